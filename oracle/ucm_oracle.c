@@ -1,0 +1,613 @@
+/*
+ * CPU oracle for the sparse-retrieval hot path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, the arithmetic of the reference's CPU
+ * retrieval path so that the HIP kernels can be checked against it bit for
+ * bit.  Nothing shipped (the package, the C-ABI library) may link or call it;
+ * only the test-suite, the smoke check and the benchmark's cpu_baseline leg do,
+ * and there only as the checker / the timed baseline.
+ *
+ * All paths below are relative to the reference tree.  Every function names
+ * the lines it follows.  Floating point order is spelled out by hand and the
+ * file is compiled with -ffp-contract=off, so results do not depend on the
+ * host ISA: the 16-lane FMA + butterfly order of the reference's AVX-512
+ * build (the canonical order of this project) is written as scalar fmaf().
+ *
+ * Pin status (what fixes each function besides this text):
+ *   orc_vector_mean / orc_q_head_mean / orc_dot16 / orc_kq_scores /
+ *   orc_topk_windows / orc_select_topk / orc_k_repre_block:
+ *       bit-exact against the reference's own translation units compiled
+ *       with -mavx512f -mfma (oracle/_ref, tests/test_oracle_pins.py) and
+ *       against the golden vectors written from that build (tests/golden).
+ *   orc_esa_retrieve: against the reference's retrieval_backend.cpp built as a
+ *       python extension (oracle/_ref) + closed form; tie order of
+ *       std::partial_sort is implementation-defined, this file defines
+ *       lower-index-first.
+ *   orc_compute_topk_len, orc_get_offset, orc_kv_gather/scatter,
+ *   orc_block_table_gather: closed forms, brute force in the tests.
+ *   orc_hash_*: closed forms (sign, LSB-first packing, <u,v> = bits-2*hamming),
+ *       brute force on tiny inputs.  The majority-vote block code is not in
+ *       the reference: parity unpinned beyond its closed form.
+ */
+#include <float.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ bf16 */
+
+ORC_API float orc_bf16_to_f32(uint16_t h)
+{
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+/* round-to-nearest-even, NaN kept quiet (what torch's float->bfloat16 does) */
+ORC_API uint16_t orc_f32_to_bf16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) { return (uint16_t)((u >> 16) | 0x0040u); }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+/* ------------------------------------------------------------ a1/a3 mean */
+
+/*
+ * ucm/sparse/gsa/offload_ops/src/vec_product.cpp:39-85 (VectorMeanImpl):
+ * mean[d] = vectors[0][d]; then += vectors[k][d] for k = 1..numK-1 in order;
+ * then *= (1.0f / numK).  Every column d is independent, so the 16-wide
+ * vector body and the scalar tail give the same value per column.
+ * `mean` may alias vectors[0] (the reference calls it in place).
+ */
+ORC_API void orc_vector_mean(const float* vectors, float* mean, uint32_t dim, uint32_t numK)
+{
+    if (numK == 0) {
+        for (uint32_t d = 0; d < dim; ++d) { mean[d] = 0.0f; }
+        return;
+    }
+    const float inv = 1.0f / (float)numK;
+    for (uint32_t d = 0; d < dim; ++d) {
+        float acc = vectors[d];
+        for (uint32_t k = 1; k < numK; ++k) { acc = acc + vectors[(size_t)k * dim + d]; }
+        mean[d] = acc * inv;
+    }
+}
+
+/*
+ * ucm/sparse/gsa/offload_ops/src/k_repre.cpp:15-35 (ComputeKRepreBlock):
+ * kArray is [kHead][blockSize][headSize] fp32, out is [kHead][headSize].
+ */
+ORC_API void orc_k_repre_block(const float* kArray, uint32_t kHead, uint32_t blockSize,
+                               uint32_t headSize, float* out)
+{
+    for (uint32_t h = 0; h < kHead; ++h) {
+        orc_vector_mean(kArray + (size_t)h * blockSize * headSize, out + (size_t)h * headSize,
+                        headSize, blockSize);
+    }
+}
+
+/*
+ * The same mean taken straight from a paged bf16 key cache
+ * [num_blocks][blockSize][kHead][headSize] (vLLM layout, k_cache = kv_cache[0],
+ * ucm/sparse/gsa/gsa.py:634-654, ucm/sparse/esa/esa.py:265-266): block
+ * block_ids[i] goes to repre row slots[i] ([kHead][headSize] fp32).
+ * round_bf16 != 0 rounds the mean to bf16 and widens it again, which is what
+ * the live path's `.mean(1)` in the model dtype followed by `.to(float32)`
+ * stores (up to torch's unspecified summation order).
+ */
+ORC_API void orc_block_mean_paged(const uint16_t* k_cache, const int32_t* block_ids,
+                                  const int32_t* slots, uint32_t n, uint32_t blockSize,
+                                  uint32_t kHead, uint32_t headSize, float* repre, int round_bf16)
+{
+    const size_t row = (size_t)kHead * headSize;
+    const float inv = 1.0f / (float)blockSize;
+#pragma omp parallel for schedule(static)
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint16_t* blk = k_cache + (size_t)block_ids[i] * blockSize * row;
+        float* out = repre + (size_t)slots[i] * row;
+        for (size_t c = 0; c < row; ++c) {
+            float acc = orc_bf16_to_f32(blk[c]);
+            for (uint32_t t = 1; t < blockSize; ++t) {
+                acc = acc + orc_bf16_to_f32(blk[(size_t)t * row + c]);
+            }
+            acc = acc * inv;
+            out[c] = round_bf16 ? orc_bf16_to_f32(orc_f32_to_bf16(acc)) : acc;
+        }
+    }
+}
+
+/*
+ * ucm/sparse/gsa/offload_ops/src/select_topk_block.cpp:101-114
+ * (ComputeQHeadMean): in place, group h of g = qHead/kHead consecutive query
+ * heads is averaged into row h.  Row h is only overwritten after group h-1..0
+ * were consumed and group h starts at row h*g >= h, so in-place is safe.
+ */
+ORC_API void orc_q_head_mean(float* q, uint32_t kHead, uint32_t qHead, uint32_t headSize)
+{
+    if (kHead == qHead) { return; }
+    const uint32_t g = qHead / kHead;
+    for (uint32_t h = 0; h < kHead; ++h) {
+        orc_vector_mean(q + (size_t)h * g * headSize, q + (size_t)h * headSize, headSize, g);
+    }
+}
+
+/* ------------------------------------------------------------- a4 scores */
+
+/*
+ * ucm/sparse/gsa/offload_ops/src/vec_product.cpp:16-37 (VectorDotImpl, AVX-512
+ * build): 16 independent lanes, lane[j] = fma(q[16i+j], k[16i+j], lane[j]) for
+ * i ascending; _mm512_reduce_add_ps (GCC avx512fintrin.h __MM512_REDUCE_OP)
+ * folds hi half onto lo half twice (16->8->4), then (x0+x2)+(x1+x3).
+ * Leftover elements (dim % 16) follow one by one as `result += q[i]*k[i]`.
+ * How that statement rounds is the compiler's choice, not the source's: GCC
+ * 11.4 at -O3 -mavx512f -mfma (the build in oracle/Makefile) vectorises the
+ * tail as an in-order reduction - groups of 8 products are rounded on their
+ * own and then added in order - and contracts the remaining (<8) elements
+ * into fused multiply-adds.  That is what is restated here so that the
+ * compiled reference can be matched for every dim; head sizes on this path
+ * are multiples of 16 and never reach the tail.
+ */
+ORC_API float orc_dot16(const float* q, const float* k, uint32_t dim)
+{
+    float lane[16];
+    for (int j = 0; j < 16; ++j) { lane[j] = 0.0f; }
+    uint32_t i = 0;
+    for (; i + 16 <= dim; i += 16) {
+        for (int j = 0; j < 16; ++j) { lane[j] = fmaf(q[i + j], k[i + j], lane[j]); }
+    }
+    float a[8], b[4];
+    for (int j = 0; j < 8; ++j) { a[j] = lane[j + 8] + lane[j]; }
+    for (int j = 0; j < 4; ++j) { b[j] = a[j + 4] + a[j]; }
+    const float c0 = b[0] + b[2];
+    const float c1 = b[1] + b[3];
+    float result = c0 + c1;
+    for (; i + 8 <= dim; i += 8) {
+        for (int j = 0; j < 8; ++j) {
+            const float p = q[i + j] * k[i + j];
+            result = result + p;
+        }
+    }
+    for (; i < dim; ++i) { result = fmaf(q[i], k[i], result); }
+    return result;
+}
+
+/*
+ * ucm/sparse/gsa/offload_ops/src/select_topk_block.cpp:53-76
+ * (ComputeBlockScore): per kv head the best (fmax, start -FLT_MAX) of the
+ * numKrepre dots, heads added in order starting from 0.0f.
+ */
+ORC_API float orc_block_score(const float* qMean, const float* blockBase, uint32_t kHead,
+                              uint32_t numKrepre, uint32_t headSize)
+{
+    float blockScore = 0.0f;
+    for (uint32_t h = 0; h < kHead; ++h) {
+        const float* q = qMean + (size_t)h * headSize;
+        const float* headBase = blockBase + (size_t)h * numKrepre * headSize;
+        float best = -FLT_MAX;
+        for (uint32_t r = 0; r < numKrepre; ++r) {
+            best = fmaxf(best, orc_dot16(q, headBase + (size_t)r * headSize, headSize));
+        }
+        blockScore = blockScore + best;
+    }
+    return blockScore;
+}
+
+/* select_topk_block.cpp:84-99 (ComputeKQDotScores); blocks are independent */
+ORC_API void orc_kq_scores(const float* qMean, const float* kRepre, uint32_t numBlock,
+                           uint32_t kHead, uint32_t numKrepre, uint32_t headSize, float* scores)
+{
+    const size_t blockOffset = (size_t)kHead * numKrepre * headSize;
+#pragma omp parallel for schedule(static)
+    for (uint32_t b = 0; b < numBlock; ++b) {
+        scores[b] = orc_block_score(qMean, kRepre + b * blockOffset, kHead, numKrepre, headSize);
+    }
+}
+
+/* --------------------------------------------------------------- a5 top-k */
+
+/* stable merge sort of indices by score descending (std::stable_sort with
+ * comparator scores[l] > scores[r]: equal scores keep their original order) */
+static void orc_stable_sort_desc(uint32_t* idx, uint32_t* tmp, uint32_t n, const float* scores)
+{
+    for (uint32_t width = 1; width < n; width *= 2) {
+        for (uint32_t lo = 0; lo < n; lo += 2 * width) {
+            uint32_t mid = lo + width < n ? lo + width : n;
+            uint32_t hi = lo + 2 * width < n ? lo + 2 * width : n;
+            uint32_t i = lo, j = mid, o = lo;
+            while (i < mid && j < hi) {
+                /* take from the right run only if it is strictly better */
+                if (scores[idx[j]] > scores[idx[i]]) { tmp[o++] = idx[j++]; }
+                else { tmp[o++] = idx[i++]; }
+            }
+            while (i < mid) { tmp[o++] = idx[i++]; }
+            while (j < hi) { tmp[o++] = idx[j++]; }
+        }
+        memcpy(idx, tmp, (size_t)n * sizeof(uint32_t));
+    }
+}
+
+static int orc_cmp_i32(const void* a, const void* b)
+{
+    const int32_t x = *(const int32_t*)a, y = *(const int32_t*)b;
+    return (x > y) - (x < y);
+}
+
+/*
+ * ucm/sparse/gsa/offload_ops/src/select_topk_block.cpp:20-51 (TopKImpl),
+ * windows from include/select_topk_block.h:20 (1 and 2 by default).
+ * Returns how many entries of `out` are meaningful: n on the identity path,
+ * k otherwise.  For 0 < k < startW+endW < n the reference writes startW+endW
+ * entries and sorts only the first k (they already ascend); the same first k
+ * are produced here and the overrun is not.
+ */
+ORC_API int32_t orc_topk_windows(const float* scores, uint32_t n, uint32_t k, uint32_t startW,
+                                 uint32_t endW, int32_t* out)
+{
+    if (startW + endW >= n || k >= n || k == 0) {
+        for (uint32_t i = 0; i < n; ++i) { out[i] = (int32_t)i; }
+        return (int32_t)n;
+    }
+    int32_t* full = (int32_t*)malloc(((size_t)k + startW + endW) * sizeof(int32_t));
+    uint32_t o = 0;
+    for (uint32_t i = 0; i < startW; ++i) { full[o++] = (int32_t)i; }
+    const int32_t midCount = (int32_t)k - (int32_t)startW - (int32_t)endW;
+    if (midCount > 0) {
+        const uint32_t m = n - startW - endW;
+        uint32_t* idx = (uint32_t*)malloc((size_t)m * sizeof(uint32_t));
+        uint32_t* tmp = (uint32_t*)malloc((size_t)m * sizeof(uint32_t));
+        for (uint32_t i = 0; i < m; ++i) { idx[i] = startW + i; }
+        orc_stable_sort_desc(idx, tmp, m, scores);
+        for (int32_t i = 0; i < midCount; ++i) { full[o++] = (int32_t)idx[i]; }
+        free(idx);
+        free(tmp);
+    }
+    for (uint32_t i = 0; i < endW; ++i) { full[o++] = (int32_t)(n - endW + i); }
+    qsort(full, k, sizeof(int32_t), orc_cmp_i32);
+    memcpy(out, full, (size_t)k * sizeof(int32_t));
+    free(full);
+    return (int32_t)k;
+}
+
+/*
+ * select_topk_block.cpp:116-129 (SelectTopK): group-mean the query in place,
+ * score every block, select.  `scores_out` (numBlock floats, may be NULL)
+ * additionally hands back the scores, which the reference keeps private.
+ */
+ORC_API int32_t orc_select_topk(float* q, const float* kRepre, uint32_t numBlock, uint32_t kHead,
+                                uint32_t qHead, uint32_t numKrepre, uint32_t headSize,
+                                uint32_t topkLength, uint32_t startW, uint32_t endW,
+                                int32_t* topkResult, float* scores_out)
+{
+    if (!q || !kRepre || !numBlock || !kHead || !qHead || !numKrepre || !headSize ||
+        !topkResult || !topkLength) {
+        return 0;
+    }
+    orc_q_head_mean(q, kHead, qHead, headSize);
+    float* scores = scores_out ? scores_out : (float*)malloc((size_t)numBlock * sizeof(float));
+    orc_kq_scores(q, kRepre, numBlock, kHead, numKrepre, headSize, scores);
+    const int32_t cnt = orc_topk_windows(scores, numBlock, topkLength, startW, endW, topkResult);
+    if (!scores_out) { free(scores); }
+    return cnt;
+}
+
+/*
+ * select_topk_block.cpp:131-149 (SelectTopKBS) over a ragged batch held in one
+ * representative table: request r owns rows seg_off[r] .. seg_off[r]+seg_len[r]-1
+ * (the contiguous per-request segment of ucm/sparse/gsa/gsa.py:188-190,
+ * cal_kpre_and_topk.cpp:219-241).  q is [numBatch][qHead][headSize] and is
+ * overwritten like in the reference.  Output row r starts at out + r*out_stride;
+ * out_count[r] receives the number of entries.  Requests are serial, blocks
+ * parallel - the reference's own schedule.
+ */
+ORC_API void orc_select_topk_bs(float* q, const float* repre, const int32_t* seg_off,
+                                const int32_t* seg_len, const int32_t* topk_len, uint32_t numBatch,
+                                uint32_t kHead, uint32_t qHead, uint32_t numKrepre,
+                                uint32_t headSize, uint32_t startW, uint32_t endW, int32_t* out,
+                                uint32_t out_stride, int32_t* out_count, float* scores_out)
+{
+    const size_t row = (size_t)kHead * numKrepre * headSize;
+    for (uint32_t r = 0; r < numBatch; ++r) {
+        out_count[r] = orc_select_topk(q + (size_t)r * qHead * headSize,
+                                       repre + (size_t)seg_off[r] * row, (uint32_t)seg_len[r],
+                                       kHead, qHead, numKrepre, headSize, (uint32_t)topk_len[r],
+                                       startW, endW, out + (size_t)r * out_stride,
+                                       scores_out ? scores_out + seg_off[r] : NULL);
+    }
+}
+
+/* ucm/sparse/utils.py:30-36 (compute_topk_len) with MIN 32 / MAX 48 (utils.py:6-7) */
+ORC_API int32_t orc_compute_topk_len(int32_t raw_seq_len)
+{
+    int32_t t = (int32_t)((double)raw_seq_len * 0.3);
+    if (t < 32) { t = raw_seq_len < 32 ? raw_seq_len : 32; }
+    else if (t > 48) { t = 48; }
+    return t;
+}
+
+/* ------------------------------------------------------------------- ESA */
+
+typedef struct { float score; int32_t idx; uint32_t pos; } orc_pair;
+
+static int orc_cmp_pair_desc(const void* a, const void* b)
+{
+    const orc_pair* x = (const orc_pair*)a;
+    const orc_pair* y = (const orc_pair*)b;
+    if (x->score > y->score) { return -1; }
+    if (x->score < y->score) { return 1; }
+    return (x->pos > y->pos) - (x->pos < y->pos);   /* defined here: earlier entry first */
+}
+
+/*
+ * ucm/sparse/esa/retrieval/cpy/retrieval_backend.cpp:170-190 (worker_loop,
+ * "for precision" branch): for every allowed slot a strictly sequential
+ * score += q[d] * data[slot*dim + d] (separate multiply and add; the module is
+ * built without FMA), then the best min(n_allowed, topk) by score descending.
+ * `indexes` is one row of the padded index matrix; entries equal to -1 are
+ * skipped (retrieval_backend.cpp:60-65).  Returns the number of results.
+ */
+ORC_API int32_t orc_esa_retrieve(const float* data, uint32_t dim, const float* q,
+                                 const int32_t* indexes, uint32_t n_indexes, int32_t topk,
+                                 int32_t* out_idx, float* out_scores)
+{
+    orc_pair* heap = (orc_pair*)malloc(((size_t)n_indexes + 1) * sizeof(orc_pair));
+    uint32_t m = 0;
+    for (uint32_t j = 0; j < n_indexes; ++j) {
+        const int32_t idx = indexes[j];
+        if (idx == -1) { continue; }
+        float score = 0.0f;
+        const float* row = data + (size_t)idx * dim;
+        for (uint32_t d = 0; d < dim; ++d) {
+            const float p = q[d] * row[d];
+            score = score + p;
+        }
+        heap[m].score = score;
+        heap[m].idx = idx;
+        heap[m].pos = m;
+        ++m;
+    }
+    int32_t cur = (int32_t)m < topk ? (int32_t)m : topk;
+    if (cur < 0) { cur = 0; }
+    qsort(heap, m, sizeof(orc_pair), orc_cmp_pair_desc);
+    for (int32_t i = 0; i < cur; ++i) {
+        out_idx[i] = heap[i].idx;
+        out_scores[i] = heap[i].score;
+    }
+    free(heap);
+    return cur;
+}
+
+/* -------------------------------------------------------- a6 block tables */
+
+/*
+ * ucm/sparse/gsa/prefetch/prefetch_engine.py:507-553 (_no_gsa_input_deal):
+ * use_block_table[:count] = block_table[topk_idx]; sparse sequence length is
+ * count*block_size when the last block is full, else
+ * count*block_size - block_size + seq_len % block_size.
+ */
+ORC_API int32_t orc_block_table_gather(const int32_t* block_table, const int32_t* topk_idx,
+                                       int32_t count, int32_t seq_len, int32_t block_size,
+                                       int32_t* phys_out)
+{
+    for (int32_t i = 0; i < count; ++i) { phys_out[i] = block_table[topk_idx[i]]; }
+    const int32_t rem = seq_len % block_size;
+    return rem == 0 ? count * block_size : count * block_size - block_size + rem;
+}
+
+/* ------------------------------------------------------ a7 paged KV moves */
+
+/*
+ * ucm/sparse/esa/esa.py:124-135 (get_offset): byte offset of one layer's K or
+ * V slice of one TP rank inside a stored block laid out [layer][K|V][rank].
+ */
+ORC_API int64_t orc_get_offset(int64_t block_size, int64_t kv_heads_per_tp, int64_t head_size,
+                               int64_t rank, int64_t tp_size, int64_t precision, int64_t layer_id,
+                               int is_v, int is_mla)
+{
+    const int64_t k_sz = block_size * kv_heads_per_tp * head_size * precision;
+    const int64_t v_sz = is_mla ? 0 : k_sz;
+    const int64_t layer_size = (k_sz + v_sz) * tp_size;
+    const int64_t k_off = is_mla ? layer_size * layer_id
+                                 : layer_size * layer_id + layer_size / tp_size * rank;
+    return is_v ? k_off + k_sz : k_off;
+}
+
+/*
+ * ucm/store/device/cuda/cuda_device.cu:47-69 (H2DKernel / D2HKernel): `num`
+ * independent copies of `size` bytes, dst[i] <- src[i].
+ */
+ORC_API void orc_copy_batch(uint8_t* const* dst, const uint8_t* const* src, size_t num, size_t size)
+{
+    for (size_t i = 0; i < num; ++i) { memcpy(dst[i], src[i], size); }
+}
+
+/*
+ * Whole-block moves between a paged cache and a staging buffer in the stored
+ * block format (ucm/sparse/esa/esa.py:222-263 launch_transfer_task with
+ * get_offset, tp_size 1): staging block i holds [layer][K|V] slices of
+ * block_bytes each; layer l's cache is layers[l] with the K plane at 0 and the
+ * V plane at kv_stride bytes (vLLM (2, num_blocks, ...) layout,
+ * ucm/sparse/gsa/gsa.py:772-778).  to_staging != 0 gathers (dump), else
+ * scatters (load).
+ */
+ORC_API void orc_kv_move_blocks(uint8_t* const* layers, uint32_t n_layers, size_t kv_stride,
+                                size_t block_bytes, const int32_t* block_ids, uint32_t n,
+                                uint8_t* staging, int to_staging)
+{
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t l = 0; l < n_layers; ++l) {
+            for (uint32_t kv = 0; kv < 2; ++kv) {
+                uint8_t* c = layers[l] + kv * kv_stride + (size_t)block_ids[i] * block_bytes;
+                uint8_t* s = staging + (((size_t)i * n_layers + l) * 2 + kv) * block_bytes;
+                if (to_staging) { memcpy(s, c, block_bytes); } else { memcpy(c, s, block_bytes); }
+            }
+        }
+    }
+}
+
+/*
+ * Gather of the selected blocks of every (layer, request) into one contiguous
+ * buffer per request: request r's region starts at dst_off[r] blocks and holds
+ * [layer][K|V][count[l][r]] blocks (the per-request buffer of the benchmark
+ * definition; the reference moves the same blocks one tensor view at a time,
+ * ucm/sparse/esa/esa.py:254-258).  phys is [n_layers][n_req][phys_stride].
+ * Regions are sized with count_max[r] = the largest count over layers.
+ */
+ORC_API void orc_kv_gather_selected(const uint8_t* const* layers, uint32_t n_layers,
+                                    size_t kv_stride, size_t block_bytes, const int32_t* phys,
+                                    const int32_t* count, uint32_t n_req, uint32_t phys_stride,
+                                    const int64_t* dst_off, const int32_t* region_k,
+                                    uint8_t* staging)
+{
+    for (uint32_t l = 0; l < n_layers; ++l) {
+        for (uint32_t r = 0; r < n_req; ++r) {
+            const int32_t c = count[(size_t)l * n_req + r];
+            for (uint32_t kv = 0; kv < 2; ++kv) {
+                for (int32_t j = 0; j < c; ++j) {
+                    const int32_t id = phys[((size_t)l * n_req + r) * phys_stride + j];
+                    const uint8_t* s = layers[l] + kv * kv_stride + (size_t)id * block_bytes;
+                    uint8_t* d = staging + ((size_t)dst_off[r] +
+                                            ((size_t)l * 2 + kv) * region_k[r] + j) * block_bytes;
+                    memcpy(d, s, block_bytes);
+                }
+            }
+        }
+    }
+}
+
+/* --------------------------------------------------------- a8 hash codes */
+
+/*
+ * ucm/sparse/kvcomp/hash_encoder.py:99-157 (compute_hash): bit c of the code is
+ * (x . W[:, c] > 0), packed LSB first: bit j of byte b is column 8b+j
+ * (hash_encoder.py:92-97,139-149).  x is [n][dim] bf16, W is [dim][bits] fp32.
+ * The projection is accumulated here in double, d ascending; the reference
+ * leaves the matmul's order to the library, so signs of projections within
+ * rounding of zero are not pinned by it.
+ */
+ORC_API void orc_hash_encode(const uint16_t* x, const float* W, uint32_t n, uint32_t dim,
+                             uint32_t bits, uint8_t* codes)
+{
+    const uint32_t nbytes = bits / 8;
+#pragma omp parallel for schedule(static)
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t b = 0; b < nbytes; ++b) {
+            uint8_t byte = 0;
+            for (uint32_t j = 0; j < 8; ++j) {
+                double acc = 0.0;
+                for (uint32_t d = 0; d < dim; ++d) {
+                    acc += (double)orc_bf16_to_f32(x[(size_t)i * dim + d]) *
+                           (double)W[(size_t)d * bits + 8 * b + j];
+                }
+                if (acc > 0.0) { byte |= (uint8_t)(1u << j); }
+            }
+            codes[(size_t)i * nbytes + b] = byte;
+        }
+    }
+}
+
+static int32_t orc_popcount_xor(const uint8_t* a, const uint8_t* b, uint32_t nbytes)
+{
+    int32_t h = 0;
+    for (uint32_t i = 0; i < nbytes; ++i) { h += __builtin_popcount((unsigned)(a[i] ^ b[i])); }
+    return h;
+}
+
+/*
+ * ucm/sparse/kvcomp/kvcomp.py:237-247 (retrieval): block score = sum over query
+ * heads i, kv heads j and the block's tokens s of <u(q_i), u(k_{n,j,s})> with
+ * u = +-1 per bit, i.e. sum of (bits - 2*hamming).  Exact in int32 (the
+ * reference rounds the same integers through fp16).  key_codes is
+ * [n_blocks][kv_heads][block_size][nbytes] (kvcomp.py:341-342), q_codes
+ * [q_heads][nbytes].
+ */
+ORC_API void orc_hash_scores_sum(const uint8_t* q_codes, uint32_t q_heads, const uint8_t* key_codes,
+                                 uint32_t n_blocks, uint32_t kv_heads, uint32_t block_size,
+                                 uint32_t nbytes, int32_t* scores)
+{
+    const int32_t bits = (int32_t)nbytes * 8;
+#pragma omp parallel for schedule(static)
+    for (uint32_t n = 0; n < n_blocks; ++n) {
+        int64_t s = 0;
+        for (uint32_t i = 0; i < q_heads; ++i) {
+            for (uint32_t j = 0; j < kv_heads; ++j) {
+                for (uint32_t t = 0; t < block_size; ++t) {
+                    const uint8_t* kc = key_codes + (((size_t)n * kv_heads + j) * block_size + t) * nbytes;
+                    s += bits - 2 * orc_popcount_xor(q_codes + (size_t)i * nbytes, kc, nbytes);
+                }
+            }
+        }
+        scores[n] = (int32_t)s;
+    }
+}
+
+/*
+ * Majority-vote block code (the benchmark's hash variant; not present in the
+ * reference): bit c of the block code of (block, kv head) is 1 when more than
+ * half of the block's tokens have bit c set; an exact tie gives 0.
+ * token_codes is [n_blocks][block_size][kv_heads][nbytes] (cache order),
+ * block_codes [n_blocks][kv_heads][nbytes].
+ */
+ORC_API void orc_hash_majority(const uint8_t* token_codes, uint32_t n_blocks, uint32_t block_size,
+                               uint32_t kv_heads, uint32_t nbytes, uint8_t* block_codes)
+{
+#pragma omp parallel for schedule(static)
+    for (uint32_t n = 0; n < n_blocks; ++n) {
+        for (uint32_t h = 0; h < kv_heads; ++h) {
+            for (uint32_t b = 0; b < nbytes; ++b) {
+                uint8_t byte = 0;
+                for (uint32_t j = 0; j < 8; ++j) {
+                    uint32_t ones = 0;
+                    for (uint32_t t = 0; t < block_size; ++t) {
+                        ones += (token_codes[(((size_t)n * block_size + t) * kv_heads + h) * nbytes + b] >> j) & 1u;
+                    }
+                    if (2 * ones > block_size) { byte |= (uint8_t)(1u << j); }
+                }
+                block_codes[((size_t)n * kv_heads + h) * nbytes + b] = byte;
+            }
+        }
+    }
+}
+
+/*
+ * Popcount similarity of the benchmark's hash variant: score[b] = sum over kv
+ * heads h of (bits - hamming(qcode[h], blockcode[b][h])).  q_codes is
+ * [kv_heads][nbytes] (one code per kv head, taken from the group-mean query).
+ */
+ORC_API void orc_hash_scores_block(const uint8_t* q_codes, const uint8_t* block_codes,
+                                   uint32_t n_blocks, uint32_t kv_heads, uint32_t nbytes,
+                                   int32_t* scores)
+{
+    const int32_t bits = (int32_t)nbytes * 8;
+    for (uint32_t b = 0; b < n_blocks; ++b) {
+        int32_t s = 0;
+        for (uint32_t h = 0; h < kv_heads; ++h) {
+            s += bits - orc_popcount_xor(q_codes + (size_t)h * nbytes,
+                                         block_codes + ((size_t)b * kv_heads + h) * nbytes, nbytes);
+        }
+        scores[b] = s;
+    }
+}
+
+/*
+ * Integer twin of orc_topk_windows for the hash variant (same rule:
+ * ucm/sparse/kvcomp/kvcomp.py:202-258 keeps init 1 / local 2 blocks out of the
+ * candidates and index-sorts the result; ties go to the lower index here,
+ * torch.topk's tie order being unspecified).
+ */
+ORC_API int32_t orc_topk_windows_i32(const int32_t* scores, uint32_t n, uint32_t k, uint32_t startW,
+                                     uint32_t endW, int32_t* out)
+{
+    float* f = (float*)malloc((size_t)(n ? n : 1) * sizeof(float));
+    /* |score| < 2^24 for every supported shape, so the conversion is exact */
+    for (uint32_t i = 0; i < n; ++i) { f[i] = (float)scores[i]; }
+    const int32_t c = orc_topk_windows(f, n, k, startW, endW, out);
+    free(f);
+    return c;
+}

@@ -1,0 +1,291 @@
+"""Pins the CPU oracle (oracle/ucm_oracle.c) before anything is compared with
+it: (1) against the golden vectors written from the reference's own C++
+(tests/golden/make_golden.py), (2) against that compiled C++ directly where
+oracle/_ref exists, (3) against closed forms / brute force chosen so that a
+dropped term, a wrong index or a flipped comparison fails."""
+import itertools
+
+import numpy as np
+import pytest
+
+import oracle as O
+import synth
+from golden.make_golden import cases_select, select_inputs
+
+bits = lambda a: np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+# ------------------------------------------------------------------ golden
+
+def test_golden_select_cases(golden):
+    z, meta = golden
+    assert meta["simd"] == "x86_64 AVX512F"
+    assert [c[0] for c in meta["select"]] == [c[0] for c in cases_select()]
+    for name, seed, n, hq, hkv, d, k, sw, ew, b16 in meta["select"]:
+        q, repre = select_inputs(seed, n, hq, hkv, d, b16)
+        qm = O.q_head_mean(q, hkv)
+        assert np.array_equal(bits(qm), bits(z[f"select/{name}/qmean"])), name
+        assert np.array_equal(bits(O.kq_scores(qm, repre)), bits(z[f"select/{name}/scores"])), name
+        idx, scores = O.select_topk(q, repre, k, sw, ew)
+        assert np.array_equal(idx, z[f"select/{name}/idx"]), name
+        assert np.array_equal(bits(scores), bits(z[f"select/{name}/scores"])), name
+
+
+def test_golden_dot_mean_krepre(golden):
+    z, meta = golden
+    for dim, s1, s2 in meta["dot"]:
+        got = O.dot16(synth.normal_f32(s1, (dim,)), synth.normal_f32(s2, (dim,)))
+        assert bits(got)[()] == bits(z[f"dot/{dim}"])[0], dim
+    for num_k, dim, seed in meta["mean"]:
+        v = synth.normal_bf16_as_f32(seed, (num_k, dim))
+        assert np.array_equal(bits(O.vector_mean(v)), bits(z[f"mean/{num_k}x{dim}"]))
+    kb = synth.normal_bf16_as_f32(450, (8, 128, 128))
+    want = z["krepre/8x128x128"]
+    assert np.array_equal(bits(O.k_repre_block(kb)), bits(want))
+    # the paged-cache entry point reads [T][H][D] bf16 instead of [H][T][D] fp32
+    cache = synth.bf16_round_bits(kb.transpose(1, 0, 2))[None]
+    repre = np.zeros((3, 8 * 128), np.float32)
+    O.block_mean_paged(cache, [0], [2], repre)
+    assert np.array_equal(bits(repre[2]), bits(want.reshape(-1)))
+    assert not repre[:2].any()
+
+
+def test_golden_ties(golden):
+    z, meta = golden
+    for i, n, k, sw, ew, seed in meta["ties"]:
+        sc = synth.ints(seed, n, 0, 3).astype(np.float32)
+        assert np.array_equal(O.topk_windows(sc, k, sw, ew), z[f"ties/{i}"]), (i, n, k, sw, ew)
+
+
+def test_golden_esa_backend(golden):
+    z, meta = golden
+    assert meta["esa"], "fixture was written without the ESA backend"
+    for i, rows, dim, b, m, topk, s_data, s_q, s_idx in meta["esa"]:
+        data = synth.normal_bf16_as_f32(s_data, (rows, dim))
+        q = synth.normal_bf16_as_f32(s_q, (b, dim))
+        idx = np.stack([synth.permutation(s_idx + r, rows)[:m] for r in range(b)]).astype(np.int32)
+        idx[:, m - 3:] = -1
+        for r in range(b):
+            gi, gs = O.esa_retrieve(data, q[r], idx[r], topk)
+            want_s = z[f"esa/{i}/scores"][r]
+            want_i = z[f"esa/{i}/indices"][r]
+            assert np.array_equal(bits(gs), bits(want_s))
+            assert len(np.unique(want_s)) == len(want_s)  # no ties in the fixture, so order is pinned
+            assert np.array_equal(gi, want_i)
+
+
+# ------------------------------------------- the compiled reference, live
+
+needs_ref = pytest.mark.skipif(not O.ref.available, reason="oracle/_ref not built (reference tree absent)")
+
+
+@needs_ref
+def test_ref_dot_and_mean_random():
+    rng = np.random.default_rng(5)
+    for dim in [1, 3, 16, 17, 48, 128, 130, 1024, 1037]:
+        for _ in range(60):
+            q = rng.standard_normal(dim).astype(np.float32) * np.float32(rng.uniform(1e-3, 1e3))
+            k = rng.standard_normal(dim).astype(np.float32)
+            assert bits(O.dot16(q, k))[()] == bits(O.ref.vector_dot(q, k))[()]
+    for num_k, dim in itertools.product([1, 2, 4, 8, 127, 128], [1, 16, 40, 128]):
+        v = rng.standard_normal((num_k, dim)).astype(np.float32)
+        assert np.array_equal(bits(O.vector_mean(v)), bits(O.ref.vector_mean(v)))
+
+
+@needs_ref
+def test_ref_select_random_shapes():
+    rng = np.random.default_rng(6)
+    for trial in range(40):
+        hkv = int(rng.choice([1, 2, 4, 8]))
+        g = int(rng.choice([1, 2, 4, 8]))
+        d = int(rng.choice([32, 64, 128]))
+        n = int(rng.integers(1, 200))
+        k = int(rng.integers(1, 60))
+        q = synth.normal_bf16_as_f32(2000 + trial, (hkv * g, d))
+        repre = synth.normal_f32(3000 + trial, (n, hkv, 1, d))
+        assert np.array_equal(bits(O.q_head_mean(q, hkv)), bits(O.ref.q_head_mean(q, hkv)))
+        idx, scores = O.select_topk(q, repre, k)
+        assert np.array_equal(bits(scores), bits(O.ref.kq_scores(O.ref.q_head_mean(q, hkv), repre)))
+        assert np.array_equal(idx, O.ref.select_topk(q, repre, k)), (trial, n, k)
+
+
+@needs_ref
+def test_ref_num_krepre_max():
+    """numKrepre > 1 takes the best representative per head (fmax)."""
+    for trial in range(10):
+        q = synth.normal_f32(4000 + trial, (8, 128))
+        repre = synth.normal_f32(4100 + trial, (37, 8, 3, 128))
+        assert np.array_equal(bits(O.kq_scores(q, repre)), bits(O.ref.kq_scores(q, repre)))
+
+
+@needs_ref
+def test_ref_ties_exhaustive_small():
+    q1 = np.ones((1, 1), np.float32)
+    rng = np.random.default_rng(7)
+    for _ in range(3000):
+        n = int(rng.integers(1, 15))
+        k = int(rng.integers(1, 17))
+        sw, ew = int(rng.integers(0, 3)), int(rng.integers(0, 4))
+        sc = rng.integers(0, 3, n).astype(np.float32)
+        want = O.ref.select_topk(q1, sc.reshape(n, 1, 1, 1), k, sw, ew)
+        assert np.array_equal(O.topk_windows(sc, k, sw, ew), want), (n, k, sw, ew, sc)
+
+
+@needs_ref
+def test_ref_batch_entry_point():
+    lens = np.array([5, 40, 3, 130, 64], np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    tk = np.array([O.compute_topk_len(int(n)) for n in lens], np.int32)
+    q = synth.normal_bf16_as_f32(5000, (len(lens), 32, 128))
+    repre = synth.normal_f32(5001, (int(lens.sum()), 8 * 128))
+    idx, cnt, _ = O.select_topk_bs(q, repre, off, lens, tk, 8, out_stride=140)
+    want = O.ref.select_topk_bs(q, repre, off, lens, tk, 8, out_stride=140)
+    for r in range(len(lens)):
+        assert np.array_equal(idx[r, : cnt[r]], want[r, : cnt[r]])
+
+
+@needs_ref
+def test_ref_esa_backend_live():
+    rb = O.ref.retrieval_backend_module()
+    if rb is None:
+        pytest.skip("retrieval_backend extension not built")
+    data = synth.normal_bf16_as_f32(6000, (200, 1024))
+    be = rb.RetrievalWorkerBackend(data)
+    q = synth.normal_bf16_as_f32(6001, (2, 1024))
+    idx = np.stack([synth.permutation(6002 + r, 200)[:150] for r in range(2)]).astype(np.int32)
+    rid = be.submit(q, 33, idx)
+    be.wait(rid)
+    res = be.get_result(rid)
+    for r in range(2):
+        gi, gs = O.esa_retrieve(data, q[r], idx[r], 33)
+        assert np.array_equal(bits(gs), bits(res["scores"][r]))
+        assert np.array_equal(gi, res["indices"][r])
+
+
+# ------------------------------------------------ closed forms, brute force
+
+def test_dot16_lane_structure():
+    """Each of the 16 lanes is its own fma chain; a one-hot probe at every
+    position must come back exactly, and the butterfly must be
+    ((l0+l8)+(l4+l12)) + ((l2+l10)+(l6+l14)) + ... : checked with values whose
+    sum depends on the association."""
+    for pos in range(128):
+        q = np.zeros(128, np.float32)
+        k = np.zeros(128, np.float32)
+        q[pos], k[pos] = 3.0, 0.5
+        assert O.dot16(q, k) == np.float32(1.5)
+    lane = np.array([1e8, 1, -1e8, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1], np.float32)
+    f = np.float32
+    a = [f(lane[j + 8] + lane[j]) for j in range(8)]
+    b = [f(a[j + 4] + a[j]) for j in range(4)]
+    want = f(f(b[0] + b[2]) + f(b[1] + b[3]))
+    assert O.dot16(lane, np.ones(16, np.float32)) == want
+    assert want != np.float32(np.sum(lane.astype(np.float64)))  # the probe does depend on the order
+    # fma, not mul-then-add: (1+2^-12)^2 - 1 keeps the 2^-24 term only when fused
+    x = np.float32(1 + 2.0 ** -12)
+    q = np.zeros(32, np.float32)
+    k = np.zeros(32, np.float32)
+    q[0], k[0] = 1.0, -1.0
+    q[16], k[16] = x, x
+    assert O.dot16(q, k) == np.float32(2.0 ** -11 + 2.0 ** -24)
+
+
+def test_mean_is_sequential_fp32():
+    v = np.array([[1e8], [1.0], [-1e8], [1.0]], np.float32)
+    f = np.float32
+    want = f(f(f(f(v[0, 0] + v[1, 0]) + v[2, 0]) + v[3, 0]) * f(0.25))
+    assert O.vector_mean(v)[0] == want == f(0.25)
+    q = np.arange(4 * 8, dtype=np.float32).reshape(4, 8)
+    assert np.array_equal(O.q_head_mean(q, 2), np.stack([q[:2].mean(0), q[2:].mean(0)]))
+    assert np.array_equal(O.q_head_mean(q, 4), q)
+
+
+def test_topk_windows_brute_force():
+    rng = np.random.default_rng(8)
+    for _ in range(2000):
+        n = int(rng.integers(1, 12))
+        k = int(rng.integers(0, 14))
+        sw, ew = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        sc = rng.integers(0, 4, n).astype(np.float32)
+        got = O.topk_windows(sc, k, sw, ew)
+        if sw + ew >= n or k >= n or k == 0:
+            assert np.array_equal(got, np.arange(n))
+            continue
+        mid = sorted(range(sw, n - ew), key=lambda i: (-sc[i], i))[: max(k - sw - ew, 0)]
+        full = list(range(sw)) + mid + list(range(n - ew, n))
+        want = sorted(full[:k]) if k >= sw + ew else full[:k]
+        assert list(got) == want, (n, k, sw, ew, sc)
+        assert len(got) == k and all(np.diff(got) > 0)
+
+
+def test_compute_topk_len_closed_form():
+    for n in range(0, 400):
+        t = int(n * 0.3)
+        want = min(32, n) if t < 32 else (48 if t > 48 else t)
+        assert O.compute_topk_len(n) == want
+    assert O.compute_topk_len(256) == 48 and O.compute_topk_len(20) == 20 and O.compute_topk_len(120) == 36
+
+
+def test_get_offset_and_block_table():
+    shape = (128, 8, 128)
+    k_sz = 128 * 8 * 128 * 2
+    assert O.get_offset(shape, 0, 1, 2, 0, False) == 0
+    assert O.get_offset(shape, 0, 1, 2, 0, True) == k_sz
+    assert O.get_offset(shape, 0, 1, 2, 5, False) == 5 * 2 * k_sz
+    assert O.get_offset(shape, 1, 2, 2, 3, True) == 3 * 4 * k_sz + 2 * k_sz + k_sz
+    assert O.get_offset(shape, 1, 2, 2, 3, False, is_mla=True) == 3 * 2 * k_sz
+    table = np.array([9, 4, 7, 1, 3], np.int32)
+    phys, sl = O.block_table_gather(table, [0, 2, 4], 5 * 128, 128)
+    assert list(phys) == [9, 7, 3] and sl == 3 * 128
+    _, sl = O.block_table_gather(table, [0, 2, 4], 4 * 128 + 17, 128)
+    assert sl == 2 * 128 + 17
+
+
+def test_kv_moves_round_trip():
+    n_layers, nb, bb = 3, 11, 64
+    rng = np.random.default_rng(9)
+    layers = [rng.integers(0, 256, 2 * nb * bb, dtype=np.uint8) for _ in range(n_layers)]
+    ids = np.array([7, 0, 10, 3], np.int32)
+    staging = np.zeros(len(ids) * n_layers * 2 * bb, np.uint8)
+    O.kv_move_blocks(layers, nb * bb, bb, ids, staging, True)
+    st = staging.reshape(len(ids), n_layers, 2, bb)
+    for i, b in enumerate(ids):
+        for l in range(n_layers):
+            for kv in range(2):
+                assert np.array_equal(st[i, l, kv], layers[l].reshape(2, nb, bb)[kv, b])
+                off = O.get_offset((bb, 1, 1), 0, 1, 1, l, bool(kv))
+                assert np.array_equal(staging[i * n_layers * 2 * bb + off:][:bb], st[i, l, kv])
+    fresh = [np.zeros_like(a) for a in layers]
+    O.kv_move_blocks(fresh, nb * bb, bb, ids, staging, False)
+    for l in range(n_layers):
+        f, o = fresh[l].reshape(2, nb, bb), layers[l].reshape(2, nb, bb)
+        assert np.array_equal(f[:, ids], o[:, ids])
+        rest = np.setdiff1d(np.arange(nb), ids)
+        assert not f[:, rest].any()
+
+
+def test_hash_closed_forms():
+    rng = np.random.default_rng(10)
+    dim, nbits = 16, 24
+    w = rng.standard_normal((dim, nbits)).astype(np.float32) * 2
+    xb = synth.normal_bf16_bits(7000, (5, 3, dim))
+    x = synth.bf16_widen(xb).astype(np.float64)
+    proj = x @ w.astype(np.float64)
+    want_bits = (proj > 0).astype(np.uint8).reshape(5, 3, nbits // 8, 8)
+    want = (want_bits * (1 << np.arange(8, dtype=np.uint8))).sum(-1).astype(np.uint8)
+    got = O.hash_encode(xb, w)
+    assert got.shape == (5, 3, 3) and np.array_equal(got, want)
+    # sum score == explicit +-1 inner products
+    qc = rng.integers(0, 256, (4, 3), dtype=np.uint8)
+    kc = rng.integers(0, 256, (6, 2, 5, 3), dtype=np.uint8)
+    un = lambda c: np.unpackbits(c, axis=-1, bitorder="little").astype(np.int64) * 2 - 1
+    want = np.einsum("id,njsd->n", un(qc), un(kc))
+    assert np.array_equal(O.hash_scores_sum(qc, kc), want)
+    # majority vote and popcount similarity
+    tc = rng.integers(0, 256, (3, 8, 2, 3), dtype=np.uint8)
+    ones = np.unpackbits(tc, axis=-1, bitorder="little").sum(1)
+    want_codes = np.packbits((2 * ones > 8).astype(np.uint8), axis=-1, bitorder="little")
+    assert np.array_equal(O.hash_majority(tc), want_codes)
+    q2 = rng.integers(0, 256, (2, 3), dtype=np.uint8)
+    sim = (nbits - np.unpackbits(q2[None] ^ want_codes, axis=-1).sum(-1)).sum(-1)
+    assert np.array_equal(O.hash_scores_block(q2, want_codes), sim)
