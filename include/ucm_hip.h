@@ -1,0 +1,187 @@
+/*
+ * libucm_hip.so - C ABI of the MI355X (gfx950) sparse-retrieval hot path.
+ *
+ * Plain pointers and sizes only; every pointer marked "dev" is device memory
+ * (anything a HIP kernel can dereference, which includes mapped pinned host
+ * memory for the staging side of the KV moves).  The library allocates nothing
+ * and never synchronises: each call validates its arguments on the host,
+ * enqueues its kernels on `stream` (a hipStream_t, NULL = the null stream) and
+ * returns.  Return value: 0 on success, a negative errno-style code otherwise
+ * (UCM_EINVAL bad argument, UCM_ENOTSUP shape outside what the kernels were
+ * built for, UCM_EHIP a HIP runtime error); ucm_last_error() has the text.
+ *
+ * Reference paths are relative to the upstream tree; each entry point names
+ * the reference interface it stands in for.
+ *
+ * Shared conventions
+ *   layers      dev array of n_layers pointers, one per model layer.  For the
+ *               KV moves a layer pointer is the start of that layer's
+ *               (2, num_blocks, block_size, kv_heads, head_dim) cache (K plane
+ *               first, V plane kv_stride bytes later: vLLM layout,
+ *               ucm/sparse/gsa/gsa.py:772-778).  For ucm_block_mean it is the
+ *               K plane.
+ *   repre       one table of block representatives for all layers:
+ *               fp32 [n_layers][repre_rows][kv_heads*head_dim]; layer l starts
+ *               at repre + l*repre_layer_stride floats.  A request owns the
+ *               contiguous rows seg_off[r] .. seg_off[r]+seg_len[r]-1, the
+ *               layout of the reference's kpre_caches
+ *               (ucm/sparse/gsa/prefetch/prefetch_engine.py:64-77, slots from
+ *               ucm/sparse/gsa/gsa.py:188-190).
+ */
+#ifndef UCM_HIP_H
+#define UCM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UCM_OK 0
+#define UCM_EINVAL (-22)
+#define UCM_ENOTSUP (-95)
+#define UCM_EHIP (-5)
+
+#define UCM_DTYPE_F32 0
+#define UCM_DTYPE_BF16 1
+
+/* ucm_block_mean modes */
+#define UCM_MEAN_F32 0       /* fp32 mean kept as is (the C++ KRepreComputer contract) */
+#define UCM_MEAN_BF16_ROUND 1 /* mean rounded to bf16 and widened (what the live torch path stores) */
+
+typedef void* ucm_stream_t; /* hipStream_t */
+
+/* Library version (major*10000 + minor*100 + patch) and the text of the last
+ * error raised on the calling thread ("" if none). */
+int ucm_version(void);
+const char* ucm_last_error(void);
+
+/*
+ * Block representatives: mean over the block_size tokens of each listed block,
+ * per (kv head, dim), accumulated in fp32 in token order and multiplied by
+ * 1/block_size - the arithmetic of KRepreComputer::ComputeKRepreBlock
+ * (ucm/sparse/gsa/offload_ops/src/k_repre.cpp:15-35 with VectorMeanImpl,
+ * src/vec_product.cpp:39-85), read straight from the paged bf16 key cache the
+ * way the live hooks index it (GSA.copy_k, ucm/sparse/gsa/gsa.py:634-654;
+ * ReqStatePerLayer.extract_block_repre, ucm/sparse/esa/esa.py:265-266).
+ *   k_layers   dev: n_layers pointers to bf16 [num_blocks][block_size][kv_heads][head_dim]
+ *   block_ids  dev int32[n]: cache blocks to reduce (same ids in every layer)
+ *   slots      dev int32[n]: destination row of each block in `repre`
+ *   num_blocks, repre_rows: sizes of a K plane and of one layer's table; an id
+ *              or slot outside them is skipped by the kernel, not dereferenced.
+ * Requires kv_heads*head_dim to be a multiple of 8 and 16-byte aligned planes.
+ */
+int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
+                   const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                   int kv_heads, int head_dim, float* repre, int repre_rows,
+                   int64_t repre_layer_stride, int mode, ucm_stream_t stream);
+
+/*
+ * Scores of every block of a ragged batch, all layers in one launch:
+ *   qbar[h]  = (q[h*g] + q[h*g+1] + ... + q[h*g+g-1]) * (1/g),  g = q_heads/kv_heads
+ *   score[b] = sum over kv heads h, in order, of dot(qbar[h], repre[b][h])
+ * with dot() in the 16-lane FMA + pairwise fold order of the reference's
+ * AVX-512 build, so the fp32 results equal TopkBlockSelector::ComputeQHeadMean
+ * + ComputeKQDotScores bit for bit
+ * (ucm/sparse/gsa/offload_ops/src/select_topk_block.cpp:53-114,
+ * src/vec_product.cpp:16-37; one representative per head, numKrepre = 1, as
+ * ucm/sparse/gsa/gsa.py:501 configures it).
+ *   q          dev: queries, q_dtype fp32 or bf16, [n_layers][*][q_heads][head_dim];
+ *              layer l starts q_layer_stride ELEMENTS after layer l-1; request
+ *              r reads row q_rows[r] (q_rows == NULL: row r).  This is the
+ *              reference's gsa_q_cache (gsa.py:503-512) when fp32, or the
+ *              layer's raw query tensor with q_rows = index of each request's
+ *              last token (GSA.copy_q, gsa.py:616-632) when bf16.
+ *   seg_off, seg_len  dev int32[n_req]: first representative row and number of
+ *              blocks of each request; max_seg_len >= every seg_len (host
+ *              value, sizes the grid).
+ *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x].
+ * head_dim must be 64 or 128 and kv_heads one of 1, 2, 4, 8, 16.
+ */
+int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
+                     int q_heads, const float* repre, int64_t repre_layer_stride,
+                     const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
+                     int n_layers, int kv_heads, int head_dim, float* scores,
+                     int64_t scores_layer_stride, ucm_stream_t stream);
+
+/* Tuning knob for benchmarks: blocks scored per workgroup by ucm_score_blocks
+ * (default 32).  Not part of the reference interface. */
+int ucm_set_score_tile(int tile_blocks);
+
+/*
+ * Per-request block selection with forced windows, all layers in one launch -
+ * TopkBlockSelector::TopKImpl (select_topk_block.cpp:20-51; windows 1 and 2 by
+ * default, include/select_topk_block.h:20): if start_w+end_w >= n or k >= n or
+ * k == 0 the result is 0..n-1 (n entries); otherwise the first start_w blocks,
+ * the k-start_w-end_w best of the rest by score (equal scores: lower index
+ * first, as std::stable_sort leaves them) and the last end_w blocks, sorted
+ * ascending.  k = topk_len[r] is the total (ucm/sparse/utils.py:30-36).
+ *   idx_out    dev int32: entry j of request r in layer l at
+ *              idx_out[(l*n_req + r)*out_stride + j]; out_stride must hold
+ *              max(k, n) of every request.
+ *   count_out  dev int32[n_layers][n_req]: entries written.
+ * Optionally (block_tables != NULL) the logical->physical step of
+ * GSAPrefetchBase._no_gsa_input_deal
+ * (ucm/sparse/gsa/prefetch/prefetch_engine.py:507-553) is fused in:
+ *   block_tables  dev int32[n_req][bt_stride]: cache block id of logical block i
+ *   phys_out      dev int32, same layout as idx_out: block_tables[r][idx]
+ *   seq_lens      dev int32[n_req] (may be NULL): tokens of each request;
+ *   sparse_seq_lens dev int32[n_layers][n_req]: count*block_size, minus
+ *              block_size - seq_len%block_size when the last block is partial.
+ * Up to 4096 blocks per request.
+ */
+int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off,
+                     const int32_t* seg_len, const int32_t* topk_len, int n_req, int max_seg_len,
+                     int n_layers, int start_w, int end_w, int32_t* idx_out, int out_stride,
+                     int32_t* count_out, const int32_t* block_tables, int bt_stride,
+                     int32_t* phys_out, const int32_t* seq_lens, int block_size,
+                     int32_t* sparse_seq_lens, ucm_stream_t stream);
+
+/*
+ * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched
+ * pointer-array copy of the reference's device layer (H2DKernel / D2HKernel,
+ * ucm/store/device/cuda/cuda_device.cu:47-81, reached through
+ * H2DBatchSync / D2HBatchSync :180-211).  dst/src are dev arrays of `num`
+ * pointers; size and every pointer must be multiples of 16.
+ */
+int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t size,
+                   ucm_stream_t stream);
+
+/*
+ * Whole-block dump (cache -> staging) and load (staging -> cache) driven by a
+ * list of cache block ids - launch_transfer_task's "dump"/"load"
+ * (ucm/sparse/esa/esa.py:222-263, ucm/sparse/gsa/gsa.py:518-560) without one
+ * tensor view and one memcpy per block.  Staging block i is in the stored-block
+ * format of get_offset (esa.py:124-135, tp_size 1): [layer][K|V] slices of
+ * block_bytes each, i.e. slice (i, l, kv) at ((i*n_layers + l)*2 + kv)*block_bytes.
+ * block_bytes, kv_stride and all base pointers must be multiples of 16.
+ * num_blocks is the number of blocks of one K (or V) plane; an id outside
+ * [0, num_blocks) is skipped by the kernel instead of being dereferenced.
+ */
+int ucm_kv_gather_blocks(const void* const* layers, int n_layers, size_t kv_stride,
+                         size_t block_bytes, int num_blocks, const int32_t* block_ids, int n,
+                         void* staging, ucm_stream_t stream);
+int ucm_kv_scatter_blocks(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                          int num_blocks, const int32_t* block_ids, int n, const void* staging,
+                          ucm_stream_t stream);
+
+/*
+ * Gather of the blocks chosen by ucm_topk_windows, straight from its device
+ * output (no host round trip): request r's region of `staging` starts at
+ * dst_off[r] blocks and holds [layer][K|V][region_k[r]] blocks, of which the
+ * first count[l][r] are written.  The reference moves the same blocks one
+ * tensor view at a time (esa.py:254-258).
+ *   phys   dev int32[n_layers][n_req][phys_stride], count dev int32[n_layers][n_req]
+ *   dst_off dev int64[n_req], region_k dev int32[n_req]; max_count >= every count.
+ */
+int ucm_kv_gather_selected(const void* const* layers, int n_layers, size_t kv_stride,
+                           size_t block_bytes, int num_blocks, const int32_t* phys,
+                           const int32_t* count, int n_req, int phys_stride, const int64_t* dst_off,
+                           const int32_t* region_k, int max_count, void* staging,
+                           ucm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UCM_HIP_H */

@@ -1,0 +1,64 @@
+"""ctypes binding of libucm_hip.so (declarations mirror include/ucm_hip.h)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libucm_hip.so")
+
+OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5
+DTYPE_F32, DTYPE_BF16 = 0, 1
+MEAN_F32, MEAN_BF16_ROUND = 0, 1
+
+_p, _i, _i64, _sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
+
+# name -> argtypes, in the order of include/ucm_hip.h
+SIGNATURES = {
+    "ucm_version": [],
+    "ucm_last_error": [],
+    "ucm_block_mean": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i64, _i, _p],
+    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i64, _p, _p, _i, _i, _i, _i, _i, _p, _i64, _p],
+    "ucm_set_score_tile": [_i],
+    "ucm_topk_windows": [_p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
+    "ucm_copy_batch": [_p, _p, _sz, _sz, _p],
+    "ucm_kv_gather_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
+    "ucm_kv_scatter_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
+    "ucm_kv_gather_selected": [_p, _i, _sz, _sz, _i, _p, _p, _i, _i, _p, _p, _i, _p, _p],
+}
+
+
+class UcmHipError(RuntimeError):
+    def __init__(self, fn: str, code: int, text: str):
+        super().__init__(f"{fn} failed with {code}: {text}")
+        self.code = code
+
+
+def load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python unified-cache-management_amd/build.py` "
+            "(the HIP library is the only implementation; there is no CPU fallback)"
+        )
+    lib = C.CDLL(LIB_PATH)
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
+        fn.argtypes = argtypes
+        fn.restype = C.c_char_p if name == "ucm_last_error" else C.c_int
+    return lib
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        _lib = load()
+    return _lib
+
+
+def call(name: str, *args) -> None:
+    rc = getattr(lib(), name)(*args)
+    if rc != OK:
+        raise UcmHipError(name, rc, lib().ucm_last_error().decode())

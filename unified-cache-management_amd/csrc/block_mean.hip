@@ -1,0 +1,124 @@
+// Block representatives: per (kv head, dim) mean over a cache block's tokens,
+// fp32 accumulation in token order (column-independent, so every thread owns
+// whole columns and the order inside a column is the reference's).
+//
+// HBM-bound: block_size*row*2 bytes read per block, row*4 written.  A token
+// row of the key cache ([kv_heads][head_dim] bf16) is contiguous, so a thread
+// owns 8 adjacent columns (one 16-byte load per token) and a workgroup of 128
+// threads covers 1024 columns = one whole Llama-shape row; the token loop is
+// unrolled 16 deep so 16 x 2 KiB of loads are in flight per workgroup.
+#include "common.h"
+
+namespace {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 128;
+constexpr int kCols = 8;      // bf16 columns per thread
+constexpr int kUnroll = 16;   // token rows in flight
+
+__device__ __forceinline__ float bf16_lo(unsigned w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(unsigned w) { return __uint_as_float(w & 0xffff0000u); }
+
+__device__ __forceinline__ float round_bf16(float x)
+{
+    unsigned u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) { return __uint_as_float((u | 0x00400000u) & 0xffff0000u); }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return __uint_as_float(u & 0xffff0000u);
+}
+
+__device__ __forceinline__ void widen(const u32x4 v, float (&f)[kCols])
+{
+    f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x);
+    f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+    f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z);
+    f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+}
+
+// grid: x = block index in the list * col_groups + column group of 1024, y = layer
+__global__ __launch_bounds__(kThreads) void block_mean_kernel(
+    const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
+    const int32_t* __restrict__ slots, unsigned num_blocks, unsigned repre_rows, unsigned block_size,
+    unsigned row /* kv_heads*head_dim */, float* __restrict__ repre, int64_t repre_layer_stride,
+    int round_to_bf16, unsigned col_groups)
+{
+    const unsigned item = blockIdx.x / col_groups;
+    const unsigned col = ((blockIdx.x % col_groups) * kThreads + threadIdx.x) * kCols;
+    if (col >= row) { return; }
+    const unsigned id = static_cast<unsigned>(block_ids[item]);
+    const unsigned slot = static_cast<unsigned>(slots[item]);
+    if (id >= num_blocks || slot >= repre_rows) { return; }  // never dereference a bad id
+
+    const uint16_t* base = static_cast<const uint16_t*>(k_layers[blockIdx.y]) +
+                           static_cast<size_t>(id) * block_size * row + col;
+    float acc[kCols];
+    widen(*reinterpret_cast<const u32x4*>(base), acc);  // acc = token 0
+
+    unsigned t = 1;
+    // full groups of kUnroll tokens: loads first, then the ordered adds
+    for (; t + kUnroll <= block_size; t += kUnroll) {
+        u32x4 v[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            v[u] = __builtin_nontemporal_load(
+                reinterpret_cast<const u32x4*>(base + static_cast<size_t>(t + u) * row));
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+            float f[kCols];
+            widen(v[u], f);
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
+        }
+    }
+    for (; t < block_size; ++t) {
+        float f[kCols];
+        widen(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + static_cast<size_t>(t) * row)), f);
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
+    }
+
+    const float inv = 1.0f / static_cast<float>(block_size);
+#pragma unroll
+    for (int c = 0; c < kCols; ++c) {
+        acc[c] = acc[c] * inv;
+        if (round_to_bf16) { acc[c] = round_bf16(acc[c]); }
+    }
+    float* out = repre + static_cast<int64_t>(blockIdx.y) * repre_layer_stride +
+                 static_cast<size_t>(slot) * row + col;
+    f32x4 lo = {acc[0], acc[1], acc[2], acc[3]};
+    f32x4 hi = {acc[4], acc[5], acc[6], acc[7]};
+    *reinterpret_cast<f32x4*>(out) = lo;
+    *reinterpret_cast<f32x4*>(out + 4) = hi;
+}
+
+}  // namespace
+
+extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
+                              const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                              int kv_heads, int head_dim, float* repre, int repre_rows,
+                              int64_t repre_layer_stride, int mode, ucm_stream_t stream)
+{
+    UCM_REQUIRE(k_layers && block_ids && slots && repre, "ucm_block_mean: null pointer");
+    UCM_REQUIRE(n_layers > 0 && n_layers <= 65535, "ucm_block_mean: n_layers=%d", n_layers);
+    UCM_REQUIRE(n >= 0, "ucm_block_mean: n=%d", n);
+    UCM_REQUIRE(block_size > 0 && kv_heads > 0 && head_dim > 0 && num_blocks > 0 && repre_rows > 0,
+                "ucm_block_mean: non-positive shape");
+    UCM_REQUIRE(mode == UCM_MEAN_F32 || mode == UCM_MEAN_BF16_ROUND, "ucm_block_mean: mode=%d", mode);
+    const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
+    UCM_SUPPORTED(row % kCols == 0, "ucm_block_mean: kv_heads*head_dim=%u must be a multiple of %d", row, kCols);
+    UCM_REQUIRE(repre_layer_stride >= static_cast<int64_t>(repre_rows) * row || n_layers == 1,
+                "ucm_block_mean: repre_layer_stride=%lld smaller than one layer's table",
+                static_cast<long long>(repre_layer_stride));
+    UCM_REQUIRE(ucm::aligned16(repre) && (repre_layer_stride % 4 == 0), "ucm_block_mean: repre not 16-byte aligned");
+    if (n == 0) { return UCM_OK; }
+    const unsigned gx = (row / kCols + kThreads - 1) / kThreads;
+    UCM_REQUIRE(static_cast<uint64_t>(n) * gx <= 0x7fffffffull, "ucm_block_mean: too many blocks for one launch");
+    hipLaunchKernelGGL(block_mean_kernel, dim3(static_cast<unsigned>(n) * gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream),
+                       k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
+                       static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row, repre,
+                       repre_layer_stride, mode == UCM_MEAN_BF16_ROUND ? 1 : 0, gx);
+    UCM_LAUNCH_CHECK("ucm_block_mean");
+}

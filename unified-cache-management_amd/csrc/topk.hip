@@ -1,0 +1,158 @@
+// Per-request block selection with forced windows: one 64-wide wavefront per
+// (layer, request), the request's scores held in registers as order-preserving
+// 32-bit keys (element i lives in lane i%64, register i/64).
+//
+// Selection is a radix select, one bit per step from the top: the threshold T
+// is grown greedily while at least m candidates have key >= T, each count being
+// a wave ballot + popcount.  Candidates with key > T are all taken; of those
+// with key == T the first `m - count(key > T)` in index order are taken, which
+// is exactly where a stable descending sort leaves equal scores.  Output
+// positions are ballot prefix counts in index order, so the result comes out
+// sorted ascending with no sort at all, and the logical->physical block-table
+// lookup is applied on the way out.
+//
+// A few KB in, a few hundred bytes out per wave: this kernel is latency-bound,
+// not bandwidth-bound; it only has to stay small next to scoring and gather.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ unsigned ordered_key(float f)
+{
+    f = f + 0.0f;  // -0.0 -> +0.0, so that the two zeros tie like they do under operator>
+    const unsigned u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ unsigned lanes_below(unsigned long long mask)
+{
+    return __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
+}
+
+// grid: x = request, y = layer; block = one wave
+template <int kEpl>
+__global__ __launch_bounds__(64) void topk_windows_kernel(
+    const float* __restrict__ scores, int64_t scores_layer_stride, const int32_t* __restrict__ seg_off,
+    const int32_t* __restrict__ seg_len, const int32_t* __restrict__ topk_len, int n_req, int start_w,
+    int end_w, int32_t* __restrict__ idx_out, int out_stride, int32_t* __restrict__ count_out,
+    const int32_t* __restrict__ block_tables, int bt_stride, int32_t* __restrict__ phys_out,
+    const int32_t* __restrict__ seq_lens, int block_size, int32_t* __restrict__ sparse_seq_lens)
+{
+    const int r = blockIdx.x, l = blockIdx.y, lane = threadIdx.x;
+    const size_t lr = static_cast<size_t>(l) * n_req + r;
+    int n = seg_len[r];
+    n = min(n, min(out_stride, 64 * kEpl));  // host checked; clamp so nothing can run past a row
+    const int k = topk_len[r];
+    int32_t* out = idx_out + lr * out_stride;
+    int32_t* pout = phys_out ? phys_out + lr * out_stride : nullptr;
+    const int32_t* bt = block_tables ? block_tables + static_cast<size_t>(r) * bt_stride : nullptr;
+    int count = 0;
+
+    if (n <= 0) {
+        count = 0;
+    } else if (start_w + end_w >= n || k >= n || k <= 0) {
+        for (int i = lane; i < n; i += 64) {
+            out[i] = i;
+            if (pout) { pout[i] = bt[i]; }
+        }
+        count = n;
+    } else if (k < start_w + end_w) {
+        // fewer slots than forced blocks: the first k of [0..start_w) ++ [n-end_w..n)
+        for (int j = lane; j < k; j += 64) {
+            const int idx = j < start_w ? j : n - end_w + (j - start_w);
+            out[j] = idx;
+            if (pout) { pout[j] = bt[idx]; }
+        }
+        count = k;
+    } else {
+        const int m = k - start_w - end_w;       // free picks among the middle blocks
+        const int hi = n - end_w;                // candidates are start_w <= i < hi
+        const float* s = scores + static_cast<int64_t>(l) * scores_layer_stride + seg_off[r];
+        unsigned key[kEpl];
+#pragma unroll
+        for (int j = 0; j < kEpl; ++j) {
+            const int i = j * 64 + lane;
+            const bool cand = i >= start_w && i < hi;
+            key[j] = cand ? ordered_key(s[cand ? i : 0]) : 0u;
+        }
+        unsigned T = 0;
+        int need = 0;
+        if (m > 0) {
+            for (int bit = 31; bit >= 0; --bit) {
+                const unsigned c = T | (1u << bit);
+                int cnt = 0;
+#pragma unroll
+                for (int j = 0; j < kEpl; ++j) { cnt += __popcll(__ballot(key[j] >= c)); }
+                if (cnt >= m) { T = c; }
+            }
+            int greater = 0;
+#pragma unroll
+            for (int j = 0; j < kEpl; ++j) { greater += __popcll(__ballot(key[j] > T)); }
+            need = m - greater;
+        }
+        int pos = 0, ties_seen = 0;
+#pragma unroll
+        for (int j = 0; j < kEpl; ++j) {
+            if (j * 64 < n) {
+                const int i = j * 64 + lane;
+                const bool window = i < n && (i < start_w || i >= hi);
+                const bool cand = i >= start_w && i < hi;
+                const bool gt = cand && m > 0 && key[j] > T;
+                const bool eq = cand && m > 0 && key[j] == T;
+                const unsigned long long eq_mask = __ballot(eq);
+                const bool take = window || gt || (eq && ties_seen + static_cast<int>(lanes_below(eq_mask)) < need);
+                ties_seen += __popcll(eq_mask);
+                const unsigned long long take_mask = __ballot(take);
+                if (take) {
+                    const int p = pos + static_cast<int>(lanes_below(take_mask));
+                    out[p] = i;
+                    if (pout) { pout[p] = bt[i]; }
+                }
+                pos += __popcll(take_mask);
+            }
+        }
+        count = pos;
+    }
+    if (lane == 0) {
+        count_out[lr] = count;
+        if (sparse_seq_lens && seq_lens) {
+            const int rem = seq_lens[r] % block_size;
+            sparse_seq_lens[lr] = rem == 0 ? count * block_size : count * block_size - block_size + rem;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off,
+                                const int32_t* seg_len, const int32_t* topk_len, int n_req, int max_seg_len,
+                                int n_layers, int start_w, int end_w, int32_t* idx_out, int out_stride,
+                                int32_t* count_out, const int32_t* block_tables, int bt_stride,
+                                int32_t* phys_out, const int32_t* seq_lens, int block_size,
+                                int32_t* sparse_seq_lens, ucm_stream_t stream)
+{
+    UCM_REQUIRE(scores && seg_off && seg_len && topk_len && idx_out && count_out, "ucm_topk_windows: null pointer");
+    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_topk_windows: n_req=%d n_layers=%d", n_req, n_layers);
+    UCM_REQUIRE(start_w >= 0 && end_w >= 0 && max_seg_len >= 0, "ucm_topk_windows: negative window or length");
+    UCM_REQUIRE(out_stride >= max_seg_len, "ucm_topk_windows: out_stride=%d < max_seg_len=%d", out_stride, max_seg_len);
+    UCM_REQUIRE((block_tables == nullptr) == (phys_out == nullptr),
+                "ucm_topk_windows: block_tables and phys_out go together");
+    UCM_REQUIRE(!block_tables || bt_stride >= max_seg_len, "ucm_topk_windows: bt_stride=%d < max_seg_len=%d",
+                bt_stride, max_seg_len);
+    UCM_REQUIRE(!sparse_seq_lens || (seq_lens && block_size > 0), "ucm_topk_windows: sparse_seq_lens needs seq_lens and block_size");
+    UCM_SUPPORTED(max_seg_len <= 4096, "ucm_topk_windows: max_seg_len=%d (at most 4096 blocks per request)", max_seg_len);
+    if (n_req == 0) { return UCM_OK; }
+    hipStream_t s = ucm::as_stream(stream);
+    const dim3 grid(n_req, n_layers), block(64);
+#define UCM_TOPK_LAUNCH(EPL)                                                                                  \
+    hipLaunchKernelGGL(topk_windows_kernel<EPL>, grid, block, 0, s, scores, scores_layer_stride, seg_off,    \
+                       seg_len, topk_len, n_req, start_w, end_w, idx_out, out_stride, count_out, block_tables, \
+                       bt_stride, phys_out, seq_lens, block_size, sparse_seq_lens)
+    if (max_seg_len <= 64) { UCM_TOPK_LAUNCH(1); }
+    else if (max_seg_len <= 256) { UCM_TOPK_LAUNCH(4); }
+    else if (max_seg_len <= 1024) { UCM_TOPK_LAUNCH(16); }
+    else { UCM_TOPK_LAUNCH(64); }
+#undef UCM_TOPK_LAUNCH
+    UCM_LAUNCH_CHECK("ucm_topk_windows");
+}

@@ -1,0 +1,196 @@
+"""Torch-tensor front end of libucm_hip.so.
+
+Every function takes CUDA(HIP) tensors, checks shapes/dtypes/contiguity on the
+host, and enqueues the kernel on torch's current stream through the C ABI
+(raw pointers only).  Nothing here computes on the CPU.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import MEAN_BF16_ROUND, MEAN_F32, UcmHipError  # noqa: F401
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, dtype, name: str) -> int:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t.data_ptr()
+
+
+def _opt(t: Optional[torch.Tensor], dtype, name: str):
+    return None if t is None else _dev(t, dtype, name)
+
+
+class LayerPointers:
+    """Device array of per-layer base pointers (one int64 tensor, built once).
+
+    ``tensors`` are the per-layer cache tensors; they are kept alive here.
+    ``sub(l)`` is the address of entry l, i.e. a one-layer pointer array.
+    """
+
+    def __init__(self, tensors: Sequence[torch.Tensor]):
+        self.tensors = list(tensors)
+        for t in self.tensors:
+            if not t.is_cuda or not t.is_contiguous():
+                raise ValueError("layer tensors must be contiguous device tensors")
+            if t.data_ptr() % 16:
+                raise ValueError("layer tensors must be 16-byte aligned")
+        self.table = torch.tensor([t.data_ptr() for t in self.tensors], dtype=torch.int64,
+                                  device=self.tensors[0].device)
+
+    def __len__(self) -> int:
+        return len(self.tensors)
+
+    def ptr(self, first_layer: int = 0) -> int:
+        return self.table.data_ptr() + 8 * first_layer
+
+
+def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
+               block_size: int, kv_heads: int, head_dim: int, num_blocks: int, mode: int = MEAN_F32,
+               first_layer: int = 0, n_layers: Optional[int] = None) -> None:
+    """repre: fp32 [L, rows, kv_heads*head_dim]; rows ``slots`` of layers
+    first_layer.. are overwritten with the means of cache blocks ``block_ids``."""
+    if repre.dim() != 3 or repre.shape[2] != kv_heads * head_dim:
+        raise ValueError("repre must be [layers, rows, kv_heads*head_dim]")
+    n_layers = len(k_layers) - first_layer if n_layers is None else n_layers
+    if first_layer < 0 or first_layer + n_layers > min(len(k_layers), repre.shape[0]):
+        raise ValueError("layer range outside the tables")
+    if block_ids.numel() != slots.numel():
+        raise ValueError("block_ids and slots differ in length")
+    rp = _dev(repre, torch.float32, "repre") + first_layer * repre.stride(0) * 4
+    _lib.call("ucm_block_mean", k_layers.ptr(first_layer), n_layers, num_blocks,
+              _dev(block_ids, torch.int32, "block_ids"), _dev(slots, torch.int32, "slots"), block_ids.numel(),
+              block_size, kv_heads, head_dim, rp, repre.shape[1], repre.stride(0), mode, _stream())
+
+
+def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor,
+                 max_seg_len: int, kv_heads: int, scores: torch.Tensor,
+                 q_rows: Optional[torch.Tensor] = None, first_layer: int = 0,
+                 n_layers: Optional[int] = None) -> None:
+    """q: [L, rows, q_heads, head_dim] fp32 or bf16; repre: fp32 [L, rows, kv_heads*head_dim];
+    scores: fp32 [L, rows].  Layers first_layer .. first_layer+n_layers-1 are scored."""
+    if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
+        raise ValueError("q [L,rows,Hq,D], repre [L,rows,Hkv*D], scores [L,rows] expected")
+    head_dim, q_heads = q.shape[3], q.shape[2]
+    if repre.shape[2] != kv_heads * head_dim:
+        raise ValueError("repre row does not match kv_heads*head_dim")
+    if q.dtype == torch.float32:
+        qd = _lib.DTYPE_F32
+    elif q.dtype == torch.bfloat16:
+        qd = _lib.DTYPE_BF16
+    else:
+        raise ValueError("q must be float32 or bfloat16")
+    n_layers = repre.shape[0] - first_layer if n_layers is None else n_layers
+    if first_layer < 0 or first_layer + n_layers > min(q.shape[0], repre.shape[0], scores.shape[0]):
+        raise ValueError("layer range outside the tables")
+    n_req = seg_off.numel()
+    if seg_len.numel() != n_req or (q_rows is not None and q_rows.numel() != n_req):
+        raise ValueError("seg_off / seg_len / q_rows differ in length")
+    if q_rows is None and q.shape[1] < n_req:
+        raise ValueError("q has fewer rows than requests")
+    if scores.shape[1] < repre.shape[1]:
+        raise ValueError("scores row shorter than the representative table")
+    es = q.element_size()
+    _lib.call("ucm_score_blocks", _dev(q, q.dtype, "q") + first_layer * q.stride(0) * es, qd, q.stride(0),
+              _opt(q_rows, torch.int32, "q_rows"), q_heads,
+              _dev(repre, torch.float32, "repre") + first_layer * repre.stride(0) * 4, repre.stride(0),
+              _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
+              n_layers, kv_heads, head_dim,
+              _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4, scores.stride(0),
+              _stream())
+
+
+def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, topk_len: torch.Tensor,
+                 max_seg_len: int, idx_out: torch.Tensor, count_out: torch.Tensor, start_w: int = 1,
+                 end_w: int = 2, block_tables: Optional[torch.Tensor] = None,
+                 phys_out: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None,
+                 block_size: int = 0, sparse_seq_lens: Optional[torch.Tensor] = None, first_layer: int = 0,
+                 n_layers: Optional[int] = None) -> None:
+    """scores fp32 [L, rows]; idx_out/phys_out int32 [L, n_req, stride]; count_out int32 [L, n_req]."""
+    n_req = seg_off.numel()
+    if idx_out.dim() != 3 or idx_out.shape[1] != n_req or count_out.shape != idx_out.shape[:2]:
+        raise ValueError("idx_out [L,n_req,stride] and count_out [L,n_req] expected")
+    n_layers = scores.shape[0] - first_layer if n_layers is None else n_layers
+    if first_layer < 0 or first_layer + n_layers > min(scores.shape[0], idx_out.shape[0]):
+        raise ValueError("layer range outside the tables")
+    if phys_out is not None and phys_out.shape != idx_out.shape:
+        raise ValueError("phys_out must have idx_out's shape")
+    if block_tables is not None and (block_tables.dim() != 2 or block_tables.shape[0] != n_req):
+        raise ValueError("block_tables must be [n_req, stride]")
+    if sparse_seq_lens is not None and sparse_seq_lens.shape != count_out.shape:
+        raise ValueError("sparse_seq_lens must have count_out's shape")
+    o = first_layer * idx_out.stride(0) * 4
+    c = first_layer * count_out.stride(0) * 4
+    _lib.call("ucm_topk_windows", _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4,
+              scores.stride(0), _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
+              _dev(topk_len, torch.int32, "topk_len"), n_req, max_seg_len, n_layers, start_w, end_w,
+              _dev(idx_out, torch.int32, "idx_out") + o, idx_out.shape[2],
+              _dev(count_out, torch.int32, "count_out") + c,
+              _opt(block_tables, torch.int32, "block_tables"),
+              0 if block_tables is None else block_tables.shape[1],
+              None if phys_out is None else _dev(phys_out, torch.int32, "phys_out") + o,
+              _opt(seq_lens, torch.int32, "seq_lens"), block_size,
+              None if sparse_seq_lens is None else _dev(sparse_seq_lens, torch.int32, "sparse_seq_lens") + c,
+              _stream())
+
+
+def copy_batch(dst_ptrs: torch.Tensor, src_ptrs: torch.Tensor, size: int) -> None:
+    """dst_ptrs/src_ptrs: int64 device tensors of raw addresses; copies size bytes each."""
+    if dst_ptrs.numel() != src_ptrs.numel():
+        raise ValueError("pointer arrays differ in length")
+    _lib.call("ucm_copy_batch", _dev(dst_ptrs, torch.int64, "dst_ptrs"), _dev(src_ptrs, torch.int64, "src_ptrs"),
+              dst_ptrs.numel(), size, _stream())
+
+
+def _staging_ptr(staging: torch.Tensor, need: int) -> int:
+    if not (staging.is_cuda or staging.is_pinned()):
+        raise ValueError("staging must be device or pinned host memory")
+    if not staging.is_contiguous() or staging.numel() * staging.element_size() < need:
+        raise ValueError(f"staging must be contiguous and hold {need} bytes")
+    return staging.data_ptr()
+
+
+def kv_gather_blocks(layers: LayerPointers, kv_stride: int, block_bytes: int, num_blocks: int,
+                     block_ids: torch.Tensor, staging: torch.Tensor) -> None:
+    n = block_ids.numel()
+    _lib.call("ucm_kv_gather_blocks", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
+              _dev(block_ids, torch.int32, "block_ids"), n,
+              _staging_ptr(staging, n * len(layers) * 2 * block_bytes), _stream())
+
+
+def kv_scatter_blocks(layers: LayerPointers, kv_stride: int, block_bytes: int, num_blocks: int,
+                      block_ids: torch.Tensor, staging: torch.Tensor) -> None:
+    n = block_ids.numel()
+    _lib.call("ucm_kv_scatter_blocks", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
+              _dev(block_ids, torch.int32, "block_ids"), n,
+              _staging_ptr(staging, n * len(layers) * 2 * block_bytes), _stream())
+
+
+def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, num_blocks: int,
+                       phys: torch.Tensor, count: torch.Tensor, dst_off: torch.Tensor, region_k: torch.Tensor,
+                       max_count: int, staging: torch.Tensor, staging_blocks: int) -> None:
+    """phys int32 [L, n_req, stride], count int32 [L, n_req]; staging holds staging_blocks blocks."""
+    if phys.dim() != 3 or phys.shape[0] != len(layers) or count.shape != phys.shape[:2]:
+        raise ValueError("phys [L,n_req,stride] / count [L,n_req] expected")
+    n_req = phys.shape[1]
+    if dst_off.numel() != n_req or region_k.numel() != n_req:
+        raise ValueError("dst_off / region_k must have one entry per request")
+    _lib.call("ucm_kv_gather_selected", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
+              _dev(phys, torch.int32, "phys"), _dev(count, torch.int32, "count"), n_req, phys.shape[2],
+              _dev(dst_off, torch.int64, "dst_off"), _dev(region_k, torch.int32, "region_k"), max_count,
+              _staging_ptr(staging, staging_blocks * block_bytes), _stream())
+
+
+def set_score_tile(tile_blocks: int) -> None:
+    _lib.call("ucm_set_score_tile", tile_blocks)
