@@ -1,0 +1,424 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C-ABI library.
+Bar: bit-exact for indices, bytes and fp32 scores/means (the kernels reproduce
+the reference's summation order, so scores are compared bit for bit as well;
+the looser rel 1e-3 bound of the north star is implied)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+import synth
+from golden.make_golden import select_inputs
+
+pytestmark = pytest.mark.gpu
+
+bits = lambda a: np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def bf16_dev(bits_u16, dev):
+    return torch.from_numpy(np.ascontiguousarray(bits_u16).view(np.int16)).to(dev).view(torch.bfloat16)
+
+
+def i32(x, dev):
+    return torch.tensor(np.asarray(x), dtype=torch.int32, device=dev)
+
+
+def randn_bf16(dev, seed, shape):
+    """Large caches are drawn on the device (seeded) and read back for the oracle."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    t = torch.randn(shape, device=dev, generator=g).to(torch.bfloat16)
+    return t, t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# ------------------------------------------------------------ block mean
+
+@pytest.mark.parametrize("hkv,d,bs,n_layers", [(8, 128, 128, 2), (2, 64, 16, 1), (4, 128, 100, 3), (1, 8, 5, 1)])
+def test_block_mean_matches_oracle(ucm, dev, hkv, d, bs, n_layers):
+    from ucm_amd import ops
+
+    nb, rows = 23, 40
+    row = hkv * d
+    caches_h = [synth.normal_bf16_bits(100 + l, (nb, bs, hkv, d)) for l in range(n_layers)]
+    caches = [bf16_dev(c, dev) for c in caches_h]
+    lp = ops.LayerPointers(caches)
+    ids = synth.permutation(7, nb)[:15]
+    slots = synth.permutation(8, rows)[:15]
+    for mode in (ops.MEAN_F32, ops.MEAN_BF16_ROUND):
+        repre = torch.full((n_layers, rows, row), 7.0, device=dev)
+        ops.block_mean(lp, i32(ids, dev), i32(slots, dev), repre, bs, hkv, d, nb, mode=mode)
+        got = repre.cpu().numpy()
+        for l in range(n_layers):
+            want = np.full((rows, row), 7.0, np.float32)
+            O.block_mean_paged(caches_h[l], ids, slots, want, round_bf16=(mode == ops.MEAN_BF16_ROUND))
+            assert np.array_equal(bits(got[l]), bits(want)), (mode, l)
+    # the rounded mode is what torch's own mean in the model dtype stores, up to its summation order
+    t = caches[0][torch.from_numpy(ids.astype(np.int64)).to(dev)].mean(1).float().reshape(len(ids), row)
+    mine = repre[0][torch.from_numpy(slots.astype(np.int64)).to(dev)]
+    assert torch.allclose(mine, t, rtol=2 ** -7, atol=1e-6)
+
+
+def test_block_mean_skips_bad_ids_and_layer_range(ucm, dev):
+    from ucm_amd import ops
+
+    hkv, d, bs, nb, rows = 8, 128, 128, 6, 9
+    caches_h = [synth.normal_bf16_bits(200 + l, (nb, bs, hkv, d)) for l in range(3)]
+    lp = ops.LayerPointers([bf16_dev(c, dev) for c in caches_h])
+    repre = torch.zeros(3, rows, hkv * d, device=dev)
+    ids = np.array([2, -1, 99, 5, 0], np.int32)
+    slots = np.array([0, 1, 2, 100, 8], np.int32)
+    ops.block_mean(lp, i32(ids, dev), i32(slots, dev), repre, bs, hkv, d, nb, first_layer=1, n_layers=1)
+    got = repre.cpu().numpy()
+    want = np.zeros((rows, hkv * d), np.float32)
+    O.block_mean_paged(caches_h[1], [2, 0], [0, 8], want)
+    assert np.array_equal(bits(got[1]), bits(want))
+    assert not got[0].any() and not got[2].any()
+    ops.block_mean(lp, i32([], dev), i32([], dev), repre, bs, hkv, d, nb)  # empty list is a no-op
+
+
+# --------------------------------------------------------------- scoring
+
+def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=torch.float32, q_rows=None,
+               block_tables=None, seq_lens=None, block_size=128):
+    """q_np [L, rows, Hq, D] fp32 values; repre_np [L, rows, Hkv*D]."""
+    n_layers = repre_np.shape[0]
+    lens = np.asarray(lens, np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    q = torch.from_numpy(q_np).to(dev).to(q_dtype)
+    repre = torch.from_numpy(repre_np).to(dev)
+    scores = torch.full((n_layers, repre_np.shape[1]), -123.0, device=dev)
+    mx = int(lens.max(initial=0))
+    ops.score_blocks(q, repre, i32(off, dev), i32(lens, dev), mx, hkv, scores,
+                     q_rows=None if q_rows is None else i32(q_rows, dev))
+    stride = max(mx, 1)
+    idx = torch.full((n_layers, len(lens), stride), -1, dtype=torch.int32, device=dev)
+    cnt = torch.full((n_layers, len(lens)), -1, dtype=torch.int32, device=dev)
+    phys = sps = None
+    bt = None
+    if block_tables is not None:
+        bt = i32(block_tables, dev)
+        phys = torch.full_like(idx, -1)
+    sl = None
+    if seq_lens is not None:
+        sl = i32(seq_lens, dev)
+        sps = torch.full_like(cnt, -1)
+    ops.topk_windows(scores, i32(off, dev), i32(lens, dev), i32(topk, dev), mx, idx, cnt, start_w=sw, end_w=ew,
+                     block_tables=bt, phys_out=phys, seq_lens=sl, block_size=block_size, sparse_seq_lens=sps)
+    torch.cuda.synchronize()
+    out = dict(scores=scores.cpu().numpy(), idx=idx.cpu().numpy(), cnt=cnt.cpu().numpy(), off=off)
+    if phys is not None:
+        out["phys"] = phys.cpu().numpy()
+    if sps is not None:
+        out["sparse_seq_lens"] = sps.cpu().numpy()
+    return out
+
+
+def check_against_oracle(out, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_rows=None):
+    n_layers = repre_np.shape[0]
+    for l in range(n_layers):
+        ql = q_np[l] if q_rows is None else q_np[l][np.asarray(q_rows)]
+        widx, wcnt, wscores = O.select_topk_bs(ql[: len(lens)], repre_np[l], out["off"], lens, topk, hkv,
+                                               start_w=sw, end_w=ew, out_stride=out["idx"].shape[2] + sw + ew + max(topk))
+        for r, n in enumerate(lens):
+            a, b = out["off"][r], out["off"][r] + n
+            if topk[r] > 0:  # the reference (and the oracle) skip scoring when k == 0
+                assert np.array_equal(bits(out["scores"][l, a:b]), bits(wscores[a:b])), (l, r)
+                assert out["cnt"][l, r] == wcnt[r], (l, r)
+                assert np.array_equal(out["idx"][l, r, : wcnt[r]], widx[r, : wcnt[r]]), (l, r)
+
+
+def test_golden_select_cases_on_gpu(ucm, dev, golden):
+    from ucm_amd import ops
+
+    z, meta = golden
+    for name, seed, n, hq, hkv, d, k, sw, ew, b16 in meta["select"]:
+        if d not in (64, 128):
+            continue  # head sizes the kernel is not built for are refused (test_abi)
+        q, repre = select_inputs(seed, n, hq, hkv, d, b16)
+        out = run_select(ops, dev, q[None, None], repre.reshape(1, n, hkv * d), [n], [k], hkv, sw, ew)
+        assert np.array_equal(bits(out["scores"][0, :n]), bits(z[f"select/{name}/scores"])), name
+        want = z[f"select/{name}/idx"]
+        assert out["cnt"][0, 0] == len(want), name
+        assert np.array_equal(out["idx"][0, 0, : len(want)], want), name
+
+
+@pytest.mark.parametrize("hkv,g,d", [(8, 4, 128), (8, 8, 128), (1, 8, 128), (2, 2, 64), (4, 1, 64), (16, 2, 128)])
+@pytest.mark.parametrize("q_dtype", [torch.float32, torch.bfloat16])
+def test_ragged_batch_scores_and_selection(ucm, dev, hkv, g, d, q_dtype):
+    from ucm_amd import ops
+
+    n_layers = 3
+    lens = [1, 2, 3, 4, 0, 17, 64, 65, 130, 33, 257]
+    topk = [O.compute_topk_len(n) if n > 40 else max(n // 2, 1) for n in lens]
+    rows = int(np.sum(lens))
+    q = synth.normal_bf16_as_f32(31, (n_layers, len(lens), hkv * g, d))
+    repre = synth.normal_f32(32, (n_layers, rows, hkv * d)) * np.float32(0.3)
+    out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=q_dtype)
+    check_against_oracle(out, q, repre, lens, topk, hkv)
+    assert out["cnt"][0, 4] == 0  # the empty request selects nothing
+
+
+def test_q_rows_indirection_and_tile_sizes(ucm, dev):
+    from ucm_amd import ops
+
+    hkv, g, d = 8, 4, 128
+    lens = [70, 200, 9]
+    topk = [19, 40, 5]
+    q = synth.normal_bf16_as_f32(41, (2, 12, hkv * g, d))     # 12 token rows, requests read rows 11, 0, 5
+    repre = synth.normal_f32(42, (2, int(np.sum(lens)), hkv * d))
+    rows = [11, 0, 5]
+    try:
+        for tile in (1, 2, 7, 32, 4096):
+            ops.set_score_tile(tile)
+            out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=torch.bfloat16, q_rows=rows)
+            check_against_oracle(out, q, repre, lens, topk, hkv, q_rows=rows)
+    finally:
+        ops.set_score_tile(32)
+
+
+def test_config1_single_request_32k(ucm, dev):
+    """Llama-3-8B shape, 32768 tokens = 256 blocks, top-16 + first 1 + last 2, keys -> means -> scores."""
+    from ucm_amd import ops
+
+    hq, hkv, d, bs, n = 32, 8, 128, 128, 256
+    cache_d, cache_h = randn_bf16(dev, 51, (n, bs, hkv, d))
+    lp = ops.LayerPointers([cache_d])
+    table = synth.permutation(52, n)
+    repre = torch.zeros(1, n, hkv * d, device=dev)
+    ops.block_mean(lp, i32(table, dev), i32(np.arange(n), dev), repre, bs, hkv, d, n)
+    want_repre = np.zeros((n, hkv * d), np.float32)
+    O.block_mean_paged(cache_h, table, np.arange(n), want_repre)
+    assert np.array_equal(bits(repre[0].cpu().numpy()), bits(want_repre))
+    q = synth.normal_bf16_as_f32(53, (1, 1, hq, d))
+    out = run_select(ops, dev, q, want_repre[None], [n], [19], hkv, block_tables=table[None], seq_lens=[n * bs])
+    check_against_oracle(out, q, want_repre[None], [n], [19], hkv)
+    sel = out["idx"][0, 0, :19]
+    assert sel[0] == 0 and list(sel[-2:]) == [n - 2, n - 1]
+    assert np.array_equal(out["phys"][0, 0, :19], table[sel])
+    assert out["sparse_seq_lens"][0, 0] == 19 * bs
+    # independent fp64 bound on the scores (rel 1e-3 of the north star)
+    qm = q[0, 0].reshape(hkv, 4, d).astype(np.float64).mean(1)
+    ref64 = np.einsum("hd,nhd->n", qm, want_repre.reshape(n, hkv, d).astype(np.float64))
+    assert np.allclose(out["scores"][0, :n], ref64, rtol=1e-3, atol=1e-5)
+
+
+def test_config4_shape_long_context_g8(ucm, dev):
+    """Qwen2-72B shape: 64 query heads, g = 8, up to 1024 blocks, k = 2 % + windows."""
+    from ucm_amd import ops
+
+    hkv, g, d = 8, 8, 128
+    lens = [1024, 512, 777]
+    topk = [max(16, int(0.02 * n)) + 3 for n in lens]
+    q = synth.normal_bf16_as_f32(61, (2, len(lens), hkv * g, d))
+    repre = synth.normal_f32(62, (2, int(np.sum(lens)), hkv * d)) * np.float32(0.2)
+    out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=torch.bfloat16)
+    check_against_oracle(out, q, repre, lens, topk, hkv)
+
+
+def test_incremental_repre_update(ucm, dev):
+    """Decode-time update: only the newly filled block is reduced (ucm/sparse/gsa/gsa.py:234-236);
+    every other row of the table must stay untouched."""
+    from ucm_amd import ops
+
+    hkv, d, bs, nb = 8, 128, 128, 12
+    cache_h = synth.normal_bf16_bits(71, (nb, bs, hkv, d))
+    lp = ops.LayerPointers([bf16_dev(cache_h, dev)])
+    repre = torch.from_numpy(synth.normal_f32(72, (1, 20, hkv * d))).to(dev)
+    before = repre.cpu().numpy().copy()
+    ops.block_mean(lp, i32([9], dev), i32([13], dev), repre, bs, hkv, d, nb)
+    after = repre.cpu().numpy()
+    want = before.copy()
+    O.block_mean_paged(cache_h, [9], [13], want[0])
+    assert np.array_equal(bits(after), bits(want))
+    assert not np.array_equal(bits(after[0, 13]), bits(before[0, 13]))
+
+
+# ----------------------------------------------------------------- top-k
+
+def run_topk(ops, dev, score_rows, topk, sw, ew, block_tables=None):
+    lens = [len(s) for s in score_rows]
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    flat = np.concatenate([np.asarray(s, np.float32) for s in score_rows] + [np.zeros(1, np.float32)])
+    scores = torch.from_numpy(flat[None]).to(dev)
+    mx = max(max(lens), 1)
+    idx = torch.full((1, len(lens), mx), -1, dtype=torch.int32, device=dev)
+    cnt = torch.full((1, len(lens)), -1, dtype=torch.int32, device=dev)
+    ops.topk_windows(scores, i32(off, dev), i32(lens, dev), i32(topk, dev), max(lens), idx, cnt, start_w=sw, end_w=ew)
+    torch.cuda.synchronize()
+    return idx.cpu().numpy()[0], cnt.cpu().numpy()[0]
+
+
+def test_topk_golden_ties_on_gpu(ucm, dev, golden):
+    from ucm_amd import ops
+
+    z, meta = golden
+    for i, n, k, sw, ew, seed in meta["ties"]:
+        sc = synth.ints(seed, n, 0, 3).astype(np.float32)
+        idx, cnt = run_topk(ops, dev, [sc], [k], sw, ew)
+        want = z[f"ties/{i}"]
+        assert cnt[0] == len(want) and np.array_equal(idx[0, : cnt[0]], want), (i, n, k, sw, ew)
+
+
+@pytest.mark.parametrize("sw,ew", [(1, 2), (0, 0), (2, 0), (0, 3), (3, 5)])
+def test_topk_many_requests_with_ties(ucm, dev, sw, ew):
+    """Hundreds of small requests in one launch, scores drawn from four values so that
+    almost every boundary is a tie; plus zeros of both signs and infinities."""
+    from ucm_amd import ops
+
+    rng = np.random.default_rng(80 + sw * 10 + ew)
+    rows, ks = [], []
+    for _ in range(300):
+        n = int(rng.integers(1, 90))
+        sc = rng.integers(-1, 3, n).astype(np.float32)
+        sc[rng.random(n) < 0.1] = -0.0
+        if rng.random() < 0.2:
+            sc[rng.integers(0, n)] = np.inf
+        if rng.random() < 0.2:
+            sc[rng.integers(0, n)] = -np.inf
+        rows.append(sc)
+        ks.append(int(rng.integers(0, n + 3)))
+    idx, cnt = run_topk(ops, dev, rows, ks, sw, ew)
+    for r, sc in enumerate(rows):
+        want = O.topk_windows(sc, ks[r], sw, ew)
+        assert cnt[r] == len(want), (r, len(sc), ks[r])
+        assert np.array_equal(idx[r, : cnt[r]], want), (r, len(sc), ks[r], sc)
+
+
+@pytest.mark.parametrize("n", [64, 65, 256, 257, 1024, 1025, 4096])
+def test_topk_register_tiers(ucm, dev, n):
+    """Each register tier of the selection kernel (64 / 256 / 1024 / 4096 blocks per request)."""
+    from ucm_amd import ops
+
+    sc = synth.normal_f32(90 + n, (n,))
+    sc[::7] = sc[3]  # a large tie class that straddles the boundary for some k
+    for k in (4, n // 3, n - 1):
+        idx, cnt = run_topk(ops, dev, [sc, sc[: n // 2]], [k, k], 1, 2)
+        for r, s in enumerate([sc, sc[: n // 2]]):
+            want = O.topk_windows(s, k, 1, 2)
+            assert cnt[r] == len(want) and np.array_equal(idx[r, : cnt[r]], want), (n, k, r)
+
+
+# -------------------------------------------------------------- KV moves
+
+def make_caches(dev, n_layers, nb, bb, seed):
+    hs = [np.frombuffer(synth.u64(seed + l, 2 * nb * bb // 8).tobytes(), np.uint8).copy() for l in range(n_layers)]
+    ds = [torch.from_numpy(h).to(dev) for h in hs]
+    return hs, ds
+
+
+@pytest.mark.parametrize("bb", [262144, 4096, 48, 16 + 32768])
+def test_kv_dump_load_round_trip(ucm, dev, bb):
+    """Config-3 shape in small: random block table, scatter staging->cache, gather cache->staging, byte exact."""
+    from ucm_amd import ops
+
+    n_layers, nb, n = 3, 37, 11
+    hs, ds = make_caches(dev, n_layers, nb, bb, 300)
+    lp = ops.LayerPointers(ds)
+    ids = synth.permutation(301, nb)[:n]
+    staging = torch.zeros(n * n_layers * 2 * bb, dtype=torch.uint8, device=dev)
+    ops.kv_gather_blocks(lp, nb * bb, bb, nb, i32(ids, dev), staging)
+    want = np.zeros(n * n_layers * 2 * bb, np.uint8)
+    O.kv_move_blocks(hs, nb * bb, bb, ids, want, True)
+    assert np.array_equal(staging.cpu().numpy(), want)
+    # load into a fresh cache: only the listed blocks change, and they equal the source
+    fresh = [torch.zeros_like(t) for t in ds]
+    lp2 = ops.LayerPointers(fresh)
+    ops.kv_scatter_blocks(lp2, nb * bb, bb, nb, i32(ids, dev), staging)
+    hfresh = [np.zeros_like(h) for h in hs]
+    O.kv_move_blocks(hfresh, nb * bb, bb, ids, want, False)
+    for l in range(n_layers):
+        assert np.array_equal(fresh[l].cpu().numpy(), hfresh[l])
+    # ids outside the plane are skipped
+    ops.kv_gather_blocks(lp, nb * bb, bb, nb, i32([nb, -3], dev), staging)
+    assert np.array_equal(staging.cpu().numpy(), want)
+
+
+def test_copy_batch_pointer_arrays(ucm, dev):
+    from ucm_amd import ops
+
+    size, num = 65536 + 16, 9
+    src = torch.from_numpy(np.frombuffer(synth.u64(310, num * size // 8).tobytes(), np.uint8).copy()).to(dev)
+    dst = torch.zeros_like(src)
+    order = synth.permutation(311, num).astype(np.int64)
+    sp = torch.tensor([src.data_ptr() + int(i) * size for i in range(num)], dtype=torch.int64, device=dev)
+    dp = torch.tensor([dst.data_ptr() + int(order[i]) * size for i in range(num)], dtype=torch.int64, device=dev)
+    ops.copy_batch(dp, sp, size)
+    got = dst.cpu().numpy().reshape(num, size)
+    want = src.cpu().numpy().reshape(num, size)
+    for i in range(num):
+        assert np.array_equal(got[order[i]], want[i])
+    ops.copy_batch(dp[:0], sp[:0], size)
+
+
+def test_copy_batch_to_pinned_host(ucm, dev):
+    """The staging side may be mapped pinned host memory (the reference's D2H kernel writes there)."""
+    from ucm_amd import ops
+
+    size, num = 8192, 5
+    src = torch.from_numpy(np.frombuffer(synth.u64(320, num * size // 8).tobytes(), np.uint8).copy()).to(dev)
+    host = torch.zeros(num * size, dtype=torch.uint8, pin_memory=True)
+    sp = torch.tensor([src.data_ptr() + i * size for i in range(num)], dtype=torch.int64, device=dev)
+    dp = torch.tensor([host.data_ptr() + i * size for i in range(num)], dtype=torch.int64, device=dev)
+    ops.copy_batch(dp, sp, size)
+    torch.cuda.synchronize()
+    assert np.array_equal(host.numpy(), src.cpu().numpy())
+
+
+def test_gather_selected_matches_oracle(ucm, dev):
+    from ucm_amd import ops
+
+    n_layers, nb, bb, n_req, stride = 4, 50, 8192, 3, 12
+    hs, ds = make_caches(dev, n_layers, nb, bb, 330)
+    lp = ops.LayerPointers(ds)
+    count = synth.ints(331, n_layers * n_req, 0, 9).astype(np.int32).reshape(n_layers, n_req)
+    phys = synth.ints(332, n_layers * n_req * stride, 0, nb - 1).astype(np.int32).reshape(n_layers, n_req, stride)
+    region = count.max(0).astype(np.int32) + 1
+    dst_off = np.concatenate([[0], np.cumsum(region * n_layers * 2)[:-1]]).astype(np.int64)
+    total = int((region * n_layers * 2).sum())
+    staging = torch.full((total * bb,), 0xAB, dtype=torch.uint8, device=dev)
+    ops.kv_gather_selected(lp, nb * bb, bb, nb, i32(phys, dev), i32(count, dev),
+                           torch.from_numpy(dst_off).to(dev), i32(region, dev), int(count.max()), staging, total)
+    want = np.full(total * bb, 0xAB, np.uint8)
+    O.kv_gather_selected(hs, nb * bb, bb, phys, count, dst_off, region, want)
+    assert np.array_equal(staging.cpu().numpy(), want)
+
+
+def test_retrieval_then_gather_end_to_end(ucm, dev):
+    """Config-2 shape in small: means -> scores -> selection -> gather, no host round trip in between."""
+    from ucm_amd import ops
+
+    n_layers, hq, hkv, d, bs = 4, 32, 8, 128, 128
+    lens = synth.ragged_lengths(340, 6, 4096, 16384)
+    lens = np.minimum(lens, 60).astype(np.int32)
+    topk = np.array([max(16, int(0.03 * n)) + 3 for n in lens], np.int32)
+    nb = int(lens.sum()) + 4
+    bb = bs * hkv * d * 2
+    pairs = [randn_bf16(dev, 341 + l, (2, nb, bs, hkv, d)) for l in range(n_layers)]
+    ds, caches_h = [p[0] for p in pairs], [p[1] for p in pairs]
+    lp = ops.LayerPointers(ds)
+    table = synth.permutation(350, nb)[: int(lens.sum())]
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    rows = int(lens.sum())
+    repre = torch.zeros(n_layers, rows, hkv * d, device=dev)
+    ops.block_mean(lp, i32(table, dev), i32(np.arange(rows), dev), repre, bs, hkv, d, nb)
+    q = synth.normal_bf16_as_f32(351, (n_layers, len(lens), hq, d))
+    bt = np.zeros((len(lens), int(lens.max())), np.int32)
+    for r, n in enumerate(lens):
+        bt[r, :n] = table[off[r] : off[r] + n]
+    repre_h = repre.cpu().numpy()
+    out = run_select(ops, dev, q, repre_h, lens, topk, hkv, q_dtype=torch.bfloat16, block_tables=bt)
+    check_against_oracle(out, q, repre_h, lens, topk, hkv)
+    for l in range(n_layers):
+        want_rep = np.zeros((rows, hkv * d), np.float32)
+        O.block_mean_paged(caches_h[l][0], table, np.arange(rows), want_rep)
+        assert np.array_equal(bits(repre_h[l]), bits(want_rep))
+    region = topk.copy()
+    dst_off = np.concatenate([[0], np.cumsum(region.astype(np.int64) * n_layers * 2)[:-1]]).astype(np.int64)
+    total = int((region.astype(np.int64) * n_layers * 2).sum())
+    staging = torch.zeros(total * bb, dtype=torch.uint8, device=dev)
+    ops.kv_gather_selected(lp, nb * bb, bb, nb, i32(out["phys"], dev), i32(out["cnt"], dev),
+                           torch.from_numpy(dst_off).to(dev), i32(region, dev), int(topk.max()), staging, total)
+    want = np.zeros(total * bb, np.uint8)
+    O.kv_gather_selected([c.view(np.uint8).reshape(-1) for c in caches_h], nb * bb, bb, out["phys"], out["cnt"],
+                         dst_off, region, want)
+    assert np.array_equal(staging.cpu().numpy(), want)

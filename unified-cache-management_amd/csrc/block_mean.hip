@@ -101,9 +101,10 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
                               int kv_heads, int head_dim, float* repre, int repre_rows,
                               int64_t repre_layer_stride, int mode, ucm_stream_t stream)
 {
+    UCM_REQUIRE(n >= 0, "ucm_block_mean: n=%d", n);
+    if (n == 0) { return UCM_OK; }  // an empty list has no pointers to check
     UCM_REQUIRE(k_layers && block_ids && slots && repre, "ucm_block_mean: null pointer");
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535, "ucm_block_mean: n_layers=%d", n_layers);
-    UCM_REQUIRE(n >= 0, "ucm_block_mean: n=%d", n);
     UCM_REQUIRE(block_size > 0 && kv_heads > 0 && head_dim > 0 && num_blocks > 0 && repre_rows > 0,
                 "ucm_block_mean: non-positive shape");
     UCM_REQUIRE(mode == UCM_MEAN_F32 || mode == UCM_MEAN_BF16_ROUND, "ucm_block_mean: mode=%d", mode);
@@ -113,7 +114,6 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
                 "ucm_block_mean: repre_layer_stride=%lld smaller than one layer's table",
                 static_cast<long long>(repre_layer_stride));
     UCM_REQUIRE(ucm::aligned16(repre) && (repre_layer_stride % 4 == 0), "ucm_block_mean: repre not 16-byte aligned");
-    if (n == 0) { return UCM_OK; }
     const unsigned gx = (row / kCols + kThreads - 1) / kThreads;
     UCM_REQUIRE(static_cast<uint64_t>(n) * gx <= 0x7fffffffull, "ucm_block_mean: too many blocks for one launch");
     hipLaunchKernelGGL(block_mean_kernel, dim3(static_cast<unsigned>(n) * gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream),

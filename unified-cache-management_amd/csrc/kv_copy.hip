@@ -99,7 +99,7 @@ int check_block_args(const void* layers, int n_layers, size_t kv_stride, size_t 
 {
     UCM_REQUIRE(num_blocks > 0 && static_cast<size_t>(num_blocks) * block_bytes <= kv_stride,
                 "kv move: num_blocks=%d does not fit kv_stride=%zu", num_blocks, kv_stride);
-    UCM_REQUIRE(layers && ids && staging, "kv move: null pointer");
+    UCM_REQUIRE(n == 0 || (layers && ids && staging), "kv move: null pointer");
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535, "kv move: n_layers=%d out of range", n_layers);
     UCM_REQUIRE(n >= 0, "kv move: n=%d", n);
     UCM_REQUIRE(block_bytes > 0 && block_bytes % 16 == 0 && kv_stride % 16 == 0,
@@ -115,9 +115,9 @@ int check_block_args(const void* layers, int n_layers, size_t kv_stride, size_t 
 extern "C" int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t size,
                               ucm_stream_t stream)
 {
-    UCM_REQUIRE(dst && src, "ucm_copy_batch: null pointer array");
     UCM_REQUIRE(size % 16 == 0, "ucm_copy_batch: size=%zu must be a multiple of 16", size);
     if (num == 0 || size == 0) { return UCM_OK; }
+    UCM_REQUIRE(dst && src, "ucm_copy_batch: null pointer array");
     const unsigned chunks = chunks_of(size);
     UCM_REQUIRE(num * chunks <= 0x7fffffffull, "ucm_copy_batch: too many chunks for one launch");
     hipLaunchKernelGGL(copy_batch_kernel, dim3(static_cast<unsigned>(num * chunks)), dim3(kThreads), 0,
@@ -159,7 +159,7 @@ extern "C" int ucm_kv_gather_selected(const void* const* layers, int n_layers, s
                                       const int32_t* region_k, int max_count, void* staging,
                                       ucm_stream_t stream)
 {
-    UCM_REQUIRE(layers && phys && count && dst_off && region_k && staging,
+    UCM_REQUIRE(n_req == 0 || max_count == 0 || (layers && phys && count && dst_off && region_k && staging),
                 "ucm_kv_gather_selected: null pointer");
     UCM_REQUIRE(n_layers > 0 && n_layers * 2 <= 65535, "ucm_kv_gather_selected: n_layers=%d", n_layers);
     UCM_REQUIRE(num_blocks > 0 && static_cast<size_t>(num_blocks) * block_bytes <= kv_stride,

@@ -152,7 +152,8 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
                                 int n_layers, int kv_heads, int head_dim, float* scores,
                                 int64_t scores_layer_stride, ucm_stream_t stream)
 {
-    UCM_REQUIRE(q && repre && seg_off && seg_len && scores, "ucm_score_blocks: null pointer");
+    UCM_REQUIRE(n_req == 0 || max_seg_len == 0 || (q && repre && seg_off && seg_len && scores),
+                "ucm_score_blocks: null pointer");
     UCM_REQUIRE(q_dtype == UCM_DTYPE_F32 || q_dtype == UCM_DTYPE_BF16, "ucm_score_blocks: q_dtype=%d", q_dtype);
     UCM_REQUIRE(n_req >= 0 && n_req <= 65535 && n_layers > 0 && n_layers <= 65535,
                 "ucm_score_blocks: n_req=%d n_layers=%d", n_req, n_layers);

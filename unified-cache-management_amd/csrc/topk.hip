@@ -132,7 +132,8 @@ extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride
                                 int32_t* phys_out, const int32_t* seq_lens, int block_size,
                                 int32_t* sparse_seq_lens, ucm_stream_t stream)
 {
-    UCM_REQUIRE(scores && seg_off && seg_len && topk_len && idx_out && count_out, "ucm_topk_windows: null pointer");
+    UCM_REQUIRE(n_req == 0 || (scores && seg_off && seg_len && topk_len && idx_out && count_out),
+                "ucm_topk_windows: null pointer");
     UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_topk_windows: n_req=%d n_layers=%d", n_req, n_layers);
     UCM_REQUIRE(start_w >= 0 && end_w >= 0 && max_seg_len >= 0, "ucm_topk_windows: negative window or length");
     UCM_REQUIRE(out_stride >= max_seg_len, "ucm_topk_windows: out_stride=%d < max_seg_len=%d", out_stride, max_seg_len);
