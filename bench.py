@@ -1,0 +1,312 @@
+"""Decode-step benchmark of the sparse-retrieval hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[1]): a ragged continuous batch of 16 requests,
+context lengths uniform in [4096, 65536] tokens rounded to the 128-token block,
+Llama-3-8B attention shape (32 query heads / 8 kv heads / head_dim 128, bf16),
+all 32 layers.  One step = for every layer and request: score all block
+representatives against the request's query, select top-k = max(16, 3 % of the
+blocks) plus the first block and the last two, and gather the selected K and V
+blocks from the bf16 paged cache into a contiguous per-request buffer.
+Three launches per step (score, select, gather), no host round trip between.
+
+Prints ONE JSON line.  `value` is microseconds per decode step with all inputs
+resident in HBM; `roofline` describes the dominant kernel (the gather),
+`roofline_score` the scoring kernel, `cpu_baseline` the same step on the host
+(the reference's CPU retrieval algorithm + a memcpy gather).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+N_REQ, N_LAYERS, HQ, HKV, D, BS = 16, 32, 32, 8, 128, 128
+ROW = HKV * D
+BLOCK_BYTES = BS * ROW * 2
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--seed", type=int, default=2024)
+    ap.add_argument("--layers", type=int, default=N_LAYERS, help="fewer layers only for quick experiments")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the oracle check of the last step")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled against a kernel of known traffic")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the retrieval path is per-GPU and this build has no multi-GPU leg "
+              f"(--gpus {args.gpus} refused)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import __graft_entry__ as ge
+
+    ge.load_package()
+    from ucm_amd import ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    n_layers = args.layers
+    rng = np.random.default_rng(args.seed)
+    lens = rng.integers(4096 // BS, 65536 // BS + 1, N_REQ).astype(np.int32)       # blocks per request
+    topk = np.array([max(16, int(0.03 * n)) + 3 for n in lens], np.int32)          # total incl. windows
+    rows = int(lens.sum())
+    nb = rows                                                                        # pool = exactly the live blocks
+    seg_off_h = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    table_h = rng.permutation(nb).astype(np.int32)                                  # random block table over the pool
+    max_len, max_k = int(lens.max()), int(topk.max())
+
+    # ---- device state: paged KV cache, block tables, representatives
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    caches = []
+    for _ in range(n_layers):
+        c = torch.empty((2, nb, BS, HKV, D), dtype=torch.bfloat16, device=dev)
+        c.normal_(generator=g)
+        caches.append(c)
+    layers = ops.LayerPointers(caches)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=dev)
+    seg_off, seg_len, topk_d, table = i32(seg_off_h), i32(lens), i32(topk), i32(table_h)
+    bt_h = np.zeros((N_REQ, max_len), np.int32)
+    for r in range(N_REQ):
+        bt_h[r, : lens[r]] = table_h[seg_off_h[r] : seg_off_h[r] + lens[r]]
+    bt = i32(bt_h)
+    repre = torch.zeros(n_layers, rows, ROW, device=dev)
+    slots = torch.arange(rows, dtype=torch.int32, device=dev)
+
+    def prefill():
+        ops.block_mean(layers, table, slots, repre, BS, HKV, D, nb)
+
+    prefill()
+    torch.cuda.synchronize()
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    a, b = ev(), ev()
+    a.record()
+    prefill()
+    b.record()
+    torch.cuda.synchronize()
+    mean_ms = a.elapsed_time(b)
+    mean_bytes = n_layers * rows * (BLOCK_BYTES + ROW * 4)
+
+    n_q = args.steps + args.warmup
+    qs = torch.empty((n_q, n_layers, N_REQ, HQ, D), dtype=torch.bfloat16, device=dev)
+    qs.normal_(generator=g)
+    scores = torch.zeros(n_layers, rows, device=dev)
+    idx = torch.full((n_layers, N_REQ, max_len), -1, dtype=torch.int32, device=dev)
+    phys = torch.full_like(idx, -1)
+    cnt = torch.zeros(n_layers, N_REQ, dtype=torch.int32, device=dev)
+    region_h = topk.copy()
+    dst_off_h = np.concatenate([[0], np.cumsum(region_h.astype(np.int64) * n_layers * 2)[:-1]]).astype(np.int64)
+    total_blocks = int((region_h.astype(np.int64) * n_layers * 2).sum())
+    region, dst_off = i32(region_h), torch.from_numpy(dst_off_h).to(dev)
+    staging = torch.empty(total_blocks * BLOCK_BYTES, dtype=torch.uint8, device=dev)
+    kv_stride = nb * BLOCK_BYTES
+
+    def step(q, events=None):
+        if events:
+            events[0].record()
+        ops.score_blocks(q, repre, seg_off, seg_len, max_len, HKV, scores, total_blocks=rows)
+        if events:
+            events[1].record()
+        ops.topk_windows(scores, seg_off, seg_len, topk_d, max_len, idx, cnt, block_tables=bt, phys_out=phys)
+        if events:
+            events[2].record()
+        ops.kv_gather_selected(layers, kv_stride, BLOCK_BYTES, nb, phys, cnt, dst_off, region, max_k, staging,
+                               total_blocks)
+        if events:
+            events[3].record()
+
+    if args.calibrate_copy:
+        gib = 1 << 30
+        src = torch.empty(gib, dtype=torch.uint8, device=dev).random_(generator=g)
+        dst = torch.empty_like(src)
+        ops.copy_batch(torch.tensor([dst.data_ptr()], dtype=torch.int64, device=dev),
+                       torch.tensor([src.data_ptr()], dtype=torch.int64, device=dev), gib)
+        torch.cuda.synchronize()
+        assert torch.equal(src, dst)
+        del src, dst
+
+    for w in range(args.warmup):
+        step(qs[w])
+    torch.cuda.synchronize()
+    all_events = [[ev() for _ in range(4)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        step(qs[args.warmup + s], all_events[s])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    k_ms = np.array([[e[i].elapsed_time(e[i + 1]) for i in range(3)] for e in all_events]).mean(0)
+    score_ms, topk_ms, gather_ms = (float(x) for x in k_ms)
+
+    n_sel = int(topk.astype(np.int64).sum()) * n_layers
+    gather_bytes = 2 * n_sel * 2 * BLOCK_BYTES                                     # K and V, read + write
+    score_bytes = n_layers * (rows * ROW * 4 + N_REQ * HQ * D * 2 + rows * 4)     # fp32 representatives + bf16 q + scores
+    gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+
+    # ---- check the last step against the CPU oracle (selection, scores, gathered bytes)
+    checked = None
+    if not args.no_check:
+        import oracle  # checker only
+
+        q_last = qs[n_q - 1].float().cpu().numpy()
+        idx_h, cnt_h, phys_h = idx.cpu().numpy(), cnt.cpu().numpy(), phys.cpu().numpy()
+        scores_h = scores.cpu().numpy()
+        for l in range(n_layers):
+            rep = repre[l].cpu().numpy()
+            widx, wcnt, wsc = oracle.select_topk_bs(q_last[l], rep, seg_off_h, lens, topk, HKV, out_stride=max_len + 4)
+            assert np.array_equal(wsc.view(np.uint32), scores_h[l].view(np.uint32)), f"scores differ in layer {l}"
+            assert np.array_equal(wcnt, cnt_h[l]), f"counts differ in layer {l}"
+            for r in range(N_REQ):
+                assert np.array_equal(widx[r, : wcnt[r]], idx_h[l, r, : wcnt[r]]), f"selection differs ({l},{r})"
+                assert np.array_equal(phys_h[l, r, : wcnt[r]], bt_h[r][widx[r, : wcnt[r]]])
+        # gathered bytes: every staged block equals its source block (device-side compare, all of them)
+        st = staging.view(torch.bfloat16).view(-1, BS, HKV, D)
+        for l in range(n_layers):
+            for r in range(N_REQ):
+                k = int(topk[r])
+                sel = phys[l, r, :k].long()
+                for kv in range(2):
+                    o = int(dst_off_h[r]) + (l * 2 + kv) * k
+                    assert torch.equal(st[o : o + k], caches[l][kv][sel]), f"gathered bytes differ ({l},{r},{kv})"
+        checked = "last step: fp32 scores, selected indices, block-table lookup and all gathered bytes equal the CPU oracle / source blocks"
+
+    # ---- CPU baseline: the reference's CPU retrieval (same arithmetic, its threading) + memcpy gather
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+
+        threads = min(16, os.cpu_count() or 1)
+        os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+        rep_h = repre.cpu().numpy()
+        q_h = qs[0].float().cpu().numpy()
+        use_ref = oracle.ref.available and _cpu_has_avx512()
+        out_stride = max_len + 4
+
+        def cpu_retrieval():
+            for l in range(n_layers):
+                if use_ref:
+                    oracle.ref.select_topk_bs(q_h[l], rep_h[l], seg_off_h, lens, topk, HKV, out_stride=out_stride)
+                else:
+                    oracle.select_topk_bs(q_h[l], rep_h[l], seg_off_h, lens, topk, HKV, out_stride=out_stride)
+
+        cpu_retrieval()
+        reps, t_acc = 0, 0.0
+        while t_acc < args.cpu_seconds * 0.6 and reps < 200:
+            s0 = time.perf_counter()
+            cpu_retrieval()
+            t_acc += time.perf_counter() - s0
+            reps += 1
+        cpu_retr_us = t_acc / reps * 1e6
+        # gather sample: a few layers of the cache on the host, memcpy of the selected blocks, scaled to all layers
+        g_layers = min(2, n_layers)
+        host_layers = [caches[l].view(torch.uint8).reshape(-1).cpu().numpy() for l in range(g_layers)]
+        g_total = int((region_h.astype(np.int64) * g_layers * 2).sum())
+        g_off = np.concatenate([[0], np.cumsum(region_h.astype(np.int64) * g_layers * 2)[:-1]]).astype(np.int64)
+        g_stage = np.empty(g_total * BLOCK_BYTES, np.uint8)
+        ph, ch = phys.cpu().numpy()[:g_layers].copy(), cnt.cpu().numpy()[:g_layers].copy()
+        oracle.kv_gather_selected(host_layers, kv_stride, BLOCK_BYTES, ph, ch, g_off, region_h, g_stage)
+        greps, g_acc = 0, 0.0
+        while g_acc < args.cpu_seconds * 0.4 and greps < 50:
+            s0 = time.perf_counter()
+            oracle.kv_gather_selected(host_layers, kv_stride, BLOCK_BYTES, ph, ch, g_off, region_h, g_stage)
+            g_acc += time.perf_counter() - s0
+            greps += 1
+        cpu_gather_us = g_acc / greps * 1e6 * (n_layers / g_layers)
+        cpu = {
+            "value": round(cpu_retr_us + cpu_gather_us, 1),
+            "unit": "us/step",
+            "cores": threads,
+            "kind": "reference" if use_ref else "port",
+            "retrieval_us": round(cpu_retr_us, 1),
+            "gather_us": round(cpu_gather_us, 1),
+            "sample": (f"retrieval: {reps} full steps (all {n_layers} layers x {N_REQ} requests, fp32 representatives "
+                       f"resident in host DRAM, {threads} OpenMP threads over blocks, requests and layers serial); "
+                       f"gather: {greps} passes over {g_layers} of {n_layers} layers with one memcpy thread, scaled x{n_layers // g_layers}"),
+            "host_cpus": os.cpu_count(),
+        }
+
+    out = {
+        "metric": "us per decode step (32-layer retrieval+gather)",
+        "value": round(ms_per_step * 1e3, 1),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 keys/queries, fp32 scores, u8 block bytes",
+        "data": "synthetic (seeded N(0,1) bf16 keys, values and queries; random block table)",
+        "config": {
+            "workload": "configs[1]: ragged batch of 16 requests, 4096-65536 tokens, Llama-3-8B attention shape, "
+                        f"{n_layers} layers, k = max(16, 3%) + 1 first + 2 last, full gather of selected K and V blocks",
+            "blocks_per_request": [int(x) for x in lens],
+            "total_blocks": rows,
+            "selected_blocks_per_step": n_sel,
+            "kv_cache_GB": round(n_layers * 2 * nb * BLOCK_BYTES / 1e9, 1),
+        },
+        "kernels_us": {"score": round(score_ms * 1e3, 1), "select": round(topk_ms * 1e3, 1),
+                       "gather": round(gather_ms * 1e3, 1)},
+        "retrieval_us": round((score_ms + topk_ms) * 1e3, 1),
+        "roofline": {
+            "kernel": "kv_gather_selected_kernel",
+            "bound": "hbm",
+            "achieved": round(gbs(gather_bytes, gather_ms), 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs(gather_bytes, gather_ms) / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes": gather_bytes,
+        },
+        "roofline_score": {
+            "kernel": "score_kernel",
+            "bound": "hbm",
+            "achieved": round(gbs(score_bytes, score_ms), 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs(score_bytes, score_ms) / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes": score_bytes,
+        },
+        "block_mean_prefill": {"ms": round(mean_ms, 3), "GBps": round(gbs(mean_bytes, mean_ms), 1),
+                               "frac": round(gbs(mean_bytes, mean_ms) / HBM_PEAK_GBS, 4)},
+        "cpu_baseline": cpu,
+        "checked": checked,
+    }
+    print(json.dumps(out))
+
+
+def _cpu_has_avx512() -> bool:
+    try:
+        with open("/proc/cpuinfo") as f:
+            return "avx512f" in f.read()
+    except OSError:
+        return False
+
+
+if __name__ == "__main__":
+    main()

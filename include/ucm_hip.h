@@ -95,14 +95,15 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *              last token (GSA.copy_q, gsa.py:616-632) when bf16.
  *   seg_off, seg_len  dev int32[n_req]: first representative row and number of
  *              blocks of each request; max_seg_len >= every seg_len (host
- *              value, sizes the grid).
+ *              value, sizes the grid); total_blocks = sum of seg_len when the
+ *              host knows it (a tighter grid), else 0.
  *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x].
  * head_dim must be 64 or 128 and kv_heads one of 1, 2, 4, 8, 16.
  */
 int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
                      int q_heads, const float* repre, int64_t repre_layer_stride,
                      const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
-                     int n_layers, int kv_heads, int head_dim, float* scores,
+                     int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
                      int64_t scores_layer_stride, ucm_stream_t stream);
 
 /* Tuning knob for benchmarks: blocks scored per workgroup by ucm_score_blocks

@@ -176,6 +176,35 @@ def test_q_rows_indirection_and_tile_sizes(ucm, dev):
         ops.set_score_tile(32)
 
 
+def test_many_requests_dense_tile_lookup(ucm, dev):
+    """More requests than one wavefront scans at once (the tile -> request lookup runs in trips of 64),
+    with empty requests in between, and the grid sized from the host-known total."""
+    from ucm_amd import ops
+
+    hkv, g, d = 4, 2, 64
+    lens = synth.ints(45, 150, 0, 40).astype(np.int32)
+    lens[[0, 63, 64, 65, 149]] = [0, 33, 0, 1, 40]
+    topk = np.maximum(lens // 3, 1).astype(np.int32)
+    rows = int(lens.sum())
+    q = synth.normal_bf16_as_f32(46, (2, len(lens), hkv * g, d))
+    repre = synth.normal_f32(47, (2, rows, hkv * d))
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    try:
+        for tile in (3, 32):
+            ops.set_score_tile(tile)
+            for total in (0, rows):
+                scores = torch.full((2, rows), -5.0, device=dev)
+                ops.score_blocks(torch.from_numpy(q).to(dev), torch.from_numpy(repre).to(dev), i32(off, dev),
+                                 i32(lens, dev), int(lens.max()), hkv, scores, total_blocks=total)
+                got = scores.cpu().numpy()
+                for l in range(2):
+                    _, _, want = O.select_topk_bs(q[l], repre[l], off, lens, topk, hkv)
+                    live = np.concatenate([np.arange(off[r], off[r] + lens[r]) for r in range(len(lens))])
+                    assert np.array_equal(bits(got[l][live]), bits(want[live])), (tile, total, l)
+    finally:
+        ops.set_score_tile(32)
+
+
 def test_config1_single_request_32k(ucm, dev):
     """Llama-3-8B shape, 32768 tokens = 256 blocks, top-16 + first 1 + last 2, keys -> means -> scores."""
     from ucm_amd import ops

@@ -77,9 +77,10 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
 def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor,
                  max_seg_len: int, kv_heads: int, scores: torch.Tensor,
                  q_rows: Optional[torch.Tensor] = None, first_layer: int = 0,
-                 n_layers: Optional[int] = None) -> None:
+                 n_layers: Optional[int] = None, total_blocks: int = 0) -> None:
     """q: [L, rows, q_heads, head_dim] fp32 or bf16; repre: fp32 [L, rows, kv_heads*head_dim];
-    scores: fp32 [L, rows].  Layers first_layer .. first_layer+n_layers-1 are scored."""
+    scores: fp32 [L, rows].  Layers first_layer .. first_layer+n_layers-1 are scored.
+    total_blocks: sum of seg_len when the host knows it (tighter grid), else 0."""
     if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
         raise ValueError("q [L,rows,Hq,D], repre [L,rows,Hkv*D], scores [L,rows] expected")
     head_dim, q_heads = q.shape[3], q.shape[2]
@@ -106,7 +107,7 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
               _opt(q_rows, torch.int32, "q_rows"), q_heads,
               _dev(repre, torch.float32, "repre") + first_layer * repre.stride(0) * 4, repre.stride(0),
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
-              n_layers, kv_heads, head_dim,
+              total_blocks, n_layers, kv_heads, head_dim,
               _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4, scores.stride(0),
               _stream())
 
