@@ -129,7 +129,9 @@ int ucm_set_score_tile(int tile_blocks);
  *   phys_out      dev int32, same layout as idx_out: block_tables[r][idx]
  *   seq_lens      dev int32[n_req] (may be NULL): tokens of each request;
  *   sparse_seq_lens dev int32[n_layers][n_req]: count*block_size, minus
- *              block_size - seq_len%block_size when the last block is partial.
+ *              block_size - seq_len%block_size when the last block is partial;
+ *              seq_len itself when every block was kept (the reference's
+ *              non-sparsified branch, prefetch_engine.py:547-553).
  * Up to 4096 blocks per request.
  */
 int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off,
@@ -138,6 +140,29 @@ int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, const int
                      int32_t* count_out, const int32_t* block_tables, int bt_stride,
                      int32_t* phys_out, const int32_t* seq_lens, int block_size,
                      int32_t* sparse_seq_lens, ucm_stream_t stream);
+
+/*
+ * The ESA retrieval backend's computation for a batch of requests -
+ * RetrievalWorkerBackend::worker_loop
+ * (ucm/sparse/esa/retrieval/cpy/retrieval_backend.cpp:135-203): for request b,
+ * every entry of indexes[b][0..m) that is not -1 names a row of `data`
+ * (fp32 [n_items][dim], the table the backend is constructed over, :19-26); its
+ * score is the strictly sequential sum over d of q[b][d]*data[row][d] with
+ * separately rounded multiply and add (:175-181); the min(valid entries, topk)
+ * best are returned in descending score order with their scores (:182-189).
+ * Equal scores come out in index-row order (the reference's std::partial_sort
+ * leaves that order unspecified).  Entries that are -1 or outside
+ * [0, n_items) are skipped.
+ *   q          dev fp32 [batch][dim]
+ *   indexes    dev int32 [batch][m], padded with -1 (submit(), :43-74)
+ *   scores_ws  dev fp32 [batch][m]: workspace for all candidate scores
+ *   out_idx / out_scores  dev [batch][out_stride]; out_count dev int32[batch]
+ * dim must be a multiple of 4, m at most 8192.
+ */
+int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
+                     const int32_t* indexes, int batch, int m, int topk, float* scores_ws,
+                     int32_t* out_idx, float* out_scores, int32_t* out_count, int out_stride,
+                     ucm_stream_t stream);
 
 /*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched

@@ -1,0 +1,323 @@
+"""The host-side mirror of the reference's plugin / worker interfaces, driven the
+way patched vLLM drives it (stand-in objects instead of vLLM's), with every
+result checked against the CPU oracle."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+import synth
+
+pytestmark = pytest.mark.gpu
+
+bits = lambda a: np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+# ------------------------------------------------------- retrieval worker
+
+def test_retrieval_worker_golden_vectors(ucm, dev, golden):
+    """submit / wait / get_result against what the reference's own backend returned."""
+    from ucm_amd.sparse.esa.retrieval_worker import HipRetrievalBackend, RetrievalWorker
+
+    z, meta = golden
+    for i, rows, dim, b, m, topk, s_data, s_q, s_idx in meta["esa"]:
+        data = torch.from_numpy(synth.normal_bf16_as_f32(s_data, (rows, dim))).to(dev)
+        q = torch.from_numpy(synth.normal_bf16_as_f32(s_q, (b, dim))).to(dev).to(torch.bfloat16)
+        idx = np.stack([synth.permutation(s_idx + r, rows)[:m] for r in range(b)]).astype(np.int32)
+        idx[:, m - 3:] = -1
+        worker = RetrievalWorker(HipRetrievalBackend(data))
+        rid = worker.submit(q, topk=topk, indexes=idx)
+        worker.wait(rid)
+        assert worker.poll(rid)
+        res = worker.get_result(rid)
+        assert res["indices"].dtype == np.int32 and res["scores"].dtype == np.float32
+        assert np.array_equal(res["indices"], z[f"esa/{i}/indices"])
+        assert np.array_equal(bits(res["scores"]), bits(z[f"esa/{i}/scores"]))
+        with pytest.raises(RuntimeError, match="Result not ready"):
+            worker.get_result(rid)  # a result is handed out once
+
+
+def test_retrieval_worker_protocol_and_errors(ucm, dev):
+    from ucm_amd.sparse.esa.retrieval_worker import HipRetrievalBackend, RetrievalWorker
+
+    rows, dim = 500, 1024
+    data = torch.from_numpy(synth.normal_bf16_as_f32(700, (rows, dim))).to(dev)
+    backend = HipRetrievalBackend(data)
+    worker = RetrievalWorker(backend)
+    with pytest.raises(RuntimeError, match="Query dim mismatch"):
+        backend.submit(torch.zeros(1, dim - 1, device=dev), 3, [[1, 2]])
+    with pytest.raises(RuntimeError, match="Query and indexes batch mismatch"):
+        backend.submit(torch.zeros(2, dim, device=dev), 3, [[1, 2]])
+    with pytest.raises(RuntimeError, match="Bad req_id"):
+        backend.wait(12345)
+    # the way ESA calls it: one request, a python list of slot lists (esa.py:297-301)
+    slots = [int(s) for s in synth.permutation(701, rows)[:333]]
+    q = torch.from_numpy(synth.normal_bf16_as_f32(702, (1, dim))).to(dev)
+    ids = [worker.submit(q, topk=40, indexes=[slots]) for _ in range(3)]
+    assert ids == sorted(set(ids))  # fresh increasing ids
+    for rid in ids:
+        worker.wait(rid)
+        res = worker.get_result(rid)
+        wi, ws = O.esa_retrieve(data.cpu().numpy(), q.cpu().numpy()[0], np.array(slots, np.int32), 40)
+        assert np.array_equal(res["indices"][0], wi) and np.array_equal(bits(res["scores"][0]), bits(ws))
+    # topk larger than the candidate list returns every candidate, best first
+    rid = worker.submit(q, topk=5000, indexes=[slots[:17]])
+    worker.wait(rid)
+    res = worker.get_result(rid)
+    assert res["indices"].shape == (1, 17) and np.all(np.diff(res["scores"][0]) <= 0)
+    # rows written after construction are visible: the table is aliased, not copied
+    data[slots[5]] = 100.0 * q[0]
+    rid = worker.submit(q, topk=1, indexes=[slots])
+    worker.wait(rid)
+    assert worker.get_result(rid)["indices"][0, 0] == slots[5]
+    # ties: equal rows come out in index-row order
+    data[7] = data[3]
+    rid = worker.submit(q, topk=2, indexes=[[7, 3]])
+    worker.wait(rid)
+    assert list(worker.get_result(rid)["indices"][0]) == [7, 3]
+
+
+def test_esa_retrieve_wide_and_ragged_rows(ucm, dev):
+    """Batch of requests, -1 padding in the middle, out-of-range slots, dims that are not a multiple of the tile."""
+    from ucm_amd import ops
+
+    for rows, dim, b, m, topk in [(900, 1024, 4, 700, 210), (64, 36, 3, 9, 4), (3000, 256, 2, 2500, 900)]:
+        data_h = synth.normal_bf16_as_f32(710 + dim, (rows, dim))
+        q_h = synth.normal_bf16_as_f32(711 + dim, (b, dim))
+        idx = np.stack([synth.permutation(712 + r, rows)[:m] for r in range(b)]).astype(np.int32)
+        idx[:, ::5] = -1
+        idx[0, 1] = rows + 7  # outside the table: skipped like a padding entry
+        out_idx = torch.full((b, min(topk, m)), -1, dtype=torch.int32, device=dev)
+        out_scores = torch.zeros((b, min(topk, m)), device=dev)
+        out_cnt = torch.zeros(b, dtype=torch.int32, device=dev)
+        ws = torch.empty(b, m, device=dev)
+        ops.esa_retrieve(torch.from_numpy(data_h).to(dev), torch.from_numpy(q_h).to(dev),
+                         torch.from_numpy(idx).to(dev), topk, ws, out_idx, out_scores, out_cnt)
+        for r in range(b):
+            row = idx[r].copy()
+            row[row >= rows] = -1
+            wi, wsc = O.esa_retrieve(data_h, q_h[r], row, topk)
+            c = int(out_cnt[r])
+            assert c == len(wi)
+            assert np.array_equal(out_idx[r, :c].cpu().numpy(), wi)
+            assert np.array_equal(bits(out_scores[r, :c].cpu().numpy()), bits(wsc))
+
+
+# ------------------------------------------------ CalKpreAndTopk surface
+
+def test_cal_kpre_and_topk_surface(ucm, dev):
+    """The reference's call sequence (gsa.py:484-512, :914-954, :616-632) against the GPU object."""
+    from ucm_amd.sparse.gsa.offload_ops import CalKpreAndTopk
+
+    L, bs, max_bs, hq, hkv, d, max_blocks = 3, 128, 8, 32, 8, 128, 64
+    obj = CalKpreAndTopk(L, bs, max_bs, hq, d, device=dev)
+    obj.set_kpre_method_param(hkv, 1)
+    kpre_all = torch.from_numpy(synth.normal_f32(720, (L, max_bs * max_blocks, 1, hkv, d))).to(dev)
+    obj.set_kpre_cache(list(kpre_all.unbind(0)))
+    # batch of 4: entries 0 and 2 decode with 50 and 37 blocks, 1 and 3 do not
+    is_decode = [True, False, True, False]
+    lens = [50, 0, 37, 0]
+    slot_map = [[max_blocks * (i + 1) + j for j in range(max(n, 1))] for i, n in enumerate(lens)]
+    topk_lens = [O.compute_topk_len(50), O.compute_topk_len(37)]
+    topk_cache = [torch.full((4, max_blocks), -1, dtype=torch.int32, device=dev) for _ in range(L)]
+    obj.set_common_param([0, 2], is_decode)
+    obj.set_topk_param(slot_map)
+    obj.set_topk_cache(topk_cache, topk_lens)
+    q = synth.normal_bf16_as_f32(721, (L, 4, hq, d))
+    for l in range(L):
+        qd = torch.from_numpy(q[l]).to(dev).to(torch.bfloat16)
+        obj.add_copy_req(False, l, [5, -1, 9, -1], qd)   # locations: -1 = not a decode entry
+    torch.cuda.synchronize()
+    assert obj.is_calculate_finish()
+    kp = kpre_all.cpu().numpy().reshape(L, max_bs * max_blocks, hkv * d)
+    for l in range(L):
+        got = topk_cache[l].cpu().numpy()
+        for i, j in ((0, 0), (2, 1)):
+            want, _ = O.select_topk(q[l, i], kp[l, slot_map[i][0] : slot_map[i][0] + lens[i]].reshape(lens[i], hkv, 1, d),
+                                    topk_lens[j])
+            assert np.array_equal(got[i, : len(want)], want), (l, i)
+        assert np.all(got[1] == -1) and np.all(got[3] == -1)
+        assert np.array_equal(obj.q_cache[l][0].cpu().numpy(), q[l, 0])
+    with pytest.raises(NotImplementedError):
+        obj.set_kpre_method_param(hkv, 2)
+
+
+# ------------------------------------------------------------ GSA plugin
+
+class _ModelConfig:
+    def __init__(self, hq, hkv, d, layers, max_model_len):
+        self.hq, self.hkv, self.d, self.layers, self.max_model_len = hq, hkv, d, layers, max_model_len
+
+    def get_num_kv_heads(self, pc):
+        return self.hkv
+
+    def get_num_attention_heads(self, pc):
+        return self.hq
+
+    def get_head_size(self):
+        return self.d
+
+    def get_num_layers(self, pc):
+        return self.layers
+
+
+def make_config(hq, hkv, d, layers, block_size, max_model_len, gsa_cfg):
+    ns = types.SimpleNamespace
+    return ns(model_config=_ModelConfig(hq, hkv, d, layers, max_model_len), parallel_config=ns(rank=0, tensor_parallel_size=1),
+              cache_config=ns(block_size=block_size), scheduler_config=ns(max_num_seqs=4),
+              kv_transfer_config=ns(kv_connector_extra_config={"ucm_sparse_config": {"GSA": gsa_cfg}}))
+
+
+def topk_len(n, lo, hi):
+    t = int(n * 0.3)
+    return min(lo, n) if t < lo else min(t, hi)
+
+
+def test_gsa_plugin_decode_flow(ucm, dev):
+    """Two requests through prefill and 40 decode steps, two layers: after every attention_begin the
+    layer's block table and sequence lengths must be what the oracle selects from the same cache."""
+    from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
+    from ucm_amd.sparse.factory import UcmSparseFactory
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 120
+    lo, hi = 6, 10
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 60, {"seg_prefill_threshold": 100, "min_topk_len": lo, "max_topk_len": hi})
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    assert isinstance(plugin, GSA)
+    assert plugin.estimate_num_slots_sparsed(ns()) == INVALID_SLOT
+    plugin.request_begin("A", [])
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    caches = [torch.zeros(2, nb, bs, hkv, d, dtype=torch.bfloat16, device=dev) for _ in range(L)]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
+    free_blocks = [int(x) for x in synth.permutation(730, nb)]
+    prompts = {"A": 300, "B": 50}
+    reqs = {r: ns(block_ids=[[]], num_computed_tokens=0, prompt_token_ids=[1] * n, output_token_ids=[]) for r, n in prompts.items()}
+    repre_h = {r: [np.zeros((60, hkv * d), np.float32) for _ in range(L)] for r in prompts}
+    done_blocks = {r: 0 for r in prompts}
+    saw_sparse = 0
+
+    for step in range(41):
+        sched = {}
+        for r, st in reqs.items():
+            n_new = prompts[r] if step == 0 else 1
+            need = -(-(st.num_computed_tokens + n_new) // bs)
+            while len(st.block_ids[0]) < need:
+                st.block_ids[0].append(free_blocks.pop())
+            sched[r] = n_new
+        so = ns(num_scheduled_tokens=sched, scheduled_new_reqs=[ns(req_id=r) for r in reqs] if step == 0 else [],
+                scheduled_cached_reqs=ns(req_ids=[] if step == 0 else list(reqs)))
+        ib = ns(req_id_to_index={"A": 0, "B": 1})
+        n_tok = sum(sched.values())
+        seq_lens = [reqs[r].num_computed_tokens + sched[r] for r in ("A", "B")]
+        width = 60
+        bt = torch.zeros(2, width, dtype=torch.int32, device=dev)
+        for i, r in enumerate(("A", "B")):
+            bt[i, : len(reqs[r].block_ids[0])] = torch.tensor(reqs[r].block_ids[0], dtype=torch.int32)
+        plugin.build_sparse_meta(so, reqs, ib, None)
+        plugin.execute_begin(so)
+        for l in range(L):
+            md = ns(block_table=bt.clone(), seq_lens=torch.tensor(seq_lens, dtype=torch.int32, device=dev))
+            fc.attn_metadata = {names[l]: md}
+            query = torch.randn(n_tok, hq, d, device=dev, generator=g).to(torch.bfloat16)
+            key = torch.randn(n_tok, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+            # the model writes this step's keys into the paged cache before attention runs
+            t0 = 0
+            for r in ("A", "B"):
+                for t in range(sched[r]):
+                    pos = reqs[r].num_computed_tokens + t
+                    caches[l][0, reqs[r].block_ids[0][pos // bs], pos % bs] = key[t0 + t]
+                t0 += sched[r]
+            plugin.attention_begin(query, key, key, names[l], fc)
+            torch.cuda.synchronize()
+            if step > 0:
+                # request A is sparsified, B keeps everything
+                nA = len(reqs["A"].block_ids[0])
+                k = topk_len(nA, lo, hi)
+                qA = query[0].float().cpu().numpy()  # A's only (= last) token is row 0 of the batch
+                want_idx, _ = O.select_topk(qA, repre_h["A"][l][:nA].reshape(nA, hkv, 1, d), k)
+                phys, want_len = O.block_table_gather(reqs["A"].block_ids[0], want_idx, seq_lens[0], bs)
+                got_bt, got_len = md.block_table.cpu().numpy(), md.seq_lens.cpu().numpy()
+                assert got_len[0] == want_len, (step, l)
+                assert np.array_equal(got_bt[0, : len(phys)], phys), (step, l)
+                nB = len(reqs["B"].block_ids[0])
+                assert got_len[1] == seq_lens[1] and np.array_equal(got_bt[1, :nB], reqs["B"].block_ids[0])
+                saw_sparse += int(len(phys) < nA)
+            else:
+                assert md.block_table.data_ptr() != plugin.block_tables_mp.data_ptr()  # prefill: untouched
+            plugin.attention_finished(query, key, key, None, names[l], fc)
+            # oracle-side table: a block is reduced after the step that fills it
+            for r in ("A", "B"):
+                full = min(seq_lens[("A", "B").index(r)] // bs, len(reqs[r].block_ids[0]))
+                todo = list(range(done_blocks[r], full))
+                if todo:
+                    kc = caches[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+                    O.block_mean_paged(kc, [reqs[r].block_ids[0][i] for i in todo], todo, repre_h[r][l])
+        for r in ("A", "B"):
+            done_blocks[r] = max(done_blocks[r], min(seq_lens[("A", "B").index(r)] // bs, len(reqs[r].block_ids[0])))
+        plugin.execute_finished()
+        torch.cuda.synchronize()
+        # the device table equals the oracle's
+        offA = plugin.gsa_stats["A"].slot_offset
+        for l in range(L):
+            got = plugin.kpre_caches[l, offA : offA + done_blocks["A"]].cpu().numpy()
+            assert np.array_equal(bits(got), bits(repre_h["A"][l][: done_blocks["A"]])), (step, l)
+        for r, st in reqs.items():
+            st.num_computed_tokens += sched[r]
+            st.output_token_ids.append(7)
+    assert saw_sparse >= 2 * 39  # every decode step of every layer really dropped blocks
+    plugin.request_finished_in_worker("A")
+    assert "A" not in plugin.gsa_stats and not plugin.topk_kpre_manger.is_exist("A")
+
+
+def test_gsa_retrieval_stride_reuses_scores(ucm, dev):
+    """With retrieval_stride 3 the scores of the last retrieval are re-selected with the current lengths
+    on the steps in between (the last two blocks are always kept, so the newest block is never missing);
+    a request is scored on its first sparsified step whatever the stride."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 64, 1, 16, 64
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 40, {"seg_prefill_threshold": 10, "min_topk_len": 5, "max_topk_len": 5,
+                                                   "retrieval_stride": 3})
+    plugin = GSA(cfg, UcmSparseRole.WORKER)
+    cache = torch.randn(2, nb, bs, hkv, d, device=dev).to(torch.bfloat16)
+    name = "model.layers.0.self_attn.attn"
+    fc = ns(no_compile_layers={name: ns(kv_cache=[cache])}, virtual_engine=0, attn_metadata=None)
+    st = ns(block_ids=[list(range(20))], num_computed_tokens=0, prompt_token_ids=[1] * 318, output_token_ids=[])
+    ib = ns(req_id_to_index={"A": 0})
+    tables, scored = [], []
+    for step in range(5):
+        n_new = 318 if step == 0 else 1
+        if step == 3:
+            st.block_ids[0].append(33)  # token 320 opens block 21
+        so = ns(num_scheduled_tokens={"A": n_new}, scheduled_new_reqs=[ns(req_id="A")] if step == 0 else [])
+        plugin.build_sparse_meta(so, {"A": st}, ib, None)
+        plugin.execute_begin(so)
+        scored.append(plugin.model_input["is_topk"])
+        md = ns(block_table=None, seq_lens=None)
+        fc.attn_metadata = md
+        q = torch.randn(n_new, hq, d, device=dev).to(torch.bfloat16)
+        plugin.attention_begin(q, None, None, name, fc)
+        plugin.attention_finished(q, None, None, None, name, fc)
+        plugin.execute_finished()
+        torch.cuda.synchronize()
+        st.num_computed_tokens += n_new
+        st.output_token_ids.append(1)
+        if step > 0:
+            cnt = int(plugin.topk_counts[0, 0])
+            tables.append((md.block_table[0, :cnt].cpu().tolist(), int(md.seq_lens[0])))
+        else:
+            assert md.block_table is None  # prefill: the layer's metadata is left alone
+    assert scored == [False, True, False, True, False]
+    assert tables[0][0] == tables[1][0] and tables[0][0][-2:] == [18, 19]     # step 2 re-selects step 1's scores
+    assert tables[2][0][-2:] == [19, 33] and tables[3][0] == tables[2][0]      # the new block is in the local window
+    assert all(len(t[0]) == 5 and t[0][0] == 0 for t in tables)
+    assert [t[1] for t in tables] == [4 * 16 + 15, 5 * 16, 4 * 16 + 1, 4 * 16 + 2]

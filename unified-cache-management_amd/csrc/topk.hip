@@ -48,6 +48,7 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
     int32_t* pout = phys_out ? phys_out + lr * out_stride : nullptr;
     const int32_t* bt = block_tables ? block_tables + static_cast<size_t>(r) * bt_stride : nullptr;
     int count = 0;
+    bool kept_all = false;
 
     if (n <= 0) {
         count = 0;
@@ -57,6 +58,7 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
             if (pout) { pout[i] = bt[i]; }
         }
         count = n;
+        kept_all = true;
     } else if (k < start_w + end_w) {
         // fewer slots than forced blocks: the first k of [0..start_w) ++ [n-end_w..n)
         for (int j = lane; j < k; j += 64) {
@@ -117,8 +119,9 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
     if (lane == 0) {
         count_out[lr] = count;
         if (sparse_seq_lens && seq_lens) {
-            const int rem = seq_lens[r] % block_size;
-            sparse_seq_lens[lr] = rem == 0 ? count * block_size : count * block_size - block_size + rem;
+            const int len = seq_lens[r], rem = len % block_size;
+            // every block kept: the request keeps its length; otherwise `count` blocks, the last one partial
+            sparse_seq_lens[lr] = kept_all ? len : (rem == 0 ? count * block_size : count * block_size - block_size + rem);
         }
     }
 }

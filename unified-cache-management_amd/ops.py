@@ -146,6 +146,24 @@ def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Ten
               _stream())
 
 
+def esa_retrieve(data: torch.Tensor, q: torch.Tensor, indexes: torch.Tensor, topk: int, scores_ws: torch.Tensor,
+                 out_idx: torch.Tensor, out_scores: torch.Tensor, out_count: torch.Tensor,
+                 stream: Optional[int] = None) -> None:
+    """data fp32 [N, dim]; q fp32 [B, dim]; indexes int32 [B, M] (-1 padded); outputs [B, stride]."""
+    if data.dim() != 2 or q.dim() != 2 or indexes.dim() != 2:
+        raise ValueError("data [N,dim], q [B,dim], indexes [B,M] expected")
+    batch, m = indexes.shape
+    if q.shape != (batch, data.shape[1]):
+        raise ValueError("q must be [B, dim]")
+    if scores_ws.numel() < batch * m or out_idx.shape != out_scores.shape or out_idx.shape[0] != batch:
+        raise ValueError("workspace / outputs too small")
+    _lib.call("ucm_esa_retrieve", _dev(data, torch.float32, "data"), data.shape[0], data.shape[1],
+              _dev(q, torch.float32, "q"), _dev(indexes, torch.int32, "indexes"), batch, m, int(topk),
+              _dev(scores_ws, torch.float32, "scores_ws"), _dev(out_idx, torch.int32, "out_idx"),
+              _dev(out_scores, torch.float32, "out_scores"), _dev(out_count, torch.int32, "out_count"),
+              out_idx.shape[1], _stream() if stream is None else stream)
+
+
 def copy_batch(dst_ptrs: torch.Tensor, src_ptrs: torch.Tensor, size: int) -> None:
     """dst_ptrs/src_ptrs: int64 device tensors of raw addresses; copies size bytes each."""
     if dst_ptrs.numel() != src_ptrs.numel():

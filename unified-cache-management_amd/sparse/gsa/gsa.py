@@ -1,0 +1,351 @@
+"""GSA-shaped sparse-attention plugin whose retrieval runs on the GPU.
+
+Same hook surface and per-step flow as the reference's ``GSA``
+(ucm/sparse/gsa/gsa.py:415-1031): block representatives are refreshed after
+each layer's attention (``copy_k``, :634-654), each request's last query token
+drives a top-k over its block representatives (``copy_q`` :616-632 +
+``CalKpreAndTopk``), and ``attention_begin`` swaps the layer's block table and
+sequence lengths for sparse ones (:656-686, built by
+``GSAPrefetchBase._no_gsa_input_deal``,
+ucm/sparse/gsa/prefetch/prefetch_engine.py:507-553).
+
+What differs is where it runs.  The reference moves queries and block means to
+the host, scores them with OpenMP loops and uses the result a few steps later.
+Here the representative table, the scores and the per-layer sparse block
+tables never leave HBM: ``attention_begin`` enqueues the scoring and selection
+kernels of that layer on the model's own stream, and the attention kernel of
+the same layer already reads the fresh table.  No host synchronisation happens
+in any hook; per-step metadata goes down in one pinned-memory copy.
+
+vLLM is not imported: the hooks only touch attributes of the objects they are
+handed (``scheduler_output.num_scheduled_tokens``, ``requests[id].block_ids``,
+``forward_context.no_compile_layers[name].kv_cache``, ``attn_metadata.block_table``
+...), so stand-in objects drive the class in the tests.
+"""
+from __future__ import annotations
+
+import math
+from itertools import accumulate
+from typing import Dict, List, Optional, Union
+
+import torch
+
+from ... import ops
+from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
+from ..utils import (
+    INIT_WINDOW_BLOCKS,
+    LOCAL_WINDOW_BLOCKS,
+    MAX_BS,
+    MAX_TOPK_LEN,
+    MIN_TOPK_LEN,
+    SEG_PREFILL_THRESHOLD,
+    compute_topk_len,
+)
+
+ReqType = Union[str, int]
+
+
+class GSAReqStat:
+    """Per-request bookkeeping (role of the reference's GSAReqStat, gsa.py:66-239):
+    the request's cache blocks, the representative rows they map to, and which
+    blocks need their representative (re)computed after this step."""
+
+    def __init__(self, req_id: ReqType, slot_offset: int, block_size: int, threshold: int):
+        self.req_id = req_id
+        self.slot_offset = slot_offset
+        self.block_size = block_size
+        self.threshold = threshold
+        self.blocks: List[int] = []
+        self.calc_block_table: List[int] = []
+        self.calc_repre_slot_mapping: List[int] = []
+        self.num_computed_tokens = 0
+        self.num_scheduled_tokens = 0
+        self.num_prompt_tokens = 0
+        self.num_output_tokens = 0
+        self.index_in_batch = 0
+        self._repre_done = 0  # blocks [0, _repre_done) have a representative
+
+    # -- state queries (same meaning as the reference's) ---------------------
+    def is_decode(self) -> bool:
+        return self.num_prompt_tokens <= self.num_computed_tokens
+
+    def is_gsa(self) -> bool:
+        return self.num_prompt_tokens > self.threshold and self.is_decode()
+
+    def is_last_chunk(self) -> bool:
+        return self.num_computed_tokens + self.num_scheduled_tokens >= self.num_prompt_tokens
+
+    def get_seq_len(self) -> int:
+        return self.num_computed_tokens + self.num_scheduled_tokens
+
+    @property
+    def repre_slot_mapping(self) -> List[int]:
+        return [self.slot_offset + i for i in range(len(self.blocks))]
+
+    def update(self, num_scheduled_tokens: int, req_state, index_in_batch: int) -> None:
+        self.num_computed_tokens = req_state.num_computed_tokens
+        self.num_scheduled_tokens = num_scheduled_tokens
+        self.num_prompt_tokens = len(req_state.prompt_token_ids)
+        self.num_output_tokens = len(req_state.output_token_ids)
+        self.index_in_batch = index_in_batch
+        self.blocks = list(req_state.block_ids[0])
+        # A block gets its representative once every one of its tokens is in
+        # the cache, i.e. after the step that fills it.
+        full_after_step = self.get_seq_len() // self.block_size
+        full_after_step = min(full_after_step, len(self.blocks))
+        todo = range(self._repre_done, full_after_step)
+        self.calc_block_table = [self.blocks[i] for i in todo]
+        self.calc_repre_slot_mapping = [self.slot_offset + i for i in todo]
+        self._repre_done = max(self._repre_done, full_after_step)
+
+
+class GSAMetaData(UcmSparseMetadata):
+    def __init__(self, block_size: int, device):
+        self.gsa_stats: Dict[ReqType, GSAReqStat] = {}
+        self.block_size = block_size
+        self.device = device
+
+
+class TopKAndKpreManger:
+    """Hands each live request one of max_num row ranges of the representative
+    table (gsa.py:323-351; spelling of the class name kept)."""
+
+    def __init__(self, max_num: int):
+        self.cache_map: Dict[ReqType, int] = {}
+        self.max_num = max_num
+        self.free_cache = list(range(max_num))
+
+    def free(self, req_id: ReqType) -> bool:
+        if req_id not in self.cache_map:
+            return False
+        self.free_cache.append(self.cache_map.pop(req_id))
+        return True
+
+    def alloc(self, req_id: ReqType) -> Optional[int]:
+        if not self.free_cache:
+            return None
+        self.cache_map[req_id] = self.free_cache.pop(0)
+        return self.cache_map[req_id]
+
+    def is_exist(self, req_id: ReqType) -> bool:
+        return req_id in self.cache_map
+
+
+class GSA(UcmSparseBase):
+    def __init__(self, vllm_config, role: UcmSparseRole):
+        super().__init__(vllm_config, role)
+        mc, pc = vllm_config.model_config, vllm_config.parallel_config
+        self.block_size = vllm_config.cache_config.block_size
+        self.num_key_heads = mc.get_num_kv_heads(pc)
+        self.num_q_heads = mc.get_num_attention_heads(pc)
+        self.head_size = mc.get_head_size()
+        self.layer_num = mc.get_num_layers(pc)
+        self.max_block_len = math.ceil(mc.max_model_len / self.block_size)
+        sched = getattr(vllm_config, "scheduler_config", None)
+        self.max_bs = min(MAX_BS, getattr(sched, "max_num_seqs", MAX_BS))
+        extra = vllm_config.kv_transfer_config.kv_connector_extra_config
+        cfg = dict((extra.get("ucm_sparse_config") or {}).get("GSA") or {})
+        self.threshold = int(cfg.get("seg_prefill_threshold", SEG_PREFILL_THRESHOLD))
+        self.retrieval_stride = max(1, int(cfg.get("retrieval_stride", 1)))
+        self.min_topk = int(cfg.get("min_topk_len", MIN_TOPK_LEN))
+        self.max_topk = int(cfg.get("max_topk_len", MAX_TOPK_LEN))
+        self.topk_ratio = float(cfg.get("sparse_ratio", 0.3))
+        self.init_window = int(cfg.get("init_window_sz", INIT_WINDOW_BLOCKS))
+        self.local_window = int(cfg.get("local_window_sz", LOCAL_WINDOW_BLOCKS))
+        self.repre_mode = ops.MEAN_BF16_ROUND if cfg.get("repre_dtype", "float32") == "bfloat16" else ops.MEAN_F32
+
+        self.topk_kpre_manger = TopKAndKpreManger(self.max_bs)
+        self.gsa_stats: Dict[ReqType, GSAReqStat] = {}
+        self.gsa_metadata: Optional[GSAMetaData] = None
+        self.model_input: dict = {}
+        self.step_count = 0
+        self.k_cache: Dict[int, torch.Tensor] = {}
+        self.v_cache: Dict[int, torch.Tensor] = {}
+        self._dev_ready = False
+        self._layer_ptrs: Dict[int, ops.LayerPointers] = {}
+        self._scored: set = set()  # sparsified requests whose blocks have been scored at least once
+
+    # ------------------------------------------------------------------ device state
+    def _ensure_device_state(self, device) -> None:
+        if self._dev_ready:
+            return
+        rows = self.max_bs * self.max_block_len
+        row = self.num_key_heads * self.head_size
+        L = self.layer_num
+        self.device = device
+        self.kpre_caches = torch.zeros((L, rows, row), dtype=torch.float32, device=device)
+        self.scores = torch.zeros((L, rows), dtype=torch.float32, device=device)
+        self.topk_caches = torch.zeros((L, self.max_bs, self.max_block_len), dtype=torch.int32, device=device)
+        self.block_tables_mp = torch.zeros_like(self.topk_caches)
+        self.topk_counts = torch.zeros((L, self.max_bs), dtype=torch.int32, device=device)
+        self.gsa_seq_len = torch.zeros((L, self.max_bs), dtype=torch.int32, device=device)
+        # two pinned staging buffers for the per-step descriptors, used alternately
+        cap = (5 + 3 * self.max_block_len) * self.max_bs
+        self._host_desc = [torch.zeros(cap, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._host_free = [None, None]  # event recorded after each buffer's last upload
+        self._dev_ready = True
+
+    def register_kv_caches(self, kv_caches: dict) -> None:
+        for name, cache in kv_caches.items():
+            self._register_layer(int(name.split(".")[2]), cache)
+
+    def _register_layer(self, layer_id: int, kv_cache) -> None:
+        if layer_id in self._layer_ptrs and self.k_cache[layer_id].data_ptr() == kv_cache[0].data_ptr():
+            return
+        self.k_cache[layer_id], self.v_cache[layer_id] = kv_cache[0], kv_cache[1]
+        self._layer_ptrs[layer_id] = ops.LayerPointers([kv_cache[0]])
+        self._ensure_device_state(kv_cache[0].device)
+
+    def maybe_register_kv_cache(self, forward_context, layer_name: str) -> None:
+        attn = forward_context.no_compile_layers[layer_name]
+        self._register_layer(int(layer_name.split(".")[2]), attn.kv_cache[forward_context.virtual_engine])
+
+    # ------------------------------------------------------------------ per-step metadata
+    def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata) -> None:
+        meta = GSAMetaData(self.block_size, getattr(self, "device", None))
+        meta.gsa_stats = self.gsa_stats
+        new_ids = {r.req_id for r in getattr(scheduler_output, "scheduled_new_reqs", [])}
+        for req_id, n_tok in scheduler_output.num_scheduled_tokens.items():
+            if req_id in new_ids and req_id in self.gsa_stats:
+                self.request_finished_in_worker(req_id)  # id reused by a new request
+            if not self.topk_kpre_manger.is_exist(req_id):
+                if self.topk_kpre_manger.alloc(req_id) is None:
+                    raise RuntimeError("more live requests than representative-table partitions")
+            if req_id not in self.gsa_stats:
+                self.gsa_stats[req_id] = GSAReqStat(
+                    req_id, self.max_block_len * self.topk_kpre_manger.cache_map[req_id], self.block_size,
+                    self.threshold)
+            self.gsa_stats[req_id].update(n_tok, requests[req_id], input_batch.req_id_to_index[req_id])
+        self.gsa_metadata = meta
+        self._sparse_metadata = meta
+
+        batch = len(scheduler_output.num_scheduled_tokens)
+        by_index: List[Optional[GSAReqStat]] = [None] * batch
+        query_locals = [0] * (batch + 1)
+        calc_blocks: List[int] = []
+        calc_slots: List[int] = []
+        for req_id, n_tok in scheduler_output.num_scheduled_tokens.items():
+            st = self.gsa_stats[req_id]
+            by_index[st.index_in_batch] = st
+            query_locals[st.index_in_batch + 1] = n_tok
+            calc_blocks += st.calc_block_table
+            calc_slots += st.calc_repre_slot_mapping
+        query_locals = list(accumulate(query_locals))
+        self.model_input = {
+            "calc_block_table": calc_blocks,
+            "calc_repre_slot_mapping": calc_slots,
+            "query_locals": query_locals,
+            "batch": by_index,
+        }
+
+    def execute_begin(self, scheduler_output) -> None:
+        """Packs this step's descriptors and sends them down in one copy."""
+        by_index: List[Optional[GSAReqStat]] = self.model_input.get("batch", [])
+        batch = len(by_index)
+        gsa_ids = {st.req_id for st in by_index if st is not None and st.is_gsa()}
+        any_gsa = bool(gsa_ids)
+        self.model_input["any_gsa"] = any_gsa
+        # score on every retrieval_stride-th step, and whenever a request is sparsified for the first time
+        is_topk = any_gsa and (self.step_count % self.retrieval_stride == 0 or not gsa_ids <= self._scored)
+        self.model_input["is_topk"] = is_topk
+        if is_topk:
+            self._scored |= gsa_ids
+        if not any_gsa or not self._dev_ready:
+            return
+        width = self.max_block_len
+        n_calc = len(self.model_input["calc_block_table"])
+        # one int32 host buffer: 5 descriptor rows, the block tables, then the block-mean lists
+        slot = self.step_count & 1
+        if self._host_free[slot] is not None:
+            self._host_free[slot].synchronize()  # upload of two steps ago; long finished
+        host = self._host_desc[slot][: 5 * batch + batch * width + 2 * n_calc]
+        host.zero_()
+        desc = host[: 5 * batch].view(5, batch)
+        tables = host[5 * batch : 5 * batch + batch * width].view(batch, width)
+        max_len = total = 0
+        for i, st in enumerate(by_index):
+            if st is None:
+                continue
+            n = len(st.blocks)
+            desc[0, i], desc[1, i] = st.slot_offset, n
+            k = compute_topk_len(n, self.min_topk, self.max_topk, self.topk_ratio) if st.is_gsa() else n
+            desc[2, i] = max(k, 1)          # k >= n keeps every block (short or prefilling requests)
+            desc[3, i] = self.model_input["query_locals"][i + 1] - 1
+            desc[4, i] = st.get_seq_len()
+            tables[i, :n] = torch.tensor(st.blocks, dtype=torch.int32)
+            max_len, total = max(max_len, n), total + n
+        tail = host[5 * batch + batch * width :]
+        tail[:n_calc] = torch.tensor(self.model_input["calc_block_table"], dtype=torch.int32)
+        tail[n_calc:] = torch.tensor(self.model_input["calc_repre_slot_mapping"], dtype=torch.int32)
+        dev = host.to(self.device, non_blocking=True)
+        self._host_free[slot] = torch.cuda.Event()
+        self._host_free[slot].record()
+        d = dev[: 5 * batch].view(5, batch)
+        self.model_input.update(
+            seg_off=d[0], seg_len=d[1], topk_len=d[2], q_rows=d[3], seq_lens=d[4],
+            block_tables=dev[5 * batch : 5 * batch + batch * width].view(batch, width),
+            calc_blocks_dev=dev[5 * batch + batch * width : 5 * batch + batch * width + n_calc],
+            calc_slots_dev=dev[5 * batch + batch * width + n_calc :],
+            max_len=max_len, total=total, n_batch=batch,
+        )
+
+    def execute_finished(self) -> None:
+        self.step_count += 1
+
+    # ------------------------------------------------------------------ per-layer hooks
+    def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        self.maybe_register_kv_cache(forward_context, layer_name)
+        mi = self.model_input
+        if not mi.get("any_gsa") or "seg_off" not in mi:
+            return
+        l = int(layer_name.split(".")[2])
+        n = mi["n_batch"]
+        if mi["is_topk"]:
+            q = query.view(1, query.shape[0], self.num_q_heads, self.head_size)
+            ops.score_blocks(q, self.kpre_caches[l : l + 1], mi["seg_off"], mi["seg_len"], mi["max_len"],
+                             self.num_key_heads, self.scores[l : l + 1], q_rows=mi["q_rows"],
+                             total_blocks=mi["total"])
+        # selection (fresh scores, or the last ones with this step's lengths), block-table lookup, sparse lengths
+        ops.topk_windows(self.scores[l : l + 1], mi["seg_off"], mi["seg_len"], mi["topk_len"], mi["max_len"],
+                         self.topk_caches[l : l + 1, :n], self.topk_counts[l : l + 1, :n],
+                         start_w=self.init_window, end_w=self.local_window, block_tables=mi["block_tables"],
+                         phys_out=self.block_tables_mp[l : l + 1, :n], seq_lens=mi["seq_lens"],
+                         block_size=self.block_size, sparse_seq_lens=self.gsa_seq_len[l : l + 1, :n])
+        md = forward_context.attn_metadata
+        md = md[layer_name] if isinstance(md, dict) else md
+        md.block_table = self.block_tables_mp[l, :n]
+        md.seq_lens = self.gsa_seq_len[l, :n]
+
+    def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
+        self.maybe_register_kv_cache(forward_context, layer_name)
+        self.copy_k(layer_name, forward_context)
+
+    def copy_k(self, layer_name: str, forward_context) -> None:
+        """Representatives of the blocks this step filled (gsa.py:634-654), reduced in place on the device."""
+        blocks = self.model_input.get("calc_block_table") or []
+        if not blocks:
+            return
+        l = int(layer_name.split(".")[2])
+        if "calc_blocks_dev" in self.model_input:
+            ids, slots = self.model_input["calc_blocks_dev"], self.model_input["calc_slots_dev"]
+        else:  # a step without any sparsified request still has to keep the table current
+            ids = torch.tensor(blocks, dtype=torch.int32, device=self.device)
+            slots = torch.tensor(self.model_input["calc_repre_slot_mapping"], dtype=torch.int32, device=self.device)
+            self.model_input["calc_blocks_dev"], self.model_input["calc_slots_dev"] = ids, slots
+        k_cache = self.k_cache[l]
+        ops.block_mean(self._layer_ptrs[l], ids, slots, self.kpre_caches[l : l + 1], self.block_size,
+                       self.num_key_heads, self.head_size, k_cache.shape[0], mode=self.repre_mode)
+
+    def request_finished_in_worker(self, request_id: ReqType) -> None:
+        self.topk_kpre_manger.free(request_id)
+        self.gsa_stats.pop(request_id, None)
+        self._scored.discard(request_id)
+
+    # ------------------------------------------------------------------ scheduler side
+    def request_begin(self, request_id: ReqType, prompt_token_ids: List[int]) -> None:
+        pass
+
+    def estimate_num_slots_sparsed(self, request) -> int:
+        # blocks are not freed by this plugin (the reference returns INVALID_SLOT too
+        # unless its prefetch path is compiled in, gsa.py:891-912)
+        return INVALID_SLOT
