@@ -1,0 +1,160 @@
+"""Host-side logic that needs no GPU: the hook surface, the registry, request
+bookkeeping and the top-k length rule."""
+import inspect
+import types
+
+import pytest
+
+import oracle as O
+
+ns = types.SimpleNamespace
+
+
+class _ModelConfig:
+    max_model_len = 4096
+
+    def get_num_kv_heads(self, pc):
+        return 8
+
+    def get_num_attention_heads(self, pc):
+        return 32
+
+    def get_head_size(self):
+        return 128
+
+    def get_num_layers(self, pc):
+        return 4
+
+
+def make_config(name="GSA", cfg=None):
+    return ns(model_config=_ModelConfig(), parallel_config=ns(), cache_config=ns(block_size=128),
+              scheduler_config=ns(max_num_seqs=8),
+              kv_transfer_config=ns(kv_connector_extra_config={"ucm_sparse_config": {name: cfg or {}}}))
+
+
+def test_hook_surface_matches_the_patched_call_sites(ucm):
+    """Names and positional parameters vLLM's patched call sites use
+    (vllm-adapt.patch:80-115, :359-364, :573-574, :1159-1176)."""
+    from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseBase
+
+    want = {
+        "bind_sparse_metadata": ["sparse_metadata"],
+        "clear_sparse_metadata": [],
+        "register_kv_caches": ["kv_caches"],
+        "execute_begin": ["scheduler_output"],
+        "execute_finished": [],
+        "attention_begin": ["query", "key", "value", "layer_name", "forward_context"],
+        "attention_finished": ["query", "key", "value", "attn_output", "layer_name", "forward_context"],
+        "request_finished_in_worker": ["request_id"],
+        "request_begin": ["request_id", "prompt_token_ids"],
+        "request_finished_in_scheduler": ["request_id"],
+        "estimate_num_slots_sparsed": ["request"],
+        "update_state_after_alloc": ["request", "num_blocks"],
+        "build_sparse_meta": ["scheduler_output", "requests", "input_batch", "attn_metadata"],
+        "allocate_slots": ["request", "num_slots_sparsed", "coordinator", "block_pool", "kv_cache_groups"],
+    }
+    for name, params in want.items():
+        sig = inspect.signature(getattr(UcmSparseBase, name))
+        assert list(sig.parameters)[1:] == params, name
+    assert INVALID_SLOT == -1
+    with pytest.raises(TypeError):
+        UcmSparseBase(None, None)  # request_begin is abstract, as in the reference
+
+    class Minimal(UcmSparseBase):
+        def request_begin(self, request_id, prompt_token_ids):
+            pass
+
+    m = Minimal(None, None)
+    assert m.estimate_num_slots_sparsed(None) == INVALID_SLOT and m.allocate_slots(1, 2, 3, 4, 5) is None
+    with pytest.raises(AssertionError):
+        m._get_sparse_metadata()
+    m.bind_sparse_metadata("x")
+    assert m._get_sparse_metadata() == "x"
+    m.clear_sparse_metadata()
+
+
+def test_factory_and_process_state(ucm):
+    from ucm_amd.sparse import state
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.factory import UcmSparseFactory
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    state.reset_ucm_sparse()
+    assert not state.has_ucm_sparse()
+    with pytest.raises(RuntimeError, match="not initialized"):
+        state.get_ucm_sparse()
+    state.ensure_ucm_sparse_initialized(ns(kv_transfer_config=None))
+    state.ensure_ucm_sparse_initialized(ns(kv_transfer_config=ns(kv_connector_extra_config={})))
+    assert not state.has_ucm_sparse()
+    state.ensure_ucm_sparse_initialized(make_config(), UcmSparseRole.SCHEDULER)
+    agent = state.get_ucm_sparse()
+    assert isinstance(agent, GSA) and agent.role == UcmSparseRole.SCHEDULER
+    state.ensure_ucm_sparse_initialized(make_config())
+    assert state.get_ucm_sparse() is agent  # created once per process
+    state.reset_ucm_sparse()
+    with pytest.raises(ValueError, match="Unsupported sparse method"):
+        UcmSparseFactory.create_sparse_method(make_config("NoSuchMethod"), UcmSparseRole.WORKER)
+    with pytest.raises(ValueError, match="already registered"):
+        UcmSparseFactory.register_sparse_method("GSA", "x", "y")
+
+
+def test_compute_topk_len_matches_the_oracle(ucm):
+    from ucm_amd.sparse.utils import compute_topk_len
+
+    for n in range(0, 600):
+        assert compute_topk_len(n) == O.compute_topk_len(n)
+    assert compute_topk_len(30, 6, 10) == 9 and compute_topk_len(10, 6, 10) == 6 and compute_topk_len(4, 6, 10) == 4
+
+
+def test_request_bookkeeping(ucm):
+    from ucm_amd.sparse.gsa.gsa import GSAReqStat, TopKAndKpreManger
+
+    mgr = TopKAndKpreManger(2)
+    assert mgr.alloc("a") == 0 and mgr.alloc("b") == 1 and mgr.alloc("c") is None
+    assert mgr.free("a") and not mgr.free("a") and mgr.alloc("c") == 0 and mgr.is_exist("c")
+
+    st = GSAReqStat("r", slot_offset=1000, block_size=16, threshold=40)
+    req = ns(block_ids=[[5, 9, 2]], num_computed_tokens=0, prompt_token_ids=[0] * 60, output_token_ids=[])
+    st.update(40, req, 0)                       # first prefill chunk: 40 of 60 tokens -> blocks 0 and 1 are full
+    assert st.calc_block_table == [5, 9] and st.calc_repre_slot_mapping == [1000, 1001]
+    assert not st.is_decode() and not st.is_gsa() and not st.is_last_chunk()
+    req.num_computed_tokens, req.block_ids = 40, [[5, 9, 2, 7]]
+    st.update(20, req, 0)                       # last chunk: 60 tokens -> block 2 full, block 3 partial
+    assert st.is_last_chunk() and st.calc_block_table == [2] and st.calc_repre_slot_mapping == [1002]
+    req.num_computed_tokens, req.output_token_ids = 60, [1]
+    st.update(1, req, 3)                        # decode, 61 tokens
+    assert st.is_decode() and st.is_gsa() and st.calc_block_table == [] and st.index_in_batch == 3
+    assert st.repre_slot_mapping == [1000, 1001, 1002, 1003]
+    req.num_computed_tokens = 63
+    st.update(1, req, 0)                        # token 64 fills block 3
+    assert st.calc_block_table == [7] and st.calc_repre_slot_mapping == [1003] and st.get_seq_len() == 64
+    req.num_computed_tokens, req.block_ids = 64, [[5, 9, 2, 7, 11]]
+    st.update(1, req, 0)
+    assert st.calc_block_table == []            # the new block has one token; nothing to reduce yet
+    short = GSAReqStat("s", 0, 16, threshold=40)
+    short.update(30, ns(block_ids=[[1, 2]], num_computed_tokens=0, prompt_token_ids=[0] * 30, output_token_ids=[]), 0)
+    assert not short.is_gsa()
+
+
+def test_gsa_plugin_metadata_without_a_gpu(ucm):
+    """build_sparse_meta is pure host work: slots, block-mean lists and query offsets for a mixed batch."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    plugin = GSA(make_config(cfg={"seg_prefill_threshold": 200}), UcmSparseRole.WORKER)
+    assert plugin.max_block_len == 32 and plugin.max_bs == 8 and plugin.layer_num == 4
+    reqs = {
+        "x": ns(block_ids=[[3, 4, 5]], num_computed_tokens=0, prompt_token_ids=[0] * 300, output_token_ids=[]),
+        "y": ns(block_ids=[[8]], num_computed_tokens=0, prompt_token_ids=[0] * 100, output_token_ids=[]),
+    }
+    so = ns(num_scheduled_tokens={"x": 300, "y": 100}, scheduled_new_reqs=[ns(req_id="x"), ns(req_id="y")])
+    plugin.build_sparse_meta(so, reqs, ns(req_id_to_index={"x": 1, "y": 0}), None)
+    mi = plugin.model_input
+    assert mi["query_locals"] == [0, 100, 400]
+    assert mi["calc_block_table"] == [3, 4] and mi["calc_repre_slot_mapping"] == [0, 1]  # x owns partition 0
+    assert plugin.gsa_stats["y"].slot_offset == 32 and mi["batch"][0].req_id == "y"
+    plugin.execute_begin(so)
+    assert mi["any_gsa"] is False and mi["is_topk"] is False
+    plugin.execute_finished()
+    plugin.request_finished_in_worker("x")
+    assert "x" not in plugin.gsa_stats and plugin.topk_kpre_manger.free_cache[-1] == 0
