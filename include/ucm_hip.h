@@ -165,6 +165,57 @@ int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
                      ucm_stream_t stream);
 
 /*
+ * Hash-code retrieval (KvComp).  A vector's code has bit c = (x . W[:, c] > 0),
+ * packed LSB first (bit j of byte b is column 8b+j) - HashEncoder.compute_hash
+ * (ucm/sparse/kvcomp/hash_encoder.py:99-157, bit order :92-97,139-149; W is
+ * [head_dim][bits] in the model dtype, :65-71).  The sign is that of the exactly
+ * accumulated product (matrix cores, with an fp64 redo of every result inside
+ * the fp32 error bound).  head_dim = bits = 128.
+ *
+ * ucm_hash_encode_blocks: codes of the keys of the listed cache blocks
+ * (ReqStatePerLayer.extract_block_repre, ucm/sparse/kvcomp/kvcomp.py:314-347),
+ * read from the paged bf16 key cache like ucm_block_mean reads it.  Per block:
+ *   token_codes  dev u8 [n_layers][rows][block_size][kv_heads][16] (cache order;
+ *                may be NULL), layer stride in BYTES
+ *   colsum       dev int16 [n_layers][rows][kv_heads][128]: #ones - #zeros of
+ *                each bit over the block's tokens, layer stride in ELEMENTS
+ *   block_codes  dev u8 [n_layers][rows][kv_heads][16]: majority vote of each bit
+ *                (colsum > 0; an exact tie gives 0), layer stride in BYTES
+ * ucm_hash_encode_queries: per (layer, request) the codes of all query heads
+ * (q_codes u8 [L][n_req][q_heads][16]), their +-1 sum over heads (q_sum int16
+ * [L][n_req][128]) and the code of every kv head's group-mean query
+ * (qbar_codes u8 [L][n_req][kv_heads][16]); q is bf16 laid out as for
+ * ucm_score_blocks.
+ * ucm_hash_score_blocks: fp32 scores of all blocks of a ragged batch, written
+ * where ucm_topk_windows reads them.
+ *   mode 0  the reference's score (kvcomp.py:237-247): the sum over query heads,
+ *           kv heads and the block's tokens of the +-1 inner products, computed
+ *           as <q_sum, sum_h colsum[h]> (the same integer); round_fp16 != 0
+ *           rounds it to fp16 as the reference's fp16 sum does.
+ *   mode 1  sum over kv heads of (128 - hamming(qbar code, majority block code)),
+ *           the benchmark's block-code variant (not present in the reference).
+ * The reference keeps init 1 / local 2 blocks out of the candidates and
+ * index-sorts its picks (kvcomp.py:219-221,249-254): ucm_topk_windows with the
+ * matching windows gives the same set.
+ */
+int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers, int num_blocks,
+                           const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                           int kv_heads, int head_dim, const void* w_bf16, int bits, int rows,
+                           uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                           int64_t colsum_layer_stride, uint8_t* block_codes,
+                           int64_t block_codes_layer_stride, ucm_stream_t stream);
+int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows,
+                            int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
+                            const void* w_bf16, int bits, uint8_t* q_codes, int16_t* q_sum,
+                            uint8_t* qbar_codes, ucm_stream_t stream);
+int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_codes,
+                          const int16_t* colsum, int64_t colsum_layer_stride,
+                          const uint8_t* block_codes, int64_t block_codes_layer_stride,
+                          const int32_t* seg_off, const int32_t* seg_len, int n_req,
+                          int64_t total_blocks, int n_layers, int kv_heads, int bits, float* scores,
+                          int64_t scores_layer_stride, int round_fp16, ucm_stream_t stream);
+
+/*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched
  * pointer-array copy of the reference's device layer (H2DKernel / D2HKernel,
  * ucm/store/device/cuda/cuda_device.cu:47-81, reached through

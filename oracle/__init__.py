@@ -70,6 +70,8 @@ _orc_get_offset = _sig(_orc, "orc_get_offset", _i64, _i64, _i64, _i64, _i64, _i6
 _orc_kv_move_blocks = _sig(_orc, "orc_kv_move_blocks", None, _p, _u32, C.c_size_t, C.c_size_t, _p, _u32, _p, C.c_int)
 _orc_kv_gather_selected = _sig(_orc, "orc_kv_gather_selected", None, _p, _u32, C.c_size_t, C.c_size_t, _p, _p, _u32, _u32, _p, _p, _p)
 _orc_hash_encode = _sig(_orc, "orc_hash_encode", None, _p, _p, _u32, _u32, _u32, _p)
+_orc_hash_encode_f32 = _sig(_orc, "orc_hash_encode_f32", None, _p, _p, _u32, _u32, _u32, _p)
+_orc_hash_colsum = _sig(_orc, "orc_hash_colsum", None, _p, _u32, _u32, _u32, _u32, _p)
 _orc_hash_scores_sum = _sig(_orc, "orc_hash_scores_sum", None, _p, _u32, _p, _u32, _u32, _u32, _u32, _p)
 _orc_hash_majority = _sig(_orc, "orc_hash_majority", None, _p, _u32, _u32, _u32, _u32, _p)
 _orc_hash_scores_block = _sig(_orc, "orc_hash_scores_block", None, _p, _p, _u32, _u32, _u32, _p)
@@ -233,6 +235,25 @@ def hash_encode(x_bits: np.ndarray, w: np.ndarray) -> np.ndarray:
     out = np.empty((n, bits // 8), np.uint8)
     _orc_hash_encode(_ptr(xb), _ptr(ww), n, dim, bits, _ptr(out))
     return out.reshape(xb.shape[:-1] + (bits // 8,))
+
+
+def hash_encode_f32(x: np.ndarray, w: np.ndarray) -> np.ndarray:
+    """x fp32 [..., dim], w fp32 [dim, bits] -> uint8 [..., bits/8]."""
+    xx, ww = _c(x, np.float32), _c(w, np.float32)
+    dim, bits = ww.shape
+    n = xx.size // dim
+    out = np.empty((n, bits // 8), np.uint8)
+    _orc_hash_encode_f32(_ptr(xx), _ptr(ww), n, dim, bits, _ptr(out))
+    return out.reshape(xx.shape[:-1] + (bits // 8,))
+
+
+def hash_colsum(token_codes: np.ndarray) -> np.ndarray:
+    """token_codes [n, block_size, kv_heads, nbytes] -> int16 [n, kv_heads, nbytes*8] (#ones - #zeros)."""
+    tc = _c(token_codes, np.uint8)
+    n, t, h, nb = tc.shape
+    out = np.empty((n, h, nb * 8), np.int16)
+    _orc_hash_colsum(_ptr(tc), n, t, h, nb, _ptr(out))
+    return out
 
 
 def hash_scores_sum(q_codes: np.ndarray, key_codes: np.ndarray) -> np.ndarray:

@@ -512,6 +512,49 @@ ORC_API void orc_hash_encode(const uint16_t* x, const float* W, uint32_t n, uint
     }
 }
 
+/* Same projection and packing for fp32 inputs (the group-mean query of the
+ * block-code variant is an fp32 vector). */
+ORC_API void orc_hash_encode_f32(const float* x, const float* W, uint32_t n, uint32_t dim,
+                                 uint32_t bits, uint8_t* codes)
+{
+    const uint32_t nbytes = bits / 8;
+    for (uint32_t i = 0; i < n; ++i) {
+        for (uint32_t b = 0; b < nbytes; ++b) {
+            uint8_t byte = 0;
+            for (uint32_t j = 0; j < 8; ++j) {
+                double acc = 0.0;
+                for (uint32_t d = 0; d < dim; ++d) {
+                    acc += (double)x[(size_t)i * dim + d] * (double)W[(size_t)d * bits + 8 * b + j];
+                }
+                if (acc > 0.0) { byte |= (uint8_t)(1u << j); }
+            }
+            codes[(size_t)i * nbytes + b] = byte;
+        }
+    }
+}
+
+/*
+ * Per (block, kv head, bit) column sums of the +-1 token codes,
+ * S = #ones - #zeros over the block's tokens: the quantity both block scores
+ * are functions of.  token_codes is [n_blocks][block_size][kv_heads][nbytes]
+ * (cache order), out is int16 [n_blocks][kv_heads][nbytes*8].
+ */
+ORC_API void orc_hash_colsum(const uint8_t* token_codes, uint32_t n_blocks, uint32_t block_size,
+                             uint32_t kv_heads, uint32_t nbytes, int16_t* out)
+{
+    for (uint32_t n = 0; n < n_blocks; ++n) {
+        for (uint32_t h = 0; h < kv_heads; ++h) {
+            for (uint32_t c = 0; c < nbytes * 8; ++c) {
+                int32_t ones = 0;
+                for (uint32_t t = 0; t < block_size; ++t) {
+                    ones += (token_codes[(((size_t)n * block_size + t) * kv_heads + h) * nbytes + c / 8] >> (c % 8)) & 1u;
+                }
+                out[((size_t)n * kv_heads + h) * nbytes * 8 + c] = (int16_t)(2 * ones - (int32_t)block_size);
+            }
+        }
+    }
+}
+
 static int32_t orc_popcount_xor(const uint8_t* a, const uint8_t* b, uint32_t nbytes)
 {
     int32_t h = 0;

@@ -1,0 +1,135 @@
+"""Hash-code retrieval (KvComp style) against the oracle: token codes, block
+summaries, query codes, both integer block scores and the selection.  All
+results are integers / bit strings, so every comparison is exact."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def i32(x, dev):
+    return torch.tensor(np.asarray(x), dtype=torch.int32, device=dev)
+
+
+def bf16_dev(bits_u16, dev):
+    return torch.from_numpy(np.ascontiguousarray(bits_u16).view(np.int16)).to(dev).view(torch.bfloat16)
+
+
+def make_weights(seed):
+    """N(0, 2^2) weights in bf16, as HashEncoder draws them (hash_encoder.py:65-71)."""
+    bits = synth.bf16_round_bits(synth.normal_f32(seed, (128, 128)) * np.float32(2.0))
+    return bits, synth.bf16_widen(bits)
+
+
+@pytest.mark.parametrize("hkv,bs", [(8, 128), (2, 16), (4, 64), (1, 32)])
+def test_hash_encode_blocks(ucm, dev, hkv, bs):
+    from ucm_amd import ops
+
+    n_layers, nb, rows = 2, 9, 12
+    w_bits, w_f32 = make_weights(800)
+    caches_h = [synth.normal_bf16_bits(801 + l, (nb, bs, hkv, 128)) for l in range(n_layers)]
+    # adversarial rows: exact cancellation (projection exactly 0 -> bit 0), near cancellation, huge dynamic range
+    w2 = w_f32.copy()
+    for l in range(n_layers):
+        c = caches_h[l]
+        c[0, 0, 0, :] = 0
+        c[0, 1, 0, :] = 0
+        c[0, 1, 0, 5] = synth.bf16_round_bits(np.array([3.0], np.float32))[0]
+        big = synth.bf16_round_bits(np.array([1.0e4, -1.0e4, 1.0e-4], np.float32))
+        c[1, 2, 0, :3] = big
+        c[2, 3, 0, :] = c[2, 4, 0, :] ^ np.uint16(0x8000)  # exact negation of another row
+    caches = [bf16_dev(c, dev) for c in caches_h]
+    lp = ops.LayerPointers(caches)
+    ids = synth.permutation(810, nb)[:7]
+    slots = synth.permutation(811, rows)[:7]
+    colsum = torch.full((n_layers, rows, hkv, 128), 77, dtype=torch.int16, device=dev)
+    bcodes = torch.full((n_layers, rows, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    tcodes = torch.full((n_layers, rows, bs, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_blocks(lp, i32(ids, dev), i32(slots, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv, nb,
+                           colsum, bcodes, token_codes=tcodes)
+    torch.cuda.synchronize()
+    got_t, got_s, got_b = tcodes.cpu().numpy(), colsum.cpu().numpy(), bcodes.cpu().numpy()
+    for l in range(n_layers):
+        want_t = O.hash_encode(caches_h[l][ids], w2)                # [7, bs, hkv, 16]
+        assert np.array_equal(got_t[l][slots], want_t), l
+        assert np.array_equal(got_s[l][slots], O.hash_colsum(want_t)), l
+        assert np.array_equal(got_b[l][slots], O.hash_majority(want_t)), l
+        rest = np.setdiff1d(np.arange(rows), slots)
+        assert np.all(got_t[l][rest] == 0xEE) and np.all(got_s[l][rest] == 77) and np.all(got_b[l][rest] == 0xEE)
+    # the all-zero vector projects to exactly 0 everywhere: every bit is 0
+    s0 = slots[list(ids).index(0)] if 0 in ids else None
+    if s0 is not None:
+        assert not got_t[0][s0, 0, 0].any()
+    # without the token codes the summaries are the same
+    colsum2, bcodes2 = torch.zeros_like(colsum), torch.zeros_like(bcodes)
+    ops.hash_encode_blocks(lp, i32(ids, dev), i32(slots, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv, nb,
+                           colsum2, bcodes2)
+    assert torch.equal(colsum2[:, torch.from_numpy(slots.astype(np.int64)).to(dev)],
+                       colsum[:, torch.from_numpy(slots.astype(np.int64)).to(dev)])
+
+
+def test_hash_queries_scores_and_selection(ucm, dev):
+    """Config-5 shape in small: ragged batch, 8 kv heads, 32 query heads, 2 layers."""
+    from ucm_amd import ops
+
+    n_layers, hq, hkv, bs = 2, 32, 8, 128
+    lens = np.array([5, 33, 1, 64, 17, 3], np.int32)
+    rows = int(lens.sum())
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    w_bits, w_f32 = make_weights(820)
+    g = torch.Generator(device=dev)
+    g.manual_seed(821)
+    caches = [torch.randn(rows, bs, hkv, 128, device=dev, generator=g).to(torch.bfloat16) for _ in range(n_layers)]
+    lp = ops.LayerPointers(caches)
+    colsum = torch.zeros((n_layers, rows, hkv, 128), dtype=torch.int16, device=dev)
+    bcodes = torch.zeros((n_layers, rows, hkv, 16), dtype=torch.uint8, device=dev)
+    tcodes = torch.zeros((n_layers, rows, bs, hkv, 16), dtype=torch.uint8, device=dev)
+    wd = bf16_dev(w_bits, dev)
+    ops.hash_encode_blocks(lp, None, None, rows, wd, bs, hkv, rows, colsum, bcodes, token_codes=tcodes)
+    q_h = synth.normal_bf16_bits(822, (n_layers, len(lens) + 2, hq, 128))
+    q_rows = np.array([3, 0, 7, 1, 2, 5], np.int32)
+    q_codes = torch.zeros((n_layers, len(lens), hq, 16), dtype=torch.uint8, device=dev)
+    q_sum = torch.zeros((n_layers, len(lens), 128), dtype=torch.int16, device=dev)
+    qbar = torch.zeros((n_layers, len(lens), hkv, 16), dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(bf16_dev(q_h, dev), wd, hkv, q_codes, q_sum, qbar, len(lens), q_rows=i32(q_rows, dev))
+    torch.cuda.synchronize()
+    tc = tcodes.cpu().numpy()
+    for l in range(n_layers):
+        kc = caches[l].view(torch.int16).cpu().numpy().view(np.uint16)
+        assert np.array_equal(tc[l], O.hash_encode(kc, w_f32)), l
+        want_q = O.hash_encode(q_h[l][q_rows], w_f32)
+        assert np.array_equal(q_codes[l].cpu().numpy(), want_q)
+        pm = np.unpackbits(want_q, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
+        assert np.array_equal(q_sum[l].cpu().numpy(), pm.sum(1))
+        qm = np.stack([O.q_head_mean(synth.bf16_widen(q_h[l][r]), hkv) for r in q_rows])
+        assert np.array_equal(qbar[l].cpu().numpy(), O.hash_encode_f32(qm, w_f32))
+
+    for mode, rnd in ((ops.HASH_SCORE_SUM, False), (ops.HASH_SCORE_SUM, True), (ops.HASH_SCORE_BLOCK_CODE, False)):
+        scores = torch.full((n_layers, rows), -1.0, device=dev)
+        ops.hash_score_blocks(mode, q_sum, qbar, colsum, bcodes, i32(off, dev), i32(lens, dev), rows, scores,
+                              round_fp16=rnd)
+        topk = np.array([max(2, n // 3) + 2 for n in lens], np.int32)
+        idx = torch.full((n_layers, len(lens), int(lens.max())), -1, dtype=torch.int32, device=dev)
+        cnt = torch.zeros((n_layers, len(lens)), dtype=torch.int32, device=dev)
+        # KvComp keeps the first block and the last one out of the candidates (kvcomp.py:219-221)
+        ops.topk_windows(scores, i32(off, dev), i32(lens, dev), i32(topk, dev), int(lens.max()), idx, cnt,
+                         start_w=1, end_w=1)
+        torch.cuda.synchronize()
+        sc = scores.cpu().numpy()
+        for l in range(n_layers):
+            for r, n in enumerate(lens):
+                a = off[r]
+                if mode == ops.HASH_SCORE_SUM:
+                    key_codes = tc[l][a : a + n].transpose(0, 2, 1, 3)      # [n, hkv, bs, 16] as the reference stores them
+                    want = O.hash_scores_sum(q_codes[l, r].cpu().numpy(), key_codes).astype(np.float32)
+                    if rnd:
+                        want = want.astype(np.float16).astype(np.float32)
+                else:
+                    want = O.hash_scores_block(qbar[l, r].cpu().numpy(), bcodes[l, a : a + n].cpu().numpy()).astype(np.float32)
+                assert np.array_equal(sc[l, a : a + n], want), (mode, rnd, l, r)
+                sel = O.topk_windows(want, int(topk[r]), 1, 1)
+                assert cnt[l, r] == len(sel) and np.array_equal(idx[l, r, : len(sel)].cpu().numpy(), sel), (mode, l, r)

@@ -164,6 +164,61 @@ def esa_retrieve(data: torch.Tensor, q: torch.Tensor, indexes: torch.Tensor, top
               out_idx.shape[1], _stream() if stream is None else stream)
 
 
+HASH_SCORE_SUM, HASH_SCORE_BLOCK_CODE = 0, 1
+
+
+def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                       n: int, w: torch.Tensor, block_size: int, kv_heads: int, num_blocks: int,
+                       colsum: torch.Tensor, block_codes: torch.Tensor,
+                       token_codes: Optional[torch.Tensor] = None) -> None:
+    """w bf16 [128, 128]; colsum int16 [L, rows, kv_heads, 128]; block_codes uint8 [L, rows, kv_heads, 16];
+    token_codes uint8 [L, rows, block_size, kv_heads, 16] or None."""
+    if w.shape != (128, 128):
+        raise ValueError("w must be [128, 128] bfloat16")
+    n_layers, rows = colsum.shape[0], colsum.shape[1]
+    if colsum.shape != (n_layers, rows, kv_heads, 128) or block_codes.shape != (n_layers, rows, kv_heads, 16):
+        raise ValueError("colsum [L,rows,Hkv,128] / block_codes [L,rows,Hkv,16] expected")
+    if n_layers != len(k_layers):
+        raise ValueError("one output layer per cache layer")
+    if token_codes is not None and token_codes.shape != (n_layers, rows, block_size, kv_heads, 16):
+        raise ValueError("token_codes must be [L, rows, block_size, kv_heads, 16]")
+    _lib.call("ucm_hash_encode_blocks", k_layers.ptr(), n_layers, num_blocks, _opt(block_ids, torch.int32, "block_ids"),
+              _opt(slots, torch.int32, "slots"), n, block_size, kv_heads, 128, _dev(w, torch.bfloat16, "w"), 128, rows,
+              _opt(token_codes, torch.uint8, "token_codes"), 0 if token_codes is None else token_codes.stride(0),
+              _dev(colsum, torch.int16, "colsum"), colsum.stride(0), _dev(block_codes, torch.uint8, "block_codes"),
+              block_codes.stride(0), _stream())
+
+
+def hash_encode_queries(q: torch.Tensor, w: torch.Tensor, kv_heads: int, q_codes: torch.Tensor, q_sum: torch.Tensor,
+                        qbar_codes: torch.Tensor, n_req: int, q_rows: Optional[torch.Tensor] = None) -> None:
+    """q bf16 [L, rows, q_heads, 128]; q_codes u8 [L, n_req, q_heads, 16]; q_sum int16 [L, n_req, 128];
+    qbar_codes u8 [L, n_req, kv_heads, 16]."""
+    n_layers, _, q_heads, d = q.shape
+    if q_codes.shape != (n_layers, n_req, q_heads, 16) or q_sum.shape != (n_layers, n_req, 128) \
+            or qbar_codes.shape != (n_layers, n_req, kv_heads, 16):
+        raise ValueError("query code outputs have the wrong shape")
+    if q_rows is None and q.shape[1] < n_req:
+        raise ValueError("q has fewer rows than requests")
+    _lib.call("ucm_hash_encode_queries", _dev(q, torch.bfloat16, "q"), q.stride(0), _opt(q_rows, torch.int32, "q_rows"),
+              n_req, n_layers, q_heads, kv_heads, d, _dev(w, torch.bfloat16, "w"), 128,
+              _dev(q_codes, torch.uint8, "q_codes"), _dev(q_sum, torch.int16, "q_sum"),
+              _dev(qbar_codes, torch.uint8, "qbar_codes"), _stream())
+
+
+def hash_score_blocks(mode: int, q_sum: torch.Tensor, qbar_codes: torch.Tensor, colsum: torch.Tensor,
+                      block_codes: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, total_blocks: int,
+                      scores: torch.Tensor, round_fp16: bool = False) -> None:
+    n_layers, rows, kv_heads, _ = colsum.shape
+    n_req = seg_off.numel()
+    if scores.dim() != 2 or scores.shape[0] != n_layers or scores.shape[1] < rows:
+        raise ValueError("scores must be [L, >= rows]")
+    _lib.call("ucm_hash_score_blocks", mode, _dev(q_sum, torch.int16, "q_sum"), _dev(qbar_codes, torch.uint8, "qbar_codes"),
+              _dev(colsum, torch.int16, "colsum"), colsum.stride(0), _dev(block_codes, torch.uint8, "block_codes"),
+              block_codes.stride(0), _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
+              n_req, total_blocks, n_layers, kv_heads, 128, _dev(scores, torch.float32, "scores"), scores.stride(0),
+              int(round_fp16), _stream())
+
+
 def copy_batch(dst_ptrs: torch.Tensor, src_ptrs: torch.Tensor, size: int) -> None:
     """dst_ptrs/src_ptrs: int64 device tensors of raw addresses; copies size bytes each."""
     if dst_ptrs.numel() != src_ptrs.numel():
