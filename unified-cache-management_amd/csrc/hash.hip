@@ -227,51 +227,74 @@ __global__ __launch_bounds__(kThreads) void hash_encode_blocks_kernel(
     }
 }
 
-// Query side, one workgroup per (request, layer): codes of every query head
-// (exact fp64 projection, there are only q_heads*128 of them), their +-1 sum
-// Q[c] over all heads, and the code of each kv head's group-mean query.
-// grid: x = request, y = layer; 128 threads = one per code bit
-__global__ __launch_bounds__(kBits) void hash_query_kernel(
+// Query side, one workgroup of 1024 threads per (request, layer): thread
+// (bit c, head group hg) projects heads hg, hg+8, ... exactly (fp64, d
+// ascending; there are only q_heads*128 such dot products), the +-1 sum over
+// all heads is combined through LDS, and each head group also produces the code
+// of the group-mean query of kv heads hg, hg+8, ...  W and the request's query
+// rows are staged in LDS once.
+// grid: x = request, y = layer
+constexpr int kQueryGroups = 8;
+constexpr int kQueryThreads = kBits * kQueryGroups;
+constexpr int kMaxQHeads = 128;
+
+__global__ __launch_bounds__(kQueryThreads) void hash_query_kernel(
     const unsigned short* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows,
     unsigned q_heads, unsigned kv_heads, const unsigned short* __restrict__ w, unsigned n_req,
     unsigned* __restrict__ q_codes /*[L][n_req][q_heads][4]*/, short* __restrict__ q_sum /*[L][n_req][128]*/,
     unsigned* __restrict__ qbar_codes /*[L][n_req][kv_heads][4]*/)
 {
-    const unsigned r = blockIdx.x, l = blockIdx.y, c = threadIdx.x;
+    __shared__ unsigned short w_s[kDim * kBits];            // [d][c]: lanes read consecutive c
+    __shared__ unsigned short q_s[kMaxQHeads * kDim];
+    __shared__ int part[kQueryGroups][kBits];
+
+    const unsigned r = blockIdx.x, l = blockIdx.y;
+    const unsigned c = threadIdx.x % kBits, hg = threadIdx.x / kBits;
     const unsigned short* qp = q + static_cast<int64_t>(l) * q_layer_stride +
                                static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kDim;
+    for (unsigned e = threadIdx.x; e < kDim * kBits; e += kQueryThreads) { w_s[e] = w[e]; }
+    for (unsigned e = threadIdx.x; e < q_heads * kDim; e += kQueryThreads) { q_s[e] = qp[e]; }
+    __syncthreads();
+
     const size_t lr = static_cast<size_t>(l) * n_req + r;
     const unsigned g = q_heads / kv_heads;
     int sum = 0;
-    for (unsigned i = 0; i < q_heads; ++i) {
+    for (unsigned i = hg; i < q_heads; i += kQueryGroups) {
         double acc = 0.0;
         for (int d = 0; d < kDim; ++d) {
-            acc += static_cast<double>(bf16_to_f32(qp[i * kDim + d])) * static_cast<double>(bf16_to_f32(w[d * kBits + c]));
+            acc += static_cast<double>(bf16_to_f32(q_s[i * kDim + d])) * static_cast<double>(bf16_to_f32(w_s[d * kBits + c]));
         }
         const bool pos = acc > 0.0;
         sum += pos ? 1 : -1;
-        const unsigned long long m = __ballot(pos);      // two waves: bits 0-63 and 64-127
+        const unsigned long long m = __ballot(pos);      // a wave covers 64 consecutive bits of one head
         if ((c & 63) == 0) {
             q_codes[(lr * q_heads + i) * 4 + (c >> 6) * 2] = static_cast<unsigned>(m);
             q_codes[(lr * q_heads + i) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(m >> 32);
         }
     }
-    q_sum[lr * kBits + c] = static_cast<short>(sum);
+    part[hg][c] = sum;
     // group-mean query: fp32 sequential adds * (1/g), the scoring path's own mean, then projected exactly
     const float inv = 1.0f / static_cast<float>(g);
-    for (unsigned h = 0; h < kv_heads; ++h) {
+    for (unsigned h = hg; h < kv_heads; h += kQueryGroups) {
         double acc = 0.0;
         for (int d = 0; d < kDim; ++d) {
-            float m = bf16_to_f32(qp[(h * g) * kDim + d]);
-            for (unsigned j = 1; j < g; ++j) { m = m + bf16_to_f32(qp[(h * g + j) * kDim + d]); }
+            float m = bf16_to_f32(q_s[(h * g) * kDim + d]);
+            for (unsigned j = 1; j < g; ++j) { m = m + bf16_to_f32(q_s[(h * g + j) * kDim + d]); }
             if (g != 1) { m = m * inv; }
-            acc += static_cast<double>(m) * static_cast<double>(bf16_to_f32(w[d * kBits + c]));
+            acc += static_cast<double>(m) * static_cast<double>(bf16_to_f32(w_s[d * kBits + c]));
         }
         const unsigned long long mk = __ballot(acc > 0.0);
         if ((c & 63) == 0) {
             qbar_codes[(lr * kv_heads + h) * 4 + (c >> 6) * 2] = static_cast<unsigned>(mk);
             qbar_codes[(lr * kv_heads + h) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(mk >> 32);
         }
+    }
+    __syncthreads();
+    if (hg == 0) {
+        int total = 0;
+#pragma unroll
+        for (int k = 0; k < kQueryGroups; ++k) { total += part[k][c]; }
+        q_sum[lr * kBits + c] = static_cast<short>(total);
     }
 }
 
@@ -281,48 +304,64 @@ __device__ __forceinline__ float half_round(float x)
     return static_cast<float>(static_cast<_Float16>(x));
 }
 
-// grid: x = 64 representative rows of the ragged batch (dense numbering), y = layer; one thread per block
+typedef short i16x8 __attribute__((ext_vector_type(8)));
+
+// Integer block scores.  Sixteen lanes share one block: in mode 0 lane j owns
+// bits 8j..8j+7 of the 128-entry column-sum row (one 16-byte load per kv head,
+// 256 contiguous bytes per 16 lanes), in mode 1 lanes 0..kv_heads*4-1 each own
+// one 32-bit word of the block code; a 16-lane DPP-free shuffle reduction adds
+// the partial scores.  Requests are found by a scan of the segment lengths
+// (they are few; rows are many).
+// grid: x = 16 rows of the ragged batch (dense numbering), y = layer; 256 threads
 template <int kMode>
-__global__ __launch_bounds__(64) void hash_score_kernel(
+__global__ __launch_bounds__(256) void hash_score_kernel(
     const short* __restrict__ q_sum, const unsigned* __restrict__ qbar_codes,
     const short* __restrict__ colsum, int64_t cs_layer_stride, const unsigned* __restrict__ block_codes,
     int64_t bc_layer_stride, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
     unsigned n_req, unsigned kv_heads, float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16)
 {
-    // owner request of dense row index: linear scan (requests are few, rows are many)
     const unsigned l = blockIdx.y;
-    int dense = blockIdx.x * 64 + threadIdx.x;
+    const unsigned sub = threadIdx.x & 15;
+    int dense = blockIdx.x * 16 + (threadIdx.x >> 4);
     int r = -1, local = 0;
     for (unsigned i = 0; i < n_req; ++i) {
         const int n = max(seg_len[i], 0);
         if (dense < n) { r = static_cast<int>(i); local = dense; break; }
         dense -= n;
     }
-    if (r < 0) { return; }
-    const int64_t row = static_cast<int64_t>(seg_off[r]) + local;
-    const size_t lr = static_cast<size_t>(l) * n_req + r;
     int score = 0;
-    if (kMode == 0) {
-        // <sum_i u(q_i), sum_h S[h]>
-        const short* cs = colsum + static_cast<int64_t>(l) * cs_layer_stride + row * kv_heads * kBits;
-        const short* qs = q_sum + lr * kBits;
-        for (int c = 0; c < kBits; ++c) {
-            int s = 0;
-            for (unsigned h = 0; h < kv_heads; ++h) { s += cs[h * kBits + c]; }
-            score += static_cast<int>(qs[c]) * s;
-        }
-    } else {
-        // sum over kv heads of (bits - hamming(code of the group-mean query, majority code of the block))
-        const unsigned* bc = block_codes + static_cast<int64_t>(l) * bc_layer_stride + row * kv_heads * 4;
-        const unsigned* qc = qbar_codes + lr * kv_heads * 4;
-        for (unsigned h = 0; h < kv_heads; ++h) {
+    int64_t row = 0;
+    if (r >= 0) {
+        row = static_cast<int64_t>(seg_off[r]) + local;
+        const size_t lr = static_cast<size_t>(l) * n_req + r;
+        if (kMode == 0) {
+            // <sum_i u(q_i), sum_h S[h]>
+            const short* cs = colsum + static_cast<int64_t>(l) * cs_layer_stride + row * kv_heads * kBits + sub * 8;
+            const i16x8 qv = *reinterpret_cast<const i16x8*>(q_sum + lr * kBits + sub * 8);
+            int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (unsigned h = 0; h < kv_heads; ++h) {
+                const i16x8 v = *reinterpret_cast<const i16x8*>(cs + h * kBits);
 #pragma unroll
-            for (int wd = 0; wd < 4; ++wd) { score += 32 - __popc(bc[h * 4 + wd] ^ qc[h * 4 + wd]); }
+                for (int k = 0; k < 8; ++k) { s[k] += v[k]; }
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { score += static_cast<int>(qv[k]) * s[k]; }
+        } else {
+            // sum over kv heads of (bits - hamming(code of the group-mean query, majority code of the block))
+            const unsigned* bc = block_codes + static_cast<int64_t>(l) * bc_layer_stride + row * kv_heads * 4;
+            const unsigned* qc = qbar_codes + lr * kv_heads * 4;
+            for (unsigned wd = sub; wd < kv_heads * 4; wd += 16) { score += 32 - __popc(bc[wd] ^ qc[wd]); }
         }
     }
-    float f = static_cast<float>(score);
-    if (round_fp16) { f = half_round(f); }
-    scores[static_cast<int64_t>(l) * scores_layer_stride + row] = f;
+    score += __shfl_xor(score, 8, 16);
+    score += __shfl_xor(score, 4, 16);
+    score += __shfl_xor(score, 2, 16);
+    score += __shfl_xor(score, 1, 16);
+    if (r >= 0 && sub == 0) {
+        float f = static_cast<float>(score);
+        if (round_fp16) { f = half_round(f); }
+        scores[static_cast<int64_t>(l) * scores_layer_stride + row] = f;
+    }
 }
 
 }  // namespace
@@ -366,9 +405,10 @@ extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_strid
     if (n_req == 0) { return UCM_OK; }
     UCM_REQUIRE(q_bf16 && w_bf16 && q_codes && q_sum && qbar_codes, "ucm_hash_encode_queries: null pointer");
     UCM_SUPPORTED(head_dim == kDim && bits == kBits, "ucm_hash_encode_queries: head_dim=%d bits=%d (128 and 128)", head_dim, bits);
-    UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0 && q_heads <= 1024,
+    UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0,
                 "ucm_hash_encode_queries: q_heads=%d kv_heads=%d", q_heads, kv_heads);
-    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kBits), 0, ucm::as_stream(stream),
+    UCM_SUPPORTED(q_heads <= kMaxQHeads, "ucm_hash_encode_queries: q_heads=%d (at most %d)", q_heads, kMaxQHeads);
+    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),
                        static_cast<const unsigned short*>(q_bf16), q_layer_stride, q_rows,
                        static_cast<unsigned>(q_heads), static_cast<unsigned>(kv_heads),
                        static_cast<const unsigned short*>(w_bf16), static_cast<unsigned>(n_req),
@@ -390,16 +430,16 @@ extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8
     UCM_REQUIRE(seg_off && seg_len && scores, "ucm_hash_score_blocks: null pointer");
     UCM_REQUIRE(mode == 0 ? (q_sum && colsum) : (qbar_codes && block_codes), "ucm_hash_score_blocks: null operand for this mode");
     UCM_SUPPORTED(bits == kBits && kv_heads >= 1 && kv_heads <= kMaxHeads, "ucm_hash_score_blocks: bits=%d kv_heads=%d", bits, kv_heads);
-    const unsigned gx = static_cast<unsigned>((total_blocks + 63) / 64);
+    const unsigned gx = static_cast<unsigned>((total_blocks + 15) / 16);
     hipStream_t s = ucm::as_stream(stream);
     if (mode == 0) {
-        hipLaunchKernelGGL(hash_score_kernel<0>, dim3(gx, n_layers), dim3(64), 0, s, q_sum,
+        hipLaunchKernelGGL(hash_score_kernel<0>, dim3(gx, n_layers), dim3(256), 0, s, q_sum,
                            reinterpret_cast<const unsigned*>(qbar_codes), colsum, colsum_layer_stride,
                            reinterpret_cast<const unsigned*>(block_codes), block_codes_layer_stride / 4, seg_off, seg_len,
                            static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores, scores_layer_stride,
                            round_fp16);
     } else {
-        hipLaunchKernelGGL(hash_score_kernel<1>, dim3(gx, n_layers), dim3(64), 0, s, q_sum,
+        hipLaunchKernelGGL(hash_score_kernel<1>, dim3(gx, n_layers), dim3(256), 0, s, q_sum,
                            reinterpret_cast<const unsigned*>(qbar_codes), colsum, colsum_layer_stride,
                            reinterpret_cast<const unsigned*>(block_codes), block_codes_layer_stride / 4, seg_off, seg_len,
                            static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores, scores_layer_stride,
