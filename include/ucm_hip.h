@@ -165,6 +165,34 @@ int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
                      ucm_stream_t stream);
 
 /*
+ * Delta loads: decides, per (layer, request), which staging slots keep their
+ * block and which missing block of the new selection goes where - the
+ * "load delta" of ReqStatePerLayer.wait_retrieval_and_start_load
+ * (ucm/sparse/esa/esa.py:312-338; the hit / miss / evict sets of
+ * GSAPrefetchEngineC::GetHitAndMissBlock, ucm/sparse/gsa/prefetch/src/kvcache_pre.cpp:206-238)
+ * computed on the device from ucm_topk_windows' output.  A block is identified
+ * by its logical index within the request.
+ *   sel, sel_phys  dev int32 [n_layers][n_req][sel_stride]: selected logical
+ *                  blocks and their cache block ids (idx_out / phys_out)
+ *   count          dev int32 [n_layers][n_req]: entries of sel that are valid
+ *   resident       dev int32 [n_layers][n_req][n_slots], in/out: logical block
+ *                  held by each staging slot, -1 = empty
+ *   load_phys      dev int32 [n_layers][n_req][n_slots], out: cache block id to
+ *                  copy into the slot, -1 = slot untouched.  It is exactly the
+ *                  `phys` argument of ucm_kv_gather_selected (count = n_slots),
+ *                  which skips the -1 entries.
+ *   slot_of_sel    dev int32, layout of sel, out: staging slot that holds each
+ *                  selected block after the load (the sparse block table)
+ *   miss_count     dev int32 [n_layers][n_req], out: blocks to load
+ * The i-th missing block (ascending) goes to the i-th freed slot (ascending);
+ * the reference pairs them in set order, which is unspecified.  At most 64
+ * slots per request and layer; selections longer than n_slots are cut there.
+ */
+int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req,
+                   int n_layers, int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys,
+                   int32_t* slot_of_sel, int32_t* miss_count, ucm_stream_t stream);
+
+/*
  * Hash-code retrieval (KvComp).  A vector's code has bit c = (x . W[:, c] > 0),
  * packed LSB first (bit j of byte b is column 8b+j) - HashEncoder.compute_hash
  * (ucm/sparse/kvcomp/hash_encoder.py:99-157, bit order :92-97,139-149; W is

@@ -69,6 +69,7 @@ _orc_block_table_gather = _sig(_orc, "orc_block_table_gather", _i32, _p, _p, _i3
 _orc_get_offset = _sig(_orc, "orc_get_offset", _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i64, C.c_int, C.c_int)
 _orc_kv_move_blocks = _sig(_orc, "orc_kv_move_blocks", None, _p, _u32, C.c_size_t, C.c_size_t, _p, _u32, _p, C.c_int)
 _orc_kv_gather_selected = _sig(_orc, "orc_kv_gather_selected", None, _p, _u32, C.c_size_t, C.c_size_t, _p, _p, _u32, _u32, _p, _p, _p)
+_orc_delta_plan = _sig(_orc, "orc_delta_plan", _i32, _p, _p, _i32, _p, _i32, _p, _p)
 _orc_hash_encode = _sig(_orc, "orc_hash_encode", None, _p, _p, _u32, _u32, _u32, _p)
 _orc_hash_encode_f32 = _sig(_orc, "orc_hash_encode_f32", None, _p, _p, _u32, _u32, _u32, _p)
 _orc_hash_colsum = _sig(_orc, "orc_hash_colsum", None, _p, _u32, _u32, _u32, _u32, _p)
@@ -225,6 +226,16 @@ def kv_gather_selected(layers, kv_stride, block_bytes, phys, count, dst_off, reg
     do, rk = _c(dst_off, np.int64), _c(region_k, np.int32)
     _orc_kv_gather_selected(_layer_ptrs(layers), n_layers, kv_stride, block_bytes, _ptr(ph), _ptr(ct), n_req,
                             stride, _ptr(do), _ptr(rk), _ptr(staging))
+
+
+def delta_plan(sel, sel_phys, resident):
+    """One (layer, request): returns (load_phys [n_slots], slot_of_sel [len(sel)], moved); resident is updated in place."""
+    s, sp = _c(sel, np.int32), _c(sel_phys, np.int32)
+    assert resident.dtype == np.int32 and resident.flags.c_contiguous
+    load = np.empty(len(resident), np.int32)
+    slot_of = np.full(max(len(s), 1), -1, np.int32)
+    moved = _orc_delta_plan(_ptr(s), _ptr(sp), len(s), _ptr(resident), len(resident), _ptr(load), _ptr(slot_of))
+    return load, slot_of[: len(s)], int(moved)
 
 
 def hash_encode(x_bits: np.ndarray, w: np.ndarray) -> np.ndarray:

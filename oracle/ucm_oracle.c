@@ -481,6 +481,49 @@ ORC_API void orc_kv_gather_selected(const uint8_t* const* layers, uint32_t n_lay
     }
 }
 
+/*
+ * Delta of a new selection against what a request's staging slots hold
+ * (ucm/sparse/esa/esa.py:312-338: blocks of the new selection that are already
+ * resident stay where they are, the others are loaded into the slots whose
+ * block is no longer wanted).  Blocks are logical indices; `resident` is
+ * updated in place (-1 = empty).  The reference pairs missing blocks and freed
+ * slots in set-iteration order; here the i-th missing block (in selection
+ * order) takes the i-th freed slot (ascending).  load_phys[j] = cache block to
+ * copy into slot j or -1; slot_of_sel[i] = slot holding sel[i] afterwards (-1
+ * if it found no slot).  Returns the number of blocks to load.
+ */
+ORC_API int32_t orc_delta_plan(const int32_t* sel, const int32_t* sel_phys, int32_t count,
+                               int32_t* resident, int32_t n_slots, int32_t* load_phys,
+                               int32_t* slot_of_sel)
+{
+    const int32_t k = count < n_slots ? count : n_slots;
+    int32_t* keep = (int32_t*)calloc((size_t)n_slots + 1, sizeof(int32_t));
+    for (int32_t i = 0; i < k; ++i) { slot_of_sel[i] = -1; }
+    for (int32_t j = 0; j < n_slots; ++j) {
+        load_phys[j] = -1;
+        for (int32_t i = 0; i < k; ++i) {
+            if (resident[j] >= 0 && resident[j] == sel[i]) { keep[j] = 1; slot_of_sel[i] = j; }
+        }
+    }
+    int32_t moved = 0, j = 0;
+    for (int32_t i = 0; i < k; ++i) {
+        if (slot_of_sel[i] >= 0) { continue; }
+        while (j < n_slots && keep[j]) { ++j; }
+        if (j == n_slots) { break; }
+        resident[j] = sel[i];
+        load_phys[j] = sel_phys[i];
+        slot_of_sel[i] = j;
+        keep[j] = 2;
+        ++moved;
+        ++j;
+    }
+    for (int32_t t = 0; t < n_slots; ++t) {
+        if (!keep[t]) { resident[t] = -1; }
+    }
+    free(keep);
+    return moved;
+}
+
 /* --------------------------------------------------------- a8 hash codes */
 
 /*

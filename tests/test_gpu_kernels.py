@@ -518,3 +518,65 @@ def test_config4_full_size_selection(ucm, dev):
         assert np.array_equal(cnt_h[l], wcnt), l
         for r in range(len(lens)):
             assert np.array_equal(idx_h[l, r, : wcnt[r]], widx[r, : wcnt[r]]), (l, r)
+
+
+def test_delta_plan_and_delta_gather(ucm, dev):
+    """Several decode steps of changing selections: the plan matches the oracle, only missing blocks move,
+    and after every step each request's staging slots hold exactly the selected blocks."""
+    from ucm_amd import ops
+
+    n_layers, n_req, n_slots, nb, bb, stride = 3, 5, 19, 300, 4096, 40
+    hs, ds = make_caches(dev, n_layers, nb, bb, 500)
+    lp = ops.LayerPointers(ds)
+    resident = torch.full((n_layers, n_req, n_slots), -1, dtype=torch.int32, device=dev)
+    res_h = np.full((n_layers, n_req, n_slots), -1, np.int32)
+    region = np.full(n_req, n_slots, np.int32)
+    dst_off = (np.arange(n_req, dtype=np.int64) * n_slots * n_layers * 2)
+    total = n_req * n_slots * n_layers * 2
+    staging = torch.zeros(total * bb, dtype=torch.uint8, device=dev)
+    tables = np.stack([synth.permutation(510 + r, nb)[:50] for r in range(n_req)]).astype(np.int32)   # logical -> cache block
+    slots_count = i32(np.full((n_layers, n_req), n_slots), dev)
+    rng = np.random.default_rng(12)
+    prev = None
+    for step in range(6):
+        cnt = rng.integers(0, n_slots + 1, (n_layers, n_req)).astype(np.int32)
+        cnt[0, 0] = n_slots
+        sel = np.full((n_layers, n_req, stride), -1, np.int32)
+        for l in range(n_layers):
+            for r in range(n_req):
+                if prev is not None and rng.random() < 0.7:       # mostly overlapping with the previous step
+                    base = set(prev[l, r][prev[l, r] >= 0].tolist())
+                    pool = list(base) + list(rng.permutation(50)[:6])
+                    pick = np.unique(np.array(pool))[: cnt[l, r]]
+                    rng.shuffle(pick)
+                    pick = np.sort(pick[: cnt[l, r]])
+                else:
+                    pick = np.sort(rng.permutation(50)[: cnt[l, r]])
+                cnt[l, r] = len(pick)
+                sel[l, r, : len(pick)] = pick
+        phys = np.where(sel >= 0, np.take_along_axis(np.broadcast_to(tables[None], (n_layers, n_req, 50)),
+                                                      np.maximum(sel, 0), axis=2), -1).astype(np.int32)
+        load = torch.full((n_layers, n_req, n_slots), -7, dtype=torch.int32, device=dev)
+        slot_of = torch.full((n_layers, n_req, stride), -7, dtype=torch.int32, device=dev)
+        miss = torch.full((n_layers, n_req), -7, dtype=torch.int32, device=dev)
+        ops.delta_plan(i32(sel, dev), i32(phys, dev), i32(cnt, dev), resident, load, slot_of, miss)
+        ops.kv_gather_selected(lp, nb * bb, bb, nb, load, slots_count, torch.from_numpy(dst_off).to(dev),
+                               i32(region, dev), n_slots, staging, total)
+        torch.cuda.synchronize()
+        load_h, slot_h, miss_h, st = load.cpu().numpy(), slot_of.cpu().numpy(), miss.cpu().numpy(), staging.cpu().numpy()
+        for l in range(n_layers):
+            for r in range(n_req):
+                k = int(cnt[l, r])
+                wl, ws, moved = O.delta_plan(sel[l, r, :k], phys[l, r, :k], res_h[l, r])
+                assert np.array_equal(load_h[l, r], wl) and miss_h[l, r] == moved, (step, l, r)
+                assert np.array_equal(slot_h[l, r, :k], ws), (step, l, r)
+                # every selected block is now in its slot, K and V
+                for i in range(k):
+                    for kv in range(2):
+                        o = (int(dst_off[r]) + (l * 2 + kv) * n_slots + int(ws[i])) * bb
+                        src = hs[l].reshape(2, nb, bb)[kv, phys[l, r, i]]
+                        assert np.array_equal(st[o : o + bb], src), (step, l, r, i, kv)
+        assert np.array_equal(resident.cpu().numpy(), res_h)
+        if step > 0:
+            assert miss_h.sum() < cnt.sum()        # overlapping selections really save loads
+        prev = sel

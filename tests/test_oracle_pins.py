@@ -289,3 +289,37 @@ def test_hash_closed_forms():
     q2 = rng.integers(0, 256, (2, 3), dtype=np.uint8)
     sim = (nbits - np.unpackbits(q2[None] ^ want_codes, axis=-1).sum(-1)).sum(-1)
     assert np.array_equal(O.hash_scores_block(q2, want_codes), sim)
+
+
+def test_delta_plan_against_set_arithmetic():
+    """The reference's delta load in terms of sets (esa.py:312-338): what stays is resident AND selected, what is
+    loaded is selected minus resident, and it goes into slots whose block is no longer selected."""
+    rng = np.random.default_rng(11)
+    for _ in range(500):
+        n_slots = int(rng.integers(1, 20))
+        k = int(rng.integers(0, n_slots + 3))
+        universe = int(rng.integers(max(k, 1), 60))
+        resident = rng.permutation(universe)[:n_slots].astype(np.int32)
+        resident = np.concatenate([resident, np.full(n_slots - len(resident), -1, np.int32)])
+        resident[rng.random(n_slots) < 0.2] = -1
+        before = resident.copy()
+        sel = np.sort(rng.permutation(universe)[:k]).astype(np.int32)
+        phys = (sel * 7 + 3).astype(np.int32)
+        load, slot_of, moved = O.delta_plan(sel, phys, resident)
+        kk = min(k, n_slots)
+        old, new = set(before[before >= 0].tolist()), set(sel[:kk].tolist())
+        assert moved == len(new - old)
+        assert set(load[load >= 0].tolist()) == {b * 7 + 3 for b in new - old}
+        for j in range(n_slots):
+            if before[j] in new:
+                assert load[j] == -1 and resident[j] == before[j]       # hit: untouched
+            elif load[j] >= 0:
+                assert resident[j] in (new - old) and load[j] == resident[j] * 7 + 3
+            else:
+                assert resident[j] == -1                                 # dropped and not refilled
+        assert set(resident[resident >= 0].tolist()) == new
+        for i in range(kk):
+            assert resident[slot_of[i]] == sel[i]
+        # misses fill freed slots in ascending order
+        filled = [j for j in range(n_slots) if load[j] >= 0]
+        assert [resident[j] for j in filled] == sorted(new - old)

@@ -160,3 +160,80 @@ extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride
 #undef UCM_TOPK_LAUNCH
     UCM_LAUNCH_CHECK("ucm_topk_windows");
 }
+
+// ---------------------------------------------------------------------------
+// Resident-set bookkeeping for delta loads: which of a request's staging slots
+// already hold a block of the new selection, and which missing block goes to
+// which freed slot.  One wave per (layer, request), slot j and selection entry
+// j in lane j; membership is a k-step broadcast compare, ranks are ballot
+// prefix counts, so the i-th missing block (ascending) lands in the i-th freed
+// slot (ascending) - a deterministic refinement of the reference's set
+// arithmetic (ucm/sparse/esa/esa.py:312-338).
+namespace {
+
+// grid: x = request, y = layer; block = one wave; n_slots <= 64
+__global__ __launch_bounds__(64) void delta_plan_kernel(
+    const int32_t* __restrict__ sel, const int32_t* __restrict__ sel_phys, const int32_t* __restrict__ count,
+    int n_req, int sel_stride, int32_t* __restrict__ resident, int n_slots, int32_t* __restrict__ load_phys,
+    int32_t* __restrict__ slot_of_sel, int32_t* __restrict__ miss_count)
+{
+    const int r = blockIdx.x, l = blockIdx.y, lane = threadIdx.x;
+    const size_t lr = static_cast<size_t>(l) * n_req + r;
+    const int k = min(count[lr], n_slots);          // selections beyond the slot budget cannot be resident
+    const int32_t* s = sel + lr * sel_stride;
+    const int32_t* sp = sel_phys + lr * sel_stride;
+    int32_t* res = resident + lr * n_slots;
+
+    const int my_sel = lane < k ? s[lane] : -1;
+    const int my_phys = lane < k ? sp[lane] : -1;
+    const int my_res = lane < n_slots ? res[lane] : -1;
+
+    // selection entry `lane` already resident?  slot `lane` still wanted?
+    bool hit = false, keep = false;
+    int hit_slot = -1;
+    for (int j = 0; j < 64; ++j) {
+        const int rj = __shfl(my_res, j, 64);
+        const int sj = __shfl(my_sel, j, 64);
+        if (j < n_slots && rj >= 0 && rj == my_sel && my_sel >= 0) { hit = true; hit_slot = j; }
+        if (j < k && sj >= 0 && sj == my_res && my_res >= 0) { keep = true; }
+    }
+    const bool miss = lane < k && !hit;
+    const bool freed = lane < n_slots && !keep;
+    const unsigned long long miss_mask = __ballot(miss), free_mask = __ballot(freed);
+    const int miss_rank = static_cast<int>(lanes_below(miss_mask));
+    const int free_rank = static_cast<int>(lanes_below(free_mask));
+
+    // the slot with free rank q receives the miss with miss rank q (exchanged through LDS)
+    __shared__ int32_t miss_sel[64], miss_phys[64], free_slot[64];
+    if (miss) { miss_sel[miss_rank] = my_sel; miss_phys[miss_rank] = my_phys; }
+    if (freed) { free_slot[free_rank] = lane; }
+    __syncthreads();
+    const int n_move = min(__popcll(miss_mask), __popcll(free_mask));
+    int dst_slot = hit_slot;
+    int take_sel = -1, take_phys = -1;
+    if (freed && free_rank < n_move) { take_sel = miss_sel[free_rank]; take_phys = miss_phys[free_rank]; }
+    if (miss && miss_rank < n_move) { dst_slot = free_slot[miss_rank]; }
+    if (lane < n_slots) {
+        load_phys[lr * n_slots + lane] = take_phys;              // -1: slot keeps what it holds
+        if (take_sel >= 0) { res[lane] = take_sel; }
+        else if (freed) { res[lane] = -1; }                      // block dropped, nothing to replace it
+    }
+    if (lane < k) { slot_of_sel[lr * sel_stride + lane] = dst_slot; }
+    if (lane == 0) { miss_count[lr] = n_move; }
+}
+
+}  // namespace
+
+extern "C" int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req,
+                              int n_layers, int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys,
+                              int32_t* slot_of_sel, int32_t* miss_count, ucm_stream_t stream)
+{
+    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_delta_plan: n_req=%d n_layers=%d", n_req, n_layers);
+    if (n_req == 0) { return UCM_OK; }
+    UCM_REQUIRE(sel && sel_phys && count && resident && load_phys && slot_of_sel && miss_count, "ucm_delta_plan: null pointer");
+    UCM_SUPPORTED(n_slots >= 1 && n_slots <= 64, "ucm_delta_plan: n_slots=%d (1..64 staging slots per request and layer)", n_slots);
+    UCM_REQUIRE(sel_stride >= 1, "ucm_delta_plan: sel_stride=%d", sel_stride);
+    hipLaunchKernelGGL(delta_plan_kernel, dim3(n_req, n_layers), dim3(64), 0, ucm::as_stream(stream), sel, sel_phys,
+                       count, n_req, sel_stride, resident, n_slots, load_phys, slot_of_sel, miss_count);
+    UCM_LAUNCH_CHECK("ucm_delta_plan");
+}

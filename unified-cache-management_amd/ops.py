@@ -164,6 +164,21 @@ def esa_retrieve(data: torch.Tensor, q: torch.Tensor, indexes: torch.Tensor, top
               out_idx.shape[1], _stream() if stream is None else stream)
 
 
+def delta_plan(sel: torch.Tensor, sel_phys: torch.Tensor, count: torch.Tensor, resident: torch.Tensor,
+               load_phys: torch.Tensor, slot_of_sel: torch.Tensor, miss_count: torch.Tensor) -> None:
+    """sel / sel_phys / slot_of_sel int32 [L, n_req, stride]; count / miss_count int32 [L, n_req];
+    resident / load_phys int32 [L, n_req, n_slots] (resident is updated in place)."""
+    n_layers, n_req, stride = sel.shape
+    if sel_phys.shape != sel.shape or slot_of_sel.shape != sel.shape or count.shape != (n_layers, n_req) \
+            or miss_count.shape != count.shape or resident.shape[:2] != (n_layers, n_req) \
+            or load_phys.shape != resident.shape:
+        raise ValueError("delta_plan: inconsistent shapes")
+    _lib.call("ucm_delta_plan", _dev(sel, torch.int32, "sel"), _dev(sel_phys, torch.int32, "sel_phys"),
+              _dev(count, torch.int32, "count"), n_req, n_layers, stride, _dev(resident, torch.int32, "resident"),
+              resident.shape[2], _dev(load_phys, torch.int32, "load_phys"),
+              _dev(slot_of_sel, torch.int32, "slot_of_sel"), _dev(miss_count, torch.int32, "miss_count"), _stream())
+
+
 HASH_SCORE_SUM, HASH_SCORE_BLOCK_CODE = 0, 1
 
 
