@@ -8,9 +8,11 @@
 // Only the SIGN of each projection is kept, and it has to be the sign of the
 // exactly accumulated dot product (the CPU oracle accumulates in fp64), so
 // every result whose magnitude is within the fp32 accumulation error bound
-//     |acc| <= 2^-15 * ||x|| * ||w_c||
+//     |acc| < 2^-15 * ||x|| * ||w_c||
 // is queued and redone by one lane in fp64, d ascending; a few bits per ten
-// thousand take that path.
+// thousand take that path (a one-compare filter with the tile's largest row
+// norm flags column blocks; only flagged ones get the per-row look).  The next tile's
+// keys are in flight while the current one goes through the matrix cores.
 //
 // Per cache block the kernel emits: the token codes (LSB-first packing: bit j
 // of byte b is column 8b+j), the per-(kv head, bit) column sums over the
@@ -35,28 +37,74 @@ constexpr int kQueueCap = 256;
 constexpr int kMaxHeads = 8;
 constexpr float kTau2 = 0x1p-30f;   // (2^-15)^2
 
+__device__ __forceinline__ unsigned lanes_below(unsigned long long mask)
+{
+    return __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
+}
+
 __device__ __forceinline__ float bf16_to_f32(unsigned short h) { return __uint_as_float(static_cast<unsigned>(h) << 16); }
 
 struct __attribute__((aligned(16))) WaveScratch {
     float row_norm2[32];
-    unsigned code_words[32][4];
     unsigned queue[kQueueCap];
+    float acc_copy[16][64];         // one column block's accumulators, for the second look
     int colsum[kMaxHeads][kBits];   // corrections + final per-head ones counts
 };
 
 // Exact sign of x . W[:, col]: fp64 accumulation, d ascending (the oracle's order).
+// Both 256-byte rows are fetched with sixteen 16-byte loads issued together, so
+// the redo costs one memory latency, not 128 of them.
 __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict__ x,
                                                const unsigned short* __restrict__ wt_col)
 {
+    u32x4 xv[kDim / 8], wv[kDim / 8];
+#pragma unroll
+    for (int i = 0; i < kDim / 8; ++i) {
+        xv[i] = *reinterpret_cast<const u32x4*>(x + i * 8);
+        wv[i] = *reinterpret_cast<const u32x4*>(wt_col + i * 8);
+    }
     double acc = 0.0;
-    for (int d = 0; d < kDim; ++d) {
-        acc += static_cast<double>(bf16_to_f32(x[d])) * static_cast<double>(bf16_to_f32(wt_col[d]));
+#pragma unroll
+    for (int i = 0; i < kDim / 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned xa = xv[i][j], wa = wv[i][j];
+            acc += static_cast<double>(__uint_as_float(xa << 16)) * static_cast<double>(__uint_as_float(wa << 16));
+            acc += static_cast<double>(__uint_as_float(xa & 0xffff0000u)) *
+                   static_cast<double>(__uint_as_float(wa & 0xffff0000u));
+        }
     }
     return acc > 0.0;
 }
 
+// Queued results are redone exactly, 64 at a time, one per lane.  Entries are
+// queued after their tile's code words were stored, so the fix goes to memory.
+// Kept out of line: it is called from 64 unrolled places and runs rarely.
+__device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen, int lane,
+                                                      const unsigned short* __restrict__ blk,
+                                                      const unsigned short* __restrict__ wt,
+                                                      unsigned* __restrict__ tc_out, unsigned kv_heads)
+{
+    // the code words stored by this wave must have reached L2 before they are patched there;
+    // waiting for the stores' acknowledgements is enough (a device-scope fence would write back the whole L2)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    for (int base = 0; base < qlen; base += 64) {
+        if (base + lane < qlen) {
+            const unsigned e = ws.queue[base + lane];
+            const unsigned v = e >> 8, col = (e >> 1) & 127u, prov = e & 1u;
+            const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &wt[col * kWtStride]);
+            if (static_cast<unsigned>(pos) != prov) {
+                if (tc_out) { atomicXor(&tc_out[v * 4 + (col >> 5)], 1u << (col & 31)); }
+                atomicAdd(&ws.colsum[v % kv_heads][col], pos ? 1 : -1);
+            }
+        }
+    }
+}
+
 // grid: x = group of kWaves items (cache blocks), y = layer
-__global__ __launch_bounds__(kThreads) void hash_encode_blocks_kernel(
+__global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows,
     unsigned tokens, unsigned kv_heads, const unsigned short* __restrict__ w,
@@ -108,33 +156,33 @@ __global__ __launch_bounds__(kThreads) void hash_encode_blocks_kernel(
     unsigned* tc_out = token_codes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
                                                     static_cast<int64_t>(slot) * n_vec * 4) : nullptr;
 
-    // Queued results are redone exactly, 64 at a time, one per lane.  Code words of
-    // tiles before `open_tile` are already in memory and are patched there; those
-    // of the tile being reduced are still in LDS.
-    auto drain_queue = [&](unsigned open_tile) {
-        __threadfence();
-        for (int base = 0; base < qlen; base += 64) {
-            if (base + lane < qlen) {
-                const unsigned e = ws.queue[base + lane];
-                const unsigned v = e >> 8, col = (e >> 1) & 127u, prov = e & 1u;
-                const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &wt[col * kWtStride]);
-                if (static_cast<unsigned>(pos) != prov) {
-                    if (v / 32 == open_tile) { atomicXor(&ws.code_words[v % 32][col >> 5], 1u << (col & 31)); }
-                    else if (tc_out) { atomicXor(&tc_out[v * 4 + (col >> 5)], 1u << (col & 31)); }
-                    atomicAdd(&ws.colsum[v % kv_heads][col], pos ? 1 : -1);
-                }
-            }
-        }
+    auto drain_queue = [&]() {
+        drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
         qlen = 0;
     };
 
     const unsigned n_tiles = n_vec / 32;
-    for (unsigned tile = 0; tile < n_tiles; ++tile) {
-        // A fragments: lane (row lr, k-half `half`) holds dims ks*16 + half*8 .. +8 of vector tile*32 + lr
-        const unsigned short* xrow = blk + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 8;
-        bf16x8 a[8];
+    // A fragments.  The contraction index may be visited in any order as long as A
+    // and B agree, so MFMA step ks of lane (row lr, k-half `half`) takes dims
+    // half*64 + ks*8 .. +8: a lane's eight 16-byte loads are then one contiguous
+    // 128-byte line of vector tile*32 + lr, fetched from L2 once.
+    auto load_tile = [&](bf16x8 (&a)[8], unsigned tile) {
+        const unsigned short* xrow = blk + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 64;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) { a[ks] = *reinterpret_cast<const bf16x8*>(xrow + ks * 16); }
+        for (int ks = 0; ks < 8; ++ks) { a[ks] = *reinterpret_cast<const bf16x8*>(xrow + ks * 8); }
+    };
+    // which ballot carries this lane's row (lanes 0..31 assemble the code words of row `lane`):
+    // kept as 16 all-ones / all-zeros masks in vector registers so that no scalar state is tied up
+    const int i_sel = ((lr >> 3) << 2) | (lr & 3);
+    const bool use_hi = (lr & 4) != 0;
+    unsigned sel_mask[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { sel_mask[i] = i == i_sel ? 0xffffffffu : 0u; }
+    float sw[4];                                         // sqrt(tau^2 * ||w_col||^2) for this lane's 4 columns
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) { sw[nb] = sqrtf(kTau2 * w_norm2[nb * 32 + lr]); }
+
+    auto reduce_tile = [&](const bf16x8 (&a)[8], unsigned tile) {
         float ss = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
@@ -144,8 +192,12 @@ __global__ __launch_bounds__(kThreads) void hash_encode_blocks_kernel(
                 ss = __builtin_fmaf(v, v, ss);
             }
         }
-        ss += __shfl_xor(ss, 32, 64);
+        ss += __shfl_xor(ss, 32, 64);                    // ||x_row||^2, row = lr
         if (half == 0) { ws.row_norm2[lr] = ss; }
+        float mx = ss;                                   // largest row norm of the tile: a cheap first filter
+#pragma unroll
+        for (int d = 16; d >= 1; d >>= 1) { mx = fmaxf(mx, __shfl_xor(mx, d, 64)); }
+        const float smx = sqrtf(mx) * 1.0001f;
 
         f32x16 acc[4];
 #pragma unroll
@@ -157,48 +209,74 @@ __global__ __launch_bounds__(kThreads) void hash_encode_blocks_kernel(
         for (int ks = 0; ks < 8; ++ks) {
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-                const bf16x8 b = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + ks * 16 + half * 8]);
+                const bf16x8 b = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64 + ks * 8]);
                 acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], b, acc[nb], 0, 0, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);           // keep the weight fragments of later steps out of registers
         }
 
         // accumulator i of lane (half, lr): row (i/4)*8 + half*4 + i%4, column nb*32 + lr
+        unsigned long long doubt[4];                     // per column block: lanes that may need the exact redo
+        unsigned words[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
         for (int nb = 0; nb < 4; ++nb) {
-            const float wn = w_norm2[nb * 32 + lr];
+            float min_abs = __builtin_inff();
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int row = (i >> 2) * 8 + half * 4 + (i & 3);
                 const float v = acc[nb][i];
                 const bool pos = v > 0.0f;
-                const float bound = kTau2 * ws.row_norm2[row] * wn;   // 0 only when x or w is all zero: exact 0 either way
-                const bool unsure = bound > 0.0f && v * v <= bound;
                 const unsigned long long m = __ballot(pos);
-                if (lane == 0) {
-                    ws.code_words[(i >> 2) * 8 + (i & 3)][nb] = static_cast<unsigned>(m);
-                    ws.code_words[(i >> 2) * 8 + 4 + (i & 3)][nb] = static_cast<unsigned>(m >> 32);
-                }
                 ones[nb][i & 3] += pos ? 1 : 0;
-                const unsigned long long um = __ballot(unsure);
-                if (um) {
-                    if (qlen + __popcll(um) > kQueueCap) { drain_queue(tile); }
-                    if (unsure) {
-                        const int p = qlen + static_cast<int>(__builtin_amdgcn_mbcnt_hi(
-                                                 static_cast<unsigned>(um >> 32),
-                                                 __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(um), 0u)));
-                        ws.queue[p] = ((tile * 32 + row) << 8) | ((nb * 32 + lr) << 1) | (pos ? 1u : 0u);
+                min_abs = fminf(min_abs, fabsf(v));
+                const unsigned mine = use_hi ? static_cast<unsigned>(m >> 32) : static_cast<unsigned>(m);
+                words[nb] |= mine & sel_mask[i];
+                if ((i & 3) == 3) { __builtin_amdgcn_sched_barrier(0); }   // consume the ballots before making more
+            }
+            doubt[nb] = __ballot(min_abs < sw[nb] * smx);
+        }
+        // this tile's code words: 32 rows x 16 B, contiguous
+        if (tc_out && lane < 32) {
+            const u32x4 cw = {words[0], words[1], words[2], words[3]};
+            *reinterpret_cast<u32x4*>(tc_out + (static_cast<size_t>(tile) * 32 + lane) * 4) = cw;
+        }
+        // second look, only at the flagged column blocks, with each row's own norm; what
+        // stays doubtful is queued for the exact redo.  The block's accumulators go
+        // through LDS so that this rare path is one rolled loop with one call site.
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+            if (doubt[nb]) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { ws.acc_copy[i][lane] = acc[nb][i]; }
+                const float wn = kTau2 * w_norm2[nb * 32 + lr];
+#pragma unroll 1
+                for (int i = 0; i < 16; ++i) {
+                    const int row = (i >> 2) * 8 + half * 4 + (i & 3);
+                    const float v = ws.acc_copy[i][lane];
+                    const bool unsure = v * v < wn * ws.row_norm2[row];   // strict: an all-zero row is exactly 0
+                    const unsigned long long um = __ballot(unsure);
+                    if (um) {
+                        if (qlen + 64 > kQueueCap) { drain_queue(); }
+                        if (unsure) {
+                            ws.queue[qlen + static_cast<int>(lanes_below(um))] =
+                                ((tile * 32 + row) << 8) | ((nb * 32 + lr) << 1) | (v > 0.0f ? 1u : 0u);
+                        }
+                        qlen += __popcll(um);
                     }
-                    qlen += __popcll(um);
                 }
             }
         }
-        // flush this tile's code words: 32 rows x 16 B, contiguous
-        if (tc_out && lane < 32) {
-            const u32x4 cw = *reinterpret_cast<const u32x4*>(&ws.code_words[lane][0]);
-            *reinterpret_cast<u32x4*>(tc_out + (static_cast<size_t>(tile) * 32 + lane) * 4) = cw;
-        }
+    };
+
+    bf16x8 a_cur[8], a_nxt[8];
+    if (n_tiles > 0) { load_tile(a_cur, 0); }
+#pragma unroll 1
+    for (unsigned tile = 0; tile < n_tiles; ++tile) {
+        if (tile + 1 < n_tiles) { load_tile(a_nxt, tile + 1); }   // in flight during this tile's MFMAs
+        reduce_tile(a_cur, tile);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) { a_cur[ks] = a_nxt[ks]; }
     }
-    if (qlen > 0) { drain_queue(n_tiles); }
+    if (qlen > 0) { drain_queue(); }
 
     // ---- block summaries
 #pragma unroll

@@ -2,11 +2,12 @@
 // the stored-block layout, and the gather of selected blocks from a device
 // block table.  Pure HBM traffic: every byte is read once and written once, so
 // the kernels are 16-byte vector copies with non-temporal hints, one
-// 1024-thread workgroup per slice (a 256 KiB K or V block = 4 trips of 64 KiB
+// 1024-thread workgroup per slice (a 256 KiB K or V block = 2 trips of 128 KiB
 // in flight), launched with far more workgroups than the 256 CUs.  Of the
 // shapes tried on MI355X (8 KiB .. 256 KiB per workgroup, 64 .. 1024 threads,
-// persistent grids, with and without the non-temporal hint) this one was the
-// fastest; all of them sit between 5.2 and 5.7 TB/s for a 1:1 read/write mix.
+// 1 .. 16 loads in flight per thread, persistent grids, with and without the
+// non-temporal hint) this one was the fastest; all of them sit between 5.2 and
+// 6.0 TB/s for a 1:1 read/write mix.
 #include "common.h"
 
 namespace {
@@ -14,12 +15,12 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 1024;
-constexpr int kUnroll = 4;
-constexpr size_t kStep = static_cast<size_t>(kThreads) * 16 * kUnroll;  // 64 KiB per trip
+constexpr int kUnroll = 8;
+constexpr size_t kStep = static_cast<size_t>(kThreads) * 16 * kUnroll;  // 128 KiB per trip
 
-// One workgroup copies one whole slice (a 256 KiB K or V block = 4 trips).
+// One workgroup copies one whole slice (a 256 KiB K or V block = 2 trips).
 // size is a multiple of 16.  All loads of a trip are issued before its first
-// store so that 64 KiB are in flight per workgroup.
+// store so that 128 KiB are in flight per workgroup.
 __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src, size_t size)
 {
     size_t o = 0;
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(kThreads) void kv_gather_selected_kernel(
     copy_slice(dst, src, block_bytes);
 }
 
-constexpr size_t kBatchPiece = 4 * kStep;  // 256 KiB
+constexpr size_t kBatchPiece = 2 * kStep;  // 256 KiB
 
 int check_block_args(const void* layers, int n_layers, size_t kv_stride, size_t block_bytes,
                      int num_blocks, const void* ids, int n, const void* staging)
