@@ -321,3 +321,165 @@ def test_gsa_retrieval_stride_reuses_scores(ucm, dev):
     assert tables[2][0][-2:] == [19, 33] and tables[3][0] == tables[2][0]      # the new block is in the local window
     assert all(len(t[0]) == 5 and t[0][0] == 0 for t in tables)
     assert [t[1] for t in tables] == [4 * 16 + 15, 5 * 16, 4 * 16 + 1, 4 * 16 + 2]
+
+
+# ------------------------------------------------- block store + ESA plugin
+
+def test_hip_block_store_round_trip(ucm, dev):
+    """dump / load through the store surface of the reference (one tensor view per block, byte offsets
+    inside the stored block) move exactly the bytes, as one batched launch per call."""
+    from ucm_amd.sparse.esa.esa import get_offset
+    from ucm_amd.store.hip_block_store import FAILURE, SUCCESS, UcmHipBlockStore
+
+    L, nb, bs, hkv, d = 3, 20, 16, 2, 64
+    shape = (bs, hkv, d)
+    slice_bytes = bs * hkv * d * 2
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 6 * L * 2 * slice_bytes, "role": "worker"})
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev).to(torch.bfloat16) for _ in range(L)]
+    hashes = [f"h{i}" for i in range(6)]
+    ids = [3, 17, 0, 9, 11, 5]
+    assert store.create(hashes) == [SUCCESS] * 6 and store.create(["overflow"]) == [FAILURE]
+    assert store.lookup(hashes) == [False] * 6
+    tasks = []
+    for l in range(L):
+        for kv in range(2):
+            off = [get_offset(shape, 0, 1, 2, l, bool(kv))] * 6
+            tasks.append(store.dump(hashes, off, [caches[l][kv][i] for i in ids]))
+    assert all(store.wait(t) == SUCCESS for t in tasks)
+    store.commit(hashes, True)
+    assert store.lookup(hashes + ["nope"]) == [True] * 6 + [False]
+    # stored-block layout is [layer][K|V] at get_offset, one slot per hash
+    buf = store._buffer.view(store.max_block_num, L, 2, slice_bytes)
+    for j, i in enumerate(ids):
+        for l in range(L):
+            for kv in range(2):
+                assert torch.equal(buf[store.slot_of[hashes[j]], l, kv], caches[l][kv][i].reshape(-1).view(torch.uint8))
+    # load a permuted subset into other cache blocks
+    fresh = [torch.zeros_like(c) for c in caches]
+    pick, dst = [4, 1, 2], [7, 8, 19]
+    tasks = []
+    for l in range(L):
+        for kv in range(2):
+            off = [get_offset(shape, 0, 1, 2, l, bool(kv))] * 3
+            tasks.append(store.load([hashes[p] for p in pick], off, [fresh[l][kv][b] for b in dst]))
+    assert all(store.check(t)[0] == SUCCESS for t in tasks)
+    assert all(store.wait(t) == SUCCESS for t in tasks)
+    for l in range(L):
+        for kv in range(2):
+            for p, b in zip(pick, dst):
+                assert torch.equal(fresh[l][kv][b], caches[l][kv][ids[p]])
+            rest = [b for b in range(nb) if b not in dst]
+            assert not fresh[l][kv][rest].any()
+    assert store.wait(store.load(["unknown"], [0], [fresh[0][0][0]])) == FAILURE
+    # a store in pinned host memory behaves the same
+    host = UcmHipBlockStore({"kv_block_size": slice_bytes, "max_cache_size": 4 * slice_bytes, "device": "pinned"})
+    t = host.dump(["a"], [0], [caches[0][0][2]])
+    assert host.wait(t) == SUCCESS
+    out = torch.zeros_like(caches[0][0][2])
+    assert host.wait(host.load(["a"], [0], [out])) == SUCCESS and torch.equal(out, caches[0][0][2])
+
+
+def test_esa_plugin_flow(ucm, dev):
+    """Prefill + decode of one request through the ESA-shaped plugin: representatives at the last prefill chunk,
+    retrieval through the worker, delta loads from the store into the request's first top_k cache blocks."""
+    from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
+    from ucm_amd.sparse.esa.esa import ESA, block_hash_func, get_offset
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 64
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
+    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"ESA": {
+        "init_window_sz": 1, "local_window_sz": 2, "min_blocks": 4, "sparse_ratio": 0.3, "retrieval_stride": 5}}}
+    slice_bytes = bs * hkv * d * 2
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 40 * L * 2 * slice_bytes})
+    plugin = ESA(cfg, UcmSparseRole.WORKER, store=store)
+    n_prompt = 20 * bs + 5                                   # 20 full blocks + 5 tokens
+    prompt = [int(x) for x in synth.ints(900, n_prompt, 0, 30000)]
+    block_ids = [int(x) for x in synth.permutation(901, nb)[:22]]
+    req = ns(block_ids=[block_ids], num_computed_tokens=0, prompt_token_ids=prompt, output_token_ids=[],
+             num_prompt_tokens=n_prompt, num_output_tokens=0, request_id="A")
+    assert plugin.estimate_num_slots_sparsed(req) == INVALID_SLOT          # nothing to sparsify during prefill
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev).to(torch.bfloat16) for _ in range(L)]
+    original = [c.clone() for c in caches]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
+    ib = ns(req_id_to_index={"A": 0})
+    md = ns(query_start_loc=torch.tensor([0, 1]))
+    sparse_range, top_k = 19, 5                              # 20 - (local_window_sz - 1); int(19 * 0.3)
+
+    def run_step(n_tok):
+        so = ns(num_scheduled_tokens={"A": n_tok})
+        plugin.build_sparse_meta(so, {"A": req}, ib, md)
+        qs = []
+        for l in range(L):
+            q = torch.randn(n_tok, hq, d, device=dev).to(torch.bfloat16)
+            qs.append(q)
+            plugin.attention_begin(q, None, None, names[l], fc)
+            plugin.attention_finished(q, None, None, None, names[l], fc)
+        req.num_computed_tokens += n_tok
+        return qs
+
+    run_step(n_prompt)                                       # prefill: representatives of the first 19 blocks
+    torch.cuda.synchronize()
+    states = plugin.req_states["A"]
+    hashes, parent = [], None
+    for b in range(20):
+        parent = block_hash_func(parent, tuple(prompt[b * bs : (b + 1) * bs]))
+        hashes.append(str(parent))
+    assert states[0].block_hashes == hashes and states[0].sparse_range == sparse_range
+    rep_h = []
+    for l in range(L):
+        assert len(states[l].slots) == sparse_range
+        kc = original[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+        want = np.zeros((plugin.num_slots, hkv * d), np.float32)
+        O.block_mean_paged(kc, block_ids[:sparse_range], states[l].slots, want, round_bf16=True)
+        assert np.array_equal(bits(plugin.data[l].cpu().numpy()), bits(want))
+        rep_h.append(want)
+    # what the prefix-cache connector does after prefill: every full prompt block goes to the store
+    for l in range(L):
+        for kv in range(2):
+            off = [get_offset((bs, hkv, d), 0, 1, 2, l, bool(kv))] * 20
+            assert store.wait(store.dump(hashes, off, [caches[l][kv][b] for b in block_ids[:20]])) == 0
+    store.commit(hashes)
+
+    def expected_selection(l, q):
+        qm = q[0].view(hkv, hq // hkv, d).mean(1).float().reshape(-1).cpu().numpy()   # the plugin's mean is taken in bf16
+        idx, _ = O.esa_retrieve(rep_h[l], qm, np.array(states[l].slots, np.int32), top_k)
+        return [states[l].slots_to_relative_indexes[int(s)] for s in idx]
+
+    resident = block_ids[:top_k]
+    held = [dict() for _ in range(L)]                        # cache block -> logical block it holds after the loads
+    for step in range(1, 8):
+        req.output_token_ids.append(1)
+        req.num_output_tokens = step
+        # the retrieval of steps 2 (submitted in attention_finished) is consumed at step 5
+        qs = run_step(1)
+        torch.cuda.synchronize()
+        for l in range(L):
+            st = states[l]
+            if step == 1:
+                want = expected_selection(l, qs[l])
+                assert sorted(st.pre_topk_block_hashes.values()) == sorted(hashes[i] for i in want)
+                held[l] = {b: hashes.index(h) for b, h in st.pre_topk_block_hashes.items()}
+                assert set(held[l]) <= set(resident) and len(st.last_loaded) == top_k
+            if step == 2:
+                pending_q = qs
+                assert st.retrieval_task is not None
+            if step == 5:
+                want = set(expected_selection(l, pending_q[l]))
+                new_held = {b: hashes.index(h) for b, h in st.pre_topk_block_hashes.items()}
+                assert set(new_held.values()) == want
+                kept = {b for b in new_held if held[l].get(b) == new_held[b]}
+                assert {b for b, _ in st.last_loaded} == set(new_held) - kept       # only missing blocks were loaded
+                held[l] = new_held
+            if step >= 6:
+                assert not st.tasks                           # transfers were waited for at step % stride == 1
+            if step in (1, 6, 7):
+                # the request's first top_k cache blocks hold exactly the selected blocks, K and V
+                for b, logical in held[l].items():
+                    for kv in range(2):
+                        assert torch.equal(caches[l][kv][b], original[l][kv][block_ids[logical]]), (step, l, b)
+    assert plugin.estimate_num_slots_sparsed(req) == top_k * bs + (5 + bs * 1 + 7)
+    plugin.request_finished_in_worker("A")
+    assert "A" not in plugin.req_states and len(plugin.layer_pools[0].allocated) == 0

@@ -158,3 +158,56 @@ def test_gsa_plugin_metadata_without_a_gpu(ucm):
     plugin.execute_finished()
     plugin.request_finished_in_worker("x")
     assert "x" not in plugin.gsa_stats and plugin.topk_kpre_manger.free_cache[-1] == 0
+
+
+def test_esa_scheduler_side_and_helpers(ucm):
+    """ESA's slot estimate, block keeping and hash chain are host arithmetic (esa.py:124-150, :537-587)."""
+    import hashlib
+    import pickle
+
+    from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
+    from ucm_amd.sparse.esa.esa import ESA, ReprePool, block_hash_func, get_offset
+    from ucm_amd.sparse.factory import UcmSparseFactory
+
+    cfg = make_config("ESA", {"init_window_sz": 1, "local_window_sz": 2, "min_blocks": 4, "sparse_ratio": 0.3,
+                              "retrieval_stride": 5})
+    esa = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.SCHEDULER)
+    assert isinstance(esa, ESA) and esa.num_slots == 4096 * 8 // 128
+
+    def request(n_prompt, n_out):
+        return ns(request_id="r", prompt_token_ids=[0] * n_prompt, num_prompt_tokens=n_prompt, num_output_tokens=n_out)
+
+    assert esa.estimate_num_slots_sparsed(request(2000, 0)) == INVALID_SLOT      # still prefilling
+    assert esa.estimate_num_slots_sparsed(request(300, 3)) == INVALID_SLOT       # shorter than min_blocks blocks
+    # 2048 tokens = 16 full blocks: sparse_range 14, keep int(14*0.3)=4 blocks + 2 local blocks + outputs
+    assert esa.estimate_num_slots_sparsed(request(2048, 3)) == 4 * 128 + 2 * 128 + 3
+    # 2000 tokens: 15 full blocks + 80: sparse_range 14, local = 80 + 128 + outputs
+    assert esa.estimate_num_slots_sparsed(request(2000, 7)) == 4 * 128 + 80 + 128 + 7
+
+    freed, evicted = [], []
+    blocks = list(range(100, 116))
+    mgr = ns(req_to_blocks={"r": blocks})
+    coordinator = ns(get_blocks=lambda rid: [blocks], single_type_managers=[mgr],
+                     get_num_blocks_to_allocate=lambda request_id, num_tokens, new_computed_blocks: 1,
+                     allocate_new_blocks=lambda rid, n: None)
+    pool = ns(_maybe_evict_cached_block=evicted.append, free_blocks=freed.extend, get_num_free_blocks=lambda: 5)
+    out = esa.allocate_slots(request(2048, 3), 4 * 128 + 2 * 128 + 3, coordinator, pool, [None])
+    assert mgr.req_to_blocks["r"] == blocks[-7:] and freed == blocks[:-7] and evicted == blocks
+    assert out.blocks == (blocks[-7:],)
+    pool.get_num_free_blocks = lambda: 0
+    assert esa.allocate_slots(request(2048, 3), 771, coordinator, pool, [None]) is None
+
+    seed = int.from_bytes(hashlib.md5(pickle.dumps("UCMHASHSEED", protocol=pickle.HIGHEST_PROTOCOL)).digest(), "big")
+    h1 = block_hash_func(None, (1, 2, 3))
+    assert h1 == int.from_bytes(hashlib.md5(pickle.dumps((seed, (1, 2, 3)), protocol=pickle.HIGHEST_PROTOCOL)).digest(), "big")
+    assert block_hash_func(h1, [4, 5]) == block_hash_func(h1, (4, 5)) != h1
+    for args in [((128, 8, 128), 0, 1, 2, 0, False), ((128, 8, 128), 1, 2, 2, 3, True), ((128, 8, 128), 0, 1, 2, 5, True)]:
+        assert get_offset(*args) == O.get_offset(*args)
+
+    pool2 = ReprePool(5)
+    a = pool2.allocate(3)
+    assert a == [0, 1, 2] and pool2.allocated == {0, 1, 2}
+    pool2.free([1])
+    assert pool2.allocate(3) == [1, 3, 4]
+    with pytest.raises(AssertionError):
+        pool2.allocate(1)
