@@ -312,6 +312,12 @@ def main():
             "host_cpus": os.cpu_count(),
         }
 
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly this workload
+    # (profiles/bench_config2_kernels.md); other workloads have no measurement
+    default_workload = n_layers == N_LAYERS and args.seed == 2024
+    traffic_gather = 10201500000 if default_workload else None
+    traffic_score = 535400000 if default_workload else None
+
     out = {
         "metric": "us per decode step (32-layer retrieval+gather)",
         "value": round(ms_per_step * 1e3, 1),
@@ -343,7 +349,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs(gather_bytes, gather_ms) / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": traffic_gather,
             "algorithmic_bytes": gather_bytes,
         },
         "roofline_score": {
@@ -353,7 +359,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs(score_bytes, score_ms) / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": traffic_score,
             "algorithmic_bytes": score_bytes,
         },
         "block_mean_prefill": {"ms": round(mean_ms, 3), "GBps": round(gbs(mean_bytes, mean_ms), 1),
