@@ -49,6 +49,9 @@ def parse():
     ap.add_argument("--delta-rho", type=float, default=0.95,
                     help="correlation of consecutive decode queries in the delta-gather leg (0 = independent)")
     ap.add_argument("--no-delta", action="store_true", help="skip the delta-gather leg")
+    ap.add_argument("--repre-dtype", choices=["bf16", "f32"], default="bf16",
+                    help="element type of the representative table: bf16 = the rounded means the live reference "
+                         "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -96,11 +99,13 @@ def main():
     for r in range(N_REQ):
         bt_h[r, : lens[r]] = table_h[seg_off_h[r] : seg_off_h[r] + lens[r]]
     bt = i32(bt_h)
-    repre = torch.zeros(n_layers, rows, ROW, device=dev)
+    repre = torch.zeros(n_layers, rows, ROW, device=dev,
+                        dtype=torch.bfloat16 if args.repre_dtype == "bf16" else torch.float32)
+    rep_es = repre.element_size()
     slots = torch.arange(rows, dtype=torch.int32, device=dev)
 
     def prefill():
-        ops.block_mean(layers, table, slots, repre, BS, HKV, D, nb)
+        ops.block_mean(layers, table, slots, repre, BS, HKV, D, nb, mode=ops.MEAN_BF16_ROUND)
 
     prefill()
     torch.cuda.synchronize()
@@ -111,7 +116,7 @@ def main():
     b.record()
     torch.cuda.synchronize()
     mean_ms = a.elapsed_time(b)
-    mean_bytes = n_layers * rows * (BLOCK_BYTES + ROW * 4)
+    mean_bytes = n_layers * rows * (BLOCK_BYTES + ROW * rep_es)
 
     n_q = args.steps + args.warmup
     qs = torch.empty((n_q, n_layers, N_REQ, HQ, D), dtype=torch.bfloat16, device=dev)
@@ -166,7 +171,7 @@ def main():
 
     n_sel = int(topk.astype(np.int64).sum()) * n_layers
     gather_bytes = 2 * n_sel * 2 * BLOCK_BYTES                                     # K and V, read + write
-    score_bytes = n_layers * (rows * ROW * 4 + N_REQ * HQ * D * 2 + rows * 4)     # fp32 representatives + bf16 q + scores
+    score_bytes = n_layers * (rows * ROW * rep_es + N_REQ * HQ * D * 2 + rows * 4)  # representatives + bf16 q + scores
     gbs = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
 
     # ---- delta-gather leg: staging slots keep their blocks between steps, only missing blocks move
@@ -239,7 +244,7 @@ def main():
         idx_h, cnt_h, phys_h = idx.cpu().numpy(), cnt.cpu().numpy(), phys.cpu().numpy()
         scores_h = scores.cpu().numpy()
         for l in range(n_layers):
-            rep = repre[l].cpu().numpy()
+            rep = repre[l].float().cpu().numpy()
             widx, wcnt, wsc = oracle.select_topk_bs(q_last[l], rep, seg_off_h, lens, topk, HKV, out_stride=max_len + 4)
             assert np.array_equal(wsc.view(np.uint32), scores_h[l].view(np.uint32)), f"scores differ in layer {l}"
             assert np.array_equal(wcnt, cnt_h[l]), f"counts differ in layer {l}"
@@ -264,7 +269,7 @@ def main():
 
         threads = min(16, os.cpu_count() or 1)
         os.environ.setdefault("OMP_NUM_THREADS", str(threads))
-        rep_h = repre.cpu().numpy()
+        rep_h = repre.float().cpu().numpy()
         q_h = qs[0].float().cpu().numpy()
         use_ref = oracle.ref.available and _cpu_has_avx512()
         out_stride = max_len + 4
@@ -316,7 +321,7 @@ def main():
     # (profiles/bench_config2_kernels.md); other workloads have no measurement
     default_workload = n_layers == N_LAYERS and args.seed == 2024
     traffic_gather = 10201500000 if default_workload else None
-    traffic_score = 535400000 if default_workload else None
+    traffic_score = {"f32": 535400000}.get(args.repre_dtype) if default_workload else None
 
     out = {
         "metric": "us per decode step (32-layer retrieval+gather)",
@@ -334,6 +339,8 @@ def main():
         "config": {
             "workload": "configs[1]: ragged batch of 16 requests, 4096-65536 tokens, Llama-3-8B attention shape, "
                         f"{n_layers} layers, k = max(16, 3%) + 1 first + 2 last, full gather of selected K and V blocks",
+            "representatives": ("bf16 table (block means rounded to the model dtype, as the live reference path stores them)"
+                                if args.repre_dtype == "bf16" else "fp32 table holding the bf16-rounded block means"),
             "blocks_per_request": [int(x) for x in lens],
             "total_blocks": rows,
             "selected_blocks_per_step": n_sel,

@@ -49,6 +49,7 @@ extern "C" {
 /* ucm_block_mean modes */
 #define UCM_MEAN_F32 0       /* fp32 mean kept as is (the C++ KRepreComputer contract) */
 #define UCM_MEAN_BF16_ROUND 1 /* mean rounded to bf16 and widened (what the live torch path stores) */
+#define UCM_MEAN_BF16_STORE 2 /* the same rounded mean kept as bf16: `repre` is a bf16 table */
 
 typedef void* ucm_stream_t; /* hipStream_t */
 
@@ -70,11 +71,16 @@ const char* ucm_last_error(void);
  *   slots      dev int32[n]: destination row of each block in `repre`
  *   num_blocks, repre_rows: sizes of a K plane and of one layer's table; an id
  *              or slot outside them is skipped by the kernel, not dereferenced.
+ *   repre      dev: fp32 [n_layers][repre_rows][kv_heads*head_dim] for modes
+ *              UCM_MEAN_F32 / UCM_MEAN_BF16_ROUND, bf16 of the same shape for
+ *              UCM_MEAN_BF16_STORE (the dtype the live path keeps its
+ *              representatives in, gsa.py:640-652); repre_layer_stride in
+ *              ELEMENTS of that type.
  * Requires kv_heads*head_dim to be a multiple of 8 and 16-byte aligned planes.
  */
 int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
                    const int32_t* block_ids, const int32_t* slots, int n, int block_size,
-                   int kv_heads, int head_dim, float* repre, int repre_rows,
+                   int kv_heads, int head_dim, void* repre, int repre_rows,
                    int64_t repre_layer_stride, int mode, ucm_stream_t stream);
 
 /*
@@ -93,6 +99,10 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *              reference's gsa_q_cache (gsa.py:503-512) when fp32, or the
  *              layer's raw query tensor with q_rows = index of each request's
  *              last token (GSA.copy_q, gsa.py:616-632) when bf16.
+ *   repre      dev: representative table, repre_dtype fp32 or bf16 (what
+ *              ucm_block_mean wrote), layer stride in ELEMENTS.  A bf16 table
+ *              is widened exactly, so it scores like the fp32 table holding
+ *              the same bf16-rounded means, at half the bytes streamed.
  *   seg_off, seg_len  dev int32[n_req]: first representative row and number of
  *              blocks of each request; max_seg_len >= every seg_len (host
  *              value, sizes the grid); total_blocks = sum of seg_len when the
@@ -101,13 +111,14 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  * head_dim must be 64 or 128 and kv_heads one of 1, 2, 4, 8, 16.
  */
 int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
-                     int q_heads, const float* repre, int64_t repre_layer_stride,
+                     int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
                      const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
                      int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
                      int64_t scores_layer_stride, ucm_stream_t stream);
 
-/* Tuning knob for benchmarks: blocks scored per workgroup by ucm_score_blocks
- * (default 32).  Not part of the reference interface. */
+/* Tuning knob for benchmarks: blocks scored per workgroup by ucm_score_blocks;
+ * 0 (the default) sizes a workgroup's share to 128 KiB of representatives.
+ * Not part of the reference interface. */
 int ucm_set_score_tile(int tile_blocks);
 
 /*

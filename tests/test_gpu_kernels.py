@@ -79,13 +79,15 @@ def test_block_mean_skips_bad_ids_and_layer_range(ucm, dev):
 # --------------------------------------------------------------- scoring
 
 def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=torch.float32, q_rows=None,
-               block_tables=None, seq_lens=None, block_size=128):
-    """q_np [L, rows, Hq, D] fp32 values; repre_np [L, rows, Hkv*D]."""
+               block_tables=None, seq_lens=None, block_size=128, repre_dtype=torch.float32):
+    """q_np [L, rows, Hq, D] fp32 values; repre_np [L, rows, Hkv*D] (values that
+    repre_dtype holds exactly, so the oracle sees the same numbers)."""
     n_layers = repre_np.shape[0]
     lens = np.asarray(lens, np.int32)
     off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
     q = torch.from_numpy(q_np).to(dev).to(q_dtype)
-    repre = torch.from_numpy(repre_np).to(dev)
+    repre = torch.from_numpy(repre_np).to(dev).to(repre_dtype)
+    assert torch.equal(repre.float().cpu(), torch.from_numpy(repre_np))
     scores = torch.full((n_layers, repre_np.shape[1]), -123.0, device=dev)
     mx = int(lens.max(initial=0))
     ops.score_blocks(q, repre, i32(off, dev), i32(lens, dev), mx, hkv, scores,
@@ -158,6 +160,60 @@ def test_ragged_batch_scores_and_selection(ucm, dev, hkv, g, d, q_dtype):
     assert out["cnt"][0, 4] == 0  # the empty request selects nothing
 
 
+def as_bf16_values(a):
+    """fp32 array rounded to the nearest bf16 value (torch's rounding, ties to even)."""
+    return torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(torch.bfloat16).float().numpy()
+
+
+@pytest.mark.parametrize("hkv,g,d", [(8, 4, 128), (8, 8, 128), (1, 8, 128), (2, 2, 64), (4, 1, 64), (16, 2, 128)])
+@pytest.mark.parametrize("q_dtype", [torch.float32, torch.bfloat16])
+def test_bf16_table_scores_like_the_widened_table(ucm, dev, hkv, g, d, q_dtype):
+    """A bf16 representative table holds what the live path stores (ucm/sparse/gsa/gsa.py:640-652);
+    scores and selections must equal the oracle's on the same values widened to fp32, bit for bit."""
+    from ucm_amd import ops
+
+    n_layers = 2
+    lens = [1, 2, 3, 0, 17, 31, 32, 33, 64, 65, 130, 257]
+    topk = [O.compute_topk_len(n) if n > 40 else max(n // 2, 1) for n in lens]
+    rows = int(np.sum(lens))
+    q = synth.normal_bf16_as_f32(33, (n_layers, len(lens), hkv * g, d))
+    repre = as_bf16_values(synth.normal_f32(34, (n_layers, rows, hkv * d)) * np.float32(0.3))
+    try:
+        for tile in (5, 32):
+            ops.set_score_tile(tile)
+            out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=q_dtype, repre_dtype=torch.bfloat16)
+            check_against_oracle(out, q, repre, lens, topk, hkv)
+    finally:
+        ops.set_score_tile(0)
+
+
+def test_bf16_table_from_the_paged_cache(ucm, dev):
+    """keys -> bf16 means -> scores, against the oracle's rounded means; the bf16 table is the
+    fp32 table of UCM_MEAN_BF16_ROUND with the low halves dropped."""
+    from ucm_amd import ops
+
+    hq, hkv, d, bs, nb, n_layers = 32, 8, 128, 128, 70, 2
+    caches_h = [synth.normal_bf16_bits(81 + l, (nb, bs, hkv, d)) for l in range(n_layers)]
+    lp = ops.LayerPointers([bf16_dev(c, dev) for c in caches_h])
+    table = synth.permutation(83, nb)[:67]
+    n = len(table)
+    slots = np.arange(n)
+    t16 = torch.full((n_layers, n + 2, hkv * d), 3.0, device=dev, dtype=torch.bfloat16)
+    t32 = torch.full((n_layers, n + 2, hkv * d), 3.0, device=dev)
+    ops.block_mean(lp, i32(table, dev), i32(slots, dev), t16, bs, hkv, d, nb)
+    ops.block_mean(lp, i32(table, dev), i32(slots, dev), t32, bs, hkv, d, nb, mode=ops.MEAN_BF16_ROUND)
+    assert torch.equal(t16.float(), t32)
+    want = np.full((n_layers, n + 2, hkv * d), 3.0, np.float32)
+    for l in range(n_layers):
+        O.block_mean_paged(caches_h[l], table, slots, want[l], round_bf16=True)
+    assert np.array_equal(bits(t16.float().cpu().numpy()), bits(want))
+    with pytest.raises(ValueError):
+        ops.block_mean(lp, i32(table, dev), i32(slots, dev), t32, bs, hkv, d, nb, mode=ops.MEAN_BF16_STORE)
+    q = synth.normal_bf16_as_f32(84, (n_layers, 1, hq, d))
+    out = run_select(ops, dev, q, want[:, :n], [n], [24], hkv, q_dtype=torch.bfloat16, repre_dtype=torch.bfloat16)
+    check_against_oracle(out, q, want[:, :n], [n], [24], hkv)
+
+
 def test_q_rows_indirection_and_tile_sizes(ucm, dev):
     from ucm_amd import ops
 
@@ -173,7 +229,7 @@ def test_q_rows_indirection_and_tile_sizes(ucm, dev):
             out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=torch.bfloat16, q_rows=rows)
             check_against_oracle(out, q, repre, lens, topk, hkv, q_rows=rows)
     finally:
-        ops.set_score_tile(32)
+        ops.set_score_tile(0)
 
 
 def test_many_requests_dense_tile_lookup(ucm, dev):
@@ -202,7 +258,7 @@ def test_many_requests_dense_tile_lookup(ucm, dev):
                     live = np.concatenate([np.arange(off[r], off[r] + lens[r]) for r in range(len(lens))])
                     assert np.array_equal(bits(got[l][live]), bits(want[live])), (tile, total, l)
     finally:
-        ops.set_score_tile(32)
+        ops.set_score_tile(0)
 
 
 def test_config1_single_request_32k(ucm, dev):

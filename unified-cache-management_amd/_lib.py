@@ -9,7 +9,7 @@ LIB_PATH = os.path.join(_HERE, "libucm_hip.so")
 
 OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5
 DTYPE_F32, DTYPE_BF16 = 0, 1
-MEAN_F32, MEAN_BF16_ROUND = 0, 1
+MEAN_F32, MEAN_BF16_ROUND, MEAN_BF16_STORE = 0, 1, 2
 
 _p, _i, _i64, _sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
 
@@ -18,7 +18,7 @@ SIGNATURES = {
     "ucm_version": [],
     "ucm_last_error": [],
     "ucm_block_mean": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i64, _i, _p],
-    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _p],
+    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _p],
     "ucm_set_score_tile": [_i],
     "ucm_topk_windows": [_p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
     "ucm_esa_retrieve": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _p, _i, _p],

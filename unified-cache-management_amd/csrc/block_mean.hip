@@ -86,6 +86,18 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
         acc[c] = acc[c] * inv;
         if (round_to_bf16) { acc[c] = round_bf16(acc[c]); }
     }
+    if (round_to_bf16 == 2) {
+        // bf16 table: the rounded means themselves, 16 bytes per thread
+        uint16_t* out16 = reinterpret_cast<uint16_t*>(repre) + static_cast<int64_t>(blockIdx.y) * repre_layer_stride +
+                          static_cast<size_t>(slot) * row + col;
+        u32x4 packed;
+        packed.x = (__float_as_uint(acc[0]) >> 16) | (__float_as_uint(acc[1]) & 0xffff0000u);
+        packed.y = (__float_as_uint(acc[2]) >> 16) | (__float_as_uint(acc[3]) & 0xffff0000u);
+        packed.z = (__float_as_uint(acc[4]) >> 16) | (__float_as_uint(acc[5]) & 0xffff0000u);
+        packed.w = (__float_as_uint(acc[6]) >> 16) | (__float_as_uint(acc[7]) & 0xffff0000u);
+        *reinterpret_cast<u32x4*>(out16) = packed;
+        return;
+    }
     float* out = repre + static_cast<int64_t>(blockIdx.y) * repre_layer_stride +
                  static_cast<size_t>(slot) * row + col;
     f32x4 lo = {acc[0], acc[1], acc[2], acc[3]};
@@ -98,7 +110,7 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
 
 extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
                               const int32_t* block_ids, const int32_t* slots, int n, int block_size,
-                              int kv_heads, int head_dim, float* repre, int repre_rows,
+                              int kv_heads, int head_dim, void* repre, int repre_rows,
                               int64_t repre_layer_stride, int mode, ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_block_mean: n=%d", n);
@@ -107,18 +119,20 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535, "ucm_block_mean: n_layers=%d", n_layers);
     UCM_REQUIRE(block_size > 0 && kv_heads > 0 && head_dim > 0 && num_blocks > 0 && repre_rows > 0,
                 "ucm_block_mean: non-positive shape");
-    UCM_REQUIRE(mode == UCM_MEAN_F32 || mode == UCM_MEAN_BF16_ROUND, "ucm_block_mean: mode=%d", mode);
+    UCM_REQUIRE(mode == UCM_MEAN_F32 || mode == UCM_MEAN_BF16_ROUND || mode == UCM_MEAN_BF16_STORE,
+                "ucm_block_mean: mode=%d", mode);
     const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
     UCM_SUPPORTED(row % kCols == 0, "ucm_block_mean: kv_heads*head_dim=%u must be a multiple of %d", row, kCols);
     UCM_REQUIRE(repre_layer_stride >= static_cast<int64_t>(repre_rows) * row || n_layers == 1,
                 "ucm_block_mean: repre_layer_stride=%lld smaller than one layer's table",
                 static_cast<long long>(repre_layer_stride));
-    UCM_REQUIRE(ucm::aligned16(repre) && (repre_layer_stride % 4 == 0), "ucm_block_mean: repre not 16-byte aligned");
+    UCM_REQUIRE(ucm::aligned16(repre) && (repre_layer_stride % (mode == UCM_MEAN_BF16_STORE ? 8 : 4) == 0),
+                "ucm_block_mean: repre not 16-byte aligned");
     const unsigned gx = (row / kCols + kThreads - 1) / kThreads;
     UCM_REQUIRE(static_cast<uint64_t>(n) * gx <= 0x7fffffffull, "ucm_block_mean: too many blocks for one launch");
     hipLaunchKernelGGL(block_mean_kernel, dim3(static_cast<unsigned>(n) * gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream),
                        k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
-                       static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row, repre,
-                       repre_layer_stride, mode == UCM_MEAN_BF16_ROUND ? 1 : 0, gx);
+                       static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row,
+                       static_cast<float*>(repre), repre_layer_stride, mode, gx);
     UCM_LAUNCH_CHECK("ucm_block_mean");
 }

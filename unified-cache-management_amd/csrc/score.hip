@@ -75,12 +75,17 @@ __device__ __forceinline__ f32x4 group_mean4_any(const QT* src, int head_stride,
     return acc * inv;
 }
 
+// Plain loads on purpose: one instruction touches only 64 bytes (32 for the bf16
+// table) of each 128-byte line and the next steps touch the rest, so the line
+// has to stay in the vector L1 between them.  Nontemporal loads do not keep it
+// there and every step then fetches the line from L2 again (bf16 table: 88 us
+// instead of 47 us at 16 requests x 32 layers).
 template <int kSteps>
 __device__ __forceinline__ void load_pass(f32x4 (&kv)[kSteps], const float* p)
 {
 #pragma unroll
     for (int i = 0; i < kSteps; ++i) {
-        kv[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + 16 * i));
+        kv[i] = *reinterpret_cast<const f32x4*>(p + 16 * i);
     }
 }
 
@@ -218,31 +223,163 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
     }
 }
 
+// ---- bf16 representative table ------------------------------------------------
+// The live reference path stores block means rounded to the model dtype
+// (ucm/sparse/gsa/gsa.py:640-652); keeping them as bf16 halves the bytes this
+// kernel streams and widens to the same fp32 values.  Two adjacent threads own
+// one (block, head) vector: thread p holds AVX lanes 8p..8p+7 and reads eight
+// bf16 (16 bytes) per 16-dim step, a wave covers 32 vectors = 8 KiB per pass;
+// the j/j+8 fold crosses the pair (one DPP), the j/j+4 and final folds are
+// in-register.  Same arithmetic, same order, same bits as the fp32-table kernel.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int kSteps>
+__device__ __forceinline__ void load_pass_bf16(u32x4 (&kv)[kSteps], const uint16_t* p)
+{
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i) {
+        kv[i] = *reinterpret_cast<const u32x4*>(p + 16 * i);
+    }
+}
+
+template <int kSteps>
+__device__ __forceinline__ float pair_dot(const f32x4 (&qlo)[kSteps], const f32x4 (&qhi)[kSteps],
+                                          const u32x4 (&kv)[kSteps])
+{
+    float a[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i) {
+        a[0] = __builtin_fmaf(qlo[i].x, __uint_as_float(kv[i].x << 16), a[0]);
+        a[1] = __builtin_fmaf(qlo[i].y, __uint_as_float(kv[i].x & 0xffff0000u), a[1]);
+        a[2] = __builtin_fmaf(qlo[i].z, __uint_as_float(kv[i].y << 16), a[2]);
+        a[3] = __builtin_fmaf(qlo[i].w, __uint_as_float(kv[i].y & 0xffff0000u), a[3]);
+        a[4] = __builtin_fmaf(qhi[i].x, __uint_as_float(kv[i].z << 16), a[4]);
+        a[5] = __builtin_fmaf(qhi[i].y, __uint_as_float(kv[i].z & 0xffff0000u), a[5]);
+        a[6] = __builtin_fmaf(qhi[i].z, __uint_as_float(kv[i].w << 16), a[6]);
+        a[7] = __builtin_fmaf(qhi[i].w, __uint_as_float(kv[i].w & 0xffff0000u), a[7]);
+    }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) { a[c] = quad_perm<kQuadXor1>(a[c]) + a[c]; }   // lanes j and j+8: the other thread
+    const float b0 = a[4] + a[0], b1 = a[5] + a[1], b2 = a[6] + a[2], b3 = a[7] + a[3];   // j and j+4
+    return (b0 + b2) + (b1 + b3);
+}
+
 template <int kD, typename QT>
-void launch(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const float* repre,
+__global__ __launch_bounds__(kThreads) void score_kernel_bf16(
+    const QT* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows, int q_heads,
+    const uint16_t* __restrict__ repre, int64_t repre_layer_stride, const int32_t* __restrict__ seg_off,
+    const int32_t* __restrict__ seg_len, int n_req, int kv_heads, float* __restrict__ scores,
+    int64_t scores_layer_stride, int tile_blocks)
+{
+    constexpr int kSteps = kD / 16;
+    __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l = blockIdx.y;
+    int r, tile;
+    if (!find_tile(seg_len, n_req, tile_blocks, blockIdx.x, lane, r, tile)) { return; }
+    const int n = seg_len[r];
+    const int tile0 = tile * tile_blocks;
+    const int tile_end = min(tile0 + tile_blocks, n);
+    const int row = kv_heads * kD;
+
+    const int p = lane & 1;                 // which 8 of the 16 lanes of the dot product
+    const int v = lane >> 1;                // vector of this pass: 0..31
+    const int blocks_per_pass = 32 / kv_heads;
+    const int bl = v / kv_heads;
+    const int h = v - bl * kv_heads;
+    const int stride = kWaves * blocks_per_pass;
+    const int seg0 = seg_off[r];
+
+    const uint16_t* rbase = repre + static_cast<int64_t>(l) * repre_layer_stride +
+                            static_cast<int64_t>(seg0) * row + h * kD + 8 * p;
+    float* sout = scores + static_cast<int64_t>(l) * scores_layer_stride + seg0;
+
+    int b0 = tile0 + wave * blocks_per_pass;
+    u32x4 kv_a[kSteps], kv_b[kSteps];
+    if (b0 < tile_end) { load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row); }
+
+    {
+        const int g = q_heads / kv_heads;
+        const float inv = 1.0f / static_cast<float>(g);
+        const QT* qp = q + static_cast<int64_t>(l) * q_layer_stride +
+                       static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kD;
+        for (int e = threadIdx.x * 4; e < row; e += kThreads * 4) {
+            const int hh = e / kD, d = e - hh * kD;
+            const f32x4 mean = group_mean4_any(qp + static_cast<int64_t>(hh) * g * kD + d, kD, g, inv);
+            *reinterpret_cast<f32x4*>(&qbar[e]) = mean;
+        }
+    }
+    __syncthreads();
+
+    f32x4 qlo[kSteps], qhi[kSteps];
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i) {
+        qlo[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p]);
+        qhi[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p + 4]);
+    }
+
+    auto finish = [&](const u32x4 (&kv)[kSteps], int base) {
+        const float dot = pair_dot<kSteps>(qlo, qhi, kv);
+        float s = 0.0f;
+        for (int hh = 0; hh < kv_heads; ++hh) {
+            const float dh = __shfl(dot, (bl * kv_heads + hh) * 2, 64);
+            s = s + fmaxf(-FLT_MAX, dh);
+        }
+        const int b = base + bl;
+        if (b < tile_end && h == 0 && p == 0) { sout[b] = s; }
+    };
+    while (b0 < tile_end) {
+        const int b1 = b0 + stride;
+        if (b1 < tile_end) { load_pass_bf16<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row); }
+        finish(kv_a, b0);
+        if (b1 >= tile_end) { break; }
+        const int b2 = b1 + stride;
+        if (b2 < tile_end) { load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row); }
+        finish(kv_b, b1);
+        b0 = b2;
+    }
+}
+
+template <int kD, typename QT>
+void launch_bf16(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
+                 int64_t repre_layer_stride, const int32_t* seg_off, const int32_t* seg_len, int n_req,
+                 int64_t tile_bound, int n_layers, int kv_heads, float* scores, int64_t scores_layer_stride,
+                 int tile_blocks, hipStream_t stream)
+{
+    hipLaunchKernelGGL((score_kernel_bf16<kD, QT>), dim3(static_cast<unsigned>(tile_bound), n_layers), dim3(kThreads), 0,
+                       stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads,
+                       static_cast<const uint16_t*>(repre), repre_layer_stride, seg_off, seg_len, n_req, kv_heads,
+                       scores, scores_layer_stride, tile_blocks);
+}
+
+template <int kD, typename QT>
+void launch(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
             int64_t repre_layer_stride, const int32_t* seg_off, const int32_t* seg_len, int n_req,
             int64_t tile_bound, int n_layers, int kv_heads, float* scores, int64_t scores_layer_stride,
             int tile_blocks, hipStream_t stream)
 {
     hipLaunchKernelGGL((score_kernel<kD, QT>), dim3(static_cast<unsigned>(tile_bound), n_layers), dim3(kThreads), 0,
-                       stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads, repre, repre_layer_stride,
+                       stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads,
+                       static_cast<const float*>(repre), repre_layer_stride,
                        seg_off, seg_len, n_req, kv_heads, scores, scores_layer_stride, tile_blocks);
 }
 
-int g_tile_blocks = 32;
+int g_tile_blocks = 0;  // 0: sized from the row bytes at each call
 
 }  // namespace
 
-// Tuning knob for benchmarks: blocks scored per workgroup (default 32).
+// Tuning knob for benchmarks: blocks scored per workgroup; 0 restores the
+// default, 128 KiB of representatives per workgroup.
 extern "C" int ucm_set_score_tile(int tile_blocks)
 {
-    UCM_REQUIRE(tile_blocks >= 1 && tile_blocks <= 4096, "ucm_set_score_tile: %d", tile_blocks);
+    UCM_REQUIRE(tile_blocks >= 0 && tile_blocks <= 4096, "ucm_set_score_tile: %d", tile_blocks);
     g_tile_blocks = tile_blocks;
     return UCM_OK;
 }
 
 extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
-                                int q_heads, const float* repre, int64_t repre_layer_stride,
+                                int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
                                 const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
                                 int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
                                 int64_t scores_layer_stride, ucm_stream_t stream)
@@ -250,6 +387,7 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
     UCM_REQUIRE(n_req == 0 || max_seg_len == 0 || (q && repre && seg_off && seg_len && scores),
                 "ucm_score_blocks: null pointer");
     UCM_REQUIRE(q_dtype == UCM_DTYPE_F32 || q_dtype == UCM_DTYPE_BF16, "ucm_score_blocks: q_dtype=%d", q_dtype);
+    UCM_REQUIRE(repre_dtype == UCM_DTYPE_F32 || repre_dtype == UCM_DTYPE_BF16, "ucm_score_blocks: repre_dtype=%d", repre_dtype);
     UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535,
                 "ucm_score_blocks: n_req=%d n_layers=%d", n_req, n_layers);
     UCM_REQUIRE(max_seg_len >= 0 && total_blocks >= 0, "ucm_score_blocks: max_seg_len=%d total_blocks=%lld",
@@ -258,21 +396,28 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
                 "ucm_score_blocks: q_heads=%d kv_heads=%d", q_heads, kv_heads);
     UCM_SUPPORTED(head_dim == 64 || head_dim == 128, "ucm_score_blocks: head_dim=%d (64 or 128)", head_dim);
     UCM_SUPPORTED(kv_heads <= 16 && 16 % kv_heads == 0, "ucm_score_blocks: kv_heads=%d (1, 2, 4, 8 or 16)", kv_heads);
-    UCM_REQUIRE(ucm::aligned16(repre) && repre_layer_stride % 4 == 0, "ucm_score_blocks: repre not 16-byte aligned");
+    UCM_REQUIRE(ucm::aligned16(repre) && repre_layer_stride % (repre_dtype == UCM_DTYPE_BF16 ? 8 : 4) == 0,
+                "ucm_score_blocks: repre not 16-byte aligned");
+    UCM_SUPPORTED(repre_dtype == UCM_DTYPE_F32 || 32 % kv_heads == 0, "ucm_score_blocks: kv_heads=%d", kv_heads);
     UCM_REQUIRE(ucm::aligned16(q) && q_layer_stride % 8 == 0, "ucm_score_blocks: q not 16-byte aligned");
     if (n_req == 0 || max_seg_len == 0) { return UCM_OK; }
     hipStream_t s = ucm::as_stream(stream);
     // upper bound of sum(ceil(seg_len / tile)): exact to within n_req when the host knows the total
-    const int64_t per_req = (static_cast<int64_t>(max_seg_len) + g_tile_blocks - 1) / g_tile_blocks;
+    const int row_bytes = kv_heads * head_dim * (repre_dtype == UCM_DTYPE_BF16 ? 2 : 4);
+    const int tile_blocks = g_tile_blocks > 0 ? g_tile_blocks : std::max(8, (128 * 1024) / row_bytes);
+    const int64_t per_req = (static_cast<int64_t>(max_seg_len) + tile_blocks - 1) / tile_blocks;
     int64_t tile_bound = per_req * n_req;
-    if (total_blocks > 0) { tile_bound = std::min(tile_bound, (total_blocks + g_tile_blocks - 1) / g_tile_blocks + n_req); }
+    if (total_blocks > 0) { tile_bound = std::min(tile_bound, (total_blocks + tile_blocks - 1) / tile_blocks + n_req); }
     UCM_REQUIRE(tile_bound <= 0x7fffffffll, "ucm_score_blocks: too many tiles for one launch");
 #define UCM_SCORE_ARGS q, q_layer_stride, q_rows, q_heads, repre, repre_layer_stride, seg_off, seg_len, n_req, \
-                       tile_bound, n_layers, kv_heads, scores, scores_layer_stride, g_tile_blocks, s
-    if (head_dim == 128) {
-        if (q_dtype == UCM_DTYPE_F32) { launch<128, float>(UCM_SCORE_ARGS); } else { launch<128, uint16_t>(UCM_SCORE_ARGS); }
+                       tile_bound, n_layers, kv_heads, scores, scores_layer_stride, tile_blocks, s
+    const bool qf = q_dtype == UCM_DTYPE_F32;
+    if (repre_dtype == UCM_DTYPE_F32) {
+        if (head_dim == 128) { if (qf) { launch<128, float>(UCM_SCORE_ARGS); } else { launch<128, uint16_t>(UCM_SCORE_ARGS); } }
+        else { if (qf) { launch<64, float>(UCM_SCORE_ARGS); } else { launch<64, uint16_t>(UCM_SCORE_ARGS); } }
     } else {
-        if (q_dtype == UCM_DTYPE_F32) { launch<64, float>(UCM_SCORE_ARGS); } else { launch<64, uint16_t>(UCM_SCORE_ARGS); }
+        if (head_dim == 128) { if (qf) { launch_bf16<128, float>(UCM_SCORE_ARGS); } else { launch_bf16<128, uint16_t>(UCM_SCORE_ARGS); } }
+        else { if (qf) { launch_bf16<64, float>(UCM_SCORE_ARGS); } else { launch_bf16<64, uint16_t>(UCM_SCORE_ARGS); } }
     }
 #undef UCM_SCORE_ARGS
     UCM_LAUNCH_CHECK("ucm_score_blocks");

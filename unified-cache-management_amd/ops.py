@@ -11,7 +11,7 @@ from typing import Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import MEAN_BF16_ROUND, MEAN_F32, UcmHipError  # noqa: F401
+from ._lib import MEAN_BF16_ROUND, MEAN_BF16_STORE, MEAN_F32, UcmHipError  # noqa: F401
 
 
 def _stream() -> int:
@@ -59,7 +59,8 @@ class LayerPointers:
 def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                block_size: int, kv_heads: int, head_dim: int, num_blocks: int, mode: int = MEAN_F32,
                first_layer: int = 0, n_layers: Optional[int] = None) -> None:
-    """repre: fp32 [L, rows, kv_heads*head_dim]; rows ``slots`` of layers
+    """repre: [L, rows, kv_heads*head_dim], fp32 (mode MEAN_F32 / MEAN_BF16_ROUND) or
+    bf16 (the mode is then MEAN_BF16_STORE whatever was passed); rows ``slots`` of layers
     first_layer.. are overwritten with the means of cache blocks ``block_ids``."""
     if repre.dim() != 3 or repre.shape[2] != kv_heads * head_dim:
         raise ValueError("repre must be [layers, rows, kv_heads*head_dim]")
@@ -68,7 +69,13 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
         raise ValueError("layer range outside the tables")
     if block_ids.numel() != slots.numel():
         raise ValueError("block_ids and slots differ in length")
-    rp = _dev(repre, torch.float32, "repre") + first_layer * repre.stride(0) * 4
+    if repre.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("repre must be float32 or bfloat16")
+    if repre.dtype == torch.bfloat16:
+        mode = MEAN_BF16_STORE
+    elif mode == MEAN_BF16_STORE:
+        raise ValueError("MEAN_BF16_STORE needs a bfloat16 table")
+    rp = _dev(repre, repre.dtype, "repre") + first_layer * repre.stride(0) * repre.element_size()
     _lib.call("ucm_block_mean", k_layers.ptr(first_layer), n_layers, num_blocks,
               _dev(block_ids, torch.int32, "block_ids"), _dev(slots, torch.int32, "slots"), block_ids.numel(),
               block_size, kv_heads, head_dim, rp, repre.shape[1], repre.stride(0), mode, _stream())
@@ -78,7 +85,7 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
                  max_seg_len: int, kv_heads: int, scores: torch.Tensor,
                  q_rows: Optional[torch.Tensor] = None, first_layer: int = 0,
                  n_layers: Optional[int] = None, total_blocks: int = 0) -> None:
-    """q: [L, rows, q_heads, head_dim] fp32 or bf16; repre: fp32 [L, rows, kv_heads*head_dim];
+    """q: [L, rows, q_heads, head_dim] fp32 or bf16; repre: fp32 or bf16 [L, rows, kv_heads*head_dim];
     scores: fp32 [L, rows].  Layers first_layer .. first_layer+n_layers-1 are scored.
     total_blocks: sum of seg_len when the host knows it (tighter grid), else 0."""
     if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
@@ -86,6 +93,8 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
     head_dim, q_heads = q.shape[3], q.shape[2]
     if repre.shape[2] != kv_heads * head_dim:
         raise ValueError("repre row does not match kv_heads*head_dim")
+    if repre.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("repre must be float32 or bfloat16")
     if q.dtype == torch.float32:
         qd = _lib.DTYPE_F32
     elif q.dtype == torch.bfloat16:
@@ -105,7 +114,8 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
     es = q.element_size()
     _lib.call("ucm_score_blocks", _dev(q, q.dtype, "q") + first_layer * q.stride(0) * es, qd, q.stride(0),
               _opt(q_rows, torch.int32, "q_rows"), q_heads,
-              _dev(repre, torch.float32, "repre") + first_layer * repre.stride(0) * 4, repre.stride(0),
+              _dev(repre, repre.dtype, "repre") + first_layer * repre.stride(0) * repre.element_size(),
+              _lib.DTYPE_BF16 if repre.dtype == torch.bfloat16 else _lib.DTYPE_F32, repre.stride(0),
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
               total_blocks, n_layers, kv_heads, head_dim,
               _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4, scores.stride(0),
