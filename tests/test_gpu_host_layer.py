@@ -175,9 +175,11 @@ def topk_len(n, lo, hi):
     return min(lo, n) if t < lo else min(t, hi)
 
 
-def test_gsa_plugin_decode_flow(ucm, dev):
+@pytest.mark.parametrize("repre_dtype", ["float32", "bfloat16"])
+def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
     """Two requests through prefill and 40 decode steps, two layers: after every attention_begin the
-    layer's block table and sequence lengths must be what the oracle selects from the same cache."""
+    layer's block table and sequence lengths must be what the oracle selects from the same cache.
+    With a bfloat16 table the representatives are the rounded means of the live reference path."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.gsa.gsa import GSA
@@ -185,9 +187,11 @@ def test_gsa_plugin_decode_flow(ucm, dev):
     ns = types.SimpleNamespace
     hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 120
     lo, hi = 6, 10
-    cfg = make_config(hq, hkv, d, L, bs, 16 * 60, {"seg_prefill_threshold": 100, "min_topk_len": lo, "max_topk_len": hi})
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 60, {"seg_prefill_threshold": 100, "min_topk_len": lo, "max_topk_len": hi,
+                                                   "repre_dtype": repre_dtype})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     assert isinstance(plugin, GSA)
+    assert plugin.kpre_caches.dtype == getattr(torch, repre_dtype)
     assert plugin.estimate_num_slots_sparsed(ns()) == INVALID_SLOT
     plugin.request_begin("A", [])
 
@@ -258,7 +262,8 @@ def test_gsa_plugin_decode_flow(ucm, dev):
                 todo = list(range(done_blocks[r], full))
                 if todo:
                     kc = caches[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
-                    O.block_mean_paged(kc, [reqs[r].block_ids[0][i] for i in todo], todo, repre_h[r][l])
+                    O.block_mean_paged(kc, [reqs[r].block_ids[0][i] for i in todo], todo, repre_h[r][l],
+                                       round_bf16=(repre_dtype == "bfloat16"))
         for r in ("A", "B"):
             done_blocks[r] = max(done_blocks[r], min(seq_lens[("A", "B").index(r)] // bs, len(reqs[r].block_ids[0])))
         plugin.execute_finished()
@@ -266,7 +271,7 @@ def test_gsa_plugin_decode_flow(ucm, dev):
         # the device table equals the oracle's
         offA = plugin.gsa_stats["A"].slot_offset
         for l in range(L):
-            got = plugin.kpre_caches[l, offA : offA + done_blocks["A"]].cpu().numpy()
+            got = plugin.kpre_caches[l, offA : offA + done_blocks["A"]].float().cpu().numpy()
             assert np.array_equal(bits(got), bits(repre_h["A"][l][: done_blocks["A"]])), (step, l)
         for r, st in reqs.items():
             st.num_computed_tokens += sched[r]

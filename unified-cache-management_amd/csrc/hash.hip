@@ -4,15 +4,17 @@
 // The projection [vectors x 128] . [128 x 128] is the one real contraction on
 // the whole retrieval path (128 flop per byte of key), so it runs on the matrix
 // cores: v_mfma_f32_32x32x16_bf16, one wave per cache block, 32-vector tiles,
-// the weight matrix staged once per workgroup in LDS (transposed, padded rows).
+// the weight matrix staged once per workgroup in LDS (transposed, padded rows,
+// sign flipped).
 // Only the SIGN of each projection is kept, and it has to be the sign of the
 // exactly accumulated dot product (the CPU oracle accumulates in fp64), so
 // every result whose magnitude is within the fp32 accumulation error bound
 //     |acc| < 2^-15 * ||x|| * ||w_c||
 // is queued and redone by one lane in fp64, d ascending; a few bits per ten
-// thousand take that path (a one-compare filter with the tile's largest row
-// norm flags column blocks; only flagged ones get the per-row look).  The next tile's
-// keys are in flight while the current one goes through the matrix cores.
+// thousand take that path (a one-compare filter with the largest column norm
+// of a 32-column block flags blocks; only flagged ones get the per-column look).
+// The next tile's keys are in flight while the current one goes through the
+// matrix cores.
 //
 // Per cache block the kernel emits: the token codes (LSB-first packing: bit j
 // of byte b is column 8b+j), the per-(kv head, bit) column sums over the
@@ -20,6 +22,8 @@
 // (bit c of head h = S[h][c] > 0).  Both block scores used downstream are
 // integer functions of these: the reference's sum over all (query head, kv
 // head, token) of +-1 inner products equals <sum_i u(q_i), sum_h S[h]>.
+#include <algorithm>
+
 #include "common.h"
 
 namespace {
@@ -46,23 +50,37 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long mask)
 __device__ __forceinline__ float bf16_to_f32(unsigned short h) { return __uint_as_float(static_cast<unsigned>(h) << 16); }
 
 struct __attribute__((aligned(16))) WaveScratch {
-    float row_norm2[32];
     unsigned queue[kQueueCap];
     float acc_copy[16][64];         // one column block's accumulators, for the second look
-    int colsum[kMaxHeads][kBits];   // corrections + final per-head ones counts
+    int colsum[kMaxHeads][kBits];   // per-head ones counts of the block being encoded
 };
 
-// Exact sign of x . W[:, col]: fp64 accumulation, d ascending (the oracle's order).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// sum of squares of 8 bf16 values added to s (v_dot2c_f32_bf16); only used for error bounds
+__device__ __forceinline__ float norm2_acc(const u32x4 v, float s)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const bf16x2 p = __builtin_bit_cast(bf16x2, v[j]);
+        s = __builtin_amdgcn_fdot2_f32_bf16(p, p, s, false);
+    }
+    return s;
+}
+
+// Exact sign of x . W[:, col] from the NEGATED weight row kept in LDS: fp64
+// accumulation, d ascending (the oracle's order; negation is exact and
+// rounding is symmetric, so the sum is the oracle's with its sign flipped).
 // Both 256-byte rows are fetched with sixteen 16-byte loads issued together, so
 // the redo costs one memory latency, not 128 of them.
 __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict__ x,
-                                               const unsigned short* __restrict__ wt_col)
+                                               const unsigned short* __restrict__ neg_wt_col)
 {
     u32x4 xv[kDim / 8], wv[kDim / 8];
 #pragma unroll
     for (int i = 0; i < kDim / 8; ++i) {
         xv[i] = *reinterpret_cast<const u32x4*>(x + i * 8);
-        wv[i] = *reinterpret_cast<const u32x4*>(wt_col + i * 8);
+        wv[i] = *reinterpret_cast<const u32x4*>(neg_wt_col + i * 8);
     }
     double acc = 0.0;
 #pragma unroll
@@ -75,15 +93,15 @@ __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict_
                    static_cast<double>(__uint_as_float(wa & 0xffff0000u));
         }
     }
-    return acc > 0.0;
+    return acc < 0.0;
 }
 
 // Queued results are redone exactly, 64 at a time, one per lane.  Entries are
 // queued after their tile's code words were stored, so the fix goes to memory.
-// Kept out of line: it is called from 64 unrolled places and runs rarely.
+// Kept out of line: it has several call sites and runs rarely.
 __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen, int lane,
                                                       const unsigned short* __restrict__ blk,
-                                                      const unsigned short* __restrict__ wt,
+                                                      const unsigned short* __restrict__ neg_wt,
                                                       unsigned* __restrict__ tc_out, unsigned kv_heads)
 {
     // the code words stored by this wave must have reached L2 before they are patched there;
@@ -94,7 +112,7 @@ __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen,
         if (base + lane < qlen) {
             const unsigned e = ws.queue[base + lane];
             const unsigned v = e >> 8, col = (e >> 1) & 127u, prov = e & 1u;
-            const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &wt[col * kWtStride]);
+            const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &neg_wt[col * kWtStride]);
             if (static_cast<unsigned>(pos) != prov) {
                 if (tc_out) { atomicXor(&tc_out[v * 4 + (col >> 5)], 1u << (col & 31)); }
                 atomicAdd(&ws.colsum[v % kv_heads][col], pos ? 1 : -1);
@@ -103,7 +121,58 @@ __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen,
     }
 }
 
-// grid: x = group of kWaves items (cache blocks), y = layer
+// Bit-sliced counters: plane p holds bit p of 32 independent counts, one per bit
+// position of the words added.  Six planes count to 63.
+constexpr int kPlanes = 6;
+constexpr unsigned kFlushTiles = 63;
+
+__device__ __forceinline__ void planes_add(unsigned (&pl)[kPlanes], unsigned x)
+{
+#pragma unroll
+    for (int p = 0; p < kPlanes; ++p) {
+        const unsigned carry = pl[p] & x;
+        pl[p] ^= x;
+        x = carry;
+    }
+}
+
+// Adds the 32 counts of a plane set to the per-head column sums in LDS and clears
+// it.  Bit b of word pair `wp` is column (2*wp + b/16)*32 + ((b%16)/4)*8 + half*4 + b%4.
+__device__ __forceinline__ void planes_flush(unsigned (&pl)[kPlanes], int* __restrict__ head_row, int wp, int half)
+{
+#pragma unroll 4
+    for (int b = 0; b < 32; ++b) {
+        int cnt = 0;
+#pragma unroll
+        for (int p = 0; p < kPlanes; ++p) { cnt |= static_cast<int>((pl[p] >> b) & 1u) << p; }
+        const int col = (2 * wp + (b >> 4)) * 32 + ((b & 15) >> 2) * 8 + half * 4 + (b & 3);
+        if (cnt) { atomicAdd(&head_row[col], cnt); }
+    }
+#pragma unroll
+    for (int p = 0; p < kPlanes; ++p) { pl[p] = 0u; }
+}
+
+// nibble g of the low 16 bits of x moves to the low nibble of byte g
+__device__ __forceinline__ unsigned spread_nibbles(unsigned x)
+{
+    x = (x | (x << 8)) & 0x00ff00ffu;
+    return (x | (x << 4)) & 0x0f0f0f0fu;
+}
+
+// The product is taken transposed, C^T = (-W)^T . X^T: the matrix cores' A
+// operand is the (negated) weight fragment and B the key fragment, so that lane
+// (half, lr) ends up with sixteen columns per 32-column block of ITS OWN vector
+// lr in registers: accumulator i of block nb is column
+//     nb*32 + (i/4)*8 + half*4 + i%4.
+// With the weights negated, a projection is positive exactly when its
+// accumulator has the sign bit set (and an all-zero key gives +0: bit clear), so
+// one v_alignbit per result shifts the bit into the lane's code word, the two
+// halves are merged with one cross-lane move, and the per-column counts over a
+// block's tokens are kept in bit-sliced counters (a lane's vectors all belong to
+// one kv head because kv_heads divides 32) that are added to LDS once per block.
+// Workgroups are persistent over the list of blocks so that staging the weight
+// matrix is paid once per workgroup, not once per four blocks.
+// grid: x = workgroup (wave w of workgroup g takes items g*kWaves + w, then steps by the grid), y = layer
 __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows,
@@ -112,194 +181,196 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     short* __restrict__ colsum_out, int64_t cs_layer_stride,
     unsigned* __restrict__ block_codes, int64_t bc_layer_stride)
 {
-    __shared__ __attribute__((aligned(16))) unsigned short wt[kBits * kWtStride];  // wt[col][d]
+    __shared__ __attribute__((aligned(16))) unsigned short wt[kBits * kWtStride];  // wt[col][d] = -W[d][col]
     __shared__ float w_norm2[kBits];
     __shared__ WaveScratch scratch[kWaves];
 
-    // ---- weights: global [d][col] -> LDS [col][d]
-    for (int e = threadIdx.x; e < kDim * kBits; e += kThreads) {
-        const int d = e / kBits, c = e - d * kBits;
-        wt[c * kWtStride + d] = w[e];
+    // ---- weights: global [d][col] -> LDS [col][d], sign flipped
+    for (int e8 = threadIdx.x; e8 < kDim * kBits / 8; e8 += kThreads) {
+        const int d = e8 / (kBits / 8), c0 = (e8 % (kBits / 8)) * 8;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(w + d * kBits + c0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            wt[(c0 + 2 * j) * kWtStride + d] = static_cast<unsigned short>((v[j] & 0xffffu) ^ 0x8000u);
+            wt[(c0 + 2 * j + 1) * kWtStride + d] = static_cast<unsigned short>((v[j] >> 16) ^ 0x8000u);
+        }
     }
     __syncthreads();
-    if (threadIdx.x < kBits) {
+    {
+        const int c = threadIdx.x >> 1, part = threadIdx.x & 1;   // two threads per column, 64 dims each
         float s = 0.0f;
-        for (int d = 0; d < kDim; ++d) {
-            const float v = bf16_to_f32(wt[threadIdx.x * kWtStride + d]);
-            s = __builtin_fmaf(v, v, s);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            s = norm2_acc(*reinterpret_cast<const u32x4*>(&wt[c * kWtStride + part * 64 + k * 8]), s);
         }
-        w_norm2[threadIdx.x] = s;
+        s += __shfl_xor(s, 1, 64);
+        if (part == 0) { w_norm2[c] = s; }
     }
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned item = blockIdx.x * kWaves + wave;
-    if (item >= n_items) { return; }
-    const unsigned id = block_ids ? static_cast<unsigned>(block_ids[item]) : item;
-    const unsigned slot = slots ? static_cast<unsigned>(slots[item]) : item;
-    if (id >= num_blocks || slot >= rows) { return; }
-    const unsigned l = blockIdx.y;
-    const unsigned n_vec = tokens * kv_heads;            // vectors of kDim bf16 in the block
-    const unsigned short* blk = static_cast<const unsigned short*>(k_layers[l]) +
-                                static_cast<size_t>(id) * n_vec * kDim;
-    WaveScratch& ws = scratch[wave];
-    for (int e = lane; e < kMaxHeads * kBits; e += 64) { (&ws.colsum[0][0])[e] = 0; }
-
     const int half = lane >> 5, lr = lane & 31;
-    int ones[4][4];                                      // [column block][row % 4]: rows of head (half*4 + e) % kv_heads
+    const unsigned l = blockIdx.y;
+    const unsigned n_vec = tokens * kv_heads;            // vectors of kDim bf16 in a block
+    const unsigned n_tiles = n_vec / 32;
+    WaveScratch& ws = scratch[wave];
+    int* head_row = &ws.colsum[lr % kv_heads][0];        // vector tile*32 + lr is a row of head lr % kv_heads
+
+    float sw[4];                                         // tau * largest ||w_col|| of each 32-column block
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
+        float m = w_norm2[nb * 32 + lr];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { ones[nb][e] = 0; }
+        for (int d = 16; d >= 1; d >>= 1) { m = fmaxf(m, __shfl_xor(m, d, 64)); }
+        sw[nb] = sqrtf(kTau2 * m) * 1.0001f;
     }
-    int qlen = 0;
-    unsigned* tc_out = token_codes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
-                                                    static_cast<int64_t>(slot) * n_vec * 4) : nullptr;
 
-    auto drain_queue = [&]() {
-        drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
-        qlen = 0;
-    };
+    for (unsigned item = blockIdx.x * kWaves + wave; item < n_items; item += gridDim.x * kWaves) {
+        const unsigned id = block_ids ? static_cast<unsigned>(block_ids[item]) : item;
+        const unsigned slot = slots ? static_cast<unsigned>(slots[item]) : item;
+        if (id >= num_blocks || slot >= rows) { continue; }   // never dereference a bad id
+        const unsigned short* blk = static_cast<const unsigned short*>(k_layers[l]) +
+                                    static_cast<size_t>(id) * n_vec * kDim;
+        unsigned* tc_out = token_codes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
+                                                        static_cast<int64_t>(slot) * n_vec * 4) : nullptr;
+        for (int e = lane; e < kMaxHeads * kBits; e += 64) { (&ws.colsum[0][0])[e] = 0; }
 
-    const unsigned n_tiles = n_vec / 32;
-    // A fragments.  The contraction index may be visited in any order as long as A
-    // and B agree, so MFMA step ks of lane (row lr, k-half `half`) takes dims
-    // half*64 + ks*8 .. +8: a lane's eight 16-byte loads are then one contiguous
-    // 128-byte line of vector tile*32 + lr, fetched from L2 once.
-    auto load_tile = [&](bf16x8 (&a)[8], unsigned tile) {
-        const unsigned short* xrow = blk + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 64;
+        unsigned planes01[kPlanes], planes23[kPlanes];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) { a[ks] = *reinterpret_cast<const bf16x8*>(xrow + ks * 8); }
-    };
-    // which ballot carries this lane's row (lanes 0..31 assemble the code words of row `lane`):
-    // kept as 16 all-ones / all-zeros masks in vector registers so that no scalar state is tied up
-    const int i_sel = ((lr >> 3) << 2) | (lr & 3);
-    const bool use_hi = (lr & 4) != 0;
-    unsigned sel_mask[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) { sel_mask[i] = i == i_sel ? 0xffffffffu : 0u; }
-    float sw[4];                                         // sqrt(tau^2 * ||w_col||^2) for this lane's 4 columns
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) { sw[nb] = sqrtf(kTau2 * w_norm2[nb * 32 + lr]); }
+        for (int p = 0; p < kPlanes; ++p) { planes01[p] = 0u; planes23[p] = 0u; }
+        unsigned pending = 0;                            // tiles counted in the planes
+        int qlen = 0;
 
-    auto reduce_tile = [&](const bf16x8 (&a)[8], unsigned tile) {
-        float ss = 0.0f;
+        // B fragments (keys).  The contraction index may be visited in any order as
+        // long as both operands agree, so MFMA step ks of lane (vector lr, k-half
+        // `half`) takes dims half*64 + ks*8 .. +8: a lane's eight 16-byte loads are
+        // then one contiguous 128-byte line of vector tile*32 + lr.
+        u32x4 k_cur[8], k_nxt[8];
+        auto load_tile = [&](u32x4 (&kf)[8], unsigned tile) {
+            const unsigned short* xrow = blk + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 64;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float v = static_cast<float>(a[ks][j]);
-                ss = __builtin_fmaf(v, v, ss);
-            }
-        }
-        ss += __shfl_xor(ss, 32, 64);                    // ||x_row||^2, row = lr
-        if (half == 0) { ws.row_norm2[lr] = ss; }
-        float mx = ss;                                   // largest row norm of the tile: a cheap first filter
-#pragma unroll
-        for (int d = 16; d >= 1; d >>= 1) { mx = fmaxf(mx, __shfl_xor(mx, d, 64)); }
-        const float smx = sqrtf(mx) * 1.0001f;
+            for (int ks = 0; ks < 8; ++ks) { kf[ks] = *reinterpret_cast<const u32x4*>(xrow + ks * 8); }
+        };
+        if (n_tiles > 0) { load_tile(k_cur, 0); }
+#pragma unroll 1
+        for (unsigned tile = 0; tile < n_tiles; ++tile) {
+            if (tile + 1 < n_tiles) { load_tile(k_nxt, tile + 1); }   // in flight during this tile's work
 
-        f32x16 acc[4];
+            float xn2 = 0.0f;                            // ||x||^2 of vector lr
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { acc[nb][i] = 0.0f; }
-        }
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
+            for (int ks = 0; ks < 8; ++ks) { xn2 = norm2_acc(k_cur[ks], xn2); }
+            xn2 += __shfl_xor(xn2, 32, 64);
+            const float sx = sqrtf(xn2);
+
+            f32x16 acc[4];
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-                const bf16x8 b = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64 + ks * 8]);
-                acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks], b, acc[nb], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { acc[nb][i] = 0.0f; }
             }
-            __builtin_amdgcn_sched_barrier(0);           // keep the weight fragments of later steps out of registers
-        }
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const bf16x8 kf = __builtin_bit_cast(bf16x8, k_cur[ks]);
+#pragma unroll
+                for (int nb = 0; nb < 4; ++nb) {
+                    const bf16x8 wf = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64 + ks * 8]);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, kf, acc[nb], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);       // keep the weight fragments of later steps out of registers
+            }
 
-        // accumulator i of lane (half, lr): row (i/4)*8 + half*4 + i%4, column nb*32 + lr
-        unsigned long long doubt[4];                     // per column block: lanes that may need the exact redo
-        unsigned words[4] = {0u, 0u, 0u, 0u};
+            // sign bits -> compact words: bit 16*(nb%2) + i of pair nb/2 is accumulator i of block nb
+            unsigned pair[2];
+            unsigned long long doubt[4];
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-            float min_abs = __builtin_inff();
+            for (int wp = 0; wp < 2; ++wp) {
+                unsigned wbits = 0u;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float v = acc[nb][i];
-                const bool pos = v > 0.0f;
-                const unsigned long long m = __ballot(pos);
-                ones[nb][i & 3] += pos ? 1 : 0;
-                min_abs = fminf(min_abs, fabsf(v));
-                const unsigned mine = use_hi ? static_cast<unsigned>(m >> 32) : static_cast<unsigned>(m);
-                words[nb] |= mine & sel_mask[i];
-                if ((i & 3) == 3) { __builtin_amdgcn_sched_barrier(0); }   // consume the ballots before making more
+                for (int sub = 1; sub >= 0; --sub) {
+                    const int nb = 2 * wp + sub;
+                    float mn = __builtin_inff();
+#pragma unroll
+                    for (int i = 15; i >= 0; --i) {
+                        wbits = __builtin_amdgcn_alignbit(wbits, __float_as_uint(acc[nb][i]), 31);
+                        mn = __builtin_fminf(mn, __builtin_fabsf(acc[nb][i]));
+                    }
+                    doubt[nb] = __ballot(mn < sw[nb] * sx);
+                }
+                pair[wp] = wbits;
             }
-            doubt[nb] = __ballot(min_abs < sw[nb] * smx);
-        }
-        // this tile's code words: 32 rows x 16 B, contiguous
-        if (tc_out && lane < 32) {
-            const u32x4 cw = {words[0], words[1], words[2], words[3]};
-            *reinterpret_cast<u32x4*>(tc_out + (static_cast<size_t>(tile) * 32 + lane) * 4) = cw;
-        }
-        // second look, only at the flagged column blocks, with each row's own norm; what
-        // stays doubtful is queued for the exact redo.  The block's accumulators go
-        // through LDS so that this rare path is one rolled loop with one call site.
+            planes_add(planes01, pair[0]);
+            planes_add(planes23, pair[1]);
+            ++pending;
+
+            // this tile's code words: 32 vectors x 16 B, contiguous
+            unsigned words[4];
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-            if (doubt[nb]) {
+            for (int nb = 0; nb < 4; ++nb) {
+                const unsigned own = spread_nibbles((pair[nb >> 1] >> (16 * (nb & 1))) & 0xffffu) << (4 * half);
+                words[nb] = own | __shfl_xor(own, 32, 64);
+            }
+            if (tc_out && lane < 32) {
+                const u32x4 cw = {words[0], words[1], words[2], words[3]};
+                *reinterpret_cast<u32x4*>(tc_out + (static_cast<size_t>(tile) * 32 + lane) * 4) = cw;
+            }
+
+            // second look, only at the flagged column blocks, column by column; what stays
+            // doubtful is queued for the exact redo.  The block's accumulators go through
+            // LDS so that this rare path is one rolled loop with one call site.
 #pragma unroll
-                for (int i = 0; i < 16; ++i) { ws.acc_copy[i][lane] = acc[nb][i]; }
-                const float wn = kTau2 * w_norm2[nb * 32 + lr];
+            for (int nb = 0; nb < 4; ++nb) {
+                if (doubt[nb]) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) { ws.acc_copy[i][lane] = acc[nb][i]; }
 #pragma unroll 1
-                for (int i = 0; i < 16; ++i) {
-                    const int row = (i >> 2) * 8 + half * 4 + (i & 3);
-                    const float v = ws.acc_copy[i][lane];
-                    const bool unsure = v * v < wn * ws.row_norm2[row];   // strict: an all-zero row is exactly 0
-                    const unsigned long long um = __ballot(unsure);
-                    if (um) {
-                        if (qlen + 64 > kQueueCap) { drain_queue(); }
-                        if (unsure) {
-                            ws.queue[qlen + static_cast<int>(lanes_below(um))] =
-                                ((tile * 32 + row) << 8) | ((nb * 32 + lr) << 1) | (v > 0.0f ? 1u : 0u);
+                    for (int i = 0; i < 16; ++i) {
+                        const int col = nb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                        const float v = ws.acc_copy[i][lane];
+                        const bool unsure = v * v < kTau2 * w_norm2[col] * xn2;   // strict: an all-zero key is exactly 0
+                        const unsigned long long um = __ballot(unsure);
+                        if (um) {
+                            if (qlen + 64 > kQueueCap) {
+                                drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
+                                qlen = 0;
+                            }
+                            if (unsure) {
+                                ws.queue[qlen + static_cast<int>(lanes_below(um))] =
+                                    ((tile * 32 + lr) << 8) | (static_cast<unsigned>(col) << 1) | (__float_as_uint(v) >> 31);
+                            }
+                            qlen += __popcll(um);
                         }
-                        qlen += __popcll(um);
                     }
                 }
             }
-        }
-    };
 
-    bf16x8 a_cur[8], a_nxt[8];
-    if (n_tiles > 0) { load_tile(a_cur, 0); }
-#pragma unroll 1
-    for (unsigned tile = 0; tile < n_tiles; ++tile) {
-        if (tile + 1 < n_tiles) { load_tile(a_nxt, tile + 1); }   // in flight during this tile's MFMAs
-        reduce_tile(a_cur, tile);
+            if (pending == kFlushTiles) {
+                planes_flush(planes01, head_row, 0, half);
+                planes_flush(planes23, head_row, 1, half);
+                pending = 0;
+            }
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) { a_cur[ks] = a_nxt[ks]; }
-    }
-    if (qlen > 0) { drain_queue(); }
-
-    // ---- block summaries
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            atomicAdd(&ws.colsum[(half * 4 + e) % kv_heads][nb * 32 + lr], ones[nb][e]);
+            for (int ks = 0; ks < 8; ++ks) { k_cur[ks] = k_nxt[ks]; }
         }
-    }
-    // (LDS operations of one wave complete in order; no barrier is needed inside the wave)
-    short* cs = colsum_out + (static_cast<int64_t>(l) * cs_layer_stride + static_cast<int64_t>(slot) * kv_heads * kBits);
-    unsigned* bc = block_codes + (static_cast<int64_t>(l) * bc_layer_stride + static_cast<int64_t>(slot) * kv_heads * 4);
-    for (unsigned h = 0; h < kv_heads; ++h) {
+        if (qlen > 0) { drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
+        planes_flush(planes01, head_row, 0, half);
+        planes_flush(planes23, head_row, 1, half);
+
+        // ---- block summaries
+        // (LDS operations of one wave complete in order; no barrier is needed inside the wave)
+        short* cs = colsum_out + (static_cast<int64_t>(l) * cs_layer_stride + static_cast<int64_t>(slot) * kv_heads * kBits);
+        unsigned* bc = block_codes + (static_cast<int64_t>(l) * bc_layer_stride + static_cast<int64_t>(slot) * kv_heads * 4);
+        for (unsigned h = 0; h < kv_heads; ++h) {
 #pragma unroll
-        for (int part = 0; part < 2; ++part) {
-            const int col = part * 64 + lane;
-            const int n_ones = ws.colsum[h][col];
-            const int s = 2 * n_ones - static_cast<int>(tokens);
-            cs[h * kBits + col] = static_cast<short>(s);
-            const unsigned long long m = __ballot(s > 0);
-            if (lane == 0) {
-                bc[h * 4 + part * 2] = static_cast<unsigned>(m);
-                bc[h * 4 + part * 2 + 1] = static_cast<unsigned>(m >> 32);
+            for (int part = 0; part < 2; ++part) {
+                const int col = part * 64 + lane;
+                const int n_ones = ws.colsum[h][col];
+                const int sgn = 2 * n_ones - static_cast<int>(tokens);
+                cs[h * kBits + col] = static_cast<short>(sgn);
+                const unsigned long long m = __ballot(sgn > 0);
+                if (lane == 0) {
+                    bc[h * 4 + part * 2] = static_cast<unsigned>(m);
+                    bc[h * 4 + part * 2 + 1] = static_cast<unsigned>(m >> 32);
+                }
             }
         }
     }
@@ -465,7 +536,10 @@ extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers,
                 "ucm_hash_encode_blocks: token_codes must be 16-byte aligned");
     UCM_REQUIRE(token_codes_layer_stride % 4 == 0 && block_codes_layer_stride % 4 == 0,
                 "ucm_hash_encode_blocks: code strides are in bytes and must be multiples of 4");
-    hipLaunchKernelGGL(hash_encode_blocks_kernel, dim3((n + kWaves - 1) / kWaves, n_layers), dim3(kThreads), 0,
+    // persistent workgroups: about 4096 of them over all layers, each wave stepping through the list
+    const int groups = (n + kWaves - 1) / kWaves;
+    const int gx = std::min(groups, std::max(1, (4096 + n_layers - 1) / n_layers));
+    hipLaunchKernelGGL(hash_encode_blocks_kernel, dim3(gx, n_layers), dim3(kThreads), 0,
                        ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
                        static_cast<unsigned>(n), static_cast<unsigned>(rows), static_cast<unsigned>(block_size),
                        static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16),

@@ -152,7 +152,10 @@ class GSA(UcmSparseBase):
         self.topk_ratio = float(cfg.get("sparse_ratio", 0.3))
         self.init_window = int(cfg.get("init_window_sz", INIT_WINDOW_BLOCKS))
         self.local_window = int(cfg.get("local_window_sz", LOCAL_WINDOW_BLOCKS))
-        self.repre_mode = ops.MEAN_BF16_ROUND if cfg.get("repre_dtype", "float32") == "bfloat16" else ops.MEAN_F32
+        # "bfloat16": the table keeps the rounded means the live reference path stores (gsa.py:640-652) in
+        # that type, half the bytes to score; "float32": fp32 means, the KRepreComputer contract
+        self.repre_dtype = torch.bfloat16 if cfg.get("repre_dtype", "float32") == "bfloat16" else torch.float32
+        self.repre_mode = ops.MEAN_BF16_STORE if self.repre_dtype == torch.bfloat16 else ops.MEAN_F32
 
         self.topk_kpre_manger = TopKAndKpreManger(self.max_bs)
         self.gsa_stats: Dict[ReqType, GSAReqStat] = {}
@@ -173,7 +176,7 @@ class GSA(UcmSparseBase):
         row = self.num_key_heads * self.head_size
         L = self.layer_num
         self.device = device
-        self.kpre_caches = torch.zeros((L, rows, row), dtype=torch.float32, device=device)
+        self.kpre_caches = torch.zeros((L, rows, row), dtype=self.repre_dtype, device=device)
         self.scores = torch.zeros((L, rows), dtype=torch.float32, device=device)
         self.topk_caches = torch.zeros((L, self.max_bs, self.max_block_len), dtype=torch.int32, device=device)
         self.block_tables_mp = torch.zeros_like(self.topk_caches)
