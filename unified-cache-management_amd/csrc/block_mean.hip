@@ -54,7 +54,7 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     const uint16_t* base = static_cast<const uint16_t*>(k_layers[blockIdx.y]) +
                            static_cast<size_t>(id) * block_size * row + col;
     float acc[kCols];
-    widen(*reinterpret_cast<const u32x4*>(base), acc);  // acc = token 0
+    widen(ucm::gload16(base), acc);  // acc = token 0
 
     unsigned t = 1;
     // full groups of kUnroll tokens: loads first, then the ordered adds
@@ -62,8 +62,7 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
         u32x4 v[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            v[u] = __builtin_nontemporal_load(
-                reinterpret_cast<const u32x4*>(base + static_cast<size_t>(t + u) * row));
+            v[u] = ucm::gload16_nt(base + static_cast<size_t>(t + u) * row);
         }
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
@@ -75,7 +74,7 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     }
     for (; t < block_size; ++t) {
         float f[kCols];
-        widen(__builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + static_cast<size_t>(t) * row)), f);
+        widen(ucm::gload16_nt(base + static_cast<size_t>(t) * row), f);
 #pragma unroll
         for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
     }

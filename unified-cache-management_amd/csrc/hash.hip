@@ -11,8 +11,9 @@
 // every result whose magnitude is within the fp32 accumulation error bound
 //     |acc| < 2^-15 * ||x|| * ||w_c||
 // is queued and redone by one lane in fp64, d ascending; a few bits per ten
-// thousand take that path (a one-compare filter with the largest column norm
-// of a 32-column block flags blocks; only flagged ones get the per-column look).
+// thousand take that path (the bound uses the largest column norm of each
+// 32-column block; a min over a lane's sixteen results flags blocks, and only
+// flagged ones get the per-result look).
 // The next tile's keys are in flight while the current one goes through the
 // matrix cores.
 //
@@ -51,7 +52,6 @@ __device__ __forceinline__ float bf16_to_f32(unsigned short h) { return __uint_a
 
 struct __attribute__((aligned(16))) WaveScratch {
     unsigned queue[kQueueCap];
-    float acc_copy[16][64];         // one column block's accumulators, for the second look
     int colsum[kMaxHeads][kBits];   // per-head ones counts of the block being encoded
 };
 
@@ -62,7 +62,8 @@ __device__ __forceinline__ float norm2_acc(const u32x4 v, float s)
 {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const bf16x2 p = __builtin_bit_cast(bf16x2, v[j]);
+        const unsigned e = v[j];   // (a bit_cast of v[j] itself reads element 0 four times with this compiler)
+        const bf16x2 p = __builtin_bit_cast(bf16x2, e);
         s = __builtin_amdgcn_fdot2_f32_bf16(p, p, s, false);
     }
     return s;
@@ -79,7 +80,7 @@ __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict_
     u32x4 xv[kDim / 8], wv[kDim / 8];
 #pragma unroll
     for (int i = 0; i < kDim / 8; ++i) {
-        xv[i] = *reinterpret_cast<const u32x4*>(x + i * 8);
+        xv[i] = ucm::gload16(x + i * 8);
         wv[i] = *reinterpret_cast<const u32x4*>(neg_wt_col + i * 8);
     }
     double acc = 0.0;
@@ -173,6 +174,7 @@ __device__ __forceinline__ unsigned spread_nibbles(unsigned x)
 // Workgroups are persistent over the list of blocks so that staging the weight
 // matrix is paid once per workgroup, not once per four blocks.
 // grid: x = workgroup (wave w of workgroup g takes items g*kWaves + w, then steps by the grid), y = layer
+template <bool kTokenCodes>
 __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows,
@@ -231,7 +233,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         if (id >= num_blocks || slot >= rows) { continue; }   // never dereference a bad id
         const unsigned short* blk = static_cast<const unsigned short*>(k_layers[l]) +
                                     static_cast<size_t>(id) * n_vec * kDim;
-        unsigned* tc_out = token_codes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
+        unsigned* tc_out = kTokenCodes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
                                                         static_cast<int64_t>(slot) * n_vec * 4) : nullptr;
         for (int e = lane; e < kMaxHeads * kBits; e += 64) { (&ws.colsum[0][0])[e] = 0; }
 
@@ -241,6 +243,21 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         unsigned pending = 0;                            // tiles counted in the planes
         int qlen = 0;
 
+        // A tile's code words are stored one trip late: the wait for the next tile's keys
+        // (all counters to zero, that is what the compiler emits at the loop head) would
+        // otherwise also wait for a store issued just before it.  The exact redo patches
+        // code words in memory, so whatever is still held here is stored before a drain.
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        constexpr unsigned kNoTile = 0xffffffffu;
+        u32x2 pend_cw = {0u, 0u};
+        unsigned pend_tile = kNoTile;
+        auto flush_codes = [&]() {
+            if (kTokenCodes && pend_tile != kNoTile) {
+                *reinterpret_cast<u32x2*>(tc_out + (static_cast<size_t>(pend_tile) * 32 + lr) * 4 + half * 2) = pend_cw;
+                pend_tile = kNoTile;
+            }
+        };
+
         // B fragments (keys).  The contraction index may be visited in any order as
         // long as both operands agree, so MFMA step ks of lane (vector lr, k-half
         // `half`) takes dims half*64 + ks*8 .. +8: a lane's eight 16-byte loads are
@@ -249,12 +266,18 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         auto load_tile = [&](u32x4 (&kf)[8], unsigned tile) {
             const unsigned short* xrow = blk + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 64;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) { kf[ks] = *reinterpret_cast<const u32x4*>(xrow + ks * 8); }
+            for (int ks = 0; ks < 8; ++ks) { kf[ks] = ucm::gload16(xrow + ks * 8); }
         };
         if (n_tiles > 0) { load_tile(k_cur, 0); }
+        // The first tile is waited for here, and the prefetch below is unconditional (the
+        // last trip fetches its own tile again): with a skipped prefetch on one path, the
+        // compiler's wait-count bookkeeping at the loop head falls back to "everything
+        // outstanding", which waits for the prefetch it has just issued.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll 1
         for (unsigned tile = 0; tile < n_tiles; ++tile) {
-            if (tile + 1 < n_tiles) { load_tile(k_nxt, tile + 1); }   // in flight during this tile's work
+            load_tile(k_nxt, min(tile + 1, n_tiles - 1));   // in flight during this tile's work
+            flush_codes();
 
             float xn2 = 0.0f;                            // ||x||^2 of vector lr
 #pragma unroll
@@ -309,36 +332,44 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                 const unsigned own = spread_nibbles((pair[nb >> 1] >> (16 * (nb & 1))) & 0xffffu) << (4 * half);
                 words[nb] = own | __shfl_xor(own, 32, 64);
             }
-            if (tc_out && lane < 32) {
-                const u32x4 cw = {words[0], words[1], words[2], words[3]};
-                *reinterpret_cast<u32x4*>(tc_out + (static_cast<size_t>(tile) * 32 + lane) * 4) = cw;
+            if (kTokenCodes) {
+                // lane lr keeps words 0-1 of its vector, lane lr+32 words 2-3; they are stored at the
+                // top of the next trip (see flush_codes)
+                pend_cw.x = half ? words[2] : words[0];
+                pend_cw.y = half ? words[3] : words[1];
+                pend_tile = tile;
             }
 
-            // second look, only at the flagged column blocks, column by column; what stays
-            // doubtful is queued for the exact redo.  The block's accumulators go through
-            // LDS so that this rare path is one rolled loop with one call site.
+            // second look, only at the flagged column blocks: the sign of |acc| - bound marks
+            // the doubtful ones of a lane's sixteen results (one sub and one v_alignbit each,
+            // no LDS, no branches), and the lanes that have any pop them into the queue.
+            // The provisional bit of an entry is read back from the packed sign word.
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
                 if (doubt[nb]) {
+                    const float bound = sw[nb] * sx;     // an all-zero key has bound 0: nothing is below it
+                    unsigned mask = 0u;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) { ws.acc_copy[i][lane] = acc[nb][i]; }
-#pragma unroll 1
-                    for (int i = 0; i < 16; ++i) {
-                        const int col = nb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                        const float v = ws.acc_copy[i][lane];
-                        const bool unsure = v * v < kTau2 * w_norm2[col] * xn2;   // strict: an all-zero key is exactly 0
-                        const unsigned long long um = __ballot(unsure);
-                        if (um) {
-                            if (qlen + 64 > kQueueCap) {
-                                drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
-                                qlen = 0;
-                            }
-                            if (unsure) {
-                                ws.queue[qlen + static_cast<int>(lanes_below(um))] =
-                                    ((tile * 32 + lr) << 8) | (static_cast<unsigned>(col) << 1) | (__float_as_uint(v) >> 31);
-                            }
-                            qlen += __popcll(um);
+                    for (int i = 15; i >= 0; --i) {
+                        mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(__builtin_fabsf(acc[nb][i]) - bound), 31);
+                    }
+                    const unsigned signs = pair[nb >> 1] >> (16 * (nb & 1));
+                    unsigned long long um = __ballot(mask != 0u);
+                    while (um) {
+                        if (qlen + 64 > kQueueCap) {
+                            flush_codes();
+                            drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
+                            qlen = 0;
                         }
+                        if (mask) {
+                            const unsigned i = static_cast<unsigned>(__builtin_ctz(mask));
+                            mask &= mask - 1u;
+                            const unsigned col = nb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                            ws.queue[qlen + static_cast<int>(lanes_below(um))] =
+                                ((tile * 32 + lr) << 8) | (col << 1) | ((signs >> i) & 1u);
+                        }
+                        qlen += __popcll(um);
+                        um = __ballot(mask != 0u);
                     }
                 }
             }
@@ -351,6 +382,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) { k_cur[ks] = k_nxt[ks]; }
         }
+        flush_codes();
         if (qlen > 0) { drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
         planes_flush(planes01, head_row, 0, half);
         planes_flush(planes23, head_row, 1, half);
@@ -539,12 +571,14 @@ extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers,
     // persistent workgroups: about 4096 of them over all layers, each wave stepping through the list
     const int groups = (n + kWaves - 1) / kWaves;
     const int gx = std::min(groups, std::max(1, (4096 + n_layers - 1) / n_layers));
-    hipLaunchKernelGGL(hash_encode_blocks_kernel, dim3(gx, n_layers), dim3(kThreads), 0,
-                       ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
-                       static_cast<unsigned>(n), static_cast<unsigned>(rows), static_cast<unsigned>(block_size),
-                       static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16),
-                       reinterpret_cast<unsigned*>(token_codes), token_codes_layer_stride / 4, colsum,
-                       colsum_layer_stride, reinterpret_cast<unsigned*>(block_codes), block_codes_layer_stride / 4);
+#define UCM_HASH_ENCODE_ARGS dim3(gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream), k_layers, block_ids, slots, \
+        static_cast<unsigned>(num_blocks), static_cast<unsigned>(n), static_cast<unsigned>(rows),                        \
+        static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16),  \
+        reinterpret_cast<unsigned*>(token_codes), token_codes_layer_stride / 4, colsum, colsum_layer_stride,             \
+        reinterpret_cast<unsigned*>(block_codes), block_codes_layer_stride / 4
+    if (token_codes) { hipLaunchKernelGGL(hash_encode_blocks_kernel<true>, UCM_HASH_ENCODE_ARGS); }
+    else { hipLaunchKernelGGL(hash_encode_blocks_kernel<false>, UCM_HASH_ENCODE_ARGS); }
+#undef UCM_HASH_ENCODE_ARGS
     UCM_LAUNCH_CHECK("ucm_hash_encode_blocks");
 }
 

@@ -12,7 +12,7 @@
 
 namespace {
 
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+using ucm::u32x4;
 
 constexpr int kThreads = 1024;
 constexpr int kUnroll = 8;
@@ -29,18 +29,19 @@ __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst, const uint
         u32x4 v[kUnroll];
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            v[u] = __builtin_nontemporal_load(
-                reinterpret_cast<const u32x4*>(src + base + static_cast<size_t>(u) * kThreads * 16));
+            v[u] = ucm::gload16_nt(src + base + static_cast<size_t>(u) * kThreads * 16);
         }
+        // every load of the trip has landed before its first store goes out: stores that
+        // start as the loads trickle in mix reads and writes on the HBM channels and cost
+        // about 6 % of the copy rate (1.64 ms -> 1.75 ms for the 5.1 GB gather)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
         for (int u = 0; u < kUnroll; ++u) {
-            __builtin_nontemporal_store(
-                v[u], reinterpret_cast<u32x4*>(dst + base + static_cast<size_t>(u) * kThreads * 16));
+            ucm::gstore16_nt(dst + base + static_cast<size_t>(u) * kThreads * 16, v[u]);
         }
     }
     for (size_t p = o + threadIdx.x * 16u; p < size; p += static_cast<size_t>(kThreads) * 16) {
-        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + p));
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst + p));
+        ucm::gstore16_nt(dst + p, ucm::gload16_nt(src + p));
     }
 }
 
