@@ -121,6 +121,12 @@ int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const i
  * Not part of the reference interface. */
 int ucm_set_score_tile(int tile_blocks);
 
+/* Tuning knob for benchmarks and tests: number of workgroups
+ * ucm_hash_encode_blocks launches over all layers; each of their waves steps
+ * through the list of blocks.  0 restores the default (4096).  Not part of the
+ * reference interface. */
+int ucm_set_hash_encode_groups(int workgroups);
+
 /*
  * Per-request block selection with forced windows, all layers in one launch -
  * TopkBlockSelector::TopKImpl (select_topk_block.cpp:20-51; windows 1 and 2 by

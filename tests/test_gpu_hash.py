@@ -72,6 +72,71 @@ def test_hash_encode_blocks(ucm, dev, hkv, bs):
                        colsum[:, torch.from_numpy(slots.astype(np.int64)).to(dev)])
 
 
+@pytest.mark.parametrize("hkv,bs", [(8, 128), (2, 48), (1, 160), (4, 8)])
+def test_hash_encode_persistent_waves_and_queue_overflow(ucm, dev, hkv, bs):
+    """One workgroup per layer walks the whole list (every wave takes several blocks, the
+    next block's first keys are fetched while the current one is finished), with odd and
+    single tile counts, bad ids in the list, and blocks whose every projection needs the
+    exact redo: x = (+B at dim 0, s at dim 8, -B at dim 16) against weights with row 16
+    equal to row 0 cancels to s*w[8][c] exactly, while fp32 accumulation loses s next to B,
+    so the matrix-core sign is wrong for about half of the columns and thousands of queue
+    entries per tile have to be redone and patched."""
+    from ucm_amd import ops
+
+    n_layers, nb, rows = 2, 23, 30
+    w = synth.normal_f32(830, (128, 128)) * np.float32(2.0)
+    w[16] = w[0]
+    w_bits = synth.bf16_round_bits(w)
+    w_f32 = synth.bf16_widen(w_bits)
+    one = lambda v: synth.bf16_round_bits(np.array([v], np.float32))[0]
+    caches_h = [synth.normal_bf16_bits(831 + l, (nb, bs, hkv, 128)) for l in range(n_layers)]
+    for l in range(n_layers):
+        c = caches_h[l]
+        for blk in (2, 3, 11, 20):                      # whole blocks of cancelling keys
+            c[blk] = 0
+            c[blk, :, :, 0] = one(4096.0)
+            c[blk, :, :, 16] = one(-4096.0)
+            small = np.array([one(((-1.0) ** (t + h)) * 2.0 ** -20 * (1 + ((t * 7 + h) % 8) / 8.0))
+                              for t in range(bs) for h in range(hkv)], np.uint16).reshape(bs, hkv)
+            c[blk, :, :, 8] = small
+        c[5, bs // 2:] = 0                              # half a block of all-zero keys
+    caches = [bf16_dev(c, dev) for c in caches_h]
+    lp = ops.LayerPointers(caches)
+    ids = np.concatenate([synth.permutation(832, nb), [2, 3]]).astype(np.int32)
+    slots = synth.permutation(833, rows)[: len(ids)].astype(np.int32)
+    ids_bad, slots_bad = ids.copy(), slots.copy()
+    ids_bad[[1, 6, 7, 13]] = [-1, nb, 1 << 30, nb + 5]      # skipped, never dereferenced
+    slots_bad[[9, 20]] = [rows, -3]
+    live = np.array([i for i in range(len(ids)) if 0 <= ids_bad[i] < nb and 0 <= slots_bad[i] < rows])
+    try:
+        for groups in (n_layers, 2 * n_layers, 0):
+            ops.set_hash_encode_groups(groups)
+            colsum = torch.full((n_layers, rows, hkv, 128), 77, dtype=torch.int16, device=dev)
+            bcodes = torch.full((n_layers, rows, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+            tcodes = torch.full((n_layers, rows, bs, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+            ops.hash_encode_blocks(lp, i32(ids_bad, dev), i32(slots_bad, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv,
+                                   nb, colsum, bcodes, token_codes=tcodes)
+            colsum2, bcodes2 = torch.full_like(colsum, 77), torch.full_like(bcodes, 0xEE)
+            ops.hash_encode_blocks(lp, i32(ids_bad, dev), i32(slots_bad, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv,
+                                   nb, colsum2, bcodes2)
+            torch.cuda.synchronize()
+            got_t, got_s, got_b = tcodes.cpu().numpy(), colsum.cpu().numpy(), bcodes.cpu().numpy()
+            assert torch.equal(colsum, colsum2) and torch.equal(bcodes, bcodes2), groups
+            for l in range(n_layers):
+                want_t = O.hash_encode(caches_h[l][ids_bad[live]], w_f32)
+                assert np.array_equal(got_t[l][slots_bad[live]], want_t), (groups, l)
+                assert np.array_equal(got_s[l][slots_bad[live]], O.hash_colsum(want_t)), (groups, l)
+                assert np.array_equal(got_b[l][slots_bad[live]], O.hash_majority(want_t)), (groups, l)
+                rest = np.setdiff1d(np.arange(rows), slots_bad[live])
+                assert np.all(got_t[l][rest] == 0xEE) and np.all(got_s[l][rest] == 77) and np.all(got_b[l][rest] == 0xEE)
+                # the construction did what it is for: the cancelling keys' codes follow sign(s * w[8][c])
+                k = list(live).index(len(ids) - 2)      # block 2, appended at the end of the list
+                sgn = synth.bf16_widen(caches_h[l][2, :, :, 8])[..., None] * w_f32[8][None, None, :] > 0
+                assert np.array_equal(np.unpackbits(want_t[k], axis=-1, bitorder="little").astype(bool), sgn)
+    finally:
+        ops.set_hash_encode_groups(0)
+
+
 def test_hash_queries_scores_and_selection(ucm, dev):
     """Config-5 shape in small: ragged batch, 8 kv heads, 32 query heads, 2 layers."""
     from ucm_amd import ops

@@ -227,12 +227,37 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         sw[nb] = sqrtf(kTau2 * m) * 1.0001f;
     }
 
-    for (unsigned item = blockIdx.x * kWaves + wave; item < n_items; item += gridDim.x * kWaves) {
-        const unsigned id = block_ids ? static_cast<unsigned>(block_ids[item]) : item;
-        const unsigned slot = slots ? static_cast<unsigned>(slots[item]) : item;
-        if (id >= num_blocks || slot >= rows) { continue; }   // never dereference a bad id
-        const unsigned short* blk = static_cast<const unsigned short*>(k_layers[l]) +
-                                    static_cast<size_t>(id) * n_vec * kDim;
+    // keys of item i, or null when its block id or slot is out of range (never dereferenced)
+    auto item_keys = [&](unsigned i, unsigned& slot_out) -> const unsigned short* {
+        if (i >= n_items) { return nullptr; }
+        const unsigned id = block_ids ? static_cast<unsigned>(block_ids[i]) : i;
+        slot_out = slots ? static_cast<unsigned>(slots[i]) : i;
+        if (id >= num_blocks || slot_out >= rows) { return nullptr; }
+        return static_cast<const unsigned short*>(k_layers[l]) + static_cast<size_t>(id) * n_vec * kDim;
+    };
+
+    // B fragments (keys).  The contraction index may be visited in any order as
+    // long as both operands agree, so MFMA step ks of lane (vector lr, k-half
+    // `half`) takes dims half*64 + ks*8 .. +8: a lane's eight 16-byte loads are
+    // then one contiguous 128-byte line of vector tile*32 + lr.
+    u32x4 k_a[8], k_b[8];
+    auto load_tile = [&](u32x4 (&kf)[8], const unsigned short* from, unsigned tile) {
+        const unsigned short* xrow = from + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 64;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) { kf[ks] = ucm::gload16(xrow + ks * 8); }
+    };
+    bool prefetched = false;                             // k_a / k_b already hold (or await) this item's first tiles
+
+    const unsigned item_step = gridDim.x * kWaves;
+    for (unsigned item = blockIdx.x * kWaves + wave; item < n_items; item += item_step) {
+        unsigned slot = 0, next_slot = 0;
+        const unsigned short* blk = item_keys(item, slot);
+        if (!blk) { prefetched = false; continue; }
+        // the tiles after this item's last one come from the next item of this wave, so its
+        // first keys are on their way while this item's summaries are written
+        const unsigned short* next_blk = item_keys(item + item_step, next_slot);
+        const bool chain = next_blk != nullptr && n_tiles >= 2;
+        if (!chain) { next_blk = blk; }
         unsigned* tc_out = kTokenCodes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
                                                         static_cast<int64_t>(slot) * n_vec * 4) : nullptr;
         for (int e = lane; e < kMaxHeads * kBits; e += 64) { (&ws.colsum[0][0])[e] = 0; }
@@ -243,45 +268,45 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         unsigned pending = 0;                            // tiles counted in the planes
         int qlen = 0;
 
-        // A tile's code words are stored one trip late: the wait for the next tile's keys
-        // (all counters to zero, that is what the compiler emits at the loop head) would
-        // otherwise also wait for a store issued just before it.  The exact redo patches
-        // code words in memory, so whatever is still held here is stored before a drain.
+        // A tile's code words are stored one trip late, at the start of the next tile's work:
+        // a store issued just before the wait for the next keys would be waited for as well.
+        // The store is unconditional (a branch around it would make the compiler's wait-count
+        // bookkeeping pessimistic): the first trip writes zeros to tile 0's slot, which the
+        // second trip overwrites.  The exact redo patches code words in memory, so what is
+        // held here is stored before a drain and read back after it.
         typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-        constexpr unsigned kNoTile = 0xffffffffu;
         u32x2 pend_cw = {0u, 0u};
-        unsigned pend_tile = kNoTile;
-        auto flush_codes = [&]() {
-            if (kTokenCodes && pend_tile != kNoTile) {
+        unsigned pend_tile = 0;
+        auto store_codes = [&]() {
+            if (kTokenCodes) {
                 *reinterpret_cast<u32x2*>(tc_out + (static_cast<size_t>(pend_tile) * 32 + lr) * 4 + half * 2) = pend_cw;
-                pend_tile = kNoTile;
+            }
+        };
+        auto drain_queue = [&]() {
+            store_codes();
+            drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
+            qlen = 0;
+            if (kTokenCodes) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the patches have been applied
+                unsigned* p = tc_out + (static_cast<size_t>(pend_tile) * 32 + lr) * 4 + half * 2;
+                pend_cw.x = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                pend_cw.y = __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // consumed here, so that the wait for these two loads stays on this rare path
+                asm volatile("" : "+v"(pend_cw.x), "+v"(pend_cw.y));
             }
         };
 
-        // B fragments (keys).  The contraction index may be visited in any order as
-        // long as both operands agree, so MFMA step ks of lane (vector lr, k-half
-        // `half`) takes dims half*64 + ks*8 .. +8: a lane's eight 16-byte loads are
-        // then one contiguous 128-byte line of vector tile*32 + lr.
-        u32x4 k_cur[8], k_nxt[8];
-        auto load_tile = [&](u32x4 (&kf)[8], unsigned tile) {
-            const unsigned short* xrow = blk + (static_cast<size_t>(tile) * 32 + lr) * kDim + half * 64;
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) { kf[ks] = ucm::gload16(xrow + ks * 8); }
-        };
-        if (n_tiles > 0) { load_tile(k_cur, 0); }
-        // The first tile is waited for here, and the prefetch below is unconditional (the
-        // last trip fetches its own tile again): with a skipped prefetch on one path, the
-        // compiler's wait-count bookkeeping at the loop head falls back to "everything
-        // outstanding", which waits for the prefetch it has just issued.
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll 1
-        for (unsigned tile = 0; tile < n_tiles; ++tile) {
-            load_tile(k_nxt, min(tile + 1, n_tiles - 1));   // in flight during this tile's work
-            flush_codes();
+        // One tile.  `kb` holds its keys; as soon as the matrix cores have consumed them the
+        // same registers are reloaded with the tile after next (of the next item at the end
+        // of this one), so two tiles are in flight per wave for most of the time without a
+        // third buffer.  The reload is unconditional: one skipped on some path would make
+        // the compiler wait for everything outstanding.
+        auto process = [&](u32x4 (&kb)[8], unsigned tile) {
+            store_codes();
 
             float xn2 = 0.0f;                            // ||x||^2 of vector lr
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) { xn2 = norm2_acc(k_cur[ks], xn2); }
+            for (int ks = 0; ks < 8; ++ks) { xn2 = norm2_acc(kb[ks], xn2); }
             xn2 += __shfl_xor(xn2, 32, 64);
             const float sx = sqrtf(xn2);
 
@@ -293,7 +318,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
             }
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                const bf16x8 kf = __builtin_bit_cast(bf16x8, k_cur[ks]);
+                const bf16x8 kf = __builtin_bit_cast(bf16x8, kb[ks]);
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) {
                     const bf16x8 wf = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64 + ks * 8]);
@@ -301,6 +326,12 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                 }
                 __builtin_amdgcn_sched_barrier(0);       // keep the weight fragments of later steps out of registers
             }
+            {
+                const unsigned t2 = tile + 2;
+                const bool over = t2 >= n_tiles;
+                load_tile(kb, over ? next_blk : blk, over ? (chain ? t2 - n_tiles : n_tiles - 1) : t2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
 
             // sign bits -> compact words: bit 16*(nb%2) + i of pair nb/2 is accumulator i of block nb
             unsigned pair[2];
@@ -334,7 +365,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
             }
             if (kTokenCodes) {
                 // lane lr keeps words 0-1 of its vector, lane lr+32 words 2-3; they are stored at the
-                // top of the next trip (see flush_codes)
+                // start of the next tile (see store_codes)
                 pend_cw.x = half ? words[2] : words[0];
                 pend_cw.y = half ? words[3] : words[1];
                 pend_tile = tile;
@@ -356,11 +387,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                     const unsigned signs = pair[nb >> 1] >> (16 * (nb & 1));
                     unsigned long long um = __ballot(mask != 0u);
                     while (um) {
-                        if (qlen + 64 > kQueueCap) {
-                            flush_codes();
-                            drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
-                            qlen = 0;
-                        }
+                        if (qlen + 64 > kQueueCap) { drain_queue(); }
                         if (mask) {
                             const unsigned i = static_cast<unsigned>(__builtin_ctz(mask));
                             mask &= mask - 1u;
@@ -379,10 +406,28 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                 planes_flush(planes23, head_row, 1, half);
                 pending = 0;
             }
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) { k_cur[ks] = k_nxt[ks]; }
+        };
+
+        if (!prefetched) {
+            load_tile(k_a, blk, 0);
+            load_tile(k_b, blk, min(1u, n_tiles - 1));
         }
-        flush_codes();
+        prefetched = chain;
+        unsigned tile = 0;
+#pragma unroll 1
+        for (; tile + 1 < n_tiles; tile += 2) {
+            process(k_a, tile);
+            process(k_b, tile + 1);
+        }
+        if (tile < n_tiles) {
+            process(k_a, tile);
+            // an odd tile count leaves the next item's tile 0 in k_b and its tile 1 in k_a
+            if (chain) {
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) { const u32x4 t = k_a[ks]; k_a[ks] = k_b[ks]; k_b[ks] = t; }
+            }
+        }
+        store_codes();
         if (qlen > 0) { drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
         planes_flush(planes01, head_row, 0, half);
         planes_flush(planes23, head_row, 1, half);
@@ -545,7 +590,18 @@ __global__ __launch_bounds__(256) void hash_score_kernel(
     }
 }
 
+int g_encode_groups = 4096;
+
 }  // namespace
+
+// Tuning knob for benchmarks and tests: workgroups launched by
+// ucm_hash_encode_blocks over all layers (0 restores the default, 4096).
+extern "C" int ucm_set_hash_encode_groups(int workgroups)
+{
+    UCM_REQUIRE(workgroups >= 0 && workgroups <= (1 << 20), "ucm_set_hash_encode_groups: %d", workgroups);
+    g_encode_groups = workgroups > 0 ? workgroups : 4096;
+    return UCM_OK;
+}
 
 extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers, int num_blocks,
                                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
@@ -570,7 +626,7 @@ extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers,
                 "ucm_hash_encode_blocks: code strides are in bytes and must be multiples of 4");
     // persistent workgroups: about 4096 of them over all layers, each wave stepping through the list
     const int groups = (n + kWaves - 1) / kWaves;
-    const int gx = std::min(groups, std::max(1, (4096 + n_layers - 1) / n_layers));
+    const int gx = std::min(groups, std::max(1, (g_encode_groups + n_layers - 1) / n_layers));
 #define UCM_HASH_ENCODE_ARGS dim3(gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream), k_layers, block_ids, slots, \
         static_cast<unsigned>(num_blocks), static_cast<unsigned>(n), static_cast<unsigned>(rows),                        \
         static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16),  \

@@ -293,3 +293,7 @@ def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, 
 
 def set_score_tile(tile_blocks: int) -> None:
     _lib.call("ucm_set_score_tile", tile_blocks)
+
+
+def set_hash_encode_groups(workgroups: int) -> None:
+    _lib.call("ucm_set_hash_encode_groups", workgroups)
