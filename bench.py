@@ -52,6 +52,8 @@ def parse():
     ap.add_argument("--repre-dtype", choices=["bf16", "f32"], default="bf16",
                     help="element type of the representative table: bf16 = the rounded means the live reference "
                          "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
+    ap.add_argument("--hash-leg", action="store_true",
+                    help="also time the hash-code retrieval variant (BASELINE configs[4] shape) on the same caches")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -232,6 +234,81 @@ def main():
                     "q' = rho*q + sqrt(1-rho^2)*noise (synthetic); staging verified against the source blocks",
         }
 
+    # ---- hash-code retrieval leg (configs[4]): 32 requests of 64-256 blocks, 32 layers, 128-bit codes.
+    # The key blocks are the K and V planes of the caches above read as one pool of 2*nb blocks.
+    hash_leg = None
+    if args.hash_leg:
+        h_req = 32
+        h_lens = rng.integers(64, 257, h_req).astype(np.int32)
+        h_rows = int(h_lens.sum())
+        h_off = np.concatenate([[0], np.cumsum(h_lens)[:-1]]).astype(np.int32)
+        pool = 2 * nb
+        h_ids_h = (rng.permutation(pool)[:h_rows] if h_rows <= pool else rng.integers(0, pool, h_rows)).astype(np.int32)
+        h_ids, h_slots = i32(h_ids_h), torch.arange(h_rows, dtype=torch.int32, device=dev)
+        w_hash = (torch.randn(128, 128, device=dev, generator=g) * 2.0).to(torch.bfloat16)
+        colsum = torch.zeros((n_layers, h_rows, HKV, 128), dtype=torch.int16, device=dev)
+        bcodes = torch.zeros((n_layers, h_rows, HKV, 16), dtype=torch.uint8, device=dev)
+        tcodes = torch.zeros((n_layers, h_rows, BS, HKV, 16), dtype=torch.uint8, device=dev)
+        hq = torch.empty((n_layers, h_req, HQ, D), dtype=torch.bfloat16, device=dev).normal_(generator=g)
+        q_codes = torch.zeros((n_layers, h_req, HQ, 16), dtype=torch.uint8, device=dev)
+        q_sum = torch.zeros((n_layers, h_req, 128), dtype=torch.int16, device=dev)
+        qbar = torch.zeros((n_layers, h_req, HKV, 16), dtype=torch.uint8, device=dev)
+        h_scores = torch.zeros(n_layers, h_rows, device=dev)
+        h_topk = np.maximum(16, (0.03 * h_lens).astype(np.int32)) + 3
+        h_idx = torch.zeros((n_layers, h_req, int(h_lens.max())), dtype=torch.int32, device=dev)
+        h_cnt = torch.zeros((n_layers, h_req), dtype=torch.int32, device=dev)
+        h_so, h_sl, h_tk = i32(h_off), i32(h_lens), i32(h_topk)
+
+        def timed(fn, reps):
+            fn()
+            torch.cuda.synchronize()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / reps
+
+        enc = lambda tc: ops.hash_encode_blocks(layers, h_ids, h_slots, h_rows, w_hash, BS, HKV, pool, colsum, bcodes,
+                                                token_codes=tc)
+        enc_ms = timed(lambda: enc(tcodes), 3)
+        enc_sum_ms = timed(lambda: enc(None), 3)
+        enc(tcodes)
+        q_ms = timed(lambda: ops.hash_encode_queries(hq, w_hash, HKV, q_codes, q_sum, qbar, h_req), 10)
+        sc_ms = timed(lambda: ops.hash_score_blocks(0, q_sum, qbar, colsum, bcodes, h_so, h_sl, h_rows, h_scores), 10)
+        tk_ms = timed(lambda: ops.topk_windows(h_scores, h_so, h_sl, h_tk, int(h_lens.max()), h_idx, h_cnt), 10)
+        key_bytes = n_layers * h_rows * BLOCK_BYTES
+        enc_bytes = key_bytes + n_layers * h_rows * (BS * HKV * 16 + HKV * 128 * 2 + HKV * 16)
+        hash_checked = None
+        if not args.no_check:
+            import oracle  # checker only
+
+            w_f32 = w_hash.float().cpu().numpy()
+            for l in (0, n_layers - 1):
+                pool_l = caches[l].view(2 * nb, BS, HKV, D)
+                for row in (0, h_rows // 2, h_rows - 1):
+                    keys = pool_l[int(h_ids_h[row])].view(torch.int16).cpu().numpy().view(np.uint16)
+                    want = oracle.hash_encode(keys[None], w_f32)
+                    assert np.array_equal(tcodes[l, row].cpu().numpy(), want[0]), "token codes differ"
+                    assert np.array_equal(colsum[l, row].cpu().numpy(), oracle.hash_colsum(want)[0]), "column sums differ"
+                    assert np.array_equal(bcodes[l, row].cpu().numpy(), oracle.hash_majority(want)[0]), "block codes differ"
+            hash_checked = "token codes, column sums and majority codes of 6 sampled blocks equal the CPU oracle"
+        hash_leg = {
+            "workload": f"configs[4]: {h_req} requests, {h_rows} blocks of 128 tokens, {n_layers} layers, 8 kv heads, 128-bit codes",
+            "encode_ms": round(enc_ms, 3),
+            "encode_read_GBps": round(gbs(key_bytes, enc_ms), 1),
+            "roofline": {"kernel": "hash_encode_blocks_kernel", "bound": "hbm", "achieved": round(gbs(enc_bytes, enc_ms), 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs(enc_bytes, enc_ms) / HBM_PEAK_GBS, 4),
+                         "traffic": None, "algorithmic_bytes": enc_bytes,
+                         "mfma_TFLOPs": round(2.0 * n_layers * h_rows * BS * HKV * 128 * 128 / (enc_ms * 1e-3) / 1e12, 1)},
+            "encode_summaries_only_ms": round(enc_sum_ms, 3),
+            "decode_step_us": {"query_codes": round(q_ms * 1e3, 1), "score": round(sc_ms * 1e3, 1),
+                               "select": round(tk_ms * 1e3, 1)},
+            "checked": hash_checked,
+        }
+        del colsum, bcodes, tcodes
+
     # ---- check the last step against the CPU oracle (selection, scores, gathered bytes)
     if not args.no_check:
         step(qs[n_q - 1])                                             # re-run the last full step: the delta leg reused the buffers
@@ -372,6 +449,7 @@ def main():
         "block_mean_prefill": {"ms": round(mean_ms, 3), "GBps": round(gbs(mean_bytes, mean_ms), 1),
                                "frac": round(gbs(mean_bytes, mean_ms) / HBM_PEAK_GBS, 4)},
         "delta_gather": delta,
+        "hash_retrieval": hash_leg,
         "cpu_baseline": cpu,
         "checked": checked,
     }

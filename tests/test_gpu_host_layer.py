@@ -191,7 +191,7 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
                                                    "repre_dtype": repre_dtype})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     assert isinstance(plugin, GSA)
-    assert plugin.kpre_caches.dtype == getattr(torch, repre_dtype)
+    assert plugin.repre_dtype == getattr(torch, repre_dtype)   # the table itself is allocated at the first step
     assert plugin.estimate_num_slots_sparsed(ns()) == INVALID_SLOT
     plugin.request_begin("A", [])
 
@@ -271,6 +271,7 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
         # the device table equals the oracle's
         offA = plugin.gsa_stats["A"].slot_offset
         for l in range(L):
+            assert plugin.kpre_caches.dtype == getattr(torch, repre_dtype)
             got = plugin.kpre_caches[l, offA : offA + done_blocks["A"]].float().cpu().numpy()
             assert np.array_equal(bits(got), bits(repre_h["A"][l][: done_blocks["A"]])), (step, l)
         for r, st in reqs.items():
