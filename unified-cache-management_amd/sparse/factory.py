@@ -30,3 +30,4 @@ class UcmSparseFactory:
 _PKG = __name__.rsplit(".", 1)[0]
 UcmSparseFactory.register_sparse_method("GSA", _PKG + ".gsa.gsa", "GSA")
 UcmSparseFactory.register_sparse_method("ESA", _PKG + ".esa.esa", "ESA")
+UcmSparseFactory.register_sparse_method("KvComp", _PKG + ".kvcomp.kvcomp", "KvComp")
