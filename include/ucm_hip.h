@@ -261,6 +261,56 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
                           int64_t scores_layer_stride, int round_fp16, ucm_stream_t stream);
 
 /*
+ * KVStar multi-query softmax-vote retrieval.
+ *
+ * ucm_kvstar_block_repre: the sub-block representatives of
+ * ReqPerLayerState.extract_block_repre (ucm/sparse/kvstar/multistep.py:279-316)
+ * read straight from the paged bf16 key cache: each listed block is cut into
+ * M = block_size/merge sub-blocks, the `merge` tokens of a sub-block are
+ * averaged per (kv head, kept channel) - fp32 sum in token order, *(1/merge),
+ * rounded to bf16 (the model dtype the reference's mean() returns) and stored
+ * as fp16 (its .to(torch.float16), :495-497).
+ *   pruned   dev int32[kv_heads][d_pruned]: channel of every kept dim (the
+ *            reference's d_pruned_index, :288-304), or NULL when d_pruned ==
+ *            head_dim
+ *   repre    dev fp16 [n_layers][repre_rows][M][kv_heads][d_pad], d_pad >=
+ *            d_pruned (columns past d_pruned are written as zero);
+ *            repre_layer_stride in elements.
+ *
+ * ucm_kvstar_votes: the arithmetic of KVStar::Execute
+ * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:817-990)
+ * for n_tasks (request, layer) tasks in one go: scores of n_tokens x q_heads
+ * query rows against all sub-block representatives of the task, softmax of
+ * every row over the task's sub-blocks, votes[block] = sum over rows and over
+ * the block's sub-blocks of the probabilities.  The top-k of the votes is
+ * taken by ucm_topk_windows (init_w = local_w = 0).  fp32 on the matrix cores;
+ * agrees with the reference's scalar loop to rounding, not bit for bit.
+ *   q_f16    dev fp16; task t's [n_tokens][q_heads][d_orig] block starts
+ *            q_off[t] elements in (dev int64[n_tasks])
+ *   pruned   dev int32[*][kv_heads][d_pruned] channel lists, pruned_sel dev
+ *            int32[n_tasks] picks one per task (-1: none); both NULL when
+ *            d_pruned == d_orig
+ *   repre_f16  dev fp16 [rows][sub_blocks][kv_heads][d_pad]; task t owns rows
+ *            seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >= every seg_len
+ *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
+ *            returns; votes dev fp32, task t's votes at votes[seg_off[t] + b].
+ * n_tokens * (q_heads/kv_heads) <= 64, kv_heads <= 8, d_pad a multiple of 16
+ * and <= 128, sub_blocks in {1, 2, 4, 8, 16, 32}.
+ */
+int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
+                           const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                           int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
+                           int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
+                           ucm_stream_t stream);
+int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int max_blocks, int sub_blocks,
+                                int64_t* max_floats, int64_t* part_floats);
+int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                     const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
+                     const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                     int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+                     float* ws_part, float* votes, ucm_stream_t stream);
+
+/*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched
  * pointer-array copy of the reference's device layer (H2DKernel / D2HKernel,
  * ucm/store/device/cuda/cuda_device.cu:47-81, reached through

@@ -76,6 +76,12 @@ _orc_hash_colsum = _sig(_orc, "orc_hash_colsum", None, _p, _u32, _u32, _u32, _u3
 _orc_hash_scores_sum = _sig(_orc, "orc_hash_scores_sum", None, _p, _u32, _p, _u32, _u32, _u32, _u32, _p)
 _orc_hash_majority = _sig(_orc, "orc_hash_majority", None, _p, _u32, _u32, _u32, _u32, _p)
 _orc_hash_scores_block = _sig(_orc, "orc_hash_scores_block", None, _p, _p, _u32, _u32, _u32, _p)
+_orc_f16_to_f32 = _sig(_orc, "orc_f16_to_f32", _f32, C.c_uint16)
+_orc_f32_to_f16 = _sig(_orc, "orc_f32_to_f16", C.c_uint16, _f32)
+_orc_kvstar_block_repre = _sig(_orc, "orc_kvstar_block_repre", None, _p, _p, _p, _u32, _u32, _u32, _u32, _u32, _p, _u32,
+                               _u32, _p)
+_orc_kvstar_retrieve = _sig(_orc, "orc_kvstar_retrieve", _i32, _p, _u32, _u32, _u32, _p, _u32, _u32, _u32, _u32, _u32, _p,
+                            _u32, _p, _p)
 _orc_f32_to_bf16 = _sig(_orc, "orc_f32_to_bf16", C.c_uint16, _f32)
 
 
@@ -294,6 +300,42 @@ def hash_scores_block(q_codes: np.ndarray, block_codes: np.ndarray) -> np.ndarra
 
 
 # ------------------------------------------- the reference's own compiled TUs
+
+def f16_to_f32(h: int) -> float:
+    return float(_orc_f16_to_f32(int(h)))
+
+
+def f32_to_f16(f: float) -> int:
+    return int(_orc_f32_to_f16(float(f)))
+
+
+def kvstar_block_repre(cache_bits: np.ndarray, block_ids, slots, merge: int, repre: np.ndarray, pruned=None) -> None:
+    """cache_bits uint16 [num_blocks, block_size, kv_heads, head_dim] (bf16); repre uint16 (fp16)
+    [rows, M, kv_heads, d_pad], rows ``slots`` are overwritten; pruned int32 [kv_heads, d_pruned] or None."""
+    cb = _c(cache_bits, np.uint16)
+    _, bs, h, d = cb.shape
+    ids, sl = _c(block_ids, np.int32), _c(slots, np.int32)
+    assert repre.dtype == np.uint16 and repre.flags.c_contiguous and repre.shape[1] == bs // merge and repre.shape[2] == h
+    pr = None if pruned is None else _c(pruned, np.int32)
+    dp = d if pr is None else pr.shape[1]
+    _orc_kvstar_block_repre(_ptr(cb), _ptr(ids), _ptr(sl), len(ids), bs, h, d, merge, None if pr is None else _ptr(pr),
+                            dp, repre.shape[3], _ptr(repre))
+
+
+def kvstar_retrieve(q_bits: np.ndarray, repre: np.ndarray, topk: int, pruned=None, d_pruned: int | None = None):
+    """q_bits uint16 (fp16) [tokens, q_heads, d_orig]; repre uint16 (fp16) [n_blocks, M, kv_heads, d_pad]
+    -> (top-k block indices by descending score, final scores fp32 [n_blocks])."""
+    qb, rp = _c(q_bits, np.uint16), _c(repre, np.uint16)
+    x, hq, d = qb.shape
+    n, m, h, d_pad = rp.shape
+    pr = None if pruned is None else _c(pruned, np.int32)
+    dp = (d_pad if d_pruned is None else d_pruned) if pr is None else pr.shape[1]
+    final = np.zeros(n, np.float32)
+    idx = np.zeros(max(min(topk, n), 1), np.int32)
+    k = _orc_kvstar_retrieve(_ptr(qb), x, hq, d, _ptr(rp), n, m, h, dp, d_pad, None if pr is None else _ptr(pr), topk,
+                             _ptr(final), _ptr(idx))
+    return idx[:k].copy(), final
+
 
 class _Ref:
     """Lazy handle on oracle/_ref (present only where the reference tree was)."""

@@ -28,6 +28,11 @@
  *   orc_hash_*: closed forms (sign, LSB-first packing, <u,v> = bits-2*hamming),
  *       brute force on tiny inputs.  The majority-vote block code is not in
  *       the reference: parity unpinned beyond its closed form.
+ *   orc_kvstar_*: PARITY UNPINNED against a build of the reference (its
+ *       translation unit needs spdlog, absent here).  Pinned by what the
+ *       mathematics fixes: an fp64 softmax-vote in numpy, sum(final) = number
+ *       of (token, head) rows, shift invariance, brute force on tiny inputs,
+ *       and the half-precision conversions against numpy's float16.
  */
 #include <float.h>
 #include <math.h>
@@ -696,4 +701,142 @@ ORC_API int32_t orc_topk_windows_i32(const int32_t* scores, uint32_t n, uint32_t
     const int32_t c = orc_topk_windows(f, n, k, startW, endW, out);
     free(f);
     return c;
+}
+
+/* ------------------------------------------------ KVStar softmax-vote retrieval */
+
+/* IEEE binary16 <-> binary32, round-to-nearest-even, subnormals kept */
+ORC_API float orc_f16_to_f32(uint16_t h)
+{
+    const uint32_t s = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu, u;
+    if (e == 0) {
+        if (m == 0) { u = s; }
+        else {
+            int shift = 0;
+            while ((m & 0x400u) == 0) { m <<= 1; ++shift; }
+            u = s | ((uint32_t)(113 - shift) << 23) | ((m & 0x3ffu) << 13);
+        }
+    } else if (e == 0x1fu) { u = s | 0x7f800000u | (m << 13); }
+    else { u = s | ((e + 112u) << 23) | (m << 13); }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+ORC_API uint16_t orc_f32_to_f16(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t s = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) { return (uint16_t)(s | 0x7e00u); }            /* NaN */
+    if (a >= 0x477ff000u) { return (uint16_t)(s | 0x7c00u); }           /* rounds to inf (>= 65520) */
+    if (a < 0x33000001u) { return s; }                                  /* <= 2^-25: rounds to zero */
+    int32_t e = (int32_t)(a >> 23) - 127;
+    uint32_t m = (a & 0x7fffffu) | 0x800000u;                           /* 24-bit significand */
+    int shift = e >= -14 ? 13 : 13 + (-14 - e);                         /* bits dropped */
+    uint32_t q = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) { ++q; }
+    if (e >= -14) { return (uint16_t)(s | (uint16_t)(((uint32_t)(e + 15) << 10) + (q - 0x400u))); }
+    return (uint16_t)(s | (uint16_t)q);                                 /* subnormal (a carry makes 2^-14) */
+}
+
+/*
+ * Sub-block representatives of KVStar (ucm/sparse/kvstar/multistep.py:279-316):
+ * for each listed cache block, the `merge` consecutive tokens of each of the
+ * M = block_size / merge sub-blocks are averaged per (kv head, kept channel);
+ * the reference does this with torch's mean in the model dtype (bf16) and then
+ * casts to fp16 (:495-497).  Restated as: fp32 sum in token order, * (1/merge),
+ * round to bf16, round to fp16.  (torch's own summation order is not pinned; the
+ * result can differ from it by one bf16 ulp.)
+ *   cache   bf16 [num_blocks][block_size][kv_heads][head_dim]
+ *   pruned  int32 [kv_heads][d_pruned] channel of each kept dim, or NULL (d_pruned == head_dim)
+ *   repre   fp16 [rows][M][kv_heads][d_pad], d_pad >= d_pruned; the pad is zero
+ */
+ORC_API void orc_kvstar_block_repre(const uint16_t* cache, const int32_t* block_ids, const int32_t* slots, uint32_t n,
+                                    uint32_t block_size, uint32_t kv_heads, uint32_t head_dim, uint32_t merge,
+                                    const int32_t* pruned, uint32_t d_pruned, uint32_t d_pad, uint16_t* repre)
+{
+    const uint32_t M = block_size / merge;
+    const float inv = 1.0f / (float)merge;
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint16_t* blk = cache + (size_t)block_ids[i] * block_size * kv_heads * head_dim;
+        uint16_t* out = repre + (size_t)slots[i] * M * kv_heads * d_pad;
+        for (uint32_t m = 0; m < M; ++m) {
+            for (uint32_t h = 0; h < kv_heads; ++h) {
+                for (uint32_t p = 0; p < d_pad; ++p) {
+                    uint16_t v = 0;
+                    if (p < d_pruned) {
+                        const uint32_t d = pruned ? (uint32_t)pruned[h * d_pruned + p] : p;
+                        float acc = orc_bf16_to_f32(blk[((size_t)(m * merge) * kv_heads + h) * head_dim + d]);
+                        for (uint32_t t = 1; t < merge; ++t) {
+                            acc = acc + orc_bf16_to_f32(blk[((size_t)(m * merge + t) * kv_heads + h) * head_dim + d]);
+                        }
+                        acc = acc * inv;
+                        v = orc_f32_to_f16(orc_bf16_to_f32(orc_f32_to_bf16(acc)));
+                    }
+                    out[((size_t)m * kv_heads + h) * d_pad + p] = v;
+                }
+            }
+        }
+    }
+}
+
+/*
+ * The retrieval itself, following the reference's portable path
+ * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:817-990,
+ * scalar_impl::execute_impl; its AVX2 and NEON twins at :635-764 and :270-390
+ * compute the same quantity with other summation orders and a polynomial exp):
+ *   score[x][H][s] = sum_d q[x][H][dp(d)] * k[s][h(H)][d]      fp32, d ascending, mul then add
+ *   p = softmax over s of each (x, H) row                        max, expf, sum in s order, divide
+ *   final[n] = sum over rows, then over the M sub-blocks of block n, of p     row-major order
+ *   top-k of final: the min-heap of :953-975 replaces its smallest entry only
+ *   by a strictly larger score, so of equal scores at the threshold the lower
+ *   index stays; the AVX2 twin uses std::nth_element (unordered, ties
+ *   unspecified).  Defined here: descending score, lower index first.
+ *   q      fp16 [x][H][d_orig]; pruned as above (the query is gathered by it)
+ *   repre  fp16 [n_blocks][M][kv_heads][d_pad] (d_pad >= d_pruned, pad ignored)
+ *   final  fp32 [n_blocks] out; topk_idx int32 [min(topk, n_blocks)] out; returns the count
+ */
+ORC_API int32_t orc_kvstar_retrieve(const uint16_t* q, uint32_t n_tokens, uint32_t q_heads, uint32_t d_orig,
+                                    const uint16_t* repre, uint32_t n_blocks, uint32_t M, uint32_t kv_heads,
+                                    uint32_t d_pruned, uint32_t d_pad, const int32_t* pruned, uint32_t topk,
+                                    float* final_scores, int32_t* topk_idx)
+{
+    const uint32_t g = q_heads / kv_heads, S = n_blocks * M;
+    float* row = (float*)malloc((size_t)(S ? S : 1) * sizeof(float));
+    float* qv = (float*)malloc((size_t)d_pruned * sizeof(float));
+    for (uint32_t b = 0; b < n_blocks; ++b) { final_scores[b] = 0.0f; }
+    for (uint32_t x = 0; x < n_tokens; ++x) {
+        for (uint32_t H = 0; H < q_heads; ++H) {
+            const uint32_t h = H / g;
+            for (uint32_t p = 0; p < d_pruned; ++p) {
+                const uint32_t d = pruned ? (uint32_t)pruned[h * d_pruned + p] : p;
+                qv[p] = orc_f16_to_f32(q[((size_t)x * q_heads + H) * d_orig + d]);
+            }
+            for (uint32_t s = 0; s < S; ++s) {
+                const uint16_t* kvec = repre + ((size_t)s * kv_heads + h) * d_pad;
+                float sc = 0.0f;
+                for (uint32_t p = 0; p < d_pruned; ++p) { sc = sc + qv[p] * orc_f16_to_f32(kvec[p]); }
+                row[s] = sc;
+            }
+            if (S == 0) { continue; }
+            float mx = row[0];
+            for (uint32_t s = 1; s < S; ++s) { if (row[s] > mx) { mx = row[s]; } }
+            float sum = 0.0f;
+            for (uint32_t s = 0; s < S; ++s) { row[s] = expf(row[s] - mx); sum = sum + row[s]; }
+            if (sum > 1e-9f) { for (uint32_t s = 0; s < S; ++s) { row[s] = row[s] / sum; } }
+            for (uint32_t s = 0; s < S; ++s) { final_scores[s / M] = final_scores[s / M] + row[s]; }
+        }
+    }
+    free(row);
+    free(qv);
+    const uint32_t k = topk < n_blocks ? topk : n_blocks;
+    orc_pair* pr = (orc_pair*)malloc((size_t)(n_blocks ? n_blocks : 1) * sizeof(orc_pair));
+    for (uint32_t b = 0; b < n_blocks; ++b) { pr[b].score = final_scores[b]; pr[b].idx = (int32_t)b; pr[b].pos = b; }
+    qsort(pr, n_blocks, sizeof(orc_pair), orc_cmp_pair_desc);
+    for (uint32_t i = 0; i < k; ++i) { topk_idx[i] = pr[i].idx; }
+    free(pr);
+    return (int32_t)k;
 }

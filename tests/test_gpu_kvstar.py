@@ -1,0 +1,173 @@
+"""KVStar softmax-vote retrieval: HIP kernels against the CPU oracle (fp32, tolerance stated per check)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+import synth
+
+pytestmark = pytest.mark.gpu
+
+# votes are sums of softmax probabilities; kernel and oracle differ in fp32 summation order and in exp()
+VOTE_RTOL, VOTE_ATOL = 2e-4, 2e-6
+
+
+def f16_bits(a):
+    return np.ascontiguousarray(a, np.float32).astype(np.float16).view(np.uint16)
+
+
+def dev_f16(bits, dev):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(dev).view(torch.float16)
+
+
+def check_selection(got_idx, want_final, k):
+    """The selected set may differ from the oracle's only by blocks whose votes tie within tolerance."""
+    n = len(want_final)
+    k = min(k, n)
+    assert len(got_idx) == k and len(set(got_idx)) == k
+    if k == 0:
+        return
+    order = np.argsort(-want_final, kind="stable")
+    kth = want_final[order[k - 1]]
+    tol = VOTE_ATOL + VOTE_RTOL * abs(kth) * 4
+    for i in got_idx:
+        assert want_final[i] >= kth - tol, (i, want_final[i], kth)
+    for i in order[:k]:
+        if want_final[i] > kth + tol:
+            assert i in got_idx, (i, want_final[i], kth)
+
+
+@pytest.mark.parametrize("merge,hkv,d,bs", [(16, 8, 128, 128), (32, 2, 64, 128), (4, 4, 128, 16), (128, 1, 128, 128), (16, 2, 128, 32)])
+def test_kvstar_block_repre(ucm, dev, merge, hkv, d, bs):
+    from ucm_amd import ops
+
+    n_layers, nb, rows = 2, 11, 14
+    caches_h = [synth.normal_bf16_bits(1000 + l, (nb, bs, hkv, d)) for l in range(n_layers)]
+    caches = [torch.from_numpy(c.view(np.int16)).to(dev).view(torch.bfloat16) for c in caches_h]
+    lp = ops.LayerPointers(caches)
+    ids = synth.permutation(1010, nb)[:9].astype(np.int32)
+    slots = synth.permutation(1011, rows)[:9].astype(np.int32)
+    M = bs // merge
+    for d_pruned in (d, d - 13, 16):
+        pruned = None if d_pruned == d else np.stack([synth.permutation(1020 + h, d)[:d_pruned] for h in range(hkv)]).astype(np.int32)
+        d_pad = (d_pruned + 15) // 16 * 16
+        repre = torch.full((n_layers, rows, M, hkv, d_pad), 3.0, dtype=torch.float16, device=dev)
+        ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge,
+                               pruned=None if pruned is None else torch.from_numpy(pruned).to(dev))
+        got = repre.view(torch.int16).cpu().numpy().view(np.uint16)
+        for l in range(n_layers):
+            want = np.full((rows, M, hkv, d_pad), np.float16(3.0).view(np.uint16), np.uint16)
+            O.kvstar_block_repre(caches_h[l], ids, slots, merge, want, pruned=pruned)
+            assert np.array_equal(got[l], want), (d_pruned, l)
+    # against torch's own mean in the model dtype (what the reference calls): equal up to one bf16 step of the summation order
+    t = caches[0][torch.from_numpy(ids.astype(np.int64)).to(dev)].reshape(9, M, merge, hkv, d).mean(dim=2).to(torch.float16)
+    repre = torch.zeros((n_layers, rows, M, hkv, d), dtype=torch.float16, device=dev)
+    ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge)
+    mine = repre[0][torch.from_numpy(slots.astype(np.int64)).to(dev)]
+    assert torch.allclose(mine.float(), t.float(), rtol=2 ** -7, atol=1e-6)
+
+
+def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None, pruned_sel=None, d_pruned=None):
+    """q_bits_list: per task uint16 [x, hq, d]; repre_bits uint16 [rows, M, hkv, d_pad]; tasks own consecutive row ranges."""
+    lens = np.asarray(lens, np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    q = dev_f16(np.stack(q_bits_list), dev)
+    q_off = torch.arange(len(lens), dtype=torch.int64, device=dev) * q[0].numel()
+    table = dev_f16(repre_bits, dev)
+    rows, M, hkv, _ = repre_bits.shape
+    votes = torch.full((rows,), -7.0, device=dev)
+    ws = ops.kvstar_workspace(len(lens), hkv, int(lens.max(initial=0)), M, dev)
+    ops.kvstar_votes(q, q_off, n_tokens, hq, table, torch.from_numpy(off).to(dev), torch.from_numpy(lens).to(dev),
+                     int(lens.max(initial=0)), votes, ws, d_pruned=d_pruned,
+                     pruned=None if pruned is None else torch.from_numpy(pruned).to(dev),
+                     pruned_sel=None if pruned_sel is None else torch.tensor(pruned_sel, dtype=torch.int32, device=dev))
+    torch.cuda.synchronize()
+    return votes.cpu().numpy(), off
+
+
+@pytest.mark.parametrize("x,hq,hkv,d,M", [(8, 32, 8, 128, 8), (8, 16, 2, 64, 4), (3, 8, 8, 128, 1), (1, 4, 1, 128, 32),
+                                          (5, 24, 4, 96, 2), (8, 64, 8, 128, 16)])
+def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
+    from ucm_amd import ops
+
+    lens = [37, 1, 0, 130, 64, 257] if M <= 8 else [37, 1, 0, 70]
+    rows = int(np.sum(lens))
+    scale = np.float32(0.25)                                  # keeps the softmax from collapsing onto one sub-block
+    repre = f16_bits(synth.normal_f32(1100, (rows, M, hkv, d)) * scale)
+    qs = [f16_bits(synth.normal_f32(1101 + t, (x, hq, d)) * scale) for t in range(len(lens))]
+    got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
+    for t, n in enumerate(lens):
+        if n == 0:
+            continue
+        idx, want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=max(n // 3, 1))
+        assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
+        # what the mathematics fixes whatever the order: every row's probabilities add up to one
+        assert abs(got[off[t] : off[t] + n].sum() - x * hq) < 1e-3 * x * hq
+    assert np.all(got[off[2] : off[2]] == -7.0)              # the empty task writes nothing
+
+
+def test_kvstar_pruned_channels_and_selection(ucm, dev):
+    from ucm_amd import ops
+
+    x, hq, hkv, d, M, dp = 8, 32, 8, 128, 8, 77              # 77 kept channels: table rows padded to 80
+    lens = [90, 33]
+    rows = int(np.sum(lens))
+    pruned = np.stack([[synth.permutation(1200 + 10 * t + h, d)[:dp] for h in range(hkv)] for t in range(2)]).astype(np.int32)
+    d_pad = 80
+    repre = np.zeros((rows, M, hkv, d_pad), np.uint16)
+    repre[..., :dp] = f16_bits(synth.normal_f32(1201, (rows, M, hkv, dp)) * np.float32(0.3))
+    qs = [f16_bits(synth.normal_f32(1202 + t, (x, hq, d)) * np.float32(0.3)) for t in range(2)]
+    got, off = run_votes(ops, dev, qs, repre, lens, x, hq, pruned=pruned, pruned_sel=[1, 0])
+    for t, n in enumerate(lens):
+        sel = [1, 0][t]
+        idx, want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=n // 4, pruned=pruned[sel])
+        assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), t
+        k = n // 4
+        seg_off, seg_len = torch.tensor([off[t]], dtype=torch.int32, device=dev), torch.tensor([n], dtype=torch.int32, device=dev)
+        out = torch.zeros((1, 1, n), dtype=torch.int32, device=dev)
+        cnt = torch.zeros((1, 1), dtype=torch.int32, device=dev)
+        ops.topk_windows(torch.from_numpy(got).to(dev).view(1, -1), seg_off, seg_len, torch.tensor([k], dtype=torch.int32, device=dev),
+                         n, out, cnt, start_w=0, end_w=0)
+        check_selection(out[0, 0, : int(cnt[0, 0])].tolist(), want, k)
+
+
+def test_kvstar_retrieve_module_surface(ucm, dev):
+    """The reference's kvstar_retrieve calls, on device tensors: keys -> sub-block means (with channel pruning)
+    -> AsyncRetrieveByCPU / Wait / GetTaskResult."""
+    from ucm_amd.sparse.kvstar import retrieve as kvstar_retrieve
+
+    hq, hkv, d, bs, nb, merge = 16, 4, 128, 32, 40, 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    k_cache = (torch.randn(nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+    ids = [int(i) for i in synth.permutation(1300, nb)[:30]]
+    kvstar_retrieve.Setup(kvstar_retrieve.SetupParam([0], 8, 0.5, 0, kvstar_retrieve.CPU, 1, 0))
+    for ratio in (1.0, 0.6):
+        repre, index = kvstar_retrieve.extract_block_repre(k_cache, ids, merge, prune_ratio=ratio, prune_dim_enable=True)
+        dp = round(d * ratio)
+        assert repre.shape == (30, bs // merge, hkv, (dp + 15) // 16 * 16) and repre.dtype == torch.float16
+        assert (index is None) == (ratio == 1.0)
+        cache_bits = k_cache.view(torch.int16).cpu().numpy().view(np.uint16)
+        want = np.zeros(tuple(repre.shape), np.uint16)
+        pr = None if index is None else index.cpu().numpy().astype(np.int32)
+        O.kvstar_block_repre(cache_bits, ids, np.arange(30), merge, want, pruned=pr)
+        assert np.array_equal(repre.view(torch.int16).cpu().numpy().view(np.uint16), want)
+        if index is not None:                                  # the kept channels are those with the largest mean |k|
+            am = k_cache[torch.tensor(ids, device=dev)].reshape(-1, hkv, d).float().abs().mean(0)
+            assert torch.equal(index, torch.topk(am, dp, dim=-1).indices)
+        blk = repre[1:-2][..., :dp].contiguous()               # the reference keeps [init:-local] (multistep.py:495-497)
+        q = (torch.randn(8, hq, d, device=dev, generator=g) * 0.3).to(torch.float16)
+        tid = kvstar_retrieve.AsyncRetrieveByCPU(q, blk, index, 9, 7, kvstar_retrieve.CPU)
+        kvstar_retrieve.Wait(tid)
+        res = kvstar_retrieve.GetTaskResult(tid)
+        assert res["status"] == "SUCCESS" and len(res["data"]) == 9
+        padded = want[1:-2]
+        idx, final = O.kvstar_retrieve(q.view(torch.int16).cpu().numpy().view(np.uint16), padded, 9, pruned=pr, d_pruned=dp)
+        check_selection(res["data"], final, 9)
+        assert all(final[a] >= final[b] - 1e-5 for a, b in zip(res["data"], res["data"][1:]))   # descending votes
+    # errors arrive through the task result, with the reference's messages
+    bad = kvstar_retrieve.AsyncRetrieveByCPU(q[0], blk, index, 3, 7, kvstar_retrieve.CPU)
+    assert kvstar_retrieve.GetTaskResult(bad) == {"status": "FAILURE", "error": "Query shape must be 3D (x, H, d)."}
+    bad = kvstar_retrieve.AsyncRetrieveByCPU(q[:, :6], blk, index, 3, 7, kvstar_retrieve.CPU)
+    assert kvstar_retrieve.GetTaskResult(bad)["error"] == "Num_q_heads must be a divisible by num_kv_heads."
+    assert kvstar_retrieve.GetTaskResult(123456) is None

@@ -323,3 +323,102 @@ def test_delta_plan_against_set_arithmetic():
         # misses fill freed slots in ascending order
         filled = [j for j in range(n_slots) if load[j] >= 0]
         assert [resident[j] for j in filled] == sorted(new - old)
+
+
+def test_half_conversions_against_numpy():
+    """orc_f16_to_f32 over every bit pattern, orc_f32_to_f16 on values around every rounding boundary."""
+    allh = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    want = allh.view(np.float16).astype(np.float32)
+    for h in range(65536):
+        got = O.f16_to_f32(h)
+        assert (np.isnan(got) and np.isnan(want[h])) or got == want[h], h
+    rng = np.random.default_rng(5)
+    vals = [0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001, 6.1e-5, 6.0e-5, 2.0 ** -14]
+    vals += list(rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000).astype(np.float32))
+    # exact midpoints between neighbouring halves (ties to even) and their float neighbours
+    for h in rng.integers(0, 0x7bff, 2000):
+        a, b = np.uint16(h).view(np.float16).astype(np.float32), np.uint16(h + 1).view(np.float16).astype(np.float32)
+        mid = np.float32((np.float64(a) + np.float64(b)) / 2)
+        vals += [mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9)), -mid]
+    with np.errstate(over="ignore"):
+        for v in vals:
+            v = np.float32(v)
+            assert O.f32_to_f16(float(v)) == int(v.astype(np.float16).view(np.uint16)), v
+
+
+def _votes_fp64(q, rep):
+    """Softmax-vote in float64 straight from its definition."""
+    x, hq, d = q.shape
+    n, m, hkv, _ = rep.shape
+    g = hq // hkv
+    keys = rep.astype(np.float64).reshape(n * m, hkv, -1)
+    votes = np.zeros(n)
+    for t in range(x):
+        for head in range(hq):
+            s = keys[:, head // g, :] @ q[t, head].astype(np.float64)
+            p = np.exp(s - s.max())
+            votes += (p / p.sum()).reshape(n, m).sum(1)
+    return votes
+
+
+def test_kvstar_retrieve_closed_forms():
+    """No build of the reference pins the KVStar restatement (it needs spdlog); what does: the definition
+    evaluated in float64, sum(votes) = rows, invariance under a per-row shift of the scores, the channel
+    gather, sub-block means by hand, brute force on a tiny case with a tie."""
+    for seed, (x, hq, hkv, d, m, n) in enumerate([(5, 8, 2, 64, 4, 23), (1, 4, 4, 16, 1, 7), (8, 32, 8, 128, 8, 40), (3, 6, 3, 48, 2, 1)]):
+        rep = (synth.normal_f32(40 + seed, (n, m, hkv, d)) * np.float32(0.3)).astype(np.float16)
+        q = (synth.normal_f32(50 + seed, (x, hq, d)) * np.float32(0.3)).astype(np.float16)
+        k = max(n // 3, 1)
+        idx, final = O.kvstar_retrieve(q.view(np.uint16), rep.view(np.uint16), k)
+        want = _votes_fp64(q, rep)
+        assert np.allclose(final, want, rtol=1e-5, atol=1e-6)
+        assert abs(final.sum() - x * hq) < 1e-4 * x * hq
+        assert list(idx) == list(np.argsort(-want, kind="stable")[:k]) or np.min(np.diff(np.sort(want))) < 1e-6
+        # a dropped or transposed head mapping would show here: zeroing the keys of one kv head flattens its rows' softmax
+        rep0 = rep.copy()
+        rep0[:, :, 0, :] = 0
+        _, f0 = O.kvstar_retrieve(q.view(np.uint16), rep0.view(np.uint16), k)
+        assert np.allclose(f0, _votes_fp64(q, rep0), rtol=1e-5, atol=1e-6)
+        # channel gather: scoring pruned keys against the full query equals scoring them against the gathered query
+        dp = max(d // 2, 1)
+        pr = np.stack([synth.permutation(60 + seed * 8 + h, d)[:dp] for h in range(hkv)]).astype(np.int32)
+        rep_p = np.ascontiguousarray(rep[..., :dp])
+        _, fp = O.kvstar_retrieve(q.view(np.uint16), rep_p.view(np.uint16), k, pruned=pr)
+        g = hq // hkv
+        q_g = np.stack([q[:, h, :][:, pr[h // g]] for h in range(hq)], axis=1)
+        assert np.allclose(fp, _votes_fp64(q_g, rep_p), rtol=1e-5, atol=1e-6)
+        # padded table columns are ignored
+        pad = np.zeros((n, m, hkv, dp + 5), np.float16)
+        pad[..., :dp] = rep_p
+        pad[..., dp:] = 9.0
+        _, fpad = O.kvstar_retrieve(q.view(np.uint16), pad.view(np.uint16), k, pruned=pr)
+        assert np.array_equal(fpad, fp)
+    # ties: identical blocks get identical votes and the lower index comes first
+    rep = np.zeros((4, 2, 1, 16), np.float16)
+    rep[1] = rep[3] = 0.5
+    q = np.ones((1, 1, 16), np.float16)
+    idx, final = O.kvstar_retrieve(q.view(np.uint16), rep.view(np.uint16), 3)
+    assert final[1] == final[3] and final[0] == final[2] and list(idx) == [1, 3, 0]
+
+
+def test_kvstar_block_repre_by_hand():
+    bs, hkv, d, merge = 8, 2, 4, 4
+    cache = synth.normal_bf16_bits(70, (3, bs, hkv, d))
+    out = np.zeros((5, bs // merge, hkv, 16), np.uint16)
+    pr = np.array([[2, 0, 3], [1, 3, 0]], np.int32)
+    O.kvstar_block_repre(cache, [2, 0], [4, 1], merge, out, pruned=pr)
+    wide = synth.bf16_widen(cache)
+    for blk, slot in ((2, 4), (0, 1)):
+        for m in range(bs // merge):
+            for h in range(hkv):
+                for p in range(3):
+                    acc = np.float32(0)
+                    vals = wide[blk, m * merge : (m + 1) * merge, h, pr[h, p]]
+                    acc = vals[0]
+                    for v in vals[1:]:
+                        acc = np.float32(acc + v)
+                    acc = np.float32(acc * np.float32(1.0 / merge))
+                    b16 = synth.bf16_widen(synth.bf16_round_bits(np.array([acc], np.float32)))[0]
+                    assert out[slot, m, h, p] == np.float32(b16).astype(np.float16).view(np.uint16)
+                assert not out[slot, m, h, 3:].any()
+    assert not out[[0, 2, 3]].any()

@@ -291,6 +291,63 @@ def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, 
               _staging_ptr(staging, staging_blocks * block_bytes), _stream())
 
 
+def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
+                       block_size: int, kv_heads: int, head_dim: int, num_blocks: int, merge: int,
+                       pruned: Optional[torch.Tensor] = None) -> None:
+    """repre fp16 [L, rows, M, kv_heads, d_pad]; pruned int32 [kv_heads, d_pruned] or None."""
+    if repre.dim() != 5 or repre.dtype != torch.float16 or repre.shape[2] * merge != block_size or repre.shape[3] != kv_heads:
+        raise ValueError("repre must be float16 [L, rows, block_size/merge, kv_heads, d_pad]")
+    if len(k_layers) != repre.shape[0]:
+        raise ValueError("one table layer per cache layer")
+    if block_ids.numel() != slots.numel():
+        raise ValueError("block_ids and slots differ in length")
+    d_pruned = head_dim if pruned is None else pruned.shape[1]
+    if pruned is not None and pruned.shape[0] != kv_heads:
+        raise ValueError("pruned must be [kv_heads, d_pruned]")
+    _lib.call("ucm_kvstar_block_repre", k_layers.ptr(), repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
+              _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
+              _opt(pruned, torch.int32, "pruned"), d_pruned, repre.shape[4], _dev(repre, torch.float16, "repre"),
+              repre.shape[1], repre.stride(0), _stream())
+
+
+def kvstar_workspace(n_tasks: int, kv_heads: int, max_blocks: int, sub_blocks: int, device) -> tuple:
+    import ctypes as C
+
+    a, b = C.c_int64(0), C.c_int64(0)
+    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, max_blocks, sub_blocks, C.addressof(a), C.addressof(b))
+    return (torch.empty(max(a.value, 1), dtype=torch.float32, device=device),
+            torch.empty(max(b.value, 1), dtype=torch.float32, device=device))
+
+
+def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: int, repre: torch.Tensor,
+                 seg_off: torch.Tensor, seg_len: torch.Tensor, max_blocks: int, votes: torch.Tensor, workspace: tuple,
+                 d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
+                 pruned_sel: Optional[torch.Tensor] = None) -> None:
+    """q fp16 (any shape; task t reads [n_tokens, q_heads, d_orig] from element q_off[t]); repre fp16
+    [rows, M, kv_heads, d_pad]; votes fp32 [>= rows]; pruned int32 [n_lists, kv_heads, d_pruned]."""
+    if repre.dim() != 4 or repre.dtype != torch.float16:
+        raise ValueError("repre must be float16 [rows, M, kv_heads, d_pad]")
+    d_orig = q.shape[-1]
+    n_tasks = seg_off.numel()
+    if seg_len.numel() != n_tasks or q_off.numel() != n_tasks:
+        raise ValueError("q_off / seg_off / seg_len differ in length")
+    if pruned is not None:
+        if pruned.dim() != 3 or pruned.shape[1] != repre.shape[2] or pruned_sel is None or pruned_sel.numel() != n_tasks:
+            raise ValueError("pruned must be [n_lists, kv_heads, d_pruned] with one pruned_sel entry per task")
+        d_pruned = pruned.shape[2]
+    elif d_pruned is None:
+        d_pruned = d_orig
+    if votes.numel() < repre.shape[0]:
+        raise ValueError("votes shorter than the representative table")
+    ws_max, ws_part = workspace
+    _lib.call("ucm_kvstar_votes", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
+              _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"),
+              _dev(repre, torch.float16, "repre"), _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
+              n_tasks, max_blocks, repre.shape[1], repre.shape[2], d_pruned, repre.shape[3],
+              _dev(ws_max, torch.float32, "ws_max"), _dev(ws_part, torch.float32, "ws_part"),
+              _dev(votes, torch.float32, "votes"), _stream())
+
+
 def set_score_tile(tile_blocks: int) -> None:
     _lib.call("ucm_set_score_tile", tile_blocks)
 
