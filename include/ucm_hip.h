@@ -293,7 +293,7 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   repre_f16  dev fp16 [rows][sub_blocks][kv_heads][d_pad]; task t owns rows
  *            seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >= every seg_len
  *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
- *            returns; votes dev fp32, task t's votes at votes[seg_off[t] + b].
+ *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev fp32, task t's votes at votes[seg_off[t] + b].
  * n_tokens * (q_heads/kv_heads) <= 64, kv_heads <= 8, d_pad a multiple of 16
  * and <= 128, sub_blocks in {1, 2, 4, 8, 16, 32}.
  */
@@ -302,8 +302,11 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
                            int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
                            int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
                            ucm_stream_t stream);
-int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int max_blocks, int sub_blocks,
-                                int64_t* max_floats, int64_t* part_floats);
+/* Tuning knob for benchmarks: kv heads per workgroup of the KVStar score kernel
+ * (1..8, default 1).  Not part of the reference interface. */
+int ucm_set_kvstar_heads_per_group(int heads);
+int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks,
+                                int sub_blocks, int64_t* max_floats, int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                      const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
                      const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,

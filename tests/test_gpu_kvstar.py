@@ -76,7 +76,7 @@ def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None
     table = dev_f16(repre_bits, dev)
     rows, M, hkv, _ = repre_bits.shape
     votes = torch.full((rows,), -7.0, device=dev)
-    ws = ops.kvstar_workspace(len(lens), hkv, int(lens.max(initial=0)), M, dev)
+    ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, dev)
     ops.kvstar_votes(q, q_off, n_tokens, hq, table, torch.from_numpy(off).to(dev), torch.from_numpy(lens).to(dev),
                      int(lens.max(initial=0)), votes, ws, d_pruned=d_pruned,
                      pruned=None if pruned is None else torch.from_numpy(pruned).to(dev),
@@ -95,15 +95,20 @@ def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
     scale = np.float32(0.25)                                  # keeps the softmax from collapsing onto one sub-block
     repre = f16_bits(synth.normal_f32(1100, (rows, M, hkv, d)) * scale)
     qs = [f16_bits(synth.normal_f32(1101 + t, (x, hq, d)) * scale) for t in range(len(lens))]
-    got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
-    for t, n in enumerate(lens):
-        if n == 0:
-            continue
-        idx, want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=max(n // 3, 1))
-        assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
-        # what the mathematics fixes whatever the order: every row's probabilities add up to one
-        assert abs(got[off[t] : off[t] + n].sum() - x * hq) < 1e-3 * x * hq
-    assert np.all(got[off[2] : off[2]] == -7.0)              # the empty task writes nothing
+    wants = {t: O.kvstar_retrieve(qs[t], repre[sum(lens[:t]) : sum(lens[:t]) + n], topk=max(n // 3, 1))[1]
+             for t, n in enumerate(lens) if n}
+    try:
+        for heads_per_group in (1, 3, 8):                     # kv heads one workgroup walks
+            ops.set_kvstar_heads_per_group(heads_per_group)
+            got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
+            for t, n in enumerate(lens):
+                if n == 0:
+                    continue
+                assert np.allclose(got[off[t] : off[t] + n], wants[t], rtol=VOTE_RTOL, atol=VOTE_ATOL), (heads_per_group, t, n)
+                # what the mathematics fixes whatever the order: every row's probabilities add up to one
+                assert abs(got[off[t] : off[t] + n].sum() - x * hq) < 1e-3 * x * hq
+    finally:
+        ops.set_kvstar_heads_per_group(1)
 
 
 def test_kvstar_pruned_channels_and_selection(ucm, dev):

@@ -36,8 +36,7 @@ constexpr int kWaves = 4;
 constexpr int kMaxRows = 64;          // tokens * group size per kv head
 constexpr int kMaxDim = 128;
 constexpr int kQStride = kMaxDim + 8; // fp16 elements per staged query row (272 B: spreads LDS banks)
-constexpr int kTilesPerWave = 8;      // 32-sub-block tiles a wave walks per workgroup
-constexpr int kChunk = kWaves * kTilesPerWave * 32;
+constexpr int kTileSub = 32;          // sub-blocks per MFMA tile
 
 __device__ __forceinline__ unsigned short f32_to_f16_bits(float f)
 {
@@ -135,37 +134,59 @@ __device__ __forceinline__ void block_sums(const float (&e)[16], int half, float
     }
 }
 
-// grid: x = chunk of kChunk sub-blocks, y = kv head, z = task
-template <int kM>
-__global__ __launch_bounds__(kThreads) void kvstar_score_kernel(
+// grid: x = chunk of sub-blocks, y = group of kv heads, z = task.  A workgroup walks the heads of its
+// group for its sub-blocks (a sub-block's vectors of all kv heads lie side by side in the table:
+// kv_heads * d_pad * 2 bytes, 2 KiB at 8 x 128); the queries of those heads are staged in LDS once
+// per workgroup.  The host picks the group size (one head by default, see ucm_kvstar_votes).
+template <int kM, bool kTwoRowTiles>
+__global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_kernel(
     const unsigned short* __restrict__ q, const int64_t* __restrict__ q_off, unsigned n_tokens, unsigned q_heads,
     unsigned d_orig, const int32_t* __restrict__ pruned, const int32_t* __restrict__ pruned_sel,
     const unsigned short* __restrict__ table, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad,
-    float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles)
+    float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
+    unsigned tiles_per_wave, unsigned row_pad, unsigned heads_per_group)
 {
-    __shared__ __attribute__((aligned(16))) unsigned short q_s[kMaxRows * kQStride];
+    extern __shared__ __attribute__((aligned(16))) unsigned short q_s[];   // [heads_per_group][row_pad][kQStride]
 
-    const unsigned task = blockIdx.z, h = blockIdx.y;
+    const unsigned task = blockIdx.z;
+    const unsigned h_first = blockIdx.y * heads_per_group;
+    const unsigned nh = min(heads_per_group, kv_heads - h_first);
     const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
     const unsigned S = n_blocks * kM;
-    const unsigned s_chunk = blockIdx.x * kChunk;
+    const unsigned chunk = kWaves * tiles_per_wave * kTileSub;
+    const unsigned s_chunk = blockIdx.x * chunk;
     if (s_chunk >= S) { return; }
     const unsigned g = q_heads / kv_heads, R = n_tokens * g;
     const int32_t psel = pruned_sel ? pruned_sel[task] : -1;
-    const int32_t* pr = (pruned && psel >= 0) ? pruned + (static_cast<size_t>(psel) * kv_heads + h) * d_pruned : nullptr;
+    const int32_t* pr0 = (pruned && psel >= 0) ? pruned + static_cast<size_t>(psel) * kv_heads * d_pruned : nullptr;
 
-    // ---- this head's query rows, gathered by the kept channels, zero padded
+    // ---- the group's query rows, gathered by the kept channels, zero padded (rows up to row_pad, columns up to d_pad)
     const unsigned short* qt = q + q_off[task];
-    for (unsigned e = threadIdx.x; e < kMaxRows * d_pad; e += kThreads) {
-        const unsigned rho = e / d_pad, p = e - rho * d_pad;
-        unsigned short v = 0;
-        if (rho < R && p < d_pruned) {
-            const unsigned xt = rho / g, gg = rho - xt * g;
-            const unsigned d = pr ? static_cast<unsigned>(pr[p]) : p;
-            if (d < d_orig) { v = qt[(static_cast<size_t>(xt) * q_heads + h * g + gg) * d_orig + d]; }
+    if (!pr0 && d_pruned == d_pad && (d_orig % 8) == 0 && (reinterpret_cast<uintptr_t>(qt) & 15u) == 0) {
+        const unsigned cpr = d_pad / 8;                  // 16-byte pieces per row
+        for (unsigned e = threadIdx.x; e < nh * row_pad * cpr; e += kThreads) {
+            const unsigned hr = e / cpr, c = e - hr * cpr;
+            const unsigned hh = hr / row_pad, rho = hr - hh * row_pad;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (rho < R) {
+                const unsigned xt = rho / g, gg = rho - xt * g;
+                v = ucm::gload16(qt + (static_cast<size_t>(xt) * q_heads + (h_first + hh) * g + gg) * d_orig + c * 8);
+            }
+            *reinterpret_cast<u32x4*>(&q_s[hr * kQStride + c * 8]) = v;
         }
-        q_s[rho * kQStride + p] = v;
+    } else {
+        for (unsigned e = threadIdx.x; e < nh * row_pad * d_pad; e += kThreads) {
+            const unsigned hr = e / d_pad, p = e - hr * d_pad;
+            const unsigned hh = hr / row_pad, rho = hr - hh * row_pad;
+            unsigned short v = 0;
+            if (rho < R && p < d_pruned) {
+                const unsigned xt = rho / g, gg = rho - xt * g;
+                const unsigned d = pr0 ? static_cast<unsigned>(pr0[(h_first + hh) * d_pruned + p]) : p;
+                if (d < d_orig) { v = qt[(static_cast<size_t>(xt) * q_heads + (h_first + hh) * g + gg) * d_orig + d]; }
+            }
+            q_s[hr * kQStride + p] = v;
+        }
     }
     __syncthreads();
 
@@ -173,116 +194,157 @@ __global__ __launch_bounds__(kThreads) void kvstar_score_kernel(
     const int half = lane >> 5, lr = lane & 31;
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes dims half*(d_pad/2) + ks*8 .. +8
     const unsigned hoff = half * (d_pad / 2);
-    const bool two_row_tiles = R > 32;
-    const unsigned short* tbase = table + static_cast<size_t>(seg_off[task]) * kM * kv_heads * d_pad + static_cast<size_t>(h) * d_pad;
+    constexpr bool two_row_tiles = kTwoRowTiles;   // 33..64 query rows per kv head
     const size_t vec_stride = static_cast<size_t>(kv_heads) * d_pad;
+    const unsigned short* tbase = table + static_cast<size_t>(seg_off[task]) * kM * vec_stride +
+                                  static_cast<size_t>(h_first) * d_pad + hoff;
 
-    float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h) * kMaxRows * max_tiles;
-    float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * kMaxRows * max_blocks;
-
-    for (unsigned t = wave; t < kWaves * kTilesPerWave; t += kWaves) {
-        const unsigned s0 = s_chunk + t * 32;
+    // A (tile, head) step's keys: eight 16-byte loads per lane, one contiguous half vector.  Everything is
+    // unconditional - MFMA steps past d_pad reload piece 0 and are multiplied with a zero query fragment,
+    // lanes and tiles past the end reload the last vector and are masked - so that the loads of the NEXT
+    // step can be issued before this step's arithmetic without a branch around them.
+    auto load_keys = [&](u32x4 (&kf)[kMaxDim / 16], unsigned s0, unsigned hh) {
+        const unsigned s_mine = min(s0 + lr, S - 1);
+        const unsigned short* krow = tbase + static_cast<size_t>(s_mine) * vec_stride + hh * d_pad;
+#pragma unroll
+        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = ucm::gload16(krow + (ks < ksteps ? ks : 0u) * 8); }
+    };
+    u32x4 kf[kMaxDim / 16], kn[kMaxDim / 16];
+    const unsigned t_end = kWaves * tiles_per_wave;
+    unsigned rot = (wave * 3u + blockIdx.x + task) % nh;
+    load_keys(kf, s_chunk + wave * kTileSub, rot);
+    for (unsigned t = wave; t < t_end; t += kWaves, rot = (rot + 1) % nh) {
+        const unsigned s0 = s_chunk + t * kTileSub;
         if (s0 >= S) { break; }
-        const unsigned s_mine = min(s0 + lr, S - 1);     // clamp: lanes past the end read a valid vector and are masked below
-        const unsigned short* krow = tbase + static_cast<size_t>(s_mine) * vec_stride + hoff;
-        u32x4 kf[kMaxDim / 16];
+        const unsigned tile = s0 / kTileSub;
+        for (unsigned hi = 0; hi < nh; ++hi) {
+            // heads are visited in an order rotated per wave and tile: consecutive vectors of one head are
+            // kv_heads*d_pad*2 bytes apart, so one head's loads fall on a fraction of the memory channels,
+            // and waves that all walked the heads in the same order would crowd onto the same ones
+            const unsigned hh = (hi + rot) % nh;
+            {   // one load site (selects, no branch): the next head of this tile, or the first head of the wave's next tile
+                const bool last = hi + 1 == nh;
+                load_keys(kn, last ? s0 + kWaves * kTileSub : s0, (last ? rot + 1 : hi + 1 + rot) % nh);
+            }
+            const unsigned short* qh = q_s + static_cast<size_t>(hh) * row_pad * kQStride;
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            f32x16 acc0, acc1;
 #pragma unroll
-        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-            if (ks < ksteps) { kf[ks] = ucm::gload16(krow + ks * 8); }
-        }
-        f32x16 acc0, acc1;
+            for (int i = 0; i < 16; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
+            for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
+                const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 8;
+                const u32x4 braw = *reinterpret_cast<const u32x4*>(&qh[lr * kQStride + col]);
+                const f16x8 b0 = __builtin_bit_cast(f16x8, ks < ksteps ? braw : zero);
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), b0, acc0, 0, 0, 0);
+            }
+            if (two_row_tiles) {
 #pragma unroll
-        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-            if (ks < ksteps) {
-                const f16x8 a = __builtin_bit_cast(f16x8, kf[ks]);
-                const f16x8 b0 = *reinterpret_cast<const f16x8*>(&q_s[lr * kQStride + hoff + ks * 8]);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0, 0, 0, 0);
-                if (two_row_tiles) {
-                    const f16x8 b1 = *reinterpret_cast<const f16x8*>(&q_s[(32 + lr) * kQStride + hoff + ks * 8]);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1, 0, 0, 0);
+                for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
+                    const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 8;
+                    const u32x4 braw = *reinterpret_cast<const u32x4*>(&qh[(32 + lr) * kQStride + col]);
+                    const f16x8 b1 = __builtin_bit_cast(f16x8, ks < ksteps ? braw : zero);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), b1, acc1, 0, 0, 0);
                 }
             }
-        }
-        const unsigned tile = s0 / 32;
+            float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h_first + hh) * row_pad * max_tiles;
+            float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h_first + hh) * row_pad * max_blocks;
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-            if (rt == 1 && !two_row_tiles) { break; }
-            const unsigned rho = rt * 32 + lr;
-            float sc[16];
-            float mx = -INFINITY;
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt == 1 && !two_row_tiles) { break; }
+                const unsigned rho = rt * 32 + lr;
+                float sc[16];
+                float mx = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
-                const float v = rt == 0 ? acc0[i] : acc1[i];
-                sc[i] = s < S ? v : -INFINITY;
-                mx = fmaxf(mx, sc[i]);
+                for (int i = 0; i < 16; ++i) {
+                    const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
+                    const float v = rt == 0 ? acc0[i] : acc1[i];
+                    sc[i] = s < S ? v : -INFINITY;
+                    mx = fmaxf(mx, sc[i]);
+                }
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the tile has at least one live sub-block, so mx is finite
+                float e[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { e[i] = __expf(sc[i] - mx); }
+                // rows past R hold zero queries: they are computed like the rest and never read
+                if (half == 0) { wmax[static_cast<size_t>(rho) * max_tiles + tile] = mx; }
+                block_sums<kM>(e, half, wpart + static_cast<size_t>(rho) * max_blocks, s0 / kM, n_blocks);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));      // the tile has at least one live sub-block, so mx is finite
-            float e[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { e[i] = __expf(sc[i] - mx); }
-            // rows past R hold zero queries: they are computed like the rest and never read
-            if (half == 0) { wmax[static_cast<size_t>(rho) * max_tiles + tile] = mx; }
-            block_sums<kM>(e, half, wpart + static_cast<size_t>(rho) * max_blocks, s0 / kM, n_blocks);
+            for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = kn[ks]; }
         }
     }
 }
 
 // ---- votes: rescale to the row maximum, normalise, add the rows ---------------------------------------
-// grid: x = task; one workgroup
-__global__ __launch_bounds__(kThreads) void kvstar_combine_kernel(
-    const float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, unsigned n_tokens, unsigned q_heads, unsigned kv_heads, unsigned M,
-    unsigned max_blocks, unsigned max_tiles, float* __restrict__ votes)
+// Phase 1, grid: x = (kv head, row) of the task, y = task; one wave per workgroup.  The row's global
+// maximum and softmax denominator are reduced over its tiles, and each tile maximum in the workspace
+// is replaced by the factor exp(tile max - row max) / denominator its partial sums have to be
+// multiplied with.
+__global__ __launch_bounds__(64) void kvstar_rowscale_kernel(
+    float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_len,
+    unsigned n_tokens, unsigned q_heads, unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles,
+    unsigned row_pad)
 {
-    __shared__ float row_max[8 * kMaxRows];
-    __shared__ float row_inv[8 * kMaxRows];
-    const unsigned task = blockIdx.x;
+    const unsigned task = blockIdx.y;
     const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
-    if (n_blocks == 0) { return; }
     const unsigned g = q_heads / kv_heads, R = n_tokens * g;
-    const unsigned n_tiles = (n_blocks * M + 31) / 32;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float* wmax = ws_max + static_cast<size_t>(task) * kv_heads * kMaxRows * max_tiles;
-    const float* wpart = ws_part + static_cast<size_t>(task) * kv_heads * kMaxRows * max_blocks;
-
-    // one wave per (kv head, row): global maximum, then the softmax denominator
-    for (unsigned row = wave; row < kv_heads * R; row += kWaves) {
-        const unsigned h = row / R, rho = row - h * R;
-        const float* tm = wmax + (static_cast<size_t>(h) * kMaxRows + rho) * max_tiles;
-        const float* pp = wpart + (static_cast<size_t>(h) * kMaxRows + rho) * max_blocks;
-        float mx = -INFINITY;
-        for (unsigned t = lane; t < n_tiles; t += 64) { mx = fmaxf(mx, tm[t]); }
+    const unsigned h = blockIdx.x / R, rho = blockIdx.x - h * R;
+    if (n_blocks == 0 || h >= kv_heads) { return; }
+    const unsigned n_tiles = (n_blocks * M + kTileSub - 1) / kTileSub;
+    const int lane = threadIdx.x;
+    float* tm = ws_max + ((static_cast<size_t>(task) * kv_heads + h) * row_pad + rho) * max_tiles;
+    const float* pp = ws_part + ((static_cast<size_t>(task) * kv_heads + h) * row_pad + rho) * max_blocks;
+    float mx = -INFINITY;
+    for (unsigned t = lane; t < n_tiles; t += 64) { mx = fmaxf(mx, tm[t]); }
 #pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) { mx = fmaxf(mx, __shfl_xor(mx, d, 64)); }
-        float den = 0.0f;
-        for (unsigned b = lane; b < n_blocks; b += 64) { den += pp[b] * __expf(tm[(b * M) / 32] - mx); }
+    for (int d = 32; d >= 1; d >>= 1) { mx = fmaxf(mx, __shfl_xor(mx, d, 64)); }
+    float den = 0.0f;
+    for (unsigned b = lane; b < n_blocks; b += 64) { den += pp[b] * __expf(tm[(b * M) / kTileSub] - mx); }
 #pragma unroll
-        for (int d = 32; d >= 1; d >>= 1) { den += __shfl_xor(den, d, 64); }
-        if (lane == 0) {
-            row_max[h * kMaxRows + rho] = mx;
-            row_inv[h * kMaxRows + rho] = den > 1e-9f ? 1.0f / den : 1.0f;   // the reference skips the division then
-        }
-    }
-    __syncthreads();
-    float* out = votes + seg_off[task];
-    for (unsigned b = threadIdx.x; b < n_blocks; b += kThreads) {
-        const unsigned tile = (b * M) / 32;
-        float v = 0.0f;
-        for (unsigned h = 0; h < kv_heads; ++h) {
-            for (unsigned rho = 0; rho < R; ++rho) {
-                const size_t r = static_cast<size_t>(h) * kMaxRows + rho;
-                v += wpart[r * max_blocks + b] * __expf(wmax[r * max_tiles + tile] - row_max[h * kMaxRows + rho]) *
-                     row_inv[h * kMaxRows + rho];
-            }
-        }
-        out[b] = v;
-    }
+    for (int d = 32; d >= 1; d >>= 1) { den += __shfl_xor(den, d, 64); }
+    const float inv = den > 1e-9f ? 1.0f / den : 1.0f;   // the reference skips the division then
+    for (unsigned t = lane; t < n_tiles; t += 64) { tm[t] = __expf(tm[t] - mx) * inv; }
 }
 
+// Phase 2, grid: x = 256 blocks of the task, y = task: votes[b] = sum over rows of partial * factor.
+__global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
+    const float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_off,
+    const int32_t* __restrict__ seg_len, unsigned n_tokens, unsigned q_heads, unsigned kv_heads, unsigned M,
+    unsigned max_blocks, unsigned max_tiles, unsigned row_pad, float* __restrict__ votes)
+{
+    const unsigned task = blockIdx.y;
+    const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
+    const unsigned b = blockIdx.x * kThreads + threadIdx.x;
+    if (b >= n_blocks) { return; }
+    const unsigned g = q_heads / kv_heads, R = n_tokens * g;
+    const unsigned tile = (b * M) / kTileSub;
+    const float* wmax = ws_max + static_cast<size_t>(task) * kv_heads * row_pad * max_tiles;
+    const float* wpart = ws_part + static_cast<size_t>(task) * kv_heads * row_pad * max_blocks;
+    float v0 = 0.0f, v1 = 0.0f;
+    for (unsigned h = 0; h < kv_heads; ++h) {
+        const size_t r0 = static_cast<size_t>(h) * row_pad;
+        unsigned rho = 0;
+        for (; rho + 1 < R; rho += 2) {
+            v0 += wpart[(r0 + rho) * max_blocks + b] * wmax[(r0 + rho) * max_tiles + tile];
+            v1 += wpart[(r0 + rho + 1) * max_blocks + b] * wmax[(r0 + rho + 1) * max_tiles + tile];
+        }
+        if (rho < R) { v0 += wpart[(r0 + rho) * max_blocks + b] * wmax[(r0 + rho) * max_tiles + tile]; }
+    }
+    votes[seg_off[task] + b] = v0 + v1;
+}
+
+unsigned g_heads_per_group = 1;
+
 }  // namespace
+
+// Tuning knob for benchmarks: kv heads one workgroup of the KVStar score kernel walks (default 1).
+extern "C" int ucm_set_kvstar_heads_per_group(int heads)
+{
+    UCM_REQUIRE(heads >= 1 && heads <= 8, "ucm_set_kvstar_heads_per_group: %d", heads);
+    g_heads_per_group = static_cast<unsigned>(heads);
+    return UCM_OK;
+}
 
 extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
                                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
@@ -311,14 +373,15 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
 }
 
-extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int max_blocks, int sub_blocks, int64_t* max_floats,
-                                           int64_t* part_floats)
+extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks,
+                                           int64_t* max_floats, int64_t* part_floats)
 {
-    UCM_REQUIRE(n_tasks >= 0 && kv_heads > 0 && max_blocks >= 0 && sub_blocks > 0 && max_floats && part_floats,
-                "ucm_kvstar_workspace_floats: bad argument");
-    const int64_t tiles = (static_cast<int64_t>(max_blocks) * sub_blocks + 31) / 32;
-    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * kMaxRows * std::max<int64_t>(tiles, 1);
-    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * kMaxRows * std::max(max_blocks, 1);
+    UCM_REQUIRE(n_tasks >= 0 && kv_heads > 0 && rows_per_head > 0 && rows_per_head <= kMaxRows && max_blocks >= 0 &&
+                    sub_blocks > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
+    const int64_t tiles = (static_cast<int64_t>(max_blocks) * sub_blocks + kTileSub - 1) / kTileSub;
+    const int64_t row_pad = rows_per_head > 32 ? 64 : 32;
+    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * std::max<int64_t>(tiles, 1);
+    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * std::max(max_blocks, 1);
     return UCM_OK;
 }
 
@@ -347,26 +410,62 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
                       sub_blocks == 32, "ucm_kvstar_votes: sub_blocks=%d (1, 2, 4, 8, 16 or 32)", sub_blocks);
     UCM_REQUIRE(ucm::aligned16(repre_f16), "ucm_kvstar_votes: representatives not 16-byte aligned");
     const int64_t S = static_cast<int64_t>(max_blocks) * sub_blocks;
-    const unsigned chunks = static_cast<unsigned>((S + kChunk - 1) / kChunk);
-    const unsigned max_tiles = static_cast<unsigned>((S + 31) / 32);
+    const unsigned max_tiles = static_cast<unsigned>((S + kTileSub - 1) / kTileSub);
+    const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
+    const unsigned row_pad = R > 32 ? 64 : 32;
+    // heads per workgroup (at most what fits 72 KiB of LDS: 8 at 32 rows per head, 4 at 64).  One head per
+    // workgroup measured fastest on MI355X (1.07 ms against 1.4-1.6 ms with 2-8 heads for 512 tasks of 32-512
+    // blocks), although several heads make a workgroup's reads contiguous; ucm_set_kvstar_heads_per_group changes it.
+    const unsigned per_head_lds = row_pad * kQStride * 2;
+    const unsigned heads_per_group = std::max(1u, std::min<unsigned>(std::min<unsigned>(kv_heads, g_heads_per_group),
+                                                                     (72u * 1024u) / per_head_lds));
+    const unsigned head_groups = (kv_heads + heads_per_group - 1) / heads_per_group;
+    const unsigned lds_bytes = heads_per_group * per_head_lds;
+    // a workgroup stages its queries once, so it should walk many tiles; the longest task is still cut into
+    // enough chunks that about 2048 workgroups exist
+    const unsigned tiles_per_wg_all = (max_tiles + kWaves - 1) / kWaves;
+    const unsigned want_chunks = std::max(1u, 2048u / static_cast<unsigned>(n_tasks * head_groups));
+    const unsigned tiles_per_wave = std::max(1u, (tiles_per_wg_all + want_chunks - 1) / want_chunks);
+    const unsigned chunks = (max_tiles + kWaves * tiles_per_wave - 1) / (kWaves * tiles_per_wave);
     hipStream_t s = ucm::as_stream(stream);
-#define UCM_KVSTAR_ARGS dim3(chunks, kv_heads, n_tasks), dim3(kThreads), 0, s, static_cast<const unsigned short*>(q_f16), q_off, \
+#define UCM_KVSTAR_ARGS dim3(chunks, head_groups, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), seg_off, seg_len, static_cast<unsigned>(kv_heads),                     \
         static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), ws_max, ws_part, static_cast<unsigned>(max_blocks),    \
-        max_tiles
+        max_tiles, tiles_per_wave, row_pad, heads_per_group
+#define UCM_KVSTAR_LAUNCH2(M, TWO)                                                                                    \
+    do {                                                                                                             \
+        if (lds_bytes > 48u * 1024u) {                                                                               \
+            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_score_kernel<M, TWO>),   \
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize,                   \
+                                                      static_cast<int>(lds_bytes));                                \
+            if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_votes (LDS size)"); }                      \
+        }                                                                                                            \
+        hipLaunchKernelGGL((kvstar_score_kernel<M, TWO>), UCM_KVSTAR_ARGS);                                          \
+    } while (0)
+#define UCM_KVSTAR_LAUNCH(M)                                                                                          \
+    do {                                                                                                             \
+        if (R > 32) { UCM_KVSTAR_LAUNCH2(M, true); } else { UCM_KVSTAR_LAUNCH2(M, false); }                          \
+    } while (0)
     switch (sub_blocks) {
-    case 1: hipLaunchKernelGGL(kvstar_score_kernel<1>, UCM_KVSTAR_ARGS); break;
-    case 2: hipLaunchKernelGGL(kvstar_score_kernel<2>, UCM_KVSTAR_ARGS); break;
-    case 4: hipLaunchKernelGGL(kvstar_score_kernel<4>, UCM_KVSTAR_ARGS); break;
-    case 8: hipLaunchKernelGGL(kvstar_score_kernel<8>, UCM_KVSTAR_ARGS); break;
-    case 16: hipLaunchKernelGGL(kvstar_score_kernel<16>, UCM_KVSTAR_ARGS); break;
-    default: hipLaunchKernelGGL(kvstar_score_kernel<32>, UCM_KVSTAR_ARGS); break;
+    case 1: UCM_KVSTAR_LAUNCH(1); break;
+    case 2: UCM_KVSTAR_LAUNCH(2); break;
+    case 4: UCM_KVSTAR_LAUNCH(4); break;
+    case 8: UCM_KVSTAR_LAUNCH(8); break;
+    case 16: UCM_KVSTAR_LAUNCH(16); break;
+    default: UCM_KVSTAR_LAUNCH(32); break;
     }
+#undef UCM_KVSTAR_LAUNCH
+#undef UCM_KVSTAR_LAUNCH2
 #undef UCM_KVSTAR_ARGS
     if (hipError_t e = hipGetLastError(); e != hipSuccess) { return ucm::check_hip(e, "ucm_kvstar_votes (scores)"); }
-    hipLaunchKernelGGL(kvstar_combine_kernel, dim3(n_tasks), dim3(kThreads), 0, s, ws_max, ws_part, seg_off, seg_len,
-                       static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(kv_heads),
-                       static_cast<unsigned>(sub_blocks), static_cast<unsigned>(max_blocks), max_tiles, votes);
+    hipLaunchKernelGGL(kvstar_rowscale_kernel, dim3(static_cast<unsigned>(kv_heads) * R, n_tasks), dim3(64), 0, s, ws_max,
+                       ws_part, seg_len, static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads),
+                       static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks), static_cast<unsigned>(max_blocks),
+                       max_tiles, row_pad);
+    hipLaunchKernelGGL(kvstar_vote_kernel, dim3((max_blocks + kThreads - 1) / kThreads, n_tasks), dim3(kThreads), 0, s, ws_max,
+                       ws_part, seg_off, seg_len, static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads),
+                       static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks), static_cast<unsigned>(max_blocks),
+                       max_tiles, row_pad, votes);
     UCM_LAUNCH_CHECK("ucm_kvstar_votes");
 }

@@ -310,11 +310,13 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
               repre.shape[1], repre.stride(0), _stream())
 
 
-def kvstar_workspace(n_tasks: int, kv_heads: int, max_blocks: int, sub_blocks: int, device) -> tuple:
+def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks: int, sub_blocks: int, device) -> tuple:
+    """Scratch of ucm_kvstar_votes; rows_per_head = query tokens * (q_heads / kv_heads)."""
     import ctypes as C
 
     a, b = C.c_int64(0), C.c_int64(0)
-    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, max_blocks, sub_blocks, C.addressof(a), C.addressof(b))
+    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, C.addressof(a),
+              C.addressof(b))
     return (torch.empty(max(a.value, 1), dtype=torch.float32, device=device),
             torch.empty(max(b.value, 1), dtype=torch.float32, device=device))
 
@@ -350,6 +352,10 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
 
 def set_score_tile(tile_blocks: int) -> None:
     _lib.call("ucm_set_score_tile", tile_blocks)
+
+
+def set_kvstar_heads_per_group(heads: int) -> None:
+    _lib.call("ucm_set_kvstar_heads_per_group", heads)
 
 
 def set_hash_encode_groups(workgroups: int) -> None:

@@ -120,7 +120,7 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
             if n > 0 and k > 0:
                 seg_off = torch.zeros(1, dtype=torch.int32, device=dev)
                 seg_len = torch.full((1,), n, dtype=torch.int32, device=dev)
-                ws = ops.kvstar_workspace(1, h, n, m, dev)
+                ws = ops.kvstar_workspace(1, h, x * (hq // h), n, m, dev)
                 ops.kvstar_votes(q, torch.zeros(1, dtype=torch.int64, device=dev), x, hq, table, seg_off, seg_len, n, votes,
                                  ws, d_pruned=dp, pruned=pruned, pruned_sel=sel)
                 ops.topk_windows(votes.view(1, -1), seg_off, seg_len, torch.full((1,), k, dtype=torch.int32, device=dev), n,
