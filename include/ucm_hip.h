@@ -273,9 +273,11 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   pruned   dev int32[kv_heads][d_pruned]: channel of every kept dim (the
  *            reference's d_pruned_index, :288-304), or NULL when d_pruned ==
  *            head_dim
- *   repre    dev fp16 [n_layers][repre_rows][M][kv_heads][d_pad], d_pad >=
- *            d_pruned (columns past d_pruned are written as zero);
- *            repre_layer_stride in elements.
+ *   repre    dev fp16, HEAD-MAJOR: [n_layers][kv_heads][repre_rows][M][d_pad],
+ *            d_pad >= d_pruned (columns past d_pruned are written as zero);
+ *            repre_layer_stride and repre_head_stride in elements.  (The
+ *            reference keeps [row][M][kv head][d]; head-major makes the vectors
+ *            a workgroup streams for one head contiguous.)
  *
  * ucm_kvstar_votes: the arithmetic of KVStar::Execute
  * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:817-990)
@@ -290,7 +292,8 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   pruned   dev int32[*][kv_heads][d_pruned] channel lists, pruned_sel dev
  *            int32[n_tasks] picks one per task (-1: none); both NULL when
  *            d_pruned == d_orig
- *   repre_f16  dev fp16 [rows][sub_blocks][kv_heads][d_pad]; task t owns rows
+ *   repre_f16  dev fp16 head-major [kv_heads][rows][sub_blocks][d_pad], head
+ *            planes repre_head_stride elements apart; task t owns rows
  *            seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >= every seg_len
  *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
  *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev fp32, task t's votes at votes[seg_off[t] + b].
@@ -301,7 +304,7 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
                            const int32_t* block_ids, const int32_t* slots, int n, int block_size,
                            int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
                            int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
-                           ucm_stream_t stream);
+                           int64_t repre_head_stride, ucm_stream_t stream);
 /* Tuning knob for benchmarks: kv heads per workgroup of the KVStar score kernel
  * (1..8, default 1).  Not part of the reference interface. */
 int ucm_set_kvstar_heads_per_group(int heads);
@@ -309,7 +312,8 @@ int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, in
                                 int sub_blocks, int64_t* max_floats, int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                      const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                     const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                     int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len,
+                     int n_tasks, int max_blocks,
                      int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                      float* ws_part, float* votes, ucm_stream_t stream);
 

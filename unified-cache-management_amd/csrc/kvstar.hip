@@ -50,7 +50,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
     unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
-    unsigned short* __restrict__ repre, int64_t layer_stride)
+    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride)
 {
     const unsigned M = block_size / merge;
     const unsigned item = blockIdx.x / M, m = blockIdx.x % M;
@@ -61,7 +61,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const unsigned short* blk = static_cast<const unsigned short*>(k_layers[blockIdx.y]) +
                                 (static_cast<size_t>(id) * block_size + static_cast<size_t>(m) * merge) * row;
     unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride +
-                          (static_cast<size_t>(slot) * M + m) * kv_heads * d_pad;
+                          (static_cast<size_t>(slot) * M + m) * d_pad;   // + h * head_stride + p
     const float inv = 1.0f / static_cast<float>(merge);
     for (unsigned e = threadIdx.x; e < kv_heads * d_pad; e += kThreads) {
         const unsigned h = e / d_pad, p = e - h * d_pad;
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
                 v = f32_to_f16_bits(__uint_as_float(u & 0xffff0000u));
             }
         }
-        out[e] = v;
+        out[static_cast<int64_t>(h) * head_stride + p] = v;
     }
 }
 
@@ -134,16 +134,16 @@ __device__ __forceinline__ void block_sums(const float (&e)[16], int half, float
     }
 }
 
-// grid: x = chunk of sub-blocks, y = group of kv heads, z = task.  A workgroup walks the heads of its
-// group for its sub-blocks (a sub-block's vectors of all kv heads lie side by side in the table:
-// kv_heads * d_pad * 2 bytes, 2 KiB at 8 x 128); the queries of those heads are staged in LDS once
-// per workgroup.  The host picks the group size (one head by default, see ucm_kvstar_votes).
+// grid: x = chunk of sub-blocks, y = group of kv heads, z = task.  The table is head-major
+// ([kv head][row][sub-block][d_pad]), so the vectors one workgroup streams for a head are contiguous
+// (in the reference's [row][sub-block][kv head][d] order each vector of a head sits kv_heads*d*2
+// bytes from the next).  The queries of the group's heads are staged in LDS once per workgroup.
 template <int kM, bool kTwoRowTiles>
 __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_kernel(
     const unsigned short* __restrict__ q, const int64_t* __restrict__ q_off, unsigned n_tokens, unsigned q_heads,
     unsigned d_orig, const int32_t* __restrict__ pruned, const int32_t* __restrict__ pruned_sel,
     const unsigned short* __restrict__ table, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad,
+    const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
     float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
     unsigned tiles_per_wave, unsigned row_pad, unsigned heads_per_group)
 {
@@ -195,9 +195,9 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes dims half*(d_pad/2) + ks*8 .. +8
     const unsigned hoff = half * (d_pad / 2);
     constexpr bool two_row_tiles = kTwoRowTiles;   // 33..64 query rows per kv head
-    const size_t vec_stride = static_cast<size_t>(kv_heads) * d_pad;
-    const unsigned short* tbase = table + static_cast<size_t>(seg_off[task]) * kM * vec_stride +
-                                  static_cast<size_t>(h_first) * d_pad + hoff;
+    // head-major table: head h's vectors of all sub-blocks are contiguous, d_pad elements each
+    const unsigned short* tbase = table + static_cast<int64_t>(h_first) * head_stride +
+                                  static_cast<size_t>(seg_off[task]) * kM * d_pad + hoff;
 
     // A (tile, head) step's keys: eight 16-byte loads per lane, one contiguous half vector.  Everything is
     // unconditional - MFMA steps past d_pad reload piece 0 and are multiplied with a zero query fragment,
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
     // step can be issued before this step's arithmetic without a branch around them.
     auto load_keys = [&](u32x4 (&kf)[kMaxDim / 16], unsigned s0, unsigned hh) {
         const unsigned s_mine = min(s0 + lr, S - 1);
-        const unsigned short* krow = tbase + static_cast<size_t>(s_mine) * vec_stride + hh * d_pad;
+        const unsigned short* krow = tbase + static_cast<int64_t>(hh) * head_stride + static_cast<size_t>(s_mine) * d_pad;
 #pragma unroll
         for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = ucm::gload16(krow + (ks < ksteps ? ks : 0u) * 8); }
     };
@@ -350,7 +350,7 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
                                       int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
                                       int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
-                                      ucm_stream_t stream)
+                                      int64_t repre_head_stride, ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_kvstar_block_repre: n=%d", n);
     if (n == 0) { return UCM_OK; }
@@ -363,13 +363,16 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                 d_pruned, d_pad);
     UCM_REQUIRE(pruned || d_pruned == head_dim, "ucm_kvstar_block_repre: d_pruned < head_dim needs the channel list");
     const int M = block_size / merge;
+    UCM_REQUIRE(repre_head_stride >= static_cast<int64_t>(repre_rows) * M * d_pad,
+                "ucm_kvstar_block_repre: repre_head_stride=%lld smaller than one head's plane",
+                static_cast<long long>(repre_head_stride));
     UCM_REQUIRE(static_cast<int64_t>(n) * M <= 0x7fffffffll, "ucm_kvstar_block_repre: too many blocks for one launch");
     hipLaunchKernelGGL(kvstar_repre_kernel, dim3(static_cast<unsigned>(n) * M, n_layers), dim3(kThreads), 0,
                        ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
                        static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),
                        static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), static_cast<unsigned>(merge),
                        pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),
-                       static_cast<unsigned short*>(repre_f16), repre_layer_stride);
+                       static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride);
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
 }
 
@@ -387,7 +390,8 @@ extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_p
 
 extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                                 const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                                const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                                int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                                int max_blocks,
                                 int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, float* ws_part,
                                 float* votes, ucm_stream_t stream)
 {
@@ -408,14 +412,14 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     UCM_REQUIRE(pruned_sel != nullptr || d_pruned == d_orig, "ucm_kvstar_votes: d_pruned < d_orig needs the channel lists");
     UCM_SUPPORTED(sub_blocks == 1 || sub_blocks == 2 || sub_blocks == 4 || sub_blocks == 8 || sub_blocks == 16 ||
                       sub_blocks == 32, "ucm_kvstar_votes: sub_blocks=%d (1, 2, 4, 8, 16 or 32)", sub_blocks);
-    UCM_REQUIRE(ucm::aligned16(repre_f16), "ucm_kvstar_votes: representatives not 16-byte aligned");
+    UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0,
+                "ucm_kvstar_votes: representatives not 16-byte aligned");
     const int64_t S = static_cast<int64_t>(max_blocks) * sub_blocks;
     const unsigned max_tiles = static_cast<unsigned>((S + kTileSub - 1) / kTileSub);
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
     const unsigned row_pad = R > 32 ? 64 : 32;
-    // heads per workgroup (at most what fits 72 KiB of LDS: 8 at 32 rows per head, 4 at 64).  One head per
-    // workgroup measured fastest on MI355X (1.07 ms against 1.4-1.6 ms with 2-8 heads for 512 tasks of 32-512
-    // blocks), although several heads make a workgroup's reads contiguous; ucm_set_kvstar_heads_per_group changes it.
+    // heads per workgroup (at most what fits 72 KiB of LDS: 8 at 32 rows per head, 4 at 64); one by default,
+    // ucm_set_kvstar_heads_per_group changes it
     const unsigned per_head_lds = row_pad * kQStride * 2;
     const unsigned heads_per_group = std::max(1u, std::min<unsigned>(std::min<unsigned>(kv_heads, g_heads_per_group),
                                                                      (72u * 1024u) / per_head_lds));
@@ -431,7 +435,8 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
 #define UCM_KVSTAR_ARGS dim3(chunks, head_groups, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), seg_off, seg_len, static_cast<unsigned>(kv_heads),                     \
-        static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), ws_max, ws_part, static_cast<unsigned>(max_blocks),    \
+        static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, ws_max, ws_part,                   \
+        static_cast<unsigned>(max_blocks),                                                                                   \
         max_tiles, tiles_per_wave, row_pad, heads_per_group
 #define UCM_KVSTAR_LAUNCH2(M, TWO)                                                                                    \
     do {                                                                                                             \

@@ -294,9 +294,9 @@ def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, 
 def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                        block_size: int, kv_heads: int, head_dim: int, num_blocks: int, merge: int,
                        pruned: Optional[torch.Tensor] = None) -> None:
-    """repre fp16 [L, rows, M, kv_heads, d_pad]; pruned int32 [kv_heads, d_pruned] or None."""
-    if repre.dim() != 5 or repre.dtype != torch.float16 or repre.shape[2] * merge != block_size or repre.shape[3] != kv_heads:
-        raise ValueError("repre must be float16 [L, rows, block_size/merge, kv_heads, d_pad]")
+    """repre fp16, head-major [L, kv_heads, rows, M, d_pad]; pruned int32 [kv_heads, d_pruned] or None."""
+    if repre.dim() != 5 or repre.dtype != torch.float16 or repre.shape[3] * merge != block_size or repre.shape[1] != kv_heads:
+        raise ValueError("repre must be float16 [L, kv_heads, rows, block_size/merge, d_pad]")
     if len(k_layers) != repre.shape[0]:
         raise ValueError("one table layer per cache layer")
     if block_ids.numel() != slots.numel():
@@ -307,7 +307,7 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
     _lib.call("ucm_kvstar_block_repre", k_layers.ptr(), repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
               _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
               _opt(pruned, torch.int32, "pruned"), d_pruned, repre.shape[4], _dev(repre, torch.float16, "repre"),
-              repre.shape[1], repre.stride(0), _stream())
+              repre.shape[2], repre.stride(0), repre.stride(1), _stream())
 
 
 def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks: int, sub_blocks: int, device) -> tuple:
@@ -326,27 +326,31 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
                  d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
                  pruned_sel: Optional[torch.Tensor] = None) -> None:
     """q fp16 (any shape; task t reads [n_tokens, q_heads, d_orig] from element q_off[t]); repre fp16
-    [rows, M, kv_heads, d_pad]; votes fp32 [>= rows]; pruned int32 [n_lists, kv_heads, d_pruned]."""
-    if repre.dim() != 4 or repre.dtype != torch.float16:
-        raise ValueError("repre must be float16 [rows, M, kv_heads, d_pad]")
+    head-major [kv_heads, rows, M, d_pad] (head planes may be strided: a row slice of a bigger table is fine);
+    votes fp32 [>= rows]; pruned int32 [n_lists, kv_heads, d_pruned]."""
+    if repre.dim() != 4 or repre.dtype != torch.float16 or not repre.is_cuda:
+        raise ValueError("repre must be a float16 device tensor [kv_heads, rows, M, d_pad]")
+    kv_heads, rows, m, d_pad = repre.shape
+    if repre.stride(3) != 1 or repre.stride(2) != d_pad or repre.stride(1) != m * d_pad:
+        raise ValueError("repre rows must be dense ([rows, M, d_pad] contiguous inside each head plane)")
     d_orig = q.shape[-1]
     n_tasks = seg_off.numel()
     if seg_len.numel() != n_tasks or q_off.numel() != n_tasks:
         raise ValueError("q_off / seg_off / seg_len differ in length")
     if pruned is not None:
-        if pruned.dim() != 3 or pruned.shape[1] != repre.shape[2] or pruned_sel is None or pruned_sel.numel() != n_tasks:
+        if pruned.dim() != 3 or pruned.shape[1] != kv_heads or pruned_sel is None or pruned_sel.numel() != n_tasks:
             raise ValueError("pruned must be [n_lists, kv_heads, d_pruned] with one pruned_sel entry per task")
         d_pruned = pruned.shape[2]
     elif d_pruned is None:
         d_pruned = d_orig
-    if votes.numel() < repre.shape[0]:
+    if votes.numel() < rows:
         raise ValueError("votes shorter than the representative table")
     ws_max, ws_part = workspace
+    head_stride = repre.stride(0) if kv_heads > 1 else rows * m * d_pad
     _lib.call("ucm_kvstar_votes", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
-              _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"),
-              _dev(repre, torch.float16, "repre"), _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
-              n_tasks, max_blocks, repre.shape[1], repre.shape[2], d_pruned, repre.shape[3],
-              _dev(ws_max, torch.float32, "ws_max"), _dev(ws_part, torch.float32, "ws_part"),
+              _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), repre.data_ptr(), head_stride,
+              _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
+              d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), _dev(ws_part, torch.float32, "ws_part"),
               _dev(votes, torch.float32, "votes"), _stream())
 
 

@@ -9,7 +9,10 @@ surface (ucm/sparse/kvstar/retrieve/py_intf/py_intf.cpp:14-133):
 d_pruned]`` as in ``ReqPerLayerState.retrieval_async`` (ucm/sparse/kvstar/multistep.py:240-265),
 but both live on the device: the reference's thread pool (retrieve_task_manager.cpp,
 retrieve_task_runner.cpp) becomes a side stream, a task's completion an event.
-``extract_block_repre`` is the device twin of multistep.py:279-316.
+``extract_block_repre`` is the device twin of multistep.py:279-316; what it returns has the
+reference's shape but is a view of head-major storage (``[kv_heads, n, M, d_pad]``, the
+order the score kernel streams), and stays one under row slices such as ``[init:-local]``.
+A tensor in any other memory order is accepted too and repacked once per call.
 
 Block order in ``data``: descending vote, lower index first among equals (what the
 reference's portable kernel returns; its AVX2 build returns the same set unordered).
@@ -69,12 +72,18 @@ def Setup(param: SetupParam) -> None:  # noqa: N802 (reference name)
         _stream = torch.cuda.Stream()  # default priority
 
 
-def _pad16(t: torch.Tensor) -> torch.Tensor:
-    d = t.shape[-1]
-    if d % 16 == 0 and t.is_contiguous():
-        return t
-    out = torch.zeros(t.shape[:-1] + ((d + 15) // 16 * 16,), dtype=t.dtype, device=t.device)
-    out[..., :d] = t
+def _head_major(blk_repre: torch.Tensor) -> torch.Tensor:
+    """[n, M, h, dp] (reference order of the dims) -> fp16 [h, n, M, d_pad] whose (n, M, d_pad) part is dense."""
+    n, m, h, dp = blk_repre.shape
+    hm = blk_repre.permute(2, 0, 1, 3)
+    d_phys = hm.stride(2) if m > 1 or n > 1 else dp
+    if hm.stride(3) == 1 and d_phys % 16 == 0 and 0 <= d_phys - dp < 16 and hm.stride(2) == d_phys \
+            and hm.stride(1) == m * d_phys and hm.data_ptr() % 16 == 0 \
+            and (h == 1 or (hm.stride(0) % 8 == 0 and hm.stride(0) >= n * m * d_phys)):
+        # already head-major (what extract_block_repre hands out); widen the view to the padded columns (zeros)
+        return torch.as_strided(hm, (h, n, m, d_phys), (hm.stride(0), m * d_phys, d_phys, 1))
+    out = torch.zeros((h, n, m, (dp + 15) // 16 * 16), dtype=blk_repre.dtype, device=blk_repre.device)
+    out[..., :dp] = hm
     return out
 
 
@@ -110,7 +119,7 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
         ready.record()
         with torch.cuda.stream(_stream):
             _stream.wait_event(ready)
-            table = _pad16(blk_repre)
+            table = _head_major(blk_repre)
             q = query_group.contiguous()
             votes = torch.zeros(max(n, 1), dtype=torch.float32, device=dev)
             k = min(int(topk), n)
@@ -162,8 +171,8 @@ def GetTaskResult(task_id: int):  # noqa: N802
 def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge: int, prune_ratio: float = 1.0,
                         d_pruned_index: Optional[torch.Tensor] = None, prune_dim_enable: bool = False):
     """Sub-block representatives of cache blocks ``vllm_block_ids`` (multistep.py:279-316).
-    Returns (fp16 [n, M, kv_heads, d_pad] with zero columns past d_pruned, d_pruned_index int64 [kv_heads,
-    d_pruned] or None).  With ``prune_dim_enable`` and a ratio below 0.98 the channels with the largest mean |k|
+    Returns (fp16 of shape [n, M, kv_heads, d_pad] - a view of head-major storage - with zero columns past
+    d_pruned, d_pruned_index int64 [kv_heads, d_pruned] or None).  With ``prune_dim_enable`` and a ratio below 0.98 the channels with the largest mean |k|
     over these blocks are kept per head (the reference's choice, :284-292); otherwise a given index is reused."""
     n_total, block_size, kv_heads, head_dim = k_cache.shape
     dev = k_cache.device
@@ -174,8 +183,8 @@ def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge:
         d_pruned_index = d_pruned_index.contiguous()
     d_pruned = head_dim if d_pruned_index is None else d_pruned_index.shape[1]
     d_pad = (d_pruned + 15) // 16 * 16
-    repre = torch.empty((1, len(vllm_block_ids), block_size // merge, kv_heads, d_pad), dtype=torch.float16, device=dev)
+    repre = torch.empty((1, kv_heads, len(vllm_block_ids), block_size // merge, d_pad), dtype=torch.float16, device=dev)
     pruned32 = None if d_pruned_index is None else d_pruned_index.to(torch.int32).contiguous()
     ops.kvstar_block_repre(ops.LayerPointers([k_cache]), ids, torch.arange(len(vllm_block_ids), dtype=torch.int32, device=dev),
                            repre, block_size, kv_heads, head_dim, n_total, merge, pruned=pruned32)
-    return repre[0], d_pruned_index
+    return repre[0].permute(1, 2, 0, 3), d_pruned_index
