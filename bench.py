@@ -54,6 +54,9 @@ def parse():
                          "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
     ap.add_argument("--hash-leg", action="store_true",
                     help="also time the hash-code retrieval variant (BASELINE configs[4] shape) on the same caches")
+    ap.add_argument("--kvstar-leg", action="store_true",
+                    help="also time the multi-query softmax-vote retrieval (KVStar shape: 8 query tokens per request, "
+                         "8 sub-block representatives per block) on the same ragged batch")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -311,6 +314,71 @@ def main():
         }
         del colsum, bcodes, tcodes
 
+    # ---- KVStar leg: every (layer, request) is one task; 8 query tokens x 32 heads vote over the request's
+    # blocks through 8 sub-block representatives each (16-token means of the same key cache, fp16, head-major)
+    kvstar_leg = None
+    if args.kvstar_leg:
+        kx, merge = 8, 16
+        km = BS // merge
+        ktab = torch.empty((n_layers, HKV, rows, km, D), dtype=torch.float16, device=dev)
+        ev0, ev1 = ev(), ev()
+        ev0.record()
+        ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge)
+        ev1.record()
+        torch.cuda.synchronize()
+        krep_ms = ev0.elapsed_time(ev1)
+        n_tasks = n_layers * N_REQ
+        # one flat head-major table over all layers: row of (layer l, block b) = l * rows + b
+        flat = ktab.permute(1, 0, 2, 3, 4).reshape(HKV, n_layers * rows, km, D).contiguous()
+        k_off = (seg_off_h[None, :].astype(np.int64) + (np.arange(n_layers, dtype=np.int64) * rows)[:, None]).reshape(-1)
+        k_len = np.tile(lens, n_layers)
+        kq = (torch.randn(n_tasks, kx, HQ, D, device=dev, generator=g) * 0.25).to(torch.float16)
+        kq_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (kx * HQ * D)
+        kvotes = torch.zeros(n_layers * rows, device=dev)
+        kws = ops.kvstar_workspace(n_tasks, HKV, kx * HQ // HKV, max_len, km, dev)
+        kso, ksl = i32(k_off), i32(k_len)
+        ktk = i32(np.tile(topk, n_layers))
+        kidx = torch.zeros((1, n_tasks, max_len), dtype=torch.int32, device=dev)
+        kcnt = torch.zeros((1, n_tasks), dtype=torch.int32, device=dev)
+
+        def kvstar_step():
+            ops.kvstar_votes(kq, kq_off, kx, HQ, flat, kso, ksl, max_len, kvotes, kws)
+            ops.topk_windows(kvotes.view(1, -1), kso, ksl, ktk, max_len, kidx, kcnt, start_w=0, end_w=0)
+
+        for _ in range(2):
+            kvstar_step()
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(args.steps):
+            kvstar_step()
+        ev1.record()
+        torch.cuda.synchronize()
+        kv_ms = ev0.elapsed_time(ev1) / args.steps
+        kv_bytes = flat.numel() * 2 + kq.numel() * 2 + kvotes.numel() * 4
+        kv_checked = None
+        if not args.no_check:
+            import oracle  # checker only
+
+            for t_ in (0, n_tasks // 2 + 3, n_tasks - 1):
+                a_, n_ = int(k_off[t_]), int(k_len[t_])
+                rep_ref = flat[:, a_ : a_ + n_].permute(1, 2, 0, 3).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+                _, want = oracle.kvstar_retrieve(kq[t_].view(torch.int16).cpu().numpy().view(np.uint16), rep_ref, int(topk[t_ % N_REQ]))
+                got = kvotes[a_ : a_ + n_].cpu().numpy()
+                assert np.allclose(got, want, rtol=2e-4, atol=2e-6), "KVStar votes differ from the CPU oracle"
+            kv_checked = "votes of 3 sampled tasks within rtol 2e-4 / atol 2e-6 of the CPU oracle (fp32, other summation order)"
+        kvstar_leg = {
+            "workload": f"{n_tasks} tasks (layer x request), {kx} query tokens x {HQ} heads, {rows} blocks x {km} sub-block "
+                        f"representatives per layer, fp16",
+            "block_repre_ms": round(krep_ms, 3),
+            "us_per_step": round(kv_ms * 1e3, 1),
+            "roofline": {"kernel": "kvstar_score_kernel (+ rowscale, vote, select)", "bound": "hbm",
+                         "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": kv_bytes,
+                         "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * D / (kv_ms * 1e-3) / 1e12, 1)},
+            "checked": kv_checked,
+        }
+        del ktab, flat, kws
+
     # ---- check the last step against the CPU oracle (selection, scores, gathered bytes)
     if not args.no_check:
         step(qs[n_q - 1])                                             # re-run the last full step: the delta leg reused the buffers
@@ -452,6 +520,7 @@ def main():
                                "frac": round(gbs(mean_bytes, mean_ms) / HBM_PEAK_GBS, 4)},
         "delta_gather": delta,
         "hash_retrieval": hash_leg,
+        "kvstar_retrieval": kvstar_leg,
         "cpu_baseline": cpu,
         "checked": checked,
     }
