@@ -315,12 +315,14 @@ def main():
         del colsum, bcodes, tcodes
 
     # ---- KVStar leg: every (layer, request) is one task; 8 query tokens x 32 heads vote over the request's
-    # blocks through 8 sub-block representatives each (16-token means of the same key cache, fp16, head-major)
+    # blocks through 8 sub-block representatives each (16-token means of the same key cache, fp16, kv head outermost)
     kvstar_leg = None
     if args.kvstar_leg:
         kx, merge = 8, 16
         km = BS // merge
-        ktab = torch.empty((n_layers, HKV, rows, km, D), dtype=torch.float16, device=dev)
+        # one table over all layers, kv head outermost: row of (layer l, block b) = l * rows + b
+        flat = torch.empty((HKV, n_layers * rows, D // 8, km, 8), dtype=torch.float16, device=dev)
+        ktab = flat.view(HKV, n_layers, rows, D // 8, km, 8).permute(1, 0, 2, 3, 4, 5)
         ev0, ev1 = ev(), ev()
         ev0.record()
         ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge)
@@ -328,8 +330,6 @@ def main():
         torch.cuda.synchronize()
         krep_ms = ev0.elapsed_time(ev1)
         n_tasks = n_layers * N_REQ
-        # one flat head-major table over all layers: row of (layer l, block b) = l * rows + b
-        flat = ktab.permute(1, 0, 2, 3, 4).reshape(HKV, n_layers * rows, km, D).contiguous()
         k_off = (seg_off_h[None, :].astype(np.int64) + (np.arange(n_layers, dtype=np.int64) * rows)[:, None]).reshape(-1)
         k_len = np.tile(lens, n_layers)
         kq = (torch.randn(n_tasks, kx, HQ, D, device=dev, generator=g) * 0.25).to(torch.float16)
@@ -361,7 +361,7 @@ def main():
 
             for t_ in (0, n_tasks // 2 + 3, n_tasks - 1):
                 a_, n_ = int(k_off[t_]), int(k_len[t_])
-                rep_ref = flat[:, a_ : a_ + n_].permute(1, 2, 0, 3).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+                rep_ref = ops.kvstar_table_to_reference(flat[:, a_ : a_ + n_]).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
                 _, want = oracle.kvstar_retrieve(kq[t_].view(torch.int16).cpu().numpy().view(np.uint16), rep_ref, int(topk[t_ % N_REQ]))
                 got = kvotes[a_ : a_ + n_].cpu().numpy()
                 assert np.allclose(got, want, rtol=2e-4, atol=2e-6), "KVStar votes differ from the CPU oracle"

@@ -51,19 +51,19 @@ def test_kvstar_block_repre(ucm, dev, merge, hkv, d, bs):
     for d_pruned in (d, d - 13, 16):
         pruned = None if d_pruned == d else np.stack([synth.permutation(1020 + h, d)[:d_pruned] for h in range(hkv)]).astype(np.int32)
         d_pad = (d_pruned + 15) // 16 * 16
-        repre = torch.full((n_layers, hkv, rows, M, d_pad), 3.0, dtype=torch.float16, device=dev)   # head-major
+        repre = ops.kvstar_table(n_layers, hkv, rows, M, d_pad, dev).fill_(3.0)      # [L, h, rows, d_pad/8, M, 8]
         ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge,
                                pruned=None if pruned is None else torch.from_numpy(pruned).to(dev))
-        got = repre.permute(0, 2, 3, 1, 4).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)   # oracle's order
+        got = ops.kvstar_table_to_reference(repre).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)   # oracle's order
         for l in range(n_layers):
             want = np.full((rows, M, hkv, d_pad), np.float16(3.0).view(np.uint16), np.uint16)
             O.kvstar_block_repre(caches_h[l], ids, slots, merge, want, pruned=pruned)
             assert np.array_equal(got[l], want), (d_pruned, l)
     # against torch's own mean in the model dtype (what the reference calls): equal up to one bf16 step of the summation order
     t = caches[0][torch.from_numpy(ids.astype(np.int64)).to(dev)].reshape(9, M, merge, hkv, d).mean(dim=2).to(torch.float16)
-    repre = torch.zeros((n_layers, hkv, rows, M, d), dtype=torch.float16, device=dev)
+    repre = ops.kvstar_table(n_layers, hkv, rows, M, d, dev).zero_()
     ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge)
-    mine = repre[0].permute(1, 2, 0, 3)[torch.from_numpy(slots.astype(np.int64)).to(dev)]
+    mine = ops.kvstar_table_to_reference(repre[0])[torch.from_numpy(slots.astype(np.int64)).to(dev)]
     assert torch.allclose(mine.float(), t.float(), rtol=2 ** -7, atol=1e-6)
 
 
@@ -74,7 +74,8 @@ def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None
     q = dev_f16(np.stack(q_bits_list), dev)
     q_off = torch.arange(len(lens), dtype=torch.int64, device=dev) * q[0].numel()
     rows, M, hkv, _ = repre_bits.shape
-    table = dev_f16(np.ascontiguousarray(repre_bits.transpose(2, 0, 1, 3)), dev)      # the kernels take it head-major
+    table = ops.kvstar_table_from_reference(dev_f16(repre_bits, dev))                 # the kernels' order: [h, rows, d_pad/8, M, 8]
+    assert torch.equal(ops.kvstar_table_to_reference(table), dev_f16(repre_bits, dev))
     votes = torch.full((rows,), -7.0, device=dev)
     ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, dev)
     ops.kvstar_votes(q, q_off, n_tokens, hq, table, torch.from_numpy(off).to(dev), torch.from_numpy(lens).to(dev),
@@ -150,20 +151,21 @@ def test_kvstar_retrieve_module_surface(ucm, dev):
     for ratio in (1.0, 0.6):
         repre, index = kvstar_retrieve.extract_block_repre(k_cache, ids, merge, prune_ratio=ratio, prune_dim_enable=True)
         dp = round(d * ratio)
-        assert repre.shape == (30, bs // merge, hkv, (dp + 15) // 16 * 16) and repre.dtype == torch.float16
-        assert repre.permute(2, 0, 1, 3).is_contiguous()          # a view of head-major storage
+        assert repre.shape == (30, bs // merge, hkv, dp) and repre.dtype == torch.float16 and repre.dim() == 4
+        assert repre.table.shape == (hkv, 30, (dp + 15) // 16 * 2, bs // merge, 8)   # the score kernel's order
         assert (index is None) == (ratio == 1.0)
         cache_bits = k_cache.view(torch.int16).cpu().numpy().view(np.uint16)
-        want = np.zeros(tuple(repre.shape), np.uint16)
+        want = np.zeros((30, bs // merge, hkv, (dp + 15) // 16 * 16), np.uint16)
         pr = None if index is None else index.cpu().numpy().astype(np.int32)
         O.kvstar_block_repre(cache_bits, ids, np.arange(30), merge, want, pruned=pr)
-        assert np.array_equal(repre.contiguous().view(torch.int16).cpu().numpy().view(np.uint16), want)
+        assert np.array_equal(repre.dense().view(torch.int16).cpu().numpy().view(np.uint16), want[..., :dp])
         if index is not None:                                  # the kept channels are those with the largest mean |k|
             am = k_cache[torch.tensor(ids, device=dev)].reshape(-1, hkv, d).float().abs().mean(0)
             assert torch.equal(index, torch.topk(am, dp, dim=-1).indices)
-        blk = repre[1:-2][..., :dp]                            # the reference keeps [init:-local] (multistep.py:495-497): still a view
+        blk = repre[1:-2]                                      # the reference keeps [init:-local] (multistep.py:495-497): still a view
+        assert blk.shape == (27, bs // merge, hkv, dp) and blk.table.data_ptr() != repre.table.data_ptr()
         if ratio == 1.0:
-            blk = blk.contiguous()                             # and a plain [n, M, h, d] tensor is accepted as well
+            blk = blk.dense()                                  # and a plain [n, M, h, d] tensor is accepted as well
         q = (torch.randn(8, hq, d, device=dev, generator=g) * 0.3).to(torch.float16)
         tid = kvstar_retrieve.AsyncRetrieveByCPU(q, blk, index, 9, 7, kvstar_retrieve.CPU)
         kvstar_retrieve.Wait(tid)

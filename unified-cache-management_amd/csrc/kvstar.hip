@@ -45,43 +45,97 @@ __device__ __forceinline__ unsigned short f32_to_f16_bits(float f)
 }
 
 // ---- sub-block representatives -------------------------------------------------------------
-// grid: x = listed block * M + sub-block, y = layer; thread = (kv head, kept channel)
+// Table layout, per kv head: [row (block slot)][piece = d_pad/8][sub-block m][8 channels], fp16.  A
+// block's representatives are one contiguous M*d_pad*2 bytes; inside it the 16-byte pieces of the M
+// sub-blocks that an MFMA step multiplies together are adjacent, so one load instruction of the
+// score kernel reads whole 128-byte lines (M*16 bytes per piece and block) instead of 16 bytes out
+// of each of 64 lines.
+//
+// grid: x = listed block, y = layer.  Phase 1: a thread owns 8 adjacent columns of a token row
+// (one 16-byte load per token, `merge` tokens accumulated in token order in fp32), the means -
+// rounded to bf16 and then fp16, what mean() in the model dtype followed by .to(float16) gives -
+// are parked in LDS as [M][kv_heads*head_dim].  Phase 2 gathers the kept channels from LDS and
+// writes the block's pieces, consecutive threads to consecutive 16 bytes.
+constexpr int kRepreUnroll = 16;
+
+__device__ __forceinline__ unsigned mean_to_f16x2(float lo, float hi, float inv)
+{
+    unsigned a = __float_as_uint(lo * inv), b = __float_as_uint(hi * inv);
+    a += 0x7fffu + ((a >> 16) & 1u);
+    b += 0x7fffu + ((b >> 16) & 1u);
+    return static_cast<unsigned>(f32_to_f16_bits(__uint_as_float(a & 0xffff0000u))) |
+           (static_cast<unsigned>(f32_to_f16_bits(__uint_as_float(b & 0xffff0000u))) << 16);
+}
+
+__device__ __forceinline__ void add_bf16x8(float (&acc)[8], const u32x4 v)
+{
+    acc[0] = acc[0] + __uint_as_float(v.x << 16); acc[1] = acc[1] + __uint_as_float(v.x & 0xffff0000u);
+    acc[2] = acc[2] + __uint_as_float(v.y << 16); acc[3] = acc[3] + __uint_as_float(v.y & 0xffff0000u);
+    acc[4] = acc[4] + __uint_as_float(v.z << 16); acc[5] = acc[5] + __uint_as_float(v.z & 0xffff0000u);
+    acc[6] = acc[6] + __uint_as_float(v.w << 16); acc[7] = acc[7] + __uint_as_float(v.w & 0xffff0000u);
+}
+
 __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
     unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
     unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride)
 {
+    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [M][row]
     const unsigned M = block_size / merge;
-    const unsigned item = blockIdx.x / M, m = blockIdx.x % M;
-    const unsigned id = static_cast<unsigned>(block_ids[item]);
-    const unsigned slot = static_cast<unsigned>(slots[item]);
-    if (id >= num_blocks || slot >= rows) { return; }
-    const unsigned row = kv_heads * head_dim;
+    const unsigned id = static_cast<unsigned>(block_ids[blockIdx.x]);
+    const unsigned slot = static_cast<unsigned>(slots[blockIdx.x]);
+    if (id >= num_blocks || slot >= rows) { return; }   // whole workgroup: never dereference a bad id
+    const unsigned row = kv_heads * head_dim, ncg = row / 8;
     const unsigned short* blk = static_cast<const unsigned short*>(k_layers[blockIdx.y]) +
-                                (static_cast<size_t>(id) * block_size + static_cast<size_t>(m) * merge) * row;
-    unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride +
-                          (static_cast<size_t>(slot) * M + m) * d_pad;   // + h * head_stride + p
+                                static_cast<size_t>(id) * block_size * row;
     const float inv = 1.0f / static_cast<float>(merge);
-    for (unsigned e = threadIdx.x; e < kv_heads * d_pad; e += kThreads) {
-        const unsigned h = e / d_pad, p = e - h * d_pad;
-        unsigned short v = 0;
-        if (p < d_pruned) {
-            const unsigned d = pruned ? static_cast<unsigned>(pruned[h * d_pruned + p]) : p;
-            if (d < head_dim) {
-                const UCM_GLOBAL unsigned short* src = (const UCM_GLOBAL unsigned short*)(blk + h * head_dim + d);
-                float acc = __uint_as_float(static_cast<unsigned>(src[0]) << 16);
-                for (unsigned t = 1; t < merge; ++t) {
-                    acc = acc + __uint_as_float(static_cast<unsigned>(src[static_cast<size_t>(t) * row]) << 16);
-                }
-                acc = acc * inv;
-                // to bf16 (round to nearest even), then to fp16: what mean() in the model dtype followed by .to(float16) gives
-                unsigned u = __float_as_uint(acc);
-                u += 0x7fffu + ((u >> 16) & 1u);
-                v = f32_to_f16_bits(__uint_as_float(u & 0xffff0000u));
-            }
+    for (unsigned w = threadIdx.x; w < M * ncg; w += kThreads) {
+        const unsigned m = w / ncg, cg = w - m * ncg;
+        const unsigned short* src = blk + static_cast<size_t>(m) * merge * row + cg * 8;
+        float acc[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
+        unsigned t = 0;
+        for (; t + kRepreUnroll <= merge; t += kRepreUnroll) {
+            u32x4 v[kRepreUnroll];
+#pragma unroll
+            for (int u = 0; u < kRepreUnroll; ++u) { v[u] = ucm::gload16_nt(src + static_cast<size_t>(t + u) * row); }
+#pragma unroll
+            for (int u = 0; u < kRepreUnroll; ++u) { add_bf16x8(acc, v[u]); }
         }
-        out[static_cast<int64_t>(h) * head_stride + p] = v;
+        for (; t < merge; ++t) { add_bf16x8(acc, ucm::gload16_nt(src + static_cast<size_t>(t) * row)); }
+        u32x4 o;
+        o.x = mean_to_f16x2(acc[0], acc[1], inv);
+        o.y = mean_to_f16x2(acc[2], acc[3], inv);
+        o.z = mean_to_f16x2(acc[4], acc[5], inv);
+        o.w = mean_to_f16x2(acc[6], acc[7], inv);
+        *reinterpret_cast<u32x4*>(&stage[m * row + cg * 8]) = o;
+    }
+    __syncthreads();
+    const unsigned pieces = d_pad / 8;
+    unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<size_t>(slot) * M * d_pad;
+    for (unsigned e = threadIdx.x; e < kv_heads * pieces * M; e += kThreads) {
+        const unsigned h = e / (pieces * M), rem = e - h * (pieces * M);
+        const unsigned piece = rem / M, m = rem - piece * M;
+        const unsigned short* srow = stage + m * row + h * head_dim;
+        unsigned short c[8];
+#pragma unroll
+        for (unsigned j = 0; j < 8; ++j) {
+            const unsigned p = piece * 8 + j;
+            unsigned short v = 0;
+            if (p < d_pruned) {
+                const unsigned d = pruned ? static_cast<unsigned>(pruned[h * d_pruned + p]) : p;
+                if (d < head_dim) { v = srow[d]; }
+            }
+            c[j] = v;
+        }
+        u32x4 o;
+        o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
+        o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
+        o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
+        o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
+        ucm::gstore16(out + static_cast<int64_t>(h) * head_stride + static_cast<size_t>(rem) * 8, o);
     }
 }
 
@@ -134,10 +188,11 @@ __device__ __forceinline__ void block_sums(const float (&e)[16], int half, float
     }
 }
 
-// grid: x = chunk of sub-blocks, y = group of kv heads, z = task.  The table is head-major
-// ([kv head][row][sub-block][d_pad]), so the vectors one workgroup streams for a head are contiguous
-// (in the reference's [row][sub-block][kv head][d] order each vector of a head sits kv_heads*d*2
-// bytes from the next).  The queries of the group's heads are staged in LDS once per workgroup.
+// grid: x = chunk of sub-blocks, y = group of kv heads, z = task.  The table is head-major and
+// piece-interleaved inside a block (see above), so what one workgroup streams for a head is one
+// contiguous run read in whole lines (in the reference's [row][sub-block][kv head][d] order each
+// vector of a head sits kv_heads*d*2 bytes from the next).  The queries of the group's heads are
+// staged in LDS once per workgroup.
 template <int kM, bool kTwoRowTiles>
 __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_kernel(
     const unsigned short* __restrict__ q, const int64_t* __restrict__ q_off, unsigned n_tokens, unsigned q_heads,
@@ -192,22 +247,24 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = lane >> 5, lr = lane & 31;
-    const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes dims half*(d_pad/2) + ks*8 .. +8
-    const unsigned hoff = half * (d_pad / 2);
+    const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes piece 2*ks + half
+    const unsigned hoff = half * 8;
     constexpr bool two_row_tiles = kTwoRowTiles;   // 33..64 query rows per kv head
     // head-major table: head h's vectors of all sub-blocks are contiguous, d_pad elements each
     const unsigned short* tbase = table + static_cast<int64_t>(h_first) * head_stride +
-                                  static_cast<size_t>(seg_off[task]) * kM * d_pad + hoff;
+                                  static_cast<size_t>(seg_off[task]) * kM * d_pad + half * (8 * kM);
 
-    // A (tile, head) step's keys: eight 16-byte loads per lane, one contiguous half vector.  Everything is
+    // A (tile, head) step's keys: eight 16-byte loads per lane, piece 2*ks + half of its sub-block; the
+    // lanes of one instruction cover M*16 contiguous bytes per block and lane half.  Everything is
     // unconditional - MFMA steps past d_pad reload piece 0 and are multiplied with a zero query fragment,
     // lanes and tiles past the end reload the last vector and are masked - so that the loads of the NEXT
     // step can be issued before this step's arithmetic without a branch around them.
     auto load_keys = [&](u32x4 (&kf)[kMaxDim / 16], unsigned s0, unsigned hh) {
         const unsigned s_mine = min(s0 + lr, S - 1);
-        const unsigned short* krow = tbase + static_cast<int64_t>(hh) * head_stride + static_cast<size_t>(s_mine) * d_pad;
+        const unsigned short* krow = tbase + static_cast<int64_t>(hh) * head_stride +
+                                     static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
 #pragma unroll
-        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = ucm::gload16(krow + (ks < ksteps ? ks : 0u) * 8); }
+        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = ucm::gload16(krow + (ks < ksteps ? ks : 0u) * (16 * kM)); }
     };
     u32x4 kf[kMaxDim / 16], kn[kMaxDim / 16];
     const unsigned t_end = kWaves * tiles_per_wave;
@@ -233,7 +290,7 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
             for (int i = 0; i < 16; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
 #pragma unroll
             for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-                const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 8;
+                const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 16;
                 const u32x4 braw = *reinterpret_cast<const u32x4*>(&qh[lr * kQStride + col]);
                 const f16x8 b0 = __builtin_bit_cast(f16x8, ks < ksteps ? braw : zero);
                 acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), b0, acc0, 0, 0, 0);
@@ -241,7 +298,7 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
             if (two_row_tiles) {
 #pragma unroll
                 for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-                    const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 8;
+                    const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 16;
                     const u32x4 braw = *reinterpret_cast<const u32x4*>(&qh[(32 + lr) * kQStride + col]);
                     const f16x8 b1 = __builtin_bit_cast(f16x8, ks < ksteps ? braw : zero);
                     acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), b1, acc1, 0, 0, 0);
@@ -366,8 +423,19 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_REQUIRE(repre_head_stride >= static_cast<int64_t>(repre_rows) * M * d_pad,
                 "ucm_kvstar_block_repre: repre_head_stride=%lld smaller than one head's plane",
                 static_cast<long long>(repre_head_stride));
-    UCM_REQUIRE(static_cast<int64_t>(n) * M <= 0x7fffffffll, "ucm_kvstar_block_repre: too many blocks for one launch");
-    hipLaunchKernelGGL(kvstar_repre_kernel, dim3(static_cast<unsigned>(n) * M, n_layers), dim3(kThreads), 0,
+    const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
+    UCM_SUPPORTED(row % 8 == 0 && d_pad % 8 == 0, "ucm_kvstar_block_repre: kv_heads*head_dim=%u and d_pad=%d must be multiples of 8",
+                  row, d_pad);
+    const size_t lds_bytes = static_cast<size_t>(M) * row * 2;
+    UCM_SUPPORTED(lds_bytes <= 64u * 1024u, "ucm_kvstar_block_repre: %d sub-blocks of %u channels exceed 64 KiB of LDS", M, row);
+    UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_layer_stride % 8 == 0 && repre_head_stride % 8 == 0,
+                "ucm_kvstar_block_repre: table not 16-byte aligned");
+    if (lds_bytes > 48u * 1024u) {
+        const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_kernel),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+        if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }
+    }
+    hipLaunchKernelGGL(kvstar_repre_kernel, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes,
                        ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
                        static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),
                        static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), static_cast<unsigned>(merge),

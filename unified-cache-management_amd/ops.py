@@ -291,12 +291,40 @@ def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, 
               _staging_ptr(staging, staging_blocks * block_bytes), _stream())
 
 
+def kvstar_table(n_layers: int, kv_heads: int, rows: int, sub_blocks: int, d_pad: int, device) -> torch.Tensor:
+    """Empty KVStar representative table, fp16 [L, kv_heads, rows, d_pad/8, M, 8]: per kv head and block the
+    16-byte pieces (8 channels) of the M sub-blocks lie side by side, the order the score kernel streams."""
+    if d_pad % 16 != 0:
+        raise ValueError("d_pad must be a multiple of 16")
+    return torch.empty((n_layers, kv_heads, rows, d_pad // 8, sub_blocks, 8), dtype=torch.float16, device=device)
+
+
+def kvstar_table_to_reference(table: torch.Tensor) -> torch.Tensor:
+    """[..., kv_heads, rows, d_pad/8, M, 8] -> the reference's [..., rows, M, kv_heads, d_pad] (a copy)."""
+    h, rows, pieces, m, _ = table.shape[-5:]
+    lead = tuple(range(table.dim() - 5))
+    k = len(lead)
+    return table.permute(*lead, k + 1, k + 3, k, k + 2, k + 4).reshape(*table.shape[:-5], rows, m, h, pieces * 8)
+
+
+def kvstar_table_from_reference(repre: torch.Tensor) -> torch.Tensor:
+    """The reference's [rows, M, kv_heads, d] -> fp16 [kv_heads, rows, d_pad/8, M, 8], columns zero padded to 16."""
+    rows, m, h, d = repre.shape
+    d_pad = (d + 15) // 16 * 16
+    padded = torch.zeros((rows, m, h, d_pad), dtype=torch.float16, device=repre.device)
+    padded[..., :d] = repre
+    return padded.view(rows, m, h, d_pad // 8, 8).permute(2, 0, 3, 1, 4).contiguous()
+
+
 def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                        block_size: int, kv_heads: int, head_dim: int, num_blocks: int, merge: int,
                        pruned: Optional[torch.Tensor] = None) -> None:
-    """repre fp16, head-major [L, kv_heads, rows, M, d_pad]; pruned int32 [kv_heads, d_pruned] or None."""
-    if repre.dim() != 5 or repre.dtype != torch.float16 or repre.shape[3] * merge != block_size or repre.shape[1] != kv_heads:
-        raise ValueError("repre must be float16 [L, kv_heads, rows, block_size/merge, d_pad]")
+    """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); pruned int32 [kv_heads, d_pruned] or None."""
+    if repre.dim() != 6 or repre.dtype != torch.float16 or repre.shape[4] * merge != block_size or \
+            repre.shape[1] != kv_heads or repre.shape[5] != 8:
+        raise ValueError("repre must be float16 [L, kv_heads, rows, d_pad/8, block_size/merge, 8]")
+    if not repre[0, 0].is_contiguous():
+        raise ValueError("a head's plane of the table must be contiguous")
     if len(k_layers) != repre.shape[0]:
         raise ValueError("one table layer per cache layer")
     if block_ids.numel() != slots.numel():
@@ -306,7 +334,7 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
         raise ValueError("pruned must be [kv_heads, d_pruned]")
     _lib.call("ucm_kvstar_block_repre", k_layers.ptr(), repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
               _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
-              _opt(pruned, torch.int32, "pruned"), d_pruned, repre.shape[4], _dev(repre, torch.float16, "repre"),
+              _opt(pruned, torch.int32, "pruned"), d_pruned, repre.shape[3] * 8, repre.data_ptr(),
               repre.shape[2], repre.stride(0), repre.stride(1), _stream())
 
 
@@ -325,14 +353,15 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
                  seg_off: torch.Tensor, seg_len: torch.Tensor, max_blocks: int, votes: torch.Tensor, workspace: tuple,
                  d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
                  pruned_sel: Optional[torch.Tensor] = None) -> None:
-    """q fp16 (any shape; task t reads [n_tokens, q_heads, d_orig] from element q_off[t]); repre fp16
-    head-major [kv_heads, rows, M, d_pad] (head planes may be strided: a row slice of a bigger table is fine);
-    votes fp32 [>= rows]; pruned int32 [n_lists, kv_heads, d_pruned]."""
-    if repre.dim() != 4 or repre.dtype != torch.float16 or not repre.is_cuda:
-        raise ValueError("repre must be a float16 device tensor [kv_heads, rows, M, d_pad]")
-    kv_heads, rows, m, d_pad = repre.shape
-    if repre.stride(3) != 1 or repre.stride(2) != d_pad or repre.stride(1) != m * d_pad:
-        raise ValueError("repre rows must be dense ([rows, M, d_pad] contiguous inside each head plane)")
+    """q fp16 (any shape; task t reads [n_tokens, q_heads, d_orig] from element q_off[t]); repre: one layer of a
+    kvstar_table, fp16 [kv_heads, rows, d_pad/8, M, 8] (head planes may be strided: a row slice of a bigger
+    table is fine); votes fp32 [>= rows]; pruned int32 [n_lists, kv_heads, d_pruned]."""
+    if repre.dim() != 5 or repre.dtype != torch.float16 or not repre.is_cuda or repre.shape[4] != 8:
+        raise ValueError("repre must be a float16 device tensor [kv_heads, rows, d_pad/8, M, 8]")
+    kv_heads, rows, pieces, m, _ = repre.shape
+    d_pad = pieces * 8
+    if rows and not repre[0].is_contiguous():
+        raise ValueError("repre rows must be dense ([rows, d_pad/8, M, 8] contiguous inside each head plane)")
     d_orig = q.shape[-1]
     n_tasks = seg_off.numel()
     if seg_len.numel() != n_tasks or q_off.numel() != n_tasks:

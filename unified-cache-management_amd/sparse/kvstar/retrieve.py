@@ -9,10 +9,11 @@ surface (ucm/sparse/kvstar/retrieve/py_intf/py_intf.cpp:14-133):
 d_pruned]`` as in ``ReqPerLayerState.retrieval_async`` (ucm/sparse/kvstar/multistep.py:240-265),
 but both live on the device: the reference's thread pool (retrieve_task_manager.cpp,
 retrieve_task_runner.cpp) becomes a side stream, a task's completion an event.
-``extract_block_repre`` is the device twin of multistep.py:279-316; what it returns has the
-reference's shape but is a view of head-major storage (``[kv_heads, n, M, d_pad]``, the
-order the score kernel streams), and stays one under row slices such as ``[init:-local]``.
-A tensor in any other memory order is accepted too and repacked once per call.
+``extract_block_repre`` is the device twin of multistep.py:279-316; it returns a ``BlockRepre``,
+which reports the reference's shape ``(n, M, kv_heads, d_pruned)`` and supports the block slices
+the plugin takes (``[init:-local]``, multistep.py:495-497) but keeps the values in the order the
+score kernel streams (``[kv_heads, n, d_pad/8, M, 8]``); ``dense()`` gives the reference's tensor.
+A plain ``[n, M, kv_heads, d_pruned]`` tensor is accepted too and repacked once per call.
 
 Block order in ``data``: descending vote, lower index first among equals (what the
 reference's portable kernel returns; its AVX2 build returns the same set unordered).
@@ -72,19 +73,36 @@ def Setup(param: SetupParam) -> None:  # noqa: N802 (reference name)
         _stream = torch.cuda.Stream()  # default priority
 
 
-def _head_major(blk_repre: torch.Tensor) -> torch.Tensor:
-    """[n, M, h, dp] (reference order of the dims) -> fp16 [h, n, M, d_pad] whose (n, M, d_pad) part is dense."""
-    n, m, h, dp = blk_repre.shape
-    hm = blk_repre.permute(2, 0, 1, 3)
-    d_phys = hm.stride(2) if m > 1 or n > 1 else dp
-    if hm.stride(3) == 1 and d_phys % 16 == 0 and 0 <= d_phys - dp < 16 and hm.stride(2) == d_phys \
-            and hm.stride(1) == m * d_phys and hm.data_ptr() % 16 == 0 \
-            and (h == 1 or (hm.stride(0) % 8 == 0 and hm.stride(0) >= n * m * d_phys)):
-        # already head-major (what extract_block_repre hands out); widen the view to the padded columns (zeros)
-        return torch.as_strided(hm, (h, n, m, d_phys), (hm.stride(0), m * d_phys, d_phys, 1))
-    out = torch.zeros((h, n, m, (dp + 15) // 16 * 16), dtype=blk_repre.dtype, device=blk_repre.device)
-    out[..., :dp] = hm
-    return out
+class BlockRepre:
+    """Sub-block representatives of n blocks in the score kernel's order; ``table`` is fp16
+    [kv_heads, n, d_pad/8, M, 8] (possibly a block slice of a bigger table)."""
+
+    def __init__(self, table: torch.Tensor, d_pruned: int):
+        self.table = table
+        self.d_pruned = int(d_pruned)
+
+    @property
+    def shape(self) -> torch.Size:
+        h, n, _, m, _ = self.table.shape
+        return torch.Size((n, m, h, self.d_pruned))
+
+    dtype = property(lambda self: self.table.dtype)
+    device = property(lambda self: self.table.device)
+
+    def dim(self) -> int:
+        return 4
+
+    def __len__(self) -> int:
+        return self.table.shape[1]
+
+    def __getitem__(self, blocks) -> "BlockRepre":
+        if not isinstance(blocks, slice) or blocks.step not in (None, 1):
+            raise TypeError("BlockRepre supports contiguous block slices only; use dense() for anything else")
+        return BlockRepre(self.table[:, blocks], self.d_pruned)
+
+    def dense(self) -> torch.Tensor:
+        """The reference's [n, M, kv_heads, d_pruned] tensor (a copy)."""
+        return ops.kvstar_table_to_reference(self.table)[..., : self.d_pruned].contiguous()
 
 
 def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pruned_index, topk: int, req_id: int,
@@ -100,6 +118,7 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
             raise RuntimeError("Query shape must be 3D (x, H, d).")
         if blk_repre.dim() != 4:
             raise RuntimeError("BlockRep shape must be 4D (n, M, h, d).")
+        packed = isinstance(blk_repre, BlockRepre)
         x, hq, d_orig = query_group.shape
         n, m, h, dp = blk_repre.shape
         if hq % h != 0:
@@ -119,7 +138,7 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
         ready.record()
         with torch.cuda.stream(_stream):
             _stream.wait_event(ready)
-            table = _head_major(blk_repre)
+            table = blk_repre.table if packed else ops.kvstar_table_from_reference(blk_repre)
             q = query_group.contiguous()
             votes = torch.zeros(max(n, 1), dtype=torch.float32, device=dev)
             k = min(int(topk), n)
@@ -171,8 +190,7 @@ def GetTaskResult(task_id: int):  # noqa: N802
 def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge: int, prune_ratio: float = 1.0,
                         d_pruned_index: Optional[torch.Tensor] = None, prune_dim_enable: bool = False):
     """Sub-block representatives of cache blocks ``vllm_block_ids`` (multistep.py:279-316).
-    Returns (fp16 of shape [n, M, kv_heads, d_pad] - a view of head-major storage - with zero columns past
-    d_pruned, d_pruned_index int64 [kv_heads, d_pruned] or None).  With ``prune_dim_enable`` and a ratio below 0.98 the channels with the largest mean |k|
+    Returns (BlockRepre of shape (n, M, kv_heads, d_pruned), d_pruned_index int64 [kv_heads, d_pruned] or None).  With ``prune_dim_enable`` and a ratio below 0.98 the channels with the largest mean |k|
     over these blocks are kept per head (the reference's choice, :284-292); otherwise a given index is reused."""
     n_total, block_size, kv_heads, head_dim = k_cache.shape
     dev = k_cache.device
@@ -183,8 +201,8 @@ def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge:
         d_pruned_index = d_pruned_index.contiguous()
     d_pruned = head_dim if d_pruned_index is None else d_pruned_index.shape[1]
     d_pad = (d_pruned + 15) // 16 * 16
-    repre = torch.empty((1, kv_heads, len(vllm_block_ids), block_size // merge, d_pad), dtype=torch.float16, device=dev)
+    table = ops.kvstar_table(1, kv_heads, len(vllm_block_ids), block_size // merge, d_pad, dev)
     pruned32 = None if d_pruned_index is None else d_pruned_index.to(torch.int32).contiguous()
     ops.kvstar_block_repre(ops.LayerPointers([k_cache]), ids, torch.arange(len(vllm_block_ids), dtype=torch.int32, device=dev),
-                           repre, block_size, kv_heads, head_dim, n_total, merge, pruned=pruned32)
-    return repre[0].permute(1, 2, 0, 3), d_pruned_index
+                           table, block_size, kv_heads, head_dim, n_total, merge, pruned=pruned32)
+    return BlockRepre(table[0], d_pruned), d_pruned_index
