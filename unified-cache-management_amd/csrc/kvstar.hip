@@ -148,9 +148,11 @@ struct Task {
 };
 
 template <int kM>
-__device__ __forceinline__ void block_sums(const float (&e)[16], int half, float* __restrict__ prow, unsigned blk0,
-                                           unsigned n_blocks)
+__device__ __forceinline__ void block_sums(const float (&e)[16], int half, float* __restrict__ prow, unsigned row_pad,
+                                           unsigned blk0, unsigned n_blocks)
 {
+    // prow points at this lane's row inside block 0 of the [block][row_pad] plane: the 32 rows of one
+    // block are one 128-byte line, written by one store instruction
     // e[i] belongs to sub-block (i/4)*8 + half*4 + i%4 of the tile
     float p4[4];
 #pragma unroll
@@ -164,26 +166,26 @@ __device__ __forceinline__ void block_sums(const float (&e)[16], int half, float
 #pragma unroll
             for (int g = 0; g < kGroups; ++g) { s += p4[b * kGroups + g]; }
             s += __shfl_xor(s, 32, 64);
-            if (half == 0 && blk0 + b < n_blocks) { prow[blk0 + b] = s; }
+            if (half == 0 && blk0 + b < n_blocks) { prow[static_cast<size_t>(blk0 + b) * row_pad] = s; }
         }
     } else if constexpr (kM == 4) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const unsigned b = blk0 + 2 * g + half;
-            if (b < n_blocks) { prow[b] = p4[g]; }
+            if (b < n_blocks) { prow[static_cast<size_t>(b) * row_pad] = p4[g]; }
         }
     } else if constexpr (kM == 2) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const unsigned b = blk0 + 4 * g + 2 * half;
-            if (b < n_blocks) { prow[b] = e[4 * g] + e[4 * g + 1]; }
-            if (b + 1 < n_blocks) { prow[b + 1] = e[4 * g + 2] + e[4 * g + 3]; }
+            if (b < n_blocks) { prow[static_cast<size_t>(b) * row_pad] = e[4 * g] + e[4 * g + 1]; }
+            if (b + 1 < n_blocks) { prow[static_cast<size_t>(b + 1) * row_pad] = e[4 * g + 2] + e[4 * g + 3]; }
         }
     } else {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const unsigned b = blk0 + (i >> 2) * 8 + half * 4 + (i & 3);
-            if (b < n_blocks) { prow[b] = e[i]; }
+            if (b < n_blocks) { prow[static_cast<size_t>(b) * row_pad] = e[i]; }
         }
     }
 }
@@ -275,9 +277,8 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
         if (s0 >= S) { break; }
         const unsigned tile = s0 / kTileSub;
         for (unsigned hi = 0; hi < nh; ++hi) {
-            // heads are visited in an order rotated per wave and tile: consecutive vectors of one head are
-            // kv_heads*d_pad*2 bytes apart, so one head's loads fall on a fraction of the memory channels,
-            // and waves that all walked the heads in the same order would crowd onto the same ones
+            // heads are visited in an order rotated per wave and tile, so that the waves of a workgroup
+            // are not all inside the same head's plane at once
             const unsigned hh = (hi + rot) % nh;
             {   // one load site (selects, no branch): the next head of this tile, or the first head of the wave's next tile
                 const bool last = hi + 1 == nh;
@@ -324,8 +325,8 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
 #pragma unroll
                 for (int i = 0; i < 16; ++i) { e[i] = __expf(sc[i] - mx); }
                 // rows past R hold zero queries: they are computed like the rest and never read
-                if (half == 0) { wmax[static_cast<size_t>(rho) * max_tiles + tile] = mx; }
-                block_sums<kM>(e, half, wpart + static_cast<size_t>(rho) * max_blocks, s0 / kM, n_blocks);
+                if (half == 0) { wmax[static_cast<size_t>(tile) * row_pad + rho] = mx; }
+                block_sums<kM>(e, half, wpart + rho, row_pad, s0 / kM, n_blocks);
             }
 #pragma unroll
             for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = kn[ks]; }
@@ -334,61 +335,71 @@ __global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_k
 }
 
 // ---- votes: rescale to the row maximum, normalise, add the rows ---------------------------------------
-// Phase 1, grid: x = (kv head, row) of the task, y = task; one wave per workgroup.  The row's global
-// maximum and softmax denominator are reduced over its tiles, and each tile maximum in the workspace
-// is replaced by the factor exp(tile max - row max) / denominator its partial sums have to be
-// multiplied with.
-__global__ __launch_bounds__(64) void kvstar_rowscale_kernel(
+// The workspace planes of a (task, kv head) are [tile][row_pad] (tile maxima) and [block][row_pad]
+// (partial sums): the rows of one tile or block are adjacent, so the score kernel's stores and the
+// loads below move whole 128-byte lines.
+//
+// Phase 1, grid: x = kv head, y = task; thread = (group of tiles/blocks, row).  The row's global maximum
+// and softmax denominator are reduced over its tiles, and each tile maximum in the workspace is
+// replaced by the factor exp(tile max - row max) / denominator its partial sums have to be multiplied
+// with.  Rows past tokens*group hold zero queries and are carried along.
+__global__ __launch_bounds__(kThreads) void kvstar_rowscale_kernel(
     float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_len,
-    unsigned n_tokens, unsigned q_heads, unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles,
-    unsigned row_pad)
+    unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles, unsigned row_pad)
 {
-    const unsigned task = blockIdx.y;
+    __shared__ float red[kThreads];
+    const unsigned task = blockIdx.y, h = blockIdx.x;
     const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
-    const unsigned g = q_heads / kv_heads, R = n_tokens * g;
-    const unsigned h = blockIdx.x / R, rho = blockIdx.x - h * R;
-    if (n_blocks == 0 || h >= kv_heads) { return; }
+    if (n_blocks == 0) { return; }
     const unsigned n_tiles = (n_blocks * M + kTileSub - 1) / kTileSub;
-    const int lane = threadIdx.x;
-    float* tm = ws_max + ((static_cast<size_t>(task) * kv_heads + h) * row_pad + rho) * max_tiles;
-    const float* pp = ws_part + ((static_cast<size_t>(task) * kv_heads + h) * row_pad + rho) * max_blocks;
+    const unsigned rho = threadIdx.x % row_pad, grp = threadIdx.x / row_pad, ngrp = kThreads / row_pad;
+    float* tm = ws_max + (static_cast<size_t>(task) * kv_heads + h) * row_pad * max_tiles + rho;
+    const float* pp = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * max_blocks + rho;
     float mx = -INFINITY;
-    for (unsigned t = lane; t < n_tiles; t += 64) { mx = fmaxf(mx, tm[t]); }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) { mx = fmaxf(mx, __shfl_xor(mx, d, 64)); }
+    for (unsigned t = grp; t < n_tiles; t += ngrp) { mx = fmaxf(mx, tm[static_cast<size_t>(t) * row_pad]); }
+    red[threadIdx.x] = mx;
+    __syncthreads();
+    mx = red[rho];
+    for (unsigned g = 1; g < ngrp; ++g) { mx = fmaxf(mx, red[g * row_pad + rho]); }
+    __syncthreads();
     float den = 0.0f;
-    for (unsigned b = lane; b < n_blocks; b += 64) { den += pp[b] * __expf(tm[(b * M) / kTileSub] - mx); }
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) { den += __shfl_xor(den, d, 64); }
+    for (unsigned b = grp; b < n_blocks; b += ngrp) {
+        den += pp[static_cast<size_t>(b) * row_pad] * __expf(tm[static_cast<size_t>((b * M) / kTileSub) * row_pad] - mx);
+    }
+    red[threadIdx.x] = den;
+    __syncthreads();   // also: every read of the tile maxima above precedes the writes below
+    den = red[rho];
+    for (unsigned g = 1; g < ngrp; ++g) { den += red[g * row_pad + rho]; }
     const float inv = den > 1e-9f ? 1.0f / den : 1.0f;   // the reference skips the division then
-    for (unsigned t = lane; t < n_tiles; t += 64) { tm[t] = __expf(tm[t] - mx) * inv; }
+    for (unsigned t = grp; t < n_tiles; t += ngrp) {
+        tm[static_cast<size_t>(t) * row_pad] = __expf(tm[static_cast<size_t>(t) * row_pad] - mx) * inv;
+    }
 }
 
-// Phase 2, grid: x = 256 blocks of the task, y = task: votes[b] = sum over rows of partial * factor.
+// Phase 2, grid: x = 8 blocks of the task, y = task; 32 lanes per block: votes[b] = sum over kv heads and
+// rows of partial * factor.
 __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
     const float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, unsigned n_tokens, unsigned q_heads, unsigned kv_heads, unsigned M,
-    unsigned max_blocks, unsigned max_tiles, unsigned row_pad, float* __restrict__ votes)
+    const int32_t* __restrict__ seg_len, unsigned R, unsigned kv_heads, unsigned M, unsigned max_blocks,
+    unsigned max_tiles, unsigned row_pad, float* __restrict__ votes)
 {
     const unsigned task = blockIdx.y;
     const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
-    const unsigned b = blockIdx.x * kThreads + threadIdx.x;
-    if (b >= n_blocks) { return; }
-    const unsigned g = q_heads / kv_heads, R = n_tokens * g;
+    if (blockIdx.x * 8 >= n_blocks) { return; }
+    const unsigned b = blockIdx.x * 8 + (threadIdx.x >> 5), l32 = threadIdx.x & 31;
+    const bool live = b < n_blocks;
     const unsigned tile = (b * M) / kTileSub;
-    const float* wmax = ws_max + static_cast<size_t>(task) * kv_heads * row_pad * max_tiles;
-    const float* wpart = ws_part + static_cast<size_t>(task) * kv_heads * row_pad * max_blocks;
-    float v0 = 0.0f, v1 = 0.0f;
-    for (unsigned h = 0; h < kv_heads; ++h) {
-        const size_t r0 = static_cast<size_t>(h) * row_pad;
-        unsigned rho = 0;
-        for (; rho + 1 < R; rho += 2) {
-            v0 += wpart[(r0 + rho) * max_blocks + b] * wmax[(r0 + rho) * max_tiles + tile];
-            v1 += wpart[(r0 + rho + 1) * max_blocks + b] * wmax[(r0 + rho + 1) * max_tiles + tile];
+    float v = 0.0f;
+    if (live) {
+        for (unsigned h = 0; h < kv_heads; ++h) {
+            const float* wpart = ws_part + ((static_cast<size_t>(task) * kv_heads + h) * max_blocks + b) * row_pad;
+            const float* wfac = ws_max + ((static_cast<size_t>(task) * kv_heads + h) * max_tiles + tile) * row_pad;
+            for (unsigned rho = l32; rho < R; rho += 32) { v += wpart[rho] * wfac[rho]; }
         }
-        if (rho < R) { v0 += wpart[(r0 + rho) * max_blocks + b] * wmax[(r0 + rho) * max_tiles + tile]; }
     }
-    votes[seg_off[task] + b] = v0 + v1;
+#pragma unroll
+    for (int d = 16; d >= 1; d >>= 1) { v += __shfl_xor(v, d, 64); }
+    if (live && l32 == 0) { votes[seg_off[task] + b] = v; }
 }
 
 unsigned g_heads_per_group = 1;
@@ -532,13 +543,11 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
 #undef UCM_KVSTAR_LAUNCH2
 #undef UCM_KVSTAR_ARGS
     if (hipError_t e = hipGetLastError(); e != hipSuccess) { return ucm::check_hip(e, "ucm_kvstar_votes (scores)"); }
-    hipLaunchKernelGGL(kvstar_rowscale_kernel, dim3(static_cast<unsigned>(kv_heads) * R, n_tasks), dim3(64), 0, s, ws_max,
-                       ws_part, seg_len, static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads),
-                       static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks), static_cast<unsigned>(max_blocks),
-                       max_tiles, row_pad);
-    hipLaunchKernelGGL(kvstar_vote_kernel, dim3((max_blocks + kThreads - 1) / kThreads, n_tasks), dim3(kThreads), 0, s, ws_max,
-                       ws_part, seg_off, seg_len, static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads),
-                       static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks), static_cast<unsigned>(max_blocks),
-                       max_tiles, row_pad, votes);
+    hipLaunchKernelGGL(kvstar_rowscale_kernel, dim3(static_cast<unsigned>(kv_heads), n_tasks), dim3(kThreads), 0, s, ws_max,
+                       ws_part, seg_len, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
+                       static_cast<unsigned>(max_blocks), max_tiles, row_pad);
+    hipLaunchKernelGGL(kvstar_vote_kernel, dim3((max_blocks + 7) / 8, n_tasks), dim3(kThreads), 0, s, ws_max, ws_part, seg_off,
+                       seg_len, R, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
+                       static_cast<unsigned>(max_blocks), max_tiles, row_pad, votes);
     UCM_LAUNCH_CHECK("ucm_kvstar_votes");
 }
