@@ -273,11 +273,14 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   pruned   dev int32[kv_heads][d_pruned]: channel of every kept dim (the
  *            reference's d_pruned_index, :288-304), or NULL when d_pruned ==
  *            head_dim
- *   repre    dev fp16, HEAD-MAJOR: [n_layers][kv_heads][repre_rows][M][d_pad],
- *            d_pad >= d_pruned (columns past d_pruned are written as zero);
- *            repre_layer_stride and repre_head_stride in elements.  (The
- *            reference keeps [row][M][kv head][d]; head-major makes the vectors
- *            a workgroup streams for one head contiguous.)
+ *   repre    dev fp16, [n_layers][kv_heads][repre_rows][d_pad/8][M][8]: kv
+ *            head outermost, and inside a block the 16-byte pieces (8
+ *            channels) of its M sub-blocks side by side; d_pad >= d_pruned, a
+ *            multiple of 8 (16 for ucm_kvstar_votes), columns past d_pruned
+ *            are written as zero; repre_layer_stride and repre_head_stride in
+ *            elements.  (The reference keeps [row][M][kv head][d]; this order
+ *            makes what a workgroup streams for one head contiguous and every
+ *            load instruction of the score kernel a run of whole cache lines.)
  *
  * ucm_kvstar_votes: the arithmetic of KVStar::Execute
  * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:817-990)
@@ -292,8 +295,8 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   pruned   dev int32[*][kv_heads][d_pruned] channel lists, pruned_sel dev
  *            int32[n_tasks] picks one per task (-1: none); both NULL when
  *            d_pruned == d_orig
- *   repre_f16  dev fp16 head-major [kv_heads][rows][sub_blocks][d_pad], head
- *            planes repre_head_stride elements apart; task t owns rows
+ *   repre_f16  dev fp16 [kv_heads][rows][d_pad/8][sub_blocks][8] (one layer of
+ *            the table above), head planes repre_head_stride elements apart; task t owns rows
  *            seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >= every seg_len
  *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
  *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev fp32, task t's votes at votes[seg_off[t] + b].
@@ -305,9 +308,15 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
                            int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
                            int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
                            int64_t repre_head_stride, ucm_stream_t stream);
-/* Tuning knob for benchmarks: kv heads per workgroup of the KVStar score kernel
- * (1..8, default 1).  Not part of the reference interface. */
-int ucm_set_kvstar_heads_per_group(int heads);
+/* Tuning knob for benchmarks and tests.  ucm_kvstar_votes has two paths: one
+ * workgroup per (task, kv head) that keeps the task's per-(block, query row)
+ * sums in LDS and stores only the head's share of the votes (taken when there
+ * are at least 1024 such pairs and the plane fits 159 KiB), and a workspace
+ * path that may cut a task into chunks.  tiles > 0: the workspace path with
+ * that many 32-sub-block tiles per wave (four waves per workgroup); -1: the
+ * in-LDS path whenever the plane fits; 0: automatic.  Not part of the
+ * reference interface. */
+int ucm_set_kvstar_tiles_per_wave(int tiles);
 int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks,
                                 int sub_blocks, int64_t* max_floats, int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,

@@ -99,21 +99,49 @@ def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
     wants = {t: O.kvstar_retrieve(qs[t], repre[sum(lens[:t]) : sum(lens[:t]) + n], topk=max(n // 3, 1))[1]
              for t, n in enumerate(lens) if n}
     try:
-        for heads_per_group in (1, 3, 8):                     # kv heads one workgroup walks
-            ops.set_kvstar_heads_per_group(heads_per_group)
+        for tiles_per_wave in (0, -1, 1, 3):                  # 0: automatic, -1: per-task plane in LDS, n: chunks of 4n tiles
+            ops.set_kvstar_tiles_per_wave(tiles_per_wave)
             got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
             for t, n in enumerate(lens):
                 if n == 0:
                     continue
-                assert np.allclose(got[off[t] : off[t] + n], wants[t], rtol=VOTE_RTOL, atol=VOTE_ATOL), (heads_per_group, t, n)
+                assert np.allclose(got[off[t] : off[t] + n], wants[t], rtol=VOTE_RTOL, atol=VOTE_ATOL), (tiles_per_wave, t, n)
                 # what the mathematics fixes whatever the order: every row's probabilities add up to one
                 assert abs(got[off[t] : off[t] + n].sum() - x * hq) < 1e-3 * x * hq
     finally:
-        ops.set_kvstar_heads_per_group(1)
+        ops.set_kvstar_tiles_per_wave(0)
 
 
-def test_kvstar_pruned_channels_and_selection(ucm, dev):
+def test_kvstar_many_short_tasks_take_the_in_lds_path(ucm, dev):
+    """Enough (task, kv head) pairs that the automatic choice is one workgroup per pair with the task's
+    per-block sums in LDS; ragged lengths including empty tasks."""
     from ucm_amd import ops
+
+    x, hq, hkv, d, M = 8, 32, 8, 128, 8
+    lens = [int(v) for v in synth.permutation(1150, 150) % 41]     # 0..40 blocks, 150 tasks -> 1200 pairs
+    rows = int(np.sum(lens))
+    repre = f16_bits(synth.normal_f32(1151, (rows, M, hkv, d)) * np.float32(0.25))
+    qs = [f16_bits(synth.normal_f32(1152 + t, (x, hq, d)) * np.float32(0.25)) for t in range(len(lens))]
+    got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
+    for t, n in enumerate(lens):
+        if n == 0:
+            continue
+        want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=1)[1]
+        assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
+
+
+@pytest.mark.parametrize("tiles_per_wave", [0, -1])
+def test_kvstar_pruned_channels_and_selection(ucm, dev, tiles_per_wave):
+    from ucm_amd import ops
+
+    ops.set_kvstar_tiles_per_wave(tiles_per_wave)
+    try:
+        _pruned_channels_and_selection(ops, dev)
+    finally:
+        ops.set_kvstar_tiles_per_wave(0)
+
+
+def _pruned_channels_and_selection(ops, dev):
 
     x, hq, hkv, d, M, dp = 8, 32, 8, 128, 8, 77              # 77 kept channels: table rows padded to 80
     lens = [90, 33]

@@ -37,6 +37,8 @@ constexpr int kMaxRows = 64;          // tokens * group size per kv head
 constexpr int kMaxDim = 128;
 constexpr int kQStride = kMaxDim + 8; // fp16 elements per staged query row (272 B: spreads LDS banks)
 constexpr int kTileSub = 32;          // sub-blocks per MFMA tile
+constexpr int64_t kLdsPathMinGroups = 1024;           // (task, kv head) pairs from which the in-LDS path is taken
+constexpr size_t kLdsPathMaxBytes = 159 * 1024;       // of the 160 KiB a compute unit has
 
 __device__ __forceinline__ unsigned short f32_to_f16_bits(float f)
 {
@@ -147,12 +149,12 @@ struct Task {
     unsigned n_blocks;
 };
 
-template <int kM>
-__device__ __forceinline__ void block_sums(const float (&e)[16], int half, float* __restrict__ prow, unsigned row_pad,
-                                           unsigned blk0, unsigned n_blocks)
+// Hands the per-block sums of a tile's 32 exponentials for this lane's row to put(block within the tile,
+// sum) and returns their total (both lane halves included).  put is called unconditionally by all 64 lanes:
+// a store the compiler has to branch around would make it wait for ALL outstanding memory operations.
+template <int kM, typename Put>
+__device__ __forceinline__ float block_sums(const float (&e)[16], int half, Put put)
 {
-    // prow points at this lane's row inside block 0 of the [block][row_pad] plane: the 32 rows of one
-    // block are one 128-byte line, written by one store instruction
     // e[i] belongs to sub-block (i/4)*8 + half*4 + i%4 of the tile
     float p4[4];
 #pragma unroll
@@ -160,219 +162,383 @@ __device__ __forceinline__ void block_sums(const float (&e)[16], int half, float
     if constexpr (kM >= 8) {
         constexpr int kGroups = kM / 8;                  // 8-sub-block groups per block
         constexpr int kBlocks = 4 / kGroups;             // blocks per tile
+        float sum[kBlocks];
+        float total = 0.0f;
 #pragma unroll
         for (int b = 0; b < kBlocks; ++b) {
-            float s = 0.0f;
+            float v = 0.0f;
 #pragma unroll
-            for (int g = 0; g < kGroups; ++g) { s += p4[b * kGroups + g]; }
-            s += __shfl_xor(s, 32, 64);
-            if (half == 0 && blk0 + b < n_blocks) { prow[static_cast<size_t>(blk0 + b) * row_pad] = s; }
+            for (int g = 0; g < kGroups; ++g) { v += p4[b * kGroups + g]; }
+            sum[b] = v + __shfl_xor(v, 32, 64);          // both halves now hold the block's sum
+            total += sum[b];
         }
-    } else if constexpr (kM == 4) {
+        if constexpr (kBlocks == 1) {
+            put(0u, sum[0]);                             // the two halves put the same value in the same place
+        } else {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const unsigned b = blk0 + 2 * g + half;
-            if (b < n_blocks) { prow[static_cast<size_t>(b) * row_pad] = p4[g]; }
+            for (int j = 0; j < kBlocks / 2; ++j) {      // lower half: block 2j, upper half: block 2j+1
+                put(static_cast<unsigned>(2 * j + half), half ? sum[2 * j + 1] : sum[2 * j]);
+            }
         }
-    } else if constexpr (kM == 2) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const unsigned b = blk0 + 4 * g + 2 * half;
-            if (b < n_blocks) { prow[static_cast<size_t>(b) * row_pad] = e[4 * g] + e[4 * g + 1]; }
-            if (b + 1 < n_blocks) { prow[static_cast<size_t>(b + 1) * row_pad] = e[4 * g + 2] + e[4 * g + 3]; }
-        }
+        return total;
     } else {
+        if constexpr (kM == 4) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const unsigned b = blk0 + (i >> 2) * 8 + half * 4 + (i & 3);
-            if (b < n_blocks) { prow[static_cast<size_t>(b) * row_pad] = e[i]; }
+            for (int g = 0; g < 4; ++g) { put(static_cast<unsigned>(2 * g + half), p4[g]); }
+        } else if constexpr (kM == 2) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                put(static_cast<unsigned>(4 * g + 2 * half), e[4 * g] + e[4 * g + 1]);
+                put(static_cast<unsigned>(4 * g + 2 * half + 1), e[4 * g + 2] + e[4 * g + 3]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { put(static_cast<unsigned>((i >> 2) * 8 + half * 4 + (i & 3)), e[i]); }
         }
+        float total = (p4[0] + p4[1]) + (p4[2] + p4[3]);
+        total += __shfl_xor(total, 32, 64);
+        return total;
     }
 }
 
-// grid: x = chunk of sub-blocks, y = group of kv heads, z = task.  The table is head-major and
-// piece-interleaved inside a block (see above), so what one workgroup streams for a head is one
-// contiguous run read in whole lines (in the reference's [row][sub-block][kv head][d] order each
-// vector of a head sits kv_heads*d*2 bytes from the next).  The queries of the group's heads are
-// staged in LDS once per workgroup.
-template <int kM, bool kTwoRowTiles>
-__global__ __launch_bounds__(kThreads, kTwoRowTiles ? 2 : 3) void kvstar_score_kernel(
+constexpr float kLog2e = 1.4426950408889634f;
+
+// grid: x = chunk of sub-blocks, y = kv head, z = task.  The table is head-major and piece-interleaved
+// inside a block (see above), so what one workgroup streams is one contiguous run read in whole lines
+// (in the reference's [row][sub-block][kv head][d] order each vector of a head sits kv_heads*d*2 bytes
+// from the next).  The head's query rows are staged in LDS once per workgroup.
+//
+// kLds == false (any task length; a task may be cut into chunks): per 32-sub-block tile and query row
+// the kernel leaves the tile's maximum and sum of exponentials ([tile][2][row_pad]) and the per-block
+// sums ([block][row_pad], blocks padded to whole tiles) in the workspace for the two kernels below.
+//
+// kLds == true (one workgroup walks the whole task and the task's [block][row_pad] plane fits LDS): the
+// plane stays in LDS, as log2 of each block's sum of exponentials (one number instead of a sum and the
+// maximum it is relative to), the workgroup itself reduces every row's maximum and denominator when it
+// is through, and only this head's share of the votes ([task][kv head][max_blocks], in ws_part) goes
+// to memory: 1/32 of the other path's stores, whose number per compute unit - not their bytes - is
+// what that path pays for.
+template <int kM, bool kTwoRowTiles, bool kLds>
+__global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const unsigned short* __restrict__ q, const int64_t* __restrict__ q_off, unsigned n_tokens, unsigned q_heads,
     unsigned d_orig, const int32_t* __restrict__ pruned, const int32_t* __restrict__ pruned_sel,
     const unsigned short* __restrict__ table, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
     float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
-    unsigned tiles_per_wave, unsigned row_pad, unsigned heads_per_group)
+    unsigned tiles_per_wave, unsigned row_pad, unsigned plane_offset)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned short q_s[];   // [heads_per_group][row_pad][kQStride]
+    extern __shared__ __attribute__((aligned(16))) unsigned short q_s[];   // [row_pad][kQStride]
+    // kLds: [block][row_pad] floats from byte plane_offset on (0 with one row tile: the queries then live in
+    // registers once the loop starts), followed by the waves' [wave][2][row_pad] running (maximum, sum) pairs
+    float* plane = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(q_s) + plane_offset);
 
-    const unsigned task = blockIdx.z;
-    const unsigned h_first = blockIdx.y * heads_per_group;
-    const unsigned nh = min(heads_per_group, kv_heads - h_first);
-    const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
+    const unsigned task = blockIdx.z, h = blockIdx.y;
+    const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);   // the planes are sized for max_blocks
     const unsigned S = n_blocks * kM;
     const unsigned chunk = kWaves * tiles_per_wave * kTileSub;
     const unsigned s_chunk = blockIdx.x * chunk;
     if (s_chunk >= S) { return; }
+    const unsigned s_last = min(S, s_chunk + chunk) - 1;  // last sub-block of this workgroup
     const unsigned g = q_heads / kv_heads, R = n_tokens * g;
     const int32_t psel = pruned_sel ? pruned_sel[task] : -1;
-    const int32_t* pr0 = (pruned && psel >= 0) ? pruned + static_cast<size_t>(psel) * kv_heads * d_pruned : nullptr;
-
-    // ---- the group's query rows, gathered by the kept channels, zero padded (rows up to row_pad, columns up to d_pad)
-    const unsigned short* qt = q + q_off[task];
-    if (!pr0 && d_pruned == d_pad && (d_orig % 8) == 0 && (reinterpret_cast<uintptr_t>(qt) & 15u) == 0) {
-        const unsigned cpr = d_pad / 8;                  // 16-byte pieces per row
-        for (unsigned e = threadIdx.x; e < nh * row_pad * cpr; e += kThreads) {
-            const unsigned hr = e / cpr, c = e - hr * cpr;
-            const unsigned hh = hr / row_pad, rho = hr - hh * row_pad;
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (rho < R) {
-                const unsigned xt = rho / g, gg = rho - xt * g;
-                v = ucm::gload16(qt + (static_cast<size_t>(xt) * q_heads + (h_first + hh) * g + gg) * d_orig + c * 8);
-            }
-            *reinterpret_cast<u32x4*>(&q_s[hr * kQStride + c * 8]) = v;
-        }
-    } else {
-        for (unsigned e = threadIdx.x; e < nh * row_pad * d_pad; e += kThreads) {
-            const unsigned hr = e / d_pad, p = e - hr * d_pad;
-            const unsigned hh = hr / row_pad, rho = hr - hh * row_pad;
-            unsigned short v = 0;
-            if (rho < R && p < d_pruned) {
-                const unsigned xt = rho / g, gg = rho - xt * g;
-                const unsigned d = pr0 ? static_cast<unsigned>(pr0[(h_first + hh) * d_pruned + p]) : p;
-                if (d < d_orig) { v = qt[(static_cast<size_t>(xt) * q_heads + (h_first + hh) * g + gg) * d_orig + d]; }
-            }
-            q_s[hr * kQStride + p] = v;
-        }
-    }
-    __syncthreads();
+    const int32_t* pr = (pruned && psel >= 0) ? pruned + (static_cast<size_t>(psel) * kv_heads + h) * d_pruned : nullptr;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = lane >> 5, lr = lane & 31;
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes piece 2*ks + half
-    const unsigned hoff = half * 8;
-    constexpr bool two_row_tiles = kTwoRowTiles;   // 33..64 query rows per kv head
-    // head-major table: head h's vectors of all sub-blocks are contiguous, d_pad elements each
-    const unsigned short* tbase = table + static_cast<int64_t>(h_first) * head_stride +
+    constexpr int kRowTiles = kTwoRowTiles ? 2 : 1;      // 33..64 query rows per kv head take two
+    constexpr unsigned kStride = kWaves * kTileSub;      // from one tile of a wave to its next
+    const unsigned short* tbase = table + static_cast<int64_t>(h) * head_stride +
                                   static_cast<size_t>(seg_off[task]) * kM * d_pad + half * (8 * kM);
 
-    // A (tile, head) step's keys: eight 16-byte loads per lane, piece 2*ks + half of its sub-block; the
-    // lanes of one instruction cover M*16 contiguous bytes per block and lane half.  Everything is
-    // unconditional - MFMA steps past d_pad reload piece 0 and are multiplied with a zero query fragment,
-    // lanes and tiles past the end reload the last vector and are masked - so that the loads of the NEXT
-    // step can be issued before this step's arithmetic without a branch around them.
-    auto load_keys = [&](u32x4 (&kf)[kMaxDim / 16], unsigned s0, unsigned hh) {
-        const unsigned s_mine = min(s0 + lr, S - 1);
-        const unsigned short* krow = tbase + static_cast<int64_t>(hh) * head_stride +
-                                     static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
+    // A tile's keys: eight 16-byte loads per lane, piece 2*ks + half of its sub-block; the lanes of one
+    // instruction cover M*16 contiguous bytes per block and lane half.  Everything is unconditional - MFMA
+    // steps past d_pad reload piece 0 and are multiplied with a zero query fragment, lanes and tiles past
+    // the workgroup's end reload its last vector and are masked or never used.
+    //
+    // Three key buffers rotate, so two tiles are in flight while one is worked on.  The loads and the waits
+    // for them are written as assembly: left to itself the compiler sinks a prefetch down to the tile that
+    // consumes it (there is nothing but a loop exit in between), which leaves nothing in flight.  Vector
+    // memory operations complete in issue order, loads and stores alike, so "the loads of tile t have
+    // landed" is "at most as many operations outstanding as were issued after them" (keys_landed below).
+    auto load_keys = [&](u32x4 (&kf)[kMaxDim / 16], unsigned s0) {
+        const unsigned s_mine = min(s0 + lr, s_last);
+        const unsigned short* krow = tbase + static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
 #pragma unroll
-        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = ucm::gload16(krow + (ks < ksteps ? ks : 0u) * (16 * kM)); }
+        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
+            const unsigned short* p = krow + (ks < ksteps ? ks : 0u) * (16 * kM);
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kf[ks]) : "v"(p) : "memory");
+        }
     };
-    u32x4 kf[kMaxDim / 16], kn[kMaxDim / 16];
-    const unsigned t_end = kWaves * tiles_per_wave;
-    unsigned rot = (wave * 3u + blockIdx.x + task) % nh;
-    load_keys(kf, s_chunk + wave * kTileSub, rot);
-    for (unsigned t = wave; t < t_end; t += kWaves, rot = (rot + 1) % nh) {
-        const unsigned s0 = s_chunk + t * kTileSub;
-        if (s0 >= S) { break; }
-        const unsigned tile = s0 / kTileSub;
-        for (unsigned hi = 0; hi < nh; ++hi) {
-            // heads are visited in an order rotated per wave and tile, so that the waves of a workgroup
-            // are not all inside the same head's plane at once
-            const unsigned hh = (hi + rot) % nh;
-            {   // one load site (selects, no branch): the next head of this tile, or the first head of the wave's next tile
-                const bool last = hi + 1 == nh;
-                load_keys(kn, last ? s0 + kWaves * kTileSub : s0, (last ? rot + 1 : hi + 1 + rot) % nh);
+    u32x4 k0[kMaxDim / 16], k1[kMaxDim / 16], k2[kMaxDim / 16];
+    const unsigned s_first = s_chunk + wave * kTileSub;
+    load_keys(k0, s_first);
+    load_keys(k1, s_first + kStride);
+    load_keys(k2, s_first + 2 * kStride);
+
+    // ---- the head's query rows, gathered by the kept channels, zero padded (rows up to row_pad, columns up to d_pad)
+    const unsigned short* qt = q + q_off[task];
+    if (!pr && d_pruned == d_pad && (d_orig % 8) == 0 && (reinterpret_cast<uintptr_t>(qt) & 15u) == 0) {
+        const unsigned cpr = d_pad / 8;                  // 16-byte pieces per row
+        for (unsigned e = threadIdx.x; e < row_pad * cpr; e += kThreads) {
+            const unsigned rho = e / cpr, c = e - rho * cpr;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (rho < R) {
+                const unsigned xt = rho / g, gg = rho - xt * g;
+                v = ucm::gload16(qt + (static_cast<size_t>(xt) * q_heads + h * g + gg) * d_orig + c * 8);
             }
-            const unsigned short* qh = q_s + static_cast<size_t>(hh) * row_pad * kQStride;
-            const u32x4 zero = {0u, 0u, 0u, 0u};
-            f32x16 acc0, acc1;
+            *reinterpret_cast<u32x4*>(&q_s[rho * kQStride + c * 8]) = v;
+        }
+    } else {
+        for (unsigned e = threadIdx.x; e < row_pad * d_pad; e += kThreads) {
+            const unsigned rho = e / d_pad, p = e - rho * d_pad;
+            unsigned short v = 0;
+            if (rho < R && p < d_pruned) {
+                const unsigned xt = rho / g, gg = rho - xt * g;
+                const unsigned d = pr ? static_cast<unsigned>(pr[p]) : p;
+                if (d < d_orig) { v = qt[(static_cast<size_t>(xt) * q_heads + h * g + gg) * d_orig + d]; }
+            }
+            q_s[rho * kQStride + p] = v;
+        }
+    }
+    __syncthreads();
+
+    // the query fragments do not change from tile to tile: with one row tile they stay in registers
+    u32x4 bq[kTwoRowTiles ? 1 : kMaxDim / 16];
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    if constexpr (!kTwoRowTiles) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { acc0[i] = 0.0f; acc1[i] = 0.0f; }
+        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
+            const u32x4 braw = *reinterpret_cast<const u32x4*>(&q_s[lr * kQStride + half * 8 + (ks < ksteps ? ks : 0u) * 16]);
+            bq[ks] = ks < ksteps ? braw : zero;
+        }
+    }
+
+    if constexpr (kLds) { __syncthreads(); }             // every wave has its query fragments: the plane may overwrite them
+
+    float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h) * (2 * row_pad) * max_tiles;          // [tile][2][row_pad]
+    float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * (kTileSub / kM) * max_tiles;  // [block][row_pad]
+
+    float m_run[kRowTiles], d_run[kRowTiles];            // kLds only
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt) { m_run[rt] = -INFINITY; d_run[rt] = 0.0f; }
+
+    auto process = [&](const u32x4 (&kf)[kMaxDim / 16], unsigned s0) {
+        const unsigned tile = s0 / kTileSub;
+        f32x16 acc[kRowTiles];
+#pragma unroll
+        for (int rt = 0; rt < kRowTiles; ++rt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { acc[rt][i] = 0.0f; }
 #pragma unroll
             for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-                const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 16;
-                const u32x4 braw = *reinterpret_cast<const u32x4*>(&qh[lr * kQStride + col]);
-                const f16x8 b0 = __builtin_bit_cast(f16x8, ks < ksteps ? braw : zero);
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), b0, acc0, 0, 0, 0);
-            }
-            if (two_row_tiles) {
-#pragma unroll
-                for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-                    const unsigned col = hoff + (ks < ksteps ? ks : 0u) * 16;
-                    const u32x4 braw = *reinterpret_cast<const u32x4*>(&qh[(32 + lr) * kQStride + col]);
-                    const f16x8 b1 = __builtin_bit_cast(f16x8, ks < ksteps ? braw : zero);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), b1, acc1, 0, 0, 0);
+                u32x4 b;
+                if constexpr (kTwoRowTiles) {
+                    const u32x4 braw = *reinterpret_cast<const u32x4*>(
+                        &q_s[(rt * 32 + lr) * kQStride + half * 8 + (ks < ksteps ? ks : 0u) * 16]);
+                    b = ks < ksteps ? braw : zero;
+                } else {
+                    b = bq[ks];
                 }
+                acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), __builtin_bit_cast(f16x8, b),
+                                                                acc[rt], 0, 0, 0);
             }
-            float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h_first + hh) * row_pad * max_tiles;
-            float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h_first + hh) * row_pad * max_blocks;
+        }
+        const bool full = s0 + kTileSub <= S;            // wave-uniform: only a task's last tile needs the mask
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
-                if (rt == 1 && !two_row_tiles) { break; }
-                const unsigned rho = rt * 32 + lr;
-                float sc[16];
-                float mx = -INFINITY;
+        for (int rt = 0; rt < kRowTiles; ++rt) {
+            const unsigned rho = rt * 32 + lr;
+            float sc[16];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
-                    const float v = rt == 0 ? acc0[i] : acc1[i];
-                    sc[i] = s < S ? v : -INFINITY;
-                    mx = fmaxf(mx, sc[i]);
-                }
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // the tile has at least one live sub-block, so mx is finite
-                float e[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) { e[i] = __expf(sc[i] - mx); }
-                // rows past R hold zero queries: they are computed like the rest and never read
-                if (half == 0) { wmax[static_cast<size_t>(tile) * row_pad + rho] = mx; }
-                block_sums<kM>(e, half, wpart + rho, row_pad, s0 / kM, n_blocks);
+            for (int i = 0; i < 16; ++i) {
+                const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
+                sc[i] = (full || s < S) ? acc[rt][i] : -INFINITY;
             }
+            float mx = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
 #pragma unroll
-            for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) { kf[ks] = kn[ks]; }
+            for (int i = 3; i < 15; i += 2) { mx = fmaxf(fmaxf(mx, sc[i]), sc[i + 1]); }
+            mx = fmaxf(mx, sc[15]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));      // the tile has at least one live sub-block, so mx is finite
+            const float nmx = -mx * kLog2e;
+            float e[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], kLog2e, nmx)); }
+            // rows past R hold zero queries: they are computed like the rest and never read
+            const unsigned blk0 = tile * (kTileSub / kM);
+            if constexpr (kLds) {
+                const float mx2 = mx * kLog2e;
+                const float total = block_sums<kM>(e, half, [&](unsigned b, float v) {
+                    plane[(blk0 + b) * row_pad + rho] = mx2 + __builtin_amdgcn_logf(v);   // log2 of the block's sum of 2^(score*log2e)
+                });
+                // the wave's running (maximum, sum of 2^(x - maximum)) of the row, in the same log2 units
+                const float m_new = fmaxf(m_run[rt], mx2);
+                d_run[rt] = d_run[rt] * __builtin_amdgcn_exp2f(m_run[rt] - m_new) + total * __builtin_amdgcn_exp2f(mx2 - m_new);
+                m_run[rt] = m_new;
+            } else {
+                const float total = block_sums<kM>(e, half, [&](unsigned b, float v) {
+                    wpart[static_cast<size_t>(blk0 + b) * row_pad + rho] = v;
+                });
+                wmax[(static_cast<size_t>(tile) * 2 + half) * row_pad + rho] = half ? total : mx;
+            }
+        }
+    };
+
+    // Operations issued after a tile's loads when the wave turns to it: the loads of the two tiles behind it
+    // (16) and the stores of the tiles worked on since - none for the wave's first tile, one tile's for its
+    // second, two tiles' from then on.
+    constexpr unsigned kStores = kLds ? 0 : kRowTiles * (1 + (kM >= 16 ? 1 : kM == 8 ? 2 : kM == 4 ? 4 : kM == 2 ? 8 : 16));
+    constexpr unsigned kAfter0 = 16, kAfter1 = 16 + kStores > 63 ? 63 : 16 + kStores,
+                       kAfter2 = 16 + 2 * kStores > 63 ? 63 : 16 + 2 * kStores;
+#define UCM_KEYS_LANDED(k, n)                                                                                              \
+    asm volatile("s_waitcnt vmcnt(%8)"                                                                                     \
+                 : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]), "+v"(k[4]), "+v"(k[5]), "+v"(k[6]), "+v"(k[7])         \
+                 : "n"(n)                                                                                                  \
+                 : "memory")
+    const unsigned s_end = min(S, s_chunk + chunk);
+    unsigned s0 = s_first;
+    if (s0 < s_end) {                                    // the wave's first two tiles, with fewer stores behind them
+        UCM_KEYS_LANDED(k0, kAfter0);
+        process(k0, s0);
+        load_keys(k0, s0 + 3 * kStride);
+        s0 += kStride;
+        if (s0 < s_end) {
+            UCM_KEYS_LANDED(k1, kAfter1);
+            process(k1, s0);
+            load_keys(k1, s0 + 3 * kStride);
+            s0 += kStride;
+        }
+    }
+    while (s0 < s_end) {                                 // buffers k2, k0, k1, k2, ... from here on
+        UCM_KEYS_LANDED(k2, kAfter2);
+        process(k2, s0);
+        load_keys(k2, s0 + 3 * kStride);
+        s0 += kStride;
+        if (s0 >= s_end) { break; }
+        UCM_KEYS_LANDED(k0, kAfter2);
+        process(k0, s0);
+        load_keys(k0, s0 + 3 * kStride);
+        s0 += kStride;
+        if (s0 >= s_end) { break; }
+        UCM_KEYS_LANDED(k1, kAfter2);
+        process(k1, s0);
+        load_keys(k1, s0 + 3 * kStride);
+        s0 += kStride;
+    }
+#undef UCM_KEYS_LANDED
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the prefetches past the end: nothing stays in flight
+
+    if constexpr (kLds) {
+        // ---- this head's share of the votes, from the plane in LDS
+        float* red = plane + static_cast<size_t>(max_tiles) * (kTileSub / kM) * row_pad;   // [wave][2][row_pad]
+        if (half == 0) {
+#pragma unroll
+            for (int rt = 0; rt < kRowTiles; ++rt) {
+                red[(wave * 2 + 0) * row_pad + rt * 32 + lr] = m_run[rt];
+                red[(wave * 2 + 1) * row_pad + rt * 32 + lr] = d_run[rt];
+            }
+        }
+        __syncthreads();                                 // the plane and the waves' pairs are complete
+        float row_m = 0.0f, row_w = 0.0f;
+        if (threadIdx.x < row_pad) {
+            row_m = red[threadIdx.x];                    // wave 0 always has a tile, so this is finite
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) { row_m = fmaxf(row_m, red[(w * 2) * row_pad + threadIdx.x]); }
+            float den = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                den += red[(w * 2 + 1) * row_pad + threadIdx.x] * __builtin_amdgcn_exp2f(red[(w * 2) * row_pad + threadIdx.x] - row_m);
+            }
+            row_w = threadIdx.x < R ? 1.0f / den : 0.0f; // den >= 1: the row's largest term is 2^0; padding rows do not vote
+        }
+        __syncthreads();                                 // (a thread reads only its own column of the pairs)
+        if (threadIdx.x < row_pad) {
+            red[threadIdx.x] = row_m;
+            red[row_pad + threadIdx.x] = row_w;
+        }
+        __syncthreads();
+        // one thread per block walks the block's rows, starting at a row of its own so that the lanes of a
+        // wave spread over the LDS banks
+        float* vh = ws_part + (static_cast<size_t>(task) * kv_heads + h) * max_blocks;
+        for (unsigned b = threadIdx.x; b < n_blocks; b += kThreads) {
+            float v = 0.0f;
+            for (unsigned r = 0; r < row_pad; ++r) {
+                const unsigned rr = (r + b) & (row_pad - 1);
+                v += __builtin_amdgcn_exp2f(plane[b * row_pad + rr] - red[rr]) * red[row_pad + rr];
+            }
+            vh[b] = v;
         }
     }
 }
 
+// kLds path, grid: x = 256 blocks of the task, y = task: adds up the kv heads' shares of the votes.
+__global__ __launch_bounds__(kThreads) void kvstar_headsum_kernel(
+    const float* __restrict__ head_votes, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
+    unsigned kv_heads, unsigned max_blocks, float* __restrict__ votes)
+{
+    const unsigned task = blockIdx.y, b = blockIdx.x * kThreads + threadIdx.x;
+    if (b >= min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks)) { return; }
+    float v = 0.0f;
+    for (unsigned h = 0; h < kv_heads; ++h) { v += head_votes[(static_cast<size_t>(task) * kv_heads + h) * max_blocks + b]; }
+    votes[seg_off[task] + b] = v;
+}
+
 // ---- votes: rescale to the row maximum, normalise, add the rows ---------------------------------------
-// The workspace planes of a (task, kv head) are [tile][row_pad] (tile maxima) and [block][row_pad]
-// (partial sums): the rows of one tile or block are adjacent, so the score kernel's stores and the
-// loads below move whole 128-byte lines.
+// The workspace planes of a (task, kv head) keep the rows of one tile or block adjacent
+// ([tile][2][row_pad], [block][row_pad]), so the score kernel's stores and the loads below move whole
+// 128-byte lines.
 //
-// Phase 1, grid: x = kv head, y = task; thread = (group of tiles/blocks, row).  The row's global maximum
-// and softmax denominator are reduced over its tiles, and each tile maximum in the workspace is
-// replaced by the factor exp(tile max - row max) / denominator its partial sums have to be multiplied
+// Phase 1, grid: x = kv head, y = task; thread = (group of tiles, row).  The tiles' (maximum, sum) pairs
+// give the row's global maximum and softmax denominator; each tile maximum in the workspace is replaced
+// by the factor exp(tile max - row max) / denominator the tile's partial sums have to be multiplied
 // with.  Rows past tokens*group hold zero queries and are carried along.
 __global__ __launch_bounds__(kThreads) void kvstar_rowscale_kernel(
-    float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_len,
-    unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles, unsigned row_pad)
+    float* __restrict__ ws_max, const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned M, unsigned max_blocks,
+    unsigned max_tiles, unsigned row_pad)
 {
     __shared__ float red[kThreads];
     const unsigned task = blockIdx.y, h = blockIdx.x;
-    const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
+    const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);
     if (n_blocks == 0) { return; }
     const unsigned n_tiles = (n_blocks * M + kTileSub - 1) / kTileSub;
     const unsigned rho = threadIdx.x % row_pad, grp = threadIdx.x / row_pad, ngrp = kThreads / row_pad;
-    float* tm = ws_max + (static_cast<size_t>(task) * kv_heads + h) * row_pad * max_tiles + rho;
-    const float* pp = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * max_blocks + rho;
+    float* tm = ws_max + (static_cast<size_t>(task) * kv_heads + h) * (2 * row_pad) * max_tiles + rho;   // [tile][2][row_pad]
+    constexpr unsigned kMine = 16;                       // tiles a thread keeps in registers; the rest is re-read
+    float mxs[kMine], sums[kMine];
     float mx = -INFINITY;
-    for (unsigned t = grp; t < n_tiles; t += ngrp) { mx = fmaxf(mx, tm[static_cast<size_t>(t) * row_pad]); }
+#pragma unroll
+    for (unsigned u = 0; u < kMine; ++u) {
+        const unsigned t = min(grp + u * ngrp, n_tiles - 1);   // clamped: unconditional loads, all in flight at once
+        mxs[u] = tm[static_cast<size_t>(2 * t) * row_pad];
+        sums[u] = tm[static_cast<size_t>(2 * t + 1) * row_pad];
+    }
+#pragma unroll
+    for (unsigned u = 0; u < kMine; ++u) { mx = fmaxf(mx, mxs[u]); }
+    for (unsigned t = grp + kMine * ngrp; t < n_tiles; t += ngrp) { mx = fmaxf(mx, tm[static_cast<size_t>(2 * t) * row_pad]); }
     red[threadIdx.x] = mx;
     __syncthreads();
     mx = red[rho];
     for (unsigned g = 1; g < ngrp; ++g) { mx = fmaxf(mx, red[g * row_pad + rho]); }
     __syncthreads();
     float den = 0.0f;
-    for (unsigned b = grp; b < n_blocks; b += ngrp) {
-        den += pp[static_cast<size_t>(b) * row_pad] * __expf(tm[static_cast<size_t>((b * M) / kTileSub) * row_pad] - mx);
+#pragma unroll
+    for (unsigned u = 0; u < kMine; ++u) {
+        if (grp + u * ngrp < n_tiles) { den += sums[u] * __expf(mxs[u] - mx); }
+    }
+    for (unsigned t = grp + kMine * ngrp; t < n_tiles; t += ngrp) {
+        den += tm[static_cast<size_t>(2 * t + 1) * row_pad] * __expf(tm[static_cast<size_t>(2 * t) * row_pad] - mx);
     }
     red[threadIdx.x] = den;
-    __syncthreads();   // also: every read of the tile maxima above precedes the writes below
+    __syncthreads();
     den = red[rho];
     for (unsigned g = 1; g < ngrp; ++g) { den += red[g * row_pad + rho]; }
     const float inv = den > 1e-9f ? 1.0f / den : 1.0f;   // the reference skips the division then
-    for (unsigned t = grp; t < n_tiles; t += ngrp) {
-        tm[static_cast<size_t>(t) * row_pad] = __expf(tm[static_cast<size_t>(t) * row_pad] - mx) * inv;
+#pragma unroll
+    for (unsigned u = 0; u < kMine; ++u) {
+        const unsigned t = grp + u * ngrp;
+        if (t < n_tiles) { tm[static_cast<size_t>(2 * t) * row_pad] = __expf(mxs[u] - mx) * inv; }
+    }
+    for (unsigned t = grp + kMine * ngrp; t < n_tiles; t += ngrp) {
+        tm[static_cast<size_t>(2 * t) * row_pad] = __expf(tm[static_cast<size_t>(2 * t) * row_pad] - mx) * inv;
     }
 }
 
@@ -380,21 +546,30 @@ __global__ __launch_bounds__(kThreads) void kvstar_rowscale_kernel(
 // rows of partial * factor.
 __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
     const float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, unsigned R, unsigned kv_heads, unsigned M, unsigned max_blocks,
-    unsigned max_tiles, unsigned row_pad, float* __restrict__ votes)
+    const int32_t* __restrict__ seg_len, unsigned R, unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles,
+    unsigned row_pad, float* __restrict__ votes)
 {
+    constexpr unsigned kMaxHeads = 8;
     const unsigned task = blockIdx.y;
-    const unsigned n_blocks = static_cast<unsigned>(max(seg_len[task], 0));
+    const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);
     if (blockIdx.x * 8 >= n_blocks) { return; }
-    const unsigned b = blockIdx.x * 8 + (threadIdx.x >> 5), l32 = threadIdx.x & 31;
-    const bool live = b < n_blocks;
+    const unsigned b = min(blockIdx.x * 8 + (threadIdx.x >> 5), n_blocks - 1), l32 = threadIdx.x & 31;
+    const bool live = blockIdx.x * 8 + (threadIdx.x >> 5) < n_blocks;
     const unsigned tile = (b * M) / kTileSub;
+    const size_t plane_blocks = static_cast<size_t>(max_tiles) * (kTileSub / M);
     float v = 0.0f;
-    if (live) {
-        for (unsigned h = 0; h < kv_heads; ++h) {
-            const float* wpart = ws_part + ((static_cast<size_t>(task) * kv_heads + h) * max_blocks + b) * row_pad;
-            const float* wfac = ws_max + ((static_cast<size_t>(task) * kv_heads + h) * max_tiles + tile) * row_pad;
-            for (unsigned rho = l32; rho < R; rho += 32) { v += wpart[rho] * wfac[rho]; }
+    for (unsigned r0 = 0; r0 < R; r0 += 32) {
+        const unsigned rho = min(r0 + l32, R - 1);       // clamped: every load is unconditional, the product is masked
+        float p[kMaxHeads], f[kMaxHeads];
+#pragma unroll
+        for (unsigned h = 0; h < kMaxHeads; ++h) {
+            const unsigned hh = min(h, kv_heads - 1);
+            p[h] = ws_part[((static_cast<size_t>(task) * kv_heads + hh) * plane_blocks + b) * row_pad + rho];
+            f[h] = ws_max[((static_cast<size_t>(task) * kv_heads + hh) * max_tiles + tile) * (2 * row_pad) + rho];
+        }
+        if (r0 + l32 < R) {
+#pragma unroll
+            for (unsigned h = 0; h < kMaxHeads; ++h) { if (h < kv_heads) { v += p[h] * f[h]; } }
         }
     }
 #pragma unroll
@@ -402,15 +577,17 @@ __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
     if (live && l32 == 0) { votes[seg_off[task] + b] = v; }
 }
 
-unsigned g_heads_per_group = 1;
+int g_tiles_per_wave = 0;
+
 
 }  // namespace
 
-// Tuning knob for benchmarks: kv heads one workgroup of the KVStar score kernel walks (default 1).
-extern "C" int ucm_set_kvstar_heads_per_group(int heads)
+// Tuning knob for benchmarks and tests: n > 0 takes the workspace path with n 32-sub-block tiles per wave
+// of a score workgroup, -1 the in-LDS path whenever a task's plane fits, 0 chooses automatically.
+extern "C" int ucm_set_kvstar_tiles_per_wave(int tiles)
 {
-    UCM_REQUIRE(heads >= 1 && heads <= 8, "ucm_set_kvstar_heads_per_group: %d", heads);
-    g_heads_per_group = static_cast<unsigned>(heads);
+    UCM_REQUIRE(tiles >= -1, "ucm_set_kvstar_tiles_per_wave: %d", tiles);
+    g_tiles_per_wave = tiles;
     return UCM_OK;
 }
 
@@ -462,8 +639,10 @@ extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_p
                     sub_blocks > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
     const int64_t tiles = (static_cast<int64_t>(max_blocks) * sub_blocks + kTileSub - 1) / kTileSub;
     const int64_t row_pad = rows_per_head > 32 ? 64 : 32;
-    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * std::max<int64_t>(tiles, 1);
-    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * std::max(max_blocks, 1);
+    UCM_REQUIRE(sub_blocks <= kTileSub && kTileSub % sub_blocks == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
+    // per (task, kv head): a (maximum, sum) pair per tile and row; a partial sum per block and row, blocks padded to whole tiles
+    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * 2 * std::max<int64_t>(tiles, 1);
+    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * (kTileSub / sub_blocks) * std::max<int64_t>(tiles, 1);
     return UCM_OK;
 }
 
@@ -497,35 +676,42 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     const unsigned max_tiles = static_cast<unsigned>((S + kTileSub - 1) / kTileSub);
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
     const unsigned row_pad = R > 32 ? 64 : 32;
-    // heads per workgroup (at most what fits 72 KiB of LDS: 8 at 32 rows per head, 4 at 64); one by default,
-    // ucm_set_kvstar_heads_per_group changes it
-    const unsigned per_head_lds = row_pad * kQStride * 2;
-    const unsigned heads_per_group = std::max(1u, std::min<unsigned>(std::min<unsigned>(kv_heads, g_heads_per_group),
-                                                                     (72u * 1024u) / per_head_lds));
-    const unsigned head_groups = (kv_heads + heads_per_group - 1) / heads_per_group;
-    const unsigned lds_bytes = heads_per_group * per_head_lds;
+    const unsigned q_bytes = row_pad * kQStride * 2;
+    // One workgroup per (task, kv head) with the task's [block][row_pad] plane in LDS, when there are enough
+    // such workgroups to fill the device and the plane fits; otherwise the workspace path, which may cut a
+    // task into chunks.  ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
+    const unsigned plane_offset = R > 32 ? q_bytes : 0u;
+    const size_t lds_plane = plane_offset + static_cast<size_t>(max_tiles) * (kTileSub / sub_blocks) * row_pad * 4 +
+                             2 * kWaves * row_pad * 4;
+    const bool use_lds = g_tiles_per_wave <= 0 && lds_plane <= kLdsPathMaxBytes &&
+                         (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
+    const unsigned lds_bytes = use_lds ? static_cast<unsigned>(std::max<size_t>(lds_plane, q_bytes)) : q_bytes;
     // a workgroup stages its queries once, so it should walk many tiles; the longest task is still cut into
     // enough chunks that about 2048 workgroups exist
     const unsigned tiles_per_wg_all = (max_tiles + kWaves - 1) / kWaves;
-    const unsigned want_chunks = std::max(1u, 2048u / static_cast<unsigned>(n_tasks * head_groups));
-    const unsigned tiles_per_wave = std::max(1u, (tiles_per_wg_all + want_chunks - 1) / want_chunks);
+    const unsigned want_chunks = use_lds ? 1u : std::max(1u, 2048u / static_cast<unsigned>(n_tasks * kv_heads));
+    const unsigned tiles_per_wave = g_tiles_per_wave > 0 ? static_cast<unsigned>(g_tiles_per_wave)
+                                                         : std::max(1u, (tiles_per_wg_all + want_chunks - 1) / want_chunks);
     const unsigned chunks = (max_tiles + kWaves * tiles_per_wave - 1) / (kWaves * tiles_per_wave);
     hipStream_t s = ucm::as_stream(stream);
-#define UCM_KVSTAR_ARGS dim3(chunks, head_groups, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
+#define UCM_KVSTAR_ARGS dim3(chunks, kv_heads, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), seg_off, seg_len, static_cast<unsigned>(kv_heads),                     \
         static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, ws_max, ws_part,                   \
-        static_cast<unsigned>(max_blocks),                                                                                   \
-        max_tiles, tiles_per_wave, row_pad, heads_per_group
-#define UCM_KVSTAR_LAUNCH2(M, TWO)                                                                                    \
+        static_cast<unsigned>(max_blocks), max_tiles, tiles_per_wave, row_pad, plane_offset
+#define UCM_KVSTAR_LAUNCH3(M, TWO, LDS)                                                                               \
     do {                                                                                                             \
         if (lds_bytes > 48u * 1024u) {                                                                               \
-            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_score_kernel<M, TWO>),   \
+            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_score_kernel<M, TWO, LDS>), \
                                                       hipFuncAttributeMaxDynamicSharedMemorySize,                   \
                                                       static_cast<int>(lds_bytes));                                \
             if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_votes (LDS size)"); }                      \
         }                                                                                                            \
-        hipLaunchKernelGGL((kvstar_score_kernel<M, TWO>), UCM_KVSTAR_ARGS);                                          \
+        hipLaunchKernelGGL((kvstar_score_kernel<M, TWO, LDS>), UCM_KVSTAR_ARGS);                                     \
+    } while (0)
+#define UCM_KVSTAR_LAUNCH2(M, TWO)                                                                                    \
+    do {                                                                                                             \
+        if (use_lds) { UCM_KVSTAR_LAUNCH3(M, TWO, true); } else { UCM_KVSTAR_LAUNCH3(M, TWO, false); }               \
     } while (0)
 #define UCM_KVSTAR_LAUNCH(M)                                                                                          \
     do {                                                                                                             \
@@ -541,13 +727,19 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     }
 #undef UCM_KVSTAR_LAUNCH
 #undef UCM_KVSTAR_LAUNCH2
+#undef UCM_KVSTAR_LAUNCH3
 #undef UCM_KVSTAR_ARGS
     if (hipError_t e = hipGetLastError(); e != hipSuccess) { return ucm::check_hip(e, "ucm_kvstar_votes (scores)"); }
-    hipLaunchKernelGGL(kvstar_rowscale_kernel, dim3(static_cast<unsigned>(kv_heads), n_tasks), dim3(kThreads), 0, s, ws_max,
-                       ws_part, seg_len, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
-                       static_cast<unsigned>(max_blocks), max_tiles, row_pad);
-    hipLaunchKernelGGL(kvstar_vote_kernel, dim3((max_blocks + 7) / 8, n_tasks), dim3(kThreads), 0, s, ws_max, ws_part, seg_off,
-                       seg_len, R, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
-                       static_cast<unsigned>(max_blocks), max_tiles, row_pad, votes);
+    if (use_lds) {
+        hipLaunchKernelGGL(kvstar_headsum_kernel, dim3((max_blocks + kThreads - 1) / kThreads, n_tasks), dim3(kThreads), 0, s,
+                           ws_part, seg_off, seg_len, static_cast<unsigned>(kv_heads), static_cast<unsigned>(max_blocks), votes);
+    } else {
+        hipLaunchKernelGGL(kvstar_rowscale_kernel, dim3(static_cast<unsigned>(kv_heads), n_tasks), dim3(kThreads), 0, s, ws_max,
+                           seg_len, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
+                           static_cast<unsigned>(max_blocks), max_tiles, row_pad);
+        hipLaunchKernelGGL(kvstar_vote_kernel, dim3((max_blocks + 7) / 8, n_tasks), dim3(kThreads), 0, s, ws_max, ws_part,
+                           seg_off, seg_len, R, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
+                           static_cast<unsigned>(max_blocks), max_tiles, row_pad, votes);
+    }
     UCM_LAUNCH_CHECK("ucm_kvstar_votes");
 }

@@ -387,8 +387,8 @@ def set_score_tile(tile_blocks: int) -> None:
     _lib.call("ucm_set_score_tile", tile_blocks)
 
 
-def set_kvstar_heads_per_group(heads: int) -> None:
-    _lib.call("ucm_set_kvstar_heads_per_group", heads)
+def set_kvstar_tiles_per_wave(tiles: int) -> None:
+    _lib.call("ucm_set_kvstar_tiles_per_wave", tiles)
 
 
 def set_hash_encode_groups(workgroups: int) -> None:
