@@ -371,7 +371,7 @@ def main():
                         f"representatives per layer, fp16",
             "block_repre_ms": round(krep_ms, 3),
             "us_per_step": round(kv_ms * 1e3, 1),
-            "roofline": {"kernel": "kvstar_score_kernel (+ rowscale, vote, select)", "bound": "hbm",
+            "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select)", "bound": "hbm",
                          "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": kv_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * D / (kv_ms * 1e-3) / 1e12, 1)},

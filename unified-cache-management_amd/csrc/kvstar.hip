@@ -15,9 +15,11 @@
 // queries as B, which leaves a lane with ONE query row and sixteen of a tile's
 // 32 sub-blocks in registers: the row's maximum and the per-block sums of
 // exp(score - max) are in-register work plus one exchange between the two lane
-// halves.  Every 32-sub-block tile emits its row maxima and per-block partial
-// sums (1/M of the score matrix); a second kernel rescales them to the global
-// row maximum, normalises and adds the rows up.  fp32 throughout; the summation
+// halves.  What a tile leaves behind is 1/M of the score matrix, one number per
+// (block, query row); it stays in LDS when a whole task fits there (the
+// workgroup then finishes the votes of its kv head itself) and goes through a
+// workspace in memory otherwise (two more kernels rescale to the global row
+// maximum, normalise and add the rows up).  fp32 throughout; the summation
 // order differs from the reference's scalar loop, so results agree with it to
 // rounding (a few 1e-6 relative), not bit for bit.
 #include <algorithm>
@@ -142,13 +144,6 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
 }
 
 // ---- scores -> per-tile row maxima and per-block partial sums ------------------------------------
-struct Task {
-    const unsigned short* q;     // [tokens][q_heads][d_orig] of this task
-    const int32_t* pruned;       // [kv_heads][d_pruned] or null
-    const unsigned short* table; // first representative of the task: [n_blocks][M][kv_heads][d_pad]
-    unsigned n_blocks;
-};
-
 // Hands the per-block sums of a tile's 32 exponentials for this lane's row to put(block within the tile,
 // sum) and returns their total (both lane halves included).  put is called unconditionally by all 64 lanes:
 // a store the compiler has to branch around would make it wait for ALL outstanding memory operations.
