@@ -1,5 +1,6 @@
 """Host-side logic that needs no GPU: the hook surface, the registry, request
 bookkeeping and the top-k length rule."""
+import math
 import inspect
 import types
 
@@ -211,3 +212,72 @@ def test_esa_scheduler_side_and_helpers(ucm):
     assert pool2.allocate(3) == [1, 3, 4]
     with pytest.raises(AssertionError):
         pool2.allocate(1)
+
+
+def test_kvstar_req_meta_query_offload_info(ucm):
+    """Which places of the retrieval group a prefill chunk fills (multistep.py:103-130): only the prompt's last
+    `retrieval_stride` tokens are kept, whatever the chunking."""
+    from ucm_amd.sparse.kvstar.multistep import ReqMeta, ReqStage
+
+    def meta(computed, scheduled, prompt=100, out=0, stride=8):
+        return ReqMeta("r", 0, prompt, out, scheduled, computed, 0, [], 16, [0] * prompt, 0, scheduled, stride)
+
+    assert meta(0, 50).query_offload_info is None                     # ends before token 92
+    assert meta(0, 100).query_offload_info == list(range(8))          # one chunk: all eight places
+    assert meta(50, 45).query_offload_info == [0, 1, 2]               # tokens 92..94
+    assert meta(95, 5).query_offload_info == [3, 4, 5, 6, 7]
+    assert meta(0, 93).query_offload_info == [0]
+    assert meta(97, 3, prompt=100).query_offload_info == [5, 6, 7]
+    m = meta(100, 1, out=13)
+    assert m.stage == ReqStage.DECODE and m.query_offload_info == [13 % 8] and m.step == 13
+    assert meta(0, 99).is_last_chunk is False and meta(60, 40).is_last_chunk is True
+    hashes = ReqMeta("r", 0, 40, 0, 40, 0, 0, [], 16, list(range(40))).req_block_hashes
+    assert len(hashes) == 2 and len(set(hashes)) == 2                 # full blocks only, chained
+
+
+def test_kvstar_scheduler_side(ucm):
+    """estimate_num_slots_sparsed / allocate_slots are host arithmetic (multistep.py:775-846)."""
+    from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
+    from ucm_amd.sparse.kvstar.multistep import KVStarMultiStep
+
+    ns = types.SimpleNamespace
+    cfg = make_config("KVStarMultiStep", {"sparse_ratio": 0.25})
+    cfg.cache_config.block_size = 16
+    cfg.parallel_config = ns(rank=0, tensor_parallel_size=1)
+    cfg.model_config.hf_config = ns(num_hidden_layers=2)
+    plugin = KVStarMultiStep(cfg, UcmSparseRole.SCHEDULER)
+    assert plugin.estimate_num_slots_sparsed(ns(num_output_tokens=0)) == INVALID_SLOT
+    for n_prompt, n_out in [(16 * 40 + 3, 1), (16 * 40, 7), (16 * 2 + 1, 5), (16 * 41, 16)]:
+        req = ns(num_output_tokens=n_out, num_prompt_tokens=n_prompt, num_tokens=n_prompt + n_out)
+        full = n_prompt // 16
+        fixed = min(3, full)
+        saved = math.ceil((full - fixed) * 0.25)
+        blocks = math.ceil((n_prompt + n_out) / 16) - (full - saved - fixed)
+        tail = (n_prompt + n_out) % 16
+        assert plugin.estimate_num_slots_sparsed(req) == ((blocks - 1) * 16 + tail if tail else blocks * 16)
+
+    class Pool:
+        def __init__(self):
+            self.freed, self.evicted = [], []
+
+        def _maybe_evict_cached_block(self, b):
+            self.evicted.append(b)
+
+        def free_blocks(self, bl):
+            self.freed.extend(bl)
+
+        def get_num_free_blocks(self):
+            return 1
+
+    held = list(range(100, 110))
+    mgr = ns(req_to_blocks={})
+    calls = []
+    coord = ns(get_blocks=lambda rid: [held], single_type_managers=[mgr],
+               get_num_blocks_to_allocate=lambda request_id, num_tokens, new_computed_blocks: calls.append(num_tokens) or 1,
+               allocate_new_blocks=lambda rid, n: calls.append(("alloc", n)))
+    pool = Pool()
+    got = plugin.allocate_slots(ns(request_id="A"), 16 * 3 + 2, coord, pool, [None])
+    assert mgr.req_to_blocks["A"] == held[-4:] and pool.freed == held[:-4] and pool.evicted == held
+    assert got.blocks == (held[-4:],) and calls == [50, ("alloc", 50)]
+    coord.get_num_blocks_to_allocate = lambda request_id, num_tokens, new_computed_blocks: 2
+    assert plugin.allocate_slots(ns(request_id="A"), 50, coord, Pool(), [None]) is None

@@ -31,3 +31,4 @@ _PKG = __name__.rsplit(".", 1)[0]
 UcmSparseFactory.register_sparse_method("GSA", _PKG + ".gsa.gsa", "GSA")
 UcmSparseFactory.register_sparse_method("ESA", _PKG + ".esa.esa", "ESA")
 UcmSparseFactory.register_sparse_method("KvComp", _PKG + ".kvcomp.kvcomp", "KvComp")
+UcmSparseFactory.register_sparse_method("KVStarMultiStep", _PKG + ".kvstar.multistep", "KVStarMultiStep")

@@ -1,0 +1,445 @@
+"""KVStar multi-step sparse-attention plugin: every ``retrieval_stride`` decode
+steps the queries of the last stride vote for the prompt blocks to keep; the
+winners are loaded from the KV store into the request's candidate cache blocks
+two strides later, so a retrieval never stalls a decode step.
+
+Follows the reference's ``KVStarMultiStep`` (ucm/sparse/kvstar/multistep.py:607-846)
+and ``ReqPerLayerState`` (:175-604) hook for hook and keeps its bookkeeping names
+(``standby_query_group``, ``step_group_retrieve_result``, ``task_waiter``, the
+``"prefill"`` / ``"decode<N>"`` group records):
+
+* prefill: the queries of the last ``retrieval_stride`` prompt tokens are parked
+  (``offload_prefill_query`` :388-408); at the last chunk the sub-block
+  representatives of all full prompt blocks are taken (``compute_block_repre``
+  :483-501, with channel pruning when ``blk_repre_dim_prune_ratio < 0.98``) and
+  the init / local window blocks are copied aside;
+* decode step 1: windows written back, the prefill group's retrieval runs and
+  its result is loaded into the candidate blocks (:377-387);
+* decode step s: the query joins group ``decode<1 + stride*((s-1)//stride)>``
+  (:461-481); at ``s % stride == 0`` that group's retrieval is queued (:370-374),
+  and from ``s >= 2*stride`` the result of the group before it is loaded in
+  ``attention_finished`` (:513-521), waited for at ``s % stride == 1`` (:387).
+
+What changes underneath: queries, representatives and votes stay on the device
+(``retrieve.py``: the reference's CPU thread pool is a side stream), the
+representatives come from one kernel over the paged cache, and there is no NUMA
+binding to do.  Block hashes are the chained md5 of the prompt's token blocks
+(``utils.py:22-36``), the ones the connector dumped the blocks under.
+"""
+from __future__ import annotations
+
+import enum
+import math
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Union
+
+import torch
+
+from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
+from ..esa.esa import _kv_cache_blocks, block_hash_func, get_offset
+from . import retrieve as kvstar_retrieve
+
+ReqType = Union[str, int]
+
+DEFAULTS = {
+    "init_window_sz": 1,
+    "local_window_sz": 2,
+    "sparse_ratio": 0.25,
+    "retrieval_stride": 8,
+    "blk_repre_dim_prune_ratio": 0.25,
+    "blk_repre_inner_token_merge": 2,
+}
+
+
+class ReqStage(enum.Enum):
+    PREFILL = enum.auto()
+    DECODE = enum.auto()
+
+
+@dataclass
+class ReqMeta:
+    """multistep.py:43-130."""
+    request_id: ReqType
+    index_in_batch: int
+    num_prompt_tokens: int
+    num_output_tokens: int
+    num_scheduled_tokens: int
+    num_computed_tokens: int
+    num_sparsed_tokens: int
+    vllm_block_ids: List[int]
+    token_blk_size: int
+    prompt_token_ids: List[int]
+    query_start_loc: int = -1
+    query_len: int = -1
+    retrieval_stride: int = 8
+    block_hashes: List[str] = field(default_factory=list)
+
+    def set_block_hashes(self, token_ids) -> List[str]:
+        hashes, parent = [], None
+        for start in range(0, len(token_ids), self.token_blk_size):
+            chunk = token_ids[start : start + self.token_blk_size]
+            if len(chunk) < self.token_blk_size:
+                break
+            parent = block_hash_func(parent, tuple(chunk))
+            hashes.append(str(parent))
+        return hashes
+
+    @property
+    def req_block_hashes(self) -> List[str]:
+        if not self.block_hashes:
+            self.block_hashes = self.set_block_hashes(self.prompt_token_ids)
+        return self.block_hashes
+
+    @property
+    def step(self) -> int:
+        return self.num_output_tokens
+
+    @property
+    def stage(self) -> ReqStage:
+        return ReqStage.DECODE if self.num_output_tokens > 0 else ReqStage.PREFILL
+
+    @property
+    def is_last_chunk(self) -> bool:
+        return self.num_computed_tokens + self.num_scheduled_tokens >= self.num_prompt_tokens
+
+    @property
+    def prefill_fully_blk_num(self) -> int:
+        return self.num_prompt_tokens // self.token_blk_size
+
+    @property
+    def query_offload_info(self) -> Optional[List[int]]:
+        """Places in the retrieval group of the tokens this step contributes: in prefill the chunk's share of
+        the prompt's last ``retrieval_stride`` tokens (None if it has none), in decode the step's own place."""
+        if self.stage == ReqStage.PREFILL:
+            end_pos = self.num_computed_tokens + self.num_scheduled_tokens
+            if end_pos < self.num_prompt_tokens - self.retrieval_stride:
+                return None
+            end_in_group = self.retrieval_stride - (self.num_prompt_tokens - end_pos)
+            count = min(end_in_group, self.num_scheduled_tokens)
+            return list(range(end_in_group - count, end_in_group))
+        return [self.num_output_tokens % self.retrieval_stride]
+
+
+@dataclass
+class KVStarMultiStepSparseMetaData(UcmSparseMetadata):
+    requests: List[ReqMeta] = field(default_factory=list)
+    finished_req_ids: List[ReqType] = field(default_factory=list)
+
+    def add_request(self, *args, **kwargs) -> None:
+        self.requests.append(ReqMeta(*args, **kwargs))
+
+
+class ReqPerLayerState:
+    """One request in one layer (multistep.py:175-604)."""
+
+    def __init__(self, req_meta: ReqMeta, layer_name: str, rank: int, tp_size: int, store_instance, store_name, sparse_cfg):
+        self.sparse_cfg = sparse_cfg
+        self.layer_name = layer_name
+        self.layer_id = int(layer_name.split(".")[2])
+        self.blk_repre = None                           # kvstar_retrieve.BlockRepre of the blocks between the windows
+        self.block_hashes: List[str] = []
+        self.num_tokens = 0
+        self.store_instance, self.store_name = store_instance, store_name
+        self.req_meta = req_meta
+        self.init_window = self.local_window = None
+        self.init_window_sz, self.local_window_sz = sparse_cfg["init_window_sz"], sparse_cfg["local_window_sz"]
+        self.block_size = None
+        self.k_cache = self.v_cache = None
+        self.d_pruned_index = None
+        self.local_tp_rank, self.total_tp_size = rank, tp_size
+        self.blk_trans_tasks: Dict[int, object] = {}
+        self.standby_query_group: Dict[str, list] = {}
+        self.do_retrieve_query_group: Dict[str, torch.Tensor] = {}
+        self.step_group_retrieve_result: Dict[str, List[str]] = {}
+        self.step_group_retrieve_indices: Dict[str, List[int]] = {}   # the same results as indices into blk_repre
+        self.task_waiter: Dict[str, int] = {}
+        self.num_blocks_dumped = 0
+
+    @classmethod
+    def block_hash(cls, request_id, block_id) -> str:
+        return f"req_{request_id}_blk_{block_id}"
+
+    # ---- retrieval -----------------------------------------------------------------------
+    def get_retrieve_record(self, cur_step: int) -> str:
+        return "prefill" if cur_step == 1 else "decode" + str(cur_step - self.sparse_cfg["retrieval_stride"])
+
+    def retrieval_async(self, cur_step: int, topk: int, retrieve_device: str = "cpu") -> None:
+        """Queues the vote of one query group over the request's representatives (multistep.py:240-268)."""
+        record = self.get_retrieve_record(cur_step)
+        if topk == 0:
+            self.step_group_retrieve_result[record] = []
+            self.step_group_retrieve_indices[record] = []
+            return
+        group = [x for x in self.standby_query_group[record] if x is not None]
+        self.do_retrieve_query_group[record] = torch.stack(group).to(torch.float16).contiguous()
+        self.task_waiter[record] = kvstar_retrieve.AsyncRetrieveByCPU(
+            self.do_retrieve_query_group[record], self.blk_repre, self.d_pruned_index, topk,
+            hash(self.req_meta.request_id) & 0x7FFFFFFF, kvstar_retrieve.CPU)
+
+    def extract_block_repre(self, vllm_block_ids: List[int], prune_dim_enable: bool = False):
+        """Sub-block representatives of the listed cache blocks (multistep.py:279-316)."""
+        if not vllm_block_ids or vllm_block_ids[-1] < 2:          # the reference's own guard, kept as it is (:280-281)
+            return None
+        repre, index = kvstar_retrieve.extract_block_repre(
+            self.k_cache, vllm_block_ids, self.sparse_cfg["blk_repre_inner_token_merge"],
+            prune_ratio=self.sparse_cfg["blk_repre_dim_prune_ratio"], d_pruned_index=self.d_pruned_index,
+            prune_dim_enable=prune_dim_enable)
+        self.d_pruned_index = index
+        return repre
+
+    def get_retrieve_candidate_block_ids(self) -> List[int]:
+        n_keep = math.ceil(self.blk_repre.shape[0] * self.sparse_cfg["sparse_ratio"])
+        return self.req_meta.vllm_block_ids[self.init_window_sz : n_keep + self.init_window_sz]
+
+    def get_decode_step_record(self):
+        stride = self.sparse_cfg["retrieval_stride"]
+        step = self.req_meta.step
+        return "decode" + str(((step - 1) // stride) * stride + 1), (step - 1) % stride
+
+    def save_to_standby(self, group_record: str, in_query_group_idx: int, query_relative_idx: int, tokens_to_offload) -> None:
+        if group_record not in self.standby_query_group:
+            self.standby_query_group[group_record] = [None] * self.sparse_cfg["retrieval_stride"]
+        self.standby_query_group[group_record][in_query_group_idx] = tokens_to_offload[query_relative_idx].clone()
+
+    def offload_prefill_query(self, query, query_len: int, query_start_loc: int) -> None:
+        places = self.req_meta.query_offload_info
+        if not places:
+            return
+        assert query_len >= len(places)
+        tail = query[query_start_loc + query_len - len(places) : query_start_loc + query_len]
+        for rel, place in enumerate(places):
+            self.save_to_standby("prefill", place, rel, tail)
+
+    def load_retrieve_result_async(self, load_step: int, candidate_swap_vllm_block_ids: List[int]) -> None:
+        """Collects the result of the group two strides back (the prefill group early on) and starts loading
+        the chosen blocks into the candidate cache blocks (multistep.py:410-450)."""
+        stride = self.sparse_cfg["retrieval_stride"]
+        if load_step <= stride * 2:
+            record = "prefill"
+        else:
+            record = "decode" + str((int(math.ceil(load_step / stride)) - 3) * stride + 1)
+        if self.step_group_retrieve_result.get(record) is None:
+            task_id = self.task_waiter[record]
+            kvstar_retrieve.Wait(task_id)
+            result = kvstar_retrieve.GetTaskResult(task_id)
+            del self.standby_query_group[record]
+            del self.do_retrieve_query_group[record]
+            if result["status"] != "SUCCESS":
+                raise RuntimeError(f"retrieval task {task_id} of layer {self.layer_id} failed: {result}")
+            chosen = [int(i) for i in result["data"]]
+            self.step_group_retrieve_indices[record] = chosen
+            self.step_group_retrieve_result[record] = [self.block_hashes[i + self.init_window_sz] for i in chosen]
+        hashes = self.step_group_retrieve_result[record]
+        if (record != "prefill" or load_step == 1) and len(hashes) > 0:
+            self.launch_transfer_task("load", hashes, candidate_swap_vllm_block_ids)
+
+    # ---- windows -------------------------------------------------------------------------
+    def prepare_init_and_local_window(self) -> None:
+        ids = self.req_meta.vllm_block_ids
+        self.k_cache[ids[: self.init_window_sz]] = self.init_window[0]
+        self.v_cache[ids[: self.init_window_sz]] = self.init_window[1]
+        if self.local_window is None:
+            return
+        n_local = self.local_window[0].shape[0]
+        self.k_cache[ids[-n_local:]] = self.local_window[0]
+        self.v_cache[ids[-n_local:]] = self.local_window[1]
+
+    def construct_init_and_local_window(self) -> None:
+        ids = self.req_meta.vllm_block_ids
+        head = ids[: self.init_window_sz]
+        self.init_window = (self.k_cache[head].clone(), self.v_cache[head].clone())
+        n_local = min(self.local_window_sz, len(ids[self.init_window_sz :]))
+        if n_local > 0:
+            tail = ids[-n_local:]
+            self.local_window = (self.k_cache[tail].clone(), self.v_cache[tail].clone())
+
+    def compute_block_repre(self, num_blocks_need_dump: int) -> None:
+        if self.req_meta.stage != ReqStage.PREFILL or not self.req_meta.is_last_chunk:
+            return
+        repre = self.extract_block_repre(self.req_meta.vllm_block_ids[: self.num_blocks_dumped + num_blocks_need_dump],
+                                         prune_dim_enable=True)
+        if repre is not None:
+            repre = None if repre.shape[0] <= 2 else repre[self.init_window_sz : -self.local_window_sz]
+        self.blk_repre = repre
+        self.construct_init_and_local_window()
+
+    # ---- hooks ---------------------------------------------------------------------------
+    def attention_begin(self, query, key, value, forward_context) -> None:
+        meta = self.req_meta
+        if meta.stage == ReqStage.PREFILL:
+            self.offload_prefill_query(query, meta.query_len, meta.query_start_loc)
+            return
+        if self.blk_repre is None:
+            return
+        assert meta.query_len == 1, "KVStar series sparse attention doesn't support spec_decode now"
+        stride = self.sparse_cfg["retrieval_stride"]
+        group_record, place = self.get_decode_step_record()
+        self.save_to_standby(group_record, place, meta.query_start_loc, query)
+        if meta.step % stride == 0:
+            self.retrieval_async(meta.step + 1, len(self.get_retrieve_candidate_block_ids()))
+        if meta.step == 1:
+            self.prepare_init_and_local_window()
+            candidates = self.get_retrieve_candidate_block_ids()
+            self.wait_for_blk_transfer_task_done()
+            self.retrieval_async(meta.step, len(candidates))
+            self.load_retrieve_result_async(meta.step, candidates)
+        if meta.step % stride == 1:
+            self.wait_for_blk_transfer_task_done()
+
+    def attention_finished(self, query, key, value, attn_output, forward_context) -> None:
+        meta = self.req_meta
+        if meta.stage != ReqStage.PREFILL:
+            stride = self.sparse_cfg["retrieval_stride"]
+            if self.blk_repre is not None and meta.step >= stride * 2 and meta.step % stride == 0:
+                self.load_retrieve_result_async(meta.step + 1, self.get_retrieve_candidate_block_ids())
+            return
+        self.maybe_register_kv_cache(forward_context)
+        updated = meta.num_computed_tokens + meta.num_scheduled_tokens
+        need_dump = updated // self.block_size - self.num_blocks_dumped
+        self.num_tokens = updated
+        self.compute_block_repre(need_dump)
+
+    def maybe_register_kv_cache(self, forward_context) -> None:
+        if self.block_size:
+            return
+        attn = forward_context.no_compile_layers[self.layer_name]
+        kv_cache = attn.kv_cache[forward_context.virtual_engine]
+        self.k_cache, self.v_cache = kv_cache[0], kv_cache[1]
+        self.block_size = self.k_cache.shape[1]
+        self.num_key_heads, self.head_size = self.k_cache.shape[2], self.k_cache.shape[3]
+        self.block_hashes = self.req_meta.req_block_hashes
+
+    def update_meta(self, req_meta: ReqMeta, forward_context=None) -> None:
+        self.req_meta = req_meta
+
+    # ---- transfers -----------------------------------------------------------------------
+    def launch_transfer_task(self, transfer_type: str, block_hashes: List[str], vllm_block_ids: List[int]) -> None:
+        n = min(len(block_hashes), len(vllm_block_ids))
+        if n == 0:
+            return
+        block_hashes, vllm_block_ids = list(block_hashes[:n]), list(vllm_block_ids[:n])
+        fn = getattr(self.store_instance, transfer_type)
+        shape = (self.block_size, self.num_key_heads, self.head_size)
+        precision = self.k_cache.element_size()
+        off_k = [get_offset(shape, self.local_tp_rank, self.total_tp_size, precision, self.layer_id, False)] * n
+        off_v = [get_offset(shape, self.local_tp_rank, self.total_tp_size, precision, self.layer_id, True)] * n
+        self.blk_trans_tasks[hash((tuple(block_hashes), transfer_type, "key"))] = fn(
+            block_hashes, off_k, [self.k_cache[i] for i in vllm_block_ids])
+        self.blk_trans_tasks[hash((tuple(block_hashes), transfer_type, "value"))] = fn(
+            block_hashes, off_v, [self.v_cache[i] for i in vllm_block_ids])
+
+    def wait_for_blk_transfer_task_done(self) -> None:
+        for task in self.blk_trans_tasks.values():
+            self.store_instance.wait(task)
+        self.blk_trans_tasks.clear()
+
+
+class KVStarMultiStep(UcmSparseBase):
+    """Plugin object (multistep.py:607-846).  ``store``: anything with the ``UcmKVStoreBase`` load / wait
+    methods; under vLLM it is the connector of the KV transfer group."""
+
+    def __init__(self, vllm_config, role: UcmSparseRole, store=None):
+        super().__init__(vllm_config=vllm_config, role=role)
+        self.req_states: Dict[ReqType, List[Optional[ReqPerLayerState]]] = {}
+        self.local_tp_rank = vllm_config.parallel_config.rank
+        self.total_tp_size = vllm_config.parallel_config.tensor_parallel_size
+        hf_config = getattr(vllm_config.model_config, "hf_config", None)
+        self.total_num_hidden_layers = (hf_config.num_hidden_layers if hf_config is not None
+                                        else vllm_config.model_config.get_num_layers(vllm_config.parallel_config))
+        extra = vllm_config.kv_transfer_config.kv_connector_extra_config
+        self.kvstar_multistep_cfg = dict(DEFAULTS)
+        self.kvstar_multistep_cfg.update(extra["ucm_sparse_config"].get("KVStarMultiStep") or {})
+        self.connector_name = extra.get("ucm_connector_name")
+        self.connector = store
+        self.token_blk_size = vllm_config.cache_config.block_size
+        if role == UcmSparseRole.WORKER:
+            kvstar_retrieve.Setup(kvstar_retrieve.SetupParam(
+                cpuNumaIds=[], physicalCorePerNuma=0, allocRatio=0.75, blkRepreSize=4096, deviceType=kvstar_retrieve.CPU,
+                totalTpSize=self.total_tp_size, localRankId=self.local_tp_rank))
+            if self.connector is None:
+                try:  # under vLLM: the connector of the KV transfer group, as the reference takes it (:637-642)
+                    from vllm.distributed.kv_transfer import get_kv_transfer_group  # type: ignore
+
+                    self.connector = get_kv_transfer_group().connector
+                except Exception:
+                    self.connector = None
+
+    def create_layerwise_req_state(self, req_meta: ReqMeta, layer_name: str) -> ReqPerLayerState:
+        layer_id = int(layer_name.split(".")[2])
+        states = self.req_states.setdefault(req_meta.request_id, [None] * self.total_num_hidden_layers)
+        if states[layer_id] is None:
+            states[layer_id] = ReqPerLayerState(req_meta, layer_name, self.local_tp_rank, self.total_tp_size, self.connector,
+                                                self.connector_name, self.kvstar_multistep_cfg)
+        return states[layer_id]
+
+    def request_begin(self, request_id: ReqType, prompt_token_ids: List[int]) -> None:
+        pass
+
+    # ---- worker side ---------------------------------------------------------------------
+    def request_finished_in_worker(self, request_id: ReqType) -> None:
+        self.req_states.pop(request_id, None)
+
+    def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        for req_meta in self._sparse_metadata.requests:
+            state = self.create_layerwise_req_state(req_meta, layer_name)
+            state.update_meta(req_meta, forward_context)
+            state.attention_begin(query, key, value, forward_context)
+
+    def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
+        for req_meta in self._sparse_metadata.requests:
+            state = self.create_layerwise_req_state(req_meta, layer_name)
+            state.update_meta(req_meta, forward_context)
+            state.attention_finished(query, key, value, attn_output, forward_context)
+
+    def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata=None) -> None:
+        meta = KVStarMultiStepSparseMetaData()
+        if isinstance(attn_metadata, dict):
+            attn_metadata = next(iter(attn_metadata.values()))
+        starts = attn_metadata.query_start_loc
+        for req_id, n_sched in scheduler_output.num_scheduled_tokens.items():
+            req = requests[req_id]
+            if len(req.prompt_token_ids) <= self.token_blk_size:
+                continue
+            row = input_batch.req_id_to_index[req_id]
+            q_start = int(starts[row])
+            meta.add_request(req_id, row, len(req.prompt_token_ids), len(req.output_token_ids), n_sched,
+                             req.num_computed_tokens, scheduler_output.req_sparsed_slots[req_id], req.block_ids[0],
+                             self.token_blk_size, req.prompt_token_ids, q_start, int(starts[row + 1]) - q_start,
+                             self.kvstar_multistep_cfg["retrieval_stride"])
+        self._sparse_metadata = meta
+
+    # ---- scheduler side ------------------------------------------------------------------
+    def estimate_num_slots_sparsed(self, request) -> int:
+        """Token slots of a decoding request: the windows, sparse_ratio of the prompt blocks between them,
+        and everything generated since (multistep.py:775-814)."""
+        if request.num_output_tokens == 0:
+            return INVALID_SLOT
+        bs = self.token_blk_size
+        cfg = self.kvstar_multistep_cfg
+        n_prefill = request.num_prompt_tokens // bs
+        n_fixed = min(cfg["init_window_sz"] + cfg["local_window_sz"], n_prefill)
+        n_saved = math.ceil((n_prefill - n_fixed) * cfg["sparse_ratio"])
+        n_dense = math.ceil(request.num_tokens / bs)
+        budget = n_dense - (n_prefill - n_saved - n_fixed)
+        tail = request.num_tokens % bs
+        return (budget - 1) * bs + tail if tail else budget * bs
+
+    def allocate_slots(self, request, num_slots_sparsed, coordinator, block_pool, kv_cache_groups):
+        """Keeps the last ceil(slots/block_size) blocks of the request, returns the others to the pool and
+        allocates for the sparsified length (multistep.py:816-846)."""
+        need = math.ceil(num_slots_sparsed / self.token_blk_size)
+        blocks = coordinator.get_blocks(request.request_id)[0]
+        first_kept = len(blocks) - need
+        kept, returned = [], []
+        for i, block in enumerate(blocks):
+            (kept if i >= first_kept else returned).append(block)
+            block_pool._maybe_evict_cached_block(block)
+        block_pool.free_blocks(returned)
+        coordinator.single_type_managers[0].req_to_blocks[request.request_id] = kept
+        empty = tuple([] for _ in range(len(kv_cache_groups)))
+        n_new = coordinator.get_num_blocks_to_allocate(request_id=request.request_id, num_tokens=num_slots_sparsed,
+                                                       new_computed_blocks=empty)
+        if n_new > block_pool.get_num_free_blocks():
+            return None
+        coordinator.allocate_new_blocks(request.request_id, num_slots_sparsed)
+        return _kv_cache_blocks(kept)
