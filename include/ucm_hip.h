@@ -301,7 +301,7 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
  *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev fp32, task t's votes at votes[seg_off[t] + b].
  * n_tokens * (q_heads/kv_heads) <= 64, kv_heads <= 8, d_pad a multiple of 16
- * and <= 128, sub_blocks in {1, 2, 4, 8, 16, 32}.
+ * and <= 128, sub_blocks a power of two up to 128.
  */
 int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
                            const int32_t* block_ids, const int32_t* slots, int n, int block_size,
@@ -311,7 +311,7 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
 /* Tuning knob for benchmarks and tests.  ucm_kvstar_votes has two paths: one
  * workgroup per (task, kv head) that keeps the task's per-(block, query row)
  * sums in LDS and stores only the head's share of the votes (taken when there
- * are at least 1024 such pairs and the plane fits 159 KiB), and a workspace
+ * are at least 128 such pairs and the plane fits 159 KiB), and a workspace
  * path that may cut a task into chunks.  tiles > 0: the workspace path with
  * that many 32-sub-block tiles per wave (four waves per workgroup); -1: the
  * in-LDS path whenever the plane fits; 0: automatic.  Not part of the

@@ -37,7 +37,8 @@ def check_selection(got_idx, want_final, k):
             assert i in got_idx, (i, want_final[i], kth)
 
 
-@pytest.mark.parametrize("merge,hkv,d,bs", [(16, 8, 128, 128), (32, 2, 64, 128), (4, 4, 128, 16), (128, 1, 128, 128), (16, 2, 128, 32)])
+@pytest.mark.parametrize("merge,hkv,d,bs", [(16, 8, 128, 128), (32, 2, 64, 128), (4, 4, 128, 16), (128, 1, 128, 128), (16, 2, 128, 32),
+                                            (2, 8, 128, 128), (1, 2, 64, 128)])   # the last two: 64 and 128 sub-blocks per block
 def test_kvstar_block_repre(ucm, dev, merge, hkv, d, bs):
     from ucm_amd import ops
 
@@ -87,7 +88,7 @@ def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None
 
 
 @pytest.mark.parametrize("x,hq,hkv,d,M", [(8, 32, 8, 128, 8), (8, 16, 2, 64, 4), (3, 8, 8, 128, 1), (1, 4, 1, 128, 32),
-                                          (5, 24, 4, 96, 2), (8, 64, 8, 128, 16)])
+                                          (5, 24, 4, 96, 2), (8, 64, 8, 128, 16), (8, 32, 8, 128, 64), (4, 8, 2, 64, 128)])
 def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
     from ucm_amd import ops
 
@@ -118,7 +119,7 @@ def test_kvstar_many_short_tasks_take_the_in_lds_path(ucm, dev):
     from ucm_amd import ops
 
     x, hq, hkv, d, M = 8, 32, 8, 128, 8
-    lens = [int(v) for v in synth.permutation(1150, 150) % 41]     # 0..40 blocks, 150 tasks -> 1200 pairs
+    lens = [int(v) for v in synth.permutation(1150, 150) % 41]     # 0..40 blocks, 150 tasks -> 1200 (task, kv head) pairs
     rows = int(np.sum(lens))
     repre = f16_bits(synth.normal_f32(1151, (rows, M, hkv, d)) * np.float32(0.25))
     qs = [f16_bits(synth.normal_f32(1152 + t, (x, hq, d)) * np.float32(0.25)) for t in range(len(lens))]

@@ -39,7 +39,7 @@ constexpr int kMaxRows = 64;          // tokens * group size per kv head
 constexpr int kMaxDim = 128;
 constexpr int kQStride = kMaxDim + 8; // fp16 elements per staged query row (272 B: spreads LDS banks)
 constexpr int kTileSub = 32;          // sub-blocks per MFMA tile
-constexpr int64_t kLdsPathMinGroups = 1024;           // (task, kv head) pairs from which the in-LDS path is taken
+constexpr int64_t kLdsPathMinGroups = 128;            // (task, kv head) pairs from which the in-LDS path is taken
 constexpr size_t kLdsPathMaxBytes = 159 * 1024;       // of the 160 KiB a compute unit has
 
 __device__ __forceinline__ unsigned short f32_to_f16_bits(float f)
@@ -58,8 +58,9 @@ __device__ __forceinline__ unsigned short f32_to_f16_bits(float f)
 // grid: x = listed block, y = layer.  Phase 1: a thread owns 8 adjacent columns of a token row
 // (one 16-byte load per token, `merge` tokens accumulated in token order in fp32), the means -
 // rounded to bf16 and then fp16, what mean() in the model dtype followed by .to(float16) gives -
-// are parked in LDS as [M][kv_heads*head_dim].  Phase 2 gathers the kept channels from LDS and
-// writes the block's pieces, consecutive threads to consecutive 16 bytes.
+// are parked in LDS as [sub-block][kv_heads*head_dim] (as many sub-blocks at a time as fit 64 KiB).
+// Phase 2 gathers the kept channels from LDS and writes the pieces, consecutive threads to consecutive
+// 16 bytes.
 constexpr int kRepreUnroll = 16;
 
 __device__ __forceinline__ unsigned mean_to_f16x2(float lo, float hi, float inv)
@@ -83,9 +84,9 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
     unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
-    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride)
+    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [M][row]
+    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row]
     const unsigned M = block_size / merge;
     const unsigned id = static_cast<unsigned>(block_ids[blockIdx.x]);
     const unsigned slot = static_cast<unsigned>(slots[blockIdx.x]);
@@ -94,56 +95,60 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const unsigned short* blk = static_cast<const unsigned short*>(k_layers[blockIdx.y]) +
                                 static_cast<size_t>(id) * block_size * row;
     const float inv = 1.0f / static_cast<float>(merge);
-    for (unsigned w = threadIdx.x; w < M * ncg; w += kThreads) {
-        const unsigned m = w / ncg, cg = w - m * ncg;
-        const unsigned short* src = blk + static_cast<size_t>(m) * merge * row + cg * 8;
-        float acc[8];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
-        unsigned t = 0;
-        for (; t + kRepreUnroll <= merge; t += kRepreUnroll) {
-            u32x4 v[kRepreUnroll];
-#pragma unroll
-            for (int u = 0; u < kRepreUnroll; ++u) { v[u] = ucm::gload16_nt(src + static_cast<size_t>(t + u) * row); }
-#pragma unroll
-            for (int u = 0; u < kRepreUnroll; ++u) { add_bf16x8(acc, v[u]); }
-        }
-        for (; t < merge; ++t) { add_bf16x8(acc, ucm::gload16_nt(src + static_cast<size_t>(t) * row)); }
-        u32x4 o;
-        o.x = mean_to_f16x2(acc[0], acc[1], inv);
-        o.y = mean_to_f16x2(acc[2], acc[3], inv);
-        o.z = mean_to_f16x2(acc[4], acc[5], inv);
-        o.w = mean_to_f16x2(acc[6], acc[7], inv);
-        *reinterpret_cast<u32x4*>(&stage[m * row + cg * 8]) = o;
-    }
-    __syncthreads();
     const unsigned pieces = d_pad / 8;
     unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<size_t>(slot) * M * d_pad;
-    for (unsigned e = threadIdx.x; e < kv_heads * pieces * M; e += kThreads) {
-        const unsigned h = e / (pieces * M), rem = e - h * (pieces * M);
-        const unsigned piece = rem / M, m = rem - piece * M;
-        const unsigned short* srow = stage + m * row + h * head_dim;
-        unsigned short c[8];
+    for (unsigned m0 = 0; m0 < M; m0 += m_chunk) {       // m_chunk sub-blocks at a time: what fits LDS
+        const unsigned mc = min(m_chunk, M - m0);
+        for (unsigned w = threadIdx.x; w < mc * ncg; w += kThreads) {
+            const unsigned ml = w / ncg, cg = w - ml * ncg;
+            const unsigned short* src = blk + static_cast<size_t>(m0 + ml) * merge * row + cg * 8;
+            float acc[8];
 #pragma unroll
-        for (unsigned j = 0; j < 8; ++j) {
-            const unsigned p = piece * 8 + j;
-            unsigned short v = 0;
-            if (p < d_pruned) {
-                const unsigned d = pruned ? static_cast<unsigned>(pruned[h * d_pruned + p]) : p;
-                if (d < head_dim) { v = srow[d]; }
+            for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
+            unsigned t = 0;
+            for (; t + kRepreUnroll <= merge; t += kRepreUnroll) {
+                u32x4 v[kRepreUnroll];
+#pragma unroll
+                for (int u = 0; u < kRepreUnroll; ++u) { v[u] = ucm::gload16_nt(src + static_cast<size_t>(t + u) * row); }
+#pragma unroll
+                for (int u = 0; u < kRepreUnroll; ++u) { add_bf16x8(acc, v[u]); }
             }
-            c[j] = v;
+            for (; t < merge; ++t) { add_bf16x8(acc, ucm::gload16_nt(src + static_cast<size_t>(t) * row)); }
+            u32x4 o;
+            o.x = mean_to_f16x2(acc[0], acc[1], inv);
+            o.y = mean_to_f16x2(acc[2], acc[3], inv);
+            o.z = mean_to_f16x2(acc[4], acc[5], inv);
+            o.w = mean_to_f16x2(acc[6], acc[7], inv);
+            *reinterpret_cast<u32x4*>(&stage[ml * row + cg * 8]) = o;
         }
-        u32x4 o;
-        o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
-        o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
-        o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
-        o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
-        ucm::gstore16(out + static_cast<int64_t>(h) * head_stride + static_cast<size_t>(rem) * 8, o);
+        __syncthreads();
+        for (unsigned e = threadIdx.x; e < kv_heads * pieces * mc; e += kThreads) {
+            const unsigned h = e / (pieces * mc), rem = e - h * (pieces * mc);
+            const unsigned piece = rem / mc, ml = rem - piece * mc;
+            const unsigned short* srow = stage + ml * row + h * head_dim;
+            unsigned short c[8];
+#pragma unroll
+            for (unsigned j = 0; j < 8; ++j) {
+                const unsigned p = piece * 8 + j;
+                unsigned short v = 0;
+                if (p < d_pruned) {
+                    const unsigned d = pruned ? static_cast<unsigned>(pruned[h * d_pruned + p]) : p;
+                    if (d < head_dim) { v = srow[d]; }
+                }
+                c[j] = v;
+            }
+            u32x4 o;
+            o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
+            o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
+            o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
+            o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
+            ucm::gstore16(out + static_cast<int64_t>(h) * head_stride + (static_cast<size_t>(piece) * M + m0 + ml) * 8, o);
+        }
+        __syncthreads();                                 // the next chunk overwrites the staged means
     }
 }
 
-// ---- scores -> per-tile row maxima and per-block partial sums ------------------------------------
+// kM here: sub-blocks per part (a block, or a tile's share of a bigger block; at most 32).
 // Hands the per-block sums of a tile's 32 exponentials for this lane's row to put(block within the tile,
 // sum) and returns their total (both lane halves included).  put is called unconditionally by all 64 lanes:
 // a store the compiler has to branch around would make it wait for ALL outstanding memory operations.
@@ -243,6 +248,10 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes piece 2*ks + half
     constexpr int kRowTiles = kTwoRowTiles ? 2 : 1;      // 33..64 query rows per kv head take two
     constexpr unsigned kStride = kWaves * kTileSub;      // from one tile of a wave to its next
+    // Sums are kept per "part": a block, or - when a block has more sub-blocks than a tile - the block's share
+    // of one tile; kParts parts make a block
+    constexpr int kPartSub = kM < kTileSub ? kM : kTileSub;
+    constexpr unsigned kParts = kM / kPartSub;
     const unsigned short* tbase = table + static_cast<int64_t>(h) * head_stride +
                                   static_cast<size_t>(seg_off[task]) * kM * d_pad + half * (8 * kM);
 
@@ -312,7 +321,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     if constexpr (kLds) { __syncthreads(); }             // every wave has its query fragments: the plane may overwrite them
 
     float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h) * (2 * row_pad) * max_tiles;          // [tile][2][row_pad]
-    float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * (kTileSub / kM) * max_tiles;  // [block][row_pad]
+    float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * (kTileSub / kPartSub) * max_tiles;  // [part][row_pad]
 
     float m_run[kRowTiles], d_run[kRowTiles];            // kLds only
 #pragma unroll
@@ -359,10 +368,10 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 #pragma unroll
             for (int i = 0; i < 16; ++i) { e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], kLog2e, nmx)); }
             // rows past R hold zero queries: they are computed like the rest and never read
-            const unsigned blk0 = tile * (kTileSub / kM);
+            const unsigned blk0 = tile * (kTileSub / kPartSub);   // first part of the tile
             if constexpr (kLds) {
                 const float mx2 = mx * kLog2e;
-                const float total = block_sums<kM>(e, half, [&](unsigned b, float v) {
+                const float total = block_sums<kPartSub>(e, half, [&](unsigned b, float v) {
                     plane[(blk0 + b) * row_pad + rho] = mx2 + __builtin_amdgcn_logf(v);   // log2 of the block's sum of 2^(score*log2e)
                 });
                 // the wave's running (maximum, sum of 2^(x - maximum)) of the row, in the same log2 units
@@ -370,7 +379,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
                 d_run[rt] = d_run[rt] * __builtin_amdgcn_exp2f(m_run[rt] - m_new) + total * __builtin_amdgcn_exp2f(mx2 - m_new);
                 m_run[rt] = m_new;
             } else {
-                const float total = block_sums<kM>(e, half, [&](unsigned b, float v) {
+                const float total = block_sums<kPartSub>(e, half, [&](unsigned b, float v) {
                     wpart[static_cast<size_t>(blk0 + b) * row_pad + rho] = v;
                 });
                 wmax[(static_cast<size_t>(tile) * 2 + half) * row_pad + rho] = half ? total : mx;
@@ -382,6 +391,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     // (16) and the stores of the tiles worked on since - none for the wave's first tile, one tile's for its
     // second, two tiles' from then on.
     constexpr unsigned kStores = kLds ? 0 : kRowTiles * (1 + (kM >= 16 ? 1 : kM == 8 ? 2 : kM == 4 ? 4 : kM == 2 ? 8 : 16));
+    static_assert(kM == 1 || kM == 2 || kM == 4 || kM == 8 || kM == 16 || kM == 32 || kM == 64 || kM == 128, "sub-blocks per block");
     constexpr unsigned kAfter0 = 16, kAfter1 = 16 + kStores > 63 ? 63 : 16 + kStores,
                        kAfter2 = 16 + 2 * kStores > 63 ? 63 : 16 + 2 * kStores;
 #define UCM_KEYS_LANDED(k, n)                                                                                              \
@@ -424,7 +434,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 
     if constexpr (kLds) {
         // ---- this head's share of the votes, from the plane in LDS
-        float* red = plane + static_cast<size_t>(max_tiles) * (kTileSub / kM) * row_pad;   // [wave][2][row_pad]
+        float* red = plane + static_cast<size_t>(max_tiles) * (kTileSub / kPartSub) * row_pad;   // [wave][2][row_pad]
         if (half == 0) {
 #pragma unroll
             for (int rt = 0; rt < kRowTiles; ++rt) {
@@ -456,9 +466,11 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
         float* vh = ws_part + (static_cast<size_t>(task) * kv_heads + h) * max_blocks;
         for (unsigned b = threadIdx.x; b < n_blocks; b += kThreads) {
             float v = 0.0f;
-            for (unsigned r = 0; r < row_pad; ++r) {
-                const unsigned rr = (r + b) & (row_pad - 1);
-                v += __builtin_amdgcn_exp2f(plane[b * row_pad + rr] - red[rr]) * red[row_pad + rr];
+            for (unsigned part = b * kParts; part < (b + 1) * kParts; ++part) {
+                for (unsigned r = 0; r < row_pad; ++r) {
+                    const unsigned rr = (r + b) & (row_pad - 1);
+                    v += __builtin_amdgcn_exp2f(plane[part * row_pad + rr] - red[rr]) * red[row_pad + rr];
+                }
             }
             vh[b] = v;
         }
@@ -550,21 +562,24 @@ __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
     if (blockIdx.x * 8 >= n_blocks) { return; }
     const unsigned b = min(blockIdx.x * 8 + (threadIdx.x >> 5), n_blocks - 1), l32 = threadIdx.x & 31;
     const bool live = blockIdx.x * 8 + (threadIdx.x >> 5) < n_blocks;
-    const unsigned tile = (b * M) / kTileSub;
-    const size_t plane_blocks = static_cast<size_t>(max_tiles) * (kTileSub / M);
+    const unsigned part_sub = min(M, static_cast<unsigned>(kTileSub)), parts = M / part_sub;   // see kvstar_score_kernel
+    const size_t plane_parts = static_cast<size_t>(max_tiles) * (kTileSub / part_sub);
     float v = 0.0f;
-    for (unsigned r0 = 0; r0 < R; r0 += 32) {
-        const unsigned rho = min(r0 + l32, R - 1);       // clamped: every load is unconditional, the product is masked
-        float p[kMaxHeads], f[kMaxHeads];
+    for (unsigned part = b * parts; part < (b + 1) * parts; ++part) {
+        const unsigned tile = (part * part_sub) / kTileSub;
+        for (unsigned r0 = 0; r0 < R; r0 += 32) {
+            const unsigned rho = min(r0 + l32, R - 1);   // clamped: every load is unconditional, the product is masked
+            float p[kMaxHeads], f[kMaxHeads];
 #pragma unroll
-        for (unsigned h = 0; h < kMaxHeads; ++h) {
-            const unsigned hh = min(h, kv_heads - 1);
-            p[h] = ws_part[((static_cast<size_t>(task) * kv_heads + hh) * plane_blocks + b) * row_pad + rho];
-            f[h] = ws_max[((static_cast<size_t>(task) * kv_heads + hh) * max_tiles + tile) * (2 * row_pad) + rho];
-        }
-        if (r0 + l32 < R) {
+            for (unsigned h = 0; h < kMaxHeads; ++h) {
+                const unsigned hh = min(h, kv_heads - 1);
+                p[h] = ws_part[((static_cast<size_t>(task) * kv_heads + hh) * plane_parts + part) * row_pad + rho];
+                f[h] = ws_max[((static_cast<size_t>(task) * kv_heads + hh) * max_tiles + tile) * (2 * row_pad) + rho];
+            }
+            if (r0 + l32 < R) {
 #pragma unroll
-            for (unsigned h = 0; h < kMaxHeads; ++h) { if (h < kv_heads) { v += p[h] * f[h]; } }
+                for (unsigned h = 0; h < kMaxHeads; ++h) { if (h < kv_heads) { v += p[h] * f[h]; } }
+            }
         }
     }
 #pragma unroll
@@ -609,8 +624,9 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
     UCM_SUPPORTED(row % 8 == 0 && d_pad % 8 == 0, "ucm_kvstar_block_repre: kv_heads*head_dim=%u and d_pad=%d must be multiples of 8",
                   row, d_pad);
-    const size_t lds_bytes = static_cast<size_t>(M) * row * 2;
-    UCM_SUPPORTED(lds_bytes <= 64u * 1024u, "ucm_kvstar_block_repre: %d sub-blocks of %u channels exceed 64 KiB of LDS", M, row);
+    UCM_SUPPORTED(row <= 32768u, "ucm_kvstar_block_repre: kv_heads*head_dim=%u (at most 32768)", row);
+    const unsigned m_chunk = std::min<unsigned>(static_cast<unsigned>(M), 32768u / row);   // sub-blocks staged at a time: 64 KiB of LDS
+    const size_t lds_bytes = static_cast<size_t>(m_chunk) * row * 2;
     UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_layer_stride % 8 == 0 && repre_head_stride % 8 == 0,
                 "ucm_kvstar_block_repre: table not 16-byte aligned");
     if (lds_bytes > 48u * 1024u) {
@@ -623,7 +639,7 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                        static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),
                        static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), static_cast<unsigned>(merge),
                        pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),
-                       static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride);
+                       static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk);
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
 }
 
@@ -634,10 +650,12 @@ extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_p
                     sub_blocks > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
     const int64_t tiles = (static_cast<int64_t>(max_blocks) * sub_blocks + kTileSub - 1) / kTileSub;
     const int64_t row_pad = rows_per_head > 32 ? 64 : 32;
-    UCM_REQUIRE(sub_blocks <= kTileSub && kTileSub % sub_blocks == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
-    // per (task, kv head): a (maximum, sum) pair per tile and row; a partial sum per block and row, blocks padded to whole tiles
+    UCM_REQUIRE(sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
+    // per (task, kv head): a (maximum, sum) pair per tile and row; a partial sum per row and block (per tile,
+    // for blocks of more than 32 sub-blocks), padded to whole tiles
+    const int64_t parts_per_tile = kTileSub / std::min(sub_blocks, kTileSub);
     *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * 2 * std::max<int64_t>(tiles, 1);
-    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * (kTileSub / sub_blocks) * std::max<int64_t>(tiles, 1);
+    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * parts_per_tile * std::max<int64_t>(tiles, 1);
     return UCM_OK;
 }
 
@@ -663,8 +681,8 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     UCM_REQUIRE(d_pruned > 0 && d_pruned <= d_pad && d_pruned <= d_orig, "ucm_kvstar_votes: d_pruned=%d", d_pruned);
     UCM_REQUIRE(pruned_sel == nullptr || pruned != nullptr, "ucm_kvstar_votes: pruned_sel without pruned");
     UCM_REQUIRE(pruned_sel != nullptr || d_pruned == d_orig, "ucm_kvstar_votes: d_pruned < d_orig needs the channel lists");
-    UCM_SUPPORTED(sub_blocks == 1 || sub_blocks == 2 || sub_blocks == 4 || sub_blocks == 8 || sub_blocks == 16 ||
-                      sub_blocks == 32, "ucm_kvstar_votes: sub_blocks=%d (1, 2, 4, 8, 16 or 32)", sub_blocks);
+    UCM_SUPPORTED(sub_blocks >= 1 && sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0,
+                  "ucm_kvstar_votes: sub_blocks=%d (a power of two up to 128)", sub_blocks);
     UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0,
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
     const int64_t S = static_cast<int64_t>(max_blocks) * sub_blocks;
@@ -676,7 +694,7 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     // such workgroups to fill the device and the plane fits; otherwise the workspace path, which may cut a
     // task into chunks.  ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
     const unsigned plane_offset = R > 32 ? q_bytes : 0u;
-    const size_t lds_plane = plane_offset + static_cast<size_t>(max_tiles) * (kTileSub / sub_blocks) * row_pad * 4 +
+    const size_t lds_plane = plane_offset + static_cast<size_t>(max_tiles) * (kTileSub / std::min(sub_blocks, kTileSub)) * row_pad * 4 +
                              2 * kWaves * row_pad * 4;
     const bool use_lds = g_tiles_per_wave <= 0 && lds_plane <= kLdsPathMaxBytes &&
                          (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
@@ -718,7 +736,9 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     case 4: UCM_KVSTAR_LAUNCH(4); break;
     case 8: UCM_KVSTAR_LAUNCH(8); break;
     case 16: UCM_KVSTAR_LAUNCH(16); break;
-    default: UCM_KVSTAR_LAUNCH(32); break;
+    case 32: UCM_KVSTAR_LAUNCH(32); break;
+    case 64: UCM_KVSTAR_LAUNCH(64); break;
+    default: UCM_KVSTAR_LAUNCH(128); break;
     }
 #undef UCM_KVSTAR_LAUNCH
 #undef UCM_KVSTAR_LAUNCH2
