@@ -88,7 +88,8 @@ def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None
 
 
 @pytest.mark.parametrize("x,hq,hkv,d,M", [(8, 32, 8, 128, 8), (8, 16, 2, 64, 4), (3, 8, 8, 128, 1), (1, 4, 1, 128, 32),
-                                          (5, 24, 4, 96, 2), (8, 64, 8, 128, 16), (8, 32, 8, 128, 64), (4, 8, 2, 64, 128)])
+                                          (5, 24, 4, 96, 2), (8, 64, 8, 128, 16), (8, 32, 8, 128, 64), (4, 8, 2, 64, 128),
+                                          (8, 32, 8, 32, 64), (4, 16, 4, 32, 2), (4, 64, 4, 32, 8), (2, 8, 8, 48, 16)])
 def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
     from ucm_amd import ops
 
@@ -131,24 +132,25 @@ def test_kvstar_many_short_tasks_take_the_in_lds_path(ucm, dev):
         assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
 
 
+@pytest.mark.parametrize("M,dp", [(8, 77), (64, 32)])          # 77 kept channels: table rows padded to 80; 64 / 32: the reference's defaults
 @pytest.mark.parametrize("tiles_per_wave", [0, -1])
-def test_kvstar_pruned_channels_and_selection(ucm, dev, tiles_per_wave):
+def test_kvstar_pruned_channels_and_selection(ucm, dev, tiles_per_wave, M, dp):
     from ucm_amd import ops
 
     ops.set_kvstar_tiles_per_wave(tiles_per_wave)
     try:
-        _pruned_channels_and_selection(ops, dev)
+        _pruned_channels_and_selection(ops, dev, M, dp)
     finally:
         ops.set_kvstar_tiles_per_wave(0)
 
 
-def _pruned_channels_and_selection(ops, dev):
+def _pruned_channels_and_selection(ops, dev, M, dp):
 
-    x, hq, hkv, d, M, dp = 8, 32, 8, 128, 8, 77              # 77 kept channels: table rows padded to 80
+    x, hq, hkv, d = 8, 32, 8, 128
     lens = [90, 33]
     rows = int(np.sum(lens))
     pruned = np.stack([[synth.permutation(1200 + 10 * t + h, d)[:dp] for h in range(hkv)] for t in range(2)]).astype(np.int32)
-    d_pad = 80
+    d_pad = (dp + 15) // 16 * 16
     repre = np.zeros((rows, M, hkv, d_pad), np.uint16)
     repre[..., :dp] = f16_bits(synth.normal_f32(1201, (rows, M, hkv, dp)) * np.float32(0.3))
     qs = [f16_bits(synth.normal_f32(1202 + t, (x, hq, d)) * np.float32(0.3)) for t in range(2)]

@@ -208,37 +208,56 @@ constexpr float kLog2e = 1.4426950408889634f;
 // (in the reference's [row][sub-block][kv head][d] order each vector of a head sits kv_heads*d*2 bytes
 // from the next).  The head's query rows are staged in LDS once per workgroup.
 //
-// kLds == false (any task length; a task may be cut into chunks): per 32-sub-block tile and query row
-// the kernel leaves the tile's maximum and sum of exponentials ([tile][2][row_pad]) and the per-block
-// sums ([block][row_pad], blocks padded to whole tiles) in the workspace for the two kernels below.
+// kSteps = MFMA steps a vector takes (d_pad <= 16*kSteps; 2, 4 or 8).  A wave always moves eight
+// 16-byte loads per lane at a time - a "span" of 8/kSteps tiles of 32 sub-blocks - so the bytes in
+// flight do not shrink with the vectors.
 //
-// kLds == true (one workgroup walks the whole task and the task's [block][row_pad] plane fits LDS): the
-// plane stays in LDS, as log2 of each block's sum of exponentials (one number instead of a sum and the
-// maximum it is relative to), the workgroup itself reduces every row's maximum and denominator when it
-// is through, and only this head's share of the votes ([task][kv head][max_blocks], in ws_part) goes
-// to memory: 1/32 of the other path's stores, whose number per compute unit - not their bytes - is
-// what that path pays for.
-template <int kM, bool kTwoRowTiles, bool kLds>
+// kLds == false (any task length; a task may be cut into chunks): per tile and query row the kernel
+// leaves the tile's maximum and sum of exponentials ([tile][2][row_pad]) and the per-block sums
+// ([part][row_pad]; a part is a block, or a tile's share of a block of more than 32 sub-blocks) in the
+// workspace for the two kernels below.
+//
+// kLds == true (one workgroup walks the whole task and the task's plane fits LDS): the plane stays in
+// LDS, as log2 of each entry's sum of exponentials (one number instead of a sum and the maximum it is
+// relative to; an entry is a block, or a span's share of a block longer than a span), the workgroup
+// itself reduces every row's maximum and denominator when it is through, and only this head's share of
+// the votes ([task][kv head][max_blocks], in ws_part) goes to memory: 1/32 of the other path's stores,
+// whose number per compute unit - not their bytes - is what that path pays for.
+template <int kM, int kSteps, bool kTwoRowTiles, bool kLds>
 __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const unsigned short* __restrict__ q, const int64_t* __restrict__ q_off, unsigned n_tokens, unsigned q_heads,
     unsigned d_orig, const int32_t* __restrict__ pruned, const int32_t* __restrict__ pruned_sel,
     const unsigned short* __restrict__ table, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
     float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
-    unsigned tiles_per_wave, unsigned row_pad, unsigned plane_offset)
+    unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset)
 {
+    static_assert(kM >= 1 && kM <= 128 && (kM & (kM - 1)) == 0, "sub-blocks per block");
+    static_assert(kSteps == 2 || kSteps == 4 || kSteps == 8, "MFMA steps per vector");
+    constexpr int kLoads = kMaxDim / 16;                 // 16-byte loads per lane and span
+    constexpr int kSpanTiles = kLoads / kSteps;
+    constexpr unsigned kSpan = kSpanTiles * kTileSub;    // sub-blocks per span
+    constexpr int kRowTiles = kTwoRowTiles ? 2 : 1;      // 33..64 query rows per kv head take two
+    constexpr unsigned kStride = kWaves * kSpan;         // from one span of a wave to its next
+    constexpr int kTilePart = kM < kTileSub ? kM : kTileSub;          // sub-blocks of one block inside one tile
+    constexpr unsigned kPartsPerTile = kTileSub / kTilePart;
+    constexpr unsigned kEntrySub = kM < static_cast<int>(kSpan) ? kM : kSpan;   // kLds: sub-blocks per plane entry
+    constexpr unsigned kEntryTiles = kEntrySub > kTileSub ? kEntrySub / kTileSub : 1;
+    constexpr unsigned kEntriesPerBlock = kM / kEntrySub;
+
     extern __shared__ __attribute__((aligned(16))) unsigned short q_s[];   // [row_pad][kQStride]
-    // kLds: [block][row_pad] floats from byte plane_offset on (0 with one row tile: the queries then live in
+    // kLds: [entry][row_pad] floats from byte plane_offset on (0 with one row tile: the queries then live in
     // registers once the loop starts), followed by the waves' [wave][2][row_pad] running (maximum, sum) pairs
     float* plane = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(q_s) + plane_offset);
 
     const unsigned task = blockIdx.z, h = blockIdx.y;
     const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);   // the planes are sized for max_blocks
     const unsigned S = n_blocks * kM;
-    const unsigned chunk = kWaves * tiles_per_wave * kTileSub;
+    const unsigned chunk = kWaves * spans_per_wave * kSpan;
     const unsigned s_chunk = blockIdx.x * chunk;
     if (s_chunk >= S) { return; }
-    const unsigned s_last = min(S, s_chunk + chunk) - 1;  // last sub-block of this workgroup
+    const unsigned s_end = min(S, s_chunk + chunk);
+    const unsigned s_last = s_end - 1;                   // last sub-block of this workgroup
     const unsigned g = q_heads / kv_heads, R = n_tokens * g;
     const int32_t psel = pruned_sel ? pruned_sel[task] : -1;
     const int32_t* pr = (pruned && psel >= 0) ? pruned + (static_cast<size_t>(psel) * kv_heads + h) * d_pruned : nullptr;
@@ -246,44 +265,43 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = lane >> 5, lr = lane & 31;
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes piece 2*ks + half
-    constexpr int kRowTiles = kTwoRowTiles ? 2 : 1;      // 33..64 query rows per kv head take two
-    constexpr unsigned kStride = kWaves * kTileSub;      // from one tile of a wave to its next
-    // Sums are kept per "part": a block, or - when a block has more sub-blocks than a tile - the block's share
-    // of one tile; kParts parts make a block
-    constexpr int kPartSub = kM < kTileSub ? kM : kTileSub;
-    constexpr unsigned kParts = kM / kPartSub;
     const unsigned short* tbase = table + static_cast<int64_t>(h) * head_stride +
                                   static_cast<size_t>(seg_off[task]) * kM * d_pad + half * (8 * kM);
 
-    // A tile's keys: eight 16-byte loads per lane, piece 2*ks + half of its sub-block; the lanes of one
-    // instruction cover M*16 contiguous bytes per block and lane half.  Everything is unconditional - MFMA
-    // steps past d_pad reload piece 0 and are multiplied with a zero query fragment, lanes and tiles past
-    // the workgroup's end reload its last vector and are masked or never used.
+    // A span's keys: for each of its tiles, kSteps 16-byte loads per lane, piece 2*ks + half of the lane's
+    // sub-block; the lanes of one instruction cover M*16 contiguous bytes per block and lane half.
+    // Everything is unconditional - MFMA steps past d_pad reload piece 0 and are multiplied with a zero
+    // query fragment, lanes and tiles past the workgroup's end reload its last vector and are masked or
+    // never used.
     //
-    // Three key buffers rotate, so two tiles are in flight while one is worked on.  The loads and the waits
-    // for them are written as assembly: left to itself the compiler sinks a prefetch down to the tile that
+    // Three key buffers rotate, so two spans are in flight while one is worked on.  The loads and the waits
+    // for them are written as assembly: left to itself the compiler sinks a prefetch down to the span that
     // consumes it (there is nothing but a loop exit in between), which leaves nothing in flight.  Vector
-    // memory operations complete in issue order, loads and stores alike, so "the loads of tile t have
-    // landed" is "at most as many operations outstanding as were issued after them" (keys_landed below).
-    auto load_keys = [&](u32x4 (&kf)[kMaxDim / 16], unsigned s0) {
-        const unsigned s_mine = min(s0 + lr, s_last);
-        const unsigned short* krow = tbase + static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
+    // memory operations complete in issue order, loads and stores alike, so "the loads of span t have
+    // landed" is "at most as many operations outstanding as were issued after them".
+    auto load_keys = [&](u32x4 (&kf)[kLoads], unsigned s0) {
 #pragma unroll
-        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-            const unsigned short* p = krow + (ks < ksteps ? ks : 0u) * (16 * kM);
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kf[ks]) : "v"(p) : "memory");
+        for (int t = 0; t < kSpanTiles; ++t) {
+            const unsigned s_mine = min(s0 + t * kTileSub + lr, s_last);
+            const unsigned short* krow = tbase + static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
+#pragma unroll
+            for (int ks = 0; ks < kSteps; ++ks) {
+                const unsigned short* p = krow + (static_cast<unsigned>(ks) < ksteps ? ks : 0) * (16 * kM);
+                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kf[t * kSteps + ks]) : "v"(p) : "memory");
+            }
         }
     };
-    u32x4 k0[kMaxDim / 16], k1[kMaxDim / 16], k2[kMaxDim / 16];
-    const unsigned s_first = s_chunk + wave * kTileSub;
+    u32x4 k0[kLoads], k1[kLoads], k2[kLoads];
+    const unsigned s_first = s_chunk + wave * kSpan;
     load_keys(k0, s_first);
     load_keys(k1, s_first + kStride);
     load_keys(k2, s_first + 2 * kStride);
 
-    // ---- the head's query rows, gathered by the kept channels, zero padded (rows up to row_pad, columns up to d_pad)
+    // ---- the head's query rows, gathered by the kept channels, zero padded (rows up to row_pad, columns up to 16*kSteps)
+    constexpr unsigned kCols = 16 * kSteps;
     const unsigned short* qt = q + q_off[task];
-    if (!pr && d_pruned == d_pad && (d_orig % 8) == 0 && (reinterpret_cast<uintptr_t>(qt) & 15u) == 0) {
-        const unsigned cpr = d_pad / 8;                  // 16-byte pieces per row
+    if (!pr && d_pruned == kCols && (d_orig % 8) == 0 && (reinterpret_cast<uintptr_t>(qt) & 15u) == 0) {
+        constexpr unsigned cpr = kCols / 8;              // 16-byte pieces per row
         for (unsigned e = threadIdx.x; e < row_pad * cpr; e += kThreads) {
             const unsigned rho = e / cpr, c = e - rho * cpr;
             u32x4 v = {0u, 0u, 0u, 0u};
@@ -294,8 +312,8 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
             *reinterpret_cast<u32x4*>(&q_s[rho * kQStride + c * 8]) = v;
         }
     } else {
-        for (unsigned e = threadIdx.x; e < row_pad * d_pad; e += kThreads) {
-            const unsigned rho = e / d_pad, p = e - rho * d_pad;
+        for (unsigned e = threadIdx.x; e < row_pad * kCols; e += kThreads) {
+            const unsigned rho = e / kCols, p = e - rho * kCols;
             unsigned short v = 0;
             if (rho < R && p < d_pruned) {
                 const unsigned xt = rho / g, gg = rho - xt * g;
@@ -308,100 +326,121 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     __syncthreads();
 
     // the query fragments do not change from tile to tile: with one row tile they stay in registers
-    u32x4 bq[kTwoRowTiles ? 1 : kMaxDim / 16];
-    const u32x4 zero = {0u, 0u, 0u, 0u};
+    // (columns from d_pad to 16*kSteps are zero, so the reloaded key pieces of those steps do not count)
+    u32x4 bq[kTwoRowTiles ? 1 : kSteps];
     if constexpr (!kTwoRowTiles) {
 #pragma unroll
-        for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-            const u32x4 braw = *reinterpret_cast<const u32x4*>(&q_s[lr * kQStride + half * 8 + (ks < ksteps ? ks : 0u) * 16]);
-            bq[ks] = ks < ksteps ? braw : zero;
+        for (int ks = 0; ks < kSteps; ++ks) {
+            bq[ks] = *reinterpret_cast<const u32x4*>(&q_s[lr * kQStride + half * 8 + ks * 16]);
         }
+        if constexpr (kLds) { __syncthreads(); }         // every wave has its query fragments: the plane may overwrite them
     }
 
-    if constexpr (kLds) { __syncthreads(); }             // every wave has its query fragments: the plane may overwrite them
-
     float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h) * (2 * row_pad) * max_tiles;          // [tile][2][row_pad]
-    float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * (kTileSub / kPartSub) * max_tiles;  // [part][row_pad]
-
+    float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * kPartsPerTile * max_tiles;  // [part][row_pad]
     float m_run[kRowTiles], d_run[kRowTiles];            // kLds only
 #pragma unroll
     for (int rt = 0; rt < kRowTiles; ++rt) { m_run[rt] = -INFINITY; d_run[rt] = 0.0f; }
 
-    auto process = [&](const u32x4 (&kf)[kMaxDim / 16], unsigned s0) {
-        const unsigned tile = s0 / kTileSub;
-        f32x16 acc[kRowTiles];
+    auto process = [&](const u32x4 (&kf)[kLoads], unsigned s_span) {
+        float e_max[kRowTiles], e_sum[kRowTiles];        // kLds, blocks longer than a tile: the plane entry being gathered
 #pragma unroll
-        for (int rt = 0; rt < kRowTiles; ++rt) {
+        for (int t = 0; t < kSpanTiles; ++t) {
+            const unsigned s0 = s_span + t * kTileSub;
+            const unsigned tile = s0 / kTileSub;
+            const bool live = s0 < S;                    // wave-uniform; a dead tile is computed on reloaded keys
+            const bool full = s0 + kTileSub <= S;        // and stored to padding: only a task's last tile needs the mask
+            f32x16 acc[kRowTiles];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { acc[rt][i] = 0.0f; }
+            for (int rt = 0; rt < kRowTiles; ++rt) {
 #pragma unroll
-            for (unsigned ks = 0; ks < kMaxDim / 16; ++ks) {
-                u32x4 b;
-                if constexpr (kTwoRowTiles) {
-                    const u32x4 braw = *reinterpret_cast<const u32x4*>(
-                        &q_s[(rt * 32 + lr) * kQStride + half * 8 + (ks < ksteps ? ks : 0u) * 16]);
-                    b = ks < ksteps ? braw : zero;
-                } else {
-                    b = bq[ks];
+                for (int i = 0; i < 16; ++i) { acc[rt][i] = 0.0f; }
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks) {
+                    u32x4 b;
+                    if constexpr (kTwoRowTiles) {
+                        b = *reinterpret_cast<const u32x4*>(&q_s[(rt * 32 + lr) * kQStride + half * 8 + ks * 16]);
+                    } else {
+                        b = bq[ks];
+                    }
+                    acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[t * kSteps + ks]),
+                                                                    __builtin_bit_cast(f16x8, b), acc[rt], 0, 0, 0);
                 }
-                acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[ks]), __builtin_bit_cast(f16x8, b),
-                                                                acc[rt], 0, 0, 0);
             }
-        }
-        const bool full = s0 + kTileSub <= S;            // wave-uniform: only a task's last tile needs the mask
 #pragma unroll
-        for (int rt = 0; rt < kRowTiles; ++rt) {
-            const unsigned rho = rt * 32 + lr;
-            float sc[16];
+            for (int rt = 0; rt < kRowTiles; ++rt) {
+                const unsigned rho = rt * 32 + lr;
+                float sc[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
-                sc[i] = (full || s < S) ? acc[rt][i] : -INFINITY;
-            }
-            float mx = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
+                for (int i = 0; i < 16; ++i) {
+                    const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
+                    sc[i] = (full || s < S) ? acc[rt][i] : -INFINITY;
+                }
+                float mx = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
 #pragma unroll
-            for (int i = 3; i < 15; i += 2) { mx = fmaxf(fmaxf(mx, sc[i]), sc[i + 1]); }
-            mx = fmaxf(mx, sc[15]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));      // the tile has at least one live sub-block, so mx is finite
-            const float nmx = -mx * kLog2e;
-            float e[16];
+                for (int i = 3; i < 15; i += 2) { mx = fmaxf(fmaxf(mx, sc[i]), sc[i + 1]); }
+                mx = fmaxf(mx, sc[15]);
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // a live tile has at least one live sub-block, so mx is finite
+                const float nmx = -mx * kLog2e;
+                float e[16];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], kLog2e, nmx)); }
-            // rows past R hold zero queries: they are computed like the rest and never read
-            const unsigned blk0 = tile * (kTileSub / kPartSub);   // first part of the tile
-            if constexpr (kLds) {
-                const float mx2 = mx * kLog2e;
-                const float total = block_sums<kPartSub>(e, half, [&](unsigned b, float v) {
-                    plane[(blk0 + b) * row_pad + rho] = mx2 + __builtin_amdgcn_logf(v);   // log2 of the block's sum of 2^(score*log2e)
-                });
-                // the wave's running (maximum, sum of 2^(x - maximum)) of the row, in the same log2 units
-                const float m_new = fmaxf(m_run[rt], mx2);
-                d_run[rt] = d_run[rt] * __builtin_amdgcn_exp2f(m_run[rt] - m_new) + total * __builtin_amdgcn_exp2f(mx2 - m_new);
-                m_run[rt] = m_new;
-            } else {
-                const float total = block_sums<kPartSub>(e, half, [&](unsigned b, float v) {
-                    wpart[static_cast<size_t>(blk0 + b) * row_pad + rho] = v;
-                });
-                wmax[(static_cast<size_t>(tile) * 2 + half) * row_pad + rho] = half ? total : mx;
+                for (int i = 0; i < 16; ++i) { e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], kLog2e, nmx)); }
+                // rows past R hold zero queries: they are computed like the rest and never read
+                const unsigned part0 = tile * kPartsPerTile;   // first part of the tile
+                if constexpr (kLds) {
+                    const float mx2 = mx * kLog2e;
+                    float total;
+                    if constexpr (kEntryTiles == 1) {
+                        // an entry lies inside this tile: log2 of the block's sum of 2^(score*log2e)
+                        total = block_sums<kTilePart>(e, half, [&](unsigned b, float v) {
+                            plane[(part0 + b) * row_pad + rho] = mx2 + __builtin_amdgcn_logf(v);
+                        });
+                    } else {
+                        // an entry spans kEntryTiles tiles of this span: gather (maximum, sum) over them
+                        total = block_sums<kTilePart>(e, half, [](unsigned, float) {});
+                        const float lt = live ? mx2 + __builtin_amdgcn_logf(total) : -INFINITY;
+                        if (t % kEntryTiles == 0) {
+                            e_max[rt] = lt;
+                            e_sum[rt] = 1.0f;
+                        } else {
+                            const float m_new = fmaxf(e_max[rt], lt);
+                            e_sum[rt] = e_sum[rt] * __builtin_amdgcn_exp2f(e_max[rt] - m_new) + __builtin_amdgcn_exp2f(lt - m_new);
+                            e_max[rt] = m_new;
+                        }
+                        if (t % kEntryTiles == kEntryTiles - 1) {
+                            plane[(tile / kEntryTiles) * row_pad + rho] = e_max[rt] + __builtin_amdgcn_logf(e_sum[rt]);
+                        }
+                    }
+                    // the wave's running (maximum, sum of 2^(x - maximum)) of the row, in the same log2 units
+                    if (live) {
+                        const float m_new = fmaxf(m_run[rt], mx2);
+                        d_run[rt] = d_run[rt] * __builtin_amdgcn_exp2f(m_run[rt] - m_new) + total * __builtin_amdgcn_exp2f(mx2 - m_new);
+                        m_run[rt] = m_new;
+                    }
+                } else {
+                    const float total = block_sums<kTilePart>(e, half, [&](unsigned b, float v) {
+                        wpart[static_cast<size_t>(part0 + b) * row_pad + rho] = v;
+                    });
+                    wmax[(static_cast<size_t>(tile) * 2 + half) * row_pad + rho] = half ? total : mx;
+                }
             }
         }
     };
 
-    // Operations issued after a tile's loads when the wave turns to it: the loads of the two tiles behind it
-    // (16) and the stores of the tiles worked on since - none for the wave's first tile, one tile's for its
-    // second, two tiles' from then on.
-    constexpr unsigned kStores = kLds ? 0 : kRowTiles * (1 + (kM >= 16 ? 1 : kM == 8 ? 2 : kM == 4 ? 4 : kM == 2 ? 8 : 16));
-    static_assert(kM == 1 || kM == 2 || kM == 4 || kM == 8 || kM == 16 || kM == 32 || kM == 64 || kM == 128, "sub-blocks per block");
-    constexpr unsigned kAfter0 = 16, kAfter1 = 16 + kStores > 63 ? 63 : 16 + kStores,
-                       kAfter2 = 16 + 2 * kStores > 63 ? 63 : 16 + 2 * kStores;
+    // Operations issued after a span's loads when the wave turns to it: the loads of the two spans behind it
+    // (16) and the stores of the spans worked on since - none for the wave's first span, one span's for its
+    // second, two spans' from then on.
+    constexpr unsigned kStores =
+        kLds ? 0 : kSpanTiles * kRowTiles * (1 + (kTilePart >= 16 ? 1 : kTilePart == 8 ? 2 : kTilePart == 4 ? 4 : kTilePart == 2 ? 8 : 16));
+    constexpr unsigned kAfter0 = 2 * kLoads, kAfter1 = kAfter0 + kStores > 63 ? 63 : kAfter0 + kStores,
+                       kAfter2 = kAfter0 + 2 * kStores > 63 ? 63 : kAfter0 + 2 * kStores;
 #define UCM_KEYS_LANDED(k, n)                                                                                              \
     asm volatile("s_waitcnt vmcnt(%8)"                                                                                     \
                  : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]), "+v"(k[4]), "+v"(k[5]), "+v"(k[6]), "+v"(k[7])         \
                  : "n"(n)                                                                                                  \
                  : "memory")
-    const unsigned s_end = min(S, s_chunk + chunk);
     unsigned s0 = s_first;
-    if (s0 < s_end) {                                    // the wave's first two tiles, with fewer stores behind them
+    if (s0 < s_end) {                                    // the wave's first two spans, with fewer stores behind them
         UCM_KEYS_LANDED(k0, kAfter0);
         process(k0, s0);
         load_keys(k0, s0 + 3 * kStride);
@@ -434,7 +473,8 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 
     if constexpr (kLds) {
         // ---- this head's share of the votes, from the plane in LDS
-        float* red = plane + static_cast<size_t>(max_tiles) * (kTileSub / kPartSub) * row_pad;   // [wave][2][row_pad]
+        const unsigned plane_entries = kM < kTileSub ? max_tiles * kPartsPerTile : max_tiles / kEntryTiles;
+        float* red = plane + static_cast<size_t>(plane_entries) * row_pad;   // [wave][2][row_pad]
         if (half == 0) {
 #pragma unroll
             for (int rt = 0; rt < kRowTiles; ++rt) {
@@ -445,7 +485,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
         __syncthreads();                                 // the plane and the waves' pairs are complete
         float row_m = 0.0f, row_w = 0.0f;
         if (threadIdx.x < row_pad) {
-            row_m = red[threadIdx.x];                    // wave 0 always has a tile, so this is finite
+            row_m = red[threadIdx.x];                    // wave 0 always has a live tile, so this is finite
 #pragma unroll
             for (int w = 1; w < kWaves; ++w) { row_m = fmaxf(row_m, red[(w * 2) * row_pad + threadIdx.x]); }
             float den = 0.0f;
@@ -466,10 +506,10 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
         float* vh = ws_part + (static_cast<size_t>(task) * kv_heads + h) * max_blocks;
         for (unsigned b = threadIdx.x; b < n_blocks; b += kThreads) {
             float v = 0.0f;
-            for (unsigned part = b * kParts; part < (b + 1) * kParts; ++part) {
+            for (unsigned entry = b * kEntriesPerBlock; entry < (b + 1) * kEntriesPerBlock; ++entry) {
                 for (unsigned r = 0; r < row_pad; ++r) {
                     const unsigned rr = (r + b) & (row_pad - 1);
-                    v += __builtin_amdgcn_exp2f(plane[part * row_pad + rr] - red[rr]) * red[row_pad + rr];
+                    v += __builtin_amdgcn_exp2f(plane[entry * row_pad + rr] - red[rr]) * red[row_pad + rr];
                 }
             }
             vh[b] = v;
@@ -643,12 +683,21 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
 }
 
+namespace {
+// Tiles the planes are sized for: a wave works in spans of up to four tiles and stores all of them
+int64_t padded_tiles(int64_t sub_blocks_total)
+{
+    const int64_t tiles = (sub_blocks_total + kTileSub - 1) / kTileSub;
+    return (tiles + 3) / 4 * 4;
+}
+}  // namespace
+
 extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks,
                                            int64_t* max_floats, int64_t* part_floats)
 {
     UCM_REQUIRE(n_tasks >= 0 && kv_heads > 0 && rows_per_head > 0 && rows_per_head <= kMaxRows && max_blocks >= 0 &&
                     sub_blocks > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
-    const int64_t tiles = (static_cast<int64_t>(max_blocks) * sub_blocks + kTileSub - 1) / kTileSub;
+    const int64_t tiles = padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks);
     const int64_t row_pad = rows_per_head > 32 ? 64 : 32;
     UCM_REQUIRE(sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
     // per (task, kv head): a (maximum, sum) pair per tile and row; a partial sum per row and block (per tile,
@@ -685,50 +734,61 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
                   "ucm_kvstar_votes: sub_blocks=%d (a power of two up to 128)", sub_blocks);
     UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0,
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
-    const int64_t S = static_cast<int64_t>(max_blocks) * sub_blocks;
-    const unsigned max_tiles = static_cast<unsigned>((S + kTileSub - 1) / kTileSub);
+    const unsigned max_tiles = static_cast<unsigned>(padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks));
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
     const unsigned row_pad = R > 32 ? 64 : 32;
     const unsigned q_bytes = row_pad * kQStride * 2;
-    // One workgroup per (task, kv head) with the task's [block][row_pad] plane in LDS, when there are enough
-    // such workgroups to fill the device and the plane fits; otherwise the workspace path, which may cut a
-    // task into chunks.  ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
+    const unsigned steps = d_pad <= 32 ? 2u : d_pad <= 64 ? 4u : 8u;     // MFMA steps per vector the kernel is built for
+    const unsigned span_tiles = 8u / steps;                                // tiles a wave moves at a time
+    // One workgroup per (task, kv head) with the task's plane in LDS, when there are enough such workgroups to
+    // fill the device and the plane fits; otherwise the workspace path, which may cut a task into chunks.
+    // ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
     const unsigned plane_offset = R > 32 ? q_bytes : 0u;
-    const size_t lds_plane = plane_offset + static_cast<size_t>(max_tiles) * (kTileSub / std::min(sub_blocks, kTileSub)) * row_pad * 4 +
-                             2 * kWaves * row_pad * 4;
+    const unsigned entry_tiles = static_cast<unsigned>(sub_blocks) <= kTileSub
+                                     ? 1u : std::min<unsigned>(sub_blocks, span_tiles * kTileSub) / kTileSub;
+    const size_t plane_entries = static_cast<unsigned>(sub_blocks) < kTileSub
+                                     ? static_cast<size_t>(max_tiles) * (kTileSub / sub_blocks) : max_tiles / entry_tiles;
+    const size_t lds_plane = plane_offset + plane_entries * row_pad * 4 + 2 * kWaves * row_pad * 4;
     const bool use_lds = g_tiles_per_wave <= 0 && lds_plane <= kLdsPathMaxBytes &&
                          (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
     const unsigned lds_bytes = use_lds ? static_cast<unsigned>(std::max<size_t>(lds_plane, q_bytes)) : q_bytes;
-    // a workgroup stages its queries once, so it should walk many tiles; the longest task is still cut into
+    // a workgroup stages its queries once, so it should walk many spans; the longest task is still cut into
     // enough chunks that about 2048 workgroups exist
-    const unsigned tiles_per_wg_all = (max_tiles + kWaves - 1) / kWaves;
+    const unsigned max_spans = (max_tiles + span_tiles - 1) / span_tiles;
+    const unsigned spans_per_wg_all = (max_spans + kWaves - 1) / kWaves;
     const unsigned want_chunks = use_lds ? 1u : std::max(1u, 2048u / static_cast<unsigned>(n_tasks * kv_heads));
-    const unsigned tiles_per_wave = g_tiles_per_wave > 0 ? static_cast<unsigned>(g_tiles_per_wave)
-                                                         : std::max(1u, (tiles_per_wg_all + want_chunks - 1) / want_chunks);
-    const unsigned chunks = (max_tiles + kWaves * tiles_per_wave - 1) / (kWaves * tiles_per_wave);
+    const unsigned spans_per_wave = g_tiles_per_wave > 0
+                                        ? (static_cast<unsigned>(g_tiles_per_wave) + span_tiles - 1) / span_tiles
+                                        : std::max(1u, (spans_per_wg_all + want_chunks - 1) / want_chunks);
+    const unsigned chunks = (max_spans + kWaves * spans_per_wave - 1) / (kWaves * spans_per_wave);
     hipStream_t s = ucm::as_stream(stream);
 #define UCM_KVSTAR_ARGS dim3(chunks, kv_heads, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), seg_off, seg_len, static_cast<unsigned>(kv_heads),                     \
         static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, ws_max, ws_part,                   \
-        static_cast<unsigned>(max_blocks), max_tiles, tiles_per_wave, row_pad, plane_offset
-#define UCM_KVSTAR_LAUNCH3(M, TWO, LDS)                                                                               \
+        static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset
+#define UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, LDS)                                                                        \
     do {                                                                                                             \
         if (lds_bytes > 48u * 1024u) {                                                                               \
-            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_score_kernel<M, TWO, LDS>), \
-                                                      hipFuncAttributeMaxDynamicSharedMemorySize,                   \
-                                                      static_cast<int>(lds_bytes));                                \
+            const hipError_t ea = hipFuncSetAttribute(                                                               \
+                reinterpret_cast<const void*>(kvstar_score_kernel<M, STEPS, TWO, LDS>),                              \
+                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));                           \
             if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_votes (LDS size)"); }                      \
         }                                                                                                            \
-        hipLaunchKernelGGL((kvstar_score_kernel<M, TWO, LDS>), UCM_KVSTAR_ARGS);                                     \
+        hipLaunchKernelGGL((kvstar_score_kernel<M, STEPS, TWO, LDS>), UCM_KVSTAR_ARGS);                              \
     } while (0)
-#define UCM_KVSTAR_LAUNCH2(M, TWO)                                                                                    \
+#define UCM_KVSTAR_LAUNCH3(M, STEPS, TWO)                                                                             \
     do {                                                                                                             \
-        if (use_lds) { UCM_KVSTAR_LAUNCH3(M, TWO, true); } else { UCM_KVSTAR_LAUNCH3(M, TWO, false); }               \
+        if (use_lds) { UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, true); } else { UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, false); } \
+    } while (0)
+#define UCM_KVSTAR_LAUNCH2(M, STEPS)                                                                                  \
+    do {                                                                                                             \
+        if (R > 32) { UCM_KVSTAR_LAUNCH3(M, STEPS, true); } else { UCM_KVSTAR_LAUNCH3(M, STEPS, false); }            \
     } while (0)
 #define UCM_KVSTAR_LAUNCH(M)                                                                                          \
     do {                                                                                                             \
-        if (R > 32) { UCM_KVSTAR_LAUNCH2(M, true); } else { UCM_KVSTAR_LAUNCH2(M, false); }                          \
+        if (steps == 2) { UCM_KVSTAR_LAUNCH2(M, 2); } else if (steps == 4) { UCM_KVSTAR_LAUNCH2(M, 4); }             \
+        else { UCM_KVSTAR_LAUNCH2(M, 8); }                                                                           \
     } while (0)
     switch (sub_blocks) {
     case 1: UCM_KVSTAR_LAUNCH(1); break;
@@ -743,6 +803,7 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
 #undef UCM_KVSTAR_LAUNCH
 #undef UCM_KVSTAR_LAUNCH2
 #undef UCM_KVSTAR_LAUNCH3
+#undef UCM_KVSTAR_LAUNCH4
 #undef UCM_KVSTAR_ARGS
     if (hipError_t e = hipGetLastError(); e != hipSuccess) { return ucm::check_hip(e, "ucm_kvstar_votes (scores)"); }
     if (use_lds) {
