@@ -30,6 +30,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+KVSTAR_TRAFFIC = None   # HBM bytes per step of the KVStar leg at its defaults (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE)
 
 N_REQ, N_LAYERS, HQ, HKV, D, BS = 16, 32, 32, 8, 128, 128
 ROW = HKV * D
@@ -55,8 +56,12 @@ def parse():
     ap.add_argument("--hash-leg", action="store_true",
                     help="also time the hash-code retrieval variant (BASELINE configs[4] shape) on the same caches")
     ap.add_argument("--kvstar-leg", action="store_true",
-                    help="also time the multi-query softmax-vote retrieval (KVStar shape: 8 query tokens per request, "
-                         "8 sub-block representatives per block) on the same ragged batch")
+                    help="also time the multi-query softmax-vote retrieval (KVStar: 8 query tokens per request) on the same "
+                         "ragged batch")
+    ap.add_argument("--kvstar-merge", type=int, default=2,
+                    help="tokens averaged into one sub-block representative (reference default 2: 64 per 128-token block)")
+    ap.add_argument("--kvstar-prune", type=float, default=0.25,
+                    help="share of the head's channels kept in the representatives (reference default 0.25; 1 = all)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
@@ -315,17 +320,30 @@ def main():
         del colsum, bcodes, tcodes
 
     # ---- KVStar leg: every (layer, request) is one task; 8 query tokens x 32 heads vote over the request's
-    # blocks through 8 sub-block representatives each (16-token means of the same key cache, fp16, kv head outermost)
+    # blocks through block_size/merge sub-block representatives each (means of `merge` tokens of the same key
+    # cache, fp16, kv head outermost), a share of the channels kept per (layer, kv head)
     kvstar_leg = None
     if args.kvstar_leg:
-        kx, merge = 8, 16
+        kx, merge = 8, args.kvstar_merge
         km = BS // merge
+        kdp = D if args.kvstar_prune >= 0.98 else round(D * args.kvstar_prune)
+        kd_pad = (kdp + 15) // 16 * 16
+        # kept channels: a seeded choice per (layer, kv head) (the reference keeps those with the largest mean |k|)
+        kpr = None
+        if kdp < D:
+            kpr = torch.stack([torch.stack([torch.randperm(D, device=dev, generator=g)[:kdp] for _ in range(HKV)])
+                               for _ in range(n_layers)]).to(torch.int32)
         # one table over all layers, kv head outermost: row of (layer l, block b) = l * rows + b
-        flat = torch.empty((HKV, n_layers * rows, D // 8, km, 8), dtype=torch.float16, device=dev)
-        ktab = flat.view(HKV, n_layers, rows, D // 8, km, 8).permute(1, 0, 2, 3, 4, 5)
+        flat = torch.empty((HKV, n_layers * rows, kd_pad // 8, km, 8), dtype=torch.float16, device=dev)
+        ktab = flat.view(HKV, n_layers, rows, kd_pad // 8, km, 8).permute(1, 0, 2, 3, 4, 5)
         ev0, ev1 = ev(), ev()
         ev0.record()
-        ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge)
+        if kpr is None:
+            ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge)
+        else:
+            for l_ in range(n_layers):                                  # a channel list per layer: one launch per layer
+                ops.kvstar_block_repre(ops.LayerPointers([caches[l_]]), table, slots, ktab[l_ : l_ + 1], BS, HKV, D, nb, merge,
+                                       pruned=kpr[l_])
         ev1.record()
         torch.cuda.synchronize()
         krep_ms = ev0.elapsed_time(ev1)
@@ -334,6 +352,7 @@ def main():
         k_len = np.tile(lens, n_layers)
         kq = (torch.randn(n_tasks, kx, HQ, D, device=dev, generator=g) * 0.25).to(torch.float16)
         kq_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (kx * HQ * D)
+        ksel = None if kpr is None else torch.arange(n_layers, dtype=torch.int32, device=dev).repeat_interleave(N_REQ)
         kvotes = torch.zeros(n_layers * rows, device=dev)
         kws = ops.kvstar_workspace(n_tasks, HKV, kx * HQ // HKV, max_len, km, dev)
         kso, ksl = i32(k_off), i32(k_len)
@@ -342,7 +361,7 @@ def main():
         kcnt = torch.zeros((1, n_tasks), dtype=torch.int32, device=dev)
 
         def kvstar_step():
-            ops.kvstar_votes(kq, kq_off, kx, HQ, flat, kso, ksl, max_len, kvotes, kws)
+            ops.kvstar_votes(kq, kq_off, kx, HQ, flat, kso, ksl, max_len, kvotes, kws, d_pruned=kdp, pruned=kpr, pruned_sel=ksel)
             ops.topk_windows(kvotes.view(1, -1), kso, ksl, ktk, max_len, kidx, kcnt, start_w=0, end_w=0)
 
         for _ in range(2):
@@ -362,23 +381,26 @@ def main():
             for t_ in (0, n_tasks // 2 + 3, n_tasks - 1):
                 a_, n_ = int(k_off[t_]), int(k_len[t_])
                 rep_ref = ops.kvstar_table_to_reference(flat[:, a_ : a_ + n_]).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
-                _, want = oracle.kvstar_retrieve(kq[t_].view(torch.int16).cpu().numpy().view(np.uint16), rep_ref, int(topk[t_ % N_REQ]))
+                pr_ = None if kpr is None else kpr[t_ // N_REQ].cpu().numpy().astype(np.int32)
+                _, want = oracle.kvstar_retrieve(kq[t_].view(torch.int16).cpu().numpy().view(np.uint16), rep_ref,
+                                                 int(topk[t_ % N_REQ]), pruned=pr_, d_pruned=kdp)
                 got = kvotes[a_ : a_ + n_].cpu().numpy()
                 assert np.allclose(got, want, rtol=2e-4, atol=2e-6), "KVStar votes differ from the CPU oracle"
             kv_checked = "votes of 3 sampled tasks within rtol 2e-4 / atol 2e-6 of the CPU oracle (fp32, other summation order)"
+        kv_default = n_layers == N_LAYERS and args.seed == 2024 and merge == 2 and kdp == 32
         kvstar_leg = {
             "workload": f"{n_tasks} tasks (layer x request), {kx} query tokens x {HQ} heads, {rows} blocks x {km} sub-block "
-                        f"representatives per layer, fp16",
+                        f"representatives per layer, {kdp} of {D} channels, fp16",
             "block_repre_ms": round(krep_ms, 3),
             "us_per_step": round(kv_ms * 1e3, 1),
             "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select)", "bound": "hbm",
                          "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4), "traffic": 2063200000 if (n_layers == N_LAYERS and args.seed == 2024) else None,
+                         "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4), "traffic": KVSTAR_TRAFFIC if kv_default else None,
                          "algorithmic_bytes": kv_bytes,
-                         "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * D / (kv_ms * 1e-3) / 1e12, 1)},
+                         "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * kd_pad / (kv_ms * 1e-3) / 1e12, 1)},
             "checked": kv_checked,
         }
-        del ktab, flat, kws
+        del ktab, flat, kws, kpr
 
     # ---- check the last step against the CPU oracle (selection, scores, gathered bytes)
     if not args.no_check:

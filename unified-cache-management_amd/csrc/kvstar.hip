@@ -80,25 +80,64 @@ __device__ __forceinline__ void add_bf16x8(float (&acc)[8], const u32x4 v)
     acc[6] = acc[6] + __uint_as_float(v.w << 16); acc[7] = acc[7] + __uint_as_float(v.w & 0xffff0000u);
 }
 
+// kMerge: the tokens per sub-block when that is 1, 2, 4 or 8 - a thread then works on 16/kMerge of its
+// (sub-block, 8 columns) items at a time so that sixteen loads are in flight - or 0 for any other count.
+template <int kMerge>
 __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
     unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
     unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row]
-    const unsigned M = block_size / merge;
+    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]: the 16 bytes of padding
+    const unsigned M = block_size / merge;                                   // spread the sub-blocks' rows over the LDS banks
     const unsigned id = static_cast<unsigned>(block_ids[blockIdx.x]);
     const unsigned slot = static_cast<unsigned>(slots[blockIdx.x]);
     if (id >= num_blocks || slot >= rows) { return; }   // whole workgroup: never dereference a bad id
-    const unsigned row = kv_heads * head_dim, ncg = row / 8;
+    const unsigned row = kv_heads * head_dim, ncg = row / 8, srow_stride = row + 8;
     const unsigned short* blk = static_cast<const unsigned short*>(k_layers[blockIdx.y]) +
                                 static_cast<size_t>(id) * block_size * row;
     const float inv = 1.0f / static_cast<float>(merge);
     const unsigned pieces = d_pad / 8;
     unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<size_t>(slot) * M * d_pad;
+    // the channel lists, read once: a load from memory per output piece would queue behind the key stream
+    int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
+    if (pruned) {
+        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = pruned[e]; }
+    }
     for (unsigned m0 = 0; m0 < M; m0 += m_chunk) {       // m_chunk sub-blocks at a time: what fits LDS
         const unsigned mc = min(m_chunk, M - m0);
+        if constexpr (kMerge > 0) {
+            constexpr unsigned kBatch = kRepreUnroll / kMerge;
+            for (unsigned w0 = threadIdx.x; w0 < mc * ncg; w0 += kThreads * kBatch) {
+                u32x4 v[kRepreUnroll];
+#pragma unroll
+                for (unsigned j = 0; j < kBatch; ++j) {
+                    const unsigned w = min(w0 + j * kThreads, mc * ncg - 1);   // clamped: loads stay unconditional
+                    const unsigned ml = w / ncg, cg = w - ml * ncg;
+                    const unsigned short* src = blk + static_cast<size_t>(m0 + ml) * kMerge * row + cg * 8;
+#pragma unroll
+                    for (unsigned t = 0; t < kMerge; ++t) { v[j * kMerge + t] = ucm::gload16_nt(src + static_cast<size_t>(t) * row); }
+                }
+#pragma unroll
+                for (unsigned j = 0; j < kBatch; ++j) {
+                    const unsigned w = w0 + j * kThreads;
+                    if (w >= mc * ncg) { break; }
+                    const unsigned ml = w / ncg, cg = w - ml * ncg;
+                    float acc[8];
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }
+#pragma unroll
+                    for (unsigned t = 0; t < kMerge; ++t) { add_bf16x8(acc, v[j * kMerge + t]); }
+                    u32x4 o;
+                    o.x = mean_to_f16x2(acc[0], acc[1], inv);
+                    o.y = mean_to_f16x2(acc[2], acc[3], inv);
+                    o.z = mean_to_f16x2(acc[4], acc[5], inv);
+                    o.w = mean_to_f16x2(acc[6], acc[7], inv);
+                    *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
+                }
+            }
+        } else {
         for (unsigned w = threadIdx.x; w < mc * ncg; w += kThreads) {
             const unsigned ml = w / ncg, cg = w - ml * ncg;
             const unsigned short* src = blk + static_cast<size_t>(m0 + ml) * merge * row + cg * 8;
@@ -119,29 +158,34 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
             o.y = mean_to_f16x2(acc[2], acc[3], inv);
             o.z = mean_to_f16x2(acc[4], acc[5], inv);
             o.w = mean_to_f16x2(acc[6], acc[7], inv);
-            *reinterpret_cast<u32x4*>(&stage[ml * row + cg * 8]) = o;
+            *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
+        }
         }
         __syncthreads();
         for (unsigned e = threadIdx.x; e < kv_heads * pieces * mc; e += kThreads) {
             const unsigned h = e / (pieces * mc), rem = e - h * (pieces * mc);
             const unsigned piece = rem / mc, ml = rem - piece * mc;
-            const unsigned short* srow = stage + ml * row + h * head_dim;
-            unsigned short c[8];
-#pragma unroll
-            for (unsigned j = 0; j < 8; ++j) {
-                const unsigned p = piece * 8 + j;
-                unsigned short v = 0;
-                if (p < d_pruned) {
-                    const unsigned d = pruned ? static_cast<unsigned>(pruned[h * d_pruned + p]) : p;
-                    if (d < head_dim) { v = srow[d]; }
-                }
-                c[j] = v;
-            }
+            const unsigned short* srow = stage + ml * srow_stride + h * head_dim;
             u32x4 o;
-            o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
-            o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
-            o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
-            o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
+            if (!pruned && piece * 8 + 8 <= d_pruned) {  // all channels kept: the piece is 16 contiguous bytes
+                o = *reinterpret_cast<const u32x4*>(srow + piece * 8);
+            } else {
+                unsigned short c[8];
+#pragma unroll
+                for (unsigned j = 0; j < 8; ++j) {
+                    const unsigned p = piece * 8 + j;
+                    unsigned short v = 0;
+                    if (p < d_pruned) {
+                        const unsigned d = pruned ? static_cast<unsigned>(kept[h * d_pruned + p]) : p;
+                        if (d < head_dim) { v = srow[d]; }
+                    }
+                    c[j] = v;
+                }
+                o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
+                o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
+                o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
+                o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
+            }
             ucm::gstore16(out + static_cast<int64_t>(h) * head_stride + (static_cast<size_t>(piece) * M + m0 + ml) * 8, o);
         }
         __syncthreads();                                 // the next chunk overwrites the staged means
@@ -230,7 +274,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const unsigned short* __restrict__ table, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
     float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
-    unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset)
+    unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset, unsigned q_full_ok)
 {
     static_assert(kM >= 1 && kM <= 128 && (kM & (kM - 1)) == 0, "sub-blocks per block");
     static_assert(kSteps == 2 || kSteps == 4 || kSteps == 8, "MFMA steps per vector");
@@ -311,6 +355,27 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
             }
             *reinterpret_cast<u32x4*>(&q_s[rho * kQStride + c * 8]) = v;
         }
+    } else if (pr && q_full_ok && (reinterpret_cast<uintptr_t>(qt) & 15u) == 0) {
+        // kept channels: whole query rows go to a second LDS area (coalesced, one round trip together with
+        // the channel list) and are gathered from there
+        unsigned short* q_full = q_s + row_pad * kQStride;
+        const unsigned cpr = d_orig / 8;
+        for (unsigned e = threadIdx.x; e < row_pad * cpr; e += kThreads) {
+            const unsigned rho = e / cpr, c = e - rho * cpr;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (rho < R) {
+                const unsigned xt = rho / g, gg = rho - xt * g;
+                v = ucm::gload16(qt + (static_cast<size_t>(xt) * q_heads + h * g + gg) * d_orig + c * 8);
+            }
+            *reinterpret_cast<u32x4*>(&q_full[rho * kQStride + c * 8]) = v;
+        }
+        const unsigned p = threadIdx.x % kCols;          // kThreads is a multiple of kCols: a thread keeps its column
+        const unsigned ch = p < d_pruned ? static_cast<unsigned>(pr[p]) : 0xffffffffu;
+        __syncthreads();
+        for (unsigned e = threadIdx.x; e < row_pad * kCols; e += kThreads) {
+            const unsigned rho = e / kCols;
+            q_s[rho * kQStride + p] = ch < d_orig ? q_full[rho * kQStride + ch] : static_cast<unsigned short>(0);
+        }
     } else {
         for (unsigned e = threadIdx.x; e < row_pad * kCols; e += kThreads) {
             const unsigned rho = e / kCols, p = e - rho * kCols;
@@ -372,9 +437,13 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
                 const unsigned rho = rt * 32 + lr;
                 float sc[16];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
-                    sc[i] = (full || s < S) ? acc[rt][i] : -INFINITY;
+                for (int i = 0; i < 16; ++i) { sc[i] = acc[rt][i]; }
+                if (!full) {                             // no memory operation in here: a branch is harmless
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
+                        sc[i] = s < S ? sc[i] : -INFINITY;
+                    }
                 }
                 float mx = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
 #pragma unroll
@@ -664,22 +733,34 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
     UCM_SUPPORTED(row % 8 == 0 && d_pad % 8 == 0, "ucm_kvstar_block_repre: kv_heads*head_dim=%u and d_pad=%d must be multiples of 8",
                   row, d_pad);
-    UCM_SUPPORTED(row <= 32768u, "ucm_kvstar_block_repre: kv_heads*head_dim=%u (at most 32768)", row);
-    const unsigned m_chunk = std::min<unsigned>(static_cast<unsigned>(M), 32768u / row);   // sub-blocks staged at a time: 64 KiB of LDS
-    const size_t lds_bytes = static_cast<size_t>(m_chunk) * row * 2;
+    UCM_SUPPORTED(row <= 32768u && head_dim % 8 == 0, "ucm_kvstar_block_repre: kv_heads*head_dim=%u (at most 32768), head_dim=%d (a multiple of 8)", row, head_dim);
+    const unsigned m_chunk = std::min<unsigned>(static_cast<unsigned>(M), 33280u / (row + 8));   // sub-blocks staged at a time: 65 KiB of LDS
+    const size_t lds_bytes = static_cast<size_t>(m_chunk) * (row + 8) * 2 + (pruned ? static_cast<size_t>(kv_heads) * d_pruned * 4 : 0);
     UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_layer_stride % 8 == 0 && repre_head_stride % 8 == 0,
                 "ucm_kvstar_block_repre: table not 16-byte aligned");
-    if (lds_bytes > 48u * 1024u) {
-        const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_kernel),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
-        if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }
+#define UCM_KVSTAR_REPRE(MERGE)                                                                                        \
+    do {                                                                                                             \
+        if (lds_bytes > 48u * 1024u) {                                                                               \
+            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_kernel<MERGE>),     \
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize,                   \
+                                                      static_cast<int>(lds_bytes));                                \
+            if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }                \
+        }                                                                                                            \
+        hipLaunchKernelGGL(kvstar_repre_kernel<MERGE>, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, \
+                           ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),    \
+                           static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),                     \
+                           static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), static_cast<unsigned>(merge), \
+                           pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),                    \
+                           static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk); \
+    } while (0)
+    switch (merge) {
+    case 1: UCM_KVSTAR_REPRE(1); break;
+    case 2: UCM_KVSTAR_REPRE(2); break;
+    case 4: UCM_KVSTAR_REPRE(4); break;
+    case 8: UCM_KVSTAR_REPRE(8); break;
+    default: UCM_KVSTAR_REPRE(0); break;
     }
-    hipLaunchKernelGGL(kvstar_repre_kernel, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes,
-                       ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
-                       static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),
-                       static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), static_cast<unsigned>(merge),
-                       pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),
-                       static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk);
+#undef UCM_KVSTAR_REPRE
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
 }
 
@@ -751,7 +832,10 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     const size_t lds_plane = plane_offset + plane_entries * row_pad * 4 + 2 * kWaves * row_pad * 4;
     const bool use_lds = g_tiles_per_wave <= 0 && lds_plane <= kLdsPathMaxBytes &&
                          (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
-    const unsigned lds_bytes = use_lds ? static_cast<unsigned>(std::max<size_t>(lds_plane, q_bytes)) : q_bytes;
+    // with channel lists, whole query rows are staged in a second area of q_bytes and gathered from there
+    const unsigned q_full_ok = pruned != nullptr && d_orig % 8 == 0 && d_orig <= kMaxDim && ucm::aligned16(q_f16) ? 1u : 0u;
+    const unsigned q_stage = q_full_ok ? 2 * q_bytes : q_bytes;
+    const unsigned lds_bytes = use_lds ? static_cast<unsigned>(std::max<size_t>(lds_plane, q_stage)) : q_stage;
     // a workgroup stages its queries once, so it should walk many spans; the longest task is still cut into
     // enough chunks that about 2048 workgroups exist
     const unsigned max_spans = (max_tiles + span_tiles - 1) / span_tiles;
@@ -766,7 +850,7 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), seg_off, seg_len, static_cast<unsigned>(kv_heads),                     \
         static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, ws_max, ws_part,                   \
-        static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset
+        static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset, q_full_ok
 #define UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, LDS)                                                                        \
     do {                                                                                                             \
         if (lds_bytes > 48u * 1024u) {                                                                               \
