@@ -30,7 +30,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-KVSTAR_TRAFFIC = None   # HBM bytes per step of the KVStar leg at its defaults (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE)
+KVSTAR_TRAFFIC = 4088600000   # HBM bytes per step of the KVStar leg at its defaults (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE)
 
 N_REQ, N_LAYERS, HQ, HKV, D, BS = 16, 32, 32, 8, 128, 128
 ROW = HKV * D
@@ -378,12 +378,16 @@ def main():
         if not args.no_check:
             import oracle  # checker only
 
+            kv_cpu_s, kv_cpu_blocks = 0.0, 0
             for t_ in (0, n_tasks // 2 + 3, n_tasks - 1):
                 a_, n_ = int(k_off[t_]), int(k_len[t_])
                 rep_ref = ops.kvstar_table_to_reference(flat[:, a_ : a_ + n_]).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
                 pr_ = None if kpr is None else kpr[t_ // N_REQ].cpu().numpy().astype(np.int32)
-                _, want = oracle.kvstar_retrieve(kq[t_].view(torch.int16).cpu().numpy().view(np.uint16), rep_ref,
-                                                 int(topk[t_ % N_REQ]), pruned=pr_, d_pruned=kdp)
+                q_ref = kq[t_].view(torch.int16).cpu().numpy().view(np.uint16)
+                t0_ = time.perf_counter()
+                _, want = oracle.kvstar_retrieve(q_ref, rep_ref, int(topk[t_ % N_REQ]), pruned=pr_, d_pruned=kdp)
+                kv_cpu_s += time.perf_counter() - t0_
+                kv_cpu_blocks += n_
                 got = kvotes[a_ : a_ + n_].cpu().numpy()
                 assert np.allclose(got, want, rtol=2e-4, atol=2e-6), "KVStar votes differ from the CPU oracle"
             kv_checked = "votes of 3 sampled tasks within rtol 2e-4 / atol 2e-6 of the CPU oracle (fp32, other summation order)"
@@ -399,6 +403,10 @@ def main():
                          "algorithmic_bytes": kv_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * kd_pad / (kv_ms * 1e-3) / 1e12, 1)},
             "checked": kv_checked,
+            "cpu_port": None if kv_checked is None else {
+                "value": round(kv_cpu_s / kv_cpu_blocks * int(k_len.sum()) * 1e6, 1), "unit": "us/step", "cores": 1, "kind": "port",
+                "sample": f"the scalar C restatement on the 3 checked tasks ({kv_cpu_blocks} of {int(k_len.sum())} (block, layer) "
+                          f"pairs), scaled by blocks"},
         }
         del ktab, flat, kws, kpr
 

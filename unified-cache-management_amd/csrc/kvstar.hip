@@ -192,6 +192,19 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     }
 }
 
+// The two halves of a wave hold the two halves of every query row's tile: one v_permlane32_swap hands each
+// lane its own and its partner's value (lower half's first), without a trip through LDS.
+__device__ __forceinline__ float halves_max(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // kM here: sub-blocks per part (a block, or a tile's share of a bigger block; at most 32).
 // Hands the per-block sums of a tile's 32 exponentials for this lane's row to put(block within the tile,
 // sum) and returns their total (both lane halves included).  put is called unconditionally by all 64 lanes:
@@ -213,7 +226,7 @@ __device__ __forceinline__ float block_sums(const float (&e)[16], int half, Put 
             float v = 0.0f;
 #pragma unroll
             for (int g = 0; g < kGroups; ++g) { v += p4[b * kGroups + g]; }
-            sum[b] = v + __shfl_xor(v, 32, 64);          // both halves now hold the block's sum
+            sum[b] = halves_sum(v);                      // both halves now hold the block's sum
             total += sum[b];
         }
         if constexpr (kBlocks == 1) {
@@ -240,7 +253,7 @@ __device__ __forceinline__ float block_sums(const float (&e)[16], int half, Put 
             for (int i = 0; i < 16; ++i) { put(static_cast<unsigned>((i >> 2) * 8 + half * 4 + (i & 3)), e[i]); }
         }
         float total = (p4[0] + p4[1]) + (p4[2] + p4[3]);
-        total += __shfl_xor(total, 32, 64);
+        total = halves_sum(total);
         return total;
     }
 }
@@ -449,7 +462,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 #pragma unroll
                 for (int i = 3; i < 15; i += 2) { mx = fmaxf(fmaxf(mx, sc[i]), sc[i + 1]); }
                 mx = fmaxf(mx, sc[15]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));  // a live tile has at least one live sub-block, so mx is finite
+                mx = halves_max(mx);                      // a live tile has at least one live sub-block, so mx is finite
                 const float nmx = -mx * kLog2e;
                 float e[16];
 #pragma unroll
