@@ -132,6 +132,27 @@ def test_kvstar_many_short_tasks_take_the_in_lds_path(ucm, dev):
         assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
 
 
+@pytest.mark.parametrize("longest", [1200, 1400])
+def test_kvstar_long_task_plane_in_lds_or_not(ucm, dev, longest):
+    """1200 blocks x 32 rows is a 150 KiB plane: the in-LDS path at its largest; 1400 blocks do not fit, and the
+    request for the in-LDS path falls back to the workspace path."""
+    from ucm_amd import ops
+
+    x, hq, hkv, d, M = 8, 8, 2, 128, 8
+    lens = [longest, 5]
+    rows = int(np.sum(lens))
+    repre = f16_bits(synth.normal_f32(1160, (rows, M, hkv, d)) * np.float32(0.25))
+    qs = [f16_bits(synth.normal_f32(1161 + t, (x, hq, d)) * np.float32(0.25)) for t in range(2)]
+    ops.set_kvstar_tiles_per_wave(-1)
+    try:
+        got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
+    finally:
+        ops.set_kvstar_tiles_per_wave(0)
+    for t, n in enumerate(lens):
+        want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=1)[1]
+        assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
+
+
 @pytest.mark.parametrize("M,dp", [(8, 77), (64, 32)])          # 77 kept channels: table rows padded to 80; 64 / 32: the reference's defaults
 @pytest.mark.parametrize("tiles_per_wave", [0, -1])
 def test_kvstar_pruned_channels_and_selection(ucm, dev, tiles_per_wave, M, dp):
