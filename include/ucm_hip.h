@@ -325,6 +325,19 @@ int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int 
                      int n_tasks, int max_blocks,
                      int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                      float* ws_part, float* votes, ucm_stream_t stream);
+/* The same for tasks whose representatives do not share one table (the
+ * reference keeps one blk_repre tensor per request and layer,
+ * ucm/sparse/kvstar/multistep.py:191,483-501): task t's table starts at
+ * task_tables[t] (dev array of n_tasks dev pointers, 16-byte aligned, laid out
+ * [kv_heads][rows][d_pad/8][sub_blocks][8] with its head planes
+ * task_head_strides[t] elements apart, a multiple of 8) and its block 0 is
+ * the table's row 0; seg_off only places the task's votes. */
+int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                            const int32_t* pruned, const int32_t* pruned_sel,
+                            const void* const* task_tables, const int64_t* task_head_strides,
+                            const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                            int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+                            float* ws_part, float* votes, ucm_stream_t stream);
 
 /*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched

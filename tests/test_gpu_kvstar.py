@@ -233,3 +233,43 @@ def test_kvstar_retrieve_module_surface(ucm, dev):
     bad = kvstar_retrieve.AsyncRetrieveByCPU(q[:, :6], blk, index, 3, 7, kvstar_retrieve.CPU)
     assert kvstar_retrieve.GetTaskResult(bad)["error"] == "Num_q_heads must be a divisible by num_kv_heads."
     assert kvstar_retrieve.GetTaskResult(123456) is None
+
+
+@pytest.mark.parametrize("ratio", [1.0, 0.25])
+def test_kvstar_retrieve_batch(ucm, dev, ratio):
+    """AsyncRetrieveBatch: the requests of a layer in one launch, each with a table (and channel list) of its own;
+    every task must return what AsyncRetrieveByCPU returns for it alone."""
+    from ucm_amd.sparse.kvstar import retrieve as kvstar_retrieve
+
+    hq, hkv, d, bs, nb, merge = 16, 4, 128, 32, 90, 2
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    k_cache = (torch.randn(nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+    order = [int(i) + 2 for i in synth.permutation(1500, nb - 2)]
+    lens, topks = [30, 1, 41, 7], [9, 1, 12, 7]
+    repres, indexes, qs, at = [], [], [], 0
+    for n in lens:
+        r, i = kvstar_retrieve.extract_block_repre(k_cache, order[at : at + n], merge, prune_ratio=ratio, prune_dim_enable=True)
+        at += n
+        repres.append(r)
+        indexes.append(i)
+        qs.append((torch.randn(8, hq, d, device=dev, generator=g) * 0.3).to(torch.float16))
+    tids = kvstar_retrieve.AsyncRetrieveBatch(qs, repres, indexes, topks)
+    assert len(tids) == len(lens)
+    for t, tid in enumerate(tids):
+        kvstar_retrieve.Wait(tid)
+        got = kvstar_retrieve.GetTaskResult(tid)
+        alone = kvstar_retrieve.AsyncRetrieveByCPU(qs[t], repres[t], indexes[t], topks[t], t, kvstar_retrieve.CPU)
+        kvstar_retrieve.Wait(alone)
+        want = kvstar_retrieve.GetTaskResult(alone)
+        assert got["status"] == "SUCCESS" and len(got["data"]) == min(topks[t], lens[t])
+        dp = repres[t].shape[3]
+        pr = None if indexes[t] is None else indexes[t].cpu().numpy().astype(np.int32)
+        padded = np.zeros((lens[t], bs // merge, hkv, (dp + 15) // 16 * 16), np.uint16)
+        padded[..., :dp] = repres[t].dense().view(torch.int16).cpu().numpy().view(np.uint16)
+        _, votes = O.kvstar_retrieve(qs[t].view(torch.int16).cpu().numpy().view(np.uint16), padded, topks[t], pruned=pr, d_pruned=dp)
+        check_selection(got["data"], votes, topks[t])
+        check_selection(want["data"], votes, topks[t])
+    bad = kvstar_retrieve.AsyncRetrieveBatch(qs[:2], [repres[0], repres[1].dense()], indexes[:2], topks[:2])
+    assert kvstar_retrieve.GetTaskResult(bad[1])["status"] == "FAILURE"
+    assert kvstar_retrieve.AsyncRetrieveBatch([], [], [], []) == []

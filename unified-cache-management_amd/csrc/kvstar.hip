@@ -284,7 +284,8 @@ template <int kM, int kSteps, bool kTwoRowTiles, bool kLds>
 __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const unsigned short* __restrict__ q, const int64_t* __restrict__ q_off, unsigned n_tokens, unsigned q_heads,
     unsigned d_orig, const int32_t* __restrict__ pruned, const int32_t* __restrict__ pruned_sel,
-    const unsigned short* __restrict__ table, const int32_t* __restrict__ seg_off,
+    const unsigned short* __restrict__ table, const void* const* __restrict__ task_tables,
+    const int64_t* __restrict__ task_head_strides, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
     float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
     unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset, unsigned q_full_ok)
@@ -322,8 +323,11 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = lane >> 5, lr = lane & 31;
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes piece 2*ks + half
-    const unsigned short* tbase = table + static_cast<int64_t>(h) * head_stride +
-                                  static_cast<size_t>(seg_off[task]) * kM * d_pad + half * (8 * kM);
+    // the task's first representative: rows seg_off[task].. of the one table, or a table of the task's own
+    const unsigned short* tbase =
+        (task_tables ? static_cast<const unsigned short*>(task_tables[task]) + static_cast<int64_t>(h) * task_head_strides[task]
+                     : table + static_cast<int64_t>(h) * head_stride + static_cast<size_t>(seg_off[task]) * kM * d_pad) +
+        half * (8 * kM);
 
     // A span's keys: for each of its tiles, kSteps 16-byte loads per lane, piece 2*ks + half of the lane's
     // sub-block; the lanes of one instruction cover M*16 contiguous bytes per block and lane half.
@@ -802,16 +806,17 @@ extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_p
     return UCM_OK;
 }
 
-extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
-                                const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                                int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
-                                int max_blocks,
-                                int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, float* ws_part,
-                                float* votes, ucm_stream_t stream)
+namespace {
+int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
+                 const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, const void* const* task_tables,
+                 const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                 int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, float* ws_part, float* votes,
+                 ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks >= 0 && max_blocks >= 0, "ucm_kvstar_votes: n_tasks=%d max_blocks=%d", n_tasks, max_blocks);
     if (n_tasks == 0 || max_blocks == 0) { return UCM_OK; }
-    UCM_REQUIRE(q_f16 && q_off && repre_f16 && seg_off && seg_len && ws_max && ws_part && votes, "ucm_kvstar_votes: null pointer");
+    UCM_REQUIRE(q_f16 && q_off && seg_off && seg_len && ws_max && ws_part && votes, "ucm_kvstar_votes: null pointer");
+    UCM_REQUIRE(task_tables ? task_head_strides != nullptr : repre_f16 != nullptr, "ucm_kvstar_votes: no representative table");
     UCM_REQUIRE(n_tasks <= 65535, "ucm_kvstar_votes: n_tasks=%d", n_tasks);
     UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0, "ucm_kvstar_votes: q_heads=%d kv_heads=%d",
                 q_heads, kv_heads);
@@ -826,7 +831,7 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     UCM_REQUIRE(pruned_sel != nullptr || d_pruned == d_orig, "ucm_kvstar_votes: d_pruned < d_orig needs the channel lists");
     UCM_SUPPORTED(sub_blocks >= 1 && sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0,
                   "ucm_kvstar_votes: sub_blocks=%d (a power of two up to 128)", sub_blocks);
-    UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0,
+    UCM_REQUIRE(task_tables || (ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0),
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
     const unsigned max_tiles = static_cast<unsigned>(padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks));
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
@@ -861,7 +866,8 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
     hipStream_t s = ucm::as_stream(stream);
 #define UCM_KVSTAR_ARGS dim3(chunks, kv_heads, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
-        static_cast<const unsigned short*>(repre_f16), seg_off, seg_len, static_cast<unsigned>(kv_heads),                     \
+        static_cast<const unsigned short*>(repre_f16), task_tables, task_head_strides, seg_off, seg_len,                      \
+        static_cast<unsigned>(kv_heads),                                                                                      \
         static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, ws_max, ws_part,                   \
         static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset, q_full_ok
 #define UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, LDS)                                                                        \
@@ -915,4 +921,26 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
                            static_cast<unsigned>(max_blocks), max_tiles, row_pad, votes);
     }
     UCM_LAUNCH_CHECK("ucm_kvstar_votes");
+}
+}  // namespace
+
+extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                                const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
+                                int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                                int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+                                float* ws_part, float* votes, ucm_stream_t stream)
+{
+    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, repre_f16, repre_head_stride, nullptr, nullptr,
+                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_part, votes, stream);
+}
+
+extern "C" int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                                       const int32_t* pruned, const int32_t* pruned_sel, const void* const* task_tables,
+                                       const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len,
+                                       int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad,
+                                       float* ws_max, float* ws_part, float* votes, ucm_stream_t stream)
+{
+    UCM_REQUIRE(n_tasks == 0 || (task_tables && task_head_strides), "ucm_kvstar_votes_tables: null table list");
+    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, nullptr, 0, task_tables, task_head_strides,
+                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_part, votes, stream);
 }

@@ -383,6 +383,43 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
               _dev(votes, torch.float32, "votes"), _stream())
 
 
+def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: int, tables, seg_off: torch.Tensor,
+                        seg_len: torch.Tensor, max_blocks: int, votes: torch.Tensor, workspace: tuple,
+                        d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
+                        pruned_sel: Optional[torch.Tensor] = None):
+    """kvstar_votes for tasks that each bring a table of their own: tables[t] fp16 [kv_heads, rows_t, d_pad/8, M, 8]
+    (block 0 of task t = its row 0); seg_off only places the votes.  Returns the pointer arrays, which the
+    caller keeps alive until the stream has run the call."""
+    n_tasks = len(tables)
+    if n_tasks == 0:
+        return None
+    kv_heads, _, pieces, m, _ = tables[0].shape
+    for t in tables:
+        if t.dim() != 5 or t.dtype != torch.float16 or not t.is_cuda or t.shape[0] != kv_heads or t.shape[2:] != tables[0].shape[2:]:
+            raise ValueError("every table must be a float16 device tensor [kv_heads, rows, d_pad/8, M, 8] of the same M and d_pad")
+        if t.shape[1] and not t[0].is_contiguous():
+            raise ValueError("table rows must be dense inside each head plane")
+    d_orig = q.shape[-1]
+    if seg_off.numel() != n_tasks or seg_len.numel() != n_tasks or q_off.numel() != n_tasks:
+        raise ValueError("q_off / seg_off / seg_len / tables differ in length")
+    if pruned is not None:
+        if pruned.dim() != 3 or pruned.shape[1] != kv_heads or pruned_sel is None or pruned_sel.numel() != n_tasks:
+            raise ValueError("pruned must be [n_lists, kv_heads, d_pruned] with one pruned_sel entry per task")
+        d_pruned = pruned.shape[2]
+    elif d_pruned is None:
+        d_pruned = d_orig
+    host = torch.tensor([[t.data_ptr() for t in tables],
+                         [t.stride(0) if kv_heads > 1 else max(t[0].numel(), 8) for t in tables]], dtype=torch.int64).pin_memory()
+    dev = host.to(tables[0].device, non_blocking=True)
+    ws_max, ws_part = workspace
+    _lib.call("ucm_kvstar_votes_tables", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
+              _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
+              _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
+              d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), _dev(ws_part, torch.float32, "ws_part"),
+              _dev(votes, torch.float32, "votes"), _stream())
+    return host, dev
+
+
 def set_score_tile(tile_blocks: int) -> None:
     _lib.call("ucm_set_score_tile", tile_blocks)
 

@@ -48,7 +48,31 @@ DEFAULTS = {
     "retrieval_stride": 8,
     "blk_repre_dim_prune_ratio": 0.25,
     "blk_repre_inner_token_merge": 2,
+    "batch_retrieval": True,      # not in the reference: one launch per layer for all requests that retrieve in a step
 }
+
+
+class _RetrievalBatch:
+    """The retrievals the requests of one layer queue during one attention_begin, launched together."""
+
+    def __init__(self):
+        self.entries = []     # (state, record, query group fp16 [x, H, d], topk)
+        self.after = []       # what the states still have to do once their tasks exist
+
+    def flush(self) -> None:
+        groups: Dict[tuple, list] = {}
+        for e in self.entries:
+            state, _, qg, _ = e
+            groups.setdefault((tuple(qg.shape), state.d_pruned_index is None, tuple(state.blk_repre.shape[1:])), []).append(e)
+        for members in groups.values():
+            ids = kvstar_retrieve.AsyncRetrieveBatch(
+                [qg for _, _, qg, _ in members], [st.blk_repre for st, _, _, _ in members],
+                [st.d_pruned_index for st, _, _, _ in members], [k for _, _, _, k in members])
+            for (st, record, _, _), task_id in zip(members, ids):
+                st.task_waiter[record] = task_id
+        for fn in self.after:
+            fn()
+        self.entries, self.after = [], []
 
 
 class ReqStage(enum.Enum):
@@ -163,8 +187,9 @@ class ReqPerLayerState:
     def get_retrieve_record(self, cur_step: int) -> str:
         return "prefill" if cur_step == 1 else "decode" + str(cur_step - self.sparse_cfg["retrieval_stride"])
 
-    def retrieval_async(self, cur_step: int, topk: int, retrieve_device: str = "cpu") -> None:
-        """Queues the vote of one query group over the request's representatives (multistep.py:240-268)."""
+    def retrieval_async(self, cur_step: int, topk: int, retrieve_device: str = "cpu", batch: Optional[_RetrievalBatch] = None) -> None:
+        """Queues the vote of one query group over the request's representatives (multistep.py:240-268); with
+        ``batch`` the task is only listed, and launched with the layer's other requests."""
         record = self.get_retrieve_record(cur_step)
         if topk == 0:
             self.step_group_retrieve_result[record] = []
@@ -172,6 +197,9 @@ class ReqPerLayerState:
             return
         group = [x for x in self.standby_query_group[record] if x is not None]
         self.do_retrieve_query_group[record] = torch.stack(group).to(torch.float16).contiguous()
+        if batch is not None:
+            batch.entries.append((self, record, self.do_retrieve_query_group[record], topk))
+            return
         self.task_waiter[record] = kvstar_retrieve.AsyncRetrieveByCPU(
             self.do_retrieve_query_group[record], self.blk_repre, self.d_pruned_index, topk,
             hash(self.req_meta.request_id) & 0x7FFFFFFF, kvstar_retrieve.CPU)
@@ -264,7 +292,7 @@ class ReqPerLayerState:
         self.construct_init_and_local_window()
 
     # ---- hooks ---------------------------------------------------------------------------
-    def attention_begin(self, query, key, value, forward_context) -> None:
+    def attention_begin(self, query, key, value, forward_context, batch: Optional[_RetrievalBatch] = None) -> None:
         meta = self.req_meta
         if meta.stage == ReqStage.PREFILL:
             self.offload_prefill_query(query, meta.query_len, meta.query_start_loc)
@@ -275,16 +303,18 @@ class ReqPerLayerState:
         stride = self.sparse_cfg["retrieval_stride"]
         group_record, place = self.get_decode_step_record()
         self.save_to_standby(group_record, place, meta.query_start_loc, query)
+        later = (lambda fn: fn()) if batch is None else batch.after.append   # with a batch: once the tasks exist
         if meta.step % stride == 0:
-            self.retrieval_async(meta.step + 1, len(self.get_retrieve_candidate_block_ids()))
+            self.retrieval_async(meta.step + 1, len(self.get_retrieve_candidate_block_ids()), batch=batch)
         if meta.step == 1:
             self.prepare_init_and_local_window()
             candidates = self.get_retrieve_candidate_block_ids()
             self.wait_for_blk_transfer_task_done()
-            self.retrieval_async(meta.step, len(candidates))
-            self.load_retrieve_result_async(meta.step, candidates)
+            self.retrieval_async(meta.step, len(candidates), batch=batch)
+            step = meta.step
+            later(lambda: self.load_retrieve_result_async(step, candidates))
         if meta.step % stride == 1:
-            self.wait_for_blk_transfer_task_done()
+            later(self.wait_for_blk_transfer_task_done)
 
     def attention_finished(self, query, key, value, attn_output, forward_context) -> None:
         meta = self.req_meta
@@ -380,10 +410,13 @@ class KVStarMultiStep(UcmSparseBase):
         self.req_states.pop(request_id, None)
 
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        batch = _RetrievalBatch() if self.kvstar_multistep_cfg["batch_retrieval"] else None
         for req_meta in self._sparse_metadata.requests:
             state = self.create_layerwise_req_state(req_meta, layer_name)
             state.update_meta(req_meta, forward_context)
-            state.attention_begin(query, key, value, forward_context)
+            state.attention_begin(query, key, value, forward_context, batch=batch)
+        if batch is not None:
+            batch.flush()
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
         for req_meta in self._sparse_metadata.requests:

@@ -54,9 +54,9 @@ class SetupParam:
 @dataclass
 class _Task:
     event: Optional[torch.cuda.Event]
-    votes: Optional[torch.Tensor]
-    idx: Optional[torch.Tensor]
-    cnt: Optional[torch.Tensor]
+    votes: Optional[torch.Tensor]       # this task's votes, one per block
+    idx: Optional[torch.Tensor]         # its selected blocks, ascending
+    cnt: Optional[torch.Tensor]         # how many of them
     keep: tuple = ()
     error: Optional[str] = None
 
@@ -156,12 +156,79 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
                 keep += (seg_off, seg_len, ws)
             event = torch.cuda.Event()
             event.record(_stream)
-        task = _Task(event, votes, idx, cnt, keep)
+        task = _Task(event, votes, idx[0, 0], cnt[0, 0], keep)
     except RuntimeError as e:
         task = _Task(None, None, None, None, error=str(e))
     with _lock:
         _tasks[task_id] = task
     return task_id
+
+
+def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_ids=None, device_type: DeviceType = CPU) -> List[int]:  # noqa: N802
+    """Several retrievals (the requests of one layer) in one launch; returns one task id per entry, to be used
+    with Wait / GetTaskResult like those of AsyncRetrieveByCPU.  Every entry must have the same number of query
+    tokens, heads and kept channels, and a BlockRepre (extract_block_repre's result) as representatives."""
+    global _stream
+    if _stream is None:
+        _stream = torch.cuda.Stream()
+    n_tasks = len(query_groups)
+    if n_tasks == 0:
+        return []
+    ids = [next(_ids) for _ in range(n_tasks)]
+    try:
+        q0, r0 = query_groups[0], blk_repres[0]
+        if any(not isinstance(r, BlockRepre) for r in blk_repres):
+            raise RuntimeError("AsyncRetrieveBatch takes BlockRepre representatives")
+        x, hq, d_orig = q0.shape
+        _, m, h, dp = r0.shape
+        for qg, r in zip(query_groups, blk_repres):
+            if tuple(qg.shape) != (x, hq, d_orig) or tuple(r.shape[1:]) != (m, h, dp) or qg.dtype != torch.float16:
+                raise RuntimeError("the entries of a batch must agree in query tokens, heads, sub-blocks and kept channels")
+        if hq % h != 0:
+            raise RuntimeError("Num_q_heads must be a divisible by num_kv_heads.")
+        with_lists = d_pruned_indexes is not None and any(i is not None for i in d_pruned_indexes)
+        if with_lists:
+            if any(i is None or tuple(i.shape) != (h, dp) for i in d_pruned_indexes):
+                raise RuntimeError("dPrunedIndex shape is inconsistent with K's shape.")
+        elif d_orig != dp:
+            raise RuntimeError("Dimension mismatch: No dPrunedIndex, but Q and K head dims differ.")
+        dev = r0.device
+        lens = [int(r.shape[0]) for r in blk_repres]
+        offs = [0]
+        for n in lens[:-1]:
+            offs.append(offs[-1] + n)
+        total, longest = sum(lens), max(lens)
+        ready = torch.cuda.Event()
+        ready.record()
+        with torch.cuda.stream(_stream):
+            _stream.wait_event(ready)
+            q = torch.stack([qg.contiguous() for qg in query_groups])
+            pruned = sel = None
+            if with_lists:
+                pruned = torch.stack([i.to(device=dev, dtype=torch.int32) for i in d_pruned_indexes]).contiguous()
+                sel = torch.arange(n_tasks, dtype=torch.int32, device=dev)
+            meta = torch.tensor([offs, lens, [min(int(k), n) for k, n in zip(topks, lens)]], dtype=torch.int32).pin_memory()
+            meta_d = meta.to(dev, non_blocking=True)
+            q_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (x * hq * d_orig)
+            votes = torch.zeros(max(total, 1), dtype=torch.float32, device=dev)
+            idx = torch.zeros((1, n_tasks, max(longest, 1)), dtype=torch.int32, device=dev)
+            cnt = torch.zeros((1, n_tasks), dtype=torch.int32, device=dev)
+            keep = (q, pruned, sel, meta, meta_d, q_off, tuple(r.table for r in blk_repres))
+            if longest > 0:
+                ws = ops.kvstar_workspace(n_tasks, h, x * (hq // h), longest, m, dev)
+                ptrs = ops.kvstar_votes_tables(q, q_off, x, hq, [r.table for r in blk_repres], meta_d[0], meta_d[1], longest, votes, ws,
+                                               d_pruned=dp, pruned=pruned, pruned_sel=sel)
+                ops.topk_windows(votes.view(1, -1), meta_d[0], meta_d[1], meta_d[2], longest, idx, cnt, start_w=0, end_w=0)
+                keep += (ws, ptrs)
+            event = torch.cuda.Event()
+            event.record(_stream)
+        tasks = [_Task(event, votes[offs[i] : offs[i] + lens[i]], idx[0, i], cnt[0, i], keep) for i in range(n_tasks)]
+    except RuntimeError as e:
+        tasks = [_Task(None, None, None, None, error=str(e)) for _ in range(n_tasks)]
+    with _lock:
+        for i, t in zip(ids, tasks):
+            _tasks[i] = t
+    return ids
 
 
 def Wait(task_id: int) -> None:  # noqa: N802
@@ -180,8 +247,8 @@ def GetTaskResult(task_id: int):  # noqa: N802
         return {"status": "FAILURE", "error": task.error}
     if not task.event.query():
         return {"status": "RUNNING"}
-    n = int(task.cnt[0, 0])
-    chosen = task.idx[0, 0, :n].long()
+    n = int(task.cnt)
+    chosen = task.idx[:n].long()
     order = torch.argsort(task.votes[chosen], descending=True, stable=True)   # chosen is ascending: ties keep the lower index first
     task.keep = ()
     return {"status": "SUCCESS", "data": chosen[order].tolist()}
