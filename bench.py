@@ -512,7 +512,8 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 keys/queries, fp32 scores, u8 block bytes",
+        "dtype": "f32",
+        "dtype_detail": "bf16 keys and queries, scores accumulated and compared in fp32, KV blocks moved as bytes",
         "data": "synthetic (seeded N(0,1) bf16 keys, values and queries; random block table)",
         "config": {
             "workload": "configs[1]: ragged batch of 16 requests, 4096-65536 tokens, Llama-3-8B attention shape, "
