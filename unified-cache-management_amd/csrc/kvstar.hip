@@ -335,11 +335,12 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     // query fragment, lanes and tiles past the workgroup's end reload its last vector and are masked or
     // never used.
     //
-    // Three key buffers rotate, so two spans are in flight while one is worked on.  The loads and the waits
-    // for them are written as assembly: left to itself the compiler sinks a prefetch down to the span that
-    // consumes it (there is nothing but a loop exit in between), which leaves nothing in flight.  Vector
-    // memory operations complete in issue order, loads and stores alike, so "the loads of span t have
-    // landed" is "at most as many operations outstanding as were issued after them".
+    // Three key buffers rotate, so two spans are in flight while one is worked on.  Every group of loads is
+    // followed by a compiler barrier (an empty asm that may touch memory): left to itself the compiler sinks
+    // a prefetch down to the span that consumes it - nothing but a loop exit lies between - and then nothing
+    // is in flight.  The waits are the compiler's own: vector memory operations complete in issue order,
+    // loads and stores alike, so it waits for "at most as many operations outstanding as were issued after
+    // the loads of this span" - which only works because no store below is skipped on any path.
     auto load_keys = [&](u32x4 (&kf)[kLoads], unsigned s0) {
 #pragma unroll
         for (int t = 0; t < kSpanTiles; ++t) {
@@ -347,10 +348,10 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
             const unsigned short* krow = tbase + static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
 #pragma unroll
             for (int ks = 0; ks < kSteps; ++ks) {
-                const unsigned short* p = krow + (static_cast<unsigned>(ks) < ksteps ? ks : 0) * (16 * kM);
-                asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(kf[t * kSteps + ks]) : "v"(p) : "memory");
+                kf[t * kSteps + ks] = ucm::gload16(krow + (static_cast<unsigned>(ks) < ksteps ? ks : 0) * (16 * kM));
             }
         }
+        asm volatile("" ::: "memory");
     };
     u32x4 k0[kLoads], k1[kLoads], k2[kLoads];
     const unsigned s_first = s_chunk + wave * kSpan;
@@ -513,49 +514,19 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
         }
     };
 
-    // Operations issued after a span's loads when the wave turns to it: the loads of the two spans behind it
-    // (16) and the stores of the spans worked on since - none for the wave's first span, one span's for its
-    // second, two spans' from then on.
-    constexpr unsigned kStores =
-        kLds ? 0 : kSpanTiles * kRowTiles * (1 + (kTilePart >= 16 ? 1 : kTilePart == 8 ? 2 : kTilePart == 4 ? 4 : kTilePart == 2 ? 8 : 16));
-    constexpr unsigned kAfter0 = 2 * kLoads, kAfter1 = kAfter0 + kStores > 63 ? 63 : kAfter0 + kStores,
-                       kAfter2 = kAfter0 + 2 * kStores > 63 ? 63 : kAfter0 + 2 * kStores;
-#define UCM_KEYS_LANDED(k, n)                                                                                              \
-    asm volatile("s_waitcnt vmcnt(%8)"                                                                                     \
-                 : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]), "+v"(k[4]), "+v"(k[5]), "+v"(k[6]), "+v"(k[7])         \
-                 : "n"(n)                                                                                                  \
-                 : "memory")
-    unsigned s0 = s_first;
-    if (s0 < s_end) {                                    // the wave's first two spans, with fewer stores behind them
-        UCM_KEYS_LANDED(k0, kAfter0);
-        process(k0, s0);
-        load_keys(k0, s0 + 3 * kStride);
-        s0 += kStride;
-        if (s0 < s_end) {
-            UCM_KEYS_LANDED(k1, kAfter1);
-            process(k1, s0);
-            load_keys(k1, s0 + 3 * kStride);
-            s0 += kStride;
-        }
-    }
-    while (s0 < s_end) {                                 // buffers k2, k0, k1, k2, ... from here on
-        UCM_KEYS_LANDED(k2, kAfter2);
-        process(k2, s0);
-        load_keys(k2, s0 + 3 * kStride);
-        s0 += kStride;
-        if (s0 >= s_end) { break; }
-        UCM_KEYS_LANDED(k0, kAfter2);
+    for (unsigned s0 = s_first; s0 < s_end;) {
         process(k0, s0);
         load_keys(k0, s0 + 3 * kStride);
         s0 += kStride;
         if (s0 >= s_end) { break; }
-        UCM_KEYS_LANDED(k1, kAfter2);
         process(k1, s0);
         load_keys(k1, s0 + 3 * kStride);
         s0 += kStride;
+        if (s0 >= s_end) { break; }
+        process(k2, s0);
+        load_keys(k2, s0 + 3 * kStride);
+        s0 += kStride;
     }
-#undef UCM_KEYS_LANDED
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the prefetches past the end: nothing stays in flight
 
     if constexpr (kLds) {
         // ---- this head's share of the votes, from the plane in LDS
