@@ -354,7 +354,7 @@ def main():
         kq_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (kx * HQ * D)
         ksel = None if kpr is None else torch.arange(n_layers, dtype=torch.int32, device=dev).repeat_interleave(N_REQ)
         kvotes = torch.zeros(n_layers * rows, device=dev)
-        kws = ops.kvstar_workspace(n_tasks, HKV, kx * HQ // HKV, max_len, km, dev)
+        kws = ops.kvstar_workspace(n_tasks, HKV, kx * HQ // HKV, max_len, km, kd_pad, dev)
         kso, ksl = i32(k_off), i32(k_len)
         ktk = i32(np.tile(topk, n_layers))
         kidx = torch.zeros((1, n_tasks, max_len), dtype=torch.int32, device=dev)

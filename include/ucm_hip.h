@@ -317,8 +317,12 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
  * in-LDS path whenever the plane fits; 0: automatic.  Not part of the
  * reference interface. */
 int ucm_set_kvstar_tiles_per_wave(int tiles);
+/* Floats of scratch ucm_kvstar_votes[_tables] needs for a call of this shape
+ * (rows_per_head = n_tokens * q_heads/kv_heads); the in-LDS path only needs
+ * room for the kv heads' vote shares.  Ask after ucm_set_kvstar_tiles_per_wave,
+ * which changes the path. */
 int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks,
-                                int sub_blocks, int64_t* max_floats, int64_t* part_floats);
+                                int sub_blocks, int d_pad, int64_t* max_floats, int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                      const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
                      int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len,

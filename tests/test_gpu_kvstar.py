@@ -78,7 +78,7 @@ def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None
     table = ops.kvstar_table_from_reference(dev_f16(repre_bits, dev))                 # the kernels' order: [h, rows, d_pad/8, M, 8]
     assert torch.equal(ops.kvstar_table_to_reference(table), dev_f16(repre_bits, dev))
     votes = torch.full((rows,), -7.0, device=dev)
-    ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, dev)
+    ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, table.shape[2] * 8, dev)
     ops.kvstar_votes(q, q_off, n_tokens, hq, table, torch.from_numpy(off).to(dev), torch.from_numpy(lens).to(dev),
                      int(lens.max(initial=0)), votes, ws, d_pruned=d_pruned,
                      pruned=None if pruned is None else torch.from_numpy(pruned).to(dev),

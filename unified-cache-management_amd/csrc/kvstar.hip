@@ -752,6 +752,7 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
 }
 
+
 namespace {
 // Tiles the planes are sized for: a wave works in spans of up to four tiles and stores all of them
 int64_t padded_tiles(int64_t sub_blocks_total)
@@ -759,21 +760,55 @@ int64_t padded_tiles(int64_t sub_blocks_total)
     const int64_t tiles = (sub_blocks_total + kTileSub - 1) / kTileSub;
     return (tiles + 3) / 4 * 4;
 }
+
+// How one call is carried out: shared by the workspace sizing and the launch
+struct VotePlan {
+    unsigned max_tiles, row_pad, q_bytes, steps, span_tiles, plane_offset;
+    size_t lds_plane;
+    bool use_lds;
+};
+
+VotePlan plan_votes(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks, int d_pad)
+{
+    VotePlan p;
+    p.max_tiles = static_cast<unsigned>(std::max<int64_t>(padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks), 4));
+    p.row_pad = rows_per_head > 32 ? 64 : 32;
+    p.q_bytes = p.row_pad * kQStride * 2;
+    p.steps = d_pad <= 32 ? 2u : d_pad <= 64 ? 4u : 8u;        // MFMA steps per vector the kernel is built for
+    p.span_tiles = 8u / p.steps;                               // tiles a wave moves at a time
+    // One workgroup per (task, kv head) with the task's plane in LDS, when there are enough such workgroups to
+    // fill the device and the plane fits; otherwise the workspace path, which may cut a task into chunks.
+    // ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
+    p.plane_offset = rows_per_head > 32 ? p.q_bytes : 0u;
+    const unsigned entry_tiles = static_cast<unsigned>(sub_blocks) <= kTileSub
+                                     ? 1u : std::min<unsigned>(sub_blocks, p.span_tiles * kTileSub) / kTileSub;
+    const size_t plane_entries = static_cast<unsigned>(sub_blocks) < kTileSub
+                                     ? static_cast<size_t>(p.max_tiles) * (kTileSub / sub_blocks) : p.max_tiles / entry_tiles;
+    p.lds_plane = p.plane_offset + plane_entries * p.row_pad * 4 + 2 * kWaves * p.row_pad * 4;
+    p.use_lds = g_tiles_per_wave <= 0 && p.lds_plane <= kLdsPathMaxBytes &&
+                (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
+    return p;
+}
 }  // namespace
 
 extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks,
-                                           int64_t* max_floats, int64_t* part_floats)
+                                           int d_pad, int64_t* max_floats, int64_t* part_floats)
 {
     UCM_REQUIRE(n_tasks >= 0 && kv_heads > 0 && rows_per_head > 0 && rows_per_head <= kMaxRows && max_blocks >= 0 &&
-                    sub_blocks > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
-    const int64_t tiles = padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks);
-    const int64_t row_pad = rows_per_head > 32 ? 64 : 32;
+                    sub_blocks > 0 && d_pad > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
     UCM_REQUIRE(sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
+    const VotePlan p = plan_votes(n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad);
+    if (p.use_lds) {
+        // only the kv heads' shares of the votes pass through memory
+        *max_floats = 1;
+        *part_floats = std::max<int64_t>(static_cast<int64_t>(n_tasks) * kv_heads * max_blocks, 1);
+        return UCM_OK;
+    }
     // per (task, kv head): a (maximum, sum) pair per tile and row; a partial sum per row and block (per tile,
     // for blocks of more than 32 sub-blocks), padded to whole tiles
     const int64_t parts_per_tile = kTileSub / std::min(sub_blocks, kTileSub);
-    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * 2 * std::max<int64_t>(tiles, 1);
-    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * row_pad * parts_per_tile * std::max<int64_t>(tiles, 1);
+    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * p.row_pad * 2 * p.max_tiles;
+    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * p.row_pad * parts_per_tile * p.max_tiles;
     return UCM_OK;
 }
 
@@ -804,23 +839,12 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
                   "ucm_kvstar_votes: sub_blocks=%d (a power of two up to 128)", sub_blocks);
     UCM_REQUIRE(task_tables || (ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0),
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
-    const unsigned max_tiles = static_cast<unsigned>(padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks));
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
-    const unsigned row_pad = R > 32 ? 64 : 32;
-    const unsigned q_bytes = row_pad * kQStride * 2;
-    const unsigned steps = d_pad <= 32 ? 2u : d_pad <= 64 ? 4u : 8u;     // MFMA steps per vector the kernel is built for
-    const unsigned span_tiles = 8u / steps;                                // tiles a wave moves at a time
-    // One workgroup per (task, kv head) with the task's plane in LDS, when there are enough such workgroups to
-    // fill the device and the plane fits; otherwise the workspace path, which may cut a task into chunks.
-    // ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
-    const unsigned plane_offset = R > 32 ? q_bytes : 0u;
-    const unsigned entry_tiles = static_cast<unsigned>(sub_blocks) <= kTileSub
-                                     ? 1u : std::min<unsigned>(sub_blocks, span_tiles * kTileSub) / kTileSub;
-    const size_t plane_entries = static_cast<unsigned>(sub_blocks) < kTileSub
-                                     ? static_cast<size_t>(max_tiles) * (kTileSub / sub_blocks) : max_tiles / entry_tiles;
-    const size_t lds_plane = plane_offset + plane_entries * row_pad * 4 + 2 * kWaves * row_pad * 4;
-    const bool use_lds = g_tiles_per_wave <= 0 && lds_plane <= kLdsPathMaxBytes &&
-                         (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
+    const VotePlan plan = plan_votes(n_tasks, kv_heads, static_cast<int>(R), max_blocks, sub_blocks, d_pad);
+    const unsigned max_tiles = plan.max_tiles, row_pad = plan.row_pad, q_bytes = plan.q_bytes, steps = plan.steps,
+                   span_tiles = plan.span_tiles, plane_offset = plan.plane_offset;
+    const size_t lds_plane = plan.lds_plane;
+    const bool use_lds = plan.use_lds;
     // with channel lists, whole query rows are staged in a second area of q_bytes and gathered from there
     const unsigned q_full_ok = pruned != nullptr && d_orig % 8 == 0 && d_orig <= kMaxDim && ucm::aligned16(q_f16) ? 1u : 0u;
     const unsigned q_stage = q_full_ok ? 2 * q_bytes : q_bytes;

@@ -338,12 +338,14 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
               repre.shape[2], repre.stride(0), repre.stride(1), _stream())
 
 
-def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks: int, sub_blocks: int, device) -> tuple:
-    """Scratch of ucm_kvstar_votes; rows_per_head = query tokens * (q_heads / kv_heads)."""
+def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks: int, sub_blocks: int, d_pad: int,
+                     device) -> tuple:
+    """Scratch of ucm_kvstar_votes for a call of this shape; rows_per_head = query tokens * (q_heads / kv_heads),
+    d_pad = padded channels per representative (the table's d_pad)."""
     import ctypes as C
 
     a, b = C.c_int64(0), C.c_int64(0)
-    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, C.addressof(a),
+    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad, C.addressof(a),
               C.addressof(b))
     return (torch.empty(max(a.value, 1), dtype=torch.float32, device=device),
             torch.empty(max(b.value, 1), dtype=torch.float32, device=device))

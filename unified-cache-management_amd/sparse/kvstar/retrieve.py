@@ -148,7 +148,7 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
             if n > 0 and k > 0:
                 seg_off = torch.zeros(1, dtype=torch.int32, device=dev)
                 seg_len = torch.full((1,), n, dtype=torch.int32, device=dev)
-                ws = ops.kvstar_workspace(1, h, x * (hq // h), n, m, dev)
+                ws = ops.kvstar_workspace(1, h, x * (hq // h), n, m, table.shape[2] * 8, dev)
                 ops.kvstar_votes(q, torch.zeros(1, dtype=torch.int64, device=dev), x, hq, table, seg_off, seg_len, n, votes,
                                  ws, d_pruned=dp, pruned=pruned, pruned_sel=sel)
                 ops.topk_windows(votes.view(1, -1), seg_off, seg_len, torch.full((1,), k, dtype=torch.int32, device=dev), n,
@@ -215,7 +215,7 @@ def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_id
             cnt = torch.zeros((1, n_tasks), dtype=torch.int32, device=dev)
             keep = (q, pruned, sel, meta, meta_d, q_off, tuple(r.table for r in blk_repres))
             if longest > 0:
-                ws = ops.kvstar_workspace(n_tasks, h, x * (hq // h), longest, m, dev)
+                ws = ops.kvstar_workspace(n_tasks, h, x * (hq // h), longest, m, r0.table.shape[2] * 8, dev)
                 ptrs = ops.kvstar_votes_tables(q, q_off, x, hq, [r.table for r in blk_repres], meta_d[0], meta_d[1], longest, votes, ws,
                                                d_pruned=dp, pruned=pruned, pruned_sel=sel)
                 ops.topk_windows(votes.view(1, -1), meta_d[0], meta_d[1], meta_d[2], longest, idx, cnt, start_w=0, end_w=0)
