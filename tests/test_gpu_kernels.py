@@ -636,3 +636,64 @@ def test_delta_plan_and_delta_gather(ucm, dev):
         if step > 0:
             assert miss_h.sum() < cnt.sum()        # overlapping selections really save loads
         prev = sel
+
+
+def test_decode_step_under_graph_capture(ucm, dev):
+    """The step's three launches (scores, selection + block table, gather) allocate and synchronise nothing, so a
+    caller may capture them in a HIP graph: three replays with fresh queries, eager work and synchronisation in
+    between, each equal to the eager result for the same queries."""
+    from ucm_amd import ops
+
+    n_layers, hq, hkv, d, bs = 3, 32, 8, 128, 16
+    lens = np.array([40, 7, 25, 3], np.int32)
+    topk = np.array([19, 7, 19, 3], np.int32)
+    rows, nb = int(lens.sum()), int(lens.sum()) + 3
+    bb = bs * hkv * d * 2
+    caches = [randn_bf16(dev, 1700 + l, (2, nb, bs, hkv, d))[0] for l in range(n_layers)]
+    lp = ops.LayerPointers(caches)
+    table = synth.permutation(1710, nb)[:rows]
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    repre = torch.zeros(n_layers, rows, hkv * d, device=dev, dtype=torch.bfloat16)
+    ops.block_mean(lp, i32(table, dev), i32(np.arange(rows), dev), repre, bs, hkv, d, nb, mode=ops.MEAN_BF16_STORE)
+    bt = np.zeros((len(lens), int(lens.max())), np.int32)
+    for r, n in enumerate(lens):
+        bt[r, :n] = table[off[r] : off[r] + n]
+    mx, kmax = int(lens.max()), int(topk.max())
+    seg_off, seg_len, topk_d, bt_d = i32(off, dev), i32(lens, dev), i32(topk, dev), i32(bt, dev)
+    region = i32(topk, dev)
+    dst_off = torch.from_numpy(np.concatenate([[0], np.cumsum(topk.astype(np.int64) * n_layers * 2)[:-1]])).to(dev)
+    total = int((topk.astype(np.int64) * n_layers * 2).sum())
+
+    def buffers():
+        return (torch.full((n_layers, rows), -5.0, device=dev), torch.full((n_layers, len(lens), mx), -1, dtype=torch.int32, device=dev),
+                torch.full((n_layers, len(lens)), -1, dtype=torch.int32, device=dev),
+                torch.full((n_layers, len(lens), mx), -1, dtype=torch.int32, device=dev),
+                torch.full((total * bb,), 7, dtype=torch.uint8, device=dev))
+
+    def step(q, scores, idx, cnt, phys, staging):
+        ops.score_blocks(q, repre, seg_off, seg_len, mx, hkv, scores)
+        ops.topk_windows(scores, seg_off, seg_len, topk_d, mx, idx, cnt, block_tables=bt_d, phys_out=phys)
+        ops.kv_gather_selected(lp, nb * bb, bb, nb, phys, cnt, dst_off, region, kmax, staging, total)
+
+    q_static = torch.zeros(n_layers, len(lens), hq, d, device=dev, dtype=torch.bfloat16)
+    g_bufs = buffers()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(q_static, *g_bufs)                                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(q_static, *g_bufs)
+    for rep in range(3):
+        q = torch.from_numpy(synth.normal_bf16_as_f32(1720 + rep, (n_layers, len(lens), hq, d))).to(dev).to(torch.bfloat16)
+        e_bufs = buffers()
+        step(q, *e_bufs)                                          # eager, on the current stream
+        torch.cuda.synchronize()
+        q_static.copy_(q)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("scores", "idx", "cnt", "phys", "staging"), g_bufs, e_bufs):
+            assert torch.equal(a, b), (rep, name)
+        assert int(e_bufs[2].min()) > 0                           # something was selected for every request
