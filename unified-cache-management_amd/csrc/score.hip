@@ -295,9 +295,14 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(
                             static_cast<int64_t>(seg0) * row + h * kD + 8 * p;
     float* sout = scores + static_cast<int64_t>(l) * scores_layer_stride + seg0;
 
+    // Loads and the store below are unconditional (rows and the output index are clamped to the tile's last
+    // block, whose score is then written more than once): an operation skipped on some path would make the
+    // compiler wait for everything outstanding, the prefetch included.  The empty asm keeps the compiler from
+    // sinking a prefetch down to its use.
     int b0 = tile0 + wave * blocks_per_pass;
     u32x4 kv_a[kSteps], kv_b[kSteps];
-    if (b0 < tile_end) { load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row); }
+    load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row);
+    asm volatile("" ::: "memory");
 
     {
         const int g = q_heads / kv_heads;
@@ -326,16 +331,17 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(
             const float dh = __shfl(dot, (bl * kv_heads + hh) * 2, 64);
             s = s + fmaxf(-FLT_MAX, dh);
         }
-        const int b = base + bl;
-        if (b < tile_end && h == 0 && p == 0) { sout[b] = s; }
+        sout[min(base + bl, tile_end - 1)] = s;   // the lanes of a block all hold its score
     };
     while (b0 < tile_end) {
         const int b1 = b0 + stride;
-        if (b1 < tile_end) { load_pass_bf16<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row); }
+        load_pass_bf16<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row);
+        asm volatile("" ::: "memory");
         finish(kv_a, b0);
         if (b1 >= tile_end) { break; }
         const int b2 = b1 + stride;
-        if (b2 < tile_end) { load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row); }
+        load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row);
+        asm volatile("" ::: "memory");
         finish(kv_b, b1);
         b0 = b2;
     }
