@@ -8,7 +8,8 @@
  * enqueues its kernels on `stream` (a hipStream_t, NULL = the null stream) and
  * returns.  Return value: 0 on success, a negative errno-style code otherwise
  * (UCM_EINVAL bad argument, UCM_ENOTSUP shape outside what the kernels were
- * built for, UCM_EHIP a HIP runtime error); ucm_last_error() has the text.
+ * built for, UCM_EHIP a HIP runtime error, UCM_ENOMEM an allocation that was
+ * refused); ucm_last_error() has the text.
  *
  * Reference paths are relative to the upstream tree; each entry point names
  * the reference interface it stands in for.
@@ -42,6 +43,7 @@ extern "C" {
 #define UCM_EINVAL (-22)
 #define UCM_ENOTSUP (-95)
 #define UCM_EHIP (-5)
+#define UCM_ENOMEM (-12)
 
 #define UCM_DTYPE_F32 0
 #define UCM_DTYPE_BF16 1
@@ -352,6 +354,63 @@ int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_token
  */
 int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t size,
                    ucm_stream_t stream);
+
+/*
+ * Transfer device of the store layer: the HIP counterpart of the reference's
+ * IDevice (ucm/store/device/idevice.h:33-58) as implemented by CudaDevice on
+ * the buffered base (ucm/store/device/cuda/cuda_device.cu:107-227,
+ * ucm/store/device/ibuffered_device.h:32-66).  One object per GPU and user:
+ * it owns a stream of default priority, `buffer_number` pinned host buffers of
+ * `buffer_size` bytes each and the device scratch of the batched copies.
+ *
+ * ucm_device_create             Setup(): selects the device, allocates the pool
+ *                               and the stream (cuda_device.cu:113-125).
+ * ucm_device_get_buffer         GetBuffer(size): a free pool slot if size fits
+ *                               one and one is free, else a pinned buffer of its
+ *                               own (ibuffered_device.h:48-62); NULL on failure.
+ * ucm_device_release_buffer     what dropping the reference's shared_ptr does:
+ *                               the slot goes back to the pool, a buffer of its
+ *                               own is freed.
+ * ucm_device_h2d_sync/d2h_sync  H2DSync / D2HSync (cuda_device.cu:126-133).
+ * ucm_device_h2d_async/d2h_async  H2DAsync / D2HAsync on the object's stream
+ *                               (:134-141).
+ * ucm_device_append_callback    AppendCallback (:142-156): cb(ok, user) runs on
+ *                               a runtime thread once everything queued before it
+ *                               on the stream has finished; ok is 1 on success.
+ *                               The callback must not call this library.
+ * ucm_device_synchronized       Synchronized (:157-160): waits for the stream.
+ * ucm_device_h2d_batch_sync     H2DBatchSync (:180-195): `number` copies of
+ *                               `count` bytes, device dArr[i] <- host hArr[i].
+ * ucm_device_d2h_batch_sync     D2HBatchSync (:196-211): host hArr[i] <- device
+ *                               dArr[i].  Both arrays are HOST arrays of
+ *                               addresses (as in the reference); the host
+ *                               addresses must be pinned memory (this object's
+ *                               buffers are), every address and `count` a multiple
+ *                               of 16.  One launch of the ucm_copy_batch kernel on
+ *                               the object's stream, then a wait.
+ * ucm_device_stream             the object's stream, for callers that order
+ *                               their own kernels against the copies.
+ *
+ * Calls on one object may come from several threads; batched copies on one
+ * object run one at a time.
+ */
+typedef struct ucm_device ucm_device_t;
+typedef void (*ucm_device_callback_t)(int ok, void* user);
+int ucm_device_create(int device_id, size_t buffer_size, size_t buffer_number, ucm_device_t** out);
+void ucm_device_destroy(ucm_device_t* dev);
+void* ucm_device_get_buffer(ucm_device_t* dev, size_t size);
+void ucm_device_release_buffer(ucm_device_t* dev, void* buffer);
+int ucm_device_h2d_sync(ucm_device_t* dev, void* dst, const void* src, size_t count);
+int ucm_device_d2h_sync(ucm_device_t* dev, void* dst, const void* src, size_t count);
+int ucm_device_h2d_async(ucm_device_t* dev, void* dst, const void* src, size_t count);
+int ucm_device_d2h_async(ucm_device_t* dev, void* dst, const void* src, size_t count);
+int ucm_device_append_callback(ucm_device_t* dev, ucm_device_callback_t cb, void* user);
+int ucm_device_synchronized(ucm_device_t* dev);
+int ucm_device_h2d_batch_sync(ucm_device_t* dev, void* const* d_arr, const void* const* h_arr,
+                              size_t number, size_t count);
+int ucm_device_d2h_batch_sync(ucm_device_t* dev, void* const* h_arr, const void* const* d_arr,
+                              size_t number, size_t count);
+ucm_stream_t ucm_device_stream(ucm_device_t* dev);
 
 /*
  * Whole-block dump (cache -> staging) and load (staging -> cache) driven by a

@@ -7,7 +7,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libucm_hip.so")
 
-OK, EINVAL, ENOTSUP, EHIP = 0, -22, -95, -5
+OK, EINVAL, ENOTSUP, EHIP, ENOMEM = 0, -22, -95, -5, -12
 DTYPE_F32, DTYPE_BF16 = 0, 1
 MEAN_F32, MEAN_BF16_ROUND, MEAN_BF16_STORE = 0, 1, 2
 
@@ -33,10 +33,35 @@ SIGNATURES = {
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_score_blocks": [_i, _p, _p, _p, _i64, _p, _i64, _p, _p, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
     "ucm_copy_batch": [_p, _p, _sz, _sz, _p],
+    "ucm_device_create": [_i, _sz, _sz, _p],
+    "ucm_device_destroy": [_p],
+    "ucm_device_get_buffer": [_p, _sz],
+    "ucm_device_release_buffer": [_p, _p],
+    "ucm_device_h2d_sync": [_p, _p, _p, _sz],
+    "ucm_device_d2h_sync": [_p, _p, _p, _sz],
+    "ucm_device_h2d_async": [_p, _p, _p, _sz],
+    "ucm_device_d2h_async": [_p, _p, _p, _sz],
+    "ucm_device_append_callback": [_p, _p, _p],
+    "ucm_device_synchronized": [_p],
+    "ucm_device_h2d_batch_sync": [_p, _p, _p, _sz, _sz],
+    "ucm_device_d2h_batch_sync": [_p, _p, _p, _sz, _sz],
+    "ucm_device_stream": [_p],
     "ucm_kv_gather_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
     "ucm_kv_scatter_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
     "ucm_kv_gather_selected": [_p, _i, _sz, _sz, _i, _p, _p, _i, _i, _p, _p, _i, _p, _p],
 }
+
+
+# entry points that do not return a status code
+RESTYPES = {
+    "ucm_last_error": C.c_char_p,
+    "ucm_device_destroy": None,
+    "ucm_device_get_buffer": C.c_void_p,
+    "ucm_device_release_buffer": None,
+    "ucm_device_stream": C.c_void_p,
+}
+
+DEVICE_CALLBACK = C.CFUNCTYPE(None, C.c_int, C.c_void_p)
 
 
 class UcmHipError(RuntimeError):
@@ -55,7 +80,7 @@ def load() -> C.CDLL:
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the library does not export a declared symbol
         fn.argtypes = argtypes
-        fn.restype = C.c_char_p if name == "ucm_last_error" else C.c_int
+        fn.restype = RESTYPES.get(name, C.c_int)
     return lib
 
 
