@@ -322,7 +322,9 @@ int ucm_set_kvstar_tiles_per_wave(int tiles);
 /* Floats of scratch ucm_kvstar_votes[_tables] needs for a call of this shape
  * (rows_per_head = n_tokens * q_heads/kv_heads); the in-LDS path only needs
  * room for the kv heads' vote shares.  Ask after ucm_set_kvstar_tiles_per_wave,
- * which changes the path. */
+ * which changes the path; the votes calls take the sizes of the two areas
+ * (ws_max_floats, ws_part_floats) and fail with UCM_EINVAL when the path they
+ * would take needs more. */
 int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks,
                                 int sub_blocks, int d_pad, int64_t* max_floats, int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
@@ -330,7 +332,8 @@ int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int 
                      int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len,
                      int n_tasks, int max_blocks,
                      int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
-                     float* ws_part, float* votes, ucm_stream_t stream);
+                     int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
+                     ucm_stream_t stream);
 /* The same for tasks whose representatives do not share one table (the
  * reference keeps one blk_repre tensor per request and layer,
  * ucm/sparse/kvstar/multistep.py:191,483-501): task t's table starts at
@@ -343,7 +346,8 @@ int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_token
                             const void* const* task_tables, const int64_t* task_head_strides,
                             const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
                             int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
-                            float* ws_part, float* votes, ucm_stream_t stream);
+                            int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
+                            ucm_stream_t stream);
 
 /*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched

@@ -132,6 +132,60 @@ def test_kvstar_many_short_tasks_take_the_in_lds_path(ucm, dev):
         assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
 
 
+@pytest.mark.parametrize("d,M", [(128, 8), (32, 64)])
+@pytest.mark.parametrize("slope", [2.0, -2.0, 7.0])
+def test_kvstar_scores_drifting_far_from_the_first_span(ucm, dev, d, M, slope):
+    """The kernel takes a wave's exponentials relative to the largest score of the wave's first span.  Scores that
+    climb by hundreds along the task make it raise that reference and redo spans (a slope of 7 per block passes
+    the limit from one span to the next); scores that fall by hundreds underflow to zero votes, as the exact
+    softmax does in fp32.  Both paths, same tolerance as everywhere."""
+    from ucm_amd import ops
+
+    x, hq, hkv, n = 4, 8, 2, 200
+    lens = [n, 3]
+    rows = int(np.sum(lens))
+    base = (np.arange(rows, dtype=np.float32) * np.float32(slope))[:, None, None, None]     # the block's score level
+    noise = synth.normal_f32(1170, (rows, M, hkv, d)) * np.float32(0.125)
+    repre = f16_bits(base * np.float32(2.0 / d) + noise)                                    # times q = 0.5: score = level + noise
+    qs = [f16_bits(np.full((x, hq, d), 0.5, dtype=np.float32) + synth.normal_f32(1171 + t, (x, hq, d)) * np.float32(0.03125))
+          for t in range(2)]
+    try:
+        for tiles_per_wave in (-1, 3):
+            ops.set_kvstar_tiles_per_wave(tiles_per_wave)
+            got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
+            for t, m in enumerate(lens):
+                want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + m], topk=1)[1]
+                assert np.isfinite(got[off[t] : off[t] + m]).all()
+                assert np.allclose(got[off[t] : off[t] + m], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (tiles_per_wave, t)
+                assert abs(got[off[t] : off[t] + m].sum() - x * hq) < 1e-3 * x * hq
+    finally:
+        ops.set_kvstar_tiles_per_wave(0)
+
+
+def test_kvstar_workspace_sized_for_another_path_is_refused(ucm, dev):
+    """The path depends on a process-wide knob; a workspace sized before the knob changed is rejected on the host."""
+    from ucm_amd import _lib, ops
+
+    x, hq, hkv, d, M, n_tasks, blocks = 8, 32, 8, 128, 8, 32, 40
+    table = torch.zeros(hkv, n_tasks * blocks, d // 8, M, 8, dtype=torch.float16, device=dev)
+    q = torch.zeros(n_tasks, x, hq, d, dtype=torch.float16, device=dev)
+    q_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (x * hq * d)
+    seg_off = torch.arange(n_tasks, dtype=torch.int32, device=dev) * blocks
+    seg_len = torch.full((n_tasks,), blocks, dtype=torch.int32, device=dev)
+    votes = torch.zeros(n_tasks * blocks, device=dev)
+    ws = ops.kvstar_workspace(n_tasks, hkv, x * hq // hkv, blocks, M, d, dev)      # 256 (task, kv head) pairs: the in-LDS path
+    try:
+        ops.set_kvstar_tiles_per_wave(3)
+        with pytest.raises(_lib.UcmHipError) as e:
+            ops.kvstar_votes(q, q_off, x, hq, table, seg_off, seg_len, blocks, votes, ws)
+        assert e.value.code == _lib.EINVAL and "workspace" in str(e.value)
+    finally:
+        ops.set_kvstar_tiles_per_wave(0)
+    ops.kvstar_votes(q, q_off, x, hq, table, seg_off, seg_len, blocks, votes, ws)  # the path it was sized for
+    torch.cuda.synchronize()
+    assert np.allclose(votes.cpu().numpy(), x * hq / blocks, rtol=1e-5)            # all-zero scores: uniform votes
+
+
 @pytest.mark.parametrize("longest", [1200, 1400])
 def test_kvstar_long_task_plane_in_lds_or_not(ucm, dev, longest):
     """1200 blocks x 32 rows is a 150 KiB plane: the in-LDS path at its largest; 1400 blocks do not fit, and the

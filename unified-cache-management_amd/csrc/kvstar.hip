@@ -270,7 +270,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 // flight do not shrink with the vectors.
 //
 // kLds == false (any task length; a task may be cut into chunks): per tile and query row the kernel
-// leaves the tile's maximum and sum of exponentials ([tile][2][row_pad]) and the per-block sums
+// leaves the reference the tile's exponentials are relative to and their sum ([tile][2][row_pad]) and the per-block sums
 // ([part][row_pad]; a part is a block, or a tile's share of a block of more than 32 sub-blocks) in the
 // workspace for the two kernels below.
 //
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 
     extern __shared__ __attribute__((aligned(16))) unsigned short q_s[];   // [row_pad][kQStride]
     // kLds: [entry][row_pad] floats from byte plane_offset on (0 with one row tile: the queries then live in
-    // registers once the loop starts), followed by the waves' [wave][2][row_pad] running (maximum, sum) pairs
+    // registers once the loop starts), followed by the waves' [wave][2][row_pad] (reference, sum) pairs
     float* plane = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(q_s) + plane_offset);
 
     const unsigned task = blockIdx.z, h = blockIdx.y;
@@ -320,7 +320,9 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const int32_t psel = pruned_sel ? pruned_sel[task] : -1;
     const int32_t* pr = (pruned && psel >= 0) ? pruned + (static_cast<size_t>(psel) * kv_heads + h) * d_pruned : nullptr;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave index through readfirstlane: the compiler then knows that everything derived from it (a span's
+    // position, whether a tile is cut by the task's end) is the same for all lanes and keeps it in scalar registers
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int half = lane >> 5, lr = lane & 31;
     const unsigned ksteps = d_pad / 16;                  // MFMA steps; lane half `half`, step ks takes piece 2*ks + half
     // the task's first representative: rows seg_off[task].. of the one table, or a table of the task's own
@@ -421,98 +423,157 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 
     float* wmax = ws_max + (static_cast<size_t>(task) * kv_heads + h) * (2 * row_pad) * max_tiles;          // [tile][2][row_pad]
     float* wpart = ws_part + (static_cast<size_t>(task) * kv_heads + h) * row_pad * kPartsPerTile * max_tiles;  // [part][row_pad]
-    float m_run[kRowTiles], d_run[kRowTiles];            // kLds only
-#pragma unroll
-    for (int rt = 0; rt < kRowTiles; ++rt) { m_run[rt] = -INFINITY; d_run[rt] = 0.0f; }
 
-    auto process = [&](const u32x4 (&kf)[kLoads], unsigned s_span) {
-        float e_max[kRowTiles], e_sum[kRowTiles];        // kLds, blocks longer than a tile: the plane entry being gathered
+    // Every exponential of a wave is taken relative to one reference per query row, the row's largest
+    // score in the wave's first span, and not to the maximum of its own tile: fp32 has 2^127 of head room
+    // above the reference, a term 2^126 below it may as well be zero, and the per-tile maxima (fifteen
+    // v_max and a cross-lane move per sixteen scores), the rescaling of running sums and the exponentials
+    // that go with it all disappear from the loop.  The negated reference is what the matrix cores start
+    // accumulating from, so a score leaves them already shifted.  Should a span's sums ever pass 2^100
+    // (a later score more than 69 above the reference), the reference is raised to that span's maximum,
+    // the running sum is rescaled and the span is done again.
+    float ref[kRowTiles], d_run[kRowTiles];              // ref: natural units; d_run: sum of exp(score - ref) so far
+    f32x16 cinit[kRowTiles];
 #pragma unroll
-        for (int t = 0; t < kSpanTiles; ++t) {
-            const unsigned s0 = s_span + t * kTileSub;
-            const unsigned tile = s0 / kTileSub;
-            const bool live = s0 < S;                    // wave-uniform; a dead tile is computed on reloaded keys
-            const bool full = s0 + kTileSub <= S;        // and stored to padding: only a task's last tile needs the mask
-            f32x16 acc[kRowTiles];
+    for (int rt = 0; rt < kRowTiles; ++rt) {
+        ref[rt] = -INFINITY;
+        d_run[rt] = 0.0f;
 #pragma unroll
-            for (int rt = 0; rt < kRowTiles; ++rt) {
+        for (int i = 0; i < 16; ++i) { cinit[rt][i] = 0.0f; }
+    }
+    auto query_fragment = [&](int rt, int ks) -> u32x4 {
+        if constexpr (kTwoRowTiles) {
+            return *reinterpret_cast<const u32x4*>(&q_s[(rt * 32 + lr) * kQStride + half * 8 + ks * 16]);
+        } else {
+            return bq[ks];
+        }
+    };
+    // one tile's scores for row tile rt, added to what c holds
+    auto tile_scores = [&](const u32x4 (&kf)[kLoads], int t, int rt, f32x16 c) -> f32x16 {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) { acc[rt][i] = 0.0f; }
+        for (int ks = 0; ks < kSteps; ++ks) {
+            c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[t * kSteps + ks]),
+                                                       __builtin_bit_cast(f16x8, query_fragment(rt, ks)), c, 0, 0, 0);
+        }
+        return c;
+    };
+    // Lanes and tiles past the workgroup's end hold reloaded vectors of the task: they may take part.
+    auto raise_ref = [&](const u32x4 (&kf)[kLoads]) {
 #pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) {
-                    u32x4 b;
-                    if constexpr (kTwoRowTiles) {
-                        b = *reinterpret_cast<const u32x4*>(&q_s[(rt * 32 + lr) * kQStride + half * 8 + ks * 16]);
-                    } else {
-                        b = bq[ks];
-                    }
-                    acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kf[t * kSteps + ks]),
-                                                                    __builtin_bit_cast(f16x8, b), acc[rt], 0, 0, 0);
-                }
+        for (int rt = 0; rt < kRowTiles; ++rt) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < kSpanTiles; ++t) {
+                f32x16 a;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { a[i] = 0.0f; }
+                a = tile_scores(kf, t, rt, a);
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { mx = fmaxf(mx, a[i]); }
             }
+            const float nref = fmaxf(ref[rt], halves_max(mx));
+            d_run[rt] *= __builtin_amdgcn_exp2f((ref[rt] - nref) * kLog2e);   // the first time: 0 * 2^-inf = 0
+            ref[rt] = nref;
 #pragma unroll
-            for (int rt = 0; rt < kRowTiles; ++rt) {
-                const unsigned rho = rt * 32 + lr;
-                float sc[16];
+            for (int i = 0; i < 16; ++i) { cinit[rt][i] = -nref; }
+        }
+    };
+
+    // One span: its sums go to the plane (or the workspace), their totals per row to span_total.
+    auto span_sums = [&](const u32x4 (&kf)[kLoads], unsigned s_span, float (&span_total)[kRowTiles]) {
+        {
+            float e_sum[kRowTiles];                      // kLds, blocks longer than a tile: the plane entry being gathered
 #pragma unroll
-                for (int i = 0; i < 16; ++i) { sc[i] = acc[rt][i]; }
-                if (!full) {                             // no memory operation in here: a branch is harmless
+            for (int rt = 0; rt < kRowTiles; ++rt) { span_total[rt] = 0.0f; e_sum[rt] = 0.0f; }
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const unsigned s = s0 + (i >> 2) * 8 + half * 4 + (i & 3);
-                        sc[i] = s < S ? sc[i] : -INFINITY;
+            for (int t = 0; t < kSpanTiles; ++t) {
+                const unsigned s0 = s_span + t * kTileSub;
+                const unsigned tile = s0 / kTileSub;
+                // a tile past the task's end is computed on reloaded keys, masked, and stored to padding
+                const bool full = s0 + kTileSub <= S;    // wave-uniform; only a task's last tile needs the mask
+                f32x16 acc[kRowTiles];
+#pragma unroll
+                for (int rt = 0; rt < kRowTiles; ++rt) { acc[rt] = tile_scores(kf, t, rt, cinit[rt]); }
+#pragma unroll
+                for (int rt = 0; rt < kRowTiles; ++rt) {
+                    const unsigned rho = rt * 32 + lr;
+                    float e[16];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) { e[i] = __builtin_amdgcn_exp2f(acc[rt][i] * kLog2e); }
+                    if constexpr (kM < kTileSub) {
+                        if (!full) {
+                            // A task's last tile, or one past its end.  Rare and wave-uniform, so it has to stay
+                            // a branch: turned into selects (with their compares hoisted to the head of the span)
+                            // it costs more instructions per tile than the exponentials do.  What depends on a
+                            // value that passed through an asm statement cannot be computed speculatively, which
+                            // keeps the compiler from doing that.
+                            unsigned left = s0 < S ? S - s0 : 0u;            // live sub-blocks of this tile
+                            asm volatile("" : "+v"(left));
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                e[i] = static_cast<unsigned>((i >> 2) * 8 + half * 4 + (i & 3)) < left ? e[i] : 0.0f;
+                            }
+                        }
                     }
-                }
-                float mx = fmaxf(fmaxf(sc[0], sc[1]), sc[2]);
-#pragma unroll
-                for (int i = 3; i < 15; i += 2) { mx = fmaxf(fmaxf(mx, sc[i]), sc[i + 1]); }
-                mx = fmaxf(mx, sc[15]);
-                mx = halves_max(mx);                      // a live tile has at least one live sub-block, so mx is finite
-                const float nmx = -mx * kLog2e;
-                float e[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) { e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[i], kLog2e, nmx)); }
-                // rows past R hold zero queries: they are computed like the rest and never read
-                const unsigned part0 = tile * kPartsPerTile;   // first part of the tile
-                if constexpr (kLds) {
-                    const float mx2 = mx * kLog2e;
+                    // rows past R hold zero queries: they are computed like the rest and never read
+                    const unsigned part0 = tile * kPartsPerTile;   // first part of the tile
+                    // with 32 or more sub-blocks per block a tile is whole or past the task's end (its sums then go to
+                    // padding and count as zero)
+                    const bool dead = kM >= kTileSub && s0 >= S;
                     float total;
-                    if constexpr (kEntryTiles == 1) {
-                        // an entry lies inside this tile: log2 of the block's sum of 2^(score*log2e)
-                        total = block_sums<kTilePart>(e, half, [&](unsigned b, float v) {
-                            plane[(part0 + b) * row_pad + rho] = mx2 + __builtin_amdgcn_logf(v);
-                        });
-                    } else {
-                        // an entry spans kEntryTiles tiles of this span: gather (maximum, sum) over them
-                        total = block_sums<kTilePart>(e, half, [](unsigned, float) {});
-                        const float lt = live ? mx2 + __builtin_amdgcn_logf(total) : -INFINITY;
-                        if (t % kEntryTiles == 0) {
-                            e_max[rt] = lt;
-                            e_sum[rt] = 1.0f;
+                    if constexpr (kLds) {
+                        const float ref2 = ref[rt] * kLog2e;
+                        if constexpr (kEntryTiles == 1) {
+                            // an entry lies inside this tile: log2 of the block's sum of 2^(score*log2e)
+                            total = block_sums<kTilePart>(e, half, [&](unsigned b, float v) {
+                                plane[(part0 + b) * row_pad + rho] = ref2 + __builtin_amdgcn_logf(v);
+                            });
+                            total = dead ? 0.0f : total;
                         } else {
-                            const float m_new = fmaxf(e_max[rt], lt);
-                            e_sum[rt] = e_sum[rt] * __builtin_amdgcn_exp2f(e_max[rt] - m_new) + __builtin_amdgcn_exp2f(lt - m_new);
-                            e_max[rt] = m_new;
+                            // an entry spans kEntryTiles tiles of this span
+                            total = block_sums<kTilePart>(e, half, [](unsigned, float) {});
+                            total = dead ? 0.0f : total;
+                            e_sum[rt] = (t % kEntryTiles == 0) ? total : e_sum[rt] + total;
+                            if (t % kEntryTiles == kEntryTiles - 1) {
+                                plane[(tile / kEntryTiles) * row_pad + rho] = ref2 + __builtin_amdgcn_logf(e_sum[rt]);
+                            }
                         }
-                        if (t % kEntryTiles == kEntryTiles - 1) {
-                            plane[(tile / kEntryTiles) * row_pad + rho] = e_max[rt] + __builtin_amdgcn_logf(e_sum[rt]);
-                        }
+                    } else {
+                        total = block_sums<kTilePart>(e, half, [&](unsigned b, float v) {
+                            wpart[static_cast<size_t>(part0 + b) * row_pad + rho] = v;
+                        });
+                        total = dead ? 0.0f : total;
+                        // the pair the next kernel reads: what the tile's sums are relative to, and their total
+                        wmax[(static_cast<size_t>(tile) * 2 + half) * row_pad + rho] = half ? total : ref[rt];
                     }
-                    // the wave's running (maximum, sum of 2^(x - maximum)) of the row, in the same log2 units
-                    if (live) {
-                        const float m_new = fmaxf(m_run[rt], mx2);
-                        d_run[rt] = d_run[rt] * __builtin_amdgcn_exp2f(m_run[rt] - m_new) + total * __builtin_amdgcn_exp2f(mx2 - m_new);
-                        m_run[rt] = m_new;
-                    }
-                } else {
-                    const float total = block_sums<kTilePart>(e, half, [&](unsigned b, float v) {
-                        wpart[static_cast<size_t>(part0 + b) * row_pad + rho] = v;
-                    });
-                    wmax[(static_cast<size_t>(tile) * 2 + half) * row_pad + rho] = half ? total : mx;
+                    span_total[rt] += total;
                 }
             }
         }
     };
+    // At most two trips: the second only after the reference was raised.  The span's position passes through
+    // an asm statement inside the loop: otherwise the compiler computes every store address of the span
+    // ahead of the loop, which takes more registers than there are.
+    auto process = [&](const u32x4 (&kf)[kLoads], unsigned s_span) {
+#pragma unroll 1
+        for (int pass = 0; pass < 2; ++pass) {
+            unsigned s_here = s_span;
+            asm volatile("" : "+s"(s_here));
+            float span_total[kRowTiles];
+            span_sums(kf, s_here, span_total);
+            bool high = false;
+#pragma unroll
+            for (int rt = 0; rt < kRowTiles; ++rt) { high = high || span_total[rt] > 0x1p100f; }
+            if (__builtin_expect(!__any(high), 1)) {
+#pragma unroll
+                for (int rt = 0; rt < kRowTiles; ++rt) { d_run[rt] += span_total[rt]; }
+                break;
+            }
+            raise_ref(kf);                               // what this pass left in the plane is written again
+        }
+    };
+
+    if (s_first < s_end) { raise_ref(k0); }
 
     for (unsigned s0 = s_first; s0 < s_end;) {
         process(k0, s0);
@@ -535,14 +596,14 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
         if (half == 0) {
 #pragma unroll
             for (int rt = 0; rt < kRowTiles; ++rt) {
-                red[(wave * 2 + 0) * row_pad + rt * 32 + lr] = m_run[rt];
+                red[(wave * 2 + 0) * row_pad + rt * 32 + lr] = ref[rt] * kLog2e;   // the same product the entries carry
                 red[(wave * 2 + 1) * row_pad + rt * 32 + lr] = d_run[rt];
             }
         }
         __syncthreads();                                 // the plane and the waves' pairs are complete
         float row_m = 0.0f, row_w = 0.0f;
         if (threadIdx.x < row_pad) {
-            row_m = red[threadIdx.x];                    // wave 0 always has a live tile, so this is finite
+            row_m = red[threadIdx.x];                    // wave 0 always has a live tile, so its reference is finite
 #pragma unroll
             for (int w = 1; w < kWaves; ++w) { row_m = fmaxf(row_m, red[(w * 2) * row_pad + threadIdx.x]); }
             float den = 0.0f;
@@ -550,7 +611,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
             for (int w = 0; w < kWaves; ++w) {
                 den += red[(w * 2 + 1) * row_pad + threadIdx.x] * __builtin_amdgcn_exp2f(red[(w * 2) * row_pad + threadIdx.x] - row_m);
             }
-            row_w = threadIdx.x < R ? 1.0f / den : 0.0f; // den >= 1: the row's largest term is 2^0; padding rows do not vote
+            row_w = threadIdx.x < R ? 1.0f / den : 0.0f; // den is about 1 or more: the reference that became row_m is one of the row's scores; padding rows do not vote
         }
         __syncthreads();                                 // (a thread reads only its own column of the pairs)
         if (threadIdx.x < row_pad) {
@@ -591,9 +652,10 @@ __global__ __launch_bounds__(kThreads) void kvstar_headsum_kernel(
 // ([tile][2][row_pad], [block][row_pad]), so the score kernel's stores and the loads below move whole
 // 128-byte lines.
 //
-// Phase 1, grid: x = kv head, y = task; thread = (group of tiles, row).  The tiles' (maximum, sum) pairs
-// give the row's global maximum and softmax denominator; each tile maximum in the workspace is replaced
-// by the factor exp(tile max - row max) / denominator the tile's partial sums have to be multiplied
+// Phase 1, grid: x = kv head, y = task; thread = (group of tiles, row).  The tiles' (reference, sum) pairs
+// give the row's largest reference - one of the row's scores, at most 2^100 below its largest - and the
+// softmax denominator relative to it; each tile's reference in the workspace is replaced by the factor
+// exp(tile reference - largest reference) / denominator the tile's partial sums have to be multiplied
 // with.  Rows past tokens*group hold zero queries and are carried along.
 __global__ __launch_bounds__(kThreads) void kvstar_rowscale_kernel(
     float* __restrict__ ws_max, const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned M, unsigned max_blocks,
@@ -791,24 +853,33 @@ VotePlan plan_votes(int n_tasks, int kv_heads, int rows_per_head, int max_blocks
 }
 }  // namespace
 
+namespace {
+// floats a call carried out as `p` stores through ws_max / ws_part
+void workspace_floats(const VotePlan& p, int n_tasks, int kv_heads, int max_blocks, int sub_blocks, int64_t* max_floats,
+                      int64_t* part_floats)
+{
+    if (p.use_lds) {
+        // only the kv heads' shares of the votes pass through memory
+        *max_floats = 1;
+        *part_floats = std::max<int64_t>(static_cast<int64_t>(n_tasks) * kv_heads * max_blocks, 1);
+        return;
+    }
+    // per (task, kv head): a (reference, sum) pair per tile and row; a partial sum per row and block (per tile,
+    // for blocks of more than 32 sub-blocks), padded to whole tiles
+    const int64_t parts_per_tile = kTileSub / std::min(sub_blocks, kTileSub);
+    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * p.row_pad * 2 * p.max_tiles;
+    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * p.row_pad * parts_per_tile * p.max_tiles;
+}
+}  // namespace
+
 extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks,
                                            int d_pad, int64_t* max_floats, int64_t* part_floats)
 {
     UCM_REQUIRE(n_tasks >= 0 && kv_heads > 0 && rows_per_head > 0 && rows_per_head <= kMaxRows && max_blocks >= 0 &&
                     sub_blocks > 0 && d_pad > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
     UCM_REQUIRE(sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
-    const VotePlan p = plan_votes(n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad);
-    if (p.use_lds) {
-        // only the kv heads' shares of the votes pass through memory
-        *max_floats = 1;
-        *part_floats = std::max<int64_t>(static_cast<int64_t>(n_tasks) * kv_heads * max_blocks, 1);
-        return UCM_OK;
-    }
-    // per (task, kv head): a (maximum, sum) pair per tile and row; a partial sum per row and block (per tile,
-    // for blocks of more than 32 sub-blocks), padded to whole tiles
-    const int64_t parts_per_tile = kTileSub / std::min(sub_blocks, kTileSub);
-    *max_floats = static_cast<int64_t>(n_tasks) * kv_heads * p.row_pad * 2 * p.max_tiles;
-    *part_floats = static_cast<int64_t>(n_tasks) * kv_heads * p.row_pad * parts_per_tile * p.max_tiles;
+    workspace_floats(plan_votes(n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad), n_tasks, kv_heads, max_blocks,
+                     sub_blocks, max_floats, part_floats);
     return UCM_OK;
 }
 
@@ -816,8 +887,8 @@ namespace {
 int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
                  const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, const void* const* task_tables,
                  const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
-                 int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, float* ws_part, float* votes,
-                 ucm_stream_t stream)
+                 int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part,
+                 int64_t ws_part_floats, float* votes, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks >= 0 && max_blocks >= 0, "ucm_kvstar_votes: n_tasks=%d max_blocks=%d", n_tasks, max_blocks);
     if (n_tasks == 0 || max_blocks == 0) { return UCM_OK; }
@@ -841,6 +912,15 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
     const VotePlan plan = plan_votes(n_tasks, kv_heads, static_cast<int>(R), max_blocks, sub_blocks, d_pad);
+    {
+        // the path depends on a process-wide knob: a workspace sized before the knob changed must not be overrun
+        int64_t need_max = 0, need_part = 0;
+        workspace_floats(plan, n_tasks, kv_heads, max_blocks, sub_blocks, &need_max, &need_part);
+        UCM_REQUIRE(ws_max_floats >= need_max && ws_part_floats >= need_part,
+                    "ucm_kvstar_votes: workspace of %lld + %lld floats, this call needs %lld + %lld (ucm_kvstar_workspace_floats)",
+                    static_cast<long long>(ws_max_floats), static_cast<long long>(ws_part_floats),
+                    static_cast<long long>(need_max), static_cast<long long>(need_part));
+    }
     const unsigned max_tiles = plan.max_tiles, row_pad = plan.row_pad, q_bytes = plan.q_bytes, steps = plan.steps,
                    span_tiles = plan.span_tiles, plane_offset = plan.plane_offset;
     const size_t lds_plane = plan.lds_plane;
@@ -923,19 +1003,23 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
                                 const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
                                 int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
                                 int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
-                                float* ws_part, float* votes, ucm_stream_t stream)
+                                int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
+                                ucm_stream_t stream)
 {
     return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, repre_f16, repre_head_stride, nullptr, nullptr,
-                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_part, votes, stream);
+                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
+                        ws_part_floats, votes, stream);
 }
 
 extern "C" int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                                        const int32_t* pruned, const int32_t* pruned_sel, const void* const* task_tables,
                                        const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len,
                                        int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad,
-                                       float* ws_max, float* ws_part, float* votes, ucm_stream_t stream)
+                                       float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
+                                       float* votes, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks == 0 || (task_tables && task_head_strides), "ucm_kvstar_votes_tables: null table list");
     return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, nullptr, 0, task_tables, task_head_strides,
-                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_part, votes, stream);
+                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
+                        ws_part_floats, votes, stream);
 }

@@ -381,7 +381,7 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
     _lib.call("ucm_kvstar_votes", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), repre.data_ptr(), head_stride,
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
-              d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), _dev(ws_part, torch.float32, "ws_part"),
+              d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
               _dev(votes, torch.float32, "votes"), _stream())
 
 
@@ -417,7 +417,7 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
     _lib.call("ucm_kvstar_votes_tables", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
-              d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), _dev(ws_part, torch.float32, "ws_part"),
+              d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
               _dev(votes, torch.float32, "votes"), _stream())
     return host, dev
 
