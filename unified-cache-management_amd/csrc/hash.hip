@@ -48,6 +48,14 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long mask)
                                      __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
 }
 
+// row of the staged (negated, transposed) weight matrix that holds weight column `col`:
+// within its 32-column block, column half*16 + i sits in row (i/4)*8 + half*4 + i%4
+__device__ __forceinline__ int row_of_col(int col)
+{
+    const int cb = col & 31, h = cb >> 4, i = cb & 15;
+    return (col & ~31) + (i >> 2) * 8 + h * 4 + (i & 3);
+}
+
 __device__ __forceinline__ float bf16_to_f32(unsigned short h) { return __uint_as_float(static_cast<unsigned>(h) << 16); }
 
 struct __attribute__((aligned(16))) WaveScratch {
@@ -113,7 +121,7 @@ __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen,
         if (base + lane < qlen) {
             const unsigned e = ws.queue[base + lane];
             const unsigned v = e >> 8, col = (e >> 1) & 127u, prov = e & 1u;
-            const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &neg_wt[col * kWtStride]);
+            const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &neg_wt[row_of_col(col) * kWtStride]);
             if (static_cast<unsigned>(pos) != prov) {
                 if (tc_out) { atomicXor(&tc_out[v * 4 + (col >> 5)], 1u << (col & 31)); }
                 atomicAdd(&ws.colsum[v % kv_heads][col], pos ? 1 : -1);
@@ -138,7 +146,7 @@ __device__ __forceinline__ void planes_add(unsigned (&pl)[kPlanes], unsigned x)
 }
 
 // Adds the 32 counts of a plane set to the per-head column sums in LDS and clears
-// it.  Bit b of word pair `wp` is column (2*wp + b/16)*32 + ((b%16)/4)*8 + half*4 + b%4.
+// it.  Bit b of word pair `wp` is column (2*wp + b/16)*32 + half*16 + b%16.
 __device__ __forceinline__ void planes_flush(unsigned (&pl)[kPlanes], int* __restrict__ head_row, int wp, int half)
 {
 #pragma unroll 4
@@ -146,25 +154,22 @@ __device__ __forceinline__ void planes_flush(unsigned (&pl)[kPlanes], int* __res
         int cnt = 0;
 #pragma unroll
         for (int p = 0; p < kPlanes; ++p) { cnt |= static_cast<int>((pl[p] >> b) & 1u) << p; }
-        const int col = (2 * wp + (b >> 4)) * 32 + ((b & 15) >> 2) * 8 + half * 4 + (b & 3);
+        const int col = (2 * wp + (b >> 4)) * 32 + half * 16 + (b & 15);
         if (cnt) { atomicAdd(&head_row[col], cnt); }
     }
 #pragma unroll
     for (int p = 0; p < kPlanes; ++p) { pl[p] = 0u; }
 }
 
-// nibble g of the low 16 bits of x moves to the low nibble of byte g
-__device__ __forceinline__ unsigned spread_nibbles(unsigned x)
-{
-    x = (x | (x << 8)) & 0x00ff00ffu;
-    return (x | (x << 4)) & 0x0f0f0f0fu;
-}
-
 // The product is taken transposed, C^T = (-W)^T . X^T: the matrix cores' A
 // operand is the (negated) weight fragment and B the key fragment, so that lane
-// (half, lr) ends up with sixteen columns per 32-column block of ITS OWN vector
-// lr in registers: accumulator i of block nb is column
-//     nb*32 + (i/4)*8 + half*4 + i%4.
+// (half, lr) ends up with sixteen results per 32-column block of ITS OWN vector
+// lr in registers: accumulator i of block nb is row (i/4)*8 + half*4 + i%4 of
+// the block's A operand.  Which weight column a row of A holds is free: the
+// staged copy keeps column nb*32 + half*16 + i in that row (row_of_col below),
+// so a lane's sixteen results are sixteen ADJACENT columns and the code words
+// need no bit shuffling: accumulator i of block nb is column
+//     nb*32 + half*16 + i.
 // With the weights negated, a projection is positive exactly when its
 // accumulator has the sign bit set (and an all-zero key gives +0: bit clear), so
 // one v_alignbit per result shifts the bit into the lane's code word, the two
@@ -183,8 +188,8 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     short* __restrict__ colsum_out, int64_t cs_layer_stride,
     unsigned* __restrict__ block_codes, int64_t bc_layer_stride)
 {
-    __shared__ __attribute__((aligned(16))) unsigned short wt[kBits * kWtStride];  // wt[col][d] = -W[d][col]
-    __shared__ float w_norm2[kBits];
+    __shared__ __attribute__((aligned(16))) unsigned short wt[kBits * kWtStride];  // wt[row_of_col(col)][d] = -W[d][col]
+    __shared__ float w_norm2[kBits];                     // by row of wt
     __shared__ WaveScratch scratch[kWaves];
 
     // ---- weights: global [d][col] -> LDS [col][d], sign flipped
@@ -193,8 +198,8 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         const u32x4 v = *reinterpret_cast<const u32x4*>(w + d * kBits + c0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            wt[(c0 + 2 * j) * kWtStride + d] = static_cast<unsigned short>((v[j] & 0xffffu) ^ 0x8000u);
-            wt[(c0 + 2 * j + 1) * kWtStride + d] = static_cast<unsigned short>((v[j] >> 16) ^ 0x8000u);
+            wt[row_of_col(c0 + 2 * j) * kWtStride + d] = static_cast<unsigned short>((v[j] & 0xffffu) ^ 0x8000u);
+            wt[row_of_col(c0 + 2 * j + 1) * kWtStride + d] = static_cast<unsigned short>((v[j] >> 16) ^ 0x8000u);
         }
     }
     __syncthreads();
@@ -356,18 +361,16 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
             planes_add(planes23, pair[1]);
             ++pending;
 
-            // this tile's code words: 32 vectors x 16 B, contiguous
-            unsigned words[4];
-#pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                const unsigned own = spread_nibbles((pair[nb >> 1] >> (16 * (nb & 1))) & 0xffffu) << (4 * half);
-                words[nb] = own | __shfl_xor(own, 32, 64);
-            }
             if (kTokenCodes) {
-                // lane lr keeps words 0-1 of its vector, lane lr+32 words 2-3; they are stored at the
-                // start of the next tile (see store_codes)
-                pend_cw.x = half ? words[2] : words[0];
-                pend_cw.y = half ? words[3] : words[1];
+                // This tile's code words: 32 vectors x 16 B, contiguous.  A lane holds the lower (half 0)
+                // or upper (half 1) sixteen bits of all four words of its vector; lane lr keeps words 0-1,
+                // lane lr+32 words 2-3 (stored at the start of the next tile, see store_codes).  One
+                // exchange between the lane halves brings both parts of a lane's two words together:
+                // lower lanes then hold (own pair 0, partner's pair 0), upper lanes (partner's pair 1,
+                // own pair 1), lower sixteen columns first either way.
+                const auto both = __builtin_amdgcn_permlane32_swap(pair[0], pair[1], false, false);
+                pend_cw.x = __builtin_amdgcn_perm(both[1], both[0], 0x05040100u);
+                pend_cw.y = __builtin_amdgcn_perm(both[1], both[0], 0x07060302u);
                 pend_tile = tile;
             }
 
@@ -391,7 +394,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                         if (mask) {
                             const unsigned i = static_cast<unsigned>(__builtin_ctz(mask));
                             mask &= mask - 1u;
-                            const unsigned col = nb * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                            const unsigned col = nb * 32 + half * 16 + i;
                             ws.queue[qlen + static_cast<int>(lanes_below(um))] =
                                 ((tile * 32 + lr) << 8) | (col << 1) | ((signs >> i) & 1u);
                         }
