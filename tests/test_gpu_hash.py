@@ -137,6 +137,65 @@ def test_hash_encode_persistent_waves_and_queue_overflow(ucm, dev, hkv, bs):
         ops.set_hash_encode_groups(0)
 
 
+def test_config5_full_size_negated_keys_give_complement_codes(ucm, dev):
+    """The hash configuration at its full size (32 requests of 64..256 blocks, 8 kv heads, 32 layers, 128-bit
+    codes), checked through what the arithmetic fixes at any size: negating a key negates its exact projection,
+    so a bit of -K's token code is the complement of K's unless the projection is exactly 0 (bit 0 both times:
+    `> 0` is strict; a few per ten million sums of bf16 products do cancel exactly), a column sum is
+    #ones - #zeros of its column over the block's tokens, and the majority code is `column sum > 0`.
+    Eight layers at a time, fresh keys each time, so that the keys and their negation stay around 22 GB."""
+    from ucm_amd import ops
+
+    hkv, bs, n_req, group = 8, 128, 32, 8
+    lens = 64 + synth.permutation(880, 4096)[:n_req] % 193          # 64..256 blocks per request
+    rows = int(lens.sum())
+    w_bits, w_f32 = make_weights(881)
+    w = bf16_dev(w_bits, dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(882)
+    ids = torch.randperm(rows, device=dev, generator=gen).to(torch.int32)
+    shifts = torch.arange(8, device=dev, dtype=torch.uint8)
+
+    def recount(tcodes_layer):                                      # [rows, bs, hkv, 16] -> #ones per (row, head, column)
+        bits = (tcodes_layer.view(rows, bs, hkv, 16, 1) >> shifts) & 1
+        return bits.view(rows, bs, hkv, 128).sum(dim=1, dtype=torch.int32)
+
+    def majority(colsum):
+        return ((colsum > 0).view(group, rows, hkv, 16, 8).to(torch.uint8) << shifts).sum(dim=-1, dtype=torch.uint8)
+
+    exact_zeros = 0
+    for part in range(32 // group):
+        caches = [torch.empty((rows, bs, hkv, 128), dtype=torch.bfloat16, device=dev).normal_(generator=gen)
+                  for _ in range(group)]
+        negated = [-c for c in caches]
+        out = []
+        for layers in (caches, negated):
+            colsum = torch.zeros((group, rows, hkv, 128), dtype=torch.int16, device=dev)
+            bcodes = torch.zeros((group, rows, hkv, 16), dtype=torch.uint8, device=dev)
+            tcodes = torch.zeros((group, rows, bs, hkv, 16), dtype=torch.uint8, device=dev)
+            ops.hash_encode_blocks(ops.LayerPointers(layers), ids, None, rows, w, bs, hkv, rows, colsum, bcodes,
+                                   token_codes=tcodes)
+            out.append((colsum, bcodes, tcodes))
+        torch.cuda.synchronize()
+        (s_pos, b_pos, t_pos), (s_neg, b_neg, t_neg) = out
+        assert not (t_pos & t_neg).any(), part                      # never positive both ways
+        both_zero = ~(t_pos | t_neg)                                # bits that are 0 both ways: exact zeros only
+        where = both_zero.nonzero()
+        assert where.shape[0] < 1e-6 * both_zero.numel() * 8, (part, where.shape[0])
+        for l, r, t, h, byte in where[:4].cpu().numpy():            # ... which a few of them are shown to be
+            x = caches[l][int(ids[r])][t, h].double().cpu().numpy()
+            cols = [8 * byte + j for j in range(8) if (int(both_zero[l, r, t, h, byte]) >> j) & 1]
+            assert cols and all(float(x @ w_f32[:, c].astype(np.float64)) == 0.0 for c in cols), (part, l, r, t, h, byte)
+        exact_zeros += where.shape[0]
+        for l in (0, group - 1):
+            ones_pos, ones_neg = recount(t_pos[l]), recount(t_neg[l])
+            assert torch.equal(s_pos[l].to(torch.int32), 2 * ones_pos - bs), (part, l)
+            assert torch.equal(s_neg[l].to(torch.int32), 2 * ones_neg - bs), (part, l)
+        assert torch.equal(b_pos, majority(s_pos)) and torch.equal(b_neg, majority(s_neg)), part
+        del caches, negated, out
+    print("exact zero projections met:", exact_zeros)
+
+
 def test_hash_queries_scores_and_selection(ucm, dev):
     """Config-5 shape in small: ragged batch, 8 kv heads, 32 query heads, 2 layers."""
     from ucm_amd import ops
