@@ -162,6 +162,47 @@ def test_kvstar_scores_drifting_far_from_the_first_span(ucm, dev, d, M, slope):
         ops.set_kvstar_tiles_per_wave(0)
 
 
+@pytest.mark.parametrize("M,d", [(64, 32), (8, 128)])
+def test_kvstar_full_size_vote_sums_and_block_order(ucm, dev, M, d):
+    """The multi-query retrieval at the size of the ragged batch of configs[1] (16 requests of 32..512 blocks x 32
+    layers = 512 tasks, 8 query tokens x 32 heads each), through what holds at any size: a task's votes are
+    probabilities summed over its 256 (token, head) rows, so they are non-negative and add up to 256; and a vote
+    belongs to its block, so a table with every task's blocks in reverse order gives the same votes reversed
+    (other summation order: equal to rounding).  Three tasks are also compared with the CPU oracle."""
+    from ucm_amd import ops
+
+    x, hq, hkv, n_layers, n_req = 8, 32, 8, 32, 16
+    lens_req = 32 + synth.permutation(1180, 4096)[:n_req] % 481            # 32..512 blocks
+    lens = np.tile(lens_req, n_layers).astype(np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    rows, n_tasks, longest = int(lens.sum()), len(lens), int(lens.max())
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1181)
+    table = (torch.empty((hkv, rows, d // 8, M, 8), device=dev).normal_(generator=gen) * 0.25).to(torch.float16)
+    q = (torch.empty((n_tasks, x, hq, d), device=dev).normal_(generator=gen) * 0.25).to(torch.float16)
+    q_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (x * hq * d)
+    seg_off, seg_len = torch.from_numpy(off).to(dev), torch.from_numpy(lens).to(dev)
+    ws = ops.kvstar_workspace(n_tasks, hkv, x * hq // hkv, longest, M, d, dev)
+    votes = torch.full((rows,), -7.0, device=dev)
+    ops.kvstar_votes(q, q_off, x, hq, table, seg_off, seg_len, longest, votes, ws)
+    # the same tasks with their blocks in reverse order
+    src = torch.cat([torch.arange(int(o) + int(n) - 1, int(o) - 1, -1) for o, n in zip(off, lens)]).to(dev)
+    votes_rev = torch.full((rows,), -7.0, device=dev)
+    ops.kvstar_votes(q, q_off, x, hq, table[:, src].contiguous(), seg_off, seg_len, longest, votes_rev, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(votes).all() and (votes >= 0).all()
+    sums = torch.zeros(n_tasks, device=dev, dtype=torch.float64).index_add_(
+        0, torch.repeat_interleave(torch.arange(n_tasks, device=dev), seg_len.long()), votes.double())
+    assert torch.allclose(sums, torch.full_like(sums, x * hq), rtol=1e-4), (sums.min().item(), sums.max().item())
+    assert torch.allclose(votes_rev[src], votes, rtol=VOTE_RTOL, atol=VOTE_ATOL)
+    ref_order = ops.kvstar_table_to_reference(table)                       # [rows, M, hkv, d]
+    for t in (0, n_tasks // 2 + 3, n_tasks - 1):
+        o, n = int(off[t]), int(lens[t])
+        want = O.kvstar_retrieve(q[t].view(torch.int16).cpu().numpy().view(np.uint16),
+                                 ref_order[o : o + n].contiguous().view(torch.int16).cpu().numpy().view(np.uint16), topk=1)[1]
+        assert np.allclose(votes[o : o + n].cpu().numpy(), want, rtol=VOTE_RTOL, atol=VOTE_ATOL), t
+
+
 def test_kvstar_workspace_sized_for_another_path_is_refused(ucm, dev):
     """The path depends on a process-wide knob; a workspace sized before the knob changed is rejected on the host."""
     from ucm_amd import _lib, ops
