@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload (BASELINE.json configs[1]): a ragged continuous batch of 16 requests,
+Workload (configs[1] of the benchmark definition): a ragged continuous batch of 16 requests,
 context lengths uniform in [4096, 65536] tokens rounded to the 128-token block,
 Llama-3-8B attention shape (32 query heads / 8 kv heads / head_dim 128, bf16),
 all 32 layers.  One step = for every layer and request: score all block
@@ -54,7 +54,7 @@ def parse():
                     help="element type of the representative table: bf16 = the rounded means the live reference "
                          "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
     ap.add_argument("--hash-leg", action="store_true",
-                    help="also time the hash-code retrieval variant (BASELINE configs[4] shape) on the same caches")
+                    help="also time the hash-code retrieval variant (the configs[4] shape of the benchmark definition) on the same caches")
     ap.add_argument("--kvstar-leg", action="store_true",
                     help="also time the multi-query softmax-vote retrieval (KVStar: 8 query tokens per request) on the same "
                          "ragged batch")

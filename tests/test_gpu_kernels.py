@@ -509,7 +509,7 @@ def test_retrieval_then_gather_end_to_end(ucm, dev):
     assert np.array_equal(staging.cpu().numpy(), want)
 
 
-# ------------------------------------------- BASELINE.json full-size cases
+# ------------------------------------------- the benchmark configurations at full size
 
 def test_config3_full_size_round_trip(ucm, dev):
     """64 requests x 2048-token budget (16 blocks) x 32 layers, K and V: 17.2 GB per direction.  A random block
