@@ -110,7 +110,8 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *              value, sizes the grid); total_blocks = sum of seg_len when the
  *              host knows it (a tighter grid), else 0.
  *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x].
- * head_dim must be 64 or 128 and kv_heads one of 1, 2, 4, 8, 16.
+ * head_dim must be 32, 64, 96, 128, 192 or 256, kv_heads one of 1, 2, 4, 8, 16 and
+ * kv_heads*head_dim at most 2048.
  */
 int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
                      int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,

@@ -45,7 +45,7 @@ def test_bad_arguments_fail_on_the_host(ucm):
     _lib.call("ucm_copy_batch", None, None, 0, 64, None)  # an empty batch is a no-op, pointers unchecked
     # head_dim the scoring kernel was not built for
     with pytest.raises(_lib.UcmHipError) as e:
-        _lib.call("ucm_score_blocks", 16, 0, 0, None, 32, 16, 0, 0, 16, 16, 1, 8, 0, 1, 8, 96, 16, 0, None)
+        _lib.call("ucm_score_blocks", 16, 0, 0, None, 32, 16, 0, 0, 16, 16, 1, 8, 0, 1, 8, 80, 16, 0, None)
     assert e.value.code == _lib.ENOTSUP and "head_dim" in str(e.value)
     with pytest.raises(_lib.UcmHipError) as e:
         _lib.call("ucm_score_blocks", 16, 0, 0, None, 30, 16, 0, 0, 16, 16, 1, 8, 0, 1, 6, 128, 16, 0, None)

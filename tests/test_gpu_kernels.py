@@ -144,7 +144,8 @@ def test_golden_select_cases_on_gpu(ucm, dev, golden):
         assert np.array_equal(out["idx"][0, 0, : len(want)], want), name
 
 
-@pytest.mark.parametrize("hkv,g,d", [(8, 4, 128), (8, 8, 128), (1, 8, 128), (2, 2, 64), (4, 1, 64), (16, 2, 128)])
+@pytest.mark.parametrize("hkv,g,d", [(8, 4, 128), (8, 8, 128), (1, 8, 128), (2, 2, 64), (4, 1, 64), (16, 2, 128),
+                                     (8, 4, 32), (2, 4, 96), (4, 2, 192), (8, 2, 256), (1, 16, 256)])
 @pytest.mark.parametrize("q_dtype", [torch.float32, torch.bfloat16])
 def test_ragged_batch_scores_and_selection(ucm, dev, hkv, g, d, q_dtype):
     from ucm_amd import ops
@@ -165,7 +166,8 @@ def as_bf16_values(a):
     return torch.from_numpy(np.ascontiguousarray(a, np.float32)).to(torch.bfloat16).float().numpy()
 
 
-@pytest.mark.parametrize("hkv,g,d", [(8, 4, 128), (8, 8, 128), (1, 8, 128), (2, 2, 64), (4, 1, 64), (16, 2, 128)])
+@pytest.mark.parametrize("hkv,g,d", [(8, 4, 128), (8, 8, 128), (1, 8, 128), (2, 2, 64), (4, 1, 64), (16, 2, 128),
+                                     (8, 4, 32), (2, 4, 96), (4, 2, 192), (8, 2, 256), (1, 16, 256)])
 @pytest.mark.parametrize("q_dtype", [torch.float32, torch.bfloat16])
 def test_bf16_table_scores_like_the_widened_table(ucm, dev, hkv, g, d, q_dtype):
     """A bf16 representative table holds what the live path stores (ucm/sparse/gsa/gsa.py:640-652);

@@ -26,7 +26,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
-constexpr int kMaxRow = 16 * 128;  // kv_heads <= 16, head_dim <= 128
+constexpr int kMaxRow = 16 * 128;  // kv_heads * head_dim: what the staged query row may hold
 
 template <int kCtrl>
 __device__ __forceinline__ float quad_perm(float x)
@@ -400,7 +400,9 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
                 max_seg_len, static_cast<long long>(total_blocks));
     UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0,
                 "ucm_score_blocks: q_heads=%d kv_heads=%d", q_heads, kv_heads);
-    UCM_SUPPORTED(head_dim == 64 || head_dim == 128, "ucm_score_blocks: head_dim=%d (64 or 128)", head_dim);
+    UCM_SUPPORTED(head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 || head_dim == 192 || head_dim == 256,
+                  "ucm_score_blocks: head_dim=%d (32, 64, 96, 128, 192 or 256)", head_dim);
+    UCM_SUPPORTED(kv_heads * head_dim <= kMaxRow, "ucm_score_blocks: kv_heads*head_dim=%d (at most %d)", kv_heads * head_dim, kMaxRow);
     UCM_SUPPORTED(kv_heads <= 16 && 16 % kv_heads == 0, "ucm_score_blocks: kv_heads=%d (1, 2, 4, 8 or 16)", kv_heads);
     UCM_REQUIRE(ucm::aligned16(repre) && repre_layer_stride % (repre_dtype == UCM_DTYPE_BF16 ? 8 : 4) == 0,
                 "ucm_score_blocks: repre not 16-byte aligned");
@@ -418,13 +420,23 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
 #define UCM_SCORE_ARGS q, q_layer_stride, q_rows, q_heads, repre, repre_layer_stride, seg_off, seg_len, n_req, \
                        tile_bound, n_layers, kv_heads, scores, scores_layer_stride, tile_blocks, s
     const bool qf = q_dtype == UCM_DTYPE_F32;
-    if (repre_dtype == UCM_DTYPE_F32) {
-        if (head_dim == 128) { if (qf) { launch<128, float>(UCM_SCORE_ARGS); } else { launch<128, uint16_t>(UCM_SCORE_ARGS); } }
-        else { if (qf) { launch<64, float>(UCM_SCORE_ARGS); } else { launch<64, uint16_t>(UCM_SCORE_ARGS); } }
-    } else {
-        if (head_dim == 128) { if (qf) { launch_bf16<128, float>(UCM_SCORE_ARGS); } else { launch_bf16<128, uint16_t>(UCM_SCORE_ARGS); } }
-        else { if (qf) { launch_bf16<64, float>(UCM_SCORE_ARGS); } else { launch_bf16<64, uint16_t>(UCM_SCORE_ARGS); } }
+#define UCM_SCORE_DIM(D)                                                                                        \
+    do {                                                                                                        \
+        if (repre_dtype == UCM_DTYPE_F32) {                                                                     \
+            if (qf) { launch<D, float>(UCM_SCORE_ARGS); } else { launch<D, uint16_t>(UCM_SCORE_ARGS); }         \
+        } else {                                                                                                \
+            if (qf) { launch_bf16<D, float>(UCM_SCORE_ARGS); } else { launch_bf16<D, uint16_t>(UCM_SCORE_ARGS); } \
+        }                                                                                                       \
+    } while (0)
+    switch (head_dim) {
+    case 32: UCM_SCORE_DIM(32); break;
+    case 64: UCM_SCORE_DIM(64); break;
+    case 96: UCM_SCORE_DIM(96); break;
+    case 128: UCM_SCORE_DIM(128); break;
+    case 192: UCM_SCORE_DIM(192); break;
+    default: UCM_SCORE_DIM(256); break;
     }
+#undef UCM_SCORE_DIM
 #undef UCM_SCORE_ARGS
     UCM_LAUNCH_CHECK("ucm_score_blocks");
 }
