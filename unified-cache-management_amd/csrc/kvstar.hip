@@ -55,7 +55,7 @@ __device__ __forceinline__ unsigned short f32_to_f16_bits(float f)
 // score kernel reads whole 128-byte lines (M*16 bytes per piece and block) instead of 16 bytes out
 // of each of 64 lines.
 //
-// grid: x = listed block, y = layer.  Phase 1: a thread owns 8 adjacent columns of a token row
+// Phase 1: a thread owns 8 adjacent columns of a token row
 // (one 16-byte load per token, `merge` tokens accumulated in token order in fp32), the means -
 // rounded to bf16 and then fp16, what mean() in the model dtype followed by .to(float16) gives -
 // are parked in LDS as [sub-block][kv_heads*head_dim] (as many sub-blocks at a time as fit 64 KiB).
@@ -80,17 +80,170 @@ __device__ __forceinline__ void add_bf16x8(float (&acc)[8], const u32x4 v)
     acc[6] = acc[6] + __uint_as_float(v.w << 16); acc[7] = acc[7] + __uint_as_float(v.w & 0xffff0000u);
 }
 
-// kMerge: the tokens per sub-block when that is 1, 2, 4 or 8 - a thread then works on 16/kMerge of its
-// (sub-block, 8 columns) items at a time so that sixteen loads are in flight - or 0 for any other count.
+// Phase 2 of the representative kernels: the kept channels of the staged means of sub-blocks m0 .. m0+mc-1,
+// gathered from LDS and written as the table's 16-byte pieces, consecutive threads to consecutive 16 bytes.
+__device__ __forceinline__ void repre_write_pieces(const unsigned short* __restrict__ stage, const int32_t* __restrict__ kept,
+                                                   bool pruned, unsigned kv_heads, unsigned head_dim, unsigned d_pruned,
+                                                   unsigned pieces, unsigned srow_stride, unsigned M, unsigned m0, unsigned mc,
+                                                   unsigned short* __restrict__ out, int64_t head_stride)
+{
+    for (unsigned e = threadIdx.x; e < kv_heads * pieces * mc; e += kThreads) {
+        const unsigned h = e / (pieces * mc), rem = e - h * (pieces * mc);
+        const unsigned piece = rem / mc, ml = rem - piece * mc;
+        const unsigned short* srow = stage + ml * srow_stride + h * head_dim;
+        u32x4 o;
+        if (!pruned && piece * 8 + 8 <= d_pruned) {      // all channels kept: the piece is 16 contiguous bytes
+            o = *reinterpret_cast<const u32x4*>(srow + piece * 8);
+        } else {
+            unsigned short c[8];
+#pragma unroll
+            for (unsigned j = 0; j < 8; ++j) {
+                const unsigned p = piece * 8 + j;
+                unsigned short v = 0;
+                if (p < d_pruned) {
+                    const unsigned d = pruned ? static_cast<unsigned>(kept[h * d_pruned + p]) : p;
+                    if (d < head_dim) { v = srow[d]; }
+                }
+                c[j] = v;
+            }
+            o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
+            o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
+            o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
+            o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
+        }
+        ucm::gstore16(out + static_cast<int64_t>(h) * head_stride + (static_cast<size_t>(piece) * M + m0 + ml) * 8, o);
+    }
+}
+
+// Sub-blocks of 1, 2, 4 or 8 tokens (kMerge).  Workgroups are persistent over the list of cache blocks
+// (grid: x = workgroup, stepping by the grid; y = layer) and the work of one is a sequence of UNITS: a unit
+// is 16 loads of 16 bytes per thread - 16/kMerge (sub-block, 8 columns) items - of one chunk of one cache
+// block.  The loads of the next unit - of the same chunk, the next chunk or the next cache block - are
+// issued before the current unit's means are formed, so key loads stay in flight through the phase that
+// writes a chunk's pieces out and across cache blocks.
 template <int kMerge>
 __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
+    const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
+    const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows, unsigned block_size,
+    unsigned kv_heads, unsigned head_dim, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
+    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
+{
+    static_assert(kMerge == 1 || kMerge == 2 || kMerge == 4 || kMerge == 8, "tokens per sub-block");
+    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]: the 16 bytes of padding
+    constexpr unsigned kBatch = kRepreUnroll / kMerge;                       // spread the sub-blocks' rows over the LDS banks
+    const unsigned M = block_size / kMerge;
+    const unsigned row = kv_heads * head_dim, ncg = row / 8, srow_stride = row + 8;
+    const float inv = 1.0f / static_cast<float>(kMerge);
+    const unsigned pieces = d_pad / 8;
+    const unsigned short* layer = static_cast<const unsigned short*>(k_layers[blockIdx.y]);
+    // the channel lists, read once: a load from memory per output piece would queue behind the key stream
+    int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
+    if (pruned) {
+        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = pruned[e]; }
+    }
+
+    struct Unit {
+        unsigned item, m0, w_first;                      // cache block in the list, first sub-block of the chunk, first work item
+        const unsigned short* blk;
+        bool valid;
+    };
+    // first usable cache block at or after `from` (a block id or slot out of range is skipped, never dereferenced)
+    auto seek = [&](Unit& u, unsigned from) {
+        for (unsigned i = from; i < n_items; i += gridDim.x) {
+            const unsigned id = static_cast<unsigned>(block_ids[i]);
+            if (id < num_blocks && static_cast<unsigned>(slots[i]) < rows) {
+                u.item = i;
+                u.m0 = 0;
+                u.w_first = 0;
+                u.blk = layer + static_cast<size_t>(id) * block_size * row;
+                return;
+            }
+        }
+        u.valid = false;
+    };
+    auto next_of = [&](const Unit& u) -> Unit {
+        Unit n = u;
+        const unsigned mc = min(m_chunk, M - u.m0);
+        n.w_first = u.w_first + kThreads * kBatch;
+        if (n.w_first >= mc * ncg) {
+            n.w_first = 0;
+            n.m0 = u.m0 + m_chunk;
+            if (n.m0 >= M) { seek(n, u.item + gridDim.x); }
+        }
+        return n;
+    };
+    // unconditional: work items past the chunk's end reload its last one
+    auto load_unit = [&](u32x4 (&v)[kRepreUnroll], const Unit& u) {
+        const unsigned last = min(m_chunk, M - u.m0) * ncg - 1;
+#pragma unroll
+        for (unsigned j = 0; j < kBatch; ++j) {
+            const unsigned w = min(u.w_first + threadIdx.x + j * kThreads, last);
+            const unsigned ml = w / ncg, cg = w - ml * ncg;
+            const unsigned short* src = u.blk + static_cast<size_t>(u.m0 + ml) * kMerge * row + cg * 8;
+#pragma unroll
+            for (unsigned t = 0; t < kMerge; ++t) { v[j * kMerge + t] = ucm::gload16_nt(src + static_cast<size_t>(t) * row); }
+        }
+        asm volatile("" ::: "memory");                   // keeps the compiler from sinking the loads to their use
+    };
+    auto finish_unit = [&](const u32x4 (&v)[kRepreUnroll], const Unit& u) {
+        const unsigned mc = min(m_chunk, M - u.m0);
+#pragma unroll
+        for (unsigned j = 0; j < kBatch; ++j) {
+            const unsigned w = u.w_first + threadIdx.x + j * kThreads;
+            if (w < mc * ncg) {                          // (LDS only: a branch is harmless)
+                const unsigned ml = w / ncg, cg = w - ml * ncg;
+                float acc[8];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
+#pragma unroll
+                for (unsigned t = 0; t < kMerge; ++t) { add_bf16x8(acc, v[j * kMerge + t]); }
+                u32x4 o;
+                o.x = mean_to_f16x2(acc[0], acc[1], inv);
+                o.y = mean_to_f16x2(acc[2], acc[3], inv);
+                o.z = mean_to_f16x2(acc[4], acc[5], inv);
+                o.w = mean_to_f16x2(acc[6], acc[7], inv);
+                *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
+            }
+        }
+        if (u.w_first + kThreads * kBatch >= mc * ncg) { // the chunk is staged: write its pieces
+            __syncthreads();
+            unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride +
+                                  static_cast<size_t>(static_cast<unsigned>(slots[u.item])) * M * d_pad;
+            repre_write_pieces(stage, kept, pruned != nullptr, kv_heads, head_dim, d_pruned, pieces, srow_stride, M, u.m0, mc,
+                               out, head_stride);
+            __syncthreads();                             // the next chunk overwrites the staged means
+        }
+    };
+
+    Unit cur{0u, 0u, 0u, nullptr, true};
+    seek(cur, blockIdx.x);
+    if (!cur.valid) { return; }                          // the whole workgroup: the unit sequence is the same for all threads
+    u32x4 va[kRepreUnroll], vb[kRepreUnroll];
+    load_unit(va, cur);
+    for (;;) {
+        Unit nxt = next_of(cur);
+        load_unit(vb, nxt.valid ? nxt : cur);
+        finish_unit(va, cur);
+        if (!nxt.valid) { break; }
+        cur = nxt;
+        nxt = next_of(cur);
+        load_unit(va, nxt.valid ? nxt : cur);
+        finish_unit(vb, cur);
+        if (!nxt.valid) { break; }
+        cur = nxt;
+    }
+}
+
+// Any other number of tokens per sub-block: one workgroup per cache block, the tokens of a sub-block summed
+// sixteen loads at a time.  grid: x = cache block of the list, y = layer.
+__global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
     unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
     unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]: the 16 bytes of padding
-    const unsigned M = block_size / merge;                                   // spread the sub-blocks' rows over the LDS banks
+    extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]
+    const unsigned M = block_size / merge;
     const unsigned id = static_cast<unsigned>(block_ids[blockIdx.x]);
     const unsigned slot = static_cast<unsigned>(slots[blockIdx.x]);
     if (id >= num_blocks || slot >= rows) { return; }   // whole workgroup: never dereference a bad id
@@ -100,44 +253,12 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const float inv = 1.0f / static_cast<float>(merge);
     const unsigned pieces = d_pad / 8;
     unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<size_t>(slot) * M * d_pad;
-    // the channel lists, read once: a load from memory per output piece would queue behind the key stream
     int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
     if (pruned) {
         for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = pruned[e]; }
     }
     for (unsigned m0 = 0; m0 < M; m0 += m_chunk) {       // m_chunk sub-blocks at a time: what fits LDS
         const unsigned mc = min(m_chunk, M - m0);
-        if constexpr (kMerge > 0) {
-            constexpr unsigned kBatch = kRepreUnroll / kMerge;
-            for (unsigned w0 = threadIdx.x; w0 < mc * ncg; w0 += kThreads * kBatch) {
-                u32x4 v[kRepreUnroll];
-#pragma unroll
-                for (unsigned j = 0; j < kBatch; ++j) {
-                    const unsigned w = min(w0 + j * kThreads, mc * ncg - 1);   // clamped: loads stay unconditional
-                    const unsigned ml = w / ncg, cg = w - ml * ncg;
-                    const unsigned short* src = blk + static_cast<size_t>(m0 + ml) * kMerge * row + cg * 8;
-#pragma unroll
-                    for (unsigned t = 0; t < kMerge; ++t) { v[j * kMerge + t] = ucm::gload16_nt(src + static_cast<size_t>(t) * row); }
-                }
-#pragma unroll
-                for (unsigned j = 0; j < kBatch; ++j) {
-                    const unsigned w = w0 + j * kThreads;
-                    if (w >= mc * ncg) { break; }
-                    const unsigned ml = w / ncg, cg = w - ml * ncg;
-                    float acc[8];
-#pragma unroll
-                    for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }
-#pragma unroll
-                    for (unsigned t = 0; t < kMerge; ++t) { add_bf16x8(acc, v[j * kMerge + t]); }
-                    u32x4 o;
-                    o.x = mean_to_f16x2(acc[0], acc[1], inv);
-                    o.y = mean_to_f16x2(acc[2], acc[3], inv);
-                    o.z = mean_to_f16x2(acc[4], acc[5], inv);
-                    o.w = mean_to_f16x2(acc[6], acc[7], inv);
-                    *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
-                }
-            }
-        } else {
         for (unsigned w = threadIdx.x; w < mc * ncg; w += kThreads) {
             const unsigned ml = w / ncg, cg = w - ml * ncg;
             const unsigned short* src = blk + static_cast<size_t>(m0 + ml) * merge * row + cg * 8;
@@ -160,34 +281,9 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
             o.w = mean_to_f16x2(acc[6], acc[7], inv);
             *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
         }
-        }
         __syncthreads();
-        for (unsigned e = threadIdx.x; e < kv_heads * pieces * mc; e += kThreads) {
-            const unsigned h = e / (pieces * mc), rem = e - h * (pieces * mc);
-            const unsigned piece = rem / mc, ml = rem - piece * mc;
-            const unsigned short* srow = stage + ml * srow_stride + h * head_dim;
-            u32x4 o;
-            if (!pruned && piece * 8 + 8 <= d_pruned) {  // all channels kept: the piece is 16 contiguous bytes
-                o = *reinterpret_cast<const u32x4*>(srow + piece * 8);
-            } else {
-                unsigned short c[8];
-#pragma unroll
-                for (unsigned j = 0; j < 8; ++j) {
-                    const unsigned p = piece * 8 + j;
-                    unsigned short v = 0;
-                    if (p < d_pruned) {
-                        const unsigned d = pruned ? static_cast<unsigned>(kept[h * d_pruned + p]) : p;
-                        if (d < head_dim) { v = srow[d]; }
-                    }
-                    c[j] = v;
-                }
-                o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
-                o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
-                o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
-                o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
-            }
-            ucm::gstore16(out + static_cast<int64_t>(h) * head_stride + (static_cast<size_t>(piece) * M + m0 + ml) * 8, o);
-        }
+        repre_write_pieces(stage, kept, pruned != nullptr, kv_heads, head_dim, d_pruned, pieces, srow_stride, M, m0, mc, out,
+                           head_stride);
         __syncthreads();                                 // the next chunk overwrites the staged means
     }
 }
@@ -788,6 +884,9 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     const size_t lds_bytes = static_cast<size_t>(m_chunk) * (row + 8) * 2 + (pruned ? static_cast<size_t>(kv_heads) * d_pruned * 4 : 0);
     UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_layer_stride % 8 == 0 && repre_head_stride % 8 == 0,
                 "ucm_kvstar_block_repre: table not 16-byte aligned");
+    hipStream_t hs = ucm::as_stream(stream);
+    // persistent workgroups for the common sub-block sizes: about 1024 over all layers (two fit a compute unit)
+    const unsigned gx = static_cast<unsigned>(std::min(n, std::max(1, (1024 + n_layers - 1) / n_layers)));
 #define UCM_KVSTAR_REPRE(MERGE)                                                                                        \
     do {                                                                                                             \
         if (lds_bytes > 48u * 1024u) {                                                                               \
@@ -796,11 +895,11 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                                                       static_cast<int>(lds_bytes));                                \
             if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }                \
         }                                                                                                            \
-        hipLaunchKernelGGL(kvstar_repre_kernel<MERGE>, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, \
-                           ucm::as_stream(stream), k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),    \
+        hipLaunchKernelGGL(kvstar_repre_kernel<MERGE>, dim3(gx, n_layers), dim3(kThreads), lds_bytes, hs, k_layers,  \
+                           block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(n),            \
                            static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),                     \
-                           static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), static_cast<unsigned>(merge), \
-                           pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),                    \
+                           static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), pruned,                 \
+                           static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),                            \
                            static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk); \
     } while (0)
     switch (merge) {
@@ -808,7 +907,18 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     case 2: UCM_KVSTAR_REPRE(2); break;
     case 4: UCM_KVSTAR_REPRE(4); break;
     case 8: UCM_KVSTAR_REPRE(8); break;
-    default: UCM_KVSTAR_REPRE(0); break;
+    default:
+        if (lds_bytes > 48u * 1024u) {
+            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_any_kernel),
+                                                      hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+            if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }
+        }
+        hipLaunchKernelGGL(kvstar_repre_any_kernel, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, hs,
+                           k_layers, block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(repre_rows),
+                           static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim),
+                           static_cast<unsigned>(merge), pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),
+                           static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk);
+        break;
     }
 #undef UCM_KVSTAR_REPRE
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
