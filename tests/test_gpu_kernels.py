@@ -371,9 +371,9 @@ def test_topk_many_requests_with_ties(ucm, dev, sw, ew):
         assert np.array_equal(idx[r, : cnt[r]], want), (r, len(sc), ks[r], sc)
 
 
-@pytest.mark.parametrize("n", [64, 65, 256, 257, 1024, 1025, 4096])
+@pytest.mark.parametrize("n", [64, 65, 128, 129, 256, 257, 512, 513, 1024, 1025, 2048, 2049, 4096])
 def test_topk_register_tiers(ucm, dev, n):
-    """Each register tier of the selection kernel (64 / 256 / 1024 / 4096 blocks per request)."""
+    """Each register tier of the selection kernel (64, 128, ... 4096 blocks per request) at both of its ends."""
     from ucm_amd import ops
 
     sc = synth.normal_f32(90 + n, (n,))

@@ -153,9 +153,14 @@ extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride
     hipLaunchKernelGGL(topk_windows_kernel<EPL>, grid, block, 0, s, scores, scores_layer_stride, seg_off,    \
                        seg_len, topk_len, n_req, start_w, end_w, idx_out, out_stride, count_out, block_tables, \
                        bt_stride, phys_out, seq_lens, block_size, sparse_seq_lens)
+    // registers per lane for the keys: the smallest tier that holds the longest request (the radix steps cost
+    // one ballot per register and bit)
     if (max_seg_len <= 64) { UCM_TOPK_LAUNCH(1); }
+    else if (max_seg_len <= 128) { UCM_TOPK_LAUNCH(2); }
     else if (max_seg_len <= 256) { UCM_TOPK_LAUNCH(4); }
+    else if (max_seg_len <= 512) { UCM_TOPK_LAUNCH(8); }
     else if (max_seg_len <= 1024) { UCM_TOPK_LAUNCH(16); }
+    else if (max_seg_len <= 2048) { UCM_TOPK_LAUNCH(32); }
     else { UCM_TOPK_LAUNCH(64); }
 #undef UCM_TOPK_LAUNCH
     UCM_LAUNCH_CHECK("ucm_topk_windows");
