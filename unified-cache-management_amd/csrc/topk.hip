@@ -72,11 +72,13 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
         const int hi = n - end_w;                // candidates are start_w <= i < hi
         const float* s = scores + static_cast<int64_t>(l) * scores_layer_stride + seg_off[r];
         unsigned key[kEpl];
-#pragma unroll
+        int32_t phys[kEpl];                      // the block table's entries, fetched with the scores: a load per
+#pragma unroll                                   // taken element on the way out would cost a memory round trip per register
         for (int j = 0; j < kEpl; ++j) {
             const int i = j * 64 + lane;
             const bool cand = i >= start_w && i < hi;
             key[j] = cand ? ordered_key(s[cand ? i : 0]) : 0u;
+            phys[j] = bt ? bt[min(i, n - 1)] : 0;
         }
         unsigned T = 0;
         int need = 0;
@@ -109,7 +111,7 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
                 if (take) {
                     const int p = pos + static_cast<int>(lanes_below(take_mask));
                     out[p] = i;
-                    if (pout) { pout[p] = bt[i]; }
+                    if (pout) { pout[p] = phys[j]; }
                 }
                 pos += __popcll(take_mask);
             }
