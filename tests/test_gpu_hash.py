@@ -196,6 +196,31 @@ def test_config5_full_size_negated_keys_give_complement_codes(ucm, dev):
     print("exact zero projections met:", exact_zeros)
 
 
+@pytest.mark.parametrize("hq,hkv", [(64, 8), (128, 8), (8, 8), (28, 4), (6, 2), (40, 1)])
+def test_hash_query_codes_for_other_head_counts(ucm, dev, hq, hkv):
+    """Query codes, their +-1 sums and the group-mean codes for head counts that take one chunk of staged
+    vectors, several, and a last chunk that is not full (the kernel stages forty vectors at a time)."""
+    from ucm_amd import ops
+
+    n_layers, n_req = 2, 3
+    w_bits, w_f32 = make_weights(840)
+    q_h = synth.normal_bf16_bits(841 + hq, (n_layers, n_req, hq, 128))
+    q_h[0, 1, 0, :] = 0                                        # an all-zero query: every projection is 0, every bit 0
+    q_codes = torch.full((n_layers, n_req, hq, 16), 0xEE, dtype=torch.uint8, device=dev)
+    q_sum = torch.full((n_layers, n_req, 128), 77, dtype=torch.int16, device=dev)
+    qbar = torch.full((n_layers, n_req, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(bf16_dev(q_h, dev), bf16_dev(w_bits, dev), hkv, q_codes, q_sum, qbar, n_req)
+    torch.cuda.synchronize()
+    for l in range(n_layers):
+        want_q = O.hash_encode(q_h[l], w_f32)
+        assert np.array_equal(q_codes[l].cpu().numpy(), want_q), l
+        pm = np.unpackbits(want_q, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
+        assert np.array_equal(q_sum[l].cpu().numpy(), pm.sum(1)), l
+        qm = np.stack([O.q_head_mean(synth.bf16_widen(q_h[l][r]), hkv) for r in range(n_req)])
+        assert np.array_equal(qbar[l].cpu().numpy(), O.hash_encode_f32(qm, w_f32)), l
+    assert not q_codes[0, 1, 0].any()
+
+
 def test_hash_queries_scores_and_selection(ucm, dev):
     """Config-5 shape in small: ragged batch, 8 kv heads, 32 query heads, 2 layers."""
     from ucm_amd import ops

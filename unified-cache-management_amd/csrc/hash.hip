@@ -456,16 +456,20 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     }
 }
 
-// Query side, one workgroup of 1024 threads per (request, layer): thread
-// (bit c, head group hg) projects heads hg, hg+8, ... exactly (fp64, d
-// ascending; there are only q_heads*128 such dot products), the +-1 sum over
-// all heads is combined through LDS, and each head group also produces the code
-// of the group-mean query of kv heads hg, hg+8, ...  W and the request's query
-// rows are staged in LDS once.
+// Query side, one workgroup of 1024 threads per (request, layer).  The vectors to project are the
+// request's q_heads query rows and the kv_heads group-mean queries (fp32 sequential adds * (1/g), the
+// scoring path's own mean); every projection is exact: fp64, d ascending (a product of two bf16 values
+// is exact in fp64 and so, for these magnitudes, is the sum).  Thread (bit c, group hg) owns column c of
+// W - 128 bf16 values held in 64 registers for the whole kernel - and projects vectors hg, hg+8, ...;
+// the vectors are staged in LDS as fp64, forty at a time, and read back two at a time as wave-wide
+// broadcasts; eight weights are widened to fp64 at a time and used for the thread's five vectors of the
+// chunk, so the inner loop is little more than one fp64 fma per vector and dimension.  The +-1 sum over
+// all heads is combined through LDS.
 // grid: x = request, y = layer
 constexpr int kQueryGroups = 8;
 constexpr int kQueryThreads = kBits * kQueryGroups;
 constexpr int kMaxQHeads = 128;
+constexpr int kQueryRows = 40;          // vectors staged at a time (a multiple of the groups): 40 KiB of fp64
 
 __global__ __launch_bounds__(kQueryThreads) void hash_query_kernel(
     const unsigned short* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows,
@@ -473,56 +477,102 @@ __global__ __launch_bounds__(kQueryThreads) void hash_query_kernel(
     unsigned* __restrict__ q_codes /*[L][n_req][q_heads][4]*/, short* __restrict__ q_sum /*[L][n_req][128]*/,
     unsigned* __restrict__ qbar_codes /*[L][n_req][kv_heads][4]*/)
 {
-    __shared__ unsigned short w_s[kDim * kBits];            // [d][c]: lanes read consecutive c
-    __shared__ unsigned short q_s[kMaxQHeads * kDim];
-    __shared__ int part[kQueryGroups][kBits];
+    extern __shared__ __attribute__((aligned(16))) unsigned char query_lds[];
+    double* rows_d = reinterpret_cast<double*>(query_lds);                                       // [kQueryRows][kDim]
+    unsigned short* wt_s = reinterpret_cast<unsigned short*>(rows_d + kQueryRows * kDim);       // [c][d], rows kWtStride apart
+    int* part = reinterpret_cast<int*>(wt_s + kBits * kWtStride);                               // [kQueryGroups][kBits]
 
     const unsigned r = blockIdx.x, l = blockIdx.y;
     const unsigned c = threadIdx.x % kBits, hg = threadIdx.x / kBits;
     const unsigned short* qp = q + static_cast<int64_t>(l) * q_layer_stride +
                                static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kDim;
-    for (unsigned e = threadIdx.x; e < kDim * kBits; e += kQueryThreads) { w_s[e] = w[e]; }
-    for (unsigned e = threadIdx.x; e < q_heads * kDim; e += kQueryThreads) { q_s[e] = qp[e]; }
+    // W transposed, so that a thread's column is sixteen 16-byte reads
+    for (unsigned e = threadIdx.x; e < kDim * kBits; e += kQueryThreads) {
+        wt_s[(e % kBits) * kWtStride + e / kBits] = w[e];
+    }
     __syncthreads();
+    u32x4 wcol[kDim / 8];
+#pragma unroll
+    for (int k = 0; k < kDim / 8; ++k) { wcol[k] = *reinterpret_cast<const u32x4*>(&wt_s[c * kWtStride + k * 8]); }
 
     const size_t lr = static_cast<size_t>(l) * n_req + r;
     const unsigned g = q_heads / kv_heads;
-    int sum = 0;
-    for (unsigned i = hg; i < q_heads; i += kQueryGroups) {
-        double acc = 0.0;
-        for (int d = 0; d < kDim; ++d) {
-            acc += static_cast<double>(bf16_to_f32(q_s[i * kDim + d])) * static_cast<double>(bf16_to_f32(w_s[d * kBits + c]));
-        }
-        const bool pos = acc > 0.0;
-        sum += pos ? 1 : -1;
-        const unsigned long long m = __ballot(pos);      // a wave covers 64 consecutive bits of one head
-        if ((c & 63) == 0) {
-            q_codes[(lr * q_heads + i) * 4 + (c >> 6) * 2] = static_cast<unsigned>(m);
-            q_codes[(lr * q_heads + i) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(m >> 32);
-        }
-    }
-    part[hg][c] = sum;
-    // group-mean query: fp32 sequential adds * (1/g), the scoring path's own mean, then projected exactly
     const float inv = 1.0f / static_cast<float>(g);
-    for (unsigned h = hg; h < kv_heads; h += kQueryGroups) {
-        double acc = 0.0;
-        for (int d = 0; d < kDim; ++d) {
-            float m = bf16_to_f32(q_s[(h * g) * kDim + d]);
-            for (unsigned j = 1; j < g; ++j) { m = m + bf16_to_f32(q_s[(h * g + j) * kDim + d]); }
-            if (g != 1) { m = m * inv; }
-            acc += static_cast<double>(m) * static_cast<double>(bf16_to_f32(w_s[d * kBits + c]));
+    const unsigned n_vec = q_heads + kv_heads;          // the query rows, then the group means
+    int sum = 0;
+    for (unsigned v0 = 0; v0 < n_vec; v0 += kQueryRows) {
+        const unsigned nv = min(static_cast<unsigned>(kQueryRows), n_vec - v0);
+        __syncthreads();                                // the chunk before has been read
+        for (unsigned e = threadIdx.x; e < nv * kDim; e += kQueryThreads) {
+            const unsigned v = v0 + e / kDim, d = e % kDim;
+            float x;
+            if (v < q_heads) {
+                x = bf16_to_f32(qp[v * kDim + d]);
+            } else {
+                const unsigned h = v - q_heads;
+                x = bf16_to_f32(qp[(h * g) * kDim + d]);
+                for (unsigned j = 1; j < g; ++j) { x = x + bf16_to_f32(qp[(h * g + j) * kDim + d]); }
+                if (g != 1) { x = x * inv; }
+            }
+            rows_d[e] = static_cast<double>(x);
         }
-        const unsigned long long mk = __ballot(acc > 0.0);
-        if ((c & 63) == 0) {
-            qbar_codes[(lr * kv_heads + h) * 4 + (c >> 6) * 2] = static_cast<unsigned>(mk);
-            qbar_codes[(lr * kv_heads + h) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(mk >> 32);
+        __syncthreads();
+        // eight weights of the column widened at a time and used for all of the thread's vectors of this chunk
+        constexpr int kMine = kQueryRows / kQueryGroups;
+        double acc[kMine];
+#pragma unroll
+        for (int vi = 0; vi < kMine; ++vi) { acc[vi] = 0.0; }
+#pragma unroll
+        for (int k = 0; k < kDim / 8; ++k) {
+            // (the empty asm keeps the compiler from widening the whole column to fp64 ahead of the chunk loop,
+            // which would take 256 registers)
+            asm volatile("" : "+v"(wcol[k]));
+            double wd[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                wd[2 * j] = static_cast<double>(__uint_as_float(wcol[k][j] << 16));
+                wd[2 * j + 1] = static_cast<double>(__uint_as_float(wcol[k][j] & 0xffff0000u));
+            }
+#pragma unroll
+            for (int vi = 0; vi < kMine; ++vi) {
+                // the same address in every lane: broadcast reads; a vector past the chunk's end re-reads the last one
+                const double* x = rows_d + min(hg + vi * kQueryGroups, nv - 1) * kDim + k * 8;
+                // (the products are exact in fp64 - at most 24 + 8 significant bits - so the fused form rounds
+                // exactly like a multiplication followed by an addition; d ascending per vector)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) { acc[vi] = __builtin_fma(x[j], wd[j], acc[vi]); }
+                __builtin_amdgcn_sched_barrier(0);      // one vector's reads at a time: with all of a step's up front the
+            }                                           // 128 registers a thread of a 1024-thread workgroup has do not suffice
+        }
+        // (used here whatever follows: otherwise the compiler moves each vector's whole fma chain down into the
+        // conditional code below and keeps every operand alive until then)
+#pragma unroll
+        for (int vi = 0; vi < kMine; ++vi) { asm volatile("" : "+v"(acc[vi])); }
+#pragma unroll
+        for (int vi = 0; vi < kMine; ++vi) {
+            const unsigned vl = hg + vi * kQueryGroups;
+            if (vl >= nv) { break; }                    // (the same for a whole wave)
+            const bool pos = acc[vi] > 0.0;
+            const unsigned long long m = __ballot(pos);  // a wave covers 64 consecutive bits of one vector
+            const unsigned v = v0 + vl;
+            if (v < q_heads) {
+                sum += pos ? 1 : -1;
+                if ((c & 63) == 0) {
+                    q_codes[(lr * q_heads + v) * 4 + (c >> 6) * 2] = static_cast<unsigned>(m);
+                    q_codes[(lr * q_heads + v) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(m >> 32);
+                }
+            } else if ((c & 63) == 0) {
+                qbar_codes[(lr * kv_heads + (v - q_heads)) * 4 + (c >> 6) * 2] = static_cast<unsigned>(m);
+                qbar_codes[(lr * kv_heads + (v - q_heads)) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(m >> 32);
+            }
         }
     }
+    part[hg * kBits + c] = sum;
     __syncthreads();
     if (hg == 0) {
         int total = 0;
 #pragma unroll
-        for (int k = 0; k < kQueryGroups; ++k) { total += part[k][c]; }
+        for (int k = 0; k < kQueryGroups; ++k) { total += part[k * kBits + c]; }
         q_sum[lr * kBits + c] = static_cast<short>(total);
     }
 }
@@ -653,7 +703,14 @@ extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_strid
     UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0,
                 "ucm_hash_encode_queries: q_heads=%d kv_heads=%d", q_heads, kv_heads);
     UCM_SUPPORTED(q_heads <= kMaxQHeads, "ucm_hash_encode_queries: q_heads=%d (at most %d)", q_heads, kMaxQHeads);
-    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),
+    constexpr size_t kQueryLds = kQueryRows * kDim * sizeof(double) + kBits * kWtStride * 2 + kQueryGroups * kBits * sizeof(int);
+    static_assert(kQueryLds <= 80 * 1024, "two query workgroups per compute unit");
+    if (const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(hash_query_kernel),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kQueryLds));
+        ea != hipSuccess) {
+        return ucm::check_hip(ea, "ucm_hash_encode_queries (LDS size)");
+    }
+    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), kQueryLds, ucm::as_stream(stream),
                        static_cast<const unsigned short*>(q_bf16), q_layer_stride, q_rows,
                        static_cast<unsigned>(q_heads), static_cast<unsigned>(kv_heads),
                        static_cast<const unsigned short*>(w_bf16), static_cast<unsigned>(n_req),
