@@ -14,8 +14,20 @@ from . import _lib
 from ._lib import MEAN_BF16_ROUND, MEAN_BF16_STORE, MEAN_F32, UcmHipError  # noqa: F401
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    """torch's current stream on the current device as a raw handle.  The plugins call this twice per layer
+    and decode step; building a torch.cuda.Stream object each time costs ~8 us, the raw query ~0.3 us."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
+
+
+def current_stream() -> int:
+    """Raw handle of torch's current stream, for callers that go to the library themselves."""
+    return _stream()
 
 
 def _dev(t: torch.Tensor, dtype, name: str) -> int:

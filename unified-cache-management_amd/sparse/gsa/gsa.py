@@ -30,7 +30,7 @@ from typing import Dict, List, Optional, Union
 
 import torch
 
-from ... import ops
+from ... import _lib, ops
 from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
 from ..utils import (
     INIT_WINDOW_BLOCKS,
@@ -186,6 +186,16 @@ class GSA(UcmSparseBase):
         cap = (5 + 3 * self.max_block_len) * self.max_bs
         self._host_desc = [torch.zeros(cap, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self._host_free = [None, None]  # event recorded after each buffer's last upload
+        # attention_begin runs once per layer and decode step: it goes to the library with addresses computed
+        # here and in execute_begin instead of slicing six tensors and re-validating them every time (the
+        # shapes are this plugin's own and do not change)
+        self._layer_addr = [
+            (self.kpre_caches[l].data_ptr(), self.scores[l].data_ptr(), self.topk_caches[l].data_ptr(),
+             self.topk_counts[l].data_ptr(), self.block_tables_mp[l].data_ptr(), self.gsa_seq_len[l].data_ptr())
+            for l in range(L)
+        ]
+        self._repre_code = _lib.DTYPE_BF16 if self.repre_dtype == torch.bfloat16 else _lib.DTYPE_F32
+        self._views: Dict[int, list] = {}  # batch size -> per-layer (block table, sequence lengths) views
         self._dev_ready = True
 
     def register_kv_caches(self, kv_caches: dict) -> None:
@@ -262,24 +272,24 @@ class GSA(UcmSparseBase):
         if self._host_free[slot] is not None:
             self._host_free[slot].synchronize()  # upload of two steps ago; long finished
         host = self._host_desc[slot][: 5 * batch + batch * width + 2 * n_calc]
-        host.zero_()
-        desc = host[: 5 * batch].view(5, batch)
-        tables = host[5 * batch : 5 * batch + batch * width].view(batch, width)
+        hn = host.numpy()                    # the same pinned memory; numpy fills it several times faster than torch indexing
+        hn[:] = 0
+        desc = hn[: 5 * batch].reshape(5, batch)
+        tables = hn[5 * batch : 5 * batch + batch * width].reshape(batch, width)
         max_len = total = 0
+        query_locals = self.model_input["query_locals"]
         for i, st in enumerate(by_index):
             if st is None:
                 continue
             n = len(st.blocks)
-            desc[0, i], desc[1, i] = st.slot_offset, n
             k = compute_topk_len(n, self.min_topk, self.max_topk, self.topk_ratio) if st.is_gsa() else n
-            desc[2, i] = max(k, 1)          # k >= n keeps every block (short or prefilling requests)
-            desc[3, i] = self.model_input["query_locals"][i + 1] - 1
-            desc[4, i] = st.get_seq_len()
-            tables[i, :n] = torch.tensor(st.blocks, dtype=torch.int32)
+            # k >= n keeps every block (short or prefilling requests)
+            desc[:, i] = (st.slot_offset, n, max(k, 1), query_locals[i + 1] - 1, st.get_seq_len())
+            tables[i, :n] = st.blocks
             max_len, total = max(max_len, n), total + n
-        tail = host[5 * batch + batch * width :]
-        tail[:n_calc] = torch.tensor(self.model_input["calc_block_table"], dtype=torch.int32)
-        tail[n_calc:] = torch.tensor(self.model_input["calc_repre_slot_mapping"], dtype=torch.int32)
+        tail = hn[5 * batch + batch * width :]
+        tail[:n_calc] = self.model_input["calc_block_table"]
+        tail[n_calc:] = self.model_input["calc_repre_slot_mapping"]
         dev = host.to(self.device, non_blocking=True)
         self._host_free[slot] = torch.cuda.Event()
         self._host_free[slot].record()
@@ -291,6 +301,8 @@ class GSA(UcmSparseBase):
             calc_slots_dev=dev[5 * batch + batch * width + n_calc :],
             max_len=max_len, total=total, n_batch=batch,
         )
+        self.model_input["addr"] = (d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), d[4].data_ptr(),
+                                    self.model_input["block_tables"].data_ptr())
 
     def execute_finished(self) -> None:
         self.step_count += 1
@@ -303,21 +315,31 @@ class GSA(UcmSparseBase):
             return
         l = int(layer_name.split(".")[2])
         n = mi["n_batch"]
+        seg_off, seg_len, topk_len, q_rows, seq_lens, tables = mi["addr"]
+        repre, scores, idx, counts, phys, sparse_len = self._layer_addr[l]
+        stream = ops.current_stream()
         if mi["is_topk"]:
-            q = query.view(1, query.shape[0], self.num_q_heads, self.head_size)
-            ops.score_blocks(q, self.kpre_caches[l : l + 1], mi["seg_off"], mi["seg_len"], mi["max_len"],
-                             self.num_key_heads, self.scores[l : l + 1], q_rows=mi["q_rows"],
-                             total_blocks=mi["total"])
+            if query.dtype == torch.bfloat16:
+                q_code = _lib.DTYPE_BF16
+            elif query.dtype == torch.float32:
+                q_code = _lib.DTYPE_F32
+            else:
+                raise ValueError("query must be bfloat16 or float32")
+            if not (query.is_cuda and query.is_contiguous()) or query.shape[-1] != self.head_size:
+                raise ValueError("query must be a contiguous device tensor [tokens, q_heads, head_size]")
+            _lib.call("ucm_score_blocks", query.data_ptr(), q_code, query.numel(), q_rows, self.num_q_heads, repre,
+                      self._repre_code, self.kpre_caches.stride(0), seg_off, seg_len, n, mi["max_len"], mi["total"], 1,
+                      self.num_key_heads, self.head_size, scores, self.scores.stride(0), stream)
         # selection (fresh scores, or the last ones with this step's lengths), block-table lookup, sparse lengths
-        ops.topk_windows(self.scores[l : l + 1], mi["seg_off"], mi["seg_len"], mi["topk_len"], mi["max_len"],
-                         self.topk_caches[l : l + 1, :n], self.topk_counts[l : l + 1, :n],
-                         start_w=self.init_window, end_w=self.local_window, block_tables=mi["block_tables"],
-                         phys_out=self.block_tables_mp[l : l + 1, :n], seq_lens=mi["seq_lens"],
-                         block_size=self.block_size, sparse_seq_lens=self.gsa_seq_len[l : l + 1, :n])
+        _lib.call("ucm_topk_windows", scores, self.scores.stride(0), seg_off, seg_len, topk_len, n, mi["max_len"], 1,
+                  self.init_window, self.local_window, idx, self.max_block_len, counts, tables, self.max_block_len, phys,
+                  seq_lens, self.block_size, sparse_len, stream)
+        views = self._views.get(n)
+        if views is None:
+            views = self._views[n] = [(self.block_tables_mp[k, :n], self.gsa_seq_len[k, :n]) for k in range(self.layer_num)]
         md = forward_context.attn_metadata
         md = md[layer_name] if isinstance(md, dict) else md
-        md.block_table = self.block_tables_mp[l, :n]
-        md.seq_lens = self.gsa_seq_len[l, :n]
+        md.block_table, md.seq_lens = views[l]
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
         self.maybe_register_kv_cache(forward_context, layer_name)
