@@ -55,6 +55,9 @@ def parse():
                          "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
     ap.add_argument("--hash-leg", action="store_true",
                     help="also time the hash-code retrieval variant (the configs[4] shape of the benchmark definition) on the same caches")
+    ap.add_argument("--moves-leg", action="store_true",
+                    help="also time the block-id driven load/dump (the configs[2] shape of the benchmark definition: 64 requests "
+                         "x 16 blocks, all layers, K and V, random block table) on the same caches")
     ap.add_argument("--kvstar-leg", action="store_true",
                     help="also time the multi-query softmax-vote retrieval (KVStar: 8 query tokens per request) on the same "
                          "ragged batch")
@@ -244,6 +247,38 @@ def main():
 
     # ---- hash-code retrieval leg (configs[4]): 32 requests of 64-256 blocks, 32 layers, 128-bit codes.
     # The key blocks are the K and V planes of the caches above read as one pool of 2*nb blocks.
+    # ---- load/dump leg: 1024 random blocks of every layer between the paged cache and a staging buffer in the
+    # stored-block order [block][layer][K|V]; the scatter writes what the gather read, so the cache is unchanged
+    moves_leg = None
+    if args.moves_leg:
+        m_blocks = 64 * 16
+        m_ids = i32(rng.permutation(nb)[:m_blocks])
+        m_stage = torch.empty(m_blocks * n_layers * 2 * BLOCK_BYTES, dtype=torch.uint8, device=dev)
+
+        def timed_move(fn, reps=10):
+            fn()
+            torch.cuda.synchronize()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / reps
+
+        gather_ms = timed_move(lambda: ops.kv_gather_blocks(layers, kv_stride, BLOCK_BYTES, nb, m_ids, m_stage))
+        scatter_ms = timed_move(lambda: ops.kv_scatter_blocks(layers, kv_stride, BLOCK_BYTES, nb, m_ids, m_stage))
+        move_bytes = 2 * m_blocks * n_layers * 2 * BLOCK_BYTES
+        moves_leg = {
+            "workload": f"configs[2]: {m_blocks} blocks x {n_layers} layers x (K, V) x {BLOCK_BYTES} B, random block table over "
+                        f"{nb} blocks per layer",
+            "algorithmic_bytes": move_bytes,
+            "gather_ms": round(gather_ms, 3), "scatter_ms": round(scatter_ms, 3),
+            "gather_GBps": round(gbs(move_bytes, gather_ms), 1), "scatter_GBps": round(gbs(move_bytes, scatter_ms), 1),
+            "frac": [round(gbs(move_bytes, gather_ms) / HBM_PEAK_GBS, 4), round(gbs(move_bytes, scatter_ms) / HBM_PEAK_GBS, 4)],
+        }
+        del m_stage
+
     hash_leg = None
     if args.hash_leg:
         h_req = 32
@@ -551,6 +586,7 @@ def main():
         "block_mean_prefill": {"ms": round(mean_ms, 3), "GBps": round(gbs(mean_bytes, mean_ms), 1),
                                "frac": round(gbs(mean_bytes, mean_ms) / HBM_PEAK_GBS, 4)},
         "delta_gather": delta,
+        "kv_moves": moves_leg,
         "hash_retrieval": hash_leg,
         "kvstar_retrieval": kvstar_leg,
         "cpu_baseline": cpu,
