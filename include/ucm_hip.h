@@ -390,9 +390,10 @@ int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t 
  *                               dArr[i].  Both arrays are HOST arrays of
  *                               addresses (as in the reference); the host
  *                               addresses must be pinned memory (this object's
- *                               buffers are), every address and `count` a multiple
- *                               of 16.  One launch of the ucm_copy_batch kernel on
- *                               the object's stream, then a wait.
+ *                               buffers are).  One launch of the ucm_copy_batch
+ *                               kernel on the object's stream, then a wait; if
+ *                               `count` or an address is not a multiple of 16,
+ *                               one runtime copy per pair instead.
  * ucm_device_stream             the object's stream, for callers that order
  *                               their own kernels against the copies.
  *

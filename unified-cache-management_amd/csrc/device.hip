@@ -41,9 +41,21 @@ int batch(ucm_device* dev, void* const* dst_host_array, const void* const* src_h
           const char* what)
 {
     UCM_REQUIRE(dev && (number == 0 || (dst_host_array && src_host_array)), "%s: null argument", what);
-    UCM_REQUIRE(count % 16 == 0, "%s: count=%zu must be a multiple of 16", what, count);
     if (number == 0 || count == 0) { return UCM_OK; }
     if (int rc = ucm::check_hip(hipSetDevice(dev->device_id), what)) { return rc; }
+    bool vector_ok = count % 16 == 0;
+    for (size_t i = 0; vector_ok && i < number; ++i) {
+        vector_ok = ucm::aligned16(dst_host_array[i]) && ucm::aligned16(src_host_array[i]);
+    }
+    if (!vector_ok) {
+        // sizes or addresses the 16-byte copy kernel cannot take: one runtime copy per pair, same stream, same wait
+        for (size_t i = 0; i < number; ++i) {
+            if (int rc = ucm::check_hip(hipMemcpyAsync(dst_host_array[i], src_host_array[i], count, hipMemcpyDefault, dev->stream), what)) {
+                return rc;
+            }
+        }
+        return ucm::check_hip(hipStreamSynchronize(dev->stream), what);
+    }
     std::lock_guard<std::mutex> guard(dev->lock);   // one batch at a time shares the pointer scratch
     if (number > dev->ptr_capacity) {
         if (dev->ptr_arrays) {
