@@ -444,12 +444,15 @@ int ucm_kv_scatter_blocks(void* const* layers, int n_layers, size_t kv_stride, s
  * tensor view at a time (esa.py:254-258).
  *   phys   dev int32[n_layers][n_req][phys_stride], count dev int32[n_layers][n_req]
  *   dst_off dev int64[n_req], region_k dev int32[n_req]; max_count >= every count.
+ *   staging_blocks  blocks the staging buffer holds: dst_off and region_k live
+ *                   in device memory, where the host cannot check them, so a
+ *                   destination at or past this bound is skipped, never written.
  */
 int ucm_kv_gather_selected(const void* const* layers, int n_layers, size_t kv_stride,
                            size_t block_bytes, int num_blocks, const int32_t* phys,
                            const int32_t* count, int n_req, int phys_stride, const int64_t* dst_off,
                            const int32_t* region_k, int max_count, void* staging,
-                           ucm_stream_t stream);
+                           int64_t staging_blocks, ucm_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -469,6 +469,24 @@ def test_gather_selected_matches_oracle(ucm, dev):
     O.kv_gather_selected(hs, nb * bb, bb, phys, count, dst_off, region, want)
     assert np.array_equal(staging.cpu().numpy(), want)
 
+    # offsets that point past the staging buffer (they live in device memory, where the host cannot check them):
+    # those destinations are skipped, everything else is written as before, nothing outside is touched
+    guard = torch.full(((total + 4) * bb,), 0xCD, dtype=torch.uint8, device=dev)
+    short = total - int(region[-1]) * 2                              # the last request's last layer does not fit
+    bad_off = dst_off.copy()
+    bad_off[0] = -5                                                   # and the first request points before the buffer
+    ops.kv_gather_selected(lp, nb * bb, bb, nb, i32(phys, dev), i32(count, dev),
+                           torch.from_numpy(bad_off).to(dev), i32(region, dev), int(count.max()), guard[: short * bb], short)
+    got = guard.cpu().numpy()
+    assert np.all(got[short * bb :] == 0xCD)
+    first_len = int(region[0]) * n_layers * 2 * bb
+    assert np.all(got[:first_len] == 0xCD)                            # request 0 was skipped entirely
+    other = np.full(total * bb, 0x12, np.uint8)                       # a second background tells written bytes from the fill
+    O.kv_gather_selected(hs, nb * bb, bb, phys, count, dst_off, region, other)
+    written = (want == other)[first_len : short * bb]
+    assert written.any() and np.array_equal(got[first_len : short * bb][written], want[first_len : short * bb][written])
+    assert np.all(got[first_len : short * bb][~written] == 0xCD)
+
 
 def test_retrieval_then_gather_end_to_end(ucm, dev):
     """Config-2 shape in small: means -> scores -> selection -> gather, no host round trip in between."""

@@ -48,7 +48,7 @@ SIGNATURES = {
     "ucm_device_stream": [_p],
     "ucm_kv_gather_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
     "ucm_kv_scatter_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
-    "ucm_kv_gather_selected": [_p, _i, _sz, _sz, _i, _p, _p, _i, _i, _p, _p, _i, _p, _p],
+    "ucm_kv_gather_selected": [_p, _i, _sz, _sz, _i, _p, _p, _i, _i, _p, _p, _i, _p, _i64, _p],
 }
 
 

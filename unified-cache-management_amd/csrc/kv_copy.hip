@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kThreads) void kv_gather_selected_kernel(
     const void* const* __restrict__ layers, size_t kv_stride, size_t block_bytes,
     const int32_t* __restrict__ phys, const int32_t* __restrict__ count, unsigned num_blocks,
     unsigned n_req, unsigned phys_stride, const int64_t* __restrict__ dst_off,
-    const int32_t* __restrict__ region_k, uint8_t* __restrict__ staging)
+    const int32_t* __restrict__ region_k, uint8_t* __restrict__ staging, uint64_t staging_blocks)
 {
     const unsigned j = blockIdx.x, r = blockIdx.y, l = blockIdx.z >> 1, kv = blockIdx.z & 1;
     const size_t lr = static_cast<size_t>(l) * n_req + r;
@@ -89,9 +89,11 @@ __global__ __launch_bounds__(kThreads) void kv_gather_selected_kernel(
     if (id >= num_blocks) { return; }
     const uint8_t* src = static_cast<const uint8_t*>(layers[l]) + kv * kv_stride +
                          static_cast<size_t>(id) * block_bytes;
-    uint8_t* dst = staging + (static_cast<size_t>(dst_off[r]) +
-                              (static_cast<size_t>(l) * 2 + kv) * region_k[r] + j) * block_bytes;
-    copy_slice(dst, src, block_bytes);
+    const int64_t off = dst_off[r], region = region_k[r];
+    if (off < 0 || region < 0) { return; }
+    const uint64_t slot = static_cast<uint64_t>(off) + (static_cast<uint64_t>(l) * 2 + kv) * static_cast<uint64_t>(region) + j;
+    if (slot >= staging_blocks) { return; }              // never write outside the staging buffer
+    copy_slice(staging + slot * block_bytes, src, block_bytes);
 }
 
 constexpr size_t kBatchPiece = 2 * kStep;  // 256 KiB
@@ -155,8 +157,9 @@ extern "C" int ucm_kv_gather_selected(const void* const* layers, int n_layers, s
                                       size_t block_bytes, int num_blocks, const int32_t* phys,
                                       const int32_t* count, int n_req, int phys_stride, const int64_t* dst_off,
                                       const int32_t* region_k, int max_count, void* staging,
-                                      ucm_stream_t stream)
+                                      int64_t staging_blocks, ucm_stream_t stream)
 {
+    UCM_REQUIRE(staging_blocks >= 0, "ucm_kv_gather_selected: staging_blocks=%lld", static_cast<long long>(staging_blocks));
     UCM_REQUIRE(n_req == 0 || max_count == 0 || (layers && phys && count && dst_off && region_k && staging),
                 "ucm_kv_gather_selected: null pointer");
     UCM_REQUIRE(n_layers > 0 && n_layers * 2 <= 65535, "ucm_kv_gather_selected: n_layers=%d", n_layers);
@@ -172,6 +175,6 @@ extern "C" int ucm_kv_gather_selected(const void* const* layers, int n_layers, s
                        dim3(static_cast<unsigned>(max_count), n_req, n_layers * 2),
                        dim3(kThreads), 0, ucm::as_stream(stream), layers, kv_stride, block_bytes, phys,
                        count, static_cast<unsigned>(num_blocks), static_cast<unsigned>(n_req), static_cast<unsigned>(phys_stride), dst_off,
-                       region_k, static_cast<uint8_t*>(staging));
+                       region_k, static_cast<uint8_t*>(staging), static_cast<uint64_t>(staging_blocks));
     UCM_LAUNCH_CHECK("ucm_kv_gather_selected");
 }

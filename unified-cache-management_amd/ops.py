@@ -300,7 +300,7 @@ def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, 
     _lib.call("ucm_kv_gather_selected", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
               _dev(phys, torch.int32, "phys"), _dev(count, torch.int32, "count"), n_req, phys.shape[2],
               _dev(dst_off, torch.int64, "dst_off"), _dev(region_k, torch.int32, "region_k"), max_count,
-              _staging_ptr(staging, staging_blocks * block_bytes), _stream())
+              _staging_ptr(staging, staging_blocks * block_bytes), staging_blocks, _stream())
 
 
 def kvstar_table(n_layers: int, kv_heads: int, rows: int, sub_blocks: int, d_pad: int, device) -> torch.Tensor:
