@@ -205,8 +205,9 @@ int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
  *                  selected block after the load (the sparse block table)
  *   miss_count     dev int32 [n_layers][n_req], out: blocks to load
  * The i-th missing block (ascending) goes to the i-th freed slot (ascending);
- * the reference pairs them in set order, which is unspecified.  At most 64
- * slots per request and layer; selections longer than n_slots are cut there.
+ * the reference pairs them in set order, which is unspecified.  At most 1024
+ * slots per request and layer (one wave up to 64 slots, a 256-thread workgroup
+ * beyond); selections longer than n_slots are cut there.
  */
 int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req,
                    int n_layers, int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys,

@@ -658,6 +658,58 @@ def test_delta_plan_and_delta_gather(ucm, dev):
         prev = sel
 
 
+@pytest.mark.parametrize("n_slots", [1, 63, 64, 65, 153, 256, 257, 512, 700, 1024])
+def test_delta_plan_slot_counts(ucm, dev, n_slots):
+    """The plan for one to 1024 staging slots (one wave up to 64, a workgroup beyond) over four steps of
+    drifting selections in score order (not ascending), with counts from empty to beyond the slot budget,
+    equals the oracle's: loads, slot of every selected block, resident sets, counts."""
+    from ucm_amd import ops
+
+    n_layers, n_req = 2, 3
+    universe = 2 * n_slots + 40
+    stride = n_slots + 9
+    rng = np.random.default_rng(1000 + n_slots)
+    resident = torch.full((n_layers, n_req, n_slots), -1, dtype=torch.int32, device=dev)
+    res_h = np.full((n_layers, n_req, n_slots), -1, np.int32)
+    table = rng.permutation(5 * universe)[:universe].astype(np.int32)
+    prev = [[None] * n_req for _ in range(n_layers)]
+    for step in range(4):
+        cnt = rng.integers(0, stride + 1, (n_layers, n_req)).astype(np.int32)
+        cnt[0, 0], cnt[1, 1] = min(stride, n_slots + 5), n_slots
+        if step == 2:
+            cnt[0, 2] = 0
+        sel = np.full((n_layers, n_req, stride), -1, np.int32)
+        for l in range(n_layers):
+            for r in range(n_req):
+                c = int(cnt[l, r])
+                if prev[l][r] is not None and len(prev[l][r]):
+                    old = prev[l][r]
+                    keep = old[rng.random(len(old)) < 0.8]
+                    fresh = np.setdiff1d(rng.permutation(universe), keep, assume_unique=True)
+                    pick = np.concatenate([keep, fresh])[:c]
+                else:
+                    pick = rng.permutation(universe)[:c]
+                pick = rng.permutation(pick).astype(np.int32)
+                sel[l, r, :c] = pick
+                prev[l][r] = pick
+        phys = np.where(sel >= 0, table[np.maximum(sel, 0)], -1).astype(np.int32)
+        load = torch.full((n_layers, n_req, n_slots), -7, dtype=torch.int32, device=dev)
+        slot_of = torch.full((n_layers, n_req, stride), -7, dtype=torch.int32, device=dev)
+        miss = torch.full((n_layers, n_req), -7, dtype=torch.int32, device=dev)
+        ops.delta_plan(i32(sel, dev), i32(phys, dev), i32(cnt, dev), resident, load, slot_of, miss)
+        torch.cuda.synchronize()
+        load_h, slot_h, miss_h = load.cpu().numpy(), slot_of.cpu().numpy(), miss.cpu().numpy()
+        for l in range(n_layers):
+            for r in range(n_req):
+                c = int(cnt[l, r])
+                wl, ws, moved = O.delta_plan(sel[l, r, :c], phys[l, r, :c], res_h[l, r])
+                k = min(c, n_slots)
+                assert np.array_equal(load_h[l, r], wl) and miss_h[l, r] == moved, (step, l, r)
+                assert np.array_equal(slot_h[l, r, :k], ws[:k]), (step, l, r)
+                assert np.all(slot_h[l, r, k:] == -7), (step, l, r)      # nothing written past the cut
+        assert np.array_equal(resident.cpu().numpy(), res_h), step
+
+
 def test_decode_step_under_graph_capture(ucm, dev):
     """The step's three launches (scores, selection + block table, gather) allocate and synchronise nothing, so a
     caller may capture them in a HIP graph: three replays with fresh queries, eager work and synchronisation in

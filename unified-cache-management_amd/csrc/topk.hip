@@ -229,6 +229,119 @@ __global__ __launch_bounds__(64) void delta_plan_kernel(
     if (lane == 0) { miss_count[lr] = n_move; }
 }
 
+// More than 64 slots: one 256-thread workgroup per (layer, request), entry
+// e*256 + thread in register e.  Both lists sit in LDS and every thread walks
+// the other list four entries per read (all threads read the same address, a
+// broadcast); ranks are ballot prefix counts plus the counts of the (register,
+// wave) groups before the thread's own, so the pairing is the same as above.
+constexpr int kPlanThreads = 256;
+constexpr int kPlanWaves = kPlanThreads / 64;
+
+template <int E>  // entries per thread: n_slots <= 256 * E
+__global__ __launch_bounds__(kPlanThreads) void delta_plan_wide_kernel(
+    const int32_t* __restrict__ sel, const int32_t* __restrict__ sel_phys, const int32_t* __restrict__ count,
+    int n_req, int sel_stride, int32_t* __restrict__ resident, int n_slots, int32_t* __restrict__ load_phys,
+    int32_t* __restrict__ slot_of_sel, int32_t* __restrict__ miss_count)
+{
+    constexpr int kCap = kPlanThreads * E;
+    const int r = blockIdx.x, l = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const size_t lr = static_cast<size_t>(l) * n_req + r;
+    const int k = min(count[lr], n_slots);
+    const int32_t* s = sel + lr * sel_stride;
+    const int32_t* sp = sel_phys + lr * sel_stride;
+    int32_t* res = resident + lr * n_slots;
+
+    __shared__ __attribute__((aligned(16))) int32_t s_sel[kCap], s_res[kCap];
+    __shared__ int32_t s_a[kCap], s_b[kCap], s_c[kCap];   // miss_sel, miss_phys, free_slot by rank
+    __shared__ int s_miss_cnt[E * kPlanWaves], s_free_cnt[E * kPlanWaves];
+
+    int my_sel[E], my_phys[E], my_res[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int i = e * kPlanThreads + tid;
+        my_sel[e] = i < k ? s[i] : -1;
+        my_phys[e] = i < k ? sp[i] : -1;
+        my_res[e] = i < n_slots ? res[i] : -1;
+        s_sel[i] = my_sel[e];          // entries past the lists hold -1, which matches nothing
+        s_res[i] = my_res[e];
+    }
+    __syncthreads();
+
+    int hit_slot[E];
+    bool keep[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) { hit_slot[e] = -1; keep[e] = false; }
+    const int res_quads = (n_slots + 3) >> 2, sel_quads = (k + 3) >> 2;
+    for (int q = 0; q < res_quads; ++q) {
+        const int4 v = *reinterpret_cast<const int4*>(&s_res[q * 4]);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            if (my_sel[e] >= 0) {   // the last matching slot wins, as in the one-wave kernel
+                if (v.x == my_sel[e]) { hit_slot[e] = q * 4; }
+                if (v.y == my_sel[e]) { hit_slot[e] = q * 4 + 1; }
+                if (v.z == my_sel[e]) { hit_slot[e] = q * 4 + 2; }
+                if (v.w == my_sel[e]) { hit_slot[e] = q * 4 + 3; }
+            }
+        }
+    }
+    for (int q = 0; q < sel_quads; ++q) {
+        const int4 v = *reinterpret_cast<const int4*>(&s_sel[q * 4]);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            if (my_res[e] >= 0 && (v.x == my_res[e] || v.y == my_res[e] || v.z == my_res[e] || v.w == my_res[e])) {
+                keep[e] = true;
+            }
+        }
+    }
+
+    bool miss[E], freed[E];
+    int miss_rank[E], free_rank[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int i = e * kPlanThreads + tid;
+        miss[e] = i < k && hit_slot[e] < 0;
+        freed[e] = i < n_slots && !keep[e];
+        const unsigned long long mm = __ballot(miss[e]), fm = __ballot(freed[e]);
+        miss_rank[e] = static_cast<int>(lanes_below(mm));
+        free_rank[e] = static_cast<int>(lanes_below(fm));
+        if (lane == 0) { s_miss_cnt[e * kPlanWaves + wave] = __popcll(mm); s_free_cnt[e * kPlanWaves + wave] = __popcll(fm); }
+    }
+    __syncthreads();
+    int n_miss = 0, n_free = 0;
+#pragma unroll
+    for (int g = 0; g < E * kPlanWaves; ++g) {
+        const int cm = s_miss_cnt[g], cf = s_free_cnt[g];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            if (g < e * kPlanWaves + wave) { miss_rank[e] += cm; free_rank[e] += cf; }
+        }
+        n_miss += cm;
+        n_free += cf;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        if (miss[e]) { s_a[miss_rank[e]] = my_sel[e]; s_b[miss_rank[e]] = my_phys[e]; }
+        if (freed[e]) { s_c[free_rank[e]] = e * kPlanThreads + tid; }
+    }
+    __syncthreads();
+    const int n_move = min(n_miss, n_free);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int i = e * kPlanThreads + tid;
+        int dst_slot = hit_slot[e], take_sel = -1, take_phys = -1;
+        if (freed[e] && free_rank[e] < n_move) { take_sel = s_a[free_rank[e]]; take_phys = s_b[free_rank[e]]; }
+        if (miss[e] && miss_rank[e] < n_move) { dst_slot = s_c[miss_rank[e]]; }
+        if (i < n_slots) {
+            load_phys[lr * n_slots + i] = take_phys;
+            if (take_sel >= 0) { res[i] = take_sel; }
+            else if (freed[e]) { res[i] = -1; }
+        }
+        if (i < k) { slot_of_sel[lr * sel_stride + i] = dst_slot; }
+    }
+    if (tid == 0) { miss_count[lr] = n_move; }
+}
+
 }  // namespace
 
 extern "C" int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req,
@@ -238,9 +351,20 @@ extern "C" int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const
     UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_delta_plan: n_req=%d n_layers=%d", n_req, n_layers);
     if (n_req == 0) { return UCM_OK; }
     UCM_REQUIRE(sel && sel_phys && count && resident && load_phys && slot_of_sel && miss_count, "ucm_delta_plan: null pointer");
-    UCM_SUPPORTED(n_slots >= 1 && n_slots <= 64, "ucm_delta_plan: n_slots=%d (1..64 staging slots per request and layer)", n_slots);
+    UCM_SUPPORTED(n_slots >= 1 && n_slots <= 1024, "ucm_delta_plan: n_slots=%d (1..1024 staging slots per request and layer)", n_slots);
     UCM_REQUIRE(sel_stride >= 1, "ucm_delta_plan: sel_stride=%d", sel_stride);
-    hipLaunchKernelGGL(delta_plan_kernel, dim3(n_req, n_layers), dim3(64), 0, ucm::as_stream(stream), sel, sel_phys,
-                       count, n_req, sel_stride, resident, n_slots, load_phys, slot_of_sel, miss_count);
+    const dim3 grid(n_req, n_layers);
+    hipStream_t s = ucm::as_stream(stream);
+#define UCM_PLAN_LAUNCH(E)                                                                                  \
+    hipLaunchKernelGGL(delta_plan_wide_kernel<E>, grid, dim3(kPlanThreads), 0, s, sel, sel_phys, count, n_req, \
+                       sel_stride, resident, n_slots, load_phys, slot_of_sel, miss_count)
+    if (n_slots <= 64) {
+        hipLaunchKernelGGL(delta_plan_kernel, grid, dim3(64), 0, s, sel, sel_phys, count, n_req, sel_stride, resident,
+                           n_slots, load_phys, slot_of_sel, miss_count);
+    }
+    else if (n_slots <= 256) { UCM_PLAN_LAUNCH(1); }
+    else if (n_slots <= 512) { UCM_PLAN_LAUNCH(2); }
+    else { UCM_PLAN_LAUNCH(4); }
+#undef UCM_PLAN_LAUNCH
     UCM_LAUNCH_CHECK("ucm_delta_plan");
 }
