@@ -221,6 +221,58 @@ def test_hash_query_codes_for_other_head_counts(ucm, dev, hq, hkv):
     assert not q_codes[0, 1, 0].any()
 
 
+def test_hash_query_codes_near_zero_projections_and_scales(ucm, dev):
+    """Query rows and group means whose projections cancel exactly, or down to one small term, and vectors
+    scaled from 2^-100 to 2^100: the kernel projects on the matrix cores in fp32 and redoes results within
+    its error bound exactly, so every sign must still be the oracle's (strict > 0: a projection of exactly
+    zero is bit 0)."""
+    from ucm_amd import ops
+
+    hq, hkv, n_layers, n_req = 32, 8, 2, 6
+    g = hq // hkv
+    w_bits, _ = make_weights(860)
+    w_bits[1] = w_bits[0]                      # two equal weight rows: (t, -t, 0, ...) projects to exactly 0
+    w_bits[5] = w_bits[4] ^ 0x8000             # and a negated pair: (t, t, ...) on dims 4, 5 cancels too
+    w_f32 = synth.bf16_widen(w_bits)
+    f = synth.normal_f32(861, (n_layers, n_req, hq, 128))
+    one, tiny = np.float32(1.0), np.float32(2.0 ** -40)
+    # request 0: rows that cancel exactly; every second one keeps a term 2^-40 of the others' size on dim 2
+    f[:, 0] = 0
+    f[:, 0, :, 0], f[:, 0, :, 1] = 3.0, -3.0
+    f[:, 0, :, 4], f[:, 0, :, 5] = 0.75, 0.75
+    f[:, 0, 1::2, 2] = tiny * np.where(np.arange(hq // 2) % 2 == 0, one, -one)
+    # request 1: heads of a group are negations of each other, so the group means are exactly zero ...
+    f[:, 1, 1::2] = -f[:, 1, 0::2]
+    # request 2: ... or cancel down to one small term
+    f[:, 2, 1::2] = -f[:, 2, 0::2]
+    # requests 3 and 4: tiny and huge vectors; request 5 mixes the scales of its rows
+    f[:, 3] *= np.float32(2.0 ** -100)
+    f[:, 4] *= np.float32(2.0 ** 100)
+    f[:, 5] *= (np.float32(2.0) ** np.linspace(-90, 90, hq)).astype(np.float32)[None, :, None]
+    q_h = synth.bf16_round_bits(f)
+    q_h[:, 1, 1::2] = q_h[:, 1, 0::2] ^ 0x8000          # exact negations after rounding as well
+    q_h[:, 2, 1::2] = q_h[:, 2, 0::2] ^ 0x8000
+    q_h[:, 2, :, 7] = 0                                 # (added to a term of size 1 it would be rounded away)
+    q_h[:, 2, 0::g, 7] = synth.bf16_round_bits(np.float32(2.0 ** -30))
+    q_codes = torch.full((n_layers, n_req, hq, 16), 0xEE, dtype=torch.uint8, device=dev)
+    q_sum = torch.full((n_layers, n_req, 128), 77, dtype=torch.int16, device=dev)
+    qbar = torch.full((n_layers, n_req, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(bf16_dev(q_h, dev), bf16_dev(w_bits, dev), hkv, q_codes, q_sum, qbar, n_req)
+    torch.cuda.synchronize()
+    for l in range(n_layers):
+        want_q = O.hash_encode(q_h[l], w_f32)
+        assert np.array_equal(q_codes[l].cpu().numpy(), want_q), l
+        pm = np.unpackbits(want_q, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
+        assert np.array_equal(q_sum[l].cpu().numpy(), pm.sum(1)), l
+        qm = np.stack([O.q_head_mean(synth.bf16_widen(q_h[l][r]), hkv) for r in range(n_req)])
+        want_bar = O.hash_encode_f32(qm, w_f32)
+        assert np.array_equal(qbar[l].cpu().numpy(), want_bar), l
+        # the cases are what they claim to be
+        assert not want_q[0, 0::2].any() and want_q[0, 1::2].any()
+        assert not want_bar[1].any() and want_bar[2].any()
+        assert want_q[3].any() and want_q[4].any()
+
+
 def test_hash_queries_scores_and_selection(ucm, dev):
     """Config-5 shape in small: ragged batch, 8 kv heads, 32 query heads, 2 layers."""
     from ucm_amd import ops

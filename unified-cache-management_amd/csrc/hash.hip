@@ -56,8 +56,6 @@ __device__ __forceinline__ int row_of_col(int col)
     return (col & ~31) + (i >> 2) * 8 + h * 4 + (i & 3);
 }
 
-__device__ __forceinline__ float bf16_to_f32(unsigned short h) { return __uint_as_float(static_cast<unsigned>(h) << 16); }
-
 struct __attribute__((aligned(16))) WaveScratch {
     unsigned queue[kQueueCap];
     int colsum[kMaxHeads][kBits];   // per-head ones counts of the block being encoded
@@ -456,124 +454,267 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     }
 }
 
-// Query side, one workgroup of 1024 threads per (request, layer).  The vectors to project are the
-// request's q_heads query rows and the kv_heads group-mean queries (fp32 sequential adds * (1/g), the
-// scoring path's own mean); every projection is exact: fp64, d ascending (a product of two bf16 values
-// is exact in fp64 and so, for these magnitudes, is the sum).  Thread (bit c, group hg) owns column c of
-// W - 128 bf16 values held in 64 registers for the whole kernel - and projects vectors hg, hg+8, ...;
-// the vectors are staged in LDS as fp64, forty at a time, and read back two at a time as wave-wide
-// broadcasts; eight weights are widened to fp64 at a time and used for the thread's five vectors of the
-// chunk, so the inner loop is little more than one fp64 fma per vector and dimension.  The +-1 sum over
-// all heads is combined through LDS.
-// grid: x = request, y = layer
-constexpr int kQueryGroups = 8;
-constexpr int kQueryThreads = kBits * kQueryGroups;
+// Query side, one workgroup of four waves per (request, layer); wave w projects every vector onto weight
+// columns 32w .. 32w+31 on the matrix cores.  The vectors are the request's q_heads query rows (32 per
+// tile) and the kv_heads group-mean queries (fp32 sequential adds * (1/g), the scoring path's own mean).
+// A mean is an fp32 number, not a bf16 one: it is cut exactly into three bf16 terms (leading 8 bits, the
+// next 8, the rest), which become rows h, 8+h and 16+h of one more tile; those three rows of a column are
+// registers i, i+4, i+8 of the same lane and are added there.  Only signs are kept, and they must be the
+// signs of the exactly accumulated products: a result whose magnitude is below
+// 2^-15 * (largest ||x|| of the tile) * ||w_col|| - more than the fp32 accumulation can be off by - is redone
+// by its lane in fp64, d ascending (a product of an fp32 and a bf16 value is exact in fp64), every lane
+// working on one of its own results at a time.  A tile whose vectors are all tiny (norm below 2^-60, where
+// bf16 subnormals and the bound itself lose bits) is redone whole.  Query rows are the A operand and weights
+// the B operand, so a lane holds one weight column and 16 vectors, and a ballot over the lanes is a vector's
+// 32-bit code word.  The weights sit in LDS in their own [d][column] order (a lane reads its column two
+// bytes at a time, neighbours in neighbouring banks); the means are formed once per workgroup, a 16-byte
+// piece per thread, and parked in LDS as their three terms.
+// grid: x = request, y = layer; 256 threads
 constexpr int kMaxQHeads = 128;
-constexpr int kQueryRows = 40;          // vectors staged at a time (a multiple of the groups): 40 KiB of fp64
+constexpr int kQueryThreads = 256;
+constexpr int kMeanStride = kDim + 8;                    // bf16 elements per staged term row (272 B)
 
-__global__ __launch_bounds__(kQueryThreads) void hash_query_kernel(
+struct __attribute__((aligned(16))) QueryLds {
+    unsigned short w[kDim * kBits];                      // [d][column]
+    unsigned short mean[3][kMaxHeads][kMeanStride];      // [term][kv head][d]
+    float mean_max2[2];                                  // largest squared norm of the means staged by waves 0 and 1
+};
+
+__device__ __forceinline__ float wave_max32(float m)
+{
+#pragma unroll
+    for (int d = 16; d >= 1; d >>= 1) { m = fmaxf(m, __shfl_xor(m, d, 64)); }
+    return m;
+}
+
+__device__ __forceinline__ void widen8(const u32x4 v, float (&x)[8])
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { x[2 * j] = __uint_as_float(v[j] << 16); x[2 * j + 1] = __uint_as_float(v[j] & 0xffff0000u); }
+}
+
+// acc += x[0..7] . W[d0 .. d0+7][col], d ascending (exact products, fp64 sums: the oracle's arithmetic)
+__device__ __forceinline__ double dot8_exact(const float (&x)[8], const unsigned short* w_s, unsigned d0, unsigned col, double acc)
+{
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float wf = __uint_as_float(static_cast<unsigned>(w_s[(d0 + j) * kBits + col]) << 16);
+        acc += static_cast<double>(x[j]) * static_cast<double>(wf);
+    }
+    return acc;
+}
+
+// exact sign of a query row . column: the row is fetched in four groups of four 16-byte pieces
+__device__ __forceinline__ bool row_exact_positive(const unsigned short* __restrict__ row, const unsigned short* w_s, unsigned col)
+{
+    double acc = 0.0;
+#pragma unroll 1
+    for (int c = 0; c < 4; ++c) {
+        u32x4 xv[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { xv[k] = ucm::gload16(row + 32 * c + 8 * k); }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float x[8];
+            widen8(xv[k], x);
+            acc = dot8_exact(x, w_s, 32 * c + 8 * k, col, acc);
+        }
+    }
+    return acc > 0.0;
+}
+
+// exact sign of a staged group mean . column; (hi + mid) + lo is the mean again, exactly
+__device__ __forceinline__ bool mean_exact_positive(const QueryLds& s, unsigned h, unsigned col)
+{
+    double acc = 0.0;
+#pragma unroll 1
+    for (int k = 0; k < kDim / 8; ++k) {
+        float hi[8], mid[8], lo[8], x[8];
+        widen8(*reinterpret_cast<const u32x4*>(&s.mean[0][h][8 * k]), hi);
+        widen8(*reinterpret_cast<const u32x4*>(&s.mean[1][h][8 * k]), mid);
+        widen8(*reinterpret_cast<const u32x4*>(&s.mean[2][h][8 * k]), lo);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { x[j] = (hi[j] + mid[j]) + lo[j]; }
+        acc = dot8_exact(x, s.w, 8 * k, col, acc);
+    }
+    return acc > 0.0;
+}
+
+__global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
     const unsigned short* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows,
     unsigned q_heads, unsigned kv_heads, const unsigned short* __restrict__ w, unsigned n_req,
     unsigned* __restrict__ q_codes /*[L][n_req][q_heads][4]*/, short* __restrict__ q_sum /*[L][n_req][128]*/,
     unsigned* __restrict__ qbar_codes /*[L][n_req][kv_heads][4]*/)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char query_lds[];
-    double* rows_d = reinterpret_cast<double*>(query_lds);                                       // [kQueryRows][kDim]
-    unsigned short* wt_s = reinterpret_cast<unsigned short*>(rows_d + kQueryRows * kDim);       // [c][d], rows kWtStride apart
-    int* part = reinterpret_cast<int*>(wt_s + kBits * kWtStride);                               // [kQueryGroups][kBits]
-
+    __shared__ QueryLds s;
     const unsigned r = blockIdx.x, l = blockIdx.y;
-    const unsigned c = threadIdx.x % kBits, hg = threadIdx.x / kBits;
+    const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned half = lane >> 5, lr32 = lane & 31;
+    const unsigned col = wave * 32 + lr32;               // the weight column this lane ends up with
     const unsigned short* qp = q + static_cast<int64_t>(l) * q_layer_stride +
                                static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kDim;
-    // W transposed, so that a thread's column is sixteen 16-byte reads
-    for (unsigned e = threadIdx.x; e < kDim * kBits; e += kQueryThreads) {
-        wt_s[(e % kBits) * kWtStride + e / kBits] = w[e];
-    }
-    __syncthreads();
-    u32x4 wcol[kDim / 8];
-#pragma unroll
-    for (int k = 0; k < kDim / 8; ++k) { wcol[k] = *reinterpret_cast<const u32x4*>(&wt_s[c * kWtStride + k * 8]); }
-
-    const size_t lr = static_cast<size_t>(l) * n_req + r;
+    const size_t lrq = static_cast<size_t>(l) * n_req + r;
     const unsigned g = q_heads / kv_heads;
     const float inv = 1.0f / static_cast<float>(g);
-    const unsigned n_vec = q_heads + kv_heads;          // the query rows, then the group means
+
+    // ---- staging: the weights as they are, and the means' three terms (thread = head, 16-byte piece)
+    {
+        u32x4 wv[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { wv[k] = ucm::gload16(w + (k * kQueryThreads + threadIdx.x) * 8); }
+        const unsigned h = threadIdx.x >> 4, piece = threadIdx.x & 15;
+        float nx2 = 0.0f;
+        if (h < kv_heads) {
+            const unsigned short* first = qp + (h * g) * kDim + 8 * piece;
+            float x[8];
+            widen8(ucm::gload16(first), x);
+#pragma unroll 4
+            for (unsigned rr = 1; rr < g; ++rr) {
+                float y[8];
+                widen8(ucm::gload16(first + rr * kDim), y);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) { x[j] = x[j] + y[j]; }
+            }
+            unsigned term[3][8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float xm = g != 1 ? x[j] * inv : x[j];
+                const float hi = __uint_as_float(__float_as_uint(xm) & 0xffff0000u);
+                const float r1 = xm - hi;                                     // exact: the trailing bits of xm
+                const float mid = __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+                const float lo = r1 - mid;                                    // exact, at most 8 significant bits
+                term[0][j] = __float_as_uint(hi) >> 16;
+                term[1][j] = __float_as_uint(mid) >> 16;
+                term[2][j] = __float_as_uint(lo) >> 16;
+                nx2 = nx2 + xm * xm;
+            }
+#pragma unroll
+            for (int p = 0; p < 3; ++p) {
+                u32x4 packed;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { packed[j] = term[p][2 * j] | (term[p][2 * j + 1] << 16); }
+                *reinterpret_cast<u32x4*>(&s.mean[p][h][8 * piece]) = packed;
+            }
+        }
+        if (wave < 2) {                                  // (waves 0 and 1 hold the at most eight heads)
+#pragma unroll
+            for (int d = 8; d >= 1; d >>= 1) { nx2 += __shfl_xor(nx2, d, 64); }      // a head's 16 pieces
+            nx2 = fmaxf(nx2, __shfl_xor(nx2, 16, 64));
+            nx2 = fmaxf(nx2, __shfl_xor(nx2, 32, 64));
+            if (lane == 0) { s.mean_max2[wave] = nx2; }
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { *reinterpret_cast<u32x4*>(&s.w[(k * kQueryThreads + threadIdx.x) * 8]) = wv[k]; }
+    }
+    __syncthreads();
+
+    // B operand: step ks covers dims 16ks .. 16ks+15, this lane holds the eight of its half for its column
+    u32x4 wb[8];
+    float nw2 = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        const unsigned short* wp = &s.w[(16 * ks + 8 * half) * kBits + col];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            wb[ks][j] = static_cast<unsigned>(wp[(2 * j) * kBits]) | (static_cast<unsigned>(wp[(2 * j + 1) * kBits]) << 16);
+        }
+        nw2 = norm2_acc(wb[ks], nw2);
+    }
+    nw2 += __shfl_xor(nw2, 32, 64);                      // the column's squared norm
+
+    // ---- the query rows, 32 per tile
     int sum = 0;
-    for (unsigned v0 = 0; v0 < n_vec; v0 += kQueryRows) {
-        const unsigned nv = min(static_cast<unsigned>(kQueryRows), n_vec - v0);
-        __syncthreads();                                // the chunk before has been read
-        for (unsigned e = threadIdx.x; e < nv * kDim; e += kQueryThreads) {
-            const unsigned v = v0 + e / kDim, d = e % kDim;
-            float x;
-            if (v < q_heads) {
-                x = bf16_to_f32(qp[v * kDim + d]);
-            } else {
-                const unsigned h = v - q_heads;
-                x = bf16_to_f32(qp[(h * g) * kDim + d]);
-                for (unsigned j = 1; j < g; ++j) { x = x + bf16_to_f32(qp[(h * g + j) * kDim + d]); }
-                if (g != 1) { x = x * inv; }
-            }
-            rows_d[e] = static_cast<double>(x);
+    for (unsigned t0 = 0; t0 < q_heads; t0 += 32) {
+        const unsigned m_in = t0 + lr32;                 // the row this lane feeds
+        u32x4 xa[8];
+        float nx2 = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            if (m_in < q_heads) { xa[ks] = ucm::gload16(qp + m_in * kDim + 16 * ks + 8 * half); }
+            else { xa[ks] = u32x4{0u, 0u, 0u, 0u}; }
+            nx2 = norm2_acc(xa[ks], nx2);
         }
-        __syncthreads();
-        // eight weights of the column widened at a time and used for all of the thread's vectors of this chunk
-        constexpr int kMine = kQueryRows / kQueryGroups;
-        double acc[kMine];
+        nx2 += __shfl_xor(nx2, 32, 64);
+        const float max2 = wave_max32(nx2);
+        const bool all_exact = max2 > 0.0f && !(max2 >= 0x1p-120f);
+        const float bound = sqrtf(kTau2 * max2) * sqrtf(nw2) * 1.01f;
+        f32x16 acc;
 #pragma unroll
-        for (int vi = 0; vi < kMine; ++vi) { acc[vi] = 0.0; }
+        for (int i = 0; i < 16; ++i) { acc[i] = 0.0f; }
 #pragma unroll
-        for (int k = 0; k < kDim / 8; ++k) {
-            // (the empty asm keeps the compiler from widening the whole column to fp64 ahead of the chunk loop,
-            // which would take 256 registers)
-            asm volatile("" : "+v"(wcol[k]));
-            double wd[8];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                wd[2 * j] = static_cast<double>(__uint_as_float(wcol[k][j] << 16));
-                wd[2 * j + 1] = static_cast<double>(__uint_as_float(wcol[k][j] & 0xffff0000u));
-            }
-#pragma unroll
-            for (int vi = 0; vi < kMine; ++vi) {
-                // the same address in every lane: broadcast reads; a vector past the chunk's end re-reads the last one
-                const double* x = rows_d + min(hg + vi * kQueryGroups, nv - 1) * kDim + k * 8;
-                // (the products are exact in fp64 - at most 24 + 8 significant bits - so the fused form rounds
-                // exactly like a multiplication followed by an addition; d ascending per vector)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) { acc[vi] = __builtin_fma(x[j], wd[j], acc[vi]); }
-                __builtin_amdgcn_sched_barrier(0);      // one vector's reads at a time: with all of a step's up front the
-            }                                           // 128 registers a thread of a 1024-thread workgroup has do not suffice
+        for (int ks = 0; ks < 8; ++ks) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xa[ks]), __builtin_bit_cast(bf16x8, wb[ks]),
+                                                          acc, 0, 0, 0);
         }
-        // (used here whatever follows: otherwise the compiler moves each vector's whole fma chain down into the
-        // conditional code below and keeps every operand alive until then)
+        // result register i is row t0 + 8*(i/4) + 4*half + i%4
+        unsigned positive = 0, redo = 0;
 #pragma unroll
-        for (int vi = 0; vi < kMine; ++vi) { asm volatile("" : "+v"(acc[vi])); }
+        for (int i = 0; i < 16; ++i) {
+            const bool valid = t0 + 8 * (i >> 2) + 4 * half + (i & 3) < q_heads;
+            if (acc[i] > 0.0f) { positive |= 1u << i; }
+            if (valid && (all_exact || !(fabsf(acc[i]) >= bound))) { redo |= 1u << i; }
+        }
+        while (redo) {
+            const unsigned i = static_cast<unsigned>(__builtin_ctz(redo));
+            redo &= redo - 1;
+            const unsigned m = t0 + 8 * (i >> 2) + 4 * half + (i & 3);
+            const bool pos = row_exact_positive(qp + m * kDim, s.w, col);
+            positive = (positive & ~(1u << i)) | (static_cast<unsigned>(pos) << i);
+        }
 #pragma unroll
-        for (int vi = 0; vi < kMine; ++vi) {
-            const unsigned vl = hg + vi * kQueryGroups;
-            if (vl >= nv) { break; }                    // (the same for a whole wave)
-            const bool pos = acc[vi] > 0.0;
-            const unsigned long long m = __ballot(pos);  // a wave covers 64 consecutive bits of one vector
-            const unsigned v = v0 + vl;
-            if (v < q_heads) {
+        for (int i = 0; i < 16; ++i) {
+            const unsigned m = t0 + 8 * (i >> 2) + 4 * half + (i & 3);
+            const bool valid = m < q_heads;
+            const bool pos = valid && ((positive >> i) & 1u);
+            const unsigned long long mask = __ballot(pos);
+            if (valid) {
                 sum += pos ? 1 : -1;
-                if ((c & 63) == 0) {
-                    q_codes[(lr * q_heads + v) * 4 + (c >> 6) * 2] = static_cast<unsigned>(m);
-                    q_codes[(lr * q_heads + v) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(m >> 32);
-                }
-            } else if ((c & 63) == 0) {
-                qbar_codes[(lr * kv_heads + (v - q_heads)) * 4 + (c >> 6) * 2] = static_cast<unsigned>(m);
-                qbar_codes[(lr * kv_heads + (v - q_heads)) * 4 + (c >> 6) * 2 + 1] = static_cast<unsigned>(m >> 32);
+                if (lr32 == 0) { q_codes[(lrq * q_heads + m) * 4 + wave] = static_cast<unsigned>(half ? mask >> 32 : mask); }
             }
         }
     }
-    part[hg * kBits + c] = sum;
-    __syncthreads();
-    if (hg == 0) {
-        int total = 0;
+    sum += __shfl_xor(sum, 32, 64);
+    if (half == 0) { q_sum[lrq * kBits + col] = static_cast<short>(sum); }
+
+    // ---- the group means: row 8*term + h of the tile is that term of head h's mean
+    {
+        const unsigned term = lr32 >> 3, h_in = lr32 & 7;
+        const bool feeds = term < 3 && h_in < kv_heads;
+        f32x16 acc;
 #pragma unroll
-        for (int k = 0; k < kQueryGroups; ++k) { total += part[k * kBits + c]; }
-        q_sum[lr * kBits + c] = static_cast<short>(total);
+        for (int i = 0; i < 16; ++i) { acc[i] = 0.0f; }
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            u32x4 xa = u32x4{0u, 0u, 0u, 0u};
+            if (feeds) { xa = *reinterpret_cast<const u32x4*>(&s.mean[term][h_in][16 * ks + 8 * half]); }
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xa), __builtin_bit_cast(bf16x8, wb[ks]),
+                                                          acc, 0, 0, 0);
+        }
+        const float max2 = fmaxf(s.mean_max2[0], s.mean_max2[1]);
+        const bool all_exact = max2 > 0.0f && !(max2 >= 0x1p-120f);
+        const float bound = sqrtf(kTau2 * max2) * sqrtf(nw2) * 1.01f;
+        unsigned positive = 0, redo = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float t = (acc[i] + acc[i + 4]) + acc[i + 8];      // the three terms of head 4*half + i
+            if (t > 0.0f) { positive |= 1u << i; }
+            if (4 * half + i < kv_heads && (all_exact || !(fabsf(t) >= bound))) { redo |= 1u << i; }
+        }
+        while (redo) {
+            const unsigned i = static_cast<unsigned>(__builtin_ctz(redo));
+            redo &= redo - 1;
+            const bool pos = mean_exact_positive(s, 4 * half + i, col);
+            positive = (positive & ~(1u << i)) | (static_cast<unsigned>(pos) << i);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned h = 4 * half + i;
+            const bool valid = h < kv_heads;
+            const unsigned long long mask = __ballot(valid && ((positive >> i) & 1u));
+            if (valid && lr32 == 0) {
+                qbar_codes[(lrq * kv_heads + h) * 4 + wave] = static_cast<unsigned>(half ? mask >> 32 : mask);
+            }
+        }
     }
 }
 
@@ -702,15 +843,9 @@ extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_strid
     UCM_SUPPORTED(head_dim == kDim && bits == kBits, "ucm_hash_encode_queries: head_dim=%d bits=%d (128 and 128)", head_dim, bits);
     UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0,
                 "ucm_hash_encode_queries: q_heads=%d kv_heads=%d", q_heads, kv_heads);
-    UCM_SUPPORTED(q_heads <= kMaxQHeads, "ucm_hash_encode_queries: q_heads=%d (at most %d)", q_heads, kMaxQHeads);
-    constexpr size_t kQueryLds = kQueryRows * kDim * sizeof(double) + kBits * kWtStride * 2 + kQueryGroups * kBits * sizeof(int);
-    static_assert(kQueryLds <= 80 * 1024, "two query workgroups per compute unit");
-    if (const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(hash_query_kernel),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kQueryLds));
-        ea != hipSuccess) {
-        return ucm::check_hip(ea, "ucm_hash_encode_queries (LDS size)");
-    }
-    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), kQueryLds, ucm::as_stream(stream),
+    UCM_SUPPORTED(q_heads <= kMaxQHeads && kv_heads <= kMaxHeads, "ucm_hash_encode_queries: q_heads=%d kv_heads=%d (at most %d and %d)",
+                  q_heads, kv_heads, kMaxQHeads, kMaxHeads);
+    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),
                        static_cast<const unsigned short*>(q_bf16), q_layer_stride, q_rows,
                        static_cast<unsigned>(q_heads), static_cast<unsigned>(kv_heads),
                        static_cast<const unsigned short*>(w_bf16), static_cast<unsigned>(n_req),
