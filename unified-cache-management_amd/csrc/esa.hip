@@ -3,15 +3,17 @@
 //
 // The reference scores each slot with a strictly sequential
 //     score = score + q[d] * data[slot][d]        (separate multiply and add)
-// so one thread owns one slot and walks its row in order; what is parallel is
-// the slots.  Rows are 4 KiB apart, so they are staged through LDS: the four
-// waves of a workgroup fetch a 64-row x 128-column tile with coalesced 16-byte
-// loads (the next tile's loads are already in flight while the current one is
-// consumed), and one wave then reads its row from LDS, conflict-free thanks to
-// an odd row stride.  Latency-bound by design (a chain of `dim` dependent adds).
+// The products do not depend on the order, the additions do: every thread of a
+// workgroup multiplies the 16-byte pieces it fetches (coalesced, rows are 4 KiB
+// apart) by the query and parks the products in LDS, column-major with an odd
+// column stride, and one wave then adds its slot's products in order - per
+// dimension one LDS read at a constant offset and one dependent add, nothing
+// else.  Two product tiles alternate, so the other waves fill the next tile
+// while the chain of the current one runs, and the loads of the tile after that
+// are in flight.  Latency-bound by design (a chain of `dim` dependent adds).
 //
-// Selection is a bitonic sort of 64-bit keys (order-preserving score bits, then
-// position ascending) in LDS, one workgroup per request.
+// Selection ranks 64-bit keys (order-preserving score bits, then position
+// ascending) by counting the keys above each, spread over workgroups.
 #include "common.h"
 
 namespace {
@@ -20,17 +22,18 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kSlots = 64;          // slots (rows) per workgroup
 constexpr int kCols = 128;          // columns per tile
-constexpr int kStride = kCols + 1;  // odd stride: lane r reading column d hits bank (r + d) % 64
+constexpr int kColStride = kSlots + 1;  // odd: lane r reading column d hits bank (r + d) % 64
 constexpr int kScoreThreads = 256;
 constexpr int kRowsPerLoad = kScoreThreads / (kCols / 4);  // 8 rows per 16-byte load instruction
 constexpr int kLoads = kSlots / kRowsPerLoad;              // 8 loads per thread per tile
+constexpr int kDepth = 2;                                  // tiles in flight per thread (an even number: two LDS buffers)
 
 // grid: x = group of 64 entries of the index row, y = request
 __global__ __launch_bounds__(kScoreThreads) void esa_score_kernel(
     const float* __restrict__ data, unsigned n_items, unsigned dim, const float* __restrict__ q,
     const int32_t* __restrict__ indexes, unsigned m, float* __restrict__ scores)
 {
-    __shared__ float tile[kSlots * kStride];
+    __shared__ float tile[2][kCols * kColStride];       // products, [column][slot]
     __shared__ int32_t slot_of[kSlots];
 
     const unsigned b = blockIdx.y, first = blockIdx.x * kSlots;
@@ -50,34 +53,51 @@ __global__ __launch_bounds__(kScoreThreads) void esa_score_kernel(
         const int32_t s = slot_of[r0 + i * kRowsPerLoad];
         row_ptr[i] = data + static_cast<size_t>(s < 0 ? 0 : s) * dim + c4 * 4;
     }
-    const float* qb = q + static_cast<size_t>(b) * dim;
+    const float* qb = q + static_cast<size_t>(b) * dim + c4 * 4;
 
-    f32x4 regs[kLoads];
-    auto fetch = [&](unsigned col0) {
+    // kDepth tiles of loads are in flight per thread: a tile's chain (128 dependent adds) is several times
+    // shorter than a trip to memory, so the chain of tile t runs while tiles t+1 .. t+kDepth-1 are on their way
+    f32x4 regs[kDepth][kLoads], qv[kDepth];
+    auto fetch = [&](int stage, unsigned col0) {
+        if (col0 + c4 * 4 < dim) {
+            qv[stage] = *reinterpret_cast<const f32x4*>(qb + col0);
 #pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            if (col0 + c4 * 4 < dim) { regs[i] = *reinterpret_cast<const f32x4*>(row_ptr[i] + col0); }
+            for (int i = 0; i < kLoads; ++i) { regs[stage][i] = *reinterpret_cast<const f32x4*>(row_ptr[i] + col0); }
         }
     };
-    fetch(0);
-    float score = 0.0f;
-    for (unsigned col0 = 0; col0 < dim; col0 += kCols) {
 #pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            float* t = &tile[(r0 + i * kRowsPerLoad) * kStride + c4 * 4];
-            t[0] = regs[i].x; t[1] = regs[i].y; t[2] = regs[i].z; t[3] = regs[i].w;
-        }
-        __syncthreads();
-        if (col0 + kCols < dim) { fetch(col0 + kCols); }
-        if (threadIdx.x < kSlots) {
-            const unsigned width = min(static_cast<unsigned>(kCols), dim - col0);
-            const float* mine = &tile[threadIdx.x * kStride];
-            for (unsigned d = 0; d < width; ++d) {
-                const float p = qb[col0 + d] * mine[d];
-                score = score + p;
+    for (int u = 0; u < kDepth; ++u) {
+        if (u * kCols < dim) { fetch(u, u * kCols); }
+    }
+    float score = 0.0f;
+    for (unsigned base = 0; base < dim; base += kDepth * kCols) {
+#pragma unroll
+        for (int u = 0; u < kDepth; ++u) {
+            const unsigned col0 = base + u * kCols;
+            if (col0 >= dim) { break; }                  // (uniform)
+            // (tiles alternate between two buffers; a buffer is rewritten two tiles later, after the barrier
+            // of the tile in between, which the chain wave only reaches when its chain is done)
+            float* tb = tile[u & 1];
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) {
+                float* t = &tb[(c4 * 4) * kColStride + r0 + i * kRowsPerLoad];
+                t[0] = qv[u].x * regs[u][i].x;
+                t[kColStride] = qv[u].y * regs[u][i].y;
+                t[2 * kColStride] = qv[u].z * regs[u][i].z;
+                t[3 * kColStride] = qv[u].w * regs[u][i].w;
+            }
+            __syncthreads();
+            if (col0 + kDepth * kCols < dim) { fetch(u, col0 + kDepth * kCols); }
+            if (threadIdx.x < kSlots) {
+                const float* mine = &tb[threadIdx.x];
+                if (col0 + kCols <= dim) {
+#pragma unroll 32
+                    for (int d = 0; d < kCols; ++d) { score = score + mine[d * kColStride]; }
+                } else {
+                    for (unsigned d = 0; d < dim - col0; ++d) { score = score + mine[d * kColStride]; }
+                }
             }
         }
-        __syncthreads();
     }
     if (threadIdx.x < kSlots && first + threadIdx.x < m) {
         scores[static_cast<size_t>(b) * m + first + threadIdx.x] = score;
@@ -91,58 +111,72 @@ __device__ __forceinline__ unsigned ordered_key(float f)
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-constexpr int kSortThreads = 1024;
+constexpr int kRankThreads = 256;
 
-// grid: x = request; dynamic LDS: n_pad 64-bit keys
-__global__ __launch_bounds__(kSortThreads) void esa_topk_kernel(
+// Selection by counting: keys are distinct (the position is part of the key), so a candidate's place in
+// the descending order is the number of keys above its own.  Every workgroup builds all keys of its request
+// in LDS; kLanes lanes share a candidate, each counting over every kLanes-th key (lanes of a wave read at
+// most kLanes different addresses at a time, the rest are broadcasts), and the best `topk` candidates write
+// themselves to their places.  No sorting network, no barrier after the keys are built; long candidate lists
+// spread over many workgroups.
+// grid: x = group of 256/kLanes candidates, y = request; dynamic LDS: n_pad 64-bit keys
+template <int kLanes>
+__global__ __launch_bounds__(kRankThreads) void esa_rank_kernel(
     const float* __restrict__ scores, const int32_t* __restrict__ indexes, unsigned n_items, unsigned m,
     unsigned n_pad, int topk, int32_t* __restrict__ out_idx, float* __restrict__ out_scores,
     int32_t* __restrict__ out_count, unsigned out_stride)
 {
-    extern __shared__ unsigned long long keys[];
+    extern __shared__ __attribute__((aligned(16))) unsigned long long keys[];
     __shared__ unsigned valid_total;
-    const unsigned b = blockIdx.x;
+    const unsigned b = blockIdx.y;
     const float* s_row = scores + static_cast<size_t>(b) * m;
     const int32_t* idx_row = indexes + static_cast<size_t>(b) * m;
     if (threadIdx.x == 0) { valid_total = 0; }
     __syncthreads();
     unsigned mine = 0;
-    for (unsigned e = threadIdx.x; e < n_pad; e += kSortThreads) {
-        unsigned long long key = 0;  // padding and skipped entries sort last
-        if (e < m) {
-            const int32_t s = idx_row[e];
-            if (s >= 0 && static_cast<unsigned>(s) < n_items) {
-                key = (static_cast<unsigned long long>(ordered_key(s_row[e])) << 32) | (0xffffffffu - e);
+    for (unsigned e0 = threadIdx.x; e0 < n_pad; e0 += 8 * kRankThreads) {
+        int32_t slot[8];
+        float sc[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {                    // both loads of all eight entries at once
+            const unsigned e = e0 + u * kRankThreads;
+            slot[u] = e < m ? idx_row[e] : -1;
+            sc[u] = e < m ? s_row[e] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const unsigned e = e0 + u * kRankThreads;
+            unsigned long long key = 0;  // padding and skipped entries: below every candidate
+            if (slot[u] >= 0 && static_cast<unsigned>(slot[u]) < n_items) {
+                key = (static_cast<unsigned long long>(ordered_key(sc[u])) << 32) | (0xffffffffu - e);
                 ++mine;
             }
+            if (e < n_pad) { keys[e] = key; }
         }
-        keys[e] = key;
     }
-    atomicAdd(&valid_total, mine);
+    if (blockIdx.x == 0) { atomicAdd(&valid_total, mine); }
     __syncthreads();
+    if (blockIdx.x == 0 && threadIdx.x == 0) { out_count[b] = max(0, min(static_cast<int>(valid_total), topk)); }
 
-    // bitonic sort, descending
-    for (unsigned size = 2; size <= n_pad; size <<= 1) {
-        for (unsigned stride = size >> 1; stride > 0; stride >>= 1) {
-            for (unsigned t = threadIdx.x; t < n_pad / 2; t += kSortThreads) {
-                const unsigned lo = 2 * t - (t & (stride - 1));
-                const unsigned hi = lo + stride;
-                const bool descending = (lo & size) == 0;
-                const unsigned long long a = keys[lo], c = keys[hi];
-                if ((a < c) == descending) { keys[lo] = c; keys[hi] = a; }
-            }
-            __syncthreads();
-        }
+    const unsigned cand = blockIdx.x * (kRankThreads / kLanes) + threadIdx.x / kLanes, sub = threadIdx.x % kLanes;
+    const unsigned long long my = cand < m ? keys[cand] : 0ull;
+    // two keys per 16-byte read, eight reads in flight; n_pad is a multiple of 16 * kLanes
+    typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+    const u64x2* pairs = reinterpret_cast<const u64x2*>(keys);
+    unsigned above = 0;
+    for (unsigned j = sub; j < n_pad / 2; j += 8 * kLanes) {
+        u64x2 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { v[u] = pairs[j + u * kLanes]; }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { above += (v[u].x > my ? 1u : 0u) + (v[u].y > my ? 1u : 0u); }
     }
-
-    const int valid = static_cast<int>(valid_total);
-    const int count = max(0, min(valid, topk));
-    for (int i = threadIdx.x; i < count; i += kSortThreads) {
-        const unsigned e = 0xffffffffu - static_cast<unsigned>(keys[i] & 0xffffffffu);
-        out_idx[static_cast<size_t>(b) * out_stride + i] = idx_row[e];
-        out_scores[static_cast<size_t>(b) * out_stride + i] = s_row[e];
+#pragma unroll
+    for (int d = 1; d < kLanes; d <<= 1) { above += __shfl_xor(above, d, 64); }
+    if (sub == 0 && my != 0ull && static_cast<int>(above) < topk) {      // (a valid key is never zero)
+        out_idx[static_cast<size_t>(b) * out_stride + above] = idx_row[cand];
+        out_scores[static_cast<size_t>(b) * out_stride + above] = s_row[cand];
     }
-    if (threadIdx.x == 0) { out_count[b] = count; }
 }
 
 }  // namespace
@@ -161,9 +195,8 @@ extern "C" int ucm_esa_retrieve(const float* data, int n_items, int dim, const f
     UCM_REQUIRE(ucm::aligned16(data) && ucm::aligned16(q), "ucm_esa_retrieve: data and q must be 16-byte aligned");
     UCM_REQUIRE(batch <= 65535, "ucm_esa_retrieve: batch=%d", batch);
     UCM_REQUIRE(out_stride >= std::min(std::max(topk, 0), m), "ucm_esa_retrieve: out_stride=%d too small", out_stride);
-    unsigned n_pad = 2;
-    while (n_pad < static_cast<unsigned>(m)) { n_pad <<= 1; }
-    UCM_SUPPORTED(n_pad <= 8192, "ucm_esa_retrieve: m=%d (at most 8192 candidates per request)", m);
+    UCM_SUPPORTED(m <= 8192, "ucm_esa_retrieve: m=%d (at most 8192 candidates per request)", m);
+    const unsigned n_pad = (static_cast<unsigned>(m) + 127u) & ~127u;    // whole rounds of the counting loop
     hipStream_t s = ucm::as_stream(stream);
     if (m > 0) {
         hipLaunchKernelGGL(esa_score_kernel, dim3((m + kSlots - 1) / kSlots, batch), dim3(kScoreThreads), 0, s,
@@ -171,8 +204,15 @@ extern "C" int ucm_esa_retrieve(const float* data, int n_items, int dim, const f
                            static_cast<unsigned>(m), scores_ws);
         if (int rc = ucm::check_hip(hipGetLastError(), "ucm_esa_retrieve(score)")) { return rc; }
     }
-    hipLaunchKernelGGL(esa_topk_kernel, dim3(batch), dim3(kSortThreads), n_pad * sizeof(unsigned long long), s,
-                       scores_ws, indexes, static_cast<unsigned>(n_items), static_cast<unsigned>(m), n_pad, topk,
-                       out_idx, out_scores, out_count, static_cast<unsigned>(out_stride));
+    if (m <= 1024) {
+        hipLaunchKernelGGL(esa_rank_kernel<1>, dim3((m + kRankThreads - 1) / kRankThreads + (m == 0), batch), dim3(kRankThreads),
+                           n_pad * sizeof(unsigned long long), s, scores_ws, indexes, static_cast<unsigned>(n_items),
+                           static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride));
+    } else {
+        constexpr int kPer = kRankThreads / 8;
+        hipLaunchKernelGGL(esa_rank_kernel<8>, dim3((m + kPer - 1) / kPer, batch), dim3(kRankThreads),
+                           n_pad * sizeof(unsigned long long), s, scores_ws, indexes, static_cast<unsigned>(n_items),
+                           static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride));
+    }
     UCM_LAUNCH_CHECK("ucm_esa_retrieve(select)");
 }

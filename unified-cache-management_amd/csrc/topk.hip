@@ -186,7 +186,7 @@ __global__ __launch_bounds__(64) void delta_plan_kernel(
 {
     const int r = blockIdx.x, l = blockIdx.y, lane = threadIdx.x;
     const size_t lr = static_cast<size_t>(l) * n_req + r;
-    const int k = min(count[lr], n_slots);          // selections beyond the slot budget cannot be resident
+    const int k = min(min(count[lr], n_slots), sel_stride);   // selections beyond the slot budget cannot be resident
     const int32_t* s = sel + lr * sel_stride;
     const int32_t* sp = sel_phys + lr * sel_stride;
     int32_t* res = resident + lr * n_slots;
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kPlanThreads) void delta_plan_wide_kernel(
     const int r = blockIdx.x, l = blockIdx.y, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const size_t lr = static_cast<size_t>(l) * n_req + r;
-    const int k = min(count[lr], n_slots);
+    const int k = min(min(count[lr], n_slots), sel_stride);   // (a count larger than a row of sel is never followed)
     const int32_t* s = sel + lr * sel_stride;
     const int32_t* sp = sel_phys + lr * sel_stride;
     int32_t* res = resident + lr * n_slots;
