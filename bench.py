@@ -58,6 +58,8 @@ def parse():
     ap.add_argument("--moves-leg", action="store_true",
                     help="also time the block-id driven load/dump (the configs[2] shape of the benchmark definition: 64 requests "
                          "x 16 blocks, all layers, K and V, random block table) on the same caches")
+    ap.add_argument("--esa-leg", action="store_true",
+                    help="also time the ESA retrieval backend (slot-list scoring + top-k) at three shapes")
     ap.add_argument("--kvstar-leg", action="store_true",
                     help="also time the multi-query softmax-vote retrieval (KVStar: 8 query tokens per request) on the same "
                          "ragged batch")
@@ -445,6 +447,32 @@ def main():
         }
         del ktab, flat, kws, kpr
 
+    # ---- ESA leg: the retrieval worker's backend call (scores of a slot list against a flat query in the
+    # reference's sequential order, best k in descending order) on a 16384-row table of 1024-wide representatives
+    esa_leg = None
+    if args.esa_leg:
+        e_data = torch.randn(16384, HKV * D, device=dev, generator=g)
+        esa_leg = []
+        for e_b, e_m, e_k in ((1, 512, 150), (64, 512, 150), (1, 8000, 3000)):
+            e_q = torch.randn(e_b, HKV * D, device=dev, generator=g)
+            e_idx = i32(np.stack([rng.permutation(16384)[:e_m] for _ in range(e_b)]))
+            e_ws = torch.zeros(e_b * e_m, device=dev)
+            e_oi = torch.zeros(e_b, e_k, dtype=torch.int32, device=dev)
+            e_os = torch.zeros(e_b, e_k, device=dev)
+            e_oc = torch.zeros(e_b, dtype=torch.int32, device=dev)
+            for _ in range(3):
+                ops.esa_retrieve(e_data, e_q, e_idx, e_k, e_ws, e_oi, e_os, e_oc)
+            torch.cuda.synchronize()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(50):
+                ops.esa_retrieve(e_data, e_q, e_idx, e_k, e_ws, e_oi, e_os, e_oc)
+            e1.record()
+            torch.cuda.synchronize()
+            esa_leg.append({"requests": e_b, "candidates": e_m, "topk": e_k,
+                            "us_per_call": round(e0.elapsed_time(e1) / 50 * 1000, 1)})
+        del e_data
+
     # ---- check the last step against the CPU oracle (selection, scores, gathered bytes)
     if not args.no_check:
         step(qs[n_q - 1])                                             # re-run the last full step: the delta leg reused the buffers
@@ -588,6 +616,7 @@ def main():
         "delta_gather": delta,
         "kv_moves": moves_leg,
         "hash_retrieval": hash_leg,
+        "esa_retrieval": esa_leg,
         "kvstar_retrieval": kvstar_leg,
         "cpu_baseline": cpu,
         "checked": checked,
