@@ -97,7 +97,10 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  * ucm/sparse/gsa/gsa.py:501 configures it).
  *   q          dev: queries, q_dtype fp32 or bf16, [n_layers][*][q_heads][head_dim];
  *              layer l starts q_layer_stride ELEMENTS after layer l-1; request
- *              r reads row q_rows[r] (q_rows == NULL: row r).  This is the
+ *              r reads row q_rows[r] (q_rows == NULL: row r); with q_rows,
+ *              q_layer_stride is also the bound of a layer's rows: a request
+ *              whose row lies outside it is skipped, its scores are left as
+ *              they were (ucm_hash_encode_queries does the same).  This is the
  *              reference's gsa_q_cache (gsa.py:503-512) when fp32, or the
  *              layer's raw query tensor with q_rows = index of each request's
  *              last token (GSA.copy_q, gsa.py:616-632) when bf16.

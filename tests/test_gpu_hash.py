@@ -273,6 +273,27 @@ def test_hash_query_codes_near_zero_projections_and_scales(ucm, dev):
         assert want_q[3].any() and want_q[4].any()
 
 
+def test_hash_query_rows_outside_the_layer_are_skipped(ucm, dev):
+    """A request whose q_rows entry is negative or past the layer's queries leaves its outputs untouched."""
+    from ucm_amd import ops
+
+    hq, hkv, n_tok = 32, 8, 5
+    w_bits, w_f32 = make_weights(870)
+    q_h = synth.normal_bf16_bits(871, (2, n_tok, hq, 128))
+    q_rows = np.array([4, -3, 5, 0], np.int32)
+    q_codes = torch.full((2, 4, hq, 16), 0xEE, dtype=torch.uint8, device=dev)
+    q_sum = torch.full((2, 4, 128), 77, dtype=torch.int16, device=dev)
+    qbar = torch.full((2, 4, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(bf16_dev(q_h, dev), bf16_dev(w_bits, dev), hkv, q_codes, q_sum, qbar, 4, q_rows=i32(q_rows, dev))
+    torch.cuda.synchronize()
+    for l in range(2):
+        for r, row in enumerate(q_rows):
+            if 0 <= row < n_tok:
+                assert np.array_equal(q_codes[l, r].cpu().numpy(), O.hash_encode(q_h[l, row], w_f32)), (l, r)
+            else:
+                assert (q_codes[l, r] == 0xEE).all() and (q_sum[l, r] == 77).all() and (qbar[l, r] == 0xEE).all(), (l, r)
+
+
 def test_hash_queries_scores_and_selection(ucm, dev):
     """Config-5 shape in small: ragged batch, 8 kv heads, 32 query heads, 2 layers."""
     from ucm_amd import ops

@@ -234,6 +234,35 @@ def test_q_rows_indirection_and_tile_sizes(ucm, dev):
         ops.set_score_tile(0)
 
 
+@pytest.mark.parametrize("repre_dtype", [torch.float32, torch.bfloat16])
+def test_query_rows_outside_the_layer_are_skipped(ucm, dev, repre_dtype):
+    """q_rows comes from device memory: a request whose query row is negative or past the layer's block of
+    queries is not followed - its scores stay as they were - and the other requests are scored as usual."""
+    from ucm_amd import ops
+
+    hkv, g, d, n_tok = 8, 4, 128, 9
+    lens = np.array([20, 70, 5, 33], np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    rows = int(lens.sum())
+    q = synth.normal_bf16_as_f32(61, (2, n_tok, hkv * g, d))
+    repre = synth.bf16_widen(synth.bf16_round_bits(synth.normal_f32(62, (2, rows, hkv * d))))
+    q_rows = np.array([3, n_tok, 8, -1], np.int32)          # the second is one past the end, the last negative
+    scores = torch.full((2, rows), -5.0, device=dev)
+    ops.score_blocks(torch.from_numpy(q).to(dev).to(torch.bfloat16), torch.from_numpy(repre).to(dev).to(repre_dtype),
+                     i32(off, dev), i32(lens, dev), int(lens.max()), hkv, scores, q_rows=i32(q_rows, dev))
+    got = scores.cpu().numpy()
+    topk = np.full(len(lens), 4, np.int32)
+    for l in range(2):
+        ql = q[l][np.clip(q_rows, 0, n_tok - 1)]
+        _, _, want = O.select_topk_bs(ql, repre[l], off, lens, topk, hkv)
+        for r, ok in enumerate([True, False, True, False]):
+            seg = slice(off[r], off[r] + lens[r])
+            if ok:
+                assert np.array_equal(bits(got[l][seg]), bits(want[seg])), (l, r)
+            else:
+                assert np.all(got[l][seg] == -5.0), (l, r)
+
+
 def test_many_requests_dense_tile_lookup(ucm, dev):
     """More requests than one wavefront scans at once (the tile -> request lookup runs in trips of 64),
     with empty requests in between, and the grid sized from the host-known total."""

@@ -551,8 +551,10 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
     const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned half = lane >> 5, lr32 = lane & 31;
     const unsigned col = wave * 32 + lr32;               // the weight column this lane ends up with
-    const unsigned short* qp = q + static_cast<int64_t>(l) * q_layer_stride +
-                               static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kDim;
+    // a row index that came from device memory is followed only inside the layer's query block
+    const int64_t q_row = q_rows ? static_cast<int64_t>(q_rows[r]) : r;
+    if (q_rows && (q_row < 0 || (q_row + 1) * q_heads * kDim > q_layer_stride)) { return; }  // (the whole workgroup)
+    const unsigned short* qp = q + static_cast<int64_t>(l) * q_layer_stride + q_row * q_heads * kDim;
     const size_t lrq = static_cast<size_t>(l) * n_req + r;
     const unsigned g = q_heads / kv_heads;
     const float inv = 1.0f / static_cast<float>(g);
@@ -843,6 +845,9 @@ extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_strid
     UCM_SUPPORTED(head_dim == kDim && bits == kBits, "ucm_hash_encode_queries: head_dim=%d bits=%d (128 and 128)", head_dim, bits);
     UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0,
                 "ucm_hash_encode_queries: q_heads=%d kv_heads=%d", q_heads, kv_heads);
+    UCM_REQUIRE(!q_rows || q_layer_stride >= static_cast<int64_t>(q_heads) * head_dim,
+                "ucm_hash_encode_queries: with q_rows, q_layer_stride=%lld bounds the rows and must hold at least one",
+                static_cast<long long>(q_layer_stride));
     UCM_SUPPORTED(q_heads <= kMaxQHeads && kv_heads <= kMaxHeads, "ucm_hash_encode_queries: q_heads=%d kv_heads=%d (at most %d and %d)",
                   q_heads, kv_heads, kMaxQHeads, kMaxHeads);
     hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),

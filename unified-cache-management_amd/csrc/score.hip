@@ -157,6 +157,9 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
     const int l = blockIdx.y;
     int r, tile;
     if (!find_tile(seg_len, n_req, tile_blocks, blockIdx.x, lane, r, tile)) { return; }
+    // a row index that came from device memory is followed only inside the layer's query block
+    const int64_t q_row = q_rows ? static_cast<int64_t>(q_rows[r]) : r;
+    if (q_rows && (q_row < 0 || (q_row + 1) * q_heads * kD > q_layer_stride)) { return; }   // (the whole workgroup)
     const int n = seg_len[r];
     const int tile0 = tile * tile_blocks;
     const int tile_end = min(tile0 + tile_blocks, n);
@@ -185,7 +188,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
         const int g = q_heads / kv_heads;
         const float inv = 1.0f / static_cast<float>(g);
         const QT* qp = q + static_cast<int64_t>(l) * q_layer_stride +
-                       static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kD;
+                       q_row * q_heads * kD;
         for (int e = threadIdx.x * 4; e < row; e += kThreads * 4) {
             const int hh = e / kD, d = e - hh * kD;
             const f32x4 mean = group_mean4_any(qp + static_cast<int64_t>(hh) * g * kD + d, kD, g, inv);
@@ -278,6 +281,9 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(
     const int l = blockIdx.y;
     int r, tile;
     if (!find_tile(seg_len, n_req, tile_blocks, blockIdx.x, lane, r, tile)) { return; }
+    // a row index that came from device memory is followed only inside the layer's query block
+    const int64_t q_row = q_rows ? static_cast<int64_t>(q_rows[r]) : r;
+    if (q_rows && (q_row < 0 || (q_row + 1) * q_heads * kD > q_layer_stride)) { return; }   // (the whole workgroup)
     const int n = seg_len[r];
     const int tile0 = tile * tile_blocks;
     const int tile_end = min(tile0 + tile_blocks, n);
@@ -308,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(
         const int g = q_heads / kv_heads;
         const float inv = 1.0f / static_cast<float>(g);
         const QT* qp = q + static_cast<int64_t>(l) * q_layer_stride +
-                       static_cast<int64_t>(q_rows ? q_rows[r] : r) * q_heads * kD;
+                       q_row * q_heads * kD;
         for (int e = threadIdx.x * 4; e < row; e += kThreads * 4) {
             const int hh = e / kD, d = e - hh * kD;
             const f32x4 mean = group_mean4_any(qp + static_cast<int64_t>(hh) * g * kD + d, kD, g, inv);
@@ -408,6 +414,9 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
                 "ucm_score_blocks: repre not 16-byte aligned");
     UCM_SUPPORTED(repre_dtype == UCM_DTYPE_F32 || 32 % kv_heads == 0, "ucm_score_blocks: kv_heads=%d", kv_heads);
     UCM_REQUIRE(ucm::aligned16(q) && q_layer_stride % 8 == 0, "ucm_score_blocks: q not 16-byte aligned");
+    UCM_REQUIRE(!q_rows || q_layer_stride >= static_cast<int64_t>(q_heads) * head_dim,
+                "ucm_score_blocks: with q_rows, q_layer_stride=%lld bounds the rows and must hold at least one",
+                static_cast<long long>(q_layer_stride));
     if (n_req == 0 || max_seg_len == 0) { return UCM_OK; }
     hipStream_t s = ucm::as_stream(stream);
     // upper bound of sum(ceil(seg_len / tile)): exact to within n_req when the host knows the total
