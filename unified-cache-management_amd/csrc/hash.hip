@@ -786,6 +786,62 @@ __global__ __launch_bounds__(256) void hash_score_kernel(
     }
 }
 
+// Block-code score on its own: 128 bytes per block, so what counts is the number of requests in flight,
+// not arithmetic.  Eight lanes share a block, lane h holding kv head h's 128-bit majority code (one
+// 16-byte load); a thread handles four blocks, 32 apart, whose loads are issued together; the owning
+// request of a block is found without an early exit, so the segment lengths arrive in a few wide scalar
+// loads.
+// grid: x = 128 rows of the ragged batch (dense numbering), y = layer; 256 threads
+constexpr int kCodeBlocksPerGroup = 128;
+
+__global__ __launch_bounds__(256) void hash_code_score_kernel(
+    const unsigned* __restrict__ qbar_codes, const unsigned* __restrict__ block_codes, int64_t bc_layer_stride,
+    const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len, unsigned n_req, unsigned kv_heads,
+    float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16)
+{
+    const unsigned l = blockIdx.y, h = threadIdx.x & 7;
+    int req[4];
+    int64_t row[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { req[u] = -1; row[u] = 0; }
+    const int first = blockIdx.x * kCodeBlocksPerGroup + (threadIdx.x >> 3);
+    int base = 0;
+    for (unsigned i = 0; i < n_req; ++i) {
+        const int n = max(seg_len[i], 0), off = seg_off[i];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int dense = first + 32 * u;
+            if (req[u] < 0 && dense < base + n) { req[u] = static_cast<int>(i); row[u] = static_cast<int64_t>(off) + (dense - base); }
+        }
+        base += n;
+    }
+    u32x4 bc[4], qc[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        bc[u] = qc[u] = u32x4{0u, 0u, 0u, 0u};
+        if (req[u] >= 0 && h < kv_heads) {
+            bc[u] = ucm::gload16(block_codes + static_cast<int64_t>(l) * bc_layer_stride + (row[u] * kv_heads + h) * 4);
+            qc[u] = ucm::gload16(qbar_codes + ((static_cast<size_t>(l) * n_req + req[u]) * kv_heads + h) * 4);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        int score = 0;
+        if (h < kv_heads) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) { score += 32 - __popc(bc[u][k] ^ qc[u][k]); }
+        }
+        score += __shfl_xor(score, 4, 8);
+        score += __shfl_xor(score, 2, 8);
+        score += __shfl_xor(score, 1, 8);
+        if (req[u] >= 0 && h == 0) {
+            float f = static_cast<float>(score);
+            if (round_fp16) { f = half_round(f); }
+            scores[static_cast<int64_t>(l) * scores_layer_stride + row[u]] = f;
+        }
+    }
+}
+
 int g_encode_groups = 4096;
 
 }  // namespace
@@ -881,11 +937,13 @@ extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8
                            static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores, scores_layer_stride,
                            round_fp16);
     } else {
-        hipLaunchKernelGGL(hash_score_kernel<1>, dim3(gx, n_layers), dim3(256), 0, s, q_sum,
-                           reinterpret_cast<const unsigned*>(qbar_codes), colsum, colsum_layer_stride,
-                           reinterpret_cast<const unsigned*>(block_codes), block_codes_layer_stride / 4, seg_off, seg_len,
-                           static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores, scores_layer_stride,
-                           round_fp16);
+        UCM_REQUIRE(ucm::aligned16(qbar_codes) && ucm::aligned16(block_codes) && block_codes_layer_stride % 16 == 0,
+                    "ucm_hash_score_blocks: codes must be 16-byte aligned");
+        const unsigned gc = static_cast<unsigned>((total_blocks + kCodeBlocksPerGroup - 1) / kCodeBlocksPerGroup);
+        hipLaunchKernelGGL(hash_code_score_kernel, dim3(gc, n_layers), dim3(256), 0, s,
+                           reinterpret_cast<const unsigned*>(qbar_codes), reinterpret_cast<const unsigned*>(block_codes),
+                           block_codes_layer_stride / 4, seg_off, seg_len, static_cast<unsigned>(n_req),
+                           static_cast<unsigned>(kv_heads), scores, scores_layer_stride, round_fp16);
     }
     UCM_LAUNCH_CHECK("ucm_hash_score_blocks");
 }

@@ -43,6 +43,7 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
     const size_t lr = static_cast<size_t>(l) * n_req + r;
     int n = seg_len[r];
     n = min(n, min(out_stride, 64 * kEpl));  // host checked; clamp so nothing can run past a row
+    if (block_tables) { n = min(n, bt_stride); }
     const int k = topk_len[r];
     int32_t* out = idx_out + lr * out_stride;
     int32_t* pout = phys_out ? phys_out + lr * out_stride : nullptr;
