@@ -728,18 +728,15 @@ __device__ __forceinline__ float half_round(float x)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 
-// Integer block scores.  Sixteen lanes share one block: in mode 0 lane j owns
-// bits 8j..8j+7 of the 128-entry column-sum row (one 16-byte load per kv head,
-// 256 contiguous bytes per 16 lanes), in mode 1 lanes 0..kv_heads*4-1 each own
-// one 32-bit word of the block code; a 16-lane DPP-free shuffle reduction adds
+// Integer block scores <sum_i u(q_i), sum_h S[h]>.  Sixteen lanes share one block:
+// lane j owns bits 8j..8j+7 of the 128-entry column-sum row (one 16-byte load per
+// kv head, 256 contiguous bytes per 16 lanes); a 16-lane shuffle reduction adds
 // the partial scores.  Requests are found by a scan of the segment lengths
 // (they are few; rows are many).
 // grid: x = 16 rows of the ragged batch (dense numbering), y = layer; 256 threads
-template <int kMode>
 __global__ __launch_bounds__(256) void hash_score_kernel(
-    const short* __restrict__ q_sum, const unsigned* __restrict__ qbar_codes,
-    const short* __restrict__ colsum, int64_t cs_layer_stride, const unsigned* __restrict__ block_codes,
-    int64_t bc_layer_stride, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
+    const short* __restrict__ q_sum, const short* __restrict__ colsum, int64_t cs_layer_stride,
+    const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
     unsigned n_req, unsigned kv_heads, float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16)
 {
     const unsigned l = blockIdx.y;
@@ -756,24 +753,16 @@ __global__ __launch_bounds__(256) void hash_score_kernel(
     if (r >= 0) {
         row = static_cast<int64_t>(seg_off[r]) + local;
         const size_t lr = static_cast<size_t>(l) * n_req + r;
-        if (kMode == 0) {
-            // <sum_i u(q_i), sum_h S[h]>
-            const short* cs = colsum + static_cast<int64_t>(l) * cs_layer_stride + row * kv_heads * kBits + sub * 8;
-            const i16x8 qv = *reinterpret_cast<const i16x8*>(q_sum + lr * kBits + sub * 8);
-            int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            for (unsigned h = 0; h < kv_heads; ++h) {
-                const i16x8 v = *reinterpret_cast<const i16x8*>(cs + h * kBits);
+        const short* cs = colsum + static_cast<int64_t>(l) * cs_layer_stride + row * kv_heads * kBits + sub * 8;
+        const i16x8 qv = *reinterpret_cast<const i16x8*>(q_sum + lr * kBits + sub * 8);
+        int s[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (unsigned h = 0; h < kv_heads; ++h) {
+            const i16x8 v = *reinterpret_cast<const i16x8*>(cs + h * kBits);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) { s[k] += v[k]; }
-            }
-#pragma unroll
-            for (int k = 0; k < 8; ++k) { score += static_cast<int>(qv[k]) * s[k]; }
-        } else {
-            // sum over kv heads of (bits - hamming(code of the group-mean query, majority code of the block))
-            const unsigned* bc = block_codes + static_cast<int64_t>(l) * bc_layer_stride + row * kv_heads * 4;
-            const unsigned* qc = qbar_codes + lr * kv_heads * 4;
-            for (unsigned wd = sub; wd < kv_heads * 4; wd += 16) { score += 32 - __popc(bc[wd] ^ qc[wd]); }
+            for (int k = 0; k < 8; ++k) { s[k] += v[k]; }
         }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { score += static_cast<int>(qv[k]) * s[k]; }
     }
     score += __shfl_xor(score, 8, 16);
     score += __shfl_xor(score, 4, 16);
@@ -786,7 +775,8 @@ __global__ __launch_bounds__(256) void hash_score_kernel(
     }
 }
 
-// Block-code score on its own: 128 bytes per block, so what counts is the number of requests in flight,
+// Block-code score: sum over kv heads of (bits - hamming(code of the group-mean query, majority code of the
+// block)).  128 bytes per block, so what counts is the number of requests in flight,
 // not arithmetic.  Eight lanes share a block, lane h holding kv head h's 128-bit majority code (one
 // 16-byte load); a thread handles four blocks, 32 apart, whose loads are issued together; the owning
 // request of a block is found without an early exit, so the segment lengths arrive in a few wide scalar
@@ -931,11 +921,9 @@ extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8
     const unsigned gx = static_cast<unsigned>((total_blocks + 15) / 16);
     hipStream_t s = ucm::as_stream(stream);
     if (mode == 0) {
-        hipLaunchKernelGGL(hash_score_kernel<0>, dim3(gx, n_layers), dim3(256), 0, s, q_sum,
-                           reinterpret_cast<const unsigned*>(qbar_codes), colsum, colsum_layer_stride,
-                           reinterpret_cast<const unsigned*>(block_codes), block_codes_layer_stride / 4, seg_off, seg_len,
-                           static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores, scores_layer_stride,
-                           round_fp16);
+        hipLaunchKernelGGL(hash_score_kernel, dim3(gx, n_layers), dim3(256), 0, s, q_sum, colsum, colsum_layer_stride,
+                           seg_off, seg_len, static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores,
+                           scores_layer_stride, round_fp16);
     } else {
         UCM_REQUIRE(ucm::aligned16(qbar_codes) && ucm::aligned16(block_codes) && block_codes_layer_stride % 16 == 0,
                     "ucm_hash_score_blocks: codes must be 16-byte aligned");
