@@ -245,7 +245,10 @@ int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* c
  *           as <q_sum, sum_h colsum[h]> (the same integer); round_fp16 != 0
  *           rounds it to fp16 as the reference's fp16 sum does.
  *   mode 1  sum over kv heads of (128 - hamming(qbar code, majority block code)),
- *           the benchmark's block-code variant (not present in the reference).
+ *           the benchmark's block-code variant (not present in the reference);
+ *           qbar_codes, block_codes and block_codes_layer_stride must be
+ *           multiples of 16 bytes (UCM_EINVAL otherwise): a kv head's code is
+ *           read as one 16-byte load.
  * The reference keeps init 1 / local 2 blocks out of the candidates and
  * index-sorts its picks (kvcomp.py:219-221,249-254): ucm_topk_windows with the
  * matching windows gives the same set.
