@@ -401,7 +401,7 @@ def main():
 
         def kvstar_step():
             ops.kvstar_votes(kq, kq_off, kx, HQ, flat, kso, ksl, max_len, kvotes, kws, d_pruned=kdp, pruned=kpr, pruned_sel=ksel)
-            ops.topk_windows(kvotes.view(1, -1), kso, ksl, ktk, max_len, kidx, kcnt, start_w=0, end_w=0)
+            ops.kvstar_topk(kvotes, kso, ksl, ktk, max_len, kidx[0], kcnt[0])
 
         for _ in range(2):
             kvstar_step()

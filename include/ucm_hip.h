@@ -298,7 +298,7 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  * query rows against all sub-block representatives of the task, softmax of
  * every row over the task's sub-blocks, votes[block] = sum over rows and over
  * the block's sub-blocks of the probabilities.  The top-k of the votes is
- * taken by ucm_topk_windows (init_w = local_w = 0).  fp32 on the matrix cores;
+ * taken by ucm_kvstar_topk.  fp32 on the matrix cores;
  * agrees with the reference's scalar loop to rounding, not bit for bit.
  *   q_f16    dev fp16; task t's [n_tokens][q_heads][d_orig] block starts
  *            q_off[t] elements in (dev int64[n_tasks])
@@ -356,6 +356,23 @@ int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_token
                             int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                             int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
                             ucm_stream_t stream);
+
+/*
+ * The selection step of KVStar::Execute on the votes of n_tasks tasks
+ * (simd_compute_kernel.cpp:955-977): a min-heap of (score, block) pairs that
+ * blocks enter in index order and that, once it holds topk pairs, replaces its
+ * smallest pair only for a strictly greater score.  Which of several blocks
+ * tied at the k-th score survive follows that process exactly (not the
+ * lowest-index rule of ucm_topk_windows).  idx_out[t*out_stride + j] holds the
+ * chosen blocks of task t in ASCENDING index order, count_out[t] =
+ * min(topk_len[t], seg_len[t]) of them; the reference returns them descending
+ * by (score, index), an order the caller restores by sorting these few
+ * entries.  votes as written by ucm_kvstar_votes (task t's at
+ * votes[seg_off[t] + b]); topk_len[t] >= 1; at most 4096 blocks per task.
+ */
+int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const int32_t* seg_len,
+                    const int32_t* topk_len, int n_tasks, int max_seg_len, int32_t* idx_out,
+                    int out_stride, int32_t* count_out, ucm_stream_t stream);
 
 /*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched

@@ -83,6 +83,7 @@ _orc_kvstar_block_repre = _sig(_orc, "orc_kvstar_block_repre", None, _p, _p, _p,
 _orc_kvstar_retrieve = _sig(_orc, "orc_kvstar_retrieve", _i32, _p, _u32, _u32, _u32, _p, _u32, _u32, _u32, _u32, _u32, _p,
                             _u32, _p, _p)
 _orc_f32_to_bf16 = _sig(_orc, "orc_f32_to_bf16", C.c_uint16, _f32)
+_orc_kvstar_topk = _sig(_orc, "orc_kvstar_topk", _i32, _p, _u32, _u32, _p)
 
 
 # ---------------------------------------------------------------- bf16 helpers
@@ -335,6 +336,18 @@ def kvstar_retrieve(q_bits: np.ndarray, repre: np.ndarray, topk: int, pruned=Non
     k = _orc_kvstar_retrieve(_ptr(qb), x, hq, d, _ptr(rp), n, m, h, dp, d_pad, None if pr is None else _ptr(pr), topk,
                              _ptr(final), _ptr(idx))
     return idx[:k].copy(), final
+
+
+def kvstar_topk(final_scores: np.ndarray, topk: int) -> np.ndarray:
+    """The heap top-k of KVStar::Execute on given per-block scores: indices, descending by (score, index)."""
+    f = _c(final_scores, np.float32)
+    out = np.zeros(max(min(int(topk), len(f)), 1), np.int32)
+    k = _orc_kvstar_topk(_ptr(f), len(f), int(topk), _ptr(out))
+    return out[:k].copy()
+
+
+def f32_to_bf16(x: float) -> int:
+    return int(_orc_f32_to_bf16(float(x)))
 
 
 class _Ref:

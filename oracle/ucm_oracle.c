@@ -784,6 +784,52 @@ ORC_API void orc_kvstar_block_repre(const uint16_t* cache, const int32_t* block_
 }
 
 /*
+ * The top-k step of KVStar::Execute
+ * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:955-977),
+ * restated literally: a min-heap of (score, index) pairs compared
+ * lexicographically (std::greater on std::pair); blocks are offered in index
+ * order; while the heap holds fewer than topk pairs a block is pushed, after
+ * that it replaces the heap's smallest pair only if its score is STRICTLY
+ * greater than that pair's score; at the end the pairs are popped smallest
+ * first and written from the back, so the output is descending by (score,
+ * index): equal scores come out higher index first.  Which of several blocks
+ * tied at the k-th score survive therefore depends on the order of arrival
+ * (see tests/test_oracle_pins.py for the closed form the device code uses).
+ * The "heap" here is a plain array searched for its smallest pair: the
+ * priority queue's internal layout never shows in its results.
+ */
+ORC_API int32_t orc_kvstar_topk(const float* final_scores, uint32_t n_blocks, uint32_t topk, int32_t* topk_idx)
+{
+    orc_pair* heap = (orc_pair*)malloc((size_t)(topk ? topk : 1) * sizeof(orc_pair));
+    uint32_t size = 0;
+    for (uint32_t n = 0; n < n_blocks; ++n) {
+        uint32_t lo = 0;   /* position of the smallest (score, index) pair */
+        for (uint32_t i = 1; i < size; ++i) {
+            if (heap[i].score < heap[lo].score || (heap[i].score == heap[lo].score && heap[i].idx < heap[lo].idx)) { lo = i; }
+        }
+        if (size < topk) {
+            heap[size].score = final_scores[n];
+            heap[size].idx = (int32_t)n;
+            ++size;
+        } else if (size > 0 && final_scores[n] > heap[lo].score) {
+            heap[lo].score = final_scores[n];
+            heap[lo].idx = (int32_t)n;
+        }
+    }
+    /* pop smallest first, fill from the back */
+    for (uint32_t left = size; left > 0; --left) {
+        uint32_t lo = 0;
+        for (uint32_t i = 1; i < left; ++i) {
+            if (heap[i].score < heap[lo].score || (heap[i].score == heap[lo].score && heap[i].idx < heap[lo].idx)) { lo = i; }
+        }
+        topk_idx[left - 1] = heap[lo].idx;
+        heap[lo] = heap[left - 1];
+    }
+    free(heap);
+    return (int32_t)size;
+}
+
+/*
  * The retrieval itself, following the reference's portable path
  * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:817-990,
  * scalar_impl::execute_impl; its AVX2 and NEON twins at :635-764 and :270-390
@@ -832,11 +878,5 @@ ORC_API int32_t orc_kvstar_retrieve(const uint16_t* q, uint32_t n_tokens, uint32
     }
     free(row);
     free(qv);
-    const uint32_t k = topk < n_blocks ? topk : n_blocks;
-    orc_pair* pr = (orc_pair*)malloc((size_t)(n_blocks ? n_blocks : 1) * sizeof(orc_pair));
-    for (uint32_t b = 0; b < n_blocks; ++b) { pr[b].score = final_scores[b]; pr[b].idx = (int32_t)b; pr[b].pos = b; }
-    qsort(pr, n_blocks, sizeof(orc_pair), orc_cmp_pair_desc);
-    for (uint32_t i = 0; i < k; ++i) { topk_idx[i] = pr[i].idx; }
-    free(pr);
-    return (int32_t)k;
+    return orc_kvstar_topk(final_scores, n_blocks, topk, topk_idx);
 }

@@ -279,8 +279,7 @@ def _pruned_channels_and_selection(ops, dev, M, dp):
         seg_off, seg_len = torch.tensor([off[t]], dtype=torch.int32, device=dev), torch.tensor([n], dtype=torch.int32, device=dev)
         out = torch.zeros((1, 1, n), dtype=torch.int32, device=dev)
         cnt = torch.zeros((1, 1), dtype=torch.int32, device=dev)
-        ops.topk_windows(torch.from_numpy(got).to(dev).view(1, -1), seg_off, seg_len, torch.tensor([k], dtype=torch.int32, device=dev),
-                         n, out, cnt, start_w=0, end_w=0)
+        ops.kvstar_topk(torch.from_numpy(got).to(dev), seg_off, seg_len, torch.tensor([k], dtype=torch.int32, device=dev), n, out[0], cnt[0])
         check_selection(out[0, 0, : int(cnt[0, 0])].tolist(), want, k)
 
 
@@ -368,3 +367,51 @@ def test_kvstar_retrieve_batch(ucm, dev, ratio):
     bad = kvstar_retrieve.AsyncRetrieveBatch(qs[:2], [repres[0], repres[1].dense()], indexes[:2], topks[:2])
     assert kvstar_retrieve.GetTaskResult(bad[1])["status"] == "FAILURE"
     assert kvstar_retrieve.AsyncRetrieveBatch([], [], [], []) == []
+
+
+@pytest.mark.parametrize("max_len", [64, 100, 256, 700, 3000])
+def test_kvstar_topk_heap_ties(ucm, dev, max_len):
+    """ucm_kvstar_topk against the oracle's literal heap on votes full of ties (few distinct values), one launch for
+    many tasks of ragged length: the chosen SET must be the heap's, and sorting it by (vote, index) descending must
+    give the heap's order."""
+    from ucm_amd import ops
+
+    rng = np.random.default_rng(max_len)
+    n_tasks = 150
+    lens = rng.integers(1, max_len + 1, n_tasks).astype(np.int32)
+    lens[0], lens[1] = max_len, 1
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    ks = np.array([max(1, int(rng.integers(1, n + 3))) for n in lens], np.int32)
+    ks[2] = lens[2]                                             # k == n: everything
+    votes = rng.integers(0, 4, int(lens.sum())).astype(np.float32) * np.float32(0.25)
+    votes[off[3] : off[3] + lens[3]] = 1.0                      # one task with all votes equal
+    idx = torch.full((n_tasks, max_len), -1, dtype=torch.int32, device=dev)
+    cnt = torch.zeros(n_tasks, dtype=torch.int32, device=dev)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    ops.kvstar_topk(t(votes), t(off), t(lens), t(ks), max_len, idx, cnt)
+    torch.cuda.synchronize()
+    idx, cnt = idx.cpu().numpy(), cnt.cpu().numpy()
+    for i in range(n_tasks):
+        v = votes[off[i] : off[i] + lens[i]]
+        want = O.kvstar_topk(v, int(ks[i]))
+        got = idx[i, : cnt[i]]
+        assert cnt[i] == len(want) == min(ks[i], lens[i])
+        assert np.all(np.diff(got) > 0)
+        assert sorted(want.tolist()) == got.tolist(), (i, lens[i], ks[i])
+        assert sorted(got.tolist(), key=lambda b: (v[b], b), reverse=True) == want.tolist()
+    assert np.all(idx[np.arange(max_len)[None, :] >= cnt[:, None]] == -1)
+
+
+def test_kvstar_get_task_result_tie_order(ucm, dev):
+    """Through the module surface: blocks 1 and 3 identical, 0 and 2 identical and lower; k = 3.  The reference's heap
+    returns [3, 1, 2] (simd_compute_kernel.cpp:955-977)."""
+    from ucm_amd.sparse.kvstar import retrieve as kvstar_retrieve
+
+    rep = torch.zeros(4, 2, 1, 16, dtype=torch.float16, device=dev)
+    rep[1] = rep[3] = 0.5
+    q = torch.ones(1, 1, 16, dtype=torch.float16, device=dev)
+    kvstar_retrieve.Setup(kvstar_retrieve.SetupParam([0], 8, 0.5, 0, kvstar_retrieve.CPU, 1, 0))
+    tid = kvstar_retrieve.AsyncRetrieveByCPU(q, rep, None, 3, 0, kvstar_retrieve.CPU)
+    kvstar_retrieve.Wait(tid)
+    res = kvstar_retrieve.GetTaskResult(tid)
+    assert res["status"] == "SUCCESS" and res["data"] == [3, 1, 2]

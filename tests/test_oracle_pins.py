@@ -364,7 +364,7 @@ def _votes_fp64(q, rep):
 def test_kvstar_retrieve_closed_forms():
     """No build of the reference pins the KVStar restatement (it needs spdlog); what does: the definition
     evaluated in float64, sum(votes) = rows, invariance under a per-row shift of the scores, the channel
-    gather, sub-block means by hand, brute force on a tiny case with a tie."""
+    gather, sub-block means by hand.  The selection step has a test of its own (test_kvstar_heap_tie_rule)."""
     for seed, (x, hq, hkv, d, m, n) in enumerate([(5, 8, 2, 64, 4, 23), (1, 4, 4, 16, 1, 7), (8, 32, 8, 128, 8, 40), (3, 6, 3, 48, 2, 1)]):
         rep = (synth.normal_f32(40 + seed, (n, m, hkv, d)) * np.float32(0.3)).astype(np.float16)
         q = (synth.normal_f32(50 + seed, (x, hq, d)) * np.float32(0.3)).astype(np.float16)
@@ -373,7 +373,8 @@ def test_kvstar_retrieve_closed_forms():
         want = _votes_fp64(q, rep)
         assert np.allclose(final, want, rtol=1e-5, atol=1e-6)
         assert abs(final.sum() - x * hq) < 1e-4 * x * hq
-        assert list(idx) == list(np.argsort(-want, kind="stable")[:k]) or np.min(np.diff(np.sort(want))) < 1e-6
+        assert sorted(idx) == sorted(np.argsort(-want, kind="stable")[:k]) or np.min(np.diff(np.sort(want))) < 1e-6
+        assert list(idx) == sorted(idx, key=lambda i: (final[i], i), reverse=True)
         # a dropped or transposed head mapping would show here: zeroing the keys of one kv head flattens its rows' softmax
         rep0 = rep.copy()
         rep0[:, :, 0, :] = 0
@@ -393,12 +394,6 @@ def test_kvstar_retrieve_closed_forms():
         pad[..., dp:] = 9.0
         _, fpad = O.kvstar_retrieve(q.view(np.uint16), pad.view(np.uint16), k, pruned=pr)
         assert np.array_equal(fpad, fp)
-    # ties: identical blocks get identical votes and the lower index comes first
-    rep = np.zeros((4, 2, 1, 16), np.float16)
-    rep[1] = rep[3] = 0.5
-    q = np.ones((1, 1, 16), np.float16)
-    idx, final = O.kvstar_retrieve(q.view(np.uint16), rep.view(np.uint16), 3)
-    assert final[1] == final[3] and final[0] == final[2] and list(idx) == [1, 3, 0]
 
 
 def test_kvstar_block_repre_by_hand():
@@ -422,3 +417,253 @@ def test_kvstar_block_repre_by_hand():
                     assert out[slot, m, h, p] == np.float32(b16).astype(np.float16).view(np.uint16)
                 assert not out[slot, m, h, 3:].any()
     assert not out[[0, 2, 3]].any()
+
+
+# ------------------------------------------ helpers the GPU tests use as ground truth
+
+def test_bf16_rounding_against_torch():
+    """orc_f32_to_bf16 (and the numpy twin the tests use) against torch's float32 -> bfloat16 conversion, a
+    library routine: random values over the whole exponent range, every exact midpoint between neighbouring
+    bf16 values with its two float neighbours (ties go to even), zeros, subnormals, overflow to inf, inf, NaN."""
+    import torch
+
+    rng = np.random.default_rng(21)
+    u = rng.integers(0, 2**32, 200000, dtype=np.uint64).astype(np.uint32)
+    hi = rng.integers(0, 2**16, 40000, dtype=np.uint64).astype(np.uint32) << 16
+    mids = hi | np.uint32(0x8000)                          # exactly half way between bf16 `hi` and the next one
+    special = np.array([0x00000000, 0x80000000, 0x00000001, 0x80000001, 0x007FFFFF, 0x00800000, 0x7F7FFFFF, 0xFF7FFFFF,
+                        0x7F7F8000, 0x7F7F7FFF, 0x7F800000, 0xFF800000, 0x7FC00000, 0x7F800001, 0xFFFFFFFF, 0x7FBFFFFF,
+                        0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001], np.uint32)
+    allu = np.concatenate([u, mids, mids - np.uint32(1), mids + np.uint32(1), special])
+    x = allu.view(np.float32)
+    want = torch.from_numpy(x.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got_np = O.bf16_bits(x)
+    nan = np.isnan(x)
+    assert np.array_equal(got_np[~nan], want[~nan])
+    assert np.all((want[nan] & 0x7F80) == 0x7F80) and np.all((got_np[nan] & 0x7F80) == 0x7F80) and np.all(got_np[nan] & 0x7F)
+    pick = np.concatenate([rng.integers(0, len(u), 3000), np.arange(len(u), len(allu))])
+    for i in pick:
+        g = O.f32_to_bf16(x[i])
+        if nan[i]:
+            assert (g & 0x7F80) == 0x7F80 and (g & 0x7F)
+        else:
+            assert g == want[i], hex(int(allu[i]))
+    assert np.array_equal(synth.bf16_round_bits(x[~nan]), want[~nan])     # the generator's own rounding, same rule
+
+
+def test_block_mean_bf16_rounding_mode():
+    """round_bf16=True stores the sequential fp32 mean rounded once to bf16 (what the live torch path keeps,
+    gsa.py:640-652): equal, bit for bit, to torch's rounding of the unrounded oracle mean; within one bf16 step of
+    the exactly (float64) computed mean rounded once, and equal to it except where the fp32 sum sits at a tie."""
+    import torch
+
+    cache = synth.normal_bf16_bits(800, (6, 128, 8, 128))
+    ids, slots = [4, 1, 5], [0, 2, 1]
+    plain = np.zeros((3, 1024), np.float32)
+    rounded = np.zeros((3, 1024), np.float32)
+    O.block_mean_paged(cache, ids, slots, plain)
+    O.block_mean_paged(cache, ids, slots, rounded, round_bf16=True)
+    want = torch.from_numpy(plain).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(bits(rounded), bits(want))
+    exact = synth.bf16_widen(cache).astype(np.float64)[ids].mean(axis=1).reshape(3, 1024)[np.argsort(slots)]
+    once = torch.from_numpy(exact).to(torch.float32).to(torch.bfloat16).to(torch.float32).numpy()
+    step = np.abs(once) * 2.0 ** -7 + 1e-30
+    assert np.all(np.abs(rounded - once) <= step)
+    assert np.mean(rounded == once) > 0.99
+
+
+def test_hash_colsum_closed_form():
+    rng = np.random.default_rng(22)
+    for n, t, h, nb in [(3, 128, 8, 16), (2, 7, 1, 3), (1, 1, 2, 1), (4, 64, 4, 16)]:
+        tc = rng.integers(0, 256, (n, t, h, nb), dtype=np.uint8)
+        ones = np.unpackbits(tc, axis=-1, bitorder="little").astype(np.int64).sum(axis=1)   # [n, h, nb*8]
+        assert np.array_equal(O.hash_colsum(tc), (2 * ones - t).astype(np.int16))
+    tc = np.zeros((1, 128, 1, 16), np.uint8)
+    tc[0, :, 0, 5] = 0x81                                   # bits 40 and 47 set in every token
+    cs = O.hash_colsum(tc)[0, 0]
+    assert cs[40] == 128 and cs[47] == 128 and cs[41] == -128 and cs.sum() == 2 * 128 - 126 * 128
+
+
+def _exact_sign_codes(x: np.ndarray, w: np.ndarray) -> np.ndarray:
+    """Bits of sign(x . W[:, c]) > 0 with the products summed exactly (python integers over a common power of two)."""
+    from fractions import Fraction
+
+    n, dim = x.shape
+    nbits = w.shape[1]
+    wf = [[Fraction(float(w[d, c])) for c in range(nbits)] for d in range(dim)]
+    out = np.zeros((n, nbits), np.uint8)
+    for i in range(n):
+        xf = [Fraction(float(v)) for v in x[i]]
+        for c in range(nbits):
+            out[i, c] = sum((xf[d] * wf[d][c] for d in range(dim) if xf[d] != 0), Fraction(0)) > 0
+    return np.packbits(out, axis=-1, bitorder="little")
+
+
+def test_hash_encode_128x128_against_exact_sign():
+    """Both encoders at the shape every kernel runs (head_dim 128, 128 bits): against the float64 matrix product of
+    numpy where the projection is clear of zero, against exactly summed products on rows built to cancel (a
+    projection of exactly 0 is NOT positive: the bit is 0), and the LSB-first packing by construction."""
+    rng = np.random.default_rng(23)
+    dim = nbits = 128
+    w = synth.bf16_widen(synth.bf16_round_bits(rng.standard_normal((dim, nbits)).astype(np.float32) * 2))
+    xb = synth.normal_bf16_bits(8100, (300, dim))
+    x = synth.bf16_widen(xb)
+    proj = x.astype(np.float64) @ w.astype(np.float64)
+    clear = np.abs(proj) > 1e-9 * (np.abs(x).astype(np.float64) @ np.abs(w).astype(np.float64))
+    assert clear.mean() > 0.999
+    want = np.packbits((proj > 0).astype(np.uint8), axis=-1, bitorder="little")
+    got_b, got_f = O.hash_encode(xb, w), O.hash_encode_f32(x, w)
+    unp = lambda c: np.unpackbits(c, axis=-1, bitorder="little")
+    assert np.array_equal(unp(got_b)[clear], unp(want)[clear]) and np.array_equal(unp(got_f)[clear], unp(want)[clear])
+    exact = _exact_sign_codes(x[:4], w)
+    assert np.array_equal(got_b[:4], exact) and np.array_equal(got_f[:4], exact)
+    # cancelling rows: x has two equal entries, column c of W has opposite entries there -> projection exactly 0
+    xc = np.zeros((3, dim), np.float32)
+    wc = w.copy()
+    xc[0, [3, 77]] = 1.5
+    wc[3, 10], wc[77, 10] = 0.625, -0.625                   # column 10: exactly zero -> bit 0
+    wc[3, 11], wc[77, 11] = 0.625, -0.5                     # column 11: +0.1875 -> bit 1
+    wc[3, 12], wc[77, 12] = 0.5, -0.625                     # column 12: negative -> bit 0
+    xc[1] = 0                                               # all-zero vector: every bit 0
+    xc[2, 127] = -2.0 ** -120                               # tiny negative times column sign
+    for enc, arg in ((O.hash_encode, synth.bf16_round_bits(xc)), (O.hash_encode_f32, xc)):
+        codes = enc(arg, wc)
+        b = unp(codes)
+        assert (b[0, 10], b[0, 11], b[0, 12]) == (0, 1, 0)
+        assert not codes[1].any()
+        assert np.array_equal(b[2], (wc[127] < 0).astype(np.uint8))
+        assert np.array_equal(codes, _exact_sign_codes(xc, wc))
+    # packing: bit j of byte b is column 8b+j
+    one = np.zeros((1, dim), np.float32)
+    one[0, 0] = 1.0
+    wp = -np.ones((dim, nbits), np.float32)
+    wp[0, 8 * 5 + 3] = 1.0
+    codes = O.hash_encode_f32(one, wp)[0]
+    assert codes[5] == 1 << 3 and codes.sum() == 1 << 3
+    # an fp32 input that is not a bf16 value must not be rounded on the way in
+    xf = np.zeros((1, dim), np.float32)
+    xf[0, 0], xf[0, 1] = np.float32(1 + 2.0 ** -20), -1.0
+    w2 = np.zeros((dim, nbits), np.float32)
+    w2[0, 0] = w2[1, 0] = 1.0
+    assert O.hash_encode_f32(xf, w2)[0, 0] & 1 == 1
+
+
+def test_kv_gather_selected_placement():
+    """orc_kv_gather_selected against the placement rule spelled out with numpy indexing, on a poisoned staging
+    buffer: request r's region starts dst_off[r] blocks in and is [layer][K|V][region_k[r]] blocks; only the first
+    count[l][r] entries of phys are followed; nothing else is touched."""
+    rng = np.random.default_rng(24)
+    n_layers, nb, bb, n_req, stride = 3, 13, 32, 4, 6
+    layers = [rng.integers(0, 256, 2 * nb * bb, dtype=np.uint8) for _ in range(n_layers)]
+    count = rng.integers(0, stride + 1, (n_layers, n_req)).astype(np.int32)
+    count[0, 1] = 0
+    phys = rng.integers(0, nb, (n_layers, n_req, stride)).astype(np.int32)
+    region_k = count.max(axis=0).astype(np.int32) + np.array([0, 2, 0, 1], np.int32)
+    order = [2, 0, 3, 1]                                     # regions need not be in request order
+    dst_off = np.zeros(n_req, np.int64)
+    pos = 1
+    for r in order:
+        dst_off[r] = pos
+        pos += n_layers * 2 * int(region_k[r]) + 1           # a one-block gap after every region
+    staging = np.full(pos * bb, 0xA5, np.uint8)
+    O.kv_gather_selected(layers, nb * bb, bb, phys, count, dst_off, region_k, staging)
+    want = np.full((pos, bb), 0xA5, np.uint8)
+    for l in range(n_layers):
+        planes = layers[l].reshape(2, nb, bb)
+        for r in range(n_req):
+            for kv in range(2):
+                for j in range(count[l, r]):
+                    want[dst_off[r] + (l * 2 + kv) * region_k[r] + j] = planes[kv, phys[l, r, j]]
+    assert np.array_equal(staging.reshape(pos, bb), want)
+    assert (want == 0xA5).all(axis=1).sum() >= n_req + 1      # the gaps and unused tails stayed poisoned
+
+
+def test_topk_windows_i32_brute_force():
+    rng = np.random.default_rng(25)
+    for _ in range(2000):
+        n = int(rng.integers(1, 14))
+        k = int(rng.integers(0, 16))
+        sw, ew = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+        sc = rng.integers(-3, 3, n).astype(np.int32) * (1 if rng.random() < 0.5 else 1 << 20)
+        got = O.topk_windows(sc, k, sw, ew)
+        assert got.dtype == np.int32
+        if sw + ew >= n or k >= n or k == 0:
+            assert np.array_equal(got, np.arange(n))
+            continue
+        mid = sorted(range(sw, n - ew), key=lambda i: (-int(sc[i]), i))[: max(k - sw - ew, 0)]
+        full = list(range(sw)) + mid + list(range(n - ew, n))
+        want = sorted(full[:k]) if k >= sw + ew else full[:k]
+        assert list(got) == want, (n, k, sw, ew, sc)
+    # scores beyond float32's 24 bits would tie after a conversion; the supported range (|s| < 2^24) does not
+    sc = np.array([0, (1 << 24) - 1, (1 << 24) - 2, 5, -(1 << 24) + 1, 0], np.int32)
+    assert list(O.topk_windows(sc, 4, 1, 2)) == [0, 1, 4, 5]
+    assert list(O.topk_windows(sc, 5, 1, 2)) == [0, 1, 2, 4, 5]
+
+
+def _heap_topk(scores, k):
+    """KVStar's selection (simd_compute_kernel.cpp:955-977) with python's heapq, whose smallest-first order over
+    (score, index) tuples is std::priority_queue<pair, vector, greater>'s."""
+    import heapq
+
+    heap = []
+    for n, s in enumerate(scores):
+        if len(heap) < k:
+            heapq.heappush(heap, (float(s), n))
+        elif heap and s > heap[0][0]:
+            heapq.heapreplace(heap, (float(s), n))
+    out = [0] * len(heap)
+    pos = len(heap) - 1
+    while heap:
+        out[pos] = heapq.heappop(heap)[1]
+        pos -= 1
+    return out
+
+
+def kvstar_heap_closed_form(scores, k):
+    """The same selection without a heap (what the device code evaluates): with T the k-th largest score, every
+    block above T is kept; ties at T enter while fewer than k blocks >= T have been seen and leave, lowest index
+    first, once per block above T that arrives later.  So with P the shortest prefix holding k blocks >= T and
+    g_P / g the blocks above T in P / in all, the ties kept are those of P from rank g - g_P on."""
+    n = len(scores)
+    if k >= n:
+        keep = list(range(n))
+    else:
+        T = sorted(scores, reverse=True)[k - 1]
+        seen = g_p = 0
+        ties_in_p = []
+        for i, s in enumerate(scores):
+            if s >= T:
+                seen += 1
+                if s > T:
+                    g_p += 1
+                else:
+                    ties_in_p.append(i)
+                if seen == k:
+                    break
+        g = sum(1 for s in scores if s > T)
+        keep = [i for i, s in enumerate(scores) if s > T] + ties_in_p[g - g_p:]
+    return sorted(keep, key=lambda i: (scores[i], i), reverse=True)
+
+
+def test_kvstar_heap_tie_rule():
+    """The worked example: votes [a, b, a, b] with b > a and k = 3.  Blocks 0, 1, 2 fill the heap; block 3 (b) is
+    greater than the smallest pair (a, 0) and replaces it; popping smallest-first from the back gives (b,3), (b,1),
+    (a,2) -> [3, 1, 2].  (A lowest-index-first sort would give [1, 3, 0]: a different block at the k boundary.)"""
+    assert list(O.kvstar_topk(np.array([1, 2, 1, 2], np.float32), 3)) == [3, 1, 2]
+    assert list(O.kvstar_topk(np.array([2, 1, 1, 1], np.float32), 2)) == [0, 1]      # equal to the minimum: not replaced
+    assert list(O.kvstar_topk(np.array([1, 1, 2, 2], np.float32), 3)) == [3, 2, 1]
+    assert list(O.kvstar_topk(np.array([5, 4], np.float32), 7)) == [0, 1]
+    rng = np.random.default_rng(26)
+    for _ in range(3000):
+        n = int(rng.integers(1, 24))
+        k = int(rng.integers(1, 26))
+        sc = rng.integers(0, 4, n).astype(np.float32)
+        want = _heap_topk(sc, k)
+        assert list(O.kvstar_topk(sc, k)) == want, (sc, k)
+        assert kvstar_heap_closed_form(list(sc), k) == want, (sc, k)
+    # through the retrieval entry point: identical blocks get identical votes
+    rep = np.zeros((4, 2, 1, 16), np.float16)
+    rep[1] = rep[3] = 0.5
+    q = np.ones((1, 1, 16), np.float16)
+    idx, final = O.kvstar_retrieve(q.view(np.uint16), rep.view(np.uint16), 3)
+    assert final[1] == final[3] and final[0] == final[2] and list(idx) == [3, 1, 2]

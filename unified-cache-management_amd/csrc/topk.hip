@@ -30,8 +30,20 @@ __device__ __forceinline__ unsigned lanes_below(unsigned long long mask)
                                      __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
 }
 
+// kHeapTies selects which blocks tied at the k-th score are kept.  false: the
+// first ones in index order (std::stable_sort).  true: the ones KVStar's
+// min-heap of (score, index) pairs ends up with
+// (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:955-977:
+// blocks arrive in index order, a full heap replaces its smallest pair only
+// for a strictly greater score).  That process has a closed form: ties enter
+// while fewer than k blocks with key >= T have arrived and leave, lowest index
+// first, once per block above T that arrives later; so with P the shortest
+// prefix holding k blocks >= T, g_P the blocks above T inside P and g those in
+// the whole list, the ties kept are the ones of P whose rank among the ties is
+// at least g - g_P.  Windows are not used with it (host checked).
+//
 // grid: x = request, y = layer; block = one wave
-template <int kEpl>
+template <int kEpl, bool kHeapTies>
 __global__ __launch_bounds__(64) void topk_windows_kernel(
     const float* __restrict__ scores, int64_t scores_layer_stride, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, const int32_t* __restrict__ topk_len, int n_req, int start_w,
@@ -83,6 +95,7 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
         }
         unsigned T = 0;
         int need = 0;
+        int tie_lo = 0, tie_hi = 0;              // kHeapTies: ranks (among the ties) that are kept
         if (m > 0) {
             for (int bit = 31; bit >= 0; --bit) {
                 const unsigned c = T | (1u << bit);
@@ -95,6 +108,31 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
 #pragma unroll
             for (int j = 0; j < kEpl; ++j) { greater += __popcll(__ballot(key[j] > T)); }
             need = m - greater;
+            if (kHeapTies) {
+                // walk the list in index order up to the k-th block with key >= T
+                int seen = 0, g_p = 0;
+#pragma unroll
+                for (int j = 0; j < kEpl; ++j) {
+                    const unsigned long long ge_mask = __ballot(key[j] >= T && key[j] != 0u);
+                    const unsigned long long gt_mask = __ballot(key[j] > T);
+                    const int c = __popcll(ge_mask);
+                    if (seen < m) {
+                        if (seen + c >= m) {
+                            // lane holding the m-th one: the (m - seen)-th set bit of ge_mask
+                            const bool is_pth = ((ge_mask >> lane) & 1ull) && seen + static_cast<int>(lanes_below(ge_mask)) + 1 == m;
+                            const unsigned long long pm = __ballot(is_pth);
+                            const int p_lane = __ffsll(static_cast<long long>(pm)) - 1;
+                            const unsigned long long upto = p_lane >= 63 ? ~0ull : ((2ull << p_lane) - 1ull);
+                            g_p += __popcll(gt_mask & upto);
+                        } else {
+                            g_p += __popcll(gt_mask);
+                        }
+                    }
+                    seen += c;
+                }
+                tie_lo = greater - g_p;          // one tie left per block above T that came after P
+                tie_hi = m - g_p;                // ties inside P
+            }
         }
         int pos = 0, ties_seen = 0;
 #pragma unroll
@@ -106,7 +144,8 @@ __global__ __launch_bounds__(64) void topk_windows_kernel(
                 const bool gt = cand && m > 0 && key[j] > T;
                 const bool eq = cand && m > 0 && key[j] == T;
                 const unsigned long long eq_mask = __ballot(eq);
-                const bool take = window || gt || (eq && ties_seen + static_cast<int>(lanes_below(eq_mask)) < need);
+                const int tie_rank = ties_seen + static_cast<int>(lanes_below(eq_mask));
+                const bool take = window || gt || (eq && (kHeapTies ? (tie_rank >= tie_lo && tie_rank < tie_hi) : tie_rank < need));
                 ties_seen += __popcll(eq_mask);
                 const unsigned long long take_mask = __ballot(take);
                 if (take) {
@@ -153,7 +192,7 @@ extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride
     hipStream_t s = ucm::as_stream(stream);
     const dim3 grid(n_req, n_layers), block(64);
 #define UCM_TOPK_LAUNCH(EPL)                                                                                  \
-    hipLaunchKernelGGL(topk_windows_kernel<EPL>, grid, block, 0, s, scores, scores_layer_stride, seg_off,    \
+    hipLaunchKernelGGL((topk_windows_kernel<EPL, false>), grid, block, 0, s, scores, scores_layer_stride, seg_off, \
                        seg_len, topk_len, n_req, start_w, end_w, idx_out, out_stride, count_out, block_tables, \
                        bt_stride, phys_out, seq_lens, block_size, sparse_seq_lens)
     // registers per lane for the keys: the smallest tier that holds the longest request (the radix steps cost
@@ -167,6 +206,32 @@ extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride
     else { UCM_TOPK_LAUNCH(64); }
 #undef UCM_TOPK_LAUNCH
     UCM_LAUNCH_CHECK("ucm_topk_windows");
+}
+
+extern "C" int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const int32_t* seg_len,
+                               const int32_t* topk_len, int n_tasks, int max_seg_len, int32_t* idx_out,
+                               int out_stride, int32_t* count_out, ucm_stream_t stream)
+{
+    UCM_REQUIRE(n_tasks >= 0 && max_seg_len >= 0, "ucm_kvstar_topk: n_tasks=%d max_seg_len=%d", n_tasks, max_seg_len);
+    if (n_tasks == 0) { return UCM_OK; }
+    UCM_REQUIRE(votes && seg_off && seg_len && topk_len && idx_out && count_out, "ucm_kvstar_topk: null pointer");
+    UCM_REQUIRE(out_stride >= max_seg_len, "ucm_kvstar_topk: out_stride=%d < max_seg_len=%d", out_stride, max_seg_len);
+    UCM_SUPPORTED(max_seg_len <= 4096, "ucm_kvstar_topk: max_seg_len=%d (at most 4096 blocks per task)", max_seg_len);
+    hipStream_t s = ucm::as_stream(stream);
+    const dim3 grid(n_tasks, 1), block(64);
+#define UCM_HEAP_LAUNCH(EPL)                                                                                   \
+    hipLaunchKernelGGL((topk_windows_kernel<EPL, true>), grid, block, 0, s, votes, int64_t{0}, seg_off, seg_len, \
+                       topk_len, n_tasks, 0, 0, idx_out, out_stride, count_out, nullptr, 0, nullptr, nullptr, 1, \
+                       nullptr)
+    if (max_seg_len <= 64) { UCM_HEAP_LAUNCH(1); }
+    else if (max_seg_len <= 128) { UCM_HEAP_LAUNCH(2); }
+    else if (max_seg_len <= 256) { UCM_HEAP_LAUNCH(4); }
+    else if (max_seg_len <= 512) { UCM_HEAP_LAUNCH(8); }
+    else if (max_seg_len <= 1024) { UCM_HEAP_LAUNCH(16); }
+    else if (max_seg_len <= 2048) { UCM_HEAP_LAUNCH(32); }
+    else { UCM_HEAP_LAUNCH(64); }
+#undef UCM_HEAP_LAUNCH
+    UCM_LAUNCH_CHECK("ucm_kvstar_topk");
 }
 
 // ---------------------------------------------------------------------------

@@ -168,6 +168,18 @@ def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Ten
               _stream())
 
 
+def kvstar_topk(votes: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, topk_len: torch.Tensor,
+                max_seg_len: int, idx_out: torch.Tensor, count_out: torch.Tensor) -> None:
+    """votes fp32 [rows]; idx_out int32 [n_tasks, stride] (ascending block indices); count_out int32 [n_tasks]."""
+    n_tasks = seg_off.numel()
+    if idx_out.dim() != 2 or idx_out.shape[0] != n_tasks or count_out.numel() != n_tasks:
+        raise ValueError("idx_out [n_tasks,stride] and count_out [n_tasks] expected")
+    _lib.call("ucm_kvstar_topk", _dev(votes, torch.float32, "votes"), _dev(seg_off, torch.int32, "seg_off"),
+              _dev(seg_len, torch.int32, "seg_len"), _dev(topk_len, torch.int32, "topk_len"), n_tasks, max_seg_len,
+              _dev(idx_out, torch.int32, "idx_out"), idx_out.shape[1], _dev(count_out, torch.int32, "count_out"),
+              _stream())
+
+
 def esa_retrieve(data: torch.Tensor, q: torch.Tensor, indexes: torch.Tensor, topk: int, scores_ws: torch.Tensor,
                  out_idx: torch.Tensor, out_scores: torch.Tensor, out_count: torch.Tensor,
                  stream: Optional[int] = None) -> None:

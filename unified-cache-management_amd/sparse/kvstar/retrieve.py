@@ -151,8 +151,7 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
                 ws = ops.kvstar_workspace(1, h, x * (hq // h), n, m, table.shape[2] * 8, dev)
                 ops.kvstar_votes(q, torch.zeros(1, dtype=torch.int64, device=dev), x, hq, table, seg_off, seg_len, n, votes,
                                  ws, d_pruned=dp, pruned=pruned, pruned_sel=sel)
-                ops.topk_windows(votes.view(1, -1), seg_off, seg_len, torch.full((1,), k, dtype=torch.int32, device=dev), n,
-                                 idx, cnt, start_w=0, end_w=0)
+                ops.kvstar_topk(votes, seg_off, seg_len, torch.full((1,), k, dtype=torch.int32, device=dev), n, idx[0], cnt[0])
                 keep += (seg_off, seg_len, ws)
             event = torch.cuda.Event()
             event.record(_stream)
@@ -218,7 +217,7 @@ def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_id
                 ws = ops.kvstar_workspace(n_tasks, h, x * (hq // h), longest, m, r0.table.shape[2] * 8, dev)
                 ptrs = ops.kvstar_votes_tables(q, q_off, x, hq, [r.table for r in blk_repres], meta_d[0], meta_d[1], longest, votes, ws,
                                                d_pruned=dp, pruned=pruned, pruned_sel=sel)
-                ops.topk_windows(votes.view(1, -1), meta_d[0], meta_d[1], meta_d[2], longest, idx, cnt, start_w=0, end_w=0)
+                ops.kvstar_topk(votes, meta_d[0], meta_d[1], meta_d[2], longest, idx[0], cnt[0])
                 keep += (ws, ptrs)
             event = torch.cuda.Event()
             event.record(_stream)
@@ -239,19 +238,28 @@ def Wait(task_id: int) -> None:  # noqa: N802
 
 
 def GetTaskResult(task_id: int):  # noqa: N802
+    """Status dictionary of a task (py_intf.cpp:55-95); None for an id that is not (or no longer) known.  A finished
+    task is handed out once: delivering "SUCCESS" or "FAILURE" forgets the task and releases its device buffers
+    (the reference keeps every result for the life of the process)."""
     with _lock:
         task = _tasks.get(task_id)
     if task is None:
         return None
     if task.error is not None:
+        with _lock:
+            _tasks.pop(task_id, None)
         return {"status": "FAILURE", "error": task.error}
     if not task.event.query():
         return {"status": "RUNNING"}
     n = int(task.cnt)
-    chosen = task.idx[:n].long()
-    order = torch.argsort(task.votes[chosen], descending=True, stable=True)   # chosen is ascending: ties keep the lower index first
-    task.keep = ()
-    return {"status": "SUCCESS", "data": chosen[order].tolist()}
+    # descending by (score, index) as the reference's heap pops them (simd_compute_kernel.cpp:969-977): the device
+    # list is ascending, so a stable sort of its reverse leaves equal scores higher index first
+    chosen = task.idx[:n].long().flip(0)
+    order = torch.argsort(task.votes[chosen], descending=True, stable=True)
+    data = chosen[order].tolist()
+    with _lock:
+        _tasks.pop(task_id, None)
+    return {"status": "SUCCESS", "data": data}
 
 
 def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge: int, prune_ratio: float = 1.0,
