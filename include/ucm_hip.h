@@ -188,6 +188,25 @@ int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
                      ucm_stream_t stream);
 
 /*
+ * ucm_esa_retrieve for callers that cannot allocate (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): it has no
+ * counterpart in the reference.  Same arguments and results as
+ * ucm_esa_retrieve, minus scores_ws: the candidate scores go to a scratch
+ * array that is part of the library image (2 MiB per GPU, held until the
+ * process ends), so the call allocates nothing.  batch*m may be at most
+ * 524288 (2^19) candidate scores; a larger call fails with UCM_ENOTSUP.
+ * The first call on a GPU looks the array's device address up (no allocation).
+ * All calls on one GPU share the array: two of them that overlap in time (on
+ * different streams or from different threads) race; calls that follow one
+ * another on a stream do not.  Nothing in the array has to be cleared
+ * between calls (every score a call reads it has written itself).
+ */
+int ucm_esa_retrieve_static(const float* data, int n_items, int dim, const float* q,
+                            const int32_t* indexes, int batch, int m, int topk, int32_t* out_idx,
+                            float* out_scores, int32_t* out_count, int out_stride,
+                            ucm_stream_t stream);
+
+/*
  * Delta loads: decides, per (layer, request), which staging slots keep their
  * block and which missing block of the new selection goes where - the
  * "load delta" of ReqStatePerLayer.wait_retrieval_and_start_load

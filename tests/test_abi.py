@@ -66,6 +66,9 @@ def test_bad_arguments_fail_on_the_host(ucm):
     with pytest.raises(_lib.UcmHipError) as e:
         _lib.call("ucm_block_mean", 16, 1, 8, 16, 16, 1, 128, 3, 3, 16, 8, 0, 0, None)  # row of 9 columns
     assert e.value.code == _lib.ENOTSUP
+    with pytest.raises(_lib.UcmHipError) as e:  # more candidate scores than the built-in scratch holds
+        _lib.call("ucm_esa_retrieve_static", 16, 100, 1024, 16, 16, 65, 8192, 4, 16, 16, 16, 4, None)
+    assert e.value.code == _lib.ENOTSUP and "scratch" in str(e.value)
 
 
 def test_ops_need_device_tensors(ucm):

@@ -29,6 +29,7 @@ SIGNATURES = {
     "ucm_kvstar_topk": [_p, _p, _p, _p, _i, _i, _p, _i, _p, _p],
     "ucm_topk_windows": [_p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
     "ucm_esa_retrieve": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _p, _i, _p],
+    "ucm_esa_retrieve_static": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _i, _p],
     "ucm_delta_plan": [_p, _p, _p, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _p],
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],

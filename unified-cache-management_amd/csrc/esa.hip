@@ -16,6 +16,9 @@
 // ascending) by counting the keys above each, spread over workgroups.
 #include "common.h"
 
+#include <algorithm>
+#include <mutex>
+
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -181,28 +184,49 @@ __global__ __launch_bounds__(kRankThreads) void esa_rank_kernel(
 
 }  // namespace
 
-extern "C" int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
-                                const int32_t* indexes, int batch, int m, int topk, float* scores_ws,
-                                int32_t* out_idx, float* out_scores, int32_t* out_count, int out_stride,
-                                ucm_stream_t stream)
+// Scratch of ucm_esa_retrieve_static: the candidate scores of one call (what the scores_ws argument of
+// ucm_esa_retrieve brings in).  Every GPU holds its own copy of the array at its own address, until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kStaticScoreFloats = size_t{1} << 19;   // 2 MiB: e.g. 64 requests x 8192 candidates
+static __device__ __align__(256) float scratch[kStaticScoreFloats];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each GPU, looked up once per GPU
+
+// Device address of the current GPU's copy of `scratch` (first call on a GPU: one symbol lookup, no allocation).
+int static_scratch(float** out)
 {
-    UCM_REQUIRE(batch >= 0 && m >= 0, "ucm_esa_retrieve: batch=%d m=%d", batch, m);
-    if (batch == 0) { return UCM_OK; }
-    UCM_REQUIRE(data && q && out_idx && out_scores && out_count, "ucm_esa_retrieve: null pointer");
-    UCM_REQUIRE(m == 0 || (indexes && scores_ws), "ucm_esa_retrieve: null index row or workspace");
-    UCM_REQUIRE(n_items > 0 && dim > 0, "ucm_esa_retrieve: n_items=%d dim=%d", n_items, dim);
-    UCM_SUPPORTED(dim % 4 == 0, "ucm_esa_retrieve: dim=%d must be a multiple of 4", dim);
-    UCM_REQUIRE(ucm::aligned16(data) && ucm::aligned16(q), "ucm_esa_retrieve: data and q must be 16-byte aligned");
-    UCM_REQUIRE(batch <= 65535, "ucm_esa_retrieve: batch=%d", batch);
-    UCM_REQUIRE(out_stride >= std::min(std::max(topk, 0), m), "ucm_esa_retrieve: out_stride=%d too small", out_stride);
-    UCM_SUPPORTED(m <= 8192, "ucm_esa_retrieve: m=%d (at most 8192 candidates per request)", m);
+    int dev = -1;
+    if (int rc = ucm::check_hip(hipGetDevice(&dev), "ucm_esa_retrieve_static(hipGetDevice)")) { return rc; }
+    if (dev < 0 || dev >= kMaxDevices) { return ucm::fail(UCM_ENOTSUP, "ucm_esa_retrieve_static: device %d (at most %d)", dev, kMaxDevices); }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        if (int rc = ucm::check_hip(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)),
+                                    "ucm_esa_retrieve_static(hipGetSymbolAddress)")) {
+            return rc;
+        }
+        if (!ptr) { return ucm::fail(UCM_EHIP, "ucm_esa_retrieve_static: no device address for the scratch array"); }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return UCM_OK;
+}
+
+int esa_retrieve_impl(const char* name, const float* data, int n_items, int dim, const float* q, const int32_t* indexes,
+                      int batch, int m, int topk, float* scores_ws, int32_t* out_idx, float* out_scores,
+                      int32_t* out_count, int out_stride, ucm_stream_t stream)
+{
     const unsigned n_pad = (static_cast<unsigned>(m) + 127u) & ~127u;    // whole rounds of the counting loop
     hipStream_t s = ucm::as_stream(stream);
     if (m > 0) {
         hipLaunchKernelGGL(esa_score_kernel, dim3((m + kSlots - 1) / kSlots, batch), dim3(kScoreThreads), 0, s,
                            data, static_cast<unsigned>(n_items), static_cast<unsigned>(dim), q, indexes,
                            static_cast<unsigned>(m), scores_ws);
-        if (int rc = ucm::check_hip(hipGetLastError(), "ucm_esa_retrieve(score)")) { return rc; }
+        if (int rc = ucm::check_hip(hipGetLastError(), name)) { return rc; }
     }
     if (m <= 1024) {
         hipLaunchKernelGGL(esa_rank_kernel<1>, dim3((m + kRankThreads - 1) / kRankThreads + (m == 0), batch), dim3(kRankThreads),
@@ -214,5 +238,44 @@ extern "C" int ucm_esa_retrieve(const float* data, int n_items, int dim, const f
                            n_pad * sizeof(unsigned long long), s, scores_ws, indexes, static_cast<unsigned>(n_items),
                            static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride));
     }
-    UCM_LAUNCH_CHECK("ucm_esa_retrieve(select)");
+    return ucm::check_hip(hipGetLastError(), name);
+}
+
+}  // namespace
+
+#define UCM_ESA_CHECK_ARGS(name, ws_ok)                                                                              \
+    UCM_REQUIRE(batch >= 0 && m >= 0, name ": batch=%d m=%d", batch, m);                                             \
+    if (batch == 0) { return UCM_OK; }                                                                               \
+    UCM_REQUIRE(data && q && out_idx && out_scores && out_count, name ": null pointer");                             \
+    UCM_REQUIRE(m == 0 || (indexes && (ws_ok)), name ": null index row or workspace");                               \
+    UCM_REQUIRE(n_items > 0 && dim > 0, name ": n_items=%d dim=%d", n_items, dim);                                   \
+    UCM_SUPPORTED(dim % 4 == 0, name ": dim=%d must be a multiple of 4", dim);                                       \
+    UCM_REQUIRE(ucm::aligned16(data) && ucm::aligned16(q), name ": data and q must be 16-byte aligned");             \
+    UCM_REQUIRE(batch <= 65535, name ": batch=%d", batch);                                                           \
+    UCM_REQUIRE(out_stride >= std::min(std::max(topk, 0), m), name ": out_stride=%d too small", out_stride);         \
+    UCM_SUPPORTED(m <= 8192, name ": m=%d (at most 8192 candidates per request)", m)
+
+extern "C" int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
+                                const int32_t* indexes, int batch, int m, int topk, float* scores_ws,
+                                int32_t* out_idx, float* out_scores, int32_t* out_count, int out_stride,
+                                ucm_stream_t stream)
+{
+    UCM_ESA_CHECK_ARGS("ucm_esa_retrieve", scores_ws != nullptr);
+    return esa_retrieve_impl("ucm_esa_retrieve", data, n_items, dim, q, indexes, batch, m, topk, scores_ws, out_idx,
+                             out_scores, out_count, out_stride, stream);
+}
+
+extern "C" int ucm_esa_retrieve_static(const float* data, int n_items, int dim, const float* q,
+                                       const int32_t* indexes, int batch, int m, int topk, int32_t* out_idx,
+                                       float* out_scores, int32_t* out_count, int out_stride, ucm_stream_t stream)
+{
+    UCM_ESA_CHECK_ARGS("ucm_esa_retrieve_static", true);
+    UCM_SUPPORTED(static_cast<size_t>(batch) * static_cast<size_t>(m) <= kStaticScoreFloats,
+                  "ucm_esa_retrieve_static: batch*m = %zu candidate scores exceed the built-in scratch of %zu "
+                  "(use ucm_esa_retrieve with a workspace of its own)",
+                  static_cast<size_t>(batch) * static_cast<size_t>(m), kStaticScoreFloats);
+    float* ws = nullptr;
+    if (int rc = static_scratch(&ws)) { return rc; }
+    return esa_retrieve_impl("ucm_esa_retrieve_static", data, n_items, dim, q, indexes, batch, m, topk, ws, out_idx,
+                             out_scores, out_count, out_stride, stream);
 }
