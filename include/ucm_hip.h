@@ -188,6 +188,35 @@ int ucm_esa_retrieve(const float* data, int n_items, int dim, const float* q,
                      ucm_stream_t stream);
 
 /*
+ * ucm_esa_retrieve over a persistent table of requests: the plugin keeps one
+ * row per live request (its slot list, ReqStatePerLayer.slots,
+ * ucm/sparse/esa/esa.py:170-175,358-362) in device memory and each call
+ * covers the requests that retrieve in this step
+ * (ReqStatePerLayer.start_retrieval, esa.py:286-301, for all of a layer's
+ * requests at once instead of one submit per request).
+ *   slot_table  dev int32 [table_rows][table_stride], -1 padded: row i = slot
+ *               list of the request that owns row i; only its first m entries
+ *               are looked at (m = the longest list among this call's
+ *               requests, so short batches do not pay for the table's width)
+ *   rows        dev int32 [batch]: table row of request b of this call (q is
+ *               [batch][dim], scores_ws [batch][m]); a row outside the table
+ *               makes that request a no-op
+ *   topk_rows   dev int32 [table_rows]: each request's own k (at most max_topk)
+ *   out_idx / out_pos / out_scores  dev [table_rows][out_stride], out_count dev
+ *               int32 [table_rows]: results of request b go to row rows[b], so
+ *               they stay with the request until a later step consumes them.
+ *               out_pos (may be NULL) is the winner's position in its slot
+ *               list, i.e. the block's index relative to the request
+ *               (slots_to_relative_indexes, esa.py:358-361) - what
+ *               ucm_delta_plan_rows takes as `sel`.
+ */
+int ucm_esa_retrieve_rows(const float* data, int n_items, int dim, const float* q,
+                          const int32_t* slot_table, int table_rows, int table_stride, int m,
+                          const int32_t* rows, int batch, const int32_t* topk_rows, int max_topk,
+                          float* scores_ws, int32_t* out_idx, int32_t* out_pos, float* out_scores,
+                          int32_t* out_count, int out_stride, ucm_stream_t stream);
+
+/*
  * ucm_esa_retrieve for callers that cannot allocate (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc): it has no
  * counterpart in the reference.  Same arguments and results as
@@ -234,6 +263,18 @@ int ucm_esa_retrieve_static(const float* data, int n_items, int dim, const float
 int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req,
                    int n_layers, int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys,
                    int32_t* slot_of_sel, int32_t* miss_count, ucm_stream_t stream);
+
+/*
+ * ucm_delta_plan over a persistent table of requests: every array is laid out
+ * [n_layers][table_rows][...] and request b of the call uses row rows[b] (dev
+ * int32 [batch]); rows outside the table are skipped.  With sel_phys == sel
+ * the plan's load_phys holds the logical block each slot is to receive, which
+ * is what ucm_kv_load_planned reads.
+ */
+int ucm_delta_plan_rows(const int32_t* sel, const int32_t* sel_phys, const int32_t* count,
+                        const int32_t* rows, int batch, int table_rows, int n_layers, int sel_stride,
+                        int32_t* resident, int n_slots, int32_t* load_phys, int32_t* slot_of_sel,
+                        int32_t* miss_count, ucm_stream_t stream);
 
 /*
  * Hash-code retrieval (KvComp).  A vector's code has bit c = (x . W[:, c] > 0),
@@ -496,6 +537,34 @@ int ucm_kv_gather_selected(const void* const* layers, int n_layers, size_t kv_st
                            const int32_t* count, int n_req, int phys_stride, const int64_t* dst_off,
                            const int32_t* region_k, int max_count, void* staging,
                            int64_t staging_blocks, ucm_stream_t stream);
+
+/*
+ * The "load" of ReqStatePerLayer.wait_retrieval_and_start_load
+ * (ucm/sparse/esa/esa.py:312-339 -> launch_transfer_task :222-263 ->
+ * store.load(block_hashes, offsets, [k_cache[id] ...])) when the store's blocks
+ * are device-addressable, driven by ucm_delta_plan_rows' output with no host
+ * round trip: for every (layer l, request row, slot j) with
+ * sel = load_sel[l][row][j] >= 0, the K and V slices of stored block
+ * src_table[row][sel] are copied into cache block dst_table[row][j] of layer l.
+ *   layers      dev array of n_layers cache pointers (as for the other KV moves)
+ *   pool        dev: stored blocks of pool_block_bytes each, slice (layer, K|V)
+ *               of a block at ((store_first_layer + l)*2 + kv)*block_bytes -
+ *               the get_offset layout (esa.py:124-135, tp_size 1);
+ *               store_first_layer is the model layer layers[0] belongs to
+ *   load_sel    dev int32 [n_layers][table_rows][n_slots] (load_phys of the plan)
+ *   src_table   dev int32 [table_rows][src_stride]: pool block holding logical
+ *               block i of the request, -1 = not stored (skipped)
+ *   dst_table   dev int32 [table_rows][dst_stride]: cache block id of slot j
+ *               (the request's first top_k vLLM blocks, esa.py:311)
+ *   rows        dev int32 [batch] or NULL (then request b uses row b)
+ * Ids outside the pool or the cache are skipped, never dereferenced.
+ */
+int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                        int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
+                        int store_first_layer, const int32_t* load_sel, int n_slots,
+                        const int32_t* src_table, int src_stride, const int32_t* dst_table,
+                        int dst_stride, const int32_t* rows, int batch, int table_rows,
+                        ucm_stream_t stream);
 
 #ifdef __cplusplus
 }

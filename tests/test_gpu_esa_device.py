@@ -1,0 +1,195 @@
+"""The ESA plugin's batched device path (retrieve -> delta plan -> planned loads, no host round trip) driven the way
+patched vLLM drives the hooks: 16 requests at different stages of their decode in every engine step, 32 layers.
+After every step the request's first top_k cache blocks must hold, K and V, exactly the blocks the oracle selects
+(orc_esa_retrieve) and places (orc_delta_plan) from the same queries.  Host time of the hooks is printed per kind
+of step."""
+import time
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+import synth
+
+pytestmark = pytest.mark.gpu
+
+bits = lambda a: np.ascontiguousarray(a, np.float32).view(np.uint32)
+ns = types.SimpleNamespace
+
+
+class _ModelConfig:
+    def __init__(self, hq, hkv, d, layers, max_model_len):
+        self.hq, self.hkv, self.d, self.layers, self.max_model_len = hq, hkv, d, layers, max_model_len
+
+    def get_num_kv_heads(self, pc):
+        return self.hkv
+
+    def get_head_size(self):
+        return self.d
+
+    def get_num_layers(self, pc):
+        return self.layers
+
+
+def _config(hq, hkv, d, layers, bs, max_model_len, max_num_seqs, esa_cfg):
+    return ns(model_config=_ModelConfig(hq, hkv, d, layers, max_model_len), parallel_config=ns(rank=0, tensor_parallel_size=1),
+              cache_config=ns(block_size=bs), scheduler_config=ns(max_num_seqs=max_num_seqs),
+              kv_transfer_config=ns(kv_connector_extra_config={"ucm_sparse_config": {"ESA": esa_cfg}}))
+
+
+@pytest.mark.parametrize("pool_where", ["cuda", "pinned"])
+def test_esa_device_path_flow(ucm, dev, pool_where):
+    from ucm_amd import ops
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.esa.esa import ESA
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+
+    hq, hkv, d, L, bs = 8, 2, 64, 32, 16
+    n_req = 16 if pool_where == "cuda" else 5
+    nb = 2048
+    stride_cfg = 5
+    max_blocks = 128 if pool_where == "cuda" else 400        # 38 sparse slots at most (one wave plans them) / 120 (a workgroup)
+    cfg = _config(hq, hkv, d, L, bs, max_blocks * bs, 24, {"init_window_sz": 1, "local_window_sz": 2, "min_blocks": 4,
+                                                     "sparse_ratio": 0.3, "retrieval_stride": stride_cfg})
+    slice_bytes = bs * hkv * d * 2
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 1800 * L * 2 * slice_bytes,
+                              "device": pool_where})
+    plugin = ESA(cfg, UcmSparseRole.WORKER, store=store)
+    g = torch.Generator(device=dev)
+    g.manual_seed(5)
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    original = [c.clone() for c in caches]
+    all_layers = ops.LayerPointers(caches)
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
+
+    # requests: different prompt lengths, each starting its prefill at a different engine step
+    perm = synth.permutation(77, nb)
+    reqs, used = {}, 0
+    for i in range(n_req):
+        n_blocks = int(synth.ints(300 + i, 1, 12, 100)[0])
+        n_prompt = n_blocks * bs + (0 if i % 3 == 0 else int(synth.ints(400 + i, 1, 1, bs - 1)[0]))
+        total = n_blocks + 3
+        ids = [int(x) for x in perm[used : used + total]]
+        used += total
+        prompt = [int(x) for x in synth.ints(500 + i, n_prompt, 0, 30000)]
+        reqs[f"r{i}"] = ns(request_id=f"r{i}", block_ids=[ids], num_computed_tokens=0, prompt_token_ids=prompt,
+                           output_token_ids=[], num_prompt_tokens=n_prompt, start=i % 4, index=i)
+    assert used <= nb
+
+    # host model of every (request, layer)
+    model = {}
+    host_ms = {"prefill": [], "first": [], "retrieve": [], "load": [], "idle": []}
+
+    def engine_step(t):
+        active = [r for r in reqs.values() if r.start <= t]
+        sched, qsl, pos = {}, [], 0
+        for r in active:
+            n_tok = r.num_prompt_tokens if r.num_computed_tokens == 0 else 1
+            sched[r.request_id] = n_tok
+            qsl.append(pos)
+            pos += n_tok
+        ib = ns(req_id_to_index={r.request_id: j for j, r in enumerate(active)})
+        md = ns(query_start_loc=torch.tensor(qsl + [pos]))
+        so = ns(num_scheduled_tokens=sched)
+        qs = [torch.randn(pos, hq, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        plugin.build_sparse_meta(so, {r.request_id: r for r in active}, ib, md)
+        for l in range(L):
+            plugin.attention_begin(qs[l], None, None, names[l], fc)
+            plugin.attention_finished(qs[l], None, None, None, names[l], fc)
+        host = (time.perf_counter() - t0) * 1e3
+        torch.cuda.synchronize()
+        p = plugin._dev.plan
+        kind = ("prefill" if p.prefill is not None else "first" if p.n_first else "load" if p.n_load else
+                "retrieve" if p.n_retrieve else "idle")
+        host_ms[kind].append(host)
+        return active, qsl, qs
+
+    def expected_selection(m, l, q_tok):
+        qm = q_tok.view(hkv, hq // hkv, d).mean(1).float().reshape(-1).cpu().numpy()      # the plugin's mean is taken in bf16
+        idx, _ = O.esa_retrieve(m["rep"][l], qm, np.array(m["slots"][l], np.int32), m["top_k"])
+        pos_of = {s: i for i, s in enumerate(m["slots"][l])}
+        return np.array([pos_of[int(s)] for s in idx], np.int32)
+
+    def check_caches(r, m):
+        ids = r.block_ids[0]
+        dst = torch.tensor(ids[: m["top_k"]], device=dev)
+        for l in range(L):
+            res = m["resident"][l]
+            held = res >= 0
+            if not held.any():
+                continue
+            src = torch.tensor([ids[b] for b in res[held]], device=dev)
+            got = caches[l].index_select(1, dst[torch.from_numpy(held).to(dev)])
+            assert torch.equal(got, original[l].index_select(1, src)), (r.request_id, l)
+
+    n_steps = 14
+    for t in range(n_steps):
+        active, qsl, qs = engine_step(t)
+        for j, r in enumerate(active):
+            rid = r.request_id
+            if r.num_computed_tokens == 0:
+                # ---- the prefill step just ran: the plugin wrote the representatives
+                st = plugin._dev.reqs[rid]
+                n_full = r.num_prompt_tokens // bs
+                sparse_range = n_full - (2 if r.num_prompt_tokens % bs == 0 else 1)
+                top_k = int(sparse_range * 0.3)
+                assert (st.sparse_range, st.top_k, st.n_repre) == (sparse_range, top_k, sparse_range)
+                m = dict(top_k=top_k, slots=[list(s) for s in st.slots], rep=[], sel=[None] * L,
+                         resident=[np.full(top_k, -1, np.int32) for _ in range(L)])
+                ids = r.block_ids[0]
+                for l in range(L):
+                    kc = original[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+                    want = np.zeros((plugin.num_slots, hkv * d), np.float32)
+                    O.block_mean_paged(kc, ids[:sparse_range], m["slots"][l], want, round_bf16=True)
+                    got = plugin.data[l][m["slots"][l]].cpu().numpy()
+                    assert np.array_equal(bits(got), bits(want[m["slots"][l]])), (rid, l)
+                    m["rep"].append(want)
+                model[rid] = m
+                # what the prefix-cache connector does after prefill: every full prompt block goes to the store
+                hashes = st.block_hashes
+                assert len(hashes) == n_full
+                assert store.create(hashes) == [0] * n_full
+                slots = [store.slot_of[h] for h in hashes]
+                assert slots == list(range(slots[0], slots[0] + n_full))
+                pool, kvb = store.device_pool()
+                ops.kv_gather_blocks(all_layers, caches[0].stride(0) * 2, slice_bytes, nb,
+                                     torch.tensor(ids[:n_full], dtype=torch.int32, device=dev), pool[slots[0] * kvb :])
+                store.commit(hashes)
+                torch.cuda.synchronize()
+                r.num_computed_tokens = r.num_prompt_tokens
+                r.output_token_ids.append(1)
+                continue
+            m, step = model[rid], len(r.output_token_ids)
+            if m["top_k"] > 0:
+                retrieve_now = step == 1 or step % stride_cfg == 2 % stride_cfg
+                load_now = step == 1 or (step % stride_cfg == 0 and m["sel"][0] is not None)
+                for l in range(L):
+                    if retrieve_now:
+                        m["sel"][l] = expected_selection(m, l, qs[l][qsl[j]])
+                    if load_now:
+                        O.delta_plan(m["sel"][l], m["sel"][l], m["resident"][l])
+                if load_now:
+                    for l in range(L):
+                        assert sorted(m["resident"][l].tolist()) == sorted(m["sel"][l].tolist())
+                    m["sel"] = [None] * L
+                check_caches(r, m)
+            r.num_computed_tokens += 1
+            r.output_token_ids.append(1)
+    # every kind of step was seen; everything outside the requests' sparse slots is untouched
+    assert all(host_ms[k] for k in ("prefill", "first", "retrieve", "load"))
+    touched = torch.zeros(nb, dtype=torch.bool, device=dev)
+    for rid, m in model.items():
+        touched[torch.tensor(reqs[rid].block_ids[0][: m["top_k"]], dtype=torch.long, device=dev)] = True
+    for l in range(L):
+        assert torch.equal(caches[l][:, ~touched], original[l][:, ~touched])
+    print("\nESA device path, %d requests x %d layers, host ms per engine step (hooks only): " % (n_req, L) +
+          ", ".join(f"{k} {np.median(v):.2f} (n={len(v)})" for k, v in host_ms.items() if v))
+    for rid in list(reqs):
+        plugin.request_finished_in_worker(rid)
+    assert not plugin._dev.reqs and len(plugin.layer_pools[0].allocated) == 0
+    assert len(plugin._dev.tables.free_rows) == 24

@@ -396,7 +396,8 @@ def test_esa_plugin_flow(ucm, dev):
     hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 64
     cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
     cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"ESA": {
-        "init_window_sz": 1, "local_window_sz": 2, "min_blocks": 4, "sparse_ratio": 0.3, "retrieval_stride": 5}}}
+        "init_window_sz": 1, "local_window_sz": 2, "min_blocks": 4, "sparse_ratio": 0.3, "retrieval_stride": 5,
+        "device_loads": False}}}                             # the per-request path through store.load (any store)
     slice_bytes = bs * hkv * d * 2
     store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 40 * L * 2 * slice_bytes})
     plugin = ESA(cfg, UcmSparseRole.WORKER, store=store)

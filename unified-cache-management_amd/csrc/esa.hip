@@ -31,22 +31,40 @@ constexpr int kRowsPerLoad = kScoreThreads / (kCols / 4);  // 8 rows per 16-byte
 constexpr int kLoads = kSlots / kRowsPerLoad;              // 8 loads per thread per tile
 constexpr int kDepth = 2;                                  // tiles in flight per thread (an even number: two LDS buffers)
 
+// Row of the index matrix (and of every per-request output) that request b uses: b itself, or rows[b] when the
+// caller keeps a persistent table of requests and a call covers some of them.  A row outside the table makes
+// the whole request a no-op.
+__device__ __forceinline__ bool request_row(const int32_t* __restrict__ rows, unsigned n_rows, unsigned b, unsigned& row)
+{
+    if (!rows) { row = b; return true; }
+    const int32_t r = rows[b];
+    row = static_cast<unsigned>(r);
+    return r >= 0 && row < n_rows;
+}
+
 // grid: x = group of 64 entries of the index row, y = request
 __global__ __launch_bounds__(kScoreThreads) void esa_score_kernel(
     const float* __restrict__ data, unsigned n_items, unsigned dim, const float* __restrict__ q,
-    const int32_t* __restrict__ indexes, unsigned m, float* __restrict__ scores)
+    const int32_t* __restrict__ indexes, unsigned m, float* __restrict__ scores,
+    const int32_t* __restrict__ rows, unsigned n_rows, unsigned idx_stride)
 {
     __shared__ float tile[2][kCols * kColStride];       // products, [column][slot]
     __shared__ int32_t slot_of[kSlots];
 
     const unsigned b = blockIdx.y, first = blockIdx.x * kSlots;
-    const int32_t* idx_row = indexes + static_cast<size_t>(b) * m;
+    unsigned row;
+    if (!request_row(rows, n_rows, b, row)) { return; }   // (uniform)
+    const int32_t* idx_row = indexes + static_cast<size_t>(row) * idx_stride;
+    int32_t my_slot = -1;
     if (threadIdx.x < kSlots) {
         const unsigned e = first + threadIdx.x;
         const int32_t s = e < m ? idx_row[e] : -1;
-        slot_of[threadIdx.x] = (s >= 0 && static_cast<unsigned>(s) < n_items) ? s : -1;
+        my_slot = (s >= 0 && static_cast<unsigned>(s) < n_items) ? s : -1;
+        slot_of[threadIdx.x] = my_slot;
     }
-    __syncthreads();
+    // a group of padding only (short requests in a wide table) has nothing to score: the selection ignores the
+    // scores of entries without a slot
+    if (!__syncthreads_or(my_slot >= 0)) { return; }
 
     // this thread's part of a tile: column group c4 (4 floats) of rows r0, r0+8, ...
     const unsigned c4 = threadIdx.x % (kCols / 4), r0 = threadIdx.x / (kCols / 4);
@@ -127,13 +145,17 @@ template <int kLanes>
 __global__ __launch_bounds__(kRankThreads) void esa_rank_kernel(
     const float* __restrict__ scores, const int32_t* __restrict__ indexes, unsigned n_items, unsigned m,
     unsigned n_pad, int topk, int32_t* __restrict__ out_idx, float* __restrict__ out_scores,
-    int32_t* __restrict__ out_count, unsigned out_stride)
+    int32_t* __restrict__ out_count, unsigned out_stride, const int32_t* __restrict__ rows, unsigned n_rows,
+    const int32_t* __restrict__ topk_rows, int32_t* __restrict__ out_pos, unsigned idx_stride)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned long long keys[];
     __shared__ unsigned valid_total;
     const unsigned b = blockIdx.y;
+    unsigned row;
+    if (!request_row(rows, n_rows, b, row)) { return; }   // (uniform)
+    if (topk_rows) { topk = min(topk, topk_rows[row]); }  // the request's own k, never beyond a row of the outputs
     const float* s_row = scores + static_cast<size_t>(b) * m;
-    const int32_t* idx_row = indexes + static_cast<size_t>(b) * m;
+    const int32_t* idx_row = indexes + static_cast<size_t>(row) * idx_stride;
     if (threadIdx.x == 0) { valid_total = 0; }
     __syncthreads();
     unsigned mine = 0;
@@ -159,7 +181,7 @@ __global__ __launch_bounds__(kRankThreads) void esa_rank_kernel(
     }
     if (blockIdx.x == 0) { atomicAdd(&valid_total, mine); }
     __syncthreads();
-    if (blockIdx.x == 0 && threadIdx.x == 0) { out_count[b] = max(0, min(static_cast<int>(valid_total), topk)); }
+    if (blockIdx.x == 0 && threadIdx.x == 0) { out_count[row] = max(0, min(static_cast<int>(valid_total), topk)); }
 
     const unsigned cand = blockIdx.x * (kRankThreads / kLanes) + threadIdx.x / kLanes, sub = threadIdx.x % kLanes;
     const unsigned long long my = cand < m ? keys[cand] : 0ull;
@@ -177,8 +199,9 @@ __global__ __launch_bounds__(kRankThreads) void esa_rank_kernel(
 #pragma unroll
     for (int d = 1; d < kLanes; d <<= 1) { above += __shfl_xor(above, d, 64); }
     if (sub == 0 && my != 0ull && static_cast<int>(above) < topk) {      // (a valid key is never zero)
-        out_idx[static_cast<size_t>(b) * out_stride + above] = idx_row[cand];
-        out_scores[static_cast<size_t>(b) * out_stride + above] = s_row[cand];
+        out_idx[static_cast<size_t>(row) * out_stride + above] = idx_row[cand];
+        out_scores[static_cast<size_t>(row) * out_stride + above] = s_row[cand];
+        if (out_pos) { out_pos[static_cast<size_t>(row) * out_stride + above] = static_cast<int32_t>(cand); }
     }
 }
 
@@ -218,25 +241,29 @@ int static_scratch(float** out)
 
 int esa_retrieve_impl(const char* name, const float* data, int n_items, int dim, const float* q, const int32_t* indexes,
                       int batch, int m, int topk, float* scores_ws, int32_t* out_idx, float* out_scores,
-                      int32_t* out_count, int out_stride, ucm_stream_t stream)
+                      int32_t* out_count, int out_stride, ucm_stream_t stream, const int32_t* rows = nullptr,
+                      int n_rows = 0, const int32_t* topk_rows = nullptr, int32_t* out_pos = nullptr, int idx_stride = -1)
 {
+    const unsigned stride = static_cast<unsigned>(idx_stride < 0 ? m : idx_stride);   // row pitch of the index matrix
     const unsigned n_pad = (static_cast<unsigned>(m) + 127u) & ~127u;    // whole rounds of the counting loop
     hipStream_t s = ucm::as_stream(stream);
     if (m > 0) {
         hipLaunchKernelGGL(esa_score_kernel, dim3((m + kSlots - 1) / kSlots, batch), dim3(kScoreThreads), 0, s,
                            data, static_cast<unsigned>(n_items), static_cast<unsigned>(dim), q, indexes,
-                           static_cast<unsigned>(m), scores_ws);
+                           static_cast<unsigned>(m), scores_ws, rows, static_cast<unsigned>(n_rows), stride);
         if (int rc = ucm::check_hip(hipGetLastError(), name)) { return rc; }
     }
     if (m <= 1024) {
         hipLaunchKernelGGL(esa_rank_kernel<1>, dim3((m + kRankThreads - 1) / kRankThreads + (m == 0), batch), dim3(kRankThreads),
                            n_pad * sizeof(unsigned long long), s, scores_ws, indexes, static_cast<unsigned>(n_items),
-                           static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride));
+                           static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride),
+                           rows, static_cast<unsigned>(n_rows), topk_rows, out_pos, stride);
     } else {
         constexpr int kPer = kRankThreads / 8;
         hipLaunchKernelGGL(esa_rank_kernel<8>, dim3((m + kPer - 1) / kPer, batch), dim3(kRankThreads),
                            n_pad * sizeof(unsigned long long), s, scores_ws, indexes, static_cast<unsigned>(n_items),
-                           static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride));
+                           static_cast<unsigned>(m), n_pad, topk, out_idx, out_scores, out_count, static_cast<unsigned>(out_stride),
+                           rows, static_cast<unsigned>(n_rows), topk_rows, out_pos, stride);
     }
     return ucm::check_hip(hipGetLastError(), name);
 }
@@ -278,4 +305,20 @@ extern "C" int ucm_esa_retrieve_static(const float* data, int n_items, int dim, 
     if (int rc = static_scratch(&ws)) { return rc; }
     return esa_retrieve_impl("ucm_esa_retrieve_static", data, n_items, dim, q, indexes, batch, m, topk, ws, out_idx,
                              out_scores, out_count, out_stride, stream);
+}
+
+extern "C" int ucm_esa_retrieve_rows(const float* data, int n_items, int dim, const float* q,
+                                     const int32_t* slot_table, int table_rows, int table_stride, int m,
+                                     const int32_t* rows, int batch, const int32_t* topk_rows, int max_topk,
+                                     float* scores_ws, int32_t* out_idx, int32_t* out_pos, float* out_scores,
+                                     int32_t* out_count, int out_stride, ucm_stream_t stream)
+{
+    const int topk = max_topk;
+    const int32_t* indexes = slot_table;
+    UCM_ESA_CHECK_ARGS("ucm_esa_retrieve_rows", scores_ws != nullptr);
+    UCM_REQUIRE(rows && topk_rows && table_rows > 0 && table_stride >= m,
+                "ucm_esa_retrieve_rows: rows, topk_rows, table_rows and table_stride >= m are required");
+    return esa_retrieve_impl("ucm_esa_retrieve_rows", data, n_items, dim, q, slot_table, batch, m, max_topk, scores_ws,
+                             out_idx, out_scores, out_count, out_stride, stream, rows, table_rows, topk_rows, out_pos,
+                             table_stride);
 }

@@ -96,6 +96,35 @@ __global__ __launch_bounds__(kThreads) void kv_gather_selected_kernel(
     copy_slice(staging + slot * block_bytes, src, block_bytes);
 }
 
+// Loads planned on the device: slot j of request row `row` receives logical block load_sel[l][row][j] (or
+// nothing, -1) from a pool of stored blocks laid out [block][layer][K|V].
+// grid: x = slot, y = request of the call, z = layer*2 + K|V
+__global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
+    void* const* __restrict__ layers, size_t kv_stride, size_t block_bytes, unsigned num_blocks,
+    const uint8_t* __restrict__ pool, uint64_t pool_blocks, size_t pool_block_bytes, unsigned store_first_layer,
+    const int32_t* __restrict__ load_sel, unsigned n_slots, const int32_t* __restrict__ src_table, unsigned src_stride,
+    const int32_t* __restrict__ dst_table, unsigned dst_stride, const int32_t* __restrict__ rows, unsigned table_rows)
+{
+    const unsigned j = blockIdx.x, b = blockIdx.y, l = blockIdx.z >> 1, kv = blockIdx.z & 1;
+    unsigned row = b;
+    if (rows) {
+        const int32_t r = rows[b];
+        if (r < 0) { return; }
+        row = static_cast<unsigned>(r);
+    }
+    if (row >= table_rows) { return; }
+    const int32_t sel = load_sel[(static_cast<size_t>(l) * table_rows + row) * n_slots + j];
+    if (sel < 0 || static_cast<unsigned>(sel) >= src_stride) { return; }     // slot keeps what it holds
+    const int32_t src = src_table[static_cast<size_t>(row) * src_stride + sel];
+    if (src < 0 || static_cast<uint64_t>(src) >= pool_blocks) { return; }   // block not in the pool
+    const unsigned dst = static_cast<unsigned>(dst_table[static_cast<size_t>(row) * dst_stride + j]);
+    if (dst >= num_blocks) { return; }
+    copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
+               pool + static_cast<size_t>(src) * pool_block_bytes +
+                   (static_cast<size_t>(store_first_layer + l) * 2 + kv) * block_bytes,
+               block_bytes);
+}
+
 constexpr size_t kBatchPiece = 2 * kStep;  // 256 KiB
 
 int check_block_args(const void* layers, int n_layers, size_t kv_stride, size_t block_bytes,
@@ -177,4 +206,36 @@ extern "C" int ucm_kv_gather_selected(const void* const* layers, int n_layers, s
                        count, static_cast<unsigned>(num_blocks), static_cast<unsigned>(n_req), static_cast<unsigned>(phys_stride), dst_off,
                        region_k, static_cast<uint8_t*>(staging), static_cast<uint64_t>(staging_blocks));
     UCM_LAUNCH_CHECK("ucm_kv_gather_selected");
+}
+
+extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                                   int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
+                                   int store_first_layer, const int32_t* load_sel, int n_slots,
+                                   const int32_t* src_table, int src_stride, const int32_t* dst_table,
+                                   int dst_stride, const int32_t* rows, int batch, int table_rows,
+                                   ucm_stream_t stream)
+{
+    UCM_REQUIRE(batch >= 0 && n_slots >= 0 && table_rows > 0, "ucm_kv_load_planned: batch=%d n_slots=%d table_rows=%d", batch,
+                n_slots, table_rows);
+    if (batch == 0 || n_slots == 0) { return UCM_OK; }
+    UCM_REQUIRE(layers && pool && load_sel && src_table && dst_table, "ucm_kv_load_planned: null pointer");
+    UCM_REQUIRE(n_layers > 0 && n_layers * 2 <= 65535 && batch <= 65535, "ucm_kv_load_planned: n_layers=%d batch=%d", n_layers, batch);
+    UCM_REQUIRE(num_blocks > 0 && static_cast<size_t>(num_blocks) * block_bytes <= kv_stride,
+                "ucm_kv_load_planned: num_blocks=%d does not fit kv_stride=%zu", num_blocks, kv_stride);
+    UCM_REQUIRE(block_bytes > 0 && block_bytes % 16 == 0 && kv_stride % 16 == 0 && pool_block_bytes % 16 == 0 &&
+                    ucm::aligned16(pool),
+                "ucm_kv_load_planned: sizes and pool must be multiples of 16");
+    UCM_REQUIRE(store_first_layer >= 0 && pool_blocks >= 0 &&
+                    static_cast<size_t>(store_first_layer + n_layers) * 2 * block_bytes <= pool_block_bytes,
+                "ucm_kv_load_planned: layers %d..%d do not fit a stored block of %zu bytes", store_first_layer,
+                store_first_layer + n_layers - 1, pool_block_bytes);
+    UCM_REQUIRE(src_stride >= 1 && dst_stride >= n_slots, "ucm_kv_load_planned: src_stride=%d dst_stride=%d n_slots=%d", src_stride,
+                dst_stride, n_slots);
+    hipLaunchKernelGGL(kv_load_planned_kernel, dim3(static_cast<unsigned>(n_slots), batch, n_layers * 2), dim3(kThreads), 0,
+                       ucm::as_stream(stream), layers, kv_stride, block_bytes, static_cast<unsigned>(num_blocks),
+                       static_cast<const uint8_t*>(pool), static_cast<uint64_t>(pool_blocks), pool_block_bytes,
+                       static_cast<unsigned>(store_first_layer), load_sel, static_cast<unsigned>(n_slots), src_table,
+                       static_cast<unsigned>(src_stride), dst_table, static_cast<unsigned>(dst_stride), rows,
+                       static_cast<unsigned>(table_rows));
+    UCM_LAUNCH_CHECK("ucm_kv_load_planned");
 }

@@ -248,9 +248,14 @@ namespace {
 __global__ __launch_bounds__(64) void delta_plan_kernel(
     const int32_t* __restrict__ sel, const int32_t* __restrict__ sel_phys, const int32_t* __restrict__ count,
     int n_req, int sel_stride, int32_t* __restrict__ resident, int n_slots, int32_t* __restrict__ load_phys,
-    int32_t* __restrict__ slot_of_sel, int32_t* __restrict__ miss_count)
+    int32_t* __restrict__ slot_of_sel, int32_t* __restrict__ miss_count, const int32_t* __restrict__ rows)
 {
-    const int r = blockIdx.x, l = blockIdx.y, lane = threadIdx.x;
+    const int l = blockIdx.y, lane = threadIdx.x;
+    int r = blockIdx.x;
+    if (rows) {   // a call over some rows of a persistent request table of n_req rows
+        r = rows[r];
+        if (r < 0 || r >= n_req) { return; }
+    }
     const size_t lr = static_cast<size_t>(l) * n_req + r;
     const int k = min(min(count[lr], n_slots), sel_stride);   // selections beyond the slot budget cannot be resident
     const int32_t* s = sel + lr * sel_stride;
@@ -307,11 +312,16 @@ template <int E>  // entries per thread: n_slots <= 256 * E
 __global__ __launch_bounds__(kPlanThreads) void delta_plan_wide_kernel(
     const int32_t* __restrict__ sel, const int32_t* __restrict__ sel_phys, const int32_t* __restrict__ count,
     int n_req, int sel_stride, int32_t* __restrict__ resident, int n_slots, int32_t* __restrict__ load_phys,
-    int32_t* __restrict__ slot_of_sel, int32_t* __restrict__ miss_count)
+    int32_t* __restrict__ slot_of_sel, int32_t* __restrict__ miss_count, const int32_t* __restrict__ rows)
 {
     constexpr int kCap = kPlanThreads * E;
-    const int r = blockIdx.x, l = blockIdx.y, tid = threadIdx.x;
+    const int l = blockIdx.y, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
+    int r = blockIdx.x;
+    if (rows) {
+        r = rows[r];
+        if (r < 0 || r >= n_req) { return; }
+    }
     const size_t lr = static_cast<size_t>(l) * n_req + r;
     const int k = min(min(count[lr], n_slots), sel_stride);   // (a count larger than a row of sel is never followed)
     const int32_t* s = sel + lr * sel_stride;
@@ -410,6 +420,30 @@ __global__ __launch_bounds__(kPlanThreads) void delta_plan_wide_kernel(
 
 }  // namespace
 
+namespace {
+
+int delta_plan_launch(const char* name, const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_rows,
+                      int n_launch, const int32_t* rows, int n_layers, int sel_stride, int32_t* resident, int n_slots,
+                      int32_t* load_phys, int32_t* slot_of_sel, int32_t* miss_count, ucm_stream_t stream)
+{
+    const dim3 grid(n_launch, n_layers);
+    hipStream_t s = ucm::as_stream(stream);
+#define UCM_PLAN_LAUNCH(E)                                                                                    \
+    hipLaunchKernelGGL(delta_plan_wide_kernel<E>, grid, dim3(kPlanThreads), 0, s, sel, sel_phys, count, n_rows, \
+                       sel_stride, resident, n_slots, load_phys, slot_of_sel, miss_count, rows)
+    if (n_slots <= 64) {
+        hipLaunchKernelGGL(delta_plan_kernel, grid, dim3(64), 0, s, sel, sel_phys, count, n_rows, sel_stride, resident,
+                           n_slots, load_phys, slot_of_sel, miss_count, rows);
+    }
+    else if (n_slots <= 256) { UCM_PLAN_LAUNCH(1); }
+    else if (n_slots <= 512) { UCM_PLAN_LAUNCH(2); }
+    else { UCM_PLAN_LAUNCH(4); }
+#undef UCM_PLAN_LAUNCH
+    return ucm::check_hip(hipGetLastError(), name);
+}
+
+}  // namespace
+
 extern "C" int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req,
                               int n_layers, int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys,
                               int32_t* slot_of_sel, int32_t* miss_count, ucm_stream_t stream)
@@ -419,18 +453,22 @@ extern "C" int ucm_delta_plan(const int32_t* sel, const int32_t* sel_phys, const
     UCM_REQUIRE(sel && sel_phys && count && resident && load_phys && slot_of_sel && miss_count, "ucm_delta_plan: null pointer");
     UCM_SUPPORTED(n_slots >= 1 && n_slots <= 1024, "ucm_delta_plan: n_slots=%d (1..1024 staging slots per request and layer)", n_slots);
     UCM_REQUIRE(sel_stride >= 1, "ucm_delta_plan: sel_stride=%d", sel_stride);
-    const dim3 grid(n_req, n_layers);
-    hipStream_t s = ucm::as_stream(stream);
-#define UCM_PLAN_LAUNCH(E)                                                                                  \
-    hipLaunchKernelGGL(delta_plan_wide_kernel<E>, grid, dim3(kPlanThreads), 0, s, sel, sel_phys, count, n_req, \
-                       sel_stride, resident, n_slots, load_phys, slot_of_sel, miss_count)
-    if (n_slots <= 64) {
-        hipLaunchKernelGGL(delta_plan_kernel, grid, dim3(64), 0, s, sel, sel_phys, count, n_req, sel_stride, resident,
-                           n_slots, load_phys, slot_of_sel, miss_count);
-    }
-    else if (n_slots <= 256) { UCM_PLAN_LAUNCH(1); }
-    else if (n_slots <= 512) { UCM_PLAN_LAUNCH(2); }
-    else { UCM_PLAN_LAUNCH(4); }
-#undef UCM_PLAN_LAUNCH
-    UCM_LAUNCH_CHECK("ucm_delta_plan");
+    return delta_plan_launch("ucm_delta_plan", sel, sel_phys, count, n_req, n_req, nullptr, n_layers, sel_stride, resident,
+                             n_slots, load_phys, slot_of_sel, miss_count, stream);
+}
+
+extern "C" int ucm_delta_plan_rows(const int32_t* sel, const int32_t* sel_phys, const int32_t* count,
+                                   const int32_t* rows, int batch, int table_rows, int n_layers, int sel_stride,
+                                   int32_t* resident, int n_slots, int32_t* load_phys, int32_t* slot_of_sel,
+                                   int32_t* miss_count, ucm_stream_t stream)
+{
+    UCM_REQUIRE(batch >= 0 && table_rows > 0 && n_layers > 0 && n_layers <= 65535,
+                "ucm_delta_plan_rows: batch=%d table_rows=%d n_layers=%d", batch, table_rows, n_layers);
+    if (batch == 0) { return UCM_OK; }
+    UCM_REQUIRE(sel && sel_phys && count && rows && resident && load_phys && slot_of_sel && miss_count,
+                "ucm_delta_plan_rows: null pointer");
+    UCM_SUPPORTED(n_slots >= 1 && n_slots <= 1024, "ucm_delta_plan_rows: n_slots=%d (1..1024 staging slots per request and layer)", n_slots);
+    UCM_REQUIRE(sel_stride >= 1, "ucm_delta_plan_rows: sel_stride=%d", sel_stride);
+    return delta_plan_launch("ucm_delta_plan_rows", sel, sel_phys, count, table_rows, batch, rows, n_layers, sel_stride,
+                             resident, n_slots, load_phys, slot_of_sel, miss_count, stream);
 }

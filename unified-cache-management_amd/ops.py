@@ -213,6 +213,69 @@ def delta_plan(sel: torch.Tensor, sel_phys: torch.Tensor, count: torch.Tensor, r
               _dev(slot_of_sel, torch.int32, "slot_of_sel"), _dev(miss_count, torch.int32, "miss_count"), _stream())
 
 
+def esa_retrieve_rows(data: torch.Tensor, q: torch.Tensor, slot_table: torch.Tensor, m: int, rows: torch.Tensor,
+                      topk_rows: torch.Tensor, max_topk: int, scores_ws: torch.Tensor, out_idx: torch.Tensor,
+                      out_pos: Optional[torch.Tensor], out_scores: torch.Tensor, out_count: torch.Tensor) -> None:
+    """data fp32 [N, dim]; q fp32 [B, dim]; slot_table int32 [table_rows, stride] (-1 padded), of which the first
+    ``m`` entries of a row are looked at; rows int32 [B]; topk_rows int32 [table_rows]; out_idx / out_pos /
+    out_scores [table_rows, out_stride]; out_count int32 [table_rows]."""
+    if data.dim() != 2 or q.dim() != 2 or slot_table.dim() != 2 or q.shape[1] != data.shape[1]:
+        raise ValueError("data [N,dim], q [B,dim], slot_table [rows,stride] expected")
+    batch, (table_rows, stride) = rows.numel(), slot_table.shape
+    if m > stride:
+        raise ValueError("m exceeds the table's row length")
+    if q.shape[0] != batch or scores_ws.numel() < batch * m:
+        raise ValueError("q / scores_ws do not cover the batch")
+    if out_idx.shape[0] != table_rows or out_scores.shape != out_idx.shape or out_count.numel() != table_rows \
+            or topk_rows.numel() != table_rows or (out_pos is not None and out_pos.shape != out_idx.shape):
+        raise ValueError("per-row outputs must have one row per table row")
+    _lib.call("ucm_esa_retrieve_rows", _dev(data, torch.float32, "data"), data.shape[0], data.shape[1],
+              _dev(q, torch.float32, "q"), _dev(slot_table, torch.int32, "slot_table"), table_rows, stride, int(m),
+              _dev(rows, torch.int32, "rows"), batch, _dev(topk_rows, torch.int32, "topk_rows"), int(max_topk),
+              _dev(scores_ws, torch.float32, "scores_ws"), _dev(out_idx, torch.int32, "out_idx"),
+              _opt(out_pos, torch.int32, "out_pos"), _dev(out_scores, torch.float32, "out_scores"),
+              _dev(out_count, torch.int32, "out_count"), out_idx.shape[1], _stream())
+
+
+def delta_plan_rows(sel: torch.Tensor, sel_phys: torch.Tensor, count: torch.Tensor, rows: torch.Tensor,
+                    resident: torch.Tensor, load_phys: torch.Tensor, slot_of_sel: torch.Tensor,
+                    miss_count: torch.Tensor) -> None:
+    """As delta_plan, every array [L, table_rows, ...]; only the rows listed in ``rows`` (int32 [B]) are planned."""
+    n_layers, table_rows, stride = sel.shape
+    if sel_phys.shape != sel.shape or slot_of_sel.shape != sel.shape or count.shape != (n_layers, table_rows) \
+            or miss_count.shape != count.shape or resident.shape[:2] != (n_layers, table_rows) \
+            or load_phys.shape != resident.shape:
+        raise ValueError("delta_plan_rows: inconsistent shapes")
+    _lib.call("ucm_delta_plan_rows", _dev(sel, torch.int32, "sel"), _dev(sel_phys, torch.int32, "sel_phys"),
+              _dev(count, torch.int32, "count"), _dev(rows, torch.int32, "rows"), rows.numel(), table_rows, n_layers,
+              stride, _dev(resident, torch.int32, "resident"), resident.shape[2],
+              _dev(load_phys, torch.int32, "load_phys"), _dev(slot_of_sel, torch.int32, "slot_of_sel"),
+              _dev(miss_count, torch.int32, "miss_count"), _stream())
+
+
+def kv_load_planned(layers: LayerPointers, ptr_first: int, store_first_layer: int, n_layers: int, kv_stride: int,
+                    block_bytes: int, num_blocks: int, pool: torch.Tensor, pool_block_bytes: int,
+                    load_sel: torch.Tensor, src_table: torch.Tensor, dst_table: torch.Tensor,
+                    rows: Optional[torch.Tensor]) -> None:
+    """pool: uint8 buffer of stored blocks ([block][layer][K|V], device or pinned host memory); load_sel int32
+    [n_layers, table_rows, n_slots]: the plan of model layers store_first_layer.., whose cache pointers are entries
+    ptr_first.. of ``layers``; src_table int32 [table_rows, M]; dst_table int32 [table_rows, >= n_slots]; rows int32
+    [B] or None (all table rows)."""
+    if load_sel.dim() != 3 or load_sel.shape[0] != n_layers:
+        raise ValueError("load_sel must be [n_layers, table_rows, n_slots]")
+    table_rows, n_slots = load_sel.shape[1], load_sel.shape[2]
+    if src_table.shape[0] != table_rows or dst_table.shape[0] != table_rows or dst_table.shape[1] < n_slots:
+        raise ValueError("src_table / dst_table must have one row per table row")
+    if ptr_first < 0 or ptr_first + n_layers > len(layers):
+        raise ValueError("layer range outside the pointer table")
+    nbytes = pool.numel() * pool.element_size()
+    _lib.call("ucm_kv_load_planned", layers.ptr(ptr_first), n_layers, kv_stride, block_bytes, num_blocks,
+              _staging_ptr(pool, 0), nbytes // pool_block_bytes, pool_block_bytes, store_first_layer,
+              _dev(load_sel, torch.int32, "load_sel"), n_slots, _dev(src_table, torch.int32, "src_table"),
+              src_table.shape[1], _dev(dst_table, torch.int32, "dst_table"), dst_table.shape[1],
+              _opt(rows, torch.int32, "rows"), table_rows if rows is None else rows.numel(), table_rows, _stream())
+
+
 HASH_SCORE_SUM, HASH_SCORE_BLOCK_CODE = 0, 1
 
 

@@ -35,6 +35,7 @@ import torch
 
 from ... import ops
 from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
+from .device_path import EsaDevicePath
 from .retrieval_worker import HipRetrievalBackend, RetrievalWorker
 
 ReqType = Union[str, int]
@@ -152,16 +153,8 @@ class ReqStatePerLayer:
 
     # ---- static data -----------------------------------------------------------
     def set_block_hashes(self, token_ids) -> None:
-        if self.block_hashes is not None:
-            return
-        self.block_hashes = []
-        parent = None
-        for start in range(0, len(token_ids), self.block_size):
-            chunk = token_ids[start : start + self.block_size]
-            if len(chunk) < self.block_size:
-                break
-            parent = block_hash_func(parent, tuple(chunk))
-            self.block_hashes.append(str(parent))
+        if self.block_hashes is None:
+            self.block_hashes = self.esa.prompt_block_hashes(token_ids)
 
     def update_meta(self, req_meta: ReqMeta) -> None:
         self.req_meta = req_meta
@@ -212,6 +205,7 @@ class ReqStatePerLayer:
         for i, slot in enumerate(new_slots):
             self.slots_to_relative_indexes[slot] = base + i
         self.slots.extend(new_slots)
+        self.slots_dev = torch.tensor([self.slots], dtype=torch.int32, device=self.k_cache.device)   # one index row
         self.esa.write_block_repre(self.layer_id, ids, new_slots)
 
     # ---- retrieval -----------------------------------------------------------------
@@ -226,8 +220,10 @@ class ReqStatePerLayer:
             query = query.view(ntokens, self.num_key_heads, -1, self.head_size).mean(2)
         elif num_q_heads < self.num_key_heads:
             query = torch.repeat_interleave(query, self.num_key_heads // num_q_heads, 1)
-        self.retrieval_task = self.retrieval_worker.submit(query.reshape(ntokens, -1), topk=self.top_k(),
-                                                           indexes=[self.slots] * ntokens)
+        # the reference submits every scheduled token's query with ONE index row (esa.py:297-301) and reads row 0
+        # of the result (:305); in decode there is one token
+        self.retrieval_task = self.retrieval_worker.submit(query.reshape(ntokens, -1)[:1], topk=self.top_k(),
+                                                           indexes=self.slots_dev)
 
     def wait_retrieval_and_start_load(self) -> None:
         self.retrieval_worker.wait(self.retrieval_task)
@@ -287,7 +283,9 @@ class ESA(UcmSparseBase):
         self.num_key_heads = mc.get_num_kv_heads(pc)
         self.head_size = mc.get_head_size()
         self.total_num_hidden_layers = mc.get_num_layers(pc)
-        self.num_slots = mc.max_model_len * vllm_config.scheduler_config.max_num_seqs // self.block_size
+        self.max_model_len = mc.max_model_len
+        self.max_num_seqs = vllm_config.scheduler_config.max_num_seqs
+        self.num_slots = self.max_model_len * self.max_num_seqs // self.block_size
         self.dim = self.num_key_heads * self.head_size
         self.connector = store  # anything with the UcmKVStoreBase load / dump / wait methods
         self.req_states: Dict[ReqType, List[Optional[ReqStatePerLayer]]] = {}
@@ -296,14 +294,32 @@ class ESA(UcmSparseBase):
         self.retrieval_workers: List[Optional[RetrievalWorker]] = [None] * self.total_num_hidden_layers
         self._layer_ptrs: Dict[int, ops.LayerPointers] = {}
         self._num_blocks: Dict[int, int] = {}
+        # "device_loads": the batched path that plans and loads on the device (needs a store whose blocks a
+        # kernel can read, i.e. one with device_pool()); False keeps the per-request host path for any store
+        self._device_loads = bool(self.esa_cfg.get("device_loads", True)) and hasattr(store, "device_pool")
+        self._dev: Optional[EsaDevicePath] = None
+
+    def prompt_block_hashes(self, token_ids) -> List[str]:
+        """Chained hashes of the prompt's full blocks (esa.py:205-219)."""
+        out, parent = [], None
+        for start in range(0, len(token_ids), self.block_size):
+            chunk = token_ids[start : start + self.block_size]
+            if len(chunk) < self.block_size:
+                break
+            parent = block_hash_func(parent, tuple(chunk))
+            out.append(str(parent))
+        return out
 
     # ---- device tables -----------------------------------------------------------------
-    def register_layer_cache(self, layer_id: int, k_cache: torch.Tensor) -> None:
+    def _allocate_tables(self, device) -> None:
         if self.data is None:
             self.data = torch.zeros((self.total_num_hidden_layers, self.num_slots, self.dim), dtype=torch.float32,
-                                    device=k_cache.device)
+                                    device=device)
             for l in range(self.total_num_hidden_layers):
                 self.retrieval_workers[l] = RetrievalWorker(HipRetrievalBackend(self.data[l]))
+
+    def register_layer_cache(self, layer_id: int, k_cache: torch.Tensor) -> None:
+        self._allocate_tables(k_cache.device)
         if layer_id not in self._layer_ptrs or self._layer_ptrs[layer_id].tensors[0].data_ptr() != k_cache.data_ptr():
             self._layer_ptrs[layer_id] = ops.LayerPointers([k_cache])
             self._num_blocks[layer_id] = k_cache.shape[0]
@@ -326,13 +342,29 @@ class ESA(UcmSparseBase):
             states[layer_id] = ReqStatePerLayer(req_meta, layer_name, self.rank, self.tp_size, self.connector, self)
         return states[layer_id]
 
+    def _device_layer(self, layer_name: str, forward_context) -> int:
+        layer_id = int(layer_name.split(".")[2])
+        if self._dev.kv_caches[layer_id] is None:
+            kv_cache = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
+            self.register_layer_cache(layer_id, kv_cache[0])
+            self._dev.register_kv_cache(layer_id, kv_cache)
+        return layer_id
+
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        if self._dev is not None:
+            if self._sparse_metadata.requests:
+                self._dev.attention_begin(self._device_layer(layer_name, forward_context), query)
+            return
         for req_meta in self._sparse_metadata.requests:
             st = self.create_layerwise_req_state(req_meta, layer_name, forward_context)
             st.update_meta(req_meta)
             st.attention_begin(query, key, value, forward_context)
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
+        if self._dev is not None:
+            if self._sparse_metadata.requests:
+                self._dev.attention_finished(self._device_layer(layer_name, forward_context), query)
+            return
         for req_meta in self._sparse_metadata.requests:
             st = self.create_layerwise_req_state(req_meta, layer_name, forward_context)
             st.update_meta(req_meta)
@@ -353,11 +385,22 @@ class ESA(UcmSparseBase):
             meta.add_request(req_id, idx, n_tok, req.num_computed_tokens, req.block_ids[0],
                              int(attn_metadata.query_start_loc[idx]), req.prompt_token_ids, req.output_token_ids)
         self._sparse_metadata = meta
+        if self._device_loads and meta.requests:
+            if self._dev is None:
+                dev = torch.device("cuda", torch.cuda.current_device())
+                pool, pool_block_bytes = self.connector.device_pool()
+                self._dev = EsaDevicePath(self, pool, pool_block_bytes, dev)
+                self._allocate_tables(dev)
+            self._dev.build_step(meta.requests)
 
     def request_finished_in_worker(self, request_id: ReqType) -> None:
+        if self._dev is not None:
+            self._dev.request_finished(request_id)
         for st in self.req_states.pop(request_id, []):
             if st is not None:
                 st.repre_pool.free(st.slots)
+                if st.retrieval_task is not None:     # a retrieval nobody will fetch: drop its device buffers
+                    st.retrieval_worker.cpp_worker.discard(st.retrieval_task)
 
     # ---- scheduler side -------------------------------------------------------------------------
     def request_begin(self, request_id: ReqType, prompt_token_ids: List[int]) -> None:

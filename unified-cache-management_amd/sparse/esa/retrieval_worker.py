@@ -63,9 +63,9 @@ class HipRetrievalBackend:
             idx_dev = idx.to(device=dev, dtype=torch.int32, non_blocking=True).contiguous()
             stride = max(min(int(topk), m), 1)
             ws = torch.empty((batch, max(m, 1)), dtype=torch.float32, device=dev)
-            out_idx = torch.full((batch, stride), -1, dtype=torch.int32, device=dev)
-            out_scores = torch.zeros((batch, stride), dtype=torch.float32, device=dev)
-            out_count = torch.zeros((batch,), dtype=torch.int32, device=dev)
+            # indices, score bits and counts share one buffer so that get_result is a single copy to the host
+            pack = torch.zeros((3, batch, stride), dtype=torch.int32, device=dev)
+            out_idx, out_scores, out_count = pack[0], pack[1].view(torch.float32), pack[2].view(-1)[:batch]
             ops.esa_retrieve(self.data, q_dev, idx_dev, int(topk), ws, out_idx, out_scores, out_count,
                              stream=self._stream.cuda_stream)
             done = torch.cuda.Event()
@@ -74,8 +74,7 @@ class HipRetrievalBackend:
             req_id = self._next_req_id
             self._next_req_id += 1
             self._known.add(req_id)
-            self._pending[req_id] = dict(done=done, out_idx=out_idx, out_scores=out_scores, out_count=out_count,
-                                         keep=(q_dev, idx_dev, ws), topk=int(topk))
+            self._pending[req_id] = dict(done=done, pack=pack, keep=(q_dev, idx_dev, ws), topk=int(topk))
         return req_id
 
     def poll(self, req_id: int) -> bool:
@@ -97,11 +96,17 @@ class HipRetrievalBackend:
             if p is None or not p["done"].query():
                 raise RuntimeError("Result not ready")
             del self._pending[req_id]  # a result can be fetched once, like the reference's erase
-        counts = p["out_count"].cpu().numpy()
-        k = int(counts[0]) if len(counts) else 0  # the reference sizes the arrays by request 0's result
-        idx = p["out_idx"][:, :k].cpu().numpy().astype(np.int32, copy=False)
-        scores = p["out_scores"][:, :k].cpu().numpy().astype(np.float32, copy=False)
-        return {"indices": idx, "scores": scores}
+        host = p["pack"].cpu().numpy()                 # [3, batch, stride]: one copy, one wait
+        batch = host.shape[1]
+        counts = host[2].reshape(-1)[:batch]
+        k = int(counts[0]) if batch else 0  # the reference sizes the arrays by request 0's result
+        return {"indices": np.ascontiguousarray(host[0][:, :k]), "scores": np.ascontiguousarray(host[1][:, :k]).view(np.float32)}
+
+    def discard(self, req_id: int) -> None:
+        """Forgets a submitted request whose result will not be fetched (its owner finished) and releases its
+        device buffers; the reference keeps such results until the process ends."""
+        with self._lock:
+            self._pending.pop(req_id, None)
 
 
 def _pad_rows(indexes) -> np.ndarray:

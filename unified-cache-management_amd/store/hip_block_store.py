@@ -69,6 +69,12 @@ class UcmHipBlockStore:
     def cc_store(self) -> int:
         return 0
 
+    def device_pool(self) -> Tuple[torch.Tensor, int]:
+        """The buffer holding every stored block (slot i at byte i*kv_block_size) and the size of a stored block:
+        what a kernel needs to read blocks in place (``slot_of`` maps a block hash to its slot).  Plugins that find
+        this method plan and run their loads on the device instead of calling ``load`` block by block."""
+        return self._ensure_buffer(), self.kv_block_size
+
     def create(self, block_ids: List[str]) -> List[int]:
         """Reserves a slot per block hash; FAILURE for those that do not fit."""
         out = []
