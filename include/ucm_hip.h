@@ -277,6 +277,49 @@ int ucm_delta_plan_rows(const int32_t* sel, const int32_t* sel_phys, const int32
                         int32_t* miss_count, ucm_stream_t stream);
 
 /*
+ * The bookkeeping of the GSA prefetch engine for a batch of requests, all
+ * layers in one launch - GSAPrefetchEngineC::RunOneBsPrefetch with
+ * GetHitAndMissBlock, RunPrefetchH2D and LoadKVToHBM
+ * (ucm/sparse/gsa/prefetch/src/kvcache_pre.cpp:206-322).  Per (request, layer):
+ * selected logical blocks that a resident cache block holds are hits, the
+ * others misses (in selection order); the free list is walked in order, entries
+ * whose block became a hit are passed over, every other takes the next miss and
+ * from then on holds that logical block; the success table lists the cache
+ * blocks of hits and served misses by logical index ascending (the row is
+ * zeroed first); the free list is rebuilt from the resident blocks outside the
+ * hit set by block id ascending.
+ *   map_block  dev int32 [table_rows][cap]: cache block of each resident slot of
+ *              a request (mBlocksMap's keys; the same in every layer), map_len
+ *              dev int32 [table_rows] slots in use
+ *   map_idx    dev int32 [n_layers][table_rows][cap], in/out: logical block each
+ *              slot holds (mBlocksMap's values; mDocsTables is the inverse)
+ *   topk_idx   dev int32 [n_layers][batch][topk_stride], topk_len dev int32
+ *              [batch]: the selections (mUseTopkIdxs, topkLensInput)
+ *   rows, bs_index  dev int32 [batch]: table row and batch slot of request i; a
+ *              request with topk_len <= 0 or a row outside the table is skipped
+ *              (CallPrefetchProcessFun, :376-381)
+ *   free_block / free_len      dev int32 [n_layers][max_bs][row_len] / [n_layers][max_bs], in/out (mFreeBlock)
+ *   success_blocks / success_len  the same shapes, out (mLoadSuccessBlocks, mSuccessTableLen)
+ *   load_blocks  dev int32 [n_layers][table_rows][cap], load_count dev int32
+ *              [n_layers][table_rows]: cache blocks that receive a load, in order
+ *              (allNeedLoadBlock, kept with the request's row);
+ *              miss_idxs dev int32 [n_layers][table_rows][topk_stride], miss_count:
+ *              ALL misses in selection order (allMissIdxs); load_blocks[j]
+ *              receives logical block miss_idxs[j].  With load_sel = miss_idxs,
+ *              dst_table = load_blocks and load_count they are the arguments of
+ *              ucm_kv_load_planned.
+ * A selection names a logical block once and the free list a block once, both
+ * blocks of the map (what the reference's Python side guarantees).  At most 256
+ * resident blocks, selected blocks and free-list entries per request.
+ */
+int ucm_prefetch_plan(const int32_t* map_block, const int32_t* map_len, int32_t* map_idx, int table_rows,
+                      int cap, const int32_t* topk_idx, int topk_stride, const int32_t* topk_len,
+                      const int32_t* rows, const int32_t* bs_index, int batch, int n_layers, int max_bs,
+                      int row_len, int32_t* free_block, int32_t* free_len, int32_t* success_blocks,
+                      int32_t* success_len, int32_t* load_blocks, int32_t* load_count, int32_t* miss_idxs,
+                      int32_t* miss_count, ucm_stream_t stream);
+
+/*
  * Hash-code retrieval (KvComp).  A vector's code has bit c = (x . W[:, c] > 0),
  * packed LSB first (bit j of byte b is column 8b+j) - HashEncoder.compute_hash
  * (ucm/sparse/kvcomp/hash_encoder.py:99-157, bit order :92-97,139-149; W is
@@ -555,7 +598,11 @@ int ucm_kv_gather_selected(const void* const* layers, int n_layers, size_t kv_st
  *   src_table   dev int32 [table_rows][src_stride]: pool block holding logical
  *               block i of the request, -1 = not stored (skipped)
  *   dst_table   dev int32 [table_rows][dst_stride]: cache block id of slot j
- *               (the request's first top_k vLLM blocks, esa.py:311)
+ *               (the request's first top_k vLLM blocks, esa.py:311); layer l
+ *               reads the table dst_layer_stride elements after layer l-1's
+ *               (0: one table for all layers)
+ *   load_count  dev int32 [n_layers][table_rows] or NULL: only the first
+ *               load_count entries of a row of load_sel are followed
  *   rows        dev int32 [batch] or NULL (then request b uses row b)
  * Ids outside the pool or the cache are skipped, never dereferenced.
  */
@@ -563,8 +610,8 @@ int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_stride, siz
                         int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
                         int store_first_layer, const int32_t* load_sel, int n_slots,
                         const int32_t* src_table, int src_stride, const int32_t* dst_table,
-                        int dst_stride, const int32_t* rows, int batch, int table_rows,
-                        ucm_stream_t stream);
+                        int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                        const int32_t* rows, int batch, int table_rows, ucm_stream_t stream);
 
 #ifdef __cplusplus
 }

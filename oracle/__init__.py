@@ -83,6 +83,7 @@ _orc_kvstar_block_repre = _sig(_orc, "orc_kvstar_block_repre", None, _p, _p, _p,
 _orc_kvstar_retrieve = _sig(_orc, "orc_kvstar_retrieve", _i32, _p, _u32, _u32, _u32, _p, _u32, _u32, _u32, _u32, _u32, _p,
                             _u32, _p, _p)
 _orc_f32_to_bf16 = _sig(_orc, "orc_f32_to_bf16", C.c_uint16, _f32)
+_orc_prefetch_run = _sig(_orc, "orc_prefetch_run", _i32, _p, _p, _i32, _p, _i32, _p, _p, _p, _i32, _p, _p, _p, _p)
 _orc_kvstar_topk = _sig(_orc, "orc_kvstar_topk", _i32, _p, _u32, _u32, _p)
 
 
@@ -346,6 +347,25 @@ def kvstar_topk(final_scores: np.ndarray, topk: int) -> np.ndarray:
     return out[:k].copy()
 
 
+def prefetch_run(map_block, map_idx, topk, free_block, free_len: int, success_cap: int):
+    """One (request, layer) of the GSA prefetch engine.  map_idx (int32 array) is updated in place.  Returns
+    (success_blocks [success_cap], success_len, load_blocks, miss_idxs, new_free_list)."""
+    mb = _c(map_block, np.int32)
+    assert map_idx.dtype == np.int32 and map_idx.flags.c_contiguous and len(map_idx) == len(mb)
+    tk = _c(topk, np.int32)
+    fb = np.zeros(max(len(mb), len(free_block), 1), np.int32)
+    fb[: len(free_block)] = free_block
+    fl, sl, nm = C.c_int32(int(free_len)), C.c_int32(0), C.c_int32(0)
+    succ = np.zeros(max(success_cap, 1), np.int32)
+    loads = np.zeros(max(len(tk), 1), np.int32)
+    miss = np.zeros(max(len(tk), 1), np.int32)
+    n_load = _orc_prefetch_run(_ptr(mb), _ptr(map_idx), len(mb), _ptr(tk), len(tk), _ptr(fb), C.byref(fl), _ptr(succ),
+                               success_cap, C.byref(sl), _ptr(loads), _ptr(miss), C.byref(nm))
+    if n_load < 0:
+        raise ValueError("free list names a block that is not in the map")
+    return succ[:success_cap], int(sl.value), loads[:n_load].copy(), miss[: nm.value].copy(), fb[: fl.value].copy()
+
+
 def f32_to_bf16(x: float) -> int:
     return int(_orc_f32_to_bf16(float(x)))
 
@@ -428,6 +448,18 @@ class _Ref:
         self.lib.ref_select_topk_bs(_ptr(w), _ptr(rp), _ptr(so), _ptr(sl), _ptr(tk), b, k_head, q_head,
                                     num_krepre, d, _ptr(out), out_stride)
         return out
+
+    def gsa_prefetch_module(self):
+        """The reference's GSA prefetch engine built as a python extension (or None)."""
+        if not os.path.isdir(_REF_DIR) or not any(f.startswith("gsa_prefetch") for f in os.listdir(_REF_DIR)):
+            return None
+        import torch  # noqa: F401  (the extension links against libtorch)
+
+        if _REF_DIR not in sys.path:
+            sys.path.insert(0, _REF_DIR)
+        import gsa_prefetch  # noqa: E402  (compiled from the reference's C++)
+
+        return gsa_prefetch
 
     def retrieval_backend_module(self):
         """The reference's ESA backend built as a python extension (or None)."""

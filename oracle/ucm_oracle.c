@@ -28,11 +28,22 @@
  *   orc_hash_*: closed forms (sign, LSB-first packing, <u,v> = bits-2*hamming),
  *       brute force on tiny inputs.  The majority-vote block code is not in
  *       the reference: parity unpinned beyond its closed form.
+ *   orc_f32_to_bf16 and the round_bf16 mode of orc_block_mean_paged: torch's
+ *       float32 -> bfloat16 conversion (ties, subnormals, overflow, inf, NaN).
+ *   orc_hash_encode / orc_hash_encode_f32 at 128 x 128: numpy float64 products
+ *       and exactly summed products on rows built to cancel; orc_hash_colsum:
+ *       2*popcount - T; orc_kv_gather_selected: closed-form placement on a
+ *       poisoned buffer; orc_topk_windows_i32: brute force.
+ *   orc_prefetch_run: the reference's kvcache_pre.cpp compiled against this
+ *       image's torch (oracle/_ref/gsa_prefetch*.so) and driven through whole
+ *       call sequences, plus the golden vectors written from it.
  *   orc_kvstar_*: PARITY UNPINNED against a build of the reference (its
  *       translation unit needs spdlog, absent here).  Pinned by what the
  *       mathematics fixes: an fp64 softmax-vote in numpy, sum(final) = number
  *       of (token, head) rows, shift invariance, brute force on tiny inputs,
- *       and the half-precision conversions against numpy's float16.
+ *       and the half-precision conversions against numpy's float16.  The
+ *       selection step (orc_kvstar_topk) restates the reference's heap
+ *       literally and is checked against python's heapq on tie-heavy inputs.
  */
 #include <float.h>
 #include <math.h>
@@ -879,4 +890,96 @@ ORC_API int32_t orc_kvstar_retrieve(const uint16_t* q, uint32_t n_tokens, uint32
     free(row);
     free(qv);
     return orc_kvstar_topk(final_scores, n_blocks, topk, topk_idx);
+}
+
+/* ------------------------------------------------- GSA prefetch engine (hit / miss / free list) */
+
+/*
+ * One (request, layer) of GSAPrefetchEngineC::RunOneBsPrefetch
+ * (ucm/sparse/gsa/prefetch/src/kvcache_pre.cpp:274-311) with the steps it calls:
+ * GetHitAndMissBlock (:206-238), RunPrefetchH2D (:240-272) and LoadKVToHBM
+ * (:313-322).
+ *
+ * State: the request's resident blocks, mBlocksMap = {cache block id -> logical
+ * block it holds}, given as the arrays map_block / map_idx (any order; the
+ * reference's std::map iterates by block id ascending) and updated in place;
+ * mDocsTables is the inverse map.  free_block / *free_len are the layer's row of
+ * mFreeBlock / mFreeBlockLen, in and out.
+ *
+ *   1. every selected logical block topk[j], in order: resident -> its cache
+ *      block joins the hit set; otherwise it is appended to the misses;
+ *   2. if there are misses: the free list is walked in order; an entry whose
+ *      block is in the hit set is passed over, any other takes the next miss
+ *      (in top-k order), joins the hit set, and the maps are rewritten so that
+ *      this cache block now holds that logical block; the walk ends when either
+ *      list does.  load_blocks = the blocks taken, in that order; miss_idxs =
+ *      ALL misses (load_blocks[i] receives miss_idxs[i]; misses beyond the free
+ *      list stay unserved);
+ *   3. the success table is zeroed and then lists the cache block of every hit
+ *      and served miss, ordered by LOGICAL index ascending (hitBlocksIdx is a
+ *      std::map);
+ *   4. the free list is rebuilt: the blocks of the map, by block id ascending,
+ *      that are not in the hit set; success_len = size of the hit set.
+ * A selection entry is assumed to occur once and every free-list entry to be a
+ * block of the map (what the Python side guarantees; the reference's operator[]
+ * would otherwise insert it).  Returns the number of loads, -1 on a free block
+ * that is not in the map.
+ */
+ORC_API int32_t orc_prefetch_run(int32_t* map_block, int32_t* map_idx, int32_t n_map, const int32_t* topk,
+                                 int32_t topk_len, int32_t* free_block, int32_t* free_len,
+                                 int32_t* success_blocks, int32_t success_cap, int32_t* success_len,
+                                 int32_t* load_blocks, int32_t* miss_idxs, int32_t* n_miss)
+{
+    uint8_t* in_hit = (uint8_t*)calloc((size_t)(n_map ? n_map : 1), 1);
+    /* hitBlocksIdx: (logical idx, block) pairs */
+    int32_t* h_idx = (int32_t*)malloc((size_t)(topk_len + 1) * sizeof(int32_t));
+    int32_t* h_blk = (int32_t*)malloc((size_t)(topk_len + 1) * sizeof(int32_t));
+    int32_t n_h = 0, misses = 0, hit_size = 0, loads = 0;
+    for (int32_t j = 0; j < topk_len; ++j) {
+        const int32_t item = topk[j];
+        int32_t e = -1;
+        for (int32_t i = 0; i < n_map; ++i) { if (map_idx[i] == item) { e = i; break; } }
+        if (e >= 0) {
+            if (!in_hit[e]) { in_hit[e] = 1; ++hit_size; }
+            h_idx[n_h] = item; h_blk[n_h] = map_block[e]; ++n_h;
+        } else {
+            miss_idxs[misses++] = item;
+        }
+    }
+    if (misses != 0) {
+        int32_t index = 0, f = 0;
+        while (f < *free_len && index < misses) {
+            const int32_t id = free_block[f];
+            int32_t e = -1;
+            for (int32_t i = 0; i < n_map; ++i) { if (map_block[i] == id) { e = i; break; } }
+            if (e < 0) { free(in_hit); free(h_idx); free(h_blk); return -1; }
+            if (in_hit[e]) { ++f; continue; }
+            load_blocks[loads++] = id;
+            in_hit[e] = 1; ++hit_size;
+            h_idx[n_h] = miss_idxs[index]; h_blk[n_h] = id; ++n_h;
+            map_idx[e] = miss_idxs[index];          /* LoadKVToHBM: the block now holds the missing logical block */
+            ++index; ++f;
+        }
+    }
+    for (int32_t i = 0; i < success_cap; ++i) { success_blocks[i] = 0; }
+    /* by logical index ascending */
+    for (int32_t a = 0; a < n_h; ++a) {
+        int32_t rank = 0;
+        for (int32_t b = 0; b < n_h; ++b) { if (h_idx[b] < h_idx[a]) { ++rank; } }
+        if (rank < success_cap) { success_blocks[rank] = h_blk[a]; }
+    }
+    /* free list: non-hit blocks by block id ascending */
+    int32_t k = 0;
+    for (int32_t a = 0; a < n_map; ++a) {
+        if (in_hit[a]) { continue; }
+        int32_t rank = 0;
+        for (int32_t b = 0; b < n_map; ++b) { if (!in_hit[b] && map_block[b] < map_block[a]) { ++rank; } }
+        free_block[rank] = map_block[a];
+        ++k;
+    }
+    *free_len = k;
+    *success_len = hit_size;
+    *n_miss = misses;
+    free(in_hit); free(h_idx); free(h_blk);
+    return loads;
 }

@@ -329,6 +329,55 @@ def test_gsa_retrieval_stride_reuses_scores(ucm, dev):
     assert [t[1] for t in tables] == [4 * 16 + 15, 5 * 16, 4 * 16 + 1, 4 * 16 + 2]
 
 
+def test_gsa_local_window_save_and_restore(ucm, dev):
+    """Prefetch mode: at the end of a long request's prefill the last `local` blocks are kept aside, K and V, every
+    layer; at its first decode step they are written into the cache blocks that now stand for the window (the last
+    `local` entries of remain_idx), whatever those blocks held (gsa.py:956-1031)."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 64, 3, 16, 200
+    lo, hi = 6, 10                                              # local window = lo - 1 = 5 blocks
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 120, {"seg_prefill_threshold": 100, "min_topk_len": lo, "max_topk_len": hi,
+                                                    "ptopk_prefetch_enable": True})
+    plugin = GSA(cfg, UcmSparseRole.WORKER)
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev).to(torch.bfloat16) for _ in range(L)]
+    plugin.register_kv_caches({f"model.layers.{l}.self_attn.attn": caches[l] for l in range(L)})
+    n_blocks = 40
+    prompt_len = n_blocks * bs
+    prompt_blocks = [int(x) for x in synth.permutation(950, nb)[:n_blocks]]
+    short_blocks = [int(x) for x in synth.permutation(951, nb)[100:104]]
+    reqs = {"long": ns(block_ids=[prompt_blocks], num_computed_tokens=0, prompt_token_ids=[1] * prompt_len, output_token_ids=[]),
+            "short": ns(block_ids=[short_blocks], num_computed_tokens=0, prompt_token_ids=[1] * 60, output_token_ids=[])}
+    ib = ns(req_id_to_index={"long": 0, "short": 1})
+    so = ns(num_scheduled_tokens={"long": prompt_len, "short": 60}, scheduled_new_reqs=[ns(req_id="long"), ns(req_id="short")])
+    plugin.build_sparse_meta(so, reqs, ib, None)
+    plugin.execute_begin(so)
+    plugin.execute_finished()                                   # the prefill step ends: the window is saved
+    st = plugin.gsa_stats["long"]
+    assert plugin.gsa_stats["short"].local_window_kv is None and st.local_window_kv.shape[:3] == (lo - 1, L, 2)
+    window = [c[:, prompt_blocks[-(lo - 1):]].clone() for c in caches]
+    # the scheduler now gives the request its sparse block list: k = compute_topk_len(40) = 10 (the cap) -> 10 + 1
+    # sparse blocks, and one more for the token being decoded; everything in the cache is overwritten in between
+    sparse_blocks = [int(x) for x in synth.permutation(952, nb)[150:162]]
+    for c in caches:
+        c.normal_()
+    before = [c.clone() for c in caches]
+    reqs["long"].block_ids = [sparse_blocks]
+    reqs["long"].num_computed_tokens = prompt_len
+    reqs["long"].output_token_ids = [1]
+    so = ns(num_scheduled_tokens={"long": 1}, scheduled_new_reqs=[])
+    plugin.build_sparse_meta(so, reqs, ns(req_id_to_index={"long": 0}), None)
+    torch.cuda.synchronize()
+    assert st.remain_idx == list(range(5)) + list(range(6, 11)) and st.prefetch_idx == [5]
+    target = [sparse_blocks[x] for x in st.remain_idx[-(lo - 1):]]
+    for l in range(L):
+        assert torch.equal(caches[l][:, target], window[l])
+        rest = [b for b in range(nb) if b not in target]
+        assert torch.equal(caches[l][:, rest], before[l][:, rest])
+
+
 # ------------------------------------------------- block store + ESA plugin
 
 def test_hip_block_store_round_trip(ucm, dev):

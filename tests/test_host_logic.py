@@ -281,3 +281,38 @@ def test_kvstar_scheduler_side(ucm):
     assert got.blocks == (held[-4:],) and calls == [50, ("alloc", 50)]
     coord.get_num_blocks_to_allocate = lambda request_id, num_tokens, new_computed_blocks: 2
     assert plugin.allocate_slots(ns(request_id="A"), 50, coord, Pool(), [None]) is None
+
+
+def test_gsa_prefetch_mode_resident_set_and_slots(ucm):
+    """The resident set of a sparsified request (gsa.py:156-186) and the slots it is given (gsa.py:891-912), checked
+    against values worked out by hand from the reference's constants (min 32, max 48, ratio 0.3, local = 31)."""
+    from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA, GSAReqStat
+
+    st = GSAReqStat("a", 0, 128, 8400)
+    st.blocks = list(range(100))                      # 100 blocks -> k = int(30.0) = 30 < 32 -> min(32, 100) = 32
+    st.num_prompt_tokens = st.num_computed_tokens = 100 * 128
+    st.get_sparse_and_free_block(True, 32, 48, 0.3)
+    # blocks 0..48 stand for the sparse cache; in use: the first 32 - 31 = 1 and the last 31; free in between
+    assert st.remain_idx == [0] + list(range(18, 49)) and st.prefetch_idx == list(range(1, 18))
+    assert st.sparse_len == 32 + 17 and len(st.remain_idx) == 32
+    st.blocks = list(range(200))                      # k = int(60.0) -> capped at 48
+    st.num_prompt_tokens = st.num_computed_tokens = 200 * 128
+    st.get_sparse_and_free_block(True, 32, 48, 0.3)
+    assert st.remain_idx == list(range(17)) + list(range(18, 49)) and st.prefetch_idx == [17] and st.sparse_len == 49
+    st.get_sparse_and_free_block(False, 32, 48, 0.3)  # prefetch mode off: everything stays
+    assert st.remain_idx == list(range(200)) and st.prefetch_idx == [] and st.sparse_len == 200
+    st.num_computed_tokens += 1                       # past the first decode step: no longer decided here
+    st.get_sparse_and_free_block(True, 32, 48, 0.3)
+    assert st.remain_idx is None and st.prefetch_idx is None
+
+    plugin = GSA(make_config(cfg={"ptopk_prefetch_enable": True}), UcmSparseRole.SCHEDULER)
+    req = ns(num_prompt_tokens=100 * 128, num_output_tokens=5, num_tokens=100 * 128 + 5)
+    # 101 blocks in all, 100 of the prompt: 1 + 32 + 17 = 50 blocks, the last one holding 5 tokens
+    assert plugin.estimate_num_slots_sparsed(req) == 50 * 128 - (128 - 5)
+    req = ns(num_prompt_tokens=200 * 128 + 7, num_output_tokens=121, num_tokens=201 * 128)
+    assert plugin.estimate_num_slots_sparsed(req) == (201 - 201 + 48 + 1) * 128
+    assert plugin.estimate_num_slots_sparsed(ns(num_prompt_tokens=8400, num_output_tokens=5, num_tokens=8405)) == INVALID_SLOT
+    assert plugin.estimate_num_slots_sparsed(ns(num_prompt_tokens=9000, num_output_tokens=0, num_tokens=9000)) == INVALID_SLOT
+    off = GSA(make_config(), UcmSparseRole.SCHEDULER)
+    assert off.estimate_num_slots_sparsed(ns(num_prompt_tokens=100 * 128, num_output_tokens=5, num_tokens=100 * 128 + 5)) == INVALID_SLOT

@@ -667,3 +667,65 @@ def test_kvstar_heap_tie_rule():
     q = np.ones((1, 1, 16), np.float16)
     idx, final = O.kvstar_retrieve(q.view(np.uint16), rep.view(np.uint16), 3)
     assert final[1] == final[3] and final[0] == final[2] and list(idx) == [3, 1, 2]
+
+
+# ------------------------------------------------ GSA prefetch engine bookkeeping
+
+@needs_ref
+def test_ref_prefetch_engine_live():
+    """orc_prefetch_run, replayed over whole call sequences, against the reference's own GSAPrefetchEngineC compiled
+    from kvcache_pre.cpp: success tables, success lengths, rebuilt free lists, loads, misses and block maps of
+    every run, every layer, every request."""
+    from golden.make_golden import prefetch_scenario, prefetch_scenarios, run_reference_prefetch
+    from prefetch_model import replay, same_result
+
+    gp = O.ref.gsa_prefetch_module()
+    if gp is None:
+        pytest.skip("gsa_prefetch extension not built")
+    cases = prefetch_scenarios() + [(3000 + 31 * i, 1 + i % 3, 1 + i % 4, 4) for i in range(12)]
+    served_short = hit_in_free = 0
+    for seed, n_layers, n_req, n_runs in cases:
+        reqs, runs = prefetch_scenario(seed, n_layers, n_req, n_runs)
+        want = run_reference_prefetch(gp, n_layers, reqs, runs)
+        got = replay(n_layers, reqs, runs)
+        for w, g in zip(want, got):
+            same_result(w, g)
+            served_short += sum(len(ld) < len(ms) for lr, mr in zip(w["loads"], w["misses"]) for ld, ms in zip(lr, mr))
+    assert served_short > 0          # the cases do include selections the free list could not serve
+
+
+def test_golden_prefetch_engine(golden):
+    from golden.make_golden import prefetch_scenario
+    from prefetch_model import replay
+
+    z, meta = golden
+    assert meta.get("prefetch"), "fixture was written without the prefetch engine"
+    flat = lambda x: np.array([v for per_req in x for per_layer in per_req for v in [len(per_layer)] + list(per_layer)], np.int32)
+    for seed, n_layers, n_req, n_runs in meta["prefetch"]:
+        reqs, runs = prefetch_scenario(seed, n_layers, n_req, n_runs)
+        for t, g in enumerate(replay(n_layers, reqs, runs)):
+            key = f"prefetch/{seed}/{t}"
+            assert np.array_equal(g["success"], z[key + "/success"]) and np.array_equal(g["success_len"], z[key + "/success_len"])
+            assert np.array_equal(g["free_len"], z[key + "/free_len"])
+            for l in range(n_layers):
+                for s in range(g["free"].shape[1]):
+                    n = g["free_len"][l, s]
+                    assert np.array_equal(g["free"][l, s, :n], z[key + "/free"][l, s, :n])
+            assert np.array_equal(flat(g["loads"]), z[key + "/loads"]) and np.array_equal(flat(g["misses"]), z[key + "/misses"])
+            maps = np.array([v for rq in reqs for m in g["maps"][rq["req_id"]]
+                             for kv in [(len(m), -1)] + sorted(m.items()) for v in kv], np.int32)
+            assert np.array_equal(maps, z[key + "/maps"])
+
+
+def test_prefetch_run_by_hand():
+    """A case small enough to follow: cache blocks 50, 60, 70, 80 hold logical blocks 0, 1, 2, 3; the free list names 70
+    then 60.  Selecting [3, 9, 1, 8]: 3 and 1 are hits (blocks 80, 60); 9 and 8 miss.  The free list offers 70 (taken
+    by 9), then 60 - a hit, passed over - and is then exhausted, so 8 stays unserved.  Success table by logical
+    index: 1 -> 60, 3 -> 80, 9 -> 70.  New free list: blocks outside the hit set by id: [50]."""
+    idx = np.array([0, 1, 2, 3], np.int32)
+    succ, sl, loads, miss, free = O.prefetch_run([50, 60, 70, 80], idx, [3, 9, 1, 8], [70, 60], 2, 6)
+    assert loads.tolist() == [70] and miss.tolist() == [9, 8]
+    assert succ.tolist() == [60, 80, 70, 0, 0, 0] and sl == 3
+    assert free.tolist() == [50] and idx.tolist() == [0, 1, 9, 3]
+    with pytest.raises(ValueError):
+        O.prefetch_run([50, 60], np.array([0, 1], np.int32), [5], [99], 1, 4)

@@ -32,7 +32,8 @@ SIGNATURES = {
     "ucm_esa_retrieve_static": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _i, _p],
     "ucm_esa_retrieve_rows": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _i, _p, _i, _p, _p, _p, _p, _p, _i, _p],
     "ucm_delta_plan_rows": [_p, _p, _p, _p, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
-    "ucm_kv_load_planned": [_p, _i, _sz, _sz, _i, _p, _i64, _sz, _i, _p, _i, _p, _i, _p, _i, _p, _i, _i, _p],
+    "ucm_kv_load_planned": [_p, _i, _sz, _sz, _i, _p, _i64, _sz, _i, _p, _i, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _p],
+    "ucm_prefetch_plan": [_p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p],
     "ucm_delta_plan": [_p, _p, _p, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _p],
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],

@@ -103,7 +103,8 @@ __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
     void* const* __restrict__ layers, size_t kv_stride, size_t block_bytes, unsigned num_blocks,
     const uint8_t* __restrict__ pool, uint64_t pool_blocks, size_t pool_block_bytes, unsigned store_first_layer,
     const int32_t* __restrict__ load_sel, unsigned n_slots, const int32_t* __restrict__ src_table, unsigned src_stride,
-    const int32_t* __restrict__ dst_table, unsigned dst_stride, const int32_t* __restrict__ rows, unsigned table_rows)
+    const int32_t* __restrict__ dst_table, unsigned dst_stride, int64_t dst_layer_stride,
+    const int32_t* __restrict__ load_count, const int32_t* __restrict__ rows, unsigned table_rows)
 {
     const unsigned j = blockIdx.x, b = blockIdx.y, l = blockIdx.z >> 1, kv = blockIdx.z & 1;
     unsigned row = b;
@@ -113,11 +114,12 @@ __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
         row = static_cast<unsigned>(r);
     }
     if (row >= table_rows) { return; }
+    if (load_count && static_cast<int32_t>(j) >= load_count[static_cast<size_t>(l) * table_rows + row]) { return; }
     const int32_t sel = load_sel[(static_cast<size_t>(l) * table_rows + row) * n_slots + j];
     if (sel < 0 || static_cast<unsigned>(sel) >= src_stride) { return; }     // slot keeps what it holds
     const int32_t src = src_table[static_cast<size_t>(row) * src_stride + sel];
     if (src < 0 || static_cast<uint64_t>(src) >= pool_blocks) { return; }   // block not in the pool
-    const unsigned dst = static_cast<unsigned>(dst_table[static_cast<size_t>(row) * dst_stride + j]);
+    const unsigned dst = static_cast<unsigned>(dst_table[l * dst_layer_stride + static_cast<int64_t>(row) * dst_stride + j]);
     if (dst >= num_blocks) { return; }
     copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
                pool + static_cast<size_t>(src) * pool_block_bytes +
@@ -212,8 +214,8 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
                                    int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
                                    int store_first_layer, const int32_t* load_sel, int n_slots,
                                    const int32_t* src_table, int src_stride, const int32_t* dst_table,
-                                   int dst_stride, const int32_t* rows, int batch, int table_rows,
-                                   ucm_stream_t stream)
+                                   int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                                   const int32_t* rows, int batch, int table_rows, ucm_stream_t stream)
 {
     UCM_REQUIRE(batch >= 0 && n_slots >= 0 && table_rows > 0, "ucm_kv_load_planned: batch=%d n_slots=%d table_rows=%d", batch,
                 n_slots, table_rows);
@@ -229,13 +231,13 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
                     static_cast<size_t>(store_first_layer + n_layers) * 2 * block_bytes <= pool_block_bytes,
                 "ucm_kv_load_planned: layers %d..%d do not fit a stored block of %zu bytes", store_first_layer,
                 store_first_layer + n_layers - 1, pool_block_bytes);
-    UCM_REQUIRE(src_stride >= 1 && dst_stride >= n_slots, "ucm_kv_load_planned: src_stride=%d dst_stride=%d n_slots=%d", src_stride,
-                dst_stride, n_slots);
+    UCM_REQUIRE(src_stride >= 1 && dst_stride >= n_slots && dst_layer_stride >= 0,
+                "ucm_kv_load_planned: src_stride=%d dst_stride=%d n_slots=%d", src_stride, dst_stride, n_slots);
     hipLaunchKernelGGL(kv_load_planned_kernel, dim3(static_cast<unsigned>(n_slots), batch, n_layers * 2), dim3(kThreads), 0,
                        ucm::as_stream(stream), layers, kv_stride, block_bytes, static_cast<unsigned>(num_blocks),
                        static_cast<const uint8_t*>(pool), static_cast<uint64_t>(pool_blocks), pool_block_bytes,
                        static_cast<unsigned>(store_first_layer), load_sel, static_cast<unsigned>(n_slots), src_table,
-                       static_cast<unsigned>(src_stride), dst_table, static_cast<unsigned>(dst_stride), rows,
-                       static_cast<unsigned>(table_rows));
+                       static_cast<unsigned>(src_stride), dst_table, static_cast<unsigned>(dst_stride), dst_layer_stride,
+                       load_count, rows, static_cast<unsigned>(table_rows));
     UCM_LAUNCH_CHECK("ucm_kv_load_planned");
 }

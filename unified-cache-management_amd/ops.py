@@ -256,24 +256,61 @@ def delta_plan_rows(sel: torch.Tensor, sel_phys: torch.Tensor, count: torch.Tens
 def kv_load_planned(layers: LayerPointers, ptr_first: int, store_first_layer: int, n_layers: int, kv_stride: int,
                     block_bytes: int, num_blocks: int, pool: torch.Tensor, pool_block_bytes: int,
                     load_sel: torch.Tensor, src_table: torch.Tensor, dst_table: torch.Tensor,
-                    rows: Optional[torch.Tensor]) -> None:
+                    rows: Optional[torch.Tensor], load_count: Optional[torch.Tensor] = None) -> None:
     """pool: uint8 buffer of stored blocks ([block][layer][K|V], device or pinned host memory); load_sel int32
     [n_layers, table_rows, n_slots]: the plan of model layers store_first_layer.., whose cache pointers are entries
-    ptr_first.. of ``layers``; src_table int32 [table_rows, M]; dst_table int32 [table_rows, >= n_slots]; rows int32
-    [B] or None (all table rows)."""
+    ptr_first.. of ``layers``; src_table int32 [table_rows, M]; dst_table int32 [table_rows, >= n_slots], or
+    [n_layers, table_rows, >= n_slots] when every layer has destinations of its own; load_count int32
+    [n_layers, table_rows] or None; rows int32 [B] or None (all table rows)."""
     if load_sel.dim() != 3 or load_sel.shape[0] != n_layers:
         raise ValueError("load_sel must be [n_layers, table_rows, n_slots]")
     table_rows, n_slots = load_sel.shape[1], load_sel.shape[2]
-    if src_table.shape[0] != table_rows or dst_table.shape[0] != table_rows or dst_table.shape[1] < n_slots:
+    per_layer = dst_table.dim() == 3
+    if src_table.shape[0] != table_rows or dst_table.shape[-2] != table_rows or dst_table.shape[-1] < n_slots \
+            or (per_layer and dst_table.shape[0] != n_layers):
         raise ValueError("src_table / dst_table must have one row per table row")
+    if load_count is not None and load_count.shape != (n_layers, table_rows):
+        raise ValueError("load_count must be [n_layers, table_rows]")
     if ptr_first < 0 or ptr_first + n_layers > len(layers):
         raise ValueError("layer range outside the pointer table")
     nbytes = pool.numel() * pool.element_size()
     _lib.call("ucm_kv_load_planned", layers.ptr(ptr_first), n_layers, kv_stride, block_bytes, num_blocks,
               _staging_ptr(pool, 0), nbytes // pool_block_bytes, pool_block_bytes, store_first_layer,
               _dev(load_sel, torch.int32, "load_sel"), n_slots, _dev(src_table, torch.int32, "src_table"),
-              src_table.shape[1], _dev(dst_table, torch.int32, "dst_table"), dst_table.shape[1],
+              src_table.shape[1], _dev(dst_table, torch.int32, "dst_table"), dst_table.shape[-1],
+              dst_table.stride(0) if per_layer else 0, _opt(load_count, torch.int32, "load_count"),
               _opt(rows, torch.int32, "rows"), table_rows if rows is None else rows.numel(), table_rows, _stream())
+
+
+def prefetch_plan(map_block: torch.Tensor, map_len: torch.Tensor, map_idx: torch.Tensor, topk_idx: torch.Tensor,
+                  topk_len: torch.Tensor, rows: torch.Tensor, bs_index: torch.Tensor, free_block: torch.Tensor,
+                  free_len: torch.Tensor, success_blocks: torch.Tensor, success_len: torch.Tensor,
+                  load_blocks: torch.Tensor, load_count: torch.Tensor, miss_idxs: torch.Tensor,
+                  miss_count: torch.Tensor) -> None:
+    """map_block int32 [table_rows, cap]; map_idx int32 [L, table_rows, cap]; topk_idx int32 [L, B, stride];
+    free_block / success_blocks int32 [L, max_bs, row_len]; free_len / success_len int32 [L, max_bs];
+    load_blocks int32 [L, table_rows, cap]; miss_idxs int32 [L, table_rows, stride]; counts int32 [L, table_rows]."""
+    n_layers, table_rows, cap = map_idx.shape
+    batch = rows.numel()
+    if map_block.shape != (table_rows, cap) or map_len.numel() != table_rows:
+        raise ValueError("map_block [table_rows, cap] / map_len [table_rows] expected")
+    if topk_idx.dim() != 3 or topk_idx.shape[:2] != (n_layers, batch) or topk_len.numel() != batch or bs_index.numel() != batch:
+        raise ValueError("topk_idx [L, B, stride], topk_len / rows / bs_index [B] expected")
+    max_bs, row_len = free_block.shape[1], free_block.shape[2]
+    if free_block.shape[0] != n_layers or success_blocks.shape != free_block.shape or free_len.shape != (n_layers, max_bs) \
+            or success_len.shape != free_len.shape:
+        raise ValueError("free / success tables must be [L, max_bs, row_len] and [L, max_bs]")
+    if load_blocks.shape != (n_layers, table_rows, cap) or miss_idxs.shape != (n_layers, table_rows, topk_idx.shape[2]) \
+            or load_count.shape != (n_layers, table_rows) or miss_count.shape != load_count.shape:
+        raise ValueError("load / miss outputs have the wrong shape")
+    _lib.call("ucm_prefetch_plan", _dev(map_block, torch.int32, "map_block"), _dev(map_len, torch.int32, "map_len"),
+              _dev(map_idx, torch.int32, "map_idx"), table_rows, cap, _dev(topk_idx, torch.int32, "topk_idx"),
+              topk_idx.shape[2], _dev(topk_len, torch.int32, "topk_len"), _dev(rows, torch.int32, "rows"),
+              _dev(bs_index, torch.int32, "bs_index"), batch, n_layers, max_bs, row_len,
+              _dev(free_block, torch.int32, "free_block"), _dev(free_len, torch.int32, "free_len"),
+              _dev(success_blocks, torch.int32, "success_blocks"), _dev(success_len, torch.int32, "success_len"),
+              _dev(load_blocks, torch.int32, "load_blocks"), _dev(load_count, torch.int32, "load_count"),
+              _dev(miss_idxs, torch.int32, "miss_idxs"), _dev(miss_count, torch.int32, "miss_count"), _stream())
 
 
 HASH_SCORE_SUM, HASH_SCORE_BLOCK_CODE = 0, 1

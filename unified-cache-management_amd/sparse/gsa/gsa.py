@@ -64,6 +64,12 @@ class GSAReqStat:
         self.num_output_tokens = 0
         self.index_in_batch = 0
         self._repre_done = 0  # blocks [0, _repre_done) have a representative
+        # prefetch mode (the reference's PTOPK_PREFETCH_ENABLE): which logical blocks stay resident once the
+        # request is sparsified, which resident blocks start out free, and the saved local window
+        self.remain_idx: Optional[List[int]] = None
+        self.prefetch_idx: Optional[List[int]] = None
+        self.sparse_len = 0
+        self.local_window_kv: Optional[torch.Tensor] = None   # [blocks, layers, K|V, block bytes]
 
     # -- state queries (same meaning as the reference's) ---------------------
     def is_decode(self) -> bool:
@@ -78,16 +84,43 @@ class GSAReqStat:
     def get_seq_len(self) -> int:
         return self.num_computed_tokens + self.num_scheduled_tokens
 
+    def get_sparse_and_free_block(self, prefetch: bool, min_topk: int, max_topk: int, ratio: float) -> None:
+        """The resident set at the first decode step (GSAReqStat._get_sparse_and_free_block, gsa.py:156-186): with
+        n blocks and k = compute_topk_len(n), logical blocks 0 .. max_topk stand for the request's sparse cache
+        blocks; the first k - local and the last local of them are in use (remain_idx), the ones in between start
+        out free (prefetch_idx); local = min_topk - 1."""
+        if self.num_prompt_tokens != self.num_computed_tokens:
+            self.remain_idx = self.prefetch_idx = None
+            return
+        n = len(self.blocks)
+        if self.num_prompt_tokens > self.threshold and prefetch:
+            local = min_topk - 1
+            remain_len = compute_topk_len(n, min_topk, max_topk, ratio)
+            if remain_len > max_topk:
+                prefetch_len, idx = 0, list(range(remain_len))
+            else:
+                prefetch_len, idx = max_topk - remain_len + 1, list(range(max_topk + 1))
+            assert local < remain_len
+            self.remain_idx = idx[: remain_len - local] + idx[-local:]
+            self.prefetch_idx = idx[remain_len - local : -local]
+            self.sparse_len = remain_len + prefetch_len
+        else:
+            self.remain_idx, self.prefetch_idx, self.sparse_len = list(range(n)), [], n
+
     @property
     def repre_slot_mapping(self) -> List[int]:
         return [self.slot_offset + i for i in range(len(self.blocks))]
 
-    def update(self, num_scheduled_tokens: int, req_state, index_in_batch: int) -> None:
+    def update(self, num_scheduled_tokens: int, req_state, index_in_batch: int, prefetch=None) -> None:
         self.num_computed_tokens = req_state.num_computed_tokens
         self.num_scheduled_tokens = num_scheduled_tokens
         self.num_prompt_tokens = len(req_state.prompt_token_ids)
         self.num_output_tokens = len(req_state.output_token_ids)
         self.index_in_batch = index_in_batch
+        if prefetch is not None and self.blocks:
+            # decided from the blocks the request held BEFORE the scheduler swapped in its sparse block list
+            # (the reference calls it ahead of touching self.blocks, gsa.py:141-149)
+            self.get_sparse_and_free_block(True, *prefetch)
         self.blocks = list(req_state.block_ids[0])
         # A block gets its representative once every one of its tokens is in
         # the cache, i.e. after the step that fills it.
@@ -154,6 +187,10 @@ class GSA(UcmSparseBase):
         self.local_window = int(cfg.get("local_window_sz", LOCAL_WINDOW_BLOCKS))
         # "bfloat16": the table keeps the rounded means the live reference path stores (gsa.py:640-652) in
         # that type, half the bytes to score; "float32": fp32 means, the KRepreComputer contract
+        # the reference's PTOPK_PREFETCH_ENABLE (ucm/sparse/utils.py:11, off as shipped): sparsified requests give
+        # most of their cache blocks back, so the local window is kept aside at the end of the prefill and
+        # written into the blocks that stand for it afterwards
+        self.ptopk_prefetch = bool(cfg.get("ptopk_prefetch_enable", False))
         self.repre_dtype = torch.bfloat16 if cfg.get("repre_dtype", "float32") == "bfloat16" else torch.float32
         self.repre_mode = ops.MEAN_BF16_STORE if self.repre_dtype == torch.bfloat16 else ops.MEAN_F32
 
@@ -166,6 +203,8 @@ class GSA(UcmSparseBase):
         self.v_cache: Dict[int, torch.Tensor] = {}
         self._dev_ready = False
         self._layer_ptrs: Dict[int, ops.LayerPointers] = {}
+        self._kv_all: Optional[ops.LayerPointers] = None   # every layer's (2, blocks, ...) cache, for whole-block moves
+        self._kv_full: Dict[int, torch.Tensor] = {}
         self._scored: set = set()  # sparsified requests whose blocks have been scored at least once
 
     # ------------------------------------------------------------------ device state
@@ -207,7 +246,47 @@ class GSA(UcmSparseBase):
             return
         self.k_cache[layer_id], self.v_cache[layer_id] = kv_cache[0], kv_cache[1]
         self._layer_ptrs[layer_id] = ops.LayerPointers([kv_cache[0]])
+        self._kv_full[layer_id] = kv_cache
+        self._kv_all = None
         self._ensure_device_state(kv_cache[0].device)
+
+    def _all_layers(self):
+        """(pointer table over every layer's cache, bytes between the K and V planes, bytes of a block, blocks)."""
+        if self._kv_all is None:
+            if len(self._kv_full) != self.layer_num or not all(isinstance(c, torch.Tensor) for c in self._kv_full.values()):
+                raise RuntimeError("whole-block moves need every layer's cache registered as one (2, blocks, ...) tensor")
+            self._kv_all = ops.LayerPointers([self._kv_full[l] for l in range(self.layer_num)])
+        kv = self._kv_full[0]
+        return self._kv_all, kv.stride(0) * kv.element_size(), kv.stride(1) * kv.element_size(), kv.shape[1]
+
+    # ------------------------------------------------------------------ local window (prefetch mode)
+    def _gsa_sparse_local_kv(self) -> None:
+        """End of the step that finishes a long request's prefill: the K and V of its last ``local`` blocks, every
+        layer, are kept aside (gsa.py:995-1031) - one gather launch instead of a clone per block, layer and plane."""
+        local = self.min_topk - 1
+        for st in self.model_input.get("batch", []):
+            if st is None or st.is_decode() or not st.is_last_chunk() or st.num_prompt_tokens <= self.threshold:
+                continue
+            layers, kv_stride, block_bytes, num_blocks = self._all_layers()
+            ids = torch.tensor(st.blocks[-local:], dtype=torch.int32, device=self.device)
+            st.local_window_kv = torch.empty((ids.numel(), self.layer_num, 2, block_bytes), dtype=torch.uint8, device=self.device)
+            ops.kv_gather_blocks(layers, kv_stride, block_bytes, num_blocks, ids, st.local_window_kv)
+
+    def _init_sparse_local_kv(self, scheduler_output, requests) -> None:
+        """First decode step of such a request: the saved window goes into the cache blocks that now stand for it,
+        the last ``local`` entries of remain_idx (gsa.py:956-993), as one scatter launch."""
+        local = self.min_topk - 1
+        for req_id in scheduler_output.num_scheduled_tokens:
+            st = self.gsa_stats.get(req_id)
+            if st is None or st.num_prompt_tokens <= self.threshold or st.local_window_kv is None:
+                continue
+            if st.num_computed_tokens != st.num_prompt_tokens:
+                continue
+            assert st.remain_idx is not None
+            blocks = requests[req_id].block_ids[0]
+            ids = torch.tensor([blocks[x] for x in st.remain_idx[-local:]], dtype=torch.int32, device=self.device)
+            layers, kv_stride, block_bytes, num_blocks = self._all_layers()
+            ops.kv_scatter_blocks(layers, kv_stride, block_bytes, num_blocks, ids, st.local_window_kv)
 
     def maybe_register_kv_cache(self, forward_context, layer_name: str) -> None:
         attn = forward_context.no_compile_layers[layer_name]
@@ -228,9 +307,12 @@ class GSA(UcmSparseBase):
                 self.gsa_stats[req_id] = GSAReqStat(
                     req_id, self.max_block_len * self.topk_kpre_manger.cache_map[req_id], self.block_size,
                     self.threshold)
-            self.gsa_stats[req_id].update(n_tok, requests[req_id], input_batch.req_id_to_index[req_id])
+            self.gsa_stats[req_id].update(n_tok, requests[req_id], input_batch.req_id_to_index[req_id],
+                                          (self.min_topk, self.max_topk, self.topk_ratio) if self.ptopk_prefetch else None)
         self.gsa_metadata = meta
         self._sparse_metadata = meta
+        if self.ptopk_prefetch:
+            self._init_sparse_local_kv(scheduler_output, requests)
 
         batch = len(scheduler_output.num_scheduled_tokens)
         by_index: List[Optional[GSAReqStat]] = [None] * batch
@@ -305,6 +387,8 @@ class GSA(UcmSparseBase):
                                     self.model_input["block_tables"].data_ptr())
 
     def execute_finished(self) -> None:
+        if self.ptopk_prefetch:
+            self._gsa_sparse_local_kv()
         self.step_count += 1
 
     # ------------------------------------------------------------------ per-layer hooks
@@ -371,6 +455,16 @@ class GSA(UcmSparseBase):
         pass
 
     def estimate_num_slots_sparsed(self, request) -> int:
-        # blocks are not freed by this plugin (the reference returns INVALID_SLOT too
-        # unless its prefetch path is compiled in, gsa.py:891-912)
-        return INVALID_SLOT
+        """Token slots of a sparsified request (gsa.py:891-912): the blocks decoded so far plus max_topk + 1 sparse
+        blocks, minus the unused tail of the last block.  INVALID_SLOT unless prefetch mode is on (the reference's
+        PTOPK_PREFETCH_ENABLE is off as shipped), during prefill and for prompts below the threshold."""
+        if not self.ptopk_prefetch or request.num_output_tokens == 0 or request.num_prompt_tokens <= self.threshold:
+            return INVALID_SLOT
+        bs = self.block_size
+        num_prompt_blocks = math.ceil(request.num_prompt_tokens / bs)
+        num_all_blocks = math.ceil(request.num_tokens / bs)
+        topk_len = compute_topk_len(num_prompt_blocks, self.min_topk, self.max_topk, self.topk_ratio)
+        prefetch_len = 0 if topk_len > self.max_topk else self.max_topk - topk_len + 1
+        num_sparse_blocks = num_all_blocks - num_prompt_blocks + topk_len + prefetch_len
+        flaw = request.num_tokens % bs
+        return num_sparse_blocks * bs - (bs - flaw if flaw else 0)
