@@ -30,7 +30,22 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-KVSTAR_TRAFFIC = 4088600000   # HBM bytes per step of the KVStar leg at its defaults (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE)
+
+
+def measured_traffic(role: str, kernel: str, default_workload: bool):
+    """HBM bytes per launch that rocprofv3 --pmc measured for `kernel` on the default workload
+    (profiles/traffic.json), or None for any other workload.  The file names the kernel each figure belongs to:
+    a figure is never quoted for a kernel other than the one this run launched."""
+    if not default_workload:
+        return None
+    with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+        entry = json.load(f)["entries"].get(role)
+    if entry is None:
+        return None
+    if entry["kernel"] != kernel:
+        raise SystemExit(f"profiles/traffic.json holds the traffic of {entry['kernel']} for '{role}', but this run launched "
+                         f"{kernel}: re-measure before quoting it")
+    return int(entry["hbm_bytes_per_launch"])
 
 N_REQ, N_LAYERS, HQ, HKV, D, BS = 16, 32, 32, 8, 128, 128
 ROW = HKV * D
@@ -349,7 +364,8 @@ def main():
             "encode_read_GBps": round(gbs(key_bytes, enc_ms), 1),
             "roofline": {"kernel": "hash_encode_blocks_kernel", "bound": "hbm", "achieved": round(gbs(enc_bytes, enc_ms), 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs(enc_bytes, enc_ms) / HBM_PEAK_GBS, 4),
-                         "traffic": 52266000000 if default_hash else None, "algorithmic_bytes": enc_bytes,
+                         "traffic": measured_traffic("hash_encode", "hash_encode_blocks_kernel", default_hash),
+                         "algorithmic_bytes": enc_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * h_rows * BS * HKV * 128 * 128 / (enc_ms * 1e-3) / 1e12, 1)},
             "encode_summaries_only_ms": round(enc_sum_ms, 3),
             "decode_step_us": {"query_codes": round(q_ms * 1e3, 1), "score": round(sc_ms * 1e3, 1),
@@ -376,16 +392,14 @@ def main():
         flat = torch.empty((HKV, n_layers * rows, kd_pad // 8, km, 8), dtype=torch.float16, device=dev)
         ktab = flat.view(HKV, n_layers, rows, kd_pad // 8, km, 8).permute(1, 0, 2, 3, 4, 5)
         ev0, ev1 = ev(), ev()
+        ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge, pruned=kpr)   # channel lists per layer
+        torch.cuda.synchronize()
         ev0.record()
-        if kpr is None:
-            ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge)
-        else:
-            for l_ in range(n_layers):                                  # a channel list per layer: one launch per layer
-                ops.kvstar_block_repre(ops.LayerPointers([caches[l_]]), table, slots, ktab[l_ : l_ + 1], BS, HKV, D, nb, merge,
-                                       pruned=kpr[l_])
+        ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge, pruned=kpr)   # one launch for all layers
         ev1.record()
         torch.cuda.synchronize()
         krep_ms = ev0.elapsed_time(ev1)
+        krep_bytes = n_layers * rows * (BLOCK_BYTES + HKV * km * kd_pad * 2)
         n_tasks = n_layers * N_REQ
         k_off = (seg_off_h[None, :].astype(np.int64) + (np.arange(n_layers, dtype=np.int64) * rows)[:, None]).reshape(-1)
         k_len = np.tile(lens, n_layers)
@@ -435,10 +449,13 @@ def main():
             "workload": f"{n_tasks} tasks (layer x request), {kx} query tokens x {HQ} heads, {rows} blocks x {km} sub-block "
                         f"representatives per layer, {kdp} of {D} channels, fp16",
             "block_repre_ms": round(krep_ms, 3),
+            "block_repre_GBps": round(gbs(krep_bytes, krep_ms), 1),
+            "block_repre_frac": round(gbs(krep_bytes, krep_ms) / HBM_PEAK_GBS, 4),
             "us_per_step": round(kv_ms * 1e3, 1),
             "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select)", "bound": "hbm",
                          "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4), "traffic": KVSTAR_TRAFFIC if kv_default else None,
+                         "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4),
+                         "traffic": measured_traffic("kvstar_votes", "kvstar_score_kernel", kv_default),
                          "algorithmic_bytes": kv_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * kd_pad / (kv_ms * 1e-3) / 1e12, 1)},
             "checked": kv_checked,
@@ -532,7 +549,8 @@ def main():
             t_acc += time.perf_counter() - s0
             reps += 1
         cpu_retr_us = t_acc / reps * 1e6
-        # gather sample: a few layers of the cache on the host, memcpy of the selected blocks, scaled to all layers
+        # gather sample: a few layers of the cache on the host, the selected blocks copied by the same host threads as
+        # the retrieval part, extrapolated to all layers
         g_layers = min(2, n_layers)
         host_layers = [caches[l].view(torch.uint8).reshape(-1).cpu().numpy() for l in range(g_layers)]
         g_total = int((region_h.astype(np.int64) * g_layers * 2).sum())
@@ -556,15 +574,17 @@ def main():
             "gather_us": round(cpu_gather_us, 1),
             "sample": (f"retrieval: {reps} full steps (all {n_layers} layers x {N_REQ} requests, fp32 representatives "
                        f"resident in host DRAM, {threads} OpenMP threads over blocks, requests and layers serial); "
-                       f"gather: {greps} passes over {g_layers} of {n_layers} layers with one memcpy thread, scaled x{n_layers // g_layers}"),
+                       f"gather: EXTRAPOLATED from {g_layers} of {n_layers} layers ({greps} passes, memcpy of the selected "
+                       f"blocks on {threads} OpenMP threads, time x{n_layers // g_layers})"),
             "host_cpus": os.cpu_count(),
         }
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly this workload
     # (profiles/bench_config2_kernels.md); other workloads have no measurement
     default_workload = n_layers == N_LAYERS and args.seed == 2024
-    traffic_gather = 10201100000 if default_workload else None
-    traffic_score = {"f32": 535400000, "bf16": 272000000}.get(args.repre_dtype) if default_workload else None
+    score_kernel_name = "score_kernel_bf16" if args.repre_dtype == "bf16" else "score_kernel"   # what ucm_score_blocks launches
+    traffic_gather = measured_traffic("gather", "kv_gather_selected_kernel", default_workload)
+    traffic_score = measured_traffic("score_" + args.repre_dtype, score_kernel_name, default_workload)
 
     out = {
         "metric": "us per decode step (32-layer retrieval+gather)",
@@ -604,7 +624,7 @@ def main():
             "algorithmic_bytes": gather_bytes,
         },
         "roofline_score": {
-            "kernel": "score_kernel",
+            "kernel": score_kernel_name,
             "bound": "hbm",
             "achieved": round(gbs(score_bytes, score_ms), 1),
             "peak": HBM_PEAK_GBS,

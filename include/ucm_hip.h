@@ -113,6 +113,9 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *              value, sizes the grid); total_blocks = sum of seg_len when the
  *              host knows it (a tighter grid), else 0.
  *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x].
+ *   tile_blocks  blocks scored per workgroup; 0 sizes a workgroup's share to 128 KiB
+ *              of representatives (a value for benchmarks and tests, not part of
+ *              the reference interface).
  * head_dim must be 32, 64, 96, 128, 192 or 256, kv_heads one of 1, 2, 4, 8, 16 and
  * kv_heads*head_dim at most 2048.
  */
@@ -120,18 +123,7 @@ int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const i
                      int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
                      const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
                      int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
-                     int64_t scores_layer_stride, ucm_stream_t stream);
-
-/* Tuning knob for benchmarks: blocks scored per workgroup by ucm_score_blocks;
- * 0 (the default) sizes a workgroup's share to 128 KiB of representatives.
- * Not part of the reference interface. */
-int ucm_set_score_tile(int tile_blocks);
-
-/* Tuning knob for benchmarks and tests: number of workgroups
- * ucm_hash_encode_blocks launches over all layers; each of their waves steps
- * through the list of blocks.  0 restores the default (4096).  Not part of the
- * reference interface. */
-int ucm_set_hash_encode_groups(int workgroups);
+                     int64_t scores_layer_stride, int tile_blocks, ucm_stream_t stream);
 
 /*
  * Per-request block selection with forced windows, all layers in one launch -
@@ -336,6 +328,8 @@ int ucm_prefetch_plan(const int32_t* map_block, const int32_t* map_len, int32_t*
  *                each bit over the block's tokens, layer stride in ELEMENTS
  *   block_codes  dev u8 [n_layers][rows][kv_heads][16]: majority vote of each bit
  *                (colsum > 0; an exact tie gives 0), layer stride in BYTES
+ *   workgroups   persistent workgroups launched over all layers, each of whose
+ *                waves steps through the list of blocks; 0 = the default (4096)
  * ucm_hash_encode_queries: per (layer, request) the codes of all query heads
  * (q_codes u8 [L][n_req][q_heads][16]), their +-1 sum over heads (q_sum int16
  * [L][n_req][128]) and the code of every kv head's group-mean query
@@ -361,7 +355,7 @@ int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers, int num_bl
                            int kv_heads, int head_dim, const void* w_bf16, int bits, int rows,
                            uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
                            int64_t colsum_layer_stride, uint8_t* block_codes,
-                           int64_t block_codes_layer_stride, ucm_stream_t stream);
+                           int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream);
 int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows,
                             int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
                             const void* w_bf16, int bits, uint8_t* q_codes, int16_t* q_sum,
@@ -385,7 +379,10 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  * as fp16 (its .to(torch.float16), :495-497).
  *   pruned   dev int32[kv_heads][d_pruned]: channel of every kept dim (the
  *            reference's d_pruned_index, :288-304), or NULL when d_pruned ==
- *            head_dim
+ *            head_dim; layer l reads the lists pruned_layer_stride elements
+ *            after layer l-1's (the reference picks the channels per layer
+ *            state; 0 = one set of lists for every layer), so one launch
+ *            covers all layers
  *   repre    dev fp16, [n_layers][kv_heads][repre_rows][d_pad/8][M][8]: kv
  *            head outermost, and inside a block the 16-byte pieces (8
  *            channels) of its M sub-blocks side by side; d_pad >= d_pruned, a
@@ -418,33 +415,34 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  */
 int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
                            const int32_t* block_ids, const int32_t* slots, int n, int block_size,
-                           int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
-                           int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
-                           int64_t repre_head_stride, ucm_stream_t stream);
-/* Tuning knob for benchmarks and tests.  ucm_kvstar_votes has two paths: one
- * workgroup per (task, kv head) that keeps the task's per-(block, query row)
- * sums in LDS and stores only the head's share of the votes (taken when there
- * are at least 128 such pairs and the plane fits 159 KiB), and a workspace
- * path that may cut a task into chunks.  tiles > 0: the workspace path with
- * that many 32-sub-block tiles per wave (four waves per workgroup); -1: the
- * in-LDS path whenever the plane fits; 0: automatic.  Not part of the
- * reference interface. */
-int ucm_set_kvstar_tiles_per_wave(int tiles);
-/* Floats of scratch ucm_kvstar_votes[_tables] needs for a call of this shape
- * (rows_per_head = n_tokens * q_heads/kv_heads); the in-LDS path only needs
- * room for the kv heads' vote shares.  Ask after ucm_set_kvstar_tiles_per_wave,
- * which changes the path; the votes calls take the sizes of the two areas
- * (ws_max_floats, ws_part_floats) and fail with UCM_EINVAL when the path they
- * would take needs more. */
+                           int kv_heads, int head_dim, int merge, const int32_t* pruned,
+                           int64_t pruned_layer_stride, int d_pruned, int d_pad, void* repre_f16,
+                           int repre_rows, int64_t repre_layer_stride, int64_t repre_head_stride,
+                           ucm_stream_t stream);
+/* ucm_kvstar_votes has two paths: one workgroup per (task, kv head) that keeps
+ * the task's per-(block, query row) sums in LDS and stores only the head's
+ * share of the votes (taken when there are at least 128 such pairs and the
+ * plane fits 159 KiB), and a workspace path that may cut a task into chunks.
+ * tiles_per_wave > 0: the workspace path with that many 32-sub-block tiles per
+ * wave (four waves per workgroup); -1: the in-LDS path whenever the plane
+ * fits; 0: automatic (what callers other than benchmarks and tests pass).
+ *
+ * ucm_kvstar_workspace_floats: floats of scratch ucm_kvstar_votes[_tables]
+ * needs for a call of this shape and tiles_per_wave (rows_per_head = n_tokens *
+ * q_heads/kv_heads); the in-LDS path only needs room for the kv heads' vote
+ * shares.  The votes calls take the sizes of the two areas (ws_max_floats,
+ * ws_part_floats) and fail with UCM_EINVAL when the path they would take needs
+ * more. */
 int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks,
-                                int sub_blocks, int d_pad, int64_t* max_floats, int64_t* part_floats);
+                                int sub_blocks, int d_pad, int tiles_per_wave, int64_t* max_floats,
+                                int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                      const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
                      int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len,
                      int n_tasks, int max_blocks,
                      int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                      int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
-                     ucm_stream_t stream);
+                     int tiles_per_wave, ucm_stream_t stream);
 /* The same for tasks whose representatives do not share one table (the
  * reference keeps one blk_repre tensor per request and layer,
  * ucm/sparse/kvstar/multistep.py:191,483-501): task t's table starts at
@@ -458,7 +456,7 @@ int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_token
                             const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
                             int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                             int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
-                            ucm_stream_t stream);
+                            int tiles_per_wave, ucm_stream_t stream);
 
 /*
  * The selection step of KVStar::Execute on the votes of n_tasks tasks
@@ -515,18 +513,28 @@ int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t 
  *                               `count` bytes, device dArr[i] <- host hArr[i].
  * ucm_device_d2h_batch_sync     D2HBatchSync (:196-211): host hArr[i] <- device
  *                               dArr[i].  Both arrays are HOST arrays of
- *                               addresses (as in the reference); the host
- *                               addresses must be pinned memory (this object's
- *                               buffers are).  One launch of the ucm_copy_batch
- *                               kernel on the object's stream, then a wait; if
- *                               `count` or an address is not a multiple of 16,
- *                               one runtime copy per pair instead.
+ *                               addresses (as in the reference).  One launch of
+ *                               the ucm_copy_batch kernel on the object's
+ *                               stream, then a wait, when every address is
+ *                               memory a kernel can touch (device memory,
+ *                               pinned host memory such as this object's
+ *                               buffers) and `count` and the addresses are
+ *                               multiples of 16; otherwise (pageable host
+ *                               memory included) one runtime copy per pair.
  * ucm_device_stream             the object's stream, for callers that order
  *                               their own kernels against the copies.
  *
  * Calls on one object may come from several threads; batched copies on one
  * object run one at a time.
  */
+/* 1 if a kernel of this library may dereference [address, address + count):
+ * device memory, pinned or registered host memory, managed memory; 0 for
+ * pageable host memory, unknown addresses and NULL.  Callers that pass raw
+ * addresses to ucm_copy_batch (as the store's fetch_data / dump_data do,
+ * ucm/store/ucmstore.py:127-167) check them with it: a kernel that touches
+ * pageable memory faults. */
+int ucm_kernel_can_access(const void* address, size_t count);
+
 typedef struct ucm_device ucm_device_t;
 typedef void (*ucm_device_callback_t)(int ok, void* user);
 int ucm_device_create(int device_id, size_t buffer_size, size_t buffer_number, ucm_device_t** out);

@@ -481,10 +481,13 @@ ORC_API void orc_kv_gather_selected(const uint8_t* const* layers, uint32_t n_lay
                                     const int64_t* dst_off, const int32_t* region_k,
                                     uint8_t* staging)
 {
+    /* every (layer, request, K|V) writes a region of its own, so the copies can run on all host threads (the
+     * timed CPU baseline uses as many as its retrieval part); the result does not depend on the schedule */
+#pragma omp parallel for collapse(3) schedule(dynamic, 1)
     for (uint32_t l = 0; l < n_layers; ++l) {
         for (uint32_t r = 0; r < n_req; ++r) {
-            const int32_t c = count[(size_t)l * n_req + r];
             for (uint32_t kv = 0; kv < 2; ++kv) {
+                const int32_t c = count[(size_t)l * n_req + r];
                 for (int32_t j = 0; j < c; ++j) {
                     const int32_t id = phys[((size_t)l * n_req + r) * phys_stride + j];
                     const uint8_t* s = layers[l] + kv * kv_stride + (size_t)id * block_bytes;

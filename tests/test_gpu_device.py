@@ -143,6 +143,38 @@ def test_batch_copies_of_odd_sizes_and_addresses(device):
         assert np.array_equal(host_array(back)[i * 1024 + 5 : i * 1024 + 5 + count], data[i * 1024 + 1 : i * 1024 + 1 + count]), i
 
 
+def test_batch_copies_with_pageable_host_memory(device):
+    """Aligned addresses in ordinary (pageable) host memory: no kernel may touch them, so the call classifies every
+    address on the host and moves such a batch with one runtime copy per pair - same bytes, no launch over memory the
+    device cannot reach.  Blocks of the hipBlockStore path (fetch_data / dump_data with raw addresses) go the same way."""
+    rng = np.random.default_rng(10)
+    number, count = 6, 4096
+    raw = np.zeros(number * count + 64, np.uint8)
+    start = (-raw.ctypes.data) % 16                                         # a 16-byte aligned window of a numpy array
+    host = raw[start : start + number * count]
+    assert host.ctypes.data % 16 == 0
+    host[:] = rng.integers(0, 256, number * count, dtype=np.uint8)
+    pool = torch.zeros(number, count, dtype=torch.uint8, device="cuda:0")
+    torch.cuda.synchronize()
+    d_arr = [pool.data_ptr() + i * count for i in range(number)]
+    device.H2DBatchSync(d_arr, [host.ctypes.data + i * count for i in range(number)], count)
+    assert np.array_equal(pool.cpu().numpy().reshape(-1), host)
+    back_raw = np.zeros(number * count + 64, np.uint8)
+    b0 = (-back_raw.ctypes.data) % 16
+    back = back_raw[b0 : b0 + number * count]
+    device.D2HBatchSync([back.ctypes.data + i * count for i in range(number)], d_arr, count)
+    assert np.array_equal(back, host)
+    # a mix: one pinned buffer among pageable ones still works (the whole batch takes the per-pair path)
+    pinned = device.GetBuffer(count)
+    host_array(pinned)[:] = 9
+    mixed = [pinned.ptr] + [host.ctypes.data + i * count for i in range(1, number)]
+    device.H2DBatchSync(d_arr, mixed, count)
+    got = pool.cpu().numpy()
+    assert (got[0] == 9).all() and np.array_equal(got[1:].reshape(-1), host[count:])
+    with pytest.raises(Exception):
+        device.H2DBatchSync(d_arr, [0] + mixed[1:], count)                  # a null address is refused on the host
+
+
 def test_device_stream_orders_library_kernels(device):
     """A kernel of the library launched on the device's stream is ordered with its copies."""
     from ucm_amd import _lib

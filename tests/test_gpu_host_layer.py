@@ -426,6 +426,13 @@ def test_hip_block_store_round_trip(ucm, dev):
             rest = [b for b in range(nb) if b not in dst]
             assert not fresh[l][kv][rest].any()
     assert store.wait(store.load(["unknown"], [0], [fresh[0][0][0]])) == FAILURE
+    # raw addresses (fetch_data / dump_data): device memory passes, pageable host memory is refused before any launch
+    raw = torch.zeros(slice_bytes, dtype=torch.uint8, device=dev)
+    assert store.wait(store.fetch_data([hashes[0]], [0], [raw.data_ptr()], [slice_bytes])) == SUCCESS
+    assert torch.equal(raw, caches[0][0][ids[0]].reshape(-1).view(torch.uint8))
+    pageable = np.zeros(slice_bytes + 64, np.uint8)
+    with pytest.raises(ValueError, match="not device or pinned"):
+        store.fetch_data([hashes[0]], [0], [pageable.ctypes.data + (-pageable.ctypes.data) % 16], [slice_bytes])
     # a store in pinned host memory behaves the same
     host = UcmHipBlockStore({"kv_block_size": slice_bytes, "max_cache_size": 4 * slice_bytes, "device": "pinned"})
     t = host.dump(["a"], [0], [caches[0][0][2]])

@@ -68,6 +68,33 @@ def test_kvstar_block_repre(ucm, dev, merge, hkv, d, bs):
     assert torch.allclose(mine.float(), t.float(), rtol=2 ** -7, atol=1e-6)
 
 
+@pytest.mark.parametrize("merge", [2, 16, 3])      # the persistent kernel, and the one for other sub-block sizes (16 and 3)
+def test_kvstar_block_repre_channel_lists_per_layer(ucm, dev, merge):
+    """One launch over all layers with a different set of kept channels in each (the reference picks them per layer
+    state, multistep.py:284-304): every layer against the oracle run with that layer's lists."""
+    from ucm_amd import ops
+
+    n_layers, nb, rows, hkv, d, bs = 5, 13, 16, 4, 128, 48
+    dp, M = 37, bs // merge
+    d_pad = (dp + 15) // 16 * 16
+    caches_h = [synth.normal_bf16_bits(1500 + l, (nb, bs, hkv, d)) for l in range(n_layers)]
+    caches = [torch.from_numpy(c.view(np.int16)).to(dev).view(torch.bfloat16) for c in caches_h]
+    ids = synth.permutation(1510, nb)[:10].astype(np.int32)
+    slots = synth.permutation(1511, rows)[:10].astype(np.int32)
+    pruned = np.stack([[synth.permutation(1520 + 10 * l + h, d)[:dp] for h in range(hkv)] for l in range(n_layers)]).astype(np.int32)
+    repre = ops.kvstar_table(n_layers, hkv, rows, M, d_pad, dev).fill_(3.0)
+    ops.kvstar_block_repre(ops.LayerPointers(caches), torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs,
+                           hkv, d, nb, merge, pruned=torch.from_numpy(pruned).to(dev))
+    got = ops.kvstar_table_to_reference(repre).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    for l in range(n_layers):
+        want = np.full((rows, M, hkv, d_pad), np.float16(3.0).view(np.uint16), np.uint16)
+        O.kvstar_block_repre(caches_h[l], ids, slots, merge, want, pruned=pruned[l])
+        assert np.array_equal(got[l], want), l
+    with pytest.raises(ValueError):
+        ops.kvstar_block_repre(ops.LayerPointers(caches), torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre,
+                               bs, hkv, d, nb, merge, pruned=torch.from_numpy(pruned[:2]).to(dev))
+
+
 def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None, pruned_sel=None, d_pruned=None):
     """q_bits_list: per task uint16 [x, hq, d]; repre_bits uint16 [rows, M, hkv, d_pad]; tasks own consecutive row ranges."""
     lens = np.asarray(lens, np.int32)

@@ -18,14 +18,11 @@ SIGNATURES = {
     "ucm_version": [],
     "ucm_last_error": [],
     "ucm_block_mean": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i64, _i, _p],
-    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _p],
-    "ucm_set_score_tile": [_i],
-    "ucm_set_hash_encode_groups": [_i],
-    "ucm_kvstar_block_repre": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _i, _p, _i, _i, _p, _i, _i64, _i64, _p],
-    "ucm_set_kvstar_tiles_per_wave": [_i],
-    "ucm_kvstar_workspace_floats": [_i, _i, _i, _i, _i, _i, _p, _p],
-    "ucm_kvstar_votes": [_p, _p, _i, _i, _i, _p, _p, _p, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _p],
-    "ucm_kvstar_votes_tables": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _p],
+    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
+    "ucm_kvstar_block_repre": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _i, _p, _i64, _i, _i, _p, _i, _i64, _i64, _p],
+    "ucm_kvstar_workspace_floats": [_i, _i, _i, _i, _i, _i, _i, _p, _p],
+    "ucm_kvstar_votes": [_p, _p, _i, _i, _i, _p, _p, _p, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
+    "ucm_kvstar_votes_tables": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
     "ucm_kvstar_topk": [_p, _p, _p, _p, _i, _i, _p, _i, _p, _p],
     "ucm_topk_windows": [_p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
     "ucm_esa_retrieve": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _p, _i, _p],
@@ -35,10 +32,11 @@ SIGNATURES = {
     "ucm_kv_load_planned": [_p, _i, _sz, _sz, _i, _p, _i64, _sz, _i, _p, _i, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _p],
     "ucm_prefetch_plan": [_p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p],
     "ucm_delta_plan": [_p, _p, _p, _i, _i, _i, _p, _i, _p, _p, _p, _p],
-    "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _p],
+    "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _i, _p],
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_score_blocks": [_i, _p, _p, _p, _i64, _p, _i64, _p, _p, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
     "ucm_copy_batch": [_p, _p, _sz, _sz, _p],
+    "ucm_kernel_can_access": [_p, _sz],
     "ucm_device_create": [_i, _sz, _sz, _p],
     "ucm_device_destroy": [_p],
     "ucm_device_get_buffer": [_p, _sz],

@@ -8,6 +8,7 @@
 // space, so the kernel reads or writes them directly).
 #include <mutex>
 #include <new>
+#include <utility>
 #include <vector>
 
 #include "common.h"
@@ -37,6 +38,39 @@ void trampoline(hipStream_t, hipError_t status, void* data)
     delete c;
 }
 
+// Can a kernel dereference this address?  The device's own pinned pool: yes.  Anything else is asked of the
+// runtime: device memory (the answer covers its whole allocation, remembered in `known` so that the many blocks of
+// one cache tensor cost one query), pinned or registered host memory and managed memory are mapped into the
+// device's address space; pageable host memory is not, and a kernel touching it would fault.
+bool kernel_can_touch(const ucm_device* dev, const void* p, size_t count, std::vector<std::pair<uintptr_t, uintptr_t>>& known)
+{
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if (dev && dev->pool) {
+        const uintptr_t lo = reinterpret_cast<uintptr_t>(dev->pool), hi = lo + dev->buffer_size * dev->buffer_number;
+        if (a >= lo && a + count <= hi) { return true; }
+    }
+    for (const auto& r : known) {
+        if (a >= r.first && a + count <= r.second) { return true; }
+    }
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();              // an unknown address is an answer, not a failure of this call
+        return false;
+    }
+    if (attr.type == hipMemoryTypeDevice) {
+        hipDeviceptr_t base = nullptr;
+        size_t size = 0;
+        if (hipMemGetAddressRange(&base, &size, const_cast<void*>(p)) == hipSuccess && size) {
+            const uintptr_t lo = reinterpret_cast<uintptr_t>(base);
+            known.emplace_back(lo, lo + size);
+            return a + count <= lo + size;
+        }
+        (void)hipGetLastError();
+        return true;
+    }
+    return attr.type == hipMemoryTypeHost || attr.type == hipMemoryTypeManaged;
+}
+
 int batch(ucm_device* dev, void* const* dst_host_array, const void* const* src_host_array, size_t number, size_t count,
           const char* what)
 {
@@ -44,11 +78,15 @@ int batch(ucm_device* dev, void* const* dst_host_array, const void* const* src_h
     if (number == 0 || count == 0) { return UCM_OK; }
     if (int rc = ucm::check_hip(hipSetDevice(dev->device_id), what)) { return rc; }
     bool vector_ok = count % 16 == 0;
+    std::vector<std::pair<uintptr_t, uintptr_t>> known;
     for (size_t i = 0; vector_ok && i < number; ++i) {
-        vector_ok = ucm::aligned16(dst_host_array[i]) && ucm::aligned16(src_host_array[i]);
+        UCM_REQUIRE(dst_host_array[i] && src_host_array[i], "%s: null address in entry %zu", what, i);
+        vector_ok = ucm::aligned16(dst_host_array[i]) && ucm::aligned16(src_host_array[i]) &&
+                    kernel_can_touch(dev, dst_host_array[i], count, known) && kernel_can_touch(dev, src_host_array[i], count, known);
     }
     if (!vector_ok) {
-        // sizes or addresses the 16-byte copy kernel cannot take: one runtime copy per pair, same stream, same wait
+        // sizes or addresses the 16-byte copy kernel cannot take (odd sizes, unaligned addresses, pageable host
+        // memory, which no kernel may touch): one runtime copy per pair, same stream, same wait
         for (size_t i = 0; i < number; ++i) {
             if (int rc = ucm::check_hip(hipMemcpyAsync(dst_host_array[i], src_host_array[i], count, hipMemcpyDefault, dev->stream), what)) {
                 return rc;
@@ -78,6 +116,13 @@ int batch(ucm_device* dev, void* const* dst_host_array, const void* const* src_h
 }
 
 }  // namespace
+
+extern "C" int ucm_kernel_can_access(const void* address, size_t count)
+{
+    if (!address) { return 0; }
+    std::vector<std::pair<uintptr_t, uintptr_t>> known;
+    return kernel_can_touch(nullptr, address, count, known) ? 1 : 0;
+}
 
 extern "C" int ucm_device_create(int device_id, size_t buffer_size, size_t buffer_number, ucm_device_t** out)
 {

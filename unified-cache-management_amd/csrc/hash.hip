@@ -832,27 +832,18 @@ __global__ __launch_bounds__(256) void hash_code_score_kernel(
     }
 }
 
-int g_encode_groups = 4096;
-
 }  // namespace
-
-// Tuning knob for benchmarks and tests: workgroups launched by
-// ucm_hash_encode_blocks over all layers (0 restores the default, 4096).
-extern "C" int ucm_set_hash_encode_groups(int workgroups)
-{
-    UCM_REQUIRE(workgroups >= 0 && workgroups <= (1 << 20), "ucm_set_hash_encode_groups: %d", workgroups);
-    g_encode_groups = workgroups > 0 ? workgroups : 4096;
-    return UCM_OK;
-}
 
 extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers, int num_blocks,
                                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
                                       int kv_heads, int head_dim, const void* w_bf16, int bits, int rows,
                                       uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
                                       int64_t colsum_layer_stride, uint8_t* block_codes,
-                                      int64_t block_codes_layer_stride, ucm_stream_t stream)
+                                      int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_hash_encode_blocks: n=%d", n);
+    UCM_REQUIRE(workgroups >= 0 && workgroups <= (1 << 20), "ucm_hash_encode_blocks: workgroups=%d", workgroups);
+    const int encode_groups = workgroups > 0 ? workgroups : 4096;
     if (n == 0) { return UCM_OK; }
     UCM_REQUIRE(k_layers && w_bf16 && colsum && block_codes, "ucm_hash_encode_blocks: null pointer");
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535 && num_blocks > 0 && rows > 0 && block_size > 0,
@@ -868,7 +859,7 @@ extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers,
                 "ucm_hash_encode_blocks: code strides are in bytes and must be multiples of 4");
     // persistent workgroups: about 4096 of them over all layers, each wave stepping through the list
     const int groups = (n + kWaves - 1) / kWaves;
-    const int gx = std::min(groups, std::max(1, (g_encode_groups + n_layers - 1) / n_layers));
+    const int gx = std::min(groups, std::max(1, (encode_groups + n_layers - 1) / n_layers));
 #define UCM_HASH_ENCODE_ARGS dim3(gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream), k_layers, block_ids, slots, \
         static_cast<unsigned>(num_blocks), static_cast<unsigned>(n), static_cast<unsigned>(rows),                        \
         static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16),  \

@@ -125,8 +125,9 @@ template <int kMerge>
 __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows, unsigned block_size,
-    unsigned kv_heads, unsigned head_dim, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
-    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
+    unsigned kv_heads, unsigned head_dim, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride,
+    unsigned d_pruned, unsigned d_pad, unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride,
+    unsigned m_chunk)
 {
     static_assert(kMerge == 1 || kMerge == 2 || kMerge == 4 || kMerge == 8, "tokens per sub-block");
     extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]: the 16 bytes of padding
@@ -138,8 +139,9 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const unsigned short* layer = static_cast<const unsigned short*>(k_layers[blockIdx.y]);
     // the channel lists, read once: a load from memory per output piece would queue behind the key stream
     int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
-    if (pruned) {
-        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = pruned[e]; }
+    if (pruned) {   // this layer's lists (a stride of 0: one set of lists for every layer)
+        const int32_t* mine = pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride;
+        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = mine[e]; }
     }
 
     struct Unit {
@@ -239,7 +241,8 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
 __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
-    unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, unsigned d_pruned, unsigned d_pad,
+    unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride, unsigned d_pruned,
+    unsigned d_pad,
     unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]
@@ -254,8 +257,9 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const unsigned pieces = d_pad / 8;
     unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<size_t>(slot) * M * d_pad;
     int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
-    if (pruned) {
-        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = pruned[e]; }
+    if (pruned) {   // this layer's lists (a stride of 0: one set of lists for every layer)
+        const int32_t* mine = pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride;
+        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = mine[e]; }
     }
     for (unsigned m0 = 0; m0 < M; m0 += m_chunk) {       // m_chunk sub-blocks at a time: what fits LDS
         const unsigned mc = min(m_chunk, M - m0);
@@ -842,23 +846,12 @@ __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
     if (live && l32 == 0) { votes[seg_off[task] + b] = v; }
 }
 
-int g_tiles_per_wave = 0;
-
-
 }  // namespace
-
-// Tuning knob for benchmarks and tests: n > 0 takes the workspace path with n 32-sub-block tiles per wave
-// of a score workgroup, -1 the in-LDS path whenever a task's plane fits, 0 chooses automatically.
-extern "C" int ucm_set_kvstar_tiles_per_wave(int tiles)
-{
-    UCM_REQUIRE(tiles >= -1, "ucm_set_kvstar_tiles_per_wave: %d", tiles);
-    g_tiles_per_wave = tiles;
-    return UCM_OK;
-}
 
 extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
                                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
-                                      int kv_heads, int head_dim, int merge, const int32_t* pruned, int d_pruned,
+                                      int kv_heads, int head_dim, int merge, const int32_t* pruned,
+                                      int64_t pruned_layer_stride, int d_pruned,
                                       int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
                                       int64_t repre_head_stride, ucm_stream_t stream)
 {
@@ -872,6 +865,8 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_REQUIRE(d_pruned > 0 && d_pruned <= head_dim && d_pad >= d_pruned, "ucm_kvstar_block_repre: d_pruned=%d d_pad=%d",
                 d_pruned, d_pad);
     UCM_REQUIRE(pruned || d_pruned == head_dim, "ucm_kvstar_block_repre: d_pruned < head_dim needs the channel list");
+    UCM_REQUIRE(pruned_layer_stride == 0 || pruned_layer_stride >= static_cast<int64_t>(kv_heads) * d_pruned,
+                "ucm_kvstar_block_repre: pruned_layer_stride=%lld", static_cast<long long>(pruned_layer_stride));
     const int M = block_size / merge;
     UCM_REQUIRE(repre_head_stride >= static_cast<int64_t>(repre_rows) * M * d_pad,
                 "ucm_kvstar_block_repre: repre_head_stride=%lld smaller than one head's plane",
@@ -899,7 +894,7 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                            block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(n),            \
                            static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),                     \
                            static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), pruned,                 \
-                           static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),                            \
+                           pruned_layer_stride, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),       \
                            static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk); \
     } while (0)
     switch (merge) {
@@ -916,7 +911,8 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
         hipLaunchKernelGGL(kvstar_repre_any_kernel, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, hs,
                            k_layers, block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(repre_rows),
                            static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim),
-                           static_cast<unsigned>(merge), pruned, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),
+                           static_cast<unsigned>(merge), pruned, pruned_layer_stride, static_cast<unsigned>(d_pruned),
+                           static_cast<unsigned>(d_pad),
                            static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk);
         break;
     }
@@ -940,7 +936,7 @@ struct VotePlan {
     bool use_lds;
 };
 
-VotePlan plan_votes(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks, int d_pad)
+VotePlan plan_votes(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks, int d_pad, int tiles_per_wave)
 {
     VotePlan p;
     p.max_tiles = static_cast<unsigned>(std::max<int64_t>(padded_tiles(static_cast<int64_t>(max_blocks) * sub_blocks), 4));
@@ -950,15 +946,15 @@ VotePlan plan_votes(int n_tasks, int kv_heads, int rows_per_head, int max_blocks
     p.span_tiles = 8u / p.steps;                               // tiles a wave moves at a time
     // One workgroup per (task, kv head) with the task's plane in LDS, when there are enough such workgroups to
     // fill the device and the plane fits; otherwise the workspace path, which may cut a task into chunks.
-    // ucm_set_kvstar_tiles_per_wave(n > 0) forces the workspace path.
+    // tiles_per_wave > 0 forces the workspace path, -1 the in-LDS path whenever the plane fits.
     p.plane_offset = rows_per_head > 32 ? p.q_bytes : 0u;
     const unsigned entry_tiles = static_cast<unsigned>(sub_blocks) <= kTileSub
                                      ? 1u : std::min<unsigned>(sub_blocks, p.span_tiles * kTileSub) / kTileSub;
     const size_t plane_entries = static_cast<unsigned>(sub_blocks) < kTileSub
                                      ? static_cast<size_t>(p.max_tiles) * (kTileSub / sub_blocks) : p.max_tiles / entry_tiles;
     p.lds_plane = p.plane_offset + plane_entries * p.row_pad * 4 + 2 * kWaves * p.row_pad * 4;
-    p.use_lds = g_tiles_per_wave <= 0 && p.lds_plane <= kLdsPathMaxBytes &&
-                (g_tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
+    p.use_lds = tiles_per_wave <= 0 && p.lds_plane <= kLdsPathMaxBytes &&
+                (tiles_per_wave < 0 || static_cast<int64_t>(n_tasks) * kv_heads >= kLdsPathMinGroups);
     return p;
 }
 }  // namespace
@@ -983,12 +979,13 @@ void workspace_floats(const VotePlan& p, int n_tasks, int kv_heads, int max_bloc
 }  // namespace
 
 extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks, int sub_blocks,
-                                           int d_pad, int64_t* max_floats, int64_t* part_floats)
+                                           int d_pad, int tiles_per_wave, int64_t* max_floats, int64_t* part_floats)
 {
+    UCM_REQUIRE(tiles_per_wave >= -1, "ucm_kvstar_workspace_floats: tiles_per_wave=%d", tiles_per_wave);
     UCM_REQUIRE(n_tasks >= 0 && kv_heads > 0 && rows_per_head > 0 && rows_per_head <= kMaxRows && max_blocks >= 0 &&
                     sub_blocks > 0 && d_pad > 0 && max_floats && part_floats, "ucm_kvstar_workspace_floats: bad argument");
     UCM_REQUIRE(sub_blocks <= 128 && (sub_blocks & (sub_blocks - 1)) == 0, "ucm_kvstar_workspace_floats: sub_blocks=%d", sub_blocks);
-    workspace_floats(plan_votes(n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad), n_tasks, kv_heads, max_blocks,
+    workspace_floats(plan_votes(n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad, tiles_per_wave), n_tasks, kv_heads, max_blocks,
                      sub_blocks, max_floats, part_floats);
     return UCM_OK;
 }
@@ -998,9 +995,10 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
                  const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, const void* const* task_tables,
                  const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
                  int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part,
-                 int64_t ws_part_floats, float* votes, ucm_stream_t stream)
+                 int64_t ws_part_floats, float* votes, int tiles_per_wave, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks >= 0 && max_blocks >= 0, "ucm_kvstar_votes: n_tasks=%d max_blocks=%d", n_tasks, max_blocks);
+    UCM_REQUIRE(tiles_per_wave >= -1, "ucm_kvstar_votes: tiles_per_wave=%d", tiles_per_wave);
     if (n_tasks == 0 || max_blocks == 0) { return UCM_OK; }
     UCM_REQUIRE(q_f16 && q_off && seg_off && seg_len && ws_max && ws_part && votes, "ucm_kvstar_votes: null pointer");
     UCM_REQUIRE(task_tables ? task_head_strides != nullptr : repre_f16 != nullptr, "ucm_kvstar_votes: no representative table");
@@ -1021,9 +1019,9 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
     UCM_REQUIRE(task_tables || (ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0),
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
-    const VotePlan plan = plan_votes(n_tasks, kv_heads, static_cast<int>(R), max_blocks, sub_blocks, d_pad);
+    const VotePlan plan = plan_votes(n_tasks, kv_heads, static_cast<int>(R), max_blocks, sub_blocks, d_pad, tiles_per_wave);
     {
-        // the path depends on a process-wide knob: a workspace sized before the knob changed must not be overrun
+        // the path depends on tiles_per_wave: a workspace sized for another value must not be overrun
         int64_t need_max = 0, need_part = 0;
         workspace_floats(plan, n_tasks, kv_heads, max_blocks, sub_blocks, &need_max, &need_part);
         UCM_REQUIRE(ws_max_floats >= need_max && ws_part_floats >= need_part,
@@ -1044,8 +1042,8 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
     const unsigned max_spans = (max_tiles + span_tiles - 1) / span_tiles;
     const unsigned spans_per_wg_all = (max_spans + kWaves - 1) / kWaves;
     const unsigned want_chunks = use_lds ? 1u : std::max(1u, 2048u / static_cast<unsigned>(n_tasks * kv_heads));
-    const unsigned spans_per_wave = g_tiles_per_wave > 0
-                                        ? (static_cast<unsigned>(g_tiles_per_wave) + span_tiles - 1) / span_tiles
+    const unsigned spans_per_wave = tiles_per_wave > 0
+                                        ? (static_cast<unsigned>(tiles_per_wave) + span_tiles - 1) / span_tiles
                                         : std::max(1u, (spans_per_wg_all + want_chunks - 1) / want_chunks);
     const unsigned chunks = (max_spans + kWaves * spans_per_wave - 1) / (kWaves * spans_per_wave);
     hipStream_t s = ucm::as_stream(stream);
@@ -1114,11 +1112,11 @@ extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_t
                                 int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
                                 int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                                 int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
-                                ucm_stream_t stream)
+                                int tiles_per_wave, ucm_stream_t stream)
 {
     return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, repre_f16, repre_head_stride, nullptr, nullptr,
                         seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
-                        ws_part_floats, votes, stream);
+                        ws_part_floats, votes, tiles_per_wave, stream);
 }
 
 extern "C" int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
@@ -1126,10 +1124,10 @@ extern "C" int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, 
                                        const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len,
                                        int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad,
                                        float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
-                                       float* votes, ucm_stream_t stream)
+                                       float* votes, int tiles_per_wave, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks == 0 || (task_tables && task_head_strides), "ucm_kvstar_votes_tables: null table list");
     return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, nullptr, 0, task_tables, task_head_strides,
                         seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
-                        ws_part_floats, votes, stream);
+                        ws_part_floats, votes, tiles_per_wave, stream);
 }

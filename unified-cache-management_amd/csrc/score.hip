@@ -377,25 +377,15 @@ void launch(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_
                        seg_off, seg_len, n_req, kv_heads, scores, scores_layer_stride, tile_blocks);
 }
 
-int g_tile_blocks = 0;  // 0: sized from the row bytes at each call
-
 }  // namespace
-
-// Tuning knob for benchmarks: blocks scored per workgroup; 0 restores the
-// default, 128 KiB of representatives per workgroup.
-extern "C" int ucm_set_score_tile(int tile_blocks)
-{
-    UCM_REQUIRE(tile_blocks >= 0 && tile_blocks <= 4096, "ucm_set_score_tile: %d", tile_blocks);
-    g_tile_blocks = tile_blocks;
-    return UCM_OK;
-}
 
 extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
                                 int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
                                 const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
                                 int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
-                                int64_t scores_layer_stride, ucm_stream_t stream)
+                                int64_t scores_layer_stride, int tile_blocks_arg, ucm_stream_t stream)
 {
+    UCM_REQUIRE(tile_blocks_arg >= 0 && tile_blocks_arg <= 4096, "ucm_score_blocks: tile_blocks=%d", tile_blocks_arg);
     UCM_REQUIRE(n_req == 0 || max_seg_len == 0 || (q && repre && seg_off && seg_len && scores),
                 "ucm_score_blocks: null pointer");
     UCM_REQUIRE(q_dtype == UCM_DTYPE_F32 || q_dtype == UCM_DTYPE_BF16, "ucm_score_blocks: q_dtype=%d", q_dtype);
@@ -421,7 +411,7 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
     hipStream_t s = ucm::as_stream(stream);
     // upper bound of sum(ceil(seg_len / tile)): exact to within n_req when the host knows the total
     const int row_bytes = kv_heads * head_dim * (repre_dtype == UCM_DTYPE_BF16 ? 2 : 4);
-    const int tile_blocks = g_tile_blocks > 0 ? g_tile_blocks : std::max(8, (128 * 1024) / row_bytes);
+    const int tile_blocks = tile_blocks_arg > 0 ? tile_blocks_arg : std::max(8, (128 * 1024) / row_bytes);
     const int64_t per_req = (static_cast<int64_t>(max_seg_len) + tile_blocks - 1) / tile_blocks;
     int64_t tile_bound = per_req * n_req;
     if (total_blocks > 0) { tile_bound = std::min(tile_bound, (total_blocks + tile_blocks - 1) / tile_blocks + n_req); }

@@ -131,7 +131,7 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
               total_blocks, n_layers, kv_heads, head_dim,
               _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4, scores.stride(0),
-              _stream())
+              _tuning["score_tile"], _stream())
 
 
 def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, topk_len: torch.Tensor,
@@ -335,7 +335,7 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
               _opt(slots, torch.int32, "slots"), n, block_size, kv_heads, 128, _dev(w, torch.bfloat16, "w"), 128, rows,
               _opt(token_codes, torch.uint8, "token_codes"), 0 if token_codes is None else token_codes.stride(0),
               _dev(colsum, torch.int16, "colsum"), colsum.stride(0), _dev(block_codes, torch.uint8, "block_codes"),
-              block_codes.stride(0), _stream())
+              block_codes.stride(0), _tuning["hash_encode_groups"], _stream())
 
 
 def hash_encode_queries(q: torch.Tensor, w: torch.Tensor, kv_heads: int, q_codes: torch.Tensor, q_sum: torch.Tensor,
@@ -443,7 +443,8 @@ def kvstar_table_from_reference(repre: torch.Tensor) -> torch.Tensor:
 def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                        block_size: int, kv_heads: int, head_dim: int, num_blocks: int, merge: int,
                        pruned: Optional[torch.Tensor] = None) -> None:
-    """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); pruned int32 [kv_heads, d_pruned] or None."""
+    """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); pruned int32 [kv_heads, d_pruned] (one set of
+    channel lists for every layer), [L, kv_heads, d_pruned] (lists per layer) or None."""
     if repre.dim() != 6 or repre.dtype != torch.float16 or repre.shape[4] * merge != block_size or \
             repre.shape[1] != kv_heads or repre.shape[5] != 8:
         raise ValueError("repre must be float16 [L, kv_heads, rows, d_pad/8, block_size/merge, 8]")
@@ -453,12 +454,14 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
         raise ValueError("one table layer per cache layer")
     if block_ids.numel() != slots.numel():
         raise ValueError("block_ids and slots differ in length")
-    d_pruned = head_dim if pruned is None else pruned.shape[1]
-    if pruned is not None and pruned.shape[0] != kv_heads:
-        raise ValueError("pruned must be [kv_heads, d_pruned]")
+    d_pruned = head_dim if pruned is None else pruned.shape[-1]
+    per_layer = pruned is not None and pruned.dim() == 3
+    if pruned is not None and (pruned.shape[-2] != kv_heads or (per_layer and pruned.shape[0] != repre.shape[0])):
+        raise ValueError("pruned must be [kv_heads, d_pruned] or [layers, kv_heads, d_pruned]")
     _lib.call("ucm_kvstar_block_repre", k_layers.ptr(), repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
               _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
-              _opt(pruned, torch.int32, "pruned"), d_pruned, repre.shape[3] * 8, repre.data_ptr(),
+              _opt(pruned, torch.int32, "pruned"), pruned.stride(0) if per_layer else 0, d_pruned, repre.shape[3] * 8,
+              repre.data_ptr(),
               repre.shape[2], repre.stride(0), repre.stride(1), _stream())
 
 
@@ -469,8 +472,8 @@ def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks
     import ctypes as C
 
     a, b = C.c_int64(0), C.c_int64(0)
-    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad, C.addressof(a),
-              C.addressof(b))
+    _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad,
+              _tuning["kvstar_tiles_per_wave"], C.addressof(a), C.addressof(b))
     return (torch.empty(max(a.value, 1), dtype=torch.float32, device=device),
             torch.empty(max(b.value, 1), dtype=torch.float32, device=device))
 
@@ -506,7 +509,7 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), repre.data_ptr(), head_stride,
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
               d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
-              _dev(votes, torch.float32, "votes"), _stream())
+              _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
 
 
 def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: int, tables, seg_off: torch.Tensor,
@@ -542,17 +545,22 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
               d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
-              _dev(votes, torch.float32, "votes"), _stream())
+              _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
     return host, dev
 
 
+# Launch-shape arguments of three entry points that only benchmarks and tests change (0 = the library's default).
+# They are plain per-call arguments of the C ABI; these helpers set what the wrappers of THIS module pass.
+_tuning = {"score_tile": 0, "hash_encode_groups": 0, "kvstar_tiles_per_wave": 0}
+
+
 def set_score_tile(tile_blocks: int) -> None:
-    _lib.call("ucm_set_score_tile", tile_blocks)
+    _tuning["score_tile"] = int(tile_blocks)
 
 
 def set_kvstar_tiles_per_wave(tiles: int) -> None:
-    _lib.call("ucm_set_kvstar_tiles_per_wave", tiles)
+    _tuning["kvstar_tiles_per_wave"] = int(tiles)
 
 
 def set_hash_encode_groups(workgroups: int) -> None:
-    _lib.call("ucm_set_hash_encode_groups", workgroups)
+    _tuning["hash_encode_groups"] = int(workgroups)

@@ -150,11 +150,23 @@ class UcmHipBlockStore:
         addrs, sizes = self._views(src_tensor)
         return self._move(block_ids, offset, addrs, sizes, to_store=True)
 
+    @staticmethod
+    def _checked(addrs: List[int], sizes: List[int]) -> List[int]:
+        """Raw addresses go straight to a copy kernel: each must be memory a kernel can touch (device memory or
+        pinned host memory); pageable host memory is refused here, on the host."""
+        from .. import _lib
+
+        can = _lib.lib().ucm_kernel_can_access
+        for a, n in zip(addrs, sizes):
+            if not can(int(a), int(n)):
+                raise ValueError(f"address {int(a):#x} is not device or pinned host memory")
+        return [int(a) for a in addrs]
+
     def fetch_data(self, block_ids: List[str], offset: List[int], dst_addr: List[int], size: List[int]) -> Task:
-        return self._move(block_ids, offset, list(dst_addr), list(size), to_store=False)
+        return self._move(block_ids, offset, self._checked(dst_addr, size), list(size), to_store=False)
 
     def dump_data(self, block_ids: List[str], offset: List[int], src_addr: List[int], size: List[int]) -> Task:
-        return self._move(block_ids, offset, list(src_addr), list(size), to_store=True)
+        return self._move(block_ids, offset, self._checked(src_addr, size), list(size), to_store=True)
 
     def wait(self, task: HipTask) -> int:
         if task.task_id == "-1":
