@@ -70,6 +70,10 @@ def parse():
                          "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
     ap.add_argument("--hash-leg", action="store_true",
                     help="also time the hash-code retrieval variant (the configs[4] shape of the benchmark definition) on the same caches")
+    ap.add_argument("--hash-distinct", type=int, default=0,
+                    help="hash leg: name only this many distinct cache blocks in the encode's block list, over and over "
+                         "(8: the key loads are served from cache, which times the compute side of the kernel on its own); "
+                         "0 = every block once")
     ap.add_argument("--moves-leg", action="store_true",
                     help="also time the block-id driven load/dump (the configs[2] shape of the benchmark definition: 64 requests "
                          "x 16 blocks, all layers, K and V, random block table) on the same caches")
@@ -78,6 +82,9 @@ def parse():
     ap.add_argument("--kvstar-leg", action="store_true",
                     help="also time the multi-query softmax-vote retrieval (KVStar: 8 query tokens per request) on the same "
                          "ragged batch")
+    ap.add_argument("--kvstar-layout", choices=["row", "head"], default="head",
+                    help="memory order of the KVStar representative table: the kv heads of a block next to each other "
+                         "(row) or a plane per kv head (head)")
     ap.add_argument("--kvstar-merge", type=int, default=2,
                     help="tokens averaged into one sub-block representative (reference default 2: 64 per 128-token block)")
     ap.add_argument("--kvstar-prune", type=float, default=0.25,
@@ -304,6 +311,8 @@ def main():
         h_off = np.concatenate([[0], np.cumsum(h_lens)[:-1]]).astype(np.int32)
         pool = 2 * nb
         h_ids_h = (rng.permutation(pool)[:h_rows] if h_rows <= pool else rng.integers(0, pool, h_rows)).astype(np.int32)
+        if args.hash_distinct > 0:
+            h_ids_h = h_ids_h[np.arange(h_rows) % args.hash_distinct]
         h_ids, h_slots = i32(h_ids_h), torch.arange(h_rows, dtype=torch.int32, device=dev)
         w_hash = (torch.randn(128, 128, device=dev, generator=g) * 2.0).to(torch.bfloat16)
         colsum = torch.zeros((n_layers, h_rows, HKV, 128), dtype=torch.int16, device=dev)
@@ -344,7 +353,7 @@ def main():
         enc_bytes = key_bytes + n_layers * h_rows * (BS * HKV * 16 + HKV * 128 * 2 + HKV * 16)
         hash_checked = None
         # HBM bytes per launch measured with rocprofv3 --pmc on exactly this workload, as for the gather below
-        default_hash = n_layers == N_LAYERS and args.seed == 2024 and h_rows == 5609
+        default_hash = n_layers == N_LAYERS and args.seed == 2024 and h_rows == 5609 and args.hash_distinct == 0
         if not args.no_check:
             import oracle  # checker only
 
@@ -359,7 +368,8 @@ def main():
                     assert np.array_equal(bcodes[l, row].cpu().numpy(), oracle.hash_majority(want)[0]), "block codes differ"
             hash_checked = "token codes, column sums and majority codes of 6 sampled blocks equal the CPU oracle"
         hash_leg = {
-            "workload": f"configs[4]: {h_req} requests, {h_rows} blocks of 128 tokens, {n_layers} layers, 8 kv heads, 128-bit codes",
+            "workload": f"configs[4]: {h_req} requests, {h_rows} blocks of 128 tokens, {n_layers} layers, 8 kv heads, 128-bit codes"
+                        + (f" (block list names {args.hash_distinct} distinct blocks: key loads served from cache)" if args.hash_distinct else ""),
             "encode_ms": round(enc_ms, 3),
             "encode_read_GBps": round(gbs(key_bytes, enc_ms), 1),
             "roofline": {"kernel": "hash_encode_blocks_kernel", "bound": "hbm", "achieved": round(gbs(enc_bytes, enc_ms), 1),
@@ -388,17 +398,25 @@ def main():
         if kdp < D:
             kpr = torch.stack([torch.stack([torch.randperm(D, device=dev, generator=g)[:kdp] for _ in range(HKV)])
                                for _ in range(n_layers)]).to(torch.int32)
-        # one table over all layers, kv head outermost: row of (layer l, block b) = l * rows + b
-        flat = torch.empty((HKV, n_layers * rows, kd_pad // 8, km, 8), dtype=torch.float16, device=dev)
-        ktab = flat.view(HKV, n_layers, rows, kd_pad // 8, km, 8).permute(1, 0, 2, 3, 4, 5)
+        # one table over all layers, indexed [kv head][row][cell]: row of (layer l, block b) = l * rows + b
+        if args.kvstar_layout == "row":      # the kv heads of a row next to each other in memory
+            kmem = torch.empty((n_layers * rows, HKV, kd_pad // 8, km, 8), dtype=torch.float16, device=dev)
+            flat = kmem.permute(1, 0, 2, 3, 4)
+            ktab = kmem.view(n_layers, rows, HKV, kd_pad // 8, km, 8).permute(0, 2, 1, 3, 4, 5)
+        else:                                # a plane per kv head
+            flat = torch.empty((HKV, n_layers * rows, kd_pad // 8, km, 8), dtype=torch.float16, device=dev)
+            ktab = flat.view(HKV, n_layers, rows, kd_pad // 8, km, 8).permute(1, 0, 2, 3, 4, 5)
         ev0, ev1 = ev(), ev()
         ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge, pruned=kpr)   # channel lists per layer
         torch.cuda.synchronize()
-        ev0.record()
-        ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge, pruned=kpr)   # one launch for all layers
-        ev1.record()
-        torch.cuda.synchronize()
-        krep_ms = ev0.elapsed_time(ev1)
+        krep_all = []
+        for _ in range(5):
+            ev0.record()
+            ops.kvstar_block_repre(layers, table, slots, ktab, BS, HKV, D, nb, merge, pruned=kpr)   # one launch for all layers
+            ev1.record()
+            torch.cuda.synchronize()
+            krep_all.append(ev0.elapsed_time(ev1))
+        krep_ms = sorted(krep_all)[len(krep_all) // 2]
         krep_bytes = n_layers * rows * (BLOCK_BYTES + HKV * km * kd_pad * 2)
         n_tasks = n_layers * N_REQ
         k_off = (seg_off_h[None, :].astype(np.int64) + (np.arange(n_layers, dtype=np.int64) * rows)[:, None]).reshape(-1)
@@ -448,7 +466,9 @@ def main():
         kvstar_leg = {
             "workload": f"{n_tasks} tasks (layer x request), {kx} query tokens x {HQ} heads, {rows} blocks x {km} sub-block "
                         f"representatives per layer, {kdp} of {D} channels, fp16",
+            "table_layout": args.kvstar_layout,
             "block_repre_ms": round(krep_ms, 3),
+            "block_repre_ms_all": [round(x, 3) for x in krep_all],
             "block_repre_GBps": round(gbs(krep_bytes, krep_ms), 1),
             "block_repre_frac": round(gbs(krep_bytes, krep_ms) / HBM_PEAK_GBS, 4),
             "us_per_step": round(kv_ms * 1e3, 1),

@@ -383,14 +383,20 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *            after layer l-1's (the reference picks the channels per layer
  *            state; 0 = one set of lists for every layer), so one launch
  *            covers all layers
- *   repre    dev fp16, [n_layers][kv_heads][repre_rows][d_pad/8][M][8]: kv
- *            head outermost, and inside a block the 16-byte pieces (8
- *            channels) of its M sub-blocks side by side; d_pad >= d_pruned, a
- *            multiple of 8 (16 for ucm_kvstar_votes), columns past d_pruned
- *            are written as zero; repre_layer_stride and repre_head_stride in
- *            elements.  (The reference keeps [row][M][kv head][d]; this order
- *            makes what a workgroup streams for one head contiguous and every
- *            load instruction of the score kernel a run of whole cache lines.)
+ *   repre    dev fp16 cells of [d_pad/8][M][8] - the 16-byte pieces (8
+ *            channels) of a block's M sub-blocks side by side - one per
+ *            (layer, kv head, row): cell (l, h, r) starts l*repre_layer_stride
+ *            + h*repre_head_stride + r*repre_row_stride elements in.  Cells
+ *            must not overlap: either head planes ([kv_heads][repre_rows]
+ *            [cell], head stride >= repre_rows * row stride) or the heads of
+ *            a row next to each other ([repre_rows][kv_heads][cell], row
+ *            stride >= kv_heads * head stride); the two measure the same,
+ *            building and reading.  d_pad >=
+ *            d_pruned, a multiple of 8 (16 for ucm_kvstar_votes), columns
+ *            past d_pruned are written as zero; all strides are multiples of
+ *            8.  (The reference keeps [row][M][kv head][d]; inside a cell
+ *            every load instruction of the score kernel is a run of whole
+ *            cache lines.)
  *
  * ucm_kvstar_votes: the arithmetic of KVStar::Execute
  * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:817-990)
@@ -405,8 +411,8 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *   pruned   dev int32[*][kv_heads][d_pruned] channel lists, pruned_sel dev
  *            int32[n_tasks] picks one per task (-1: none); both NULL when
  *            d_pruned == d_orig
- *   repre_f16  dev fp16 [kv_heads][rows][d_pad/8][sub_blocks][8] (one layer of
- *            the table above), head planes repre_head_stride elements apart; task t owns rows
+ *   repre_f16  dev fp16, one layer of the table above: cell (h, r) starts
+ *            h*repre_head_stride + r*repre_row_stride elements in; task t owns rows
  *            seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >= every seg_len
  *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
  *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev fp32, task t's votes at votes[seg_off[t] + b].
@@ -418,7 +424,7 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
                            int kv_heads, int head_dim, int merge, const int32_t* pruned,
                            int64_t pruned_layer_stride, int d_pruned, int d_pad, void* repre_f16,
                            int repre_rows, int64_t repre_layer_stride, int64_t repre_head_stride,
-                           ucm_stream_t stream);
+                           int64_t repre_row_stride, ucm_stream_t stream);
 /* ucm_kvstar_votes has two paths: one workgroup per (task, kv head) that keeps
  * the task's per-(block, query row) sums in LDS and stores only the head's
  * share of the votes (taken when there are at least 128 such pairs and the
@@ -438,22 +444,23 @@ int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, in
                                 int64_t* part_floats);
 int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                      const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                     int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len,
-                     int n_tasks, int max_blocks,
+                     int64_t repre_head_stride, int64_t repre_row_stride, const int32_t* seg_off,
+                     const int32_t* seg_len, int n_tasks, int max_blocks,
                      int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                      int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
                      int tiles_per_wave, ucm_stream_t stream);
 /* The same for tasks whose representatives do not share one table (the
  * reference keeps one blk_repre tensor per request and layer,
  * ucm/sparse/kvstar/multistep.py:191,483-501): task t's table starts at
- * task_tables[t] (dev array of n_tasks dev pointers, 16-byte aligned, laid out
- * [kv_heads][rows][d_pad/8][sub_blocks][8] with its head planes
- * task_head_strides[t] elements apart, a multiple of 8) and its block 0 is
- * the table's row 0; seg_off only places the task's votes. */
+ * task_tables[t] (dev array of n_tasks dev pointers, 16-byte aligned; cell
+ * (h, r) of task t's table starts h*task_head_strides[t] + r*task_row_stride
+ * elements in, multiples of 8) and its block 0 is the table's row 0; seg_off
+ * only places the task's votes. */
 int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                             const int32_t* pruned, const int32_t* pruned_sel,
                             const void* const* task_tables, const int64_t* task_head_strides,
-                            const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                            int64_t task_row_stride, const int32_t* seg_off, const int32_t* seg_len,
+                            int n_tasks, int max_blocks,
                             int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                             int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
                             int tiles_per_wave, ucm_stream_t stream);

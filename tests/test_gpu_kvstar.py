@@ -49,10 +49,10 @@ def test_kvstar_block_repre(ucm, dev, merge, hkv, d, bs):
     ids = synth.permutation(1010, nb)[:9].astype(np.int32)
     slots = synth.permutation(1011, rows)[:9].astype(np.int32)
     M = bs // merge
-    for d_pruned in (d, d - 13, 16):
+    for d_pruned, layout in ((d, "row"), (d - 13, "row"), (16, "row"), (d, "head"), (16, "head")):
         pruned = None if d_pruned == d else np.stack([synth.permutation(1020 + h, d)[:d_pruned] for h in range(hkv)]).astype(np.int32)
         d_pad = (d_pruned + 15) // 16 * 16
-        repre = ops.kvstar_table(n_layers, hkv, rows, M, d_pad, dev).fill_(3.0)      # [L, h, rows, d_pad/8, M, 8]
+        repre = ops.kvstar_table(n_layers, hkv, rows, M, d_pad, dev, layout).fill_(3.0)      # indexed [L, h, rows, d_pad/8, M, 8]
         ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge,
                                pruned=None if pruned is None else torch.from_numpy(pruned).to(dev))
         got = ops.kvstar_table_to_reference(repre).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)   # oracle's order
@@ -95,14 +95,14 @@ def test_kvstar_block_repre_channel_lists_per_layer(ucm, dev, merge):
                                bs, hkv, d, nb, merge, pruned=torch.from_numpy(pruned[:2]).to(dev))
 
 
-def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None, pruned_sel=None, d_pruned=None):
+def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None, pruned_sel=None, d_pruned=None, layout="head"):
     """q_bits_list: per task uint16 [x, hq, d]; repre_bits uint16 [rows, M, hkv, d_pad]; tasks own consecutive row ranges."""
     lens = np.asarray(lens, np.int32)
     off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
     q = dev_f16(np.stack(q_bits_list), dev)
     q_off = torch.arange(len(lens), dtype=torch.int64, device=dev) * q[0].numel()
     rows, M, hkv, _ = repre_bits.shape
-    table = ops.kvstar_table_from_reference(dev_f16(repre_bits, dev))                 # the kernels' order: [h, rows, d_pad/8, M, 8]
+    table = ops.kvstar_table_from_reference(dev_f16(repre_bits, dev), layout)         # indexed [h, rows, d_pad/8, M, 8]
     assert torch.equal(ops.kvstar_table_to_reference(table), dev_f16(repre_bits, dev))
     votes = torch.full((rows,), -7.0, device=dev)
     ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, table.shape[2] * 8, dev)
@@ -128,9 +128,10 @@ def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
     wants = {t: O.kvstar_retrieve(qs[t], repre[sum(lens[:t]) : sum(lens[:t]) + n], topk=max(n // 3, 1))[1]
              for t, n in enumerate(lens) if n}
     try:
-        for tiles_per_wave in (0, -1, 1, 3):                  # 0: automatic, -1: per-task plane in LDS, n: chunks of 4n tiles
+        # 0: automatic, -1: per-task plane in LDS, n: chunks of 4n tiles; table rows of kv_heads cells, or head planes
+        for tiles_per_wave, layout in ((0, "row"), (-1, "row"), (1, "row"), (3, "row"), (0, "head"), (-1, "head"), (3, "head")):
             ops.set_kvstar_tiles_per_wave(tiles_per_wave)
-            got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
+            got, off = run_votes(ops, dev, qs, repre, lens, x, hq, layout=layout)
             for t, n in enumerate(lens):
                 if n == 0:
                     continue

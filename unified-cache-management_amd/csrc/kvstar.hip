@@ -80,13 +80,64 @@ __device__ __forceinline__ void add_bf16x8(float (&acc)[8], const u32x4 v)
     acc[6] = acc[6] + __uint_as_float(v.w << 16); acc[7] = acc[7] + __uint_as_float(v.w & 0xffff0000u);
 }
 
+// With channel lists, which (kv head, 16-byte piece) pairs a thread writes is decided once per kernel when the
+// pairs divide the workgroup: kThreads / pairs threads share a pair and split its sub-blocks, and the pair's eight
+// kept channels stay in registers (-1: a padding column).  Reading the lists again for every piece and turning
+// a flat index into (head, piece, sub-block) by division cost more instructions than the key loads themselves.
+struct PieceMap {
+    bool fixed;
+    unsigned h, piece, sub, tpp;
+    int d[8];
+};
+
+__device__ __forceinline__ PieceMap make_piece_map(const int32_t* __restrict__ lists, unsigned kv_heads, unsigned head_dim,
+                                                   unsigned d_pruned, unsigned pieces)
+{
+    PieceMap m;
+    const unsigned pairs = kv_heads * pieces;
+    m.fixed = lists != nullptr && pairs <= static_cast<unsigned>(kThreads) && (kThreads % pairs) == 0;
+    m.tpp = m.fixed ? kThreads / pairs : 1u;
+    const unsigned pair = threadIdx.x / m.tpp;
+    m.sub = threadIdx.x - pair * m.tpp;
+    m.h = m.fixed ? pair / pieces : 0u;
+    m.piece = m.fixed ? pair - m.h * pieces : 0u;
+#pragma unroll
+    for (unsigned j = 0; j < 8; ++j) {
+        const unsigned p = m.piece * 8 + j;
+        int d = -1;
+        if (m.fixed && p < d_pruned) {
+            d = lists[m.h * d_pruned + p];
+            if (d < 0 || static_cast<unsigned>(d) >= head_dim) { d = -1; }
+        }
+        m.d[j] = d;
+    }
+    return m;
+}
+
 // Phase 2 of the representative kernels: the kept channels of the staged means of sub-blocks m0 .. m0+mc-1,
 // gathered from LDS and written as the table's 16-byte pieces, consecutive threads to consecutive 16 bytes.
 __device__ __forceinline__ void repre_write_pieces(const unsigned short* __restrict__ stage, const int32_t* __restrict__ kept,
                                                    bool pruned, unsigned kv_heads, unsigned head_dim, unsigned d_pruned,
                                                    unsigned pieces, unsigned srow_stride, unsigned M, unsigned m0, unsigned mc,
-                                                   unsigned short* __restrict__ out, int64_t head_stride)
+                                                   unsigned short* __restrict__ out, int64_t head_stride, const PieceMap& pm)
 {
+    if (pm.fixed) {
+        unsigned short* dst = out + static_cast<int64_t>(pm.h) * head_stride + (static_cast<size_t>(pm.piece) * M + m0) * 8;
+        const unsigned short* src = stage + pm.h * head_dim;
+        for (unsigned ml = pm.sub; ml < mc; ml += pm.tpp) {
+            const unsigned short* srow = src + ml * srow_stride;
+            unsigned short c[8];
+#pragma unroll
+            for (unsigned j = 0; j < 8; ++j) { c[j] = pm.d[j] >= 0 ? srow[pm.d[j]] : static_cast<unsigned short>(0); }
+            u32x4 o;
+            o.x = c[0] | (static_cast<unsigned>(c[1]) << 16);
+            o.y = c[2] | (static_cast<unsigned>(c[3]) << 16);
+            o.z = c[4] | (static_cast<unsigned>(c[5]) << 16);
+            o.w = c[6] | (static_cast<unsigned>(c[7]) << 16);
+            ucm::gstore16(dst + static_cast<size_t>(ml) * 8, o);
+        }
+        return;
+    }
     for (unsigned e = threadIdx.x; e < kv_heads * pieces * mc; e += kThreads) {
         const unsigned h = e / (pieces * mc), rem = e - h * (pieces * mc);
         const unsigned piece = rem / mc, ml = rem - piece * mc;
@@ -127,7 +178,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows, unsigned block_size,
     unsigned kv_heads, unsigned head_dim, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride,
     unsigned d_pruned, unsigned d_pad, unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride,
-    unsigned m_chunk)
+    int64_t row_stride, unsigned m_chunk)
 {
     static_assert(kMerge == 1 || kMerge == 2 || kMerge == 4 || kMerge == 8, "tokens per sub-block");
     extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]: the 16 bytes of padding
@@ -139,15 +190,27 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const unsigned short* layer = static_cast<const unsigned short*>(k_layers[blockIdx.y]);
     // the channel lists, read once: a load from memory per output piece would queue behind the key stream
     int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
+    const int32_t* my_lists = pruned ? pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride : nullptr;
     if (pruned) {   // this layer's lists (a stride of 0: one set of lists for every layer)
-        const int32_t* mine = pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride;
-        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = mine[e]; }
+        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = my_lists[e]; }
     }
+    const PieceMap pm = make_piece_map(my_lists, kv_heads, head_dim, d_pruned, pieces);
 
     struct Unit {
         unsigned item, m0, w_first;                      // cache block in the list, first sub-block of the chunk, first work item
+        unsigned wq, wr;                                 // w_first = wq * ncg + wr
         const unsigned short* blk;
         bool valid;
+    };
+    // (sub-block, column group) of a work item is its number divided by ncg.  One division per thread here and
+    // additions with a carry afterwards: a division per load cost as many instructions as the means themselves.
+    const unsigned tq = threadIdx.x / ncg, tr = threadIdx.x - tq * ncg;                 // this thread's offset inside a unit
+    const unsigned sq = kThreads / ncg, sr = kThreads - sq * ncg;                        // step between a thread's items
+    const unsigned uq = (kThreads * kBatch) / ncg, ur = kThreads * kBatch - uq * ncg;   // step between units
+    auto step = [&](unsigned& q, unsigned& r, unsigned dq, unsigned dr) {
+        q += dq;
+        r += dr;
+        if (r >= ncg) { r -= ncg; ++q; }
     };
     // first usable cache block at or after `from` (a block id or slot out of range is skipped, never dereferenced)
     auto seek = [&](Unit& u, unsigned from) {
@@ -157,6 +220,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
                 u.item = i;
                 u.m0 = 0;
                 u.w_first = 0;
+                u.wq = u.wr = 0;
                 u.blk = layer + static_cast<size_t>(id) * block_size * row;
                 return;
             }
@@ -167,8 +231,10 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
         Unit n = u;
         const unsigned mc = min(m_chunk, M - u.m0);
         n.w_first = u.w_first + kThreads * kBatch;
+        step(n.wq, n.wr, uq, ur);
         if (n.w_first >= mc * ncg) {
             n.w_first = 0;
+            n.wq = n.wr = 0;
             n.m0 = u.m0 + m_chunk;
             if (n.m0 >= M) { seek(n, u.item + gridDim.x); }
         }
@@ -176,63 +242,72 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     };
     // unconditional: work items past the chunk's end reload its last one
     auto load_unit = [&](u32x4 (&v)[kRepreUnroll], const Unit& u) {
-        const unsigned last = min(m_chunk, M - u.m0) * ncg - 1;
+        const unsigned mc = min(m_chunk, M - u.m0), last = mc * ncg - 1;
+        unsigned q = u.wq, r = u.wr;
+        step(q, r, tq, tr);
 #pragma unroll
         for (unsigned j = 0; j < kBatch; ++j) {
-            const unsigned w = min(u.w_first + threadIdx.x + j * kThreads, last);
-            const unsigned ml = w / ncg, cg = w - ml * ncg;
+            const bool past = u.w_first + threadIdx.x + j * kThreads > last;
+            const unsigned ml = past ? mc - 1 : q, cg = past ? ncg - 1 : r;
+            step(q, r, sq, sr);
             const unsigned short* src = u.blk + static_cast<size_t>(u.m0 + ml) * kMerge * row + cg * 8;
 #pragma unroll
             for (unsigned t = 0; t < kMerge; ++t) { v[j * kMerge + t] = ucm::gload16_nt(src + static_cast<size_t>(t) * row); }
         }
         asm volatile("" ::: "memory");                   // keeps the compiler from sinking the loads to their use
     };
-    auto finish_unit = [&](const u32x4 (&v)[kRepreUnroll], const Unit& u) {
-        const unsigned mc = min(m_chunk, M - u.m0);
+    // `live` false: the unit does not exist (the sequence has ended); its registers are still read, nothing is written
+    auto finish_unit = [&](const u32x4 (&v)[kRepreUnroll], const Unit& u, bool live) {
+        const unsigned mc = min(m_chunk, M - u.m0), n_work = live ? mc * ncg : 0u;
+        unsigned q = u.wq, r = u.wr;
+        step(q, r, tq, tr);
 #pragma unroll
         for (unsigned j = 0; j < kBatch; ++j) {
             const unsigned w = u.w_first + threadIdx.x + j * kThreads;
-            if (w < mc * ncg) {                          // (LDS only: a branch is harmless)
-                const unsigned ml = w / ncg, cg = w - ml * ncg;
-                float acc[8];
+            const unsigned ml = q, cg = r;
+            step(q, r, sq, sr);
+            // the means are formed whether or not the item exists: were the loaded registers read only under a
+            // branch, the compiler could not tell further down that their loads have returned, and would wait
+            // there for every load in flight, the next unit's included
+            float acc[8];
 #pragma unroll
-                for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
+            for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
 #pragma unroll
-                for (unsigned t = 0; t < kMerge; ++t) { add_bf16x8(acc, v[j * kMerge + t]); }
-                u32x4 o;
-                o.x = mean_to_f16x2(acc[0], acc[1], inv);
-                o.y = mean_to_f16x2(acc[2], acc[3], inv);
-                o.z = mean_to_f16x2(acc[4], acc[5], inv);
-                o.w = mean_to_f16x2(acc[6], acc[7], inv);
-                *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
-            }
+            for (unsigned t = 0; t < kMerge; ++t) { add_bf16x8(acc, v[j * kMerge + t]); }
+            u32x4 o;
+            o.x = mean_to_f16x2(acc[0], acc[1], inv);
+            o.y = mean_to_f16x2(acc[2], acc[3], inv);
+            o.z = mean_to_f16x2(acc[4], acc[5], inv);
+            o.w = mean_to_f16x2(acc[6], acc[7], inv);
+            if (w < n_work) { *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o; }
         }
-        if (u.w_first + kThreads * kBatch >= mc * ncg) { // the chunk is staged: write its pieces
+        if (live && u.w_first + kThreads * kBatch >= mc * ncg) { // the chunk is staged: write its pieces
             __syncthreads();
             unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride +
-                                  static_cast<size_t>(static_cast<unsigned>(slots[u.item])) * M * d_pad;
+                                  static_cast<int64_t>(static_cast<unsigned>(slots[u.item])) * row_stride;
             repre_write_pieces(stage, kept, pruned != nullptr, kv_heads, head_dim, d_pruned, pieces, srow_stride, M, u.m0, mc,
-                               out, head_stride);
+                               out, head_stride, pm);
             __syncthreads();                             // the next chunk overwrites the staged means
         }
     };
 
-    Unit cur{0u, 0u, 0u, nullptr, true};
-    seek(cur, blockIdx.x);
-    if (!cur.valid) { return; }                          // the whole workgroup: the unit sequence is the same for all threads
+    // Two units per round, one in each register set, and ONE way out of the loop, at its end: with a second exit
+    // between the halves the compiler joins both exits in one block that also leads back to the loop's head, and
+    // then waits at the head for the loads it believes may have just been issued - all of them, every round.
+    Unit a{0u, 0u, 0u, 0u, 0u, nullptr, true};
+    seek(a, blockIdx.x);
+    if (!a.valid) { return; }                            // the whole workgroup: the unit sequence is the same for all threads
     u32x4 va[kRepreUnroll], vb[kRepreUnroll];
-    load_unit(va, cur);
+    load_unit(va, a);
     for (;;) {
-        Unit nxt = next_of(cur);
-        load_unit(vb, nxt.valid ? nxt : cur);
-        finish_unit(va, cur);
-        if (!nxt.valid) { break; }
-        cur = nxt;
-        nxt = next_of(cur);
-        load_unit(va, nxt.valid ? nxt : cur);
-        finish_unit(vb, cur);
-        if (!nxt.valid) { break; }
-        cur = nxt;
+        const Unit b = next_of(a);                       // past the end: a reloads (16 loads per workgroup, once)
+        load_unit(vb, b.valid ? b : a);
+        finish_unit(va, a, true);
+        const Unit c = b.valid ? next_of(b) : b;
+        load_unit(va, c.valid ? c : a);
+        finish_unit(vb, b.valid ? b : a, b.valid);
+        if (!c.valid) { break; }
+        a = c;
     }
 }
 
@@ -243,7 +318,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
     unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride, unsigned d_pruned,
     unsigned d_pad,
-    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, unsigned m_chunk)
+    unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, int64_t row_stride, unsigned m_chunk)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]
     const unsigned M = block_size / merge;
@@ -255,12 +330,13 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
                                 static_cast<size_t>(id) * block_size * row;
     const float inv = 1.0f / static_cast<float>(merge);
     const unsigned pieces = d_pad / 8;
-    unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<size_t>(slot) * M * d_pad;
+    unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<int64_t>(slot) * row_stride;
     int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
+    const int32_t* my_lists = pruned ? pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride : nullptr;
     if (pruned) {   // this layer's lists (a stride of 0: one set of lists for every layer)
-        const int32_t* mine = pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride;
-        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = mine[e]; }
+        for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = my_lists[e]; }
     }
+    const PieceMap pm = make_piece_map(my_lists, kv_heads, head_dim, d_pruned, pieces);
     for (unsigned m0 = 0; m0 < M; m0 += m_chunk) {       // m_chunk sub-blocks at a time: what fits LDS
         const unsigned mc = min(m_chunk, M - m0);
         for (unsigned w = threadIdx.x; w < mc * ncg; w += kThreads) {
@@ -287,7 +363,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
         }
         __syncthreads();
         repre_write_pieces(stage, kept, pruned != nullptr, kv_heads, head_dim, d_pruned, pieces, srow_stride, M, m0, mc, out,
-                           head_stride);
+                           head_stride, pm);
         __syncthreads();                                 // the next chunk overwrites the staged means
     }
 }
@@ -387,7 +463,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const unsigned short* __restrict__ table, const void* const* __restrict__ task_tables,
     const int64_t* __restrict__ task_head_strides, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
-    float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
+    int64_t row_stride, float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
     unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset, unsigned q_full_ok)
 {
     static_assert(kM >= 1 && kM <= 128 && (kM & (kM - 1)) == 0, "sub-blocks per block");
@@ -428,7 +504,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     // the task's first representative: rows seg_off[task].. of the one table, or a table of the task's own
     const unsigned short* tbase =
         (task_tables ? static_cast<const unsigned short*>(task_tables[task]) + static_cast<int64_t>(h) * task_head_strides[task]
-                     : table + static_cast<int64_t>(h) * head_stride + static_cast<size_t>(seg_off[task]) * kM * d_pad) +
+                     : table + static_cast<int64_t>(h) * head_stride + static_cast<int64_t>(seg_off[task]) * row_stride) +
         half * (8 * kM);
 
     // A span's keys: for each of its tiles, kSteps 16-byte loads per lane, piece 2*ks + half of the lane's
@@ -447,7 +523,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 #pragma unroll
         for (int t = 0; t < kSpanTiles; ++t) {
             const unsigned s_mine = min(s0 + t * kTileSub + lr, s_last);
-            const unsigned short* krow = tbase + static_cast<size_t>(s_mine / kM) * (kM * d_pad) + (s_mine % kM) * 8;
+            const unsigned short* krow = tbase + static_cast<int64_t>(s_mine / kM) * row_stride + (s_mine % kM) * 8;
 #pragma unroll
             for (int ks = 0; ks < kSteps; ++ks) {
                 kf[t * kSteps + ks] = ucm::gload16(krow + (static_cast<unsigned>(ks) < ksteps ? ks : 0) * (16 * kM));
@@ -853,7 +929,7 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                                       int kv_heads, int head_dim, int merge, const int32_t* pruned,
                                       int64_t pruned_layer_stride, int d_pruned,
                                       int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
-                                      int64_t repre_head_stride, ucm_stream_t stream)
+                                      int64_t repre_head_stride, int64_t repre_row_stride, ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_kvstar_block_repre: n=%d", n);
     if (n == 0) { return UCM_OK; }
@@ -868,17 +944,23 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_REQUIRE(pruned_layer_stride == 0 || pruned_layer_stride >= static_cast<int64_t>(kv_heads) * d_pruned,
                 "ucm_kvstar_block_repre: pruned_layer_stride=%lld", static_cast<long long>(pruned_layer_stride));
     const int M = block_size / merge;
-    UCM_REQUIRE(repre_head_stride >= static_cast<int64_t>(repre_rows) * M * d_pad,
-                "ucm_kvstar_block_repre: repre_head_stride=%lld smaller than one head's plane",
-                static_cast<long long>(repre_head_stride));
+    // a (row, kv head) cell is M*d_pad elements; the cells must not overlap: heads outside rows (head planes) or
+    // rows outside heads (a block's heads next to each other)
+    const int64_t cell = static_cast<int64_t>(M) * d_pad;
+    UCM_REQUIRE(repre_row_stride >= cell && repre_head_stride >= cell &&
+                    (repre_head_stride >= static_cast<int64_t>(repre_rows) * repre_row_stride ||
+                     repre_row_stride >= static_cast<int64_t>(kv_heads) * repre_head_stride),
+                "ucm_kvstar_block_repre: repre_head_stride=%lld and repre_row_stride=%lld let cells of %lld elements overlap",
+                static_cast<long long>(repre_head_stride), static_cast<long long>(repre_row_stride),
+                static_cast<long long>(cell));
     const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
     UCM_SUPPORTED(row % 8 == 0 && d_pad % 8 == 0, "ucm_kvstar_block_repre: kv_heads*head_dim=%u and d_pad=%d must be multiples of 8",
                   row, d_pad);
     UCM_SUPPORTED(row <= 32768u && head_dim % 8 == 0, "ucm_kvstar_block_repre: kv_heads*head_dim=%u (at most 32768), head_dim=%d (a multiple of 8)", row, head_dim);
     const unsigned m_chunk = std::min<unsigned>(static_cast<unsigned>(M), 33280u / (row + 8));   // sub-blocks staged at a time: 65 KiB of LDS
     const size_t lds_bytes = static_cast<size_t>(m_chunk) * (row + 8) * 2 + (pruned ? static_cast<size_t>(kv_heads) * d_pruned * 4 : 0);
-    UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_layer_stride % 8 == 0 && repre_head_stride % 8 == 0,
-                "ucm_kvstar_block_repre: table not 16-byte aligned");
+    UCM_REQUIRE(ucm::aligned16(repre_f16) && repre_layer_stride % 8 == 0 && repre_head_stride % 8 == 0 &&
+                    repre_row_stride % 8 == 0, "ucm_kvstar_block_repre: table not 16-byte aligned");
     hipStream_t hs = ucm::as_stream(stream);
     // persistent workgroups for the common sub-block sizes: about 1024 over all layers (two fit a compute unit)
     const unsigned gx = static_cast<unsigned>(std::min(n, std::max(1, (1024 + n_layers - 1) / n_layers)));
@@ -895,7 +977,8 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                            static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),                     \
                            static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), pruned,                 \
                            pruned_layer_stride, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),       \
-                           static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk); \
+                           static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride,          \
+                           repre_row_stride, m_chunk);                                                               \
     } while (0)
     switch (merge) {
     case 1: UCM_KVSTAR_REPRE(1); break;
@@ -913,7 +996,8 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                            static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim),
                            static_cast<unsigned>(merge), pruned, pruned_layer_stride, static_cast<unsigned>(d_pruned),
                            static_cast<unsigned>(d_pad),
-                           static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, m_chunk);
+                           static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, repre_row_stride,
+                           m_chunk);
         break;
     }
 #undef UCM_KVSTAR_REPRE
@@ -992,8 +1076,8 @@ extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_p
 
 namespace {
 int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
-                 const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, const void* const* task_tables,
-                 const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
+                 const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, int64_t repre_row_stride,
+                 const void* const* task_tables, const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
                  int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part,
                  int64_t ws_part_floats, float* votes, int tiles_per_wave, ucm_stream_t stream)
 {
@@ -1018,6 +1102,9 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
                   "ucm_kvstar_votes: sub_blocks=%d (a power of two up to 128)", sub_blocks);
     UCM_REQUIRE(task_tables || (ucm::aligned16(repre_f16) && repre_head_stride % 8 == 0 && repre_head_stride > 0),
                 "ucm_kvstar_votes: representatives not 16-byte aligned");
+    UCM_REQUIRE(repre_row_stride % 8 == 0 && repre_row_stride >= static_cast<int64_t>(sub_blocks) * d_pad,
+                "ucm_kvstar_votes: repre_row_stride=%lld (a multiple of 8, at least sub_blocks*d_pad=%d)",
+                static_cast<long long>(repre_row_stride), sub_blocks * d_pad);
     const unsigned R = static_cast<unsigned>(n_tokens * (q_heads / kv_heads));
     const VotePlan plan = plan_votes(n_tasks, kv_heads, static_cast<int>(R), max_blocks, sub_blocks, d_pad, tiles_per_wave);
     {
@@ -1051,7 +1138,7 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), task_tables, task_head_strides, seg_off, seg_len,                      \
         static_cast<unsigned>(kv_heads),                                                                                      \
-        static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, ws_max, ws_part,                   \
+        static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, repre_row_stride, ws_max, ws_part, \
         static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset, q_full_ok
 #define UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, LDS)                                                                        \
     do {                                                                                                             \
@@ -1109,25 +1196,25 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
 
 extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                                 const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                                int64_t repre_head_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
-                                int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+                                int64_t repre_head_stride, int64_t repre_row_stride, const int32_t* seg_off,
+                                const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                                 int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
                                 int tiles_per_wave, ucm_stream_t stream)
 {
-    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, repre_f16, repre_head_stride, nullptr, nullptr,
-                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
+    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, repre_f16, repre_head_stride, repre_row_stride,
+                        nullptr, nullptr, seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
                         ws_part_floats, votes, tiles_per_wave, stream);
 }
 
 extern "C" int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
                                        const int32_t* pruned, const int32_t* pruned_sel, const void* const* task_tables,
-                                       const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len,
-                                       int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad,
+                                       const int64_t* task_head_strides, int64_t task_row_stride, const int32_t* seg_off,
+                                       const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad,
                                        float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
                                        float* votes, int tiles_per_wave, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks == 0 || (task_tables && task_head_strides), "ucm_kvstar_votes_tables: null table list");
-    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, nullptr, 0, task_tables, task_head_strides,
-                        seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
+    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, nullptr, 0, task_row_stride, task_tables,
+                        task_head_strides, seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
                         ws_part_floats, votes, tiles_per_wave, stream);
 }

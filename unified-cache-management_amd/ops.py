@@ -415,12 +415,31 @@ def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, 
               _staging_ptr(staging, staging_blocks * block_bytes), staging_blocks, _stream())
 
 
-def kvstar_table(n_layers: int, kv_heads: int, rows: int, sub_blocks: int, d_pad: int, device) -> torch.Tensor:
-    """Empty KVStar representative table, fp16 [L, kv_heads, rows, d_pad/8, M, 8]: per kv head and block the
-    16-byte pieces (8 channels) of the M sub-blocks lie side by side, the order the score kernel streams."""
+def kvstar_table(n_layers: int, kv_heads: int, rows: int, sub_blocks: int, d_pad: int, device,
+                 layout: str = "head") -> torch.Tensor:
+    """Empty KVStar representative table, fp16, indexed [L, kv_heads, rows, d_pad/8, M, 8]: per kv head and block
+    a cell with the 16-byte pieces (8 channels) of the M sub-blocks side by side, the order the score kernel
+    streams.  layout "head" keeps a plane per kv head, "row" the kv heads of a row next to each other in memory
+    (the returned tensor is then a permuted view); the kernels take either and run equally fast on both."""
     if d_pad % 16 != 0:
         raise ValueError("d_pad must be a multiple of 16")
-    return torch.empty((n_layers, kv_heads, rows, d_pad // 8, sub_blocks, 8), dtype=torch.float16, device=device)
+    if layout == "head":
+        return torch.empty((n_layers, kv_heads, rows, d_pad // 8, sub_blocks, 8), dtype=torch.float16, device=device)
+    if layout != "row":
+        raise ValueError("layout must be 'row' or 'head'")
+    return torch.empty((n_layers, rows, kv_heads, d_pad // 8, sub_blocks, 8), dtype=torch.float16,
+                       device=device).permute(0, 2, 1, 3, 4, 5)
+
+
+def _kvstar_cell_strides(t: torch.Tensor, what: str):
+    """(head stride, row stride) in elements of a [kv_heads, rows, d_pad/8, M, 8] view whose cells are dense."""
+    kv_heads, rows, pieces, m, _ = t.shape
+    cell = pieces * m * 8
+    if rows and kv_heads and not t[0, 0].is_contiguous():
+        raise ValueError(f"{what}: a (kv head, row) cell [d_pad/8, M, 8] must be contiguous")
+    row_stride = t.stride(1) if rows > 1 else cell
+    head_stride = t.stride(0) if kv_heads > 1 else max(rows, 1) * row_stride
+    return head_stride, row_stride
 
 
 def kvstar_table_to_reference(table: torch.Tensor) -> torch.Tensor:
@@ -431,13 +450,19 @@ def kvstar_table_to_reference(table: torch.Tensor) -> torch.Tensor:
     return table.permute(*lead, k + 1, k + 3, k, k + 2, k + 4).reshape(*table.shape[:-5], rows, m, h, pieces * 8)
 
 
-def kvstar_table_from_reference(repre: torch.Tensor) -> torch.Tensor:
-    """The reference's [rows, M, kv_heads, d] -> fp16 [kv_heads, rows, d_pad/8, M, 8], columns zero padded to 16."""
+def kvstar_table_from_reference(repre: torch.Tensor, layout: str = "head") -> torch.Tensor:
+    """The reference's [rows, M, kv_heads, d] -> fp16 indexed [kv_heads, rows, d_pad/8, M, 8], columns zero padded to
+    16; in memory the heads of a row next to each other (layout "row") or a plane per head ("head")."""
     rows, m, h, d = repre.shape
     d_pad = (d + 15) // 16 * 16
     padded = torch.zeros((rows, m, h, d_pad), dtype=torch.float16, device=repre.device)
     padded[..., :d] = repre
-    return padded.view(rows, m, h, d_pad // 8, 8).permute(2, 0, 3, 1, 4).contiguous()
+    cells = padded.view(rows, m, h, d_pad // 8, 8)
+    if layout == "head":
+        return cells.permute(2, 0, 3, 1, 4).contiguous()
+    if layout != "row":
+        raise ValueError("layout must be 'row' or 'head'")
+    return cells.permute(0, 2, 3, 1, 4).contiguous().permute(1, 0, 2, 3, 4)
 
 
 def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
@@ -448,8 +473,7 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
     if repre.dim() != 6 or repre.dtype != torch.float16 or repre.shape[4] * merge != block_size or \
             repre.shape[1] != kv_heads or repre.shape[5] != 8:
         raise ValueError("repre must be float16 [L, kv_heads, rows, d_pad/8, block_size/merge, 8]")
-    if not repre[0, 0].is_contiguous():
-        raise ValueError("a head's plane of the table must be contiguous")
+    head_stride, row_stride = _kvstar_cell_strides(repre[0], "repre")
     if len(k_layers) != repre.shape[0]:
         raise ValueError("one table layer per cache layer")
     if block_ids.numel() != slots.numel():
@@ -462,7 +486,7 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
               _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
               _opt(pruned, torch.int32, "pruned"), pruned.stride(0) if per_layer else 0, d_pruned, repre.shape[3] * 8,
               repre.data_ptr(),
-              repre.shape[2], repre.stride(0), repre.stride(1), _stream())
+              repre.shape[2], repre.stride(0), head_stride, row_stride, _stream())
 
 
 def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks: int, sub_blocks: int, d_pad: int,
@@ -489,8 +513,7 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
         raise ValueError("repre must be a float16 device tensor [kv_heads, rows, d_pad/8, M, 8]")
     kv_heads, rows, pieces, m, _ = repre.shape
     d_pad = pieces * 8
-    if rows and not repre[0].is_contiguous():
-        raise ValueError("repre rows must be dense ([rows, d_pad/8, M, 8] contiguous inside each head plane)")
+    head_stride, row_stride = _kvstar_cell_strides(repre, "repre")
     d_orig = q.shape[-1]
     n_tasks = seg_off.numel()
     if seg_len.numel() != n_tasks or q_off.numel() != n_tasks:
@@ -504,11 +527,10 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
     if votes.numel() < rows:
         raise ValueError("votes shorter than the representative table")
     ws_max, ws_part = workspace
-    head_stride = repre.stride(0) if kv_heads > 1 else rows * m * d_pad
     _lib.call("ucm_kvstar_votes", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), repre.data_ptr(), head_stride,
-              _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
-              d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
+              row_stride, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m,
+              kv_heads, d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
               _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
 
 
@@ -523,11 +545,17 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
     if n_tasks == 0:
         return None
     kv_heads, _, pieces, m, _ = tables[0].shape
+    cell = pieces * m * 8
+    strides = []
     for t in tables:
         if t.dim() != 5 or t.dtype != torch.float16 or not t.is_cuda or t.shape[0] != kv_heads or t.shape[2:] != tables[0].shape[2:]:
             raise ValueError("every table must be a float16 device tensor [kv_heads, rows, d_pad/8, M, 8] of the same M and d_pad")
-        if t.shape[1] and not t[0].is_contiguous():
-            raise ValueError("table rows must be dense inside each head plane")
+        strides.append(_kvstar_cell_strides(t, "table"))
+    # one row stride for the call: tables of a single row fit any
+    row_strides = {rs for t, (_, rs) in zip(tables, strides) if t.shape[1] > 1}
+    if len(row_strides) > 1:
+        raise ValueError("the tables of one call must share a row stride (all head planes, or all rows of kv_heads cells)")
+    row_stride = row_strides.pop() if row_strides else cell
     d_orig = q.shape[-1]
     if seg_off.numel() != n_tasks or seg_len.numel() != n_tasks or q_off.numel() != n_tasks:
         raise ValueError("q_off / seg_off / seg_len / tables differ in length")
@@ -538,13 +566,13 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
     elif d_pruned is None:
         d_pruned = d_orig
     host = torch.tensor([[t.data_ptr() for t in tables],
-                         [t.stride(0) if kv_heads > 1 else max(t[0].numel(), 8) for t in tables]], dtype=torch.int64).pin_memory()
+                         [hs for hs, _ in strides]], dtype=torch.int64).pin_memory()
     dev = host.to(tables[0].device, non_blocking=True)
     ws_max, ws_part = workspace
     _lib.call("ucm_kvstar_votes_tables", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
-              _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m, kv_heads,
-              d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
+              row_stride, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m,
+              kv_heads, d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
               _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
     return host, dev
 
