@@ -113,6 +113,11 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *              value, sizes the grid); total_blocks = sum of seg_len when the
  *              host knows it (a tighter grid), else 0.
  *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x].
+ *   scale      every score is multiplied by it on the way out; 1 leaves the bits
+ *              above.  1/kv_heads gives the values of the reference's torch
+ *              variant, the mean over all q heads of TopkCal.cal_topk
+ *              (ucm/sparse/gsa/gsa.py:386-412, to the rounding of its own
+ *              summation order; the ranking is the same for any positive scale).
  *   tile_blocks  blocks scored per workgroup; 0 sizes a workgroup's share to 128 KiB
  *              of representatives (a value for benchmarks and tests, not part of
  *              the reference interface).
@@ -123,7 +128,7 @@ int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const i
                      int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
                      const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
                      int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
-                     int64_t scores_layer_stride, int tile_blocks, ucm_stream_t stream);
+                     int64_t scores_layer_stride, float scale, int tile_blocks, ucm_stream_t stream);
 
 /*
  * Per-request block selection with forced windows, all layers in one launch -

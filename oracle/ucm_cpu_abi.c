@@ -1,0 +1,258 @@
+/*
+ * Host twins of the C ABI: the same prototypes as libucm_hip.so's entry points
+ * of the dense retrieval path, name + "_cpu", every "dev" pointer a host
+ * pointer, `stream` ignored, the work done before the call returns.  A caller
+ * written against one prototype switches between host and device by choosing
+ * the symbol.
+ *
+ * TEST INFRASTRUCTURE ONLY, like the rest of this directory: the arithmetic is
+ * the oracle's (ucm_oracle.c, which names the reference lines it follows) and
+ * nothing here is linked into, loaded by or shipped with the product.  The
+ * twins are compiled into liborc.so.
+ *
+ * The type of every twin is taken from the device entry point's declaration
+ * (`__typeof__`), so a twin whose parameter list drifts from the header does
+ * not compile.  Argument checks follow the device library's: UCM_EINVAL for
+ * what it calls a bad argument, ids / slots / rows outside their table are
+ * skipped, never dereferenced.
+ */
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "ucm_hip.h"
+
+#define ORC_API __attribute__((visibility("default")))
+#define TWIN(name) ORC_API extern __typeof__(name) name##_cpu
+
+TWIN(ucm_block_mean);
+TWIN(ucm_score_blocks);
+TWIN(ucm_topk_windows);
+TWIN(ucm_kv_gather_blocks);
+TWIN(ucm_kv_scatter_blocks);
+TWIN(ucm_kv_gather_selected);
+TWIN(ucm_delta_plan);
+
+/* the oracle's functions these forward to (ucm_oracle.c) */
+float orc_bf16_to_f32(uint16_t h);
+uint16_t orc_f32_to_bf16(float f);
+void orc_block_mean_paged(const uint16_t* k_cache, const int32_t* block_ids, const int32_t* slots, uint32_t n,
+                          uint32_t blockSize, uint32_t kHead, uint32_t headSize, float* repre, int round_bf16);
+void orc_q_head_mean(float* q, uint32_t kHead, uint32_t qHead, uint32_t headSize);
+void orc_kq_scores(const float* qMean, const float* kRepre, uint32_t numBlock, uint32_t kHead, uint32_t numKrepre,
+                   uint32_t headSize, float* scores);
+int32_t orc_topk_windows(const float* scores, uint32_t n, uint32_t k, uint32_t startW, uint32_t endW, int32_t* out);
+int32_t orc_block_table_gather(const int32_t* block_table, const int32_t* topk_idx, int32_t count, int32_t seq_len,
+                               int32_t block_size, int32_t* phys_out);
+int32_t orc_delta_plan(const int32_t* sel, const int32_t* sel_phys, int32_t count, int32_t* resident, int32_t n_slots,
+                       int32_t* load_phys, int32_t* slot_of_sel);
+
+int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
+                       const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, void* repre,
+                       int repre_rows, int64_t repre_layer_stride, int mode, ucm_stream_t stream)
+{
+    (void)stream;
+    if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
+    if (n == 0 || n_layers == 0) { return UCM_OK; }
+    if (!k_layers || !block_ids || !slots || !repre || num_blocks <= 0 || repre_rows <= 0 || block_size <= 0 ||
+        kv_heads <= 0 || head_dim <= 0 || mode < UCM_MEAN_F32 || mode > UCM_MEAN_BF16_STORE) {
+        return UCM_EINVAL;
+    }
+    const size_t row = (size_t)kv_heads * head_dim;
+    float* tmp = (float*)malloc(row * sizeof(float));
+    if (!tmp) { return UCM_ENOMEM; }
+    const int32_t zero = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        for (int i = 0; i < n; ++i) {
+            if (block_ids[i] < 0 || block_ids[i] >= num_blocks || slots[i] < 0 || slots[i] >= repre_rows) { continue; }
+            orc_block_mean_paged((const uint16_t*)k_layers[l], &block_ids[i], &zero, 1, (uint32_t)block_size,
+                                 (uint32_t)kv_heads, (uint32_t)head_dim, tmp, mode != UCM_MEAN_F32);
+            const size_t at = (size_t)l * (size_t)repre_layer_stride + (size_t)slots[i] * row;
+            if (mode == UCM_MEAN_BF16_STORE) {
+                for (size_t c = 0; c < row; ++c) { ((uint16_t*)repre)[at + c] = orc_f32_to_bf16(tmp[c]); }
+            } else {
+                memcpy((float*)repre + at, tmp, row * sizeof(float));
+            }
+        }
+    }
+    free(tmp);
+    return UCM_OK;
+}
+
+int ucm_score_blocks_cpu(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows, int q_heads,
+                         const void* repre, int repre_dtype, int64_t repre_layer_stride, const int32_t* seg_off,
+                         const int32_t* seg_len, int n_req, int max_seg_len, int64_t total_blocks, int n_layers,
+                         int kv_heads, int head_dim, float* scores, int64_t scores_layer_stride, float scale,
+                         int tile_blocks, ucm_stream_t stream)
+{
+    (void)stream;
+    (void)total_blocks;
+    (void)tile_blocks;
+    if (n_req < 0 || max_seg_len < 0 || n_layers < 0 || !isfinite(scale)) { return UCM_EINVAL; }
+    if (n_req == 0 || max_seg_len == 0 || n_layers == 0) { return UCM_OK; }
+    if (!q || !repre || !seg_off || !seg_len || !scores || kv_heads <= 0 || q_heads < kv_heads ||
+        q_heads % kv_heads != 0 || head_dim <= 0 || (q_dtype != UCM_DTYPE_F32 && q_dtype != UCM_DTYPE_BF16) ||
+        (repre_dtype != UCM_DTYPE_F32 && repre_dtype != UCM_DTYPE_BF16)) {
+        return UCM_EINVAL;
+    }
+    const size_t qrow = (size_t)q_heads * head_dim, row = (size_t)kv_heads * head_dim;
+    float* qf = (float*)malloc(qrow * sizeof(float));
+    float* wide = (float*)malloc((size_t)max_seg_len * row * sizeof(float));
+    if (!qf || !wide) { free(qf); free(wide); return UCM_ENOMEM; }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int r = 0; r < n_req; ++r) {
+            const int64_t qr = q_rows ? q_rows[r] : r;
+            const int32_t n = seg_len[r] < max_seg_len ? seg_len[r] : max_seg_len;
+            /* with q_rows, a layer's rows end at q_layer_stride: a request whose row lies outside is skipped */
+            if (n <= 0 || qr < 0 || (q_rows && (int64_t)(qr + 1) * (int64_t)qrow > q_layer_stride)) { continue; }
+            const size_t q_at = (size_t)l * (size_t)q_layer_stride + (size_t)qr * qrow;
+            for (size_t c = 0; c < qrow; ++c) {
+                qf[c] = q_dtype == UCM_DTYPE_F32 ? ((const float*)q)[q_at + c] : orc_bf16_to_f32(((const uint16_t*)q)[q_at + c]);
+            }
+            orc_q_head_mean(qf, (uint32_t)kv_heads, (uint32_t)q_heads, (uint32_t)head_dim);
+            const size_t t_at = (size_t)l * (size_t)repre_layer_stride + (size_t)seg_off[r] * row;
+            const float* table;
+            if (repre_dtype == UCM_DTYPE_F32) {
+                table = (const float*)repre + t_at;
+            } else {
+                for (size_t c = 0; c < (size_t)n * row; ++c) { wide[c] = orc_bf16_to_f32(((const uint16_t*)repre)[t_at + c]); }
+                table = wide;
+            }
+            float* out = scores + (size_t)l * (size_t)scores_layer_stride + seg_off[r];
+            orc_kq_scores(qf, table, (uint32_t)n, (uint32_t)kv_heads, 1, (uint32_t)head_dim, out);
+            for (int32_t b = 0; b < n; ++b) { out[b] = out[b] * scale; }
+        }
+    }
+    free(qf);
+    free(wide);
+    return UCM_OK;
+}
+
+int ucm_topk_windows_cpu(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off, const int32_t* seg_len,
+                         const int32_t* topk_len, int n_req, int max_seg_len, int n_layers, int start_w, int end_w,
+                         int32_t* idx_out, int out_stride, int32_t* count_out, const int32_t* block_tables, int bt_stride,
+                         int32_t* phys_out, const int32_t* seq_lens, int block_size, int32_t* sparse_seq_lens,
+                         ucm_stream_t stream)
+{
+    (void)stream;
+    if (n_req < 0 || n_layers < 0 || max_seg_len < 0 || start_w < 0 || end_w < 0) { return UCM_EINVAL; }
+    if (n_req == 0 || n_layers == 0) { return UCM_OK; }
+    if (!scores || !seg_off || !seg_len || !topk_len || !idx_out || !count_out || out_stride < max_seg_len ||
+        (block_tables && (!phys_out || bt_stride < max_seg_len)) || (seq_lens && (!sparse_seq_lens || block_size <= 0))) {
+        return UCM_EINVAL;
+    }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int r = 0; r < n_req; ++r) {
+            const size_t lr = (size_t)l * n_req + r;
+            const int32_t n = seg_len[r] < max_seg_len ? seg_len[r] : max_seg_len;
+            int32_t* out = idx_out + lr * (size_t)out_stride;
+            int32_t cnt = 0;
+            if (n > 0) {
+                cnt = orc_topk_windows(scores + (size_t)l * (size_t)scores_layer_stride + seg_off[r], (uint32_t)n,
+                                       (uint32_t)(topk_len[r] > 0 ? topk_len[r] : 0), (uint32_t)start_w, (uint32_t)end_w, out);
+            }
+            count_out[lr] = cnt;
+            int32_t sparse = 0;
+            if (block_tables) {
+                sparse = orc_block_table_gather(block_tables + (size_t)r * bt_stride, out, cnt, seq_lens ? seq_lens[r] : 0,
+                                                block_size > 0 ? block_size : 1, phys_out + lr * (size_t)out_stride);
+            }
+            if (seq_lens) {
+                if (!block_tables) {
+                    const int32_t rem = seq_lens[r] % block_size;
+                    sparse = rem == 0 ? cnt * block_size : cnt * block_size - block_size + rem;
+                }
+                /* every block kept: the request is not sparsified and keeps its length (prefetch_engine.py:547-553) */
+                sparse_seq_lens[lr] = cnt >= n ? seq_lens[r] : sparse;
+            }
+        }
+    }
+    return UCM_OK;
+}
+
+static int kv_move(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                   const int32_t* block_ids, int n, void* staging, int to_staging)
+{
+    if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
+    if (n == 0 || n_layers == 0) { return UCM_OK; }
+    if (!layers || !block_ids || !staging || num_blocks <= 0 || block_bytes == 0) { return UCM_EINVAL; }
+    for (int i = 0; i < n; ++i) {
+        if (block_ids[i] < 0 || block_ids[i] >= num_blocks) { continue; }
+        for (int l = 0; l < n_layers; ++l) {
+            for (int kv = 0; kv < 2; ++kv) {
+                uint8_t* c = (uint8_t*)layers[l] + (size_t)kv * kv_stride + (size_t)block_ids[i] * block_bytes;
+                uint8_t* s = (uint8_t*)staging + (((size_t)i * n_layers + l) * 2 + kv) * block_bytes;
+                if (to_staging) { memcpy(s, c, block_bytes); } else { memcpy(c, s, block_bytes); }
+            }
+        }
+    }
+    return UCM_OK;
+}
+
+int ucm_kv_gather_blocks_cpu(const void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                             const int32_t* block_ids, int n, void* staging, ucm_stream_t stream)
+{
+    (void)stream;
+    return kv_move((void* const*)layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging, 1);
+}
+
+int ucm_kv_scatter_blocks_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                              const int32_t* block_ids, int n, const void* staging, ucm_stream_t stream)
+{
+    (void)stream;
+    return kv_move(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, (void*)staging, 0);
+}
+
+int ucm_kv_gather_selected_cpu(const void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                               const int32_t* phys, const int32_t* count, int n_req, int phys_stride, const int64_t* dst_off,
+                               const int32_t* region_k, int max_count, void* staging, int64_t staging_blocks,
+                               ucm_stream_t stream)
+{
+    (void)stream;
+    if (n_req < 0 || n_layers < 0 || max_count < 0) { return UCM_EINVAL; }
+    if (n_req == 0 || n_layers == 0 || max_count == 0) { return UCM_OK; }
+    if (!layers || !phys || !count || !dst_off || !region_k || !staging || num_blocks <= 0 || block_bytes == 0 ||
+        phys_stride <= 0 || staging_blocks < 0) {
+        return UCM_EINVAL;
+    }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int r = 0; r < n_req; ++r) {
+            int32_t c = count[(size_t)l * n_req + r];
+            if (c > max_count) { c = max_count; }
+            if (dst_off[r] < 0 || region_k[r] < 0) { continue; }
+            for (int kv = 0; kv < 2; ++kv) {
+                for (int32_t j = 0; j < c; ++j) {
+                    const int32_t id = phys[((size_t)l * n_req + r) * (size_t)phys_stride + j];
+                    const int64_t dst = dst_off[r] + ((int64_t)l * 2 + kv) * region_k[r] + j;
+                    /* an id outside the cache (-1 marks a slot a delta plan leaves alone) or a destination
+                     * outside the staging buffer is skipped */
+                    if (id < 0 || id >= num_blocks || dst >= staging_blocks) { continue; }
+                    memcpy((uint8_t*)staging + (size_t)dst * block_bytes,
+                           (const uint8_t*)layers[l] + (size_t)kv * kv_stride + (size_t)id * block_bytes, block_bytes);
+                }
+            }
+        }
+    }
+    return UCM_OK;
+}
+
+int ucm_delta_plan_cpu(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, int n_req, int n_layers,
+                       int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys, int32_t* slot_of_sel,
+                       int32_t* miss_count, ucm_stream_t stream)
+{
+    (void)stream;
+    if (n_req < 0 || n_layers < 0) { return UCM_EINVAL; }
+    if (n_req == 0 || n_layers == 0) { return UCM_OK; }
+    if (!sel || !sel_phys || !count || !resident || !load_phys || !slot_of_sel || !miss_count || sel_stride <= 0 ||
+        n_slots <= 0) {
+        return UCM_EINVAL;
+    }
+    for (size_t lr = 0; lr < (size_t)n_layers * n_req; ++lr) {
+        int32_t c = count[lr] < 0 ? 0 : count[lr];
+        if (c > sel_stride) { c = sel_stride; }
+        miss_count[lr] = orc_delta_plan(sel + lr * (size_t)sel_stride, sel_phys + lr * (size_t)sel_stride, c,
+                                        resident + lr * (size_t)n_slots, n_slots, load_phys + lr * (size_t)n_slots,
+                                        slot_of_sel + lr * (size_t)sel_stride);
+    }
+    return UCM_OK;
+}

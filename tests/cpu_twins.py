@@ -1,0 +1,165 @@
+"""One scripted pass over the dense retrieval path - representatives, scores, selection with block-table lookup,
+delta plan, gathers and the block moves - written once against the C ABI's prototypes and run either through
+libucm_hip.so on device buffers or through the oracle's `_cpu` twins (oracle/ucm_cpu_abi.c) on host buffers.
+The argument lists of the two runs are identical except for where the pointers point."""
+import ctypes as C
+import os
+
+import numpy as np
+
+import oracle
+import synth
+
+TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
+         "ucm_kv_gather_selected", "ucm_delta_plan"]
+
+
+def twin_caller(signatures):
+    """call(name, *args) for the host twins, bound with the argument types the device library's binding uses."""
+    lib = C.CDLL(os.path.join(os.path.dirname(oracle.__file__), "liborc.so"))
+    for name in TWINS:
+        fn = getattr(lib, name + "_cpu")
+        fn.argtypes, fn.restype = signatures[name], C.c_int
+
+    def call(name, *args):
+        rc = getattr(lib, name + "_cpu")(*args)
+        if rc != 0:
+            raise RuntimeError(f"{name}_cpu returned {rc}")
+    return call
+
+
+class HostSide:
+    def up(self, a):
+        return np.ascontiguousarray(a).copy()
+
+    def ptr(self, a):
+        return a.ctypes.data
+
+    def pointers(self, arrays):
+        self._keep = getattr(self, "_keep", []) + [np.array([a.ctypes.data for a in arrays], np.uint64)]
+        return self._keep[-1].ctypes.data
+
+    def down(self, a):
+        return a
+
+    def sync(self):
+        pass
+
+
+class DeviceSide:
+    def __init__(self, ops, dev):
+        import torch
+
+        self.torch, self.ops, self.dev = torch, ops, dev
+
+    def up(self, a):
+        a = np.ascontiguousarray(a)
+        view = a.view(np.int16) if a.dtype == np.uint16 else a
+        return self.torch.from_numpy(view.copy()).to(self.dev)
+
+    def ptr(self, t):
+        return t.data_ptr()
+
+    def pointers(self, tensors):
+        self._keep = getattr(self, "_keep", []) + [self.ops.LayerPointers(tensors)]
+        return self._keep[-1].ptr()
+
+    def down(self, t):
+        a = t.cpu().numpy()
+        return a.view(np.uint16) if a.dtype == np.int16 else a
+
+    def sync(self):
+        self.torch.cuda.synchronize()
+
+
+L, NB, BS, HKV, D, G = 2, 12, 16, 2, 64, 4
+HQ, ROW = HKV * G, HKV * D
+BLOCK_BYTES = BS * HKV * D * 2
+KV_STRIDE = NB * BLOCK_BYTES
+LENS = np.array([4, 0, 6], np.int32)
+OFF = np.array([0, 4, 4], np.int32)
+ROWS = 10
+
+
+def inputs():
+    caches = [synth.normal_bf16_bits(7000 + l, (2, NB, BS, HKV, D)) for l in range(L)]
+    ids = synth.permutation(7010, NB)[:ROWS].astype(np.int32)
+    ids_bad = np.concatenate([ids, [-1, NB]]).astype(np.int32)        # two ids the call must skip
+    slots = np.concatenate([np.arange(ROWS), [3, 4]]).astype(np.int32)
+    q32 = synth.normal_f32(7020, (L, 5, HQ, D))
+    q16 = oracle.bf16_bits(synth.normal_f32(7021, (L, 5, HQ, D)))
+    q_rows = np.array([4, 1, 2], np.int32)
+    topk = np.array([3, 1, 4], np.int32)
+    tables = np.stack([synth.permutation(7030 + r, NB)[:8] for r in range(3)]).astype(np.int32)
+    seq_lens = np.array([4 * BS - 5, 0, 6 * BS], np.int32)
+    return dict(caches=caches, ids=ids_bad, slots=slots, q32=q32, q16=q16, q_rows=q_rows, topk=topk, tables=tables,
+                seq_lens=seq_lens)
+
+
+def run(call, side):
+    """Every output of the pass, as numpy arrays."""
+    x = inputs()
+    out = {}
+    caches = [side.up(c) for c in x["caches"]]
+    k_planes = side.pointers(caches)                                 # a layer's K plane comes first
+    ids, slots = side.up(x["ids"]), side.up(x["slots"])
+    n = len(x["ids"])
+    # 1. representatives in the three modes
+    tabs = {}
+    for mode, dtype in ((0, np.float32), (1, np.float32), (2, np.uint16)):
+        t = side.up(np.full((L, ROWS, ROW), 7, dtype))
+        call("ucm_block_mean", k_planes, L, NB, side.ptr(ids), side.ptr(slots), n, BS, HKV, D, side.ptr(t), ROWS, ROWS * ROW,
+             mode, None)
+        tabs[mode] = t
+        out[f"repre{mode}"] = t
+    # 2. scores: fp32 queries on the fp32 table; bf16 queries picked by q_rows on the bf16 table, scaled
+    seg_off, seg_len = side.up(OFF), side.up(LENS)
+    s32 = side.up(np.full((L, ROWS), -3, np.float32))
+    q32 = side.up(x["q32"])
+    call("ucm_score_blocks", side.ptr(q32), 0, 5 * HQ * D, None, HQ, side.ptr(tabs[0]), 0, ROWS * ROW, side.ptr(seg_off),
+         side.ptr(seg_len), 3, 6, 10, L, HKV, D, side.ptr(s32), ROWS, 1.0, 0, None)
+    s16 = side.up(np.full((L, ROWS), -3, np.float32))
+    q16, q_rows = side.up(x["q16"]), side.up(x["q_rows"])
+    call("ucm_score_blocks", side.ptr(q16), 1, 5 * HQ * D, side.ptr(q_rows), HQ, side.ptr(tabs[2]), 1, ROWS * ROW,
+         side.ptr(seg_off), side.ptr(seg_len), 3, 6, 0, L, HKV, D, side.ptr(s16), ROWS, 0.5, 0, None)
+    out["scores32"], out["scores16"] = s32, s16
+    # 3. selection with the block-table lookup and the sparse lengths
+    topk, tables, seq_lens = side.up(x["topk"]), side.up(x["tables"]), side.up(x["seq_lens"])
+    idx, phys = side.up(np.full((L, 3, 6), -1, np.int32)), side.up(np.full((L, 3, 6), -1, np.int32))
+    cnt, sparse = side.up(np.full((L, 3), -1, np.int32)), side.up(np.full((L, 3), -1, np.int32))
+    call("ucm_topk_windows", side.ptr(s16), ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk), 3, 6, L, 1, 1,
+         side.ptr(idx), 6, side.ptr(cnt), side.ptr(tables), 8, side.ptr(phys), side.ptr(seq_lens), BS, side.ptr(sparse), None)
+    out.update(idx=idx, phys=phys, cnt=cnt, sparse=sparse)
+    # 4. delta plan, twice: empty slots first, then the other scores' selection against what the first left
+    resident = side.up(np.full((L, 3, 4), -1, np.int32))
+    load, slot_of, miss = (side.up(np.full(s, -9, np.int32)) for s in ((L, 3, 4), (L, 3, 6), (L, 3)))
+    call("ucm_delta_plan", side.ptr(idx), side.ptr(phys), side.ptr(cnt), 3, L, 6, side.ptr(resident), 4, side.ptr(load),
+         side.ptr(slot_of), side.ptr(miss), None)
+    side.sync()
+    out.update(resident1=side.up(side.down(resident)), load1=side.up(side.down(load)), miss1=side.up(side.down(miss)))
+    idx2, phys2, cnt2 = (side.up(np.full(s, -1, np.int32)) for s in ((L, 3, 6), (L, 3, 6), (L, 3)))
+    call("ucm_topk_windows", side.ptr(s32), ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk), 3, 6, L, 1, 1,
+         side.ptr(idx2), 6, side.ptr(cnt2), side.ptr(tables), 8, side.ptr(phys2), None, BS, None, None)
+    call("ucm_delta_plan", side.ptr(idx2), side.ptr(phys2), side.ptr(cnt2), 3, L, 6, side.ptr(resident), 4, side.ptr(load),
+         side.ptr(slot_of), side.ptr(miss), None)
+    out.update(idx2=idx2, resident2=resident, load2=load, slot_of2=slot_of, miss2=miss)
+    # 5. gather of the first selection, and of the second plan's loads (its -1 entries are skipped)
+    layers = side.pointers(caches)
+    dst_off, region_k = side.up(np.array([0, 16, 16], np.int64)), side.up(np.array([4, 0, 4], np.int32))
+    for name, p, c in (("gathered", phys, cnt), ("loaded", load, side.up(np.full((L, 3), 4, np.int32)))):
+        staging = side.up(np.zeros((2 * 2 * L * 4, BLOCK_BYTES), np.uint8))
+        stride = 6 if name == "gathered" else 4
+        call("ucm_kv_gather_selected", layers, L, KV_STRIDE, BLOCK_BYTES, NB, side.ptr(p), side.ptr(c), 3, stride,
+             side.ptr(dst_off), side.ptr(region_k), 4, side.ptr(staging), 2 * 2 * L * 4, None)
+        out[name] = staging
+    # 6. block moves: out of the cache, and back into an empty one
+    move = side.up(np.array([5, -2, 0, 11], np.int32))
+    staging = side.up(np.zeros((4, L, 2, BLOCK_BYTES), np.uint8))
+    call("ucm_kv_gather_blocks", layers, L, KV_STRIDE, BLOCK_BYTES, NB, side.ptr(move), 4, side.ptr(staging), None)
+    empty = [side.up(np.zeros((2, NB, BS, HKV, D), np.uint16)) for _ in range(L)]
+    call("ucm_kv_scatter_blocks", side.pointers(empty), L, KV_STRIDE, BLOCK_BYTES, NB, side.ptr(move), 4, side.ptr(staging), None)
+    out["moved"] = staging
+    for l in range(L):
+        out[f"restored{l}"] = empty[l]
+    side.sync()
+    return {k: np.array(side.down(v)) for k, v in out.items()}, x

@@ -1,0 +1,44 @@
+"""The oracle's `_cpu` twins of the C ABI (oracle/ucm_cpu_abi.c): same prototypes as the device entry points, host
+pointers.  Here, without a GPU: they load with the device binding's argument types and reproduce the oracle's own
+functions on a scripted pass; with a GPU (tests/test_gpu_kernels.py) the same pass through libucm_hip.so gives the
+same bytes."""
+import numpy as np
+
+import cpu_twins
+import oracle as O
+
+
+def test_twins_reproduce_the_oracle(ucm):
+    from ucm_amd import _lib
+
+    got, x = cpu_twins.run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    L, ROWS, ROW, HKV = cpu_twins.L, cpu_twins.ROWS, cpu_twins.ROW, cpu_twins.HKV
+    ids, slots = x["ids"][:ROWS], x["slots"][:ROWS]            # the two out-of-range ids behind them are skipped
+    for l in range(L):
+        for mode, rounded in ((0, False), (1, True)):
+            want = np.full((ROWS, ROW), 7, np.float32)
+            O.block_mean_paged(x["caches"][l][0], ids, slots, want, round_bf16=rounded)
+            assert np.array_equal(got[f"repre{mode}"][l].view(np.uint32), want.view(np.uint32))
+        assert np.array_equal(got["repre2"][l], O.bf16_bits(got["repre1"][l]))
+    # scores and selection, per request, against the oracle's batch call
+    table16 = O.bf16_to_f32(got["repre2"])
+    for l in range(L):
+        q = O.bf16_to_f32(x["q16"][l][x["q_rows"]])
+        idx, cnt, scores = O.select_topk_bs(q, table16[l], cpu_twins.OFF, cpu_twins.LENS, x["topk"], HKV, start_w=1, end_w=1,
+                                            out_stride=6)
+        for r, (a, n) in enumerate(zip(cpu_twins.OFF, cpu_twins.LENS)):
+            assert np.array_equal(got["scores16"][l, a : a + n], scores[a : a + n] * np.float32(0.5))
+            assert got["cnt"][l, r] == cnt[r] and np.array_equal(got["idx"][l, r, : cnt[r]], idx[r, : cnt[r]])
+            assert np.array_equal(got["phys"][l, r, : cnt[r]], x["tables"][r][idx[r, : cnt[r]]])
+            if n:
+                assert got["sparse"][l, r] == (x["seq_lens"][r] if cnt[r] >= n else
+                                                O.block_table_gather(x["tables"][r], idx[r, : cnt[r]], int(x["seq_lens"][r]),
+                                                                     cpu_twins.BS)[1])
+    # the first plan fills empty slots in order; the moves restore exactly the listed blocks
+    assert np.array_equal(got["resident1"][:, 0, :3], got["idx"][:, 0, :3]) and (got["resident1"][:, 1] == -1).all()
+    assert np.array_equal(got["miss1"], got["cnt"])
+    for l in range(L):
+        want = np.zeros_like(x["caches"][l])
+        for b in (5, 0, 11):
+            want[:, b] = x["caches"][l][:, b]
+        assert np.array_equal(got[f"restored{l}"], want)

@@ -189,6 +189,32 @@ def test_bf16_table_scores_like_the_widened_table(ucm, dev, hkv, g, d, q_dtype):
         ops.set_score_tile(0)
 
 
+@pytest.mark.parametrize("hkv,g,d,repre_dtype", [(8, 4, 128, torch.bfloat16), (2, 8, 64, torch.float32)])
+def test_score_scale_gives_the_torch_variants_values(ucm, dev, hkv, g, d, repre_dtype):
+    """scale = 1/kv_heads turns the score into the mean over ALL q heads of q[h] . k[kv head of h], what the
+    reference's torch variant ranks by (TopkCal.cal_topk, ucm/sparse/gsa/gsa.py:386-412, one representative per
+    block); scale = 1 leaves the bits of the unscaled call."""
+    from ucm_amd import ops
+
+    n_layers, lens = 2, np.array([37, 0, 130, 5], np.int32)
+    rows, hq = int(lens.sum()), hkv * g
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    q = torch.from_numpy(synth.normal_f32(4100, (n_layers, len(lens), hq, d))).to(dev)
+    repre = torch.from_numpy(synth.normal_f32(4101, (n_layers, rows, hkv * d))).to(dev).to(repre_dtype)
+    plain, one, scaled = (torch.full((n_layers, rows), -5.0, device=dev) for _ in range(3))
+    args = (q, repre, i32(off, dev), i32(lens, dev), int(lens.max()), hkv)
+    ops.score_blocks(*args, plain)
+    ops.score_blocks(*args, one, scale=1.0)
+    ops.score_blocks(*args, scaled, scale=1.0 / hkv)
+    assert torch.equal(plain, one)
+    assert torch.equal(scaled, plain * np.float32(1.0 / hkv))          # one fp32 multiplication of the same score
+    # the torch variant's formula, in fp64: expand every kv head to its g query heads, dot, mean over the q heads
+    k = repre.double().view(n_layers, rows, hkv, 1, d).expand(-1, -1, -1, g, -1).reshape(n_layers, rows, hq, d)
+    for r, (a, n) in enumerate(zip(off, lens)):
+        want = torch.einsum("lhd,lbhd->lhb", q[:, r].double(), k[:, a : a + n]).mean(dim=1)
+        assert torch.allclose(scaled[:, a : a + n].double(), want, rtol=1e-5, atol=1e-5), r
+
+
 def test_bf16_table_from_the_paged_cache(ucm, dev):
     """keys -> bf16 means -> scores, against the oracle's rounded means; the bf16 table is the
     fp32 table of UCM_MEAN_BF16_ROUND with the low halves dropped."""
@@ -798,3 +824,19 @@ def test_decode_step_under_graph_capture(ucm, dev):
         for name, a, b in zip(("scores", "idx", "cnt", "phys", "staging"), g_bufs, e_bufs):
             assert torch.equal(a, b), (rep, name)
         assert int(e_bufs[2].min()) > 0                           # something was selected for every request
+
+
+def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
+    """One scripted pass over the dense path (three representative modes, both score variants with q_rows and a
+    scale, selection with block tables and sparse lengths, two delta plans, both gathers, block moves with ids to
+    skip) through libucm_hip.so on device buffers and through the oracle's `_cpu` twins on host buffers: the same
+    argument lists, the same bytes out."""
+    import cpu_twins
+    from ucm_amd import _lib, ops
+
+    want, _ = cpu_twins.run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    got, _ = cpu_twins.run(_lib.call, cpu_twins.DeviceSide(ops, dev))
+    assert got.keys() == want.keys()
+    for name in want:
+        assert got[name].dtype == want[name].dtype and got[name].shape == want[name].shape, name
+        assert np.array_equal(got[name].view(np.uint8), want[name].view(np.uint8)), name

@@ -11,14 +11,14 @@ OK, EINVAL, ENOTSUP, EHIP, ENOMEM = 0, -22, -95, -5, -12
 DTYPE_F32, DTYPE_BF16 = 0, 1
 MEAN_F32, MEAN_BF16_ROUND, MEAN_BF16_STORE = 0, 1, 2
 
-_p, _i, _i64, _sz = C.c_void_p, C.c_int, C.c_int64, C.c_size_t
+_p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 
 # name -> argtypes, in the order of include/ucm_hip.h
 SIGNATURES = {
     "ucm_version": [],
     "ucm_last_error": [],
     "ucm_block_mean": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i64, _i, _p],
-    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
+    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _f, _i, _p],
     "ucm_kvstar_block_repre": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _i, _p, _i64, _i, _i, _p, _i, _i64, _i64, _i64, _p],
     "ucm_kvstar_workspace_floats": [_i, _i, _i, _i, _i, _i, _i, _p, _p],
     "ucm_kvstar_votes": [_p, _p, _i, _i, _i, _p, _p, _p, _i64, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],

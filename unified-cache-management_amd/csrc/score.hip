@@ -18,6 +18,8 @@
 #include <algorithm>
 #include <cfloat>
 
+#include <cmath>
+
 #include "common.h"
 
 namespace {
@@ -148,7 +150,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
     const QT* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows, int q_heads,
     const float* __restrict__ repre, int64_t repre_layer_stride, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, int n_req, int kv_heads, float* __restrict__ scores,
-    int64_t scores_layer_stride, int tile_blocks)
+    int64_t scores_layer_stride, int tile_blocks, float scale)
 {
     constexpr int kSteps = kD / 16;
     __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
@@ -212,7 +214,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(
             s = s + fmaxf(-FLT_MAX, dh);
         }
         const int b = base + bl;
-        if (b < tile_end && h == 0 && m == 0) { sout[b] = s; }
+        if (b < tile_end && h == 0 && m == 0) { sout[b] = s * scale; }   // (a scale of 1 changes no bit)
     };
     while (b0 < tile_end) {
         const int b1 = b0 + stride;
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(
     const QT* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows, int q_heads,
     const uint16_t* __restrict__ repre, int64_t repre_layer_stride, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, int n_req, int kv_heads, float* __restrict__ scores,
-    int64_t scores_layer_stride, int tile_blocks)
+    int64_t scores_layer_stride, int tile_blocks, float scale)
 {
     constexpr int kSteps = kD / 16;
     __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(
             const float dh = __shfl(dot, (bl * kv_heads + hh) * 2, 64);
             s = s + fmaxf(-FLT_MAX, dh);
         }
-        sout[min(base + bl, tile_end - 1)] = s;   // the lanes of a block all hold its score
+        sout[min(base + bl, tile_end - 1)] = s * scale;   // the lanes of a block all hold its score; a scale of 1 changes no bit
     };
     while (b0 < tile_end) {
         const int b1 = b0 + stride;
@@ -357,24 +359,24 @@ template <int kD, typename QT>
 void launch_bf16(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
                  int64_t repre_layer_stride, const int32_t* seg_off, const int32_t* seg_len, int n_req,
                  int64_t tile_bound, int n_layers, int kv_heads, float* scores, int64_t scores_layer_stride,
-                 int tile_blocks, hipStream_t stream)
+                 int tile_blocks, float scale, hipStream_t stream)
 {
     hipLaunchKernelGGL((score_kernel_bf16<kD, QT>), dim3(static_cast<unsigned>(tile_bound), n_layers), dim3(kThreads), 0,
                        stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads,
                        static_cast<const uint16_t*>(repre), repre_layer_stride, seg_off, seg_len, n_req, kv_heads,
-                       scores, scores_layer_stride, tile_blocks);
+                       scores, scores_layer_stride, tile_blocks, scale);
 }
 
 template <int kD, typename QT>
 void launch(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
             int64_t repre_layer_stride, const int32_t* seg_off, const int32_t* seg_len, int n_req,
             int64_t tile_bound, int n_layers, int kv_heads, float* scores, int64_t scores_layer_stride,
-            int tile_blocks, hipStream_t stream)
+            int tile_blocks, float scale, hipStream_t stream)
 {
     hipLaunchKernelGGL((score_kernel<kD, QT>), dim3(static_cast<unsigned>(tile_bound), n_layers), dim3(kThreads), 0,
                        stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads,
                        static_cast<const float*>(repre), repre_layer_stride,
-                       seg_off, seg_len, n_req, kv_heads, scores, scores_layer_stride, tile_blocks);
+                       seg_off, seg_len, n_req, kv_heads, scores, scores_layer_stride, tile_blocks, scale);
 }
 
 }  // namespace
@@ -383,8 +385,9 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
                                 int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
                                 const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
                                 int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
-                                int64_t scores_layer_stride, int tile_blocks_arg, ucm_stream_t stream)
+                                int64_t scores_layer_stride, float scale, int tile_blocks_arg, ucm_stream_t stream)
 {
+    UCM_REQUIRE(std::isfinite(scale), "ucm_score_blocks: scale is not finite");
     UCM_REQUIRE(tile_blocks_arg >= 0 && tile_blocks_arg <= 4096, "ucm_score_blocks: tile_blocks=%d", tile_blocks_arg);
     UCM_REQUIRE(n_req == 0 || max_seg_len == 0 || (q && repre && seg_off && seg_len && scores),
                 "ucm_score_blocks: null pointer");
@@ -417,7 +420,7 @@ extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stri
     if (total_blocks > 0) { tile_bound = std::min(tile_bound, (total_blocks + tile_blocks - 1) / tile_blocks + n_req); }
     UCM_REQUIRE(tile_bound <= 0x7fffffffll, "ucm_score_blocks: too many tiles for one launch");
 #define UCM_SCORE_ARGS q, q_layer_stride, q_rows, q_heads, repre, repre_layer_stride, seg_off, seg_len, n_req, \
-                       tile_bound, n_layers, kv_heads, scores, scores_layer_stride, tile_blocks, s
+                       tile_bound, n_layers, kv_heads, scores, scores_layer_stride, tile_blocks, scale, s
     const bool qf = q_dtype == UCM_DTYPE_F32;
 #define UCM_SCORE_DIM(D)                                                                                        \
     do {                                                                                                        \

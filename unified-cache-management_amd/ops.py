@@ -96,10 +96,11 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
 def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor,
                  max_seg_len: int, kv_heads: int, scores: torch.Tensor,
                  q_rows: Optional[torch.Tensor] = None, first_layer: int = 0,
-                 n_layers: Optional[int] = None, total_blocks: int = 0) -> None:
+                 n_layers: Optional[int] = None, total_blocks: int = 0, scale: float = 1.0) -> None:
     """q: [L, rows, q_heads, head_dim] fp32 or bf16; repre: fp32 or bf16 [L, rows, kv_heads*head_dim];
     scores: fp32 [L, rows].  Layers first_layer .. first_layer+n_layers-1 are scored.
-    total_blocks: sum of seg_len when the host knows it (tighter grid), else 0."""
+    total_blocks: sum of seg_len when the host knows it (tighter grid), else 0.  scale multiplies every score
+    (1/kv_heads: the mean over all q heads the reference's torch variant ranks by)."""
     if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
         raise ValueError("q [L,rows,Hq,D], repre [L,rows,Hkv*D], scores [L,rows] expected")
     head_dim, q_heads = q.shape[3], q.shape[2]
@@ -131,7 +132,7 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
               _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
               total_blocks, n_layers, kv_heads, head_dim,
               _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4, scores.stride(0),
-              _tuning["score_tile"], _stream())
+              float(scale), _tuning["score_tile"], _stream())
 
 
 def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, topk_len: torch.Tensor,

@@ -413,7 +413,7 @@ class GSA(UcmSparseBase):
                 raise ValueError("query must be a contiguous device tensor [tokens, q_heads, head_size]")
             _lib.call("ucm_score_blocks", query.data_ptr(), q_code, query.numel(), q_rows, self.num_q_heads, repre,
                       self._repre_code, self.kpre_caches.stride(0), seg_off, seg_len, n, mi["max_len"], mi["total"], 1,
-                      self.num_key_heads, self.head_size, scores, self.scores.stride(0), 0, stream)
+                      self.num_key_heads, self.head_size, scores, self.scores.stride(0), 1.0, 0, stream)
         # selection (fresh scores, or the last ones with this step's lengths), block-table lookup, sparse lengths
         _lib.call("ucm_topk_windows", scores, self.scores.stride(0), seg_off, seg_len, topk_len, n, mi["max_len"], 1,
                   self.init_window, self.local_window, idx, self.max_block_len, counts, tables, self.max_block_len, phys,
