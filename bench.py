@@ -290,16 +290,16 @@ def main():
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / reps
 
-        gather_ms = timed_move(lambda: ops.kv_gather_blocks(layers, kv_stride, BLOCK_BYTES, nb, m_ids, m_stage))
+        mv_gather_ms = timed_move(lambda: ops.kv_gather_blocks(layers, kv_stride, BLOCK_BYTES, nb, m_ids, m_stage))
         scatter_ms = timed_move(lambda: ops.kv_scatter_blocks(layers, kv_stride, BLOCK_BYTES, nb, m_ids, m_stage))
         move_bytes = 2 * m_blocks * n_layers * 2 * BLOCK_BYTES
         moves_leg = {
             "workload": f"configs[2]: {m_blocks} blocks x {n_layers} layers x (K, V) x {BLOCK_BYTES} B, random block table over "
                         f"{nb} blocks per layer",
             "algorithmic_bytes": move_bytes,
-            "gather_ms": round(gather_ms, 3), "scatter_ms": round(scatter_ms, 3),
-            "gather_GBps": round(gbs(move_bytes, gather_ms), 1), "scatter_GBps": round(gbs(move_bytes, scatter_ms), 1),
-            "frac": [round(gbs(move_bytes, gather_ms) / HBM_PEAK_GBS, 4), round(gbs(move_bytes, scatter_ms) / HBM_PEAK_GBS, 4)],
+            "gather_ms": round(mv_gather_ms, 3), "scatter_ms": round(scatter_ms, 3),
+            "gather_GBps": round(gbs(move_bytes, mv_gather_ms), 1), "scatter_GBps": round(gbs(move_bytes, scatter_ms), 1),
+            "frac": [round(gbs(move_bytes, mv_gather_ms) / HBM_PEAK_GBS, 4), round(gbs(move_bytes, scatter_ms) / HBM_PEAK_GBS, 4)],
         }
         del m_stage
 
@@ -471,6 +471,8 @@ def main():
             "block_repre_ms_all": [round(x, 3) for x in krep_all],
             "block_repre_GBps": round(gbs(krep_bytes, krep_ms), 1),
             "block_repre_frac": round(gbs(krep_bytes, krep_ms) / HBM_PEAK_GBS, 4),
+            "block_repre_traffic": measured_traffic("kvstar_repre", "kvstar_repre_kernel", kv_default),
+            "block_repre_algorithmic_bytes": krep_bytes,
             "us_per_step": round(kv_ms * 1e3, 1),
             "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select)", "bound": "hbm",
                          "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
