@@ -195,3 +195,68 @@ def test_config5_full_size_hash_retrieval(ucm, dev):
                 assert np.array_equal(sc[a : a + n], want.astype(np.float32)), (l, mode, r)
                 sel = O.topk_windows(want.astype(np.int32), int(topk[r]))
                 assert cnt_h[r] == len(sel) and np.array_equal(idx_h[r, : len(sel)], sel), (l, mode, r)
+
+
+def test_config4_full_size_long_context_scores_selection_and_incremental_update(ucm, dev):
+    """8 requests of 512..1024 blocks (65536..131072 tokens), Qwen2-72B attention shape (64 query heads, 8 kv heads,
+    head_dim 128), all 80 layers, k = max(16, 2 %) + 1 first + 2 last blocks.  The representative table is the input
+    at this size (the keys of 80 layers would not fit the device: 8 x 1024 x 80 x 512 KiB); the incremental update
+    of a decode step - only the block a request just filled is reduced, every other row stays - is done on one
+    cache block per request and layer."""
+    from ucm_amd import ops
+
+    n_req, n_layers, hq, hkv, d, bs = 8, 80, 64, 8, 128, 128
+    row = hkv * d
+    lens = synth.ragged_lengths(2040, n_req, 65536, 131072)
+    assert lens.min() >= 512 and lens.max() <= 1024
+    topk = np.array([max(16, int(0.02 * n)) + 3 for n in lens], np.int32)
+    rows = int(lens.sum())
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    max_len = int(lens.max())
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2041)
+    # bf16 values both sides hold exactly: block means of N(0,1) keys have a standard deviation of 1/sqrt(128)
+    repre = (torch.empty((n_layers, rows, row), dtype=torch.float32, device=dev).normal_(generator=gen) * 0.0884).to(torch.bfloat16)
+    q = torch.empty((n_layers, n_req, hq, d), dtype=torch.bfloat16, device=dev).normal_(generator=gen)
+    seg_off, seg_len, topk_d = i32(off, dev), i32(lens, dev), i32(topk, dev)
+    scores = torch.zeros(n_layers, rows, device=dev)
+    idx = torch.full((n_layers, n_req, max_len), -1, dtype=torch.int32, device=dev)
+    cnt = torch.zeros(n_layers, n_req, dtype=torch.int32, device=dev)
+
+    def check(layers_to_check):
+        torch.cuda.synchronize()
+        q_h, sc_h, idx_h, cnt_h = q.float().cpu().numpy(), scores.cpu().numpy(), idx.cpu().numpy(), cnt.cpu().numpy()
+        for l in layers_to_check:
+            widx, wcnt, wsc = O.select_topk_bs(q_h[l], repre[l].float().cpu().numpy(), off, lens, topk, hkv, out_stride=max_len + 4)
+            assert np.array_equal(bits(wsc), bits(sc_h[l])), f"scores differ in layer {l}"
+            assert np.array_equal(wcnt, cnt_h[l]) and np.array_equal(wcnt, topk)
+            for r in range(n_req):
+                assert np.array_equal(widx[r, : wcnt[r]], idx_h[l, r, : wcnt[r]]), (l, r)
+                # what the rule fixes whatever the scores: first block, last two, ascending, no repeats
+                got = idx_h[l, r, : wcnt[r]]
+                assert got[0] == 0 and got[-1] == lens[r] - 1 and got[-2] == lens[r] - 2 and (np.diff(got) > 0).all()
+
+    ops.score_blocks(q, repre, seg_off, seg_len, max_len, hkv, scores, total_blocks=rows)
+    ops.topk_windows(scores, seg_off, seg_len, topk_d, max_len, idx, cnt)
+    check(range(n_layers))
+
+    # ---- decode step: each request's last block has just been filled; only its row of the table changes
+    nb = 2 * n_req
+    caches = [torch.empty((nb, bs, hkv, d), dtype=torch.bfloat16, device=dev).normal_(generator=gen) for _ in range(n_layers)]
+    new_ids = synth.permutation(2042, nb)[:n_req].astype(np.int32)
+    new_rows = (off + lens - 1).astype(np.int32)
+    before = repre.clone()
+    ops.block_mean(ops.LayerPointers(caches), i32(new_ids, dev), i32(new_rows, dev), repre, bs, hkv, d, nb)
+    torch.cuda.synchronize()
+    untouched = np.ones(rows, bool)
+    untouched[new_rows] = False
+    keep = torch.from_numpy(untouched).to(dev)
+    assert torch.equal(repre[:, keep], before[:, keep])
+    for l in (0, 41, n_layers - 1):
+        want = np.zeros((n_req, row), np.float32)
+        O.block_mean_paged(caches[l].view(torch.int16).cpu().numpy().view(np.uint16), new_ids, np.arange(n_req), want, round_bf16=True)
+        assert np.array_equal(bits(repre[l, torch.from_numpy(new_rows.astype(np.int64)).to(dev)].float().cpu().numpy()), bits(want))
+    q = torch.empty((n_layers, n_req, hq, d), dtype=torch.bfloat16, device=dev).normal_(generator=gen)
+    ops.score_blocks(q, repre, seg_off, seg_len, max_len, hkv, scores, total_blocks=rows)
+    ops.topk_windows(scores, seg_off, seg_len, topk_d, max_len, idx, cnt)
+    check((0, 17, 41, n_layers - 1))
