@@ -83,7 +83,8 @@ def test_esa_retrieve_wide_and_ragged_rows(ucm, dev):
     """Batch of requests, -1 padding in the middle, out-of-range slots, dims that are not a multiple of the tile."""
     from ucm_amd import ops
 
-    for rows, dim, b, m, topk in [(900, 1024, 4, 700, 210), (64, 36, 3, 9, 4), (3000, 256, 2, 2500, 900)]:
+    # the last case: the widest row the entry point takes (8192 candidates: the rank kernel's 64 KiB of dynamic LDS)
+    for rows, dim, b, m, topk in [(900, 1024, 4, 700, 210), (64, 36, 3, 9, 4), (3000, 256, 2, 2500, 900), (9000, 64, 2, 8192, 3000)]:
         data_h = synth.normal_bf16_as_f32(710 + dim, (rows, dim))
         q_h = synth.normal_bf16_as_f32(711 + dim, (b, dim))
         idx = np.stack([synth.permutation(712 + r, rows)[:m] for r in range(b)]).astype(np.int32)
