@@ -74,6 +74,10 @@ def parse():
                     help="hash leg: name only this many distinct cache blocks in the encode's block list, over and over "
                          "(8: the key loads are served from cache, which times the compute side of the kernel on its own); "
                          "0 = every block once")
+    ap.add_argument("--prefetch-leg", action="store_true",
+                    help="also time the GSA prefetch engine's round at this batch: hits / misses / free list of every "
+                         "(request, layer) on the device plus the loads of the served misses from a device-resident "
+                         "pool of stored blocks (needs about as much memory again as the KV cache)")
     ap.add_argument("--moves-leg", action="store_true",
                     help="also time the block-id driven load/dump (the configs[2] shape of the benchmark definition: 64 requests "
                          "x 16 blocks, all layers, K and V, random block table) on the same caches")
@@ -601,6 +605,138 @@ def main():
             "host_cpus": os.cpu_count(),
         }
 
+    # ---- prefetch leg: one round of the GSA prefetch engine per decode step - which selected blocks are resident,
+    # which free cache block takes each missing one, the new block tables - and the loads it plans, from a pool of
+    # stored blocks in device memory.  Runs last: it overwrites cache blocks.
+    prefetch_leg = None
+    if args.prefetch_leg:
+        from ucm_amd.sparse.gsa.gsa import GSAReqStat
+        from ucm_amd.sparse.gsa.prefetch import GSAPrefetchEngineC
+        from ucm_amd.sparse.utils import LOCAL_WINDOW_SZ, MAX_TOPK_LEN, MIN_TOPK_LEN, compute_topk_len
+
+        width = 64                                          # table row: MAX_TOPK_LEN + 1 resident blocks fit
+        i32z = lambda *shape: torch.zeros(shape, dtype=torch.int32, device=dev)
+        p_free, p_free_len = i32z(n_layers, N_REQ, width), i32z(n_layers, N_REQ)
+        p_succ, p_succ_len = i32z(n_layers, N_REQ, width), i32z(n_layers, N_REQ)
+        eng = GSAPrefetchEngineC(p_free, p_succ, p_free_len, p_succ_len, False)
+        p_topk_h = np.array([compute_topk_len(int(n)) for n in lens], np.int32)      # 30 % of the blocks, 32..48
+        resident_h = []
+        for r in range(N_REQ):
+            n = int(lens[r])
+            st_ = GSAReqStat(r, 0, BS, 0)
+            st_.blocks = [int(x) for x in bt_h[r, :n]]
+            st_.num_prompt_tokens = st_.num_computed_tokens = n * BS
+            st_.get_sparse_and_free_block(True, MIN_TOPK_LEN, MAX_TOPK_LEN, 0.3)
+            # positions 0..MAX_TOPK_LEN of the request's block list are the cache blocks it keeps; the last
+            # LOCAL_WINDOW_SZ of the used ones hold the request's last logical blocks (prefetch_engine.py:327-379)
+            used, spare = st_.remain_idx, st_.prefetch_idx
+            logical = spare + used[:-LOCAL_WINDOW_SZ] + list(range(n - LOCAL_WINDOW_SZ, n))
+            holder = {i: st_.blocks[i] for i in spare + used[:-LOCAL_WINDOW_SZ]}
+            holder.update({n - LOCAL_WINDOW_SZ + j: st_.blocks[p_] for j, p_ in enumerate(used[-LOCAL_WINDOW_SZ:])})
+            eng.set_blocks_map(r, holder, logical)
+            p_free[:, r, : len(spare)] = i32([st_.blocks[x] for x in spare])
+            p_free_len[:, r] = len(spare)
+            resident_h.append((holder, logical, [st_.blocks[x] for x in spare]))
+        pool = torch.empty((rows, n_layers, 2, BLOCK_BYTES), dtype=torch.uint8, device=dev)
+        for l0 in range(0, rows, 256):
+            pool[l0 : l0 + 256].random_(generator=g)
+        src_table = torch.full((N_REQ, max_len), -1, dtype=torch.int32, device=dev)
+        for r in range(N_REQ):
+            src_table[eng.row_of(r), : lens[r]] = torch.arange(int(seg_off_h[r]), int(seg_off_h[r] + lens[r]), dtype=torch.int32, device=dev)
+        p_topk = i32(p_topk_h)
+        p_idx = torch.full((n_layers, N_REQ, max_len), -1, dtype=torch.int32, device=dev)
+        p_cnt = torch.zeros(n_layers, N_REQ, dtype=torch.int32, device=dev)
+        req_ids, bs_idx, tk_list = list(range(N_REQ)), list(range(N_REQ)), [int(k) for k in p_topk_h]
+        rho = args.delta_rho
+        q_cur = qs[0].float()
+        n_rounds = 4 + min(args.steps, 16)
+        ev_p = [[ev() for _ in range(4)] for _ in range(n_rounds)]
+        loads_per_round, topk_rounds = [], []
+        for t in range(n_rounds):
+            if t:
+                q_cur = rho * q_cur + (1.0 - rho * rho) ** 0.5 * torch.randn(q_cur.shape, device=dev, generator=g)
+            ops.score_blocks(q_cur.to(torch.bfloat16), repre, seg_off, seg_len, max_len, HKV, scores, total_blocks=rows)
+            ops.topk_windows(scores, seg_off, seg_len, p_topk, max_len, p_idx, p_cnt)
+            sel = p_idx[:, :, :MAX_TOPK_LEN].contiguous()
+            ev_p[t][0].record()
+            eng.set_blocks_table_info(p_succ, p_succ_len, sel, t)
+            ev_p[t][1].record()
+            eng.run_async_prefetch_bs(req_ids, tk_list, bs_idx, 0)
+            ev_p[t][2].record()
+            eng.load_missing(layers, kv_stride, BLOCK_BYTES, nb, pool.view(-1), n_layers * 2 * BLOCK_BYTES, src_table)
+            ev_p[t][3].record()
+            loads_per_round.append(eng.load_count.sum())
+            topk_rounds.append(sel)
+        torch.cuda.synchronize()
+        p_ms = np.array([[e[i].elapsed_time(e[i + 1]) for i in range(3)] for e in ev_p[4:]]).mean(0)   # rounds 0-3 warm the set up
+        loads_h = [int(x) for x in loads_per_round]
+        steady = float(np.mean(loads_h[4:]))
+        sel_per_round = int(p_topk_h.sum()) * n_layers
+        load_bytes = 2 * steady * 2 * BLOCK_BYTES
+        p_checked = None
+        if not args.no_check:
+            # the blocks the last round loaded hold the bytes of the stored blocks it named
+            lb, mi = eng.obtain_load_blocks(), eng.obtain_miss_idxs()
+            n_cmp = 0
+            for r in range(N_REQ):
+                for l in (0, n_layers // 2, n_layers - 1):
+                    for blk, idx_ in zip(lb[r][l], mi[r][l]):
+                        for kv in range(2):
+                            got = caches[l][kv][blk].view(torch.uint8).reshape(-1)
+                            assert torch.equal(got, pool[int(seg_off_h[r]) + idx_, l, kv]), f"prefetch load differs ({r},{l},{blk})"
+                        n_cmp += 1
+            p_checked = f"{n_cmp} blocks loaded by the last round (3 layers x all requests) hold the stored blocks' bytes, K and V"
+        # the reference's own engine (kvcache_pre.cpp compiled against torch into oracle/_ref) on the same rounds
+        cpu_round_us = None
+        if not args.no_cpu:
+            import oracle
+
+            gp = oracle.ref.gsa_prefetch_module()
+            if gp is not None:
+                c32 = dict(dtype=torch.int32)
+                c_free, c_free_len = torch.zeros((n_layers, N_REQ, width), **c32), torch.zeros((n_layers, N_REQ), **c32)
+                c_succ, c_succ_len = torch.zeros((n_layers, N_REQ, width), **c32), torch.zeros((n_layers, N_REQ), **c32)
+                ceng = gp.GSAPrefetchEngineC(c_free, c_succ, c_free_len, c_succ_len, False)
+                for r, (holder, logical, spare_blocks) in enumerate(resident_h):
+                    table_list = [0] * int(lens[r])
+                    for i_, b_ in holder.items():
+                        table_list[i_] = b_
+                    ceng.set_blocks_map(r, table_list, logical)
+                    c_free[:, r, : len(spare_blocks)] = torch.tensor(spare_blocks, **c32)
+                    c_free_len[:, r] = len(spare_blocks)
+                t_cpu = []
+                for t, sel in enumerate(topk_rounds):
+                    buf = sel.cpu().to(torch.int64)
+                    s0 = time.perf_counter()
+                    ceng.set_blocks_table_info(c_succ, c_succ_len, buf, t)
+                    ceng.run_async_prefetch_bs(req_ids, tk_list, bs_idx, 0)
+                    while not ceng.get_prefetch_status():
+                        time.sleep(0.00005)
+                    t_cpu.append(time.perf_counter() - s0)
+                cpu_round_us = float(np.mean(t_cpu[4:]) * 1e6)
+                assert torch.equal(c_succ_len, p_succ_len.cpu()) and torch.equal(c_succ, p_succ.cpu()), \
+                    "device and reference engines left different block tables"
+        prefetch_leg = {
+            "workload": f"{N_REQ} requests x {n_layers} layers, {MAX_TOPK_LEN + 1} cache blocks kept per request, "
+                        f"{int(p_topk_h.min())}-{int(p_topk_h.max())} blocks selected per (request, layer), consecutive queries "
+                        f"correlated with rho = {rho} (synthetic), stored blocks [block][layer][K|V] in device memory",
+            "us_per_round": round(float(p_ms.sum()) * 1e3, 1),
+            "table_info_us": round(float(p_ms[0]) * 1e3, 1),
+            "plan_us": round(float(p_ms[1]) * 1e3, 1),
+            "loads_us": round(float(p_ms[2]) * 1e3, 1),
+            "blocks_selected_per_round": sel_per_round,
+            "blocks_loaded_per_round": round(steady, 1),
+            "hit_rate": round(1.0 - steady / sel_per_round, 4),
+            "loads_GBps": round(gbs(load_bytes, float(p_ms[2])), 1) if steady else None,
+            "cpu_reference_plan_us": None if cpu_round_us is None else round(cpu_round_us, 1),
+            "cpu_reference": None if cpu_round_us is None else
+                "GSAPrefetchEngineC of the reference (kvcache_pre.cpp, its worker thread + 16 OpenMP threads over layers) on the "
+                "same selections: set_blocks_table_info + run_async_prefetch_bs until get_prefetch_status(); bookkeeping "
+                "only, the reference loads through its store connector afterwards; tables equal the device's",
+            "checked": p_checked,
+        }
+        del pool
+
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly this workload
     # (profiles/bench_config2_kernels.md); other workloads have no measurement
     default_workload = n_layers == N_LAYERS and args.seed == 2024
@@ -659,6 +795,7 @@ def main():
                                "frac": round(gbs(mean_bytes, mean_ms) / HBM_PEAK_GBS, 4)},
         "delta_gather": delta,
         "kv_moves": moves_leg,
+        "prefetch_round": prefetch_leg,
         "hash_retrieval": hash_leg,
         "esa_retrieval": esa_leg,
         "kvstar_retrieval": kvstar_leg,

@@ -98,7 +98,8 @@ __global__ __launch_bounds__(kThreads) void kv_gather_selected_kernel(
 
 // Loads planned on the device: slot j of request row `row` receives logical block load_sel[l][row][j] (or
 // nothing, -1) from a pool of stored blocks laid out [block][layer][K|V].
-// grid: x = slot, y = request of the call, z = layer*2 + K|V
+// grid: x = slot (stepping by the grid: most slots of most rows have nothing to load, and a workgroup of this
+// size that only finds that out costs microseconds), y = request of the call, z = layer*2 + K|V
 __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
     void* const* __restrict__ layers, size_t kv_stride, size_t block_bytes, unsigned num_blocks,
     const uint8_t* __restrict__ pool, uint64_t pool_blocks, size_t pool_block_bytes, unsigned store_first_layer,
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
     const int32_t* __restrict__ dst_table, unsigned dst_stride, int64_t dst_layer_stride,
     const int32_t* __restrict__ load_count, const int32_t* __restrict__ rows, unsigned table_rows)
 {
-    const unsigned j = blockIdx.x, b = blockIdx.y, l = blockIdx.z >> 1, kv = blockIdx.z & 1;
+    const unsigned b = blockIdx.y, l = blockIdx.z >> 1, kv = blockIdx.z & 1;
     unsigned row = b;
     if (rows) {
         const int32_t r = rows[b];
@@ -114,17 +115,92 @@ __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
         row = static_cast<unsigned>(r);
     }
     if (row >= table_rows) { return; }
-    if (load_count && static_cast<int32_t>(j) >= load_count[static_cast<size_t>(l) * table_rows + row]) { return; }
-    const int32_t sel = load_sel[(static_cast<size_t>(l) * table_rows + row) * n_slots + j];
-    if (sel < 0 || static_cast<unsigned>(sel) >= src_stride) { return; }     // slot keeps what it holds
-    const int32_t src = src_table[static_cast<size_t>(row) * src_stride + sel];
-    if (src < 0 || static_cast<uint64_t>(src) >= pool_blocks) { return; }   // block not in the pool
-    const unsigned dst = static_cast<unsigned>(dst_table[l * dst_layer_stride + static_cast<int64_t>(row) * dst_stride + j]);
-    if (dst >= num_blocks) { return; }
-    copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
-               pool + static_cast<size_t>(src) * pool_block_bytes +
-                   (static_cast<size_t>(store_first_layer + l) * 2 + kv) * block_bytes,
-               block_bytes);
+    unsigned limit = n_slots;
+    if (load_count) { limit = min(limit, static_cast<unsigned>(max(load_count[static_cast<size_t>(l) * table_rows + row], 0))); }
+    for (unsigned j = blockIdx.x; j < limit; j += gridDim.x) {    // (uniform: every thread of the workgroup takes the same trips)
+        const int32_t sel = load_sel[(static_cast<size_t>(l) * table_rows + row) * n_slots + j];
+        if (sel < 0 || static_cast<unsigned>(sel) >= src_stride) { continue; }     // slot keeps what it holds
+        const int32_t src = src_table[static_cast<size_t>(row) * src_stride + sel];
+        if (src < 0 || static_cast<uint64_t>(src) >= pool_blocks) { continue; }   // block not in the pool
+        const unsigned dst = static_cast<unsigned>(dst_table[l * dst_layer_stride + static_cast<int64_t>(row) * dst_stride + j]);
+        if (dst >= num_blocks) { continue; }
+        copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
+                   pool + static_cast<size_t>(src) * pool_block_bytes +
+                       (static_cast<size_t>(store_first_layer + l) * 2 + kv) * block_bytes,
+                   block_bytes);
+    }
+}
+
+// The same loads when every row says how many of its leading entries are loads (load_count): the work is
+// known exactly, so it is dealt out evenly.  Every workgroup builds the running total of the (layer, request)
+// pairs' counts in LDS (a few hundred integers), and takes the copies w, w + grid, ... of the 2 * total
+// (K and V); which pair a copy belongs to is a binary search in the totals.  grid: x = workgroup.
+constexpr unsigned kMaxPlannedPairs = 4096;
+
+__global__ __launch_bounds__(kThreads) void kv_load_counted_kernel(
+    void* const* __restrict__ layers, size_t kv_stride, size_t block_bytes, unsigned num_blocks,
+    const uint8_t* __restrict__ pool, uint64_t pool_blocks, size_t pool_block_bytes, unsigned store_first_layer,
+    const int32_t* __restrict__ load_sel, unsigned n_slots, const int32_t* __restrict__ src_table, unsigned src_stride,
+    const int32_t* __restrict__ dst_table, unsigned dst_stride, int64_t dst_layer_stride,
+    const int32_t* __restrict__ load_count, const int32_t* __restrict__ rows, unsigned table_rows, unsigned batch,
+    unsigned n_layers)
+{
+    __shared__ unsigned s_total[kMaxPlannedPairs + 1];   // s_total[p] = loads of the pairs before p
+    __shared__ unsigned s_part[kThreads];
+    const unsigned pairs = n_layers * batch;             // pair p = layer p / batch, request p % batch
+    constexpr unsigned kPer = kMaxPlannedPairs / kThreads;
+    unsigned mine[kPer], sum = 0;
+#pragma unroll
+    for (unsigned i = 0; i < kPer; ++i) {
+        const unsigned p = threadIdx.x * kPer + i;
+        unsigned c = 0;
+        if (p < pairs) {
+            const unsigned l = p / batch, b = p - l * batch;
+            const int32_t r = rows ? rows[b] : static_cast<int32_t>(b);
+            if (r >= 0 && static_cast<unsigned>(r) < table_rows) {
+                c = min(n_slots, static_cast<unsigned>(max(load_count[static_cast<size_t>(l) * table_rows + r], 0)));
+            }
+        }
+        mine[i] = c;
+        sum += c;
+    }
+    s_part[threadIdx.x] = sum;
+    __syncthreads();
+    for (unsigned d = 1; d < kThreads; d <<= 1) {         // inclusive scan of the threads' sums
+        const unsigned v = threadIdx.x >= d ? s_part[threadIdx.x - d] : 0u;
+        __syncthreads();
+        s_part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    unsigned run = s_part[threadIdx.x] - sum;
+#pragma unroll
+    for (unsigned i = 0; i < kPer; ++i) {
+        s_total[threadIdx.x * kPer + i] = run;
+        run += mine[i];
+    }
+    if (threadIdx.x == kThreads - 1) { s_total[kMaxPlannedPairs] = run; }
+    __syncthreads();
+    const unsigned copies = 2u * s_total[kMaxPlannedPairs];
+    for (unsigned w = blockIdx.x; w < copies; w += gridDim.x) {   // (uniform in the workgroup)
+        const unsigned t = w >> 1, kv = w & 1u;
+        unsigned lo = 0, hi = pairs;                     // last pair whose running total is <= t
+        while (hi - lo > 1) {
+            const unsigned mid = (lo + hi) >> 1;
+            if (s_total[mid] <= t) { lo = mid; } else { hi = mid; }
+        }
+        const unsigned l = lo / batch, b = lo - l * batch, j = t - s_total[lo];
+        const unsigned row = static_cast<unsigned>(rows ? rows[b] : static_cast<int32_t>(b));
+        const int32_t sel = load_sel[(static_cast<size_t>(l) * table_rows + row) * n_slots + j];
+        if (sel < 0 || static_cast<unsigned>(sel) >= src_stride) { continue; }
+        const int32_t src = src_table[static_cast<size_t>(row) * src_stride + sel];
+        if (src < 0 || static_cast<uint64_t>(src) >= pool_blocks) { continue; }
+        const unsigned dst = static_cast<unsigned>(dst_table[l * dst_layer_stride + static_cast<int64_t>(row) * dst_stride + j]);
+        if (dst >= num_blocks) { continue; }
+        copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
+                   pool + static_cast<size_t>(src) * pool_block_bytes +
+                       (static_cast<size_t>(store_first_layer + l) * 2 + kv) * block_bytes,
+                   block_bytes);
+    }
 }
 
 constexpr size_t kBatchPiece = 2 * kStep;  // 256 KiB
@@ -233,11 +309,23 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
                 store_first_layer + n_layers - 1, pool_block_bytes);
     UCM_REQUIRE(src_stride >= 1 && dst_stride >= n_slots && dst_layer_stride >= 0,
                 "ucm_kv_load_planned: src_stride=%d dst_stride=%d n_slots=%d", src_stride, dst_stride, n_slots);
-    hipLaunchKernelGGL(kv_load_planned_kernel, dim3(static_cast<unsigned>(n_slots), batch, n_layers * 2), dim3(kThreads), 0,
-                       ucm::as_stream(stream), layers, kv_stride, block_bytes, static_cast<unsigned>(num_blocks),
-                       static_cast<const uint8_t*>(pool), static_cast<uint64_t>(pool_blocks), pool_block_bytes,
-                       static_cast<unsigned>(store_first_layer), load_sel, static_cast<unsigned>(n_slots), src_table,
-                       static_cast<unsigned>(src_stride), dst_table, static_cast<unsigned>(dst_stride), dst_layer_stride,
-                       load_count, rows, static_cast<unsigned>(table_rows));
+    if (load_count && static_cast<unsigned>(n_layers) * static_cast<unsigned>(batch) <= kMaxPlannedPairs) {
+        // the rows' counts say exactly what there is to copy: 1024 workgroups share it evenly
+        hipLaunchKernelGGL(kv_load_counted_kernel, dim3(1024), dim3(kThreads), 0, ucm::as_stream(stream), layers, kv_stride,
+                           block_bytes, static_cast<unsigned>(num_blocks), static_cast<const uint8_t*>(pool),
+                           static_cast<uint64_t>(pool_blocks), pool_block_bytes, static_cast<unsigned>(store_first_layer),
+                           load_sel, static_cast<unsigned>(n_slots), src_table, static_cast<unsigned>(src_stride), dst_table,
+                           static_cast<unsigned>(dst_stride), dst_layer_stride, load_count, rows,
+                           static_cast<unsigned>(table_rows), static_cast<unsigned>(batch), static_cast<unsigned>(n_layers));
+    } else {
+        // the entries to load are scattered over a row (or there are too many rows for the counted kernel's table)
+        const unsigned gx = static_cast<unsigned>(std::min(n_slots, load_count ? 8 : 16));
+        hipLaunchKernelGGL(kv_load_planned_kernel, dim3(gx, batch, n_layers * 2), dim3(kThreads), 0,
+                           ucm::as_stream(stream), layers, kv_stride, block_bytes, static_cast<unsigned>(num_blocks),
+                           static_cast<const uint8_t*>(pool), static_cast<uint64_t>(pool_blocks), pool_block_bytes,
+                           static_cast<unsigned>(store_first_layer), load_sel, static_cast<unsigned>(n_slots), src_table,
+                           static_cast<unsigned>(src_stride), dst_table, static_cast<unsigned>(dst_stride), dst_layer_stride,
+                           load_count, rows, static_cast<unsigned>(table_rows));
+    }
     UCM_LAUNCH_CHECK("ucm_kv_load_planned");
 }

@@ -179,6 +179,10 @@ class GSAPrefetchEngineC:
                       for l in range(self.n_layers)] for req, row in self._row_of.items()}
 
     # ---- device-side consumers ----------------------------------------------------------------------------
+    def row_of(self, req_id: int) -> int:
+        """Row of the engine's tables (and of load_missing's src_table) that holds the request, -1 if unknown."""
+        return self._row_of.get(int(req_id), -1)
+
     def run_rows_device(self) -> torch.Tensor:
         """Table rows of the last round's requests (int32 device tensor; -1 for requests the engine does not know)."""
         return self._run_dev[1][0]
