@@ -119,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void prefetch_plan_kernel(
     const bool eligible = n_miss > 0 && free_slot >= 0 && s_hit[free_slot] == 0;
     int n_eligible;
     const int el_rank = block_rank(eligible, s_cnt, n_eligible);
-    const int n_load = min(n_eligible, n_miss);
+    const int n_load = min(min(n_eligible, n_miss), cap);   // (a free list that names a block twice could outnumber the slots)
     if (eligible && el_rank < n_load) {
         const int32_t want = s_miss[el_rank];
         load_blocks[lr * cap + el_rank] = free_id;
