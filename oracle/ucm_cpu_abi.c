@@ -32,6 +32,9 @@ TWIN(ucm_kv_gather_blocks);
 TWIN(ucm_kv_scatter_blocks);
 TWIN(ucm_kv_gather_selected);
 TWIN(ucm_delta_plan);
+TWIN(ucm_hash_encode_blocks);
+TWIN(ucm_hash_encode_queries);
+TWIN(ucm_hash_score_blocks);
 
 /* the oracle's functions these forward to (ucm_oracle.c) */
 float orc_bf16_to_f32(uint16_t h);
@@ -46,6 +49,16 @@ int32_t orc_block_table_gather(const int32_t* block_table, const int32_t* topk_i
                                int32_t block_size, int32_t* phys_out);
 int32_t orc_delta_plan(const int32_t* sel, const int32_t* sel_phys, int32_t count, int32_t* resident, int32_t n_slots,
                        int32_t* load_phys, int32_t* slot_of_sel);
+void orc_hash_encode(const uint16_t* x, const float* W, uint32_t n, uint32_t dim, uint32_t bits, uint8_t* codes);
+void orc_hash_encode_f32(const float* x, const float* W, uint32_t n, uint32_t dim, uint32_t bits, uint8_t* codes);
+void orc_hash_colsum(const uint8_t* token_codes, uint32_t n_blocks, uint32_t block_size, uint32_t kv_heads, uint32_t nbytes,
+                     int16_t* out);
+void orc_hash_majority(const uint8_t* token_codes, uint32_t n_blocks, uint32_t block_size, uint32_t kv_heads, uint32_t nbytes,
+                       uint8_t* block_codes);
+void orc_hash_scores_block(const uint8_t* q_codes, const uint8_t* block_codes, uint32_t n_blocks, uint32_t kv_heads,
+                           uint32_t nbytes, int32_t* scores);
+float orc_f16_to_f32(uint16_t h);
+uint16_t orc_f32_to_f16(float f);
 
 int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
                        const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, void* repre,
@@ -253,6 +266,147 @@ int ucm_delta_plan_cpu(const int32_t* sel, const int32_t* sel_phys, const int32_
         miss_count[lr] = orc_delta_plan(sel + lr * (size_t)sel_stride, sel_phys + lr * (size_t)sel_stride, c,
                                         resident + lr * (size_t)n_slots, n_slots, load_phys + lr * (size_t)n_slots,
                                         slot_of_sel + lr * (size_t)sel_stride);
+    }
+    return UCM_OK;
+}
+
+/* ------------------------------------------------------------ hash codes */
+
+static float* widen_weights(const void* w_bf16, int head_dim, int bits)
+{
+    float* w = (float*)malloc((size_t)head_dim * bits * sizeof(float));
+    if (w) {
+        for (size_t i = 0; i < (size_t)head_dim * bits; ++i) { w[i] = orc_bf16_to_f32(((const uint16_t*)w_bf16)[i]); }
+    }
+    return w;
+}
+
+int ucm_hash_encode_blocks_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
+                               const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, const void* w_bf16,
+                               int bits, int rows, uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                               int64_t colsum_layer_stride, uint8_t* block_codes, int64_t block_codes_layer_stride,
+                               int workgroups, ucm_stream_t stream)
+{
+    (void)stream;
+    (void)workgroups;
+    if (n < 0) { return UCM_EINVAL; }
+    if (n == 0) { return UCM_OK; }
+    if (!k_layers || !w_bf16 || !colsum || !block_codes || n_layers <= 0 || num_blocks <= 0 || rows <= 0 || block_size <= 0 ||
+        kv_heads <= 0) {
+        return UCM_EINVAL;
+    }
+    if (head_dim != 128 || bits != 128) { return UCM_ENOTSUP; }
+    const uint32_t nbytes = (uint32_t)bits / 8;
+    const size_t n_vec = (size_t)block_size * kv_heads;
+    float* w = widen_weights(w_bf16, head_dim, bits);
+    uint8_t* codes = (uint8_t*)malloc(n_vec * nbytes);
+    if (!w || !codes) { free(w); free(codes); return UCM_ENOMEM; }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int i = 0; i < n; ++i) {
+            /* block_ids NULL: item i is block i; slots NULL: it goes to row i */
+            const int64_t id = block_ids ? block_ids[i] : i, slot = slots ? slots[i] : i;
+            if (id < 0 || id >= num_blocks || slot < 0 || slot >= rows) { continue; }
+            const uint16_t* x = (const uint16_t*)k_layers[l] + (size_t)id * n_vec * head_dim;
+            orc_hash_encode(x, w, (uint32_t)n_vec, (uint32_t)head_dim, (uint32_t)bits, codes);
+            if (token_codes) {
+                memcpy(token_codes + (size_t)l * (size_t)token_codes_layer_stride + (size_t)slot * n_vec * nbytes, codes,
+                       n_vec * nbytes);
+            }
+            orc_hash_colsum(codes, 1, (uint32_t)block_size, (uint32_t)kv_heads, nbytes,
+                            colsum + (size_t)l * (size_t)colsum_layer_stride + (size_t)slot * kv_heads * bits);
+            orc_hash_majority(codes, 1, (uint32_t)block_size, (uint32_t)kv_heads, nbytes,
+                              block_codes + (size_t)l * (size_t)block_codes_layer_stride + (size_t)slot * kv_heads * nbytes);
+        }
+    }
+    free(w);
+    free(codes);
+    return UCM_OK;
+}
+
+int ucm_hash_encode_queries_cpu(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows, int n_req, int n_layers,
+                                int q_heads, int kv_heads, int head_dim, const void* w_bf16, int bits, uint8_t* q_codes,
+                                int16_t* q_sum, uint8_t* qbar_codes, ucm_stream_t stream)
+{
+    (void)stream;
+    if (n_req < 0 || n_layers < 0) { return UCM_EINVAL; }
+    if (n_req == 0 || n_layers == 0) { return UCM_OK; }
+    if (!q_bf16 || !w_bf16 || !q_codes || !q_sum || !qbar_codes || kv_heads <= 0 || q_heads < kv_heads ||
+        q_heads % kv_heads != 0) {
+        return UCM_EINVAL;
+    }
+    if (head_dim != 128 || bits != 128) { return UCM_ENOTSUP; }
+    const uint32_t nbytes = (uint32_t)bits / 8;
+    const size_t qrow = (size_t)q_heads * head_dim;
+    float* w = widen_weights(w_bf16, head_dim, bits);
+    float* qf = (float*)malloc(qrow * sizeof(float));
+    if (!w || !qf) { free(w); free(qf); return UCM_ENOMEM; }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int r = 0; r < n_req; ++r) {
+            const int64_t qr = q_rows ? q_rows[r] : r;
+            if (qr < 0 || (q_rows && (int64_t)(qr + 1) * (int64_t)qrow > q_layer_stride)) { continue; }   /* left as they were */
+            const uint16_t* x = (const uint16_t*)q_bf16 + (size_t)l * (size_t)q_layer_stride + (size_t)qr * qrow;
+            const size_t lr = (size_t)l * n_req + r;
+            uint8_t* codes = q_codes + lr * q_heads * nbytes;
+            orc_hash_encode(x, w, (uint32_t)q_heads, (uint32_t)head_dim, (uint32_t)bits, codes);
+            for (int c = 0; c < bits; ++c) {
+                int32_t ones = 0;
+                for (int h = 0; h < q_heads; ++h) { ones += (codes[(size_t)h * nbytes + c / 8] >> (c % 8)) & 1; }
+                q_sum[lr * bits + c] = (int16_t)(2 * ones - q_heads);
+            }
+            /* the kv head's group-mean query in fp32 (select_topk_block.cpp:101-114), then its code */
+            for (size_t c = 0; c < qrow; ++c) { qf[c] = orc_bf16_to_f32(x[c]); }
+            orc_q_head_mean(qf, (uint32_t)kv_heads, (uint32_t)q_heads, (uint32_t)head_dim);
+            orc_hash_encode_f32(qf, w, (uint32_t)kv_heads, (uint32_t)head_dim, (uint32_t)bits, qbar_codes + lr * kv_heads * nbytes);
+        }
+    }
+    free(w);
+    free(qf);
+    return UCM_OK;
+}
+
+int ucm_hash_score_blocks_cpu(int mode, const int16_t* q_sum, const uint8_t* qbar_codes, const int16_t* colsum,
+                              int64_t colsum_layer_stride, const uint8_t* block_codes, int64_t block_codes_layer_stride,
+                              const int32_t* seg_off, const int32_t* seg_len, int n_req, int64_t total_blocks, int n_layers,
+                              int kv_heads, int bits, float* scores, int64_t scores_layer_stride, int round_fp16,
+                              ucm_stream_t stream)
+{
+    (void)stream;
+    (void)total_blocks;
+    if (n_req < 0 || n_layers < 0 || (mode != 0 && mode != 1)) { return UCM_EINVAL; }
+    if (n_req == 0 || n_layers == 0) { return UCM_OK; }
+    if (!seg_off || !seg_len || !scores || kv_heads <= 0 || (mode == 0 && (!q_sum || !colsum)) ||
+        (mode == 1 && (!qbar_codes || !block_codes))) {
+        return UCM_EINVAL;
+    }
+    if (bits != 128) { return UCM_ENOTSUP; }
+    const uint32_t nbytes = (uint32_t)bits / 8;
+    for (int l = 0; l < n_layers; ++l) {
+        for (int r = 0; r < n_req; ++r) {
+            const size_t lr = (size_t)l * n_req + r;
+            float* out = scores + (size_t)l * (size_t)scores_layer_stride + seg_off[r];
+            for (int32_t b = 0; b < seg_len[r]; ++b) {
+                const size_t row = (size_t)seg_off[r] + b;
+                if (mode == 0) {
+                    /* <sum of the query heads' +-1 codes, sum over kv heads of the block's column sums>: the reference's
+                     * triple sum of +-1 inner products (kvcomp.py:237-247) as one integer */
+                    int64_t s = 0;
+                    const int16_t* cs = colsum + (size_t)l * (size_t)colsum_layer_stride + row * kv_heads * bits;
+                    for (int c = 0; c < bits; ++c) {
+                        int32_t col = 0;
+                        for (int h = 0; h < kv_heads; ++h) { col += cs[(size_t)h * bits + c]; }
+                        s += (int64_t)q_sum[lr * bits + c] * col;
+                    }
+                    float f = (float)s;
+                    out[b] = round_fp16 ? orc_f16_to_f32(orc_f32_to_f16(f)) : f;
+                } else {
+                    int32_t s = 0;
+                    orc_hash_scores_block(qbar_codes + lr * kv_heads * nbytes,
+                                          block_codes + (size_t)l * (size_t)block_codes_layer_stride + row * kv_heads * nbytes, 1,
+                                          (uint32_t)kv_heads, nbytes, &s);
+                    out[b] = (float)s;
+                }
+            }
+        }
     }
     return UCM_OK;
 }

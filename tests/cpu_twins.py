@@ -11,7 +11,8 @@ import oracle
 import synth
 
 TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
-         "ucm_kv_gather_selected", "ucm_delta_plan"]
+         "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
+         "ucm_hash_score_blocks"]
 
 
 def twin_caller(signatures):
@@ -54,8 +55,11 @@ class DeviceSide:
 
     def up(self, a):
         a = np.ascontiguousarray(a)
-        view = a.view(np.int16) if a.dtype == np.uint16 else a
-        return self.torch.from_numpy(view.copy()).to(self.dev)
+        view = a.view(np.int16) if a.dtype == np.uint16 else a      # torch has no uint16 arithmetic type to hold bf16 bits
+        t = self.torch.from_numpy(view.copy()).to(self.dev)
+        if a.dtype == np.uint16:
+            self._u16 = getattr(self, "_u16", set()) | {t.data_ptr()}
+        return t
 
     def ptr(self, t):
         return t.data_ptr()
@@ -66,7 +70,7 @@ class DeviceSide:
 
     def down(self, t):
         a = t.cpu().numpy()
-        return a.view(np.uint16) if a.dtype == np.int16 else a
+        return a.view(np.uint16) if t.data_ptr() in getattr(self, "_u16", set()) else a
 
     def sync(self):
         self.torch.cuda.synchronize()
@@ -161,5 +165,49 @@ def run(call, side):
     out["moved"] = staging
     for l in range(L):
         out[f"restored{l}"] = empty[l]
+    side.sync()
+    return {k: np.array(side.down(v)) for k, v in out.items()}, x
+
+
+HL, HNB, HBS, HHKV, HHQ, HD = 2, 7, 16, 2, 8, 128
+H_LENS = np.array([3, 0, 2], np.int32)
+H_OFF = np.array([0, 3, 3], np.int32)
+H_ROWS = 6
+
+
+def hash_inputs():
+    keys = [synth.normal_bf16_bits(7100 + l, (HNB, HBS, HHKV, HD)) for l in range(HL)]
+    w = oracle.bf16_bits(synth.normal_f32(7110, (HD, 128)) * np.float32(2.0))
+    q = synth.normal_bf16_bits(7111, (HL, 4, HHQ, HD))
+    ids = np.array([4, 0, 6, -3, 2, 1, 5, HNB], np.int32)              # two ids the call must skip
+    slots = np.array([0, 1, 2, 3, 3, 4, 5, 5], np.int32)
+    return dict(keys=keys, w=w, q=q, ids=ids, slots=slots, q_rows=np.array([3, 0, 1], np.int32))
+
+
+def run_hash(call, side):
+    """The hash-code path: block codes and summaries, query codes, both scores."""
+    x = hash_inputs()
+    keys = [side.up(k) for k in x["keys"]]
+    w, q = side.up(x["w"]), side.up(x["q"])
+    ids, slots, q_rows = side.up(x["ids"]), side.up(x["slots"]), side.up(x["q_rows"])
+    tcodes = side.up(np.full((HL, H_ROWS, HBS, HHKV, 16), 0xEE, np.uint8))
+    colsum = side.up(np.full((HL, H_ROWS, HHKV, 128), 77, np.int16))
+    bcodes = side.up(np.full((HL, H_ROWS, HHKV, 16), 0xEE, np.uint8))
+    call("ucm_hash_encode_blocks", side.pointers(keys), HL, HNB, side.ptr(ids), side.ptr(slots), len(x["ids"]), HBS, HHKV, HD,
+         side.ptr(w), 128, H_ROWS, side.ptr(tcodes), H_ROWS * HBS * HHKV * 16, side.ptr(colsum), H_ROWS * HHKV * 128,
+         side.ptr(bcodes), H_ROWS * HHKV * 16, 0, None)
+    q_codes = side.up(np.full((HL, 3, HHQ, 16), 0xEE, np.uint8))
+    q_sum = side.up(np.full((HL, 3, 128), 77, np.int16))
+    qbar = side.up(np.full((HL, 3, HHKV, 16), 0xEE, np.uint8))
+    call("ucm_hash_encode_queries", side.ptr(q), 4 * HHQ * HD, side.ptr(q_rows), 3, HL, HHQ, HHKV, HD, side.ptr(w), 128,
+         side.ptr(q_codes), side.ptr(q_sum), side.ptr(qbar), None)
+    seg_off, seg_len = side.up(H_OFF), side.up(H_LENS)
+    out = dict(token_codes=tcodes, colsum=colsum, block_codes=bcodes, q_codes=q_codes, q_sum=q_sum, qbar=qbar)
+    for name, mode, fp16 in (("score_sum", 0, 0), ("score_sum_fp16", 0, 1), ("score_code", 1, 0)):
+        sc = side.up(np.full((HL, H_ROWS), -3, np.float32))
+        call("ucm_hash_score_blocks", mode, side.ptr(q_sum), side.ptr(qbar), side.ptr(colsum), H_ROWS * HHKV * 128,
+             side.ptr(bcodes), H_ROWS * HHKV * 16, side.ptr(seg_off), side.ptr(seg_len), 3, 5, HL, HHKV, 128, side.ptr(sc),
+             H_ROWS, fp16, None)
+        out[name] = sc
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x

@@ -42,3 +42,29 @@ def test_twins_reproduce_the_oracle(ucm):
         for b in (5, 0, 11):
             want[:, b] = x["caches"][l][:, b]
         assert np.array_equal(got[f"restored{l}"], want)
+
+
+def test_hash_twins_reproduce_the_oracle(ucm):
+    from ucm_amd import _lib
+
+    got, x = cpu_twins.run_hash(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    w = O.bf16_to_f32(x["w"])
+    live = [i for i, b in enumerate(x["ids"]) if 0 <= b < cpu_twins.HNB]
+    # a slot named twice keeps the later block (the calls are serial on the host)
+    final = {int(x["slots"][i]): int(x["ids"][i]) for i in live}
+    for l in range(cpu_twins.HL):
+        for slot, blk in final.items():
+            codes = O.hash_encode(x["keys"][l][blk], w)                      # [tokens, kv heads, 16]
+            assert np.array_equal(got["token_codes"][l, slot], codes)
+            assert np.array_equal(got["colsum"][l, slot], O.hash_colsum(codes[None])[0])
+            assert np.array_equal(got["block_codes"][l, slot], O.hash_majority(codes[None])[0])
+        for r, row in enumerate(x["q_rows"]):
+            qc = O.hash_encode(x["q"][l, row], w)
+            assert np.array_equal(got["q_codes"][l, r], qc)
+            for a, n in ((cpu_twins.H_OFF[r], cpu_twins.H_LENS[r]),):
+                if n:
+                    keys = np.ascontiguousarray(got["token_codes"][l, a : a + n].transpose(0, 2, 1, 3))   # [block, head, token, 16]
+                    assert np.array_equal(got["score_sum"][l, a : a + n], O.hash_scores_sum(qc, keys).astype(np.float32))
+                    assert np.array_equal(got["score_code"][l, a : a + n],
+                                          O.hash_scores_block(got["qbar"][l, r], got["block_codes"][l, a : a + n]).astype(np.float32))
+    assert np.array_equal(got["score_sum_fp16"], got["score_sum"].astype(np.float16).astype(np.float32))

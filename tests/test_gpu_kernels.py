@@ -834,9 +834,10 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     import cpu_twins
     from ucm_amd import _lib, ops
 
-    want, _ = cpu_twins.run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
-    got, _ = cpu_twins.run(_lib.call, cpu_twins.DeviceSide(ops, dev))
-    assert got.keys() == want.keys()
-    for name in want:
-        assert got[name].dtype == want[name].dtype and got[name].shape == want[name].shape, name
-        assert np.array_equal(got[name].view(np.uint8), want[name].view(np.uint8)), name
+    for run in (cpu_twins.run, cpu_twins.run_hash):      # the dense path; the hash-code path
+        want, _ = run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+        got, _ = run(_lib.call, cpu_twins.DeviceSide(ops, dev))
+        assert got.keys() == want.keys()
+        for name in want:
+            assert got[name].dtype == want[name].dtype and got[name].shape == want[name].shape, name
+            assert np.array_equal(got[name].view(np.uint8), want[name].view(np.uint8)), name
