@@ -1,6 +1,6 @@
 /*
  * Host twins of the C ABI: the same prototypes as libucm_hip.so's entry points
- * of the dense retrieval path, name + "_cpu", every "dev" pointer a host
+ * of the dense retrieval path and of the hash-code path, name + "_cpu", every "dev" pointer a host
  * pointer, `stream` ignored, the work done before the call returns.  A caller
  * written against one prototype switches between host and device by choosing
  * the symbol.
