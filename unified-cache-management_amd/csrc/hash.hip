@@ -113,8 +113,10 @@ __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen,
 {
     // the code words stored by this wave must have reached L2 before they are patched there;
     // waiting for the stores' acknowledgements is enough (a device-scope fence would write back the whole L2)
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
+    if (tc_out) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+    }
     for (int base = 0; base < qlen; base += 64) {
         if (base + lane < qlen) {
             const unsigned e = ws.queue[base + lane];
@@ -154,6 +156,48 @@ __device__ __forceinline__ void planes_flush(unsigned (&pl)[kPlanes], int* __res
         for (int p = 0; p < kPlanes; ++p) { cnt |= static_cast<int>((pl[p] >> b) & 1u) << p; }
         const int col = (2 * wp + (b >> 4)) * 32 + half * 16 + (b & 15);
         if (cnt) { atomicAdd(&head_row[col], cnt); }
+    }
+#pragma unroll
+    for (int p = 0; p < kPlanes; ++p) { pl[p] = 0u; }
+}
+
+// The same for eight kv heads, without atomics: the four lanes of a lane half that hold vectors of one head
+// (lr, lr ^ 8, lr ^ 16, lr ^ 24) first add their counts up - as bytes, four to a register: a plane set counts at
+// most 63 tiles, four lanes 252 - and lane lr < 8 then owns head lr's sixteen columns of each of the two column
+// blocks outright.  (Thirty-two LDS atomics per lane with four lanes on every address took four times as long as
+// everything else a block needs at its end.)
+__device__ __forceinline__ void planes_flush_heads8(unsigned (&pl)[kPlanes], int* __restrict__ colsum, int wp, int half, int lr)
+{
+    unsigned cnt[8];                                     // byte k of cnt[j]: count of bit 4j + k
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        unsigned c = 0u;
+#pragma unroll
+        for (int p = 0; p < kPlanes; ++p) {
+            const unsigned nib = (pl[p] >> (4 * j)) & 0xfu;
+            c += ((nib * 0x00204081u) & 0x01010101u) << p;   // bit i of the nibble -> byte i
+        }
+        c += __shfl_xor(c, 8, 64);
+        c += __shfl_xor(c, 16, 64);
+        cnt[j] = c;
+    }
+    if (lr < 8) {
+        int* row = colsum + lr * kBits + half * 16;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {              // bits 16*blk .. 16*blk+15 are columns (2*wp + blk)*32 + half*16 + 0..15
+            int* dst = row + (2 * wp + blk) * 32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const unsigned c = cnt[4 * blk + q];
+                typedef int i32x4 __attribute__((ext_vector_type(4)));
+                i32x4 v = *reinterpret_cast<i32x4*>(dst + 4 * q);
+                v.x += static_cast<int>(c & 0xffu);
+                v.y += static_cast<int>((c >> 8) & 0xffu);
+                v.z += static_cast<int>((c >> 16) & 0xffu);
+                v.w += static_cast<int>(c >> 24);
+                *reinterpret_cast<i32x4*>(dst + 4 * q) = v;
+            }
+        }
     }
 #pragma unroll
     for (int p = 0; p < kPlanes; ++p) { pl[p] = 0u; }
@@ -213,7 +257,9 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     }
     __syncthreads();
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wave index through readfirstlane: the item a wave works on is then known to be the same for all lanes,
+    // and its block id and slot are read with scalar loads, which do not queue behind the key loads in flight
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int half = lane >> 5, lr = lane & 31;
     const unsigned l = blockIdx.y;
     const unsigned n_vec = tokens * kv_heads;            // vectors of kDim bf16 in a block
@@ -252,13 +298,19 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     bool prefetched = false;                             // k_a / k_b already hold (or await) this item's first tiles
 
     const unsigned item_step = gridDim.x * kWaves;
-    for (unsigned item = blockIdx.x * kWaves + wave; item < n_items; item += item_step) {
-        unsigned slot = 0, next_slot = 0;
-        const unsigned short* blk = item_keys(item, slot);
-        if (!blk) { prefetched = false; continue; }
+    const unsigned first_item = blockIdx.x * kWaves + wave;
+    unsigned carried_slot = 0;                           // the item looked up as the one before's successor
+    const unsigned short* carried_blk = item_keys(first_item, carried_slot);
+    for (unsigned item = first_item; item < n_items; item += item_step) {
+        unsigned next_slot = 0;
+        const unsigned slot = carried_slot;
+        const unsigned short* blk = carried_blk;
         // the tiles after this item's last one come from the next item of this wave, so its
         // first keys are on their way while this item's summaries are written
         const unsigned short* next_blk = item_keys(item + item_step, next_slot);
+        carried_blk = next_blk;
+        carried_slot = next_slot;
+        if (!blk) { prefetched = false; continue; }
         const bool chain = next_blk != nullptr && n_tiles >= 2;
         if (!chain) { next_blk = blk; }
         unsigned* tc_out = kTokenCodes ? token_codes + (static_cast<int64_t>(l) * tc_layer_stride +
@@ -270,6 +322,15 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         for (int p = 0; p < kPlanes; ++p) { planes01[p] = 0u; planes23[p] = 0u; }
         unsigned pending = 0;                            // tiles counted in the planes
         int qlen = 0;
+        auto flush_planes = [&]() {
+            if (kv_heads == 8) {                         // (uniform)
+                planes_flush_heads8(planes01, &ws.colsum[0][0], 0, half, lr);
+                planes_flush_heads8(planes23, &ws.colsum[0][0], 1, half, lr);
+            } else {
+                planes_flush(planes01, head_row, 0, half);
+                planes_flush(planes23, head_row, 1, half);
+            }
+        };
 
         // A tile's code words are stored one trip late, at the start of the next tile's work:
         // a store issued just before the wait for the next keys would be waited for as well.
@@ -304,12 +365,41 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         // of this one), so two tiles are in flight per wave for most of the time without a
         // third buffer.  The reload is unconditional: one skipped on some path would make
         // the compiler wait for everything outstanding.
+        // Without token codes there are sixteen registers to spare, and the weight fragments of the first step
+        // of a tile stay in them for the whole kernel: no tile then starts with a wait for LDS, and an eighth of
+        // the LDS reads is gone.  With token codes the fragments are requested first thing in a tile, ahead of
+        // the wait for the keys and of their norms.
+        constexpr bool kResidentFirst = !kTokenCodes;
+        bf16x8 wf_first[4];
+        if (kResidentFirst) {
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+                wf_first[nb] = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64]);
+            }
+        }
         auto process = [&](u32x4 (&kb)[8], unsigned tile) {
+            bf16x8 wf[2][4];
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb) {
+                if (kResidentFirst) { wf[0][nb] = wf_first[nb]; }
+                else { wf[0][nb] = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64]); }
+            }
+            __builtin_amdgcn_sched_barrier(0);
             store_codes();
 
-            float xn2 = 0.0f;                            // ||x||^2 of vector lr
+            // ||x||^2 of vector lr, in four partial sums: one chain of thirty-two dependent dot instructions
+            // would leave the wave waiting on each one's latency
+            float xp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) { xn2 = norm2_acc(kb[ks], xn2); }
+            for (int ks = 0; ks < 8; ++ks) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const unsigned e = kb[ks][j];
+                    const bf16x2 p = __builtin_bit_cast(bf16x2, e);
+                    xp[j] = __builtin_amdgcn_fdot2_f32_bf16(p, p, xp[j], false);
+                }
+            }
+            float xn2 = (xp[0] + xp[1]) + (xp[2] + xp[3]);
             xn2 += __shfl_xor(xn2, 32, 64);
             const float sx = sqrtf(xn2);
 
@@ -319,15 +409,22 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
 #pragma unroll
                 for (int i = 0; i < 16; ++i) { acc[nb][i] = 0.0f; }
             }
+            // the weight fragments of a step are read from LDS while the matrix instructions of the step before run
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 const bf16x8 kf = __builtin_bit_cast(bf16x8, kb[ks]);
+                if (ks < 7) {
+#pragma unroll
+                    for (int nb = 0; nb < 4; ++nb) {
+                        wf[(ks + 1) & 1][nb] = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64 + (ks + 1) * 8]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) {
-                    const bf16x8 wf = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 64 + ks * 8]);
-                    acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, kf, acc[nb], 0, 0, 0);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks & 1][nb], kf, acc[nb], 0, 0, 0);
                 }
-                __builtin_amdgcn_sched_barrier(0);       // keep the weight fragments of later steps out of registers
+                __builtin_amdgcn_sched_barrier(0);
             }
             {
                 const unsigned t2 = tile + 2;
@@ -372,39 +469,41 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                 pend_tile = tile;
             }
 
-            // second look, only at the flagged column blocks: the sign of |acc| - bound marks
-            // the doubtful ones of a lane's sixteen results (one sub and one v_alignbit each,
-            // no LDS, no branches), and the lanes that have any pop them into the queue.
-            // The provisional bit of an entry is read back from the packed sign word.
+            // second look, only at the flagged column blocks (with Gaussian keys about one block
+            // per tile is flagged, so all four flags are tested with one branch first): the sign of
+            // |acc| - bound marks the doubtful ones of a lane's sixteen results (one sub and one
+            // v_alignbit each, no LDS, no branches), and the lanes that have any pop them into the
+            // queue.  The provisional bit of an entry is read back from the packed sign word.
+            if (doubt[0] | doubt[1] | doubt[2] | doubt[3]) {
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
-                if (doubt[nb]) {
-                    const float bound = sw[nb] * sx;     // an all-zero key has bound 0: nothing is below it
-                    unsigned mask = 0u;
+                for (int nb = 0; nb < 4; ++nb) {
+                    if (doubt[nb]) {
+                        const float bound = sw[nb] * sx;     // an all-zero key has bound 0: nothing is below it
+                        unsigned mask = 0u;
 #pragma unroll
-                    for (int i = 15; i >= 0; --i) {
-                        mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(__builtin_fabsf(acc[nb][i]) - bound), 31);
-                    }
-                    const unsigned signs = pair[nb >> 1] >> (16 * (nb & 1));
-                    unsigned long long um = __ballot(mask != 0u);
-                    while (um) {
-                        if (qlen + 64 > kQueueCap) { drain_queue(); }
-                        if (mask) {
-                            const unsigned i = static_cast<unsigned>(__builtin_ctz(mask));
-                            mask &= mask - 1u;
-                            const unsigned col = nb * 32 + half * 16 + i;
-                            ws.queue[qlen + static_cast<int>(lanes_below(um))] =
-                                ((tile * 32 + lr) << 8) | (col << 1) | ((signs >> i) & 1u);
+                        for (int i = 15; i >= 0; --i) {
+                            mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(__builtin_fabsf(acc[nb][i]) - bound), 31);
                         }
-                        qlen += __popcll(um);
-                        um = __ballot(mask != 0u);
+                        const unsigned signs = pair[nb >> 1] >> (16 * (nb & 1));
+                        unsigned long long um = __ballot(mask != 0u);
+                        while (um) {
+                            if (qlen + 64 > kQueueCap) { drain_queue(); }
+                            if (mask) {
+                                const unsigned i = static_cast<unsigned>(__builtin_ctz(mask));
+                                mask &= mask - 1u;
+                                const unsigned col = nb * 32 + half * 16 + i;
+                                ws.queue[qlen + static_cast<int>(lanes_below(um))] =
+                                    ((tile * 32 + lr) << 8) | (col << 1) | ((signs >> i) & 1u);
+                            }
+                            qlen += __popcll(um);
+                            um = __ballot(mask != 0u);
+                        }
                     }
                 }
             }
 
             if (pending == kFlushTiles) {
-                planes_flush(planes01, head_row, 0, half);
-                planes_flush(planes23, head_row, 1, half);
+                flush_planes();
                 pending = 0;
             }
         };
@@ -430,8 +529,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         }
         store_codes();
         if (qlen > 0) { drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
-        planes_flush(planes01, head_row, 0, half);
-        planes_flush(planes23, head_row, 1, half);
+        flush_planes();
 
         // ---- block summaries
         // (LDS operations of one wave complete in order; no barrier is needed inside the wave)
