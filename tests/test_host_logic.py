@@ -316,3 +316,29 @@ def test_gsa_prefetch_mode_resident_set_and_slots(ucm):
     assert plugin.estimate_num_slots_sparsed(ns(num_prompt_tokens=9000, num_output_tokens=0, num_tokens=9000)) == INVALID_SLOT
     off = GSA(make_config(), UcmSparseRole.SCHEDULER)
     assert off.estimate_num_slots_sparsed(ns(num_prompt_tokens=100 * 128, num_output_tokens=5, num_tokens=100 * 128 + 5)) == INVALID_SLOT
+
+
+def test_kvcomp_reads_the_reference_config_file(ucm, tmp_path):
+    """KvComp takes head_dim and hash_bits from the reference's JSON (kvcomp_config.py:36-80; the files under
+    kvcomp/configs have these keys) and refuses one written for a model with another number of layers
+    (kvcomp.py:452-464)."""
+    import json
+
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.kvcomp.kvcomp import KvComp
+
+    js = {"model_name": "Qwen/Qwen3-4B", "is_mla": False, "hash_weight_type": "random", "num_hidden_layers": 36,
+          "seq_len_threshhold": 2048, "chunk_size": 128, "chunk_repre_method": "max", "head_dim": 128,
+          "hash_bits": 128, "top_k_ratio_per_layer": [1, 1] + [0.3] * 34, "top_k_index_reuse": [-1] * 36,
+          "must_select_blocks": [0, -2, -1], "hash_weight": None}
+    path = tmp_path / "kvcomp.json"
+    path.write_text(json.dumps(js))
+    cfg = make_config("KvComp", {})
+    cfg.parallel_config = ns(rank=0, tensor_parallel_size=1)
+    cfg.kv_transfer_config.kv_connector_extra_config["kvcomp_config_path"] = str(path)
+    cfg.model_config.hf_text_config = ns(num_hidden_layers=36)
+    plugin = KvComp(cfg, UcmSparseRole.SCHEDULER)
+    assert plugin.cfg["head_dim"] == 128 and plugin.cfg["hash_bits"] == 128
+    cfg.model_config.hf_text_config = ns(num_hidden_layers=32)
+    with pytest.raises(AssertionError, match="num_hidden_layers 36"):
+        KvComp(cfg, UcmSparseRole.SCHEDULER)

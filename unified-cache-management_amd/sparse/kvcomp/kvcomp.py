@@ -232,6 +232,12 @@ class KvComp(UcmSparseBase):
                 js = json.load(f)
             self.cfg.setdefault("head_dim", js.get("head_dim", 128))
             self.cfg.setdefault("hash_bits", js.get("hash_bits", 128))
+            # the reference refuses a file written for another model (kvcomp.py:458-464)
+            n_model = getattr(getattr(mc, "hf_text_config", None), "num_hidden_layers", None)
+            n_file = js.get("num_hidden_layers")
+            assert n_model is None or n_file is None or n_file == n_model, (
+                f"kvcomp_config.num_hidden_layers {n_file} != "
+                f"vllm_config.model_config.hf_text_config.num_hidden_layers {n_model}")
         for key, default in (("init_window_sz", INIT_WINDOW_SZ), ("local_window_sz", LOCAL_WINDOW_SZ),
                              ("sparse_ratio", SPARSE_RATIO), ("retrieval_stride", RETRIEVAL_STRIDE),
                              ("hash_bits", 128), ("fp16_scores", True), ("keep_token_codes", False)):
