@@ -1,6 +1,6 @@
 /*
  * Host twins of the C ABI: the same prototypes as libucm_hip.so's entry points
- * of the dense retrieval path and of the hash-code path, name + "_cpu", every "dev" pointer a host
+ * of the dense retrieval path, of the ESA retrieval worker and of the hash-code path, name + "_cpu", every "dev" pointer a host
  * pointer, `stream` ignored, the work done before the call returns.  A caller
  * written against one prototype switches between host and device by choosing
  * the symbol.
@@ -32,6 +32,9 @@ TWIN(ucm_kv_gather_blocks);
 TWIN(ucm_kv_scatter_blocks);
 TWIN(ucm_kv_gather_selected);
 TWIN(ucm_delta_plan);
+TWIN(ucm_delta_plan_rows);
+TWIN(ucm_esa_retrieve);
+TWIN(ucm_esa_retrieve_rows);
 TWIN(ucm_hash_encode_blocks);
 TWIN(ucm_hash_encode_queries);
 TWIN(ucm_hash_score_blocks);
@@ -47,6 +50,8 @@ void orc_kq_scores(const float* qMean, const float* kRepre, uint32_t numBlock, u
 int32_t orc_topk_windows(const float* scores, uint32_t n, uint32_t k, uint32_t startW, uint32_t endW, int32_t* out);
 int32_t orc_block_table_gather(const int32_t* block_table, const int32_t* topk_idx, int32_t count, int32_t seq_len,
                                int32_t block_size, int32_t* phys_out);
+int32_t orc_esa_retrieve(const float* data, uint32_t dim, const float* q, const int32_t* indexes, uint32_t n_indexes,
+                         int32_t topk, int32_t* out_idx, float* out_scores);
 int32_t orc_delta_plan(const int32_t* sel, const int32_t* sel_phys, int32_t count, int32_t* resident, int32_t n_slots,
                        int32_t* load_phys, int32_t* slot_of_sel);
 void orc_hash_encode(const uint16_t* x, const float* W, uint32_t n, uint32_t dim, uint32_t bits, uint8_t* codes);
@@ -266,6 +271,117 @@ int ucm_delta_plan_cpu(const int32_t* sel, const int32_t* sel_phys, const int32_
         miss_count[lr] = orc_delta_plan(sel + lr * (size_t)sel_stride, sel_phys + lr * (size_t)sel_stride, c,
                                         resident + lr * (size_t)n_slots, n_slots, load_phys + lr * (size_t)n_slots,
                                         slot_of_sel + lr * (size_t)sel_stride);
+    }
+    return UCM_OK;
+}
+
+int ucm_delta_plan_rows_cpu(const int32_t* sel, const int32_t* sel_phys, const int32_t* count, const int32_t* rows, int batch,
+                            int table_rows, int n_layers, int sel_stride, int32_t* resident, int n_slots, int32_t* load_phys,
+                            int32_t* slot_of_sel, int32_t* miss_count, ucm_stream_t stream)
+{
+    (void)stream;
+    if (batch < 0 || table_rows <= 0 || n_layers <= 0) { return UCM_EINVAL; }
+    if (batch == 0) { return UCM_OK; }
+    if (!sel || !sel_phys || !count || !rows || !resident || !load_phys || !slot_of_sel || !miss_count || sel_stride < 1) {
+        return UCM_EINVAL;
+    }
+    if (n_slots < 1 || n_slots > 1024) { return UCM_ENOTSUP; }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int b = 0; b < batch; ++b) {
+            if (rows[b] < 0 || rows[b] >= table_rows) { continue; }
+            const size_t lr = (size_t)l * table_rows + rows[b];
+            int32_t c = count[lr] < 0 ? 0 : count[lr];
+            if (c > sel_stride) { c = sel_stride; }
+            miss_count[lr] = orc_delta_plan(sel + lr * (size_t)sel_stride, sel_phys + lr * (size_t)sel_stride, c,
+                                            resident + lr * (size_t)n_slots, n_slots, load_phys + lr * (size_t)n_slots,
+                                            slot_of_sel + lr * (size_t)sel_stride);
+        }
+    }
+    return UCM_OK;
+}
+
+/* ------------------------------------------------------- ESA retrieval */
+
+/*
+ * One request: the list entries that name a row of the table go to orc_esa_retrieve in list order (it breaks ties by
+ * that order); a winner's position in the list is the first position not yet given out that holds its row.
+ */
+static int esa_one(const float* data, int n_items, int dim, const float* q, const int32_t* list, int m, int topk,
+                   int32_t* out_idx, int32_t* out_pos, float* out_scores)
+{
+    int32_t* keep = (int32_t*)malloc(((size_t)m + 1) * sizeof(int32_t));
+    int32_t* pos = (int32_t*)malloc(((size_t)m + 1) * sizeof(int32_t));
+    int32_t* win = (int32_t*)malloc(((size_t)m + 1) * sizeof(int32_t));
+    float* win_s = (float*)malloc(((size_t)m + 1) * sizeof(float));
+    char* used = (char*)calloc((size_t)m + 1, 1);
+    int n = 0, got = -1;
+    if (keep && pos && win && win_s && used) {
+        for (int j = 0; j < m; ++j) {
+            if (list[j] >= 0 && list[j] < n_items) { keep[n] = list[j]; pos[n] = j; ++n; }
+        }
+        got = orc_esa_retrieve(data, (uint32_t)dim, q, keep, (uint32_t)n, topk, win, win_s);
+        for (int i = 0; i < got; ++i) {
+            int at = 0;
+            while (used[at] || keep[at] != win[i]) { ++at; }
+            used[at] = 1;
+            out_idx[i] = win[i];
+            out_scores[i] = win_s[i];
+            if (out_pos) { out_pos[i] = pos[at]; }
+        }
+    }
+    free(keep); free(pos); free(win); free(win_s); free(used);
+    return got;
+}
+
+static int esa_check(const float* data, int n_items, int dim, const float* q, const void* lists, int batch, int m, int topk,
+                     const void* ws, const void* out_idx, const void* out_scores, const void* out_count, int out_stride)
+{
+    if (batch < 0 || m < 0) { return UCM_EINVAL; }
+    if (batch == 0) { return 1; }                        /* nothing to do */
+    if (!data || !q || !out_idx || !out_scores || !out_count || (m > 0 && (!lists || !ws)) || n_items <= 0 || dim <= 0) {
+        return UCM_EINVAL;
+    }
+    if (dim % 4 != 0) { return UCM_ENOTSUP; }
+    const int k = topk < 0 ? 0 : topk;
+    if (batch > 65535 || out_stride < (k < m ? k : m)) { return UCM_EINVAL; }
+    return m > 8192 ? UCM_ENOTSUP : UCM_OK;
+}
+
+int ucm_esa_retrieve_cpu(const float* data, int n_items, int dim, const float* q, const int32_t* indexes, int batch, int m,
+                         int topk, float* scores_ws, int32_t* out_idx, float* out_scores, int32_t* out_count, int out_stride,
+                         ucm_stream_t stream)
+{
+    (void)stream;
+    const int rc = esa_check(data, n_items, dim, q, indexes, batch, m, topk, scores_ws, out_idx, out_scores, out_count, out_stride);
+    if (rc != UCM_OK) { return rc == 1 ? UCM_OK : rc; }
+    for (int b = 0; b < batch; ++b) {
+        const int got = esa_one(data, n_items, dim, q + (size_t)b * dim, indexes + (size_t)b * m, m, topk,
+                                out_idx + (size_t)b * out_stride, NULL, out_scores + (size_t)b * out_stride);
+        if (got < 0) { return UCM_ENOMEM; }
+        out_count[b] = got;
+    }
+    return UCM_OK;
+}
+
+int ucm_esa_retrieve_rows_cpu(const float* data, int n_items, int dim, const float* q, const int32_t* slot_table,
+                              int table_rows, int table_stride, int m, const int32_t* rows, int batch, const int32_t* topk_rows,
+                              int max_topk, float* scores_ws, int32_t* out_idx, int32_t* out_pos, float* out_scores,
+                              int32_t* out_count, int out_stride, ucm_stream_t stream)
+{
+    (void)stream;
+    const int rc = esa_check(data, n_items, dim, q, slot_table, batch, m, max_topk, scores_ws, out_idx, out_scores, out_count,
+                             out_stride);
+    if (rc != UCM_OK) { return rc == 1 ? UCM_OK : rc; }
+    if (!rows || !topk_rows || table_rows <= 0 || table_stride < m) { return UCM_EINVAL; }
+    for (int b = 0; b < batch; ++b) {
+        const int row = rows[b];
+        if (row < 0 || row >= table_rows) { continue; }
+        const int k = topk_rows[row] < max_topk ? topk_rows[row] : max_topk;
+        const int got = esa_one(data, n_items, dim, q + (size_t)b * dim, slot_table + (size_t)row * table_stride, m, k,
+                                out_idx + (size_t)row * out_stride, out_pos ? out_pos + (size_t)row * out_stride : NULL,
+                                out_scores + (size_t)row * out_stride);
+        if (got < 0) { return UCM_ENOMEM; }
+        out_count[row] = got;
     }
     return UCM_OK;
 }

@@ -12,7 +12,7 @@ import synth
 
 TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
-         "ucm_hash_score_blocks"]
+         "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows"]
 
 
 def twin_caller(signatures):
@@ -211,3 +211,70 @@ def run_hash(call, side):
         out[name] = sc
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x
+
+
+E_ITEMS, E_DIM, E_M, E_ROWS, E_L, E_SLOTS = 40, 64, 12, 5, 2, 6
+
+
+def esa_inputs():
+    data = synth.normal_f32(7200, (E_ITEMS, E_DIM))
+    data[7] = data[3]                                                  # equal scores: the earlier list entry wins
+    data[11] = 0.0
+    data[12] = -0.0 * np.ones(E_DIM, np.float32)                       # +0 and -0 rank as equal
+    q = synth.normal_f32(7201, (3, E_DIM))
+    lists = np.full((3, E_M), -1, np.int32)
+    lists[0, :9] = [5, 3, -1, 7, E_ITEMS, 11, 12, 30, 2]               # a hole, an id outside the table
+    lists[1, :2] = [9, 9]                                              # the same row twice
+    lists[2] = synth.permutation(7202, E_ITEMS)[:E_M]
+    table = np.full((E_ROWS, E_M + 3), -1, np.int32)                   # persistent rows, wider than m
+    table[4, :E_M], table[0, :E_M], table[2, :E_M] = lists[0], lists[1], lists[2]
+    rows = np.array([4, 0, 2, E_ROWS, -1], np.int32)                   # two requests outside the table: no-ops
+    topk_rows = np.array([1, 9, 4, 9, 3], np.int32)
+    return dict(data=data, q=q, lists=lists, table=table, rows=rows, topk_rows=topk_rows)
+
+
+def run_esa(call, side):
+    """The ESA worker's retrieval, batched and over a persistent table, and the resident-set plan of its winners."""
+    x = esa_inputs()
+    data, q = side.up(x["data"]), side.up(x["q"])
+    lists, table, rows, topk_rows = side.up(x["lists"]), side.up(x["table"]), side.up(x["rows"]), side.up(x["topk_rows"])
+    ws = side.up(np.zeros((5, E_M), np.float32))
+    out = {}
+    for topk in (4, 0, 20):
+        oi, os_, oc = (side.up(np.full((3, E_M), -7, np.int32)), side.up(np.full((3, E_M), -7, np.float32)),
+                       side.up(np.full(3, -7, np.int32)))
+        call("ucm_esa_retrieve", side.ptr(data), E_ITEMS, E_DIM, side.ptr(q), side.ptr(lists), 3, E_M, topk, side.ptr(ws),
+             side.ptr(oi), side.ptr(os_), side.ptr(oc), E_M, None)
+        out.update({f"idx{topk}": oi, f"scores{topk}": os_, f"count{topk}": oc})
+    q5 = side.up(np.concatenate([x["q"], x["q"][:2]]))                 # five requests, two of them without a row
+    ri, rp, rs, rc = (side.up(np.full((E_ROWS, 5), -7, np.int32)), side.up(np.full((E_ROWS, 5), -7, np.int32)),
+                      side.up(np.full((E_ROWS, 5), -7, np.float32)), side.up(np.full(E_ROWS, -7, np.int32)))
+    call("ucm_esa_retrieve_rows", side.ptr(data), E_ITEMS, E_DIM, side.ptr(q5), side.ptr(table), E_ROWS, E_M + 3, E_M,
+         side.ptr(rows), 5, side.ptr(topk_rows), 5, side.ptr(ws), side.ptr(ri), side.ptr(rp), side.ptr(rs), side.ptr(rc), 5, None)
+    out.update(rows_idx=ri, rows_pos=rp, rows_scores=rs, rows_count=rc)
+    # the winners' list positions are the request's logical blocks: two plans in a row over [layers][rows][slots]
+    resident = side.up(np.full((E_L, E_ROWS, E_SLOTS), -1, np.int32))
+    load, slot_of, miss = (side.up(np.full((E_L, E_ROWS, E_SLOTS), -7, np.int32)), side.up(np.full((E_L, E_ROWS, 5), -7, np.int32)),
+                           side.up(np.full((E_L, E_ROWS), -7, np.int32)))
+    side.sync()
+    pos_h, cnt_h = np.array(side.down(rp)), np.array(side.down(rc))
+    sel_h = np.stack([pos_h, pos_h[:, ::-1].copy()])                   # layer 1 sees the winners in another order
+    cnt_l = np.stack([cnt_h, cnt_h])
+    for r in range(E_ROWS):
+        if cnt_h[r] >= 0:
+            sel_h[1, r, : cnt_h[r]] = pos_h[r, : cnt_h[r]][::-1]
+    sel, cnt = side.up(sel_h.astype(np.int32)), side.up(cnt_l.astype(np.int32))
+    for step in (1, 2):
+        if step == 2:                                                  # second step: one winner replaced per request
+            sel_h = sel_h.copy()
+            for r in range(E_ROWS):
+                if cnt_h[r] > 0:                                       # by the lowest position that did not win
+                    sel_h[:, r, 0] = min(set(range(E_M)) - set(pos_h[r, : cnt_h[r]].tolist()))
+            sel = side.up(sel_h.astype(np.int32))
+        call("ucm_delta_plan_rows", side.ptr(sel), side.ptr(sel), side.ptr(cnt), side.ptr(rows), 5, E_ROWS, E_L, 5,
+             side.ptr(resident), E_SLOTS, side.ptr(load), side.ptr(slot_of), side.ptr(miss), None)
+        side.sync()
+        out.update({f"resident{step}": np.array(side.down(resident)).copy(), f"load{step}": np.array(side.down(load)).copy(),
+                    f"slot_of{step}": np.array(side.down(slot_of)).copy(), f"miss{step}": np.array(side.down(miss)).copy()})
+    side.sync()
+    return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x

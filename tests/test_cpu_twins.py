@@ -68,3 +68,41 @@ def test_hash_twins_reproduce_the_oracle(ucm):
                     assert np.array_equal(got["score_code"][l, a : a + n],
                                           O.hash_scores_block(got["qbar"][l, r], got["block_codes"][l, a : a + n]).astype(np.float32))
     assert np.array_equal(got["score_sum_fp16"], got["score_sum"].astype(np.float16).astype(np.float32))
+
+
+def test_esa_twins_reproduce_the_oracle(ucm):
+    from ucm_amd import _lib
+
+    got, x = cpu_twins.run_esa(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    n_items = cpu_twins.E_ITEMS
+    for topk in (4, 0, 20):
+        for b in range(3):
+            live = x["lists"][b][(x["lists"][b] >= 0) & (x["lists"][b] < n_items)]      # holes and foreign ids are skipped
+            idx, sc = O.esa_retrieve(x["data"], x["q"][b], live, topk)
+            n = got[f"count{topk}"][b]
+            assert n == len(idx) == min(len(live), topk)
+            assert np.array_equal(got[f"idx{topk}"][b, :n], idx)
+            assert np.array_equal(got[f"scores{topk}"][b, :n].view(np.uint32), sc.view(np.uint32))
+            assert (got[f"idx{topk}"][b, n:] == -7).all()
+    # worked by hand: rows 11 (+0) and 12 (-0) tie at 0 and come in list order; the duplicate of row 3 follows row 3
+    order = got["idx20"][0, :7].tolist()
+    assert order.index(11) + 1 == order.index(12) and order.index(3) + 1 == order.index(7)
+    # the table variant: request b -> row rows[b], its own k, positions within the slot list
+    for b, row in enumerate(x["rows"][:3]):
+        k = min(5, int(x["topk_rows"][row]))
+        lst = x["table"][row, : cpu_twins.E_M]
+        live = lst[(lst >= 0) & (lst < n_items)]
+        idx, sc = O.esa_retrieve(x["data"], x["q"][b], live, k)
+        n = got["rows_count"][row]
+        assert n == len(idx) and np.array_equal(got["rows_idx"][row, :n], idx)
+        assert np.array_equal(lst[got["rows_pos"][row, :n]], idx)
+    assert (got["rows_count"][[1, 3]] == -7).all()                     # rows no request of the call owns
+    # plans: first step loads every winner; second step loads exactly the one replaced, into the slot it freed
+    for l in range(cpu_twins.E_L):
+        for row in (4, 0, 2):
+            n = got["rows_count"][row]
+            assert got["miss1"][l, row] == n and sorted(got["resident1"][l, row, :n]) == sorted(got["rows_pos"][row, :n])
+            assert got["miss2"][l, row] == 1 and (got["load2"][l, row] >= 0).sum() == 1
+            slot = int(np.argmax(got["load2"][l, row] >= 0))
+            assert got["resident2"][l, row, slot] == got["load2"][l, row, slot]
+            assert got["resident1"][l, row, slot] not in got["resident2"][l, row]

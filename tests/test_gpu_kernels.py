@@ -829,12 +829,13 @@ def test_decode_step_under_graph_capture(ucm, dev):
 def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     """One scripted pass over the dense path (three representative modes, both score variants with q_rows and a
     scale, selection with block tables and sparse lengths, two delta plans, both gathers, block moves with ids to
-    skip) through libucm_hip.so on device buffers and through the oracle's `_cpu` twins on host buffers: the same
+    skip; the hash-code path; the ESA worker's retrieval, batched and over a persistent table, with two plans of its
+    winners) through libucm_hip.so on device buffers and through the oracle's `_cpu` twins on host buffers: the same
     argument lists, the same bytes out."""
     import cpu_twins
     from ucm_amd import _lib, ops
 
-    for run in (cpu_twins.run, cpu_twins.run_hash):      # the dense path; the hash-code path
+    for run in (cpu_twins.run, cpu_twins.run_hash, cpu_twins.run_esa):   # the dense path; hash codes; the ESA worker
         want, _ = run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
         got, _ = run(_lib.call, cpu_twins.DeviceSide(ops, dev))
         assert got.keys() == want.keys()
