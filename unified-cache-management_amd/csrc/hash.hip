@@ -161,42 +161,40 @@ __device__ __forceinline__ void planes_flush(unsigned (&pl)[kPlanes], int* __res
     for (int p = 0; p < kPlanes; ++p) { pl[p] = 0u; }
 }
 
-// The same for eight kv heads, without atomics: the four lanes of a lane half that hold vectors of one head
-// (lr, lr ^ 8, lr ^ 16, lr ^ 24) first add their counts up - as bytes, four to a register: a plane set counts at
-// most 63 tiles, four lanes 252 - and lane lr < 8 then owns head lr's sixteen columns of each of the two column
-// blocks outright.  (Thirty-two LDS atomics per lane with four lanes on every address took four times as long as
-// everything else a block needs at its end.)
-__device__ __forceinline__ void planes_flush_heads8(unsigned (&pl)[kPlanes], int* __restrict__ colsum, int wp, int half, int lr)
+// The same without atomics, for kHeads = 8, 4, 2 or 1 kv heads: the 32 / kHeads lanes of a lane half that hold
+// vectors of one head (lr, lr ^ kHeads, lr ^ 2 kHeads, ...) first add their counts up with shuffles - as bytes, four
+// to a register, for the first two levels (a plane set counts at most 63 tiles, four lanes 252), as halfwords for the
+// levels beyond - and lane lr < kHeads then owns head lr's sixteen columns of each of the two column blocks outright.
+// (Thirty-two LDS atomics per lane, with 32 / kHeads lanes on every address, took four times as long as everything
+// else a block of eight heads needs at its end, and more than the block's tiles for one head.)
+template <int kHeads>
+__device__ __forceinline__ void planes_flush_owner(unsigned (&pl)[kPlanes], int* __restrict__ colsum, int wp, int half, int lr)
 {
-    unsigned cnt[8];                                     // byte k of cnt[j]: count of bit 4j + k
+    typedef int i32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        unsigned c = 0u;
+    for (int j = 0; j < 8; ++j) {                        // bits 4j .. 4j+3: columns (2*wp + j/4)*32 + half*16 + 4*(j%4) + 0..3
+        unsigned c = 0u;                                 // byte k: count of bit 4j + k
 #pragma unroll
         for (int p = 0; p < kPlanes; ++p) {
             const unsigned nib = (pl[p] >> (4 * j)) & 0xfu;
             c += ((nib * 0x00204081u) & 0x01010101u) << p;   // bit i of the nibble -> byte i
         }
-        c += __shfl_xor(c, 8, 64);
-        c += __shfl_xor(c, 16, 64);
-        cnt[j] = c;
-    }
-    if (lr < 8) {
-        int* row = colsum + lr * kBits + half * 16;
+        c += __shfl_xor(c, kHeads, 64);
+        c += __shfl_xor(c, 2 * kHeads, 64);
+        unsigned even = c & 0x00ff00ffu, odd = (c >> 8) & 0x00ff00ffu;   // counts of bits 4j, 4j+2 / 4j+1, 4j+3
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {              // bits 16*blk .. 16*blk+15 are columns (2*wp + blk)*32 + half*16 + 0..15
-            int* dst = row + (2 * wp + blk) * 32;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const unsigned c = cnt[4 * blk + q];
-                typedef int i32x4 __attribute__((ext_vector_type(4)));
-                i32x4 v = *reinterpret_cast<i32x4*>(dst + 4 * q);
-                v.x += static_cast<int>(c & 0xffu);
-                v.y += static_cast<int>((c >> 8) & 0xffu);
-                v.z += static_cast<int>((c >> 16) & 0xffu);
-                v.w += static_cast<int>(c >> 24);
-                *reinterpret_cast<i32x4*>(dst + 4 * q) = v;
-            }
+        for (int s = 4 * kHeads; s < 32; s <<= 1) {
+            even += __shfl_xor(even, s, 64);
+            odd += __shfl_xor(odd, s, 64);
+        }
+        if (lr < kHeads) {
+            int* dst = colsum + lr * kBits + (2 * wp + (j >> 2)) * 32 + half * 16 + 4 * (j & 3);
+            i32x4 v = *reinterpret_cast<i32x4*>(dst);
+            v.x += static_cast<int>(even & 0xffffu);
+            v.y += static_cast<int>(odd & 0xffffu);
+            v.z += static_cast<int>(even >> 16);
+            v.w += static_cast<int>(odd >> 16);
+            *reinterpret_cast<i32x4*>(dst) = v;
         }
     }
 #pragma unroll
@@ -322,13 +320,23 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         for (int p = 0; p < kPlanes; ++p) { planes01[p] = 0u; planes23[p] = 0u; }
         unsigned pending = 0;                            // tiles counted in the planes
         int qlen = 0;
+        // inside a block of more than 63 tiles (once per 63 tiles; the three copies of the tile code each hold one)
         auto flush_planes = [&]() {
             if (kv_heads == 8) {                         // (uniform)
-                planes_flush_heads8(planes01, &ws.colsum[0][0], 0, half, lr);
-                planes_flush_heads8(planes23, &ws.colsum[0][0], 1, half, lr);
+                planes_flush_owner<8>(planes01, &ws.colsum[0][0], 0, half, lr);
+                planes_flush_owner<8>(planes23, &ws.colsum[0][0], 1, half, lr);
             } else {
                 planes_flush(planes01, head_row, 0, half);
                 planes_flush(planes23, head_row, 1, half);
+            }
+        };
+        // at the end of every block
+        auto flush_planes_last = [&]() {
+            switch (kv_heads) {                          // (uniform)
+            case 8: planes_flush_owner<8>(planes01, &ws.colsum[0][0], 0, half, lr); planes_flush_owner<8>(planes23, &ws.colsum[0][0], 1, half, lr); break;
+            case 4: planes_flush_owner<4>(planes01, &ws.colsum[0][0], 0, half, lr); planes_flush_owner<4>(planes23, &ws.colsum[0][0], 1, half, lr); break;
+            case 2: planes_flush_owner<2>(planes01, &ws.colsum[0][0], 0, half, lr); planes_flush_owner<2>(planes23, &ws.colsum[0][0], 1, half, lr); break;
+            default: planes_flush_owner<1>(planes01, &ws.colsum[0][0], 0, half, lr); planes_flush_owner<1>(planes23, &ws.colsum[0][0], 1, half, lr); break;
             }
         };
 
@@ -529,7 +537,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         }
         store_codes();
         if (qlen > 0) { drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
-        flush_planes();
+        flush_planes_last();
 
         // ---- block summaries
         // (LDS operations of one wave complete in order; no barrier is needed inside the wave)
