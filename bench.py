@@ -74,6 +74,9 @@ def parse():
                     help="hash leg: name only this many distinct cache blocks in the encode's block list, over and over "
                          "(8: the key loads are served from cache, which times the compute side of the kernel on its own); "
                          "0 = every block once")
+    ap.add_argument("--hash-heads-sweep", action="store_true",
+                    help="hash leg: also time the summaries-only encode with the same cache bytes read as blocks of 4, 2 "
+                         "and 1 kv heads (what a tensor-parallel rank holds)")
     ap.add_argument("--prefetch-leg", action="store_true",
                     help="also time the GSA prefetch engine's round at this batch: hits / misses / free list of every "
                          "(request, layer) on the device plus the loads of the served misses from a device-resident "
@@ -353,6 +356,19 @@ def main():
         sc1_ms = timed(lambda: ops.hash_score_blocks(1, q_sum, qbar, colsum, bcodes, h_so, h_sl, h_rows, h_scores), 10)
         ops.hash_score_blocks(0, q_sum, qbar, colsum, bcodes, h_so, h_sl, h_rows, h_scores)
         tk_ms = timed(lambda: ops.topk_windows(h_scores, h_so, h_sl, h_tk, int(h_lens.max()), h_idx, h_cnt), 10)
+        heads_sweep = None
+        if args.hash_heads_sweep:
+            # the same bytes as blocks of fewer heads: a [128][8][128] block is 8/h blocks of [128][h][128], and the
+            # block list names all of them; the summary tables keep their size
+            heads_sweep = {}
+            for h in (8, 4, 2, 1):
+                f = HKV // h
+                ids_h = (h_ids.view(-1, 1) * f + torch.arange(f, dtype=torch.int32, device=dev)).reshape(-1).contiguous()
+                slots_h = torch.arange(h_rows * f, dtype=torch.int32, device=dev)
+                cs_h, bc_h = colsum.view(n_layers, h_rows * f, h, 128), bcodes.view(n_layers, h_rows * f, h, 16)
+                ms = timed(lambda: ops.hash_encode_blocks(layers, ids_h, slots_h, h_rows * f, w_hash, BS, h, pool * f, cs_h, bc_h), 3)
+                heads_sweep[str(h)] = {"blocks": h_rows * f, "ms": round(ms, 3)}
+            enc(tcodes)                                  # the tables hold the 8-head results again
         key_bytes = n_layers * h_rows * BLOCK_BYTES
         enc_bytes = key_bytes + n_layers * h_rows * (BS * HKV * 16 + HKV * 128 * 2 + HKV * 16)
         hash_checked = None
@@ -382,6 +398,7 @@ def main():
                          "algorithmic_bytes": enc_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * h_rows * BS * HKV * 128 * 128 / (enc_ms * 1e-3) / 1e12, 1)},
             "encode_summaries_only_ms": round(enc_sum_ms, 3),
+            "encode_summaries_only_ms_by_kv_heads": heads_sweep,
             "decode_step_us": {"query_codes": round(q_ms * 1e3, 1), "score": round(sc_ms * 1e3, 1),
                                "score_block_code": round(sc1_ms * 1e3, 1), "select": round(tk_ms * 1e3, 1)},
             "checked": hash_checked,
