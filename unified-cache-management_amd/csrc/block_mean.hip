@@ -37,15 +37,25 @@ __device__ __forceinline__ void widen(const u32x4 v, float (&f)[kCols])
     f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
 }
 
-// grid: x = block index in the list * col_groups + column group of 1024, y = layer
+// grid: x = block index in the list * col_groups + column group of 1024, y = layer; rows narrower than 1024
+// columns whose thread count divides the workgroup (a tensor-parallel rank's 4, 2 or 1 kv heads of 128) share a
+// workgroup, items_per_group list entries side by side, so that no lane idles
 __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned repre_rows, unsigned block_size,
     unsigned row /* kv_heads*head_dim */, float* __restrict__ repre, int64_t repre_layer_stride,
-    int round_to_bf16, unsigned col_groups)
+    int round_to_bf16, unsigned col_groups, unsigned items_per_group, unsigned n_items)
 {
-    const unsigned item = blockIdx.x / col_groups;
-    const unsigned col = ((blockIdx.x % col_groups) * kThreads + threadIdx.x) * kCols;
+    unsigned item, col;
+    if (items_per_group > 1) {
+        const unsigned per_item = kThreads / items_per_group;
+        item = blockIdx.x * items_per_group + threadIdx.x / per_item;
+        col = (threadIdx.x % per_item) * kCols;
+        if (item >= n_items) { return; }
+    } else {
+        item = blockIdx.x / col_groups;
+        col = ((blockIdx.x % col_groups) * kThreads + threadIdx.x) * kCols;
+    }
     if (col >= row) { return; }
     const unsigned id = static_cast<unsigned>(block_ids[item]);
     const unsigned slot = static_cast<unsigned>(slots[item]);
@@ -129,9 +139,12 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
                 "ucm_block_mean: repre not 16-byte aligned");
     const unsigned gx = (row / kCols + kThreads - 1) / kThreads;
     UCM_REQUIRE(static_cast<uint64_t>(n) * gx <= 0x7fffffffull, "ucm_block_mean: too many blocks for one launch");
-    hipLaunchKernelGGL(block_mean_kernel, dim3(static_cast<unsigned>(n) * gx, n_layers), dim3(kThreads), 0, ucm::as_stream(stream),
+    const unsigned per_item = row / kCols;               // threads a list entry needs
+    const unsigned share = (per_item < kThreads && kThreads % per_item == 0) ? kThreads / per_item : 1u;
+    const unsigned groups = share > 1 ? (static_cast<unsigned>(n) + share - 1) / share : static_cast<unsigned>(n) * gx;
+    hipLaunchKernelGGL(block_mean_kernel, dim3(groups, n_layers), dim3(kThreads), 0, ucm::as_stream(stream),
                        k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
                        static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row,
-                       static_cast<float*>(repre), repre_layer_stride, mode, gx);
+                       static_cast<float*>(repre), repre_layer_stride, mode, gx, share, static_cast<unsigned>(n));
     UCM_LAUNCH_CHECK("ucm_block_mean");
 }
