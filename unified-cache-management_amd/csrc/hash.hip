@@ -95,9 +95,10 @@ __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict_
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const unsigned xa = xv[i][j], wa = wv[i][j];
-            acc += static_cast<double>(__uint_as_float(xa << 16)) * static_cast<double>(__uint_as_float(wa << 16));
-            acc += static_cast<double>(__uint_as_float(xa & 0xffff0000u)) *
-                   static_cast<double>(__uint_as_float(wa & 0xffff0000u));
+            // (a product of two bf16 values is exact in fp64, so the fused form rounds exactly as multiply-then-add does)
+            acc = __builtin_fma(static_cast<double>(__uint_as_float(xa << 16)), static_cast<double>(__uint_as_float(wa << 16)), acc);
+            acc = __builtin_fma(static_cast<double>(__uint_as_float(xa & 0xffff0000u)),
+                                static_cast<double>(__uint_as_float(wa & 0xffff0000u)), acc);
         }
     }
     return acc < 0.0;
