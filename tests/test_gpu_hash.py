@@ -25,8 +25,8 @@ def make_weights(seed):
     return bits, synth.bf16_widen(bits)
 
 
-# (8, 272) and (4, 520): more than 63 tiles in a block, so the column counters are flushed inside the tile loop too
-@pytest.mark.parametrize("hkv,bs", [(8, 128), (2, 16), (4, 64), (1, 32), (8, 272), (4, 520)])
+# the last four: more than 63 tiles in a block, so the column counters are flushed inside the tile loop too
+@pytest.mark.parametrize("hkv,bs", [(8, 128), (2, 16), (4, 64), (1, 32), (8, 272), (4, 520), (2, 1040), (1, 2080)])
 def test_hash_encode_blocks(ucm, dev, hkv, bs):
     from ucm_amd import ops
 
