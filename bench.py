@@ -74,6 +74,9 @@ def parse():
                     help="hash leg: name only this many distinct cache blocks in the encode's block list, over and over "
                          "(8: the key loads are served from cache, which times the compute side of the kernel on its own); "
                          "0 = every block once")
+    ap.add_argument("--no-legs", action="store_true",
+                    help="only the decode step (and its delta-gather leg): none of the --*-leg measurements.  Without this "
+                         "flag and without any --*-leg flag, every leg runs; naming legs runs exactly those.")
     ap.add_argument("--hash-heads-sweep", action="store_true",
                     help="hash leg: also time the summaries-only encode with the same cache bytes read as blocks of 4, 2 "
                          "and 1 kv heads (what a tensor-parallel rank holds)")
@@ -99,7 +102,12 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
-    return ap.parse_args()
+    args = ap.parse_args()
+    leg_flags = ("hash_leg", "prefetch_leg", "moves_leg", "esa_leg", "kvstar_leg")
+    run_all = not args.no_legs and not any(getattr(args, f) for f in leg_flags)
+    for f in leg_flags:
+        setattr(args, f, run_all or (getattr(args, f) and not args.no_legs))
+    return args
 
 
 def main():
