@@ -356,3 +356,61 @@ def test_hash_queries_scores_and_selection(ucm, dev):
                 assert np.array_equal(sc[l, a : a + n], want), (mode, rnd, l, r)
                 sel = O.topk_windows(want, int(topk[r]), 1, 1)
                 assert cnt[l, r] == len(sel) and np.array_equal(idx[l, r, : len(sel)].cpu().numpy(), sel), (mode, l, r)
+
+
+def cancelling_keys(seed, w_f32, n_vec, perm):
+    """Vectors whose projection on one chosen weight column is built to cancel: the 128 dims are taken in pairs (in
+    the order `perm`), the second element of a pair being the bf16 neighbour that brings the running sum closest to
+    zero, with magnitudes that fall off at a rate drawn per vector.  The projection ends between 2^-45 and 2^-18 of
+    ||x|| ||w|| while the partial sums along the way are as large as any - the worst case for a sum accumulated in
+    fp32 in whatever order.  Returns bf16 bits [n_vec, 128] and the column each vector was built against."""
+    rng = np.random.default_rng(seed)
+    cols = rng.integers(0, 128, n_vec)
+    wc = w_f32.T[cols].astype(np.float64)                                # [n_vec, 128]
+    rate = rng.random((n_vec, 1)) * 0.35
+    a = synth.bf16_widen(synth.bf16_round_bits((rng.standard_normal((n_vec, 64)) * 2.0 ** (-rate * np.arange(64))).astype(np.float32)))
+    x = np.zeros((n_vec, 128), np.float32)
+    r = np.zeros(n_vec)
+    for i in range(64):
+        p0, p1 = perm[2 * i], perm[2 * i + 1]
+        w1 = np.where(wc[:, p1] == 0, 1.0, wc[:, p1])
+        t0 = a[:, i].astype(np.float64) * wc[:, p0]
+        ideal = (-(r + t0) / w1).astype(np.float32)
+        ideal = np.clip(ideal, -1e30, 1e30)
+        lo = (ideal.view(np.uint32) & np.uint32(0xffff0000)).view(np.float32)            # towards zero
+        hi = ((ideal.view(np.uint32) & np.uint32(0xffff0000)) + np.uint32(0x10000)).view(np.float32)
+        y = np.where(np.abs(r + t0 + lo.astype(np.float64) * w1) <= np.abs(r + t0 + hi.astype(np.float64) * w1), lo, hi)
+        y = np.where(np.isfinite(y) & (np.abs(y) < 1e20), y, np.float32(0))
+        x[:, p0], x[:, p1] = a[:, i], y
+        r = r + t0 + y.astype(np.float64) * wc[:, p1]
+    bits_ = synth.bf16_round_bits(x)
+    assert np.array_equal(synth.bf16_widen(bits_), x)                                    # every value is a bf16 value
+    return bits_, cols
+
+
+@pytest.mark.parametrize("paired", ["neighbours", "scattered"])
+def test_hash_encode_projections_built_to_cancel(ucm, dev, paired):
+    """Seven thousand key vectors, each built so that its projection on one weight column cancels down to between
+    2^-45 and 2^-18 of ||x|| ||w|| (neighbouring dims paired, or dims paired at random so that the cancellation spans
+    the matrix instructions): the signs - those the matrix cores keep and those that are redone - must be the
+    oracle's, and so must the column sums."""
+    from ucm_amd import ops
+
+    hkv, bs, nb = 8, 128, 7
+    w_bits, w_f32 = make_weights(880)
+    perm = np.arange(128) if paired == "neighbours" else np.random.default_rng(881).permutation(128)
+    x_bits, cols = cancelling_keys(882, w_f32, nb * bs * hkv, perm)
+    x64 = synth.bf16_widen(x_bits).astype(np.float64)
+    ratio = np.abs((x64 * w_f32.T[cols]).sum(1)) / (np.linalg.norm(x64, axis=1) * np.linalg.norm(w_f32.T[cols].astype(np.float64), axis=1))
+    assert np.median(ratio) < 2.0 ** -24 and (ratio > 2.0 ** -24).sum() > 500 and (ratio < 2.0 ** -30).sum() > 500
+    keys_h = x_bits.reshape(nb, bs, hkv, 128)
+    lp = ops.LayerPointers([bf16_dev(keys_h, dev)])
+    colsum = torch.zeros((1, nb, hkv, 128), dtype=torch.int16, device=dev)
+    bcodes = torch.zeros((1, nb, hkv, 16), dtype=torch.uint8, device=dev)
+    tcodes = torch.zeros((1, nb, bs, hkv, 16), dtype=torch.uint8, device=dev)
+    ops.hash_encode_blocks(lp, None, None, nb, bf16_dev(w_bits, dev), bs, hkv, nb, colsum, bcodes, token_codes=tcodes)
+    torch.cuda.synchronize()
+    want = O.hash_encode(keys_h, w_f32)
+    assert np.array_equal(tcodes[0].cpu().numpy(), want)
+    assert np.array_equal(colsum[0].cpu().numpy(), O.hash_colsum(want))
+    assert np.array_equal(bcodes[0].cpu().numpy(), O.hash_majority(want))
