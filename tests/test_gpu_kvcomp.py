@@ -53,10 +53,13 @@ def test_hash_encoder_surface(ucm, dev):
     assert np.array_equal(pm.float().cpu().numpy(), want)
 
 
-def test_kvcomp_plugin_flow(ucm, dev):
+@pytest.mark.parametrize("device_loads", [True, False])
+def test_kvcomp_plugin_flow(ucm, dev, device_loads):
     """Prefill of 20 full blocks + 5 tokens, then decode on the sparsified block list: windows restored at step 1,
     retrieval at steps 1 and 5 picks what the oracle picks from the same keys, the chosen blocks land in the
-    request's middle cache blocks in ascending order, a block filled during decode is dumped and hashed."""
+    request's middle cache blocks in ascending order, a block filled during decode is dumped and hashed.  Once
+    through the batched device path (one call per layer for all requests, loads planned on the device) and once
+    through the per-request path that works with any store."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvcomp.kvcomp import KvComp
@@ -65,7 +68,8 @@ def test_kvcomp_plugin_flow(ucm, dev):
     ns = types.SimpleNamespace
     hq, hkv, d, L, bs, nb = 8, 2, 128, 2, 16, 64
     cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
-    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KvComp": {"keep_token_codes": True}}}
+    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KvComp": {"keep_token_codes": True,
+                                                                                         "device_loads": device_loads}}}
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     assert isinstance(plugin, KvComp)
     slice_bytes = bs * hkv * d * 2
@@ -168,5 +172,123 @@ def test_kvcomp_plugin_flow(ucm, dev):
         want = O.hash_encode(bf16_bits(caches[l][0][kept[-1]])[None], w_f32)
         assert np.array_equal(plugin.token_codes[l, base + 20].cpu().numpy(), want[0])
         assert "req_A_blk_20" in store.slot_of
+    assert (plugin._dev is not None) == device_loads
     plugin.request_finished_in_worker("A")
     assert "A" not in plugin.req_states and "A" not in plugin.segment_of
+
+
+def kvcomp_scenario(dev, device_loads, timing=None, shape=(8, 2, 128, 3, 16, 256), prompts=None, start=None, n_steps=12,
+                    keep_caches=True):
+    """Three sparsified requests at different stages (one prefilled two steps after the others, so that some steps
+    mix a prompt with decode tokens and the retrieval steps of the requests do not coincide) plus one short request
+    the plugin leaves alone; returns, per engine step, every request's selections per layer and the bytes of all
+    caches."""
+    import time
+
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.factory import UcmSparseFactory
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+
+    ns = types.SimpleNamespace
+    torch.manual_seed(5)                                           # the plugin draws its hash weights from the global generator
+    hq, hkv, d, L, bs, nb = shape
+    cfg = make_config(hq, hkv, d, L, bs, bs * 64, {})
+    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KvComp": {"device_loads": device_loads}}}
+    cfg.scheduler_config.max_num_seqs = max(cfg.scheduler_config.max_num_seqs, len(prompts or ()) + 1)
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    slice_bytes = bs * hkv * d * 2
+    plugin.connector = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": nb * L * 2 * slice_bytes})
+    g = torch.Generator(device=dev)
+    g.manual_seed(21)
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    perm = [int(x) for x in synth.permutation(980, nb)]
+    prompts = prompts or {"A": 20 * bs + 5, "B": 33 * bs, "C": 9 * bs + 3, "D": bs - 2}
+    start = start or {"A": 0, "B": 0, "C": 2, "D": 0}              # engine step of the prefill
+    reqs, pos = {}, 0
+    for rid, n in prompts.items():
+        n_blk = -(-(n + 12) // bs)
+        reqs[rid] = ns(block_ids=[perm[pos : pos + n_blk]], num_computed_tokens=0, prompt_token_ids=[1] * n, output_token_ids=[],
+                       num_prompt_tokens=n, num_output_tokens=0, num_tokens=n, request_id=rid, full=perm[pos : pos + n_blk])
+        pos += n_blk
+    log = []
+    for step in range(n_steps):
+        live = [rid for rid in reqs if start[rid] <= step]
+        sched, starts, at = {}, [0], {}
+        for i, rid in enumerate(live):
+            r = reqs[rid]
+            if start[rid] < step:                                  # a decode step: one more output token
+                r.output_token_ids.append(7)
+                r.num_output_tokens += 1
+                r.num_tokens += 1
+                if r.num_output_tokens == 1 and r.num_prompt_tokens > bs:   # the scheduler shrinks the block list (kvcomp.py:571-587)
+                    slots = plugin.estimate_num_slots_sparsed(r)
+                    r.block_ids = [r.full[: -(-r.num_tokens // bs)][-(-(-slots // bs)):]]
+            sched[rid] = r.num_prompt_tokens if start[rid] == step else 1
+            at[rid] = i
+            starts.append(starts[-1] + sched[rid])
+        fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0,
+                attn_metadata=ns(query_start_loc=torch.tensor(starts)))
+        so = ns(num_scheduled_tokens=sched, req_sparsed_slots={rid: 0 for rid in live})
+        t0 = time.perf_counter()
+        plugin.build_sparse_meta(so, reqs, ns(req_id_to_index=at))
+        t_hooks = time.perf_counter() - t0
+        for l in range(L):
+            q = torch.randn(starts[-1], hq, d, device=dev, generator=g).to(torch.bfloat16)
+            t0 = time.perf_counter()
+            plugin.attention_begin(q, None, None, names[l], fc)
+            plugin.attention_finished(q, None, None, None, names[l], fc)
+            t_hooks += time.perf_counter() - t0
+        if timing is not None:
+            torch.cuda.synchronize()
+            timing.append((step, t_hooks))
+        for rid in live:
+            reqs[rid].num_computed_tokens += sched[rid]
+        torch.cuda.synchronize()
+        sel = {rid: [plugin.req_states[rid][l].last_selection for l in range(L)] for rid in live if rid in plugin.req_states}
+        log.append((sel, [c.clone() for c in caches] if keep_caches or step == n_steps - 1 else None))
+    return log
+
+
+def test_kvcomp_batched_path_equals_per_request_path(ucm, dev):
+    """The same twelve engine steps through the batched device path and through the per-request path: the same
+    selections at every step a request retrieves and the same bytes in every cache after every step."""
+    t_dev, t_host = [], []
+    a = kvcomp_scenario(dev, True, t_dev)
+    b = kvcomp_scenario(dev, False, t_host)
+    retrievals = 0
+    for step, ((sel_a, caches_a), (sel_b, caches_b)) in enumerate(zip(a, b)):
+        for l, (x, y) in enumerate(zip(caches_a, caches_b)):
+            assert torch.equal(x, y), (step, l)
+        assert sel_a.keys() == sel_b.keys()
+        for rid in sel_b:
+            for l, want in enumerate(sel_b[rid]):
+                if want is not None and sel_a[rid][l] is not None:
+                    assert sel_a[rid][l] == want, (step, rid, l)
+                    retrievals += 1
+    assert retrievals > 20 and "D" not in a[-1][0]
+    busy_dev = sorted(t for s, t in t_dev if s >= 4)
+    busy_host = sorted(t for s, t in t_host if s >= 4)
+    print(f"\nhost time of a step's hooks, median over steps 4-11: batched {busy_dev[len(busy_dev) // 2] * 1e3:.2f} ms, "
+          f"per request {busy_host[len(busy_host) // 2] * 1e3:.2f} ms; slowest {busy_dev[-1] * 1e3:.2f} / {busy_host[-1] * 1e3:.2f} ms")
+
+
+def test_kvcomp_batched_path_at_serving_size(ucm, dev):
+    """Sixteen requests of 30 to 45 blocks of 128 tokens, 32 layers, Llama-3-8B head shape: the batched path and the
+    per-request path leave the same bytes in every cache after six decode steps (two retrieval steps per request, the
+    requests not in phase); the host time of a step's hooks is printed for both."""
+    rng = np.random.default_rng(31)
+    prompts = {f"R{i}": int(rng.integers(30, 46)) * 128 + int(rng.integers(0, 128)) for i in range(16)}
+    start = {rid: int(i % 3 == 2) for i, rid in enumerate(prompts)}     # a third of them prefilled one step later
+    shape = (32, 8, 128, 32, 128, 16 * 48)
+    t_dev, t_host = [], []
+    b = kvcomp_scenario(dev, False, t_host, shape, prompts, start, n_steps=8, keep_caches=False)
+    last_b = b[-1][1]
+    del b
+    a = kvcomp_scenario(dev, True, t_dev, shape, prompts, start, n_steps=8, keep_caches=False)
+    for l, (x, y) in enumerate(zip(a[-1][1], last_b)):
+        assert torch.equal(x, y), l
+    ms = lambda t: " ".join(f"{x * 1e3:.1f}" for s, x in t)
+    print(f"\nhost time of a step's hooks, steps 0-7 (16 requests, 32 layers; prefills in steps 0 and 1, first decode "
+          f"steps - windows written back, retrieval - in 1 and 2, retrieval again in 5 and 6), ms: batched {ms(t_dev)}; "
+          f"per request {ms(t_host)}")

@@ -1,0 +1,166 @@
+"""Batched, device-resident retrieval step of the KvComp plugin.
+
+The reference scores and loads one request and one layer at a time
+(ucm/sparse/kvcomp/kvcomp.py:361-389): the query slice of the request, its
+group mean, the hash codes, the Hamming scores against the request's blocks, a
+``topk`` whose result comes back to the host as a list, the list turned into
+block hashes and two ``store.load`` calls with a tensor view per block, and a
+wait for them.  When the store's blocks are device-addressable
+(``UcmHipBlockStore.device_pool``) a layer's hook needs none of the host round
+trips and covers all requests of the step at once:
+
+* every request owns a row (its segment of the summary tables, which the plugin
+  already keeps); per step the host uploads one descriptor from pinned memory -
+  for each request that retrieves, the first candidate block, how many
+  candidates, how many to pick, which token of the step's batch is its query;
+* the hook takes the group means of all those queries with the reference's own
+  torch expression, then ONE ``ucm_hash_encode_queries``, ONE
+  ``ucm_hash_score_blocks``, ONE ``ucm_topk_windows`` (ascending picks, as the
+  reference sorts them) and ONE ``ucm_kv_load_planned`` that copies pick j of
+  every request from the store's pool into that request's j-th middle cache
+  block, K and V - what ``launch_transfer_task("load", hashes, mid)`` does
+  (:283-323), without the wait.
+
+Which steps retrieve, which blocks are candidates and how many are picked are
+the reference's rules (``ReqStatePerLayer.retrieval`` :202-258).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ... import ops
+
+
+class KvCompDevicePath:
+    def __init__(self, plugin, pool: torch.Tensor, pool_block_bytes: int, device):
+        self.plugin, self.pool, self.pool_block_bytes, self.device = plugin, pool, pool_block_bytes, device
+        L, rows, mb, h = plugin.total_num_hidden_layers, plugin.max_num_seqs, plugin.max_blocks, plugin.num_key_heads
+        i32 = dict(dtype=torch.int32, device=device)
+        self.rows, self.max_blocks = rows, mb
+        self.idx = torch.full((L, rows, mb), -1, **i32)           # picks, as offsets from the row's first candidate
+        self.cnt = torch.zeros((L, rows), **i32)
+        self.src_table = torch.full((rows, mb), -1, **i32)        # candidate i of a row -> block of the store's pool
+        self.dst_table = torch.full((rows, mb), -1, **i32)        # pick j of a row -> cache block
+        self.q_codes = torch.empty((1, rows, h, 16), dtype=torch.uint8, device=device)
+        self.q_sum = torch.empty((1, rows, 128), dtype=torch.int16, device=device)
+        self.qbar = torch.empty((1, rows, h, 16), dtype=torch.uint8, device=device)
+        # per-step descriptor, one entry per retrieving request: seg_off, seg_len, topk_len, its token in the step's
+        # query tensor, its table row; a ring of pinned buffers, the copy of one step may still be in flight while the
+        # host fills the next
+        self._ring = [torch.empty(5 * rows, dtype=torch.int32).pin_memory() for _ in range(4)]
+        self._ring_dev = [torch.empty(5 * rows, **i32) for _ in range(4)]
+        self._turn = 0
+        self.n_src: Dict[object, int] = {}                        # candidates of a request whose pool block is uploaded
+        self.dst_ids: Dict[object, tuple] = {}
+        self.active: List[object] = []                            # requests that retrieve in this step
+        self.first_of: Dict[object, int] = {}
+        self.seg_off = self.seg_len = self.topk_len = self.tokens = self.src_step = self.dst_step = None
+        self.slot_of_step: Dict[object, int] = {}
+        self.max_len = self.total = 0
+        self._kv: Dict[int, ops.LayerPointers] = {}
+        self._geom: Dict[int, tuple] = {}
+
+    def register_kv_cache(self, layer_id: int, kv_cache: torch.Tensor) -> None:
+        if layer_id not in self._kv or self._geom[layer_id][3] != kv_cache.data_ptr():
+            self._kv[layer_id] = ops.LayerPointers([kv_cache])
+            self._geom[layer_id] = (kv_cache.stride(0) * kv_cache.element_size(), kv_cache.stride(1) * kv_cache.element_size(),
+                                    kv_cache.shape[1], kv_cache.data_ptr())
+
+    # ---- per step ---------------------------------------------------------------------------
+    def build_step(self, metas, query_start: List[int]) -> None:
+        """metas: the step's requests; query_start[i]: first token of request i in the step's query tensor.  Fills
+        the descriptor for the requests that retrieve in this step (kvcomp.py:361-371, :202-215)."""
+        p = self.plugin
+        stride, init, local = p.cfg["retrieval_stride"], p.cfg["init_window_sz"], p.cfg["local_window_sz"]
+        self.active, self.max_len, self.total = [], 0, 0
+        rows = self.rows
+        host = None
+        for meta, a in zip(metas, query_start):
+            states = p.req_states.get(meta.request_id)
+            st = states[0] if states else None
+            if st is None or not st.block_size or meta.step % stride != 1 or meta.num_scheduled_tokens != 1:
+                continue
+            n_blocks = st.num_blocks_hashed
+            mid = meta.vllm_block_ids[init:-local]
+            top_k, first, end = len(mid), init, n_blocks - local + 1
+            if end <= first or top_k <= 0:
+                continue
+            count = end - first
+            k = count if top_k >= n_blocks else min(top_k, count)     # every candidate, or the best top_k of them
+            row = p.segment_base(meta.request_id) // p.max_blocks
+            if host is None:
+                self._turn = (self._turn + 1) % len(self._ring)
+                host = self._ring[self._turn].numpy().reshape(5, rows)
+            n = len(self.active)
+            host[0, n], host[1, n], host[2, n], host[3, n], host[4, n] = row * p.max_blocks + first, count, k, a, row
+            self.active.append(meta.request_id)
+            self.first_of[meta.request_id] = first
+            self.max_len = max(self.max_len, count)
+            self.total += count
+            self._sources(meta.request_id, row, first, count)
+            ids = tuple(mid[:k])
+            if self.dst_ids.get(meta.request_id) != ids:
+                self.dst_table[row, : len(ids)] = torch.tensor(ids, dtype=torch.int32, device=self.device)
+                self.dst_ids[meta.request_id] = ids
+        if host is not None:
+            n = len(self.active)
+            dev = self._ring_dev[self._turn]
+            dev.copy_(self._ring[self._turn], non_blocking=True)
+            d = dev.view(5, rows)
+            self.seg_off, self.seg_len, self.topk_len, self.tokens = d[0, :n], d[1, :n], d[2, :n], d[3, :n]
+            table_rows = d[4, :n].long()
+            self.src_step = self.src_table.index_select(0, table_rows)      # the step's requests side by side
+            self.dst_step = self.dst_table.index_select(0, table_rows)
+            self.slot_of_step = {r: i for i, r in enumerate(self.active)}
+
+    def _sources(self, request_id, row: int, first: int, count: int) -> None:
+        """Pool blocks of candidates first .. first+count-1 (the hash -> store lookup, once per block)."""
+        done = self.n_src.get(request_id, 0)
+        if done >= count:
+            return
+        from .kvcomp import ReqStatePerLayer                 # (the plugin module imports this one)
+
+        slot_of = self.plugin.connector.slot_of
+        name = ReqStatePerLayer.block_hash
+        src = [slot_of.get(name(request_id, first + i), -1) for i in range(done, count)]
+        self.src_table[row, done:count] = torch.tensor(src, dtype=torch.int32, device=self.device)
+        self.n_src[request_id] = count
+
+    # ---- hook -------------------------------------------------------------------------------
+    def attention_begin(self, layer_id: int, query: torch.Tensor) -> None:
+        if not self.active:
+            return
+        p = self.plugin
+        h, d, b = p.num_key_heads, p.head_size, len(self.active)
+        q = query.index_select(0, self.tokens.long())                 # [b, q heads, d], the model's dtype
+        hq = q.shape[1]
+        if hq > h:                                                    # kvcomp.py:228-233
+            q = q.view(b, h, -1, d).mean(2)
+        elif hq < h:
+            q = torch.repeat_interleave(q, h // hq, 1)
+        q = q.to(torch.bfloat16).reshape(1, b, h, d).contiguous()
+        q_codes, q_sum, qbar = self.q_codes[:, :b], self.q_sum[:, :b], self.qbar[:, :b]
+        ops.hash_encode_queries(q, p.hash_encoder.hash_weights, h, q_codes, q_sum, qbar, b)
+        l = slice(layer_id, layer_id + 1)
+        ops.hash_score_blocks(0, q_sum, qbar, p.colsum[l], p.block_codes[l], self.seg_off, self.seg_len, self.total,
+                              p.scores[l], round_fp16=bool(p.cfg["fp16_scores"]))
+        idx, cnt = self.idx[l, :b], self.cnt[l, :b]
+        ops.topk_windows(p.scores[l], self.seg_off, self.seg_len, self.topk_len, self.max_len, idx, cnt, start_w=0, end_w=0)
+        kv_stride, block_bytes, num_blocks, _ = self._geom[layer_id]
+        ops.kv_load_planned(self._kv[layer_id], 0, layer_id, 1, kv_stride, block_bytes, num_blocks, self.pool,
+                            self.pool_block_bytes, idx, self.src_step, self.dst_step, None, load_count=cnt)
+
+    def selection(self, layer_id: int, request_id) -> Optional[List[int]]:
+        """Logical blocks picked for the request in this layer, ascending (reads back).  Valid until the next step in
+        which any request retrieves: the tables hold the latest retrieval only."""
+        i = self.slot_of_step.get(request_id)
+        if i is None:
+            return None
+        n = int(self.cnt[layer_id, i])
+        return [self.first_of[request_id] + int(x) for x in self.idx[layer_id, i, :n].tolist()]
+
+    def request_finished(self, request_id) -> None:
+        for table in (self.n_src, self.dst_ids, self.first_of):
+            table.pop(request_id, None)

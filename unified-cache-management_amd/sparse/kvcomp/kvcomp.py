@@ -35,6 +35,7 @@ import torch
 from ... import ops
 from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
 from ..esa.esa import get_offset
+from .device_path import KvCompDevicePath
 from .hash_encoder import HashEncoder
 
 ReqType = Union[str, int]
@@ -94,7 +95,15 @@ class ReqStatePerLayer:
         self.block_size = None
         self.k_cache = self.v_cache = None
         self.tasks: Dict[int, object] = {}
-        self.last_selection: Optional[List[int]] = None  # logical block ids of the last retrieval, ascending
+        self._last_selection: Optional[List[int]] = None
+
+    @property
+    def last_selection(self) -> Optional[List[int]]:
+        """Logical block ids of the last retrieval, ascending (read back from the device tables when the batched
+        path made it)."""
+        dev = self.plugin._dev
+        got = dev.selection(self.layer_id, self.req_meta.request_id) if dev is not None else None
+        return self._last_selection if got is None else got
 
     @classmethod
     def block_hash(cls, request_id, block_id) -> str:
@@ -111,7 +120,7 @@ class ReqStatePerLayer:
         self.k_cache, self.v_cache = kv_cache[0], kv_cache[1]
         self.block_size = self.k_cache.shape[1]
         self.num_key_heads, self.head_size = self.k_cache.shape[2], self.k_cache.shape[3]
-        self.plugin.register_layer_cache(self.layer_id, self.k_cache)
+        self.plugin.register_layer_cache(self.layer_id, self.k_cache, kv_cache)
 
     # ---- retrieval -----------------------------------------------------------------------
     def retrieval(self, query: torch.Tensor, top_k: int) -> List[str]:
@@ -130,7 +139,7 @@ class ReqStatePerLayer:
             picked = self.plugin.score_and_select(self.layer_id, self.req_meta.request_id, query, first, end - first,
                                                   min(top_k, end - first))
             chosen = [first + int(i) for i in picked]
-        self.last_selection = chosen
+        self._last_selection = chosen
         return [self.block_hash(self.req_meta.request_id, b) for b in chosen]
 
     # ---- windows -------------------------------------------------------------------------
@@ -256,10 +265,21 @@ class KvComp(UcmSparseBase):
         self.colsum = self.block_codes = self.token_codes = None
         self._layer_ptrs: Dict[int, ops.LayerPointers] = {}
         self._num_blocks: Dict[int, int] = {}
+        # "device_loads": the batched retrieval step that scores, selects and loads on the device for all requests
+        # of a layer at once (needs a store whose blocks a kernel can read, i.e. one with device_pool()); False
+        # keeps the per-request path, which works with any store
+        self._device_loads = bool(self.cfg.get("device_loads", True))
+        self._dev: Optional[KvCompDevicePath] = None
+        self._dev_step_built = True
+        self._kv_caches: Dict[int, torch.Tensor] = {}
 
     # ---- device tables -------------------------------------------------------------------
-    def register_layer_cache(self, layer_id: int, k_cache: torch.Tensor) -> None:
+    def register_layer_cache(self, layer_id: int, k_cache: torch.Tensor, kv_cache: Optional[torch.Tensor] = None) -> None:
         dev = k_cache.device
+        if kv_cache is not None:
+            self._kv_caches[layer_id] = kv_cache
+            if self._dev is not None:
+                self._dev.register_kv_cache(layer_id, kv_cache)
         if self.hash_encoder is None:
             self.hash_encoder = HashEncoder(self.cfg["head_dim"], self.cfg["hash_bits"], k_cache.dtype, dev)
             L, rows, h = self.total_num_hidden_layers, self.max_num_seqs * self.max_blocks, self.num_key_heads
@@ -321,11 +341,39 @@ class KvComp(UcmSparseBase):
             states[layer_id] = ReqStatePerLayer(req_meta, layer_name, self.rank, self.tp_size, self.connector, self)
         return states[layer_id]
 
+    def _device_step(self, layer_name: str, forward_context) -> Optional[KvCompDevicePath]:
+        """The batched path, with this step's descriptor built (at the step's first hook: the token positions come
+        with the forward context), or None when the store's blocks cannot be read by a kernel."""
+        if not self._device_loads or self.hash_encoder is None or not hasattr(self.connector, "device_pool"):
+            return None
+        if self._dev is None:
+            pool, pool_block_bytes = self.connector.device_pool()
+            self._dev = KvCompDevicePath(self, pool, pool_block_bytes, self.colsum.device)
+            for layer_id, kv in self._kv_caches.items():
+                self._dev.register_kv_cache(layer_id, kv)
+        if not self._dev_step_built:
+            attn_md = forward_context.attn_metadata
+            if isinstance(attn_md, dict):
+                attn_md = attn_md[layer_name]
+            starts = attn_md.query_start_loc.tolist()
+            metas = self._sparse_metadata.requests
+            self._dev.build_step(metas, [int(starts[m.index_in_batch]) for m in metas])
+            self._dev_step_built = True
+        return self._dev
+
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        dev = self._device_step(layer_name, forward_context)
+        batched = set(dev.active) if dev is not None else ()
         for req_meta in self._sparse_metadata.requests:
             st = self._state(req_meta, layer_name)
             st.update_meta(req_meta)
-            st.attention_begin(query, key, value, forward_context)
+            if req_meta.request_id in batched:          # dumps done and windows back in place, then one call for all
+                st.wait_for_task_done()
+                st.prepare_init_and_local_window()
+            else:
+                st.attention_begin(query, key, value, forward_context)
+        if batched:
+            dev.attention_begin(int(layer_name.split(".")[2]), query)
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
         for req_meta in self._sparse_metadata.requests:
@@ -343,9 +391,12 @@ class KvComp(UcmSparseBase):
                                  len(req.output_token_ids), n_tok, req.num_computed_tokens,
                                  sparsed.get(req_id, INVALID_SLOT), req.block_ids[0])
         self._sparse_metadata = meta
+        self._dev_step_built = False
 
     def request_finished_in_worker(self, request_id: ReqType) -> None:
         self.req_states.pop(request_id, None)
+        if self._dev is not None:
+            self._dev.request_finished(request_id)
         if request_id in self.segment_of:
             self.free_segments.append(self.segment_of.pop(request_id))
 
