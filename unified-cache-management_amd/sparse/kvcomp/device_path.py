@@ -22,7 +22,9 @@ trips and covers all requests of the step at once:
   (:283-323), without the wait.
 
 Which steps retrieve, which blocks are candidates and how many are picked are
-the reference's rules (``ReqStatePerLayer.retrieval`` :202-258).
+the reference's rules (``ReqStatePerLayer.retrieval`` :202-258).  Blocks that
+became full (``save_blocks`` :325-347) are dumped into the pool and hashed for
+all requests of a layer with one pointer-array copy and one launch.
 """
 from __future__ import annotations
 
@@ -59,6 +61,8 @@ class KvCompDevicePath:
         self.seg_off = self.seg_len = self.topk_len = self.tokens = self.src_step = self.dst_step = None
         self.slot_of_step: Dict[object, int] = {}
         self.max_len = self.total = 0
+        self._save_key = None
+        self._save_src = self._save_dst = self._save_ids = self._save_rows = None
         self._kv: Dict[int, ops.LayerPointers] = {}
         self._geom: Dict[int, tuple] = {}
 
@@ -151,6 +155,38 @@ class KvCompDevicePath:
         kv_stride, block_bytes, num_blocks, _ = self._geom[layer_id]
         ops.kv_load_planned(self._kv[layer_id], 0, layer_id, 1, kv_stride, block_bytes, num_blocks, self.pool,
                             self.pool_block_bytes, idx, self.src_step, self.dst_step, None, load_count=cnt)
+
+    # ---- blocks that became full --------------------------------------------------------------
+    def save_blocks(self, layer_id: int, step_key, batch) -> bool:
+        """batch: (request, cache blocks, logical numbers) of every request with full blocks to save in this step
+        (the same lists in every layer's hook).  One pointer-array copy moves this layer's K and V slices of all of
+        them into the store's pool - what ``launch_transfer_task("dump", ...)`` does per request (kvcomp.py:325-347)
+        - and one launch writes their codes and column sums.  False (nothing done) when the store has no room."""
+        from .kvcomp import ReqStatePerLayer
+
+        p = self.plugin
+        kv_stride, block_bytes, num_blocks, base = self._geom[layer_id]
+        if step_key is not self._save_key:
+            store = p.connector
+            hashes = [ReqStatePerLayer.block_hash(r, b) for r, _, logical in batch for b in logical]
+            if any(rc != 0 for rc in store.create(hashes)):
+                return False
+            physical = [b for _, blocks, _ in batch for b in blocks]
+            rows = [p.segment_base(r) + b for r, _, logical in batch for b in logical]
+            i64 = dict(dtype=torch.int64, device=self.device)
+            src = torch.tensor(physical, **i64) * block_bytes
+            dst = torch.tensor([store.slot_of[h] for h in hashes], **i64) * self.pool_block_bytes + self.pool.data_ptr()
+            self._save_src = torch.cat([src, src + kv_stride])                  # K slices, then V slices
+            self._save_dst = torch.cat([dst, dst + block_bytes])
+            self._save_ids = torch.tensor(physical, dtype=torch.int32, device=self.device)
+            self._save_rows = torch.tensor(rows, dtype=torch.int32, device=self.device)
+            self._save_key = step_key
+        ops.copy_batch(self._save_dst + layer_id * 2 * block_bytes, self._save_src + base, block_bytes)
+        l = slice(layer_id, layer_id + 1)
+        p.hash_encoder.encode_cache_blocks(p._layer_ptrs[layer_id], self._save_ids, self._save_rows, p.block_size,
+                                           p.num_key_heads, p._num_blocks[layer_id], p.colsum[l], p.block_codes[l],
+                                           None if p.token_codes is None else p.token_codes[l])
+        return True
 
     def selection(self, layer_id: int, request_id) -> Optional[List[int]]:
         """Logical blocks picked for the request in this layer, ascending (reads back).  Valid until the next step in

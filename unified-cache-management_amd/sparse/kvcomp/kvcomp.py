@@ -185,9 +185,10 @@ class ReqStatePerLayer:
             self.store_instance.wait(task)
         self.tasks.clear()
 
-    def save_blocks(self, num_blocks_need_dump: int) -> None:
+    def blocks_to_save(self, num_blocks_need_dump: int):
+        """(cache blocks, their logical numbers) that became full (kvcomp.py:325-335), counted as saved."""
         if num_blocks_need_dump <= 0:
-            return
+            return [], []
         ids = self.req_meta.vllm_block_ids
         done = self.num_blocks_hashed
         logical = list(range(done, done + num_blocks_need_dump))
@@ -196,10 +197,16 @@ class ReqStatePerLayer:
         else:
             physical = ids[-1:]
             logical = logical[:1]
+        self.num_blocks_hashed += len(logical)
+        return physical, logical
+
+    def save_blocks(self, num_blocks_need_dump: int) -> None:
+        physical, logical = self.blocks_to_save(num_blocks_need_dump)
+        if not logical:
+            return
         hashes = [self.block_hash(self.req_meta.request_id, b) for b in logical]
         self.launch_transfer_task("dump", hashes, physical)
         self.plugin.hash_blocks(self.layer_id, self.req_meta.request_id, physical, logical)
-        self.num_blocks_hashed += len(logical)
 
     # ---- hooks ---------------------------------------------------------------------------
     def attention_begin(self, query, key, value, forward_context) -> None:
@@ -217,10 +224,18 @@ class ReqStatePerLayer:
         self.launch_transfer_task("load", hashes, mid)
         self.wait_for_task_done()
 
-    def attention_finished(self, query, key, value, attn_output, forward_context) -> None:
+    def attention_finished(self, query, key, value, attn_output, forward_context, batch=None) -> None:
+        """batch: a list the blocks to save are appended to instead of being dumped and hashed here (the plugin
+        then saves the blocks of all requests of the layer at once)."""
         self.maybe_register_kv_cache(forward_context)
         updated = self.req_meta.num_computed_tokens + self.req_meta.num_scheduled_tokens
-        self.save_blocks(updated // self.block_size - self.num_blocks_hashed)
+        n = updated // self.block_size - self.num_blocks_hashed
+        if batch is None:
+            self.save_blocks(n)
+        else:
+            physical, logical = self.blocks_to_save(n)
+            if logical:
+                batch.append((self.req_meta.request_id, physical, logical))
         if self.req_meta.is_prefill and self.req_meta.is_last_chunk:
             self.construct_init_and_local_window()
             self.wait_for_task_done()
@@ -268,7 +283,8 @@ class KvComp(UcmSparseBase):
         # "device_loads": the batched retrieval step that scores, selects and loads on the device for all requests
         # of a layer at once (needs a store whose blocks a kernel can read, i.e. one with device_pool()); False
         # keeps the per-request path, which works with any store
-        self._device_loads = bool(self.cfg.get("device_loads", True))
+        # (the stored-block layout the kernels address is the one of a single rank, get_offset with tp_size 1)
+        self._device_loads = bool(self.cfg.get("device_loads", True)) and self.tp_size == 1
         self._dev: Optional[KvCompDevicePath] = None
         self._dev_step_built = True
         self._kv_caches: Dict[int, torch.Tensor] = {}
@@ -376,10 +392,21 @@ class KvComp(UcmSparseBase):
             dev.attention_begin(int(layer_name.split(".")[2]), query)
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
+        # with a device-addressable store the full blocks of all requests are dumped and hashed in one go; the
+        # batched path exists from the first layer's first hook on (it needs the summary tables)
+        dev = self._dev if self._device_loads and hasattr(self.connector, "device_pool") else None
+        batch = [] if dev is not None else None
         for req_meta in self._sparse_metadata.requests:
             st = self._state(req_meta, layer_name)
             st.update_meta(req_meta)
-            st.attention_finished(query, key, value, attn_output, forward_context)
+            st.attention_finished(query, key, value, attn_output, forward_context, batch)
+        if batch:
+            layer_id = int(layer_name.split(".")[2])
+            if not dev.save_blocks(layer_id, self._sparse_metadata, batch):      # the store is full: block by block
+                for request_id, physical, logical in batch:
+                    st = self.req_states[request_id][layer_id]
+                    st.launch_transfer_task("dump", [st.block_hash(request_id, b) for b in logical], physical)
+                    self.hash_blocks(layer_id, request_id, physical, logical)
 
     def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata=None) -> None:
         meta = KvCompSparseMetaData()
