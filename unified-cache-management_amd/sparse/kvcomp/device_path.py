@@ -24,7 +24,9 @@ trips and covers all requests of the step at once:
 Which steps retrieve, which blocks are candidates and how many are picked are
 the reference's rules (``ReqStatePerLayer.retrieval`` :202-258).  Blocks that
 became full (``save_blocks`` :325-347) are dumped into the pool and hashed for
-all requests of a layer with one pointer-array copy and one launch.
+all requests of a layer with one pointer-array copy and one launch; the windows
+kept aside at the end of a prefill and written back at the first decode step
+(:260-274, :392-404) take one pointer-array copy per layer each way.
 """
 from __future__ import annotations
 
@@ -62,6 +64,10 @@ class KvCompDevicePath:
         self.slot_of_step: Dict[object, int] = {}
         self.max_len = self.total = 0
         self._save_key = None
+        self.windows: Dict[object, torch.Tensor] = {}              # per request: [layer][K|V][window block] bytes
+        self.win_shape: Dict[object, tuple] = {}
+        self._win_key: Dict[str, object] = {}
+        self._win_lists: Dict[str, tuple] = {}
         self._save_src = self._save_dst = self._save_ids = self._save_rows = None
         self._kv: Dict[int, ops.LayerPointers] = {}
         self._geom: Dict[int, tuple] = {}
@@ -188,6 +194,58 @@ class KvCompDevicePath:
                                            None if p.token_codes is None else p.token_codes[l])
         return True
 
+    # ---- the windows kept aside at the end of the prefill ---------------------------------------
+    def _window_blocks(self, ids: List[int], n_head: Optional[int] = None, n_tail: Optional[int] = None) -> List[int]:
+        init, local = self.plugin.cfg["init_window_sz"], self.plugin.cfg["local_window_sz"]
+        if n_head is None:                                   # kvcomp.py:260-274
+            n_head = len(ids[:init])
+            n_tail = min(local, len(ids[init:]))
+        return ids[:n_head] + (ids[-n_tail:] if n_tail > 0 else [])
+
+    def _window_copy(self, layer_id: int, step_key, which: str, metas, to_windows: bool) -> None:
+        """One pointer-array copy between the window blocks of all ``metas`` in this layer's cache and the requests'
+        window buffers ([layer][K|V][window block]); the address lists are built at the step's first hook."""
+        kv_stride, block_bytes, _, base = self._geom[layer_id]
+        if self._win_key.get(which) is not step_key:
+            cache_off, win_addr, win_lstride = [], [], []
+            L = self.plugin.total_num_hidden_layers
+            for meta in metas:
+                rid = meta.request_id
+                if to_windows:
+                    blocks = self._window_blocks(meta.vllm_block_ids)
+                    n_head = len(meta.vllm_block_ids[: self.plugin.cfg["init_window_sz"]])
+                    self.win_shape[rid] = (n_head, len(blocks) - n_head)
+                    self.windows[rid] = torch.empty(L * 2 * len(blocks) * block_bytes, dtype=torch.uint8, device=self.device)
+                else:
+                    blocks = self._window_blocks(meta.vllm_block_ids, *self.win_shape[rid])
+                n, ptr = len(blocks), self.windows[rid].data_ptr()
+                for kv in range(2):
+                    for j, b in enumerate(blocks):
+                        cache_off.append(kv * kv_stride + b * block_bytes)
+                        win_addr.append(ptr + (kv * n + j) * block_bytes)
+                        win_lstride.append(2 * n * block_bytes)
+            i64 = dict(dtype=torch.int64, device=self.device)
+            self._win_lists[which] = tuple(torch.tensor(x, **i64) for x in (cache_off, win_addr, win_lstride))
+            self._win_key[which] = step_key
+        cache_off, win_addr, win_lstride = self._win_lists[which]
+        if cache_off.numel() == 0:
+            return
+        in_cache, in_windows = cache_off + base, win_addr + win_lstride * layer_id
+        if to_windows:
+            ops.copy_batch(in_windows, in_cache, block_bytes)
+        else:
+            ops.copy_batch(in_cache, in_windows, block_bytes)
+
+    def save_windows(self, layer_id: int, step_key, metas) -> None:
+        """The first ``init_window_sz`` and last ``local_window_sz`` blocks of every request that finishes its
+        prefill in this step, copied aside (``construct_init_and_local_window``, kvcomp.py:260-274)."""
+        self._window_copy(layer_id, step_key, "save", metas, True)
+
+    def restore_windows(self, layer_id: int, step_key, metas) -> None:
+        """... and written back into the request's new first and last blocks at its first decode step
+        (``prepare_init_and_local_window``, kvcomp.py:392-404)."""
+        self._window_copy(layer_id, step_key, "restore", metas, False)
+
     def selection(self, layer_id: int, request_id) -> Optional[List[int]]:
         """Logical blocks picked for the request in this layer, ascending (reads back).  Valid until the next step in
         which any request retrieves: the tables hold the latest retrieval only."""
@@ -198,5 +256,5 @@ class KvCompDevicePath:
         return [self.first_of[request_id] + int(x) for x in self.idx[layer_id, i, :n].tolist()]
 
     def request_finished(self, request_id) -> None:
-        for table in (self.n_src, self.dst_ids, self.first_of):
+        for table in (self.n_src, self.dst_ids, self.first_of, self.windows, self.win_shape):
             table.pop(request_id, None)

@@ -237,7 +237,8 @@ class ReqStatePerLayer:
             if logical:
                 batch.append((self.req_meta.request_id, physical, logical))
         if self.req_meta.is_prefill and self.req_meta.is_last_chunk:
-            self.construct_init_and_local_window()
+            if batch is None:
+                self.construct_init_and_local_window()
             self.wait_for_task_done()
 
 
@@ -357,16 +358,27 @@ class KvComp(UcmSparseBase):
             states[layer_id] = ReqStatePerLayer(req_meta, layer_name, self.rank, self.tp_size, self.connector, self)
         return states[layer_id]
 
-    def _device_step(self, layer_name: str, forward_context) -> Optional[KvCompDevicePath]:
-        """The batched path, with this step's descriptor built (at the step's first hook: the token positions come
-        with the forward context), or None when the store's blocks cannot be read by a kernel."""
-        if not self._device_loads or self.hash_encoder is None or not hasattr(self.connector, "device_pool"):
+    def _batched(self, layer_name: str, forward_context) -> Optional[KvCompDevicePath]:
+        """The batched path (created at the first hook that sees a device-addressable store), with this layer's
+        cache registered; None when the store's blocks cannot be read by a kernel."""
+        if not self._device_loads or not hasattr(self.connector, "device_pool"):
             return None
+        layer_id = int(layer_name.split(".")[2])
+        if layer_id not in self._kv_caches:
+            kv_cache = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
+            self.register_layer_cache(layer_id, kv_cache[0], kv_cache)
         if self._dev is None:
             pool, pool_block_bytes = self.connector.device_pool()
             self._dev = KvCompDevicePath(self, pool, pool_block_bytes, self.colsum.device)
-            for layer_id, kv in self._kv_caches.items():
-                self._dev.register_kv_cache(layer_id, kv)
+            for l, kv in self._kv_caches.items():
+                self._dev.register_kv_cache(l, kv)
+        return self._dev
+
+    def _device_step(self, layer_name: str, forward_context) -> Optional[KvCompDevicePath]:
+        """The batched path, with this step's descriptor built (at the step's first hook: the token positions come
+        with the forward context), or None when the store's blocks cannot be read by a kernel."""
+        if self._batched(layer_name, forward_context) is None:
+            return None
         if not self._dev_step_built:
             attn_md = forward_context.attn_metadata
             if isinstance(attn_md, dict):
@@ -388,20 +400,29 @@ class KvComp(UcmSparseBase):
                 st.prepare_init_and_local_window()
             else:
                 st.attention_begin(query, key, value, forward_context)
-        if batched:
-            dev.attention_begin(int(layer_name.split(".")[2]), query)
+        if dev is not None:
+            layer_id = int(layer_name.split(".")[2])
+            first = [m for m in self._sparse_metadata.requests if m.step == 1 and m.request_id in dev.windows]
+            if first:
+                dev.restore_windows(layer_id, self._sparse_metadata, first)
+            if batched:
+                dev.attention_begin(layer_id, query)
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
-        # with a device-addressable store the full blocks of all requests are dumped and hashed in one go; the
-        # batched path exists from the first layer's first hook on (it needs the summary tables)
-        dev = self._dev if self._device_loads and hasattr(self.connector, "device_pool") else None
+        # with a device-addressable store the full blocks of all requests are dumped and hashed in one go, and the
+        # windows of those that finish their prefill copied aside in one go
+        dev = self._batched(layer_name, forward_context)
         batch = [] if dev is not None else None
         for req_meta in self._sparse_metadata.requests:
             st = self._state(req_meta, layer_name)
             st.update_meta(req_meta)
             st.attention_finished(query, key, value, attn_output, forward_context, batch)
+        layer_id = int(layer_name.split(".")[2])
+        if dev is not None:
+            ending = [m for m in self._sparse_metadata.requests if m.is_prefill and m.is_last_chunk]
+            if ending:
+                dev.save_windows(layer_id, self._sparse_metadata, ending)
         if batch:
-            layer_id = int(layer_name.split(".")[2])
             if not dev.save_blocks(layer_id, self._sparse_metadata, batch):      # the store is full: block by block
                 for request_id, physical, logical in batch:
                     st = self.req_states[request_id][layer_id]
