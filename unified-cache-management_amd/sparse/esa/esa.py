@@ -296,7 +296,9 @@ class ESA(UcmSparseBase):
         self._num_blocks: Dict[int, int] = {}
         # "device_loads": the batched path that plans and loads on the device (needs a store whose blocks a
         # kernel can read, i.e. one with device_pool()); False keeps the per-request host path for any store
-        self._device_loads = bool(self.esa_cfg.get("device_loads", True)) and hasattr(store, "device_pool")
+        # (the stored-block layout the load kernel addresses is a single rank's, get_offset with tp_size 1)
+        self._device_loads = (bool(self.esa_cfg.get("device_loads", True)) and hasattr(store, "device_pool")
+                              and self.tp_size == 1)
         self._dev: Optional[EsaDevicePath] = None
 
     def prompt_block_hashes(self, token_ids) -> List[str]:
