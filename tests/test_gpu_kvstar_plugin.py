@@ -18,8 +18,9 @@ def bits(t):
     return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-@pytest.mark.parametrize("prune_ratio,chunks,batched", [(1.0, 1, True), (0.5, 3, True), (0.25, 1, False)])
-def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched):
+@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads", [(1.0, 1, True, True), (0.5, 3, True, False), (0.25, 1, False, True),
+                                                                     (0.25, 1, True, False)])
+def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads):
     """Prefill (one chunk, or three) of 24 full blocks + 5 tokens, then 13 decode steps with stride 4: step 1 restores
     the windows and loads what the prefill group's vote picks; the vote of decode steps 1-4 is queued at step 4 and
     its winners are loaded at step 8; steps 5-8 at step 8 / 12.  Selections are checked against the CPU oracle on the
@@ -35,7 +36,7 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched):
     cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
     cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KVStarMultiStep": {
         "retrieval_stride": stride, "sparse_ratio": ratio, "blk_repre_dim_prune_ratio": prune_ratio,
-        "blk_repre_inner_token_merge": merge, "batch_retrieval": batched}}}
+        "blk_repre_inner_token_merge": merge, "batch_retrieval": batched, "device_loads": device_loads}}}
     slice_bytes = bs * hkv * d * 2
     store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 40 * L * 2 * slice_bytes})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)

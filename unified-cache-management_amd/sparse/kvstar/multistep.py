@@ -37,6 +37,7 @@ import torch
 
 from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
 from ..esa.esa import _kv_cache_blocks, block_hash_func, get_offset
+from ... import ops
 from . import retrieve as kvstar_retrieve
 
 ReqType = Union[str, int]
@@ -49,6 +50,8 @@ DEFAULTS = {
     "blk_repre_dim_prune_ratio": 0.25,
     "blk_repre_inner_token_merge": 2,
     "batch_retrieval": True,      # not in the reference: one launch per layer for all requests that retrieve in a step
+    "device_loads": True,         # not in the reference: with a store whose blocks a kernel can read (device_pool()),
+                                  # the blocks every request of a layer loads move in one pointer-array copy
 }
 
 
@@ -172,6 +175,7 @@ class ReqPerLayerState:
         self.d_pruned_index = None
         self.local_tp_rank, self.total_tp_size = rank, tp_size
         self.blk_trans_tasks: Dict[int, object] = {}
+        self.load_sink: Optional[list] = None            # set by the plugin: loads are collected, not issued here
         self.standby_query_group: Dict[str, list] = {}
         self.do_retrieve_query_group: Dict[str, torch.Tensor] = {}
         self.step_group_retrieve_result: Dict[str, List[str]] = {}
@@ -348,6 +352,9 @@ class ReqPerLayerState:
         if n == 0:
             return
         block_hashes, vllm_block_ids = list(block_hashes[:n]), list(vllm_block_ids[:n])
+        if transfer_type == "load" and self.load_sink is not None:
+            self.load_sink.append((block_hashes, vllm_block_ids))
+            return
         fn = getattr(self.store_instance, transfer_type)
         shape = (self.block_size, self.num_key_heads, self.head_size)
         precision = self.k_cache.element_size()
@@ -409,20 +416,60 @@ class KVStarMultiStep(UcmSparseBase):
     def request_finished_in_worker(self, request_id: ReqType) -> None:
         self.req_states.pop(request_id, None)
 
+    def _load_sink(self) -> Optional[list]:
+        """A list that collects the loads of a hook's requests, when they can be carried out as one copy: the store's
+        blocks must be readable by a kernel, in the stored layout of a single rank (get_offset with tp_size 1)."""
+        if (self.kvstar_multistep_cfg["device_loads"] and hasattr(self.connector, "device_pool")
+                and self.total_tp_size == 1):
+            return []
+        return None
+
+    def _flush_loads(self, sink: list, layer_name: str, forward_context) -> None:
+        """One pointer-array copy for every (stored block -> cache block) pair the hook's requests asked for, K and V
+        (launch_transfer_task("load", ...) per request, multistep.py:452-480).  A block the store does not hold is
+        left out (the per-request path gives up the whole request's load in that case)."""
+        if not sink:
+            return
+        layer_id = int(layer_name.split(".")[2])
+        kv = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
+        pool, pool_block_bytes = self.connector.device_pool()
+        slot_of = self.connector.slot_of
+        es = kv.element_size()
+        kv_stride, block_bytes = kv.stride(0) * es, kv.stride(1) * es
+        cache, stored = kv.data_ptr(), pool.data_ptr() + layer_id * 2 * block_bytes
+        dst, src = [], []
+        for hashes, ids in sink:
+            for h, b in zip(hashes, ids):
+                slot = slot_of.get(h)
+                if slot is None:
+                    continue
+                for plane in (0, 1):
+                    src.append(stored + slot * pool_block_bytes + plane * block_bytes)
+                    dst.append(cache + plane * kv_stride + b * block_bytes)
+        if src:
+            ptrs = torch.tensor([dst, src], dtype=torch.int64).pin_memory().to(kv.device, non_blocking=True)
+            ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
+
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
         batch = _RetrievalBatch() if self.kvstar_multistep_cfg["batch_retrieval"] else None
+        sink = self._load_sink()
         for req_meta in self._sparse_metadata.requests:
             state = self.create_layerwise_req_state(req_meta, layer_name)
             state.update_meta(req_meta, forward_context)
+            state.load_sink = sink
             state.attention_begin(query, key, value, forward_context, batch=batch)
         if batch is not None:
             batch.flush()
+        self._flush_loads(sink, layer_name, forward_context)
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
+        sink = self._load_sink()
         for req_meta in self._sparse_metadata.requests:
             state = self.create_layerwise_req_state(req_meta, layer_name)
             state.update_meta(req_meta, forward_context)
+            state.load_sink = sink
             state.attention_finished(query, key, value, attn_output, forward_context)
+        self._flush_loads(sink, layer_name, forward_context)
 
     def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata=None) -> None:
         meta = KVStarMultiStepSparseMetaData()
