@@ -18,31 +18,36 @@ constexpr int kThreads = 1024;
 constexpr int kUnroll = 8;
 constexpr size_t kStep = static_cast<size_t>(kThreads) * 16 * kUnroll;  // 128 KiB per trip
 
-// One workgroup copies one whole slice (a 256 KiB K or V block = 2 trips).
-// size is a multiple of 16.  All loads of a trip are issued before its first
-// store so that 128 KiB are in flight per workgroup.
+// kN x 16 KiB of a slice: every load is issued before the first store goes out.  Stores that start as the
+// loads trickle in mix reads and writes on the HBM channels and cost about 6 % of the copy rate (1.64 ms ->
+// 1.75 ms for the 5.1 GB gather), hence the wait for ALL of the trip's loads.
+template <int kN>
+__device__ __forceinline__ void copy_trip(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src, size_t base)
+{
+    u32x4 v[kN];
+#pragma unroll
+    for (int u = 0; u < kN; ++u) {
+        v[u] = ucm::gload16_nt(src + base + static_cast<size_t>(u) * kThreads * 16);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int u = 0; u < kN; ++u) {
+        ucm::gstore16_nt(dst + base + static_cast<size_t>(u) * kThreads * 16, v[u]);
+    }
+}
+
+// One workgroup copies one whole slice (a 256 KiB K or V block = 2 trips of 128 KiB).  size is a multiple of
+// 16.  What is left after the 128 KiB trips goes in trips of 64, 32 and 16 KiB (the slices of 64-, 32- and
+// 16-token blocks), each with all its loads in flight at once, and a last partial one.
 __device__ __forceinline__ void copy_slice(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src, size_t size)
 {
     size_t o = 0;
-    for (; o + kStep <= size; o += kStep) {
-        const size_t base = o + threadIdx.x * 16u;
-        u32x4 v[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            v[u] = ucm::gload16_nt(src + base + static_cast<size_t>(u) * kThreads * 16);
-        }
-        // every load of the trip has landed before its first store goes out: stores that
-        // start as the loads trickle in mix reads and writes on the HBM channels and cost
-        // about 6 % of the copy rate (1.64 ms -> 1.75 ms for the 5.1 GB gather)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            ucm::gstore16_nt(dst + base + static_cast<size_t>(u) * kThreads * 16, v[u]);
-        }
-    }
-    for (size_t p = o + threadIdx.x * 16u; p < size; p += static_cast<size_t>(kThreads) * 16) {
-        ucm::gstore16_nt(dst + p, ucm::gload16_nt(src + p));
-    }
+    const size_t mine = threadIdx.x * 16u;
+    for (; o + kStep <= size; o += kStep) { copy_trip<kUnroll>(dst, src, o + mine); }
+    if (o + kStep / 2 <= size) { copy_trip<kUnroll / 2>(dst, src, o + mine); o += kStep / 2; }
+    if (o + kStep / 4 <= size) { copy_trip<kUnroll / 4>(dst, src, o + mine); o += kStep / 4; }
+    if (o + kStep / 8 <= size) { copy_trip<kUnroll / 8>(dst, src, o + mine); o += kStep / 8; }
+    if (o + mine < size) { ucm::gstore16_nt(dst + o + mine, ucm::gload16_nt(src + o + mine)); }
 }
 
 __global__ __launch_bounds__(kThreads) void copy_batch_kernel(void* const* __restrict__ dst,
