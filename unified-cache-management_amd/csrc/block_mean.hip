@@ -37,6 +37,22 @@ __device__ __forceinline__ void widen(const u32x4 v, float (&f)[kCols])
     f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
 }
 
+// acc += token rows t .. t+kN-1, in that order, all kN loads issued before the first add
+template <int kN>
+__device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsigned row, unsigned t, float (&acc)[kCols])
+{
+    u32x4 v[kN];
+#pragma unroll
+    for (int u = 0; u < kN; ++u) { v[u] = ucm::gload16_nt(base + static_cast<size_t>(t + u) * row); }
+#pragma unroll
+    for (int u = 0; u < kN; ++u) {
+        float f[kCols];
+        widen(v[u], f);
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
+    }
+}
+
 // grid: x = block index in the list * col_groups + column group of 1024, y = layer; rows narrower than 1024
 // columns whose thread count divides the workgroup (a tensor-parallel rank's 4, 2 or 1 kv heads of 128) share a
 // workgroup, items_per_group list entries side by side, so that no lane idles
@@ -67,27 +83,13 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     widen(ucm::gload16(base), acc);  // acc = token 0
 
     unsigned t = 1;
-    // full groups of kUnroll tokens: loads first, then the ordered adds
-    for (; t + kUnroll <= block_size; t += kUnroll) {
-        u32x4 v[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            v[u] = ucm::gload16_nt(base + static_cast<size_t>(t + u) * row);
-        }
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-            float f[kCols];
-            widen(v[u], f);
-#pragma unroll
-            for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
-        }
-    }
-    for (; t < block_size; ++t) {
-        float f[kCols];
-        widen(ucm::gload16_nt(base + static_cast<size_t>(t) * row), f);
-#pragma unroll
-        for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
-    }
+    // full groups of kUnroll tokens: loads first, then the ordered adds; what is left (all of a 16-token block
+    // after its first token) goes in groups of 8, 4, 2 and 1, each with its loads issued together
+    for (; t + kUnroll <= block_size; t += kUnroll) { add_rows<kUnroll>(base, row, t, acc); }
+    if (t + 8 <= block_size) { add_rows<8>(base, row, t, acc); t += 8; }
+    if (t + 4 <= block_size) { add_rows<4>(base, row, t, acc); t += 4; }
+    if (t + 2 <= block_size) { add_rows<2>(base, row, t, acc); t += 2; }
+    if (t < block_size) { add_rows<1>(base, row, t, acc); }
 
     const float inv = 1.0f / static_cast<float>(block_size);
 #pragma unroll
