@@ -488,6 +488,22 @@ int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const int32_t* s
                     int out_stride, int32_t* count_out, ucm_stream_t stream);
 
 /*
+ * The order in which KVStar::Execute hands the chosen blocks back
+ * (simd_compute_kernel.cpp:969-977: the heap is emptied smallest pair first
+ * and the list reversed, so blocks come out descending by (score, index)),
+ * restored in place on ucm_kvstar_topk's output: afterwards
+ * idx_io[t*out_stride + j], j < count[t], is the j-th block the reference
+ * returns for task t.  The reference's caller loads the j-th block into the
+ * request's j-th candidate cache block (ucm/sparse/kvstar/multistep.py:410-450),
+ * so with this order ucm_kv_load_planned can follow the list without a host
+ * round trip.  votes, seg_off, seg_len as for ucm_kvstar_topk; count dev
+ * int32[n_tasks] (its count_out); max_count >= every count, at most 4096.
+ */
+int ucm_kvstar_order(const float* votes, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                     int max_count, int32_t* idx_io, int out_stride, const int32_t* count,
+                     ucm_stream_t stream);
+
+/*
  * `num` independent copies of `size` bytes, dst[i] <- src[i]: the batched
  * pointer-array copy of the reference's device layer (H2DKernel / D2HKernel,
  * ucm/store/device/cuda/cuda_device.cu:47-81, reached through

@@ -416,9 +416,12 @@ def test_kvstar_topk_heap_ties(ucm, dev, max_len):
     idx = torch.full((n_tasks, max_len), -1, dtype=torch.int32, device=dev)
     cnt = torch.zeros(n_tasks, dtype=torch.int32, device=dev)
     t = lambda a: torch.from_numpy(a).to(dev)
+    votes[off[4] : off[4] + lens[4]] *= -1.0                    # negative votes and both zeros
     ops.kvstar_topk(t(votes), t(off), t(lens), t(ks), max_len, idx, cnt)
+    ordered = idx.clone()
+    ops.kvstar_order(t(votes), t(off), t(lens), max_len, ordered, cnt)   # the reference's return order, on the device
     torch.cuda.synchronize()
-    idx, cnt = idx.cpu().numpy(), cnt.cpu().numpy()
+    idx, cnt, ordered = idx.cpu().numpy(), cnt.cpu().numpy(), ordered.cpu().numpy()
     for i in range(n_tasks):
         v = votes[off[i] : off[i] + lens[i]]
         want = O.kvstar_topk(v, int(ks[i]))
@@ -427,7 +430,9 @@ def test_kvstar_topk_heap_ties(ucm, dev, max_len):
         assert np.all(np.diff(got) > 0)
         assert sorted(want.tolist()) == got.tolist(), (i, lens[i], ks[i])
         assert sorted(got.tolist(), key=lambda b: (v[b], b), reverse=True) == want.tolist()
-    assert np.all(idx[np.arange(max_len)[None, :] >= cnt[:, None]] == -1)
+        assert ordered[i, : cnt[i]].tolist() == want.tolist(), (i, lens[i], ks[i])
+    for a in (idx, ordered):
+        assert np.all(a[np.arange(max_len)[None, :] >= cnt[:, None]] == -1)
 
 
 def test_kvstar_get_task_result_tie_order(ucm, dev):

@@ -18,9 +18,10 @@ def bits(t):
     return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads", [(1.0, 1, True, True), (0.5, 3, True, False), (0.25, 1, False, True),
-                                                                     (0.25, 1, True, False)])
-def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads):
+@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads,device_plans", [
+    (1.0, 1, True, True, True), (0.5, 3, True, False, True), (0.25, 1, False, True, True), (0.25, 1, True, False, False),
+    (0.25, 1, True, True, False), (0.5, 3, True, True, True)])
+def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads, device_plans):
     """Prefill (one chunk, or three) of 24 full blocks + 5 tokens, then 13 decode steps with stride 4: step 1 restores
     the windows and loads what the prefill group's vote picks; the vote of decode steps 1-4 is queued at step 4 and
     its winners are loaded at step 8; steps 5-8 at step 8 / 12.  Selections are checked against the CPU oracle on the
@@ -36,7 +37,8 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
     cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
     cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KVStarMultiStep": {
         "retrieval_stride": stride, "sparse_ratio": ratio, "blk_repre_dim_prune_ratio": prune_ratio,
-        "blk_repre_inner_token_merge": merge, "batch_retrieval": batched, "device_loads": device_loads}}}
+        "blk_repre_inner_token_merge": merge, "batch_retrieval": batched, "device_loads": device_loads,
+        "device_plans": device_plans}}}
     slice_bytes = bs * hkv * d * 2
     store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 40 * L * 2 * slice_bytes})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
@@ -125,6 +127,8 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
 
     def check_loaded(record, l):
         st = states[l]
+        # with the loads planned on the device nobody has read the list yet; looking at it fetches the host copy
+        assert (record in st.step_group_retrieve_indices) == (not (device_loads and device_plans))
         chosen = st.step_group_retrieve_indices[record]
         votes = expect(record, l)
         check_selection(chosen, votes, n_keep)
@@ -165,3 +169,126 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
                 assert not st.blk_trans_tasks                # waited for at the first step of a stride
     plugin.request_finished_in_worker("7")
     assert "7" not in plugin.req_states
+
+
+def kvstar_serving_scenario(dev, overrides, n_steps, timing):
+    """16 requests of 32-200 prompt blocks, 32 layers: one prefill step for all, then n_steps decode steps with the
+    reference's stride of 8 (votes queued at steps 8 and 16, the first decode group's winners loaded at 16).
+    Returns a position-weighted checksum of every layer's cache after steps 1, 8, 16 and the last one, and every
+    request's chosen lists of layer 0 and the last layer."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.esa.esa import get_offset
+    from ucm_amd.sparse.factory import UcmSparseFactory
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+    import time
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, R = 32, 8, 128, 32, 16, 16
+    lens = [32 + (37 * r * 13) % 169 for r in range(R)]
+    nb = sum(lens) + R + 8
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 256, {})
+    settings = {"retrieval_stride": 8, "sparse_ratio": 0.25, "blk_repre_dim_prune_ratio": 0.25, "blk_repre_inner_token_merge": 2}
+    settings.update(overrides)
+    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KVStarMultiStep": settings}}
+    slice_bytes = bs * hkv * d * 2
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": nb * L * 2 * slice_bytes})
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    plugin.connector = store
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    caches = [(torch.randn(2, nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(torch.bfloat16) for _ in range(L)]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    reqs, first = {}, 2
+    for r in range(R):
+        n_prompt = lens[r] * bs + 5
+        ids = list(range(first, first + lens[r] + 1))
+        first += lens[r] + 1
+        reqs[str(r)] = ns(block_ids=[ids], num_computed_tokens=0, prompt_token_ids=[int(t) for t in synth.permutation(1400 + r, 100000)[:n_prompt]],
+                          output_token_ids=[], num_prompt_tokens=n_prompt, num_output_tokens=0, num_tokens=n_prompt, request_id=str(r),
+                          full_ids=ids)
+    ib = ns(req_id_to_index={str(r): r for r in range(R)})
+
+    def run_step(n_toks, label):
+        so = ns(num_scheduled_tokens={str(r): n_toks[r] for r in range(R)}, req_sparsed_slots={str(r): 0 for r in range(R)})
+        starts = [0]
+        for n in n_toks:
+            starts.append(starts[-1] + n)
+        md = ns(query_start_loc=torch.tensor(starts))
+        fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=md)
+        q = (torch.randn(starts[-1], hq, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        plugin.build_sparse_meta(so, reqs, ib, md)
+        for l in range(L):
+            plugin.attention_begin(q, None, None, names[l], fc)
+            plugin.attention_finished(q, None, None, None, names[l], fc)
+        timing.setdefault(label, []).append(1e3 * (time.perf_counter() - t0))
+        torch.cuda.synchronize()
+        for r in range(R):
+            reqs[str(r)].num_computed_tokens += n_toks[r]
+
+    def digest():
+        weights = None
+        out = []
+        for c in caches:
+            flat = c.view(torch.int16).reshape(-1).to(torch.int64)
+            if weights is None:
+                weights = torch.arange(flat.numel(), device=dev) % 65521 + 1
+            out.append(int((flat * weights).sum()))
+        return out
+
+    run_step([reqs[str(r)].num_prompt_tokens for r in range(R)], "prefill")
+    for r in range(R):                                   # the connector's part: the prompt's blocks under their hashes
+        hashes = plugin.req_states[str(r)][0].block_hashes
+        assert store.create(hashes) == [0] * len(hashes)
+        for l in range(L):
+            for kv in range(2):
+                off = get_offset((bs, hkv, d), 0, 1, 2, l, bool(kv))
+                store.wait(store.dump(hashes, [off] * len(hashes), [caches[l][kv][i] for i in reqs[str(r)].full_ids[: len(hashes)]]))
+        store.commit(hashes)
+    for r in range(R):                                   # the scheduler shrinks every request
+        req = reqs[str(r)]
+        req.output_token_ids.append(1)
+        req.num_output_tokens, req.num_tokens = 1, req.num_prompt_tokens + 1
+        req.block_ids = [req.full_ids[-math.ceil(plugin.estimate_num_slots_sparsed(req) / bs):]]
+        for l in range(L):
+            caches[l][:, req.block_ids[0][:-1]] = 0
+    digests, chosen = {}, {}
+    for step in range(1, n_steps + 1):
+        if step > 1:
+            for r in range(R):
+                req = reqs[str(r)]
+                req.output_token_ids.append(1)
+                req.num_output_tokens, req.num_tokens = step, req.num_prompt_tokens + step
+        kind = "first decode" if step == 1 else "queue + load" if step % 8 == 0 and step >= 16 else "queue" if step % 8 == 0 else "plain"
+        run_step([1] * R, kind)
+        if step in (1, 8, 16, n_steps):
+            for r in range(R):
+                for st in (plugin.req_states[str(r)][0], plugin.req_states[str(r)][L - 1]):
+                    st.wait_for_blk_transfer_task_done()
+            torch.cuda.synchronize()
+            digests[step] = digest()
+        if step in (1, 16):
+            record = "prefill" if step == 1 else "decode1"
+            chosen[step] = [[list(plugin.req_states[str(r)][l].step_group_retrieve_indices[record]) for l in (0, L - 1)] for r in range(R)]
+    return digests, chosen
+
+
+def test_kvstar_plugin_at_serving_size(ucm, dev):
+    """The device path (loads planned from the device's own lists, window and standby copies once per layer) against
+    the host path behind the same batched retrievals (every list read back, two store.load calls per request and
+    layer): the same lists and the same bytes in every cache of every layer.  The reference's flow (one retrieval per
+    request and layer as well) runs a launch of its own per request, whose votes may differ from the batched launch's
+    in the last bits and swap two near-equal blocks of a list, so it is only timed here; the host time of the hooks
+    is printed for all three."""
+    t_dev, t_host, t_ref = {}, {}, {}
+    got = kvstar_serving_scenario(dev, {}, 17, t_dev)
+    torch.cuda.empty_cache()
+    want = kvstar_serving_scenario(dev, {"device_loads": False, "device_plans": False}, 17, t_host)
+    assert got[1] == want[1]
+    assert got[0] == want[0]
+    torch.cuda.empty_cache()
+    kvstar_serving_scenario(dev, {"batch_retrieval": False, "device_loads": False, "device_plans": False}, 17, t_ref)
+    for kind in t_dev:
+        print(f"KVStar hooks, 16 requests x 32 layers, {kind}: {np.median(t_dev[kind]):.1f} ms of host time per step "
+              f"(lists on the host {np.median(t_host[kind]):.1f} ms, the reference's flow {np.median(t_ref[kind]):.1f} ms)")

@@ -24,6 +24,7 @@ SIGNATURES = {
     "ucm_kvstar_votes": [_p, _p, _i, _i, _i, _p, _p, _p, _i64, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
     "ucm_kvstar_votes_tables": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
     "ucm_kvstar_topk": [_p, _p, _p, _p, _i, _i, _p, _i, _p, _p],
+    "ucm_kvstar_order": [_p, _p, _p, _i, _i, _p, _i, _p, _p],
     "ucm_topk_windows": [_p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
     "ucm_esa_retrieve": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _p, _i, _p],
     "ucm_esa_retrieve_static": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _i, _p],

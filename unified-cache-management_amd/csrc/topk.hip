@@ -235,6 +235,56 @@ extern "C" int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const
 }
 
 // ---------------------------------------------------------------------------
+// The order KVStar's heap hands its pairs back in (descending by (score, index),
+// simd_compute_kernel.cpp:969-977), restored on the device: a task's chosen blocks are ranked by counting - the
+// 64-bit keys (ordered score, index) are distinct, so entry j goes to position #{m : key[m] > key[j]}.  One
+// workgroup per task, the keys in LDS, every thread reading the same key at a time (a broadcast).
+namespace {
+
+constexpr int kOrderThreads = 256;
+constexpr int kOrderMax = 4096;
+
+__global__ __launch_bounds__(kOrderThreads) void kvstar_order_kernel(
+    const float* __restrict__ votes, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
+    int32_t* __restrict__ idx, int out_stride, const int32_t* __restrict__ count)
+{
+    __shared__ unsigned long long keys[kOrderMax];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int k = min(count[t], min(out_stride, kOrderMax));
+    const int n = seg_len[t];
+    int32_t* row = idx + static_cast<size_t>(t) * out_stride;
+    const float* v = votes + seg_off[t];
+    for (int j = tid; j < k; j += kOrderThreads) {
+        const int i = row[j];
+        const bool inside = i >= 0 && i < n;             // anything else was not written by the selection: never read
+        keys[j] = (static_cast<unsigned long long>(inside ? ordered_key(v[i]) : 0u) << 32) | static_cast<unsigned>(i);
+    }
+    __syncthreads();
+    for (int j = tid; j < k; j += kOrderThreads) {
+        const unsigned long long mine = keys[j];
+        int rank = 0;
+        for (int m = 0; m < k; ++m) { rank += keys[m] > mine ? 1 : 0; }
+        row[rank] = static_cast<int32_t>(static_cast<unsigned>(mine));
+    }
+}
+
+}  // namespace
+
+extern "C" int ucm_kvstar_order(const float* votes, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                                int max_count, int32_t* idx_io, int out_stride, const int32_t* count,
+                                ucm_stream_t stream)
+{
+    UCM_REQUIRE(n_tasks >= 0 && max_count >= 0, "ucm_kvstar_order: n_tasks=%d max_count=%d", n_tasks, max_count);
+    if (n_tasks == 0 || max_count == 0) { return UCM_OK; }
+    UCM_REQUIRE(votes && seg_off && seg_len && idx_io && count, "ucm_kvstar_order: null pointer");
+    UCM_REQUIRE(out_stride >= max_count, "ucm_kvstar_order: out_stride=%d < max_count=%d", out_stride, max_count);
+    UCM_SUPPORTED(max_count <= kOrderMax, "ucm_kvstar_order: max_count=%d (at most 4096 chosen blocks per task)", max_count);
+    hipLaunchKernelGGL(kvstar_order_kernel, dim3(n_tasks), dim3(kOrderThreads), 0, ucm::as_stream(stream), votes, seg_off,
+                       seg_len, idx_io, out_stride, count);
+    UCM_LAUNCH_CHECK("ucm_kvstar_order");
+}
+
+// ---------------------------------------------------------------------------
 // Resident-set bookkeeping for delta loads: which of a request's staging slots
 // already hold a block of the new selection, and which missing block goes to
 // which freed slot.  One wave per (layer, request), slot j and selection entry

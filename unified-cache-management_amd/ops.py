@@ -6,6 +6,7 @@ host, and enqueues the kernel on torch's current stream through the C ABI
 """
 from __future__ import annotations
 
+import threading
 from typing import Optional, Sequence
 
 import torch
@@ -42,6 +43,46 @@ def _dev(t: torch.Tensor, dtype, name: str) -> int:
 
 def _opt(t: Optional[torch.Tensor], dtype, name: str):
     return None if t is None else _dev(t, dtype, name)
+
+
+class _UploadRing:
+    """Pinned staging for the small descriptor tables the wrappers and plugins send to the device many times per
+    step: a slot is reused once the copy queued from it has completed (an event per slot), so no call allocates
+    pinned memory.  Anything larger than a slot takes the allocator's route."""
+
+    def __init__(self, slots: int = 64, slot_bytes: int = 1 << 16):
+        self.slots, self.slot_bytes = slots, slot_bytes
+        self.buf = None
+        self.events = [None] * slots
+        self.next = 0
+        self.lock = threading.Lock()
+
+    def put(self, host: torch.Tensor, device) -> torch.Tensor:
+        nbytes = host.numel() * host.element_size()
+        if nbytes > self.slot_bytes or nbytes == 0:
+            return host.pin_memory().to(device, non_blocking=True)
+        with self.lock:
+            if self.buf is None:
+                self.buf = torch.empty((self.slots, self.slot_bytes), dtype=torch.uint8, pin_memory=True)
+            i = self.next
+            self.next = (i + 1) % self.slots
+            if self.events[i] is None:
+                self.events[i] = torch.cuda.Event()
+            else:
+                self.events[i].synchronize()
+            stage = self.buf[i, :nbytes].view(host.dtype).view(host.shape)
+            stage.copy_(host)
+            out = stage.to(device, non_blocking=True)
+            self.events[i].record()
+        return out
+
+
+_ring = _UploadRing()
+
+
+def upload(host: torch.Tensor, device) -> torch.Tensor:
+    """A host tensor's values in a new device tensor, copied on the current stream without blocking the host."""
+    return _ring.put(host.contiguous(), device)
 
 
 class LayerPointers:
@@ -179,6 +220,18 @@ def kvstar_topk(votes: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tenso
               _dev(seg_len, torch.int32, "seg_len"), _dev(topk_len, torch.int32, "topk_len"), n_tasks, max_seg_len,
               _dev(idx_out, torch.int32, "idx_out"), idx_out.shape[1], _dev(count_out, torch.int32, "count_out"),
               _stream())
+
+
+def kvstar_order(votes: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, max_count: int, idx: torch.Tensor,
+                 count: torch.Tensor) -> None:
+    """Puts every task's chosen blocks (kvstar_topk's idx [n_tasks, stride] and count [n_tasks]) into the order the
+    reference returns them in: descending by (vote, index)."""
+    n_tasks = count.numel()
+    if idx.dim() != 2 or idx.shape[0] != n_tasks or seg_off.numel() != n_tasks or seg_len.numel() != n_tasks:
+        raise ValueError("idx [n_tasks, stride] and seg_off, seg_len, count [n_tasks] expected")
+    _lib.call("ucm_kvstar_order", _dev(votes, torch.float32, "votes"), _dev(seg_off, torch.int32, "seg_off"),
+              _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_count, _dev(idx, torch.int32, "idx"), idx.shape[1],
+              _dev(count, torch.int32, "count"), _stream())
 
 
 def esa_retrieve(data: torch.Tensor, q: torch.Tensor, indexes: torch.Tensor, topk: int, scores_ws: torch.Tensor,
@@ -540,7 +593,7 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
                         d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
                         pruned_sel: Optional[torch.Tensor] = None):
     """kvstar_votes for tasks that each bring a table of their own: tables[t] fp16 [kv_heads, rows_t, d_pad/8, M, 8]
-    (block 0 of task t = its row 0); seg_off only places the votes.  Returns the pointer arrays, which the
+    (block 0 of task t = its row 0); seg_off only places the votes.  Returns the device pointer arrays, which the
     caller keeps alive until the stream has run the call."""
     n_tasks = len(tables)
     if n_tasks == 0:
@@ -566,16 +619,14 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
         d_pruned = pruned.shape[2]
     elif d_pruned is None:
         d_pruned = d_orig
-    host = torch.tensor([[t.data_ptr() for t in tables],
-                         [hs for hs, _ in strides]], dtype=torch.int64).pin_memory()
-    dev = host.to(tables[0].device, non_blocking=True)
+    dev = upload(torch.tensor([[t.data_ptr() for t in tables], [hs for hs, _ in strides]], dtype=torch.int64), tables[0].device)
     ws_max, ws_part = workspace
     _lib.call("ucm_kvstar_votes_tables", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
               _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
               row_stride, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m,
               kv_heads, d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
               _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
-    return host, dev
+    return dev
 
 
 # Launch-shape arguments of three entry points that only benchmarks and tests change (0 = the library's default).

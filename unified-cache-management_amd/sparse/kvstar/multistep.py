@@ -51,7 +51,11 @@ DEFAULTS = {
     "blk_repre_inner_token_merge": 2,
     "batch_retrieval": True,      # not in the reference: one launch per layer for all requests that retrieve in a step
     "device_loads": True,         # not in the reference: with a store whose blocks a kernel can read (device_pool()),
-                                  # the blocks every request of a layer loads move in one pointer-array copy
+                                  # the blocks every request of a layer loads move in one pointer-array copy, and so
+                                  # do the window blocks the requests of a layer save or write back
+    "device_plans": True,         # not in the reference: with device_loads, the chosen blocks are loaded by a kernel
+                                  # that follows the retrieval's own list on the device; the host reads the list only
+                                  # when step_group_retrieve_result / _indices are looked at
 }
 
 
@@ -59,23 +63,44 @@ class _RetrievalBatch:
     """The retrievals the requests of one layer queue during one attention_begin, launched together."""
 
     def __init__(self):
-        self.entries = []     # (state, record, query group fp16 [x, H, d], topk)
+        self.entries = []     # (state, record, the group's query tokens [H, d] each, topk)
         self.after = []       # what the states still have to do once their tasks exist
 
     def flush(self) -> None:
         groups: Dict[tuple, list] = {}
         for e in self.entries:
-            state, _, qg, _ = e
-            groups.setdefault((tuple(qg.shape), state.d_pruned_index is None, tuple(state.blk_repre.shape[1:])), []).append(e)
+            state, _, tokens, _ = e
+            groups.setdefault((len(tokens), tuple(tokens[0].shape), state.d_pruned_index is None,
+                               tuple(state.blk_repre.shape[1:])), []).append(e)
         for members in groups.values():
+            # one stack and one conversion for the query groups of all members (torch.stack(...).to(float16) per
+            # request in the reference, multistep.py:252-254)
+            x = len(members[0][2])
+            q = torch.stack([t for _, _, tokens, _ in members for t in tokens]).to(torch.float16)
+            q = q.view(len(members), x, *q.shape[1:])
+            for i, (st, record, _, _) in enumerate(members):
+                st.do_retrieve_query_group[record] = q[i]
             ids = kvstar_retrieve.AsyncRetrieveBatch(
-                [qg for _, _, qg, _ in members], [st.blk_repre for st, _, _, _ in members],
-                [st.d_pruned_index for st, _, _, _ in members], [k for _, _, _, k in members])
+                q, [st.blk_repre for st, _, _, _ in members],
+                [st.d_pruned_index32 for st, _, _, _ in members], [k for _, _, _, k in members])
             for (st, record, _, _), task_id in zip(members, ids):
                 st.task_waiter[record] = task_id
         for fn in self.after:
             fn()
         self.entries, self.after = [], []
+
+
+class _Collected(dict):
+    """``step_group_retrieve_result`` / ``step_group_retrieve_indices`` of a request: a record whose blocks were
+    loaded straight from the device list is read back the first time somebody asks for it."""
+
+    def __init__(self, collect):
+        super().__init__()
+        self._collect = collect
+
+    def __missing__(self, record):
+        self._collect(record)
+        return dict.__getitem__(self, record)
 
 
 class ReqStage(enum.Enum):
@@ -176,10 +201,15 @@ class ReqPerLayerState:
         self.local_tp_rank, self.total_tp_size = rank, tp_size
         self.blk_trans_tasks: Dict[int, object] = {}
         self.load_sink: Optional[list] = None            # set by the plugin: loads are collected, not issued here
+        self.plan_sink: Optional[list] = None            # set by the plugin: loads that follow the device's own list
+        self.standby_row: Optional[torch.Tensor] = None  # set by the plugin: this step's query token, already copied aside
+        self.window_sink: Optional[list] = None          # set by the plugin: window copies are collected, not issued here
+        self._d_pruned_index32 = None
         self.standby_query_group: Dict[str, list] = {}
         self.do_retrieve_query_group: Dict[str, torch.Tensor] = {}
-        self.step_group_retrieve_result: Dict[str, List[str]] = {}
-        self.step_group_retrieve_indices: Dict[str, List[int]] = {}   # the same results as indices into blk_repre
+        self.step_group_retrieve_result: Dict[str, List[str]] = _Collected(self._collect_planned)
+        self.step_group_retrieve_indices: Dict[str, List[int]] = _Collected(self._collect_planned)   # as indices into blk_repre
+        self._planned: Dict[str, tuple] = {}             # record -> (task id, results, row) of a load planned on the device
         self.task_waiter: Dict[str, int] = {}
         self.num_blocks_dumped = 0
 
@@ -200,10 +230,10 @@ class ReqPerLayerState:
             self.step_group_retrieve_indices[record] = []
             return
         group = [x for x in self.standby_query_group[record] if x is not None]
-        self.do_retrieve_query_group[record] = torch.stack(group).to(torch.float16).contiguous()
         if batch is not None:
-            batch.entries.append((self, record, self.do_retrieve_query_group[record], topk))
+            batch.entries.append((self, record, group, topk))
             return
+        self.do_retrieve_query_group[record] = torch.stack(group).to(torch.float16).contiguous()
         self.task_waiter[record] = kvstar_retrieve.AsyncRetrieveByCPU(
             self.do_retrieve_query_group[record], self.blk_repre, self.d_pruned_index, topk,
             hash(self.req_meta.request_id) & 0x7FFFFFFF, kvstar_retrieve.CPU)
@@ -217,7 +247,15 @@ class ReqPerLayerState:
             prune_ratio=self.sparse_cfg["blk_repre_dim_prune_ratio"], d_pruned_index=self.d_pruned_index,
             prune_dim_enable=prune_dim_enable)
         self.d_pruned_index = index
+        self._d_pruned_index32 = None
         return repre
+
+    @property
+    def d_pruned_index32(self):
+        """The kept channels as the kernels take them (int32), converted once."""
+        if self.d_pruned_index is not None and self._d_pruned_index32 is None:
+            self._d_pruned_index32 = self.d_pruned_index.to(torch.int32).contiguous()
+        return self._d_pruned_index32
 
     def get_retrieve_candidate_block_ids(self) -> List[int]:
         n_keep = math.ceil(self.blk_repre.shape[0] * self.sparse_cfg["sparse_ratio"])
@@ -238,9 +276,11 @@ class ReqPerLayerState:
         if not places:
             return
         assert query_len >= len(places)
-        tail = query[query_start_loc + query_len - len(places) : query_start_loc + query_len]
+        # one copy of the chunk's share of the group; every place keeps a view of it
+        tail = query[query_start_loc + query_len - len(places) : query_start_loc + query_len].clone()
+        group = self.standby_query_group.setdefault("prefill", [None] * self.sparse_cfg["retrieval_stride"])
         for rel, place in enumerate(places):
-            self.save_to_standby("prefill", place, rel, tail)
+            group[place] = tail[rel]
 
     def load_retrieve_result_async(self, load_step: int, candidate_swap_vllm_block_ids: List[int]) -> None:
         """Collects the result of the group two strides back (the prefill group early on) and starts loading
@@ -250,6 +290,24 @@ class ReqPerLayerState:
             record = "prefill"
         else:
             record = "decode" + str((int(math.ceil(load_step / stride)) - 3) * stride + 1)
+        if (self.plan_sink is not None and record in self.task_waiter and record not in self._planned
+                and dict.get(self.step_group_retrieve_result, record) is None):
+            # the chosen blocks never come to the host: the load follows the device's list, after the side stream's
+            # event, and the bookkeeping lists are read back only if somebody looks at them
+            task_id = self.task_waiter[record]
+            found = kvstar_retrieve.DeviceResult(task_id)
+            if found is None:
+                raise RuntimeError(f"retrieval task {task_id} of layer {self.layer_id} is not known")
+            for old_task, _, _ in self._planned.values():
+                kvstar_retrieve.Forget(old_task)
+            self._planned = {record: (task_id,) + found}
+            del self.standby_query_group[record]
+            del self.do_retrieve_query_group[record]
+            if record != "prefill" or load_step == 1:
+                self.plan_sink.append((self, found[0], found[1], list(candidate_swap_vllm_block_ids)))
+            return
+        if dict.get(self.step_group_retrieve_result, record) is None and record in self._planned:
+            self._collect_planned(record)
         if self.step_group_retrieve_result.get(record) is None:
             task_id = self.task_waiter[record]
             kvstar_retrieve.Wait(task_id)
@@ -265,8 +323,29 @@ class ReqPerLayerState:
         if (record != "prefill" or load_step == 1) and len(hashes) > 0:
             self.launch_transfer_task("load", hashes, candidate_swap_vllm_block_ids)
 
+    def _collect_planned(self, record: str) -> None:
+        """The host's copy of a list whose blocks were loaded on the device (KeyError if there is none)."""
+        task_id, results, row = self._planned[record]
+        chosen = results.chosen(row)
+        dict.__setitem__(self.step_group_retrieve_indices, record, chosen)
+        dict.__setitem__(self.step_group_retrieve_result, record, [self.block_hashes[i + self.init_window_sz] for i in chosen])
+
+    def release(self) -> None:
+        for task_id, _, _ in self._planned.values():
+            kvstar_retrieve.Forget(task_id)
+        self._planned = {}
+
     # ---- windows -------------------------------------------------------------------------
+    def window_blocks(self):
+        """(cache blocks of the init window, cache blocks of the local window) as the request stands now."""
+        ids = self.req_meta.vllm_block_ids
+        n_local = min(self.local_window_sz, len(ids[self.init_window_sz :]))
+        return ids[: self.init_window_sz], (ids[-n_local:] if n_local > 0 else [])
+
     def prepare_init_and_local_window(self) -> None:
+        if self.window_sink is not None:
+            self.window_sink.append((self, "restore"))
+            return
         ids = self.req_meta.vllm_block_ids
         self.k_cache[ids[: self.init_window_sz]] = self.init_window[0]
         self.v_cache[ids[: self.init_window_sz]] = self.init_window[1]
@@ -277,6 +356,9 @@ class ReqPerLayerState:
         self.v_cache[ids[-n_local:]] = self.local_window[1]
 
     def construct_init_and_local_window(self) -> None:
+        if self.window_sink is not None:
+            self.window_sink.append((self, "save"))
+            return
         ids = self.req_meta.vllm_block_ids
         head = ids[: self.init_window_sz]
         self.init_window = (self.k_cache[head].clone(), self.v_cache[head].clone())
@@ -306,7 +388,10 @@ class ReqPerLayerState:
         assert meta.query_len == 1, "KVStar series sparse attention doesn't support spec_decode now"
         stride = self.sparse_cfg["retrieval_stride"]
         group_record, place = self.get_decode_step_record()
-        self.save_to_standby(group_record, place, meta.query_start_loc, query)
+        if self.standby_row is not None:
+            self.standby_query_group.setdefault(group_record, [None] * stride)[place] = self.standby_row
+        else:
+            self.save_to_standby(group_record, place, meta.query_start_loc, query)
         later = (lambda fn: fn()) if batch is None else batch.after.append   # with a batch: once the tasks exist
         if meta.step % stride == 0:
             self.retrieval_async(meta.step + 1, len(self.get_retrieve_candidate_block_ids()), batch=batch)
@@ -389,6 +474,8 @@ class KVStarMultiStep(UcmSparseBase):
         self.connector_name = extra.get("ucm_connector_name")
         self.connector = store
         self.token_blk_size = vllm_config.cache_config.block_size
+        self._step_cache: Dict[object, tuple] = {}       # what every layer's hooks of one step share (tables, indices)
+        self._layer_ptrs: Dict[str, tuple] = {}
         if role == UcmSparseRole.WORKER:
             kvstar_retrieve.Setup(kvstar_retrieve.SetupParam(
                 cpuNumaIds=[], physicalCorePerNuma=0, allocRatio=0.75, blkRepreSize=4096, deviceType=kvstar_retrieve.CPU,
@@ -414,7 +501,9 @@ class KVStarMultiStep(UcmSparseBase):
 
     # ---- worker side ---------------------------------------------------------------------
     def request_finished_in_worker(self, request_id: ReqType) -> None:
-        self.req_states.pop(request_id, None)
+        for state in self.req_states.pop(request_id, None) or []:
+            if state is not None:
+                state.release()
 
     def _load_sink(self) -> Optional[list]:
         """A list that collects the loads of a hook's requests, when they can be carried out as one copy: the store's
@@ -447,29 +536,143 @@ class KVStarMultiStep(UcmSparseBase):
                     src.append(stored + slot * pool_block_bytes + plane * block_bytes)
                     dst.append(cache + plane * kv_stride + b * block_bytes)
         if src:
-            ptrs = torch.tensor([dst, src], dtype=torch.int64).pin_memory().to(kv.device, non_blocking=True)
+            ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
             ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
 
-    def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
-        batch = _RetrievalBatch() if self.kvstar_multistep_cfg["batch_retrieval"] else None
+    def _flush_planned(self, plan: list, layer_name: str, forward_context) -> None:
+        """The loads whose lists stay on the device: per launch that produced them, one ucm_kv_load_planned follows
+        the ordered lists (j-th chosen block -> j-th candidate cache block, multistep.py:410-450) once the side
+        stream's event has passed.  The tables that turn a list entry into a stored block and a list position into a
+        cache block are the same for every layer of a step and are built at the first."""
+        if not plan:
+            return
+        layer_id = int(layer_name.split(".")[2])
+        kv = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
+        known = self._layer_ptrs.get(layer_name)
+        if known is None or known[0] != kv.data_ptr():
+            known = self._layer_ptrs[layer_name] = (kv.data_ptr(), ops.LayerPointers([kv]))
+        es = kv.element_size()
+        pool, pool_block_bytes = self.connector.device_pool()
+        groups: Dict[int, list] = {}
+        for entry in plan:
+            groups.setdefault(id(entry[1]), []).append(entry)
+        stream = torch.cuda.current_stream()
+        for members in groups.values():
+            results = members[0][1]
+            n_rows, width = results.idx.shape
+            key = (n_rows, width, tuple((st.req_meta.request_id, row) for st, _, row, _ in members))
+            tables = self._step_cache.get(key)
+            if tables is None:
+                slot_of = self.connector.slot_of
+                longest = max(len(st.block_hashes) for st, _, _, _ in members)
+                src = torch.full((n_rows, max(longest, 1)), -1, dtype=torch.int32)
+                dst = torch.full((n_rows, width), -1, dtype=torch.int32)
+                for st, _, row, candidates in members:
+                    first = st.init_window_sz
+                    stored = [slot_of.get(h, -1) for h in st.block_hashes[first:]]
+                    src[row, : len(stored)] = torch.tensor(stored, dtype=torch.int32)
+                    dst[row, : min(len(candidates), width)] = torch.tensor(candidates[:width], dtype=torch.int32)
+                rows = [row for _, _, row, _ in members]
+                both = ops.upload(torch.cat([src.view(-1), dst.view(-1), torch.tensor(rows, dtype=torch.int32)]), kv.device)
+                tables = self._step_cache[key] = (both[: src.numel()].view(src.shape),
+                                                   both[src.numel() : src.numel() + dst.numel()].view(dst.shape),
+                                                   None if rows == list(range(n_rows)) else both[src.numel() + dst.numel() :])
+            stream.wait_event(results.event)
+            results.idx.record_stream(stream)
+            results.cnt.record_stream(stream)
+            ops.kv_load_planned(known[1], 0, layer_id, 1, kv.stride(0) * es, kv.stride(1) * es, kv.shape[1], pool, pool_block_bytes,
+                                results.idx.unsqueeze(0), tables[0], tables[1], tables[2], load_count=results.cnt.unsqueeze(0))
+
+    def _flush_windows(self, sink: list, layer_name: str, forward_context) -> None:
+        """The window copies of a hook's requests as one pointer-array copy: "save" keeps the init and local window
+        blocks of a request that ends its prefill (multistep.py:326-346: four indexed clones per request), "restore"
+        writes them back into the blocks the request holds at its first decode step (:348-362)."""
+        if not sink:
+            return
+        kv = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
+        es = kv.element_size()
+        kv_stride, block_bytes = kv.stride(0) * es, kv.stride(1) * es
+        if not kv[0, 0].is_contiguous():
+            raise ValueError("cache blocks must be contiguous")
+        cache = kv.data_ptr()
+        dst, src = [], []
+        saves = [st for st, what in sink if what == "save"]
+        if saves:
+            counts = [tuple(len(b) for b in st.window_blocks()) for st in saves]
+            total = sum(a + b for a, b in counts)
+            kept = torch.empty((2, total) + tuple(kv.shape[2:]), dtype=kv.dtype, device=kv.device)   # [K|V][window block]
+            at = 0
+            for st, (n_init, n_local) in zip(saves, counts):
+                head, tail = st.window_blocks()
+                st.init_window = (kept[0, at : at + n_init], kept[1, at : at + n_init])
+                st.local_window = (kept[0, at + n_init : at + n_init + n_local], kept[1, at + n_init : at + n_init + n_local]) if n_local else None
+                for j, b in enumerate(list(head) + list(tail)):
+                    for plane in (0, 1):
+                        src.append(cache + plane * kv_stride + b * block_bytes)
+                        dst.append(kept.data_ptr() + (plane * total + at + j) * block_bytes)
+                at += n_init + n_local
+        for st, what in sink:
+            if what != "restore":
+                continue
+            ids = st.req_meta.vllm_block_ids
+            pairs = list(zip(ids[: st.init_window_sz], range(st.init_window_sz)))
+            for plane in (0, 1):
+                for b, j in pairs:
+                    src.append(st.init_window[plane][j].data_ptr())
+                    dst.append(cache + plane * kv_stride + b * block_bytes)
+                if st.local_window is not None:
+                    n_local = st.local_window[plane].shape[0]
+                    for j, b in enumerate(ids[-n_local:]):
+                        src.append(st.local_window[plane][j].data_ptr())
+                        dst.append(cache + plane * kv_stride + b * block_bytes)
+        if src:
+            ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
+            ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
+
+    def _standby_rows(self, query):
+        """The decoding requests' query tokens of this layer copied aside in one go (``query[start].clone()`` per
+        request in the reference, multistep.py:318-324); every request then keeps a view of its row."""
+        found = self._step_cache.get("standby")
+        if found is None:
+            place, starts = {}, []
+            for m in self._sparse_metadata.requests:
+                if m.stage == ReqStage.DECODE:
+                    place[m.request_id] = len(starts)
+                    starts.append(m.query_start_loc)
+            index = ops.upload(torch.tensor(starts, dtype=torch.int64), query.device) if len(starts) > 1 else None
+            found = self._step_cache["standby"] = (index, place)
+        if found[0] is None:
+            return None, None
+        return query.index_select(0, found[0]), found[1]
+
+    def _hook(self, which: str, layer_name: str, forward_context, *args) -> None:
+        batch = _RetrievalBatch() if which == "attention_begin" and self.kvstar_multistep_cfg["batch_retrieval"] else None
         sink = self._load_sink()
+        plan = [] if sink is not None and self.kvstar_multistep_cfg["device_plans"] else None
+        windows = [] if self.kvstar_multistep_cfg["device_loads"] else None
+        rows = place = None
+        if which == "attention_begin":
+            rows, place = self._standby_rows(args[0])
         for req_meta in self._sparse_metadata.requests:
             state = self.create_layerwise_req_state(req_meta, layer_name)
             state.update_meta(req_meta, forward_context)
-            state.load_sink = sink
-            state.attention_begin(query, key, value, forward_context, batch=batch)
+            state.load_sink, state.plan_sink, state.window_sink = sink, plan, windows
+            state.standby_row = None if rows is None or req_meta.request_id not in place else rows[place[req_meta.request_id]]
+            if which == "attention_begin":
+                state.attention_begin(*args, forward_context, batch=batch)
+            else:
+                state.attention_finished(*args, forward_context)
         if batch is not None:
             batch.flush()
+        self._flush_windows(windows, layer_name, forward_context)
         self._flush_loads(sink, layer_name, forward_context)
+        self._flush_planned(plan, layer_name, forward_context)
+
+    def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        self._hook("attention_begin", layer_name, forward_context, query, key, value)
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
-        sink = self._load_sink()
-        for req_meta in self._sparse_metadata.requests:
-            state = self.create_layerwise_req_state(req_meta, layer_name)
-            state.update_meta(req_meta, forward_context)
-            state.load_sink = sink
-            state.attention_finished(query, key, value, attn_output, forward_context)
-        self._flush_loads(sink, layer_name, forward_context)
+        self._hook("attention_finished", layer_name, forward_context, query, key, value, attn_output)
 
     def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata=None) -> None:
         meta = KVStarMultiStepSparseMetaData()
@@ -487,6 +690,7 @@ class KVStarMultiStep(UcmSparseBase):
                              self.token_blk_size, req.prompt_token_ids, q_start, int(starts[row + 1]) - q_start,
                              self.kvstar_multistep_cfg["retrieval_stride"])
         self._sparse_metadata = meta
+        self._step_cache = {}
 
     # ---- scheduler side ------------------------------------------------------------------
     def estimate_num_slots_sparsed(self, request) -> int:

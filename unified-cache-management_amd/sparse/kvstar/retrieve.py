@@ -15,8 +15,10 @@ the plugin takes (``[init:-local]``, multistep.py:495-497) but keeps the values 
 score kernel streams (``[kv_heads, n, d_pad/8, M, 8]``); ``dense()`` gives the reference's tensor.
 A plain ``[n, M, kv_heads, d_pruned]`` tensor is accepted too and repacked once per call.
 
-Block order in ``data``: descending vote, lower index first among equals (what the
-reference's portable kernel returns; its AVX2 build returns the same set unordered).
+Block order in ``data``: descending by (vote, index), the order in which the reference's heap is
+emptied (simd_compute_kernel.cpp:969-977).  It is restored on the device (``ops.kvstar_order``) and
+read back once per launch, for all its tasks, when the first of them is asked for its list; the
+device copy (``DeviceResult``) lets a caller load the chosen blocks without reading the list at all.
 """
 from __future__ import annotations
 
@@ -51,14 +53,35 @@ class SetupParam:
     localRankId: int
 
 
+class _Results:
+    """What one launch leaves behind for its tasks: the chosen blocks in the reference's order on the device
+    (``idx`` int32 [n_tasks, stride], ``cnt`` int32 [n_tasks]).  The host's copy is made when the first task of the
+    launch is asked for its list, for all of them at once."""
+
+    def __init__(self, event, votes, idx, cnt, keep=()):
+        self.event, self.votes, self.idx, self.cnt, self.keep = event, votes, idx, cnt, keep
+        self._host = None
+
+    def host(self):
+        if self._host is None:
+            self.event.synchronize()
+            self._host = (self.idx.cpu(), self.cnt.cpu())
+        return self._host
+
+    def chosen(self, row: int) -> List[int]:
+        idx, cnt = self.host()
+        return idx[row, : int(cnt[row])].tolist()
+
+
 @dataclass
 class _Task:
-    event: Optional[torch.cuda.Event]
-    votes: Optional[torch.Tensor]       # this task's votes, one per block
-    idx: Optional[torch.Tensor]         # its selected blocks, ascending
-    cnt: Optional[torch.Tensor]         # how many of them
-    keep: tuple = ()
+    results: Optional[_Results]
+    row: int = 0                        # this task's row of the launch's results
     error: Optional[str] = None
+
+    @property
+    def event(self):
+        return None if self.results is None else self.results.event
 
 
 _tasks: Dict[int, _Task] = {}
@@ -142,8 +165,8 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
             q = query_group.contiguous()
             votes = torch.zeros(max(n, 1), dtype=torch.float32, device=dev)
             k = min(int(topk), n)
-            idx = torch.zeros((1, 1, max(n, 1)), dtype=torch.int32, device=dev)
-            cnt = torch.zeros((1, 1), dtype=torch.int32, device=dev)
+            idx = torch.zeros((1, max(n, 1)), dtype=torch.int32, device=dev)
+            cnt = torch.zeros(1, dtype=torch.int32, device=dev)
             keep = (table, q, pruned, sel)
             if n > 0 and k > 0:
                 seg_off = torch.zeros(1, dtype=torch.int32, device=dev)
@@ -151,13 +174,14 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
                 ws = ops.kvstar_workspace(1, h, x * (hq // h), n, m, table.shape[2] * 8, dev)
                 ops.kvstar_votes(q, torch.zeros(1, dtype=torch.int64, device=dev), x, hq, table, seg_off, seg_len, n, votes,
                                  ws, d_pruned=dp, pruned=pruned, pruned_sel=sel)
-                ops.kvstar_topk(votes, seg_off, seg_len, torch.full((1,), k, dtype=torch.int32, device=dev), n, idx[0], cnt[0])
+                ops.kvstar_topk(votes, seg_off, seg_len, torch.full((1,), k, dtype=torch.int32, device=dev), n, idx, cnt)
+                ops.kvstar_order(votes, seg_off, seg_len, k, idx, cnt)
                 keep += (seg_off, seg_len, ws)
-            event = torch.cuda.Event()
-            event.record(_stream)
-        task = _Task(event, votes, idx[0, 0], cnt[0, 0], keep)
+            results = _Results(torch.cuda.Event(), votes, idx, cnt, keep)
+            results.event.record(_stream)
+        task = _Task(results, 0)
     except RuntimeError as e:
-        task = _Task(None, None, None, None, error=str(e))
+        task = _Task(None, error=str(e))
     with _lock:
         _tasks[task_id] = task
     return task_id
@@ -166,7 +190,8 @@ def AsyncRetrieveByCPU(query_group: torch.Tensor, blk_repre: torch.Tensor, d_pru
 def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_ids=None, device_type: DeviceType = CPU) -> List[int]:  # noqa: N802
     """Several retrievals (the requests of one layer) in one launch; returns one task id per entry, to be used
     with Wait / GetTaskResult like those of AsyncRetrieveByCPU.  Every entry must have the same number of query
-    tokens, heads and kept channels, and a BlockRepre (extract_block_repre's result) as representatives."""
+    tokens, heads and kept channels, and a BlockRepre (extract_block_repre's result) as representatives;
+    ``query_groups`` is a list of fp16 [x, q_heads, d] tensors or one fp16 tensor [n_tasks, x, q_heads, d]."""
     global _stream
     if _stream is None:
         _stream = torch.cuda.Stream()
@@ -180,8 +205,11 @@ def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_id
             raise RuntimeError("AsyncRetrieveBatch takes BlockRepre representatives")
         x, hq, d_orig = q0.shape
         _, m, h, dp = r0.shape
+        stacked = isinstance(query_groups, torch.Tensor)      # [n_tasks, x, q_heads, d] in one tensor
+        if stacked and query_groups.dtype != torch.float16:
+            raise RuntimeError("query groups must be float16")
         for qg, r in zip(query_groups, blk_repres):
-            if tuple(qg.shape) != (x, hq, d_orig) or tuple(r.shape[1:]) != (m, h, dp) or qg.dtype != torch.float16:
+            if tuple(r.shape[1:]) != (m, h, dp) or (not stacked and (tuple(qg.shape) != (x, hq, d_orig) or qg.dtype != torch.float16)):
                 raise RuntimeError("the entries of a batch must agree in query tokens, heads, sub-blocks and kept channels")
         if hq % h != 0:
             raise RuntimeError("Num_q_heads must be a divisible by num_kv_heads.")
@@ -201,29 +229,29 @@ def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_id
         ready.record()
         with torch.cuda.stream(_stream):
             _stream.wait_event(ready)
-            q = torch.stack([qg.contiguous() for qg in query_groups])
+            q = query_groups.contiguous() if stacked else torch.stack([qg.contiguous() for qg in query_groups])
             pruned = sel = None
             if with_lists:
                 pruned = torch.stack([i.to(device=dev, dtype=torch.int32) for i in d_pruned_indexes]).contiguous()
                 sel = torch.arange(n_tasks, dtype=torch.int32, device=dev)
-            meta = torch.tensor([offs, lens, [min(int(k), n) for k, n in zip(topks, lens)]], dtype=torch.int32).pin_memory()
-            meta_d = meta.to(dev, non_blocking=True)
+            meta_d = ops.upload(torch.tensor([offs, lens, [min(int(k), n) for k, n in zip(topks, lens)]], dtype=torch.int32), dev)
             q_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (x * hq * d_orig)
             votes = torch.zeros(max(total, 1), dtype=torch.float32, device=dev)
-            idx = torch.zeros((1, n_tasks, max(longest, 1)), dtype=torch.int32, device=dev)
-            cnt = torch.zeros((1, n_tasks), dtype=torch.int32, device=dev)
-            keep = (q, pruned, sel, meta, meta_d, q_off, tuple(r.table for r in blk_repres))
+            idx = torch.zeros((n_tasks, max(longest, 1)), dtype=torch.int32, device=dev)
+            cnt = torch.zeros(n_tasks, dtype=torch.int32, device=dev)
+            keep = (q, pruned, sel, meta_d, q_off, tuple(r.table for r in blk_repres))
             if longest > 0:
                 ws = ops.kvstar_workspace(n_tasks, h, x * (hq // h), longest, m, r0.table.shape[2] * 8, dev)
                 ptrs = ops.kvstar_votes_tables(q, q_off, x, hq, [r.table for r in blk_repres], meta_d[0], meta_d[1], longest, votes, ws,
                                                d_pruned=dp, pruned=pruned, pruned_sel=sel)
-                ops.kvstar_topk(votes, meta_d[0], meta_d[1], meta_d[2], longest, idx[0], cnt[0])
+                ops.kvstar_topk(votes, meta_d[0], meta_d[1], meta_d[2], longest, idx, cnt)
+                ops.kvstar_order(votes, meta_d[0], meta_d[1], longest, idx, cnt)
                 keep += (ws, ptrs)
-            event = torch.cuda.Event()
-            event.record(_stream)
-        tasks = [_Task(event, votes[offs[i] : offs[i] + lens[i]], idx[0, i], cnt[0, i], keep) for i in range(n_tasks)]
+            results = _Results(torch.cuda.Event(), votes, idx, cnt, keep)
+            results.event.record(_stream)
+        tasks = [_Task(results, i) for i in range(n_tasks)]
     except RuntimeError as e:
-        tasks = [_Task(None, None, None, None, error=str(e)) for _ in range(n_tasks)]
+        tasks = [_Task(None, error=str(e)) for _ in range(n_tasks)]
     with _lock:
         for i, t in zip(ids, tasks):
             _tasks[i] = t
@@ -251,15 +279,28 @@ def GetTaskResult(task_id: int):  # noqa: N802
         return {"status": "FAILURE", "error": task.error}
     if not task.event.query():
         return {"status": "RUNNING"}
-    n = int(task.cnt)
-    # descending by (score, index) as the reference's heap pops them (simd_compute_kernel.cpp:969-977): the device
-    # list is ascending, so a stable sort of its reverse leaves equal scores higher index first
-    chosen = task.idx[:n].long().flip(0)
-    order = torch.argsort(task.votes[chosen], descending=True, stable=True)
-    data = chosen[order].tolist()
+    data = task.results.chosen(task.row)
     with _lock:
         _tasks.pop(task_id, None)
     return {"status": "SUCCESS", "data": data}
+
+
+def DeviceResult(task_id: int):  # noqa: N802
+    """(results, row) of a queued task, for callers that use the chosen blocks on the device: ``results.idx[row,
+    :results.cnt[row]]`` are valid on any stream that has waited for ``results.event``.  Raises the task's error if
+    it failed at submission; the task stays known until GetTaskResult or Forget."""
+    with _lock:
+        task = _tasks.get(task_id)
+    if task is None:
+        return None
+    if task.error is not None:
+        raise RuntimeError(task.error)
+    return task.results, task.row
+
+
+def Forget(task_id: int) -> None:  # noqa: N802
+    with _lock:
+        _tasks.pop(task_id, None)
 
 
 def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge: int, prune_ratio: float = 1.0,
