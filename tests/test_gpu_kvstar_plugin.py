@@ -175,7 +175,8 @@ def kvstar_serving_scenario(dev, overrides, n_steps, timing):
     """16 requests of 32-200 prompt blocks, 32 layers: one prefill step for all, then n_steps decode steps with the
     reference's stride of 8 (votes queued at steps 8 and 16, the first decode group's winners loaded at 16).
     Returns a position-weighted checksum of every layer's cache after steps 1, 8, 16 and the last one, and every
-    request's chosen lists of layer 0 and the last layer."""
+    request's chosen lists of layer 0 and the last layer.  Request 5 finishes after step 12, between the queueing of its
+    votes and their load, so the load of step 16 follows 15 of the 16 rows of the launch that produced the lists."""
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.esa.esa import get_offset
     from ucm_amd.sparse.factory import UcmSparseFactory
@@ -208,11 +209,13 @@ def kvstar_serving_scenario(dev, overrides, n_steps, timing):
                           full_ids=ids)
     ib = ns(req_id_to_index={str(r): r for r in range(R)})
 
+    active = list(range(R))
+
     def run_step(n_toks, label):
-        so = ns(num_scheduled_tokens={str(r): n_toks[r] for r in range(R)}, req_sparsed_slots={str(r): 0 for r in range(R)})
-        starts = [0]
-        for n in n_toks:
-            starts.append(starts[-1] + n)
+        so = ns(num_scheduled_tokens={str(r): n_toks[r] for r in active}, req_sparsed_slots={str(r): 0 for r in active})
+        starts = [0] * (R + 1)
+        for r in range(R):
+            starts[r + 1] = starts[r] + (n_toks[r] if r in active else 0)
         md = ns(query_start_loc=torch.tensor(starts))
         fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=md)
         q = (torch.randn(starts[-1], hq, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
@@ -224,7 +227,7 @@ def kvstar_serving_scenario(dev, overrides, n_steps, timing):
             plugin.attention_finished(q, None, None, None, names[l], fc)
         timing.setdefault(label, []).append(1e3 * (time.perf_counter() - t0))
         torch.cuda.synchronize()
-        for r in range(R):
+        for r in active:
             reqs[str(r)].num_computed_tokens += n_toks[r]
 
     def digest():
@@ -255,22 +258,25 @@ def kvstar_serving_scenario(dev, overrides, n_steps, timing):
             caches[l][:, req.block_ids[0][:-1]] = 0
     digests, chosen = {}, {}
     for step in range(1, n_steps + 1):
+        if step == 13:
+            plugin.request_finished_in_worker("5")
+            active.remove(5)
         if step > 1:
-            for r in range(R):
+            for r in active:
                 req = reqs[str(r)]
                 req.output_token_ids.append(1)
                 req.num_output_tokens, req.num_tokens = step, req.num_prompt_tokens + step
         kind = "first decode" if step == 1 else "queue + load" if step % 8 == 0 and step >= 16 else "queue" if step % 8 == 0 else "plain"
         run_step([1] * R, kind)
         if step in (1, 8, 16, n_steps):
-            for r in range(R):
+            for r in active:
                 for st in (plugin.req_states[str(r)][0], plugin.req_states[str(r)][L - 1]):
                     st.wait_for_blk_transfer_task_done()
             torch.cuda.synchronize()
             digests[step] = digest()
         if step in (1, 16):
             record = "prefill" if step == 1 else "decode1"
-            chosen[step] = [[list(plugin.req_states[str(r)][l].step_group_retrieve_indices[record]) for l in (0, L - 1)] for r in range(R)]
+            chosen[step] = [[list(plugin.req_states[str(r)][l].step_group_retrieve_indices[record]) for l in (0, L - 1)] for r in active]
     return digests, chosen
 
 

@@ -122,17 +122,17 @@ class UcmHipBlockStore:
                 raise ValueError("offset outside the stored block")
             store_ptrs.append(base + self.slot_of[b] * self.kv_block_size + off)
         dev = torch.device("cuda", torch.cuda.current_device())
-        host = torch.tensor([store_ptrs, addrs], dtype=torch.int64).pin_memory()
+        host = torch.tensor([store_ptrs, addrs], dtype=torch.int64)
         ready = torch.cuda.Event()
         ready.record()                       # the caller's stream produced / will consume the tensors
         with torch.cuda.stream(self._stream):
             self._stream.wait_event(ready)
-            ptrs = host.to(dev, non_blocking=True)
+            ptrs = ops.upload(host, dev)     # staged through reused pinned memory, copied on this stream
             dst, src = (ptrs[0], ptrs[1]) if to_store else (ptrs[1], ptrs[0])
-            ops.copy_batch(dst.contiguous(), src.contiguous(), sizes[0])
+            ops.copy_batch(dst, src, sizes[0])
             task.event = torch.cuda.Event()
             task.event.record(self._stream)
-        task.keep = (host, ptrs)
+        task.keep = (ptrs,)
         return task
 
     @staticmethod
