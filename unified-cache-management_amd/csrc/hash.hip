@@ -169,11 +169,25 @@ __device__ __forceinline__ void planes_flush(unsigned (&pl)[kPlanes], int* __res
 }
 
 // The same without atomics, for kHeads = 8, 4, 2 or 1 kv heads: the 32 / kHeads lanes of a lane half that hold
-// vectors of one head (lr, lr ^ kHeads, lr ^ 2 kHeads, ...) first add their counts up with shuffles - as bytes, four
+// vectors of one head (lr, lr ^ kHeads, lr ^ 2 kHeads, ...) first add their counts up across lanes - as bytes, four
 // to a register, for the first two levels (a plane set counts at most 63 tiles, four lanes 252), as halfwords for the
 // levels beyond - and lane lr < kHeads then owns head lr's sixteen columns of each of the two column blocks outright.
 // (Thirty-two LDS atomics per lane, with 32 / kHeads lanes on every address, took four times as long as everything
 // else a block of eight heads needs at its end, and more than the block's tiles for one head.)
+// x + (x of the lane kS away), for sums over the lanes lr, lr +- kS, lr +- 2 kS, ... of a 32-lane half: within a row
+// of sixteen lanes a rotation by kS (a DPP operand, no LDS), and for kS = 16 the row exchange of v_permlane16_swap
+// (rows 1 and 3 of one copy against rows 0 and 2 of another, so the two results add up to the pair's sum in both).
+template <int kS>
+__device__ __forceinline__ unsigned coset_add(unsigned x)
+{
+    if constexpr (kS == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+        return r[0] + r[1];
+    } else {
+        return x + static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(x), 0x120 + kS, 0xf, 0xf, false));
+    }
+}
+
 template <int kHeads>
 __device__ __forceinline__ void planes_flush_owner(unsigned (&pl)[kPlanes], int* __restrict__ colsum, int wp, int half, int lr)
 {
@@ -186,14 +200,12 @@ __device__ __forceinline__ void planes_flush_owner(unsigned (&pl)[kPlanes], int*
             const unsigned nib = (pl[p] >> (4 * j)) & 0xfu;
             c += ((nib * 0x00204081u) & 0x01010101u) << p;   // bit i of the nibble -> byte i
         }
-        c += __shfl_xor(c, kHeads, 64);
-        c += __shfl_xor(c, 2 * kHeads, 64);
+        c = coset_add<kHeads>(c);
+        c = coset_add<2 * kHeads>(c);
         unsigned even = c & 0x00ff00ffu, odd = (c >> 8) & 0x00ff00ffu;   // counts of bits 4j, 4j+2 / 4j+1, 4j+3
-#pragma unroll
-        for (int s = 4 * kHeads; s < 32; s <<= 1) {
-            even += __shfl_xor(even, s, 64);
-            odd += __shfl_xor(odd, s, 64);
-        }
+        if constexpr (kHeads <= 1) { even = coset_add<4>(even); odd = coset_add<4>(odd); }
+        if constexpr (kHeads <= 2) { even = coset_add<8>(even); odd = coset_add<8>(odd); }
+        if constexpr (kHeads <= 4) { even = coset_add<16>(even); odd = coset_add<16>(odd); }
         if (lr < kHeads) {
             int* dst = colsum + lr * kBits + (2 * wp + (j >> 2)) * 32 + half * 16 + 4 * (j & 3);
             i32x4 v = *reinterpret_cast<i32x4*>(dst);
