@@ -1,6 +1,7 @@
 /*
  * Host twins of the C ABI: the same prototypes as libucm_hip.so's entry points
- * of the dense retrieval path, of the ESA retrieval worker and of the hash-code path, name + "_cpu", every "dev" pointer a host
+ * of the dense retrieval path, of the ESA retrieval worker, of the hash-code path, of the planned loads, of KVStar's
+ * selection and of the prefetch bookkeeping, name + "_cpu", every "dev" pointer a host
  * pointer, `stream` ignored, the work done before the call returns.  A caller
  * written against one prototype switches between host and device by choosing
  * the symbol.
@@ -38,6 +39,11 @@ TWIN(ucm_esa_retrieve_rows);
 TWIN(ucm_hash_encode_blocks);
 TWIN(ucm_hash_encode_queries);
 TWIN(ucm_hash_score_blocks);
+TWIN(ucm_copy_batch);
+TWIN(ucm_kv_load_planned);
+TWIN(ucm_kvstar_topk);
+TWIN(ucm_kvstar_order);
+TWIN(ucm_prefetch_plan);
 
 /* the oracle's functions these forward to (ucm_oracle.c) */
 float orc_bf16_to_f32(uint16_t h);
@@ -63,6 +69,10 @@ void orc_hash_majority(const uint8_t* token_codes, uint32_t n_blocks, uint32_t b
 void orc_hash_scores_block(const uint8_t* q_codes, const uint8_t* block_codes, uint32_t n_blocks, uint32_t kv_heads,
                            uint32_t nbytes, int32_t* scores);
 float orc_f16_to_f32(uint16_t h);
+int32_t orc_kvstar_topk(const float* final_scores, uint32_t n_blocks, uint32_t topk, int32_t* topk_idx);
+int32_t orc_prefetch_run(int32_t* map_block, int32_t* map_idx, int32_t n_map, const int32_t* topk, int32_t topk_len,
+                         int32_t* free_block, int32_t* free_len, int32_t* success_blocks, int32_t success_cap,
+                         int32_t* success_len, int32_t* load_blocks, int32_t* miss_idxs, int32_t* n_miss);
 uint16_t orc_f32_to_f16(float f);
 
 int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
@@ -526,3 +536,186 @@ int ucm_hash_score_blocks_cpu(int mode, const int16_t* q_sum, const uint8_t* qba
     }
     return UCM_OK;
 }
+
+/* ---- pointer-array copy and planned loads ------------------------------------------------------------------ */
+
+int ucm_copy_batch_cpu(void* const* dst, const void* const* src, size_t num, size_t size, ucm_stream_t stream)
+{
+    (void)stream;
+    if (num == 0 || size == 0) { return UCM_OK; }
+    if (!dst || !src || size % 16) { return UCM_EINVAL; }
+    for (size_t i = 0; i < num; ++i) {
+        if (!dst[i] || !src[i] || ((uintptr_t)dst[i] | (uintptr_t)src[i]) % 16) { return UCM_EINVAL; }
+    }
+    for (size_t i = 0; i < num; ++i) { memmove(dst[i], src[i], size); }
+    return UCM_OK;
+}
+
+int ucm_kv_load_planned_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                            const void* pool, int64_t pool_blocks, size_t pool_block_bytes, int store_first_layer,
+                            const int32_t* load_sel, int n_slots, const int32_t* src_table, int src_stride,
+                            const int32_t* dst_table, int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                            const int32_t* rows, int batch, int table_rows, ucm_stream_t stream)
+{
+    (void)stream;
+    if (batch < 0 || n_slots < 0 || table_rows <= 0) { return UCM_EINVAL; }
+    if (batch == 0 || n_slots == 0) { return UCM_OK; }
+    if (!layers || !pool || !load_sel || !src_table || !dst_table || n_layers <= 0 || num_blocks <= 0 || block_bytes == 0 ||
+        block_bytes % 16 || kv_stride % 16 || pool_block_bytes % 16 || (size_t)num_blocks * block_bytes > kv_stride ||
+        store_first_layer < 0 || pool_blocks < 0 || src_stride < 1 || dst_stride < n_slots || dst_layer_stride < 0 ||
+        (size_t)(store_first_layer + n_layers) * 2 * block_bytes > pool_block_bytes) {
+        return UCM_EINVAL;
+    }
+    for (int l = 0; l < n_layers; ++l) {
+        for (int b = 0; b < batch; ++b) {
+            const int row = rows ? rows[b] : b;
+            if (row < 0 || row >= table_rows) { continue; }
+            int limit = n_slots;
+            if (load_count) {
+                const int32_t c = load_count[(size_t)l * table_rows + row];
+                if (c < limit) { limit = c < 0 ? 0 : c; }
+            }
+            for (int j = 0; j < limit; ++j) {
+                const int32_t sel = load_sel[((size_t)l * table_rows + row) * (size_t)n_slots + j];
+                if (sel < 0 || sel >= src_stride) { continue; }
+                const int32_t from = src_table[(size_t)row * src_stride + sel];
+                if (from < 0 || from >= pool_blocks) { continue; }
+                const int32_t to = dst_table[l * dst_layer_stride + (int64_t)row * dst_stride + j];
+                if (to < 0 || to >= num_blocks) { continue; }
+                for (int kv = 0; kv < 2; ++kv) {
+                    memcpy((uint8_t*)layers[l] + (size_t)kv * kv_stride + (size_t)to * block_bytes,
+                           (const uint8_t*)pool + (size_t)from * pool_block_bytes +
+                               ((size_t)(store_first_layer + l) * 2 + kv) * block_bytes,
+                           block_bytes);
+                }
+            }
+        }
+    }
+    return UCM_OK;
+}
+
+/* ---- KVStar's selection ----------------------------------------------------------------------------------------- */
+
+static int cmp_i32(const void* a, const void* b)
+{
+    const int32_t x = *(const int32_t*)a, y = *(const int32_t*)b;
+    return (x > y) - (x < y);
+}
+
+int ucm_kvstar_topk_cpu(const float* votes, const int32_t* seg_off, const int32_t* seg_len, const int32_t* topk_len,
+                        int n_tasks, int max_seg_len, int32_t* idx_out, int out_stride, int32_t* count_out,
+                        ucm_stream_t stream)
+{
+    (void)stream;
+    if (n_tasks < 0 || max_seg_len < 0) { return UCM_EINVAL; }
+    if (n_tasks == 0) { return UCM_OK; }
+    if (!votes || !seg_off || !seg_len || !topk_len || !idx_out || !count_out || out_stride < max_seg_len) { return UCM_EINVAL; }
+    if (max_seg_len > 4096) { return UCM_ENOTSUP; }
+    for (int t = 0; t < n_tasks; ++t) {
+        int n = seg_len[t];
+        if (n > out_stride) { n = out_stride; }
+        int32_t* out = idx_out + (size_t)t * out_stride;
+        if (n <= 0) { count_out[t] = 0; continue; }
+        const int32_t k = topk_len[t];
+        int32_t got;
+        if (k <= 0 || k >= n) {                      /* everything, as ucm_topk_windows hands it out */
+            for (int i = 0; i < n; ++i) { out[i] = i; }
+            got = n;
+        } else {
+            got = orc_kvstar_topk(votes + seg_off[t], (uint32_t)n, (uint32_t)k, out);   /* the heap's order */
+            qsort(out, (size_t)got, sizeof(int32_t), cmp_i32);                          /* the device's: ascending */
+        }
+        count_out[t] = got;
+    }
+    return UCM_OK;
+}
+
+int ucm_kvstar_order_cpu(const float* votes, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_count,
+                         int32_t* idx_io, int out_stride, const int32_t* count, ucm_stream_t stream)
+{
+    (void)stream;
+    if (n_tasks < 0 || max_count < 0) { return UCM_EINVAL; }
+    if (n_tasks == 0 || max_count == 0) { return UCM_OK; }
+    if (!votes || !seg_off || !seg_len || !idx_io || !count || out_stride < max_count) { return UCM_EINVAL; }
+    if (max_count > 4096) { return UCM_ENOTSUP; }
+    for (int t = 0; t < n_tasks; ++t) {
+        int32_t* row = idx_io + (size_t)t * out_stride;
+        int k = count[t];
+        if (k > out_stride) { k = out_stride; }
+        if (k > 4096) { k = 4096; }
+        const float* v = votes + seg_off[t];
+        /* descending by (vote, index): insertion sort, the lists are short; the two zeros compare equal */
+        for (int a = 1; a < k; ++a) {
+            const int32_t cur = row[a];
+            int b = a - 1;
+            while (b >= 0 && (v[row[b]] < v[cur] || (v[row[b]] == v[cur] && row[b] < cur))) {
+                row[b + 1] = row[b];
+                --b;
+            }
+            row[b + 1] = cur;
+        }
+    }
+    return UCM_OK;
+}
+
+/* ---- GSA prefetch bookkeeping ------------------------------------------------------------------------------------ */
+
+int ucm_prefetch_plan_cpu(const int32_t* map_block, const int32_t* map_len, int32_t* map_idx, int table_rows, int cap,
+                          const int32_t* topk_idx, int topk_stride, const int32_t* topk_len, const int32_t* rows,
+                          const int32_t* bs_index, int batch, int n_layers, int max_bs, int row_len, int32_t* free_block,
+                          int32_t* free_len, int32_t* success_blocks, int32_t* success_len, int32_t* load_blocks,
+                          int32_t* load_count, int32_t* miss_idxs, int32_t* miss_count, ucm_stream_t stream)
+{
+    (void)stream;
+    if (batch < 0 || n_layers <= 0) { return UCM_EINVAL; }
+    if (batch == 0) { return UCM_OK; }
+    if (!map_block || !map_len || !map_idx || !topk_idx || !topk_len || !rows || !bs_index || !free_block || !free_len ||
+        !success_blocks || !success_len || !load_blocks || !load_count || !miss_idxs || !miss_count || table_rows <= 0 ||
+        max_bs <= 0) {
+        return UCM_EINVAL;
+    }
+    if (cap < 1 || cap > 256 || topk_stride < 1 || topk_stride > 256 || row_len < 1) { return UCM_ENOTSUP; }
+    int32_t* blocks = (int32_t*)malloc(sizeof(int32_t) * 256 * 6);
+    if (!blocks) { return UCM_ENOMEM; }
+    int32_t* loads = blocks + 256;
+    int32_t* misses = blocks + 512;
+    int32_t* free_tmp = blocks + 768;
+    int32_t* succ_tmp = blocks + 1024;                  /* 512 entries: hits and served misses */
+    int rc = UCM_OK;
+    for (int l = 0; l < n_layers && rc == UCM_OK; ++l) {
+        for (int i = 0; i < batch; ++i) {
+            const int row = rows[i], b = bs_index[i];
+            int k = topk_len[i] < topk_stride ? topk_len[i] : topk_stride;
+            if (row < 0 || row >= table_rows || b < 0 || b >= max_bs || k <= 0) {   /* the reference skips such a request */
+                if (row >= 0 && row < table_rows) {
+                    load_count[(size_t)l * table_rows + row] = 0;
+                    miss_count[(size_t)l * table_rows + row] = 0;
+                }
+                continue;
+            }
+            const size_t lb = (size_t)l * max_bs + b, lr = (size_t)l * table_rows + row;
+            int n = map_len[row] < cap ? map_len[row] : cap;
+            if (n < 0) { n = 0; }
+            int32_t f = free_len[lb] < row_len ? free_len[lb] : row_len;
+            if (f > 256) { f = 256; }
+            if (f < 0) { f = 0; }
+            memcpy(blocks, map_block + (size_t)row * cap, sizeof(int32_t) * (size_t)n);
+            memcpy(free_tmp, free_block + lb * row_len, sizeof(int32_t) * (size_t)f);
+            int32_t n_succ = 0, n_miss = 0;
+            const int32_t n_load = orc_prefetch_run(blocks, map_idx + lr * cap, n, topk_idx + ((size_t)l * batch + i) * topk_stride,
+                                                    k, free_tmp, &f, succ_tmp, 512, &n_succ, loads, misses, &n_miss);
+            if (n_load < 0) { rc = UCM_EINVAL; break; }      /* a free-list entry that is no block of the map */
+            memcpy(load_blocks + lr * cap, loads, sizeof(int32_t) * (size_t)n_load);
+            memcpy(miss_idxs + lr * topk_stride, misses, sizeof(int32_t) * (size_t)n_miss);
+            for (int p = 0; p < row_len; ++p) { success_blocks[lb * row_len + p] = p < 512 ? succ_tmp[p] : 0; }
+            memcpy(free_block + lb * row_len, free_tmp, sizeof(int32_t) * (size_t)(f < row_len ? f : row_len));
+            free_len[lb] = f;
+            success_len[lb] = n_succ;
+            load_count[lr] = n_load;
+            miss_count[lr] = n_miss;
+        }
+    }
+    free(blocks);
+    return rc;
+}
+

@@ -12,7 +12,8 @@ import synth
 
 TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
-         "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows"]
+         "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
+         "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan"]
 
 
 def twin_caller(signatures):
@@ -278,3 +279,91 @@ def run_esa(call, side):
                     f"slot_of{step}": np.array(side.down(slot_of)).copy(), f"miss{step}": np.array(side.down(miss)).copy()})
     side.sync()
     return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
+
+
+# ---- KVStar's selection, the prefetch bookkeeping and the loads that follow it --------------------------------------
+P_L, P_ROWS, P_CAP, P_TOPK, P_MAX_BS, P_ROW_LEN, P_NB, P_POOL = 2, 3, 8, 6, 4, 8, 40, 24
+P_BLOCK_BYTES = 256
+
+
+def more_inputs():
+    rng = np.random.default_rng(7300)
+    lens = np.array([7, 1, 40, 100, 0], np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    ks = np.array([3, 1, 40, 17, 2], np.int32)                         # the third task keeps everything
+    votes = (rng.integers(0, 4, int(lens.sum())) * 0.25).astype(np.float32)
+    votes[off[3] : off[3] + 10] *= -1                                  # negative votes and both zeros
+    # prefetch: per request the resident cache blocks (the same in every layer) and, per layer, what they hold
+    map_block = np.full((P_ROWS, P_CAP), -1, np.int32)
+    map_len = np.array([6, 8, 5], np.int32)
+    map_idx = np.full((P_L, P_ROWS, P_CAP), -1, np.int32)
+    for r in range(P_ROWS):
+        map_block[r, : map_len[r]] = 2 + r * P_CAP + rng.permutation(P_CAP)[: map_len[r]]
+        for l in range(P_L):
+            map_idx[l, r, : map_len[r]] = rng.permutation(12)[: map_len[r]]
+    rows = np.array([2, 0, P_ROWS, 1], np.int32)                       # the third request names no row of the table
+    bs_index = np.array([0, 3, 1, 2], np.int32)
+    topk_len = np.array([5, 6, 4, 0], np.int32)                        # the fourth selects nothing: skipped
+    topk_idx = np.stack([np.stack([rng.permutation(12)[:P_TOPK] for _ in range(4)]) for _ in range(P_L)]).astype(np.int32)
+    free_block = np.zeros((P_L, P_MAX_BS, P_ROW_LEN), np.int32)
+    free_len = np.zeros((P_L, P_MAX_BS), np.int32)
+    for l in range(P_L):
+        for i in (0, 1):                                               # a free list = some of the request's blocks
+            r, b = rows[i], bs_index[i]
+            pick = rng.permutation(map_len[r])[:4]
+            free_block[l, b, :4] = map_block[r, pick]
+            free_len[l, b] = 4
+    src_table = np.stack([rng.permutation(P_POOL)[:12] for _ in range(P_ROWS)]).astype(np.int32)
+    src_table[0, 3] = -1                                               # a logical block the store does not hold
+    pool = rng.integers(0, 256, (P_POOL, P_L, 2, P_BLOCK_BYTES)).astype(np.uint8)
+    return dict(lens=lens, off=off, ks=ks, votes=votes, map_block=map_block, map_len=map_len, map_idx=map_idx, rows=rows,
+                bs_index=bs_index, topk_len=topk_len, topk_idx=topk_idx, free_block=free_block, free_len=free_len,
+                src_table=src_table, pool=pool)
+
+
+def run_more(call, side):
+    """KVStar's selection and its return order; a pointer-array copy; a round of the prefetch bookkeeping and the
+    loads it plans, from a pool in the stored layout into two layers' caches."""
+    x = more_inputs()
+    out = {}
+    n_tasks, longest = len(x["lens"]), int(x["lens"].max())
+    votes, off, lens, ks = side.up(x["votes"]), side.up(x["off"]), side.up(x["lens"]), side.up(x["ks"])
+    idx, cnt = side.up(np.full((n_tasks, longest), -1, np.int32)), side.up(np.full(n_tasks, -1, np.int32))
+    call("ucm_kvstar_topk", side.ptr(votes), side.ptr(off), side.ptr(lens), side.ptr(ks), n_tasks, longest, side.ptr(idx),
+         longest, side.ptr(cnt), None)
+    side.sync()
+    out["chosen"] = np.array(side.down(idx)).copy()
+    call("ucm_kvstar_order", side.ptr(votes), side.ptr(off), side.ptr(lens), n_tasks, longest, side.ptr(idx), longest,
+         side.ptr(cnt), None)
+    out.update(ordered=idx, chosen_count=cnt)
+    # pointer-array copy: three pieces of 64 bytes, the last two swapped
+    a, b = side.up(np.arange(192, dtype=np.uint8)), side.up(np.zeros(192, np.uint8))
+    src = side.up(np.array([side.ptr(a), side.ptr(a) + 128, side.ptr(a) + 64], np.int64))
+    dst = side.up(np.array([side.ptr(b), side.ptr(b) + 64, side.ptr(b) + 128], np.int64))
+    call("ucm_copy_batch", side.ptr(dst), side.ptr(src), 3, 64, None)
+    out["copied"] = b
+    # one round of the prefetch bookkeeping
+    map_block, map_len, map_idx = side.up(x["map_block"]), side.up(x["map_len"]), side.up(x["map_idx"])
+    rows, bs_index, topk_len, topk_idx = side.up(x["rows"]), side.up(x["bs_index"]), side.up(x["topk_len"]), side.up(x["topk_idx"])
+    free_block, free_len = side.up(x["free_block"]), side.up(x["free_len"])
+    succ, succ_len = side.up(np.full((P_L, P_MAX_BS, P_ROW_LEN), -5, np.int32)), side.up(np.full((P_L, P_MAX_BS), -5, np.int32))
+    load_blocks, load_count = side.up(np.full((P_L, P_ROWS, P_CAP), -1, np.int32)), side.up(np.full((P_L, P_ROWS), -5, np.int32))
+    miss_idxs, miss_count = side.up(np.full((P_L, P_ROWS, P_TOPK), -1, np.int32)), side.up(np.full((P_L, P_ROWS), -5, np.int32))
+    call("ucm_prefetch_plan", side.ptr(map_block), side.ptr(map_len), side.ptr(map_idx), P_ROWS, P_CAP, side.ptr(topk_idx), P_TOPK,
+         side.ptr(topk_len), side.ptr(rows), side.ptr(bs_index), 4, P_L, P_MAX_BS, P_ROW_LEN, side.ptr(free_block),
+         side.ptr(free_len), side.ptr(succ), side.ptr(succ_len), side.ptr(load_blocks), side.ptr(load_count),
+         side.ptr(miss_idxs), side.ptr(miss_count), None)
+    out.update(map_idx=map_idx, free_block=free_block, free_len=free_len, success=succ, success_len=succ_len,
+               load_blocks=load_blocks, load_count=load_count, miss_idxs=miss_idxs, miss_count=miss_count)
+    # the loads it planned: miss j of a row goes into load block j, K and V of both layers
+    caches = [side.up(np.zeros((2, P_NB, P_BLOCK_BYTES), np.uint8)) for _ in range(P_L)]
+    layers = side.pointers(caches)
+    pool, src_table = side.up(x["pool"]), side.up(x["src_table"])
+    call("ucm_kv_load_planned", layers, P_L, P_NB * P_BLOCK_BYTES, P_BLOCK_BYTES, P_NB, side.ptr(pool), P_POOL,
+         P_L * 2 * P_BLOCK_BYTES, 0, side.ptr(miss_idxs), P_TOPK, side.ptr(src_table), 12, side.ptr(load_blocks), P_CAP,
+         P_ROWS * P_CAP, side.ptr(load_count), side.ptr(rows), 4, P_ROWS, None)
+    for l in range(P_L):
+        out[f"cache{l}"] = caches[l]
+    side.sync()
+    return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
+

@@ -106,3 +106,47 @@ def test_esa_twins_reproduce_the_oracle(ucm):
             slot = int(np.argmax(got["load2"][l, row] >= 0))
             assert got["resident2"][l, row, slot] == got["load2"][l, row, slot]
             assert got["resident1"][l, row, slot] not in got["resident2"][l, row]
+
+
+def test_selection_prefetch_and_load_twins_reproduce_the_oracle(ucm):
+    from ucm_amd import _lib
+
+    got, x = cpu_twins.run_more(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    # KVStar's selection: the oracle's literal heap gives the order, its sorted copy the ascending list
+    for t, (a, n, k) in enumerate(zip(x["off"], x["lens"], x["ks"])):
+        if n == 0:
+            assert got["chosen_count"][t] == 0
+            continue
+        want = O.kvstar_topk(x["votes"][a : a + n], int(k))
+        assert got["chosen_count"][t] == len(want)
+        assert got["chosen"][t, : len(want)].tolist() == sorted(want.tolist())
+        assert got["ordered"][t, : len(want)].tolist() == want.tolist()
+        assert (got["ordered"][t, len(want):] == -1).all()
+    assert np.array_equal(got["copied"], np.concatenate([np.arange(64), np.arange(128, 192), np.arange(64, 128)]).astype(np.uint8))
+    # the prefetch round, request by request and layer by layer, against the oracle's single run
+    P = cpu_twins
+    want_cache = [np.zeros((2, P.P_NB, P.P_BLOCK_BYTES), np.uint8) for _ in range(P.P_L)]
+    for l in range(P.P_L):
+        for i in (0, 1):
+            r, b = int(x["rows"][i]), int(x["bs_index"][i])
+            n = int(x["map_len"][r])
+            m_idx = x["map_idx"][l, r, :n].copy()
+            succ, succ_len, loads, miss, free = O.prefetch_run(x["map_block"][r, :n], m_idx, x["topk_idx"][l, i, : x["topk_len"][i]],
+                                                              x["free_block"][l, b, : x["free_len"][l, b]], int(x["free_len"][l, b]),
+                                                              P.P_ROW_LEN)
+            assert np.array_equal(got["map_idx"][l, r, :n], m_idx)
+            assert np.array_equal(got["success"][l, b], succ) and got["success_len"][l, b] == succ_len
+            assert got["load_count"][l, r] == len(loads) and np.array_equal(got["load_blocks"][l, r, : len(loads)], loads)
+            assert got["miss_count"][l, r] == len(miss) and np.array_equal(got["miss_idxs"][l, r, : len(miss)], miss)
+            assert got["free_len"][l, b] == len(free) and np.array_equal(got["free_block"][l, b, : len(free)], free)
+            for j, blk in enumerate(loads):                        # the planned loads, placed by hand
+                stored = x["src_table"][r, miss[j]]
+                if stored >= 0:
+                    want_cache[l][:, blk] = x["pool"][stored, l]
+        # rows no request of the call reached keep what they held; a request that selects nothing reports zero loads
+        assert got["load_count"][l, 1] == 0 and got["miss_count"][l, 1] == 0
+        assert np.array_equal(got["map_idx"][l, 1], x["map_idx"][l, 1])
+        assert (got["success"][l, [1, 2]] == -5).all()
+        assert np.array_equal(got[f"cache{l}"], want_cache[l])
+    assert any(c.any() for c in want_cache)
+

@@ -835,7 +835,7 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     import cpu_twins
     from ucm_amd import _lib, ops
 
-    for run in (cpu_twins.run, cpu_twins.run_hash, cpu_twins.run_esa):   # the dense path; hash codes; the ESA worker
+    for run in (cpu_twins.run, cpu_twins.run_hash, cpu_twins.run_esa, cpu_twins.run_more):   # the dense path; hash codes; the ESA worker; KVStar's selection, prefetch round, planned loads
         want, _ = run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
         got, _ = run(_lib.call, cpu_twins.DeviceSide(ops, dev))
         assert got.keys() == want.keys()
