@@ -73,16 +73,21 @@ class _UploadRing:
             stage = self.buf[i, :nbytes].view(host.dtype).view(host.shape)
             stage.copy_(host)
             out = stage.to(device, non_blocking=True)
-            self.events[i].record()
+            self.events[i].record(torch.cuda.current_stream(device))   # the stream the copy was queued on
         return out
 
 
-_ring = _UploadRing()
+_rings: dict = {}        # one per device: a slot's event belongs to the device it was first recorded on
 
 
 def upload(host: torch.Tensor, device) -> torch.Tensor:
     """A host tensor's values in a new device tensor, copied on the current stream without blocking the host."""
-    return _ring.put(host.contiguous(), device)
+    device = torch.device(device)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    ring = _rings.get(index)
+    if ring is None:
+        ring = _rings.setdefault(index, _UploadRing())
+    return ring.put(host.contiguous(), device)
 
 
 class LayerPointers:
