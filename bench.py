@@ -463,6 +463,7 @@ def main():
         def kvstar_step():
             ops.kvstar_votes(kq, kq_off, kx, HQ, flat, kso, ksl, max_len, kvotes, kws, d_pruned=kdp, pruned=kpr, pruned_sel=ksel)
             ops.kvstar_topk(kvotes, kso, ksl, ktk, max_len, kidx[0], kcnt[0])
+            ops.kvstar_order(kvotes, kso, ksl, max_len, kidx[0], kcnt[0])     # the order the reference returns them in
 
         for _ in range(2):
             kvstar_step()
@@ -490,7 +491,11 @@ def main():
                 kv_cpu_blocks += n_
                 got = kvotes[a_ : a_ + n_].cpu().numpy()
                 assert np.allclose(got, want, rtol=2e-4, atol=2e-6), "KVStar votes differ from the CPU oracle"
-            kv_checked = "votes of 3 sampled tasks within rtol 2e-4 / atol 2e-6 of the CPU oracle (fp32, other summation order)"
+                # the selection and its order are exact functions of the votes: the oracle's heap on the device's own votes
+                heap = oracle.kvstar_topk(got, int(topk[t_ % N_REQ]))
+                assert kidx[0, t_, : int(kcnt[0, t_])].cpu().numpy().tolist() == heap.tolist(), "KVStar selection differs from the heap"
+            kv_checked = ("votes of 3 sampled tasks within rtol 2e-4 / atol 2e-6 of the CPU oracle (fp32, other summation order); "
+                          "their chosen blocks, in order, equal the oracle's heap on the same votes")
         kv_default = n_layers == N_LAYERS and args.seed == 2024 and merge == 2 and kdp == 32
         kvstar_leg = {
             "workload": f"{n_tasks} tasks (layer x request), {kx} query tokens x {HQ} heads, {rows} blocks x {km} sub-block "
@@ -503,7 +508,7 @@ def main():
             "block_repre_traffic": measured_traffic("kvstar_repre", "kvstar_repre_kernel", kv_default),
             "block_repre_algorithmic_bytes": krep_bytes,
             "us_per_step": round(kv_ms * 1e3, 1),
-            "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select)", "bound": "hbm",
+            "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select, order)", "bound": "hbm",
                          "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4),
                          "traffic": measured_traffic("kvstar_votes", "kvstar_score_kernel", kv_default),
