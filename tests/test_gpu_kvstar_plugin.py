@@ -183,6 +183,9 @@ def kvstar_serving_scenario(dev, overrides, n_steps, timing):
     from ucm_amd.store.hip_block_store import UcmHipBlockStore
     import time
 
+    from ucm_amd.sparse.kvstar import retrieve as kvstar_retrieve
+
+    tasks_before = len(kvstar_retrieve._tasks)
     ns = types.SimpleNamespace
     hq, hkv, d, L, bs, R = 32, 8, 128, 32, 16, 16
     lens = [32 + (37 * r * 13) % 169 for r in range(R)]
@@ -277,6 +280,9 @@ def kvstar_serving_scenario(dev, overrides, n_steps, timing):
         if step in (1, 16):
             record = "prefill" if step == 1 else "decode1"
             chosen[step] = [[list(plugin.req_states[str(r)][l].step_group_retrieve_indices[record]) for l in (0, L - 1)] for r in active]
+    for r in active:                                     # every request ends: no retrieval task is left behind
+        plugin.request_finished_in_worker(str(r))
+    assert len(kvstar_retrieve._tasks) == tasks_before and not plugin.req_states
     return digests, chosen
 
 

@@ -331,9 +331,14 @@ class ReqPerLayerState:
         dict.__setitem__(self.step_group_retrieve_result, record, [self.block_hashes[i + self.init_window_sz] for i in chosen])
 
     def release(self) -> None:
+        """The request is over: retrievals nobody will collect are dropped, and with them the buffers of their launch
+        once its last task is gone (the reference keeps every result for the life of the process)."""
         for task_id, _, _ in self._planned.values():
             kvstar_retrieve.Forget(task_id)
+        for task_id in self.task_waiter.values():
+            kvstar_retrieve.Forget(task_id)
         self._planned = {}
+        self.task_waiter = {}
 
     # ---- windows -------------------------------------------------------------------------
     def window_blocks(self):
