@@ -2,6 +2,9 @@
 scores -> selection with block tables and sparse lengths -> two resident-set plans -> gather, each stage against
 the CPU oracle.  The fixed-shape tests pick their edge cases by hand; this one draws head counts, group sizes, head
 dims, block sizes, window sizes, empty and one-block requests, k = 0 and k beyond the request together."""
+import math
+import types
+
 import numpy as np
 import pytest
 import torch
@@ -277,3 +280,127 @@ def test_random_esa_retrieval(ucm, dev, seed):
         assert np.array_equal(lists[b][pos], idx) and len(set(pos.tolist())) == n, ("positions", b)
     others = np.setdiff1d(np.arange(table_rows), rows)
     assert (rc[torch.from_numpy(others).to(dev)] == -7).all()
+
+
+def kvstar_random_scenario(dev, seed, overrides):
+    """Five requests with drawn prompt lengths, arrival steps, prefill chunkings and lifetimes go through the KVStar
+    plugin's hooks on stand-in vLLM objects (head counts, stride, merge, sparse ratio and channel pruning drawn too);
+    the connector's part (the prompt's blocks stored under their hashes) and the scheduler's (the request shrunk to
+    its sparse budget, stale blocks zeroed) happen before a request's first decode step.  Returns, per engine step,
+    the requests scheduled and a position-weighted checksum of every layer's cache."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.esa.esa import get_offset
+    from ucm_amd.sparse.factory import UcmSparseFactory
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+    from test_gpu_host_layer import make_config
+
+    ns = types.SimpleNamespace
+    rng = np.random.default_rng(seed)
+    L, d, bs = 3, 128, 16
+    hkv = int(rng.choice([2, 4])); hq = hkv * int(rng.choice([2, 4]))
+    stride = int(rng.choice([2, 4])); merge = int(rng.choice([2, 4]))
+    ratio = float(rng.choice([0.25, 0.5])); prune = float(rng.choice([1.0, 0.5]))
+    R = 5
+    blocks = rng.integers(6, 41, R); arrive = rng.integers(0, 6, R); chunks = rng.integers(1, 4, R)
+    n_decode = rng.integers(stride * 2 + 2, stride * 4 + 4, R)
+    nb = int(blocks.sum()) + R + 4
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
+    settings = {"retrieval_stride": stride, "sparse_ratio": ratio, "blk_repre_dim_prune_ratio": prune, "blk_repre_inner_token_merge": merge}
+    settings.update(overrides)
+    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KVStarMultiStep": settings}}
+    slice_bytes = bs * hkv * d * 2
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": nb * L * 2 * slice_bytes})
+    plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+    plugin.connector = store
+    g = torch.Generator(device=dev); g.manual_seed(seed)
+    caches = [(torch.randn(2, nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(torch.bfloat16) for _ in range(L)]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    reqs, first = {}, 2
+    for r in range(R):
+        n_prompt = int(blocks[r]) * bs + int(rng.integers(1, bs))
+        ids = list(range(first, first + int(blocks[r]) + 1)); first += int(blocks[r]) + 1
+        cuts = sorted(rng.choice(np.arange(1, n_prompt), int(chunks[r]) - 1, replace=False).tolist()) if chunks[r] > 1 else []
+        sizes = [b - a for a, b in zip([0] + cuts, cuts + [n_prompt])]
+        reqs[str(r)] = ns(block_ids=[ids], num_computed_tokens=0, prompt_token_ids=[int(t) for t in synth.permutation(seed * 10 + r, 100000)[:n_prompt]],
+                          output_token_ids=[], num_prompt_tokens=n_prompt, num_output_tokens=0, num_tokens=n_prompt, request_id=str(r),
+                          full_ids=ids, sizes=sizes, left=int(n_decode[r]), done=False, stored=False)
+    ib = ns(req_id_to_index={str(r): r for r in range(R)})
+    digests = []
+    weights = None
+    t = 0
+    while not all(q.done for q in reqs.values()):
+        sched = {}
+        for r in range(R):
+            q = reqs[str(r)]
+            if q.done or arrive[r] > t:
+                continue
+            if q.sizes:
+                sched[r] = q.sizes.pop(0)
+            else:
+                if not q.stored:                       # first decode step: the connector stored the prompt, the scheduler shrank it
+                    hashes = plugin.req_states[str(r)][0].block_hashes
+                    assert store.create(hashes) == [0] * len(hashes)
+                    for l in range(L):
+                        for kv in range(2):
+                            off = get_offset((bs, hkv, d), 0, 1, 2, l, bool(kv))
+                            store.wait(store.dump(hashes, [off] * len(hashes), [caches[l][kv][i] for i in q.full_ids[: len(hashes)]]))
+                    store.commit(hashes)
+                    q.output_token_ids.append(1); q.num_output_tokens, q.num_tokens = 1, q.num_prompt_tokens + 1
+                    q.block_ids = [q.full_ids[-math.ceil(plugin.estimate_num_slots_sparsed(q) / bs):]]
+                    for l in range(L):
+                        caches[l][:, q.block_ids[0][:-1]] = 0
+                    q.stored = True
+                else:
+                    q.output_token_ids.append(1); q.num_output_tokens += 1; q.num_tokens += 1
+                sched[r] = 1
+        if sched:
+            so = ns(num_scheduled_tokens={str(r): n for r, n in sched.items()}, req_sparsed_slots={str(r): 0 for r in sched})
+            starts = [0] * (R + 1)
+            for r in range(R):
+                starts[r + 1] = starts[r] + sched.get(r, 0)
+            md = ns(query_start_loc=torch.tensor(starts))
+            fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=md)
+            qt = (torch.randn(starts[-1], hq, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+            plugin.build_sparse_meta(so, reqs, ib, md)
+            for l in range(L):
+                plugin.attention_begin(qt, None, None, names[l], fc)
+                plugin.attention_finished(qt, None, None, None, names[l], fc)
+            for r, n in sched.items():
+                q = reqs[str(r)]
+                q.num_computed_tokens += n
+                if q.stored:
+                    q.left -= 1
+                    if q.left == 0:
+                        for st in plugin.req_states[str(r)]:
+                            if st is not None: st.wait_for_blk_transfer_task_done()
+                        plugin.request_finished_in_worker(str(r)); q.done = True
+            for rr, states in plugin.req_states.items():
+                for st in states:
+                    if st is not None: st.wait_for_blk_transfer_task_done()
+            torch.cuda.synchronize()
+            row = []
+            for c in caches:
+                flat = c.view(torch.int16).reshape(-1).to(torch.int64)
+                if weights is None or weights.numel() != flat.numel():
+                    weights = torch.arange(flat.numel(), device=dev) % 65521 + 1
+                row.append(int((flat * weights).sum()))
+            digests.append((t, tuple(sorted(sched)), tuple(row)))
+        t += 1
+    return digests, (hkv, hq, stride, merge, ratio, prune, blocks.tolist(), arrive.tolist(), chunks.tolist(), n_decode.tolist())
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_kvstar_plugin_flow(ucm, dev, seed):
+    """The three ways the KVStar plugin loads what a retrieval chose - a kernel following the list on the device, one
+    pointer-array copy per layer from the lists read back, one store.load per request and K|V - behind the same
+    batched retrievals: the same bytes in every cache after every engine step, and no retrieval task left behind."""
+    from ucm_amd.sparse.kvstar import retrieve as kvstar_retrieve
+
+    before = len(kvstar_retrieve._tasks)
+    planned, drawn = kvstar_random_scenario(dev, seed, {})
+    by_request, _ = kvstar_random_scenario(dev, seed, {"device_loads": False, "device_plans": False})
+    from_lists, _ = kvstar_random_scenario(dev, seed, {"device_plans": False})
+    assert len(planned) == len(by_request) == len(from_lists) > 0
+    for a, b, c in zip(planned, by_request, from_lists):
+        assert a == b == c, (drawn, a[:2])
+    assert len(kvstar_retrieve._tasks) == before
