@@ -273,6 +273,40 @@ def test_kvcomp_batched_path_equals_per_request_path(ucm, dev):
           f"per request {busy_host[len(busy_host) // 2] * 1e3:.2f} ms; slowest {busy_dev[-1] * 1e3:.2f} / {busy_host[-1] * 1e3:.2f} ms")
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_kvcomp_paths_agree_on_drawn_scenarios(ucm, dev, seed):
+    """Head counts, block size, layers, the number of requests, their prompt lengths and the engine step of their
+    prefill drawn from a seeded generator: the batched device path and the per-request path leave the same bytes in
+    every cache after every step and make the same selections."""
+    rng = np.random.default_rng(500 + seed)
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    hq = hkv * int(rng.choice([1, 2, 4]))
+    bs = int(rng.choice([16, 32]))
+    n_layers = int(rng.integers(1, 4))
+    if hkv * bs < 32:                                              # a block is at least one tile of 32 key vectors
+        bs = 32
+    n_req = int(rng.integers(2, 6))
+    prompts = {chr(65 + i): int(rng.integers(1, 40)) * bs + int(rng.integers(0, bs)) for i in range(n_req)}
+    prompts[chr(65 + n_req)] = bs - 2                              # one the plugin leaves alone
+    start = {rid: int(rng.integers(0, 4)) for rid in prompts}
+    start[min(start, key=start.get)] = 0
+    shape = (hq, hkv, 128, n_layers, bs, sum(-(-(n + 12) // bs) for n in prompts.values()) + 8)
+    n_steps = int(rng.integers(8, 15))
+    a = kvcomp_scenario(dev, True, None, shape, dict(prompts), dict(start), n_steps)
+    b = kvcomp_scenario(dev, False, None, shape, dict(prompts), dict(start), n_steps)
+    compared = 0
+    for step, ((sel_a, caches_a), (sel_b, caches_b)) in enumerate(zip(a, b)):
+        for l, (x, y) in enumerate(zip(caches_a, caches_b)):
+            assert torch.equal(x, y), (step, l, shape, prompts, start)
+        assert sel_a.keys() == sel_b.keys()
+        for rid in sel_b:
+            for l, want in enumerate(sel_b[rid]):
+                if want is not None and sel_a[rid][l] is not None:
+                    assert sel_a[rid][l] == want, (step, rid, l)
+                    compared += 1
+    assert compared > 0
+
+
 def test_kvcomp_batched_path_at_serving_size(ucm, dev):
     """Sixteen requests of 30 to 45 blocks of 128 tokens, 32 layers, Llama-3-8B head shape: the batched path and the
     per-request path leave the same bytes in every cache after six decode steps (two retrieval steps per request, the
