@@ -335,6 +335,9 @@ int ucm_prefetch_plan(const int32_t* map_block, const int32_t* map_len, int32_t*
  *                (colsum > 0; an exact tie gives 0), layer stride in BYTES
  *   workgroups   persistent workgroups launched over all layers, each of whose
  *                waves steps through the list of blocks; 0 = the default (4096)
+ * A block is encoded in tiles of 32 key vectors: block_size * kv_heads must be
+ * a multiple of 32 (UCM_ENOTSUP otherwise; 16-token blocks need two kv heads
+ * or more), kv_heads one of 1, 2, 4, 8 and block_size at most 16383.
  * ucm_hash_encode_queries: per (layer, request) the codes of all query heads
  * (q_codes u8 [L][n_req][q_heads][16]), their +-1 sum over heads (q_sum int16
  * [L][n_req][128]) and the code of every kv head's group-mean query
