@@ -1,7 +1,7 @@
 /*
  * Host twins of the C ABI: the same prototypes as libucm_hip.so's entry points
  * of the dense retrieval path, of the ESA retrieval worker, of the hash-code path, of the planned loads, of KVStar's
- * selection and of the prefetch bookkeeping, name + "_cpu", every "dev" pointer a host
+ * representatives, votes and selection and of the prefetch bookkeeping, name + "_cpu", every "dev" pointer a host
  * pointer, `stream` ignored, the work done before the call returns.  A caller
  * written against one prototype switches between host and device by choosing
  * the symbol.
@@ -44,6 +44,9 @@ TWIN(ucm_kv_load_planned);
 TWIN(ucm_kvstar_topk);
 TWIN(ucm_kvstar_order);
 TWIN(ucm_prefetch_plan);
+TWIN(ucm_kvstar_block_repre);
+TWIN(ucm_kvstar_votes);
+TWIN(ucm_kvstar_votes_tables);
 
 /* the oracle's functions these forward to (ucm_oracle.c) */
 float orc_bf16_to_f32(uint16_t h);
@@ -70,6 +73,12 @@ void orc_hash_scores_block(const uint8_t* q_codes, const uint8_t* block_codes, u
                            uint32_t nbytes, int32_t* scores);
 float orc_f16_to_f32(uint16_t h);
 int32_t orc_kvstar_topk(const float* final_scores, uint32_t n_blocks, uint32_t topk, int32_t* topk_idx);
+void orc_kvstar_block_repre(const uint16_t* cache, const int32_t* block_ids, const int32_t* slots, uint32_t n, uint32_t block_size,
+                            uint32_t kv_heads, uint32_t head_dim, uint32_t merge, const int32_t* pruned, uint32_t d_pruned,
+                            uint32_t d_pad, uint16_t* repre);
+int32_t orc_kvstar_retrieve(const uint16_t* q, uint32_t n_tokens, uint32_t q_heads, uint32_t d_orig, const uint16_t* repre,
+                            uint32_t n_blocks, uint32_t M, uint32_t kv_heads, uint32_t d_pruned, uint32_t d_pad,
+                            const int32_t* pruned, uint32_t topk, float* final_scores, int32_t* topk_idx);
 int32_t orc_prefetch_run(int32_t* map_block, int32_t* map_idx, int32_t n_map, const int32_t* topk, int32_t topk_len,
                          int32_t* free_block, int32_t* free_len, int32_t* success_blocks, int32_t success_cap,
                          int32_t* success_len, int32_t* load_blocks, int32_t* miss_idxs, int32_t* n_miss);
@@ -717,5 +726,140 @@ int ucm_prefetch_plan_cpu(const int32_t* map_block, const int32_t* map_len, int3
     }
     free(blocks);
     return rc;
+}
+
+/* ---- KVStar's representatives and votes ------------------------------------------------------------------------
+ * The device keeps a block's sub-block representatives as cells [d_pad/8][M][8] per (layer, kv head, row) - the
+ * order the score kernel streams; the oracle's functions use the reference's [row][M][kv head][d].  The twins move
+ * between the two around the oracle's arithmetic.  The votes are the oracle's scalar loop: the device's agree with
+ * them to rounding (other summation order on the matrix cores), not bit for bit. */
+
+int ucm_kvstar_block_repre_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
+                               const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, int merge,
+                               const int32_t* pruned, int64_t pruned_layer_stride, int d_pruned, int d_pad, void* repre_f16,
+                               int repre_rows, int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
+                               ucm_stream_t stream)
+{
+    (void)stream;
+    if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
+    if (n == 0 || n_layers == 0) { return UCM_OK; }
+    if (!k_layers || !repre_f16 || num_blocks <= 0 || repre_rows <= 0 || block_size <= 0 || kv_heads <= 0 || head_dim <= 0 ||
+        merge <= 0 || block_size % merge || d_pruned <= 0 || d_pruned > head_dim || d_pad < d_pruned || d_pad % 8 ||
+        (!pruned && d_pruned != head_dim) || (pruned_layer_stride != 0 && pruned_layer_stride < (int64_t)kv_heads * d_pruned) ||
+        (repre_layer_stride | repre_head_stride | repre_row_stride) % 8) {
+        return UCM_EINVAL;
+    }
+    const int M = block_size / merge;
+    uint16_t* tmp = (uint16_t*)malloc((size_t)M * kv_heads * d_pad * sizeof(uint16_t));
+    if (!tmp) { return UCM_ENOMEM; }
+    const int32_t zero = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        const int32_t* lists = pruned ? pruned + (int64_t)l * pruned_layer_stride : NULL;
+        for (int i = 0; i < n; ++i) {
+            const int32_t id = block_ids ? block_ids[i] : i, slot = slots ? slots[i] : i;
+            if (id < 0 || id >= num_blocks || slot < 0 || slot >= repre_rows) { continue; }
+            orc_kvstar_block_repre((const uint16_t*)k_layers[l], &id, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads,
+                                   (uint32_t)head_dim, (uint32_t)merge, lists, (uint32_t)d_pruned, (uint32_t)d_pad, tmp);
+            for (int h = 0; h < kv_heads; ++h) {
+                uint16_t* cell = (uint16_t*)repre_f16 + (int64_t)l * repre_layer_stride + (int64_t)h * repre_head_stride +
+                                 (int64_t)slot * repre_row_stride;
+                for (int m = 0; m < M; ++m) {
+                    for (int p = 0; p < d_pad; ++p) {
+                        cell[((size_t)(p / 8) * M + m) * 8 + p % 8] = tmp[((size_t)m * kv_heads + h) * d_pad + p];
+                    }
+                }
+            }
+        }
+    }
+    free(tmp);
+    return UCM_OK;
+}
+
+/* votes of one task whose block b has its cell of kv head h at table + h*head_stride + b*row_stride */
+static int kvstar_task_votes(const uint16_t* q, int n_tokens, int q_heads, int d_orig, const int32_t* lists, const uint16_t* table,
+                             int64_t head_stride, int64_t row_stride, int n_blocks, int M, int kv_heads, int d_pruned, int d_pad,
+                             float* votes)
+{
+    if (n_blocks <= 0) { return UCM_OK; }
+    uint16_t* ref = (uint16_t*)malloc((size_t)n_blocks * M * kv_heads * d_pad * sizeof(uint16_t));
+    if (!ref) { return UCM_ENOMEM; }
+    for (int b = 0; b < n_blocks; ++b) {
+        for (int h = 0; h < kv_heads; ++h) {
+            const uint16_t* cell = table + (int64_t)h * head_stride + (int64_t)b * row_stride;
+            for (int m = 0; m < M; ++m) {
+                for (int p = 0; p < d_pad; ++p) {
+                    ref[(((size_t)b * M + m) * kv_heads + h) * d_pad + p] = cell[((size_t)(p / 8) * M + m) * 8 + p % 8];
+                }
+            }
+        }
+    }
+    int32_t none;
+    orc_kvstar_retrieve(q, (uint32_t)n_tokens, (uint32_t)q_heads, (uint32_t)d_orig, ref, (uint32_t)n_blocks, (uint32_t)M,
+                        (uint32_t)kv_heads, (uint32_t)d_pruned, (uint32_t)d_pad, lists, 0, votes, &none);
+    free(ref);
+    return UCM_OK;
+}
+
+static int kvstar_votes_check(const void* q, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
+                              const int32_t* pruned_sel, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                              int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, const float* votes)
+{
+    if (n_tasks < 0 || max_blocks < 0) { return UCM_EINVAL; }
+    if (n_tasks == 0) { return UCM_OK; }
+    if (!q || !q_off || !seg_off || !seg_len || !votes || n_tokens <= 0 || q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads ||
+        d_orig <= 0 || d_pruned <= 0 || d_pruned > d_orig || d_pad < d_pruned || (pruned == NULL) != (pruned_sel == NULL) ||
+        (!pruned && d_pruned != d_orig) || sub_blocks <= 0) {
+        return UCM_EINVAL;
+    }
+    if (n_tokens * (q_heads / kv_heads) > 64 || kv_heads > 8 || d_pad % 16 || d_pad > 128 || sub_blocks > 128 ||
+        (sub_blocks & (sub_blocks - 1))) {
+        return UCM_ENOTSUP;
+    }
+    return 1;   /* go on */
+}
+
+int ucm_kvstar_votes_cpu(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
+                         const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, int64_t repre_row_stride,
+                         const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads,
+                         int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
+                         float* votes, int tiles_per_wave, ucm_stream_t stream)
+{
+    (void)ws_max; (void)ws_max_floats; (void)ws_part; (void)ws_part_floats; (void)tiles_per_wave; (void)stream;
+    const int rc = kvstar_votes_check(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, seg_off, seg_len, n_tasks,
+                                      max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, votes);
+    if (rc != 1) { return rc; }
+    if (!repre_f16) { return UCM_EINVAL; }
+    for (int t = 0; t < n_tasks; ++t) {
+        const int n = seg_len[t] < max_blocks ? seg_len[t] : max_blocks;
+        const int32_t* lists = (pruned && pruned_sel[t] >= 0) ? pruned + (size_t)pruned_sel[t] * kv_heads * d_pruned : NULL;
+        const int r = kvstar_task_votes((const uint16_t*)q_f16 + q_off[t], n_tokens, q_heads, d_orig, lists,
+                                        (const uint16_t*)repre_f16 + (int64_t)seg_off[t] * repre_row_stride, repre_head_stride,
+                                        repre_row_stride, n, sub_blocks, kv_heads, d_pruned, d_pad, votes + seg_off[t]);
+        if (r != UCM_OK) { return r; }
+    }
+    return UCM_OK;
+}
+
+int ucm_kvstar_votes_tables_cpu(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                                const int32_t* pruned, const int32_t* pruned_sel, const void* const* task_tables,
+                                const int64_t* task_head_strides, int64_t task_row_stride, const int32_t* seg_off,
+                                const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned,
+                                int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
+                                float* votes, int tiles_per_wave, ucm_stream_t stream)
+{
+    (void)ws_max; (void)ws_max_floats; (void)ws_part; (void)ws_part_floats; (void)tiles_per_wave; (void)stream;
+    const int rc = kvstar_votes_check(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, seg_off, seg_len, n_tasks,
+                                      max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, votes);
+    if (rc != 1) { return rc; }
+    if (!task_tables || !task_head_strides) { return UCM_EINVAL; }
+    for (int t = 0; t < n_tasks; ++t) {
+        const int n = seg_len[t] < max_blocks ? seg_len[t] : max_blocks;
+        const int32_t* lists = (pruned && pruned_sel[t] >= 0) ? pruned + (size_t)pruned_sel[t] * kv_heads * d_pruned : NULL;
+        const int r = kvstar_task_votes((const uint16_t*)q_f16 + q_off[t], n_tokens, q_heads, d_orig, lists,
+                                        (const uint16_t*)task_tables[t], task_head_strides[t], task_row_stride, n, sub_blocks,
+                                        kv_heads, d_pruned, d_pad, votes + seg_off[t]);
+        if (r != UCM_OK) { return r; }
+    }
+    return UCM_OK;
 }
 

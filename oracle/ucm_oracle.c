@@ -851,10 +851,8 @@ ORC_API int32_t orc_kvstar_topk(const float* final_scores, uint32_t n_blocks, ui
  *   score[x][H][s] = sum_d q[x][H][dp(d)] * k[s][h(H)][d]      fp32, d ascending, mul then add
  *   p = softmax over s of each (x, H) row                        max, expf, sum in s order, divide
  *   final[n] = sum over rows, then over the M sub-blocks of block n, of p     row-major order
- *   top-k of final: the min-heap of :953-975 replaces its smallest entry only
- *   by a strictly larger score, so of equal scores at the threshold the lower
- *   index stays; the AVX2 twin uses std::nth_element (unordered, ties
- *   unspecified).  Defined here: descending score, lower index first.
+ *   top-k of final: orc_kvstar_topk above, the literal heap of :955-977 (the
+ *   AVX2 twin uses std::nth_element: unordered, ties unspecified).
  *   q      fp16 [x][H][d_orig]; pruned as above (the query is gathered by it)
  *   repre  fp16 [n_blocks][M][kv_heads][d_pad] (d_pad >= d_pruned, pad ignored)
  *   final  fp32 [n_blocks] out; topk_idx int32 [min(topk, n_blocks)] out; returns the count

@@ -13,7 +13,8 @@ import synth
 TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
-         "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan"]
+         "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
+         "ucm_kvstar_votes", "ucm_kvstar_votes_tables"]
 
 
 def twin_caller(signatures):
@@ -364,6 +365,70 @@ def run_more(call, side):
          P_ROWS * P_CAP, side.ptr(load_count), side.ptr(rows), 4, P_ROWS, None)
     for l in range(P_L):
         out[f"cache{l}"] = caches[l]
+    side.sync()
+    return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
+
+
+# ---- KVStar's representatives and votes ------------------------------------------------------------------------
+K_L, K_NB, K_BS, K_HKV, K_D, K_MERGE, K_ROWS, K_G, K_X = 2, 10, 16, 2, 64, 4, 8, 2, 2
+K_M, K_DP, K_DPAD = K_BS // K_MERGE, 20, 32
+K_OFF, K_LEN = np.array([0, 3, 3], np.int32), np.array([3, 0, 5], np.int32)
+
+
+def kvstar_inputs():
+    rng = np.random.default_rng(7400)
+    caches = [synth.normal_bf16_bits(7400 + l, (K_NB, K_BS, K_HKV, K_D)) for l in range(K_L)]
+    ids = np.array([7, 2, 9, -1, 0, 4, 5, K_NB, 1, 3], np.int32)      # two ids the call must skip
+    slots = np.array([0, 1, 2, 3, 3, 4, 5, 6, 6, 7], np.int32)
+    lists = np.stack([np.stack([np.sort(rng.permutation(K_D)[:K_DP]) for _ in range(K_HKV)]) for _ in range(K_L)]).astype(np.int32)
+    q = (rng.standard_normal((3, K_X, K_HKV * K_G, K_D)) * 0.5).astype(np.float16).view(np.uint16)
+    return dict(caches=caches, ids=ids, slots=slots, lists=lists, q=q)
+
+
+def run_kvstar(call, side):
+    """Sub-block representatives with and without channel pruning into tables of head planes, then the votes of
+    three tasks (one empty) over layer 0's pruned table, once as rows of the shared table and once as tables of
+    their own."""
+    import ctypes as C
+
+    from ucm_amd import _lib
+
+    x = kvstar_inputs()
+    out = {}
+    caches = [side.up(c) for c in x["caches"]]
+    k_layers = side.pointers(caches)
+    ids, slots, lists = side.up(x["ids"]), side.up(x["slots"]), side.up(x["lists"])
+    tables = {}
+    for name, pr, dp, d_pad in (("full", None, K_D, K_D), ("pruned", lists, K_DP, K_DPAD)):
+        cell = d_pad * K_M
+        t = side.up(np.full((K_L, K_HKV, K_ROWS, cell), 0x3c00, np.uint16))            # fp16 ones where nothing is written
+        call("ucm_kvstar_block_repre", k_layers, K_L, K_NB, side.ptr(ids), side.ptr(slots), len(x["ids"]), K_BS, K_HKV, K_D,
+             K_MERGE, None if pr is None else side.ptr(pr), 0 if pr is None else K_HKV * K_DP, dp, d_pad, side.ptr(t), K_ROWS,
+             K_HKV * K_ROWS * cell, K_ROWS * cell, cell, None)
+        tables[name] = t
+        out["table_" + name] = t
+    side.sync()
+    # votes over layer 0 of the pruned table
+    cell = K_DPAD * K_M
+    q, seg_off, seg_len = side.up(x["q"]), side.up(K_OFF), side.up(K_LEN)
+    q_off = side.up((np.arange(3) * K_X * K_HKV * K_G * K_D).astype(np.int64))
+    sel = side.up(np.zeros(3, np.int32))
+    mf, pf = C.c_int64(), C.c_int64()
+    _lib.call("ucm_kvstar_workspace_floats", 3, K_HKV, K_X * K_G, 5, K_M, K_DPAD, 0, C.byref(mf), C.byref(pf))
+    ws_max, ws_part = side.up(np.zeros(max(mf.value, 1), np.float32)), side.up(np.zeros(max(pf.value, 1), np.float32))
+    votes = side.up(np.full(K_ROWS, -3, np.float32))
+    call("ucm_kvstar_votes", side.ptr(q), side.ptr(q_off), K_X, K_HKV * K_G, K_D, side.ptr(lists), side.ptr(sel),
+         side.ptr(tables["pruned"]), K_ROWS * cell, cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M, K_HKV, K_DP, K_DPAD,
+         side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes), 0, None)
+    out["votes"] = votes
+    base = side.ptr(tables["pruned"])
+    task_tables = side.up(np.array([base + int(a) * cell * 2 for a in K_OFF], np.int64))
+    head_strides = side.up(np.full(3, K_ROWS * cell, np.int64))
+    votes_t = side.up(np.full(K_ROWS, -3, np.float32))
+    call("ucm_kvstar_votes_tables", side.ptr(q), side.ptr(q_off), K_X, K_HKV * K_G, K_D, side.ptr(lists), side.ptr(sel),
+         side.ptr(task_tables), side.ptr(head_strides), cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M, K_HKV, K_DP,
+         K_DPAD, side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes_t), 0, None)
+    out["votes_tables"] = votes_t
     side.sync()
     return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
 

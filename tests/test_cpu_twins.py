@@ -150,3 +150,31 @@ def test_selection_prefetch_and_load_twins_reproduce_the_oracle(ucm):
         assert np.array_equal(got[f"cache{l}"], want_cache[l])
     assert any(c.any() for c in want_cache)
 
+
+def test_kvstar_twins_reproduce_the_oracle(ucm):
+    from ucm_amd import _lib
+
+    got, x = cpu_twins.run_kvstar(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    K = cpu_twins
+    live = [(int(b), int(s)) for b, s in zip(x["ids"], x["slots"]) if 0 <= b < K.K_NB]
+    final = dict((s, b) for b, s in live)                              # a slot named twice keeps the later block
+    for name, d_pad in (("full", K.K_D), ("pruned", K.K_DPAD)):
+        # cells [d_pad/8][M][8] of (layer, head, row) back into the reference's [row][M][head][d]
+        cells = got["table_" + name].reshape(K.K_L, K.K_HKV, K.K_ROWS, d_pad // 8, K.K_M, 8)
+        ref = cells.transpose(0, 2, 4, 1, 3, 5).reshape(K.K_L, K.K_ROWS, K.K_M, K.K_HKV, d_pad)
+        for l in range(K.K_L):
+            want = np.full((K.K_ROWS, K.K_M, K.K_HKV, d_pad), 0x3c00, np.uint16)
+            O.kvstar_block_repre(x["caches"][l], np.array(list(final.values()), np.int32), np.array(list(final.keys()), np.int32),
+                                 K.K_MERGE, want, pruned=None if name == "full" else x["lists"][l])
+            assert np.array_equal(ref[l], want), (name, l)
+            if name == "pruned":
+                assert (ref[l][..., K.K_DP:] == 0).all() and (ref[l][..., : K.K_DP] != 0).any()
+    assert set(final) == set(range(K.K_ROWS))
+    for key in ("votes", "votes_tables"):
+        for t, (a, n) in enumerate(zip(K.K_OFF, K.K_LEN)):
+            if n:
+                _, want = O.kvstar_retrieve(x["q"][t], np.ascontiguousarray(ref[0][a : a + n]), 1, pruned=x["lists"][0])
+                assert np.array_equal(got[key][a : a + n].view(np.uint32), want.view(np.uint32)), (key, t)
+                assert abs(float(want.sum()) - K.K_X * K.K_HKV * K.K_G) < 1e-3          # every query row votes with weight one
+    assert np.array_equal(got["votes"], got["votes_tables"])
+

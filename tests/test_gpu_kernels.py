@@ -842,3 +842,10 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
         for name in want:
             assert got[name].dtype == want[name].dtype and got[name].shape == want[name].shape, name
             assert np.array_equal(got[name].view(np.uint8), want[name].view(np.uint8)), name
+    # KVStar: the tables bit for bit; the votes to rounding (the matrix cores sum in another order than the scalar loop)
+    want, _ = cpu_twins.run_kvstar(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    got, _ = cpu_twins.run_kvstar(_lib.call, cpu_twins.DeviceSide(ops, dev))
+    for name in ("table_full", "table_pruned"):
+        assert np.array_equal(got[name], want[name]), name
+    for name in ("votes", "votes_tables"):
+        assert np.allclose(got[name], want[name], rtol=2e-4, atol=2e-6), name
