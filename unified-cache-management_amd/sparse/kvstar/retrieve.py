@@ -88,6 +88,7 @@ _tasks: Dict[int, _Task] = {}
 _ids = itertools.count(1)
 _lock = threading.Lock()
 _stream: Optional[torch.cuda.Stream] = None
+_layer_pointers: Dict[int, "ops.LayerPointers"] = {}     # one pointer table per key cache seen by extract_block_repre
 
 
 def Setup(param: SetupParam) -> None:  # noqa: N802 (reference name)
@@ -310,7 +311,7 @@ def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge:
     over these blocks are kept per head (the reference's choice, :284-292); otherwise a given index is reused."""
     n_total, block_size, kv_heads, head_dim = k_cache.shape
     dev = k_cache.device
-    ids = torch.tensor(vllm_block_ids, dtype=torch.int32, device=dev)
+    ids = ops.upload(torch.tensor(vllm_block_ids, dtype=torch.int32), dev)
     if prune_dim_enable and prune_ratio < 0.98:
         absmean = k_cache[ids.long()].reshape(-1, kv_heads, head_dim).to(torch.float32).abs().mean(dim=0)
         _, d_pruned_index = torch.topk(absmean, k=round(head_dim * prune_ratio), dim=-1)
@@ -319,6 +320,11 @@ def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge:
     d_pad = (d_pruned + 15) // 16 * 16
     table = ops.kvstar_table(1, kv_heads, len(vllm_block_ids), block_size // merge, d_pad, dev)
     pruned32 = None if d_pruned_index is None else d_pruned_index.to(torch.int32).contiguous()
-    ops.kvstar_block_repre(ops.LayerPointers([k_cache]), ids, torch.arange(len(vllm_block_ids), dtype=torch.int32, device=dev),
+    known = _layer_pointers.get(k_cache.data_ptr())
+    if known is None or known.tensors[0].shape != k_cache.shape:
+        if len(_layer_pointers) > 256:                   # caches come and go with engines; the table stays small
+            _layer_pointers.clear()
+        known = _layer_pointers[k_cache.data_ptr()] = ops.LayerPointers([k_cache])
+    ops.kvstar_block_repre(known, ids, torch.arange(len(vllm_block_ids), dtype=torch.int32, device=dev),
                            table, block_size, kv_heads, head_dim, n_total, merge, pruned=pruned32)
     return BlockRepre(table[0], d_pruned), d_pruned_index
