@@ -52,6 +52,9 @@ extern "C" {
 #define UCM_MEAN_F32 0       /* fp32 mean kept as is (the C++ KRepreComputer contract) */
 #define UCM_MEAN_BF16_ROUND 1 /* mean rounded to bf16 and widened (what the live torch path stores) */
 #define UCM_MEAN_BF16_STORE 2 /* the same rounded mean kept as bf16: `repre` is a bf16 table */
+#define UCM_MEAN_ABS 4        /* or-ed to one of the above: the mean of the ABSOLUTE values, token order as before
+                               (the per-channel |k| statistic KVStar picks its channels by,
+                               ucm/sparse/kvstar/multistep.py:284-292, one block at a time) */
 
 typedef void* ucm_stream_t; /* hipStream_t */
 

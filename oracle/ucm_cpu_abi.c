@@ -92,18 +92,28 @@ int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks
     if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
     if (n == 0 || n_layers == 0) { return UCM_OK; }
     if (!k_layers || !block_ids || !slots || !repre || num_blocks <= 0 || repre_rows <= 0 || block_size <= 0 ||
-        kv_heads <= 0 || head_dim <= 0 || mode < UCM_MEAN_F32 || mode > UCM_MEAN_BF16_STORE) {
+        kv_heads <= 0 || head_dim <= 0 || (mode & ~UCM_MEAN_ABS) < UCM_MEAN_F32 || (mode & ~UCM_MEAN_ABS) > UCM_MEAN_BF16_STORE) {
         return UCM_EINVAL;
     }
+    const int of_abs = (mode & UCM_MEAN_ABS) != 0;
+    mode &= ~UCM_MEAN_ABS;
     const size_t row = (size_t)kv_heads * head_dim;
     float* tmp = (float*)malloc(row * sizeof(float));
-    if (!tmp) { return UCM_ENOMEM; }
+    uint16_t* blk = of_abs ? (uint16_t*)malloc((size_t)block_size * row * sizeof(uint16_t)) : NULL;   /* the block without its signs */
+    if (!tmp || (of_abs && !blk)) { free(tmp); free(blk); return UCM_ENOMEM; }
     const int32_t zero = 0;
     for (int l = 0; l < n_layers; ++l) {
         for (int i = 0; i < n; ++i) {
             if (block_ids[i] < 0 || block_ids[i] >= num_blocks || slots[i] < 0 || slots[i] >= repre_rows) { continue; }
-            orc_block_mean_paged((const uint16_t*)k_layers[l], &block_ids[i], &zero, 1, (uint32_t)block_size,
-                                 (uint32_t)kv_heads, (uint32_t)head_dim, tmp, mode != UCM_MEAN_F32);
+            if (of_abs) {
+                const uint16_t* src = (const uint16_t*)k_layers[l] + (size_t)block_ids[i] * block_size * row;
+                for (size_t e = 0; e < (size_t)block_size * row; ++e) { blk[e] = src[e] & 0x7fffu; }
+                orc_block_mean_paged(blk, &zero, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads, (uint32_t)head_dim, tmp,
+                                     mode != UCM_MEAN_F32);
+            } else {
+                orc_block_mean_paged((const uint16_t*)k_layers[l], &block_ids[i], &zero, 1, (uint32_t)block_size,
+                                     (uint32_t)kv_heads, (uint32_t)head_dim, tmp, mode != UCM_MEAN_F32);
+            }
             const size_t at = (size_t)l * (size_t)repre_layer_stride + (size_t)slots[i] * row;
             if (mode == UCM_MEAN_BF16_STORE) {
                 for (size_t c = 0; c < row; ++c) { ((uint16_t*)repre)[at + c] = orc_f32_to_bf16(tmp[c]); }
@@ -113,6 +123,7 @@ int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks
         }
     }
     free(tmp);
+    free(blk);
     return UCM_OK;
 }
 

@@ -112,7 +112,7 @@ def run(call, side):
     n = len(x["ids"])
     # 1. representatives in the three modes
     tabs = {}
-    for mode, dtype in ((0, np.float32), (1, np.float32), (2, np.uint16)):
+    for mode, dtype in ((0, np.float32), (1, np.float32), (2, np.uint16), (4, np.float32)):      # 4: of the absolute values
         t = side.up(np.full((L, ROWS, ROW), 7, dtype))
         call("ucm_block_mean", k_planes, L, NB, side.ptr(ids), side.ptr(slots), n, BS, HKV, D, side.ptr(t), ROWS, ROWS * ROW,
              mode, None)

@@ -20,6 +20,9 @@ def test_twins_reproduce_the_oracle(ucm):
             O.block_mean_paged(x["caches"][l][0], ids, slots, want, round_bf16=rounded)
             assert np.array_equal(got[f"repre{mode}"][l].view(np.uint32), want.view(np.uint32))
         assert np.array_equal(got["repre2"][l], O.bf16_bits(got["repre1"][l]))
+        want = np.full((ROWS, ROW), 7, np.float32)
+        O.block_mean_paged(x["caches"][l][0] & np.uint16(0x7fff), ids, slots, want)
+        assert np.array_equal(got["repre4"][l].view(np.uint32), want.view(np.uint32))
     # scores and selection, per request, against the oracle's batch call
     table16 = O.bf16_to_f32(got["repre2"])
     for l in range(L):

@@ -56,6 +56,20 @@ def test_block_mean_matches_oracle(ucm, dev, hkv, d, bs, n_layers):
     t = caches[0][torch.from_numpy(ids.astype(np.int64)).to(dev)].mean(1).float().reshape(len(ids), row)
     mine = repre[0][torch.from_numpy(slots.astype(np.int64)).to(dev)]
     assert torch.allclose(mine, t, rtol=2 ** -7, atol=1e-6)
+    # MEAN_ABS: the same sums over the keys without their signs (the oracle on a cache whose sign bits are cleared)
+    for mode in (ops.MEAN_F32, ops.MEAN_BF16_ROUND):
+        repre = torch.full((n_layers, rows, row), 7.0, device=dev)
+        ops.block_mean(lp, i32(ids, dev), i32(slots, dev), repre, bs, hkv, d, nb, mode=mode | ops.MEAN_ABS)
+        got = repre.cpu().numpy()
+        for l in range(n_layers):
+            want = np.full((rows, row), 7.0, np.float32)
+            O.block_mean_paged(caches_h[l] & np.uint16(0x7fff), ids, slots, want, round_bf16=(mode == ops.MEAN_BF16_ROUND))
+            assert np.array_equal(bits(got[l]), bits(want)), (mode, l)
+            assert (got[l][slots] >= 0).all()
+    both = torch.zeros((n_layers, rows, row), dtype=torch.bfloat16, device=dev)
+    ops.block_mean(lp, i32(ids, dev), i32(slots, dev), both, bs, hkv, d, nb, mode=ops.MEAN_ABS)   # a bf16 table of |k| means
+    assert torch.equal(both[:, torch.from_numpy(slots.astype(np.int64)).to(dev)].float(),
+                       repre[:, torch.from_numpy(slots.astype(np.int64)).to(dev)])
 
 
 def test_block_mean_skips_bad_ids_and_layer_range(ucm, dev):

@@ -29,8 +29,11 @@ __device__ __forceinline__ float round_bf16(float x)
     return __uint_as_float(u & 0xffff0000u);
 }
 
-__device__ __forceinline__ void widen(const u32x4 v, float (&f)[kCols])
+// kAbs: the absolute values (a bf16 pair loses its two sign bits with one AND)
+template <bool kAbs>
+__device__ __forceinline__ void widen(u32x4 v, float (&f)[kCols])
 {
+    if (kAbs) { v.x &= 0x7fff7fffu; v.y &= 0x7fff7fffu; v.z &= 0x7fff7fffu; v.w &= 0x7fff7fffu; }
     f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x);
     f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
     f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z);
@@ -38,7 +41,7 @@ __device__ __forceinline__ void widen(const u32x4 v, float (&f)[kCols])
 }
 
 // acc += token rows t .. t+kN-1, in that order, all kN loads issued before the first add
-template <int kN>
+template <int kN, bool kAbs>
 __device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsigned row, unsigned t, float (&acc)[kCols])
 {
     u32x4 v[kN];
@@ -47,7 +50,7 @@ __device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsi
 #pragma unroll
     for (int u = 0; u < kN; ++u) {
         float f[kCols];
-        widen(v[u], f);
+        widen<kAbs>(v[u], f);
 #pragma unroll
         for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
     }
@@ -56,6 +59,7 @@ __device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsi
 // grid: x = block index in the list * col_groups + column group of 1024, y = layer; rows narrower than 1024
 // columns whose thread count divides the workgroup (a tensor-parallel rank's 4, 2 or 1 kv heads of 128) share a
 // workgroup, items_per_group list entries side by side, so that no lane idles
+template <bool kAbs>
 __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned repre_rows, unsigned block_size,
@@ -80,16 +84,16 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     const uint16_t* base = static_cast<const uint16_t*>(k_layers[blockIdx.y]) +
                            static_cast<size_t>(id) * block_size * row + col;
     float acc[kCols];
-    widen(ucm::gload16(base), acc);  // acc = token 0
+    widen<kAbs>(ucm::gload16(base), acc);  // acc = token 0
 
     unsigned t = 1;
     // full groups of kUnroll tokens: loads first, then the ordered adds; what is left (all of a 16-token block
     // after its first token) goes in groups of 8, 4, 2 and 1, each with its loads issued together
-    for (; t + kUnroll <= block_size; t += kUnroll) { add_rows<kUnroll>(base, row, t, acc); }
-    if (t + 8 <= block_size) { add_rows<8>(base, row, t, acc); t += 8; }
-    if (t + 4 <= block_size) { add_rows<4>(base, row, t, acc); t += 4; }
-    if (t + 2 <= block_size) { add_rows<2>(base, row, t, acc); t += 2; }
-    if (t < block_size) { add_rows<1>(base, row, t, acc); }
+    for (; t + kUnroll <= block_size; t += kUnroll) { add_rows<kUnroll, kAbs>(base, row, t, acc); }
+    if (t + 8 <= block_size) { add_rows<8, kAbs>(base, row, t, acc); t += 8; }
+    if (t + 4 <= block_size) { add_rows<4, kAbs>(base, row, t, acc); t += 4; }
+    if (t + 2 <= block_size) { add_rows<2, kAbs>(base, row, t, acc); t += 2; }
+    if (t < block_size) { add_rows<1, kAbs>(base, row, t, acc); }
 
     const float inv = 1.0f / static_cast<float>(block_size);
 #pragma unroll
@@ -130,6 +134,8 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535, "ucm_block_mean: n_layers=%d", n_layers);
     UCM_REQUIRE(block_size > 0 && kv_heads > 0 && head_dim > 0 && num_blocks > 0 && repre_rows > 0,
                 "ucm_block_mean: non-positive shape");
+    const bool of_abs = (mode & UCM_MEAN_ABS) != 0;
+    mode &= ~UCM_MEAN_ABS;
     UCM_REQUIRE(mode == UCM_MEAN_F32 || mode == UCM_MEAN_BF16_ROUND || mode == UCM_MEAN_BF16_STORE,
                 "ucm_block_mean: mode=%d", mode);
     const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
@@ -144,9 +150,11 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
     const unsigned per_item = row / kCols;               // threads a list entry needs
     const unsigned share = (per_item < kThreads && kThreads % per_item == 0) ? kThreads / per_item : 1u;
     const unsigned groups = share > 1 ? (static_cast<unsigned>(n) + share - 1) / share : static_cast<unsigned>(n) * gx;
-    hipLaunchKernelGGL(block_mean_kernel, dim3(groups, n_layers), dim3(kThreads), 0, ucm::as_stream(stream),
-                       k_layers, block_ids, slots, static_cast<unsigned>(num_blocks),
-                       static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row,
-                       static_cast<float*>(repre), repre_layer_stride, mode, gx, share, static_cast<unsigned>(n));
+#define UCM_BLOCK_MEAN_ARGS dim3(groups, n_layers), dim3(kThreads), 0, ucm::as_stream(stream), k_layers, block_ids, slots, \
+        static_cast<unsigned>(num_blocks), static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row,       \
+        static_cast<float*>(repre), repre_layer_stride, mode, gx, share, static_cast<unsigned>(n)
+    if (of_abs) { hipLaunchKernelGGL(block_mean_kernel<true>, UCM_BLOCK_MEAN_ARGS); }
+    else { hipLaunchKernelGGL(block_mean_kernel<false>, UCM_BLOCK_MEAN_ARGS); }
+#undef UCM_BLOCK_MEAN_ARGS
     UCM_LAUNCH_CHECK("ucm_block_mean");
 }

@@ -12,7 +12,7 @@ from typing import Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import MEAN_BF16_ROUND, MEAN_BF16_STORE, MEAN_F32, UcmHipError  # noqa: F401
+from ._lib import MEAN_ABS, MEAN_BF16_ROUND, MEAN_BF16_STORE, MEAN_F32, UcmHipError  # noqa: F401
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -119,7 +119,8 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
                first_layer: int = 0, n_layers: Optional[int] = None) -> None:
     """repre: [L, rows, kv_heads*head_dim], fp32 (mode MEAN_F32 / MEAN_BF16_ROUND) or
     bf16 (the mode is then MEAN_BF16_STORE whatever was passed); rows ``slots`` of layers
-    first_layer.. are overwritten with the means of cache blocks ``block_ids``."""
+    first_layer.. are overwritten with the means of cache blocks ``block_ids`` (``mode | MEAN_ABS``: of their
+    absolute values)."""
     if repre.dim() != 3 or repre.shape[2] != kv_heads * head_dim:
         raise ValueError("repre must be [layers, rows, kv_heads*head_dim]")
     n_layers = len(k_layers) - first_layer if n_layers is None else n_layers
@@ -129,10 +130,13 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
         raise ValueError("block_ids and slots differ in length")
     if repre.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("repre must be float32 or bfloat16")
+    of_abs = mode & MEAN_ABS
+    mode &= ~MEAN_ABS
     if repre.dtype == torch.bfloat16:
         mode = MEAN_BF16_STORE
     elif mode == MEAN_BF16_STORE:
         raise ValueError("MEAN_BF16_STORE needs a bfloat16 table")
+    mode |= of_abs
     rp = _dev(repre, repre.dtype, "repre") + first_layer * repre.stride(0) * repre.element_size()
     _lib.call("ucm_block_mean", k_layers.ptr(first_layer), n_layers, num_blocks,
               _dev(block_ids, torch.int32, "block_ids"), _dev(slots, torch.int32, "slots"), block_ids.numel(),

@@ -311,20 +311,25 @@ def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge:
     over these blocks are kept per head (the reference's choice, :284-292); otherwise a given index is reused."""
     n_total, block_size, kv_heads, head_dim = k_cache.shape
     dev = k_cache.device
+    n = len(vllm_block_ids)
     ids = ops.upload(torch.tensor(vllm_block_ids, dtype=torch.int32), dev)
-    if prune_dim_enable and prune_ratio < 0.98:
-        absmean = k_cache[ids.long()].reshape(-1, kv_heads, head_dim).to(torch.float32).abs().mean(dim=0)
-        _, d_pruned_index = torch.topk(absmean, k=round(head_dim * prune_ratio), dim=-1)
-        d_pruned_index = d_pruned_index.contiguous()
-    d_pruned = head_dim if d_pruned_index is None else d_pruned_index.shape[1]
-    d_pad = (d_pruned + 15) // 16 * 16
-    table = ops.kvstar_table(1, kv_heads, len(vllm_block_ids), block_size // merge, d_pad, dev)
-    pruned32 = None if d_pruned_index is None else d_pruned_index.to(torch.int32).contiguous()
+    rows = torch.arange(n, dtype=torch.int32, device=dev)
     known = _layer_pointers.get(k_cache.data_ptr())
     if known is None or known.tensors[0].shape != k_cache.shape:
         if len(_layer_pointers) > 256:                   # caches come and go with engines; the table stays small
             _layer_pointers.clear()
         known = _layer_pointers[k_cache.data_ptr()] = ops.LayerPointers([k_cache])
-    ops.kvstar_block_repre(known, ids, torch.arange(len(vllm_block_ids), dtype=torch.int32, device=dev),
-                           table, block_size, kv_heads, head_dim, n_total, merge, pruned=pruned32)
+    if prune_dim_enable and prune_ratio < 0.98:
+        # mean |k| per (head, channel) over all tokens of these blocks: the blocks' own means of |k|, read from the
+        # paged cache in one pass, averaged (the reference gathers the blocks and takes one mean, :284-290)
+        per_block = torch.empty((1, n, kv_heads * head_dim), dtype=torch.float32, device=dev)
+        ops.block_mean(known, ids, rows, per_block, block_size, kv_heads, head_dim, n_total, mode=ops.MEAN_F32 | ops.MEAN_ABS)
+        absmean = per_block[0].mean(dim=0).view(kv_heads, head_dim)
+        _, d_pruned_index = torch.topk(absmean, k=round(head_dim * prune_ratio), dim=-1)
+        d_pruned_index = d_pruned_index.contiguous()
+    d_pruned = head_dim if d_pruned_index is None else d_pruned_index.shape[1]
+    d_pad = (d_pruned + 15) // 16 * 16
+    table = ops.kvstar_table(1, kv_heads, n, block_size // merge, d_pad, dev)
+    pruned32 = None if d_pruned_index is None else d_pruned_index.to(torch.int32).contiguous()
+    ops.kvstar_block_repre(known, ids, rows, table, block_size, kv_heads, head_dim, n_total, merge, pruned=pruned32)
     return BlockRepre(table[0], d_pruned), d_pruned_index
