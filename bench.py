@@ -65,6 +65,9 @@ def parse():
     ap.add_argument("--delta-rho", type=float, default=0.95,
                     help="correlation of consecutive decode queries in the delta-gather leg (0 = independent)")
     ap.add_argument("--no-delta", action="store_true", help="skip the delta-gather leg")
+    ap.add_argument("--two-launch", action="store_true",
+                    help="score and select as two launches (ucm_score_blocks, ucm_topk_windows) instead of the one-launch "
+                         "ucm_score_select")
     ap.add_argument("--repre-dtype", choices=["bf16", "f32"], default="bf16",
                     help="element type of the representative table: bf16 = the rounded means the live reference "
                          "path stores, kept as they are; f32 = the same values widened (the CPU path's table)")
@@ -184,13 +187,22 @@ def main():
     staging = torch.empty(total_blocks * BLOCK_BYTES, dtype=torch.uint8, device=dev)
     kv_stride = nb * BLOCK_BYTES
 
+    tickets = torch.zeros_like(cnt)
+
     def step(q, events=None):
         if events:
             events[0].record()
-        ops.score_blocks(q, repre, seg_off, seg_len, max_len, HKV, scores, total_blocks=rows)
-        if events:
-            events[1].record()
-        ops.topk_windows(scores, seg_off, seg_len, topk_d, max_len, idx, cnt, block_tables=bt, phys_out=phys)
+        if args.two_launch:
+            ops.score_blocks(q, repre, seg_off, seg_len, max_len, HKV, scores, total_blocks=rows)
+            if events:
+                events[1].record()
+            ops.topk_windows(scores, seg_off, seg_len, topk_d, max_len, idx, cnt, block_tables=bt, phys_out=phys)
+        else:
+            # one launch: the last scoring workgroup of a (layer, request) runs its selection
+            ops.score_select(q, repre, seg_off, seg_len, topk_d, max_len, HKV, scores, idx, cnt, tickets, block_tables=bt,
+                             phys_out=phys)
+            if events:
+                events[1].record()
         if events:
             events[2].record()
         ops.kv_gather_selected(layers, kv_stride, BLOCK_BYTES, nb, phys, cnt, dst_off, region, max_k, staging,

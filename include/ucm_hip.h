@@ -47,6 +47,7 @@ extern "C" {
 
 #define UCM_DTYPE_F32 0
 #define UCM_DTYPE_BF16 1
+#define UCM_DTYPE_F16 2
 
 /* ucm_block_mean modes */
 #define UCM_MEAN_F32 0       /* fp32 mean kept as is (the C++ KRepreComputer contract) */
@@ -91,14 +92,14 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
 /*
  * Scores of every block of a ragged batch, all layers in one launch:
  *   qbar[h]  = (q[h*g] + q[h*g+1] + ... + q[h*g+g-1]) * (1/g),  g = q_heads/kv_heads
- *   score[b] = sum over kv heads h, in order, of dot(qbar[h], repre[b][h])
+ *   score[b] = sum over kv heads h, in order, of max over r < num_repre of dot(qbar[h], repre[b][h][r])
  * with dot() in the 16-lane FMA + pairwise fold order of the reference's
  * AVX-512 build, so the fp32 results equal TopkBlockSelector::ComputeQHeadMean
  * + ComputeKQDotScores bit for bit
  * (ucm/sparse/gsa/offload_ops/src/select_topk_block.cpp:53-114,
- * src/vec_product.cpp:16-37; one representative per head, numKrepre = 1, as
- * ucm/sparse/gsa/gsa.py:501 configures it).
- *   q          dev: queries, q_dtype fp32 or bf16, [n_layers][*][q_heads][head_dim];
+ * src/vec_product.cpp:16-37; the reference configures one representative per
+ * head, numKrepre = 1, ucm/sparse/gsa/gsa.py:501).
+ *   q          dev: queries, q_dtype fp32, bf16 or fp16, [n_layers][*][q_heads][head_dim];
  *              layer l starts q_layer_stride ELEMENTS after layer l-1; request
  *              r reads row q_rows[r] (q_rows == NULL: row r); with q_rows,
  *              q_layer_stride is also the bound of a layer's rows: a request
@@ -106,16 +107,21 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *              they were (ucm_hash_encode_queries does the same).  This is the
  *              reference's gsa_q_cache (gsa.py:503-512) when fp32, or the
  *              layer's raw query tensor with q_rows = index of each request's
- *              last token (GSA.copy_q, gsa.py:616-632) when bf16.
- *   repre      dev: representative table, repre_dtype fp32 or bf16 (what
- *              ucm_block_mean wrote), layer stride in ELEMENTS.  A bf16 table
- *              is widened exactly, so it scores like the fp32 table holding
- *              the same bf16-rounded means, at half the bytes streamed.
+ *              last token (GSA.copy_q, gsa.py:616-632) in the model dtype.
+ *   repre      dev: representative table [n_layers][repre_rows][kv_heads][num_repre][head_dim],
+ *              repre_dtype fp32 or bf16 (what ucm_block_mean wrote), layer
+ *              stride in ELEMENTS.  A bf16 table is widened exactly, so it
+ *              scores like the fp32 table holding the same bf16-rounded means,
+ *              at half the bytes streamed.
  *   seg_off, seg_len  dev int32[n_req]: first representative row and number of
  *              blocks of each request; max_seg_len >= every seg_len (host
- *              value, sizes the grid); total_blocks = sum of seg_len when the
- *              host knows it (a tighter grid), else 0.
- *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x].
+ *              value, sizes the grid; a longer seg_len is cut there);
+ *              total_blocks = sum of seg_len when the host knows it (a tighter
+ *              grid), else 0.  These descriptors live in device memory, where
+ *              the host cannot check them: a request whose rows do not lie
+ *              inside [0, repre_rows) is skipped, its scores left as they were.
+ *   scores     dev fp32: score of row x of layer l at scores[l*scores_layer_stride + x];
+ *              a layer holds at least repre_rows scores.
  *   scale      every score is multiplied by it on the way out; 1 leaves the bits
  *              above.  1/kv_heads gives the values of the reference's torch
  *              variant, the mean over all q heads of TopkCal.cal_topk
@@ -124,14 +130,15 @@ int ucm_block_mean(const void* const* k_layers, int n_layers, int num_blocks,
  *   tile_blocks  blocks scored per workgroup; 0 sizes a workgroup's share to 128 KiB
  *              of representatives (a value for benchmarks and tests, not part of
  *              the reference interface).
- * head_dim must be 32, 64, 96, 128, 192 or 256, kv_heads one of 1, 2, 4, 8, 16 and
- * kv_heads*head_dim at most 2048.
+ * head_dim must be 32, 64, 96, 128, 192 or 256, kv_heads*num_repre one of 1, 2,
+ * 4, 8, 16 and kv_heads*num_repre*head_dim at most 2048.
  */
 int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
                      int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
-                     const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
-                     int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
-                     int64_t scores_layer_stride, float scale, int tile_blocks, ucm_stream_t stream);
+                     int64_t repre_rows, int num_repre, const int32_t* seg_off, const int32_t* seg_len,
+                     int n_req, int max_seg_len, int64_t total_blocks, int n_layers, int kv_heads,
+                     int head_dim, float* scores, int64_t scores_layer_stride, float scale,
+                     int tile_blocks, ucm_stream_t stream);
 
 /*
  * Per-request block selection with forced windows, all layers in one launch -
@@ -141,6 +148,8 @@ int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const i
  * the k-start_w-end_w best of the rest by score (equal scores: lower index
  * first, as std::stable_sort leaves them) and the last end_w blocks, sorted
  * ascending.  k = topk_len[r] is the total (ucm/sparse/utils.py:30-36).
+ *   scores_rows  scores a layer holds: a request whose seg_off .. seg_off+seg_len
+ *              does not lie inside [0, scores_rows) selects nothing (count 0)
  *   idx_out    dev int32: entry j of request r in layer l at
  *              idx_out[(l*n_req + r)*out_stride + j]; out_stride must hold
  *              max(k, n) of every request.
@@ -157,12 +166,83 @@ int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const i
  *              non-sparsified branch, prefetch_engine.py:547-553).
  * Up to 4096 blocks per request.
  */
-int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off,
-                     const int32_t* seg_len, const int32_t* topk_len, int n_req, int max_seg_len,
-                     int n_layers, int start_w, int end_w, int32_t* idx_out, int out_stride,
-                     int32_t* count_out, const int32_t* block_tables, int bt_stride,
+int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, int64_t scores_rows,
+                     const int32_t* seg_off, const int32_t* seg_len, const int32_t* topk_len, int n_req,
+                     int max_seg_len, int n_layers, int start_w, int end_w, int32_t* idx_out,
+                     int out_stride, int32_t* count_out, const int32_t* block_tables, int bt_stride,
                      int32_t* phys_out, const int32_t* seq_lens, int block_size,
                      int32_t* sparse_seq_lens, ucm_stream_t stream);
+
+/*
+ * ucm_score_blocks and ucm_topk_windows as ONE launch - what
+ * TopkBlockSelector::SelectTopK does per request (select_topk_block.cpp:116-129:
+ * group mean, scores, selection) for every request and layer of the call.  A
+ * request's scoring workgroups each take a ticket when their scores are visible
+ * to the whole device; the one that draws the last ticket runs the request's
+ * selection, so no second launch waits for the first to drain.  Scores and
+ * selections are bit-identical to the two calls.
+ *
+ * The arguments travel in a struct so that a caller that issues the call once
+ * per layer (the plugin's attention hook) fills it once per step and changes
+ * two fields (q, first_layer) per call.  Fields are those of the two entry
+ * points above, with these differences:
+ *   struct_size  sizeof(ucm_score_select_args_t), checked
+ *   q          the queries of layer first_layer (a layer's own query tensor);
+ *              every other pointer names layer 0 of its table, and the call
+ *              works on layers first_layer .. first_layer+n_layers-1
+ *   repre_rows  rows of a layer of `repre` AND scores a layer of `scores` holds
+ *   idx_layer_stride, count_layer_stride  elements between two layers of
+ *              idx_out / phys_out and of count_out / sparse_seq_lens / tickets;
+ *              0 = dense (n_req*out_stride and n_req).  A caller that keeps
+ *              persistent [layers][max_requests][...] tables and runs a batch of
+ *              fewer requests names the tables' own strides.
+ *   tickets    dev int32 [layers][n_req] (indexed like count_out): zero before
+ *              the first call; every call leaves it zero.  Calls that overlap
+ *              in time (different streams) need arrays of their own.
+ * Up to 1024 blocks per request (UCM_ENOTSUP beyond: use the two calls).
+ */
+typedef struct ucm_score_select_args {
+    size_t struct_size;
+    const void* q;
+    int q_dtype;
+    int q_heads;
+    int64_t q_layer_stride;
+    const int32_t* q_rows;
+    const void* repre;
+    int repre_dtype;
+    int num_repre;
+    int64_t repre_layer_stride;
+    int64_t repre_rows;
+    const int32_t* seg_off;
+    const int32_t* seg_len;
+    const int32_t* topk_len;
+    int n_req;
+    int max_seg_len;
+    int first_layer;
+    int n_layers;
+    int kv_heads;
+    int head_dim;
+    float* scores;
+    int64_t scores_layer_stride;
+    float scale;
+    int tile_blocks;
+    int start_w;
+    int end_w;
+    int32_t* idx_out;
+    int32_t* count_out;
+    int out_stride;
+    int bt_stride;
+    const int32_t* block_tables;
+    int32_t* phys_out;
+    const int32_t* seq_lens;
+    int32_t* sparse_seq_lens;
+    int block_size;
+    int reserved;
+    int32_t* tickets;
+    int64_t idx_layer_stride;
+    int64_t count_layer_stride;
+} ucm_score_select_args_t;
+int ucm_score_select(const ucm_score_select_args_t* args, ucm_stream_t stream);
 
 /*
  * The ESA retrieval backend's computation for a batch of requests -
@@ -357,6 +437,9 @@ int ucm_prefetch_plan(const int32_t* map_block, const int32_t* map_len, int32_t*
  *           qbar_codes, block_codes and block_codes_layer_stride must be
  *           multiples of 16 bytes (UCM_EINVAL otherwise): a kv head's code is
  *           read as one 16-byte load.
+ *   rows    rows of a layer of the summary tables (colsum / block_codes) and of
+ *           `scores`: a request whose seg_off .. seg_off+seg_len does not lie inside
+ *           [0, rows) is not scored (its descriptors live in device memory).
  * The reference keeps init 1 / local 2 blocks out of the candidates and
  * index-sorts its picks (kvcomp.py:219-221,249-254): ucm_topk_windows with the
  * matching windows gives the same set.
@@ -373,7 +456,7 @@ int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const in
                             uint8_t* qbar_codes, ucm_stream_t stream);
 int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_codes,
                           const int16_t* colsum, int64_t colsum_layer_stride,
-                          const uint8_t* block_codes, int64_t block_codes_layer_stride,
+                          const uint8_t* block_codes, int64_t block_codes_layer_stride, int64_t rows,
                           const int32_t* seg_off, const int32_t* seg_len, int n_req,
                           int64_t total_blocks, int n_layers, int kv_heads, int bits, float* scores,
                           int64_t scores_layer_stride, int round_fp16, ucm_stream_t stream);
@@ -417,16 +500,24 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  * the block's sub-blocks of the probabilities.  The top-k of the votes is
  * taken by ucm_kvstar_topk.  fp32 on the matrix cores;
  * agrees with the reference's scalar loop to rounding, not bit for bit.
- *   q_f16    dev fp16; task t's [n_tokens][q_heads][d_orig] block starts
- *            q_off[t] elements in (dev int64[n_tasks])
- *   pruned   dev int32[*][kv_heads][d_pruned] channel lists, pruned_sel dev
- *            int32[n_tasks] picks one per task (-1: none); both NULL when
- *            d_pruned == d_orig
+ *   q_f16    dev fp16 buffer of q_elems elements; task t's
+ *            [n_tokens][q_heads][d_orig] block starts q_off[t] elements in
+ *            (dev int64[n_tasks])
+ *   pruned   dev int32[n_pruned_lists][kv_heads][d_pruned] channel lists,
+ *            pruned_sel dev int32[n_tasks] picks one per task (-1: none); both
+ *            NULL when d_pruned == d_orig
  *   repre_f16  dev fp16, one layer of the table above: cell (h, r) starts
- *            h*repre_head_stride + r*repre_row_stride elements in; task t owns rows
- *            seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >= every seg_len
+ *            h*repre_head_stride + r*repre_row_stride elements in, r < repre_rows;
+ *            task t owns rows seg_off[t] .. seg_off[t]+seg_len[t]-1; max_blocks >=
+ *            every seg_len (a longer one is cut there)
  *   ws_max, ws_part  dev fp32 scratch of the sizes ucm_kvstar_workspace_floats
- *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev fp32, task t's votes at votes[seg_off[t] + b].
+ *            returns (rows_per_head = n_tokens * q_heads/kv_heads); votes dev
+ *            fp32 [>= repre_rows], task t's votes at votes[seg_off[t] + b].
+ * q_off, pruned_sel, seg_off and seg_len live in device memory, where the host
+ * cannot check them: a task whose query block does not lie inside the buffer,
+ * whose rows do not lie inside [0, repre_rows) or whose list index is not below
+ * n_pruned_lists is skipped by every kernel of the call (its votes stay as
+ * they were).
  * n_tokens * (q_heads/kv_heads) <= 64, kv_heads <= 8, d_pad a multiple of 16
  * and <= 128, sub_blocks a power of two up to 128.
  */
@@ -453,11 +544,11 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
 int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_per_head, int max_blocks,
                                 int sub_blocks, int d_pad, int tiles_per_wave, int64_t* max_floats,
                                 int64_t* part_floats);
-int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
-                     const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                     int64_t repre_head_stride, int64_t repre_row_stride, const int32_t* seg_off,
-                     const int32_t* seg_len, int n_tasks, int max_blocks,
-                     int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+int ucm_kvstar_votes(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads,
+                     int d_orig, const int32_t* pruned, int n_pruned_lists, const int32_t* pruned_sel,
+                     const void* repre_f16, int64_t repre_rows, int64_t repre_head_stride,
+                     int64_t repre_row_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                     int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                      int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
                      int tiles_per_wave, ucm_stream_t stream);
 /* The same for tasks whose representatives do not share one table (the
@@ -466,15 +557,16 @@ int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int 
  * task_tables[t] (dev array of n_tasks dev pointers, 16-byte aligned; cell
  * (h, r) of task t's table starts h*task_head_strides[t] + r*task_row_stride
  * elements in, multiples of 8) and its block 0 is the table's row 0; seg_off
- * only places the task's votes. */
-int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
-                            const int32_t* pruned, const int32_t* pruned_sel,
+ * only places the task's votes, inside votes[0 .. votes_rows) (a task whose
+ * votes would fall outside is skipped; the table pointers themselves are
+ * addresses the caller vouches for). */
+int ucm_kvstar_votes_tables(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads,
+                            int d_orig, const int32_t* pruned, int n_pruned_lists, const int32_t* pruned_sel,
                             const void* const* task_tables, const int64_t* task_head_strides,
-                            int64_t task_row_stride, const int32_t* seg_off, const int32_t* seg_len,
-                            int n_tasks, int max_blocks,
-                            int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+                            int64_t task_row_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                            int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                             int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
-                            int tiles_per_wave, ucm_stream_t stream);
+                            int64_t votes_rows, int tiles_per_wave, ucm_stream_t stream);
 
 /*
  * The selection step of KVStar::Execute on the votes of n_tasks tasks
@@ -487,9 +579,10 @@ int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_token
  * min(topk_len[t], seg_len[t]) of them; the reference returns them descending
  * by (score, index), an order the caller restores by sorting these few
  * entries.  votes as written by ucm_kvstar_votes (task t's at
- * votes[seg_off[t] + b]); topk_len[t] >= 1; at most 4096 blocks per task.
+ * votes[seg_off[t] + b], inside votes[0 .. votes_rows): a task outside selects
+ * nothing); topk_len[t] >= 1; at most 4096 blocks per task.
  */
-int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const int32_t* seg_len,
+int ucm_kvstar_topk(const float* votes, int64_t votes_rows, const int32_t* seg_off, const int32_t* seg_len,
                     const int32_t* topk_len, int n_tasks, int max_seg_len, int32_t* idx_out,
                     int out_stride, int32_t* count_out, ucm_stream_t stream);
 
@@ -505,8 +598,8 @@ int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const int32_t* s
  * round trip.  votes, seg_off, seg_len as for ucm_kvstar_topk; count dev
  * int32[n_tasks] (its count_out); max_count >= every count, at most 4096.
  */
-int ucm_kvstar_order(const float* votes, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
-                     int max_count, int32_t* idx_io, int out_stride, const int32_t* count,
+int ucm_kvstar_order(const float* votes, int64_t votes_rows, const int32_t* seg_off, const int32_t* seg_len,
+                     int n_tasks, int max_count, int32_t* idx_io, int out_stride, const int32_t* count,
                      ucm_stream_t stream);
 
 /*

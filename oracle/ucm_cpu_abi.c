@@ -29,6 +29,7 @@
 TWIN(ucm_block_mean);
 TWIN(ucm_score_blocks);
 TWIN(ucm_topk_windows);
+TWIN(ucm_score_select);
 TWIN(ucm_kv_gather_blocks);
 TWIN(ucm_kv_scatter_blocks);
 TWIN(ucm_kv_gather_selected);
@@ -127,23 +128,27 @@ int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks
     return UCM_OK;
 }
 
-int ucm_score_blocks_cpu(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows, int q_heads,
-                         const void* repre, int repre_dtype, int64_t repre_layer_stride, const int32_t* seg_off,
-                         const int32_t* seg_len, int n_req, int max_seg_len, int64_t total_blocks, int n_layers,
-                         int kv_heads, int head_dim, float* scores, int64_t scores_layer_stride, float scale,
-                         int tile_blocks, ucm_stream_t stream)
+static float widen_q(const void* q, int q_dtype, size_t at)
 {
-    (void)stream;
-    (void)total_blocks;
-    (void)tile_blocks;
-    if (n_req < 0 || max_seg_len < 0 || n_layers < 0 || !isfinite(scale)) { return UCM_EINVAL; }
+    if (q_dtype == UCM_DTYPE_F32) { return ((const float*)q)[at]; }
+    return q_dtype == UCM_DTYPE_BF16 ? orc_bf16_to_f32(((const uint16_t*)q)[at]) : orc_f16_to_f32(((const uint16_t*)q)[at]);
+}
+
+/* scores of the requests whose descriptors may be followed (the device library's rule: query row inside the
+ * layer's query block, rows inside [0, repre_rows)); the others are left alone */
+static int score_host(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
+                      int repre_dtype, int64_t repre_layer_stride, int64_t repre_rows, int num_repre, const int32_t* seg_off,
+                      const int32_t* seg_len, int n_req, int max_seg_len, int n_layers, int kv_heads, int head_dim, float* scores,
+                      int64_t scores_layer_stride, float scale)
+{
+    if (n_req < 0 || max_seg_len < 0 || n_layers < 0 || !isfinite(scale) || repre_rows < 0 || num_repre < 1) { return UCM_EINVAL; }
     if (n_req == 0 || max_seg_len == 0 || n_layers == 0) { return UCM_OK; }
     if (!q || !repre || !seg_off || !seg_len || !scores || kv_heads <= 0 || q_heads < kv_heads ||
-        q_heads % kv_heads != 0 || head_dim <= 0 || (q_dtype != UCM_DTYPE_F32 && q_dtype != UCM_DTYPE_BF16) ||
+        q_heads % kv_heads != 0 || head_dim <= 0 || q_dtype < UCM_DTYPE_F32 || q_dtype > UCM_DTYPE_F16 ||
         (repre_dtype != UCM_DTYPE_F32 && repre_dtype != UCM_DTYPE_BF16)) {
         return UCM_EINVAL;
     }
-    const size_t qrow = (size_t)q_heads * head_dim, row = (size_t)kv_heads * head_dim;
+    const size_t qrow = (size_t)q_heads * head_dim, row = (size_t)kv_heads * num_repre * head_dim;
     float* qf = (float*)malloc(qrow * sizeof(float));
     float* wide = (float*)malloc((size_t)max_seg_len * row * sizeof(float));
     if (!qf || !wide) { free(qf); free(wide); return UCM_ENOMEM; }
@@ -153,10 +158,9 @@ int ucm_score_blocks_cpu(const void* q, int q_dtype, int64_t q_layer_stride, con
             const int32_t n = seg_len[r] < max_seg_len ? seg_len[r] : max_seg_len;
             /* with q_rows, a layer's rows end at q_layer_stride: a request whose row lies outside is skipped */
             if (n <= 0 || qr < 0 || (q_rows && (int64_t)(qr + 1) * (int64_t)qrow > q_layer_stride)) { continue; }
+            if (seg_off[r] < 0 || (int64_t)seg_off[r] + n > repre_rows) { continue; }
             const size_t q_at = (size_t)l * (size_t)q_layer_stride + (size_t)qr * qrow;
-            for (size_t c = 0; c < qrow; ++c) {
-                qf[c] = q_dtype == UCM_DTYPE_F32 ? ((const float*)q)[q_at + c] : orc_bf16_to_f32(((const uint16_t*)q)[q_at + c]);
-            }
+            for (size_t c = 0; c < qrow; ++c) { qf[c] = widen_q(q, q_dtype, q_at + c); }
             orc_q_head_mean(qf, (uint32_t)kv_heads, (uint32_t)q_heads, (uint32_t)head_dim);
             const size_t t_at = (size_t)l * (size_t)repre_layer_stride + (size_t)seg_off[r] * row;
             const float* table;
@@ -167,7 +171,7 @@ int ucm_score_blocks_cpu(const void* q, int q_dtype, int64_t q_layer_stride, con
                 table = wide;
             }
             float* out = scores + (size_t)l * (size_t)scores_layer_stride + seg_off[r];
-            orc_kq_scores(qf, table, (uint32_t)n, (uint32_t)kv_heads, 1, (uint32_t)head_dim, out);
+            orc_kq_scores(qf, table, (uint32_t)n, (uint32_t)kv_heads, (uint32_t)num_repre, (uint32_t)head_dim, out);
             for (int32_t b = 0; b < n; ++b) { out[b] = out[b] * scale; }
         }
     }
@@ -176,14 +180,27 @@ int ucm_score_blocks_cpu(const void* q, int q_dtype, int64_t q_layer_stride, con
     return UCM_OK;
 }
 
-int ucm_topk_windows_cpu(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off, const int32_t* seg_len,
-                         const int32_t* topk_len, int n_req, int max_seg_len, int n_layers, int start_w, int end_w,
-                         int32_t* idx_out, int out_stride, int32_t* count_out, const int32_t* block_tables, int bt_stride,
-                         int32_t* phys_out, const int32_t* seq_lens, int block_size, int32_t* sparse_seq_lens,
+int ucm_score_blocks_cpu(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows, int q_heads,
+                         const void* repre, int repre_dtype, int64_t repre_layer_stride, int64_t repre_rows, int num_repre,
+                         const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len, int64_t total_blocks,
+                         int n_layers, int kv_heads, int head_dim, float* scores, int64_t scores_layer_stride, float scale,
+                         int tile_blocks, ucm_stream_t stream)
+{
+    (void)stream;
+    (void)total_blocks;
+    (void)tile_blocks;
+    return score_host(q, q_dtype, q_layer_stride, q_rows, q_heads, repre, repre_dtype, repre_layer_stride, repre_rows, num_repre,
+                      seg_off, seg_len, n_req, max_seg_len, n_layers, kv_heads, head_dim, scores, scores_layer_stride, scale);
+}
+
+int ucm_topk_windows_cpu(const float* scores, int64_t scores_layer_stride, int64_t scores_rows, const int32_t* seg_off,
+                         const int32_t* seg_len, const int32_t* topk_len, int n_req, int max_seg_len, int n_layers, int start_w,
+                         int end_w, int32_t* idx_out, int out_stride, int32_t* count_out, const int32_t* block_tables,
+                         int bt_stride, int32_t* phys_out, const int32_t* seq_lens, int block_size, int32_t* sparse_seq_lens,
                          ucm_stream_t stream)
 {
     (void)stream;
-    if (n_req < 0 || n_layers < 0 || max_seg_len < 0 || start_w < 0 || end_w < 0) { return UCM_EINVAL; }
+    if (n_req < 0 || n_layers < 0 || max_seg_len < 0 || start_w < 0 || end_w < 0 || scores_rows < 0) { return UCM_EINVAL; }
     if (n_req == 0 || n_layers == 0) { return UCM_OK; }
     if (!scores || !seg_off || !seg_len || !topk_len || !idx_out || !count_out || out_stride < max_seg_len ||
         (block_tables && (!phys_out || bt_stride < max_seg_len)) || (seq_lens && (!sparse_seq_lens || block_size <= 0))) {
@@ -192,7 +209,9 @@ int ucm_topk_windows_cpu(const float* scores, int64_t scores_layer_stride, const
     for (int l = 0; l < n_layers; ++l) {
         for (int r = 0; r < n_req; ++r) {
             const size_t lr = (size_t)l * n_req + r;
-            const int32_t n = seg_len[r] < max_seg_len ? seg_len[r] : max_seg_len;
+            int32_t n = seg_len[r] < max_seg_len ? seg_len[r] : max_seg_len;
+            /* a request whose scores do not lie inside the layer selects nothing */
+            if (n > 0 && (seg_off[r] < 0 || (int64_t)seg_off[r] + n > scores_rows)) { n = 0; }
             int32_t* out = idx_out + lr * (size_t)out_stride;
             int32_t cnt = 0;
             if (n > 0) {
@@ -216,6 +235,37 @@ int ucm_topk_windows_cpu(const float* scores, int64_t scores_layer_stride, const
         }
     }
     return UCM_OK;
+}
+
+/* the one-launch entry point: scores, then the selection from them, on layers first_layer .. */
+int ucm_score_select_cpu(const ucm_score_select_args_t* p, ucm_stream_t stream)
+{
+    if (!p || p->struct_size != sizeof(ucm_score_select_args_t) || p->n_req < 0 || p->n_layers <= 0 || p->first_layer < 0) {
+        return UCM_EINVAL;
+    }
+    if (p->n_req == 0) { return UCM_OK; }
+    if (!p->tickets || !p->scores || p->max_seg_len < 0) { return UCM_EINVAL; }
+    if (p->max_seg_len > 1024) { return UCM_ENOTSUP; }
+    const int64_t es = p->repre_dtype == UCM_DTYPE_BF16 ? 2 : 4;
+    const int first = p->first_layer;
+    const char* repre = (const char*)p->repre + (int64_t)first * p->repre_layer_stride * es;
+    float* scores = p->scores + (int64_t)first * p->scores_layer_stride;
+    const int64_t idx_ls = p->idx_layer_stride ? p->idx_layer_stride : (int64_t)p->n_req * p->out_stride;
+    const int64_t cnt_ls = p->count_layer_stride ? p->count_layer_stride : p->n_req;
+    if (idx_ls < (int64_t)p->n_req * p->out_stride || cnt_ls < p->n_req) { return UCM_EINVAL; }
+    int rc = score_host(p->q, p->q_dtype, p->q_layer_stride, p->q_rows, p->q_heads, repre, p->repre_dtype, p->repre_layer_stride,
+                        p->repre_rows, p->num_repre, p->seg_off, p->seg_len, p->n_req, p->max_seg_len, p->n_layers, p->kv_heads,
+                        p->head_dim, scores, p->scores_layer_stride, p->scale);
+    /* the selection layer by layer: the tables' layers may lie further apart than a dense layer */
+    for (int l = 0; l < p->n_layers && rc == UCM_OK; ++l) {
+        const int64_t li = (first + l) * idx_ls, lc = (first + l) * cnt_ls;
+        rc = ucm_topk_windows_cpu(scores + (int64_t)l * p->scores_layer_stride, p->scores_layer_stride, p->repre_rows, p->seg_off,
+                                  p->seg_len, p->topk_len, p->n_req, p->max_seg_len, 1, p->start_w, p->end_w, p->idx_out + li,
+                                  p->out_stride, p->count_out + lc, p->block_tables, p->bt_stride,
+                                  p->phys_out ? p->phys_out + li : NULL, p->seq_lens, p->block_size,
+                                  p->sparse_seq_lens ? p->sparse_seq_lens + lc : NULL, stream);
+    }
+    return rc;
 }
 
 static int kv_move(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
@@ -512,13 +562,13 @@ int ucm_hash_encode_queries_cpu(const void* q_bf16, int64_t q_layer_stride, cons
 
 int ucm_hash_score_blocks_cpu(int mode, const int16_t* q_sum, const uint8_t* qbar_codes, const int16_t* colsum,
                               int64_t colsum_layer_stride, const uint8_t* block_codes, int64_t block_codes_layer_stride,
-                              const int32_t* seg_off, const int32_t* seg_len, int n_req, int64_t total_blocks, int n_layers,
+                              int64_t rows, const int32_t* seg_off, const int32_t* seg_len, int n_req, int64_t total_blocks, int n_layers,
                               int kv_heads, int bits, float* scores, int64_t scores_layer_stride, int round_fp16,
                               ucm_stream_t stream)
 {
     (void)stream;
     (void)total_blocks;
-    if (n_req < 0 || n_layers < 0 || (mode != 0 && mode != 1)) { return UCM_EINVAL; }
+    if (n_req < 0 || n_layers < 0 || (mode != 0 && mode != 1) || rows < 0) { return UCM_EINVAL; }
     if (n_req == 0 || n_layers == 0) { return UCM_OK; }
     if (!seg_off || !seg_len || !scores || kv_heads <= 0 || (mode == 0 && (!q_sum || !colsum)) ||
         (mode == 1 && (!qbar_codes || !block_codes))) {
@@ -529,6 +579,8 @@ int ucm_hash_score_blocks_cpu(int mode, const int16_t* q_sum, const uint8_t* qba
     for (int l = 0; l < n_layers; ++l) {
         for (int r = 0; r < n_req; ++r) {
             const size_t lr = (size_t)l * n_req + r;
+            /* a request whose rows do not lie inside the summary tables is not scored */
+            if (seg_off[r] < 0 || (int64_t)seg_off[r] + (seg_len[r] > 0 ? seg_len[r] : 0) > rows) { continue; }
             float* out = scores + (size_t)l * (size_t)scores_layer_stride + seg_off[r];
             for (int32_t b = 0; b < seg_len[r]; ++b) {
                 const size_t row = (size_t)seg_off[r] + b;
@@ -622,18 +674,19 @@ static int cmp_i32(const void* a, const void* b)
     return (x > y) - (x < y);
 }
 
-int ucm_kvstar_topk_cpu(const float* votes, const int32_t* seg_off, const int32_t* seg_len, const int32_t* topk_len,
-                        int n_tasks, int max_seg_len, int32_t* idx_out, int out_stride, int32_t* count_out,
-                        ucm_stream_t stream)
+int ucm_kvstar_topk_cpu(const float* votes, int64_t votes_rows, const int32_t* seg_off, const int32_t* seg_len,
+                        const int32_t* topk_len, int n_tasks, int max_seg_len, int32_t* idx_out, int out_stride,
+                        int32_t* count_out, ucm_stream_t stream)
 {
     (void)stream;
-    if (n_tasks < 0 || max_seg_len < 0) { return UCM_EINVAL; }
+    if (n_tasks < 0 || max_seg_len < 0 || votes_rows < 0) { return UCM_EINVAL; }
     if (n_tasks == 0) { return UCM_OK; }
     if (!votes || !seg_off || !seg_len || !topk_len || !idx_out || !count_out || out_stride < max_seg_len) { return UCM_EINVAL; }
     if (max_seg_len > 4096) { return UCM_ENOTSUP; }
     for (int t = 0; t < n_tasks; ++t) {
-        int n = seg_len[t];
+        int n = seg_len[t] < max_seg_len ? seg_len[t] : max_seg_len;
         if (n > out_stride) { n = out_stride; }
+        if (n > 0 && (seg_off[t] < 0 || (int64_t)seg_off[t] + n > votes_rows)) { n = 0; }   /* votes outside the array */
         int32_t* out = idx_out + (size_t)t * out_stride;
         if (n <= 0) { count_out[t] = 0; continue; }
         const int32_t k = topk_len[t];
@@ -650,11 +703,11 @@ int ucm_kvstar_topk_cpu(const float* votes, const int32_t* seg_off, const int32_
     return UCM_OK;
 }
 
-int ucm_kvstar_order_cpu(const float* votes, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_count,
-                         int32_t* idx_io, int out_stride, const int32_t* count, ucm_stream_t stream)
+int ucm_kvstar_order_cpu(const float* votes, int64_t votes_rows, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                         int max_count, int32_t* idx_io, int out_stride, const int32_t* count, ucm_stream_t stream)
 {
     (void)stream;
-    if (n_tasks < 0 || max_count < 0) { return UCM_EINVAL; }
+    if (n_tasks < 0 || max_count < 0 || votes_rows < 0) { return UCM_EINVAL; }
     if (n_tasks == 0 || max_count == 0) { return UCM_OK; }
     if (!votes || !seg_off || !seg_len || !idx_io || !count || out_stride < max_count) { return UCM_EINVAL; }
     if (max_count > 4096) { return UCM_ENOTSUP; }
@@ -663,6 +716,7 @@ int ucm_kvstar_order_cpu(const float* votes, const int32_t* seg_off, const int32
         int k = count[t];
         if (k > out_stride) { k = out_stride; }
         if (k > 4096) { k = 4096; }
+        if (seg_off[t] < 0 || seg_len[t] < 0 || (int64_t)seg_off[t] + seg_len[t] > votes_rows) { continue; }
         const float* v = votes + seg_off[t];
         /* descending by (vote, index): insertion sort, the lists are short; the two zeros compare equal */
         for (int a = 1; a < k; ++a) {
@@ -811,6 +865,15 @@ static int kvstar_task_votes(const uint16_t* q, int n_tokens, int q_heads, int d
     return UCM_OK;
 }
 
+/* the device library's rule for a task's descriptors: query block inside the buffer, channel list inside the lists,
+ * rows inside the table / the votes array; a task outside any of them is skipped */
+static int kvstar_task_ok(int64_t q_elems, const int64_t* q_off, int64_t q_need, int n_lists, const int32_t* pruned_sel,
+                          int64_t rows_bound, const int32_t* seg_off, int n, int t)
+{
+    return q_off[t] >= 0 && q_off[t] + q_need <= q_elems && (!pruned_sel || pruned_sel[t] < n_lists) && seg_off[t] >= 0 &&
+           (int64_t)seg_off[t] + (n > 0 ? n : 0) <= rows_bound;
+}
+
 static int kvstar_votes_check(const void* q, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
                               const int32_t* pruned_sel, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
                               int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, const float* votes)
@@ -829,19 +892,23 @@ static int kvstar_votes_check(const void* q, const int64_t* q_off, int n_tokens,
     return 1;   /* go on */
 }
 
-int ucm_kvstar_votes_cpu(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
-                         const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, int64_t repre_row_stride,
-                         const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads,
-                         int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
-                         float* votes, int tiles_per_wave, ucm_stream_t stream)
+int ucm_kvstar_votes_cpu(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                         const int32_t* pruned, int n_pruned_lists, const int32_t* pruned_sel, const void* repre_f16,
+                         int64_t repre_rows, int64_t repre_head_stride, int64_t repre_row_stride, const int32_t* seg_off,
+                         const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned,
+                         int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
+                         int tiles_per_wave, ucm_stream_t stream)
 {
     (void)ws_max; (void)ws_max_floats; (void)ws_part; (void)ws_part_floats; (void)tiles_per_wave; (void)stream;
     const int rc = kvstar_votes_check(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, seg_off, seg_len, n_tasks,
                                       max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, votes);
     if (rc != 1) { return rc; }
-    if (!repre_f16) { return UCM_EINVAL; }
+    if (!repre_f16 || q_elems < 0 || repre_rows < 0 || n_pruned_lists < 0) { return UCM_EINVAL; }
     for (int t = 0; t < n_tasks; ++t) {
         const int n = seg_len[t] < max_blocks ? seg_len[t] : max_blocks;
+        if (!kvstar_task_ok(q_elems, q_off, (int64_t)n_tokens * q_heads * d_orig, n_pruned_lists, pruned_sel, repre_rows, seg_off, n, t)) {
+            continue;
+        }
         const int32_t* lists = (pruned && pruned_sel[t] >= 0) ? pruned + (size_t)pruned_sel[t] * kv_heads * d_pruned : NULL;
         const int r = kvstar_task_votes((const uint16_t*)q_f16 + q_off[t], n_tokens, q_heads, d_orig, lists,
                                         (const uint16_t*)repre_f16 + (int64_t)seg_off[t] * repre_row_stride, repre_head_stride,
@@ -851,20 +918,23 @@ int ucm_kvstar_votes_cpu(const void* q_f16, const int64_t* q_off, int n_tokens, 
     return UCM_OK;
 }
 
-int ucm_kvstar_votes_tables_cpu(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
-                                const int32_t* pruned, const int32_t* pruned_sel, const void* const* task_tables,
-                                const int64_t* task_head_strides, int64_t task_row_stride, const int32_t* seg_off,
-                                const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned,
-                                int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
-                                float* votes, int tiles_per_wave, ucm_stream_t stream)
+int ucm_kvstar_votes_tables_cpu(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                                const int32_t* pruned, int n_pruned_lists, const int32_t* pruned_sel,
+                                const void* const* task_tables, const int64_t* task_head_strides, int64_t task_row_stride,
+                                const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks,
+                                int kv_heads, int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part,
+                                int64_t ws_part_floats, float* votes, int64_t votes_rows, int tiles_per_wave, ucm_stream_t stream)
 {
     (void)ws_max; (void)ws_max_floats; (void)ws_part; (void)ws_part_floats; (void)tiles_per_wave; (void)stream;
     const int rc = kvstar_votes_check(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, seg_off, seg_len, n_tasks,
                                       max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, votes);
     if (rc != 1) { return rc; }
-    if (!task_tables || !task_head_strides) { return UCM_EINVAL; }
+    if (!task_tables || !task_head_strides || q_elems < 0 || votes_rows < 0 || n_pruned_lists < 0) { return UCM_EINVAL; }
     for (int t = 0; t < n_tasks; ++t) {
         const int n = seg_len[t] < max_blocks ? seg_len[t] : max_blocks;
+        if (!kvstar_task_ok(q_elems, q_off, (int64_t)n_tokens * q_heads * d_orig, n_pruned_lists, pruned_sel, votes_rows, seg_off, n, t)) {
+            continue;
+        }
         const int32_t* lists = (pruned && pruned_sel[t] >= 0) ? pruned + (size_t)pruned_sel[t] * kv_heads * d_pruned : NULL;
         const int r = kvstar_task_votes((const uint16_t*)q_f16 + q_off[t], n_tokens, q_heads, d_orig, lists,
                                         (const uint16_t*)task_tables[t], task_head_strides[t], task_row_stride, n, sub_blocks,

@@ -10,7 +10,7 @@ import numpy as np
 import oracle
 import synth
 
-TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
+TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_select", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
@@ -122,20 +122,41 @@ def run(call, side):
     seg_off, seg_len = side.up(OFF), side.up(LENS)
     s32 = side.up(np.full((L, ROWS), -3, np.float32))
     q32 = side.up(x["q32"])
-    call("ucm_score_blocks", side.ptr(q32), 0, 5 * HQ * D, None, HQ, side.ptr(tabs[0]), 0, ROWS * ROW, side.ptr(seg_off),
+    call("ucm_score_blocks", side.ptr(q32), 0, 5 * HQ * D, None, HQ, side.ptr(tabs[0]), 0, ROWS * ROW, ROWS, 1, side.ptr(seg_off),
          side.ptr(seg_len), 3, 6, 10, L, HKV, D, side.ptr(s32), ROWS, 1.0, 0, None)
     s16 = side.up(np.full((L, ROWS), -3, np.float32))
     q16, q_rows = side.up(x["q16"]), side.up(x["q_rows"])
-    call("ucm_score_blocks", side.ptr(q16), 1, 5 * HQ * D, side.ptr(q_rows), HQ, side.ptr(tabs[2]), 1, ROWS * ROW,
+    call("ucm_score_blocks", side.ptr(q16), 1, 5 * HQ * D, side.ptr(q_rows), HQ, side.ptr(tabs[2]), 1, ROWS * ROW, ROWS, 1,
          side.ptr(seg_off), side.ptr(seg_len), 3, 6, 0, L, HKV, D, side.ptr(s16), ROWS, 0.5, 0, None)
     out["scores32"], out["scores16"] = s32, s16
     # 3. selection with the block-table lookup and the sparse lengths
     topk, tables, seq_lens = side.up(x["topk"]), side.up(x["tables"]), side.up(x["seq_lens"])
     idx, phys = side.up(np.full((L, 3, 6), -1, np.int32)), side.up(np.full((L, 3, 6), -1, np.int32))
     cnt, sparse = side.up(np.full((L, 3), -1, np.int32)), side.up(np.full((L, 3), -1, np.int32))
-    call("ucm_topk_windows", side.ptr(s16), ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk), 3, 6, L, 1, 1,
+    call("ucm_topk_windows", side.ptr(s16), ROWS, ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk), 3, 6, L, 1, 1,
          side.ptr(idx), 6, side.ptr(cnt), side.ptr(tables), 8, side.ptr(phys), side.ptr(seq_lens), BS, side.ptr(sparse), None)
     out.update(idx=idx, phys=phys, cnt=cnt, sparse=sparse)
+    # 3b. the same scores and selection as one launch: every output must equal the two calls'
+    import ctypes as C
+
+    from ucm_amd import _lib
+
+    # (its output tables are kept for four requests, of which this batch uses three: layer strides of their own)
+    f_scores = side.up(np.full((L, ROWS), -3, np.float32))
+    f_idx, f_phys = side.up(np.full((L, 4, 6), -1, np.int32)), side.up(np.full((L, 4, 6), -1, np.int32))
+    f_cnt, f_sparse = side.up(np.full((L, 4), -1, np.int32)), side.up(np.full((L, 4), -1, np.int32))
+    tickets = side.up(np.zeros((L, 4), np.int32))
+    args = _lib.ScoreSelectArgs(
+        q=side.ptr(q16), q_dtype=1, q_heads=HQ, q_layer_stride=5 * HQ * D, q_rows=side.ptr(q_rows), repre=side.ptr(tabs[2]),
+        repre_dtype=1, repre_layer_stride=ROWS * ROW, repre_rows=ROWS, seg_off=side.ptr(seg_off), seg_len=side.ptr(seg_len),
+        topk_len=side.ptr(topk), n_req=3, max_seg_len=6, first_layer=0, kv_heads=HKV, head_dim=D, scores=side.ptr(f_scores),
+        scores_layer_stride=ROWS, start_w=1, end_w=1, idx_out=side.ptr(f_idx), count_out=side.ptr(f_cnt), out_stride=6,
+        bt_stride=8, block_tables=side.ptr(tables), phys_out=side.ptr(f_phys), seq_lens=side.ptr(seq_lens),
+        sparse_seq_lens=side.ptr(f_sparse), block_size=BS, tickets=side.ptr(tickets), idx_layer_stride=4 * 6,
+        count_layer_stride=4)
+    args.n_layers, args.scale = L, 0.5
+    call("ucm_score_select", C.addressof(args), None)
+    out.update(f_scores=f_scores, f_idx=f_idx, f_phys=f_phys, f_cnt=f_cnt, f_sparse=f_sparse, tickets=tickets)
     # 4. delta plan, twice: empty slots first, then the other scores' selection against what the first left
     resident = side.up(np.full((L, 3, 4), -1, np.int32))
     load, slot_of, miss = (side.up(np.full(s, -9, np.int32)) for s in ((L, 3, 4), (L, 3, 6), (L, 3)))
@@ -144,7 +165,7 @@ def run(call, side):
     side.sync()
     out.update(resident1=side.up(side.down(resident)), load1=side.up(side.down(load)), miss1=side.up(side.down(miss)))
     idx2, phys2, cnt2 = (side.up(np.full(s, -1, np.int32)) for s in ((L, 3, 6), (L, 3, 6), (L, 3)))
-    call("ucm_topk_windows", side.ptr(s32), ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk), 3, 6, L, 1, 1,
+    call("ucm_topk_windows", side.ptr(s32), ROWS, ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk), 3, 6, L, 1, 1,
          side.ptr(idx2), 6, side.ptr(cnt2), side.ptr(tables), 8, side.ptr(phys2), None, BS, None, None)
     call("ucm_delta_plan", side.ptr(idx2), side.ptr(phys2), side.ptr(cnt2), 3, L, 6, side.ptr(resident), 4, side.ptr(load),
          side.ptr(slot_of), side.ptr(miss), None)
@@ -169,6 +190,44 @@ def run(call, side):
         out[f"restored{l}"] = empty[l]
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x
+
+
+def run_bounds(call, side):
+    """Segment descriptors that point outside the tables: the call declares fewer rows than the buffers hold (the
+    table starts PAD rows into its buffer), so a descriptor that were followed would land in memory the test owns and
+    show up in the padding.  Request 0 is in range, request 1 starts below row 0, request 2 ends past the last row."""
+    import ctypes as C
+
+    from ucm_amd import _lib
+
+    PAD = 4
+    x = inputs()
+    repre_h = synth.normal_f32(7050, (L, ROWS + 2 * PAD, ROW))
+    repre = side.up(repre_h)
+    scores = side.up(np.full((L, ROWS + 2 * PAD), -3, np.float32))
+    q32 = side.up(x["q32"])
+    seg_off, seg_len = side.up(np.array([1, -2, 7], np.int32)), side.up(np.array([4, 3, 5], np.int32))
+    topk = side.up(np.array([2, 2, 2], np.int32))
+    stride_t, stride_s = (ROWS + 2 * PAD) * ROW, ROWS + 2 * PAD
+    call("ucm_score_blocks", side.ptr(q32), 0, 5 * HQ * D, None, HQ, side.ptr(repre) + PAD * ROW * 4, 0, stride_t, ROWS, 1,
+         side.ptr(seg_off), side.ptr(seg_len), 3, 6, 0, L, HKV, D, side.ptr(scores) + PAD * 4, stride_s, 1.0, 0, None)
+    idx, cnt = side.up(np.full((L, 3, 6), -1, np.int32)), side.up(np.full((L, 3), -1, np.int32))
+    call("ucm_topk_windows", side.ptr(scores) + PAD * 4, stride_s, ROWS, side.ptr(seg_off), side.ptr(seg_len), side.ptr(topk),
+         3, 6, L, 0, 0, side.ptr(idx), 6, side.ptr(cnt), None, 0, None, None, BS, None, None)
+    f_scores = side.up(np.full((L, ROWS + 2 * PAD), -3, np.float32))
+    f_idx, f_cnt = side.up(np.full((L, 3, 6), -1, np.int32)), side.up(np.full((L, 3), -1, np.int32))
+    tickets = side.up(np.zeros((L, 3), np.int32))
+    args = _lib.ScoreSelectArgs(
+        q=side.ptr(q32), q_dtype=0, q_heads=HQ, q_layer_stride=5 * HQ * D, repre=side.ptr(repre) + PAD * ROW * 4, repre_dtype=0,
+        repre_layer_stride=stride_t, repre_rows=ROWS, seg_off=side.ptr(seg_off), seg_len=side.ptr(seg_len),
+        topk_len=side.ptr(topk), n_req=3, max_seg_len=6, first_layer=0, kv_heads=HKV, head_dim=D,
+        scores=side.ptr(f_scores) + PAD * 4, scores_layer_stride=stride_s, start_w=0, end_w=0, idx_out=side.ptr(f_idx),
+        count_out=side.ptr(f_cnt), out_stride=6, tickets=side.ptr(tickets))
+    args.n_layers = L
+    call("ucm_score_select", C.addressof(args), None)
+    side.sync()
+    out = dict(scores=scores, idx=idx, cnt=cnt, f_scores=f_scores, f_idx=f_idx, f_cnt=f_cnt, tickets=tickets)
+    return {k: np.array(side.down(v)) for k, v in out.items()}, dict(repre=repre_h, q32=x["q32"], pad=PAD)
 
 
 HL, HNB, HBS, HHKV, HHQ, HD = 2, 7, 16, 2, 8, 128
@@ -208,8 +267,17 @@ def run_hash(call, side):
     for name, mode, fp16 in (("score_sum", 0, 0), ("score_sum_fp16", 0, 1), ("score_code", 1, 0)):
         sc = side.up(np.full((HL, H_ROWS), -3, np.float32))
         call("ucm_hash_score_blocks", mode, side.ptr(q_sum), side.ptr(qbar), side.ptr(colsum), H_ROWS * HHKV * 128,
-             side.ptr(bcodes), H_ROWS * HHKV * 16, side.ptr(seg_off), side.ptr(seg_len), 3, 5, HL, HHKV, 128, side.ptr(sc),
+             side.ptr(bcodes), H_ROWS * HHKV * 16, H_ROWS, side.ptr(seg_off), side.ptr(seg_len), 3, 5, HL, HHKV, 128, side.ptr(sc),
              H_ROWS, fp16, None)
+        out[name] = sc
+    # descriptors outside the summary tables: the first request starts below row 0, the third ends past the last row the
+    # call names (one row fewer than the tables hold, so a request that were followed would stay inside owned memory)
+    bad_off, bad_len = side.up(np.array([-1, 3, 3], np.int32)), side.up(np.array([2, 0, 3], np.int32))
+    for name, mode in (("score_sum_bad", 0), ("score_code_bad", 1)):
+        sc = side.up(np.full((HL, H_ROWS), -3, np.float32))
+        call("ucm_hash_score_blocks", mode, side.ptr(q_sum) , side.ptr(qbar), side.ptr(colsum), H_ROWS * HHKV * 128,
+             side.ptr(bcodes), H_ROWS * HHKV * 16, H_ROWS - 1, side.ptr(bad_off), side.ptr(bad_len), 3, 5, HL, HHKV, 128,
+             side.ptr(sc), H_ROWS, 0, None)
         out[name] = sc
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x
@@ -330,13 +398,25 @@ def run_more(call, side):
     n_tasks, longest = len(x["lens"]), int(x["lens"].max())
     votes, off, lens, ks = side.up(x["votes"]), side.up(x["off"]), side.up(x["lens"]), side.up(x["ks"])
     idx, cnt = side.up(np.full((n_tasks, longest), -1, np.int32)), side.up(np.full(n_tasks, -1, np.int32))
-    call("ucm_kvstar_topk", side.ptr(votes), side.ptr(off), side.ptr(lens), side.ptr(ks), n_tasks, longest, side.ptr(idx),
+    n_votes = len(x["votes"])
+    call("ucm_kvstar_topk", side.ptr(votes), n_votes, side.ptr(off), side.ptr(lens), side.ptr(ks), n_tasks, longest, side.ptr(idx),
          longest, side.ptr(cnt), None)
     side.sync()
     out["chosen"] = np.array(side.down(idx)).copy()
-    call("ucm_kvstar_order", side.ptr(votes), side.ptr(off), side.ptr(lens), n_tasks, longest, side.ptr(idx), longest,
+    call("ucm_kvstar_order", side.ptr(votes), n_votes, side.ptr(off), side.ptr(lens), n_tasks, longest, side.ptr(idx), longest,
          side.ptr(cnt), None)
     out.update(ordered=idx, chosen_count=cnt)
+    # the same with a votes array declared 50 entries shorter: the task that reaches past it (the fourth) selects
+    # nothing and its row is left alone by both calls; a task that starts below 0 likewise
+    off_bad = x["off"].copy()
+    off_bad[0] = -3
+    off_b = side.up(off_bad)
+    idx_b, cnt_b = side.up(np.full((n_tasks, longest), -1, np.int32)), side.up(np.full(n_tasks, -1, np.int32))
+    call("ucm_kvstar_topk", side.ptr(votes), n_votes - 50, side.ptr(off_b), side.ptr(lens), side.ptr(ks), n_tasks, longest,
+         side.ptr(idx_b), longest, side.ptr(cnt_b), None)
+    call("ucm_kvstar_order", side.ptr(votes), n_votes - 50, side.ptr(off_b), side.ptr(lens), n_tasks, longest, side.ptr(idx_b),
+         longest, side.ptr(cnt_b), None)
+    out.update(ordered_bad=idx_b, chosen_count_bad=cnt_b)
     # pointer-array copy: three pieces of 64 bytes, the last two swapped
     a, b = side.up(np.arange(192, dtype=np.uint8)), side.up(np.zeros(192, np.uint8))
     src = side.up(np.array([side.ptr(a), side.ptr(a) + 128, side.ptr(a) + 64], np.int64))
@@ -417,17 +497,32 @@ def run_kvstar(call, side):
     _lib.call("ucm_kvstar_workspace_floats", 3, K_HKV, K_X * K_G, 5, K_M, K_DPAD, 0, C.byref(mf), C.byref(pf))
     ws_max, ws_part = side.up(np.zeros(max(mf.value, 1), np.float32)), side.up(np.zeros(max(pf.value, 1), np.float32))
     votes = side.up(np.full(K_ROWS, -3, np.float32))
-    call("ucm_kvstar_votes", side.ptr(q), side.ptr(q_off), K_X, K_HKV * K_G, K_D, side.ptr(lists), side.ptr(sel),
-         side.ptr(tables["pruned"]), K_ROWS * cell, cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M, K_HKV, K_DP, K_DPAD,
-         side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes), 0, None)
+    q_elems = int(np.prod(x["q"].shape))
+    call("ucm_kvstar_votes", side.ptr(q), q_elems, side.ptr(q_off), K_X, K_HKV * K_G, K_D, side.ptr(lists), K_L, side.ptr(sel),
+         side.ptr(tables["pruned"]), K_ROWS, K_ROWS * cell, cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M, K_HKV, K_DP,
+         K_DPAD, side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes), 0, None)
     out["votes"] = votes
+    # descriptors the call must not follow: a query block that ends past the buffer (declared one task shorter), a
+    # channel list that does not exist, rows past the table (declared two rows shorter).  Each of the three tasks
+    # breaks one rule in turn, the other two vote as before.
+    q_need = K_X * K_HKV * K_G * K_D
+    for case in range(3):
+        bad_sel = np.zeros(3, np.int32)
+        bad_sel[0] = K_L if case == 1 else 0
+        sel_b = side.up(bad_sel)
+        votes_b = side.up(np.full(K_ROWS, -3, np.float32))
+        call("ucm_kvstar_votes", side.ptr(q), q_elems - (q_need if case == 0 else 0), side.ptr(q_off), K_X, K_HKV * K_G, K_D,
+             side.ptr(lists), K_L, side.ptr(sel_b), side.ptr(tables["pruned"]), K_ROWS - (2 if case == 2 else 0), K_ROWS * cell,
+             cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M, K_HKV, K_DP, K_DPAD, side.ptr(ws_max), mf.value,
+             side.ptr(ws_part), pf.value, side.ptr(votes_b), 0, None)
+        out[f"votes_bad{case}"] = votes_b
     base = side.ptr(tables["pruned"])
     task_tables = side.up(np.array([base + int(a) * cell * 2 for a in K_OFF], np.int64))
     head_strides = side.up(np.full(3, K_ROWS * cell, np.int64))
     votes_t = side.up(np.full(K_ROWS, -3, np.float32))
-    call("ucm_kvstar_votes_tables", side.ptr(q), side.ptr(q_off), K_X, K_HKV * K_G, K_D, side.ptr(lists), side.ptr(sel),
-         side.ptr(task_tables), side.ptr(head_strides), cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M, K_HKV, K_DP,
-         K_DPAD, side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes_t), 0, None)
+    call("ucm_kvstar_votes_tables", side.ptr(q), q_elems, side.ptr(q_off), K_X, K_HKV * K_G, K_D, side.ptr(lists), K_L,
+         side.ptr(sel), side.ptr(task_tables), side.ptr(head_strides), cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M,
+         K_HKV, K_DP, K_DPAD, side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes_t), K_ROWS, 0, None)
     out["votes_tables"] = votes_t
     side.sync()
     return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x

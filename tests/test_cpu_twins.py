@@ -37,6 +37,11 @@ def test_twins_reproduce_the_oracle(ucm):
                 assert got["sparse"][l, r] == (x["seq_lens"][r] if cnt[r] >= n else
                                                 O.block_table_gather(x["tables"][r], idx[r, : cnt[r]], int(x["seq_lens"][r]),
                                                                      cpu_twins.BS)[1])
+    # the one-launch entry point gives what the two calls gave, and leaves its tickets at zero
+    assert np.array_equal(got["f_scores"].view(np.uint32), got["scores16"].view(np.uint32))
+    for a, b in (("f_idx", "idx"), ("f_phys", "phys"), ("f_cnt", "cnt"), ("f_sparse", "sparse")):
+        assert np.array_equal(got[a][:, :3], got[b]) and (got[a][:, 3] == -1).all(), a      # the fourth request's row is not this batch's
+    assert not got["tickets"].any()
     # the first plan fills empty slots in order; the moves restore exactly the listed blocks
     assert np.array_equal(got["resident1"][:, 0, :3], got["idx"][:, 0, :3]) and (got["resident1"][:, 1] == -1).all()
     assert np.array_equal(got["miss1"], got["cnt"])
@@ -45,6 +50,26 @@ def test_twins_reproduce_the_oracle(ucm):
         for b in (5, 0, 11):
             want[:, b] = x["caches"][l][:, b]
         assert np.array_equal(got[f"restored{l}"], want)
+
+
+def test_descriptors_outside_the_tables_are_not_followed(ucm):
+    """seg_off / seg_len live in device memory: a request whose rows do not lie inside the table the call names is
+    skipped by the scores (its scores, and the padding around the table, keep what they held) and selects nothing."""
+    from ucm_amd import _lib
+
+    got, x = cpu_twins.run_bounds(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+    pad, rows = x["pad"], cpu_twins.ROWS
+    for key in ("scores", "f_scores"):
+        sc = got[key]
+        assert (sc[:, :pad + 1] == -3).all() and (sc[:, pad + 5:] == -3).all(), key        # only rows 1..4 were written
+        for l in range(cpu_twins.L):
+            _, _, want = O.select_topk_bs(x["q32"][l][:1], x["repre"][l][pad + 1 : pad + 5], np.array([0], np.int32),
+                                          np.array([4], np.int32), np.array([2], np.int32), cpu_twins.HKV, start_w=0, end_w=0)
+            assert np.array_equal(sc[l, pad + 1 : pad + 5].view(np.uint32), want[:4].view(np.uint32)), (key, l)
+    for ck, ik in (("cnt", "idx"), ("f_cnt", "f_idx")):
+        assert (got[ck][:, 0] == 2).all() and (got[ck][:, 1:] == 0).all(), ck
+        assert (got[ik][:, 1:] == -1).all(), ik
+    assert np.array_equal(got["idx"], got["f_idx"]) and not got["tickets"].any()
 
 
 def test_hash_twins_reproduce_the_oracle(ucm):
@@ -71,6 +96,8 @@ def test_hash_twins_reproduce_the_oracle(ucm):
                     assert np.array_equal(got["score_code"][l, a : a + n],
                                           O.hash_scores_block(got["qbar"][l, r], got["block_codes"][l, a : a + n]).astype(np.float32))
     assert np.array_equal(got["score_sum_fp16"], got["score_sum"].astype(np.float16).astype(np.float32))
+    # requests outside the declared rows were not scored; the empty one in between has nothing to score either way
+    assert (got["score_sum_bad"] == -3).all() and (got["score_code_bad"] == -3).all()
 
 
 def test_esa_twins_reproduce_the_oracle(ucm):
@@ -125,6 +152,11 @@ def test_selection_prefetch_and_load_twins_reproduce_the_oracle(ucm):
         assert got["chosen"][t, : len(want)].tolist() == sorted(want.tolist())
         assert got["ordered"][t, : len(want)].tolist() == want.tolist()
         assert (got["ordered"][t, len(want):] == -1).all()
+    # with the votes declared shorter and a task starting below them: those two select nothing, the others as before
+    assert got["chosen_count_bad"][0] == 0 and got["chosen_count_bad"][3] == 0
+    assert (got["ordered_bad"][[0, 3]] == -1).all()
+    for t in (1, 2, 4):
+        assert got["chosen_count_bad"][t] == got["chosen_count"][t] and np.array_equal(got["ordered_bad"][t], got["ordered"][t])
     assert np.array_equal(got["copied"], np.concatenate([np.arange(64), np.arange(128, 192), np.arange(64, 128)]).astype(np.uint8))
     # the prefetch round, request by request and layer by layer, against the oracle's single run
     P = cpu_twins
@@ -180,4 +212,10 @@ def test_kvstar_twins_reproduce_the_oracle(ucm):
                 assert np.array_equal(got[key][a : a + n].view(np.uint32), want.view(np.uint32)), (key, t)
                 assert abs(float(want.sum()) - K.K_X * K.K_HKV * K.K_G) < 1e-3          # every query row votes with weight one
     assert np.array_equal(got["votes"], got["votes_tables"])
+    # a task whose query block, channel list or rows lie outside what the call declares is skipped: its votes keep
+    # the fill value, the other tasks' are unchanged
+    a0, n0, a2, n2 = K.K_OFF[0], K.K_LEN[0], K.K_OFF[2], K.K_LEN[2]
+    assert (got["votes_bad0"][a2 : a2 + n2] == -3).all() and np.array_equal(got["votes_bad0"][a0 : a0 + n0], got["votes"][a0 : a0 + n0])
+    assert (got["votes_bad1"][a0 : a0 + n0] == -3).all() and np.array_equal(got["votes_bad1"][a2 : a2 + n2], got["votes"][a2 : a2 + n2])
+    assert (got["votes_bad2"][a2 : a2 + n2] == -3).all() and np.array_equal(got["votes_bad2"][a0 : a0 + n0], got["votes"][a0 : a0 + n0])
 

@@ -109,33 +109,29 @@ def test_hash_encode_persistent_waves_and_queue_overflow(ucm, dev, hkv, bs):
     ids_bad[[1, 6, 7, 13]] = [-1, nb, 1 << 30, nb + 5]      # skipped, never dereferenced
     slots_bad[[9, 20]] = [rows, -3]
     live = np.array([i for i in range(len(ids)) if 0 <= ids_bad[i] < nb and 0 <= slots_bad[i] < rows])
-    try:
-        for groups in (n_layers, 2 * n_layers, 0):
-            ops.set_hash_encode_groups(groups)
-            colsum = torch.full((n_layers, rows, hkv, 128), 77, dtype=torch.int16, device=dev)
-            bcodes = torch.full((n_layers, rows, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
-            tcodes = torch.full((n_layers, rows, bs, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
-            ops.hash_encode_blocks(lp, i32(ids_bad, dev), i32(slots_bad, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv,
-                                   nb, colsum, bcodes, token_codes=tcodes)
-            colsum2, bcodes2 = torch.full_like(colsum, 77), torch.full_like(bcodes, 0xEE)
-            ops.hash_encode_blocks(lp, i32(ids_bad, dev), i32(slots_bad, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv,
-                                   nb, colsum2, bcodes2)
-            torch.cuda.synchronize()
-            got_t, got_s, got_b = tcodes.cpu().numpy(), colsum.cpu().numpy(), bcodes.cpu().numpy()
-            assert torch.equal(colsum, colsum2) and torch.equal(bcodes, bcodes2), groups
-            for l in range(n_layers):
-                want_t = O.hash_encode(caches_h[l][ids_bad[live]], w_f32)
-                assert np.array_equal(got_t[l][slots_bad[live]], want_t), (groups, l)
-                assert np.array_equal(got_s[l][slots_bad[live]], O.hash_colsum(want_t)), (groups, l)
-                assert np.array_equal(got_b[l][slots_bad[live]], O.hash_majority(want_t)), (groups, l)
-                rest = np.setdiff1d(np.arange(rows), slots_bad[live])
-                assert np.all(got_t[l][rest] == 0xEE) and np.all(got_s[l][rest] == 77) and np.all(got_b[l][rest] == 0xEE)
-                # the construction did what it is for: the cancelling keys' codes follow sign(s * w[8][c])
-                k = list(live).index(len(ids) - 2)      # block 2, appended at the end of the list
-                sgn = synth.bf16_widen(caches_h[l][2, :, :, 8])[..., None] * w_f32[8][None, None, :] > 0
-                assert np.array_equal(np.unpackbits(want_t[k], axis=-1, bitorder="little").astype(bool), sgn)
-    finally:
-        ops.set_hash_encode_groups(0)
+    for groups in (n_layers, 2 * n_layers, 0):
+        colsum = torch.full((n_layers, rows, hkv, 128), 77, dtype=torch.int16, device=dev)
+        bcodes = torch.full((n_layers, rows, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+        tcodes = torch.full((n_layers, rows, bs, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+        ops.hash_encode_blocks(lp, i32(ids_bad, dev), i32(slots_bad, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv,
+                               nb, colsum, bcodes, token_codes=tcodes, workgroups=groups)
+        colsum2, bcodes2 = torch.full_like(colsum, 77), torch.full_like(bcodes, 0xEE)
+        ops.hash_encode_blocks(lp, i32(ids_bad, dev), i32(slots_bad, dev), len(ids), bf16_dev(w_bits, dev), bs, hkv,
+                               nb, colsum2, bcodes2, workgroups=groups)
+        torch.cuda.synchronize()
+        got_t, got_s, got_b = tcodes.cpu().numpy(), colsum.cpu().numpy(), bcodes.cpu().numpy()
+        assert torch.equal(colsum, colsum2) and torch.equal(bcodes, bcodes2), groups
+        for l in range(n_layers):
+            want_t = O.hash_encode(caches_h[l][ids_bad[live]], w_f32)
+            assert np.array_equal(got_t[l][slots_bad[live]], want_t), (groups, l)
+            assert np.array_equal(got_s[l][slots_bad[live]], O.hash_colsum(want_t)), (groups, l)
+            assert np.array_equal(got_b[l][slots_bad[live]], O.hash_majority(want_t)), (groups, l)
+            rest = np.setdiff1d(np.arange(rows), slots_bad[live])
+            assert np.all(got_t[l][rest] == 0xEE) and np.all(got_s[l][rest] == 77) and np.all(got_b[l][rest] == 0xEE)
+            # the construction did what it is for: the cancelling keys' codes follow sign(s * w[8][c])
+            k = list(live).index(len(ids) - 2)      # block 2, appended at the end of the list
+            sgn = synth.bf16_widen(caches_h[l][2, :, :, 8])[..., None] * w_f32[8][None, None, :] > 0
+            assert np.array_equal(np.unpackbits(want_t[k], axis=-1, bitorder="little").astype(bool), sgn)
 
 
 def test_config5_full_size_negated_keys_give_complement_codes(ucm, dev):

@@ -93,9 +93,10 @@ def test_block_mean_skips_bad_ids_and_layer_range(ucm, dev):
 # --------------------------------------------------------------- scoring
 
 def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=torch.float32, q_rows=None,
-               block_tables=None, seq_lens=None, block_size=128, repre_dtype=torch.float32):
+               block_tables=None, seq_lens=None, block_size=128, repre_dtype=torch.float32, tile=0):
     """q_np [L, rows, Hq, D] fp32 values; repre_np [L, rows, Hkv*D] (values that
-    repre_dtype holds exactly, so the oracle sees the same numbers)."""
+    repre_dtype holds exactly, so the oracle sees the same numbers).  Requests of up to 1024 blocks also go
+    through the one-launch entry point, whose every output must equal the two launches'."""
     n_layers = repre_np.shape[0]
     lens = np.asarray(lens, np.int32)
     off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
@@ -105,7 +106,7 @@ def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=to
     scores = torch.full((n_layers, repre_np.shape[1]), -123.0, device=dev)
     mx = int(lens.max(initial=0))
     ops.score_blocks(q, repre, i32(off, dev), i32(lens, dev), mx, hkv, scores,
-                     q_rows=None if q_rows is None else i32(q_rows, dev))
+                     q_rows=None if q_rows is None else i32(q_rows, dev), tile_blocks=tile)
     stride = max(mx, 1)
     idx = torch.full((n_layers, len(lens), stride), -1, dtype=torch.int32, device=dev)
     cnt = torch.full((n_layers, len(lens)), -1, dtype=torch.int32, device=dev)
@@ -126,6 +127,24 @@ def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=to
         out["phys"] = phys.cpu().numpy()
     if sps is not None:
         out["sparse_seq_lens"] = sps.cpu().numpy()
+    if mx <= 1024:
+        fused = dict(scores=torch.full_like(scores, -123.0), idx=torch.full_like(idx, -1), cnt=torch.full_like(cnt, -1),
+                     phys=None if phys is None else torch.full_like(phys, -1), sps=None if sps is None else torch.full_like(sps, -1))
+        tickets = torch.zeros_like(cnt)
+        for _ in range(2):                                   # twice: the tickets must come back to zero
+            ops.score_select(q, repre, i32(off, dev), i32(lens, dev), i32(topk, dev), mx, hkv, fused["scores"], fused["idx"],
+                             fused["cnt"], tickets, start_w=sw, end_w=ew, q_rows=None if q_rows is None else i32(q_rows, dev),
+                             block_tables=bt, phys_out=fused["phys"], seq_lens=sl, block_size=block_size,
+                             sparse_seq_lens=fused["sps"], tile_blocks=tile)
+            torch.cuda.synchronize()
+            assert not tickets.any(), "tickets left non-zero"
+        assert torch.equal(fused["scores"].view(torch.int32), scores.view(torch.int32)), "fused scores differ"
+        assert torch.equal(fused["cnt"], cnt), "fused counts differ"
+        assert torch.equal(fused["idx"], idx), "fused selection differs"
+        if phys is not None:
+            assert torch.equal(fused["phys"], phys), "fused block-table lookup differs"
+        if sps is not None:
+            assert torch.equal(fused["sps"], sps), "fused sparse lengths differ"
     return out
 
 
@@ -194,13 +213,9 @@ def test_bf16_table_scores_like_the_widened_table(ucm, dev, hkv, g, d, q_dtype):
     rows = int(np.sum(lens))
     q = synth.normal_bf16_as_f32(33, (n_layers, len(lens), hkv * g, d))
     repre = as_bf16_values(synth.normal_f32(34, (n_layers, rows, hkv * d)) * np.float32(0.3))
-    try:
-        for tile in (5, 32):
-            ops.set_score_tile(tile)
-            out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=q_dtype, repre_dtype=torch.bfloat16)
-            check_against_oracle(out, q, repre, lens, topk, hkv)
-    finally:
-        ops.set_score_tile(0)
+    for tile in (5, 32):
+        out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=q_dtype, repre_dtype=torch.bfloat16, tile=tile)
+        check_against_oracle(out, q, repre, lens, topk, hkv)
 
 
 @pytest.mark.parametrize("hkv,g,d,repre_dtype", [(8, 4, 128, torch.bfloat16), (2, 8, 64, torch.float32)])
@@ -265,13 +280,9 @@ def test_q_rows_indirection_and_tile_sizes(ucm, dev):
     q = synth.normal_bf16_as_f32(41, (2, 12, hkv * g, d))     # 12 token rows, requests read rows 11, 0, 5
     repre = synth.normal_f32(42, (2, int(np.sum(lens)), hkv * d))
     rows = [11, 0, 5]
-    try:
-        for tile in (1, 2, 7, 32, 4096):
-            ops.set_score_tile(tile)
-            out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=torch.bfloat16, q_rows=rows)
-            check_against_oracle(out, q, repre, lens, topk, hkv, q_rows=rows)
-    finally:
-        ops.set_score_tile(0)
+    for tile in (1, 2, 7, 32, 4096):
+        out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=torch.bfloat16, q_rows=rows, tile=tile)
+        check_against_oracle(out, q, repre, lens, topk, hkv, q_rows=rows)
 
 
 @pytest.mark.parametrize("repre_dtype", [torch.float32, torch.bfloat16])
@@ -316,20 +327,16 @@ def test_many_requests_dense_tile_lookup(ucm, dev):
     q = synth.normal_bf16_as_f32(46, (2, len(lens), hkv * g, d))
     repre = synth.normal_f32(47, (2, rows, hkv * d))
     off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
-    try:
-        for tile in (3, 32):
-            ops.set_score_tile(tile)
-            for total in (0, rows):
-                scores = torch.full((2, rows), -5.0, device=dev)
-                ops.score_blocks(torch.from_numpy(q).to(dev), torch.from_numpy(repre).to(dev), i32(off, dev),
-                                 i32(lens, dev), int(lens.max()), hkv, scores, total_blocks=total)
-                got = scores.cpu().numpy()
-                for l in range(2):
-                    _, _, want = O.select_topk_bs(q[l], repre[l], off, lens, topk, hkv)
-                    live = np.concatenate([np.arange(off[r], off[r] + lens[r]) for r in range(len(lens))])
-                    assert np.array_equal(bits(got[l][live]), bits(want[live])), (tile, total, l)
-    finally:
-        ops.set_score_tile(0)
+    for tile in (3, 32):
+        for total in (0, rows):
+            scores = torch.full((2, rows), -5.0, device=dev)
+            ops.score_blocks(torch.from_numpy(q).to(dev), torch.from_numpy(repre).to(dev), i32(off, dev),
+                             i32(lens, dev), int(lens.max()), hkv, scores, total_blocks=total, tile_blocks=tile)
+            got = scores.cpu().numpy()
+            for l in range(2):
+                _, _, want = O.select_topk_bs(q[l], repre[l], off, lens, topk, hkv)
+                live = np.concatenate([np.arange(off[r], off[r] + lens[r]) for r in range(len(lens))])
+                assert np.array_equal(bits(got[l][live]), bits(want[live])), (tile, total, l)
 
 
 def test_config1_single_request_32k(ucm, dev):
@@ -849,7 +856,8 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     import cpu_twins
     from ucm_amd import _lib, ops
 
-    for run in (cpu_twins.run, cpu_twins.run_hash, cpu_twins.run_esa, cpu_twins.run_more):   # the dense path; hash codes; the ESA worker; KVStar's selection, prefetch round, planned loads
+    # the dense path; descriptors outside the tables; hash codes; the ESA worker; KVStar's selection, prefetch round, planned loads
+    for run in (cpu_twins.run, cpu_twins.run_bounds, cpu_twins.run_hash, cpu_twins.run_esa, cpu_twins.run_more):
         want, _ = run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
         got, _ = run(_lib.call, cpu_twins.DeviceSide(ops, dev))
         assert got.keys() == want.keys()
@@ -861,5 +869,6 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     got, _ = cpu_twins.run_kvstar(_lib.call, cpu_twins.DeviceSide(ops, dev))
     for name in ("table_full", "table_pruned"):
         assert np.array_equal(got[name], want[name]), name
-    for name in ("votes", "votes_tables"):
+    for name in ("votes", "votes_tables", "votes_bad0", "votes_bad1", "votes_bad2"):
         assert np.allclose(got[name], want[name], rtol=2e-4, atol=2e-6), name
+        assert np.array_equal(got[name] == -3, want[name] == -3), name        # the same tasks were skipped

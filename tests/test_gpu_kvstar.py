@@ -95,7 +95,8 @@ def test_kvstar_block_repre_channel_lists_per_layer(ucm, dev, merge):
                                bs, hkv, d, nb, merge, pruned=torch.from_numpy(pruned[:2]).to(dev))
 
 
-def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None, pruned_sel=None, d_pruned=None, layout="head"):
+def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None, pruned_sel=None, d_pruned=None, layout="head",
+              tiles_per_wave=0):
     """q_bits_list: per task uint16 [x, hq, d]; repre_bits uint16 [rows, M, hkv, d_pad]; tasks own consecutive row ranges."""
     lens = np.asarray(lens, np.int32)
     off = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
@@ -105,11 +106,13 @@ def run_votes(ops, dev, q_bits_list, repre_bits, lens, n_tokens, hq, pruned=None
     table = ops.kvstar_table_from_reference(dev_f16(repre_bits, dev), layout)         # indexed [h, rows, d_pad/8, M, 8]
     assert torch.equal(ops.kvstar_table_to_reference(table), dev_f16(repre_bits, dev))
     votes = torch.full((rows,), -7.0, device=dev)
-    ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, table.shape[2] * 8, dev)
+    ws = ops.kvstar_workspace(len(lens), hkv, n_tokens * (hq // hkv), int(lens.max(initial=0)), M, table.shape[2] * 8, dev,
+                              tiles_per_wave=tiles_per_wave)
     ops.kvstar_votes(q, q_off, n_tokens, hq, table, torch.from_numpy(off).to(dev), torch.from_numpy(lens).to(dev),
                      int(lens.max(initial=0)), votes, ws, d_pruned=d_pruned,
                      pruned=None if pruned is None else torch.from_numpy(pruned).to(dev),
-                     pruned_sel=None if pruned_sel is None else torch.tensor(pruned_sel, dtype=torch.int32, device=dev))
+                     pruned_sel=None if pruned_sel is None else torch.tensor(pruned_sel, dtype=torch.int32, device=dev),
+                     tiles_per_wave=tiles_per_wave)
     torch.cuda.synchronize()
     return votes.cpu().numpy(), off
 
@@ -127,19 +130,15 @@ def test_kvstar_votes_match_oracle(ucm, dev, x, hq, hkv, d, M):
     qs = [f16_bits(synth.normal_f32(1101 + t, (x, hq, d)) * scale) for t in range(len(lens))]
     wants = {t: O.kvstar_retrieve(qs[t], repre[sum(lens[:t]) : sum(lens[:t]) + n], topk=max(n // 3, 1))[1]
              for t, n in enumerate(lens) if n}
-    try:
-        # 0: automatic, -1: per-task plane in LDS, n: chunks of 4n tiles; table rows of kv_heads cells, or head planes
-        for tiles_per_wave, layout in ((0, "row"), (-1, "row"), (1, "row"), (3, "row"), (0, "head"), (-1, "head"), (3, "head")):
-            ops.set_kvstar_tiles_per_wave(tiles_per_wave)
-            got, off = run_votes(ops, dev, qs, repre, lens, x, hq, layout=layout)
-            for t, n in enumerate(lens):
-                if n == 0:
-                    continue
-                assert np.allclose(got[off[t] : off[t] + n], wants[t], rtol=VOTE_RTOL, atol=VOTE_ATOL), (tiles_per_wave, t, n)
-                # what the mathematics fixes whatever the order: every row's probabilities add up to one
-                assert abs(got[off[t] : off[t] + n].sum() - x * hq) < 1e-3 * x * hq
-    finally:
-        ops.set_kvstar_tiles_per_wave(0)
+    # 0: automatic, -1: per-task plane in LDS, n: chunks of 4n tiles; table rows of kv_heads cells, or head planes
+    for tiles_per_wave, layout in ((0, "row"), (-1, "row"), (1, "row"), (3, "row"), (0, "head"), (-1, "head"), (3, "head")):
+        got, off = run_votes(ops, dev, qs, repre, lens, x, hq, layout=layout, tiles_per_wave=tiles_per_wave)
+        for t, n in enumerate(lens):
+            if n == 0:
+                continue
+            assert np.allclose(got[off[t] : off[t] + n], wants[t], rtol=VOTE_RTOL, atol=VOTE_ATOL), (tiles_per_wave, t, n)
+            # what the mathematics fixes whatever the order: every row's probabilities add up to one
+            assert abs(got[off[t] : off[t] + n].sum() - x * hq) < 1e-3 * x * hq
 
 
 def test_kvstar_many_short_tasks_take_the_in_lds_path(ucm, dev):
@@ -177,17 +176,13 @@ def test_kvstar_scores_drifting_far_from_the_first_span(ucm, dev, d, M, slope):
     repre = f16_bits(base * np.float32(2.0 / d) + noise)                                    # times q = 0.5: score = level + noise
     qs = [f16_bits(np.full((x, hq, d), 0.5, dtype=np.float32) + synth.normal_f32(1171 + t, (x, hq, d)) * np.float32(0.03125))
           for t in range(2)]
-    try:
-        for tiles_per_wave in (-1, 3):
-            ops.set_kvstar_tiles_per_wave(tiles_per_wave)
-            got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
-            for t, m in enumerate(lens):
-                want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + m], topk=1)[1]
-                assert np.isfinite(got[off[t] : off[t] + m]).all()
-                assert np.allclose(got[off[t] : off[t] + m], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (tiles_per_wave, t)
-                assert abs(got[off[t] : off[t] + m].sum() - x * hq) < 1e-3 * x * hq
-    finally:
-        ops.set_kvstar_tiles_per_wave(0)
+    for tiles_per_wave in (-1, 3):
+        got, off = run_votes(ops, dev, qs, repre, lens, x, hq, tiles_per_wave=tiles_per_wave)
+        for t, m in enumerate(lens):
+            want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + m], topk=1)[1]
+            assert np.isfinite(got[off[t] : off[t] + m]).all()
+            assert np.allclose(got[off[t] : off[t] + m], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (tiles_per_wave, t)
+            assert abs(got[off[t] : off[t] + m].sum() - x * hq) < 1e-3 * x * hq
 
 
 @pytest.mark.parametrize("M,d", [(64, 32), (8, 128)])
@@ -243,13 +238,9 @@ def test_kvstar_workspace_sized_for_another_path_is_refused(ucm, dev):
     seg_len = torch.full((n_tasks,), blocks, dtype=torch.int32, device=dev)
     votes = torch.zeros(n_tasks * blocks, device=dev)
     ws = ops.kvstar_workspace(n_tasks, hkv, x * hq // hkv, blocks, M, d, dev)      # 256 (task, kv head) pairs: the in-LDS path
-    try:
-        ops.set_kvstar_tiles_per_wave(3)
-        with pytest.raises(_lib.UcmHipError) as e:
-            ops.kvstar_votes(q, q_off, x, hq, table, seg_off, seg_len, blocks, votes, ws)
-        assert e.value.code == _lib.EINVAL and "workspace" in str(e.value)
-    finally:
-        ops.set_kvstar_tiles_per_wave(0)
+    with pytest.raises(_lib.UcmHipError) as e:
+        ops.kvstar_votes(q, q_off, x, hq, table, seg_off, seg_len, blocks, votes, ws, tiles_per_wave=3)
+    assert e.value.code == _lib.EINVAL and "workspace" in str(e.value)
     ops.kvstar_votes(q, q_off, x, hq, table, seg_off, seg_len, blocks, votes, ws)  # the path it was sized for
     torch.cuda.synchronize()
     assert np.allclose(votes.cpu().numpy(), x * hq / blocks, rtol=1e-5)            # all-zero scores: uniform votes
@@ -266,11 +257,7 @@ def test_kvstar_long_task_plane_in_lds_or_not(ucm, dev, longest):
     rows = int(np.sum(lens))
     repre = f16_bits(synth.normal_f32(1160, (rows, M, hkv, d)) * np.float32(0.25))
     qs = [f16_bits(synth.normal_f32(1161 + t, (x, hq, d)) * np.float32(0.25)) for t in range(2)]
-    ops.set_kvstar_tiles_per_wave(-1)
-    try:
-        got, off = run_votes(ops, dev, qs, repre, lens, x, hq)
-    finally:
-        ops.set_kvstar_tiles_per_wave(0)
+    got, off = run_votes(ops, dev, qs, repre, lens, x, hq, tiles_per_wave=-1)
     for t, n in enumerate(lens):
         want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=1)[1]
         assert np.allclose(got[off[t] : off[t] + n], want, rtol=VOTE_RTOL, atol=VOTE_ATOL), (t, n)
@@ -281,14 +268,10 @@ def test_kvstar_long_task_plane_in_lds_or_not(ucm, dev, longest):
 def test_kvstar_pruned_channels_and_selection(ucm, dev, tiles_per_wave, M, dp):
     from ucm_amd import ops
 
-    ops.set_kvstar_tiles_per_wave(tiles_per_wave)
-    try:
-        _pruned_channels_and_selection(ops, dev, M, dp)
-    finally:
-        ops.set_kvstar_tiles_per_wave(0)
+    _pruned_channels_and_selection(ops, dev, M, dp, tiles_per_wave)
 
 
-def _pruned_channels_and_selection(ops, dev, M, dp):
+def _pruned_channels_and_selection(ops, dev, M, dp, tiles_per_wave):
 
     x, hq, hkv, d = 8, 32, 8, 128
     lens = [90, 33]
@@ -298,7 +281,7 @@ def _pruned_channels_and_selection(ops, dev, M, dp):
     repre = np.zeros((rows, M, hkv, d_pad), np.uint16)
     repre[..., :dp] = f16_bits(synth.normal_f32(1201, (rows, M, hkv, dp)) * np.float32(0.3))
     qs = [f16_bits(synth.normal_f32(1202 + t, (x, hq, d)) * np.float32(0.3)) for t in range(2)]
-    got, off = run_votes(ops, dev, qs, repre, lens, x, hq, pruned=pruned, pruned_sel=[1, 0])
+    got, off = run_votes(ops, dev, qs, repre, lens, x, hq, pruned=pruned, pruned_sel=[1, 0], tiles_per_wave=tiles_per_wave)
     for t, n in enumerate(lens):
         sel = [1, 0][t]
         idx, want = O.kvstar_retrieve(qs[t], repre[off[t] : off[t] + n], topk=n // 4, pruned=pruned[sel])

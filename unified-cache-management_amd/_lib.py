@@ -8,7 +8,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libucm_hip.so")
 
 OK, EINVAL, ENOTSUP, EHIP, ENOMEM = 0, -22, -95, -5, -12
-DTYPE_F32, DTYPE_BF16 = 0, 1
+DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 MEAN_F32, MEAN_BF16_ROUND, MEAN_BF16_STORE = 0, 1, 2
 MEAN_ABS = 4        # or-ed to a mode: the mean of the absolute values
 
@@ -19,14 +19,15 @@ SIGNATURES = {
     "ucm_version": [],
     "ucm_last_error": [],
     "ucm_block_mean": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i64, _i, _p],
-    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _f, _i, _p],
+    "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _i64, _i, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _f, _i, _p],
+    "ucm_score_select": [_p, _p],
     "ucm_kvstar_block_repre": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _i, _p, _i64, _i, _i, _p, _i, _i64, _i64, _i64, _p],
     "ucm_kvstar_workspace_floats": [_i, _i, _i, _i, _i, _i, _i, _p, _p],
-    "ucm_kvstar_votes": [_p, _p, _i, _i, _i, _p, _p, _p, _i64, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
-    "ucm_kvstar_votes_tables": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
-    "ucm_kvstar_topk": [_p, _p, _p, _p, _i, _i, _p, _i, _p, _p],
-    "ucm_kvstar_order": [_p, _p, _p, _i, _i, _p, _i, _p, _p],
-    "ucm_topk_windows": [_p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
+    "ucm_kvstar_votes": [_p, _i64, _p, _i, _i, _i, _p, _i, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],
+    "ucm_kvstar_votes_tables": [_p, _i64, _p, _i, _i, _i, _p, _i, _p, _p, _p, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i64, _i, _p],
+    "ucm_kvstar_topk": [_p, _i64, _p, _p, _p, _i, _i, _p, _i, _p, _p],
+    "ucm_kvstar_order": [_p, _i64, _p, _p, _i, _i, _p, _i, _p, _p],
+    "ucm_topk_windows": [_p, _i64, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _i, _p, _p, _i, _p, _p],
     "ucm_esa_retrieve": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _p, _i, _p],
     "ucm_esa_retrieve_static": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _p, _p, _i, _p],
     "ucm_esa_retrieve_rows": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _i, _p, _i, _p, _p, _p, _p, _p, _i, _p],
@@ -36,7 +37,7 @@ SIGNATURES = {
     "ucm_delta_plan": [_p, _p, _p, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _i, _p],
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
-    "ucm_hash_score_blocks": [_i, _p, _p, _p, _i64, _p, _i64, _p, _p, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
+    "ucm_hash_score_blocks": [_i, _p, _p, _p, _i64, _p, _i64, _i64, _p, _p, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
     "ucm_copy_batch": [_p, _p, _sz, _sz, _p],
     "ucm_kernel_can_access": [_p, _sz],
     "ucm_device_create": [_i, _sz, _sz, _p],
@@ -68,6 +69,23 @@ RESTYPES = {
 }
 
 DEVICE_CALLBACK = C.CFUNCTYPE(None, C.c_int, C.c_void_p)
+
+
+class ScoreSelectArgs(C.Structure):
+    """ucm_score_select_args_t (include/ucm_hip.h), field for field."""
+    _fields_ = [
+        ("struct_size", _sz), ("q", _p), ("q_dtype", _i), ("q_heads", _i), ("q_layer_stride", _i64), ("q_rows", _p),
+        ("repre", _p), ("repre_dtype", _i), ("num_repre", _i), ("repre_layer_stride", _i64), ("repre_rows", _i64),
+        ("seg_off", _p), ("seg_len", _p), ("topk_len", _p), ("n_req", _i), ("max_seg_len", _i), ("first_layer", _i),
+        ("n_layers", _i), ("kv_heads", _i), ("head_dim", _i), ("scores", _p), ("scores_layer_stride", _i64),
+        ("scale", _f), ("tile_blocks", _i), ("start_w", _i), ("end_w", _i), ("idx_out", _p), ("count_out", _p),
+        ("out_stride", _i), ("bt_stride", _i), ("block_tables", _p), ("phys_out", _p), ("seq_lens", _p),
+        ("sparse_seq_lens", _p), ("block_size", _i), ("reserved", _i), ("tickets", _p),
+        ("idx_layer_stride", _i64), ("count_layer_stride", _i64),
+    ]
+
+    def __init__(self, **kw):
+        super().__init__(struct_size=C.sizeof(ScoreSelectArgs), num_repre=1, scale=1.0, n_layers=1, **kw)
 
 
 class UcmHipError(RuntimeError):

@@ -856,6 +856,14 @@ __device__ __forceinline__ float half_round(float x)
 
 typedef short i16x8 __attribute__((ext_vector_type(8)));
 
+// Blocks of a request whose rows lie inside the summary tables; a request outside them (its descriptors live in
+// device memory, where the host cannot check them) counts none and is not scored.
+__device__ __forceinline__ int seg_blocks(int off, int len, int64_t rows)
+{
+    const int n = max(len, 0);
+    return off >= 0 && static_cast<int64_t>(off) + n <= rows ? n : 0;
+}
+
 // Integer block scores <sum_i u(q_i), sum_h S[h]>.  Sixteen lanes share one block:
 // lane j owns bits 8j..8j+7 of the 128-entry column-sum row (one 16-byte load per
 // kv head, 256 contiguous bytes per 16 lanes); a 16-lane shuffle reduction adds
@@ -865,14 +873,14 @@ typedef short i16x8 __attribute__((ext_vector_type(8)));
 __global__ __launch_bounds__(256) void hash_score_kernel(
     const short* __restrict__ q_sum, const short* __restrict__ colsum, int64_t cs_layer_stride,
     const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
-    unsigned n_req, unsigned kv_heads, float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16)
+    unsigned n_req, unsigned kv_heads, float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16, int64_t rows)
 {
     const unsigned l = blockIdx.y;
     const unsigned sub = threadIdx.x & 15;
     int dense = blockIdx.x * 16 + (threadIdx.x >> 4);
     int r = -1, local = 0;
     for (unsigned i = 0; i < n_req; ++i) {
-        const int n = max(seg_len[i], 0);
+        const int n = seg_blocks(seg_off[i], seg_len[i], rows);
         if (dense < n) { r = static_cast<int>(i); local = dense; break; }
         dense -= n;
     }
@@ -915,7 +923,7 @@ constexpr int kCodeBlocksPerGroup = 128;
 __global__ __launch_bounds__(256) void hash_code_score_kernel(
     const unsigned* __restrict__ qbar_codes, const unsigned* __restrict__ block_codes, int64_t bc_layer_stride,
     const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len, unsigned n_req, unsigned kv_heads,
-    float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16)
+    float* __restrict__ scores, int64_t scores_layer_stride, int round_fp16, int64_t rows)
 {
     const unsigned l = blockIdx.y, h = threadIdx.x & 7;
     int req[4];
@@ -925,7 +933,7 @@ __global__ __launch_bounds__(256) void hash_code_score_kernel(
     const int first = blockIdx.x * kCodeBlocksPerGroup + (threadIdx.x >> 3);
     int base = 0;
     for (unsigned i = 0; i < n_req; ++i) {
-        const int n = max(seg_len[i], 0), off = seg_off[i];
+        const int off = seg_off[i], n = seg_blocks(off, seg_len[i], rows);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int dense = first + 32 * u;
@@ -1026,12 +1034,14 @@ extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_strid
 extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_codes,
                                      const int16_t* colsum, int64_t colsum_layer_stride,
                                      const uint8_t* block_codes, int64_t block_codes_layer_stride,
-                                     const int32_t* seg_off, const int32_t* seg_len, int n_req,
+                                     int64_t rows, const int32_t* seg_off, const int32_t* seg_len, int n_req,
                                      int64_t total_blocks, int n_layers, int kv_heads, int bits, float* scores,
                                      int64_t scores_layer_stride, int round_fp16, ucm_stream_t stream)
 {
-    UCM_REQUIRE(n_req >= 0 && total_blocks >= 0 && n_layers > 0 && n_layers <= 65535,
-                "ucm_hash_score_blocks: n_req=%d n_layers=%d", n_req, n_layers);
+    UCM_REQUIRE(n_req >= 0 && total_blocks >= 0 && n_layers > 0 && n_layers <= 65535 && rows >= 0,
+                "ucm_hash_score_blocks: n_req=%d n_layers=%d rows=%lld", n_req, n_layers, static_cast<long long>(rows));
+    UCM_REQUIRE(n_layers == 1 || scores_layer_stride >= rows, "ucm_hash_score_blocks: scores_layer_stride=%lld < rows=%lld",
+                static_cast<long long>(scores_layer_stride), static_cast<long long>(rows));
     if (n_req == 0 || total_blocks == 0) { return UCM_OK; }
     UCM_REQUIRE(mode == 0 || mode == 1, "ucm_hash_score_blocks: mode=%d", mode);
     UCM_REQUIRE(seg_off && seg_len && scores, "ucm_hash_score_blocks: null pointer");
@@ -1042,7 +1052,7 @@ extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8
     if (mode == 0) {
         hipLaunchKernelGGL(hash_score_kernel, dim3(gx, n_layers), dim3(256), 0, s, q_sum, colsum, colsum_layer_stride,
                            seg_off, seg_len, static_cast<unsigned>(n_req), static_cast<unsigned>(kv_heads), scores,
-                           scores_layer_stride, round_fp16);
+                           scores_layer_stride, round_fp16, rows);
     } else {
         UCM_REQUIRE(ucm::aligned16(qbar_codes) && ucm::aligned16(block_codes) && block_codes_layer_stride % 16 == 0,
                     "ucm_hash_score_blocks: codes must be 16-byte aligned");
@@ -1050,7 +1060,7 @@ extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8
         hipLaunchKernelGGL(hash_code_score_kernel, dim3(gc, n_layers), dim3(256), 0, s,
                            reinterpret_cast<const unsigned*>(qbar_codes), reinterpret_cast<const unsigned*>(block_codes),
                            block_codes_layer_stride / 4, seg_off, seg_len, static_cast<unsigned>(n_req),
-                           static_cast<unsigned>(kv_heads), scores, scores_layer_stride, round_fp16);
+                           static_cast<unsigned>(kv_heads), scores, scores_layer_stride, round_fp16, rows);
     }
     UCM_LAUNCH_CHECK("ucm_hash_score_blocks");
 }

@@ -436,6 +436,27 @@ __device__ __forceinline__ float block_sums(const float (&e)[16], int half, Put 
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// What bounds the descriptors a task brings in device memory: its rows inside the table / the votes array, its
+// query block inside the query buffer, its channel list inside the lists.  A task outside any of them counts
+// zero blocks in every kernel of the call, so none of its descriptors is followed and its votes stay as they were.
+struct TaskBounds {
+    int64_t rows_bound;     // rows of the shared table (ucm_kvstar_votes) and entries of `votes`
+    int64_t q_elems;        // fp16 elements the query buffer holds
+    int64_t q_need;         // elements a task reads from q_off[task] on: n_tokens * q_heads * d_orig
+    int n_lists;            // channel lists in `pruned`
+};
+
+__device__ __forceinline__ unsigned task_blocks(const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
+                                                const int64_t* __restrict__ q_off, const int32_t* __restrict__ pruned_sel,
+                                                unsigned task, unsigned max_blocks, const TaskBounds& tb)
+{
+    const int n = min(max(seg_len[task], 0), static_cast<int>(max_blocks));   // the planes are sized for max_blocks
+    const int64_t so = seg_off[task], qo = q_off[task];
+    const bool ok = so >= 0 && so + n <= tb.rows_bound && qo >= 0 && qo + tb.q_need <= tb.q_elems &&
+                    (!pruned_sel || pruned_sel[task] < tb.n_lists);
+    return ok ? static_cast<unsigned>(n) : 0u;
+}
+
 // grid: x = chunk of sub-blocks, y = kv head, z = task.  The table is head-major and piece-interleaved
 // inside a block (see above), so what one workgroup streams is one contiguous run read in whole lines
 // (in the reference's [row][sub-block][kv head][d] order each vector of a head sits kv_heads*d*2 bytes
@@ -464,7 +485,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     const int64_t* __restrict__ task_head_strides, const int32_t* __restrict__ seg_off,
     const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned d_pruned, unsigned d_pad, int64_t head_stride,
     int64_t row_stride, float* __restrict__ ws_max, float* __restrict__ ws_part, unsigned max_blocks, unsigned max_tiles,
-    unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset, unsigned q_full_ok)
+    unsigned spans_per_wave, unsigned row_pad, unsigned plane_offset, unsigned q_full_ok, const TaskBounds tb)
 {
     static_assert(kM >= 1 && kM <= 128 && (kM & (kM - 1)) == 0, "sub-blocks per block");
     static_assert(kSteps == 2 || kSteps == 4 || kSteps == 8, "MFMA steps per vector");
@@ -485,7 +506,7 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
     float* plane = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(q_s) + plane_offset);
 
     const unsigned task = blockIdx.z, h = blockIdx.y;
-    const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);   // the planes are sized for max_blocks
+    const unsigned n_blocks = task_blocks(seg_off, seg_len, q_off, pruned_sel, task, max_blocks, tb);
     const unsigned S = n_blocks * kM;
     const unsigned chunk = kWaves * spans_per_wave * kSpan;
     const unsigned s_chunk = blockIdx.x * chunk;
@@ -814,10 +835,11 @@ __global__ __launch_bounds__(kThreads, 2) void kvstar_score_kernel(
 // kLds path, grid: x = 256 blocks of the task, y = task: adds up the kv heads' shares of the votes.
 __global__ __launch_bounds__(kThreads) void kvstar_headsum_kernel(
     const float* __restrict__ head_votes, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
+    const int64_t* __restrict__ q_off, const int32_t* __restrict__ pruned_sel, const TaskBounds tb,
     unsigned kv_heads, unsigned max_blocks, float* __restrict__ votes)
 {
     const unsigned task = blockIdx.y, b = blockIdx.x * kThreads + threadIdx.x;
-    if (b >= min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks)) { return; }
+    if (b >= task_blocks(seg_off, seg_len, q_off, pruned_sel, task, max_blocks, tb)) { return; }
     float v = 0.0f;
     for (unsigned h = 0; h < kv_heads; ++h) { v += head_votes[(static_cast<size_t>(task) * kv_heads + h) * max_blocks + b]; }
     votes[seg_off[task] + b] = v;
@@ -834,12 +856,13 @@ __global__ __launch_bounds__(kThreads) void kvstar_headsum_kernel(
 // exp(tile reference - largest reference) / denominator the tile's partial sums have to be multiplied
 // with.  Rows past tokens*group hold zero queries and are carried along.
 __global__ __launch_bounds__(kThreads) void kvstar_rowscale_kernel(
-    float* __restrict__ ws_max, const int32_t* __restrict__ seg_len, unsigned kv_heads, unsigned M, unsigned max_blocks,
-    unsigned max_tiles, unsigned row_pad)
+    float* __restrict__ ws_max, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
+    const int64_t* __restrict__ q_off, const int32_t* __restrict__ pruned_sel, const TaskBounds tb, unsigned kv_heads,
+    unsigned M, unsigned max_blocks, unsigned max_tiles, unsigned row_pad)
 {
     __shared__ float red[kThreads];
     const unsigned task = blockIdx.y, h = blockIdx.x;
-    const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);
+    const unsigned n_blocks = task_blocks(seg_off, seg_len, q_off, pruned_sel, task, max_blocks, tb);
     if (n_blocks == 0) { return; }
     const unsigned n_tiles = (n_blocks * M + kTileSub - 1) / kTileSub;
     const unsigned rho = threadIdx.x % row_pad, grp = threadIdx.x / row_pad, ngrp = kThreads / row_pad;
@@ -888,12 +911,13 @@ __global__ __launch_bounds__(kThreads) void kvstar_rowscale_kernel(
 // rows of partial * factor.
 __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
     const float* __restrict__ ws_max, const float* __restrict__ ws_part, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, unsigned R, unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles,
+    const int32_t* __restrict__ seg_len, const int64_t* __restrict__ q_off, const int32_t* __restrict__ pruned_sel,
+    const TaskBounds tb, unsigned R, unsigned kv_heads, unsigned M, unsigned max_blocks, unsigned max_tiles,
     unsigned row_pad, float* __restrict__ votes)
 {
     constexpr unsigned kMaxHeads = 8;
     const unsigned task = blockIdx.y;
-    const unsigned n_blocks = min(static_cast<unsigned>(max(seg_len[task], 0)), max_blocks);
+    const unsigned n_blocks = task_blocks(seg_off, seg_len, q_off, pruned_sel, task, max_blocks, tb);
     if (blockIdx.x * 8 >= n_blocks) { return; }
     const unsigned b = min(blockIdx.x * 8 + (threadIdx.x >> 5), n_blocks - 1), l32 = threadIdx.x & 31;
     const bool live = blockIdx.x * 8 + (threadIdx.x >> 5) < n_blocks;
@@ -1075,13 +1099,15 @@ extern "C" int ucm_kvstar_workspace_floats(int n_tasks, int kv_heads, int rows_p
 }
 
 namespace {
-int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig, const int32_t* pruned,
-                 const int32_t* pruned_sel, const void* repre_f16, int64_t repre_head_stride, int64_t repre_row_stride,
+int kvstar_votes(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
+                 const int32_t* pruned, int n_lists, const int32_t* pruned_sel, int64_t rows_bound, const void* repre_f16, int64_t repre_head_stride, int64_t repre_row_stride,
                  const void* const* task_tables, const int64_t* task_head_strides, const int32_t* seg_off, const int32_t* seg_len, int n_tasks, int max_blocks,
                  int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max, int64_t ws_max_floats, float* ws_part,
                  int64_t ws_part_floats, float* votes, int tiles_per_wave, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks >= 0 && max_blocks >= 0, "ucm_kvstar_votes: n_tasks=%d max_blocks=%d", n_tasks, max_blocks);
+    UCM_REQUIRE(q_elems >= 0 && rows_bound >= 0 && n_lists >= 0, "ucm_kvstar_votes: q_elems=%lld rows=%lld n_lists=%d",
+                static_cast<long long>(q_elems), static_cast<long long>(rows_bound), n_lists);
     UCM_REQUIRE(tiles_per_wave >= -1, "ucm_kvstar_votes: tiles_per_wave=%d", tiles_per_wave);
     if (n_tasks == 0 || max_blocks == 0) { return UCM_OK; }
     UCM_REQUIRE(q_f16 && q_off && seg_off && seg_len && ws_max && ws_part && votes, "ucm_kvstar_votes: null pointer");
@@ -1134,12 +1160,13 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
                                         : std::max(1u, (spans_per_wg_all + want_chunks - 1) / want_chunks);
     const unsigned chunks = (max_spans + kWaves * spans_per_wave - 1) / (kWaves * spans_per_wave);
     hipStream_t s = ucm::as_stream(stream);
+    const TaskBounds tb = {rows_bound, q_elems, static_cast<int64_t>(n_tokens) * q_heads * d_orig, n_lists};
 #define UCM_KVSTAR_ARGS dim3(chunks, kv_heads, n_tasks), dim3(kThreads), lds_bytes, s, static_cast<const unsigned short*>(q_f16), q_off, \
         static_cast<unsigned>(n_tokens), static_cast<unsigned>(q_heads), static_cast<unsigned>(d_orig), pruned, pruned_sel,   \
         static_cast<const unsigned short*>(repre_f16), task_tables, task_head_strides, seg_off, seg_len,                      \
         static_cast<unsigned>(kv_heads),                                                                                      \
         static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad), repre_head_stride, repre_row_stride, ws_max, ws_part, \
-        static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset, q_full_ok
+        static_cast<unsigned>(max_blocks), max_tiles, spans_per_wave, row_pad, plane_offset, q_full_ok, tb
 #define UCM_KVSTAR_LAUNCH4(M, STEPS, TWO, LDS)                                                                        \
     do {                                                                                                             \
         if (lds_bytes > 48u * 1024u) {                                                                               \
@@ -1181,40 +1208,43 @@ int kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_he
     if (hipError_t e = hipGetLastError(); e != hipSuccess) { return ucm::check_hip(e, "ucm_kvstar_votes (scores)"); }
     if (use_lds) {
         hipLaunchKernelGGL(kvstar_headsum_kernel, dim3((max_blocks + kThreads - 1) / kThreads, n_tasks), dim3(kThreads), 0, s,
-                           ws_part, seg_off, seg_len, static_cast<unsigned>(kv_heads), static_cast<unsigned>(max_blocks), votes);
+                           ws_part, seg_off, seg_len, q_off, pruned_sel, tb, static_cast<unsigned>(kv_heads),
+                           static_cast<unsigned>(max_blocks), votes);
     } else {
         hipLaunchKernelGGL(kvstar_rowscale_kernel, dim3(static_cast<unsigned>(kv_heads), n_tasks), dim3(kThreads), 0, s, ws_max,
-                           seg_len, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
+                           seg_off, seg_len, q_off, pruned_sel, tb, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
                            static_cast<unsigned>(max_blocks), max_tiles, row_pad);
         hipLaunchKernelGGL(kvstar_vote_kernel, dim3((max_blocks + 7) / 8, n_tasks), dim3(kThreads), 0, s, ws_max, ws_part,
-                           seg_off, seg_len, R, static_cast<unsigned>(kv_heads), static_cast<unsigned>(sub_blocks),
-                           static_cast<unsigned>(max_blocks), max_tiles, row_pad, votes);
+                           seg_off, seg_len, q_off, pruned_sel, tb, R, static_cast<unsigned>(kv_heads),
+                           static_cast<unsigned>(sub_blocks), static_cast<unsigned>(max_blocks), max_tiles, row_pad, votes);
     }
     UCM_LAUNCH_CHECK("ucm_kvstar_votes");
 }
 }  // namespace
 
-extern "C" int ucm_kvstar_votes(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
-                                const int32_t* pruned, const int32_t* pruned_sel, const void* repre_f16,
-                                int64_t repre_head_stride, int64_t repre_row_stride, const int32_t* seg_off,
-                                const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+extern "C" int ucm_kvstar_votes(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads,
+                                int d_orig, const int32_t* pruned, int n_pruned_lists, const int32_t* pruned_sel,
+                                const void* repre_f16, int64_t repre_rows, int64_t repre_head_stride,
+                                int64_t repre_row_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                                int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
                                 int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
                                 int tiles_per_wave, ucm_stream_t stream)
 {
-    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, repre_f16, repre_head_stride, repre_row_stride,
-                        nullptr, nullptr, seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
-                        ws_part_floats, votes, tiles_per_wave, stream);
+    return kvstar_votes(q_f16, q_elems, q_off, n_tokens, q_heads, d_orig, pruned, n_pruned_lists, pruned_sel, repre_rows, repre_f16,
+                        repre_head_stride, repre_row_stride, nullptr, nullptr, seg_off, seg_len, n_tasks, max_blocks, sub_blocks,
+                        kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part, ws_part_floats, votes, tiles_per_wave, stream);
 }
 
-extern "C" int ucm_kvstar_votes_tables(const void* q_f16, const int64_t* q_off, int n_tokens, int q_heads, int d_orig,
-                                       const int32_t* pruned, const int32_t* pruned_sel, const void* const* task_tables,
-                                       const int64_t* task_head_strides, int64_t task_row_stride, const int32_t* seg_off,
-                                       const int32_t* seg_len, int n_tasks, int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad,
-                                       float* ws_max, int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats,
-                                       float* votes, int tiles_per_wave, ucm_stream_t stream)
+extern "C" int ucm_kvstar_votes_tables(const void* q_f16, int64_t q_elems, const int64_t* q_off, int n_tokens, int q_heads,
+                                       int d_orig, const int32_t* pruned, int n_pruned_lists, const int32_t* pruned_sel,
+                                       const void* const* task_tables, const int64_t* task_head_strides,
+                                       int64_t task_row_stride, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
+                                       int max_blocks, int sub_blocks, int kv_heads, int d_pruned, int d_pad, float* ws_max,
+                                       int64_t ws_max_floats, float* ws_part, int64_t ws_part_floats, float* votes,
+                                       int64_t votes_rows, int tiles_per_wave, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_tasks == 0 || (task_tables && task_head_strides), "ucm_kvstar_votes_tables: null table list");
-    return kvstar_votes(q_f16, q_off, n_tokens, q_heads, d_orig, pruned, pruned_sel, nullptr, 0, task_row_stride, task_tables,
-                        task_head_strides, seg_off, seg_len, n_tasks, max_blocks, sub_blocks, kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part,
-                        ws_part_floats, votes, tiles_per_wave, stream);
+    return kvstar_votes(q_f16, q_elems, q_off, n_tokens, q_heads, d_orig, pruned, n_pruned_lists, pruned_sel, votes_rows, nullptr, 0,
+                        task_row_stride, task_tables, task_head_strides, seg_off, seg_len, n_tasks, max_blocks, sub_blocks,
+                        kv_heads, d_pruned, d_pad, ws_max, ws_max_floats, ws_part, ws_part_floats, votes, tiles_per_wave, stream);
 }

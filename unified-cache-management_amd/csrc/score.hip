@@ -21,6 +21,7 @@
 #include <cmath>
 
 #include "common.h"
+#include "topk_select.h"
 
 namespace {
 
@@ -45,6 +46,16 @@ __device__ __forceinline__ f32x4 load_q4(const uint16_t* p)
     const uint2 w = *reinterpret_cast<const uint2*>(p);
     f32x4 r = {__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
                __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u)};
+    return r;
+}
+
+// fp16 queries travel as a type of their own so that the 16-bit loads pick the right widening
+struct f16bits { uint16_t v; };
+__device__ __forceinline__ f32x4 load_q4(const f16bits* p)
+{
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 w = *reinterpret_cast<const h4*>(p);
+    f32x4 r = {static_cast<float>(w.x), static_cast<float>(w.y), static_cast<float>(w.z), static_cast<float>(w.w)};
     return r;
 }
 
@@ -116,13 +127,17 @@ __device__ __forceinline__ float quad_dot(const f32x4 (&qr)[kSteps], const f32x4
 // end to end, request r contributing ceil(seg_len[r] / tile_blocks) of them).
 // Every wave does this on its own: 64 requests per trip, an inclusive wave scan
 // of their tile counts, a ballot for the first prefix that exceeds w.
-__device__ __forceinline__ bool find_tile(const int32_t* __restrict__ seg_len, int n_req, int tile_blocks,
-                                          int w, int lane, int& r_out, int& tile_out)
+// A seg_len beyond the host's max_seg_len is cut there (the grid was sized for it); with min_tiles = 1 every
+// request owns at least one tile, which the fused kernel needs: a request's last tile runs its selection.
+__device__ __forceinline__ int clamped_len(int n, int max_seg_len) { return min(max(n, 0), max_seg_len); }
+
+__device__ __forceinline__ bool find_tile(const int32_t* __restrict__ seg_len, int n_req, int tile_blocks, int max_seg_len,
+                                          int min_tiles, int w, int lane, int& r_out, int& tile_out)
 {
     int base = 0;
     for (int c = 0; c < n_req; c += 64) {
         const int r = c + lane;
-        const int t = r < n_req ? (max(seg_len[r], 0) + tile_blocks - 1) / tile_blocks : 0;
+        const int t = r < n_req ? max((clamped_len(seg_len[r], max_seg_len) + tile_blocks - 1) / tile_blocks, min_tiles) : 0;
         int incl = t;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -141,91 +156,173 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ seg_len, i
     return false;
 }
 
+// What a scoring launch reads and writes; the same for every workgroup.
+struct ScoreArgs {
+    const void* q;
+    int64_t q_layer_stride;
+    const int32_t* q_rows;
+    int q_heads;
+    const void* repre;
+    int64_t repre_layer_stride;
+    int64_t repre_rows;             // rows of a layer's table (and of a layer's scores): requests outside are skipped
+    const int32_t* seg_off;
+    const int32_t* seg_len;
+    int n_req;
+    int max_seg_len;
+    int kv_heads;
+    int num_repre;                  // representatives per (block, head): the score takes the largest of their dots
+    float* scores;
+    int64_t scores_layer_stride;
+    int tile_blocks;
+    float scale;
+    int32_t* tickets;               // fused selection: [layers][n_req] counters, zero between launches; else null
+};
+
+// What a workgroup works on: request, tile, and whether the request's descriptors may be followed.
+struct TileInfo {
+    int r, tile, n;
+    int64_t seg0, q_row;
+    bool ok;
+};
+
+template <int kD>
+__device__ __forceinline__ bool locate(const ScoreArgs& a, int lane, TileInfo& t)
+{
+    if (!find_tile(a.seg_len, a.n_req, a.tile_blocks, a.max_seg_len, a.tickets ? 1 : 0, blockIdx.x, lane, t.r, t.tile)) {
+        return false;
+    }
+    t.n = clamped_len(a.seg_len[t.r], a.max_seg_len);
+    t.seg0 = a.seg_off[t.r];
+    // indices that came from device memory are followed only inside their tables: the request's query row
+    // inside the layer's query block, its rows inside a layer of the representative table
+    t.q_row = a.q_rows ? static_cast<int64_t>(a.q_rows[t.r]) : t.r;
+    t.ok = !(a.q_rows && (t.q_row < 0 || (t.q_row + 1) * a.q_heads * kD > a.q_layer_stride)) &&
+           t.seg0 >= 0 && t.seg0 + t.n <= a.repre_rows;
+    return true;
+}
+
+// group-mean query -> LDS: sequential adds over the g heads of a group, then * (1/g)
+template <int kD, typename QT>
+__device__ __forceinline__ void stage_query(const ScoreArgs& a, int l, int64_t q_row, float* qbar)
+{
+    const int g = a.q_heads / a.kv_heads;
+    const float inv = 1.0f / static_cast<float>(g);
+    const QT* qp = static_cast<const QT*>(a.q) + static_cast<int64_t>(l) * a.q_layer_stride + q_row * a.q_heads * kD;
+    for (int e = threadIdx.x * 4; e < a.kv_heads * kD; e += kThreads * 4) {
+        const int hh = e / kD, d = e - hh * kD;
+        const f32x4 mean = group_mean4_any(qp + static_cast<int64_t>(hh) * g * kD + d, kD, g, inv);
+        *reinterpret_cast<f32x4*>(&qbar[e]) = mean;
+    }
+}
+
+// Sum over the kv heads, in order, of the largest dot among a head's representatives
+// (TopkBlockSelector::ComputeBlockScore); `first` is the lane that holds the block's first dot, `step` the lanes
+// per vector.  With one representative per head this is s + fmaxf(-FLT_MAX, dot) per head.
+__device__ __forceinline__ float head_sum(float dot, int first, int step, int kv_heads, int num_repre)
+{
+    float s = 0.0f;
+    int src = first;
+    for (int hh = 0; hh < kv_heads; ++hh) {
+        float best = -FLT_MAX;
+        for (int rr = 0; rr < num_repre; ++rr, src += step) { best = fmaxf(best, __shfl(dot, src, 64)); }
+        s = s + best;
+    }
+    return s;
+}
+
+// The fused kernel's tail.  Every workgroup of a request takes a ticket once its scores are visible to the
+// device; the one that draws the last ticket resets the counter and its first wave runs the request's
+// selection (TopkBlockSelector::TopKImpl, select_topk_block.cpp:20-51) on the scores all of them wrote.
+__device__ __forceinline__ void select_if_last(const ScoreArgs& a, const ucm::SelectArgs& sel, const TileInfo& t, int l)
+{
+    __shared__ int s_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");           // this thread's scores, before the ticket below
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int32_t* ticket = a.tickets + static_cast<int64_t>(l) * sel.cnt_layer_stride + t.r;
+        const int tiles = max((t.n + a.tile_blocks - 1) / a.tile_blocks, 1);
+        const int drawn = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = drawn == tiles - 1;
+        if (s_last) { __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    }
+    __syncthreads();
+    if (!s_last || threadIdx.x >= 64) { return; }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");           // the other workgroups' scores, after their tickets
+    const int lane = threadIdx.x;
+    // the smallest tier of key registers that holds the request (the host allows at most 1024 blocks here)
+    if (t.n <= 64) { ucm::select_wave<1, false>(sel, t.r, l, lane); }
+    else if (t.n <= 128) { ucm::select_wave<2, false>(sel, t.r, l, lane); }
+    else if (t.n <= 256) { ucm::select_wave<4, false>(sel, t.r, l, lane); }
+    else if (t.n <= 512) { ucm::select_wave<8, false>(sel, t.r, l, lane); }
+    else { ucm::select_wave<16, false>(sel, t.r, l, lane); }
+}
+
 // grid: x = dense tile index over all requests (workgroups past the last tile
 // exit), y = layer.  Tiles are numbered densely so that consecutive workgroups,
 // which the hardware deals round-robin to the 8 XCDs, always carry work: with a
 // (tile, request) grid the short requests of a ragged batch leave most XCDs idle.
 template <int kD, typename QT>
-__global__ __launch_bounds__(kThreads) void score_kernel(
-    const QT* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows, int q_heads,
-    const float* __restrict__ repre, int64_t repre_layer_stride, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, int n_req, int kv_heads, float* __restrict__ scores,
-    int64_t scores_layer_stride, int tile_blocks, float scale)
+__global__ __launch_bounds__(kThreads) void score_kernel(const ScoreArgs a, const ucm::SelectArgs sel)
 {
     constexpr int kSteps = kD / 16;
     __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l = blockIdx.y;
-    int r, tile;
-    if (!find_tile(seg_len, n_req, tile_blocks, blockIdx.x, lane, r, tile)) { return; }
-    // a row index that came from device memory is followed only inside the layer's query block
-    const int64_t q_row = q_rows ? static_cast<int64_t>(q_rows[r]) : r;
-    if (q_rows && (q_row < 0 || (q_row + 1) * q_heads * kD > q_layer_stride)) { return; }   // (the whole workgroup)
-    const int n = seg_len[r];
-    const int tile0 = tile * tile_blocks;
-    const int tile_end = min(tile0 + tile_blocks, n);
-    const int row = kv_heads * kD;
+    TileInfo t;
+    if (!locate<kD>(a, lane, t)) { return; }
+    const int tile0 = t.tile * a.tile_blocks;
+    const int tile_end = min(tile0 + a.tile_blocks, t.n);
+    if (t.ok && tile0 < tile_end) {                                  // (uniform over the workgroup)
+        const int vecs = a.kv_heads * a.num_repre;  // vectors per block
+        const int row = vecs * kD;
 
-    const int m = lane & 3;                 // which 4 of the 16 lanes of the dot product
-    const int v = lane >> 2;                // vector of this pass: 0..15
-    const int blocks_per_pass = 16 / kv_heads;
-    const int bl = v / kv_heads;            // block within the pass
-    const int h = v - bl * kv_heads;        // kv head, fixed for the whole kernel
-    const int stride = kWaves * blocks_per_pass;
-    const int seg0 = seg_off[r];
+        const int m = lane & 3;                 // which 4 of the 16 lanes of the dot product
+        const int v = lane >> 2;                // vector of this pass: 0..15
+        const int blocks_per_pass = 16 / vecs;
+        const int bl = v / vecs;                // block within the pass
+        const int vb = v - bl * vecs;           // vector within the block, fixed for the whole kernel
+        const int h = vb / a.num_repre;         // its kv head
+        const int stride = kWaves * blocks_per_pass;
 
-    const float* rbase = repre + static_cast<int64_t>(l) * repre_layer_stride +
-                         static_cast<int64_t>(seg0) * row + h * kD + 4 * m;
-    float* sout = scores + static_cast<int64_t>(l) * scores_layer_stride + seg0;
+        const float* rbase = static_cast<const float*>(a.repre) + static_cast<int64_t>(l) * a.repre_layer_stride +
+                             t.seg0 * row + vb * kD + 4 * m;
+        float* sout = a.scores + static_cast<int64_t>(l) * a.scores_layer_stride + t.seg0;
 
-    // the first pass's representatives are requested before the query is
-    // touched, so the two latencies overlap
-    int b0 = tile0 + wave * blocks_per_pass;
-    f32x4 kv_a[kSteps], kv_b[kSteps];
-    if (b0 < tile_end) { load_pass<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row); }
+        // the first pass's representatives are requested before the query is
+        // touched, so the two latencies overlap
+        int b0 = tile0 + wave * blocks_per_pass;
+        f32x4 kv_a[kSteps], kv_b[kSteps];
+        if (b0 < tile_end) { load_pass<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row); }
 
-    // group-mean query -> LDS: sequential adds over the g heads of a group, then * (1/g)
-    {
-        const int g = q_heads / kv_heads;
-        const float inv = 1.0f / static_cast<float>(g);
-        const QT* qp = q + static_cast<int64_t>(l) * q_layer_stride +
-                       q_row * q_heads * kD;
-        for (int e = threadIdx.x * 4; e < row; e += kThreads * 4) {
-            const int hh = e / kD, d = e - hh * kD;
-            const f32x4 mean = group_mean4_any(qp + static_cast<int64_t>(hh) * g * kD + d, kD, g, inv);
-            *reinterpret_cast<f32x4*>(&qbar[e]) = mean;
-        }
-    }
-    __syncthreads();
+        stage_query<kD, QT>(a, l, t.q_row, qbar);
+        __syncthreads();
 
-    f32x4 qr[kSteps];
+        f32x4 qr[kSteps];
 #pragma unroll
-    for (int i = 0; i < kSteps; ++i) {
-        qr[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 4 * m]);
-    }
-
-    // two passes per trip: the loads of the next pass are in flight while this one is reduced
-    auto finish = [&](const f32x4 (&kv)[kSteps], int base) {
-        const float dot = quad_dot<kSteps>(qr, kv);
-        float s = 0.0f;
-        for (int hh = 0; hh < kv_heads; ++hh) {
-            const float dh = __shfl(dot, (bl * kv_heads + hh) * 4, 64);
-            s = s + fmaxf(-FLT_MAX, dh);
+        for (int i = 0; i < kSteps; ++i) {
+            qr[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 4 * m]);
         }
-        const int b = base + bl;
-        if (b < tile_end && h == 0 && m == 0) { sout[b] = s * scale; }   // (a scale of 1 changes no bit)
-    };
-    while (b0 < tile_end) {
-        const int b1 = b0 + stride;
-        if (b1 < tile_end) { load_pass<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row); }
-        finish(kv_a, b0);
-        if (b1 >= tile_end) { break; }
-        const int b2 = b1 + stride;
-        if (b2 < tile_end) { load_pass<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row); }
-        finish(kv_b, b1);
-        b0 = b2;
+
+        // two passes per trip: the loads of the next pass are in flight while this one is reduced
+        auto finish = [&](const f32x4 (&kv)[kSteps], int base) {
+            const float dot = quad_dot<kSteps>(qr, kv);
+            const float s = head_sum(dot, bl * vecs * 4, 4, a.kv_heads, a.num_repre);
+            const int b = base + bl;
+            if (b < tile_end && vb == 0 && m == 0) { sout[b] = s * a.scale; }   // (a scale of 1 changes no bit)
+        };
+        while (b0 < tile_end) {
+            const int b1 = b0 + stride;
+            if (b1 < tile_end) { load_pass<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row); }
+            finish(kv_a, b0);
+            if (b1 >= tile_end) { break; }
+            const int b2 = b1 + stride;
+            if (b2 < tile_end) { load_pass<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row); }
+            finish(kv_b, b1);
+            b0 = b2;
+        }
     }
+    if (a.tickets) { select_if_last(a, sel, t, l); }
 }
 
 // ---- bf16 representative table ------------------------------------------------
@@ -270,175 +367,196 @@ __device__ __forceinline__ float pair_dot(const f32x4 (&qlo)[kSteps], const f32x
 }
 
 template <int kD, typename QT>
-__global__ __launch_bounds__(kThreads) void score_kernel_bf16(
-    const QT* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows, int q_heads,
-    const uint16_t* __restrict__ repre, int64_t repre_layer_stride, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, int n_req, int kv_heads, float* __restrict__ scores,
-    int64_t scores_layer_stride, int tile_blocks, float scale)
+__global__ __launch_bounds__(kThreads) void score_kernel_bf16(const ScoreArgs a, const ucm::SelectArgs sel)
 {
     constexpr int kSteps = kD / 16;
     __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l = blockIdx.y;
-    int r, tile;
-    if (!find_tile(seg_len, n_req, tile_blocks, blockIdx.x, lane, r, tile)) { return; }
-    // a row index that came from device memory is followed only inside the layer's query block
-    const int64_t q_row = q_rows ? static_cast<int64_t>(q_rows[r]) : r;
-    if (q_rows && (q_row < 0 || (q_row + 1) * q_heads * kD > q_layer_stride)) { return; }   // (the whole workgroup)
-    const int n = seg_len[r];
-    const int tile0 = tile * tile_blocks;
-    const int tile_end = min(tile0 + tile_blocks, n);
-    const int row = kv_heads * kD;
+    TileInfo t;
+    if (!locate<kD>(a, lane, t)) { return; }
+    const int tile0 = t.tile * a.tile_blocks;
+    const int tile_end = min(tile0 + a.tile_blocks, t.n);
+    if (t.ok && tile0 < tile_end) {                                  // (uniform over the workgroup)
+        const int vecs = a.kv_heads * a.num_repre;
+        const int row = vecs * kD;
 
-    const int p = lane & 1;                 // which 8 of the 16 lanes of the dot product
-    const int v = lane >> 1;                // vector of this pass: 0..31
-    const int blocks_per_pass = 32 / kv_heads;
-    const int bl = v / kv_heads;
-    const int h = v - bl * kv_heads;
-    const int stride = kWaves * blocks_per_pass;
-    const int seg0 = seg_off[r];
+        const int p = lane & 1;                 // which 8 of the 16 lanes of the dot product
+        const int v = lane >> 1;                // vector of this pass: 0..31
+        const int blocks_per_pass = 32 / vecs;
+        const int bl = v / vecs;
+        const int vb = v - bl * vecs;
+        const int h = vb / a.num_repre;
+        const int stride = kWaves * blocks_per_pass;
 
-    const uint16_t* rbase = repre + static_cast<int64_t>(l) * repre_layer_stride +
-                            static_cast<int64_t>(seg0) * row + h * kD + 8 * p;
-    float* sout = scores + static_cast<int64_t>(l) * scores_layer_stride + seg0;
+        const uint16_t* rbase = static_cast<const uint16_t*>(a.repre) + static_cast<int64_t>(l) * a.repre_layer_stride +
+                                t.seg0 * row + vb * kD + 8 * p;
+        float* sout = a.scores + static_cast<int64_t>(l) * a.scores_layer_stride + t.seg0;
 
-    // Loads and the store below are unconditional (rows and the output index are clamped to the tile's last
-    // block, whose score is then written more than once): an operation skipped on some path would make the
-    // compiler wait for everything outstanding, the prefetch included.  The empty asm keeps the compiler from
-    // sinking a prefetch down to its use.
-    int b0 = tile0 + wave * blocks_per_pass;
-    u32x4 kv_a[kSteps], kv_b[kSteps];
-    load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row);
-    asm volatile("" ::: "memory");
+        // Loads and the store below are unconditional (rows and the output index are clamped to the tile's last
+        // block, whose score is then written more than once): an operation skipped on some path would make the
+        // compiler wait for everything outstanding, the prefetch included.  The empty asm keeps the compiler from
+        // sinking a prefetch down to its use.
+        int b0 = tile0 + wave * blocks_per_pass;
+        u32x4 kv_a[kSteps], kv_b[kSteps];
+        load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b0 + bl, tile_end - 1)) * row);
+        asm volatile("" ::: "memory");
 
-    {
-        const int g = q_heads / kv_heads;
-        const float inv = 1.0f / static_cast<float>(g);
-        const QT* qp = q + static_cast<int64_t>(l) * q_layer_stride +
-                       q_row * q_heads * kD;
-        for (int e = threadIdx.x * 4; e < row; e += kThreads * 4) {
-            const int hh = e / kD, d = e - hh * kD;
-            const f32x4 mean = group_mean4_any(qp + static_cast<int64_t>(hh) * g * kD + d, kD, g, inv);
-            *reinterpret_cast<f32x4*>(&qbar[e]) = mean;
-        }
-    }
-    __syncthreads();
+        stage_query<kD, QT>(a, l, t.q_row, qbar);
+        __syncthreads();
 
-    f32x4 qlo[kSteps], qhi[kSteps];
+        f32x4 qlo[kSteps], qhi[kSteps];
 #pragma unroll
-    for (int i = 0; i < kSteps; ++i) {
-        qlo[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p]);
-        qhi[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p + 4]);
-    }
-
-    auto finish = [&](const u32x4 (&kv)[kSteps], int base) {
-        const float dot = pair_dot<kSteps>(qlo, qhi, kv);
-        float s = 0.0f;
-        for (int hh = 0; hh < kv_heads; ++hh) {
-            const float dh = __shfl(dot, (bl * kv_heads + hh) * 2, 64);
-            s = s + fmaxf(-FLT_MAX, dh);
+        for (int i = 0; i < kSteps; ++i) {
+            qlo[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p]);
+            qhi[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p + 4]);
         }
-        sout[min(base + bl, tile_end - 1)] = s * scale;   // the lanes of a block all hold its score; a scale of 1 changes no bit
-    };
-    while (b0 < tile_end) {
-        const int b1 = b0 + stride;
-        load_pass_bf16<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row);
-        asm volatile("" ::: "memory");
-        finish(kv_a, b0);
-        if (b1 >= tile_end) { break; }
-        const int b2 = b1 + stride;
-        load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row);
-        asm volatile("" ::: "memory");
-        finish(kv_b, b1);
-        b0 = b2;
+
+        auto finish = [&](const u32x4 (&kv)[kSteps], int base) {
+            const float dot = pair_dot<kSteps>(qlo, qhi, kv);
+            const float s = head_sum(dot, bl * vecs * 2, 2, a.kv_heads, a.num_repre);
+            sout[min(base + bl, tile_end - 1)] = s * a.scale;   // the lanes of a block all hold its score; a scale of 1 changes no bit
+        };
+        while (b0 < tile_end) {
+            const int b1 = b0 + stride;
+            load_pass_bf16<kSteps>(kv_b, rbase + static_cast<int64_t>(min(b1 + bl, tile_end - 1)) * row);
+            asm volatile("" ::: "memory");
+            finish(kv_a, b0);
+            if (b1 >= tile_end) { break; }
+            const int b2 = b1 + stride;
+            load_pass_bf16<kSteps>(kv_a, rbase + static_cast<int64_t>(min(b2 + bl, tile_end - 1)) * row);
+            asm volatile("" ::: "memory");
+            finish(kv_b, b1);
+            b0 = b2;
+        }
     }
+    if (a.tickets) { select_if_last(a, sel, t, l); }
 }
 
 template <int kD, typename QT>
-void launch_bf16(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
-                 int64_t repre_layer_stride, const int32_t* seg_off, const int32_t* seg_len, int n_req,
-                 int64_t tile_bound, int n_layers, int kv_heads, float* scores, int64_t scores_layer_stride,
-                 int tile_blocks, float scale, hipStream_t stream)
+void launch_dim(const ScoreArgs& a, const ucm::SelectArgs& sel, bool bf16_table, dim3 grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((score_kernel_bf16<kD, QT>), dim3(static_cast<unsigned>(tile_bound), n_layers), dim3(kThreads), 0,
-                       stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads,
-                       static_cast<const uint16_t*>(repre), repre_layer_stride, seg_off, seg_len, n_req, kv_heads,
-                       scores, scores_layer_stride, tile_blocks, scale);
+    if (bf16_table) { hipLaunchKernelGGL((score_kernel_bf16<kD, QT>), grid, dim3(kThreads), 0, s, a, sel); }
+    else { hipLaunchKernelGGL((score_kernel<kD, QT>), grid, dim3(kThreads), 0, s, a, sel); }
 }
 
-template <int kD, typename QT>
-void launch(const void* q, int64_t q_layer_stride, const int32_t* q_rows, int q_heads, const void* repre,
-            int64_t repre_layer_stride, const int32_t* seg_off, const int32_t* seg_len, int n_req,
-            int64_t tile_bound, int n_layers, int kv_heads, float* scores, int64_t scores_layer_stride,
-            int tile_blocks, float scale, hipStream_t stream)
+template <int kD>
+void launch_q(const ScoreArgs& a, const ucm::SelectArgs& sel, int q_dtype, bool bf16_table, dim3 grid, hipStream_t s)
 {
-    hipLaunchKernelGGL((score_kernel<kD, QT>), dim3(static_cast<unsigned>(tile_bound), n_layers), dim3(kThreads), 0,
-                       stream, static_cast<const QT*>(q), q_layer_stride, q_rows, q_heads,
-                       static_cast<const float*>(repre), repre_layer_stride,
-                       seg_off, seg_len, n_req, kv_heads, scores, scores_layer_stride, tile_blocks, scale);
+    if (q_dtype == UCM_DTYPE_F32) { launch_dim<kD, float>(a, sel, bf16_table, grid, s); }
+    else if (q_dtype == UCM_DTYPE_BF16) { launch_dim<kD, uint16_t>(a, sel, bf16_table, grid, s); }
+    else { launch_dim<kD, f16bits>(a, sel, bf16_table, grid, s); }
+}
+
+// Host checks shared by ucm_score_blocks and ucm_score_select, then the launch.  `sel` is null for scores alone.
+int score_launch(const char* name, const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows, int q_heads,
+                 const void* repre, int repre_dtype, int64_t repre_layer_stride, int64_t repre_rows, int num_repre,
+                 const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len, int64_t total_blocks,
+                 int n_layers, int kv_heads, int head_dim, float* scores, int64_t scores_layer_stride, float scale,
+                 int tile_blocks_arg, const ucm::SelectArgs* sel, int32_t* tickets, ucm_stream_t stream)
+{
+    UCM_REQUIRE(std::isfinite(scale), "%s: scale is not finite", name);
+    UCM_REQUIRE(tile_blocks_arg >= 0 && tile_blocks_arg <= 4096, "%s: tile_blocks=%d", name, tile_blocks_arg);
+    UCM_REQUIRE(n_req == 0 || max_seg_len == 0 || (q && repre && seg_off && seg_len && scores), "%s: null pointer", name);
+    UCM_REQUIRE(q_dtype == UCM_DTYPE_F32 || q_dtype == UCM_DTYPE_BF16 || q_dtype == UCM_DTYPE_F16, "%s: q_dtype=%d", name, q_dtype);
+    UCM_REQUIRE(repre_dtype == UCM_DTYPE_F32 || repre_dtype == UCM_DTYPE_BF16, "%s: repre_dtype=%d", name, repre_dtype);
+    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "%s: n_req=%d n_layers=%d", name, n_req, n_layers);
+    UCM_REQUIRE(max_seg_len >= 0 && total_blocks >= 0, "%s: max_seg_len=%d total_blocks=%lld", name, max_seg_len,
+                static_cast<long long>(total_blocks));
+    UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0, "%s: q_heads=%d kv_heads=%d", name, q_heads, kv_heads);
+    UCM_REQUIRE(num_repre >= 1, "%s: num_repre=%d", name, num_repre);
+    UCM_SUPPORTED(head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 || head_dim == 192 || head_dim == 256,
+                  "%s: head_dim=%d (32, 64, 96, 128, 192 or 256)", name, head_dim);
+    const int vecs = kv_heads * num_repre;
+    UCM_SUPPORTED(vecs * head_dim <= kMaxRow, "%s: kv_heads*num_repre*head_dim=%d (at most %d)", name, vecs * head_dim, kMaxRow);
+    UCM_SUPPORTED(vecs <= 16 && 16 % vecs == 0, "%s: kv_heads*num_repre=%d (1, 2, 4, 8 or 16)", name, vecs);
+    const int es = repre_dtype == UCM_DTYPE_BF16 ? 2 : 4;
+    UCM_REQUIRE(ucm::aligned16(repre) && repre_layer_stride % (16 / es) == 0, "%s: repre not 16-byte aligned", name);
+    UCM_REQUIRE(ucm::aligned16(q) && q_layer_stride % 8 == 0, "%s: q not 16-byte aligned", name);
+    UCM_REQUIRE(!q_rows || q_layer_stride >= static_cast<int64_t>(q_heads) * head_dim,
+                "%s: with q_rows, q_layer_stride=%lld bounds the rows and must hold at least one", name,
+                static_cast<long long>(q_layer_stride));
+    UCM_REQUIRE(repre_rows >= 0 && (n_layers == 1 || (repre_layer_stride >= repre_rows * vecs * head_dim &&
+                                                     scores_layer_stride >= repre_rows)),
+                "%s: repre_rows=%lld does not fit the layer strides", name, static_cast<long long>(repre_rows));
+    if (n_req == 0 || (max_seg_len == 0 && !sel)) { return UCM_OK; }
+    // upper bound of sum(ceil(seg_len / tile)): exact to within n_req when the host knows the total
+    const int row_bytes = vecs * head_dim * es;
+    const int tile_blocks = tile_blocks_arg > 0 ? tile_blocks_arg : std::max(8, (128 * 1024) / row_bytes);
+    const int64_t per_req = std::max<int64_t>((static_cast<int64_t>(max_seg_len) + tile_blocks - 1) / tile_blocks, sel ? 1 : 0);
+    int64_t tile_bound = per_req * n_req;
+    // (with the selection fused in, every tile of every request has to run, whatever seg_len holds: the
+    // caller's total is not used to shrink the grid)
+    if (total_blocks > 0 && !sel) { tile_bound = std::min(tile_bound, (total_blocks + tile_blocks - 1) / tile_blocks + n_req); }
+    UCM_REQUIRE(tile_bound <= 0x7fffffffll, "%s: too many tiles for one launch", name);
+    const ScoreArgs a = {q, q_layer_stride, q_rows, q_heads, repre, repre_layer_stride, repre_rows, seg_off, seg_len, n_req,
+                         max_seg_len, kv_heads, num_repre, scores, scores_layer_stride, tile_blocks, scale, sel ? tickets : nullptr};
+    const ucm::SelectArgs none = {};
+    const dim3 grid(static_cast<unsigned>(tile_bound), n_layers);
+    hipStream_t s = ucm::as_stream(stream);
+    const bool bf16_table = repre_dtype == UCM_DTYPE_BF16;
+    switch (head_dim) {
+    case 32: launch_q<32>(a, sel ? *sel : none, q_dtype, bf16_table, grid, s); break;
+    case 64: launch_q<64>(a, sel ? *sel : none, q_dtype, bf16_table, grid, s); break;
+    case 96: launch_q<96>(a, sel ? *sel : none, q_dtype, bf16_table, grid, s); break;
+    case 128: launch_q<128>(a, sel ? *sel : none, q_dtype, bf16_table, grid, s); break;
+    case 192: launch_q<192>(a, sel ? *sel : none, q_dtype, bf16_table, grid, s); break;
+    default: launch_q<256>(a, sel ? *sel : none, q_dtype, bf16_table, grid, s); break;
+    }
+    return ucm::check_hip(hipGetLastError(), name);
 }
 
 }  // namespace
 
 extern "C" int ucm_score_blocks(const void* q, int q_dtype, int64_t q_layer_stride, const int32_t* q_rows,
                                 int q_heads, const void* repre, int repre_dtype, int64_t repre_layer_stride,
-                                const int32_t* seg_off, const int32_t* seg_len, int n_req, int max_seg_len,
-                                int64_t total_blocks, int n_layers, int kv_heads, int head_dim, float* scores,
-                                int64_t scores_layer_stride, float scale, int tile_blocks_arg, ucm_stream_t stream)
+                                int64_t repre_rows, int num_repre, const int32_t* seg_off, const int32_t* seg_len,
+                                int n_req, int max_seg_len, int64_t total_blocks, int n_layers, int kv_heads,
+                                int head_dim, float* scores, int64_t scores_layer_stride, float scale,
+                                int tile_blocks, ucm_stream_t stream)
 {
-    UCM_REQUIRE(std::isfinite(scale), "ucm_score_blocks: scale is not finite");
-    UCM_REQUIRE(tile_blocks_arg >= 0 && tile_blocks_arg <= 4096, "ucm_score_blocks: tile_blocks=%d", tile_blocks_arg);
-    UCM_REQUIRE(n_req == 0 || max_seg_len == 0 || (q && repre && seg_off && seg_len && scores),
-                "ucm_score_blocks: null pointer");
-    UCM_REQUIRE(q_dtype == UCM_DTYPE_F32 || q_dtype == UCM_DTYPE_BF16, "ucm_score_blocks: q_dtype=%d", q_dtype);
-    UCM_REQUIRE(repre_dtype == UCM_DTYPE_F32 || repre_dtype == UCM_DTYPE_BF16, "ucm_score_blocks: repre_dtype=%d", repre_dtype);
-    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535,
-                "ucm_score_blocks: n_req=%d n_layers=%d", n_req, n_layers);
-    UCM_REQUIRE(max_seg_len >= 0 && total_blocks >= 0, "ucm_score_blocks: max_seg_len=%d total_blocks=%lld",
-                max_seg_len, static_cast<long long>(total_blocks));
-    UCM_REQUIRE(kv_heads > 0 && q_heads >= kv_heads && q_heads % kv_heads == 0,
-                "ucm_score_blocks: q_heads=%d kv_heads=%d", q_heads, kv_heads);
-    UCM_SUPPORTED(head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 || head_dim == 192 || head_dim == 256,
-                  "ucm_score_blocks: head_dim=%d (32, 64, 96, 128, 192 or 256)", head_dim);
-    UCM_SUPPORTED(kv_heads * head_dim <= kMaxRow, "ucm_score_blocks: kv_heads*head_dim=%d (at most %d)", kv_heads * head_dim, kMaxRow);
-    UCM_SUPPORTED(kv_heads <= 16 && 16 % kv_heads == 0, "ucm_score_blocks: kv_heads=%d (1, 2, 4, 8 or 16)", kv_heads);
-    UCM_REQUIRE(ucm::aligned16(repre) && repre_layer_stride % (repre_dtype == UCM_DTYPE_BF16 ? 8 : 4) == 0,
-                "ucm_score_blocks: repre not 16-byte aligned");
-    UCM_SUPPORTED(repre_dtype == UCM_DTYPE_F32 || 32 % kv_heads == 0, "ucm_score_blocks: kv_heads=%d", kv_heads);
-    UCM_REQUIRE(ucm::aligned16(q) && q_layer_stride % 8 == 0, "ucm_score_blocks: q not 16-byte aligned");
-    UCM_REQUIRE(!q_rows || q_layer_stride >= static_cast<int64_t>(q_heads) * head_dim,
-                "ucm_score_blocks: with q_rows, q_layer_stride=%lld bounds the rows and must hold at least one",
-                static_cast<long long>(q_layer_stride));
-    if (n_req == 0 || max_seg_len == 0) { return UCM_OK; }
-    hipStream_t s = ucm::as_stream(stream);
-    // upper bound of sum(ceil(seg_len / tile)): exact to within n_req when the host knows the total
-    const int row_bytes = kv_heads * head_dim * (repre_dtype == UCM_DTYPE_BF16 ? 2 : 4);
-    const int tile_blocks = tile_blocks_arg > 0 ? tile_blocks_arg : std::max(8, (128 * 1024) / row_bytes);
-    const int64_t per_req = (static_cast<int64_t>(max_seg_len) + tile_blocks - 1) / tile_blocks;
-    int64_t tile_bound = per_req * n_req;
-    if (total_blocks > 0) { tile_bound = std::min(tile_bound, (total_blocks + tile_blocks - 1) / tile_blocks + n_req); }
-    UCM_REQUIRE(tile_bound <= 0x7fffffffll, "ucm_score_blocks: too many tiles for one launch");
-#define UCM_SCORE_ARGS q, q_layer_stride, q_rows, q_heads, repre, repre_layer_stride, seg_off, seg_len, n_req, \
-                       tile_bound, n_layers, kv_heads, scores, scores_layer_stride, tile_blocks, scale, s
-    const bool qf = q_dtype == UCM_DTYPE_F32;
-#define UCM_SCORE_DIM(D)                                                                                        \
-    do {                                                                                                        \
-        if (repre_dtype == UCM_DTYPE_F32) {                                                                     \
-            if (qf) { launch<D, float>(UCM_SCORE_ARGS); } else { launch<D, uint16_t>(UCM_SCORE_ARGS); }         \
-        } else {                                                                                                \
-            if (qf) { launch_bf16<D, float>(UCM_SCORE_ARGS); } else { launch_bf16<D, uint16_t>(UCM_SCORE_ARGS); } \
-        }                                                                                                       \
-    } while (0)
-    switch (head_dim) {
-    case 32: UCM_SCORE_DIM(32); break;
-    case 64: UCM_SCORE_DIM(64); break;
-    case 96: UCM_SCORE_DIM(96); break;
-    case 128: UCM_SCORE_DIM(128); break;
-    case 192: UCM_SCORE_DIM(192); break;
-    default: UCM_SCORE_DIM(256); break;
-    }
-#undef UCM_SCORE_DIM
-#undef UCM_SCORE_ARGS
-    UCM_LAUNCH_CHECK("ucm_score_blocks");
+    return score_launch("ucm_score_blocks", q, q_dtype, q_layer_stride, q_rows, q_heads, repre, repre_dtype, repre_layer_stride,
+                        repre_rows, num_repre, seg_off, seg_len, n_req, max_seg_len, total_blocks, n_layers, kv_heads, head_dim,
+                        scores, scores_layer_stride, scale, tile_blocks, nullptr, nullptr, stream);
+}
+
+extern "C" int ucm_score_select(const ucm_score_select_args_t* p, ucm_stream_t stream)
+{
+    UCM_REQUIRE(p && p->struct_size == sizeof(ucm_score_select_args_t), "ucm_score_select: args missing or of another version (struct_size)");
+    const int n_req = p->n_req, n_layers = p->n_layers, first = p->first_layer;
+    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535 && first >= 0, "ucm_score_select: n_req=%d n_layers=%d first_layer=%d",
+                n_req, n_layers, first);
+    if (n_req == 0) { return UCM_OK; }
+    UCM_REQUIRE(p->seg_off && p->seg_len && p->topk_len && p->idx_out && p->count_out && p->tickets && p->scores,
+                "ucm_score_select: null pointer");
+    UCM_REQUIRE(p->start_w >= 0 && p->end_w >= 0 && p->max_seg_len >= 0, "ucm_score_select: negative window or length");
+    UCM_REQUIRE(p->out_stride >= p->max_seg_len, "ucm_score_select: out_stride=%d < max_seg_len=%d", p->out_stride, p->max_seg_len);
+    UCM_REQUIRE((p->block_tables == nullptr) == (p->phys_out == nullptr), "ucm_score_select: block_tables and phys_out go together");
+    UCM_REQUIRE(!p->block_tables || p->bt_stride >= p->max_seg_len, "ucm_score_select: bt_stride=%d < max_seg_len=%d", p->bt_stride,
+                p->max_seg_len);
+    UCM_REQUIRE(!p->sparse_seq_lens || (p->seq_lens && p->block_size > 0), "ucm_score_select: sparse_seq_lens needs seq_lens and block_size");
+    UCM_SUPPORTED(p->max_seg_len <= 1024, "ucm_score_select: max_seg_len=%d (at most 1024 blocks per request; ucm_score_blocks + "
+                  "ucm_topk_windows take up to 4096)", p->max_seg_len);
+    UCM_REQUIRE(p->kv_heads > 0 && p->head_dim > 0 && p->num_repre >= 1, "ucm_score_select: kv_heads=%d head_dim=%d num_repre=%d",
+                p->kv_heads, p->head_dim, p->num_repre);
+    // table pointers name layer 0 and move to first_layer here; q names the first layer scored
+    const int64_t es = p->repre_dtype == UCM_DTYPE_BF16 ? 2 : 4;
+    const char* repre = static_cast<const char*>(p->repre) + first * p->repre_layer_stride * es;
+    float* scores = p->scores + first * p->scores_layer_stride;
+    UCM_REQUIRE(p->idx_layer_stride >= 0 && p->count_layer_stride >= 0, "ucm_score_select: negative layer stride");
+    const int64_t idx_ls = p->idx_layer_stride ? p->idx_layer_stride : static_cast<int64_t>(n_req) * p->out_stride;
+    const int64_t cnt_ls = p->count_layer_stride ? p->count_layer_stride : n_req;
+    UCM_REQUIRE(idx_ls >= static_cast<int64_t>(n_req) * p->out_stride && cnt_ls >= n_req,
+                "ucm_score_select: layer strides shorter than a layer (%lld, %lld)", static_cast<long long>(idx_ls),
+                static_cast<long long>(cnt_ls));
+    const ucm::SelectArgs sel = {scores, p->scores_layer_stride, p->repre_rows, p->seg_off, p->seg_len, p->topk_len, n_req,
+                                 p->max_seg_len, p->start_w, p->end_w, p->idx_out + first * idx_ls, p->out_stride, idx_ls, cnt_ls,
+                                 p->count_out + first * cnt_ls, p->block_tables, p->bt_stride,
+                                 p->phys_out ? p->phys_out + first * idx_ls : nullptr, p->seq_lens, p->block_size,
+                                 p->sparse_seq_lens ? p->sparse_seq_lens + first * cnt_ls : nullptr};
+    return score_launch("ucm_score_select", p->q, p->q_dtype, p->q_layer_stride, p->q_rows, p->q_heads, repre, p->repre_dtype,
+                        p->repre_layer_stride, p->repre_rows, p->num_repre, p->seg_off, p->seg_len, n_req, p->max_seg_len, 0,
+                        n_layers, p->kv_heads, p->head_dim, scores, p->scores_layer_stride, p->scale, p->tile_blocks, &sel,
+                        p->tickets + first * cnt_ls, stream);
 }

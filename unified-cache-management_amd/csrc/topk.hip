@@ -1,200 +1,28 @@
 // Per-request block selection with forced windows: one 64-wide wavefront per
-// (layer, request), the request's scores held in registers as order-preserving
-// 32-bit keys (element i lives in lane i%64, register i/64).
-//
-// Selection is a radix select, one bit per step from the top: the threshold T
-// is grown greedily while at least m candidates have key >= T, each count being
-// a wave ballot + popcount.  Candidates with key > T are all taken; of those
-// with key == T the first `m - count(key > T)` in index order are taken, which
-// is exactly where a stable descending sort leaves equal scores.  Output
-// positions are ballot prefix counts in index order, so the result comes out
-// sorted ascending with no sort at all, and the logical->physical block-table
-// lookup is applied on the way out.
+// (layer, request); the selection itself is ucm::select_wave (topk_select.h).
 //
 // A few KB in, a few hundred bytes out per wave: this kernel is latency-bound,
 // not bandwidth-bound; it only has to stay small next to scoring and gather.
 #include "common.h"
+#include "topk_select.h"
 
 namespace {
 
-__device__ __forceinline__ unsigned ordered_key(float f)
-{
-    f = f + 0.0f;  // -0.0 -> +0.0, so that the two zeros tie like they do under operator>
-    const unsigned u = __float_as_uint(f);
-    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-}
+using ucm::lanes_below;
+using ucm::ordered_key;
 
-__device__ __forceinline__ unsigned lanes_below(unsigned long long mask)
-{
-    return __builtin_amdgcn_mbcnt_hi(static_cast<unsigned>(mask >> 32),
-                                     __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(mask), 0u));
-}
-
-// kHeapTies selects which blocks tied at the k-th score are kept.  false: the
-// first ones in index order (std::stable_sort).  true: the ones KVStar's
-// min-heap of (score, index) pairs ends up with
-// (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:955-977:
-// blocks arrive in index order, a full heap replaces its smallest pair only
-// for a strictly greater score).  That process has a closed form: ties enter
-// while fewer than k blocks with key >= T have arrived and leave, lowest index
-// first, once per block above T that arrives later; so with P the shortest
-// prefix holding k blocks >= T, g_P the blocks above T inside P and g those in
-// the whole list, the ties kept are the ones of P whose rank among the ties is
-// at least g - g_P.  Windows are not used with it (host checked).
-//
 // grid: x = request, y = layer; block = one wave
 template <int kEpl, bool kHeapTies>
-__global__ __launch_bounds__(64) void topk_windows_kernel(
-    const float* __restrict__ scores, int64_t scores_layer_stride, const int32_t* __restrict__ seg_off,
-    const int32_t* __restrict__ seg_len, const int32_t* __restrict__ topk_len, int n_req, int start_w,
-    int end_w, int32_t* __restrict__ idx_out, int out_stride, int32_t* __restrict__ count_out,
-    const int32_t* __restrict__ block_tables, int bt_stride, int32_t* __restrict__ phys_out,
-    const int32_t* __restrict__ seq_lens, int block_size, int32_t* __restrict__ sparse_seq_lens)
+__global__ __launch_bounds__(64) void topk_windows_kernel(const ucm::SelectArgs a)
 {
-    const int r = blockIdx.x, l = blockIdx.y, lane = threadIdx.x;
-    const size_t lr = static_cast<size_t>(l) * n_req + r;
-    int n = seg_len[r];
-    n = min(n, min(out_stride, 64 * kEpl));  // host checked; clamp so nothing can run past a row
-    if (block_tables) { n = min(n, bt_stride); }
-    const int k = topk_len[r];
-    int32_t* out = idx_out + lr * out_stride;
-    int32_t* pout = phys_out ? phys_out + lr * out_stride : nullptr;
-    const int32_t* bt = block_tables ? block_tables + static_cast<size_t>(r) * bt_stride : nullptr;
-    int count = 0;
-    bool kept_all = false;
-
-    if (n <= 0) {
-        count = 0;
-    } else if (start_w + end_w >= n || k >= n || k <= 0) {
-        for (int i = lane; i < n; i += 64) {
-            out[i] = i;
-            if (pout) { pout[i] = bt[i]; }
-        }
-        count = n;
-        kept_all = true;
-    } else if (k < start_w + end_w) {
-        // fewer slots than forced blocks: the first k of [0..start_w) ++ [n-end_w..n)
-        for (int j = lane; j < k; j += 64) {
-            const int idx = j < start_w ? j : n - end_w + (j - start_w);
-            out[j] = idx;
-            if (pout) { pout[j] = bt[idx]; }
-        }
-        count = k;
-    } else {
-        const int m = k - start_w - end_w;       // free picks among the middle blocks
-        const int hi = n - end_w;                // candidates are start_w <= i < hi
-        const float* s = scores + static_cast<int64_t>(l) * scores_layer_stride + seg_off[r];
-        unsigned key[kEpl];
-        int32_t phys[kEpl];                      // the block table's entries, fetched with the scores: a load per
-#pragma unroll                                   // taken element on the way out would cost a memory round trip per register
-        for (int j = 0; j < kEpl; ++j) {
-            const int i = j * 64 + lane;
-            const bool cand = i >= start_w && i < hi;
-            key[j] = cand ? ordered_key(s[cand ? i : 0]) : 0u;
-            phys[j] = bt ? bt[min(i, n - 1)] : 0;
-        }
-        unsigned T = 0;
-        int need = 0;
-        int tie_lo = 0, tie_hi = 0;              // kHeapTies: ranks (among the ties) that are kept
-        if (m > 0) {
-            for (int bit = 31; bit >= 0; --bit) {
-                const unsigned c = T | (1u << bit);
-                int cnt = 0;
-#pragma unroll
-                for (int j = 0; j < kEpl; ++j) { cnt += __popcll(__ballot(key[j] >= c)); }
-                if (cnt >= m) { T = c; }
-            }
-            int greater = 0;
-#pragma unroll
-            for (int j = 0; j < kEpl; ++j) { greater += __popcll(__ballot(key[j] > T)); }
-            need = m - greater;
-            if (kHeapTies) {
-                // walk the list in index order up to the k-th block with key >= T
-                int seen = 0, g_p = 0;
-#pragma unroll
-                for (int j = 0; j < kEpl; ++j) {
-                    const unsigned long long ge_mask = __ballot(key[j] >= T && key[j] != 0u);
-                    const unsigned long long gt_mask = __ballot(key[j] > T);
-                    const int c = __popcll(ge_mask);
-                    if (seen < m) {
-                        if (seen + c >= m) {
-                            // lane holding the m-th one: the (m - seen)-th set bit of ge_mask
-                            const bool is_pth = ((ge_mask >> lane) & 1ull) && seen + static_cast<int>(lanes_below(ge_mask)) + 1 == m;
-                            const unsigned long long pm = __ballot(is_pth);
-                            const int p_lane = __ffsll(static_cast<long long>(pm)) - 1;
-                            const unsigned long long upto = p_lane >= 63 ? ~0ull : ((2ull << p_lane) - 1ull);
-                            g_p += __popcll(gt_mask & upto);
-                        } else {
-                            g_p += __popcll(gt_mask);
-                        }
-                    }
-                    seen += c;
-                }
-                tie_lo = greater - g_p;          // one tie left per block above T that came after P
-                tie_hi = m - g_p;                // ties inside P
-            }
-        }
-        int pos = 0, ties_seen = 0;
-#pragma unroll
-        for (int j = 0; j < kEpl; ++j) {
-            if (j * 64 < n) {
-                const int i = j * 64 + lane;
-                const bool window = i < n && (i < start_w || i >= hi);
-                const bool cand = i >= start_w && i < hi;
-                const bool gt = cand && m > 0 && key[j] > T;
-                const bool eq = cand && m > 0 && key[j] == T;
-                const unsigned long long eq_mask = __ballot(eq);
-                const int tie_rank = ties_seen + static_cast<int>(lanes_below(eq_mask));
-                const bool take = window || gt || (eq && (kHeapTies ? (tie_rank >= tie_lo && tie_rank < tie_hi) : tie_rank < need));
-                ties_seen += __popcll(eq_mask);
-                const unsigned long long take_mask = __ballot(take);
-                if (take) {
-                    const int p = pos + static_cast<int>(lanes_below(take_mask));
-                    out[p] = i;
-                    if (pout) { pout[p] = phys[j]; }
-                }
-                pos += __popcll(take_mask);
-            }
-        }
-        count = pos;
-    }
-    if (lane == 0) {
-        count_out[lr] = count;
-        if (sparse_seq_lens && seq_lens) {
-            const int len = seq_lens[r], rem = len % block_size;
-            // every block kept: the request keeps its length; otherwise `count` blocks, the last one partial
-            sparse_seq_lens[lr] = kept_all ? len : (rem == 0 ? count * block_size : count * block_size - block_size + rem);
-        }
-    }
+    ucm::select_wave<kEpl, kHeapTies>(a, blockIdx.x, blockIdx.y, threadIdx.x);
 }
 
-}  // namespace
-
-extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, const int32_t* seg_off,
-                                const int32_t* seg_len, const int32_t* topk_len, int n_req, int max_seg_len,
-                                int n_layers, int start_w, int end_w, int32_t* idx_out, int out_stride,
-                                int32_t* count_out, const int32_t* block_tables, int bt_stride,
-                                int32_t* phys_out, const int32_t* seq_lens, int block_size,
-                                int32_t* sparse_seq_lens, ucm_stream_t stream)
+template <bool kHeapTies>
+void launch_select(const ucm::SelectArgs& a, int max_seg_len, int n_layers, hipStream_t s)
 {
-    UCM_REQUIRE(n_req == 0 || (scores && seg_off && seg_len && topk_len && idx_out && count_out),
-                "ucm_topk_windows: null pointer");
-    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_topk_windows: n_req=%d n_layers=%d", n_req, n_layers);
-    UCM_REQUIRE(start_w >= 0 && end_w >= 0 && max_seg_len >= 0, "ucm_topk_windows: negative window or length");
-    UCM_REQUIRE(out_stride >= max_seg_len, "ucm_topk_windows: out_stride=%d < max_seg_len=%d", out_stride, max_seg_len);
-    UCM_REQUIRE((block_tables == nullptr) == (phys_out == nullptr),
-                "ucm_topk_windows: block_tables and phys_out go together");
-    UCM_REQUIRE(!block_tables || bt_stride >= max_seg_len, "ucm_topk_windows: bt_stride=%d < max_seg_len=%d",
-                bt_stride, max_seg_len);
-    UCM_REQUIRE(!sparse_seq_lens || (seq_lens && block_size > 0), "ucm_topk_windows: sparse_seq_lens needs seq_lens and block_size");
-    UCM_SUPPORTED(max_seg_len <= 4096, "ucm_topk_windows: max_seg_len=%d (at most 4096 blocks per request)", max_seg_len);
-    if (n_req == 0) { return UCM_OK; }
-    hipStream_t s = ucm::as_stream(stream);
-    const dim3 grid(n_req, n_layers), block(64);
-#define UCM_TOPK_LAUNCH(EPL)                                                                                  \
-    hipLaunchKernelGGL((topk_windows_kernel<EPL, false>), grid, block, 0, s, scores, scores_layer_stride, seg_off, \
-                       seg_len, topk_len, n_req, start_w, end_w, idx_out, out_stride, count_out, block_tables, \
-                       bt_stride, phys_out, seq_lens, block_size, sparse_seq_lens)
+    const dim3 grid(a.n_req, n_layers), block(64);
+#define UCM_TOPK_LAUNCH(EPL) hipLaunchKernelGGL((topk_windows_kernel<EPL, kHeapTies>), grid, block, 0, s, a)
     // registers per lane for the keys: the smallest tier that holds the longest request (the radix steps cost
     // one ballot per register and bit)
     if (max_seg_len <= 64) { UCM_TOPK_LAUNCH(1); }
@@ -205,32 +33,52 @@ extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride
     else if (max_seg_len <= 2048) { UCM_TOPK_LAUNCH(32); }
     else { UCM_TOPK_LAUNCH(64); }
 #undef UCM_TOPK_LAUNCH
+}
+
+}  // namespace
+
+extern "C" int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, int64_t scores_rows,
+                                const int32_t* seg_off, const int32_t* seg_len, const int32_t* topk_len, int n_req,
+                                int max_seg_len, int n_layers, int start_w, int end_w, int32_t* idx_out,
+                                int out_stride, int32_t* count_out, const int32_t* block_tables, int bt_stride,
+                                int32_t* phys_out, const int32_t* seq_lens, int block_size,
+                                int32_t* sparse_seq_lens, ucm_stream_t stream)
+{
+    UCM_REQUIRE(n_req == 0 || (scores && seg_off && seg_len && topk_len && idx_out && count_out),
+                "ucm_topk_windows: null pointer");
+    UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_topk_windows: n_req=%d n_layers=%d", n_req, n_layers);
+    UCM_REQUIRE(start_w >= 0 && end_w >= 0 && max_seg_len >= 0, "ucm_topk_windows: negative window or length");
+    UCM_REQUIRE(scores_rows >= 0 && (n_layers == 1 || scores_layer_stride >= scores_rows),
+                "ucm_topk_windows: scores_rows=%lld does not fit scores_layer_stride=%lld",
+                static_cast<long long>(scores_rows), static_cast<long long>(scores_layer_stride));
+    UCM_REQUIRE(out_stride >= max_seg_len, "ucm_topk_windows: out_stride=%d < max_seg_len=%d", out_stride, max_seg_len);
+    UCM_REQUIRE((block_tables == nullptr) == (phys_out == nullptr),
+                "ucm_topk_windows: block_tables and phys_out go together");
+    UCM_REQUIRE(!block_tables || bt_stride >= max_seg_len, "ucm_topk_windows: bt_stride=%d < max_seg_len=%d",
+                bt_stride, max_seg_len);
+    UCM_REQUIRE(!sparse_seq_lens || (seq_lens && block_size > 0), "ucm_topk_windows: sparse_seq_lens needs seq_lens and block_size");
+    UCM_SUPPORTED(max_seg_len <= 4096, "ucm_topk_windows: max_seg_len=%d (at most 4096 blocks per request)", max_seg_len);
+    if (n_req == 0) { return UCM_OK; }
+    const ucm::SelectArgs a = {scores, scores_layer_stride, scores_rows, seg_off, seg_len, topk_len, n_req, max_seg_len,
+                               start_w, end_w, idx_out, out_stride, static_cast<int64_t>(n_req) * out_stride, n_req, count_out, block_tables, bt_stride, phys_out, seq_lens, block_size,
+                               sparse_seq_lens};
+    launch_select<false>(a, max_seg_len, n_layers, ucm::as_stream(stream));
     UCM_LAUNCH_CHECK("ucm_topk_windows");
 }
 
-extern "C" int ucm_kvstar_topk(const float* votes, const int32_t* seg_off, const int32_t* seg_len,
+extern "C" int ucm_kvstar_topk(const float* votes, int64_t votes_rows, const int32_t* seg_off, const int32_t* seg_len,
                                const int32_t* topk_len, int n_tasks, int max_seg_len, int32_t* idx_out,
                                int out_stride, int32_t* count_out, ucm_stream_t stream)
 {
-    UCM_REQUIRE(n_tasks >= 0 && max_seg_len >= 0, "ucm_kvstar_topk: n_tasks=%d max_seg_len=%d", n_tasks, max_seg_len);
+    UCM_REQUIRE(n_tasks >= 0 && max_seg_len >= 0 && votes_rows >= 0, "ucm_kvstar_topk: n_tasks=%d max_seg_len=%d votes_rows=%lld",
+                n_tasks, max_seg_len, static_cast<long long>(votes_rows));
     if (n_tasks == 0) { return UCM_OK; }
     UCM_REQUIRE(votes && seg_off && seg_len && topk_len && idx_out && count_out, "ucm_kvstar_topk: null pointer");
     UCM_REQUIRE(out_stride >= max_seg_len, "ucm_kvstar_topk: out_stride=%d < max_seg_len=%d", out_stride, max_seg_len);
     UCM_SUPPORTED(max_seg_len <= 4096, "ucm_kvstar_topk: max_seg_len=%d (at most 4096 blocks per task)", max_seg_len);
-    hipStream_t s = ucm::as_stream(stream);
-    const dim3 grid(n_tasks, 1), block(64);
-#define UCM_HEAP_LAUNCH(EPL)                                                                                   \
-    hipLaunchKernelGGL((topk_windows_kernel<EPL, true>), grid, block, 0, s, votes, int64_t{0}, seg_off, seg_len, \
-                       topk_len, n_tasks, 0, 0, idx_out, out_stride, count_out, nullptr, 0, nullptr, nullptr, 1, \
-                       nullptr)
-    if (max_seg_len <= 64) { UCM_HEAP_LAUNCH(1); }
-    else if (max_seg_len <= 128) { UCM_HEAP_LAUNCH(2); }
-    else if (max_seg_len <= 256) { UCM_HEAP_LAUNCH(4); }
-    else if (max_seg_len <= 512) { UCM_HEAP_LAUNCH(8); }
-    else if (max_seg_len <= 1024) { UCM_HEAP_LAUNCH(16); }
-    else if (max_seg_len <= 2048) { UCM_HEAP_LAUNCH(32); }
-    else { UCM_HEAP_LAUNCH(64); }
-#undef UCM_HEAP_LAUNCH
+    const ucm::SelectArgs a = {votes, 0, votes_rows, seg_off, seg_len, topk_len, n_tasks, max_seg_len, 0, 0, idx_out, out_stride, 0, 0, count_out,
+                               nullptr, 0, nullptr, nullptr, 1, nullptr};
+    launch_select<true>(a, max_seg_len, 1, ucm::as_stream(stream));
     UCM_LAUNCH_CHECK("ucm_kvstar_topk");
 }
 
@@ -245,15 +93,18 @@ constexpr int kOrderThreads = 256;
 constexpr int kOrderMax = 4096;
 
 __global__ __launch_bounds__(kOrderThreads) void kvstar_order_kernel(
-    const float* __restrict__ votes, const int32_t* __restrict__ seg_off, const int32_t* __restrict__ seg_len,
-    int32_t* __restrict__ idx, int out_stride, const int32_t* __restrict__ count)
+    const float* __restrict__ votes, int64_t votes_rows, const int32_t* __restrict__ seg_off,
+    const int32_t* __restrict__ seg_len, int32_t* __restrict__ idx, int out_stride, const int32_t* __restrict__ count)
 {
     __shared__ unsigned long long keys[kOrderMax];
     const int t = blockIdx.x, tid = threadIdx.x;
-    const int k = min(count[t], min(out_stride, kOrderMax));
     const int n = seg_len[t];
+    const int64_t seg0 = seg_off[t];
+    // a task whose votes lie outside the array is left as it is (the selection wrote nothing for it either)
+    if (seg0 < 0 || n < 0 || seg0 + n > votes_rows) { return; }
+    const int k = min(count[t], min(out_stride, kOrderMax));
     int32_t* row = idx + static_cast<size_t>(t) * out_stride;
-    const float* v = votes + seg_off[t];
+    const float* v = votes + seg0;
     for (int j = tid; j < k; j += kOrderThreads) {
         const int i = row[j];
         const bool inside = i >= 0 && i < n;             // anything else was not written by the selection: never read
@@ -270,17 +121,18 @@ __global__ __launch_bounds__(kOrderThreads) void kvstar_order_kernel(
 
 }  // namespace
 
-extern "C" int ucm_kvstar_order(const float* votes, const int32_t* seg_off, const int32_t* seg_len, int n_tasks,
-                                int max_count, int32_t* idx_io, int out_stride, const int32_t* count,
+extern "C" int ucm_kvstar_order(const float* votes, int64_t votes_rows, const int32_t* seg_off, const int32_t* seg_len,
+                                int n_tasks, int max_count, int32_t* idx_io, int out_stride, const int32_t* count,
                                 ucm_stream_t stream)
 {
-    UCM_REQUIRE(n_tasks >= 0 && max_count >= 0, "ucm_kvstar_order: n_tasks=%d max_count=%d", n_tasks, max_count);
+    UCM_REQUIRE(n_tasks >= 0 && max_count >= 0 && votes_rows >= 0, "ucm_kvstar_order: n_tasks=%d max_count=%d votes_rows=%lld",
+                n_tasks, max_count, static_cast<long long>(votes_rows));
     if (n_tasks == 0 || max_count == 0) { return UCM_OK; }
     UCM_REQUIRE(votes && seg_off && seg_len && idx_io && count, "ucm_kvstar_order: null pointer");
     UCM_REQUIRE(out_stride >= max_count, "ucm_kvstar_order: out_stride=%d < max_count=%d", out_stride, max_count);
     UCM_SUPPORTED(max_count <= kOrderMax, "ucm_kvstar_order: max_count=%d (at most 4096 chosen blocks per task)", max_count);
-    hipLaunchKernelGGL(kvstar_order_kernel, dim3(n_tasks), dim3(kOrderThreads), 0, ucm::as_stream(stream), votes, seg_off,
-                       seg_len, idx_io, out_stride, count);
+    hipLaunchKernelGGL(kvstar_order_kernel, dim3(n_tasks), dim3(kOrderThreads), 0, ucm::as_stream(stream), votes,
+                       votes_rows, seg_off, seg_len, idx_io, out_stride, count);
     UCM_LAUNCH_CHECK("ucm_kvstar_order");
 }
 

@@ -146,24 +146,21 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
 def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor,
                  max_seg_len: int, kv_heads: int, scores: torch.Tensor,
                  q_rows: Optional[torch.Tensor] = None, first_layer: int = 0,
-                 n_layers: Optional[int] = None, total_blocks: int = 0, scale: float = 1.0) -> None:
-    """q: [L, rows, q_heads, head_dim] fp32 or bf16; repre: fp32 or bf16 [L, rows, kv_heads*head_dim];
+                 n_layers: Optional[int] = None, total_blocks: int = 0, scale: float = 1.0, num_repre: int = 1,
+                 tile_blocks: int = 0) -> None:
+    """q: [L, rows, q_heads, head_dim] fp32, bf16 or fp16; repre: fp32 or bf16 [L, rows, kv_heads*num_repre*head_dim];
     scores: fp32 [L, rows].  Layers first_layer .. first_layer+n_layers-1 are scored.
     total_blocks: sum of seg_len when the host knows it (tighter grid), else 0.  scale multiplies every score
-    (1/kv_heads: the mean over all q heads the reference's torch variant ranks by)."""
+    (1/kv_heads: the mean over all q heads the reference's torch variant ranks by).  tile_blocks: blocks per
+    workgroup, 0 = the library's choice (benchmarks and tests)."""
     if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
         raise ValueError("q [L,rows,Hq,D], repre [L,rows,Hkv*D], scores [L,rows] expected")
     head_dim, q_heads = q.shape[3], q.shape[2]
-    if repre.shape[2] != kv_heads * head_dim:
-        raise ValueError("repre row does not match kv_heads*head_dim")
+    if repre.shape[2] != kv_heads * num_repre * head_dim:
+        raise ValueError("repre row does not match kv_heads*num_repre*head_dim")
     if repre.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("repre must be float32 or bfloat16")
-    if q.dtype == torch.float32:
-        qd = _lib.DTYPE_F32
-    elif q.dtype == torch.bfloat16:
-        qd = _lib.DTYPE_BF16
-    else:
-        raise ValueError("q must be float32 or bfloat16")
+    qd = _q_code(q)
     n_layers = repre.shape[0] - first_layer if n_layers is None else n_layers
     if first_layer < 0 or first_layer + n_layers > min(q.shape[0], repre.shape[0], scores.shape[0]):
         raise ValueError("layer range outside the tables")
@@ -178,11 +175,64 @@ def score_blocks(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
     _lib.call("ucm_score_blocks", _dev(q, q.dtype, "q") + first_layer * q.stride(0) * es, qd, q.stride(0),
               _opt(q_rows, torch.int32, "q_rows"), q_heads,
               _dev(repre, repre.dtype, "repre") + first_layer * repre.stride(0) * repre.element_size(),
-              _lib.DTYPE_BF16 if repre.dtype == torch.bfloat16 else _lib.DTYPE_F32, repre.stride(0),
-              _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
+              _lib.DTYPE_BF16 if repre.dtype == torch.bfloat16 else _lib.DTYPE_F32, repre.stride(0), repre.shape[1],
+              num_repre, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_req, max_seg_len,
               total_blocks, n_layers, kv_heads, head_dim,
               _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4, scores.stride(0),
-              float(scale), _tuning["score_tile"], _stream())
+              float(scale), int(tile_blocks), _stream())
+
+
+def _q_code(q: torch.Tensor) -> int:
+    code = {torch.float32: _lib.DTYPE_F32, torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}.get(q.dtype)
+    if code is None:
+        raise ValueError("q must be float32, bfloat16 or float16")
+    return code
+
+
+def score_select(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor,
+                 topk_len: torch.Tensor, max_seg_len: int, kv_heads: int, scores: torch.Tensor, idx_out: torch.Tensor,
+                 count_out: torch.Tensor, tickets: torch.Tensor, start_w: int = 1, end_w: int = 2,
+                 q_rows: Optional[torch.Tensor] = None, block_tables: Optional[torch.Tensor] = None,
+                 phys_out: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None, block_size: int = 0,
+                 sparse_seq_lens: Optional[torch.Tensor] = None, first_layer: int = 0, n_layers: Optional[int] = None,
+                 scale: float = 1.0, num_repre: int = 1, tile_blocks: int = 0) -> None:
+    """score_blocks and topk_windows as one launch (ucm_score_select): q [L, rows, q_heads, head_dim] whose layer 0
+    belongs to ``first_layer``... of the tables; tickets int32 [L, n_req], zero before the first call and left zero."""
+    if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
+        raise ValueError("q [L,rows,Hq,D], repre [L,rows,Hkv*D], scores [L,rows] expected")
+    head_dim, q_heads = q.shape[3], q.shape[2]
+    if repre.shape[2] != kv_heads * num_repre * head_dim:
+        raise ValueError("repre row does not match kv_heads*num_repre*head_dim")
+    n_req = seg_off.numel()
+    n_layers = q.shape[0] if n_layers is None else n_layers
+    if first_layer < 0 or first_layer + n_layers > min(repre.shape[0], scores.shape[0], idx_out.shape[0]) or n_layers > q.shape[0]:
+        raise ValueError("layer range outside the tables")
+    if idx_out.dim() != 3 or idx_out.shape[1] != n_req or count_out.shape != idx_out.shape[:2] or tickets.shape != count_out.shape:
+        raise ValueError("idx_out [L,n_req,stride], count_out and tickets [L,n_req] expected")
+    if scores.shape[1] < repre.shape[1]:
+        raise ValueError("scores row shorter than the representative table")
+    if phys_out is not None and phys_out.shape != idx_out.shape:
+        raise ValueError("phys_out must have idx_out's shape")
+    if sparse_seq_lens is not None and sparse_seq_lens.shape != count_out.shape:
+        raise ValueError("sparse_seq_lens must have count_out's shape")
+    args = _lib.ScoreSelectArgs(
+        q=_dev(q, q.dtype, "q"), q_dtype=_q_code(q), q_heads=q_heads, q_layer_stride=q.stride(0),
+        q_rows=_opt(q_rows, torch.int32, "q_rows"), repre=_dev(repre, repre.dtype, "repre"),
+        repre_dtype=_lib.DTYPE_BF16 if repre.dtype == torch.bfloat16 else _lib.DTYPE_F32,
+        repre_layer_stride=repre.stride(0), repre_rows=repre.shape[1], seg_off=_dev(seg_off, torch.int32, "seg_off"),
+        seg_len=_dev(seg_len, torch.int32, "seg_len"), topk_len=_dev(topk_len, torch.int32, "topk_len"), n_req=n_req,
+        max_seg_len=max_seg_len, first_layer=first_layer, kv_heads=kv_heads, head_dim=head_dim,
+        scores=_dev(scores, torch.float32, "scores"), scores_layer_stride=scores.stride(0), tile_blocks=int(tile_blocks),
+        start_w=start_w, end_w=end_w, idx_out=_dev(idx_out, torch.int32, "idx_out"),
+        count_out=_dev(count_out, torch.int32, "count_out"), out_stride=idx_out.shape[2],
+        bt_stride=0 if block_tables is None else block_tables.shape[1],
+        block_tables=_opt(block_tables, torch.int32, "block_tables"), phys_out=_opt(phys_out, torch.int32, "phys_out"),
+        seq_lens=_opt(seq_lens, torch.int32, "seq_lens"), sparse_seq_lens=_opt(sparse_seq_lens, torch.int32, "sparse_seq_lens"),
+        block_size=block_size, tickets=_dev(tickets, torch.int32, "tickets"))
+    args.n_layers, args.num_repre, args.scale = n_layers, num_repre, float(scale)
+    import ctypes as C
+
+    _lib.call("ucm_score_select", C.addressof(args), _stream())
 
 
 def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tensor, topk_len: torch.Tensor,
@@ -207,7 +257,7 @@ def topk_windows(scores: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Ten
     o = first_layer * idx_out.stride(0) * 4
     c = first_layer * count_out.stride(0) * 4
     _lib.call("ucm_topk_windows", _dev(scores, torch.float32, "scores") + first_layer * scores.stride(0) * 4,
-              scores.stride(0), _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
+              scores.stride(0), scores.shape[1], _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
               _dev(topk_len, torch.int32, "topk_len"), n_req, max_seg_len, n_layers, start_w, end_w,
               _dev(idx_out, torch.int32, "idx_out") + o, idx_out.shape[2],
               _dev(count_out, torch.int32, "count_out") + c,
@@ -225,7 +275,7 @@ def kvstar_topk(votes: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tenso
     n_tasks = seg_off.numel()
     if idx_out.dim() != 2 or idx_out.shape[0] != n_tasks or count_out.numel() != n_tasks:
         raise ValueError("idx_out [n_tasks,stride] and count_out [n_tasks] expected")
-    _lib.call("ucm_kvstar_topk", _dev(votes, torch.float32, "votes"), _dev(seg_off, torch.int32, "seg_off"),
+    _lib.call("ucm_kvstar_topk", _dev(votes, torch.float32, "votes"), votes.numel(), _dev(seg_off, torch.int32, "seg_off"),
               _dev(seg_len, torch.int32, "seg_len"), _dev(topk_len, torch.int32, "topk_len"), n_tasks, max_seg_len,
               _dev(idx_out, torch.int32, "idx_out"), idx_out.shape[1], _dev(count_out, torch.int32, "count_out"),
               _stream())
@@ -238,7 +288,7 @@ def kvstar_order(votes: torch.Tensor, seg_off: torch.Tensor, seg_len: torch.Tens
     n_tasks = count.numel()
     if idx.dim() != 2 or idx.shape[0] != n_tasks or seg_off.numel() != n_tasks or seg_len.numel() != n_tasks:
         raise ValueError("idx [n_tasks, stride] and seg_off, seg_len, count [n_tasks] expected")
-    _lib.call("ucm_kvstar_order", _dev(votes, torch.float32, "votes"), _dev(seg_off, torch.int32, "seg_off"),
+    _lib.call("ucm_kvstar_order", _dev(votes, torch.float32, "votes"), votes.numel(), _dev(seg_off, torch.int32, "seg_off"),
               _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_count, _dev(idx, torch.int32, "idx"), idx.shape[1],
               _dev(count, torch.int32, "count"), _stream())
 
@@ -382,9 +432,10 @@ HASH_SCORE_SUM, HASH_SCORE_BLOCK_CODE = 0, 1
 def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                        n: int, w: torch.Tensor, block_size: int, kv_heads: int, num_blocks: int,
                        colsum: torch.Tensor, block_codes: torch.Tensor,
-                       token_codes: Optional[torch.Tensor] = None) -> None:
+                       token_codes: Optional[torch.Tensor] = None, workgroups: int = 0) -> None:
     """w bf16 [128, 128]; colsum int16 [L, rows, kv_heads, 128]; block_codes uint8 [L, rows, kv_heads, 16];
-    token_codes uint8 [L, rows, block_size, kv_heads, 16] or None."""
+    token_codes uint8 [L, rows, block_size, kv_heads, 16] or None; workgroups: persistent workgroups over all
+    layers, 0 = the library's choice (benchmarks and tests)."""
     if w.shape != (128, 128):
         raise ValueError("w must be [128, 128] bfloat16")
     n_layers, rows = colsum.shape[0], colsum.shape[1]
@@ -398,7 +449,7 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
               _opt(slots, torch.int32, "slots"), n, block_size, kv_heads, 128, _dev(w, torch.bfloat16, "w"), 128, rows,
               _opt(token_codes, torch.uint8, "token_codes"), 0 if token_codes is None else token_codes.stride(0),
               _dev(colsum, torch.int16, "colsum"), colsum.stride(0), _dev(block_codes, torch.uint8, "block_codes"),
-              block_codes.stride(0), _tuning["hash_encode_groups"], _stream())
+              block_codes.stride(0), int(workgroups), _stream())
 
 
 def hash_encode_queries(q: torch.Tensor, w: torch.Tensor, kv_heads: int, q_codes: torch.Tensor, q_sum: torch.Tensor,
@@ -426,7 +477,7 @@ def hash_score_blocks(mode: int, q_sum: torch.Tensor, qbar_codes: torch.Tensor, 
         raise ValueError("scores must be [L, >= rows]")
     _lib.call("ucm_hash_score_blocks", mode, _dev(q_sum, torch.int16, "q_sum"), _dev(qbar_codes, torch.uint8, "qbar_codes"),
               _dev(colsum, torch.int16, "colsum"), colsum.stride(0), _dev(block_codes, torch.uint8, "block_codes"),
-              block_codes.stride(0), _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
+              block_codes.stride(0), rows, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"),
               n_req, total_blocks, n_layers, kv_heads, 128, _dev(scores, torch.float32, "scores"), scores.stride(0),
               int(round_fp16), _stream())
 
@@ -553,14 +604,14 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
 
 
 def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks: int, sub_blocks: int, d_pad: int,
-                     device) -> tuple:
+                     device, tiles_per_wave: int = 0) -> tuple:
     """Scratch of ucm_kvstar_votes for a call of this shape; rows_per_head = query tokens * (q_heads / kv_heads),
-    d_pad = padded channels per representative (the table's d_pad)."""
+    d_pad = padded channels per representative (the table's d_pad); tiles_per_wave as passed to the votes call."""
     import ctypes as C
 
     a, b = C.c_int64(0), C.c_int64(0)
     _lib.call("ucm_kvstar_workspace_floats", n_tasks, kv_heads, rows_per_head, max_blocks, sub_blocks, d_pad,
-              _tuning["kvstar_tiles_per_wave"], C.addressof(a), C.addressof(b))
+              int(tiles_per_wave), C.addressof(a), C.addressof(b))
     return (torch.empty(max(a.value, 1), dtype=torch.float32, device=device),
             torch.empty(max(b.value, 1), dtype=torch.float32, device=device))
 
@@ -568,7 +619,7 @@ def kvstar_workspace(n_tasks: int, kv_heads: int, rows_per_head: int, max_blocks
 def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: int, repre: torch.Tensor,
                  seg_off: torch.Tensor, seg_len: torch.Tensor, max_blocks: int, votes: torch.Tensor, workspace: tuple,
                  d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
-                 pruned_sel: Optional[torch.Tensor] = None) -> None:
+                 pruned_sel: Optional[torch.Tensor] = None, tiles_per_wave: int = 0) -> None:
     """q fp16 (any shape; task t reads [n_tokens, q_heads, d_orig] from element q_off[t]); repre: one layer of a
     kvstar_table, fp16 [kv_heads, rows, d_pad/8, M, 8] (head planes may be strided: a row slice of a bigger
     table is fine); votes fp32 [>= rows]; pruned int32 [n_lists, kv_heads, d_pruned]."""
@@ -590,17 +641,17 @@ def kvstar_votes(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: i
     if votes.numel() < rows:
         raise ValueError("votes shorter than the representative table")
     ws_max, ws_part = workspace
-    _lib.call("ucm_kvstar_votes", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
-              _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), repre.data_ptr(), head_stride,
-              row_stride, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m,
+    _lib.call("ucm_kvstar_votes", _dev(q, torch.float16, "q"), q.numel(), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads,
+              d_orig, _opt(pruned, torch.int32, "pruned"), 0 if pruned is None else pruned.shape[0],
+              _opt(pruned_sel, torch.int32, "pruned_sel"), repre.data_ptr(), rows, head_stride, row_stride, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m,
               kv_heads, d_pruned, d_pad, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
-              _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
+              _dev(votes, torch.float32, "votes"), int(tiles_per_wave), _stream())
 
 
 def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_heads: int, tables, seg_off: torch.Tensor,
                         seg_len: torch.Tensor, max_blocks: int, votes: torch.Tensor, workspace: tuple,
                         d_pruned: Optional[int] = None, pruned: Optional[torch.Tensor] = None,
-                        pruned_sel: Optional[torch.Tensor] = None):
+                        pruned_sel: Optional[torch.Tensor] = None, tiles_per_wave: int = 0):
     """kvstar_votes for tasks that each bring a table of their own: tables[t] fp16 [kv_heads, rows_t, d_pad/8, M, 8]
     (block 0 of task t = its row 0); seg_off only places the votes.  Returns the device pointer arrays, which the
     caller keeps alive until the stream has run the call."""
@@ -630,26 +681,10 @@ def kvstar_votes_tables(q: torch.Tensor, q_off: torch.Tensor, n_tokens: int, q_h
         d_pruned = d_orig
     dev = upload(torch.tensor([[t.data_ptr() for t in tables], [hs for hs, _ in strides]], dtype=torch.int64), tables[0].device)
     ws_max, ws_part = workspace
-    _lib.call("ucm_kvstar_votes_tables", _dev(q, torch.float16, "q"), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads, d_orig,
-              _opt(pruned, torch.int32, "pruned"), _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
+    _lib.call("ucm_kvstar_votes_tables", _dev(q, torch.float16, "q"), q.numel(), _dev(q_off, torch.int64, "q_off"), n_tokens, q_heads,
+              d_orig, _opt(pruned, torch.int32, "pruned"), 0 if pruned is None else pruned.shape[0],
+              _opt(pruned_sel, torch.int32, "pruned_sel"), dev[0].data_ptr(), dev[1].data_ptr(),
               row_stride, _dev(seg_off, torch.int32, "seg_off"), _dev(seg_len, torch.int32, "seg_len"), n_tasks, max_blocks, m,
               kv_heads, d_pruned, pieces * 8, _dev(ws_max, torch.float32, "ws_max"), ws_max.numel(), _dev(ws_part, torch.float32, "ws_part"), ws_part.numel(),
-              _dev(votes, torch.float32, "votes"), _tuning["kvstar_tiles_per_wave"], _stream())
+              _dev(votes, torch.float32, "votes"), votes.numel(), int(tiles_per_wave), _stream())
     return dev
-
-
-# Launch-shape arguments of three entry points that only benchmarks and tests change (0 = the library's default).
-# They are plain per-call arguments of the C ABI; these helpers set what the wrappers of THIS module pass.
-_tuning = {"score_tile": 0, "hash_encode_groups": 0, "kvstar_tiles_per_wave": 0}
-
-
-def set_score_tile(tile_blocks: int) -> None:
-    _tuning["score_tile"] = int(tile_blocks)
-
-
-def set_kvstar_tiles_per_wave(tiles: int) -> None:
-    _tuning["kvstar_tiles_per_wave"] = int(tiles)
-
-
-def set_hash_encode_groups(workgroups: int) -> None:
-    _tuning["hash_encode_groups"] = int(workgroups)

@@ -24,6 +24,7 @@ handed (``scheduler_output.num_scheduled_tokens``, ``requests[id].block_ids``,
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from itertools import accumulate
 from typing import Dict, List, Optional, Union
@@ -43,6 +44,7 @@ from ..utils import (
 )
 
 ReqType = Union[str, int]
+_Q_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16}
 
 
 class GSAReqStat:
@@ -206,6 +208,7 @@ class GSA(UcmSparseBase):
         self._kv_all: Optional[ops.LayerPointers] = None   # every layer's (2, blocks, ...) cache, for whole-block moves
         self._kv_full: Dict[int, torch.Tensor] = {}
         self._scored: set = set()  # sparsified requests whose blocks have been scored at least once
+        self._layer_of: Dict[str, int] = {}
 
     # ------------------------------------------------------------------ device state
     def _ensure_device_state(self, device) -> None:
@@ -235,6 +238,22 @@ class GSA(UcmSparseBase):
         ]
         self._repre_code = _lib.DTYPE_BF16 if self.repre_dtype == torch.bfloat16 else _lib.DTYPE_F32
         self._views: Dict[int, list] = {}  # batch size -> per-layer (block table, sequence lengths) views
+        # scoring and selection of a layer are ONE library call with ONE argument block: everything that does not
+        # change between layers is filled in here and in execute_begin, attention_begin sets the layer and its
+        # queries.  The ticket counters of the fused launch are zero between calls.
+        self.tickets = torch.zeros((L, self.max_bs), dtype=torch.int32, device=device)
+        self._sel = _lib.ScoreSelectArgs(
+            q_heads=self.num_q_heads, repre=self.kpre_caches.data_ptr(), repre_dtype=self._repre_code,
+            repre_layer_stride=self.kpre_caches.stride(0), repre_rows=rows, kv_heads=self.num_key_heads,
+            head_dim=self.head_size, scores=self.scores.data_ptr(), scores_layer_stride=self.scores.stride(0),
+            start_w=self.init_window, end_w=self.local_window, idx_out=self.topk_caches.data_ptr(),
+            count_out=self.topk_counts.data_ptr(), out_stride=self.max_block_len, bt_stride=self.max_block_len,
+            phys_out=self.block_tables_mp.data_ptr(), sparse_seq_lens=self.gsa_seq_len.data_ptr(),
+            block_size=self.block_size, tickets=self.tickets.data_ptr(),
+            idx_layer_stride=self.topk_caches.stride(0), count_layer_stride=self.topk_counts.stride(0))
+        self._sel_addr = ctypes.addressof(self._sel)
+        self._score_select = _lib.lib().ucm_score_select
+        self._fused_ok = self.max_block_len <= 1024     # longer requests take the two launches
         self._dev_ready = True
 
     def register_kv_caches(self, kv_caches: dict) -> None:
@@ -290,7 +309,7 @@ class GSA(UcmSparseBase):
 
     def maybe_register_kv_cache(self, forward_context, layer_name: str) -> None:
         attn = forward_context.no_compile_layers[layer_name]
-        self._register_layer(int(layer_name.split(".")[2]), attn.kv_cache[forward_context.virtual_engine])
+        self._register_layer(self._layer_id(layer_name), attn.kv_cache[forward_context.virtual_engine])
 
     # ------------------------------------------------------------------ per-step metadata
     def build_sparse_meta(self, scheduler_output, requests, input_batch, attn_metadata) -> None:
@@ -385,6 +404,9 @@ class GSA(UcmSparseBase):
         )
         self.model_input["addr"] = (d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), d[4].data_ptr(),
                                     self.model_input["block_tables"].data_ptr())
+        a = self._sel
+        a.seg_off, a.seg_len, a.topk_len, a.q_rows, a.seq_lens, a.block_tables = self.model_input["addr"]
+        a.n_req, a.max_seg_len = batch, max_len
 
     def execute_finished(self) -> None:
         if self.ptopk_prefetch:
@@ -392,32 +414,46 @@ class GSA(UcmSparseBase):
         self.step_count += 1
 
     # ------------------------------------------------------------------ per-layer hooks
+    def _layer_id(self, layer_name: str) -> int:
+        l = self._layer_of.get(layer_name)
+        if l is None:
+            l = self._layer_of[layer_name] = int(layer_name.split(".")[2])
+        return l
+
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
         self.maybe_register_kv_cache(forward_context, layer_name)
         mi = self.model_input
         if not mi.get("any_gsa") or "seg_off" not in mi:
             return
-        l = int(layer_name.split(".")[2])
+        l = self._layer_id(layer_name)
         n = mi["n_batch"]
-        seg_off, seg_len, topk_len, q_rows, seq_lens, tables = mi["addr"]
-        repre, scores, idx, counts, phys, sparse_len = self._layer_addr[l]
         stream = ops.current_stream()
         if mi["is_topk"]:
-            if query.dtype == torch.bfloat16:
-                q_code = _lib.DTYPE_BF16
-            elif query.dtype == torch.float32:
-                q_code = _lib.DTYPE_F32
-            else:
-                raise ValueError("query must be bfloat16 or float32")
+            q_code = _Q_CODES.get(query.dtype)
+            if q_code is None:
+                raise ValueError("query must be bfloat16, float16 or float32")
             if not (query.is_cuda and query.is_contiguous()) or query.shape[-1] != self.head_size:
                 raise ValueError("query must be a contiguous device tensor [tokens, q_heads, head_size]")
-            _lib.call("ucm_score_blocks", query.data_ptr(), q_code, query.numel(), q_rows, self.num_q_heads, repre,
-                      self._repre_code, self.kpre_caches.stride(0), seg_off, seg_len, n, mi["max_len"], mi["total"], 1,
-                      self.num_key_heads, self.head_size, scores, self.scores.stride(0), 1.0, 0, stream)
-        # selection (fresh scores, or the last ones with this step's lengths), block-table lookup, sparse lengths
-        _lib.call("ucm_topk_windows", scores, self.scores.stride(0), seg_off, seg_len, topk_len, n, mi["max_len"], 1,
-                  self.init_window, self.local_window, idx, self.max_block_len, counts, tables, self.max_block_len, phys,
-                  seq_lens, self.block_size, sparse_len, stream)
+        if mi["is_topk"] and self._fused_ok:
+            # scores of every block and the selection from them: one launch (the last scoring workgroup of a
+            # request runs its selection), block-table lookup and sparse lengths on the way out
+            a = self._sel
+            a.q, a.q_dtype, a.q_layer_stride, a.first_layer = query.data_ptr(), q_code, query.numel(), l
+            rc = self._score_select(self._sel_addr, stream)
+            if rc != 0:
+                raise _lib.UcmHipError("ucm_score_select", rc, _lib.lib().ucm_last_error().decode())
+        else:
+            seg_off, seg_len, topk_len, q_rows, seq_lens, tables = mi["addr"]
+            repre, scores, idx, counts, phys, sparse_len = self._layer_addr[l]
+            rows = self.kpre_caches.shape[1]
+            if mi["is_topk"]:
+                _lib.call("ucm_score_blocks", query.data_ptr(), q_code, query.numel(), q_rows, self.num_q_heads, repre,
+                          self._repre_code, self.kpre_caches.stride(0), rows, 1, seg_off, seg_len, n, mi["max_len"],
+                          mi["total"], 1, self.num_key_heads, self.head_size, scores, self.scores.stride(0), 1.0, 0, stream)
+            # selection from the last scores with this step's lengths, block-table lookup, sparse lengths
+            _lib.call("ucm_topk_windows", scores, self.scores.stride(0), rows, seg_off, seg_len, topk_len, n, mi["max_len"],
+                      1, self.init_window, self.local_window, idx, self.max_block_len, counts, tables, self.max_block_len,
+                      phys, seq_lens, self.block_size, sparse_len, stream)
         views = self._views.get(n)
         if views is None:
             views = self._views[n] = [(self.block_tables_mp[k, :n], self.gsa_seq_len[k, :n]) for k in range(self.layer_num)]
@@ -426,15 +462,16 @@ class GSA(UcmSparseBase):
         md.block_table, md.seq_lens = views[l]
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
-        self.maybe_register_kv_cache(forward_context, layer_name)
-        self.copy_k(layer_name, forward_context)
+        # (the layer's cache was looked at in attention_begin of the same step)
+        if self.model_input.get("calc_block_table"):
+            self.copy_k(layer_name, forward_context)
 
     def copy_k(self, layer_name: str, forward_context) -> None:
         """Representatives of the blocks this step filled (gsa.py:634-654), reduced in place on the device."""
         blocks = self.model_input.get("calc_block_table") or []
         if not blocks:
             return
-        l = int(layer_name.split(".")[2])
+        l = self._layer_id(layer_name)
         if "calc_blocks_dev" in self.model_input:
             ids, slots = self.model_input["calc_blocks_dev"], self.model_input["calc_slots_dev"]
         else:  # a step without any sparsified request still has to keep the table current
