@@ -200,9 +200,7 @@ def main():
         else:
             # one launch: the last scoring workgroup of a (layer, request) runs its selection
             ops.score_select(q, repre, seg_off, seg_len, topk_d, max_len, HKV, scores, idx, cnt, tickets, block_tables=bt,
-                             phys_out=phys)
-            if events:
-                events[1].record()
+                             phys_out=phys, total_blocks=rows)
         if events:
             events[2].record()
         ops.kv_gather_selected(layers, kv_stride, BLOCK_BYTES, nb, phys, cnt, dst_off, region, max_k, staging,
@@ -230,8 +228,12 @@ def main():
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    k_ms = np.array([[e[i].elapsed_time(e[i + 1]) for i in range(3)] for e in all_events]).mean(0)
-    score_ms, topk_ms, gather_ms = (float(x) for x in k_ms)
+    if args.two_launch:
+        k_ms = np.array([[e[i].elapsed_time(e[i + 1]) for i in range(3)] for e in all_events]).mean(0)
+        score_ms, topk_ms, gather_ms = (float(x) for x in k_ms)
+    else:       # one launch scores and selects: two spans per step
+        k_ms = np.array([[e[0].elapsed_time(e[2]), e[2].elapsed_time(e[3])] for e in all_events]).mean(0)
+        score_ms, topk_ms, gather_ms = float(k_ms[0]), 0.0, float(k_ms[1])
 
     n_sel = int(topk.astype(np.int64).sum()) * n_layers
     gather_bytes = 2 * n_sel * 2 * BLOCK_BYTES                                     # K and V, read + write

@@ -196,6 +196,7 @@ int ucm_topk_windows(const float* scores, int64_t scores_layer_stride, int64_t s
  *              0 = dense (n_req*out_stride and n_req).  A caller that keeps
  *              persistent [layers][max_requests][...] tables and runs a batch of
  *              fewer requests names the tables' own strides.
+ *   total_blocks  as for ucm_score_blocks (0 = unknown)
  *   tickets    dev int32 [layers][n_req] (indexed like count_out): zero before
  *              the first call; every call leaves it zero.  Calls that overlap
  *              in time (different streams) need arrays of their own.
@@ -241,6 +242,7 @@ typedef struct ucm_score_select_args {
     int32_t* tickets;
     int64_t idx_layer_stride;
     int64_t count_layer_stride;
+    int64_t total_blocks;
 } ucm_score_select_args_t;
 int ucm_score_select(const ucm_score_select_args_t* args, ucm_stream_t stream);
 

@@ -131,11 +131,13 @@ def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=to
         fused = dict(scores=torch.full_like(scores, -123.0), idx=torch.full_like(idx, -1), cnt=torch.full_like(cnt, -1),
                      phys=None if phys is None else torch.full_like(phys, -1), sps=None if sps is None else torch.full_like(sps, -1))
         tickets = torch.zeros_like(cnt)
-        for _ in range(2):                                   # twice: the tickets must come back to zero
+        # twice: the tickets must come back to zero; the second time with a total that understates the batch, so
+        # that the grid is short and workgroups go on to a second and third tile
+        for total in (0, max(int(lens.sum()) // 3, 1)):
             ops.score_select(q, repre, i32(off, dev), i32(lens, dev), i32(topk, dev), mx, hkv, fused["scores"], fused["idx"],
                              fused["cnt"], tickets, start_w=sw, end_w=ew, q_rows=None if q_rows is None else i32(q_rows, dev),
                              block_tables=bt, phys_out=fused["phys"], seq_lens=sl, block_size=block_size,
-                             sparse_seq_lens=fused["sps"], tile_blocks=tile)
+                             sparse_seq_lens=fused["sps"], tile_blocks=tile, total_blocks=total)
             torch.cuda.synchronize()
             assert not tickets.any(), "tickets left non-zero"
         assert torch.equal(fused["scores"].view(torch.int32), scores.view(torch.int32)), "fused scores differ"

@@ -81,7 +81,7 @@ class ScoreSelectArgs(C.Structure):
         ("scale", _f), ("tile_blocks", _i), ("start_w", _i), ("end_w", _i), ("idx_out", _p), ("count_out", _p),
         ("out_stride", _i), ("bt_stride", _i), ("block_tables", _p), ("phys_out", _p), ("seq_lens", _p),
         ("sparse_seq_lens", _p), ("block_size", _i), ("reserved", _i), ("tickets", _p),
-        ("idx_layer_stride", _i64), ("count_layer_stride", _i64),
+        ("idx_layer_stride", _i64), ("count_layer_stride", _i64), ("total_blocks", _i64),
     ]
 
     def __init__(self, **kw):

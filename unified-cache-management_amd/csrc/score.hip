@@ -188,7 +188,7 @@ struct TileInfo {
 template <int kD>
 __device__ __forceinline__ bool locate(const ScoreArgs& a, int lane, TileInfo& t)
 {
-    if (!find_tile(a.seg_len, a.n_req, a.tile_blocks, a.max_seg_len, a.tickets ? 1 : 0, blockIdx.x, lane, t.r, t.tile)) {
+    if (!find_tile(a.seg_len, a.n_req, a.tile_blocks, a.max_seg_len, a.tickets ? 1 : 0, blockIdx.y, lane, t.r, t.tile)) {
         return false;
     }
     t.n = clamped_len(a.seg_len[t.r], a.max_seg_len);
@@ -230,37 +230,51 @@ __device__ __forceinline__ float head_sum(float dot, int first, int step, int kv
     return s;
 }
 
-// The fused kernel's tail.  Every workgroup of a request takes a ticket once its scores are visible to the
-// device; the one that draws the last ticket resets the counter and its first wave runs the request's
-// selection (TopkBlockSelector::TopKImpl, select_topk_block.cpp:20-51) on the scores all of them wrote.
-__device__ __forceinline__ void select_if_last(const ScoreArgs& a, const ucm::SelectArgs& sel, const TileInfo& t, int l)
+// A score on its way out.  With the selection fused in, another workgroup of this launch reads it: the store then
+// goes through to memory at device scope (no cache of another part of the chip keeps it back), and the reader
+// uses device-scope loads.
+__device__ __forceinline__ void store_score(float* p, float v, bool through)
 {
-    __shared__ int s_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");           // this thread's scores, before the ticket below
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int32_t* ticket = a.tickets + static_cast<int64_t>(l) * sel.cnt_layer_stride + t.r;
-        const int tiles = max((t.n + a.tile_blocks - 1) / a.tile_blocks, 1);
-        const int drawn = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = drawn == tiles - 1;
-        if (s_last) { __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-    }
-    __syncthreads();
-    if (!s_last || threadIdx.x >= 64) { return; }
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");           // the other workgroups' scores, after their tickets
-    const int lane = threadIdx.x;
-    // the smallest tier of key registers that holds the request (the host allows at most 1024 blocks here)
-    if (t.n <= 64) { ucm::select_wave<1, false>(sel, t.r, l, lane); }
-    else if (t.n <= 128) { ucm::select_wave<2, false>(sel, t.r, l, lane); }
-    else if (t.n <= 256) { ucm::select_wave<4, false>(sel, t.r, l, lane); }
-    else if (t.n <= 512) { ucm::select_wave<8, false>(sel, t.r, l, lane); }
-    else { ucm::select_wave<16, false>(sel, t.r, l, lane); }
+    if (through) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    else { *p = v; }
 }
 
-// grid: x = dense tile index over all requests (workgroups past the last tile
-// exit), y = layer.  Tiles are numbered densely so that consecutive workgroups,
-// which the hardware deals round-robin to the 8 XCDs, always carry work: with a
-// (tile, request) grid the short requests of a ragged batch leave most XCDs idle.
+// The fused kernel's tail.  Every workgroup of a request takes a ticket once its scores have reached memory; the
+// one that draws the last ticket resets the counter and its first wave runs the request's selection
+// (TopkBlockSelector::TopKImpl, select_topk_block.cpp:20-51) on the scores all of them wrote.  Ordering: a wave's
+// score stores are device-scope write-through stores, complete when the wave's memory counter reaches zero (the
+// workgroup-scope fence below waits for that); the barrier then orders all waves' stores before thread 0's ticket;
+// the last workgroup reads the scores with device-scope loads after it has seen every other ticket.  (A
+// device-scope release/acquire pair would also do, but it writes the whole L2 back per wave: 7x the kernel's time.)
+__device__ __forceinline__ void select_if_last(const ScoreArgs& a, const ucm::SelectArgs& sel, const TileInfo& t, int l)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x >= 64) { return; }                           // the other waves are done: their registers are free again
+    const int lane = threadIdx.x;
+    int drawn = 0;
+    int32_t* ticket = a.tickets + static_cast<int64_t>(l) * sel.cnt_layer_stride + t.r;
+    if (lane == 0) { drawn = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    drawn = __builtin_amdgcn_readfirstlane(drawn);
+    const int tiles = max((t.n + a.tile_blocks - 1) / a.tile_blocks, 1);
+    if (drawn != tiles - 1) { return; }
+    if (lane == 0) { __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    // the smallest tier of key registers that holds the request (the host allows at most 1024 blocks here)
+    if (t.n <= 64) { ucm::select_wave<1, false, true>(sel, t.r, l, lane); }
+    else if (t.n <= 128) { ucm::select_wave<2, false, true>(sel, t.r, l, lane); }
+    else if (t.n <= 256) { ucm::select_wave<4, false, true>(sel, t.r, l, lane); }
+    else if (t.n <= 512) { ucm::select_wave<8, false, true>(sel, t.r, l, lane); }
+    else { ucm::select_wave<16, false, true>(sel, t.r, l, lane); }
+}
+
+// grid: x = layer, y = dense tile index over all requests (workgroups past the
+// last tile exit).  Tiles are numbered densely and the layers run fastest, so that
+// consecutive workgroups, which the hardware deals round-robin to the 8 XCDs,
+// always carry work (with a (tile, request) grid the short requests of a ragged
+// batch leave most XCDs idle) and the workgroups without a tile - the host sizes
+// the grid from its own bounds on the segment lengths - are dispatched last: in
+// between the others each of them held a workgroup's registers and LDS for the
+// time it takes to find that out (12 us for 1600 of them among 2500).
 template <int kD, typename QT>
 __global__ __launch_bounds__(kThreads) void score_kernel(const ScoreArgs a, const ucm::SelectArgs sel)
 {
@@ -268,7 +282,8 @@ __global__ __launch_bounds__(kThreads) void score_kernel(const ScoreArgs a, cons
     __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int l = blockIdx.y;
+    const int l = blockIdx.x;
+    const bool fused = a.tickets != nullptr;
     TileInfo t;
     if (!locate<kD>(a, lane, t)) { return; }
     const int tile0 = t.tile * a.tile_blocks;
@@ -309,7 +324,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(const ScoreArgs a, cons
             const float dot = quad_dot<kSteps>(qr, kv);
             const float s = head_sum(dot, bl * vecs * 4, 4, a.kv_heads, a.num_repre);
             const int b = base + bl;
-            if (b < tile_end && vb == 0 && m == 0) { sout[b] = s * a.scale; }   // (a scale of 1 changes no bit)
+            if (b < tile_end && vb == 0 && m == 0) { store_score(sout + b, s * a.scale, fused); }   // (a scale of 1 changes no bit)
         };
         while (b0 < tile_end) {
             const int b1 = b0 + stride;
@@ -322,7 +337,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel(const ScoreArgs a, cons
             b0 = b2;
         }
     }
-    if (a.tickets) { select_if_last(a, sel, t, l); }
+    if (fused) { select_if_last(a, sel, t, l); }
 }
 
 // ---- bf16 representative table ------------------------------------------------
@@ -373,7 +388,8 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(const ScoreArgs a,
     __shared__ __attribute__((aligned(16))) float qbar[kMaxRow];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int l = blockIdx.y;
+    const int l = blockIdx.x;
+    const bool fused = a.tickets != nullptr;
     TileInfo t;
     if (!locate<kD>(a, lane, t)) { return; }
     const int tile0 = t.tile * a.tile_blocks;
@@ -416,7 +432,8 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(const ScoreArgs a,
         auto finish = [&](const u32x4 (&kv)[kSteps], int base) {
             const float dot = pair_dot<kSteps>(qlo, qhi, kv);
             const float s = head_sum(dot, bl * vecs * 2, 2, a.kv_heads, a.num_repre);
-            sout[min(base + bl, tile_end - 1)] = s * a.scale;   // the lanes of a block all hold its score; a scale of 1 changes no bit
+            // the lanes of a block all hold its score; a scale of 1 changes no bit
+            store_score(sout + min(base + bl, tile_end - 1), s * a.scale, fused);
         };
         while (b0 < tile_end) {
             const int b1 = b0 + stride;
@@ -431,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(const ScoreArgs a,
             b0 = b2;
         }
     }
-    if (a.tickets) { select_if_last(a, sel, t, l); }
+    if (fused) { select_if_last(a, sel, t, l); }
 }
 
 template <int kD, typename QT>
@@ -489,11 +506,11 @@ int score_launch(const char* name, const void* q, int q_dtype, int64_t q_layer_s
     // (with the selection fused in, every tile of every request has to run, whatever seg_len holds: the
     // caller's total is not used to shrink the grid)
     if (total_blocks > 0 && !sel) { tile_bound = std::min(tile_bound, (total_blocks + tile_blocks - 1) / tile_blocks + n_req); }
-    UCM_REQUIRE(tile_bound <= 0x7fffffffll, "%s: too many tiles for one launch", name);
+    UCM_REQUIRE(tile_bound <= 65535, "%s: too many tiles for one launch (%lld)", name, static_cast<long long>(tile_bound));
     const ScoreArgs a = {q, q_layer_stride, q_rows, q_heads, repre, repre_layer_stride, repre_rows, seg_off, seg_len, n_req,
                          max_seg_len, kv_heads, num_repre, scores, scores_layer_stride, tile_blocks, scale, sel ? tickets : nullptr};
     const ucm::SelectArgs none = {};
-    const dim3 grid(static_cast<unsigned>(tile_bound), n_layers);
+    const dim3 grid(n_layers, static_cast<unsigned>(tile_bound));
     hipStream_t s = ucm::as_stream(stream);
     const bool bf16_table = repre_dtype == UCM_DTYPE_BF16;
     switch (head_dim) {
@@ -556,7 +573,8 @@ extern "C" int ucm_score_select(const ucm_score_select_args_t* p, ucm_stream_t s
                                  p->phys_out ? p->phys_out + first * idx_ls : nullptr, p->seq_lens, p->block_size,
                                  p->sparse_seq_lens ? p->sparse_seq_lens + first * cnt_ls : nullptr};
     return score_launch("ucm_score_select", p->q, p->q_dtype, p->q_layer_stride, p->q_rows, p->q_heads, repre, p->repre_dtype,
-                        p->repre_layer_stride, p->repre_rows, p->num_repre, p->seg_off, p->seg_len, n_req, p->max_seg_len, 0,
+                        p->repre_layer_stride, p->repre_rows, p->num_repre, p->seg_off, p->seg_len, n_req, p->max_seg_len,
+                        p->total_blocks,
                         n_layers, p->kv_heads, p->head_dim, scores, p->scores_layer_stride, p->scale, p->tile_blocks, &sel,
                         p->tickets + first * cnt_ls, stream);
 }

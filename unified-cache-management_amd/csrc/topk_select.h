@@ -69,7 +69,11 @@ struct SelectArgs {
 //
 // Called by all 64 lanes of one wave for request r of layer l; kEpl * 64 is the
 // longest request the instance holds (longer ones are cut there: host checked).
-template <int kEpl, bool kHeapTies>
+//
+// kCoherent: the scores were written by other workgroups of the SAME launch (device-scope stores that went through
+// to memory); they are read with device-scope loads, which do not take a line that an L2 of another part of the
+// chip may still hold in an older state.
+template <int kEpl, bool kHeapTies, bool kCoherent = false>
 __device__ __forceinline__ void select_wave(const SelectArgs& a, int r, int l, int lane)
 {
     const int start_w = a.start_w, end_w = a.end_w, out_stride = a.out_stride;
@@ -116,7 +120,9 @@ __device__ __forceinline__ void select_wave(const SelectArgs& a, int r, int l, i
         for (int j = 0; j < kEpl; ++j) {
             const int i = j * 64 + lane;
             const bool cand = i >= start_w && i < hi;
-            key[j] = cand ? ordered_key(s[cand ? i : 0]) : 0u;
+            const float* sp = s + (cand ? i : 0);
+            const float sv = kCoherent ? __hip_atomic_load(sp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *sp;
+            key[j] = cand ? ordered_key(sv) : 0u;
             phys[j] = bt ? bt[min(i, n - 1)] : 0;
         }
         unsigned T = 0;

@@ -195,7 +195,7 @@ def score_select(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
                  q_rows: Optional[torch.Tensor] = None, block_tables: Optional[torch.Tensor] = None,
                  phys_out: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None, block_size: int = 0,
                  sparse_seq_lens: Optional[torch.Tensor] = None, first_layer: int = 0, n_layers: Optional[int] = None,
-                 scale: float = 1.0, num_repre: int = 1, tile_blocks: int = 0) -> None:
+                 scale: float = 1.0, num_repre: int = 1, tile_blocks: int = 0, total_blocks: int = 0) -> None:
     """score_blocks and topk_windows as one launch (ucm_score_select): q [L, rows, q_heads, head_dim] whose layer 0
     belongs to ``first_layer``... of the tables; tickets int32 [L, n_req], zero before the first call and left zero."""
     if q.dim() != 4 or repre.dim() != 3 or scores.dim() != 2:
@@ -229,7 +229,7 @@ def score_select(q: torch.Tensor, repre: torch.Tensor, seg_off: torch.Tensor, se
         block_tables=_opt(block_tables, torch.int32, "block_tables"), phys_out=_opt(phys_out, torch.int32, "phys_out"),
         seq_lens=_opt(seq_lens, torch.int32, "seq_lens"), sparse_seq_lens=_opt(sparse_seq_lens, torch.int32, "sparse_seq_lens"),
         block_size=block_size, tickets=_dev(tickets, torch.int32, "tickets"))
-    args.n_layers, args.num_repre, args.scale = n_layers, num_repre, float(scale)
+    args.n_layers, args.num_repre, args.scale, args.total_blocks = n_layers, num_repre, float(scale), int(total_blocks)
     import ctypes as C
 
     _lib.call("ucm_score_select", C.addressof(args), _stream())

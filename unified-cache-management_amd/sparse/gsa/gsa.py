@@ -406,7 +406,7 @@ class GSA(UcmSparseBase):
                                     self.model_input["block_tables"].data_ptr())
         a = self._sel
         a.seg_off, a.seg_len, a.topk_len, a.q_rows, a.seq_lens, a.block_tables = self.model_input["addr"]
-        a.n_req, a.max_seg_len = batch, max_len
+        a.n_req, a.max_seg_len, a.total_blocks = batch, max_len, total
 
     def execute_finished(self) -> None:
         if self.ptopk_prefetch:
