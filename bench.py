@@ -9,7 +9,9 @@ all 32 layers.  One step = for every layer and request: score all block
 representatives against the request's query, select top-k = max(16, 3 % of the
 blocks) plus the first block and the last two, and gather the selected K and V
 blocks from the bf16 paged cache into a contiguous per-request buffer.
-Three launches per step (score, select, gather), no host round trip between.
+Two launches per step (scores with each request's selection run by its last scoring
+workgroup, then the gather), no host round trip between; --two-launch scores and
+selects in launches of their own.
 
 Prints ONE JSON line.  `value` is microseconds per decode step with all inputs
 resident in HBM; `roofline` describes the dominant kernel (the gather),
@@ -23,6 +25,7 @@ import json
 import os
 import sys
 import time
+import zlib
 
 import numpy as np
 
@@ -32,15 +35,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 
 
-def measured_traffic(role: str, kernel: str, default_workload: bool):
-    """HBM bytes per launch that rocprofv3 --pmc measured for `kernel` on the default workload
-    (profiles/traffic.json), or None for any other workload.  The file names the kernel each figure belongs to:
-    a figure is never quoted for a kernel other than the one this run launched."""
-    if not default_workload:
-        return None
+def measured_traffic(role: str, kernel: str, workload: dict):
+    """HBM bytes per launch that rocprofv3 --pmc measured for `kernel` (profiles/traffic.json), or None when the
+    file has no entry for this role whose workload (layers, seed, blocks ...) is exactly this run's.  The file
+    names the kernel each figure belongs to: a figure is never quoted for a kernel other than the one this run
+    launched."""
     with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
         entry = json.load(f)["entries"].get(role)
-    if entry is None:
+    if entry is None or entry.get("workload") != workload:
         return None
     if entry["kernel"] != kernel:
         raise SystemExit(f"profiles/traffic.json holds the traffic of {entry['kernel']} for '{role}', but this run launched "
@@ -62,8 +64,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the oracle check of the last step")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
-    ap.add_argument("--delta-rho", type=float, default=0.95,
-                    help="correlation of consecutive decode queries in the delta-gather leg (0 = independent)")
+    ap.add_argument("--delta-rho", type=float, nargs="+", default=[0.95, 0.0, 0.9, 0.99],
+                    help="correlation(s) of consecutive decode queries in the delta-gather leg (0 = independent); the "
+                         "first one is the `delta_gather` object of the line, all of them its `by_correlation` list")
     ap.add_argument("--no-delta", action="store_true", help="skip the delta-gather leg")
     ap.add_argument("--two-launch", action="store_true",
                     help="score and select as two launches (ucm_score_blocks, ucm_topk_windows) instead of the one-launch "
@@ -92,6 +95,15 @@ def parse():
                          "x 16 blocks, all layers, K and V, random block table) on the same caches")
     ap.add_argument("--esa-leg", action="store_true",
                     help="also time the ESA retrieval backend (slot-list scoring + top-k) at three shapes")
+    ap.add_argument("--config1-leg", action="store_true",
+                    help="also time configs[0] of the benchmark definition: one request of 32768 tokens (256 blocks), one layer")
+    ap.add_argument("--config4-leg", action="store_true",
+                    help="also time configs[3]: 8 requests of 512-1024 blocks, 64 query heads (groups of 8), 80 layers, bf16 "
+                         "and fp32 representative tables, with the block mean of the one block per request that fills up")
+    ap.add_argument("--plugin-leg", action="store_true",
+                    help="also run the four plugins' hooks (GSA, ESA, KvComp, KVStar) on this batch with stand-in objects for "
+                         "vLLM's and report the host time and the host-inclusive time of their steps (plugin_bench.py; "
+                         "needs about as much memory again as the KV cache for the store the loads come from)")
     ap.add_argument("--kvstar-leg", action="store_true",
                     help="also time the multi-query softmax-vote retrieval (KVStar: 8 query tokens per request) on the same "
                          "ragged batch")
@@ -106,7 +118,7 @@ def parse():
                     help="also launch one plain 1 GiB copy (copy_batch_kernel) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled against a kernel of known traffic")
     args = ap.parse_args()
-    leg_flags = ("hash_leg", "prefetch_leg", "moves_leg", "esa_leg", "kvstar_leg")
+    leg_flags = ("hash_leg", "prefetch_leg", "moves_leg", "esa_leg", "kvstar_leg", "config1_leg", "config4_leg", "plugin_leg")
     run_all = not args.no_legs and not any(getattr(args, f) for f in leg_flags)
     for f in leg_flags:
         setattr(args, f, run_all or (getattr(args, f) and not args.no_legs))
@@ -142,6 +154,20 @@ def main():
     # ---- device state: paged KV cache, block tables, representatives
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
+
+    def score_name(f32_table: bool) -> str:
+        return "score_kernel" if f32_table else "score_kernel_bf16"
+
+    def leg_rng(name: str):
+        """Every leg draws from generators of its own (seeded by the run's seed and the leg's name), so that its
+        workload does not depend on which other legs ran before it."""
+        return np.random.default_rng([args.seed, zlib.crc32(name.encode())])
+
+    def leg_gen(name: str):
+        gen = torch.Generator(device=dev)
+        gen.manual_seed((args.seed << 32) + zlib.crc32(name.encode()))
+        return gen
+
     caches = []
     for _ in range(n_layers):
         c = torch.empty((2, nb, BS, HKV, D), dtype=torch.bfloat16, device=dev)
@@ -210,7 +236,7 @@ def main():
 
     if args.calibrate_copy:
         gib = 1 << 30
-        src = torch.empty(gib, dtype=torch.uint8, device=dev).random_(generator=g)
+        src = torch.empty(gib, dtype=torch.uint8, device=dev).random_(generator=leg_gen("calibrate"))
         dst = torch.empty_like(src)
         ops.copy_batch(torch.tensor([dst.data_ptr()], dtype=torch.int64, device=dev),
                        torch.tensor([src.data_ptr()], dtype=torch.int64, device=dev), gib)
@@ -244,59 +270,63 @@ def main():
     delta = None
     if not args.no_delta:
         n_slots = max_k
-        resident = torch.full((n_layers, N_REQ, n_slots), -1, dtype=torch.int32, device=dev)
-        load_phys = torch.empty_like(resident)
+        load_phys = torch.empty((n_layers, N_REQ, n_slots), dtype=torch.int32, device=dev)
         slot_of = torch.empty_like(idx)
         miss = torch.zeros_like(cnt)
         slots_count = torch.full_like(cnt, n_slots)
-        rho = float(args.delta_rho)
-        q_t = qs[0].float()
-        noise = torch.empty_like(q_t)
-
-        def delta_step(record=None):
-            nonlocal q_t
-            noise.normal_(generator=g)
-            q_t = rho * q_t + (1.0 - rho * rho) ** 0.5 * noise       # stationary N(0,1) sequence
-            qb = q_t.to(torch.bfloat16)
-            if record:
-                record[0].record()
-            ops.score_blocks(qb, repre, seg_off, seg_len, max_len, HKV, scores, total_blocks=rows)
-            ops.topk_windows(scores, seg_off, seg_len, topk_d, max_len, idx, cnt, block_tables=bt, phys_out=phys)
-            ops.delta_plan(idx, phys, cnt, resident, load_phys, slot_of, miss)
-            ops.kv_gather_selected(layers, kv_stride, BLOCK_BYTES, nb, load_phys, slots_count, dst_off, region, n_slots,
-                                   staging, total_blocks)
-            if record:
-                record[1].record()
-
-        for _ in range(max(args.warmup, 2)):
-            delta_step()                                              # the first step fills every slot
-        torch.cuda.synchronize()
-        d_events = [(ev(), ev()) for _ in range(args.steps)]
-        moved = torch.zeros((), dtype=torch.int64, device=dev)
-        for s_ in range(args.steps):
-            delta_step(d_events[s_])
-            moved += miss.sum()
-        torch.cuda.synchronize()
-        d_ms = float(np.mean([a_.elapsed_time(b_) for a_, b_ in d_events]))
-        moved_per_step = float(moved.item()) / args.steps
-        # the staging slots must hold exactly the selected blocks (checked on a sample of layers)
+        noise = torch.empty(qs[0].shape, dtype=torch.float32, device=dev)
         st = staging.view(torch.bfloat16).view(-1, BS, HKV, D)
-        for l in (0, n_layers // 2, n_layers - 1):
-            for r in range(N_REQ):
-                k = int(cnt[l, r])
-                slots_lr = slot_of[l, r, :k].long()
-                for kv in range(2):
-                    o = int(dst_off_h[r]) + (l * 2 + kv) * n_slots
-                    assert torch.equal(st[o + slots_lr], caches[l][kv][phys[l, r, :k].long()]), "delta staging differs"
-        delta = {
-            "us_per_step": round(d_ms * 1e3, 1),
-            "query_correlation": rho,
-            "blocks_moved_per_step": round(moved_per_step, 1),
+
+        def delta_run(rho: float) -> dict:
+            gen = leg_gen(f"delta {rho}")
+            resident = torch.full((n_layers, N_REQ, n_slots), -1, dtype=torch.int32, device=dev)
+            q_t = qs[0].float()
+
+            def delta_step(record=None):
+                nonlocal q_t
+                noise.normal_(generator=gen)
+                q_t = rho * q_t + (1.0 - rho * rho) ** 0.5 * noise       # stationary N(0,1) sequence
+                qb = q_t.to(torch.bfloat16)
+                if record:
+                    record[0].record()
+                ops.score_select(qb, repre, seg_off, seg_len, topk_d, max_len, HKV, scores, idx, cnt, tickets, block_tables=bt,
+                                 phys_out=phys, total_blocks=rows)
+                ops.delta_plan(idx, phys, cnt, resident, load_phys, slot_of, miss)
+                ops.kv_gather_selected(layers, kv_stride, BLOCK_BYTES, nb, load_phys, slots_count, dst_off, region, n_slots,
+                                       staging, total_blocks)
+                if record:
+                    record[1].record()
+
+            for _ in range(max(args.warmup, 2)):
+                delta_step()                                              # the first step fills every slot
+            torch.cuda.synchronize()
+            d_events = [(ev(), ev()) for _ in range(args.steps)]
+            moved = torch.zeros((), dtype=torch.int64, device=dev)
+            for s_ in range(args.steps):
+                delta_step(d_events[s_])
+                moved += miss.sum()
+            torch.cuda.synchronize()
+            d_ms = float(np.mean([a_.elapsed_time(b_) for a_, b_ in d_events]))
+            moved_per_step = float(moved.item()) / args.steps
+            # the staging slots must hold exactly the selected blocks (checked on a sample of layers)
+            for l in (0, n_layers // 2, n_layers - 1):
+                for r in range(N_REQ):
+                    k = int(cnt[l, r])
+                    slots_lr = slot_of[l, r, :k].long()
+                    for kv in range(2):
+                        o = int(dst_off_h[r]) + (l * 2 + kv) * n_slots
+                        assert torch.equal(st[o + slots_lr], caches[l][kv][phys[l, r, :k].long()]), "delta staging differs"
+            return {"query_correlation": rho, "us_per_step": round(d_ms * 1e3, 1), "blocks_moved_per_step": round(moved_per_step, 1),
+                    "hit_rate": round(1.0 - moved_per_step / n_sel, 4)}
+
+        runs = [delta_run(float(rho)) for rho in args.delta_rho]
+        delta = dict(runs[0])
+        delta.update({
             "blocks_selected_per_step": n_sel,
-            "hit_rate": round(1.0 - moved_per_step / n_sel, 4),
-            "note": "score + select + resident-set plan + gather of missing blocks only; consecutive queries follow "
+            "by_correlation": runs,
+            "note": "score + select (one launch) + resident-set plan + gather of missing blocks only; consecutive queries follow "
                     "q' = rho*q + sqrt(1-rho^2)*noise (synthetic); staging verified against the source blocks",
-        }
+        })
 
     # ---- hash-code retrieval leg (configs[4]): 32 requests of 64-256 blocks, 32 layers, 128-bit codes.
     # The key blocks are the K and V planes of the caches above read as one pool of 2*nb blocks.
@@ -305,7 +335,7 @@ def main():
     moves_leg = None
     if args.moves_leg:
         m_blocks = 64 * 16
-        m_ids = i32(rng.permutation(nb)[:m_blocks])
+        m_ids = i32(leg_rng("moves").permutation(nb)[:m_blocks])
         m_stage = torch.empty(m_blocks * n_layers * 2 * BLOCK_BYTES, dtype=torch.uint8, device=dev)
 
         def timed_move(fn, reps=10):
@@ -335,19 +365,20 @@ def main():
     hash_leg = None
     if args.hash_leg:
         h_req = 32
-        h_lens = rng.integers(64, 257, h_req).astype(np.int32)
+        h_rng, h_gen = leg_rng("hash"), leg_gen("hash")
+        h_lens = h_rng.integers(64, 257, h_req).astype(np.int32)
         h_rows = int(h_lens.sum())
         h_off = np.concatenate([[0], np.cumsum(h_lens)[:-1]]).astype(np.int32)
         pool = 2 * nb
-        h_ids_h = (rng.permutation(pool)[:h_rows] if h_rows <= pool else rng.integers(0, pool, h_rows)).astype(np.int32)
+        h_ids_h = (h_rng.permutation(pool)[:h_rows] if h_rows <= pool else h_rng.integers(0, pool, h_rows)).astype(np.int32)
         if args.hash_distinct > 0:
             h_ids_h = h_ids_h[np.arange(h_rows) % args.hash_distinct]
         h_ids, h_slots = i32(h_ids_h), torch.arange(h_rows, dtype=torch.int32, device=dev)
-        w_hash = (torch.randn(128, 128, device=dev, generator=g) * 2.0).to(torch.bfloat16)
+        w_hash = (torch.randn(128, 128, device=dev, generator=h_gen) * 2.0).to(torch.bfloat16)
         colsum = torch.zeros((n_layers, h_rows, HKV, 128), dtype=torch.int16, device=dev)
         bcodes = torch.zeros((n_layers, h_rows, HKV, 16), dtype=torch.uint8, device=dev)
         tcodes = torch.zeros((n_layers, h_rows, BS, HKV, 16), dtype=torch.uint8, device=dev)
-        hq = torch.empty((n_layers, h_req, HQ, D), dtype=torch.bfloat16, device=dev).normal_(generator=g)
+        hq = torch.empty((n_layers, h_req, HQ, D), dtype=torch.bfloat16, device=dev).normal_(generator=h_gen)
         q_codes = torch.zeros((n_layers, h_req, HQ, 16), dtype=torch.uint8, device=dev)
         q_sum = torch.zeros((n_layers, h_req, 128), dtype=torch.int16, device=dev)
         qbar = torch.zeros((n_layers, h_req, HKV, 16), dtype=torch.uint8, device=dev)
@@ -395,7 +426,7 @@ def main():
         enc_bytes = key_bytes + n_layers * h_rows * (BS * HKV * 16 + HKV * 128 * 2 + HKV * 16)
         hash_checked = None
         # HBM bytes per launch measured with rocprofv3 --pmc on exactly this workload, as for the gather below
-        default_hash = n_layers == N_LAYERS and args.seed == 2024 and h_rows == 5609 and args.hash_distinct == 0
+        hash_workload = {"seed": args.seed, "layers": n_layers, "blocks": h_rows, "distinct": args.hash_distinct}
         if not args.no_check:
             import oracle  # checker only
 
@@ -416,7 +447,7 @@ def main():
             "encode_read_GBps": round(gbs(key_bytes, enc_ms), 1),
             "roofline": {"kernel": "hash_encode_blocks_kernel", "bound": "hbm", "achieved": round(gbs(enc_bytes, enc_ms), 1),
                          "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(gbs(enc_bytes, enc_ms) / HBM_PEAK_GBS, 4),
-                         "traffic": measured_traffic("hash_encode", "hash_encode_blocks_kernel", default_hash),
+                         "traffic": measured_traffic("hash_encode", "hash_encode_blocks_kernel", hash_workload),
                          "algorithmic_bytes": enc_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * h_rows * BS * HKV * 128 * 128 / (enc_ms * 1e-3) / 1e12, 1)},
             "encode_summaries_only_ms": round(enc_sum_ms, 3),
@@ -433,13 +464,14 @@ def main():
     kvstar_leg = None
     if args.kvstar_leg:
         kx, merge = 8, args.kvstar_merge
+        k_gen = leg_gen("kvstar")
         km = BS // merge
         kdp = D if args.kvstar_prune >= 0.98 else round(D * args.kvstar_prune)
         kd_pad = (kdp + 15) // 16 * 16
         # kept channels: a seeded choice per (layer, kv head) (the reference keeps those with the largest mean |k|)
         kpr = None
         if kdp < D:
-            kpr = torch.stack([torch.stack([torch.randperm(D, device=dev, generator=g)[:kdp] for _ in range(HKV)])
+            kpr = torch.stack([torch.stack([torch.randperm(D, device=dev, generator=k_gen)[:kdp] for _ in range(HKV)])
                                for _ in range(n_layers)]).to(torch.int32)
         # one table over all layers, indexed [kv head][row][cell]: row of (layer l, block b) = l * rows + b
         if args.kvstar_layout == "row":      # the kv heads of a row next to each other in memory
@@ -464,7 +496,7 @@ def main():
         n_tasks = n_layers * N_REQ
         k_off = (seg_off_h[None, :].astype(np.int64) + (np.arange(n_layers, dtype=np.int64) * rows)[:, None]).reshape(-1)
         k_len = np.tile(lens, n_layers)
-        kq = (torch.randn(n_tasks, kx, HQ, D, device=dev, generator=g) * 0.25).to(torch.float16)
+        kq = (torch.randn(n_tasks, kx, HQ, D, device=dev, generator=k_gen) * 0.25).to(torch.float16)
         kq_off = torch.arange(n_tasks, dtype=torch.int64, device=dev) * (kx * HQ * D)
         ksel = None if kpr is None else torch.arange(n_layers, dtype=torch.int32, device=dev).repeat_interleave(N_REQ)
         kvotes = torch.zeros(n_layers * rows, device=dev)
@@ -510,7 +542,7 @@ def main():
                 assert kidx[0, t_, : int(kcnt[0, t_])].cpu().numpy().tolist() == heap.tolist(), "KVStar selection differs from the heap"
             kv_checked = ("votes of 3 sampled tasks within rtol 2e-4 / atol 2e-6 of the CPU oracle (fp32, other summation order); "
                           "their chosen blocks, in order, equal the oracle's heap on the same votes")
-        kv_default = n_layers == N_LAYERS and args.seed == 2024 and merge == 2 and kdp == 32
+        kv_workload = {"seed": args.seed, "layers": n_layers, "blocks": rows, "merge": merge, "channels": kdp}
         kvstar_leg = {
             "workload": f"{n_tasks} tasks (layer x request), {kx} query tokens x {HQ} heads, {rows} blocks x {km} sub-block "
                         f"representatives per layer, {kdp} of {D} channels, fp16",
@@ -519,13 +551,13 @@ def main():
             "block_repre_ms_all": [round(x, 3) for x in krep_all],
             "block_repre_GBps": round(gbs(krep_bytes, krep_ms), 1),
             "block_repre_frac": round(gbs(krep_bytes, krep_ms) / HBM_PEAK_GBS, 4),
-            "block_repre_traffic": measured_traffic("kvstar_repre", "kvstar_repre_kernel", kv_default),
+            "block_repre_traffic": measured_traffic("kvstar_repre", "kvstar_repre_kernel", kv_workload),
             "block_repre_algorithmic_bytes": krep_bytes,
             "us_per_step": round(kv_ms * 1e3, 1),
             "roofline": {"kernel": "kvstar_score_kernel (+ head sum, select, order)", "bound": "hbm",
                          "achieved": round(gbs(kv_bytes, kv_ms), 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(gbs(kv_bytes, kv_ms) / HBM_PEAK_GBS, 4),
-                         "traffic": measured_traffic("kvstar_votes", "kvstar_score_kernel", kv_default),
+                         "traffic": measured_traffic("kvstar_votes", "kvstar_score_kernel", kv_workload),
                          "algorithmic_bytes": kv_bytes,
                          "mfma_TFLOPs": round(2.0 * n_layers * rows * km * HQ * kx * kd_pad / (kv_ms * 1e-3) / 1e12, 1)},
             "checked": kv_checked,
@@ -540,11 +572,12 @@ def main():
     # reference's sequential order, best k in descending order) on a 16384-row table of 1024-wide representatives
     esa_leg = None
     if args.esa_leg:
-        e_data = torch.randn(16384, HKV * D, device=dev, generator=g)
+        e_rng, e_gen = leg_rng("esa"), leg_gen("esa")
+        e_data = torch.randn(16384, HKV * D, device=dev, generator=e_gen)
         esa_leg = []
         for e_b, e_m, e_k in ((1, 512, 150), (64, 512, 150), (1, 8000, 3000)):
-            e_q = torch.randn(e_b, HKV * D, device=dev, generator=g)
-            e_idx = i32(np.stack([rng.permutation(16384)[:e_m] for _ in range(e_b)]))
+            e_q = torch.randn(e_b, HKV * D, device=dev, generator=e_gen)
+            e_idx = i32(np.stack([e_rng.permutation(16384)[:e_m] for _ in range(e_b)]))
             e_ws = torch.zeros(e_b * e_m, device=dev)
             e_oi = torch.zeros(e_b, e_k, dtype=torch.int32, device=dev)
             e_os = torch.zeros(e_b, e_k, device=dev)
@@ -561,6 +594,188 @@ def main():
             esa_leg.append({"requests": e_b, "candidates": e_m, "topk": e_k,
                             "us_per_call": round(e0.elapsed_time(e1) / 50 * 1000, 1)})
         del e_data
+
+    # ---- configs[0]: one request of 32768 tokens (256 blocks), one layer: block means from the paged cache, then
+    # scores + selection (k = 16 + first 1 + last 2) in one launch.  Latency-bound at this size: the figures are
+    # times, the bandwidths only say how far from streaming a single small launch is.
+    config1_leg = None
+    if args.config1_leg:
+        c_rng, c_gen = leg_rng("config1"), leg_gen("config1")
+        c_n, c_k = 256, 19
+        c_ids = i32(c_rng.permutation(nb)[:c_n])
+        c_slots = torch.arange(c_n, dtype=torch.int32, device=dev)
+        c_rep = torch.zeros((1, c_n, ROW), dtype=repre.dtype, device=dev)
+        c_layer = ops.LayerPointers([caches[0][0]])
+        c_q = torch.empty((1, 1, HQ, D), dtype=torch.bfloat16, device=dev).normal_(generator=c_gen)
+        c_off, c_len, c_topk = i32([0]), i32([c_n]), i32([c_k])
+        c_scores = torch.zeros(1, c_n, device=dev)
+        c_idx = torch.full((1, 1, c_n), -1, dtype=torch.int32, device=dev)
+        c_cnt, c_tickets = torch.zeros((1, 1), dtype=torch.int32, device=dev), torch.zeros((1, 1), dtype=torch.int32, device=dev)
+
+        def timed_us(fn, reps=50):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = ev(), ev()
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / reps * 1e3
+
+        c_mean_us = timed_us(lambda: ops.block_mean(c_layer, c_ids, c_slots, c_rep, BS, HKV, D, nb, mode=ops.MEAN_BF16_ROUND))
+        c_retr_us = timed_us(lambda: ops.score_select(c_q, c_rep, c_off, c_len, c_topk, c_n, HKV, c_scores, c_idx, c_cnt, c_tickets,
+                                                      total_blocks=c_n))
+        c_two_us = timed_us(lambda: (ops.score_blocks(c_q, c_rep, c_off, c_len, c_n, HKV, c_scores, total_blocks=c_n),
+                                     ops.topk_windows(c_scores, c_off, c_len, c_topk, c_n, c_idx, c_cnt)))
+        c_cpu_us = c_checked = None
+        if not args.no_check or not args.no_cpu:
+            import oracle  # checker / baseline only
+
+            c_rep_h = c_rep[0].float().cpu().numpy()
+            c_q_h = c_q[0].float().cpu().numpy()
+            lens1, off1, k1 = np.array([c_n], np.int32), np.array([0], np.int32), np.array([c_k], np.int32)
+            if not args.no_check:
+                kc = caches[0][0].view(torch.int16)[c_ids.long()].cpu().numpy().view(np.uint16)
+                want_rep = np.zeros((c_n, ROW), np.float32)
+                oracle.block_mean_paged(kc, np.arange(c_n, dtype=np.int32), np.arange(c_n, dtype=np.int32), want_rep, round_bf16=True)
+                assert np.array_equal(want_rep.view(np.uint32), c_rep_h.view(np.uint32)), "configs[0]: block means differ"
+                widx, wcnt, wsc = oracle.select_topk_bs(c_q_h, c_rep_h, off1, lens1, k1, HKV, out_stride=c_n + 4)
+                assert np.array_equal(wsc.view(np.uint32), c_scores[0].cpu().numpy().view(np.uint32)), "configs[0]: scores differ"
+                assert int(c_cnt[0, 0]) == int(wcnt[0]) and np.array_equal(c_idx[0, 0, : wcnt[0]].cpu().numpy(), widx[0, : wcnt[0]])
+                c_checked = "block means, fp32 scores and the selection equal the CPU oracle"
+            if not args.no_cpu:
+                ref_ok = oracle.ref.available and _cpu_has_avx512()
+                fn = oracle.ref.select_topk_bs if ref_ok else oracle.select_topk_bs
+                fn(c_q_h, c_rep_h, off1, lens1, k1, HKV, out_stride=c_n + 4)
+                s0 = time.perf_counter()
+                for _ in range(200):
+                    fn(c_q_h, c_rep_h, off1, lens1, k1, HKV, out_stride=c_n + 4)
+                c_cpu_us = (time.perf_counter() - s0) / 200 * 1e6
+        c_mean_bytes = c_n * (BLOCK_BYTES + ROW * rep_es)
+        c_score_bytes = c_n * ROW * rep_es + HQ * D * 2 + c_n * 4
+        config1_leg = {
+            "workload": f"configs[0]: 1 request x {c_n} blocks (32768 tokens), 1 layer, k = 16 + 1 first + 2 last, "
+                        f"{args.repre_dtype} representatives",
+            "block_mean_us": round(c_mean_us, 1), "retrieval_us": round(c_retr_us, 1), "retrieval_two_launches_us": round(c_two_us, 1),
+            "roofline_block_mean": {"kernel": "block_mean_kernel", "bound": "hbm", "achieved": round(c_mean_bytes / c_mean_us / 1e3, 1),
+                                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(c_mean_bytes / c_mean_us / 1e3 / HBM_PEAK_GBS, 4),
+                                    "traffic": None, "algorithmic_bytes": c_mean_bytes},
+            "roofline": {"kernel": score_name(args.repre_dtype == "f32"), "bound": "hbm", "achieved": round(c_score_bytes / c_retr_us / 1e3, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(c_score_bytes / c_retr_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "traffic": None, "algorithmic_bytes": c_score_bytes,
+                         "note": "one workgroup chain of a few microseconds: launch latency, not bandwidth, is what this size measures"},
+            "cpu_reference_retrieval_us": None if c_cpu_us is None else round(c_cpu_us, 1),
+            "checked": c_checked,
+        }
+
+    # ---- configs[3]: 8 requests of 512-1024 blocks, 64 query heads in groups of 8, 80 layers; one decode step =
+    # scores + selection of all layers (one launch), and - on the steps in which a request's last block fills up -
+    # the block mean of one block per request, every layer.  The tables hold random bf16 values: the step does not
+    # read the KV cache, and 80 layers of it would not fit beside the 32-layer one.
+    config4_leg = None
+    if args.config4_leg:
+        f_rng, f_gen = leg_rng("config4"), leg_gen("config4")
+        f_req, f_layers, f_hq = 8, 80, 64
+        f_lens = f_rng.integers(512, 1025, f_req).astype(np.int32)
+        f_rows, f_max = int(f_lens.sum()), int(f_lens.max())
+        f_off_h = np.concatenate([[0], np.cumsum(f_lens)[:-1]]).astype(np.int32)
+        f_topk_h = np.array([max(16, int(0.02 * n)) + 3 for n in f_lens], np.int32)
+        f_off, f_len, f_topk = i32(f_off_h), i32(f_lens), i32(f_topk_h)
+        f_q = torch.empty((f_layers, f_req, f_hq, D), dtype=torch.bfloat16, device=dev).normal_(generator=f_gen)
+        f_scores = torch.zeros(f_layers, f_rows, device=dev)
+        f_idx = torch.full((f_layers, f_req, f_max), -1, dtype=torch.int32, device=dev)
+        f_cnt, f_tickets = torch.zeros((f_layers, f_req), dtype=torch.int32, device=dev), torch.zeros((f_layers, f_req), dtype=torch.int32, device=dev)
+        f_tab16 = torch.empty((f_layers, f_rows, ROW), dtype=torch.bfloat16, device=dev).normal_(generator=f_gen)
+        f_out = {}
+        f_e0, f_e1 = ev(), ev()
+        for name, tab in (("bf16", f_tab16), ("f32", None)):
+            if tab is None:
+                tab = f_tab16.float()                                   # the same values widened: the CPU path's table
+            run = lambda: ops.score_select(f_q, tab, f_off, f_len, f_topk, f_max, HKV, f_scores, f_idx, f_cnt, f_tickets,
+                                           total_blocks=f_rows)
+            for _ in range(3):
+                run()
+            torch.cuda.synchronize()
+            f_e0.record()
+            for _ in range(args.steps):
+                run()
+            f_e1.record()
+            torch.cuda.synchronize()
+            us = f_e0.elapsed_time(f_e1) / args.steps * 1e3
+            nbytes = f_layers * (f_rows * ROW * tab.element_size() + f_req * f_hq * D * 2 + f_rows * 4)
+            f_out[name] = {"retrieval_us": round(us, 1),
+                           "roofline": {"kernel": "score_kernel_bf16" if name == "bf16" else "score_kernel", "bound": "hbm",
+                                        "achieved": round(nbytes / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                        "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": nbytes}}
+            if name == "f32":
+                f_tab32 = tab
+        # the incremental representative: the block that filled up, one per request, all 80 layers in one launch
+        # (the 80 key planes are the 32 layers' K planes named again and again)
+        f_planes = ops.LayerPointers([caches[l % n_layers][0] for l in range(f_layers)])
+        f_new_ids = [i32(f_rng.permutation(nb)[:f_req]) for _ in range(args.steps + 3)]   # other blocks every time: nothing cached
+        f_new_slots = i32(f_off_h + f_lens - 1)
+        inc = lambda i: ops.block_mean(f_planes, f_new_ids[i], f_new_slots, f_tab16, BS, HKV, D, nb, mode=ops.MEAN_BF16_ROUND)
+        for i in range(3):
+            inc(i)
+        torch.cuda.synchronize()
+        f_e0.record()
+        for i in range(args.steps):
+            inc(3 + i)
+        f_e1.record()
+        torch.cuda.synchronize()
+        f_inc_us = f_e0.elapsed_time(f_e1) / args.steps * 1e3
+        f_inc_bytes = f_layers * f_req * (BLOCK_BYTES + ROW * 2)
+        f_cpu_us = f_checked = None
+        if not args.no_check or not args.no_cpu:
+            import oracle  # checker / baseline only
+
+            ops.score_select(f_q, f_tab32, f_off, f_len, f_topk, f_max, HKV, f_scores, f_idx, f_cnt, f_tickets, total_blocks=f_rows)
+            torch.cuda.synchronize()
+            f_q_h = f_q.float().cpu().numpy()
+            if not args.no_check:
+                for l in (0, f_layers // 2, f_layers - 1):
+                    widx, wcnt, wsc = oracle.select_topk_bs(f_q_h[l], f_tab32[l].cpu().numpy(), f_off_h, f_lens, f_topk_h, HKV,
+                                                            out_stride=f_max + 4)
+                    assert np.array_equal(wsc.view(np.uint32), f_scores[l].cpu().numpy().view(np.uint32)), f"configs[3]: scores differ ({l})"
+                    got_i, got_c = f_idx[l].cpu().numpy(), f_cnt[l].cpu().numpy()
+                    for r in range(f_req):
+                        assert got_c[r] == wcnt[r] and np.array_equal(got_i[r, : wcnt[r]], widx[r, : wcnt[r]]), f"configs[3]: selection differs ({l},{r})"
+                f_checked = "fp32 scores and selections of 3 of the 80 layers equal the CPU oracle"
+            if not args.no_cpu:
+                ref_ok = oracle.ref.available and _cpu_has_avx512()
+                fn = oracle.ref.select_topk_bs if ref_ok else oracle.select_topk_bs
+                f_rep_h = f_tab32.cpu().numpy()
+
+                def f_cpu_step():
+                    for l in range(f_layers):
+                        fn(f_q_h[l], f_rep_h[l], f_off_h, f_lens, f_topk_h, HKV, out_stride=f_max + 4)
+
+                f_cpu_step()
+                f_reps, f_acc = 0, 0.0
+                while f_acc < 4.0 and f_reps < 50:
+                    s0 = time.perf_counter()
+                    f_cpu_step()
+                    f_acc += time.perf_counter() - s0
+                    f_reps += 1
+                f_cpu_us = f_acc / f_reps * 1e6
+                del f_rep_h
+        config4_leg = {
+            "workload": f"configs[3]: {f_req} requests, {f_rows} blocks ({int(f_lens.min())}-{f_max} each), {f_hq} query heads in groups of "
+                        f"{f_hq // HKV}, {f_layers} layers, k = max(16, 2%) + 1 first + 2 last",
+            "bf16_table": f_out["bf16"], "f32_table": f_out["f32"],
+            "incremental_block_mean": {"blocks_per_launch": f_req * f_layers, "us": round(f_inc_us, 1),
+                                       "GBps": round(f_inc_bytes / f_inc_us / 1e3, 1),
+                                       "note": "one block per request and layer, 80 layers in one launch; runs on the steps in "
+                                               "which a request's last block fills up (every 128th per request)"},
+            "cpu_reference_retrieval_us": None if f_cpu_us is None else round(f_cpu_us, 1),
+            "cpu_reference": None if f_cpu_us is None else
+                f"the reference's own translation units where AVX-512 is present (else the port), {min(16, os.cpu_count() or 1)} OpenMP "
+                "threads over blocks, requests and layers serial, fp32 table in host memory",
+            "checked": f_checked,
+        }
+        del f_tab16, f_tab32, f_scores, f_idx
 
     # ---- check the last step against the CPU oracle (selection, scores, gathered bytes)
     if not args.no_check:
@@ -658,6 +873,7 @@ def main():
         from ucm_amd.sparse.gsa.prefetch import GSAPrefetchEngineC
         from ucm_amd.sparse.utils import LOCAL_WINDOW_SZ, MAX_TOPK_LEN, MIN_TOPK_LEN, compute_topk_len
 
+        p_gen = leg_gen("prefetch")
         width = 64                                          # table row: MAX_TOPK_LEN + 1 resident blocks fit
         i32z = lambda *shape: torch.zeros(shape, dtype=torch.int32, device=dev)
         p_free, p_free_len = i32z(n_layers, N_REQ, width), i32z(n_layers, N_REQ)
@@ -683,7 +899,7 @@ def main():
             resident_h.append((holder, logical, [st_.blocks[x] for x in spare]))
         pool = torch.empty((rows, n_layers, 2, BLOCK_BYTES), dtype=torch.uint8, device=dev)
         for l0 in range(0, rows, 256):
-            pool[l0 : l0 + 256].random_(generator=g)
+            pool[l0 : l0 + 256].random_(generator=p_gen)
         src_table = torch.full((N_REQ, max_len), -1, dtype=torch.int32, device=dev)
         for r in range(N_REQ):
             src_table[eng.row_of(r), : lens[r]] = torch.arange(int(seg_off_h[r]), int(seg_off_h[r] + lens[r]), dtype=torch.int32, device=dev)
@@ -691,14 +907,14 @@ def main():
         p_idx = torch.full((n_layers, N_REQ, max_len), -1, dtype=torch.int32, device=dev)
         p_cnt = torch.zeros(n_layers, N_REQ, dtype=torch.int32, device=dev)
         req_ids, bs_idx, tk_list = list(range(N_REQ)), list(range(N_REQ)), [int(k) for k in p_topk_h]
-        rho = args.delta_rho
+        rho = float(args.delta_rho[0])
         q_cur = qs[0].float()
         n_rounds = 4 + min(args.steps, 16)
         ev_p = [[ev() for _ in range(4)] for _ in range(n_rounds)]
         loads_per_round, topk_rounds = [], []
         for t in range(n_rounds):
             if t:
-                q_cur = rho * q_cur + (1.0 - rho * rho) ** 0.5 * torch.randn(q_cur.shape, device=dev, generator=g)
+                q_cur = rho * q_cur + (1.0 - rho * rho) ** 0.5 * torch.randn(q_cur.shape, device=dev, generator=p_gen)
             ops.score_blocks(q_cur.to(torch.bfloat16), repre, seg_off, seg_len, max_len, HKV, scores, total_blocks=rows)
             ops.topk_windows(scores, seg_off, seg_len, p_topk, max_len, p_idx, p_cnt)
             sel = p_idx[:, :, :MAX_TOPK_LEN].contiguous()
@@ -781,12 +997,31 @@ def main():
         }
         del pool
 
+    # ---- plugin leg: the four plugins' hooks on this batch, host time included (runs last: loads overwrite cache blocks)
+    plugin_leg = None
+    if args.plugin_leg:
+        import plugin_bench
+
+        block_lists = [[int(x) for x in bt_h[r, : lens[r]]] for r in range(N_REQ)]
+        del staging
+        torch.cuda.empty_cache()
+        plugin_leg = {"note": "hooks driven by stand-in objects for vLLM's (plugin_bench.py), 16 requests x "
+                              f"{n_layers} layers; host_us = the hooks' time on the model-runner thread, wall_us = until the "
+                              "device has finished what they queued (no model runs in between); medians per kind of step"}
+        for name, leg in (("GSA", lambda: plugin_bench.gsa_leg(torch, dev, caches, lens, block_lists, args.steps, args.seed)),
+                          ("ESA", lambda: plugin_bench.esa_leg(torch, dev, caches, lens, block_lists, args.seed)),
+                          ("KvComp", lambda: plugin_bench.kvcomp_leg(torch, dev, caches, lens, block_lists, args.seed)),
+                          ("KVStar", lambda: plugin_bench.kvstar_leg(torch, dev, caches, lens, block_lists, args.seed))):
+            plugin_leg[name] = leg()
+            torch.cuda.empty_cache()
+
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly this workload
     # (profiles/bench_config2_kernels.md); other workloads have no measurement
-    default_workload = n_layers == N_LAYERS and args.seed == 2024
-    score_kernel_name = "score_kernel_bf16" if args.repre_dtype == "bf16" else "score_kernel"   # what ucm_score_blocks launches
-    traffic_gather = measured_traffic("gather", "kv_gather_selected_kernel", default_workload)
-    traffic_score = measured_traffic("score_" + args.repre_dtype, score_kernel_name, default_workload)
+    main_workload = {"seed": args.seed, "layers": n_layers, "blocks": rows}
+    score_kernel_name = "score_kernel_bf16" if args.repre_dtype == "bf16" else "score_kernel"   # what the scoring calls launch
+    traffic_gather = measured_traffic("gather", "kv_gather_selected_kernel", main_workload)
+    traffic_score = measured_traffic("score_" + args.repre_dtype + ("" if args.two_launch else "_select"), score_kernel_name,
+                                     main_workload)
 
     out = {
         "metric": "us per decode step (32-layer retrieval+gather)",
@@ -812,8 +1047,9 @@ def main():
             "selected_blocks_per_step": n_sel,
             "kv_cache_GB": round(n_layers * 2 * nb * BLOCK_BYTES / 1e9, 1),
         },
-        "kernels_us": {"score": round(score_ms * 1e3, 1), "select": round(topk_ms * 1e3, 1),
-                       "gather": round(gather_ms * 1e3, 1)},
+        "kernels_us": ({"score": round(score_ms * 1e3, 1), "select": round(topk_ms * 1e3, 1), "gather": round(gather_ms * 1e3, 1)}
+                       if args.two_launch else {"score_select": round(score_ms * 1e3, 1), "gather": round(gather_ms * 1e3, 1)}),
+        "launches_per_step": 3 if args.two_launch else 2,
         "retrieval_us": round((score_ms + topk_ms) * 1e3, 1),
         "roofline": {
             "kernel": "kv_gather_selected_kernel",
@@ -826,7 +1062,7 @@ def main():
             "algorithmic_bytes": gather_bytes,
         },
         "roofline_score": {
-            "kernel": score_kernel_name,
+            "kernel": score_kernel_name + ("" if args.two_launch else " (scores, and each request's selection by its last workgroup)"),
             "bound": "hbm",
             "achieved": round(gbs(score_bytes, score_ms), 1),
             "peak": HBM_PEAK_GBS,
@@ -838,6 +1074,9 @@ def main():
         "block_mean_prefill": {"ms": round(mean_ms, 3), "GBps": round(gbs(mean_bytes, mean_ms), 1),
                                "frac": round(gbs(mean_bytes, mean_ms) / HBM_PEAK_GBS, 4)},
         "delta_gather": delta,
+        "config1": config1_leg,
+        "config4": config4_leg,
+        "plugin_steps": plugin_leg,
         "kv_moves": moves_leg,
         "prefetch_round": prefetch_leg,
         "hash_retrieval": hash_leg,

@@ -26,7 +26,7 @@ from __future__ import annotations
 
 import ctypes
 import math
-from itertools import accumulate
+from itertools import accumulate, count
 from typing import Dict, List, Optional, Union
 
 import torch
@@ -44,6 +44,8 @@ from ..utils import (
 )
 
 ReqType = Union[str, int]
+_serials = count()
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _Q_CODES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32, torch.float16: _lib.DTYPE_F16}
 
 
@@ -58,6 +60,8 @@ class GSAReqStat:
         self.block_size = block_size
         self.threshold = threshold
         self.blocks: List[int] = []
+        self.blocks_version = 0           # counts the changes of `blocks`
+        self.serial = next(_serials)      # a request id may come back with another request behind it
         self.calc_block_table: List[int] = []
         self.calc_repre_slot_mapping: List[int] = []
         self.num_computed_tokens = 0
@@ -123,7 +127,13 @@ class GSAReqStat:
             # decided from the blocks the request held BEFORE the scheduler swapped in its sparse block list
             # (the reference calls it ahead of touching self.blocks, gsa.py:141-149)
             self.get_sparse_and_free_block(True, *prefetch)
-        self.blocks = list(req_state.block_ids[0])
+        src = req_state.block_ids[0]
+        # (a decoding request's list only grows at its end: the copy is made when the list changed)
+        mid = len(src) // 2
+        if len(src) != len(self.blocks) or (src and (src[-1] != self.blocks[-1] or src[0] != self.blocks[0]
+                                                     or src[mid] != self.blocks[mid])):
+            self.blocks = list(src)
+            self.blocks_version += 1
         # A block gets its representative once every one of its tokens is in
         # the cache, i.e. after the step that fills it.
         full_after_step = self.get_seq_len() // self.block_size
@@ -209,6 +219,8 @@ class GSA(UcmSparseBase):
         self._kv_full: Dict[int, torch.Tensor] = {}
         self._scored: set = set()  # sparsified requests whose blocks have been scored at least once
         self._layer_of: Dict[str, int] = {}
+        self._tables_signature = None     # (request, blocks, last block) per batch slot of the block tables on the device
+        self._tables_dev: Optional[torch.Tensor] = None
 
     # ------------------------------------------------------------------ device state
     def _ensure_device_state(self, device) -> None:
@@ -218,6 +230,7 @@ class GSA(UcmSparseBase):
         row = self.num_key_heads * self.head_size
         L = self.layer_num
         self.device = device
+        self._dev_index = device.index if device.index is not None else torch.cuda.current_device()
         self.kpre_caches = torch.zeros((L, rows, row), dtype=self.repre_dtype, device=device)
         self.scores = torch.zeros((L, rows), dtype=torch.float32, device=device)
         self.topk_caches = torch.zeros((L, self.max_bs, self.max_block_len), dtype=torch.int32, device=device)
@@ -261,7 +274,9 @@ class GSA(UcmSparseBase):
             self._register_layer(int(name.split(".")[2]), cache)
 
     def _register_layer(self, layer_id: int, kv_cache) -> None:
-        if layer_id in self._layer_ptrs and self.k_cache[layer_id].data_ptr() == kv_cache[0].data_ptr():
+        known = self._kv_full.get(layer_id)
+        if known is kv_cache or (known is not None and isinstance(kv_cache, torch.Tensor) and isinstance(known, torch.Tensor)
+                                 and known.data_ptr() == kv_cache.data_ptr()):
             return
         self.k_cache[layer_id], self.v_cache[layer_id] = kv_cache[0], kv_cache[1]
         self._layer_ptrs[layer_id] = ops.LayerPointers([kv_cache[0]])
@@ -368,15 +383,22 @@ class GSA(UcmSparseBase):
             return
         width = self.max_block_len
         n_calc = len(self.model_input["calc_block_table"])
-        # one int32 host buffer: 5 descriptor rows, the block tables, then the block-mean lists
+        # The block tables go down only when a request's list changed or the batch was reordered (a decoding
+        # request's list grows by one entry every block_size steps); the five descriptor rows and the block-mean
+        # lists go down every step.  One int32 host buffer, one copy.
+        signature = tuple((st.serial, st.blocks_version) if st is not None else None for st in by_index)
+        tables_known = signature == self._tables_signature
         slot = self.step_count & 1
         if self._host_free[slot] is not None:
             self._host_free[slot].synchronize()  # upload of two steps ago; long finished
-        host = self._host_desc[slot][: 5 * batch + batch * width + 2 * n_calc]
+        n_tables = 0 if tables_known else batch * width
+        host = self._host_desc[slot][: 5 * batch + n_tables + 2 * n_calc]
         hn = host.numpy()                    # the same pinned memory; numpy fills it several times faster than torch indexing
-        hn[:] = 0
         desc = hn[: 5 * batch].reshape(5, batch)
-        tables = hn[5 * batch : 5 * batch + batch * width].reshape(batch, width)
+        desc[:] = 0
+        if not tables_known:
+            tables = hn[5 * batch : 5 * batch + n_tables].reshape(batch, width)
+            tables[:] = 0
         max_len = total = 0
         query_locals = self.model_input["query_locals"]
         for i, st in enumerate(by_index):
@@ -386,24 +408,29 @@ class GSA(UcmSparseBase):
             k = compute_topk_len(n, self.min_topk, self.max_topk, self.topk_ratio) if st.is_gsa() else n
             # k >= n keeps every block (short or prefilling requests)
             desc[:, i] = (st.slot_offset, n, max(k, 1), query_locals[i + 1] - 1, st.get_seq_len())
-            tables[i, :n] = st.blocks
+            if not tables_known:
+                tables[i, :n] = st.blocks
             max_len, total = max(max_len, n), total + n
-        tail = hn[5 * batch + batch * width :]
+        tail = hn[5 * batch + n_tables :]
         tail[:n_calc] = self.model_input["calc_block_table"]
         tail[n_calc:] = self.model_input["calc_repre_slot_mapping"]
         dev = host.to(self.device, non_blocking=True)
         self._host_free[slot] = torch.cuda.Event()
         self._host_free[slot].record()
         d = dev[: 5 * batch].view(5, batch)
+        if not tables_known:
+            self._tables_dev = dev[5 * batch : 5 * batch + n_tables].view(batch, width)
+            self._tables_signature = signature
         self.model_input.update(
             seg_off=d[0], seg_len=d[1], topk_len=d[2], q_rows=d[3], seq_lens=d[4],
-            block_tables=dev[5 * batch : 5 * batch + batch * width].view(batch, width),
-            calc_blocks_dev=dev[5 * batch + batch * width : 5 * batch + batch * width + n_calc],
-            calc_slots_dev=dev[5 * batch + batch * width + n_calc :],
+            block_tables=self._tables_dev,
+            calc_blocks_dev=dev[5 * batch + n_tables : 5 * batch + n_tables + n_calc],
+            calc_slots_dev=dev[5 * batch + n_tables + n_calc :],
             max_len=max_len, total=total, n_batch=batch,
         )
-        self.model_input["addr"] = (d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), d[4].data_ptr(),
-                                    self.model_input["block_tables"].data_ptr())
+        base = d.data_ptr()
+        self.model_input["addr"] = (base, base + 4 * batch, base + 8 * batch, base + 12 * batch, base + 16 * batch,
+                                    self._tables_dev.data_ptr())
         a = self._sel
         a.seg_off, a.seg_len, a.topk_len, a.q_rows, a.seq_lens, a.block_tables = self.model_input["addr"]
         a.n_req, a.max_seg_len, a.total_blocks = batch, max_len, total
@@ -427,7 +454,7 @@ class GSA(UcmSparseBase):
             return
         l = self._layer_id(layer_name)
         n = mi["n_batch"]
-        stream = ops.current_stream()
+        stream = _raw_stream(self._dev_index) if _raw_stream is not None else ops.current_stream()
         if mi["is_topk"]:
             q_code = _Q_CODES.get(query.dtype)
             if q_code is None:
