@@ -21,6 +21,7 @@ resident in HBM; `roofline` describes the dominant kernel (the gather),
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -1013,6 +1014,7 @@ def main():
                           ("KvComp", lambda: plugin_bench.kvcomp_leg(torch, dev, caches, lens, block_lists, args.seed)),
                           ("KVStar", lambda: plugin_bench.kvstar_leg(torch, dev, caches, lens, block_lists, args.seed))):
             plugin_leg[name] = leg()
+            gc.collect()                                     # the leg's plugin and its store (a KV cache's worth of memory)
             torch.cuda.empty_cache()
 
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on exactly this workload

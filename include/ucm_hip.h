@@ -479,6 +479,11 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
  *            after layer l-1's (the reference picks the channels per layer
  *            state; 0 = one set of lists for every layer), so one launch
  *            covers all layers
+ *   pruned_sel  dev int32[n] or NULL: with it a layer has n_pruned_lists
+ *            lists ([n_pruned_lists][kv_heads][d_pruned]) and listed block i is
+ *            pruned by list pruned_sel[i] - the blocks of several requests,
+ *            each with channels of its own, in one launch (a block that names
+ *            a list outside [0, n_pruned_lists) is skipped); NULL: list 0
  *   repre    dev fp16 cells of [d_pad/8][M][8] - the 16-byte pieces (8
  *            channels) of a block's M sub-blocks side by side - one per
  *            (layer, kv head, row): cell (l, h, r) starts l*repre_layer_stride
@@ -526,9 +531,23 @@ int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_co
 int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
                            const int32_t* block_ids, const int32_t* slots, int n, int block_size,
                            int kv_heads, int head_dim, int merge, const int32_t* pruned,
-                           int64_t pruned_layer_stride, int d_pruned, int d_pad, void* repre_f16,
-                           int repre_rows, int64_t repre_layer_stride, int64_t repre_head_stride,
-                           int64_t repre_row_stride, ucm_stream_t stream);
+                           int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
+                           int d_pruned, int d_pad, void* repre_f16, int repre_rows,
+                           int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
+                           ucm_stream_t stream);
+/*
+ * The query tokens a step contributes to its requests' retrieval groups, copied aside as fp16 - save_to_standby
+ * (ucm/sparse/kvstar/multistep.py:318-324, one clone per request and layer) together with the .to(float16) of
+ * retrieval_async (:252-254), for all requests of a layer in one launch:
+ *   ring_f16[dst_off[i] .. dst_off[i]+row_elems) = fp16(q[src_rows[i]][0 .. row_elems))
+ *   q          dev: [q_rows][row_elems] fp32, bf16 or fp16 (a layer's query tensor, row_elems = q_heads*head_dim)
+ *   src_rows   dev int32[n], dst_off dev int64[n] (elements into the ring, multiples of 8)
+ * A row outside [0, q_rows) or a place outside [0, ring_elems) is skipped.  The groups then are the `q_f16`
+ * of ucm_kvstar_votes with q_off pointing into the ring.
+ */
+int ucm_kvstar_park_queries(const void* q, int q_dtype, int64_t q_rows, int row_elems, const int32_t* src_rows,
+                            const int64_t* dst_off, int n, void* ring_f16, int64_t ring_elems, ucm_stream_t stream);
+
 /* ucm_kvstar_votes has two paths: one workgroup per (task, kv head) that keeps
  * the task's per-(block, query row) sums in LDS and stores only the head's
  * share of the votes (taken when there are at least 128 such pairs and the

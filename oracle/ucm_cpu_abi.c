@@ -48,6 +48,7 @@ TWIN(ucm_prefetch_plan);
 TWIN(ucm_kvstar_block_repre);
 TWIN(ucm_kvstar_votes);
 TWIN(ucm_kvstar_votes_tables);
+TWIN(ucm_kvstar_park_queries);
 
 /* the oracle's functions these forward to (ucm_oracle.c) */
 float orc_bf16_to_f32(uint16_t h);
@@ -801,12 +802,12 @@ int ucm_prefetch_plan_cpu(const int32_t* map_block, const int32_t* map_len, int3
 
 int ucm_kvstar_block_repre_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
                                const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, int merge,
-                               const int32_t* pruned, int64_t pruned_layer_stride, int d_pruned, int d_pad, void* repre_f16,
-                               int repre_rows, int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
-                               ucm_stream_t stream)
+                               const int32_t* pruned, int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
+                               int d_pruned, int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
+                               int64_t repre_head_stride, int64_t repre_row_stride, ucm_stream_t stream)
 {
     (void)stream;
-    if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
+    if (n < 0 || n_layers < 0 || (pruned_sel && (!pruned || n_pruned_lists < 1))) { return UCM_EINVAL; }
     if (n == 0 || n_layers == 0) { return UCM_OK; }
     if (!k_layers || !repre_f16 || num_blocks <= 0 || repre_rows <= 0 || block_size <= 0 || kv_heads <= 0 || head_dim <= 0 ||
         merge <= 0 || block_size % merge || d_pruned <= 0 || d_pruned > head_dim || d_pad < d_pruned || d_pad % 8 ||
@@ -823,8 +824,10 @@ int ucm_kvstar_block_repre_cpu(const void* const* k_layers, int n_layers, int nu
         for (int i = 0; i < n; ++i) {
             const int32_t id = block_ids ? block_ids[i] : i, slot = slots ? slots[i] : i;
             if (id < 0 || id >= num_blocks || slot < 0 || slot >= repre_rows) { continue; }
+            if (pruned_sel && (pruned_sel[i] < 0 || pruned_sel[i] >= n_pruned_lists)) { continue; }   /* a list that does not exist */
+            const int32_t* mine = (lists && pruned_sel) ? lists + (size_t)pruned_sel[i] * kv_heads * d_pruned : lists;
             orc_kvstar_block_repre((const uint16_t*)k_layers[l], &id, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads,
-                                   (uint32_t)head_dim, (uint32_t)merge, lists, (uint32_t)d_pruned, (uint32_t)d_pad, tmp);
+                                   (uint32_t)head_dim, (uint32_t)merge, mine, (uint32_t)d_pruned, (uint32_t)d_pad, tmp);
             for (int h = 0; h < kv_heads; ++h) {
                 uint16_t* cell = (uint16_t*)repre_f16 + (int64_t)l * repre_layer_stride + (int64_t)h * repre_head_stride +
                                  (int64_t)slot * repre_row_stride;
@@ -837,6 +840,31 @@ int ucm_kvstar_block_repre_cpu(const void* const* k_layers, int n_layers, int nu
         }
     }
     free(tmp);
+    return UCM_OK;
+}
+
+int ucm_kvstar_park_queries_cpu(const void* q, int q_dtype, int64_t q_rows, int row_elems, const int32_t* src_rows,
+                                const int64_t* dst_off, int n, void* ring_f16, int64_t ring_elems, ucm_stream_t stream)
+{
+    (void)stream;
+    if (n < 0 || q_rows < 0 || ring_elems < 0) { return UCM_EINVAL; }
+    if (n == 0) { return UCM_OK; }
+    if (!q || !src_rows || !dst_off || !ring_f16 || q_dtype < UCM_DTYPE_F32 || q_dtype > UCM_DTYPE_F16 || row_elems <= 0 ||
+        row_elems % 8) {
+        return UCM_EINVAL;
+    }
+    for (int i = 0; i < n; ++i) {
+        const int64_t src = src_rows[i], dst = dst_off[i];
+        if (src < 0 || src >= q_rows || dst < 0 || dst + row_elems > ring_elems || (dst & 7)) { continue; }
+        for (int e = 0; e < row_elems; ++e) {
+            const size_t at = (size_t)src * row_elems + e;
+            uint16_t h;
+            if (q_dtype == UCM_DTYPE_F16) { h = ((const uint16_t*)q)[at]; }
+            else if (q_dtype == UCM_DTYPE_BF16) { h = orc_f32_to_f16(orc_bf16_to_f32(((const uint16_t*)q)[at])); }
+            else { h = orc_f32_to_f16(((const float*)q)[at]); }
+            ((uint16_t*)ring_f16)[dst + e] = h;
+        }
+    }
     return UCM_OK;
 }
 

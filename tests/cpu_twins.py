@@ -14,7 +14,7 @@ TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_se
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
-         "ucm_kvstar_votes", "ucm_kvstar_votes_tables"]
+         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries"]
 
 
 def twin_caller(signatures):
@@ -483,10 +483,21 @@ def run_kvstar(call, side):
         cell = d_pad * K_M
         t = side.up(np.full((K_L, K_HKV, K_ROWS, cell), 0x3c00, np.uint16))            # fp16 ones where nothing is written
         call("ucm_kvstar_block_repre", k_layers, K_L, K_NB, side.ptr(ids), side.ptr(slots), len(x["ids"]), K_BS, K_HKV, K_D,
-             K_MERGE, None if pr is None else side.ptr(pr), 0 if pr is None else K_HKV * K_DP, dp, d_pad, side.ptr(t), K_ROWS,
-             K_HKV * K_ROWS * cell, K_ROWS * cell, cell, None)
+             K_MERGE, None if pr is None else side.ptr(pr), 0 if pr is None else K_HKV * K_DP, None, 0, dp, d_pad, side.ptr(t),
+             K_ROWS, K_HKV * K_ROWS * cell, K_ROWS * cell, cell, None)
         tables[name] = t
         out["table_" + name] = t
+    # every listed block pruned by a list of its own choice: the two layers' lists as the two lists of EVERY layer,
+    # blocks alternating between them, one naming a list that does not exist (skipped)
+    cell = K_DPAD * K_M
+    sel_h = (np.arange(len(x["ids"])) % 2).astype(np.int32)
+    sel_h[5] = 2
+    t, sel_in = side.up(np.full((K_L, K_HKV, K_ROWS, cell), 0x3c00, np.uint16)), side.up(sel_h)
+    call("ucm_kvstar_block_repre", k_layers, K_L, K_NB, side.ptr(ids), side.ptr(slots), len(x["ids"]), K_BS, K_HKV, K_D, K_MERGE,
+         side.ptr(lists), 0, side.ptr(sel_in), K_L, K_DP, K_DPAD, side.ptr(t), K_ROWS, K_HKV * K_ROWS * cell, K_ROWS * cell,
+         cell, None)
+    out["table_by_block"] = t
+    x["list_sel"] = sel_h
     side.sync()
     # votes over layer 0 of the pruned table
     cell = K_DPAD * K_M
@@ -524,6 +535,22 @@ def run_kvstar(call, side):
          side.ptr(sel), side.ptr(task_tables), side.ptr(head_strides), cell, side.ptr(seg_off), side.ptr(seg_len), 3, 5, K_M,
          K_HKV, K_DP, K_DPAD, side.ptr(ws_max), mf.value, side.ptr(ws_part), pf.value, side.ptr(votes_t), K_ROWS, 0, None)
     out["votes_tables"] = votes_t
+    # query tokens parked as fp16 from bf16, fp16 and fp32 queries: rows out of order, one row and one place out of range
+    row_elems = K_HKV * K_G * K_D
+    rng = np.random.default_rng(7410)
+    qf = (rng.standard_normal((6, row_elems)) * np.array([1e-6, 1.0, 300.0, 7e4, 1.0, 1.0], np.float32)[:, None]).astype(np.float32)
+    qf[4, :4] = [np.inf, -np.inf, 0.0, -0.0]
+    src = side.up(np.array([5, 0, 6, 3, 2, 1], np.int32))                  # 6 is past the queries
+    dst = side.up((np.array([0, 2, 3, 1, 9, 4], np.int64)) * row_elems)     # 9 is past the ring of 6 rows
+    with np.errstate(over="ignore"):
+        q_half = qf.astype(np.float16).view(np.uint16)
+    for name, code, arr in (("park_f32", 0, qf), ("park_bf16", 1, oracle.bf16_bits(qf)), ("park_f16", 2, q_half)):
+        ring, q_in = side.up(np.full((6, row_elems), 0x3c00, np.uint16)), side.up(arr)
+        call("ucm_kvstar_park_queries", side.ptr(q_in), code, 6, row_elems, side.ptr(src), side.ptr(dst), 6, side.ptr(ring),
+             6 * row_elems, None)
+        side.sync()
+        out[name] = ring
+    x["park_q"] = qf
     side.sync()
     return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
 

@@ -205,6 +205,19 @@ def test_kvstar_twins_reproduce_the_oracle(ucm):
             if name == "pruned":
                 assert (ref[l][..., K.K_DP:] == 0).all() and (ref[l][..., : K.K_DP] != 0).any()
     assert set(final) == set(range(K.K_ROWS))
+    # a list per listed block: every block against the oracle run with the list it names; the one that names no list is skipped
+    cells = got["table_by_block"].reshape(K.K_L, K.K_HKV, K.K_ROWS, K.K_DPAD // 8, K.K_M, 8)
+    by_block = cells.transpose(0, 2, 4, 1, 3, 5).reshape(K.K_L, K.K_ROWS, K.K_M, K.K_HKV, K.K_DPAD)
+    last = {}
+    for i, (b, s_) in enumerate(zip(x["ids"], x["slots"])):
+        if 0 <= b < K.K_NB and x["list_sel"][i] < K.K_L:
+            last[int(s_)] = (int(b), int(x["list_sel"][i]))
+    for l in range(K.K_L):
+        want = np.full((K.K_ROWS, K.K_M, K.K_HKV, K.K_DPAD), 0x3c00, np.uint16)
+        for slot, (b, which) in last.items():
+            O.kvstar_block_repre(x["caches"][l], np.array([b], np.int32), np.array([slot], np.int32), K.K_MERGE, want,
+                                 pruned=x["lists"][which])
+        assert np.array_equal(by_block[l], want), l
     for key in ("votes", "votes_tables"):
         for t, (a, n) in enumerate(zip(K.K_OFF, K.K_LEN)):
             if n:
@@ -212,6 +225,19 @@ def test_kvstar_twins_reproduce_the_oracle(ucm):
                 assert np.array_equal(got[key][a : a + n].view(np.uint32), want.view(np.uint32)), (key, t)
                 assert abs(float(want.sum()) - K.K_X * K.K_HKV * K.K_G) < 1e-3          # every query row votes with weight one
     assert np.array_equal(got["votes"], got["votes_tables"])
+    # parked query tokens: numpy's own float32 -> float16 conversion (round to nearest even, overflow to inf); the row
+    # past the queries and the place past the ring change nothing
+    qf = x["park_q"]
+    want = np.full((6, qf.shape[1]), 0x3c00, np.uint16)
+    with np.errstate(over="ignore"):
+        for s_, d_ in ((5, 0), (0, 2), (3, 1), (1, 4)):
+            want[d_] = qf[s_].astype(np.float16).view(np.uint16)
+        assert np.array_equal(got["park_f32"], want), np.argwhere(got["park_f32"] != want)[:4]
+        want16 = want.copy()
+        for s_, d_ in ((5, 0), (0, 2), (3, 1), (1, 4)):
+            want16[d_] = O.bf16_to_f32(O.bf16_bits(qf[s_])).astype(np.float16).view(np.uint16)
+        assert np.array_equal(got["park_bf16"], want16)
+        assert np.array_equal(got["park_f16"][[0, 2, 1, 4]], qf[[5, 0, 3, 1]].astype(np.float16).view(np.uint16))
     # a task whose query block, channel list or rows lie outside what the call declares is skipped: its votes keep
     # the fill value, the other tasks' are unchanged
     a0, n0, a2, n2 = K.K_OFF[0], K.K_LEN[0], K.K_OFF[2], K.K_LEN[2]

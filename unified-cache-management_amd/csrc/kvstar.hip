@@ -177,6 +177,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows, unsigned block_size,
     unsigned kv_heads, unsigned head_dim, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride,
+    const int32_t* __restrict__ list_sel, unsigned n_lists,
     unsigned d_pruned, unsigned d_pad, unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride,
     int64_t row_stride, unsigned m_chunk)
 {
@@ -194,7 +195,11 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     if (pruned) {   // this layer's lists (a stride of 0: one set of lists for every layer)
         for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = my_lists[e]; }
     }
-    const PieceMap pm = make_piece_map(my_lists, kv_heads, head_dim, d_pruned, pieces);
+    PieceMap pm = make_piece_map(my_lists, kv_heads, head_dim, d_pruned, pieces);
+    // list_sel: every listed block names the list of the layer's n_lists it is pruned by (the blocks of several
+    // requests in one launch, each request with channels of its own); the list in use is replaced when a block
+    // names another one, which is once per request and workgroup
+    unsigned cur_list = 0;
 
     struct Unit {
         unsigned item, m0, w_first;                      // cache block in the list, first sub-block of the chunk, first work item
@@ -216,7 +221,8 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     auto seek = [&](Unit& u, unsigned from) {
         for (unsigned i = from; i < n_items; i += gridDim.x) {
             const unsigned id = static_cast<unsigned>(block_ids[i]);
-            if (id < num_blocks && static_cast<unsigned>(slots[i]) < rows) {
+            if (id < num_blocks && static_cast<unsigned>(slots[i]) < rows &&
+                (!list_sel || static_cast<unsigned>(list_sel[i]) < n_lists)) {
                 u.item = i;
                 u.m0 = 0;
                 u.w_first = 0;
@@ -282,6 +288,13 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
             if (w < n_work) { *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o; }
         }
         if (live && u.w_first + kThreads * kBatch >= mc * ncg) { // the chunk is staged: write its pieces
+            if (list_sel && static_cast<unsigned>(list_sel[u.item]) != cur_list) {      // (the same for all threads)
+                cur_list = static_cast<unsigned>(list_sel[u.item]);
+                const int32_t* lists = my_lists + static_cast<size_t>(cur_list) * kv_heads * d_pruned;
+                __syncthreads();                         // nobody reads the old list any more
+                for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = lists[e]; }
+                pm = make_piece_map(lists, kv_heads, head_dim, d_pruned, pieces);
+            }
             __syncthreads();
             unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride +
                                   static_cast<int64_t>(static_cast<unsigned>(slots[u.item])) * row_stride;
@@ -316,15 +329,16 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
 __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
-    unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride, unsigned d_pruned,
-    unsigned d_pad,
+    unsigned head_dim, unsigned merge, const int32_t* __restrict__ pruned, int64_t pruned_layer_stride,
+    const int32_t* __restrict__ list_sel, unsigned n_lists, unsigned d_pruned, unsigned d_pad,
     unsigned short* __restrict__ repre, int64_t layer_stride, int64_t head_stride, int64_t row_stride, unsigned m_chunk)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned short stage[];   // [m_chunk][row + 8]
     const unsigned M = block_size / merge;
     const unsigned id = static_cast<unsigned>(block_ids[blockIdx.x]);
     const unsigned slot = static_cast<unsigned>(slots[blockIdx.x]);
-    if (id >= num_blocks || slot >= rows) { return; }   // whole workgroup: never dereference a bad id
+    const unsigned sel = list_sel ? static_cast<unsigned>(list_sel[blockIdx.x]) : 0u;
+    if (id >= num_blocks || slot >= rows || (list_sel && sel >= n_lists)) { return; }   // whole workgroup: never dereference a bad id
     const unsigned row = kv_heads * head_dim, ncg = row / 8, srow_stride = row + 8;
     const unsigned short* blk = static_cast<const unsigned short*>(k_layers[blockIdx.y]) +
                                 static_cast<size_t>(id) * block_size * row;
@@ -332,8 +346,10 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const unsigned pieces = d_pad / 8;
     unsigned short* out = repre + static_cast<int64_t>(blockIdx.y) * layer_stride + static_cast<int64_t>(slot) * row_stride;
     int32_t* kept = reinterpret_cast<int32_t*>(stage + static_cast<size_t>(m_chunk) * srow_stride);
-    const int32_t* my_lists = pruned ? pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride : nullptr;
-    if (pruned) {   // this layer's lists (a stride of 0: one set of lists for every layer)
+    // this layer's lists (a stride of 0: one set of lists for every layer), and of them the one the block names
+    const int32_t* my_lists = pruned ? pruned + static_cast<int64_t>(blockIdx.y) * pruned_layer_stride +
+                                           static_cast<size_t>(sel) * kv_heads * d_pruned : nullptr;
+    if (pruned) {
         for (unsigned e = threadIdx.x; e < kv_heads * d_pruned; e += kThreads) { kept[e] = my_lists[e]; }
     }
     const PieceMap pm = make_piece_map(my_lists, kv_heads, head_dim, d_pruned, pieces);
@@ -948,14 +964,80 @@ __global__ __launch_bounds__(kThreads) void kvstar_vote_kernel(
 
 }  // namespace
 
+// ---- query groups ----------------------------------------------------------------------------------
+// The query tokens a step contributes to its requests' retrieval groups, copied aside as fp16: the reference clones
+// one token per request and layer (save_to_standby, ucm/sparse/kvstar/multistep.py:318-324) and converts a group
+// when it is retrieved (torch.stack(...).to(torch.float16), :252-254).  One workgroup per row; the conversion is
+// the round-to-nearest-even one of that .to().
+namespace {
+
+template <int kType>   // UCM_DTYPE_*
+__global__ __launch_bounds__(kThreads) void kvstar_park_kernel(
+    const void* __restrict__ q, int64_t q_rows, unsigned row_elems, const int32_t* __restrict__ src_rows,
+    const int64_t* __restrict__ dst_off, unsigned short* __restrict__ ring, int64_t ring_elems)
+{
+    const int64_t src = src_rows[blockIdx.x], dst = dst_off[blockIdx.x];
+    // rows and places come from device memory: a row outside the queries or a place outside the ring is skipped
+    if (src < 0 || src >= q_rows || dst < 0 || dst + row_elems > ring_elems || (dst & 7) != 0) { return; }
+    unsigned short* out = ring + dst;
+    for (unsigned e = threadIdx.x * 8; e < row_elems; e += kThreads * 8) {
+        unsigned short h[8];
+        if constexpr (kType == UCM_DTYPE_F16) {
+            *reinterpret_cast<u32x4*>(h) = ucm::gload16(static_cast<const unsigned short*>(q) + src * row_elems + e);
+        } else if constexpr (kType == UCM_DTYPE_BF16) {
+            const u32x4 v = ucm::gload16(static_cast<const unsigned short*>(q) + src * row_elems + e);
+            const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                h[2 * j] = f32_to_f16_bits(__uint_as_float(w[j] << 16));
+                h[2 * j + 1] = f32_to_f16_bits(__uint_as_float(w[j] & 0xffff0000u));
+            }
+        } else {
+            const float* f = static_cast<const float*>(q) + src * row_elems + e;
+            const u32x4 a = ucm::gload16(f), b = ucm::gload16(f + 4);
+            const unsigned w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { h[j] = f32_to_f16_bits(__uint_as_float(w[j])); }
+        }
+        ucm::gstore16(out + e, *reinterpret_cast<const u32x4*>(h));
+    }
+}
+
+}  // namespace
+
+extern "C" int ucm_kvstar_park_queries(const void* q, int q_dtype, int64_t q_rows, int row_elems, const int32_t* src_rows,
+                                       const int64_t* dst_off, int n, void* ring_f16, int64_t ring_elems, ucm_stream_t stream)
+{
+    UCM_REQUIRE(n >= 0 && q_rows >= 0 && ring_elems >= 0, "ucm_kvstar_park_queries: n=%d q_rows=%lld ring_elems=%lld", n,
+                static_cast<long long>(q_rows), static_cast<long long>(ring_elems));
+    if (n == 0) { return UCM_OK; }
+    UCM_REQUIRE(q && src_rows && dst_off && ring_f16, "ucm_kvstar_park_queries: null pointer");
+    UCM_REQUIRE(q_dtype == UCM_DTYPE_F32 || q_dtype == UCM_DTYPE_BF16 || q_dtype == UCM_DTYPE_F16, "ucm_kvstar_park_queries: q_dtype=%d", q_dtype);
+    UCM_REQUIRE(row_elems > 0 && row_elems % 8 == 0, "ucm_kvstar_park_queries: row_elems=%d (a positive multiple of 8)", row_elems);
+    UCM_REQUIRE(ucm::aligned16(q) && ucm::aligned16(ring_f16), "ucm_kvstar_park_queries: q and ring must be 16-byte aligned");
+    UCM_REQUIRE(n <= 0x7fffffff, "ucm_kvstar_park_queries: n=%d", n);
+    hipStream_t hs = ucm::as_stream(stream);
+#define UCM_PARK(T)                                                                                                   \
+    hipLaunchKernelGGL(kvstar_park_kernel<T>, dim3(static_cast<unsigned>(n)), dim3(kThreads), 0, hs, q, q_rows,       \
+                       static_cast<unsigned>(row_elems), src_rows, dst_off, static_cast<unsigned short*>(ring_f16), ring_elems)
+    if (q_dtype == UCM_DTYPE_F16) { UCM_PARK(UCM_DTYPE_F16); }
+    else if (q_dtype == UCM_DTYPE_BF16) { UCM_PARK(UCM_DTYPE_BF16); }
+    else { UCM_PARK(UCM_DTYPE_F32); }
+#undef UCM_PARK
+    UCM_LAUNCH_CHECK("ucm_kvstar_park_queries");
+}
+
 extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
                                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
                                       int kv_heads, int head_dim, int merge, const int32_t* pruned,
-                                      int64_t pruned_layer_stride, int d_pruned,
-                                      int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
-                                      int64_t repre_head_stride, int64_t repre_row_stride, ucm_stream_t stream)
+                                      int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
+                                      int d_pruned, int d_pad, void* repre_f16, int repre_rows,
+                                      int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
+                                      ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_kvstar_block_repre: n=%d", n);
+    UCM_REQUIRE(!pruned_sel || (pruned && n_pruned_lists >= 1), "ucm_kvstar_block_repre: pruned_sel needs the lists and their number");
+    const int lists_per_layer = pruned_sel ? n_pruned_lists : 1;
     if (n == 0) { return UCM_OK; }
     UCM_REQUIRE(k_layers && block_ids && slots && repre_f16, "ucm_kvstar_block_repre: null pointer");
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535 && num_blocks > 0 && repre_rows > 0 && block_size > 0 && kv_heads > 0 &&
@@ -965,7 +1047,7 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     UCM_REQUIRE(d_pruned > 0 && d_pruned <= head_dim && d_pad >= d_pruned, "ucm_kvstar_block_repre: d_pruned=%d d_pad=%d",
                 d_pruned, d_pad);
     UCM_REQUIRE(pruned || d_pruned == head_dim, "ucm_kvstar_block_repre: d_pruned < head_dim needs the channel list");
-    UCM_REQUIRE(pruned_layer_stride == 0 || pruned_layer_stride >= static_cast<int64_t>(kv_heads) * d_pruned,
+    UCM_REQUIRE(pruned_layer_stride == 0 || pruned_layer_stride >= static_cast<int64_t>(lists_per_layer) * kv_heads * d_pruned,
                 "ucm_kvstar_block_repre: pruned_layer_stride=%lld", static_cast<long long>(pruned_layer_stride));
     const int M = block_size / merge;
     // a (row, kv head) cell is M*d_pad elements; the cells must not overlap: heads outside rows (head planes) or
@@ -1000,7 +1082,8 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                            block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(n),            \
                            static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),                     \
                            static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), pruned,                 \
-                           pruned_layer_stride, static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),       \
+                           pruned_layer_stride, pruned_sel, static_cast<unsigned>(lists_per_layer),                  \
+                           static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),                            \
                            static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride,          \
                            repre_row_stride, m_chunk);                                                               \
     } while (0)
@@ -1018,8 +1101,8 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
         hipLaunchKernelGGL(kvstar_repre_any_kernel, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, hs,
                            k_layers, block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(repre_rows),
                            static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim),
-                           static_cast<unsigned>(merge), pruned, pruned_layer_stride, static_cast<unsigned>(d_pruned),
-                           static_cast<unsigned>(d_pad),
+                           static_cast<unsigned>(merge), pruned, pruned_layer_stride, pruned_sel,
+                           static_cast<unsigned>(lists_per_layer), static_cast<unsigned>(d_pruned), static_cast<unsigned>(d_pad),
                            static_cast<unsigned short*>(repre_f16), repre_layer_stride, repre_head_stride, repre_row_stride,
                            m_chunk);
         break;

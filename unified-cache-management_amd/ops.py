@@ -581,9 +581,10 @@ def kvstar_table_from_reference(repre: torch.Tensor, layout: str = "head") -> to
 
 def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                        block_size: int, kv_heads: int, head_dim: int, num_blocks: int, merge: int,
-                       pruned: Optional[torch.Tensor] = None) -> None:
+                       pruned: Optional[torch.Tensor] = None, pruned_sel: Optional[torch.Tensor] = None) -> None:
     """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); pruned int32 [kv_heads, d_pruned] (one set of
-    channel lists for every layer), [L, kv_heads, d_pruned] (lists per layer) or None."""
+    channel lists for every layer), [L, kv_heads, d_pruned] (lists per layer) or None.  With pruned_sel (int32 [n]:
+    the list each listed block is pruned by) pruned is [n_lists, kv_heads, d_pruned] or [L, n_lists, kv_heads, d_pruned]."""
     if repre.dim() != 6 or repre.dtype != torch.float16 or repre.shape[4] * merge != block_size or \
             repre.shape[1] != kv_heads or repre.shape[5] != 8:
         raise ValueError("repre must be float16 [L, kv_heads, rows, d_pad/8, block_size/merge, 8]")
@@ -593,12 +594,20 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
     if block_ids.numel() != slots.numel():
         raise ValueError("block_ids and slots differ in length")
     d_pruned = head_dim if pruned is None else pruned.shape[-1]
-    per_layer = pruned is not None and pruned.dim() == 3
+    n_lists = 0
+    if pruned_sel is not None:
+        if pruned is None or pruned.dim() not in (3, 4) or pruned_sel.numel() != block_ids.numel():
+            raise ValueError("pruned_sel needs pruned [n_lists, kv_heads, d_pruned] (or one such set per layer) and one entry per block")
+        per_layer = pruned.dim() == 4
+        n_lists = pruned.shape[-3]
+    else:
+        per_layer = pruned is not None and pruned.dim() == 3
     if pruned is not None and (pruned.shape[-2] != kv_heads or (per_layer and pruned.shape[0] != repre.shape[0])):
         raise ValueError("pruned must be [kv_heads, d_pruned] or [layers, kv_heads, d_pruned]")
     _lib.call("ucm_kvstar_block_repre", k_layers.ptr(), repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
               _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
-              _opt(pruned, torch.int32, "pruned"), pruned.stride(0) if per_layer else 0, d_pruned, repre.shape[3] * 8,
+              _opt(pruned, torch.int32, "pruned"), pruned.stride(0) if per_layer else 0,
+              _opt(pruned_sel, torch.int32, "pruned_sel"), n_lists, d_pruned, repre.shape[3] * 8,
               repre.data_ptr(),
               repre.shape[2], repre.stride(0), head_stride, row_stride, _stream())
 

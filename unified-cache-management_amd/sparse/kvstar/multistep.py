@@ -204,6 +204,7 @@ class ReqPerLayerState:
         self.plan_sink: Optional[list] = None            # set by the plugin: loads that follow the device's own list
         self.standby_row: Optional[torch.Tensor] = None  # set by the plugin: this step's query token, already copied aside
         self.window_sink: Optional[list] = None          # set by the plugin: window copies are collected, not issued here
+        self.repre_sink: Optional[list] = None           # set by the plugin: representatives of a layer's requests in one go
         self._d_pruned_index32 = None
         self.standby_query_group: Dict[str, list] = {}
         self.do_retrieve_query_group: Dict[str, torch.Tensor] = {}
@@ -375,8 +376,15 @@ class ReqPerLayerState:
     def compute_block_repre(self, num_blocks_need_dump: int) -> None:
         if self.req_meta.stage != ReqStage.PREFILL or not self.req_meta.is_last_chunk:
             return
-        repre = self.extract_block_repre(self.req_meta.vllm_block_ids[: self.num_blocks_dumped + num_blocks_need_dump],
-                                         prune_dim_enable=True)
+        ids = self.req_meta.vllm_block_ids[: self.num_blocks_dumped + num_blocks_need_dump]
+        if self.repre_sink is not None and ids and ids[-1] >= 2:
+            self.repre_sink.append((self, list(ids)))   # taken with the layer's other requests (set_block_repre follows)
+            return
+        self.set_block_repre(self.extract_block_repre(ids, prune_dim_enable=True))
+
+    def set_block_repre(self, repre) -> None:
+        """The representatives of all full prompt blocks are in: the ones between the windows are kept, the window
+        blocks copied aside (multistep.py:483-501)."""
         if repre is not None:
             repre = None if repre.shape[0] <= 2 else repre[self.init_window_sz : -self.local_window_sz]
         self.blk_repre = repre
@@ -634,6 +642,56 @@ class KVStarMultiStep(UcmSparseBase):
             ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
             ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
 
+    def _flush_repre(self, sink: list, layer_name: str, forward_context) -> None:
+        """Sub-block representatives and channel choice of every request that ends its prefill in this step, for one
+        layer: one pass over the paged cache for the blocks' mean |k| (of all requests), one mean per request over
+        its blocks, one top-k for the kept channels, one launch that writes every request's representatives with its
+        own channels (``extract_block_repre`` per request in the reference, multistep.py:279-316).  The requests'
+        tables are row ranges of one tensor."""
+        if not sink:
+            return
+        cfg = self.kvstar_multistep_cfg
+        kv = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
+        k_cache = kv[0]
+        n_total, block_size, kv_heads, head_dim = k_cache.shape
+        dev = k_cache.device
+        known = self._layer_ptrs.get(("k", layer_name))
+        if known is None or known[0] != k_cache.data_ptr():
+            known = self._layer_ptrs[("k", layer_name)] = (k_cache.data_ptr(), ops.LayerPointers([k_cache]))
+        key = ("repre", tuple(st.req_meta.request_id for st, _ in sink))
+        shared = self._step_cache.get(key)
+        if shared is None:        # the same for every layer of the step
+            counts = [len(ids) for _, ids in sink]
+            flat = [b for _, ids in sink for b in ids]
+            which = [r for r, n in enumerate(counts) for _ in range(n)]
+            both = ops.upload(torch.tensor([flat, which], dtype=torch.int32), dev)
+            shared = self._step_cache[key] = (both[0], both[1], torch.arange(len(flat), dtype=torch.int32, device=dev),
+                                               torch.tensor(counts, dtype=torch.int64, device=dev), counts)
+        ids_dev, which_dev, rows, counts_dev, counts = shared
+        n = ids_dev.numel()
+        merge, ratio = cfg["blk_repre_inner_token_merge"], cfg["blk_repre_dim_prune_ratio"]
+        index = lists32 = None
+        if ratio < 0.98:
+            # mean |k| per (head, channel) over all tokens of a request's blocks: the blocks' own means of |k|, read
+            # from the paged cache in one pass, averaged per request
+            per_block = torch.empty((1, n, kv_heads * head_dim), dtype=torch.float32, device=dev)
+            ops.block_mean(known[1], ids_dev, rows, per_block, block_size, kv_heads, head_dim, n_total,
+                           mode=ops.MEAN_F32 | ops.MEAN_ABS)
+            absmean = torch.segment_reduce(per_block[0], "mean", lengths=counts_dev, axis=0, unsafe=True)
+            _, index = torch.topk(absmean.view(len(counts), kv_heads, head_dim), k=round(head_dim * ratio), dim=-1)
+            lists32 = index.to(torch.int32)
+        d_pruned = head_dim if index is None else index.shape[-1]
+        d_pad = (d_pruned + 15) // 16 * 16
+        table = ops.kvstar_table(1, kv_heads, n, block_size // merge, d_pad, dev)
+        ops.kvstar_block_repre(known[1], ids_dev, rows, table, block_size, kv_heads, head_dim, n_total, merge, pruned=lists32,
+                               pruned_sel=None if lists32 is None else which_dev)
+        at = 0
+        for r, (st, _) in enumerate(sink):
+            if index is not None:
+                st.d_pruned_index, st._d_pruned_index32 = index[r], lists32[r]
+            st.set_block_repre(kvstar_retrieve.BlockRepre(table[0][:, at : at + counts[r]], d_pruned))
+            at += counts[r]
+
     def _standby_rows(self, query):
         """The decoding requests' query tokens of this layer copied aside in one go (``query[start].clone()`` per
         request in the reference, multistep.py:318-324); every request then keeps a view of its row."""
@@ -655,13 +713,14 @@ class KVStarMultiStep(UcmSparseBase):
         sink = self._load_sink()
         plan = [] if sink is not None and self.kvstar_multistep_cfg["device_plans"] else None
         windows = [] if self.kvstar_multistep_cfg["device_loads"] else None
+        repres = [] if which == "attention_finished" else None
         rows = place = None
         if which == "attention_begin":
             rows, place = self._standby_rows(args[0])
         for req_meta in self._sparse_metadata.requests:
             state = self.create_layerwise_req_state(req_meta, layer_name)
             state.update_meta(req_meta, forward_context)
-            state.load_sink, state.plan_sink, state.window_sink = sink, plan, windows
+            state.load_sink, state.plan_sink, state.window_sink, state.repre_sink = sink, plan, windows, repres
             state.standby_row = None if rows is None or req_meta.request_id not in place else rows[place[req_meta.request_id]]
             if which == "attention_begin":
                 state.attention_begin(*args, forward_context, batch=batch)
@@ -669,6 +728,7 @@ class KVStarMultiStep(UcmSparseBase):
                 state.attention_finished(*args, forward_context)
         if batch is not None:
             batch.flush()
+        self._flush_repre(repres, layer_name, forward_context)      # (before the windows: it queues the ending requests' saves)
         self._flush_windows(windows, layer_name, forward_context)
         self._flush_loads(sink, layer_name, forward_context)
         self._flush_planned(plan, layer_name, forward_context)
