@@ -39,6 +39,7 @@ from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
 from ..esa.esa import _kv_cache_blocks, block_hash_func, get_offset
 from ... import ops
 from . import retrieve as kvstar_retrieve
+from .layer_path import KVStarLayerPath
 
 ReqType = Union[str, int]
 
@@ -193,10 +194,11 @@ class ReqPerLayerState:
         self.num_tokens = 0
         self.store_instance, self.store_name = store_instance, store_name
         self.req_meta = req_meta
-        self.init_window = self.local_window = None
+        self._init_window = self._local_window = None
+        self._kept = None                                # (buffer [K|V][window block], first, init blocks, local blocks)
         self.init_window_sz, self.local_window_sz = sparse_cfg["init_window_sz"], sparse_cfg["local_window_sz"]
         self.block_size = None
-        self.k_cache = self.v_cache = None
+        self._kv = None                                  # the layer's cache [K|V][block][token][head][channel]
         self.d_pruned_index = None
         self.local_tp_rank, self.total_tp_size = rank, tp_size
         self.blk_trans_tasks: Dict[int, object] = {}
@@ -213,6 +215,30 @@ class ReqPerLayerState:
         self._planned: Dict[str, tuple] = {}             # record -> (task id, results, row) of a load planned on the device
         self.task_waiter: Dict[str, int] = {}
         self.num_blocks_dumped = 0
+
+    # the layer's K and V planes and the window copies, as the reference's attributes of these names; the views are made
+    # when somebody asks for them (the paths that handle a layer's requests together work on addresses)
+    k_cache = property(lambda self: None if self._kv is None else self._kv[0])
+    v_cache = property(lambda self: None if self._kv is None else self._kv[1])
+
+    def _window(self, which: int):
+        if self._kept is None:
+            return self._local_window if which else self._init_window
+        kept, at, n_init, n_local = self._kept
+        if which == 0:
+            return kept[0, at : at + n_init], kept[1, at : at + n_init]
+        return (kept[0, at + n_init : at + n_init + n_local], kept[1, at + n_init : at + n_init + n_local]) if n_local else None
+
+    def _set_window(self, which: int, value) -> None:
+        if self._kept is not None:                       # leaving the shared buffer: both windows become plain tensors
+            self._init_window, self._local_window, self._kept = self._window(0), self._window(1), None
+        if which:
+            self._local_window = value
+        else:
+            self._init_window = value
+
+    init_window = property(lambda self: self._window(0), lambda self, v: self._set_window(0, v))
+    local_window = property(lambda self: self._window(1), lambda self, v: self._set_window(1, v))
 
     @classmethod
     def block_hash(cls, request_id, block_id) -> str:
@@ -326,7 +352,14 @@ class ReqPerLayerState:
 
     def _collect_planned(self, record: str) -> None:
         """The host's copy of a list whose blocks were loaded on the device (KeyError if there is none)."""
-        task_id, results, row = self._planned[record]
+        found = self._planned.get(record)
+        if found is None:
+            # (a load issued for the layer's requests together leaves no entry per request: the task itself is asked)
+            found = kvstar_retrieve.DeviceResult(self.task_waiter[record])
+            if found is None:
+                raise KeyError(record)
+            found = (None,) + found
+        _, results, row = found
         chosen = results.chosen(row)
         dict.__setitem__(self.step_group_retrieve_indices, record, chosen)
         dict.__setitem__(self.step_group_retrieve_result, record, [self.block_hashes[i + self.init_window_sz] for i in chosen])
@@ -435,10 +468,8 @@ class ReqPerLayerState:
         if self.block_size:
             return
         attn = forward_context.no_compile_layers[self.layer_name]
-        kv_cache = attn.kv_cache[forward_context.virtual_engine]
-        self.k_cache, self.v_cache = kv_cache[0], kv_cache[1]
-        self.block_size = self.k_cache.shape[1]
-        self.num_key_heads, self.head_size = self.k_cache.shape[2], self.k_cache.shape[3]
+        self._kv = attn.kv_cache[forward_context.virtual_engine]
+        _, _, self.block_size, self.num_key_heads, self.head_size = self._kv.shape
         self.block_hashes = self.req_meta.req_block_hashes
 
     def update_meta(self, req_meta: ReqMeta, forward_context=None) -> None:
@@ -489,6 +520,10 @@ class KVStarMultiStep(UcmSparseBase):
         self.token_blk_size = vllm_config.cache_config.block_size
         self._step_cache: Dict[object, tuple] = {}       # what every layer's hooks of one step share (tables, indices)
         self._layer_ptrs: Dict[str, tuple] = {}
+        self._layer_ids: Dict[str, int] = {}
+        self._layer_slots: Dict[str, int] = {}             # layers in the order their hooks first ran
+        self._n_slots = 0                                  # how many there were in a complete step (0: none seen yet)
+        self._path: Optional[KVStarLayerPath] = None       # the decode steps of a layer's requests at once (see _hook)
         if role == UcmSparseRole.WORKER:
             kvstar_retrieve.Setup(kvstar_retrieve.SetupParam(
                 cpuNumaIds=[], physicalCorePerNuma=0, allocRatio=0.75, blkRepreSize=4096, deviceType=kvstar_retrieve.CPU,
@@ -517,6 +552,16 @@ class KVStarMultiStep(UcmSparseBase):
         for state in self.req_states.pop(request_id, None) or []:
             if state is not None:
                 state.release()
+        if self._path is not None:
+            self._path.request_finished(request_id)
+
+    def _layer_path(self) -> Optional[KVStarLayerPath]:
+        """The path that handles a layer's requests together (layer_path.py); it needs what the three switches stand
+        for: batched retrieval, a store whose blocks a kernel can read, loads that follow the device's lists."""
+        cfg = self.kvstar_multistep_cfg
+        if self._path is None and cfg["batch_retrieval"] and cfg["device_plans"] and self._load_sink() is not None:
+            self._path = KVStarLayerPath(self, None)
+        return self._path
 
     def _load_sink(self) -> Optional[list]:
         """A list that collects the loads of a hook's requests, when they can be carried out as one copy: the store's
@@ -596,6 +641,18 @@ class KVStarMultiStep(UcmSparseBase):
             ops.kv_load_planned(known[1], 0, layer_id, 1, kv.stride(0) * es, kv.stride(1) * es, kv.shape[1], pool, pool_block_bytes,
                                 results.idx.unsqueeze(0), tables[0], tables[1], tables[2], load_count=results.cnt.unsqueeze(0))
 
+    def _of_all_layers(self, what, layer_name: str, make):
+        """Layer ``layer_name``'s part of a buffer that every layer of this step needs in the same shape: once the
+        number of layers is known (a step has gone by), ``make(n)`` allocates for all of them at the first, instead
+        of one device allocation per layer."""
+        slot = self._layer_slots.setdefault(layer_name, len(self._layer_slots))
+        if slot >= self._n_slots:
+            return make(1)[0]
+        whole = self._step_cache.get(what)
+        if whole is None:
+            whole = self._step_cache[what] = make(self._n_slots)
+        return whole[slot]
+
     def _flush_windows(self, sink: list, layer_name: str, forward_context) -> None:
         """The window copies of a hook's requests as one pointer-array copy: "save" keeps the init and local window
         blocks of a request that ends its prefill (multistep.py:326-346: four indexed clones per request), "restore"
@@ -609,34 +666,42 @@ class KVStarMultiStep(UcmSparseBase):
             raise ValueError("cache blocks must be contiguous")
         cache = kv.data_ptr()
         dst, src = [], []
-        saves = [st for st, what in sink if what == "save"]
+        saves = [(st, st.window_blocks()) for st, what in sink if what == "save"]
         if saves:
-            counts = [tuple(len(b) for b in st.window_blocks()) for st in saves]
-            total = sum(a + b for a, b in counts)
-            kept = torch.empty((2, total) + tuple(kv.shape[2:]), dtype=kv.dtype, device=kv.device)   # [K|V][window block]
-            at = 0
-            for st, (n_init, n_local) in zip(saves, counts):
-                head, tail = st.window_blocks()
-                st.init_window = (kept[0, at : at + n_init], kept[1, at : at + n_init])
-                st.local_window = (kept[0, at + n_init : at + n_init + n_local], kept[1, at + n_init : at + n_init + n_local]) if n_local else None
+            total = sum(len(head) + len(tail) for _, (head, tail) in saves)
+            kept = self._of_all_layers(("kept", total), layer_name, lambda n: torch.empty(
+                (n, 2, total) + tuple(kv.shape[2:]), dtype=kv.dtype, device=kv.device))                # [K|V][window block]
+            base, at = kept.data_ptr(), 0
+            for st, (head, tail) in saves:
+                st._init_window = st._local_window = None
+                st._kept = (kept, at, len(head), len(tail))
                 for j, b in enumerate(list(head) + list(tail)):
                     for plane in (0, 1):
                         src.append(cache + plane * kv_stride + b * block_bytes)
-                        dst.append(kept.data_ptr() + (plane * total + at + j) * block_bytes)
-                at += n_init + n_local
+                        dst.append(base + (plane * total + at + j) * block_bytes)
+                at += len(head) + len(tail)
         for st, what in sink:
             if what != "restore":
                 continue
             ids = st.req_meta.vllm_block_ids
-            pairs = list(zip(ids[: st.init_window_sz], range(st.init_window_sz)))
+            if st._kept is not None:
+                kept, at, n_init, n_local = st._kept
+                base, total = kept.data_ptr(), kept.shape[1]
+                blocks = list(ids[: st.init_window_sz][:n_init]) + (list(ids[-n_local:]) if n_local else [])
+                for plane in (0, 1):
+                    for j, b in enumerate(blocks):
+                        src.append(base + (plane * total + at + j) * block_bytes)
+                        dst.append(cache + plane * kv_stride + b * block_bytes)
+                continue
+            init, local = st.init_window, st.local_window
             for plane in (0, 1):
-                for b, j in pairs:
-                    src.append(st.init_window[plane][j].data_ptr())
+                for j, b in enumerate(ids[: st.init_window_sz]):
+                    src.append(init[plane][j].data_ptr())
                     dst.append(cache + plane * kv_stride + b * block_bytes)
-                if st.local_window is not None:
-                    n_local = st.local_window[plane].shape[0]
+                if local is not None:
+                    n_local = local[plane].shape[0]
                     for j, b in enumerate(ids[-n_local:]):
-                        src.append(st.local_window[plane][j].data_ptr())
+                        src.append(local[plane][j].data_ptr())
                         dst.append(cache + plane * kv_stride + b * block_bytes)
         if src:
             ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
@@ -682,7 +747,8 @@ class KVStarMultiStep(UcmSparseBase):
             lists32 = index.to(torch.int32)
         d_pruned = head_dim if index is None else index.shape[-1]
         d_pad = (d_pruned + 15) // 16 * 16
-        table = ops.kvstar_table(1, kv_heads, n, block_size // merge, d_pad, dev)
+        table = self._of_all_layers(("table", n, d_pad), layer_name, lambda layers: ops.kvstar_table(
+            layers, kv_heads, n, block_size // merge, d_pad, dev)).unsqueeze(0)
         ops.kvstar_block_repre(known[1], ids_dev, rows, table, block_size, kv_heads, head_dim, n_total, merge, pruned=lists32,
                                pruned_sel=None if lists32 is None else which_dev)
         at = 0
@@ -709,6 +775,23 @@ class KVStarMultiStep(UcmSparseBase):
         return query.index_select(0, found[0]), found[1]
 
     def _hook(self, which: str, layer_name: str, forward_context, *args) -> None:
+        requests = self._sparse_metadata.requests
+        path = self._path
+        if path is not None:
+            if path.step.get("owner") is not self._sparse_metadata:      # metadata bound by somebody else
+                path.build_step(self._sparse_metadata, ReqStage)
+            # decode steps: nothing per request; what is left for the per-request objects are the requests that end
+            # their prefill in this step (representatives, channel choice, windows aside)
+            layer_id = self._layer_ids.get(layer_name)
+            if layer_id is None:
+                layer_id = self._layer_ids[layer_name] = int(layer_name.split(".")[2])
+            if which == "attention_begin":
+                path.attention_begin(layer_id, layer_name, args[0], forward_context)
+                return
+            path.attention_finished(layer_id, layer_name, forward_context)
+            requests = path.step["ending"]
+            if not requests:
+                return
         batch = _RetrievalBatch() if which == "attention_begin" and self.kvstar_multistep_cfg["batch_retrieval"] else None
         sink = self._load_sink()
         plan = [] if sink is not None and self.kvstar_multistep_cfg["device_plans"] else None
@@ -717,7 +800,7 @@ class KVStarMultiStep(UcmSparseBase):
         rows = place = None
         if which == "attention_begin":
             rows, place = self._standby_rows(args[0])
-        for req_meta in self._sparse_metadata.requests:
+        for req_meta in requests:
             state = self.create_layerwise_req_state(req_meta, layer_name)
             state.update_meta(req_meta, forward_context)
             state.load_sink, state.plan_sink, state.window_sink, state.repre_sink = sink, plan, windows, repres
@@ -756,6 +839,10 @@ class KVStarMultiStep(UcmSparseBase):
                              self.kvstar_multistep_cfg["retrieval_stride"])
         self._sparse_metadata = meta
         self._step_cache = {}
+        self._n_slots = len(self._layer_slots)
+        path = self._layer_path() if self.role == UcmSparseRole.WORKER else None
+        if path is not None:
+            path.build_step(meta, ReqStage)
 
     # ---- scheduler side ------------------------------------------------------------------
     def estimate_num_slots_sparsed(self, request) -> int:

@@ -259,6 +259,16 @@ def AsyncRetrieveBatch(query_groups, blk_repres, d_pruned_indexes, topks, req_id
     return ids
 
 
+def RegisterBatch(results: _Results, n_tasks: int) -> List[int]:  # noqa: N802
+    """Task ids for the rows of a launch somebody else queued (``results.event`` recorded after it): row i becomes
+    a task that Wait / GetTaskResult / DeviceResult / Forget treat like one of AsyncRetrieveBatch's."""
+    ids = [next(_ids) for _ in range(n_tasks)]
+    with _lock:
+        for row, task_id in enumerate(ids):
+            _tasks[task_id] = _Task(results, row)
+    return ids
+
+
 def Wait(task_id: int) -> None:  # noqa: N802
     with _lock:
         task = _tasks.get(task_id)
@@ -302,6 +312,12 @@ def DeviceResult(task_id: int):  # noqa: N802
 def Forget(task_id: int) -> None:  # noqa: N802
     with _lock:
         _tasks.pop(task_id, None)
+
+
+def ForgetBatch(task_ids) -> None:  # noqa: N802
+    with _lock:
+        for task_id in task_ids:
+            _tasks.pop(task_id, None)
 
 
 def extract_block_repre(k_cache: torch.Tensor, vllm_block_ids: List[int], merge: int, prune_ratio: float = 1.0,
