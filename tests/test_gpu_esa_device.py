@@ -193,3 +193,82 @@ def test_esa_device_path_flow(ucm, dev, pool_where):
         plugin.request_finished_in_worker(rid)
     assert not plugin._dev.reqs and len(plugin.layer_pools[0].allocated) == 0
     assert len(plugin._dev.tables.free_rows) == 24
+
+
+def test_esa_device_path_store_hole(ucm, dev):
+    """The store lacks every other prompt block when the first load is due: the load leaves them out and says so (a
+    warning, a counter); once they are there, the plugin finds them, forgets what it believed resident and the next
+    load brings every selected block in - after which the cache holds what the resident lists say."""
+    from ucm_amd import ops
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.esa.esa import ESA
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+
+    hq, hkv, d, L, bs, nb, stride = 8, 2, 64, 2, 16, 128, 5
+    cfg = _config(hq, hkv, d, L, bs, 64 * bs, 4, {"init_window_sz": 1, "local_window_sz": 2, "min_blocks": 4,
+                                                 "sparse_ratio": 0.3, "retrieval_stride": stride})
+    slice_bytes = bs * hkv * d * 2
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 64 * L * 2 * slice_bytes})
+    plugin = ESA(cfg, UcmSparseRole.WORKER, store=store)
+    g = torch.Generator(device=dev)
+    g.manual_seed(9)
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    original = [c.clone() for c in caches]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
+    n_full = 40
+    ids = [int(x) for x in synth.permutation(78, nb)[: n_full + 3]]
+    req = ns(request_id="h", block_ids=[ids], num_computed_tokens=0, output_token_ids=[], num_prompt_tokens=n_full * bs + 3,
+             prompt_token_ids=[int(x) for x in synth.ints(501, n_full * bs + 3, 0, 30000)])
+
+    def engine_step():
+        n_tok = req.num_prompt_tokens if req.num_computed_tokens == 0 else 1
+        md = ns(query_start_loc=torch.tensor([0, n_tok]))
+        plugin.build_sparse_meta(ns(num_scheduled_tokens={"h": n_tok}), {"h": req}, ns(req_id_to_index={"h": 0}), md)
+        for l in range(L):
+            q = torch.randn(n_tok, hq, d, device=dev, generator=g).to(torch.bfloat16)
+            plugin.attention_begin(q, None, None, names[l], fc)
+            plugin.attention_finished(q, None, None, None, names[l], fc)
+        torch.cuda.synchronize()
+        req.num_computed_tokens += n_tok
+        req.output_token_ids.append(1)
+
+    def to_store(which):
+        hashes = plugin._dev.reqs["h"].block_hashes
+        some = [hashes[i] for i in which]
+        assert store.create(some) == [0] * len(some)
+        pool, kvb = store.device_pool()
+        for i, h in zip(which, some):
+            ops.kv_gather_blocks(ops.LayerPointers(original), original[0].stride(0) * 2, slice_bytes, nb,
+                                 torch.tensor([ids[i]], dtype=torch.int32, device=dev), pool[store.slot_of[h] * kvb :])
+        store.commit(some)
+        torch.cuda.synchronize()
+
+    def held_blocks_match():
+        st, t = plugin._dev.reqs["h"], plugin._dev.tables
+        for l in range(L):
+            res = t.resident[l, st.row, : st.top_k].cpu().numpy()
+            assert (res >= 0).all()
+            for j, b in enumerate(res):
+                if not torch.equal(caches[l][:, ids[j]], original[l][:, ids[int(b)]]):
+                    return False
+        return True
+
+    engine_step()                                            # prefill: representatives
+    late = list(range(0, n_full, 2))
+    to_store([i for i in range(n_full) if i not in late])
+    st = plugin._dev.reqs["h"]
+    n_late = len([i for i in late if i < st.sparse_range])
+    with pytest.warns(RuntimeWarning, match="does not hold"):
+        engine_step()                                        # decode step 1: retrieve, plan, load - with holes
+    assert plugin.load_misses == n_late and not st.src_ready and st.skipped
+    assert not held_blocks_match()                           # (blocks were left out; the lists say they are there)
+    to_store(late)
+    for step in range(2, 2 * stride + 1):                    # retrieval at step 2 and 7, loads at 5 and 10
+        engine_step()
+        if step == 2:
+            assert st.src_ready and not st.skipped and plugin.load_misses == n_late
+            assert int((plugin._dev.tables.resident[:, st.row] >= 0).sum()) == 0
+        if step in (stride, 2 * stride):
+            assert held_blocks_match()
+    plugin.request_finished_in_worker("h")

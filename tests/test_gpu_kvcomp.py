@@ -53,13 +53,15 @@ def test_hash_encoder_surface(ucm, dev):
     assert np.array_equal(pm.float().cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("device_loads", [True, False])
-def test_kvcomp_plugin_flow(ucm, dev, device_loads):
+@pytest.mark.parametrize("device_loads,hole", [(True, False), (False, False), (True, True)])
+def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole):
     """Prefill of 20 full blocks + 5 tokens, then decode on the sparsified block list: windows restored at step 1,
     retrieval at steps 1 and 5 picks what the oracle picks from the same keys, the chosen blocks land in the
     request's middle cache blocks in ascending order, a block filled during decode is dumped and hashed.  Once
     through the batched device path (one call per layer for all requests, loads planned on the device) and once
-    through the per-request path that works with any store."""
+    through the per-request path that works with any store.  ``hole``: at the first retrieval the store lacks every
+    other block - the load leaves those out, says so (a warning, a counter), and finds them at the next retrieval,
+    by which time they are back."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvcomp.kvcomp import KvComp
@@ -136,12 +138,21 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads):
         order = np.argsort(-sc.astype(np.float32), kind="stable")[:mid]
         return sorted(first + int(i) for i in order)
 
+    away = {}
+    if hole:
+        away = {b: store.slot_of.pop(f"req_A_blk_{b}") for b in range(1, 19, 2)}
     for step in range(1, 7):
         if step > 1:
             req.output_token_ids.append(7)
             req.num_output_tokens = step
             req.num_tokens = n_prompt + step
-        qs = run_step(1)
+        before = [c.clone() for c in caches]
+        if hole and step == 1:
+            with pytest.warns(RuntimeWarning, match="does not hold"):
+                qs = run_step(1)
+            assert plugin.load_misses == len(away)
+        else:
+            qs = run_step(1)
         torch.cuda.synchronize()
         for l in range(L):
             st = states[l]
@@ -150,13 +161,22 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads):
                 assert st.last_selection == want, (step, l)
                 for kv in range(2):
                     got = caches[l][kv][kept[1 : 1 + mid]]
-                    assert torch.equal(got, original[l][kv][[full_ids[b] for b in want]]), (step, l, kv)
+                    should = original[l][kv][[full_ids[b] for b in want]]
+                    for j, b in enumerate(want):             # a block the store lacked: the cache block keeps what it held
+                        if step == 1 and b in away:
+                            should[j] = before[l][kv][kept[1 + j]]
+                    assert torch.equal(got, should), (step, l, kv)
                     # windows: logical block 0 in the first kept block, the last two logical blocks in the last two
                     assert torch.equal(caches[l][kv][kept[0]], original[l][kv][full_ids[0]])
             else:
                 assert st.last_selection == expected(l, qs_at[l], 20) if step < 5 else True
         if step in (1, 5):
             qs_at = qs
+        if hole and step == 1:
+            for b, slot in away.items():
+                store.slot_of[f"req_A_blk_{b}"] = slot
+    if hole:
+        assert plugin.load_misses == len(away)               # the second retrieval found every block
     # step 1 restored the local window as it was at the end of prefill (blocks 19 and 20 of the prompt)
     # and decode kept writing into the last block; the block that filled up is dumped and hashed
     req.output_token_ids.extend([7] * 12)

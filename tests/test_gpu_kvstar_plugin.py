@@ -18,14 +18,16 @@ def bits(t):
     return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads,device_plans", [
-    (1.0, 1, True, True, True), (0.5, 3, True, False, True), (0.25, 1, False, True, True), (0.25, 1, True, False, False),
-    (0.25, 1, True, True, False), (0.5, 3, True, True, True)])
-def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads, device_plans):
+@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads,device_plans,hole", [
+    (1.0, 1, True, True, True, False), (0.5, 3, True, False, True, False), (0.25, 1, False, True, True, False),
+    (0.25, 1, True, False, False, False), (0.25, 1, True, True, False, False), (0.5, 3, True, True, True, False),
+    (0.25, 1, True, True, True, True), (0.25, 1, False, True, True, True), (0.25, 1, True, True, False, True)])
+def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads, device_plans, hole):
     """Prefill (one chunk, or three) of 24 full blocks + 5 tokens, then 13 decode steps with stride 4: step 1 restores
     the windows and loads what the prefill group's vote picks; the vote of decode steps 1-4 is queued at step 4 and
     its winners are loaded at step 8; steps 5-8 at step 8 / 12.  Selections are checked against the CPU oracle on the
-    same keys and queries."""
+    same keys and queries.  ``hole``: at the first load the store lacks some of the prompt's blocks - the load leaves them
+    out, says so (a warning, a counter) and looks again at the next load, by which time they have arrived."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvstar.multistep import KVStarMultiStep
@@ -83,13 +85,19 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
     assert len(hashes) == n_full and hashes == states[1].block_hashes
 
     # what the connector does in a deployment: the prompt's full blocks are in the store under their chained hashes
-    assert store.create(hashes) == [0] * n_full
     from ucm_amd.sparse.esa.esa import get_offset
-    for l in range(L):
-        for kv in range(2):
-            off = get_offset((bs, hkv, d), 0, 1, 2, l, bool(kv))
-            store.wait(store.dump(hashes, [off] * n_full, [original[l][kv][i] for i in full_ids[:n_full]]))
-    store.commit(hashes)
+
+    def to_store(which):
+        some = [hashes[i] for i in which]
+        assert store.create(some) == [0] * len(some)
+        for l in range(L):
+            for kv in range(2):
+                off = get_offset((bs, hkv, d), 0, 1, 2, l, bool(kv))
+                store.wait(store.dump(some, [off] * len(some), [original[l][kv][full_ids[i]] for i in which]))
+        store.commit(some)
+
+    late = list(range(1, n_full - 2, 2)) if hole else []     # every other block between the windows arrives late
+    to_store([i for i in range(n_full) if i not in late])
 
     # representatives: blocks 1 .. 21 (init window 1, local window 2), against the oracle on the same keys
     want_repre, pruned = [], []
@@ -125,7 +133,7 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
         _, votes = O.kvstar_retrieve(bits(qg), want_repre[l], n_keep, pruned=pruned[l], d_pruned=dp)
         return votes
 
-    def check_loaded(record, l):
+    def check_loaded(record, l, absent=(), before=None):
         st = states[l]
         # with the loads planned on the device nobody has read the list yet; looking at it fetches the host copy
         assert (record in st.step_group_retrieve_indices) == (not (device_loads and device_plans))
@@ -136,14 +144,29 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
         assert st.step_group_retrieve_result[record] == [hashes[i + 1] for i in chosen]
         for kv in range(2):                                  # candidate block j holds the j-th winner, K and V
             got = caches[l][kv][kept[1 : 1 + n_keep]]
-            assert torch.equal(got, original[l][kv][[full_ids[i + 1] for i in chosen]]), (record, l, kv)
+            want = original[l][kv][[full_ids[i + 1] for i in chosen]]
+            if absent:                                       # a block the store lacked: the cache block keeps what it held
+                for j, i in enumerate(chosen):
+                    if i + 1 in absent:
+                        want[j] = before[l][kv][kept[1 + j]]
+            assert torch.equal(got, want), (record, l, kv)
 
     decode_q = {l: [] for l in range(L)}
     for step in range(1, 14):
         if step > 1:
             req.output_token_ids.append(1)
             req.num_output_tokens, req.num_tokens = step, n_prompt + step
-        for l, q in enumerate(run_step(1)):
+        before = [c.clone() for c in caches]
+        if hole and step == 1:
+            with pytest.warns(RuntimeWarning, match="does not hold"):
+                qs = run_step(1)
+            assert plugin.load_misses >= 1
+        else:
+            qs = run_step(1)
+        if hole and step == 1:
+            to_store(late)
+            seen = plugin.load_misses
+        for l, q in enumerate(qs):
             decode_q[l].append(q[0])
         if step % stride == 0:
             groups["decode" + str(step - stride + 1)] = [torch.stack(decode_q[l][-stride:]) for l in range(L)]
@@ -152,7 +175,7 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
             st = states[l]
             if step == 1:
                 st.wait_for_blk_transfer_task_done()
-                check_loaded("prefill", l)
+                check_loaded("prefill", l, late, before)
                 for kv in range(2):                          # windows written back around the candidates
                     assert torch.equal(caches[l][kv][kept[0]], original[l][kv][full_ids[0]])
                     assert torch.equal(caches[l][kv][kept[-2:]], original[l][kv][full_ids[-2:]])
@@ -167,6 +190,8 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
                 check_loaded("decode5", l)
             if step in (9, 13):
                 assert not st.blk_trans_tasks                # waited for at the first step of a stride
+    if hole:
+        assert plugin.load_misses == seen                    # nothing was missing any more at the later loads
     plugin.request_finished_in_worker("7")
     assert "7" not in plugin.req_states
 

@@ -10,6 +10,7 @@ imported here, which keeps the surface testable with stand-in objects.
 from __future__ import annotations
 
 import enum
+import warnings
 from abc import ABC, abstractmethod
 from typing import Any, List, Optional, Union
 
@@ -30,10 +31,19 @@ class UcmSparseBase(ABC):
         self._vllm_config = vllm_config
         self._role = role
         self._sparse_metadata: Optional[UcmSparseMetadata] = None
+        self.load_misses = 0            # blocks a device-side load wanted from the KV store and did not find there
 
     @property
     def role(self) -> UcmSparseRole:
         return self._role
+
+    def _report_missing(self, n: int) -> None:
+        """A load that a kernel carries out leaves out a block the store does not hold: the cache block that should
+        receive it keeps what it has.  That is counted and said aloud instead of passing unnoticed, and the plugins
+        look the block up again at their next load."""
+        self.load_misses += n
+        warnings.warn(f"{type(self).__name__}: the KV store does not hold {n} of the blocks a load of this step may ask "
+                      "for; cache blocks that should receive them keep what they hold", RuntimeWarning, stacklevel=3)
 
     # ---- worker side -----------------------------------------------------
     def bind_sparse_metadata(self, sparse_metadata: UcmSparseMetadata) -> None:

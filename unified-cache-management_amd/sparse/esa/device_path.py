@@ -42,7 +42,9 @@ class DeviceRequest:
     n_repre: int = 0                                          # representatives written (blocks)
     pending: bool = False                                     # a retrieval waits to be turned into loads
     dst_ids: tuple = ()                                       # cache blocks of the first top_k vLLM blocks, as uploaded
-    src_ready: bool = False
+    src_ready: bool = False                                   # every block of the sparse range was found in the store
+    src_missing: int = 0                                      # how many were not, at the last look
+    skipped: bool = False                                     # a load ran while some were missing
 
 
 class StepPlan:
@@ -75,11 +77,7 @@ class EsaDeviceTables:
         self.dst_table = torch.full((max_rows, max_slots), -1, **i32)
         self.scores_ws = torch.empty(max_rows * max_blocks, dtype=torch.float32, device=device)
         self.free_rows = list(range(max_rows - 1, -1, -1))
-        # per-step descriptor: a ring of pinned buffers (the copy of step s may still be in flight while the host
-        # fills step s+1) and one device twin per ring entry
-        self._ring = [torch.empty(5 * max_rows, dtype=torch.int32).pin_memory() for _ in range(4)]
-        self._ring_dev = [torch.empty(5 * max_rows, **i32) for _ in range(4)]
-        self._turn = 0
+        self.device = device
 
     def allocate_row(self) -> int:
         if not self.free_rows:
@@ -96,23 +94,17 @@ class EsaDeviceTables:
         self.free_rows.append(row)
 
     def upload(self, parts: List[List[int]]) -> List[Optional[torch.Tensor]]:
-        """Concatenates the integer lists into one pinned buffer, copies it once and returns a device view per
-        list (None for an empty one)."""
-        self._turn = (self._turn + 1) % len(self._ring)
-        host, dev = self._ring[self._turn], self._ring_dev[self._turn]
-        flat = host.numpy()
+        """The integer lists side by side in one device tensor, sent in one copy (pinned staging whose reuse waits
+        for the copy that last read it); returns a view per list, None for an empty one."""
+        flat = [x for p in parts for x in p]
+        if not flat:
+            return [None] * len(parts)
+        dev = ops.upload(torch.tensor(flat, dtype=torch.int32), self.device)
         views, pos = [], 0
         for p in parts:
-            n = len(p)
-            if n:
-                flat[pos : pos + n] = p
-                views.append((pos, n))
-            else:
-                views.append(None)
-            pos += n
-        if pos:
-            dev[:pos].copy_(host[:pos], non_blocking=True)
-        return [None if v is None else dev[v[0] : v[0] + v[1]] for v in views]
+            views.append(dev[pos : pos + len(p)] if p else None)
+            pos += len(p)
+        return views
 
 
 class EsaDevicePath:
@@ -174,6 +166,9 @@ class EsaDevicePath:
             if ids != st.dst_ids:
                 t.dst_table[st.row, : len(ids)] = torch.tensor(ids, dtype=torch.int32, device=self.device)
                 st.dst_ids = ids
+            if st.src_missing and (step == 1 or (step % stride == 0 and st.pending)):
+                esa._report_missing(st.src_missing)
+                st.skipped = True
             if step == 1:
                 first.append(st.row)
                 first_q.append(meta.query_start_loc)
@@ -212,12 +207,19 @@ class EsaDevicePath:
         return st
 
     def _upload_sources(self, st: DeviceRequest) -> None:
-        """hash -> pool block of the request's sparse range, once (esa.py:306-310 looks hashes up per retrieval)."""
+        """hash -> pool block of the request's sparse range (esa.py:306-310 looks hashes up per retrieval): once, when
+        the store holds them all; otherwise again at every step until it does.  A load that ran in between left the
+        missing blocks out while the plan counted them as present, so once more of them are found the request's
+        resident lists are forgotten and its next load brings in everything it selects."""
         slot_of = self.esa.connector.slot_of
         src = [slot_of.get(h, -1) for h in st.block_hashes[: st.sparse_range]]
+        missing = src.count(-1)
         if src:
-            self.tables.src_table[st.row, : len(src)] = torch.tensor(src, dtype=torch.int32, device=self.device)
-        st.src_ready = True
+            self.tables.src_table[st.row, : len(src)] = ops.upload(torch.tensor(src, dtype=torch.int32), self.device)
+        if st.skipped and missing < st.src_missing:
+            self.tables.resident[:, st.row].fill_(-1)
+            st.skipped = False
+        st.src_missing, st.src_ready = missing, missing == 0
 
     def _allocate_repre(self, prefill):
         """Rows of every layer's table for the requests that finish their prefill in this step

@@ -51,12 +51,10 @@ class KvCompDevicePath:
         self.q_sum = torch.empty((1, rows, 128), dtype=torch.int16, device=device)
         self.qbar = torch.empty((1, rows, h, 16), dtype=torch.uint8, device=device)
         # per-step descriptor, one entry per retrieving request: seg_off, seg_len, topk_len, its token in the step's
-        # query tensor, its table row; a ring of pinned buffers, the copy of one step may still be in flight while the
-        # host fills the next
-        self._ring = [torch.empty(5 * rows, dtype=torch.int32).pin_memory() for _ in range(4)]
-        self._ring_dev = [torch.empty(5 * rows, **i32) for _ in range(4)]
-        self._turn = 0
+        # query tensor, its table row; filled on the host and sent in one copy
+        self._desc = torch.empty((5, rows), dtype=torch.int32)
         self.n_src: Dict[object, int] = {}                        # candidates of a request whose pool block is uploaded
+        self.src_absent: Dict[object, List[int]] = {}             # ... and those the store did not hold at the last look
         self.dst_ids: Dict[object, tuple] = {}
         self.active: List[object] = []                            # requests that retrieve in this step
         self.first_of: Dict[object, int] = {}
@@ -101,8 +99,7 @@ class KvCompDevicePath:
             k = count if top_k >= n_blocks else min(top_k, count)     # every candidate, or the best top_k of them
             row = p.segment_base(meta.request_id) // p.max_blocks
             if host is None:
-                self._turn = (self._turn + 1) % len(self._ring)
-                host = self._ring[self._turn].numpy().reshape(5, rows)
+                host = self._desc.numpy()
             n = len(self.active)
             host[0, n], host[1, n], host[2, n], host[3, n], host[4, n] = row * p.max_blocks + first, count, k, a, row
             self.active.append(meta.request_id)
@@ -116,9 +113,7 @@ class KvCompDevicePath:
                 self.dst_ids[meta.request_id] = ids
         if host is not None:
             n = len(self.active)
-            dev = self._ring_dev[self._turn]
-            dev.copy_(self._ring[self._turn], non_blocking=True)
-            d = dev.view(5, rows)
+            d = ops.upload(self._desc[:, :n], self.device)      # (pinned staging whose reuse waits for its last copy)
             self.seg_off, self.seg_len, self.topk_len, self.tokens = d[0, :n], d[1, :n], d[2, :n], d[3, :n]
             table_rows = d[4, :n].long()
             self.src_step = self.src_table.index_select(0, table_rows)      # the step's requests side by side
@@ -126,17 +121,32 @@ class KvCompDevicePath:
             self.slot_of_step = {r: i for i, r in enumerate(self.active)}
 
     def _sources(self, request_id, row: int, first: int, count: int) -> None:
-        """Pool blocks of candidates first .. first+count-1 (the hash -> store lookup, once per block)."""
+        """Pool blocks of candidates first .. first+count-1: the hash -> store lookup, once per block the store holds;
+        one it does not hold (its dump found no room, or has not happened) is looked up again at every retrieval, and
+        reported while it stays away - the retrieval's load leaves it out."""
         done = self.n_src.get(request_id, 0)
-        if done >= count:
+        absent = self.src_absent.get(request_id)
+        if done >= count and not absent:
             return
         from .kvcomp import ReqStatePerLayer                 # (the plugin module imports this one)
 
         slot_of = self.plugin.connector.slot_of
         name = ReqStatePerLayer.block_hash
-        src = [slot_of.get(name(request_id, first + i), -1) for i in range(done, count)]
-        self.src_table[row, done:count] = torch.tensor(src, dtype=torch.int32, device=self.device)
-        self.n_src[request_id] = count
+        if absent:
+            found = [(i, slot_of[name(request_id, first + i)]) for i in absent if name(request_id, first + i) in slot_of]
+            if found:
+                at = torch.tensor([i for i, _ in found], dtype=torch.int64, device=self.device)
+                self.src_table[row].index_copy_(0, at, ops.upload(torch.tensor([s for _, s in found], dtype=torch.int32), self.device))
+                gone = {i for i, _ in found}
+                absent = [i for i in absent if i not in gone]
+        if done < count:
+            src = [slot_of.get(name(request_id, first + i), -1) for i in range(done, count)]
+            self.src_table[row, done:count] = ops.upload(torch.tensor(src, dtype=torch.int32), self.device)
+            absent = (absent or []) + [done + i for i, s in enumerate(src) if s < 0]
+            self.n_src[request_id] = count
+        self.src_absent[request_id] = absent or []
+        if absent:
+            self.plugin._report_missing(len(absent))
 
     # ---- hook -------------------------------------------------------------------------------
     def attention_begin(self, layer_id: int, query: torch.Tensor) -> None:
@@ -256,5 +266,5 @@ class KvCompDevicePath:
         return [self.first_of[request_id] + int(x) for x in self.idx[layer_id, i, :n].tolist()]
 
     def request_finished(self, request_id) -> None:
-        for table in (self.n_src, self.dst_ids, self.first_of, self.windows, self.win_shape):
+        for table in (self.n_src, self.src_absent, self.dst_ids, self.first_of, self.windows, self.win_shape):
             table.pop(request_id, None)

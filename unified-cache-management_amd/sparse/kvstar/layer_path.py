@@ -23,7 +23,6 @@ The schedule over ``step % retrieval_stride`` is the reference's (multistep.py:3
 from __future__ import annotations
 
 import math
-import warnings
 from typing import Dict, List, Optional
 
 import torch
@@ -74,7 +73,6 @@ class KVStarLayerPath:
         self.step: dict = {}
         self.side = None
         self.reading: Dict[int, object] = {}               # layer -> event of the side stream's last launch that reads its ring
-        self.load_misses = 0                               # chosen blocks the store did not hold when their load was due
         self._dev_index = 0
 
     # ---- rows of the rings ------------------------------------------------------------------------------------
@@ -359,10 +357,7 @@ class KVStarLayerPath:
                 missing += stored.count(-1)
                 src[row, : len(stored)] = torch.tensor(stored, dtype=torch.int32)
             if missing:
-                self.load_misses += missing
-                warnings.warn(f"KVStar: the KV store does not hold {missing} prompt blocks of the requests that load in this "
-                              "step; a cache block that should receive one of them keeps what it holds", RuntimeWarning,
-                              stacklevel=2)
+                self.plugin._report_missing(missing)
             batch.src_table = ops.upload(src, self.device)
             batch.src_complete = missing == 0
         width = batch.dst_host.shape[1]

@@ -574,7 +574,7 @@ class KVStarMultiStep(UcmSparseBase):
     def _flush_loads(self, sink: list, layer_name: str, forward_context) -> None:
         """One pointer-array copy for every (stored block -> cache block) pair the hook's requests asked for, K and V
         (launch_transfer_task("load", ...) per request, multistep.py:452-480).  A block the store does not hold is
-        left out (the per-request path gives up the whole request's load in that case)."""
+        left out and reported (the per-request path gives up the whole request's load in that case)."""
         if not sink:
             return
         layer_id = int(layer_name.split(".")[2])
@@ -585,14 +585,18 @@ class KVStarMultiStep(UcmSparseBase):
         kv_stride, block_bytes = kv.stride(0) * es, kv.stride(1) * es
         cache, stored = kv.data_ptr(), pool.data_ptr() + layer_id * 2 * block_bytes
         dst, src = [], []
+        missing = 0
         for hashes, ids in sink:
             for h, b in zip(hashes, ids):
                 slot = slot_of.get(h)
                 if slot is None:
+                    missing += 1
                     continue
                 for plane in (0, 1):
                     src.append(stored + slot * pool_block_bytes + plane * block_bytes)
                     dst.append(cache + plane * kv_stride + b * block_bytes)
+        if missing:
+            self._report_missing(missing)
         if src:
             ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
             ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
@@ -625,11 +629,15 @@ class KVStarMultiStep(UcmSparseBase):
                 longest = max(len(st.block_hashes) for st, _, _, _ in members)
                 src = torch.full((n_rows, max(longest, 1)), -1, dtype=torch.int32)
                 dst = torch.full((n_rows, width), -1, dtype=torch.int32)
+                missing = 0
                 for st, _, row, candidates in members:
                     first = st.init_window_sz
                     stored = [slot_of.get(h, -1) for h in st.block_hashes[first:]]
+                    missing += stored[: st.blk_repre.shape[0]].count(-1)
                     src[row, : len(stored)] = torch.tensor(stored, dtype=torch.int32)
                     dst[row, : min(len(candidates), width)] = torch.tensor(candidates[:width], dtype=torch.int32)
+                if missing:
+                    self._report_missing(missing)
                 rows = [row for _, _, row, _ in members]
                 both = ops.upload(torch.cat([src.view(-1), dst.view(-1), torch.tensor(rows, dtype=torch.int32)]), kv.device)
                 tables = self._step_cache[key] = (both[: src.numel()].view(src.shape),
