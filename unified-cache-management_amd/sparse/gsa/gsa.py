@@ -29,6 +29,7 @@ import math
 from itertools import accumulate, count
 from typing import Dict, List, Optional, Union
 
+import numpy as np
 import torch
 
 from ... import _lib, ops
@@ -219,6 +220,8 @@ class GSA(UcmSparseBase):
         self._kv_full: Dict[int, torch.Tensor] = {}
         self._scored: set = set()  # sparsified requests whose blocks have been scored at least once
         self._layer_of: Dict[str, int] = {}
+        self._fast: Optional[list] = None   # set by execute_begin for a step that takes the one-launch path in every layer
+        self._seen_layers = None          # the engine's table of layers once every layer's cache has been registered from it
         self._tables_signature = None     # (request, blocks, last block) per batch slot of the block tables on the device
         self._tables_dev: Optional[torch.Tensor] = None
 
@@ -345,6 +348,7 @@ class GSA(UcmSparseBase):
                                           (self.min_topk, self.max_topk, self.topk_ratio) if self.ptopk_prefetch else None)
         self.gsa_metadata = meta
         self._sparse_metadata = meta
+        self._fast = None
         if self.ptopk_prefetch:
             self._init_sparse_local_kv(scheduler_output, requests)
 
@@ -377,6 +381,7 @@ class GSA(UcmSparseBase):
         # score on every retrieval_stride-th step, and whenever a request is sparsified for the first time
         is_topk = any_gsa and (self.step_count % self.retrieval_stride == 0 or not gsa_ids <= self._scored)
         self.model_input["is_topk"] = is_topk
+        self._fast = None
         if is_topk:
             self._scored |= gsa_ids
         if not any_gsa or not self._dev_ready:
@@ -395,27 +400,34 @@ class GSA(UcmSparseBase):
         host = self._host_desc[slot][: 5 * batch + n_tables + 2 * n_calc]
         hn = host.numpy()                    # the same pinned memory; numpy fills it several times faster than torch indexing
         desc = hn[: 5 * batch].reshape(5, batch)
-        desc[:] = 0
         if not tables_known:
             tables = hn[5 * batch : 5 * batch + n_tables].reshape(batch, width)
             tables[:] = 0
         max_len = total = 0
         query_locals = self.model_input["query_locals"]
+        rows = []                            # per request: first table row, blocks, k, its last query token, tokens so far
+        min_topk, max_topk, ratio = self.min_topk, self.max_topk, self.topk_ratio
         for i, st in enumerate(by_index):
             if st is None:
+                rows.append((0, 0, 0, 0, 0))
                 continue
             n = len(st.blocks)
-            k = compute_topk_len(n, self.min_topk, self.max_topk, self.topk_ratio) if st.is_gsa() else n
             # k >= n keeps every block (short or prefilling requests)
-            desc[:, i] = (st.slot_offset, n, max(k, 1), query_locals[i + 1] - 1, st.get_seq_len())
+            k = compute_topk_len(n, min_topk, max_topk, ratio) if st.is_gsa() else n
+            rows.append((st.slot_offset, n, k if k > 1 else 1, query_locals[i + 1] - 1,
+                         st.num_computed_tokens + st.num_scheduled_tokens))
             if not tables_known:
                 tables[i, :n] = st.blocks
-            max_len, total = max(max_len, n), total + n
+            if n > max_len:
+                max_len = n
+            total += n
+        desc[:] = np.array(rows, dtype=np.int32).T
         tail = hn[5 * batch + n_tables :]
         tail[:n_calc] = self.model_input["calc_block_table"]
         tail[n_calc:] = self.model_input["calc_repre_slot_mapping"]
         dev = host.to(self.device, non_blocking=True)
-        self._host_free[slot] = torch.cuda.Event()
+        if self._host_free[slot] is None:
+            self._host_free[slot] = torch.cuda.Event()
         self._host_free[slot].record()
         d = dev[: 5 * batch].view(5, batch)
         if not tables_known:
@@ -434,6 +446,15 @@ class GSA(UcmSparseBase):
         a = self._sel
         a.seg_off, a.seg_len, a.topk_len, a.q_rows, a.seq_lens, a.block_tables = self.model_input["addr"]
         a.n_req, a.max_seg_len, a.total_blocks = batch, max_len, total
+        if is_topk and self._fused_ok and _raw_stream is not None:
+            self._fast = self._batch_views(batch)
+
+    def _batch_views(self, n: int) -> list:
+        """Per layer: (sparse block table, sparse sequence lengths) of a batch of n requests."""
+        views = self._views.get(n)
+        if views is None:
+            views = self._views[n] = [(self.block_tables_mp[k, :n], self.gsa_seq_len[k, :n]) for k in range(self.layer_num)]
+        return views
 
     def execute_finished(self) -> None:
         if self.ptopk_prefetch:
@@ -448,11 +469,35 @@ class GSA(UcmSparseBase):
         return l
 
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
-        self.maybe_register_kv_cache(forward_context, layer_name)
+        # the layer's cache is looked at when the engine's table of layers is not the one seen before (the caches are
+        # allocated once; the reference re-reads them in every hook, gsa.py:866-877)
+        layers = forward_context.no_compile_layers
+        if layers is not self._seen_layers or layer_name not in self._layer_of:
+            self.maybe_register_kv_cache(forward_context, layer_name)
+            if len(self._kv_full) == self.layer_num:
+                self._seen_layers = layers
+        fast = self._fast
+        if fast is not None:
+            # the step scores and selects with the one-launch call: everything but the layer and its queries was
+            # filled in by execute_begin
+            l = self._layer_of[layer_name]
+            q_code = _Q_CODES.get(query.dtype)
+            if q_code is None or not query.is_contiguous() or query.shape[-1] != self.head_size:
+                raise ValueError("query must be a contiguous bfloat16, float16 or float32 device tensor [tokens, q_heads, head_size]")
+            a = self._sel
+            a.q, a.q_dtype, a.q_layer_stride, a.first_layer = query.data_ptr(), q_code, query.numel(), l
+            rc = self._score_select(self._sel_addr, _raw_stream(self._dev_index))
+            if rc != 0:
+                raise _lib.UcmHipError("ucm_score_select", rc, _lib.lib().ucm_last_error().decode())
+            md = forward_context.attn_metadata
+            if isinstance(md, dict):
+                md = md[layer_name]
+            md.block_table, md.seq_lens = fast[l]
+            return
         mi = self.model_input
         if not mi.get("any_gsa") or "seg_off" not in mi:
             return
-        l = self._layer_id(layer_name)
+        l = self._layer_of[layer_name]
         n = mi["n_batch"]
         stream = _raw_stream(self._dev_index) if _raw_stream is not None else ops.current_stream()
         if mi["is_topk"]:
@@ -481,9 +526,7 @@ class GSA(UcmSparseBase):
             _lib.call("ucm_topk_windows", scores, self.scores.stride(0), rows, seg_off, seg_len, topk_len, n, mi["max_len"],
                       1, self.init_window, self.local_window, idx, self.max_block_len, counts, tables, self.max_block_len,
                       phys, seq_lens, self.block_size, sparse_len, stream)
-        views = self._views.get(n)
-        if views is None:
-            views = self._views[n] = [(self.block_tables_mp[k, :n], self.gsa_seq_len[k, :n]) for k in range(self.layer_num)]
+        views = self._batch_views(n)
         md = forward_context.attn_metadata
         md = md[layer_name] if isinstance(md, dict) else md
         md.block_table, md.seq_lens = views[l]
