@@ -141,8 +141,28 @@ def test_cal_kpre_and_topk_surface(ucm, dev):
             assert np.array_equal(got[i, : len(want)], want), (l, i)
         assert np.all(got[1] == -1) and np.all(got[3] == -1)
         assert np.array_equal(obj.q_cache[l][0].cpu().numpy(), q[l, 0])
-    with pytest.raises(NotImplementedError):
-        obj.set_kpre_method_param(hkv, 2)
+    with pytest.raises(ValueError):
+        obj.set_kpre_method_param(hkv, 3)
+    # two representatives per (block, kv head): a row of the cache is read [kv head][representative][channel], as
+    # the reference's kernel reads it
+    obj = CalKpreAndTopk(L, bs, max_bs, hq, d, device=dev)
+    obj.set_kpre_method_param(hkv, 2)
+    kpre_all = torch.from_numpy(synth.normal_f32(722, (L, max_bs * max_blocks, 2, hkv, d))).to(dev)
+    obj.set_kpre_cache(list(kpre_all.unbind(0)))
+    topk_cache = [torch.full((4, max_blocks), -1, dtype=torch.int32, device=dev) for _ in range(L)]
+    obj.set_common_param([0, 2], is_decode)
+    obj.set_topk_param(slot_map)
+    obj.set_topk_cache(topk_cache, topk_lens)
+    for l in range(L):
+        obj.add_copy_req(False, l, [5, -1, 9, -1], torch.from_numpy(q[l]).to(dev).to(torch.bfloat16))
+    torch.cuda.synchronize()
+    kp = kpre_all.cpu().numpy().reshape(L, max_bs * max_blocks, hkv * 2 * d)
+    for l in range(L):
+        got = topk_cache[l].cpu().numpy()
+        for i, j in ((0, 0), (2, 1)):
+            want, _ = O.select_topk(q[l, i], kp[l, slot_map[i][0] : slot_map[i][0] + lens[i]].reshape(lens[i], hkv, 2, d),
+                                    topk_lens[j])
+            assert np.array_equal(got[i, : len(want)], want), (l, i)
 
 
 # ------------------------------------------------------------ GSA plugin

@@ -93,7 +93,7 @@ def test_block_mean_skips_bad_ids_and_layer_range(ucm, dev):
 # --------------------------------------------------------------- scoring
 
 def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=torch.float32, q_rows=None,
-               block_tables=None, seq_lens=None, block_size=128, repre_dtype=torch.float32, tile=0):
+               block_tables=None, seq_lens=None, block_size=128, repre_dtype=torch.float32, tile=0, num_repre=1):
     """q_np [L, rows, Hq, D] fp32 values; repre_np [L, rows, Hkv*D] (values that
     repre_dtype holds exactly, so the oracle sees the same numbers).  Requests of up to 1024 blocks also go
     through the one-launch entry point, whose every output must equal the two launches'."""
@@ -106,7 +106,7 @@ def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=to
     scores = torch.full((n_layers, repre_np.shape[1]), -123.0, device=dev)
     mx = int(lens.max(initial=0))
     ops.score_blocks(q, repre, i32(off, dev), i32(lens, dev), mx, hkv, scores,
-                     q_rows=None if q_rows is None else i32(q_rows, dev), tile_blocks=tile)
+                     q_rows=None if q_rows is None else i32(q_rows, dev), tile_blocks=tile, num_repre=num_repre)
     stride = max(mx, 1)
     idx = torch.full((n_layers, len(lens), stride), -1, dtype=torch.int32, device=dev)
     cnt = torch.full((n_layers, len(lens)), -1, dtype=torch.int32, device=dev)
@@ -137,7 +137,7 @@ def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=to
             ops.score_select(q, repre, i32(off, dev), i32(lens, dev), i32(topk, dev), mx, hkv, fused["scores"], fused["idx"],
                              fused["cnt"], tickets, start_w=sw, end_w=ew, q_rows=None if q_rows is None else i32(q_rows, dev),
                              block_tables=bt, phys_out=fused["phys"], seq_lens=sl, block_size=block_size,
-                             sparse_seq_lens=fused["sps"], tile_blocks=tile, total_blocks=total)
+                             sparse_seq_lens=fused["sps"], tile_blocks=tile, total_blocks=total, num_repre=num_repre)
             torch.cuda.synchronize()
             assert not tickets.any(), "tickets left non-zero"
         assert torch.equal(fused["scores"].view(torch.int32), scores.view(torch.int32)), "fused scores differ"
@@ -150,11 +150,11 @@ def run_select(ops, dev, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_dtype=to
     return out
 
 
-def check_against_oracle(out, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_rows=None):
+def check_against_oracle(out, q_np, repre_np, lens, topk, hkv, sw=1, ew=2, q_rows=None, num_repre=1):
     n_layers = repre_np.shape[0]
     for l in range(n_layers):
         ql = q_np[l] if q_rows is None else q_np[l][np.asarray(q_rows)]
-        widx, wcnt, wscores = O.select_topk_bs(ql[: len(lens)], repre_np[l], out["off"], lens, topk, hkv,
+        widx, wcnt, wscores = O.select_topk_bs(ql[: len(lens)], repre_np[l], out["off"], lens, topk, hkv, num_krepre=num_repre,
                                                start_w=sw, end_w=ew, out_stride=out["idx"].shape[2] + sw + ew + max(topk))
         for r, n in enumerate(lens):
             a, b = out["off"][r], out["off"][r] + n
@@ -194,6 +194,28 @@ def test_ragged_batch_scores_and_selection(ucm, dev, hkv, g, d, q_dtype):
     out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=q_dtype)
     check_against_oracle(out, q, repre, lens, topk, hkv)
     assert out["cnt"][0, 4] == 0  # the empty request selects nothing
+
+
+@pytest.mark.parametrize("hkv,g,d,num_repre", [(8, 4, 128, 2), (4, 8, 128, 2), (2, 2, 64, 4), (1, 8, 128, 2), (4, 2, 64, 4)])
+@pytest.mark.parametrize("q_dtype,repre_dtype", [(torch.float32, torch.float32), (torch.float16, torch.float32),
+                                                 (torch.bfloat16, torch.bfloat16), (torch.float16, torch.bfloat16)])
+def test_several_representatives_per_head_and_fp16_queries(ucm, dev, hkv, g, d, num_repre, q_dtype, repre_dtype):
+    """numKrepre > 1: a block's score takes, per kv head, the largest of the dots with that head's representatives
+    (k_repre rows laid out [kv head][representative][channel], cal_kpre_and_topk.cpp's kRepre); queries in any of the
+    three types the model may run in, widened exactly."""
+    from ucm_amd import ops
+
+    lens = [3, 40, 0, 65, 130, 257]
+    topk = [max(n // 3, 1) for n in lens]
+    rows = int(np.sum(lens))
+    q = synth.normal_bf16_as_f32(41, (2, len(lens), hkv * g, d))
+    if q_dtype == torch.float16:
+        q = torch.from_numpy(q).to(torch.float16).float().numpy()        # values fp16 holds exactly
+    repre = synth.normal_f32(42, (2, rows, hkv * num_repre * d)) * np.float32(0.3)
+    if repre_dtype == torch.bfloat16:
+        repre = torch.from_numpy(repre).to(torch.bfloat16).float().numpy()
+    out = run_select(ops, dev, q, repre, lens, topk, hkv, q_dtype=q_dtype, repre_dtype=repre_dtype, num_repre=num_repre)
+    check_against_oracle(out, q, repre, lens, topk, hkv, num_repre=num_repre)
 
 
 def as_bf16_values(a):

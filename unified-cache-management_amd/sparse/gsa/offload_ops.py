@@ -12,9 +12,10 @@ scoring and selection kernels of that layer; results land in the caller-owned
 is an event query.
 
 All tensors handed in (kpre caches, top-k caches) must live on the device; the
-representatives are fp32 ``[rows, 1, kv_heads, head_dim]`` per layer, exactly
-the shape of the reference's ``kpre_caches``
-(ucm/sparse/gsa/prefetch/prefetch_engine.py:64-77).
+representatives are fp32 ``[rows, numKpre, kv_heads, head_dim]`` per layer, the
+shape of the reference's ``kpre_caches``
+(ucm/sparse/gsa/prefetch/prefetch_engine.py:64-77); with numKpre > 1 a row is
+read as the reference's kernel reads it, kv head outermost.
 """
 from __future__ import annotations
 
@@ -67,15 +68,18 @@ class CalKpreAndTopk:
 
     # ---- configuration ---------------------------------------------------
     def set_kpre_method_param(self, num_heads: int, num_kpre: int) -> None:
-        if num_kpre != 1:
-            raise NotImplementedError("one representative per (block, kv head): numKpre must be 1")
+        """num_kpre representatives per (block, kv head): a block's score then takes, per head, the largest of the
+        dots with them.  A row of the kpre caches is read the way the reference's kernel reads it, [kv head]
+        [representative][channel] (select_topk_block.cpp: headBase = h * numKrepre * headSize)."""
+        if num_kpre < 1 or num_heads * num_kpre > 16 or 16 % (num_heads * num_kpre):
+            raise ValueError("kv heads x numKpre must be 1, 2, 4, 8 or 16")
         self.kv_heads, self.num_kpre = num_heads, num_kpre
 
     def set_kpre_cache(self, kpre_cache: Sequence[torch.Tensor]) -> None:
-        row = self.kv_heads * self.head_size
+        row = self.kv_heads * self.num_kpre * self.head_size
         for t in kpre_cache:
             if not t.is_cuda or t.dtype != torch.float32 or not t.is_contiguous() or t[0].numel() != row:
-                raise ValueError("kpre caches must be contiguous float32 device tensors [rows, 1, kv_heads, head_dim]")
+                raise ValueError("kpre caches must be contiguous float32 device tensors [rows, numKpre, kv_heads, head_dim]")
         self._kpre = list(kpre_cache)
         self._kpre_stride = _common_layer_stride(self._kpre)
 
@@ -151,7 +155,7 @@ class CalKpreAndTopk:
             scores = self._scores_buffer(rows)
             counts = self._counts_buffer(d["n"])
             ops.score_blocks(self.q_cache[layer_idx].unsqueeze(0), repre, seg_off, seg_len, d["max_len"],
-                             self.kv_heads, scores, q_rows=q_rows, total_blocks=d["total"])
+                             self.kv_heads, scores, q_rows=q_rows, total_blocks=d["total"], num_repre=self.num_kpre)
             ops.topk_windows(scores, seg_off, seg_len, topk, d["max_len"], out[: d["n"]].unsqueeze(0), counts,
                              start_w=self.init_window, end_w=self.local_window)
         if layer_idx == self.layer_num - 1:
