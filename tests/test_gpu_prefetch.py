@@ -95,6 +95,8 @@ def test_prefetch_engine_skips_and_errors(ucm, dev):
     assert success[:, 1].eq(5).all() and success_len[:, 1].tolist() == [9, 9]
     eng.run_async_prefetch_bs([1], [0], [2])                          # topk_len 0: skipped
     assert success[:, 2].eq(5).all()
+    with pytest.raises(ValueError, match="selection of more than 3"):
+        eng.run_async_prefetch_bs([1], [4], [2])                      # longer than the round's buffer: refused, not cut
     eng.del_blocks_map(1)
     eng.del_blocks_map(1)
     assert eng.obtain_blocks_map() == {}

@@ -317,6 +317,40 @@ def test_gsa_prefetch_mode_resident_set_and_slots(ucm):
     off = GSA(make_config(), UcmSparseRole.SCHEDULER)
     assert off.estimate_num_slots_sparsed(ns(num_prompt_tokens=100 * 128, num_output_tokens=5, num_tokens=100 * 128 + 5)) == INVALID_SLOT
 
+    # the scheduler's half (not in the reference): at the first decode step the request keeps its first max_topk + 1
+    # blocks and what it holds beyond its prompt, later steps only allocate
+    class Pool:
+        def __init__(self):
+            self.freed, self.evicted = [], []
+
+        def _maybe_evict_cached_block(self, b):
+            self.evicted.append(b)
+
+        def free_blocks(self, bl):
+            self.freed.extend(bl)
+
+        def get_num_free_blocks(self):
+            return 1
+
+    held = list(range(500, 602))                      # 101 blocks of the prompt (100 full + 5 tokens... ) and one more
+    mgr = ns(req_to_blocks={})
+    calls = []
+    coord = ns(get_blocks=lambda rid: [held], single_type_managers=[mgr],
+               get_num_blocks_to_allocate=lambda request_id, num_tokens, new_computed_blocks: calls.append(num_tokens) or 1,
+               allocate_new_blocks=lambda rid, n: calls.append(("alloc", n)))
+    pool = Pool()
+    req = ns(request_id="A", num_prompt_tokens=100 * 128 + 5, num_computed_tokens=100 * 128 + 5, num_output_tokens=1,
+             num_tokens=100 * 128 + 6)
+    got = plugin.allocate_slots(req, 4000, coord, pool, [None])
+    assert mgr.req_to_blocks["A"] == held[:49] + held[101:] and pool.freed == held[49:101] and pool.evicted == held
+    assert got.blocks == (held[:49] + held[101:],) and calls == [4000, ("alloc", 4000)]
+    req.num_computed_tokens += 1                      # a later step: nothing is returned any more
+    pool2, mgr.req_to_blocks = Pool(), {}
+    got = plugin.allocate_slots(req, 4001, coord, pool2, [None])
+    assert pool2.freed == [] and mgr.req_to_blocks == {} and got.blocks == (held,)
+    coord.get_num_blocks_to_allocate = lambda request_id, num_tokens, new_computed_blocks: 2
+    assert plugin.allocate_slots(req, 4001, coord, Pool(), [None]) is None
+
 
 def test_kvcomp_reads_the_reference_config_file(ucm, tmp_path):
     """KvComp takes head_dim and hash_bits from the reference's JSON (kvcomp_config.py:36-80; the files under

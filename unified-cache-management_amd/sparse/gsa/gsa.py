@@ -77,6 +77,9 @@ class GSAReqStat:
         self.prefetch_idx: Optional[List[int]] = None
         self.sparse_len = 0
         self.local_window_kv: Optional[torch.Tensor] = None   # [blocks, layers, K|V, block bytes]
+        self.phys: List[int] = []         # prefetch mode, decode: the cache blocks the request holds (the scheduler's list)
+        self.prompt_blocks = 0            # ... and how many logical blocks it had when it was sparsified
+        self.calc_logical: List[int] = [] # logical numbers of the blocks in calc_block_table
 
     # -- state queries (same meaning as the reference's) ---------------------
     def is_decode(self) -> bool:
@@ -124,11 +127,10 @@ class GSAReqStat:
         self.num_prompt_tokens = len(req_state.prompt_token_ids)
         self.num_output_tokens = len(req_state.output_token_ids)
         self.index_in_batch = index_in_batch
-        if prefetch is not None and self.blocks:
-            # decided from the blocks the request held BEFORE the scheduler swapped in its sparse block list
-            # (the reference calls it ahead of touching self.blocks, gsa.py:141-149)
-            self.get_sparse_and_free_block(True, *prefetch)
         src = req_state.block_ids[0]
+        if prefetch is not None and self.blocks and self.is_decode():
+            self._update_sparsified(src, prefetch)
+            return
         # (a decoding request's list only grows at its end: the copy is made when the list changed)
         mid = len(src) // 2
         if len(src) != len(self.blocks) or (src and (src[-1] != self.blocks[-1] or src[0] != self.blocks[0]
@@ -142,7 +144,32 @@ class GSAReqStat:
         todo = range(self._repre_done, full_after_step)
         self.calc_block_table = [self.blocks[i] for i in todo]
         self.calc_repre_slot_mapping = [self.slot_offset + i for i in todo]
+        self.calc_logical = list(todo)
         self._repre_done = max(self._repre_done, full_after_step)
+
+    def _update_sparsified(self, src: List[int], prefetch) -> None:
+        """A decoding request in prefetch mode (GSAReqStat.updata_req_state, gsa.py:133-154): ``blocks`` stays the
+        list of LOGICAL blocks - one entry per block of the sequence, a block the request grows by is appended -
+        while the cache blocks it really holds are the scheduler's list ``phys``: the resident blocks first, then
+        the blocks decoded into.  The block being written is always the last of ``phys``; it gets its
+        representative (and goes to the store) after the step that fills it."""
+        # decided from the blocks the request held BEFORE the scheduler swapped in its sparse block list
+        self.get_sparse_and_free_block(True, *prefetch)
+        if self.remain_idx is not None:
+            self.prompt_blocks = len(self.blocks)
+        self.phys = list(src)
+        if len(src) != self.sparse_len:
+            self.blocks = self.blocks + [src[-1]]
+            self.blocks_version += 1
+            self.sparse_len = len(src)
+        full_after_step = min(self.get_seq_len() // self.block_size, len(self.blocks))
+        self.calc_block_table, self.calc_repre_slot_mapping, self.calc_logical = [], [], []
+        if full_after_step > self._repre_done:
+            last = len(self.blocks) - 1
+            self.calc_block_table = [src[-1]]
+            self.calc_repre_slot_mapping = [self.slot_offset + last]
+            self.calc_logical = [last]
+            self._repre_done = full_after_step
 
 
 class GSAMetaData(UcmSparseMetadata):
@@ -178,8 +205,9 @@ class TopKAndKpreManger:
 
 
 class GSA(UcmSparseBase):
-    def __init__(self, vllm_config, role: UcmSparseRole):
+    def __init__(self, vllm_config, role: UcmSparseRole, store=None):
         super().__init__(vllm_config, role)
+        self.connector = store            # prefetch mode: the KV store the request's blocks go to and come back from
         mc, pc = vllm_config.model_config, vllm_config.parallel_config
         self.block_size = vllm_config.cache_config.block_size
         self.num_key_heads = mc.get_num_kv_heads(pc)
@@ -204,6 +232,8 @@ class GSA(UcmSparseBase):
         # most of their cache blocks back, so the local window is kept aside at the end of the prefill and
         # written into the blocks that stand for it afterwards
         self.ptopk_prefetch = bool(cfg.get("ptopk_prefetch_enable", False))
+        self.prefetch_stride = max(1, int(cfg.get("prefetch_stride", 6)))   # steps between two rounds of the prefetch engine
+        self._pf = None                   # prefetch mode's tables and engine (prefetch_mode.py), built with the device state
         self.repre_dtype = torch.bfloat16 if cfg.get("repre_dtype", "float32") == "bfloat16" else torch.float32
         self.repre_mode = ops.MEAN_BF16_STORE if self.repre_dtype == torch.bfloat16 else ops.MEAN_F32
 
@@ -271,6 +301,16 @@ class GSA(UcmSparseBase):
         self._score_select = _lib.lib().ucm_score_select
         self._fused_ok = self.max_block_len <= 1024     # longer requests take the two launches
         self._dev_ready = True
+
+    def _topk_len(self, n_blocks: int) -> int:
+        return compute_topk_len(n_blocks, self.min_topk, self.max_topk, self.topk_ratio)
+
+    def _prefetch_mode(self):
+        if self._pf is None:
+            from .prefetch_mode import GsaPrefetchMode
+
+            self._pf = GsaPrefetchMode(self, self.connector, self.device)
+        return self._pf
 
     def register_kv_caches(self, kv_caches: dict) -> None:
         for name, cache in kv_caches.items():
@@ -380,6 +420,8 @@ class GSA(UcmSparseBase):
         self.model_input["any_gsa"] = any_gsa
         # score on every retrieval_stride-th step, and whenever a request is sparsified for the first time
         is_topk = any_gsa and (self.step_count % self.retrieval_stride == 0 or not gsa_ids <= self._scored)
+        if any_gsa and self.ptopk_prefetch and self._dev_ready and self._prefetch_mode().round_due():
+            is_topk = True                # the round at the end of this step reads this step's selection
         self.model_input["is_topk"] = is_topk
         self._fast = None
         if is_topk:
@@ -446,7 +488,11 @@ class GSA(UcmSparseBase):
         a = self._sel
         a.seg_off, a.seg_len, a.topk_len, a.q_rows, a.seq_lens, a.block_tables = self.model_input["addr"]
         a.n_req, a.max_seg_len, a.total_blocks = batch, max_len, total
-        if is_topk and self._fused_ok and _raw_stream is not None:
+        if self.ptopk_prefetch:
+            # attention reads the engine's tables; the selection is kept as logical block numbers for the next round
+            a.block_tables = a.phys_out = a.sparse_seq_lens = None
+            self._prefetch_mode().begin_step(by_index)
+        elif is_topk and self._fused_ok and _raw_stream is not None:
             self._fast = self._batch_views(batch)
 
     def _batch_views(self, n: int) -> list:
@@ -459,6 +505,8 @@ class GSA(UcmSparseBase):
     def execute_finished(self) -> None:
         if self.ptopk_prefetch:
             self._gsa_sparse_local_kv()
+            if self._pf is not None:
+                self._pf.end_step()
         self.step_count += 1
 
     # ------------------------------------------------------------------ per-layer hooks
@@ -514,9 +562,11 @@ class GSA(UcmSparseBase):
             rc = self._score_select(self._sel_addr, stream)
             if rc != 0:
                 raise _lib.UcmHipError("ucm_score_select", rc, _lib.lib().ucm_last_error().decode())
-        else:
+        elif mi["is_topk"] or not self.ptopk_prefetch:
             seg_off, seg_len, topk_len, q_rows, seq_lens, tables = mi["addr"]
             repre, scores, idx, counts, phys, sparse_len = self._layer_addr[l]
+            if self.ptopk_prefetch:
+                tables = phys = sparse_len = None
             rows = self.kpre_caches.shape[1]
             if mi["is_topk"]:
                 _lib.call("ucm_score_blocks", query.data_ptr(), q_code, query.numel(), q_rows, self.num_q_heads, repre,
@@ -526,15 +576,20 @@ class GSA(UcmSparseBase):
             _lib.call("ucm_topk_windows", scores, self.scores.stride(0), rows, seg_off, seg_len, topk_len, n, mi["max_len"],
                       1, self.init_window, self.local_window, idx, self.max_block_len, counts, tables, self.max_block_len,
                       phys, seq_lens, self.block_size, sparse_len, stream)
-        views = self._batch_views(n)
         md = forward_context.attn_metadata
         md = md[layer_name] if isinstance(md, dict) else md
-        md.block_table, md.seq_lens = views[l]
+        if self.ptopk_prefetch:
+            md.block_table, md.seq_lens = self._pf.bt_step[l], self._pf.seq_step[l]
+        else:
+            md.block_table, md.seq_lens = self._batch_views(n)[l]
 
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
         # (the layer's cache was looked at in attention_begin of the same step)
         if self.model_input.get("calc_block_table"):
             self.copy_k(layer_name, forward_context)
+            if self.ptopk_prefetch:
+                l = self._layer_id(layer_name)
+                self._prefetch_mode().save_blocks(l, self._kv_full[l])
 
     def copy_k(self, layer_name: str, forward_context) -> None:
         """Representatives of the blocks this step filled (gsa.py:634-654), reduced in place on the device."""
@@ -556,6 +611,8 @@ class GSA(UcmSparseBase):
         self.topk_kpre_manger.free(request_id)
         self.gsa_stats.pop(request_id, None)
         self._scored.discard(request_id)
+        if self._pf is not None:
+            self._pf.request_finished(request_id)
 
     # ------------------------------------------------------------------ scheduler side
     def request_begin(self, request_id: ReqType, prompt_token_ids: List[int]) -> None:
@@ -575,3 +632,30 @@ class GSA(UcmSparseBase):
         num_sparse_blocks = num_all_blocks - num_prompt_blocks + topk_len + prefetch_len
         flaw = request.num_tokens % bs
         return num_sparse_blocks * bs - (bs - flaw if flaw else 0)
+
+    def allocate_slots(self, request, num_slots_sparsed, coordinator, block_pool, kv_cache_groups):
+        """Prefetch mode, scheduler side.  The reference leaves this to the base class, which does nothing; what its
+        worker side assumes (_first_topk_deal reads the resident blocks at positions 0 .. max_topk of the request's
+        block list, prefetch_engine.py:327-379) is written out here: at its first decode step a long request keeps
+        its first ``max_topk + 1`` blocks - they still hold logical blocks 0 .. max_topk - and whatever it holds
+        beyond its prompt's blocks, returns the rest to the pool, and is then allocated for the sparsified length."""
+        blocks = coordinator.get_blocks(request.request_id)[0]
+        kept = list(blocks)
+        if request.num_computed_tokens == request.num_prompt_tokens:
+            n_prompt = math.ceil(request.num_prompt_tokens / self.block_size)
+            k = self._topk_len(n_prompt)
+            keep = k + (0 if k > self.max_topk else self.max_topk - k + 1)
+            kept, returned = list(blocks[:keep]) + list(blocks[n_prompt:]), list(blocks[keep:n_prompt])
+            for block in blocks:
+                block_pool._maybe_evict_cached_block(block)
+            block_pool.free_blocks(returned)
+            coordinator.single_type_managers[0].req_to_blocks[request.request_id] = kept
+        empty = tuple([] for _ in range(len(kv_cache_groups)))
+        n_new = coordinator.get_num_blocks_to_allocate(request_id=request.request_id, num_tokens=num_slots_sparsed,
+                                                       new_computed_blocks=empty)
+        if n_new > block_pool.get_num_free_blocks():
+            return None
+        coordinator.allocate_new_blocks(request.request_id, num_slots_sparsed)
+        from ..esa.esa import _kv_cache_blocks
+
+        return _kv_cache_blocks(kept)

@@ -18,6 +18,10 @@ results stay on the device: ``load_missing`` moves the missed blocks from a
 device-addressable pool into the cache blocks chosen for them without the host
 seeing either list.  The ``obtain_*`` accessors copy them back for callers
 written against the reference's surface.
+
+Limits (the reference's containers have none): 256 resident blocks and 256
+selected blocks per request; ``set_blocks_map`` / ``add_blocks_map`` and
+``run_async_prefetch_bs`` raise ``ValueError`` beyond them.
 """
 from __future__ import annotations
 
@@ -53,6 +57,7 @@ class GSAPrefetchEngineC:
         self._row_of: Dict[int, int] = {}
         self._blocks: Dict[int, List[int]] = {}          # host mirror of map_block rows (block ids never change on the device)
         self._topk: Optional[torch.Tensor] = None
+        self._topk_width = 0
         self._step = 0
         self._done: Optional[torch.cuda.Event] = None
         self._status = True
@@ -120,6 +125,7 @@ class GSAPrefetchEngineC:
         topk = torch.zeros((self.n_layers, input_topk_buf.shape[1], self.topk_stride), dtype=torch.int32, device=self.device)
         topk[:, :, :width] = input_topk_buf[:, :, :width].to(device=self.device, dtype=torch.int32)
         self._topk = topk
+        self._topk_width = width
         self._step = step
 
     def run_async_prefetch_bs(self, req_ids: List[int], topk_lens: List[int], bs_indexes: List[int], rank: int = 0) -> None:
@@ -132,6 +138,9 @@ class GSAPrefetchEngineC:
         rows = [self._row_of.get(int(r), -1) for r in req_ids]       # unknown requests are skipped by the kernel
         if self._topk.shape[1] < len(req_ids):
             raise ValueError("selection buffer has fewer rows than requests")
+        if max((int(k) for k in topk_lens), default=0) > min(self.topk_stride, self._topk_width):
+            raise ValueError(f"a selection of more than {min(self.topk_stride, self._topk_width)} blocks: the engine holds "
+                             f"{self.topk_stride} per request and the buffer of this round {self._topk_width}")
         meta = torch.tensor([rows, [int(k) for k in topk_lens], [int(b) for b in bs_indexes]], dtype=torch.int32).pin_memory()
         meta_d = meta.to(self.device, non_blocking=True)
         topk = self._topk[:, : len(req_ids)].contiguous()
