@@ -720,6 +720,23 @@ int ucm_kv_scatter_blocks(void* const* layers, int n_layers, size_t kv_stride, s
                           ucm_stream_t stream);
 
 /*
+ * The same moves, and ucm_kv_load_planned below, for one rank of a
+ * tensor-parallel group whose ranks share the stored block: get_offset
+ * (ucm/sparse/esa/esa.py:124-135) puts rank r's K slice of layer l at
+ * 2*block_bytes*tp_size*l + 2*block_bytes*r and its V slice block_bytes later
+ * (block_bytes = the rank's own slice: block_size x its kv heads x head_dim),
+ * so a stored (or staging) block is n_layers*2*block_bytes*tp_size bytes and a
+ * rank touches only its own slices.  0 <= rank < tp_size; (0, 1) is the plain
+ * entry point.
+ */
+int ucm_kv_gather_blocks_tp(const void* const* layers, int n_layers, size_t kv_stride,
+                            size_t block_bytes, int num_blocks, const int32_t* block_ids, int n,
+                            void* staging, int rank, int tp_size, ucm_stream_t stream);
+int ucm_kv_scatter_blocks_tp(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                             int num_blocks, const int32_t* block_ids, int n, const void* staging,
+                             int rank, int tp_size, ucm_stream_t stream);
+
+/*
  * Gather of the blocks chosen by ucm_topk_windows, straight from its device
  * output (no host round trip): request r's region of `staging` starts at
  * dst_off[r] blocks and holds [layer][K|V][region_k[r]] blocks, of which the
@@ -768,6 +785,13 @@ int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_stride, siz
                         const int32_t* src_table, int src_stride, const int32_t* dst_table,
                         int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
                         const int32_t* rows, int batch, int table_rows, ucm_stream_t stream);
+int ucm_kv_load_planned_tp(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                           int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
+                           int store_first_layer, const int32_t* load_sel, int n_slots,
+                           const int32_t* src_table, int src_stride, const int32_t* dst_table,
+                           int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                           const int32_t* rows, int batch, int table_rows, int rank, int tp_size,
+                           ucm_stream_t stream);
 
 #ifdef __cplusplus
 }

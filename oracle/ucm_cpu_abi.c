@@ -32,6 +32,9 @@ TWIN(ucm_topk_windows);
 TWIN(ucm_score_select);
 TWIN(ucm_kv_gather_blocks);
 TWIN(ucm_kv_scatter_blocks);
+TWIN(ucm_kv_gather_blocks_tp);
+TWIN(ucm_kv_scatter_blocks_tp);
+TWIN(ucm_kv_load_planned_tp);
 TWIN(ucm_kv_gather_selected);
 TWIN(ucm_delta_plan);
 TWIN(ucm_delta_plan_rows);
@@ -269,10 +272,19 @@ int ucm_score_select_cpu(const ucm_score_select_args_t* p, ucm_stream_t stream)
     return rc;
 }
 
-static int kv_move(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
-                   const int32_t* block_ids, int n, void* staging, int to_staging)
+int64_t orc_get_offset(int64_t block_size, int64_t kv_heads_per_tp, int64_t head_size, int64_t rank, int64_t tp_size,
+                       int64_t precision, int64_t layer_id, int is_v, int is_mla);
+
+/* where get_offset puts a rank's K or V slice of a layer inside a stored block (a slice is block_bytes long) */
+static size_t stored_slice(size_t block_bytes, int rank, int tp_size, int layer, int kv)
 {
-    if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
+    return (size_t)orc_get_offset((int64_t)block_bytes, 1, 1, rank, tp_size, 1, layer, kv, 0);
+}
+
+static int kv_move(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                   const int32_t* block_ids, int n, void* staging, int to_staging, int rank, int tp_size)
+{
+    if (n < 0 || n_layers < 0 || tp_size < 1 || rank < 0 || rank >= tp_size) { return UCM_EINVAL; }
     if (n == 0 || n_layers == 0) { return UCM_OK; }
     if (!layers || !block_ids || !staging || num_blocks <= 0 || block_bytes == 0) { return UCM_EINVAL; }
     for (int i = 0; i < n; ++i) {
@@ -280,7 +292,8 @@ static int kv_move(void* const* layers, int n_layers, size_t kv_stride, size_t b
         for (int l = 0; l < n_layers; ++l) {
             for (int kv = 0; kv < 2; ++kv) {
                 uint8_t* c = (uint8_t*)layers[l] + (size_t)kv * kv_stride + (size_t)block_ids[i] * block_bytes;
-                uint8_t* s = (uint8_t*)staging + (((size_t)i * n_layers + l) * 2 + kv) * block_bytes;
+                uint8_t* s = (uint8_t*)staging + (size_t)i * n_layers * 2 * block_bytes * tp_size +
+                             stored_slice(block_bytes, rank, tp_size, l, kv);
                 if (to_staging) { memcpy(s, c, block_bytes); } else { memcpy(c, s, block_bytes); }
             }
         }
@@ -292,14 +305,29 @@ int ucm_kv_gather_blocks_cpu(const void* const* layers, int n_layers, size_t kv_
                              const int32_t* block_ids, int n, void* staging, ucm_stream_t stream)
 {
     (void)stream;
-    return kv_move((void* const*)layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging, 1);
+    return kv_move((void* const*)layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging, 1, 0, 1);
+}
+
+int ucm_kv_gather_blocks_tp_cpu(const void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                                const int32_t* block_ids, int n, void* staging, int rank, int tp_size, ucm_stream_t stream)
+{
+    (void)stream;
+    return kv_move((void* const*)layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging, 1, rank, tp_size);
 }
 
 int ucm_kv_scatter_blocks_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
                               const int32_t* block_ids, int n, const void* staging, ucm_stream_t stream)
 {
     (void)stream;
-    return kv_move(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, (void*)staging, 0);
+    return kv_move(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, (void*)staging, 0, 0, 1);
+}
+
+int ucm_kv_scatter_blocks_tp_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                                 const int32_t* block_ids, int n, const void* staging, int rank, int tp_size,
+                                 ucm_stream_t stream)
+{
+    (void)stream;
+    return kv_move(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, (void*)staging, 0, rank, tp_size);
 }
 
 int ucm_kv_gather_selected_cpu(const void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
@@ -624,19 +652,19 @@ int ucm_copy_batch_cpu(void* const* dst, const void* const* src, size_t num, siz
     return UCM_OK;
 }
 
-int ucm_kv_load_planned_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
-                            const void* pool, int64_t pool_blocks, size_t pool_block_bytes, int store_first_layer,
-                            const int32_t* load_sel, int n_slots, const int32_t* src_table, int src_stride,
-                            const int32_t* dst_table, int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
-                            const int32_t* rows, int batch, int table_rows, ucm_stream_t stream)
+int ucm_kv_load_planned_tp_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                               const void* pool, int64_t pool_blocks, size_t pool_block_bytes, int store_first_layer,
+                               const int32_t* load_sel, int n_slots, const int32_t* src_table, int src_stride,
+                               const int32_t* dst_table, int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                               const int32_t* rows, int batch, int table_rows, int rank, int tp_size, ucm_stream_t stream)
 {
     (void)stream;
-    if (batch < 0 || n_slots < 0 || table_rows <= 0) { return UCM_EINVAL; }
+    if (batch < 0 || n_slots < 0 || table_rows <= 0 || tp_size < 1 || rank < 0 || rank >= tp_size) { return UCM_EINVAL; }
     if (batch == 0 || n_slots == 0) { return UCM_OK; }
     if (!layers || !pool || !load_sel || !src_table || !dst_table || n_layers <= 0 || num_blocks <= 0 || block_bytes == 0 ||
         block_bytes % 16 || kv_stride % 16 || pool_block_bytes % 16 || (size_t)num_blocks * block_bytes > kv_stride ||
         store_first_layer < 0 || pool_blocks < 0 || src_stride < 1 || dst_stride < n_slots || dst_layer_stride < 0 ||
-        (size_t)(store_first_layer + n_layers) * 2 * block_bytes > pool_block_bytes) {
+        (size_t)(store_first_layer + n_layers) * 2 * block_bytes * tp_size > pool_block_bytes) {
         return UCM_EINVAL;
     }
     for (int l = 0; l < n_layers; ++l) {
@@ -658,13 +686,24 @@ int ucm_kv_load_planned_cpu(void* const* layers, int n_layers, size_t kv_stride,
                 for (int kv = 0; kv < 2; ++kv) {
                     memcpy((uint8_t*)layers[l] + (size_t)kv * kv_stride + (size_t)to * block_bytes,
                            (const uint8_t*)pool + (size_t)from * pool_block_bytes +
-                               ((size_t)(store_first_layer + l) * 2 + kv) * block_bytes,
+                               stored_slice(block_bytes, rank, tp_size, store_first_layer + l, kv),
                            block_bytes);
                 }
             }
         }
     }
     return UCM_OK;
+}
+
+int ucm_kv_load_planned_cpu(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes, int num_blocks,
+                            const void* pool, int64_t pool_blocks, size_t pool_block_bytes, int store_first_layer,
+                            const int32_t* load_sel, int n_slots, const int32_t* src_table, int src_stride,
+                            const int32_t* dst_table, int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                            const int32_t* rows, int batch, int table_rows, ucm_stream_t stream)
+{
+    return ucm_kv_load_planned_tp_cpu(layers, n_layers, kv_stride, block_bytes, num_blocks, pool, pool_blocks, pool_block_bytes,
+                                      store_first_layer, load_sel, n_slots, src_table, src_stride, dst_table, dst_stride,
+                                      dst_layer_stride, load_count, rows, batch, table_rows, 0, 1, stream);
 }
 
 /* ---- KVStar's selection ----------------------------------------------------------------------------------------- */

@@ -420,7 +420,7 @@ ORC_API int32_t orc_block_table_gather(const int32_t* block_table, const int32_t
 
 /*
  * ucm/sparse/esa/esa.py:124-135 (get_offset): byte offset of one layer's K or
- * V slice of one TP rank inside a stored block laid out [layer][K|V][rank].
+ * V slice of one TP rank inside a stored block laid out [layer][rank][K|V].
  */
 ORC_API int64_t orc_get_offset(int64_t block_size, int64_t kv_heads_per_tp, int64_t head_size,
                                int64_t rank, int64_t tp_size, int64_t precision, int64_t layer_id,

@@ -11,6 +11,7 @@ import oracle
 import synth
 
 TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_select", "ucm_kv_gather_blocks", "ucm_kv_scatter_blocks",
+         "ucm_kv_gather_blocks_tp", "ucm_kv_scatter_blocks_tp", "ucm_kv_load_planned_tp",
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
@@ -188,6 +189,15 @@ def run(call, side):
     out["moved"] = staging
     for l in range(L):
         out[f"restored{l}"] = empty[l]
+    # 7. the same moves for rank 1 of 3 ranks that share the stored block: only that rank's slices are touched
+    wide = side.up(np.full((4, L, 3, 2, BLOCK_BYTES), 0xEE, np.uint8))
+    call("ucm_kv_gather_blocks_tp", layers, L, KV_STRIDE, BLOCK_BYTES, NB, side.ptr(move), 4, side.ptr(wide), 1, 3, None)
+    empty_tp = [side.up(np.zeros((2, NB, BS, HKV, D), np.uint16)) for _ in range(L)]
+    call("ucm_kv_scatter_blocks_tp", side.pointers(empty_tp), L, KV_STRIDE, BLOCK_BYTES, NB, side.ptr(move), 4, side.ptr(wide), 1, 3,
+         None)
+    out["moved_tp"] = wide
+    for l in range(L):
+        out[f"restored_tp{l}"] = empty_tp[l]
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x
 
@@ -445,6 +455,16 @@ def run_more(call, side):
          P_ROWS * P_CAP, side.ptr(load_count), side.ptr(rows), 4, P_ROWS, None)
     for l in range(P_L):
         out[f"cache{l}"] = caches[l]
+    # the same loads out of stored blocks that two ranks share, for rank 1: [block][layer][rank][K|V]
+    caches_tp = [side.up(np.zeros((2, P_NB, P_BLOCK_BYTES), np.uint8)) for _ in range(P_L)]
+    pool_tp = np.full((P_POOL, P_L, 2, 2, P_BLOCK_BYTES), 0xEE, np.uint8)
+    pool_tp[:, :, 1] = np.asarray(x["pool"]).reshape(P_POOL, P_L, 2, P_BLOCK_BYTES)
+    pool_tp = side.up(pool_tp)
+    call("ucm_kv_load_planned_tp", side.pointers(caches_tp), P_L, P_NB * P_BLOCK_BYTES, P_BLOCK_BYTES, P_NB, side.ptr(pool_tp),
+         P_POOL, P_L * 4 * P_BLOCK_BYTES, 0, side.ptr(miss_idxs), P_TOPK, side.ptr(src_table), 12, side.ptr(load_blocks), P_CAP,
+         P_ROWS * P_CAP, side.ptr(load_count), side.ptr(rows), 4, P_ROWS, 1, 2, None)
+    for l in range(P_L):
+        out[f"cache_tp{l}"] = caches_tp[l]
     side.sync()
     return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
 

@@ -50,6 +50,17 @@ def test_twins_reproduce_the_oracle(ucm):
         for b in (5, 0, 11):
             want[:, b] = x["caches"][l][:, b]
         assert np.array_equal(got[f"restored{l}"], want)
+        assert np.array_equal(got[f"restored_tp{l}"], want)
+    # one rank of three that share the stored block: its slices sit where get_offset says, the others' bytes stay
+    wide = got["moved_tp"]                               # [4 blocks][layer][rank][K|V][bytes]
+    flat = wide.reshape(4, -1)
+    assert (wide[:, :, [0, 2]] == 0xEE).all() and (wide[1] == 0xEE).all()
+    for i, b in ((0, 5), (2, 0), (3, 11)):
+        for l in range(L):
+            for kv in (0, 1):
+                at = O.get_offset((1, 1, cpu_twins.BLOCK_BYTES), 1, 3, 1, l, bool(kv))
+                want = x["caches"][l][kv, b].reshape(-1).view(np.uint8)
+                assert np.array_equal(flat[i, at : at + cpu_twins.BLOCK_BYTES], want), (i, l, kv)
 
 
 def test_descriptors_outside_the_tables_are_not_followed(ucm):
@@ -183,6 +194,7 @@ def test_selection_prefetch_and_load_twins_reproduce_the_oracle(ucm):
         assert np.array_equal(got["map_idx"][l, 1], x["map_idx"][l, 1])
         assert (got["success"][l, [1, 2]] == -5).all()
         assert np.array_equal(got[f"cache{l}"], want_cache[l])
+        assert np.array_equal(got[f"cache_tp{l}"], want_cache[l])      # the same blocks out of rank 1's slices of wider stored blocks
     assert any(c.any() for c in want_cache)
 
 

@@ -567,3 +567,59 @@ def test_esa_plugin_flow(ucm, dev):
     assert plugin.estimate_num_slots_sparsed(req) == top_k * bs + (5 + bs * 1 + 7)
     plugin.request_finished_in_worker("A")
     assert "A" not in plugin.req_states and len(plugin.layer_pools[0].allocated) == 0
+
+
+def test_hip_block_store_spills_to_pinned_host_and_reloads(ucm, dev):
+    """A pool of 4 slots in HBM with a tier of 6 pinned buffers behind it: the fifth block pushes the one used longest
+    ago out (an asynchronous copy on the store's stream, finished by a callback), loading a spilled block brings it
+    back, held blocks stay, and every block reads back the bytes that were dumped."""
+    from ucm_amd.store.hip_block_store import FAILURE, SUCCESS, UcmHipBlockStore
+
+    kvb = 2 * 4096
+    store = UcmHipBlockStore({"kv_block_size": kvb, "max_cache_size": 4 * kvb, "host_spill_blocks": 6})
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    data = [torch.randint(0, 255, (kvb,), dtype=torch.uint8, device=dev, generator=g) for _ in range(10)]
+    names = [f"b{i}" for i in range(10)]
+
+    def put(i):
+        assert store.create([names[i]]) == [SUCCESS]
+        assert store.wait(store.dump([names[i]], [0], [data[i]])) == SUCCESS
+        store.commit([names[i]])
+
+    def get(i):
+        out = torch.zeros(kvb, dtype=torch.uint8, device=dev)
+        assert store.wait(store.load([names[i]], [0], [out])) == SUCCESS
+        return out
+
+    for i in range(4):
+        put(i)
+    assert store.spills == 0 and store.generation == 0
+    assert torch.equal(get(0), data[0])                      # touching b0 makes b1 the coldest
+    put(4)
+    assert store.spills == 1 and "b1" in store.host_of and "b1" not in store.slot_of and store.generation == 1
+    assert store.lookup(names[:5]) == [True] * 5
+    held = store.hold(["b2", "b3"])                          # kernels will read these in place: they may not leave
+    assert held == [store.slot_of["b2"], store.slot_of["b3"]]
+    put(5)
+    put(6)
+    assert set(store.host_of) == {"b1", "b0", "b4"} and store.spills == 3
+    assert store.create(["b7"]) == [FAILURE] or "b7" in store.slot_of   # only b5 / b6 can leave now
+    store.release(["b2", "b3"])
+    # a spilled block comes back through load (and pushes another one out), bytes intact; so does one through hold
+    assert torch.equal(get(1), data[1]) and "b1" in store.slot_of and store.reloads == 1
+    slot = store.hold(["b0"])[0]
+    assert slot == store.slot_of["b0"] and store.reloads == 2
+    pool, _ = store.device_pool()
+    torch.cuda.synchronize()
+    assert torch.equal(pool[slot * kvb : (slot + 1) * kvb], data[0])
+    store.release(["b0"])
+    for i in range(7):
+        if names[i] in store.slot_of or names[i] in store.host_of:
+            assert torch.equal(get(i), data[i]), i
+    store._device.Synchronized()
+    assert store.spills_done == store.spills                 # every spill's callback has run
+    # the tier is bounded too: 4 slots + 6 buffers hold 10 blocks, the eleventh is refused
+    for i in range(7, 10):
+        put(i)
+    assert store.create(["b10"]) == [FAILURE]

@@ -520,6 +520,48 @@ def test_kv_dump_load_round_trip(ucm, dev, bb):
     assert np.array_equal(staging.cpu().numpy(), want)
 
 
+def test_kv_moves_of_one_tensor_parallel_rank(ucm, dev):
+    """Four ranks share the stored block; each moves its own K and V slices to where get_offset (esa.py:124-135) puts
+    them, leaves the others' bytes alone, and reads them back - through the block moves and through the planned load."""
+    from ucm_amd import ops
+
+    n_layers, nb, n, tp, bb = 3, 23, 7, 4, 4096
+    ids = synth.permutation(311, nb)[:n]
+    staging = torch.full((n, n_layers * 2 * bb * tp), 0xEE, dtype=torch.uint8, device=dev)
+    ranks = []
+    for rank in range(tp):
+        hs, ds = make_caches(dev, n_layers, nb, bb, 320 + rank)
+        ranks.append((hs, ds))
+        ops.kv_gather_blocks(ops.LayerPointers(ds), nb * bb, bb, nb, i32(ids, dev), staging, rank=rank, tp_size=tp)
+        got = staging.cpu().numpy()
+        for r2 in range(tp):                                         # ranks not yet written still hold the fill
+            for l in range(n_layers):
+                for kv in (0, 1):
+                    at = O.get_offset((bb, 1, 1), r2, tp, 1, l, bool(kv))
+                    for i, b in enumerate(ids):
+                        piece = got[i, at : at + bb]
+                        if r2 <= rank:
+                            assert np.array_equal(piece, ranks[r2][0][l].reshape(2, nb, bb)[kv, b]), (rank, r2, l, kv, i)
+                        else:
+                            assert (piece == 0xEE).all()
+    for rank in (2, 0):
+        hs, _ = ranks[rank]
+        fresh = [torch.zeros(2, nb, bb, dtype=torch.uint8, device=dev) for _ in range(n_layers)]
+        ops.kv_scatter_blocks(ops.LayerPointers(fresh), nb * bb, bb, nb, i32(ids, dev), staging, rank=rank, tp_size=tp)
+        # the planned load reads the same slices: logical block j of the one request is stored block j, slot j takes it
+        planned = [torch.zeros(2, nb, bb, dtype=torch.uint8, device=dev) for _ in range(n_layers)]
+        sel = torch.arange(n, dtype=torch.int32, device=dev).repeat(n_layers, 1, 1)
+        src = torch.arange(n, dtype=torch.int32, device=dev).view(1, n)
+        ops.kv_load_planned(ops.LayerPointers(planned), 0, 0, n_layers, nb * bb, bb, nb, staging, n_layers * 2 * bb * tp, sel, src,
+                            i32(ids, dev).view(1, n), None, rank=rank, tp_size=tp)
+        for l in range(n_layers):
+            want = np.zeros((2, nb, bb), np.uint8)
+            want[:, ids] = hs[l].reshape(2, nb, bb)[:, ids]
+            assert np.array_equal(fresh[l].cpu().numpy(), want) and np.array_equal(planned[l].cpu().numpy(), want), (rank, l)
+    with pytest.raises(ops.UcmHipError):
+        ops.kv_gather_blocks(ops.LayerPointers(ranks[0][1]), nb * bb, bb, nb, i32(ids, dev), staging, rank=4, tp_size=4)
+
+
 def test_copy_batch_pointer_arrays(ucm, dev):
     from ucm_amd import ops
 

@@ -21,13 +21,16 @@ def bits(t):
 @pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads,device_plans,hole", [
     (1.0, 1, True, True, True, False), (0.5, 3, True, False, True, False), (0.25, 1, False, True, True, False),
     (0.25, 1, True, False, False, False), (0.25, 1, True, True, False, False), (0.5, 3, True, True, True, False),
-    (0.25, 1, True, True, True, True), (0.25, 1, False, True, True, True), (0.25, 1, True, True, False, True)])
+    (0.25, 1, True, True, True, True), (0.25, 1, False, True, True, True), (0.25, 1, True, True, False, True),
+    (0.25, 1, True, True, True, "spill"), (0.25, 1, False, True, True, "spill"), (0.25, 1, True, True, False, "spill")])
 def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads, device_plans, hole):
     """Prefill (one chunk, or three) of 24 full blocks + 5 tokens, then 13 decode steps with stride 4: step 1 restores
     the windows and loads what the prefill group's vote picks; the vote of decode steps 1-4 is queued at step 4 and
     its winners are loaded at step 8; steps 5-8 at step 8 / 12.  Selections are checked against the CPU oracle on the
     same keys and queries.  ``hole``: at the first load the store lacks some of the prompt's blocks - the load leaves them
-    out, says so (a warning, a counter) and looks again at the next load, by which time they have arrived."""
+    out, says so (a warning, a counter) and looks again at the next load, by which time they have arrived.  ``hole ==
+    "spill"``: the store's pool is smaller than the prompt and has pinned host memory behind it - the blocks a load may
+    ask for come back into the pool when the request first loads, and stay."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvstar.multistep import KVStarMultiStep
@@ -42,7 +45,9 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
         "blk_repre_inner_token_merge": merge, "batch_retrieval": batched, "device_loads": device_loads,
         "device_plans": device_plans}}}
     slice_bytes = bs * hkv * d * 2
-    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 40 * L * 2 * slice_bytes})
+    spill, hole = hole == "spill", hole is True
+    store = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": (22 if spill else 40) * L * 2 * slice_bytes,
+                              "host_spill_blocks": 8 if spill else 0})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     assert isinstance(plugin, KVStarMultiStep)
     plugin.connector = store
@@ -97,7 +102,12 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
         store.commit(some)
 
     late = list(range(1, n_full - 2, 2)) if hole else []     # every other block between the windows arrives late
-    to_store([i for i in range(n_full) if i not in late])
+    if spill:                                                # 24 blocks into 22 slots: the two stored first leave the pool
+        to_store(list(range(12)))
+        to_store(list(range(12, n_full)))
+        assert store.spills == 2 and set(store.host_of) == {hashes[0], hashes[1]}
+    else:
+        to_store([i for i in range(n_full) if i not in late])
 
     # representatives: blocks 1 .. 21 (init window 1, local window 2), against the oracle on the same keys
     want_repre, pruned = [], []
@@ -192,6 +202,10 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
                 assert not st.blk_trans_tasks                # waited for at the first step of a stride
     if hole:
         assert plugin.load_misses == seen                    # nothing was missing any more at the later loads
+    if spill:
+        assert plugin.load_misses == 0
+        if device_plans:                                     # (the lists stay on the device: every block a list may name was held)
+            assert store.reloads >= 1 and hashes[1] in store.slot_of
     plugin.request_finished_in_worker("7")
     assert "7" not in plugin.req_states
 

@@ -34,6 +34,7 @@ SIGNATURES = {
     "ucm_esa_retrieve_rows": [_p, _i, _i, _p, _p, _i, _i, _i, _p, _i, _p, _i, _p, _p, _p, _p, _p, _i, _p],
     "ucm_delta_plan_rows": [_p, _p, _p, _p, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_kv_load_planned": [_p, _i, _sz, _sz, _i, _p, _i64, _sz, _i, _p, _i, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _p],
+    "ucm_kv_load_planned_tp": [_p, _i, _sz, _sz, _i, _p, _i64, _sz, _i, _p, _i, _p, _i, _p, _i, _i64, _p, _p, _i, _i, _i, _i, _p],
     "ucm_prefetch_plan": [_p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p],
     "ucm_delta_plan": [_p, _p, _p, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _i, _p],
@@ -56,6 +57,8 @@ SIGNATURES = {
     "ucm_device_stream": [_p],
     "ucm_kv_gather_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
     "ucm_kv_scatter_blocks": [_p, _i, _sz, _sz, _i, _p, _i, _p, _p],
+    "ucm_kv_gather_blocks_tp": [_p, _i, _sz, _sz, _i, _p, _i, _p, _i, _i, _p],
+    "ucm_kv_scatter_blocks_tp": [_p, _i, _sz, _sz, _i, _p, _i, _p, _i, _i, _p],
     "ucm_kv_gather_selected": [_p, _i, _sz, _sz, _i, _p, _p, _i, _i, _p, _p, _i, _p, _i64, _p],
 }
 

@@ -62,20 +62,31 @@ __global__ __launch_bounds__(kThreads) void copy_batch_kernel(void* const* __res
     copy_slice(static_cast<uint8_t*>(dst[i]) + off, static_cast<const uint8_t*>(src[i]) + off, len);
 }
 
+// Where a cache block's K and V slices of a layer sit inside a stored block: at layer * layer_pitch + slice_base
+// (K) and block_bytes later (V).  One rank's blocks: layer_pitch = 2 * block_bytes, slice_base = 0; rank r of tp
+// ranks that share the stored block: layer_pitch = 2 * block_bytes * tp, slice_base = 2 * block_bytes * r.
+struct StoredLayout {
+    size_t layer_pitch, slice_base;
+    __host__ __device__ size_t slice(size_t layer, unsigned kv, size_t block_bytes) const
+    {
+        return layer * layer_pitch + slice_base + kv * block_bytes;
+    }
+};
+
 // grid: x = index into block_ids, y = layer, z = K|V
 template <bool kToStaging>
 __global__ __launch_bounds__(kThreads) void kv_blocks_kernel(void* const* __restrict__ layers,
                                                              size_t kv_stride, size_t block_bytes,
                                                              const int32_t* __restrict__ block_ids,
                                                              unsigned num_blocks,
-                                                             uint8_t* __restrict__ staging)
+                                                             uint8_t* __restrict__ staging, StoredLayout lay)
 {
     const unsigned i = blockIdx.x, l = blockIdx.y, kv = blockIdx.z, n_layers = gridDim.y;
     const unsigned id = static_cast<unsigned>(block_ids[i]);
     if (id >= num_blocks) { return; }  // ids outside the cache are skipped, never dereferenced
     uint8_t* cache = static_cast<uint8_t*>(layers[l]) + kv * kv_stride +
                      static_cast<size_t>(id) * block_bytes;
-    uint8_t* stage = staging + ((static_cast<size_t>(i) * n_layers + l) * 2 + kv) * block_bytes;
+    uint8_t* stage = staging + static_cast<size_t>(i) * n_layers * lay.layer_pitch + lay.slice(l, kv, block_bytes);
     if (kToStaging) { copy_slice(stage, cache, block_bytes); }
     else { copy_slice(cache, stage, block_bytes); }
 }
@@ -110,7 +121,7 @@ __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
     const uint8_t* __restrict__ pool, uint64_t pool_blocks, size_t pool_block_bytes, unsigned store_first_layer,
     const int32_t* __restrict__ load_sel, unsigned n_slots, const int32_t* __restrict__ src_table, unsigned src_stride,
     const int32_t* __restrict__ dst_table, unsigned dst_stride, int64_t dst_layer_stride,
-    const int32_t* __restrict__ load_count, const int32_t* __restrict__ rows, unsigned table_rows)
+    const int32_t* __restrict__ load_count, const int32_t* __restrict__ rows, unsigned table_rows, StoredLayout lay)
 {
     const unsigned b = blockIdx.y, l = blockIdx.z >> 1, kv = blockIdx.z & 1;
     unsigned row = b;
@@ -130,8 +141,7 @@ __global__ __launch_bounds__(kThreads) void kv_load_planned_kernel(
         const unsigned dst = static_cast<unsigned>(dst_table[l * dst_layer_stride + static_cast<int64_t>(row) * dst_stride + j]);
         if (dst >= num_blocks) { continue; }
         copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
-                   pool + static_cast<size_t>(src) * pool_block_bytes +
-                       (static_cast<size_t>(store_first_layer + l) * 2 + kv) * block_bytes,
+                   pool + static_cast<size_t>(src) * pool_block_bytes + lay.slice(store_first_layer + l, kv, block_bytes),
                    block_bytes);
     }
 }
@@ -148,7 +158,7 @@ __global__ __launch_bounds__(kThreads) void kv_load_counted_kernel(
     const int32_t* __restrict__ load_sel, unsigned n_slots, const int32_t* __restrict__ src_table, unsigned src_stride,
     const int32_t* __restrict__ dst_table, unsigned dst_stride, int64_t dst_layer_stride,
     const int32_t* __restrict__ load_count, const int32_t* __restrict__ rows, unsigned table_rows, unsigned batch,
-    unsigned n_layers)
+    unsigned n_layers, StoredLayout lay)
 {
     __shared__ unsigned s_total[kMaxPlannedPairs + 1];   // s_total[p] = loads of the pairs before p
     __shared__ unsigned s_part[kThreads];
@@ -202,8 +212,7 @@ __global__ __launch_bounds__(kThreads) void kv_load_counted_kernel(
         const unsigned dst = static_cast<unsigned>(dst_table[l * dst_layer_stride + static_cast<int64_t>(row) * dst_stride + j]);
         if (dst >= num_blocks) { continue; }
         copy_slice(static_cast<uint8_t*>(layers[l]) + kv * kv_stride + static_cast<size_t>(dst) * block_bytes,
-                   pool + static_cast<size_t>(src) * pool_block_bytes +
-                       (static_cast<size_t>(store_first_layer + l) * 2 + kv) * block_bytes,
+                   pool + static_cast<size_t>(src) * pool_block_bytes + lay.slice(store_first_layer + l, kv, block_bytes),
                    block_bytes);
     }
 }
@@ -224,6 +233,14 @@ int check_block_args(const void* layers, int n_layers, size_t kv_stride, size_t 
     return UCM_OK;
 }
 
+int stored_layout(const char* name, size_t block_bytes, int rank, int tp_size, StoredLayout* lay)
+{
+    UCM_REQUIRE(tp_size >= 1 && rank >= 0 && rank < tp_size, "%s: rank=%d tp_size=%d", name, rank, tp_size);
+    lay->layer_pitch = 2 * block_bytes * static_cast<size_t>(tp_size);
+    lay->slice_base = 2 * block_bytes * static_cast<size_t>(rank);
+    return UCM_OK;
+}
+
 }  // namespace
 
 extern "C" int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t size,
@@ -239,30 +256,48 @@ extern "C" int ucm_copy_batch(void* const* dst, const void* const* src, size_t n
     UCM_LAUNCH_CHECK("ucm_copy_batch");
 }
 
-extern "C" int ucm_kv_gather_blocks(const void* const* layers, int n_layers, size_t kv_stride,
-                                    size_t block_bytes, int num_blocks, const int32_t* block_ids,
-                                    int n, void* staging, ucm_stream_t stream)
+extern "C" int ucm_kv_gather_blocks_tp(const void* const* layers, int n_layers, size_t kv_stride,
+                                       size_t block_bytes, int num_blocks, const int32_t* block_ids,
+                                       int n, void* staging, int rank, int tp_size, ucm_stream_t stream)
 {
     if (int rc = check_block_args(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging)) { return rc; }
+    StoredLayout lay;
+    if (int rc = stored_layout("ucm_kv_gather_blocks", block_bytes, rank, tp_size, &lay)) { return rc; }
     if (n == 0) { return UCM_OK; }
     hipLaunchKernelGGL(kv_blocks_kernel<true>, dim3(static_cast<unsigned>(n), n_layers, 2),
                        dim3(kThreads), 0, ucm::as_stream(stream), const_cast<void* const*>(layers),
                        kv_stride, block_bytes, block_ids, static_cast<unsigned>(num_blocks),
-                       static_cast<uint8_t*>(staging));
+                       static_cast<uint8_t*>(staging), lay);
     UCM_LAUNCH_CHECK("ucm_kv_gather_blocks");
+}
+
+extern "C" int ucm_kv_gather_blocks(const void* const* layers, int n_layers, size_t kv_stride,
+                                    size_t block_bytes, int num_blocks, const int32_t* block_ids,
+                                    int n, void* staging, ucm_stream_t stream)
+{
+    return ucm_kv_gather_blocks_tp(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging, 0, 1, stream);
+}
+
+extern "C" int ucm_kv_scatter_blocks_tp(void* const* layers, int n_layers, size_t kv_stride,
+                                        size_t block_bytes, int num_blocks, const int32_t* block_ids,
+                                        int n, const void* staging, int rank, int tp_size, ucm_stream_t stream)
+{
+    if (int rc = check_block_args(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging)) { return rc; }
+    StoredLayout lay;
+    if (int rc = stored_layout("ucm_kv_scatter_blocks", block_bytes, rank, tp_size, &lay)) { return rc; }
+    if (n == 0) { return UCM_OK; }
+    hipLaunchKernelGGL(kv_blocks_kernel<false>, dim3(static_cast<unsigned>(n), n_layers, 2),
+                       dim3(kThreads), 0, ucm::as_stream(stream), layers, kv_stride, block_bytes,
+                       block_ids, static_cast<unsigned>(num_blocks),
+                       static_cast<uint8_t*>(const_cast<void*>(staging)), lay);
+    UCM_LAUNCH_CHECK("ucm_kv_scatter_blocks");
 }
 
 extern "C" int ucm_kv_scatter_blocks(void* const* layers, int n_layers, size_t kv_stride,
                                      size_t block_bytes, int num_blocks, const int32_t* block_ids,
                                      int n, const void* staging, ucm_stream_t stream)
 {
-    if (int rc = check_block_args(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging)) { return rc; }
-    if (n == 0) { return UCM_OK; }
-    hipLaunchKernelGGL(kv_blocks_kernel<false>, dim3(static_cast<unsigned>(n), n_layers, 2),
-                       dim3(kThreads), 0, ucm::as_stream(stream), layers, kv_stride, block_bytes,
-                       block_ids, static_cast<unsigned>(num_blocks),
-                       static_cast<uint8_t*>(const_cast<void*>(staging)));
-    UCM_LAUNCH_CHECK("ucm_kv_scatter_blocks");
+    return ucm_kv_scatter_blocks_tp(layers, n_layers, kv_stride, block_bytes, num_blocks, block_ids, n, staging, 0, 1, stream);
 }
 
 extern "C" int ucm_kv_gather_selected(const void* const* layers, int n_layers, size_t kv_stride,
@@ -291,13 +326,16 @@ extern "C" int ucm_kv_gather_selected(const void* const* layers, int n_layers, s
     UCM_LAUNCH_CHECK("ucm_kv_gather_selected");
 }
 
-extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
-                                   int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
-                                   int store_first_layer, const int32_t* load_sel, int n_slots,
-                                   const int32_t* src_table, int src_stride, const int32_t* dst_table,
-                                   int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
-                                   const int32_t* rows, int batch, int table_rows, ucm_stream_t stream)
+extern "C" int ucm_kv_load_planned_tp(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                                      int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
+                                      int store_first_layer, const int32_t* load_sel, int n_slots,
+                                      const int32_t* src_table, int src_stride, const int32_t* dst_table,
+                                      int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                                      const int32_t* rows, int batch, int table_rows, int rank, int tp_size,
+                                      ucm_stream_t stream)
 {
+    StoredLayout lay;
+    if (int rc = stored_layout("ucm_kv_load_planned", block_bytes, rank, tp_size, &lay)) { return rc; }
     UCM_REQUIRE(batch >= 0 && n_slots >= 0 && table_rows > 0, "ucm_kv_load_planned: batch=%d n_slots=%d table_rows=%d", batch,
                 n_slots, table_rows);
     if (batch == 0 || n_slots == 0) { return UCM_OK; }
@@ -309,7 +347,7 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
                     ucm::aligned16(pool),
                 "ucm_kv_load_planned: sizes and pool must be multiples of 16");
     UCM_REQUIRE(store_first_layer >= 0 && pool_blocks >= 0 &&
-                    static_cast<size_t>(store_first_layer + n_layers) * 2 * block_bytes <= pool_block_bytes,
+                    static_cast<size_t>(store_first_layer + n_layers) * lay.layer_pitch <= pool_block_bytes,
                 "ucm_kv_load_planned: layers %d..%d do not fit a stored block of %zu bytes", store_first_layer,
                 store_first_layer + n_layers - 1, pool_block_bytes);
     UCM_REQUIRE(src_stride >= 1 && dst_stride >= n_slots && dst_layer_stride >= 0,
@@ -321,7 +359,7 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
                            static_cast<uint64_t>(pool_blocks), pool_block_bytes, static_cast<unsigned>(store_first_layer),
                            load_sel, static_cast<unsigned>(n_slots), src_table, static_cast<unsigned>(src_stride), dst_table,
                            static_cast<unsigned>(dst_stride), dst_layer_stride, load_count, rows,
-                           static_cast<unsigned>(table_rows), static_cast<unsigned>(batch), static_cast<unsigned>(n_layers));
+                           static_cast<unsigned>(table_rows), static_cast<unsigned>(batch), static_cast<unsigned>(n_layers), lay);
     } else {
         // the entries to load are scattered over a row (or there are too many rows for the counted kernel's table)
         const unsigned gx = static_cast<unsigned>(std::min(n_slots, load_count ? 8 : 16));
@@ -330,7 +368,19 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
                            static_cast<const uint8_t*>(pool), static_cast<uint64_t>(pool_blocks), pool_block_bytes,
                            static_cast<unsigned>(store_first_layer), load_sel, static_cast<unsigned>(n_slots), src_table,
                            static_cast<unsigned>(src_stride), dst_table, static_cast<unsigned>(dst_stride), dst_layer_stride,
-                           load_count, rows, static_cast<unsigned>(table_rows));
+                           load_count, rows, static_cast<unsigned>(table_rows), lay);
     }
     UCM_LAUNCH_CHECK("ucm_kv_load_planned");
+}
+
+extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_stride, size_t block_bytes,
+                                   int num_blocks, const void* pool, int64_t pool_blocks, size_t pool_block_bytes,
+                                   int store_first_layer, const int32_t* load_sel, int n_slots,
+                                   const int32_t* src_table, int src_stride, const int32_t* dst_table,
+                                   int dst_stride, int64_t dst_layer_stride, const int32_t* load_count,
+                                   const int32_t* rows, int batch, int table_rows, ucm_stream_t stream)
+{
+    return ucm_kv_load_planned_tp(layers, n_layers, kv_stride, block_bytes, num_blocks, pool, pool_blocks, pool_block_bytes,
+                                  store_first_layer, load_sel, n_slots, src_table, src_stride, dst_table, dst_stride,
+                                  dst_layer_stride, load_count, rows, batch, table_rows, 0, 1, stream);
 }

@@ -369,12 +369,14 @@ def delta_plan_rows(sel: torch.Tensor, sel_phys: torch.Tensor, count: torch.Tens
 def kv_load_planned(layers: LayerPointers, ptr_first: int, store_first_layer: int, n_layers: int, kv_stride: int,
                     block_bytes: int, num_blocks: int, pool: torch.Tensor, pool_block_bytes: int,
                     load_sel: torch.Tensor, src_table: torch.Tensor, dst_table: torch.Tensor,
-                    rows: Optional[torch.Tensor], load_count: Optional[torch.Tensor] = None) -> None:
+                    rows: Optional[torch.Tensor], load_count: Optional[torch.Tensor] = None, rank: int = 0,
+                    tp_size: int = 1) -> None:
     """pool: uint8 buffer of stored blocks ([block][layer][K|V], device or pinned host memory); load_sel int32
     [n_layers, table_rows, n_slots]: the plan of model layers store_first_layer.., whose cache pointers are entries
     ptr_first.. of ``layers``; src_table int32 [table_rows, M]; dst_table int32 [table_rows, >= n_slots], or
     [n_layers, table_rows, >= n_slots] when every layer has destinations of its own; load_count int32
-    [n_layers, table_rows] or None; rows int32 [B] or None (all table rows)."""
+    [n_layers, table_rows] or None; rows int32 [B] or None (all table rows).  tp_size > 1: the stored blocks are the ones
+    tp_size ranks share ([layer][rank][K|V] slices of block_bytes each) and ``rank``'s slices are read."""
     if load_sel.dim() != 3 or load_sel.shape[0] != n_layers:
         raise ValueError("load_sel must be [n_layers, table_rows, n_slots]")
     table_rows, n_slots = load_sel.shape[1], load_sel.shape[2]
@@ -387,12 +389,13 @@ def kv_load_planned(layers: LayerPointers, ptr_first: int, store_first_layer: in
     if ptr_first < 0 or ptr_first + n_layers > len(layers):
         raise ValueError("layer range outside the pointer table")
     nbytes = pool.numel() * pool.element_size()
-    _lib.call("ucm_kv_load_planned", layers.ptr(ptr_first), n_layers, kv_stride, block_bytes, num_blocks,
+    _lib.call("ucm_kv_load_planned_tp", layers.ptr(ptr_first), n_layers, kv_stride, block_bytes, num_blocks,
               _staging_ptr(pool, 0), nbytes // pool_block_bytes, pool_block_bytes, store_first_layer,
               _dev(load_sel, torch.int32, "load_sel"), n_slots, _dev(src_table, torch.int32, "src_table"),
               src_table.shape[1], _dev(dst_table, torch.int32, "dst_table"), dst_table.shape[-1],
               dst_table.stride(0) if per_layer else 0, _opt(load_count, torch.int32, "load_count"),
-              _opt(rows, torch.int32, "rows"), table_rows if rows is None else rows.numel(), table_rows, _stream())
+              _opt(rows, torch.int32, "rows"), table_rows if rows is None else rows.numel(), table_rows, int(rank),
+              int(tp_size), _stream())
 
 
 def prefetch_plan(map_block: torch.Tensor, map_len: torch.Tensor, map_idx: torch.Tensor, topk_idx: torch.Tensor,
@@ -499,19 +502,21 @@ def _staging_ptr(staging: torch.Tensor, need: int) -> int:
 
 
 def kv_gather_blocks(layers: LayerPointers, kv_stride: int, block_bytes: int, num_blocks: int,
-                     block_ids: torch.Tensor, staging: torch.Tensor) -> None:
+                     block_ids: torch.Tensor, staging: torch.Tensor, rank: int = 0, tp_size: int = 1) -> None:
+    """Cache blocks ``block_ids`` of every layer into ``staging`` in the stored-block layout; with tp_size > 1 the
+    staging blocks are the wider ones tp_size ranks share ([layer][rank][K|V]) and only ``rank``'s slices are written."""
     n = block_ids.numel()
-    _lib.call("ucm_kv_gather_blocks", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
+    _lib.call("ucm_kv_gather_blocks_tp", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
               _dev(block_ids, torch.int32, "block_ids"), n,
-              _staging_ptr(staging, n * len(layers) * 2 * block_bytes), _stream())
+              _staging_ptr(staging, n * len(layers) * 2 * block_bytes * tp_size), int(rank), int(tp_size), _stream())
 
 
 def kv_scatter_blocks(layers: LayerPointers, kv_stride: int, block_bytes: int, num_blocks: int,
-                      block_ids: torch.Tensor, staging: torch.Tensor) -> None:
+                      block_ids: torch.Tensor, staging: torch.Tensor, rank: int = 0, tp_size: int = 1) -> None:
     n = block_ids.numel()
-    _lib.call("ucm_kv_scatter_blocks", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
+    _lib.call("ucm_kv_scatter_blocks_tp", layers.ptr(), len(layers), kv_stride, block_bytes, num_blocks,
               _dev(block_ids, torch.int32, "block_ids"), n,
-              _staging_ptr(staging, n * len(layers) * 2 * block_bytes), _stream())
+              _staging_ptr(staging, n * len(layers) * 2 * block_bytes * tp_size), int(rank), int(tp_size), _stream())
 
 
 def kv_gather_selected(layers: LayerPointers, kv_stride: int, block_bytes: int, num_blocks: int,

@@ -29,6 +29,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ... import ops
+from ..utils import HeldBlocks
 
 
 @dataclass
@@ -45,6 +46,7 @@ class DeviceRequest:
     src_ready: bool = False                                   # every block of the sparse range was found in the store
     src_missing: int = 0                                      # how many were not, at the last look
     skipped: bool = False                                     # a load ran while some were missing
+    held: Optional[HeldBlocks] = None                         # its stored blocks stay in the store's pool while it lives
 
 
 class StepPlan:
@@ -146,6 +148,9 @@ class EsaDevicePath:
         step (esa.py:366-399) and uploads the index arrays."""
         esa, t = self.esa, self.tables
         stride = esa.esa_cfg["retrieval_stride"]
+        wait = getattr(esa.connector, "wait_for_writes", None)
+        if wait is not None:
+            wait()                       # blocks dumped through the store's stream are read in place by this step's loads
         first, first_q, retr, retr_q, load = [], [], [], [], []
         m_first = m_retr = 0
         prefill = []
@@ -211,8 +216,9 @@ class EsaDevicePath:
         the store holds them all; otherwise again at every step until it does.  A load that ran in between left the
         missing blocks out while the plan counted them as present, so once more of them are found the request's
         resident lists are forgotten and its next load brings in everything it selects."""
-        slot_of = self.esa.connector.slot_of
-        src = [slot_of.get(h, -1) for h in st.block_hashes[: st.sparse_range]]
+        if st.held is None:
+            st.held = HeldBlocks(self.esa.connector)
+        src = st.held.slots(st.block_hashes[: st.sparse_range])
         missing = src.count(-1)
         if src:
             self.tables.src_table[st.row, : len(src)] = ops.upload(torch.tensor(src, dtype=torch.int32), self.device)
@@ -307,4 +313,6 @@ class EsaDevicePath:
             return
         for l, slots in enumerate(st.slots):
             self.esa.layer_pools[l].free(slots)
+        if st.held is not None:
+            st.held.release()
         self.tables.release_row(st.row)

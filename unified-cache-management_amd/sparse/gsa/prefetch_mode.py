@@ -38,6 +38,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ... import ops
+from ..utils import HeldBlocks
 from .prefetch import GSAPrefetchEngineC
 
 
@@ -66,6 +67,7 @@ class GsaPrefetchMode:
         self.to_map: Dict[object, List[tuple]] = {}               # blocks to tell the engine about at the next round
         self.to_table: Dict[object, List[int]] = {}               # ... and to append to the table that round activates
         self.batch: List = []
+        self.held: Dict[object, HeldBlocks] = {}                  # per request: its stored blocks stay in the store's pool
         self.ready = set()                                        # requests whose table rows have been set up
         self.bt_step = self.seq_step = None
         self._save_key = None
@@ -188,11 +190,13 @@ class GsaPrefetchMode:
 
     def _sources(self, st, engine_row: int, logical) -> None:
         """Where the store keeps the request's logical blocks (the hash -> pool block lookup, once per block)."""
-        slot_of = self.store.slot_of
         logical = list(logical)
         if not logical:
             return
-        slots = [slot_of.get(self.block_hash(st.req_id, i), -1) for i in logical]
+        held = self.held.get(st.req_id)
+        if held is None:
+            held = self.held[st.req_id] = HeldBlocks(self.store)
+        slots = held.slots([self.block_hash(st.req_id, i) for i in logical])
         # (the request's last block is still being written and comes to the store when it is full; it is inside the
         # selection's window until then and never asked for)
         missing = sum(1 for i, s in zip(logical, slots) if s < 0 and i < st._repre_done)
@@ -231,7 +235,7 @@ class GsaPrefetchMode:
             for (st, logical), slot in zip(owners, slots):       # a sparsified request can be asked for them from now on
                 eid = self.engine_id.get(st.req_id)
                 if eid is not None and self.engine.row_of(eid) >= 0:
-                    self.src_table[self.engine.row_of(eid), logical] = slot
+                    self._sources(st, self.engine.row_of(eid), [logical])
         if self._save is None:
             return
         src, dst, block_bytes, hashes = self._save
@@ -287,3 +291,6 @@ class GsaPrefetchMode:
         self.to_map.pop(request_id, None)
         self.to_table.pop(request_id, None)
         self.ready.discard(request_id)
+        held = self.held.pop(request_id, None)
+        if held is not None:
+            held.release()

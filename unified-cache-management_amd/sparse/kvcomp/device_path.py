@@ -35,6 +35,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ... import ops
+from ..utils import HeldBlocks
 
 
 class KvCompDevicePath:
@@ -55,6 +56,7 @@ class KvCompDevicePath:
         self._desc = torch.empty((5, rows), dtype=torch.int32)
         self.n_src: Dict[object, int] = {}                        # candidates of a request whose pool block is uploaded
         self.src_absent: Dict[object, List[int]] = {}             # ... and those the store did not hold at the last look
+        self.held: Dict[object, HeldBlocks] = {}                  # per request: its stored blocks stay in the store's pool
         self.dst_ids: Dict[object, tuple] = {}
         self.active: List[object] = []                            # requests that retrieve in this step
         self.first_of: Dict[object, int] = {}
@@ -130,17 +132,20 @@ class KvCompDevicePath:
             return
         from .kvcomp import ReqStatePerLayer                 # (the plugin module imports this one)
 
-        slot_of = self.plugin.connector.slot_of
+        held = self.held.get(request_id)
+        if held is None:
+            held = self.held[request_id] = HeldBlocks(self.plugin.connector)
         name = ReqStatePerLayer.block_hash
         if absent:
-            found = [(i, slot_of[name(request_id, first + i)]) for i in absent if name(request_id, first + i) in slot_of]
+            looked = held.slots([name(request_id, first + i) for i in absent])
+            found = [(i, slot) for i, slot in zip(absent, looked) if slot >= 0]
             if found:
                 at = torch.tensor([i for i, _ in found], dtype=torch.int64, device=self.device)
                 self.src_table[row].index_copy_(0, at, ops.upload(torch.tensor([s for _, s in found], dtype=torch.int32), self.device))
                 gone = {i for i, _ in found}
                 absent = [i for i in absent if i not in gone]
         if done < count:
-            src = [slot_of.get(name(request_id, first + i), -1) for i in range(done, count)]
+            src = held.slots([name(request_id, first + i) for i in range(done, count)])
             self.src_table[row, done:count] = ops.upload(torch.tensor(src, dtype=torch.int32), self.device)
             absent = (absent or []) + [done + i for i, s in enumerate(src) if s < 0]
             self.n_src[request_id] = count
@@ -185,7 +190,9 @@ class KvCompDevicePath:
         if step_key is not self._save_key:
             store = p.connector
             hashes = [ReqStatePerLayer.block_hash(r, b) for r, _, logical in batch for b in logical]
+            made = [h for h in hashes if h not in store.slot_of]
             if any(rc != 0 for rc in store.create(hashes)):
+                store.commit(made, False)        # the slots this call reserved go back: nothing was written into them
                 return False
             physical = [b for _, blocks, _ in batch for b in blocks]
             rows = [p.segment_base(r) + b for r, _, logical in batch for b in logical]
@@ -266,5 +273,8 @@ class KvCompDevicePath:
         return [self.first_of[request_id] + int(x) for x in self.idx[layer_id, i, :n].tolist()]
 
     def request_finished(self, request_id) -> None:
+        held = self.held.pop(request_id, None)
+        if held is not None:
+            held.release()
         for table in (self.n_src, self.src_absent, self.dst_ids, self.first_of, self.windows, self.win_shape):
             table.pop(request_id, None)

@@ -28,6 +28,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ... import _lib, ops
+from ...sparse.utils import HeldBlocks
 from . import retrieve as kvstar_retrieve
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -70,6 +71,7 @@ class KVStarLayerPath:
         self.rings: Dict[int, torch.Tensor] = {}          # layer -> fp16 [rows, 2 groups, stride, q_heads * head_dim]
         self.row_elems = 0
         self.batches: Dict[tuple, _Batch] = {}
+        self.held: Dict[object, HeldBlocks] = {}           # per request: its stored blocks stay in the store's pool
         self.step: dict = {}
         self.side = None
         self.reading: Dict[int, object] = {}               # layer -> event of the side stream's last launch that reads its ring
@@ -97,6 +99,9 @@ class KVStarLayerPath:
         row = self.rows.pop(request_id, None)
         if row is not None:
             self.free_rows.append(row)
+        held = self.held.pop(request_id, None)
+        if held is not None:
+            held.release()
         for key in [k for k in self.batches if request_id in k[0]]:
             del self.batches[key]
 
@@ -348,12 +353,15 @@ class KVStarLayerPath:
         warned about); a request's destinations when its candidate blocks have changed."""
         if not batch.src_complete and ("src", id(batch)) not in self.step["cache"]:
             self.step["cache"][("src", id(batch))] = True           # once per step, not once per layer
-            slot_of = self.plugin.connector.slot_of
             src = torch.full((batch.n, max(batch.longest, 1)), -1, dtype=torch.int32)
             missing = 0
             for row, states in enumerate(batch.states):
                 st = states[0]
-                stored = [slot_of.get(h, -1) for h in st.block_hashes[st.init_window_sz : st.init_window_sz + batch.lens[row]]]
+                rid = st.req_meta.request_id
+                held = self.held.get(rid)
+                if held is None:
+                    held = self.held[rid] = HeldBlocks(self.plugin.connector)
+                stored = held.slots(st.block_hashes[st.init_window_sz : st.init_window_sz + batch.lens[row]])
                 missing += stored.count(-1)
                 src[row, : len(stored)] = torch.tensor(stored, dtype=torch.int32)
             if missing:

@@ -37,6 +37,7 @@ import torch
 
 from ..base import INVALID_SLOT, UcmSparseBase, UcmSparseMetadata, UcmSparseRole
 from ..esa.esa import _kv_cache_blocks, block_hash_func, get_offset
+from ..utils import HeldBlocks
 from ... import ops
 from . import retrieve as kvstar_retrieve
 from .layer_path import KVStarLayerPath
@@ -580,16 +581,17 @@ class KVStarMultiStep(UcmSparseBase):
         layer_id = int(layer_name.split(".")[2])
         kv = forward_context.no_compile_layers[layer_name].kv_cache[forward_context.virtual_engine]
         pool, pool_block_bytes = self.connector.device_pool()
-        slot_of = self.connector.slot_of
         es = kv.element_size()
         kv_stride, block_bytes = kv.stride(0) * es, kv.stride(1) * es
         cache, stored = kv.data_ptr(), pool.data_ptr() + layer_id * 2 * block_bytes
         dst, src = [], []
         missing = 0
+        # (held while the copy is queued: a store with a tier behind its pool brings spilled blocks back first, and
+        # orders whatever it does to these slots later after this stream's work)
+        held = HeldBlocks(self.connector)
         for hashes, ids in sink:
-            for h, b in zip(hashes, ids):
-                slot = slot_of.get(h)
-                if slot is None:
+            for slot, b in zip(held.slots(hashes), ids):
+                if slot < 0:
                     missing += 1
                     continue
                 for plane in (0, 1):
@@ -600,6 +602,7 @@ class KVStarMultiStep(UcmSparseBase):
         if src:
             ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
             ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
+        held.release()
 
     def _flush_planned(self, plan: list, layer_name: str, forward_context) -> None:
         """The loads whose lists stay on the device: per launch that produced them, one ucm_kv_load_planned follows
@@ -625,15 +628,15 @@ class KVStarMultiStep(UcmSparseBase):
             key = (n_rows, width, tuple((st.req_meta.request_id, row) for st, _, row, _ in members))
             tables = self._step_cache.get(key)
             if tables is None:
-                slot_of = self.connector.slot_of
+                held = self._step_cache.setdefault("held", HeldBlocks(self.connector))   # until the step's last layer
                 longest = max(len(st.block_hashes) for st, _, _, _ in members)
                 src = torch.full((n_rows, max(longest, 1)), -1, dtype=torch.int32)
                 dst = torch.full((n_rows, width), -1, dtype=torch.int32)
                 missing = 0
                 for st, _, row, candidates in members:
                     first = st.init_window_sz
-                    stored = [slot_of.get(h, -1) for h in st.block_hashes[first:]]
-                    missing += stored[: st.blk_repre.shape[0]].count(-1)
+                    stored = held.slots(st.block_hashes[first : first + st.blk_repre.shape[0]])
+                    missing += stored.count(-1)
                     src[row, : len(stored)] = torch.tensor(stored, dtype=torch.int32)
                     dst[row, : min(len(candidates), width)] = torch.tensor(candidates[:width], dtype=torch.int32)
                 if missing:
@@ -846,6 +849,9 @@ class KVStarMultiStep(UcmSparseBase):
                              self.token_blk_size, req.prompt_token_ids, q_start, int(starts[row + 1]) - q_start,
                              self.kvstar_multistep_cfg["retrieval_stride"])
         self._sparse_metadata = meta
+        held = self._step_cache.get("held")
+        if held is not None:
+            held.release()
         self._step_cache = {}
         self._n_slots = len(self._layer_slots)
         path = self._layer_path() if self.role == UcmSparseRole.WORKER else None
