@@ -706,10 +706,14 @@ def main():
             torch.cuda.synchronize()
             us = f_e0.elapsed_time(f_e1) / args.steps * 1e3
             nbytes = f_layers * (f_rows * ROW * tab.element_size() + f_req * f_hq * D * 2 + f_rows * 4)
+            f_kernel = "score_kernel_bf16" if name == "bf16" else "score_kernel"
             f_out[name] = {"retrieval_us": round(us, 1),
-                           "roofline": {"kernel": "score_kernel_bf16" if name == "bf16" else "score_kernel", "bound": "hbm",
+                           "roofline": {"kernel": f_kernel, "bound": "hbm",
                                         "achieved": round(nbytes / us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                        "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": nbytes}}
+                                        "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                                        "traffic": measured_traffic(f"config4_score_{name}_select", f_kernel,
+                                                                    {"seed": args.seed, "layers": f_layers, "blocks": f_rows}),
+                                        "algorithmic_bytes": nbytes}}
             if name == "f32":
                 f_tab32 = tab
         # the incremental representative: the block that filled up, one per request, all 80 layers in one launch

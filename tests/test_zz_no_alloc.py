@@ -25,9 +25,14 @@ def _both(ucm, dev, data, q, idx, topk):
         head = (data.data_ptr(), data.shape[0], data.shape[1], q.data_ptr(), idx.data_ptr(), batch, m, topk)
         tail = (out_i.data_ptr(), out_s.data_ptr(), out_c.data_ptr(), stride, stream)
         if static:
-            before = torch.cuda.memory_allocated(dev)
+            # neither torch's allocator nor the driver hands out memory during the call (a hipMalloc inside the
+            # library would not show in torch's own count, it does in the device's free memory)
+            torch.cuda.synchronize()
+            before, free_before = torch.cuda.memory_allocated(dev), torch.cuda.mem_get_info(dev)[0]
             _lib.call("ucm_esa_retrieve_static", *head, *tail)
+            torch.cuda.synchronize()
             assert torch.cuda.memory_allocated(dev) == before
+            assert torch.cuda.mem_get_info(dev)[0] == free_before
         else:
             ws = torch.zeros(batch * m, dtype=torch.float32, device=dev)
             _lib.call("ucm_esa_retrieve", *head, ws.data_ptr(), *tail)
