@@ -56,6 +56,9 @@ extern "C" {
 #define UCM_MEAN_ABS 4        /* or-ed to one of the above: the mean of the ABSOLUTE values, token order as before
                                (the per-channel |k| statistic KVStar picks its channels by,
                                ucm/sparse/kvstar/multistep.py:284-292, one block at a time) */
+#define UCM_MEAN_KEYS_F16 8   /* or-ed to UCM_MEAN_F32 or UCM_MEAN_BF16_ROUND: the key cache is fp16 (a model that runs in
+                              * float16), and "rounded" then means rounded to fp16, the cache's own type, and widened.
+                              * UCM_MEAN_BF16_STORE is not offered for fp16 caches (UCM_ENOTSUP). */
 
 typedef void* ucm_stream_t; /* hipStream_t */
 
@@ -73,6 +76,7 @@ const char* ucm_last_error(void);
  * way the live hooks index it (GSA.copy_k, ucm/sparse/gsa/gsa.py:634-654;
  * ReqStatePerLayer.extract_block_repre, ucm/sparse/esa/esa.py:265-266).
  *   k_layers   dev: n_layers pointers to bf16 [num_blocks][block_size][kv_heads][head_dim]
+ *              (fp16 with UCM_MEAN_KEYS_F16 or-ed to the mode)
  *   block_ids  dev int32[n]: cache blocks to reduce (same ids in every layer)
  *   slots      dev int32[n]: destination row of each block in `repre`
  *   num_blocks, repre_rows: sizes of a K plane and of one layer's table; an id

@@ -56,6 +56,7 @@ def _sig(lib, name, restype, *argtypes):
 _orc_vector_mean = _sig(_orc, "orc_vector_mean", None, _p, _p, _u32, _u32)
 _orc_k_repre_block = _sig(_orc, "orc_k_repre_block", None, _p, _u32, _u32, _u32, _p)
 _orc_block_mean_paged = _sig(_orc, "orc_block_mean_paged", None, _p, _p, _p, _u32, _u32, _u32, _u32, _p, C.c_int)
+_orc_block_mean_paged_f16 = _sig(_orc, "orc_block_mean_paged_f16", None, _p, _p, _p, _u32, _u32, _u32, _u32, _p, C.c_int)
 _orc_q_head_mean = _sig(_orc, "orc_q_head_mean", None, _p, _u32, _u32, _u32)
 _orc_dot16 = _sig(_orc, "orc_dot16", _f32, _p, _p, _u32)
 _orc_kq_scores = _sig(_orc, "orc_kq_scores", None, _p, _p, _u32, _u32, _u32, _u32, _p)
@@ -121,13 +122,15 @@ def k_repre_block(k_array: np.ndarray) -> np.ndarray:
     return out
 
 
-def block_mean_paged(k_cache_bits, block_ids, slots, repre, round_bf16=False) -> None:
-    """k_cache_bits uint16 [num_blocks, T, H, D]; writes repre[slots[i]] in place."""
+def block_mean_paged(k_cache_bits, block_ids, slots, repre, round_bf16=False, keys_f16=False) -> None:
+    """k_cache_bits uint16 [num_blocks, T, H, D] (bf16 bit patterns, or fp16 ones with keys_f16: round_bf16 then
+    rounds to fp16, the cache's own type); writes repre[slots[i]] in place."""
     kc = _c(k_cache_bits, np.uint16)
     _, t, h, d = kc.shape
     ids, sl = _c(block_ids, np.int32), _c(slots, np.int32)
     assert repre.dtype == np.float32 and repre.flags.c_contiguous
-    _orc_block_mean_paged(_ptr(kc), _ptr(ids), _ptr(sl), len(ids), t, h, d, _ptr(repre), int(round_bf16))
+    fn = _orc_block_mean_paged_f16 if keys_f16 else _orc_block_mean_paged
+    fn(_ptr(kc), _ptr(ids), _ptr(sl), len(ids), t, h, d, _ptr(repre), int(round_bf16))
 
 
 def q_head_mean(q: np.ndarray, k_head: int) -> np.ndarray:

@@ -56,6 +56,8 @@ TWIN(ucm_kvstar_park_queries);
 /* the oracle's functions these forward to (ucm_oracle.c) */
 float orc_bf16_to_f32(uint16_t h);
 uint16_t orc_f32_to_bf16(float f);
+void orc_block_mean_paged_f16(const uint16_t* k_cache, const int32_t* block_ids, const int32_t* slots, uint32_t n,
+                              uint32_t blockSize, uint32_t kHead, uint32_t headSize, float* repre, int round_f16);
 void orc_block_mean_paged(const uint16_t* k_cache, const int32_t* block_ids, const int32_t* slots, uint32_t n,
                           uint32_t blockSize, uint32_t kHead, uint32_t headSize, float* repre, int round_bf16);
 void orc_q_head_mean(float* q, uint32_t kHead, uint32_t qHead, uint32_t headSize);
@@ -97,11 +99,15 @@ int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks
     if (n < 0 || n_layers < 0) { return UCM_EINVAL; }
     if (n == 0 || n_layers == 0) { return UCM_OK; }
     if (!k_layers || !block_ids || !slots || !repre || num_blocks <= 0 || repre_rows <= 0 || block_size <= 0 ||
-        kv_heads <= 0 || head_dim <= 0 || (mode & ~UCM_MEAN_ABS) < UCM_MEAN_F32 || (mode & ~UCM_MEAN_ABS) > UCM_MEAN_BF16_STORE) {
+        kv_heads <= 0 || head_dim <= 0 || (mode & ~(UCM_MEAN_ABS | UCM_MEAN_KEYS_F16)) < UCM_MEAN_F32 ||
+        (mode & ~(UCM_MEAN_ABS | UCM_MEAN_KEYS_F16)) > UCM_MEAN_BF16_STORE) {
         return UCM_EINVAL;
     }
-    const int of_abs = (mode & UCM_MEAN_ABS) != 0;
-    mode &= ~UCM_MEAN_ABS;
+    const int of_abs = (mode & UCM_MEAN_ABS) != 0, keys_f16 = (mode & UCM_MEAN_KEYS_F16) != 0;
+    mode &= ~(UCM_MEAN_ABS | UCM_MEAN_KEYS_F16);
+    if (keys_f16 && mode == UCM_MEAN_BF16_STORE) { return UCM_ENOTSUP; }
+    void (*mean)(const uint16_t*, const int32_t*, const int32_t*, uint32_t, uint32_t, uint32_t, uint32_t, float*, int) =
+        keys_f16 ? orc_block_mean_paged_f16 : orc_block_mean_paged;
     const size_t row = (size_t)kv_heads * head_dim;
     float* tmp = (float*)malloc(row * sizeof(float));
     uint16_t* blk = of_abs ? (uint16_t*)malloc((size_t)block_size * row * sizeof(uint16_t)) : NULL;   /* the block without its signs */
@@ -113,11 +119,10 @@ int ucm_block_mean_cpu(const void* const* k_layers, int n_layers, int num_blocks
             if (of_abs) {
                 const uint16_t* src = (const uint16_t*)k_layers[l] + (size_t)block_ids[i] * block_size * row;
                 for (size_t e = 0; e < (size_t)block_size * row; ++e) { blk[e] = src[e] & 0x7fffu; }
-                orc_block_mean_paged(blk, &zero, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads, (uint32_t)head_dim, tmp,
-                                     mode != UCM_MEAN_F32);
+                mean(blk, &zero, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads, (uint32_t)head_dim, tmp, mode != UCM_MEAN_F32);
             } else {
-                orc_block_mean_paged((const uint16_t*)k_layers[l], &block_ids[i], &zero, 1, (uint32_t)block_size,
-                                     (uint32_t)kv_heads, (uint32_t)head_dim, tmp, mode != UCM_MEAN_F32);
+                mean((const uint16_t*)k_layers[l], &block_ids[i], &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads,
+                     (uint32_t)head_dim, tmp, mode != UCM_MEAN_F32);
             }
             const size_t at = (size_t)l * (size_t)repre_layer_stride + (size_t)slots[i] * row;
             if (mode == UCM_MEAN_BF16_STORE) {

@@ -34,6 +34,8 @@
  *       and exactly summed products on rows built to cancel; orc_hash_colsum:
  *       2*popcount - T; orc_kv_gather_selected: closed-form placement on a
  *       poisoned buffer; orc_topk_windows_i32: brute force.
+ *   orc_block_mean_paged_f16: sequential fp32 sums in numpy on small blocks; its conversions are the
+ *       half-precision ones pinned against numpy's float16.
  *   orc_prefetch_run: the reference's kvcache_pre.cpp compiled against this
  *       image's torch (oracle/_ref/gsa_prefetch*.so) and driven through whole
  *       call sequences, plus the golden vectors written from it.
@@ -754,6 +756,28 @@ ORC_API uint16_t orc_f32_to_f16(float f)
     if (rem > half || (rem == half && (q & 1u))) { ++q; }
     if (e >= -14) { return (uint16_t)(s | (uint16_t)(((uint32_t)(e + 15) << 10) + (q - 0x400u))); }
     return (uint16_t)(s | (uint16_t)q);                                 /* subnormal (a carry makes 2^-14) */
+}
+
+/*
+ * orc_block_mean_paged for a paged fp16 key cache (a model that runs in float16): the same fp32 accumulation in
+ * token order; round_f16 != 0 rounds the mean to fp16 and widens it again - the model-dtype mean the live torch
+ * path stores (ucm/sparse/gsa/gsa.py:640-652, ucm/sparse/esa/esa.py:265-266 take the mean in the cache's dtype).
+ */
+ORC_API void orc_block_mean_paged_f16(const uint16_t* k_cache, const int32_t* block_ids, const int32_t* slots, uint32_t n,
+                                      uint32_t blockSize, uint32_t kHead, uint32_t headSize, float* repre, int round_f16)
+{
+    const size_t row = (size_t)kHead * headSize;
+    const float inv = 1.0f / (float)blockSize;
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint16_t* blk = k_cache + (size_t)block_ids[i] * blockSize * row;
+        float* out = repre + (size_t)slots[i] * row;
+        for (size_t c = 0; c < row; ++c) {
+            float acc = orc_f16_to_f32(blk[c]);
+            for (uint32_t t = 1; t < blockSize; ++t) { acc = acc + orc_f16_to_f32(blk[(size_t)t * row + c]); }
+            acc = acc * inv;
+            out[c] = round_f16 ? orc_f16_to_f32(orc_f32_to_f16(acc)) : acc;
+        }
+    }
 }
 
 /*

@@ -196,11 +196,12 @@ def topk_len(n, lo, hi):
     return min(lo, n) if t < lo else min(t, hi)
 
 
-@pytest.mark.parametrize("repre_dtype", ["float32", "bfloat16"])
-def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
+@pytest.mark.parametrize("repre_dtype,model", [("float32", "bfloat16"), ("bfloat16", "bfloat16"), ("float32", "float16")])
+def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
     """Two requests through prefill and 40 decode steps, two layers: after every attention_begin the
     layer's block table and sequence lengths must be what the oracle selects from the same cache.
-    With a bfloat16 table the representatives are the rounded means of the live reference path."""
+    With a bfloat16 table the representatives are the rounded means of the live reference path; a model that runs
+    in float16 (cache, keys and queries) goes through the same hooks with an fp32 table."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.gsa.gsa import GSA
@@ -218,7 +219,8 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
 
     g = torch.Generator(device=dev)
     g.manual_seed(5)
-    caches = [torch.zeros(2, nb, bs, hkv, d, dtype=torch.bfloat16, device=dev) for _ in range(L)]
+    model = getattr(torch, model)
+    caches = [torch.zeros(2, nb, bs, hkv, d, dtype=model, device=dev) for _ in range(L)]
     names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
     fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
     free_blocks = [int(x) for x in synth.permutation(730, nb)]
@@ -250,8 +252,8 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
         for l in range(L):
             md = ns(block_table=bt.clone(), seq_lens=torch.tensor(seq_lens, dtype=torch.int32, device=dev))
             fc.attn_metadata = {names[l]: md}
-            query = torch.randn(n_tok, hq, d, device=dev, generator=g).to(torch.bfloat16)
-            key = torch.randn(n_tok, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+            query = torch.randn(n_tok, hq, d, device=dev, generator=g).to(model)
+            key = torch.randn(n_tok, hkv, d, device=dev, generator=g).to(model)
             # the model writes this step's keys into the paged cache before attention runs
             t0 = 0
             for r in ("A", "B"):
@@ -284,7 +286,7 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype):
                 if todo:
                     kc = caches[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
                     O.block_mean_paged(kc, [reqs[r].block_ids[0][i] for i in todo], todo, repre_h[r][l],
-                                       round_bf16=(repre_dtype == "bfloat16"))
+                                       round_bf16=(repre_dtype == "bfloat16"), keys_f16=(model == torch.float16))
         for r in ("A", "B"):
             done_blocks[r] = max(done_blocks[r], min(seq_lens[("A", "B").index(r)] // bs, len(reqs[r].block_ids[0])))
         plugin.execute_finished()

@@ -72,6 +72,32 @@ def test_block_mean_matches_oracle(ucm, dev, hkv, d, bs, n_layers):
                        repre[:, torch.from_numpy(slots.astype(np.int64)).to(dev)])
 
 
+@pytest.mark.parametrize("hkv,d,bs", [(8, 128, 128), (2, 64, 16), (1, 8, 5)])
+def test_block_mean_of_fp16_caches(ucm, dev, hkv, d, bs):
+    """A model that runs in float16: the wrapper sees the cache's type, the kernel widens fp16 keys, and the rounding
+    mode rounds to fp16 (the cache's type); a bf16 table from an fp16 cache is refused."""
+    from ucm_amd import ops
+
+    nb, rows, n_layers = 19, 30, 2
+    row = hkv * d
+    caches = [(torch.from_numpy(synth.normal_f32(130 + l, (nb, bs, hkv, d))) * 3).to(torch.float16).to(dev) for l in range(n_layers)]
+    caches_h = [c.cpu().numpy().view(np.uint16) for c in caches]
+    lp = ops.LayerPointers(caches)
+    ids, slots = synth.permutation(9, nb)[:11], synth.permutation(10, rows)[:11]
+    for mode in (ops.MEAN_F32, ops.MEAN_BF16_ROUND, ops.MEAN_F32 | ops.MEAN_ABS):
+        repre = torch.full((n_layers, rows, row), 7.0, device=dev)
+        ops.block_mean(lp, i32(ids, dev), i32(slots, dev), repre, bs, hkv, d, nb, mode=mode)
+        got = repre.cpu().numpy()
+        for l in range(n_layers):
+            want = np.full((rows, row), 7.0, np.float32)
+            keys = caches_h[l] & np.uint16(0x7fff) if mode & ops.MEAN_ABS else caches_h[l]
+            O.block_mean_paged(keys, ids, slots, want, round_bf16=(mode == ops.MEAN_BF16_ROUND), keys_f16=True)
+            assert np.array_equal(bits(got[l]), bits(want)), (mode, l)
+    with pytest.raises(ops.UcmHipError):
+        ops.block_mean(lp, i32(ids, dev), i32(slots, dev), torch.zeros((n_layers, rows, row), dtype=torch.bfloat16, device=dev),
+                       bs, hkv, d, nb)
+
+
 def test_block_mean_skips_bad_ids_and_layer_range(ucm, dev):
     from ucm_amd import ops
 

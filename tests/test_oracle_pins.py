@@ -472,6 +472,39 @@ def test_block_mean_bf16_rounding_mode():
     assert np.mean(rounded == once) > 0.99
 
 
+def test_block_mean_of_fp16_keys():
+    """The fp16-cache variant: numpy's own float16 -> float32 widening, fp32 adds in token order written out as a loop,
+    * (1/T); rounded once to float16 by numpy in the rounding mode.  Also through the C-ABI twin with its key-type flag."""
+    import ctypes as C
+
+    rng = np.random.default_rng(801)
+    keys = (rng.standard_normal((5, 16, 2, 8)) * 3).astype(np.float16)
+    keys[0, 3, 1, 2], keys[1, 0, 0, 0] = np.float16(6.1e-5), np.float16(-65504.0)     # a subnormal-range and the largest value
+    cache = keys.view(np.uint16)
+    ids, slots = [3, 0, 1], [1, 2, 0]
+    plain, rounded = np.zeros((3, 16), np.float32), np.zeros((3, 16), np.float32)
+    O.block_mean_paged(cache, ids, slots, plain, keys_f16=True)
+    O.block_mean_paged(cache, ids, slots, rounded, round_bf16=True, keys_f16=True)
+    for b, s in zip(ids, slots):
+        acc = keys[b, 0].astype(np.float32).reshape(-1)
+        for t in range(1, 16):
+            acc = acc + keys[b, t].astype(np.float32).reshape(-1)
+        want = acc * np.float32(1.0 / 16)
+        assert np.array_equal(bits(plain[s]), bits(want))
+        assert np.array_equal(bits(rounded[s]), bits(want.astype(np.float16).astype(np.float32)))
+    # the twin: flag 8 selects the fp16 reading, mode 1 the rounding, mode 2 (a bf16 table) is not offered
+    lib = C.CDLL(O._ORC_PATH)
+    layers = (C.c_void_p * 1)(cache.ctypes.data)
+    ids_a, slots_a = np.array(ids, np.int32), np.array(slots, np.int32)
+    for mode, want in ((8, plain), (9, rounded)):
+        out = np.zeros((3, 16), np.float32)
+        rc = lib.ucm_block_mean_cpu(layers, 1, 5, ids_a.ctypes.data_as(C.c_void_p), slots_a.ctypes.data_as(C.c_void_p), 3, 16, 2, 8,
+                                    out.ctypes.data_as(C.c_void_p), 3, C.c_int64(48), mode, None)
+        assert rc == 0 and np.array_equal(bits(out), bits(want))
+    assert lib.ucm_block_mean_cpu(layers, 1, 5, ids_a.ctypes.data_as(C.c_void_p), slots_a.ctypes.data_as(C.c_void_p), 3, 16, 2, 8,
+                                  out.ctypes.data_as(C.c_void_p), 3, C.c_int64(48), 10, None) == -95
+
+
 def test_hash_colsum_closed_form():
     rng = np.random.default_rng(22)
     for n, t, h, nb in [(3, 128, 8, 16), (2, 7, 1, 3), (1, 1, 2, 1), (4, 64, 4, 16)]:

@@ -11,6 +11,7 @@ OK, EINVAL, ENOTSUP, EHIP, ENOMEM = 0, -22, -95, -5, -12
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 MEAN_F32, MEAN_BF16_ROUND, MEAN_BF16_STORE = 0, 1, 2
 MEAN_ABS = 4        # or-ed to a mode: the mean of the absolute values
+MEAN_KEYS_F16 = 8   # or-ed to MEAN_F32 / MEAN_BF16_ROUND: fp16 key cache; the rounding is then to fp16
 
 _p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
 

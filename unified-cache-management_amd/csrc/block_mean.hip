@@ -3,7 +3,7 @@
 // whole columns and the order inside a column is the reference's).
 //
 // HBM-bound: block_size*row*2 bytes read per block, row*4 written.  A token
-// row of the key cache ([kv_heads][head_dim] bf16) is contiguous, so a thread
+// row of the key cache ([kv_heads][head_dim] bf16, or fp16 for a model that runs in float16) is contiguous, so a thread
 // owns 8 adjacent columns (one 16-byte load per token) and a workgroup of 128
 // threads covers 1024 columns = one whole Llama-shape row; the token loop is
 // unrolled 16 deep so 16 x 2 KiB of loads are in flight per workgroup.
@@ -29,11 +29,33 @@ __device__ __forceinline__ float round_bf16(float x)
     return __uint_as_float(u & 0xffff0000u);
 }
 
-// kAbs: the absolute values (a bf16 pair loses its two sign bits with one AND)
-template <bool kAbs>
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// fp32 -> fp16 -> fp32, the fp32 value rounded once more.  The value is made opaque first: handed a product, the
+// compiler otherwise folds the multiplication into a mixed-precision instruction that rounds the exact product
+// straight to fp16 - one rounding instead of the two the reference's arithmetic has (seen at a tie: 1/5 of a sum).
+__device__ __forceinline__ float round_f16(float x)
+{
+    asm volatile("" : "+v"(x));
+    return static_cast<float>(static_cast<_Float16>(x));
+}
+
+// kAbs: the absolute values (a pair of 16-bit floats of either kind loses its two sign bits with one AND);
+// kF16: the cache holds fp16 keys, not bf16 ones
+template <bool kAbs, bool kF16>
 __device__ __forceinline__ void widen(u32x4 v, float (&f)[kCols])
 {
     if (kAbs) { v.x &= 0x7fff7fffu; v.y &= 0x7fff7fffu; v.z &= 0x7fff7fffu; v.w &= 0x7fff7fffu; }
+    if (kF16) {
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const f16x2 p = __builtin_bit_cast(f16x2, w[j]);
+            f[2 * j] = static_cast<float>(p[0]);
+            f[2 * j + 1] = static_cast<float>(p[1]);
+        }
+        return;
+    }
     f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x);
     f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
     f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z);
@@ -41,7 +63,7 @@ __device__ __forceinline__ void widen(u32x4 v, float (&f)[kCols])
 }
 
 // acc += token rows t .. t+kN-1, in that order, all kN loads issued before the first add
-template <int kN, bool kAbs>
+template <int kN, bool kAbs, bool kF16>
 __device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsigned row, unsigned t, float (&acc)[kCols])
 {
     u32x4 v[kN];
@@ -50,7 +72,7 @@ __device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsi
 #pragma unroll
     for (int u = 0; u < kN; ++u) {
         float f[kCols];
-        widen<kAbs>(v[u], f);
+        widen<kAbs, kF16>(v[u], f);
 #pragma unroll
         for (int c = 0; c < kCols; ++c) { acc[c] = acc[c] + f[c]; }
     }
@@ -59,7 +81,7 @@ __device__ __forceinline__ void add_rows(const uint16_t* __restrict__ base, unsi
 // grid: x = block index in the list * col_groups + column group of 1024, y = layer; rows narrower than 1024
 // columns whose thread count divides the workgroup (a tensor-parallel rank's 4, 2 or 1 kv heads of 128) share a
 // workgroup, items_per_group list entries side by side, so that no lane idles
-template <bool kAbs>
+template <bool kAbs, bool kF16>
 __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned repre_rows, unsigned block_size,
@@ -84,22 +106,22 @@ __global__ __launch_bounds__(kThreads) void block_mean_kernel(
     const uint16_t* base = static_cast<const uint16_t*>(k_layers[blockIdx.y]) +
                            static_cast<size_t>(id) * block_size * row + col;
     float acc[kCols];
-    widen<kAbs>(ucm::gload16(base), acc);  // acc = token 0
+    widen<kAbs, kF16>(ucm::gload16(base), acc);  // acc = token 0
 
     unsigned t = 1;
     // full groups of kUnroll tokens: loads first, then the ordered adds; what is left (all of a 16-token block
     // after its first token) goes in groups of 8, 4, 2 and 1, each with its loads issued together
-    for (; t + kUnroll <= block_size; t += kUnroll) { add_rows<kUnroll, kAbs>(base, row, t, acc); }
-    if (t + 8 <= block_size) { add_rows<8, kAbs>(base, row, t, acc); t += 8; }
-    if (t + 4 <= block_size) { add_rows<4, kAbs>(base, row, t, acc); t += 4; }
-    if (t + 2 <= block_size) { add_rows<2, kAbs>(base, row, t, acc); t += 2; }
-    if (t < block_size) { add_rows<1, kAbs>(base, row, t, acc); }
+    for (; t + kUnroll <= block_size; t += kUnroll) { add_rows<kUnroll, kAbs, kF16>(base, row, t, acc); }
+    if (t + 8 <= block_size) { add_rows<8, kAbs, kF16>(base, row, t, acc); t += 8; }
+    if (t + 4 <= block_size) { add_rows<4, kAbs, kF16>(base, row, t, acc); t += 4; }
+    if (t + 2 <= block_size) { add_rows<2, kAbs, kF16>(base, row, t, acc); t += 2; }
+    if (t < block_size) { add_rows<1, kAbs, kF16>(base, row, t, acc); }
 
     const float inv = 1.0f / static_cast<float>(block_size);
 #pragma unroll
     for (int c = 0; c < kCols; ++c) {
         acc[c] = acc[c] * inv;
-        if (round_to_bf16) { acc[c] = round_bf16(acc[c]); }
+        if (round_to_bf16) { acc[c] = kF16 ? round_f16(acc[c]) : round_bf16(acc[c]); }
     }
     if (round_to_bf16 == 2) {
         // bf16 table: the rounded means themselves, 16 bytes per thread
@@ -134,10 +156,12 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
     UCM_REQUIRE(n_layers > 0 && n_layers <= 65535, "ucm_block_mean: n_layers=%d", n_layers);
     UCM_REQUIRE(block_size > 0 && kv_heads > 0 && head_dim > 0 && num_blocks > 0 && repre_rows > 0,
                 "ucm_block_mean: non-positive shape");
-    const bool of_abs = (mode & UCM_MEAN_ABS) != 0;
-    mode &= ~UCM_MEAN_ABS;
+    const bool of_abs = (mode & UCM_MEAN_ABS) != 0, keys_f16 = (mode & UCM_MEAN_KEYS_F16) != 0;
+    mode &= ~(UCM_MEAN_ABS | UCM_MEAN_KEYS_F16);
     UCM_REQUIRE(mode == UCM_MEAN_F32 || mode == UCM_MEAN_BF16_ROUND || mode == UCM_MEAN_BF16_STORE,
                 "ucm_block_mean: mode=%d", mode);
+    UCM_SUPPORTED(!(keys_f16 && mode == UCM_MEAN_BF16_STORE), "ucm_block_mean: no bf16 table from an fp16 key cache "
+                  "(UCM_MEAN_F32 or UCM_MEAN_BF16_ROUND, which then rounds to fp16)");
     const unsigned row = static_cast<unsigned>(kv_heads) * static_cast<unsigned>(head_dim);
     UCM_SUPPORTED(row % kCols == 0, "ucm_block_mean: kv_heads*head_dim=%u must be a multiple of %d", row, kCols);
     UCM_REQUIRE(repre_layer_stride >= static_cast<int64_t>(repre_rows) * row || n_layers == 1,
@@ -153,8 +177,14 @@ extern "C" int ucm_block_mean(const void* const* k_layers, int n_layers, int num
 #define UCM_BLOCK_MEAN_ARGS dim3(groups, n_layers), dim3(kThreads), 0, ucm::as_stream(stream), k_layers, block_ids, slots, \
         static_cast<unsigned>(num_blocks), static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size), row,       \
         static_cast<float*>(repre), repre_layer_stride, mode, gx, share, static_cast<unsigned>(n)
-    if (of_abs) { hipLaunchKernelGGL(block_mean_kernel<true>, UCM_BLOCK_MEAN_ARGS); }
-    else { hipLaunchKernelGGL(block_mean_kernel<false>, UCM_BLOCK_MEAN_ARGS); }
+    if (keys_f16) {
+        if (of_abs) { hipLaunchKernelGGL((block_mean_kernel<true, true>), UCM_BLOCK_MEAN_ARGS); }
+        else { hipLaunchKernelGGL((block_mean_kernel<false, true>), UCM_BLOCK_MEAN_ARGS); }
+    } else if (of_abs) {
+        hipLaunchKernelGGL((block_mean_kernel<true, false>), UCM_BLOCK_MEAN_ARGS);
+    } else {
+        hipLaunchKernelGGL((block_mean_kernel<false, false>), UCM_BLOCK_MEAN_ARGS);
+    }
 #undef UCM_BLOCK_MEAN_ARGS
     UCM_LAUNCH_CHECK("ucm_block_mean");
 }

@@ -12,7 +12,7 @@ from typing import Optional, Sequence
 import torch
 
 from . import _lib
-from ._lib import MEAN_ABS, MEAN_BF16_ROUND, MEAN_BF16_STORE, MEAN_F32, UcmHipError  # noqa: F401
+from ._lib import MEAN_ABS, MEAN_BF16_ROUND, MEAN_BF16_STORE, MEAN_F32, MEAN_KEYS_F16, UcmHipError  # noqa: F401
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -114,13 +114,19 @@ class LayerPointers:
         return self.table.data_ptr() + 8 * first_layer
 
 
+def _bf16_keys_only(layers: LayerPointers, what: str) -> None:
+    if layers.tensors and layers.tensors[0].dtype == torch.float16:
+        raise ValueError(f"{what} reads bfloat16 key caches only (a float16 cache is taken by block_mean and the scoring calls)")
+
+
 def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                block_size: int, kv_heads: int, head_dim: int, num_blocks: int, mode: int = MEAN_F32,
                first_layer: int = 0, n_layers: Optional[int] = None) -> None:
     """repre: [L, rows, kv_heads*head_dim], fp32 (mode MEAN_F32 / MEAN_BF16_ROUND) or
     bf16 (the mode is then MEAN_BF16_STORE whatever was passed); rows ``slots`` of layers
     first_layer.. are overwritten with the means of cache blocks ``block_ids`` (``mode | MEAN_ABS``: of their
-    absolute values)."""
+    absolute values).  The caches behind ``k_layers`` are bfloat16 or float16; with float16 ones MEAN_BF16_ROUND rounds
+    to float16 (the cache's type) and a bfloat16 table is refused."""
     if repre.dim() != 3 or repre.shape[2] != kv_heads * head_dim:
         raise ValueError("repre must be [layers, rows, kv_heads*head_dim]")
     n_layers = len(k_layers) - first_layer if n_layers is None else n_layers
@@ -131,7 +137,9 @@ def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Te
     if repre.dtype not in (torch.float32, torch.bfloat16):
         raise ValueError("repre must be float32 or bfloat16")
     of_abs = mode & MEAN_ABS
-    mode &= ~MEAN_ABS
+    mode &= ~(MEAN_ABS | MEAN_KEYS_F16)
+    if k_layers.tensors[first_layer].dtype == torch.float16:
+        of_abs |= MEAN_KEYS_F16
     if repre.dtype == torch.bfloat16:
         mode = MEAN_BF16_STORE
     elif mode == MEAN_BF16_STORE:
@@ -439,6 +447,7 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
     """w bf16 [128, 128]; colsum int16 [L, rows, kv_heads, 128]; block_codes uint8 [L, rows, kv_heads, 16];
     token_codes uint8 [L, rows, block_size, kv_heads, 16] or None; workgroups: persistent workgroups over all
     layers, 0 = the library's choice (benchmarks and tests)."""
+    _bf16_keys_only(k_layers, "hash_encode_blocks")
     if w.shape != (128, 128):
         raise ValueError("w must be [128, 128] bfloat16")
     n_layers, rows = colsum.shape[0], colsum.shape[1]
@@ -590,6 +599,7 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
     """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); pruned int32 [kv_heads, d_pruned] (one set of
     channel lists for every layer), [L, kv_heads, d_pruned] (lists per layer) or None.  With pruned_sel (int32 [n]:
     the list each listed block is pruned by) pruned is [n_lists, kv_heads, d_pruned] or [L, n_lists, kv_heads, d_pruned]."""
+    _bf16_keys_only(k_layers, "kvstar_block_repre")
     if repre.dim() != 6 or repre.dtype != torch.float16 or repre.shape[4] * merge != block_size or \
             repre.shape[1] != kv_heads or repre.shape[5] != 8:
         raise ValueError("repre must be float16 [L, kv_heads, rows, d_pad/8, block_size/merge, 8]")

@@ -321,6 +321,8 @@ class GSA(UcmSparseBase):
         if known is kv_cache or (known is not None and isinstance(kv_cache, torch.Tensor) and isinstance(known, torch.Tensor)
                                  and known.data_ptr() == kv_cache.data_ptr()):
             return
+        if kv_cache[0].dtype == torch.float16 and self.repre_dtype == torch.bfloat16:
+            raise ValueError("a float16 KV cache needs repre_dtype float32: the bfloat16 table holds the means of a bfloat16 model")
         self.k_cache[layer_id], self.v_cache[layer_id] = kv_cache[0], kv_cache[1]
         self._layer_ptrs[layer_id] = ops.LayerPointers([kv_cache[0]])
         self._kv_full[layer_id] = kv_cache
