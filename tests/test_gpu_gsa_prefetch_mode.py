@@ -51,21 +51,24 @@ def test_gsa_prefetch_mode_flow(ucm, dev, stride):
     fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
 
     perm = [int(x) for x in synth.permutation(960, nb)]
-    pool_free = perm[150:]                              # blocks the scheduler hands out during decode
-    # A: 40 full blocks + 5 tokens; B: exactly 35 blocks (its first decoded token opens a block); C: short, never sparse
-    shapes = {"A": (41, 40 * bs + 5), "B": (35, 35 * bs), "C": (4, 60)}
+    pool_free = perm[200:]                              # blocks the scheduler hands out during decode
+    # A: 40 full blocks + 5 tokens; B: exactly 35 blocks (its first decoded token opens a block) - it ends after engine
+    # step 25; C: short, never sparse; D: 38 blocks + 9 tokens, arrives at engine step 10, while the others decode
+    shapes = {"A": (41, 40 * bs + 5), "B": (35, 35 * bs), "C": (4, 60), "D": (39, 38 * bs + 9)}
+    arrive, leave = {"A": 0, "B": 0, "C": 0, "D": 10}, {"B": 25}
     reqs, models, at = {}, {}, 0
     for rid, (n_blocks, n_tok) in shapes.items():
         ids = perm[at : at + n_blocks]
         at += n_blocks
         reqs[rid] = ns(block_ids=[list(ids)], num_computed_tokens=0, prompt_token_ids=[1] * n_tok, output_token_ids=[])
         models[rid] = Model(rid, ids, n_tok, L)
-    order = ["A", "B", "C"]
-    ib = ns(req_id_to_index={r: i for i, r in enumerate(order)})
-    truth = {rid: [dict() for _ in range(L)] for rid in order}     # per layer {logical block: its K and V}
+    truth = {rid: [dict() for _ in range(L)] for rid in shapes}    # per layer {logical block: its K and V}
+    tokens = {r: 0 for r in shapes}                                 # tokens in the sequence so far
+    k_of = lambda n: topk_len(n, lo, hi)
 
-    def run_step(n_tokens, new=()):
-        so = ns(num_scheduled_tokens=dict(n_tokens), scheduled_new_reqs=[ns(req_id=r) for r in new])
+    def run_step(order, n_tokens, new=()):
+        so = ns(num_scheduled_tokens={r: n_tokens[r] for r in order}, scheduled_new_reqs=[ns(req_id=r) for r in new])
+        ib = ns(req_id_to_index={r: i for i, r in enumerate(order)})
         starts = np.concatenate([[0], np.cumsum([n_tokens[r] for r in order])])
         md = ns(query_start_loc=torch.tensor(starts), block_table=None, seq_lens=None)
         fc.attn_metadata = md
@@ -84,9 +87,9 @@ def test_gsa_prefetch_mode_flow(ucm, dev, stride):
             reqs[r].num_computed_tokens += n_tokens[r]
         return seen
 
-    # ---- prefill: representatives, every full block to the store, the local windows aside
-    run_step({r: shapes[r][1] for r in order}, new=order)
-    for rid in order:
+    def after_prefill(rid):
+        """Every full block is in the store; then the scheduler's part (GSA.allocate_slots): a long request keeps its
+        first sparse_len blocks, the rest is somebody else's."""
         m = models[rid]
         n_full = shapes[rid][1] // bs
         for j in range(len(m.prompt_ids)):
@@ -94,20 +97,17 @@ def test_gsa_prefetch_mode_flow(ucm, dev, stride):
                 truth[rid][l][j] = caches[l][:, m.prompt_ids[j]].clone()
         assert all(store.lookup([f"req_{rid}_blk_{j}"]) == [True] for j in range(n_full))
         assert f"req_{rid}_blk_{n_full}" not in store.slot_of
-
-    # ---- first decode step: the scheduler keeps the first sparse_len blocks of a long request (GSA.allocate_slots)
-    k_of = lambda n: topk_len(n, lo, hi)
-    for rid in ("A", "B"):
-        m = models[rid]
+        tokens[rid] = shapes[rid][1]
+        if shapes[rid][1] <= 100:
+            return
         n_p = len(m.prompt_ids)
         k = k_of(n_p)
         sparse_len = k + (0 if k > hi else hi - k + 1)
         released = m.prompt_ids[sparse_len:]
         m.phys = m.prompt_ids[:sparse_len]
-        m.sparse, m.sparse_len, m.n_p = True, sparse_len, n_p
-        for l in range(L):                              # what was released is somebody else's now
+        m.sparse, m.n_p = True, n_p
+        for l in range(L):
             caches[l][:, released] = 7.0
-    tokens = {r: shapes[r][1] for r in order}             # tokens in the sequence so far
 
     def grow(rid):
         """The scheduler's part of a decode step: a block for the token if it opens one."""
@@ -133,25 +133,48 @@ def test_gsa_prefetch_mode_flow(ucm, dev, stride):
             assert torch.equal(caches[l][:, b], truth[m.rid][l][j]), (step, l, m.rid, b, j)
 
     pf = None
-    space = 0
-    rounds = n_loaded = 0
-    for step in range(1, 40):
-        grown = {}
+    space = rounds = n_loaded = 0
+    decoded = {r: 0 for r in shapes}                                # decode steps a request has taken
+    live = []
+    for step in range(0, 40):
+        for rid in [r for r in live if leave.get(r, 99) < step]:
+            plugin.request_finished_in_worker(rid)
+            live.remove(rid)
+            assert rid not in pf.engine_id and rid not in pf.ready
+        new = [r for r in shapes if arrive[r] == step]
+        live += new
+        order = list(live)
+        n_tokens, grown = {}, {}
         for rid in order:
+            if rid in new:
+                n_tokens[rid] = shapes[rid][1]
+                continue
             grown[rid] = grow(rid)
             tokens[rid] += 1
+            decoded[rid] += 1
             reqs[rid].output_token_ids.append(1)
             reqs[rid].block_ids = [list(models[rid].phys)]
-        seen = run_step({r: 1 for r in order})
+            n_tokens[rid] = 1
+        seen = run_step(order, n_tokens, new)
+        for rid in new:
+            after_prefill(rid)
+        if step == 0:
+            assert all(t is None for t, _ in seen)                   # nobody decodes: the layer's metadata is left alone
+            continue
         pf = plugin._pf
         round_now = space >= stride - 1
         space = 0 if round_now else space + 1
         # ---- replay: first deal, lengths, growth
-        for i, rid in enumerate(order):
+        for rid in order:
             m = models[rid]
-            seq = tokens[rid]
-            slot = seq % bs
-            if step == 1:
+            if rid in new:                                          # a prefill step: its own blocks, its real length
+                m.use = [list(m.prompt_ids) for _ in range(L)]
+                m.succ = None
+                m.seq_want = [shapes[rid][1]] * L
+                m.to_map, m.to_table = [], []
+                continue
+            slot = tokens[rid] % bs
+            if decoded[rid] == 1:
                 if m.sparse:
                     n_p, k = m.n_p, k_of(m.n_p)
                     idx = list(range(hi + 1)) if k <= hi else list(range(k))
@@ -188,13 +211,15 @@ def test_gsa_prefetch_mode_flow(ucm, dev, stride):
                 assert int(lens[i]) == m.seq_want[l], (step, l, rid)
                 n = len(m.use[l])
                 assert table[i, :n].tolist() == m.use[l], (step, l, rid)
-                if m.sparse and not round_now:
+                if m.sparse and rid not in new and not round_now:
                     holds_what_the_maps_say(step, l, m)
         # ---- the round at the end of the step
         if round_now:
             rounds += 1
             for i, rid in enumerate(order):
                 m = models[rid]
+                if rid in new:
+                    continue                                        # (its rows are set up again at its first decode step)
                 m.use, m.succ = m.succ, m.use
                 for j, b in m.to_map:
                     if m.sparse:
@@ -231,11 +256,13 @@ def test_gsa_prefetch_mode_flow(ucm, dev, stride):
                     assert pf.use_table[l, row, : len(m.use[l])].tolist() == m.use[l] and int(pf.use_len[l, row]) == len(m.use[l])
                     holds_what_the_maps_say(step, l, m)
             got = pf.engine.obtain_blocks_map()
-            for rid in ("A", "B"):
-                for l in range(L):
-                    assert got[pf.engine_id[rid]][l] == models[rid].map[l], (step, l, rid)
+            for rid in order:
+                if models[rid].sparse and rid not in new:
+                    for l in range(L):
+                        assert got[pf.engine_id[rid]][l] == models[rid].map[l], (step, l, rid)
     assert rounds == pf.rounds and rounds >= 39 // stride - 1
     assert plugin.load_misses == 0 and n_loaded > 0
-    for rid in order:
+    assert sorted(live) == ["A", "C", "D"] and decoded["D"] == 29
+    for rid in live:
         plugin.request_finished_in_worker(rid)
     assert not pf.engine_id and not pf.ready
