@@ -903,8 +903,8 @@ def main():
             p_free_len[:, r] = len(spare)
             resident_h.append((holder, logical, [st_.blocks[x] for x in spare]))
         pool = torch.empty((rows, n_layers, 2, BLOCK_BYTES), dtype=torch.uint8, device=dev)
-        for l0 in range(0, rows, 256):
-            pool[l0 : l0 + 256].random_(generator=p_gen)
+        for l0 in range(0, rows, 256):                      # stored blocks are K and V values like the caches' (the loads
+            pool[l0 : l0 + 256].view(torch.bfloat16).normal_(generator=p_gen)       # write them into the caches later legs read)
         src_table = torch.full((N_REQ, max_len), -1, dtype=torch.int32, device=dev)
         for r in range(N_REQ):
             src_table[eng.row_of(r), : lens[r]] = torch.arange(int(seg_off_h[r]), int(seg_off_h[r] + lens[r]), dtype=torch.int32, device=dev)
@@ -1009,8 +1009,10 @@ def main():
 
         block_lists = [[int(x) for x in bt_h[r, : lens[r]]] for r in range(N_REQ)]
         del staging
+        gc.collect()
         torch.cuda.empty_cache()
-        plugin_leg = {"note": "hooks driven by stand-in objects for vLLM's (plugin_bench.py), 16 requests x "
+        plugin_leg = {"device_memory_free_GB": round(torch.cuda.mem_get_info(dev)[0] / 1e9, 1),
+                      "note": "hooks driven by stand-in objects for vLLM's (plugin_bench.py), 16 requests x "
                               f"{n_layers} layers; host_us = the hooks' time on the model-runner thread, wall_us = until the "
                               "device has finished what they queued (no model runs in between); medians per kind of step"}
         for name, leg in (("GSA", lambda: plugin_bench.gsa_leg(torch, dev, caches, lens, block_lists, args.steps, args.seed)),

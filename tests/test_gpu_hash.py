@@ -410,3 +410,77 @@ def test_hash_encode_projections_built_to_cancel(ucm, dev, paired):
     assert np.array_equal(tcodes[0].cpu().numpy(), want)
     assert np.array_equal(colsum[0].cpu().numpy(), O.hash_colsum(want))
     assert np.array_equal(bcodes[0].cpu().numpy(), O.hash_majority(want))
+
+
+def test_hash_encode_keys_beyond_the_fp32_range(ucm, dev):
+    """Keys whose fp32 sums overflow on the way (components up to 3e38: the exact sum may be finite and of either
+    sign where the matrix cores hold an infinity or a NaN), keys with infinite components and keys with NaN: the
+    codes are still the signs of the sums accumulated exactly, d ascending (NaN is not > 0: bit 0), because a key
+    without a finite error bound has all its results redone."""
+    from ucm_amd import ops
+
+    hkv, bs, nb = 8, 128, 6
+    w_bits, w_f32 = make_weights(890)
+    rng = np.random.default_rng(891)
+    keys_h = synth.normal_bf16_bits(892, (nb, bs, hkv, 128))
+    raw = rng.integers(0, 1 << 16, size=(bs, hkv, 128), dtype=np.uint16)
+    keys_h[0] = raw                                                    # any bit pattern: NaN, infinities, 1e38 next to 1e-38
+    finite = raw.copy()
+    finite[(finite & 0x7F80) == 0x7F80] &= 0xFF7F                      # exponent 255 -> 254: the same without NaN and infinity
+    keys_h[1] = finite
+    huge = synth.bf16_round_bits((rng.standard_normal((bs, hkv, 128)) * 1e38).clip(-3e38, 3e38).astype(np.float32))
+    keys_h[2] = huge                                                   # every partial sum is out of range
+    keys_h[3, ::3, :, 17] = 0x7F80                                     # one +inf in otherwise ordinary keys
+    keys_h[3, 1::3, :, 40] = 0xFF80                                    # ... or +inf and -inf
+    keys_h[3, 1::3, :, 90] = 0x7F80
+    keys_h[4, ::2, :, 5] = 0x7FC0                                      # one NaN
+    keys_h[5, :, ::2, 0] = synth.bf16_round_bits(np.array([2.5e38], np.float32))[0]    # one component that alone overflows
+    lp = ops.LayerPointers([bf16_dev(keys_h, dev)])
+    colsum = torch.zeros((1, nb, hkv, 128), dtype=torch.int16, device=dev)
+    bcodes = torch.zeros((1, nb, hkv, 16), dtype=torch.uint8, device=dev)
+    tcodes = torch.zeros((1, nb, bs, hkv, 16), dtype=torch.uint8, device=dev)
+    ops.hash_encode_blocks(lp, None, None, nb, bf16_dev(w_bits, dev), bs, hkv, nb, colsum, bcodes, token_codes=tcodes)
+    torch.cuda.synchronize()
+    with np.errstate(all="ignore"):
+        want = O.hash_encode(keys_h, w_f32)
+    # the cases are what they claim to be: fp32 sums of block 2 are not finite, its exact sums have both signs
+    x2 = synth.bf16_widen(huge).reshape(-1, 128)
+    with np.errstate(all="ignore"):
+        assert not np.isfinite(x2 @ w_f32).any()
+    assert 0.3 < np.unpackbits(want[2]).mean() < 0.7
+    assert not want[4, ::2].any() and want[4, 1::2].any()
+    got = tcodes[0].cpu().numpy()
+    for b in range(nb):
+        assert np.array_equal(got[b], want[b]), b
+    assert np.array_equal(colsum[0].cpu().numpy(), O.hash_colsum(want))
+    assert np.array_equal(bcodes[0].cpu().numpy(), O.hash_majority(want))
+    # the summaries alone (no token codes) take the same path
+    colsum2, bcodes2 = torch.zeros_like(colsum), torch.zeros_like(bcodes)
+    ops.hash_encode_blocks(lp, None, None, nb, bf16_dev(w_bits, dev), bs, hkv, nb, colsum2, bcodes2)
+    assert torch.equal(colsum2, colsum) and torch.equal(bcodes2, bcodes)
+
+
+def test_hash_query_codes_beyond_the_fp32_range(ucm, dev):
+    """Query rows with components up to 3e38 (one head per kv head, so that the group mean is the row itself): a
+    tile whose largest norm is not finite is redone whole, the signs are those of the exact sums."""
+    from ucm_amd import ops
+
+    hq = hkv = 8
+    n_layers, n_req = 1, 4
+    w_bits, w_f32 = make_weights(895)
+    rng = np.random.default_rng(896)
+    q_h = synth.normal_bf16_bits(897, (n_layers, n_req, hq, 128))
+    q_h[0, 1] = synth.bf16_round_bits((rng.standard_normal((hq, 128)) * 1e38).clip(-3e38, 3e38).astype(np.float32))
+    q_h[0, 2, ::2] = q_h[0, 1, ::2]                                    # huge rows next to ordinary ones
+    q_h[0, 3, :, 9] = synth.bf16_round_bits(np.array([2.5e38], np.float32))[0]
+    q_codes = torch.full((n_layers, n_req, hq, 16), 0xEE, dtype=torch.uint8, device=dev)
+    q_sum = torch.full((n_layers, n_req, 128), 77, dtype=torch.int16, device=dev)
+    qbar = torch.full((n_layers, n_req, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(bf16_dev(q_h, dev), bf16_dev(w_bits, dev), hkv, q_codes, q_sum, qbar, n_req)
+    torch.cuda.synchronize()
+    want_q = O.hash_encode(q_h[0], w_f32)
+    assert 0.3 < np.unpackbits(want_q[1]).mean() < 0.7
+    assert np.array_equal(q_codes[0].cpu().numpy(), want_q)
+    pm = np.unpackbits(want_q, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
+    assert np.array_equal(q_sum[0].cpu().numpy(), pm.sum(1))
+    assert np.array_equal(qbar[0].cpu().numpy(), want_q)               # a group of one head: the mean is the row

@@ -472,13 +472,16 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
 #pragma unroll
                 for (int sub = 1; sub >= 0; --sub) {
                     const int nb = 2 * wp + sub;
-                    float mn = __builtin_inff();
+                    // (the minimum starts at the largest finite value and the test is "not at or above", so that a
+                    // bound of infinity or NaN - a key with a component beyond 1e19, infinite or NaN, whose sums
+                    // may have overflowed on the way - flags the column block whatever the results are)
+                    float mn = 0x1.fffffep+127f;
 #pragma unroll
                     for (int i = 15; i >= 0; --i) {
                         wbits = __builtin_amdgcn_alignbit(wbits, __float_as_uint(acc[nb][i]), 31);
                         mn = __builtin_fminf(mn, __builtin_fabsf(acc[nb][i]));
                     }
-                    doubt[nb] = __ballot(mn < sw[nb] * sx);
+                    doubt[nb] = __ballot(!(mn >= sw[nb] * sx));
                 }
                 pair[wp] = wbits;
             }
@@ -514,6 +517,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
                         for (int i = 15; i >= 0; --i) {
                             mask = __builtin_amdgcn_alignbit(mask, __float_as_uint(__builtin_fabsf(acc[nb][i]) - bound), 31);
                         }
+                        if (!(bound < __builtin_inff())) { mask = 0xffffu; }    // no finite bound: all sixteen are redone
                         const unsigned signs = pair[nb >> 1] >> (16 * (nb & 1));
                         unsigned long long um = __ballot(mask != 0u);
                         while (um) {
@@ -766,7 +770,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         }
         nx2 += __shfl_xor(nx2, 32, 64);
         const float max2 = wave_max32(nx2);
-        const bool all_exact = max2 > 0.0f && !(max2 >= 0x1p-120f);
+        const bool all_exact = (max2 > 0.0f && !(max2 >= 0x1p-120f)) || !(max2 < __builtin_inff());   // tiny norms, or none that is finite
         const float bound = sqrtf(kTau2 * max2) * sqrtf(nw2) * 1.01f;
         f32x16 acc;
 #pragma unroll
@@ -821,7 +825,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
                                                           acc, 0, 0, 0);
         }
         const float max2 = fmaxf(s.mean_max2[0], s.mean_max2[1]);
-        const bool all_exact = max2 > 0.0f && !(max2 >= 0x1p-120f);
+        const bool all_exact = (max2 > 0.0f && !(max2 >= 0x1p-120f)) || !(max2 < __builtin_inff());   // tiny norms, or none that is finite
         const float bound = sqrtf(kTau2 * max2) * sqrtf(nw2) * 1.01f;
         unsigned positive = 0, redo = 0;
 #pragma unroll
