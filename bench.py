@@ -1016,6 +1016,7 @@ def main():
                               f"{n_layers} layers; host_us = the hooks' time on the model-runner thread, wall_us = until the "
                               "device has finished what they queued (no model runs in between); medians per kind of step"}
         for name, leg in (("GSA", lambda: plugin_bench.gsa_leg(torch, dev, caches, lens, block_lists, args.steps, args.seed)),
+                          ("GSA, retrieval_lag 1", lambda: plugin_bench.gsa_leg(torch, dev, caches, lens, block_lists, args.steps, args.seed, 1)),
                           ("ESA", lambda: plugin_bench.esa_leg(torch, dev, caches, lens, block_lists, args.seed)),
                           ("KvComp", lambda: plugin_bench.kvcomp_leg(torch, dev, caches, lens, block_lists, args.seed)),
                           ("KVStar", lambda: plugin_bench.kvstar_leg(torch, dev, caches, lens, block_lists, args.seed))):

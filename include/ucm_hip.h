@@ -638,6 +638,19 @@ int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t 
                    ucm_stream_t stream);
 
 /*
+ * Rows of one array copied into rows of another: dst[dst_idx[i]] <- src[src_idx[i]],
+ * i < n, `row_bytes` each.  This is copy_q of the reference's GSA
+ * (ucm/sparse/gsa/gsa.py:616-632, `gsa_q_cache[layer][:len(ids)].copy_(query[ids])`):
+ * the last query token of every request of a layer kept for the selection that
+ * the next step applies.  src is [src_rows][row_bytes], dst [dst_rows][row_bytes],
+ * both dev and 16-byte aligned, row_bytes a multiple of 16; src_idx dev int32[n];
+ * dst_idx dev int32[n] or NULL (row i).  A pair with either index outside its
+ * array is skipped.  Destination rows named twice get one of the sources.
+ */
+int ucm_park_rows(const void* src, int64_t src_rows, const int32_t* src_idx, void* dst, int64_t dst_rows,
+                  const int32_t* dst_idx, int n, size_t row_bytes, ucm_stream_t stream);
+
+/*
  * Transfer device of the store layer: the HIP counterpart of the reference's
  * IDevice (ucm/store/device/idevice.h:33-58) as implemented by CudaDevice on
  * the buffered base (ucm/store/device/cuda/cuda_device.cu:107-227,

@@ -52,6 +52,7 @@ TWIN(ucm_kvstar_block_repre);
 TWIN(ucm_kvstar_votes);
 TWIN(ucm_kvstar_votes_tables);
 TWIN(ucm_kvstar_park_queries);
+TWIN(ucm_park_rows);
 
 /* the oracle's functions these forward to (ucm_oracle.c) */
 float orc_bf16_to_f32(uint16_t h);
@@ -654,6 +655,21 @@ int ucm_copy_batch_cpu(void* const* dst, const void* const* src, size_t num, siz
         if (!dst[i] || !src[i] || ((uintptr_t)dst[i] | (uintptr_t)src[i]) % 16) { return UCM_EINVAL; }
     }
     for (size_t i = 0; i < num; ++i) { memmove(dst[i], src[i], size); }
+    return UCM_OK;
+}
+
+int ucm_park_rows_cpu(const void* src, int64_t src_rows, const int32_t* src_idx, void* dst, int64_t dst_rows,
+                      const int32_t* dst_idx, int n, size_t row_bytes, ucm_stream_t stream)
+{
+    (void)stream;
+    if (n < 0 || src_rows < 0 || dst_rows < 0 || row_bytes == 0 || row_bytes % 16) { return UCM_EINVAL; }
+    if (n == 0) { return UCM_OK; }
+    if (!src || !src_idx || !dst || ((uintptr_t)src | (uintptr_t)dst) % 16) { return UCM_EINVAL; }
+    for (int i = 0; i < n; ++i) {
+        const int64_t from = src_idx[i], to = dst_idx ? dst_idx[i] : i;
+        if (from < 0 || from >= src_rows || to < 0 || to >= dst_rows) { continue; }
+        memmove((char*)dst + (size_t)to * row_bytes, (const char*)src + (size_t)from * row_bytes, row_bytes);
+    }
     return UCM_OK;
 }
 

@@ -131,14 +131,15 @@ def _prompt_shape(lens):
     return [int(n - 1) * BS + 40 for n in lens]
 
 
-def gsa_leg(torch, dev, caches, lens, block_tables, steps: int, seed: int) -> dict:
+def gsa_leg(torch, dev, caches, lens, block_tables, steps: int, seed: int, lag: int = 0) -> dict:
     """GSA: every decode step scores all blocks of every request and swaps each layer's block table and sequence
-    lengths for the sparse ones (one library call per layer)."""
+    lengths for the sparse ones - one library call per layer with the layer's own queries (lag 0), or the layer's
+    hook only keeps the queries and the next step scores every layer in one launch before its model runs (lag 1)."""
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.gsa.gsa import GSA
 
     n_layers = len(caches)
-    cfg = make_config(n_layers, 65536, len(lens), "GSA", {"seg_prefill_threshold": 0, "repre_dtype": "bfloat16"})
+    cfg = make_config(n_layers, 65536, len(lens), "GSA", {"seg_prefill_threshold": 0, "repre_dtype": "bfloat16", "retrieval_lag": lag})
     plugin = GSA(cfg, UcmSparseRole.WORKER)
 
     def wave(w: int) -> dict:

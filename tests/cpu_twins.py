@@ -15,7 +15,7 @@ TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_se
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
-         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries"]
+         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries", "ucm_park_rows"]
 
 
 def twin_caller(signatures):
@@ -571,6 +571,17 @@ def run_kvstar(call, side):
         side.sync()
         out[name] = ring
     x["park_q"] = qf
+    # rows of one array into rows of another (a step's query rows kept for the next step's selection): out of order,
+    # a source row past the array, a negative one, a destination past the array; with and without destination indices
+    rows_src = side.up(np.arange(7 * 48, dtype=np.int32).reshape(7, 48))
+    pick = side.up(np.array([6, 0, 7, 3, -1, 2], np.int32))
+    put = side.up(np.array([1, 4, 0, 5, 2, 9], np.int32))
+    for name, where in (("rows_indexed", put), ("rows_in_order", None)):
+        rows_dst = side.up(np.full((6, 48), -5, np.int32))
+        call("ucm_park_rows", side.ptr(rows_src), 7, side.ptr(pick), side.ptr(rows_dst), 6, None if where is None else side.ptr(where),
+             6, 48 * 4, None)
+        side.sync()
+        out[name] = rows_dst
     side.sync()
     return {k: (v if isinstance(v, np.ndarray) else np.array(side.down(v))) for k, v in out.items()}, x
 

@@ -250,6 +250,14 @@ def test_kvstar_twins_reproduce_the_oracle(ucm):
             want16[d_] = O.bf16_to_f32(O.bf16_bits(qf[s_])).astype(np.float16).view(np.uint16)
         assert np.array_equal(got["park_bf16"], want16)
         assert np.array_equal(got["park_f16"][[0, 2, 1, 4]], qf[[5, 0, 3, 1]].astype(np.float16).view(np.uint16))
+    # rows moved by index: pairs (6 -> 1), (0 -> 4), (3 -> 5) land, the rest name a row outside an array
+    src_rows = np.arange(7 * 48, dtype=np.int32).reshape(7, 48)
+    want_rows = np.full((6, 48), -5, np.int32)
+    want_rows[[1, 4, 5]] = src_rows[[6, 0, 3]]
+    assert np.array_equal(got["rows_indexed"], want_rows)
+    want_rows = np.full((6, 48), -5, np.int32)
+    want_rows[[0, 1, 3, 5]] = src_rows[[6, 0, 3, 2]]
+    assert np.array_equal(got["rows_in_order"], want_rows)
     # a task whose query block, channel list or rows lie outside what the call declares is skipped: its votes keep
     # the fill value, the other tasks' are unchanged
     a0, n0, a2, n2 = K.K_OFF[0], K.K_LEN[0], K.K_OFF[2], K.K_LEN[2]

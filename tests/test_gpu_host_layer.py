@@ -196,12 +196,15 @@ def topk_len(n, lo, hi):
     return min(lo, n) if t < lo else min(t, hi)
 
 
-@pytest.mark.parametrize("repre_dtype,model", [("float32", "bfloat16"), ("bfloat16", "bfloat16"), ("float32", "float16")])
-def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
+@pytest.mark.parametrize("repre_dtype,model,lag", [("float32", "bfloat16", 0), ("bfloat16", "bfloat16", 0), ("float32", "float16", 0),
+                                                   ("bfloat16", "bfloat16", 1), ("float32", "float16", 1)])
+def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model, lag):
     """Two requests through prefill and 40 decode steps, two layers: after every attention_begin the
     layer's block table and sequence lengths must be what the oracle selects from the same cache.
     With a bfloat16 table the representatives are the rounded means of the live reference path; a model that runs
-    in float16 (cache, keys and queries) goes through the same hooks with an fp32 table."""
+    in float16 (cache, keys and queries) goes through the same hooks with an fp32 table.  With retrieval_lag 1 a
+    step's selection comes from the queries of the step before (the request's first sparsified step apart), scored
+    over the table and the block lists of the step that uses it, in one launch before the first layer runs."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.gsa.gsa import GSA
@@ -210,7 +213,7 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
     hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 120
     lo, hi = 6, 10
     cfg = make_config(hq, hkv, d, L, bs, 16 * 60, {"seg_prefill_threshold": 100, "min_topk_len": lo, "max_topk_len": hi,
-                                                   "repre_dtype": repre_dtype})
+                                                   "repre_dtype": repre_dtype, "retrieval_lag": lag})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     assert isinstance(plugin, GSA)
     assert plugin.repre_dtype == getattr(torch, repre_dtype)   # the table itself is allocated at the first step
@@ -229,6 +232,8 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
     repre_h = {r: [np.zeros((60, hkv * d), np.float32) for _ in range(L)] for r in prompts}
     done_blocks = {r: 0 for r in prompts}
     saw_sparse = 0
+    q_before = [None] * L                    # request A's query of the step before, per layer
+    lagged_steps = 0
 
     for step in range(41):
         sched = {}
@@ -249,6 +254,9 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
             bt[i, : len(reqs[r].block_ids[0])] = torch.tensor(reqs[r].block_ids[0], dtype=torch.int32)
         plugin.build_sparse_meta(so, reqs, ib, None)
         plugin.execute_begin(so)
+        # with the lag, every step after the first sparsified one has its selection before the model runs
+        assert (plugin._lagged is not None) == (lag == 1 and step >= 2)
+        lagged_steps += int(plugin._lagged is not None)
         for l in range(L):
             md = ns(block_table=bt.clone(), seq_lens=torch.tensor(seq_lens, dtype=torch.int32, device=dev))
             fc.attn_metadata = {names[l]: md}
@@ -268,6 +276,10 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
                 nA = len(reqs["A"].block_ids[0])
                 k = topk_len(nA, lo, hi)
                 qA = query[0].float().cpu().numpy()  # A's only (= last) token is row 0 of the batch
+                if lag and step >= 2:
+                    qA, q_before[l] = q_before[l], qA
+                else:
+                    q_before[l] = qA
                 want_idx, _ = O.select_topk(qA, repre_h["A"][l][:nA].reshape(nA, hkv, 1, d), k)
                 phys, want_len = O.block_table_gather(reqs["A"].block_ids[0], want_idx, seq_lens[0], bs)
                 got_bt, got_len = md.block_table.cpu().numpy(), md.seq_lens.cpu().numpy()
@@ -301,6 +313,7 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model):
             st.num_computed_tokens += sched[r]
             st.output_token_ids.append(7)
     assert saw_sparse >= 2 * 39  # every decode step of every layer really dropped blocks
+    assert lagged_steps == (39 if lag else 0)
     plugin.request_finished_in_worker("A")
     assert "A" not in plugin.gsa_stats and not plugin.topk_kpre_manger.is_exist("A")
 

@@ -959,7 +959,7 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     # KVStar: the tables bit for bit; the votes to rounding (the matrix cores sum in another order than the scalar loop)
     want, _ = cpu_twins.run_kvstar(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
     got, _ = cpu_twins.run_kvstar(_lib.call, cpu_twins.DeviceSide(ops, dev))
-    for name in ("table_full", "table_pruned", "table_by_block", "park_f32", "park_bf16", "park_f16"):
+    for name in ("table_full", "table_pruned", "table_by_block", "park_f32", "park_bf16", "park_f16", "rows_indexed", "rows_in_order"):
         assert np.array_equal(got[name], want[name]), name
     for name in ("votes", "votes_tables", "votes_bad0", "votes_bad1", "votes_bad2"):
         assert np.allclose(got[name], want[name], rtol=2e-4, atol=2e-6), name

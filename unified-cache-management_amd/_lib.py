@@ -42,6 +42,7 @@ SIGNATURES = {
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_score_blocks": [_i, _p, _p, _p, _i64, _p, _i64, _i64, _p, _p, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
     "ucm_copy_batch": [_p, _p, _sz, _sz, _p],
+    "ucm_park_rows": [_p, _i64, _p, _p, _i64, _p, _i, _sz, _p],
     "ucm_kernel_can_access": [_p, _sz],
     "ucm_device_create": [_i, _sz, _sz, _p],
     "ucm_device_destroy": [_p],

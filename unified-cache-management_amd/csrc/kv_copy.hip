@@ -241,6 +241,34 @@ int stored_layout(const char* name, size_t block_bytes, int rank, int tp_size, S
     return UCM_OK;
 }
 
+// dst row dst_idx[i] = src row src_idx[i]: one 256-thread workgroup per pair (a step's query rows are a few KiB each,
+// so the launch is all latency: every thread has its loads in flight before its first store)
+constexpr int kRowThreads = 256;
+
+__global__ __launch_bounds__(kRowThreads) void park_rows_kernel(const uint8_t* __restrict__ src, long long src_rows,
+                                                                const int32_t* __restrict__ src_idx, uint8_t* __restrict__ dst,
+                                                                long long dst_rows, const int32_t* __restrict__ dst_idx,
+                                                                size_t row_bytes)
+{
+    const long long from = src_idx[blockIdx.x], to = dst_idx ? dst_idx[blockIdx.x] : static_cast<long long>(blockIdx.x);
+    if (from < 0 || from >= src_rows || to < 0 || to >= dst_rows) { return; }
+    const uint8_t* s = src + static_cast<size_t>(from) * row_bytes;
+    uint8_t* d = dst + static_cast<size_t>(to) * row_bytes;
+    for (size_t o = threadIdx.x * 16u; o < row_bytes; o += static_cast<size_t>(kRowThreads) * 16 * 4) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t at = o + static_cast<size_t>(u) * kRowThreads * 16;
+            if (at < row_bytes) { v[u] = ucm::gload16(s + at); }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const size_t at = o + static_cast<size_t>(u) * kRowThreads * 16;
+            if (at < row_bytes) { ucm::gstore16(d + at, v[u]); }
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int ucm_copy_batch(void* const* dst, const void* const* src, size_t num, size_t size,
@@ -383,4 +411,19 @@ extern "C" int ucm_kv_load_planned(void* const* layers, int n_layers, size_t kv_
     return ucm_kv_load_planned_tp(layers, n_layers, kv_stride, block_bytes, num_blocks, pool, pool_blocks, pool_block_bytes,
                                   store_first_layer, load_sel, n_slots, src_table, src_stride, dst_table, dst_stride,
                                   dst_layer_stride, load_count, rows, batch, table_rows, 0, 1, stream);
+}
+
+extern "C" int ucm_park_rows(const void* src, int64_t src_rows, const int32_t* src_idx, void* dst, int64_t dst_rows,
+                             const int32_t* dst_idx, int n, size_t row_bytes, ucm_stream_t stream)
+{
+    UCM_REQUIRE(n >= 0 && src_rows >= 0 && dst_rows >= 0, "ucm_park_rows: n=%d src_rows=%lld dst_rows=%lld", n,
+                static_cast<long long>(src_rows), static_cast<long long>(dst_rows));
+    UCM_REQUIRE(row_bytes > 0 && row_bytes % 16 == 0, "ucm_park_rows: row_bytes=%zu must be a positive multiple of 16", row_bytes);
+    if (n == 0) { return UCM_OK; }
+    UCM_REQUIRE(src && src_idx && dst, "ucm_park_rows: null pointer");
+    UCM_REQUIRE(ucm::aligned16(src) && ucm::aligned16(dst), "ucm_park_rows: src and dst must be 16-byte aligned");
+    hipLaunchKernelGGL(park_rows_kernel, dim3(static_cast<unsigned>(n)), dim3(kRowThreads), 0, ucm::as_stream(stream),
+                       static_cast<const uint8_t*>(src), static_cast<long long>(src_rows), src_idx, static_cast<uint8_t*>(dst),
+                       static_cast<long long>(dst_rows), dst_idx, row_bytes);
+    UCM_LAUNCH_CHECK("ucm_park_rows");
 }

@@ -502,6 +502,21 @@ def copy_batch(dst_ptrs: torch.Tensor, src_ptrs: torch.Tensor, size: int) -> Non
               dst_ptrs.numel(), size, _stream())
 
 
+def park_rows(src: torch.Tensor, src_idx: torch.Tensor, dst: torch.Tensor, dst_idx: Optional[torch.Tensor] = None) -> None:
+    """dst[dst_idx[i]] = src[src_idx[i]] for 2-D (or flattened to rows) contiguous device tensors of one dtype and row
+    size; dst_idx None: row i.  Pairs with an index outside its tensor are skipped."""
+    if src.dtype != dst.dtype or not (src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()):
+        raise ValueError("src and dst must be contiguous device tensors of one dtype")
+    if src.dim() < 2 or dst.dim() < 2 or src.shape[1:] != dst.shape[1:]:
+        raise ValueError("src and dst must be arrays of rows of one shape")
+    n = src_idx.numel()
+    if dst_idx is not None and dst_idx.numel() != n:
+        raise ValueError("index arrays differ in length")
+    row_bytes = src[0].numel() * src.element_size()
+    _lib.call("ucm_park_rows", src.data_ptr(), src.shape[0], _dev(src_idx, torch.int32, "src_idx"), dst.data_ptr(),
+              dst.shape[0], _opt(dst_idx, torch.int32, "dst_idx"), n, row_bytes, _stream())
+
+
 def _staging_ptr(staging: torch.Tensor, need: int) -> int:
     if not (staging.is_cuda or staging.is_pinned()):
         raise ValueError("staging must be device or pinned host memory")

@@ -234,6 +234,14 @@ class GSA(UcmSparseBase):
         self.ptopk_prefetch = bool(cfg.get("ptopk_prefetch_enable", False))
         self.prefetch_stride = max(1, int(cfg.get("prefetch_stride", 6)))   # steps between two rounds of the prefetch engine
         self._pf = None                   # prefetch mode's tables and engine (prefetch_mode.py), built with the device state
+        # 0: a layer's blocks are scored with the layer's own queries just before its attention (one launch per layer).
+        # 1: the reference's timing - a layer's hook only keeps the step's last query tokens (copy_q, gsa.py:616-632) and
+        # the step after scores every layer with them in ONE launch before the model runs, as the reference's block
+        # tables of a step come from queries of an earlier one (gsa.py:672-679); a request's first sparsified step
+        # still scores layer by layer.  Prefetch mode keeps its own timing (its rounds read the step's selection).
+        self.retrieval_lag = int(cfg.get("retrieval_lag", 0))
+        if self.retrieval_lag not in (0, 1):
+            raise ValueError("retrieval_lag must be 0 (same step) or 1 (the step after)")
         self.repre_dtype = torch.bfloat16 if cfg.get("repre_dtype", "float32") == "bfloat16" else torch.float32
         self.repre_mode = ops.MEAN_BF16_STORE if self.repre_dtype == torch.bfloat16 else ops.MEAN_F32
 
@@ -254,6 +262,10 @@ class GSA(UcmSparseBase):
         self._seen_layers = None          # the engine's table of layers once every layer's cache has been registered from it
         self._tables_signature = None     # (request, blocks, last block) per batch slot of the block tables on the device
         self._tables_dev: Optional[torch.Tensor] = None
+        self.q_stage: Optional[torch.Tensor] = None   # retrieval_lag 1: [layers, table partitions, q_heads, head_size], the kept queries
+        self._parked: set = set()         # requests whose queries of the step before are in q_stage, every layer
+        self._parking: Optional[tuple] = None   # this step keeps its queries: (requests, source rows, partitions, n)
+        self._lagged: Optional[list] = None     # this step's selection was made in execute_begin: per-layer views
 
     # ------------------------------------------------------------------ device state
     def _ensure_device_state(self, device) -> None:
@@ -271,7 +283,7 @@ class GSA(UcmSparseBase):
         self.topk_counts = torch.zeros((L, self.max_bs), dtype=torch.int32, device=device)
         self.gsa_seq_len = torch.zeros((L, self.max_bs), dtype=torch.int32, device=device)
         # two pinned staging buffers for the per-step descriptors, used alternately
-        cap = (5 + 3 * self.max_block_len) * self.max_bs
+        cap = (6 + 3 * self.max_block_len) * self.max_bs
         self._host_desc = [torch.zeros(cap, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self._host_free = [None, None]  # event recorded after each buffer's last upload
         # attention_begin runs once per layer and decode step: it goes to the library with addresses computed
@@ -298,6 +310,11 @@ class GSA(UcmSparseBase):
             block_size=self.block_size, tickets=self.tickets.data_ptr(),
             idx_layer_stride=self.topk_caches.stride(0), count_layer_stride=self.topk_counts.stride(0))
         self._sel_addr = ctypes.addressof(self._sel)
+        # retrieval_lag 1: the same call over every layer at once, its queries the kept ones
+        self._sel_all = _lib.ScoreSelectArgs()
+        ctypes.memmove(ctypes.addressof(self._sel_all), self._sel_addr, ctypes.sizeof(self._sel))
+        self._sel_all.first_layer, self._sel_all.n_layers = 0, L
+        self._park_rows = _lib.lib().ucm_park_rows
         self._score_select = _lib.lib().ucm_score_select
         self._fused_ok = self.max_block_len <= 1024     # longer requests take the two launches
         self._dev_ready = True
@@ -425,7 +442,7 @@ class GSA(UcmSparseBase):
         if any_gsa and self.ptopk_prefetch and self._dev_ready and self._prefetch_mode().round_due():
             is_topk = True                # the round at the end of this step reads this step's selection
         self.model_input["is_topk"] = is_topk
-        self._fast = None
+        self._fast = self._lagged = self._parking = None
         if is_topk:
             self._scored |= gsa_ids
         if not any_gsa or not self._dev_ready:
@@ -433,7 +450,7 @@ class GSA(UcmSparseBase):
         width = self.max_block_len
         n_calc = len(self.model_input["calc_block_table"])
         # The block tables go down only when a request's list changed or the batch was reordered (a decoding
-        # request's list grows by one entry every block_size steps); the five descriptor rows and the block-mean
+        # request's list grows by one entry every block_size steps); the six descriptor rows and the block-mean
         # lists go down every step.  One int32 host buffer, one copy.
         signature = tuple((st.serial, st.blocks_version) if st is not None else None for st in by_index)
         tables_known = signature == self._tables_signature
@@ -441,47 +458,47 @@ class GSA(UcmSparseBase):
         if self._host_free[slot] is not None:
             self._host_free[slot].synchronize()  # upload of two steps ago; long finished
         n_tables = 0 if tables_known else batch * width
-        host = self._host_desc[slot][: 5 * batch + n_tables + 2 * n_calc]
+        host = self._host_desc[slot][: 6 * batch + n_tables + 2 * n_calc]
         hn = host.numpy()                    # the same pinned memory; numpy fills it several times faster than torch indexing
-        desc = hn[: 5 * batch].reshape(5, batch)
+        desc = hn[: 6 * batch].reshape(6, batch)
         if not tables_known:
-            tables = hn[5 * batch : 5 * batch + n_tables].reshape(batch, width)
+            tables = hn[6 * batch : 6 * batch + n_tables].reshape(batch, width)
             tables[:] = 0
         max_len = total = 0
         query_locals = self.model_input["query_locals"]
-        rows = []                            # per request: first table row, blocks, k, its last query token, tokens so far
+        rows = []                            # per request: first table row, blocks, k, its last query token, tokens so far, table partition
         min_topk, max_topk, ratio = self.min_topk, self.max_topk, self.topk_ratio
         for i, st in enumerate(by_index):
             if st is None:
-                rows.append((0, 0, 0, 0, 0))
+                rows.append((0, 0, 0, 0, 0, -1))
                 continue
             n = len(st.blocks)
             # k >= n keeps every block (short or prefilling requests)
             k = compute_topk_len(n, min_topk, max_topk, ratio) if st.is_gsa() else n
             rows.append((st.slot_offset, n, k if k > 1 else 1, query_locals[i + 1] - 1,
-                         st.num_computed_tokens + st.num_scheduled_tokens))
+                         st.num_computed_tokens + st.num_scheduled_tokens, st.slot_offset // width))
             if not tables_known:
                 tables[i, :n] = st.blocks
             if n > max_len:
                 max_len = n
             total += n
         desc[:] = np.array(rows, dtype=np.int32).T
-        tail = hn[5 * batch + n_tables :]
+        tail = hn[6 * batch + n_tables :]
         tail[:n_calc] = self.model_input["calc_block_table"]
         tail[n_calc:] = self.model_input["calc_repre_slot_mapping"]
         dev = host.to(self.device, non_blocking=True)
         if self._host_free[slot] is None:
             self._host_free[slot] = torch.cuda.Event()
         self._host_free[slot].record()
-        d = dev[: 5 * batch].view(5, batch)
+        d = dev[: 6 * batch].view(6, batch)
         if not tables_known:
-            self._tables_dev = dev[5 * batch : 5 * batch + n_tables].view(batch, width)
+            self._tables_dev = dev[6 * batch : 6 * batch + n_tables].view(batch, width)
             self._tables_signature = signature
         self.model_input.update(
             seg_off=d[0], seg_len=d[1], topk_len=d[2], q_rows=d[3], seq_lens=d[4],
             block_tables=self._tables_dev,
-            calc_blocks_dev=dev[5 * batch + n_tables : 5 * batch + n_tables + n_calc],
-            calc_slots_dev=dev[5 * batch + n_tables + n_calc :],
+            calc_blocks_dev=dev[6 * batch + n_tables : 6 * batch + n_tables + n_calc],
+            calc_slots_dev=dev[6 * batch + n_tables + n_calc :],
             max_len=max_len, total=total, n_batch=batch,
         )
         base = d.data_ptr()
@@ -490,10 +507,24 @@ class GSA(UcmSparseBase):
         a = self._sel
         a.seg_off, a.seg_len, a.topk_len, a.q_rows, a.seq_lens, a.block_tables = self.model_input["addr"]
         a.n_req, a.max_seg_len, a.total_blocks = batch, max_len, total
+        lag = self.retrieval_lag and not self.ptopk_prefetch and self._fused_ok and _raw_stream is not None
+        if lag and (self.retrieval_stride == 1 or (self.step_count + 1) % self.retrieval_stride == 0):
+            # the step after may select with this step's queries: every layer keeps them
+            self._parking = ({st.req_id for st in by_index if st is not None}, base + 12 * batch, base + 20 * batch, batch)
         if self.ptopk_prefetch:
             # attention reads the engine's tables; the selection is kept as logical block numbers for the next round
             a.block_tables = a.phys_out = a.sparse_seq_lens = None
             self._prefetch_mode().begin_step(by_index)
+        elif lag and is_topk and self.q_stage is not None and gsa_ids <= self._parked:
+            # every sparsified request's queries of the step before are at hand: one launch for all layers, now
+            b = self._sel_all
+            b.seg_off, b.seg_len, b.topk_len, b.seq_lens, b.block_tables = a.seg_off, a.seg_len, a.topk_len, a.seq_lens, a.block_tables
+            b.q_rows = base + 20 * batch
+            b.n_req, b.max_seg_len, b.total_blocks = batch, max_len, total
+            rc = self._score_select(ctypes.addressof(b), _raw_stream(self._dev_index))
+            if rc != 0:
+                raise _lib.UcmHipError("ucm_score_select", rc, _lib.lib().ucm_last_error().decode())
+            self._lagged = self._batch_views(batch)
         elif is_topk and self._fused_ok and _raw_stream is not None:
             self._fast = self._batch_views(batch)
 
@@ -509,6 +540,8 @@ class GSA(UcmSparseBase):
             self._gsa_sparse_local_kv()
             if self._pf is not None:
                 self._pf.end_step()
+        self._parked = self._parking[0] if self._parking is not None else set()
+        self._parking = None
         self.step_count += 1
 
     # ------------------------------------------------------------------ per-layer hooks
@@ -526,6 +559,25 @@ class GSA(UcmSparseBase):
             self.maybe_register_kv_cache(forward_context, layer_name)
             if len(self._kv_full) == self.layer_num:
                 self._seen_layers = layers
+        parking = self._parking
+        if parking is not None:
+            # the last query token of every request goes to the request's row of the kept queries of this layer
+            # (copy_q, gsa.py:616-632), for the selection the next step makes before its model runs
+            l = self._layer_of[layer_name]
+            if self.q_stage is None:
+                self._make_stage(query)
+            if query.dtype is not self._stage_dtype or query.shape[1:] != self._stage_row or not query.is_contiguous():
+                raise ValueError("query must be a contiguous device tensor [tokens, q_heads, head_size] of the type the first step had")
+            rc = self._park_rows(query.data_ptr(), query.shape[0], parking[1], self._stage_addr[l], self.max_bs, parking[2],
+                                 parking[3], self._stage_row_bytes, _raw_stream(self._dev_index))
+            if rc != 0:
+                raise _lib.UcmHipError("ucm_park_rows", rc, _lib.lib().ucm_last_error().decode())
+        if self._lagged is not None:
+            md = forward_context.attn_metadata
+            if isinstance(md, dict):
+                md = md[layer_name]
+            md.block_table, md.seq_lens = self._lagged[self._layer_of[layer_name]]
+            return
         fast = self._fast
         if fast is not None:
             # the step scores and selects with the one-launch call: everything but the layer and its queries was
@@ -585,6 +637,18 @@ class GSA(UcmSparseBase):
         else:
             md.block_table, md.seq_lens = self._batch_views(n)[l]
 
+    def _make_stage(self, query) -> None:
+        """The kept queries [layers, table partitions, q_heads, head_size], in the type of the model's queries."""
+        if _Q_CODES.get(query.dtype) is None:
+            raise ValueError("query must be bfloat16, float16 or float32")
+        stage = self.q_stage = torch.zeros((self.layer_num, self.max_bs, self.num_q_heads, self.head_size),
+                                           dtype=query.dtype, device=self.device)
+        b = self._sel_all
+        b.q, b.q_dtype, b.q_layer_stride = stage.data_ptr(), _Q_CODES[query.dtype], stage.stride(0)
+        self._stage_dtype, self._stage_row = query.dtype, stage.shape[2:]
+        self._stage_row_bytes = stage.stride(1) * stage.element_size()
+        self._stage_addr = [stage[l].data_ptr() for l in range(self.layer_num)]
+
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
         # (the layer's cache was looked at in attention_begin of the same step)
         if self.model_input.get("calc_block_table"):
@@ -613,6 +677,7 @@ class GSA(UcmSparseBase):
         self.topk_kpre_manger.free(request_id)
         self.gsa_stats.pop(request_id, None)
         self._scored.discard(request_id)
+        self._parked.discard(request_id)
         if self._pf is not None:
             self._pf.request_finished(request_id)
 
