@@ -539,6 +539,16 @@ int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_bl
                            int d_pruned, int d_pad, void* repre_f16, int repre_rows,
                            int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
                            ucm_stream_t stream);
+/* The same for a cache of key_dtype UCM_DTYPE_BF16 (what ucm_kvstar_block_repre takes) or UCM_DTYPE_F16: a float16
+ * model's means are rounded once, to float16 (the .mean(dim=2) in the model's type, ucm/sparse/kvstar/multistep.py:310-314;
+ * the .to(torch.float16) that follows, :494-499, then changes nothing). */
+int ucm_kvstar_block_repre_keys(const void* const* k_layers, int key_dtype, int n_layers, int num_blocks,
+                                const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                                int kv_heads, int head_dim, int merge, const int32_t* pruned,
+                                int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
+                                int d_pruned, int d_pad, void* repre_f16, int repre_rows,
+                                int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
+                                ucm_stream_t stream);
 /*
  * The query tokens a step contributes to its requests' retrieval groups, copied aside as fp16 - save_to_standby
  * (ucm/sparse/kvstar/multistep.py:318-324, one clone per request and layer) together with the .to(float16) of

@@ -81,6 +81,8 @@ _orc_f16_to_f32 = _sig(_orc, "orc_f16_to_f32", _f32, C.c_uint16)
 _orc_f32_to_f16 = _sig(_orc, "orc_f32_to_f16", C.c_uint16, _f32)
 _orc_kvstar_block_repre = _sig(_orc, "orc_kvstar_block_repre", None, _p, _p, _p, _u32, _u32, _u32, _u32, _u32, _p, _u32,
                                _u32, _p)
+_orc_kvstar_block_repre_f16 = _sig(_orc, "orc_kvstar_block_repre_f16", None, _p, _p, _p, _u32, _u32, _u32, _u32, _u32, _p, _u32,
+                                   _u32, _p)
 _orc_kvstar_retrieve = _sig(_orc, "orc_kvstar_retrieve", _i32, _p, _u32, _u32, _u32, _p, _u32, _u32, _u32, _u32, _u32, _p,
                             _u32, _p, _p)
 _orc_f32_to_bf16 = _sig(_orc, "orc_f32_to_bf16", C.c_uint16, _f32)
@@ -314,8 +316,9 @@ def f32_to_f16(f: float) -> int:
     return int(_orc_f32_to_f16(float(f)))
 
 
-def kvstar_block_repre(cache_bits: np.ndarray, block_ids, slots, merge: int, repre: np.ndarray, pruned=None) -> None:
-    """cache_bits uint16 [num_blocks, block_size, kv_heads, head_dim] (bf16); repre uint16 (fp16)
+def kvstar_block_repre(cache_bits: np.ndarray, block_ids, slots, merge: int, repre: np.ndarray, pruned=None,
+                       keys_f16: bool = False) -> None:
+    """cache_bits uint16 [num_blocks, block_size, kv_heads, head_dim] (bf16, or fp16 with keys_f16); repre uint16 (fp16)
     [rows, M, kv_heads, d_pad], rows ``slots`` are overwritten; pruned int32 [kv_heads, d_pruned] or None."""
     cb = _c(cache_bits, np.uint16)
     _, bs, h, d = cb.shape
@@ -323,8 +326,8 @@ def kvstar_block_repre(cache_bits: np.ndarray, block_ids, slots, merge: int, rep
     assert repre.dtype == np.uint16 and repre.flags.c_contiguous and repre.shape[1] == bs // merge and repre.shape[2] == h
     pr = None if pruned is None else _c(pruned, np.int32)
     dp = d if pr is None else pr.shape[1]
-    _orc_kvstar_block_repre(_ptr(cb), _ptr(ids), _ptr(sl), len(ids), bs, h, d, merge, None if pr is None else _ptr(pr),
-                            dp, repre.shape[3], _ptr(repre))
+    fn = _orc_kvstar_block_repre_f16 if keys_f16 else _orc_kvstar_block_repre
+    fn(_ptr(cb), _ptr(ids), _ptr(sl), len(ids), bs, h, d, merge, None if pr is None else _ptr(pr), dp, repre.shape[3], _ptr(repre))
 
 
 def kvstar_retrieve(q_bits: np.ndarray, repre: np.ndarray, topk: int, pruned=None, d_pruned: int | None = None):

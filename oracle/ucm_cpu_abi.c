@@ -49,6 +49,7 @@ TWIN(ucm_kvstar_topk);
 TWIN(ucm_kvstar_order);
 TWIN(ucm_prefetch_plan);
 TWIN(ucm_kvstar_block_repre);
+TWIN(ucm_kvstar_block_repre_keys);
 TWIN(ucm_kvstar_votes);
 TWIN(ucm_kvstar_votes_tables);
 TWIN(ucm_kvstar_park_queries);
@@ -82,6 +83,9 @@ void orc_hash_scores_block(const uint8_t* q_codes, const uint8_t* block_codes, u
 float orc_f16_to_f32(uint16_t h);
 int32_t orc_kvstar_topk(const float* final_scores, uint32_t n_blocks, uint32_t topk, int32_t* topk_idx);
 void orc_kvstar_block_repre(const uint16_t* cache, const int32_t* block_ids, const int32_t* slots, uint32_t n, uint32_t block_size,
+                            uint32_t kv_heads, uint32_t head_dim, uint32_t merge, const int32_t* pruned, uint32_t d_pruned,
+                            uint32_t d_pad, uint16_t* repre);
+void orc_kvstar_block_repre_f16(const uint16_t* cache, const int32_t* block_ids, const int32_t* slots, uint32_t n, uint32_t block_size,
                             uint32_t kv_heads, uint32_t head_dim, uint32_t merge, const int32_t* pruned, uint32_t d_pruned,
                             uint32_t d_pad, uint16_t* repre);
 int32_t orc_kvstar_retrieve(const uint16_t* q, uint32_t n_tokens, uint32_t q_heads, uint32_t d_orig, const uint16_t* repre,
@@ -866,7 +870,20 @@ int ucm_kvstar_block_repre_cpu(const void* const* k_layers, int n_layers, int nu
                                int d_pruned, int d_pad, void* repre_f16, int repre_rows, int64_t repre_layer_stride,
                                int64_t repre_head_stride, int64_t repre_row_stride, ucm_stream_t stream)
 {
+    return ucm_kvstar_block_repre_keys_cpu(k_layers, UCM_DTYPE_BF16, n_layers, num_blocks, block_ids, slots, n, block_size, kv_heads,
+                                           head_dim, merge, pruned, pruned_layer_stride, pruned_sel, n_pruned_lists, d_pruned, d_pad,
+                                           repre_f16, repre_rows, repre_layer_stride, repre_head_stride, repre_row_stride, stream);
+}
+
+int ucm_kvstar_block_repre_keys_cpu(const void* const* k_layers, int key_dtype, int n_layers, int num_blocks,
+                                    const int32_t* block_ids, const int32_t* slots, int n, int block_size, int kv_heads,
+                                    int head_dim, int merge, const int32_t* pruned, int64_t pruned_layer_stride,
+                                    const int32_t* pruned_sel, int n_pruned_lists, int d_pruned, int d_pad, void* repre_f16,
+                                    int repre_rows, int64_t repre_layer_stride, int64_t repre_head_stride,
+                                    int64_t repre_row_stride, ucm_stream_t stream)
+{
     (void)stream;
+    if (key_dtype != UCM_DTYPE_BF16 && key_dtype != UCM_DTYPE_F16) { return UCM_EINVAL; }
     if (n < 0 || n_layers < 0 || (pruned_sel && (!pruned || n_pruned_lists < 1))) { return UCM_EINVAL; }
     if (n == 0 || n_layers == 0) { return UCM_OK; }
     if (!k_layers || !repre_f16 || num_blocks <= 0 || repre_rows <= 0 || block_size <= 0 || kv_heads <= 0 || head_dim <= 0 ||
@@ -886,8 +903,9 @@ int ucm_kvstar_block_repre_cpu(const void* const* k_layers, int n_layers, int nu
             if (id < 0 || id >= num_blocks || slot < 0 || slot >= repre_rows) { continue; }
             if (pruned_sel && (pruned_sel[i] < 0 || pruned_sel[i] >= n_pruned_lists)) { continue; }   /* a list that does not exist */
             const int32_t* mine = (lists && pruned_sel) ? lists + (size_t)pruned_sel[i] * kv_heads * d_pruned : lists;
-            orc_kvstar_block_repre((const uint16_t*)k_layers[l], &id, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads,
-                                   (uint32_t)head_dim, (uint32_t)merge, mine, (uint32_t)d_pruned, (uint32_t)d_pad, tmp);
+            (key_dtype == UCM_DTYPE_F16 ? orc_kvstar_block_repre_f16 : orc_kvstar_block_repre)(
+                (const uint16_t*)k_layers[l], &id, &zero, 1, (uint32_t)block_size, (uint32_t)kv_heads, (uint32_t)head_dim,
+                (uint32_t)merge, mine, (uint32_t)d_pruned, (uint32_t)d_pad, tmp);
             for (int h = 0; h < kv_heads; ++h) {
                 uint16_t* cell = (uint16_t*)repre_f16 + (int64_t)l * repre_layer_stride + (int64_t)h * repre_head_stride +
                                  (int64_t)slot * repre_row_stride;

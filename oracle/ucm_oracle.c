@@ -821,6 +821,38 @@ ORC_API void orc_kvstar_block_repre(const uint16_t* cache, const int32_t* block_
     }
 }
 
+/* The same for a float16 cache: the sums are the same fp32 sums of the (exactly widened) keys, the mean is rounded
+ * once, to float16 - .mean() in a float16 model (multistep.py:310-314); the .to(torch.float16) that follows is then
+ * the identity. */
+ORC_API void orc_kvstar_block_repre_f16(const uint16_t* cache, const int32_t* block_ids, const int32_t* slots, uint32_t n,
+                                        uint32_t block_size, uint32_t kv_heads, uint32_t head_dim, uint32_t merge,
+                                        const int32_t* pruned, uint32_t d_pruned, uint32_t d_pad, uint16_t* repre)
+{
+    const uint32_t M = block_size / merge;
+    const float inv = 1.0f / (float)merge;
+    for (uint32_t i = 0; i < n; ++i) {
+        const uint16_t* blk = cache + (size_t)block_ids[i] * block_size * kv_heads * head_dim;
+        uint16_t* out = repre + (size_t)slots[i] * M * kv_heads * d_pad;
+        for (uint32_t m = 0; m < M; ++m) {
+            for (uint32_t h = 0; h < kv_heads; ++h) {
+                for (uint32_t p = 0; p < d_pad; ++p) {
+                    uint16_t v = 0;
+                    if (p < d_pruned) {
+                        const uint32_t d = pruned ? (uint32_t)pruned[h * d_pruned + p] : p;
+                        float acc = orc_f16_to_f32(blk[((size_t)(m * merge) * kv_heads + h) * head_dim + d]);
+                        for (uint32_t t = 1; t < merge; ++t) {
+                            acc = acc + orc_f16_to_f32(blk[((size_t)(m * merge + t) * kv_heads + h) * head_dim + d]);
+                        }
+                        acc = acc * inv;
+                        v = orc_f32_to_f16(acc);
+                    }
+                    out[((size_t)m * kv_heads + h) * d_pad + p] = v;
+                }
+            }
+        }
+    }
+}
+
 /*
  * The top-k step of KVStar::Execute
  * (ucm/sparse/kvstar/retrieve/core/domain/retrieve_task/simd_compute_kernel.cpp:955-977),

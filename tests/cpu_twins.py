@@ -15,7 +15,7 @@ TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_se
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
-         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries", "ucm_park_rows"]
+         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries", "ucm_park_rows", "ucm_kvstar_block_repre_keys"]
 
 
 def twin_caller(signatures):

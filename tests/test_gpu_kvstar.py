@@ -68,6 +68,39 @@ def test_kvstar_block_repre(ucm, dev, merge, hkv, d, bs):
     assert torch.allclose(mine.float(), t.float(), rtol=2 ** -7, atol=1e-6)
 
 
+@pytest.mark.parametrize("merge,hkv,d,bs", [(2, 8, 128, 128), (4, 2, 64, 32), (16, 4, 128, 128), (3, 2, 64, 48)])
+def test_kvstar_block_repre_of_fp16_keys(ucm, dev, merge, hkv, d, bs):
+    """A float16 model: the cache is float16, the means are rounded once to float16 (merge 3 goes through the kernel
+    for arbitrary sub-block sizes); the result is what torch's mean() gives in float16 up to the order of the sums."""
+    from ucm_amd import ops
+
+    n_layers, nb, rows = 2, 9, 12
+    rng = np.random.default_rng(1090 + merge)
+    caches_h = [(rng.standard_normal((nb, bs, hkv, d)) * rng.choice([1e-3, 1.0, 40.0], size=(nb, 1, 1, d))).astype(np.float16)
+                for _ in range(n_layers)]
+    caches = [torch.from_numpy(c).to(dev) for c in caches_h]
+    lp = ops.LayerPointers(caches)
+    ids = synth.permutation(1091, nb)[:7].astype(np.int32)
+    slots = synth.permutation(1092, rows)[:7].astype(np.int32)
+    M = bs // merge
+    for d_pruned, layout in ((d, "head"), (16, "head"), (d - 8, "row")):
+        pruned = None if d_pruned == d else np.stack([synth.permutation(1093 + h, d)[:d_pruned] for h in range(hkv)]).astype(np.int32)
+        d_pad = (d_pruned + 15) // 16 * 16
+        repre = ops.kvstar_table(n_layers, hkv, rows, M, d_pad, dev, layout).fill_(3.0)
+        ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge,
+                               pruned=None if pruned is None else torch.from_numpy(pruned).to(dev))
+        got = ops.kvstar_table_to_reference(repre).contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+        for l in range(n_layers):
+            want = np.full((rows, M, hkv, d_pad), np.float16(3.0).view(np.uint16), np.uint16)
+            O.kvstar_block_repre(caches_h[l].view(np.uint16), ids, slots, merge, want, pruned=pruned, keys_f16=True)
+            assert np.array_equal(got[l], want), (d_pruned, l)
+    t = caches[0][torch.from_numpy(ids.astype(np.int64)).to(dev)].reshape(7, M, merge, hkv, d).mean(dim=2)
+    repre = ops.kvstar_table(n_layers, hkv, rows, M, d, dev).zero_()
+    ops.kvstar_block_repre(lp, torch.from_numpy(ids).to(dev), torch.from_numpy(slots).to(dev), repre, bs, hkv, d, nb, merge)
+    mine = ops.kvstar_table_to_reference(repre[0])[torch.from_numpy(slots.astype(np.int64)).to(dev)]
+    assert torch.allclose(mine.float(), t.float(), rtol=2 ** -10, atol=1e-6)
+
+
 @pytest.mark.parametrize("merge", [2, 16, 3])      # the persistent kernel, and the one for other sub-block sizes (16 and 3)
 def test_kvstar_block_repre_channel_lists_per_layer(ucm, dev, merge):
     """One launch over all layers with a different set of kept channels in each (the reference picks them per layer

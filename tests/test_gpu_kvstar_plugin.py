@@ -18,19 +18,23 @@ def bits(t):
     return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads,device_plans,hole", [
-    (1.0, 1, True, True, True, False), (0.5, 3, True, False, True, False), (0.25, 1, False, True, True, False),
-    (0.25, 1, True, False, False, False), (0.25, 1, True, True, False, False), (0.5, 3, True, True, True, False),
-    (0.25, 1, True, True, True, True), (0.25, 1, False, True, True, True), (0.25, 1, True, True, False, True),
-    (0.25, 1, True, True, True, "spill"), (0.25, 1, False, True, True, "spill"), (0.25, 1, True, True, False, "spill")])
-def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads, device_plans, hole):
+@pytest.mark.parametrize("prune_ratio,chunks,batched,device_loads,device_plans,hole,model", [
+    (1.0, 1, True, True, True, False, "bfloat16"), (0.5, 3, True, False, True, False, "bfloat16"),
+    (0.25, 1, False, True, True, False, "bfloat16"), (0.25, 1, True, False, False, False, "bfloat16"),
+    (0.25, 1, True, True, False, False, "bfloat16"), (0.5, 3, True, True, True, False, "bfloat16"),
+    (0.25, 1, True, True, True, True, "bfloat16"), (0.25, 1, False, True, True, True, "bfloat16"),
+    (0.25, 1, True, True, False, True, "bfloat16"), (0.25, 1, True, True, True, "spill", "bfloat16"),
+    (0.25, 1, False, True, True, "spill", "bfloat16"), (0.25, 1, True, True, False, "spill", "bfloat16"),
+    (0.25, 1, True, True, True, False, "float16"), (1.0, 3, False, True, True, False, "float16")])
+def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads, device_plans, hole, model):
     """Prefill (one chunk, or three) of 24 full blocks + 5 tokens, then 13 decode steps with stride 4: step 1 restores
     the windows and loads what the prefill group's vote picks; the vote of decode steps 1-4 is queued at step 4 and
     its winners are loaded at step 8; steps 5-8 at step 8 / 12.  Selections are checked against the CPU oracle on the
     same keys and queries.  ``hole``: at the first load the store lacks some of the prompt's blocks - the load leaves them
     out, says so (a warning, a counter) and looks again at the next load, by which time they have arrived.  ``hole ==
     "spill"``: the store's pool is smaller than the prompt and has pinned host memory behind it - the blocks a load may
-    ask for come back into the pool when the request first loads, and stay."""
+    ask for come back into the pool when the request first loads, and stay.  ``model``: the type of the cache and of the
+    queries (a float16 model's representatives are rounded once, to float16)."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvstar.multistep import KVStarMultiStep
@@ -59,7 +63,8 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
              num_prompt_tokens=n_prompt, num_output_tokens=0, num_tokens=n_prompt, request_id="7")
     g = torch.Generator(device=dev)
     g.manual_seed(21)
-    caches = [(torch.randn(2, nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(torch.bfloat16) for _ in range(L)]
+    model = getattr(torch, model)
+    caches = [(torch.randn(2, nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(model) for _ in range(L)]
     original = [c.clone() for c in caches]
     names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
     ib = ns(req_id_to_index={"7": 0})
@@ -71,7 +76,7 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
         plugin.build_sparse_meta(so, {"7": req}, ib, md)
         qs = []
         for l in range(L):
-            q = (torch.randn(n_tok, hq, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+            q = (torch.randn(n_tok, hq, d, device=dev, generator=g) * 0.3).to(model)
             qs.append(q)
             plugin.attention_begin(q, None, None, names[l], fc)
             plugin.attention_finished(q, None, None, None, names[l], fc)
@@ -118,7 +123,7 @@ def test_kvstar_plugin_flow(ucm, dev, prune_ratio, chunks, batched, device_loads
         pr = None if prune_ratio >= 0.98 else st.d_pruned_index.cpu().numpy().astype(np.int32)
         w = np.zeros((n_full, bs // merge, hkv, (dp + 15) // 16 * 16), np.uint16)
         O.kvstar_block_repre(bits(original[l][0]), np.array(full_ids[:n_full], np.int32), np.arange(n_full, dtype=np.int32), merge, w,
-                             pruned=pr)
+                             pruned=pr, keys_f16=(model == torch.float16))
         assert np.array_equal(bits(st.blk_repre.dense()), w[1:-2][..., :dp])
         want_repre.append(w[1:-2])
         pruned.append(pr)

@@ -419,6 +419,31 @@ def test_kvstar_block_repre_by_hand():
     assert not out[[0, 2, 3]].any()
 
 
+def test_kvstar_block_repre_of_fp16_keys_by_hand():
+    """A float16 cache: sequential fp32 sums of the widened keys, times 1/merge, rounded once to float16 - numpy's own
+    float16 conversions on both ends; merges 4 (the product is exact) and 3 (it is rounded to fp32 first)."""
+    for merge, bs in ((4, 8), (3, 12)):
+        hkv, d = 2, 4
+        rng = np.random.default_rng(71 + merge)
+        keys = (rng.standard_normal((3, bs, hkv, d)) * np.array([1.0, 300.0, 1e-4, 30.0])).astype(np.float16)
+        out = np.zeros((5, bs // merge, hkv, 16), np.uint16)
+        pr = np.array([[2, 0, 3], [1, 3, 0]], np.int32)
+        O.kvstar_block_repre(keys.view(np.uint16), [2, 0], [4, 1], merge, out, pruned=pr, keys_f16=True)
+        wide = keys.astype(np.float32)
+        for blk, slot in ((2, 4), (0, 1)):
+            for m in range(bs // merge):
+                for h in range(hkv):
+                    for p in range(3):
+                        vals = wide[blk, m * merge : (m + 1) * merge, h, pr[h, p]]
+                        acc = vals[0]
+                        for v in vals[1:]:
+                            acc = np.float32(acc + v)
+                        acc = np.float32(acc * np.float32(1.0 / merge))
+                        assert out[slot, m, h, p] == acc.astype(np.float16).view(np.uint16), (merge, blk, m, h, p)
+                    assert not out[slot, m, h, 3:].any()
+        assert not out[[0, 2, 3]].any()
+
+
 # ------------------------------------------ helpers the GPU tests use as ground truth
 
 def test_bf16_rounding_against_torch():

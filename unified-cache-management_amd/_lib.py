@@ -23,6 +23,7 @@ SIGNATURES = {
     "ucm_score_blocks": [_p, _i, _i64, _p, _i, _p, _i, _i64, _i64, _i, _p, _p, _i, _i, _i64, _i, _i, _i, _p, _i64, _f, _i, _p],
     "ucm_score_select": [_p, _p],
     "ucm_kvstar_block_repre": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _i, _p, _i64, _p, _i, _i, _i, _p, _i, _i64, _i64, _i64, _p],
+    "ucm_kvstar_block_repre_keys": [_p, _i, _i, _i, _p, _p, _i, _i, _i, _i, _i, _p, _i64, _p, _i, _i, _i, _p, _i, _i64, _i64, _i64, _p],
     "ucm_kvstar_park_queries": [_p, _i, _i64, _i, _p, _p, _i, _p, _i64, _p],
     "ucm_kvstar_workspace_floats": [_i, _i, _i, _i, _i, _i, _i, _p, _p],
     "ucm_kvstar_votes": [_p, _i64, _p, _i, _i, _i, _p, _i, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i64, _p, _i64, _p, _i, _p],

@@ -80,6 +80,38 @@ __device__ __forceinline__ void add_bf16x8(float (&acc)[8], const u32x4 v)
     acc[6] = acc[6] + __uint_as_float(v.w << 16); acc[7] = acc[7] + __uint_as_float(v.w & 0xffff0000u);
 }
 
+// float16 keys: the mean is rounded once, to float16 - what mean() gives in a float16 model (the .to(float16) that
+// follows changes nothing)
+__device__ __forceinline__ unsigned mean_f16keys_to_f16x2(float lo, float hi, float inv)
+{
+    float a = lo * inv, b = hi * inv;
+    asm volatile("" : "+v"(a), "+v"(b));     // the product is rounded to fp32 first, as torch's mean is, then converted
+    return static_cast<unsigned>(f32_to_f16_bits(a)) | (static_cast<unsigned>(f32_to_f16_bits(b)) << 16);
+}
+
+__device__ __forceinline__ void add_f16x8(float (&acc)[8], const u32x4 v)
+{
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        acc[2 * j] = acc[2 * j] + static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(w[j] & 0xffffu)));
+        acc[2 * j + 1] = acc[2 * j + 1] + static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(w[j] >> 16)));
+    }
+}
+
+template <bool kF16>
+__device__ __forceinline__ void add_keys8(float (&acc)[8], const u32x4 v)
+{
+    if (kF16) { add_f16x8(acc, v); } else { add_bf16x8(acc, v); }
+}
+
+template <bool kF16>
+__device__ __forceinline__ unsigned mean_pair(float lo, float hi, float inv)
+{
+    return kF16 ? mean_f16keys_to_f16x2(lo, hi, inv) : mean_to_f16x2(lo, hi, inv);
+}
+
+
 // With channel lists, which (kv head, 16-byte piece) pairs a thread writes is decided once per kernel when the
 // pairs divide the workgroup: kThreads / pairs threads share a pair and split its sub-blocks, and the pair's eight
 // kept channels stay in registers (-1: a padding column).  Reading the lists again for every piece and turning
@@ -172,7 +204,7 @@ __device__ __forceinline__ void repre_write_pieces(const unsigned short* __restr
 // block.  The loads of the next unit - of the same chunk, the next chunk or the next cache block - are
 // issued before the current unit's means are formed, so key loads stay in flight through the phase that
 // writes a chunk's pieces out and across cache blocks.
-template <int kMerge>
+template <int kMerge, bool kF16>
 __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows, unsigned block_size,
@@ -279,12 +311,12 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
 #pragma unroll
             for (int c = 0; c < 8; ++c) { acc[c] = -0.0f; }   // -0 + x == x for every x, signed zeros included
 #pragma unroll
-            for (unsigned t = 0; t < kMerge; ++t) { add_bf16x8(acc, v[j * kMerge + t]); }
+            for (unsigned t = 0; t < kMerge; ++t) { add_keys8<kF16>(acc, v[j * kMerge + t]); }
             u32x4 o;
-            o.x = mean_to_f16x2(acc[0], acc[1], inv);
-            o.y = mean_to_f16x2(acc[2], acc[3], inv);
-            o.z = mean_to_f16x2(acc[4], acc[5], inv);
-            o.w = mean_to_f16x2(acc[6], acc[7], inv);
+            o.x = mean_pair<kF16>(acc[0], acc[1], inv);
+            o.y = mean_pair<kF16>(acc[2], acc[3], inv);
+            o.z = mean_pair<kF16>(acc[4], acc[5], inv);
+            o.w = mean_pair<kF16>(acc[6], acc[7], inv);
             if (w < n_work) { *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o; }
         }
         if (live && u.w_first + kThreads * kBatch >= mc * ncg) { // the chunk is staged: write its pieces
@@ -326,6 +358,7 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_kernel(
 
 // Any other number of tokens per sub-block: one workgroup per cache block, the tokens of a sub-block summed
 // sixteen loads at a time.  grid: x = cache block of the list, y = layer.
+template <bool kF16>
 __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned rows, unsigned block_size, unsigned kv_heads,
@@ -367,14 +400,14 @@ __global__ __launch_bounds__(kThreads) void kvstar_repre_any_kernel(
 #pragma unroll
                 for (int u = 0; u < kRepreUnroll; ++u) { v[u] = ucm::gload16_nt(src + static_cast<size_t>(t + u) * row); }
 #pragma unroll
-                for (int u = 0; u < kRepreUnroll; ++u) { add_bf16x8(acc, v[u]); }
+                for (int u = 0; u < kRepreUnroll; ++u) { add_keys8<kF16>(acc, v[u]); }
             }
-            for (; t < merge; ++t) { add_bf16x8(acc, ucm::gload16_nt(src + static_cast<size_t>(t) * row)); }
+            for (; t < merge; ++t) { add_keys8<kF16>(acc, ucm::gload16_nt(src + static_cast<size_t>(t) * row)); }
             u32x4 o;
-            o.x = mean_to_f16x2(acc[0], acc[1], inv);
-            o.y = mean_to_f16x2(acc[2], acc[3], inv);
-            o.z = mean_to_f16x2(acc[4], acc[5], inv);
-            o.w = mean_to_f16x2(acc[6], acc[7], inv);
+            o.x = mean_pair<kF16>(acc[0], acc[1], inv);
+            o.y = mean_pair<kF16>(acc[2], acc[3], inv);
+            o.z = mean_pair<kF16>(acc[4], acc[5], inv);
+            o.w = mean_pair<kF16>(acc[6], acc[7], inv);
             *reinterpret_cast<u32x4*>(&stage[ml * srow_stride + cg * 8]) = o;
         }
         __syncthreads();
@@ -1027,15 +1060,18 @@ extern "C" int ucm_kvstar_park_queries(const void* q, int q_dtype, int64_t q_row
     UCM_LAUNCH_CHECK("ucm_kvstar_park_queries");
 }
 
-extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
-                                      const int32_t* block_ids, const int32_t* slots, int n, int block_size,
-                                      int kv_heads, int head_dim, int merge, const int32_t* pruned,
-                                      int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
-                                      int d_pruned, int d_pad, void* repre_f16, int repre_rows,
-                                      int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
-                                      ucm_stream_t stream)
+extern "C" int ucm_kvstar_block_repre_keys(const void* const* k_layers, int key_dtype, int n_layers, int num_blocks,
+                                           const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                                           int kv_heads, int head_dim, int merge, const int32_t* pruned,
+                                           int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
+                                           int d_pruned, int d_pad, void* repre_f16, int repre_rows,
+                                           int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
+                                           ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_kvstar_block_repre: n=%d", n);
+    UCM_REQUIRE(key_dtype == UCM_DTYPE_BF16 || key_dtype == UCM_DTYPE_F16, "ucm_kvstar_block_repre: key_dtype=%d (bfloat16 or float16)",
+                key_dtype);
+    const bool f16 = key_dtype == UCM_DTYPE_F16;
     UCM_REQUIRE(!pruned_sel || (pruned && n_pruned_lists >= 1), "ucm_kvstar_block_repre: pruned_sel needs the lists and their number");
     const int lists_per_layer = pruned_sel ? n_pruned_lists : 1;
     if (n == 0) { return UCM_OK; }
@@ -1072,13 +1108,17 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     const unsigned gx = static_cast<unsigned>(std::min(n, std::max(1, (1024 + n_layers - 1) / n_layers)));
 #define UCM_KVSTAR_REPRE(MERGE)                                                                                        \
     do {                                                                                                             \
+        if (f16) { UCM_KVSTAR_REPRE_T(MERGE, true); } else { UCM_KVSTAR_REPRE_T(MERGE, false); }                     \
+    } while (0)
+#define UCM_KVSTAR_REPRE_T(MERGE, F16)                                                                                 \
+    do {                                                                                                             \
         if (lds_bytes > 48u * 1024u) {                                                                               \
-            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_kernel<MERGE>),     \
+            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_kernel<MERGE, F16>), \
                                                       hipFuncAttributeMaxDynamicSharedMemorySize,                   \
                                                       static_cast<int>(lds_bytes));                                \
             if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }                \
         }                                                                                                            \
-        hipLaunchKernelGGL(kvstar_repre_kernel<MERGE>, dim3(gx, n_layers), dim3(kThreads), lds_bytes, hs, k_layers,  \
+        hipLaunchKernelGGL((kvstar_repre_kernel<MERGE, F16>), dim3(gx, n_layers), dim3(kThreads), lds_bytes, hs, k_layers,  \
                            block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(n),            \
                            static_cast<unsigned>(repre_rows), static_cast<unsigned>(block_size),                     \
                            static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim), pruned,                 \
@@ -1092,13 +1132,14 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
     case 2: UCM_KVSTAR_REPRE(2); break;
     case 4: UCM_KVSTAR_REPRE(4); break;
     case 8: UCM_KVSTAR_REPRE(8); break;
-    default:
+    default: {
+        auto* any = f16 ? kvstar_repre_any_kernel<true> : kvstar_repre_any_kernel<false>;
         if (lds_bytes > 48u * 1024u) {
-            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(kvstar_repre_any_kernel),
+            const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(any),
                                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
             if (ea != hipSuccess) { return ucm::check_hip(ea, "ucm_kvstar_block_repre (LDS size)"); }
         }
-        hipLaunchKernelGGL(kvstar_repre_any_kernel, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, hs,
+        hipLaunchKernelGGL(any, dim3(static_cast<unsigned>(n), n_layers), dim3(kThreads), lds_bytes, hs,
                            k_layers, block_ids, slots, static_cast<unsigned>(num_blocks), static_cast<unsigned>(repre_rows),
                            static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<unsigned>(head_dim),
                            static_cast<unsigned>(merge), pruned, pruned_layer_stride, pruned_sel,
@@ -1107,8 +1148,23 @@ extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers,
                            m_chunk);
         break;
     }
+    }
 #undef UCM_KVSTAR_REPRE
+#undef UCM_KVSTAR_REPRE_T
     UCM_LAUNCH_CHECK("ucm_kvstar_block_repre");
+}
+
+extern "C" int ucm_kvstar_block_repre(const void* const* k_layers, int n_layers, int num_blocks,
+                                      const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                                      int kv_heads, int head_dim, int merge, const int32_t* pruned,
+                                      int64_t pruned_layer_stride, const int32_t* pruned_sel, int n_pruned_lists,
+                                      int d_pruned, int d_pad, void* repre_f16, int repre_rows,
+                                      int64_t repre_layer_stride, int64_t repre_head_stride, int64_t repre_row_stride,
+                                      ucm_stream_t stream)
+{
+    return ucm_kvstar_block_repre_keys(k_layers, UCM_DTYPE_BF16, n_layers, num_blocks, block_ids, slots, n, block_size, kv_heads,
+                                       head_dim, merge, pruned, pruned_layer_stride, pruned_sel, n_pruned_lists, d_pruned, d_pad,
+                                       repre_f16, repre_rows, repre_layer_stride, repre_head_stride, repre_row_stride, stream);
 }
 
 

@@ -422,15 +422,21 @@ __global__ __launch_bounds__(kThreads) void score_kernel_bf16(const ScoreArgs a,
         stage_query<kD, QT>(a, l, t.q_row, qbar);
         __syncthreads();
 
-        f32x4 qlo[kSteps], qhi[kSteps];
+        // Half of the thread's query values stay in registers, the other half is read from LDS again in every pass
+        // (broadcast reads, after the memory clobber that follows the prefetch): with all of them in registers the
+        // kernel needs 158 VGPRs and runs three waves per SIMD, with half it needs 126 and runs four, which is worth
+        // 8 % on long requests (80 layers x 8 requests x 523-981 blocks: 239 -> 220 us) and costs the ragged batch
+        // of 16 short requests nothing; all of them from LDS (97 VGPRs, still four waves) was 211 us there but 56
+        // instead of 51 us on the ragged batch, whose workgroups make only a few passes.
+        const float* qmine = &qbar[h * kD + 8 * p];
+        f32x4 ql[kSteps];
 #pragma unroll
-        for (int i = 0; i < kSteps; ++i) {
-            qlo[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p]);
-            qhi[i] = *reinterpret_cast<const f32x4*>(&qbar[h * kD + 16 * i + 8 * p + 4]);
-        }
-
+        for (int i = 0; i < kSteps; ++i) { ql[i] = *reinterpret_cast<const f32x4*>(qmine + 16 * i); }
         auto finish = [&](const u32x4 (&kv)[kSteps], int base) {
-            const float dot = pair_dot<kSteps>(qlo, qhi, kv);
+            f32x4 qh[kSteps];
+#pragma unroll
+            for (int i = 0; i < kSteps; ++i) { qh[i] = *reinterpret_cast<const f32x4*>(qmine + 16 * i + 4); }
+            const float dot = pair_dot<kSteps>(ql, qh, kv);
             const float s = head_sum(dot, bl * vecs * 2, 2, a.kv_heads, a.num_repre);
             // the lanes of a block all hold its score; a scale of 1 changes no bit
             store_score(sout + min(base + bl, tile_end - 1), s * a.scale, fused);

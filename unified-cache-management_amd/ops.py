@@ -116,7 +116,7 @@ class LayerPointers:
 
 def _bf16_keys_only(layers: LayerPointers, what: str) -> None:
     if layers.tensors and layers.tensors[0].dtype == torch.float16:
-        raise ValueError(f"{what} reads bfloat16 key caches only (a float16 cache is taken by block_mean and the scoring calls)")
+        raise ValueError(f"{what} reads bfloat16 key caches only (a float16 cache is taken by block_mean, kvstar_block_repre and the scoring calls)")
 
 
 def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
@@ -611,10 +611,10 @@ def kvstar_table_from_reference(repre: torch.Tensor, layout: str = "head") -> to
 def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                        block_size: int, kv_heads: int, head_dim: int, num_blocks: int, merge: int,
                        pruned: Optional[torch.Tensor] = None, pruned_sel: Optional[torch.Tensor] = None) -> None:
-    """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); pruned int32 [kv_heads, d_pruned] (one set of
+    """repre: a kvstar_table ([L, kv_heads, rows, d_pad/8, M, 8] fp16); the caches bfloat16 or float16; pruned int32 [kv_heads, d_pruned] (one set of
     channel lists for every layer), [L, kv_heads, d_pruned] (lists per layer) or None.  With pruned_sel (int32 [n]:
     the list each listed block is pruned by) pruned is [n_lists, kv_heads, d_pruned] or [L, n_lists, kv_heads, d_pruned]."""
-    _bf16_keys_only(k_layers, "kvstar_block_repre")
+    key_dtype = _lib.DTYPE_F16 if k_layers.tensors and k_layers.tensors[0].dtype == torch.float16 else _lib.DTYPE_BF16
     if repre.dim() != 6 or repre.dtype != torch.float16 or repre.shape[4] * merge != block_size or \
             repre.shape[1] != kv_heads or repre.shape[5] != 8:
         raise ValueError("repre must be float16 [L, kv_heads, rows, d_pad/8, block_size/merge, 8]")
@@ -634,7 +634,7 @@ def kvstar_block_repre(k_layers: LayerPointers, block_ids: torch.Tensor, slots: 
         per_layer = pruned is not None and pruned.dim() == 3
     if pruned is not None and (pruned.shape[-2] != kv_heads or (per_layer and pruned.shape[0] != repre.shape[0])):
         raise ValueError("pruned must be [kv_heads, d_pruned] or [layers, kv_heads, d_pruned]")
-    _lib.call("ucm_kvstar_block_repre", k_layers.ptr(), repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
+    _lib.call("ucm_kvstar_block_repre_keys", k_layers.ptr(), key_dtype, repre.shape[0], num_blocks, _dev(block_ids, torch.int32, "block_ids"),
               _dev(slots, torch.int32, "slots"), block_ids.numel(), block_size, kv_heads, head_dim, merge,
               _opt(pruned, torch.int32, "pruned"), pruned.stride(0) if per_layer else 0,
               _opt(pruned_sel, torch.int32, "pruned_sel"), n_lists, d_pruned, repre.shape[3] * 8,
