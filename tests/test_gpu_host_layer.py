@@ -318,17 +318,102 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model, lag):
     assert "A" not in plugin.gsa_stats and not plugin.topk_kpre_manger.is_exist("A")
 
 
-def test_gsa_retrieval_stride_reuses_scores(ucm, dev):
+def test_gsa_retrieval_lag_with_a_request_that_arrives_later(ucm, dev):
+    """retrieval_lag 1 while the batch changes: request A decodes from step 1, request C's prompt arrives at step 4 (A
+    decoding beside it) and C decodes from step 5.  Every selection a layer's attention sees must be the oracle's for
+    the query the request had in the step before - for C's first decode step that is the last token of its prompt, kept
+    during the step that prefilled it - over the representatives and block lists of the step that uses it."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 160
+    lo, hi = 6, 10
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 60, {"seg_prefill_threshold": 100, "min_topk_len": lo, "max_topk_len": hi,
+                                                   "repre_dtype": "bfloat16", "retrieval_lag": 1})
+    plugin = GSA(cfg, UcmSparseRole.WORKER)
+    g = torch.Generator(device=dev)
+    g.manual_seed(9)
+    caches = [torch.zeros(2, nb, bs, hkv, d, dtype=torch.bfloat16, device=dev) for _ in range(L)]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
+    free_blocks = [int(x) for x in synth.permutation(731, nb)]
+    prompts, arrives = {"A": 290, "C": 410}, {"A": 0, "C": 4}
+    reqs = {r: ns(block_ids=[[]], num_computed_tokens=0, prompt_token_ids=[1] * n, output_token_ids=[]) for r, n in prompts.items()}
+    repre_h = {r: [np.zeros((60, hkv * d), np.float32) for _ in range(L)] for r in prompts}
+    done_blocks = {r: 0 for r in prompts}
+    q_before = {r: [None] * L for r in prompts}
+    lagged, checked = [], 0
+    for step in range(10):
+        live = [r for r in prompts if arrives[r] <= step]
+        sched = {r: (prompts[r] if step == arrives[r] else 1) for r in live}
+        for r in live:
+            need = -(-(reqs[r].num_computed_tokens + sched[r]) // bs)
+            while len(reqs[r].block_ids[0]) < need:
+                reqs[r].block_ids[0].append(free_blocks.pop())
+        so = ns(num_scheduled_tokens=sched, scheduled_new_reqs=[ns(req_id=r) for r in live if step == arrives[r]])
+        ib = ns(req_id_to_index={r: i for i, r in enumerate(live)})
+        seq_lens = {r: reqs[r].num_computed_tokens + sched[r] for r in live}
+        plugin.build_sparse_meta(so, {r: reqs[r] for r in live}, ib, None)
+        plugin.execute_begin(so)
+        lagged.append(plugin._lagged is not None)
+        for l in range(L):
+            md = ns(block_table=None, seq_lens=None)
+            fc.attn_metadata = {names[l]: md}
+            n_tok = sum(sched.values())
+            query = torch.randn(n_tok, hq, d, device=dev, generator=g).to(torch.bfloat16)
+            key = torch.randn(n_tok, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+            t0, last_row = 0, {}
+            for r in live:
+                for t in range(sched[r]):
+                    pos = reqs[r].num_computed_tokens + t
+                    caches[l][0, reqs[r].block_ids[0][pos // bs], pos % bs] = key[t0 + t]
+                t0 += sched[r]
+                last_row[r] = t0 - 1
+            plugin.attention_begin(query, key, key, names[l], fc)
+            torch.cuda.synchronize()
+            for i, r in enumerate(live):
+                q_now = query[last_row[r]].float().cpu().numpy()
+                if step > arrives[r]:                                     # a decode step of a sparsified request
+                    n = len(reqs[r].block_ids[0])
+                    q_use = q_before[r][l] if lagged[-1] else q_now
+                    want_idx, _ = O.select_topk(q_use, repre_h[r][l][:n].reshape(n, hkv, 1, d), topk_len(n, lo, hi))
+                    phys, want_len = O.block_table_gather(reqs[r].block_ids[0], want_idx, seq_lens[r], bs)
+                    assert int(md.seq_lens[i]) == want_len, (step, l, r)
+                    assert np.array_equal(md.block_table[i, : len(phys)].cpu().numpy(), phys), (step, l, r)
+                    checked += 1
+                q_before[r][l] = q_now
+            plugin.attention_finished(query, key, key, None, names[l], fc)
+            for r in live:
+                full = min(seq_lens[r] // bs, len(reqs[r].block_ids[0]))
+                todo = list(range(done_blocks[r], full))
+                if todo:
+                    kc = caches[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+                    O.block_mean_paged(kc, [reqs[r].block_ids[0][i] for i in todo], todo, repre_h[r][l], round_bf16=True)
+        for r in live:
+            done_blocks[r] = max(done_blocks[r], min(seq_lens[r] // bs, len(reqs[r].block_ids[0])))
+            reqs[r].num_computed_tokens += sched[r]
+            reqs[r].output_token_ids.append(7)
+        plugin.execute_finished()
+    # step 1 scores layer by layer (nothing was kept during the prefill-only step 0); from step 2 on one launch per step,
+    # the step C's prompt runs beside A's decode and C's first decode step included
+    assert lagged == [False, False] + [True] * 8
+    assert checked == L * (9 + 5)
+
+
+@pytest.mark.parametrize("lag", [0, 1])
+def test_gsa_retrieval_stride_reuses_scores(ucm, dev, lag):
     """With retrieval_stride 3 the scores of the last retrieval are re-selected with the current lengths
     on the steps in between (the last two blocks are always kept, so the newest block is never missing);
-    a request is scored on its first sparsified step whatever the stride."""
+    a request is scored on its first sparsified step whatever the stride.  With retrieval_lag 1 the queries are kept
+    only on the step before a retrieval, and that retrieval (step 3) is the one launch before the model runs."""
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.gsa.gsa import GSA
 
     ns = types.SimpleNamespace
     hq, hkv, d, L, bs, nb = 8, 2, 64, 1, 16, 64
     cfg = make_config(hq, hkv, d, L, bs, 16 * 40, {"seg_prefill_threshold": 10, "min_topk_len": 5, "max_topk_len": 5,
-                                                   "retrieval_stride": 3})
+                                                   "retrieval_stride": 3, "retrieval_lag": lag})
     plugin = GSA(cfg, UcmSparseRole.WORKER)
     cache = torch.randn(2, nb, bs, hkv, d, device=dev).to(torch.bfloat16)
     name = "model.layers.0.self_attn.attn"
@@ -344,6 +429,8 @@ def test_gsa_retrieval_stride_reuses_scores(ucm, dev):
         plugin.build_sparse_meta(so, {"A": st}, ib, None)
         plugin.execute_begin(so)
         scored.append(plugin.model_input["is_topk"])
+        assert (plugin._lagged is not None) == (lag == 1 and step == 3)
+        assert (plugin._parking is not None) == (lag == 1 and step == 2)
         md = ns(block_table=None, seq_lens=None)
         fc.attn_metadata = md
         q = torch.randn(n_new, hq, d, device=dev).to(torch.bfloat16)
