@@ -1019,6 +1019,8 @@ def main():
                           ("GSA, retrieval_lag 1", lambda: plugin_bench.gsa_leg(torch, dev, caches, lens, block_lists, args.steps, args.seed, 1)),
                           ("ESA", lambda: plugin_bench.esa_leg(torch, dev, caches, lens, block_lists, args.seed)),
                           ("KvComp", lambda: plugin_bench.kvcomp_leg(torch, dev, caches, lens, block_lists, args.seed)),
+                          ("KvComp, delta_loads (decode queries drift with correlation 0.95 per step)",
+                           lambda: plugin_bench.kvcomp_leg(torch, dev, caches, lens, block_lists, args.seed, True, 0.95)),
                           ("KVStar", lambda: plugin_bench.kvstar_leg(torch, dev, caches, lens, block_lists, args.seed))):
             plugin_leg[name] = leg()
             gc.collect()                                     # the leg's plugin and its store (a KV cache's worth of memory)

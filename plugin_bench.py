@@ -74,6 +74,8 @@ class Harness:
         self.g = torch.Generator(device=dev)
         self.g.manual_seed(seed)
         self.times = {}
+        self.rho = 0.0                 # correlation of a layer's decode queries from one step to the next (0: independent draws)
+        self._last_q = None
 
     def decode_token(self) -> None:
         """Every request has produced one more token (what the engine does between two decode steps)."""
@@ -94,6 +96,12 @@ class Harness:
         rows = starts[-1] if query_rows is None else query_rows
         draw = lambda: torch.empty((rows, HQ, D), dtype=torch.bfloat16, device=self.dev).normal_(0.0, 0.3, generator=self.g)
         qs = [draw()] * self.n_layers if one_query else [draw() for _ in range(self.n_layers)]
+        if self.rho > 0.0 and not one_query:
+            # decode queries that drift: q_t = rho q_(t-1) + sqrt(1 - rho^2) noise, layer by layer (the same batch as before)
+            if self._last_q is not None and self._last_q[0].shape == qs[0].shape:
+                qs = [(self.rho * a.float() + math.sqrt(1.0 - self.rho ** 2) * b.float()).to(torch.bfloat16)
+                      for a, b in zip(self._last_q, qs)]
+            self._last_q = qs
         so = ns(num_scheduled_tokens=dict((rid, n_tokens[rid]) for rid in live), req_sparsed_slots={rid: 0 for rid in live},
                 scheduled_new_reqs=[ns(req_id=rid) for rid in live if self.reqs[rid].num_computed_tokens == 0],
                 scheduled_cached_reqs=ns(req_ids=[rid for rid in live if self.reqs[rid].num_computed_tokens > 0]))
@@ -226,20 +234,23 @@ def esa_leg(torch, dev, caches, lens, block_tables, seed: int) -> dict:
     return _second_wave(wave)
 
 
-def kvcomp_leg(torch, dev, caches, lens, block_tables, seed: int) -> dict:
+def kvcomp_leg(torch, dev, caches, lens, block_tables, seed: int, delta: bool = False, rho: float = 0.0) -> dict:
     """KvComp, device path: hash codes of every prompt block at the end of the prefill (and the blocks into the
-    store), the scheduler shrinks the block lists, then a retrieval every fourth decode step."""
+    store), the scheduler shrinks the block lists, then a retrieval every fourth decode step.  ``delta``: the
+    retrieval's load moves only the picks the middle cache blocks do not hold yet (how many depends on how far the
+    queries drift between retrievals: ``rho`` per step)."""
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
 
     n_layers = len(caches)
     torch.manual_seed(seed)                                            # the plugin draws its hash weights from the global generator
-    cfg = make_config(n_layers, 65536, len(lens) + 1, "KvComp", {"device_loads": True})
+    cfg = make_config(n_layers, 65536, len(lens) + 1, "KvComp", {"device_loads": True, "delta_loads": delta})
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     plugin.connector = _store(torch, n_layers, int(sum(lens)))
 
     def wave(w: int) -> dict:
         h = Harness(torch, dev, plugin, caches, _prompt_shape(lens), block_tables, seed)
+        h.rho = rho
         h.step("prefill end (hash codes + blocks to the store, 32 layers)", {rid: r.num_prompt_tokens for rid, r in h.reqs.items()},
                query_rows=16)
         for step in range(1, 10):
@@ -260,6 +271,9 @@ def kvcomp_leg(torch, dev, caches, lens, block_tables, seed: int) -> dict:
                                     "wall_us": round(float(np.median(busy[:, 1])), 1)}
         out["plain step"] = {"steps": len(plain), "host_us": round(float(np.median(plain[:, 0])), 1),
                              "wall_us": round(float(np.median(plain[:, 1])), 1)}
+        if delta and plugin._dev is not None and plugin._dev.miss_step is not None:
+            picks = int(plugin._dev.cnt[:, : len(lens)].sum())
+            out["blocks_moved_by_the_last_retrieval"] = {"moved": int(plugin._dev.miss_step.sum()), "picked": picks}
         for rid in list(h.reqs):
             plugin.request_finished_in_worker(rid)
         return out

@@ -53,15 +53,17 @@ def test_hash_encoder_surface(ucm, dev):
     assert np.array_equal(pm.float().cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("device_loads,hole", [(True, False), (False, False), (True, True)])
-def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole):
+@pytest.mark.parametrize("device_loads,hole,delta", [(True, False, False), (False, False, False), (True, True, False),
+                                                     (True, False, True), (True, True, True)])
+def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
     """Prefill of 20 full blocks + 5 tokens, then decode on the sparsified block list: windows restored at step 1,
     retrieval at steps 1 and 5 picks what the oracle picks from the same keys, the chosen blocks land in the
     request's middle cache blocks in ascending order, a block filled during decode is dumped and hashed.  Once
     through the batched device path (one call per layer for all requests, loads planned on the device) and once
     through the per-request path that works with any store.  ``hole``: at the first retrieval the store lacks every
     other block - the load leaves those out, says so (a warning, a counter), and finds them at the next retrieval,
-    by which time they are back."""
+    by which time they are back.  ``delta``: the load moves only the picks that are not in the middle cache blocks
+    already - the same set of blocks there, each in the block the plan names, fewer bytes moved."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvcomp.kvcomp import KvComp
@@ -71,7 +73,8 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole):
     hq, hkv, d, L, bs, nb = 8, 2, 128, 2, 16, 64
     cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
     cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KvComp": {"keep_token_codes": True,
-                                                                                         "device_loads": device_loads}}}
+                                                                                         "device_loads": device_loads,
+                                                                                         "delta_loads": delta}}}
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     assert isinstance(plugin, KvComp)
     slice_bytes = bs * hkv * d * 2
@@ -138,7 +141,7 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole):
         order = np.argsort(-sc.astype(np.float32), kind="stable")[:mid]
         return sorted(first + int(i) for i in order)
 
-    away = {}
+    away, first_picks, first_placed = {}, {}, {}
     if hole:
         away = {b: store.slot_of.pop(f"req_A_blk_{b}") for b in range(1, 19, 2)}
     for step in range(1, 7):
@@ -159,13 +162,34 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole):
             if step in (1, 5):
                 want = expected(l, qs[l], 20)
                 assert st.last_selection == want, (step, l)
+                placed = want
+                if delta:
+                    # the plan's own record of what each middle block holds: the picks, every one once ...
+                    placed = plugin._dev.resident_blocks(l, "A")
+                    if hole and step == 1:                   # the load left blocks out: the record is dropped (the next
+                        assert placed == [-1] * mid          # retrieval loads everything); an empty row is filled in pick order
+                        placed = want
+                    assert sorted(placed) == want, (step, l, placed)
+                    moved = int(plugin._dev.miss_step[l, 0])
+                    if step == 1:
+                        assert moved == mid
+                    elif not hole:                           # ... and at the second retrieval only the new ones moved,
+                        assert moved == len(set(want) - set(first_picks[l])), (step, l)       # the others stayed where they were
+                        assert all(b == a for a, b in zip(first_placed[l], placed) if a in want)
+                    else:
+                        assert moved == mid                  # (after a load that left blocks out everything is loaded afresh)
+                    if step == 1:
+                        first_picks[l], first_placed[l] = want, placed
                 for kv in range(2):
                     got = caches[l][kv][kept[1 : 1 + mid]]
-                    should = original[l][kv][[full_ids[b] for b in want]]
+                    should = original[l][kv][[full_ids[b] for b in placed]]
+                    want_order = want
+                    want = placed
                     for j, b in enumerate(want):             # a block the store lacked: the cache block keeps what it held
                         if step == 1 and b in away:
                             should[j] = before[l][kv][kept[1 + j]]
                     assert torch.equal(got, should), (step, l, kv)
+                    want = want_order
                     # windows: logical block 0 in the first kept block, the last two logical blocks in the last two
                     assert torch.equal(caches[l][kv][kept[0]], original[l][kv][full_ids[0]])
             else:

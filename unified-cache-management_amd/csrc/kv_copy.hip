@@ -390,7 +390,12 @@ extern "C" int ucm_kv_load_planned_tp(void* const* layers, int n_layers, size_t 
                            static_cast<unsigned>(table_rows), static_cast<unsigned>(batch), static_cast<unsigned>(n_layers), lay);
     } else {
         // the entries to load are scattered over a row (or there are too many rows for the counted kernel's table)
-        const unsigned gx = static_cast<unsigned>(std::min(n_slots, load_count ? 8 : 16));
+        // A small launch (one layer's plan for a batch) takes a workgroup per slot: the slots that load are scattered,
+        // and with 16 workgroups stepping through a row some copy three blocks while others copy none (a layer of 16
+        // requests with 40 % of 48 slots to load: 190 us stepping, about as long as loading all of them).  A big one (every
+        // layer's plan in one launch) keeps the stepping: there the workgroups that find nothing are the many.
+        const int64_t per_slot = static_cast<int64_t>(n_slots) * batch * n_layers * 2;
+        const unsigned gx = static_cast<unsigned>(per_slot <= 8192 ? n_slots : std::min(n_slots, load_count ? 8 : 16));
         hipLaunchKernelGGL(kv_load_planned_kernel, dim3(gx, batch, n_layers * 2), dim3(kThreads), 0,
                            ucm::as_stream(stream), layers, kv_stride, block_bytes, static_cast<unsigned>(num_blocks),
                            static_cast<const uint8_t*>(pool), static_cast<uint64_t>(pool_blocks), pool_block_bytes,

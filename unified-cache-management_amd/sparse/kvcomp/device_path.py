@@ -21,6 +21,12 @@ trips and covers all requests of the step at once:
   block, K and V - what ``launch_transfer_task("load", hashes, mid)`` does
   (:283-323), without the wait.
 
+With ``"delta_loads": true`` the load is a delta: the plugin remembers which candidate each middle cache block
+holds (per layer and request), ``ucm_delta_plan`` keeps the picks that are already there where they are and pairs the
+missing ones with the blocks whose candidate was not picked again, and ``ucm_kv_load_planned`` moves only those - the
+same set of blocks in the request's middle cache blocks as the reference leaves there, in another order (the reference
+reloads every pick at every retrieval, :283-323, pick j into the j-th block).
+
 Which steps retrieve, which blocks are candidates and how many are picked are
 the reference's rules (``ReqStatePerLayer.retrieval`` :202-258).  Blocks that
 became full (``save_blocks`` :325-347) are dumped into the pool and hashed for
@@ -54,6 +60,12 @@ class KvCompDevicePath:
         # per-step descriptor, one entry per retrieving request: seg_off, seg_len, topk_len, its token in the step's
         # query tensor, its table row; filled on the host and sent in one copy
         self._desc = torch.empty((5, rows), dtype=torch.int32)
+        # delta loads: the candidate (offset from the row's first) each middle cache block holds, -1 = none of them
+        self.delta = bool(plugin.cfg.get("delta_loads", False))
+        self.resident = torch.full((L, rows, mb), -1, **i32) if self.delta else None
+        self.res_step = self.load_step = self.slot_step = self.miss_step = self._res_rows = None
+        self._forget: List[int] = []                              # rows whose load left blocks out: planned afresh next time
+        self.n_layers = L
         self.n_src: Dict[object, int] = {}                        # candidates of a request whose pool block is uploaded
         self.src_absent: Dict[object, List[int]] = {}             # ... and those the store did not hold at the last look
         self.held: Dict[object, HeldBlocks] = {}                  # per request: its stored blocks stay in the store's pool
@@ -84,6 +96,7 @@ class KvCompDevicePath:
         the descriptor for the requests that retrieve in this step (kvcomp.py:361-371, :202-215)."""
         p = self.plugin
         stride, init, local = p.cfg["retrieval_stride"], p.cfg["init_window_sz"], p.cfg["local_window_sz"]
+        self._commit_resident()
         self.active, self.max_len, self.total = [], 0, 0
         rows = self.rows
         host = None
@@ -113,6 +126,10 @@ class KvCompDevicePath:
             if self.dst_ids.get(meta.request_id) != ids:
                 self.dst_table[row, : len(ids)] = torch.tensor(ids, dtype=torch.int32, device=self.device)
                 self.dst_ids[meta.request_id] = ids
+                if self.delta:
+                    self.resident[:, row] = -1               # other cache blocks: what they hold is not known
+            if self.delta and self.src_absent.get(meta.request_id):
+                self._forget.append(row)                     # the plan will count blocks as loaded that the load leaves out
         if host is not None:
             n = len(self.active)
             d = ops.upload(self._desc[:, :n], self.device)      # (pinned staging whose reuse waits for its last copy)
@@ -121,6 +138,25 @@ class KvCompDevicePath:
             self.src_step = self.src_table.index_select(0, table_rows)      # the step's requests side by side
             self.dst_step = self.dst_table.index_select(0, table_rows)
             self.slot_of_step = {r: i for i, r in enumerate(self.active)}
+            if self.delta:
+                w = max(len(self.dst_ids[r]) for r in self.active)           # middle cache blocks of the widest request
+                if w > 1024:
+                    raise ValueError(f"delta_loads plans at most 1024 middle blocks per request ({w} here)")
+                # [layers, the step's requests, middle blocks]
+                self.res_step = self.resident.index_select(1, table_rows)[:, :, :w].contiguous()
+                self.load_step, self.slot_step = torch.empty_like(self.res_step), torch.empty_like(self.idx[:, :n])
+                self.miss_step = torch.zeros((self.n_layers, n), dtype=torch.int32, device=self.device)
+                self._res_rows = table_rows
+
+    def _commit_resident(self) -> None:
+        """What the step's plans left in the middle blocks goes back into the requests' rows (after the last layer's
+        hook, or before the next step is built)."""
+        if self._res_rows is not None:
+            self.resident[:, :, : self.res_step.shape[2]].index_copy_(1, self._res_rows, self.res_step)
+            self._res_rows = None
+        if self._forget:
+            self.resident[:, torch.tensor(self._forget, dtype=torch.int64, device=self.device)] = -1
+            self._forget = []
 
     def _sources(self, request_id, row: int, first: int, count: int) -> None:
         """Pool blocks of candidates first .. first+count-1: the hash -> store lookup, once per block the store holds;
@@ -174,6 +210,13 @@ class KvCompDevicePath:
         idx, cnt = self.idx[l, :b], self.cnt[l, :b]
         ops.topk_windows(p.scores[l], self.seg_off, self.seg_len, self.topk_len, self.max_len, idx, cnt, start_w=0, end_w=0)
         kv_stride, block_bytes, num_blocks, _ = self._geom[layer_id]
+        if self.delta:
+            ops.delta_plan(idx, idx, cnt, self.res_step[l], self.load_step[l], self.slot_step[l], self.miss_step[l])
+            ops.kv_load_planned(self._kv[layer_id], 0, layer_id, 1, kv_stride, block_bytes, num_blocks, self.pool,
+                                self.pool_block_bytes, self.load_step[l], self.src_step, self.dst_step, None)
+            if layer_id == self.n_layers - 1:
+                self._commit_resident()
+            return
         ops.kv_load_planned(self._kv[layer_id], 0, layer_id, 1, kv_stride, block_bytes, num_blocks, self.pool,
                             self.pool_block_bytes, idx, self.src_step, self.dst_step, None, load_count=cnt)
 
@@ -272,7 +315,22 @@ class KvCompDevicePath:
         n = int(self.cnt[layer_id, i])
         return [self.first_of[request_id] + int(x) for x in self.idx[layer_id, i, :n].tolist()]
 
+    def resident_blocks(self, layer_id: int, request_id) -> Optional[List[int]]:
+        """Delta loads: the logical block each middle cache block of the request holds after its latest retrieval (-1:
+        none), in the order of the request's middle cache blocks (reads back)."""
+        if not self.delta or request_id not in self.dst_ids:
+            return None
+        self._commit_resident()
+        p = self.plugin
+        row = p.segment_base(request_id) // p.max_blocks
+        first = self.first_of[request_id]
+        return [first + int(x) if x >= 0 else -1 for x in self.resident[layer_id, row, : len(self.dst_ids[request_id])].tolist()]
+
     def request_finished(self, request_id) -> None:
+        if self.delta and request_id in self.dst_ids:
+            self._commit_resident()
+            p = self.plugin
+            self.resident[:, p.segment_base(request_id) // p.max_blocks] = -1
         held = self.held.pop(request_id, None)
         if held is not None:
             held.release()
