@@ -460,6 +460,22 @@ int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const in
                             int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
                             const void* w_bf16, int bits, uint8_t* q_codes, int16_t* q_sum,
                             uint8_t* qbar_codes, ucm_stream_t stream);
+/*
+ * The same two calls for a float16 model: keys (or queries) and weights are float16 - HashEncoder draws its weights
+ * in the model's type (ucm/sparse/kvcomp/hash_encoder.py:65-71) - and the codes are the signs of the exactly
+ * accumulated float16 products.  The query call takes one query head per kv head only (q_heads == kv_heads, what the
+ * plugin passes after its own group mean, kvcomp.py:228-233); UCM_ENOTSUP otherwise.
+ */
+int ucm_hash_encode_blocks_f16(const void* const* k_layers, int n_layers, int num_blocks,
+                               const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                               int kv_heads, int head_dim, const void* w_f16, int bits, int rows,
+                               uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                               int64_t colsum_layer_stride, uint8_t* block_codes,
+                               int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream);
+int ucm_hash_encode_queries_f16(const void* q_f16, int64_t q_layer_stride, const int32_t* q_rows,
+                                int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
+                                const void* w_f16, int bits, uint8_t* q_codes, int16_t* q_sum,
+                                uint8_t* qbar_codes, ucm_stream_t stream);
 int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_codes,
                           const int16_t* colsum, int64_t colsum_layer_stride,
                           const uint8_t* block_codes, int64_t block_codes_layer_stride, int64_t rows,

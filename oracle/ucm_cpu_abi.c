@@ -42,6 +42,8 @@ TWIN(ucm_esa_retrieve);
 TWIN(ucm_esa_retrieve_rows);
 TWIN(ucm_hash_encode_blocks);
 TWIN(ucm_hash_encode_queries);
+TWIN(ucm_hash_encode_blocks_f16);
+TWIN(ucm_hash_encode_queries_f16);
 TWIN(ucm_hash_score_blocks);
 TWIN(ucm_copy_batch);
 TWIN(ucm_kv_load_planned);
@@ -507,23 +509,27 @@ int ucm_esa_retrieve_rows_cpu(const float* data, int n_items, int dim, const flo
 
 /* ------------------------------------------------------------ hash codes */
 
-static float* widen_weights(const void* w_bf16, int head_dim, int bits)
+/* bfloat16 or float16 values widened to fp32 (exact either way) */
+static void widen_to_f32(const void* src, int f16, size_t n, float* dst)
+{
+    for (size_t i = 0; i < n; ++i) {
+        const uint16_t h = ((const uint16_t*)src)[i];
+        dst[i] = f16 ? orc_f16_to_f32(h) : orc_bf16_to_f32(h);
+    }
+}
+
+static float* widen_weights(const void* w16, int f16, int head_dim, int bits)
 {
     float* w = (float*)malloc((size_t)head_dim * bits * sizeof(float));
-    if (w) {
-        for (size_t i = 0; i < (size_t)head_dim * bits; ++i) { w[i] = orc_bf16_to_f32(((const uint16_t*)w_bf16)[i]); }
-    }
+    if (w) { widen_to_f32(w16, f16, (size_t)head_dim * bits, w); }
     return w;
 }
 
-int ucm_hash_encode_blocks_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
-                               const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, const void* w_bf16,
-                               int bits, int rows, uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
-                               int64_t colsum_layer_stride, uint8_t* block_codes, int64_t block_codes_layer_stride,
-                               int workgroups, ucm_stream_t stream)
+static int hash_encode_blocks_host(int f16, const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
+                                   const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, const void* w_bf16,
+                                   int bits, int rows, uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                                   int64_t colsum_layer_stride, uint8_t* block_codes, int64_t block_codes_layer_stride)
 {
-    (void)stream;
-    (void)workgroups;
     if (n < 0) { return UCM_EINVAL; }
     if (n == 0) { return UCM_OK; }
     if (!k_layers || !w_bf16 || !colsum || !block_codes || n_layers <= 0 || num_blocks <= 0 || rows <= 0 || block_size <= 0 ||
@@ -533,16 +539,22 @@ int ucm_hash_encode_blocks_cpu(const void* const* k_layers, int n_layers, int nu
     if (head_dim != 128 || bits != 128) { return UCM_ENOTSUP; }
     const uint32_t nbytes = (uint32_t)bits / 8;
     const size_t n_vec = (size_t)block_size * kv_heads;
-    float* w = widen_weights(w_bf16, head_dim, bits);
+    float* w = widen_weights(w_bf16, f16, head_dim, bits);
     uint8_t* codes = (uint8_t*)malloc(n_vec * nbytes);
-    if (!w || !codes) { free(w); free(codes); return UCM_ENOMEM; }
+    float* xf = f16 ? (float*)malloc(n_vec * head_dim * sizeof(float)) : NULL;
+    if (!w || !codes || (f16 && !xf)) { free(w); free(codes); free(xf); return UCM_ENOMEM; }
     for (int l = 0; l < n_layers; ++l) {
         for (int i = 0; i < n; ++i) {
             /* block_ids NULL: item i is block i; slots NULL: it goes to row i */
             const int64_t id = block_ids ? block_ids[i] : i, slot = slots ? slots[i] : i;
             if (id < 0 || id >= num_blocks || slot < 0 || slot >= rows) { continue; }
             const uint16_t* x = (const uint16_t*)k_layers[l] + (size_t)id * n_vec * head_dim;
-            orc_hash_encode(x, w, (uint32_t)n_vec, (uint32_t)head_dim, (uint32_t)bits, codes);
+            if (f16) {
+                widen_to_f32(x, 1, n_vec * head_dim, xf);
+                orc_hash_encode_f32(xf, w, (uint32_t)n_vec, (uint32_t)head_dim, (uint32_t)bits, codes);
+            } else {
+                orc_hash_encode(x, w, (uint32_t)n_vec, (uint32_t)head_dim, (uint32_t)bits, codes);
+            }
             if (token_codes) {
                 memcpy(token_codes + (size_t)l * (size_t)token_codes_layer_stride + (size_t)slot * n_vec * nbytes, codes,
                        n_vec * nbytes);
@@ -555,24 +567,50 @@ int ucm_hash_encode_blocks_cpu(const void* const* k_layers, int n_layers, int nu
     }
     free(w);
     free(codes);
+    free(xf);
     return UCM_OK;
 }
 
-int ucm_hash_encode_queries_cpu(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows, int n_req, int n_layers,
-                                int q_heads, int kv_heads, int head_dim, const void* w_bf16, int bits, uint8_t* q_codes,
-                                int16_t* q_sum, uint8_t* qbar_codes, ucm_stream_t stream)
+int ucm_hash_encode_blocks_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
+                               const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, const void* w_bf16,
+                               int bits, int rows, uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                               int64_t colsum_layer_stride, uint8_t* block_codes, int64_t block_codes_layer_stride,
+                               int workgroups, ucm_stream_t stream)
 {
     (void)stream;
+    (void)workgroups;
+    return hash_encode_blocks_host(0, k_layers, n_layers, num_blocks, block_ids, slots, n, block_size, kv_heads, head_dim, w_bf16,
+                                   bits, rows, token_codes, token_codes_layer_stride, colsum, colsum_layer_stride, block_codes,
+                                   block_codes_layer_stride);
+}
+
+int ucm_hash_encode_blocks_f16_cpu(const void* const* k_layers, int n_layers, int num_blocks, const int32_t* block_ids,
+                                   const int32_t* slots, int n, int block_size, int kv_heads, int head_dim, const void* w_f16,
+                                   int bits, int rows, uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                                   int64_t colsum_layer_stride, uint8_t* block_codes, int64_t block_codes_layer_stride,
+                                   int workgroups, ucm_stream_t stream)
+{
+    (void)stream;
+    (void)workgroups;
+    return hash_encode_blocks_host(1, k_layers, n_layers, num_blocks, block_ids, slots, n, block_size, kv_heads, head_dim, w_f16,
+                                   bits, rows, token_codes, token_codes_layer_stride, colsum, colsum_layer_stride, block_codes,
+                                   block_codes_layer_stride);
+}
+
+static int hash_encode_queries_host(int f16, const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows, int n_req,
+                                    int n_layers, int q_heads, int kv_heads, int head_dim, const void* w_bf16, int bits,
+                                    uint8_t* q_codes, int16_t* q_sum, uint8_t* qbar_codes)
+{
     if (n_req < 0 || n_layers < 0) { return UCM_EINVAL; }
     if (n_req == 0 || n_layers == 0) { return UCM_OK; }
     if (!q_bf16 || !w_bf16 || !q_codes || !q_sum || !qbar_codes || kv_heads <= 0 || q_heads < kv_heads ||
         q_heads % kv_heads != 0) {
         return UCM_EINVAL;
     }
-    if (head_dim != 128 || bits != 128) { return UCM_ENOTSUP; }
+    if (head_dim != 128 || bits != 128 || (f16 && q_heads != kv_heads)) { return UCM_ENOTSUP; }
     const uint32_t nbytes = (uint32_t)bits / 8;
     const size_t qrow = (size_t)q_heads * head_dim;
-    float* w = widen_weights(w_bf16, head_dim, bits);
+    float* w = widen_weights(w_bf16, f16, head_dim, bits);
     float* qf = (float*)malloc(qrow * sizeof(float));
     if (!w || !qf) { free(w); free(qf); return UCM_ENOMEM; }
     for (int l = 0; l < n_layers; ++l) {
@@ -582,14 +620,14 @@ int ucm_hash_encode_queries_cpu(const void* q_bf16, int64_t q_layer_stride, cons
             const uint16_t* x = (const uint16_t*)q_bf16 + (size_t)l * (size_t)q_layer_stride + (size_t)qr * qrow;
             const size_t lr = (size_t)l * n_req + r;
             uint8_t* codes = q_codes + lr * q_heads * nbytes;
-            orc_hash_encode(x, w, (uint32_t)q_heads, (uint32_t)head_dim, (uint32_t)bits, codes);
+            widen_to_f32(x, f16, qrow, qf);
+            orc_hash_encode_f32(qf, w, (uint32_t)q_heads, (uint32_t)head_dim, (uint32_t)bits, codes);
             for (int c = 0; c < bits; ++c) {
                 int32_t ones = 0;
                 for (int h = 0; h < q_heads; ++h) { ones += (codes[(size_t)h * nbytes + c / 8] >> (c % 8)) & 1; }
                 q_sum[lr * bits + c] = (int16_t)(2 * ones - q_heads);
             }
             /* the kv head's group-mean query in fp32 (select_topk_block.cpp:101-114), then its code */
-            for (size_t c = 0; c < qrow; ++c) { qf[c] = orc_bf16_to_f32(x[c]); }
             orc_q_head_mean(qf, (uint32_t)kv_heads, (uint32_t)q_heads, (uint32_t)head_dim);
             orc_hash_encode_f32(qf, w, (uint32_t)kv_heads, (uint32_t)head_dim, (uint32_t)bits, qbar_codes + lr * kv_heads * nbytes);
         }
@@ -597,6 +635,24 @@ int ucm_hash_encode_queries_cpu(const void* q_bf16, int64_t q_layer_stride, cons
     free(w);
     free(qf);
     return UCM_OK;
+}
+
+int ucm_hash_encode_queries_cpu(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows, int n_req, int n_layers,
+                                int q_heads, int kv_heads, int head_dim, const void* w_bf16, int bits, uint8_t* q_codes,
+                                int16_t* q_sum, uint8_t* qbar_codes, ucm_stream_t stream)
+{
+    (void)stream;
+    return hash_encode_queries_host(0, q_bf16, q_layer_stride, q_rows, n_req, n_layers, q_heads, kv_heads, head_dim, w_bf16, bits,
+                                    q_codes, q_sum, qbar_codes);
+}
+
+int ucm_hash_encode_queries_f16_cpu(const void* q_f16, int64_t q_layer_stride, const int32_t* q_rows, int n_req, int n_layers,
+                                    int q_heads, int kv_heads, int head_dim, const void* w_f16, int bits, uint8_t* q_codes,
+                                    int16_t* q_sum, uint8_t* qbar_codes, ucm_stream_t stream)
+{
+    (void)stream;
+    return hash_encode_queries_host(1, q_f16, q_layer_stride, q_rows, n_req, n_layers, q_heads, kv_heads, head_dim, w_f16, bits,
+                                    q_codes, q_sum, qbar_codes);
 }
 
 int ucm_hash_score_blocks_cpu(int mode, const int16_t* q_sum, const uint8_t* qbar_codes, const int16_t* colsum,

@@ -15,7 +15,8 @@ TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_se
          "ucm_kv_gather_selected", "ucm_delta_plan", "ucm_hash_encode_blocks", "ucm_hash_encode_queries",
          "ucm_hash_score_blocks", "ucm_esa_retrieve", "ucm_esa_retrieve_rows", "ucm_delta_plan_rows", "ucm_copy_batch",
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
-         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries", "ucm_park_rows", "ucm_kvstar_block_repre_keys"]
+         "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries", "ucm_park_rows", "ucm_kvstar_block_repre_keys",
+         "ucm_hash_encode_blocks_f16", "ucm_hash_encode_queries_f16"]
 
 
 def twin_caller(signatures):
@@ -252,7 +253,13 @@ def hash_inputs():
     q = synth.normal_bf16_bits(7111, (HL, 4, HHQ, HD))
     ids = np.array([4, 0, 6, -3, 2, 1, 5, HNB], np.int32)              # two ids the call must skip
     slots = np.array([0, 1, 2, 3, 3, 4, 5, 5], np.int32)
-    return dict(keys=keys, w=w, q=q, ids=ids, slots=slots, q_rows=np.array([3, 0, 1], np.int32))
+    # a float16 model: keys, queries (one head per kv head) and weights in float16, subnormal components among them
+    rng = np.random.default_rng(7120)
+    keys16 = [(rng.standard_normal((HNB, HBS, HHKV, HD)) * rng.choice([3e-6, 0.02, 1.0, 200.0], size=(HNB, HBS, HHKV, 1)))
+              .astype(np.float16) for _ in range(HL)]
+    w16 = (rng.standard_normal((HD, 128)) * 2.0).astype(np.float16)
+    q16 = (rng.standard_normal((HL, 4, HHKV, HD)) * rng.choice([1e-5, 1.0], size=(HL, 4, HHKV, 1))).astype(np.float16)
+    return dict(keys=keys, w=w, q=q, ids=ids, slots=slots, q_rows=np.array([3, 0, 1], np.int32), keys16=keys16, w16=w16, q16=q16)
 
 
 def run_hash(call, side):
@@ -289,6 +296,21 @@ def run_hash(call, side):
              side.ptr(bcodes), H_ROWS * HHKV * 16, H_ROWS - 1, side.ptr(bad_off), side.ptr(bad_len), 3, 5, HL, HHKV, 128,
              side.ptr(sc), H_ROWS, 0, None)
         out[name] = sc
+    # the float16 entry points on the same lists
+    keys16 = [side.up(k.view(np.uint16)) for k in x["keys16"]]
+    w16, q16 = side.up(x["w16"].view(np.uint16)), side.up(x["q16"].view(np.uint16))
+    t16 = side.up(np.full((HL, H_ROWS, HBS, HHKV, 16), 0xEE, np.uint8))
+    c16 = side.up(np.full((HL, H_ROWS, HHKV, 128), 77, np.int16))
+    b16 = side.up(np.full((HL, H_ROWS, HHKV, 16), 0xEE, np.uint8))
+    call("ucm_hash_encode_blocks_f16", side.pointers(keys16), HL, HNB, side.ptr(ids), side.ptr(slots), len(x["ids"]), HBS, HHKV, HD,
+         side.ptr(w16), 128, H_ROWS, side.ptr(t16), H_ROWS * HBS * HHKV * 16, side.ptr(c16), H_ROWS * HHKV * 128,
+         side.ptr(b16), H_ROWS * HHKV * 16, 0, None)
+    qc16 = side.up(np.full((HL, 3, HHKV, 16), 0xEE, np.uint8))
+    qs16 = side.up(np.full((HL, 3, 128), 77, np.int16))
+    qb16 = side.up(np.full((HL, 3, HHKV, 16), 0xEE, np.uint8))
+    call("ucm_hash_encode_queries_f16", side.ptr(q16), 4 * HHKV * HD, side.ptr(q_rows), 3, HL, HHKV, HHKV, HD, side.ptr(w16), 128,
+         side.ptr(qc16), side.ptr(qs16), side.ptr(qb16), None)
+    out.update(token_codes_f16=t16, colsum_f16=c16, block_codes_f16=b16, q_codes_f16=qc16, q_sum_f16=qs16, qbar_f16=qb16)
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x
 

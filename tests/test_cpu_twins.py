@@ -109,6 +109,27 @@ def test_hash_twins_reproduce_the_oracle(ucm):
     assert np.array_equal(got["score_sum_fp16"], got["score_sum"].astype(np.float16).astype(np.float32))
     # requests outside the declared rows were not scored; the empty one in between has nothing to score either way
     assert (got["score_sum_bad"] == -3).all() and (got["score_code_bad"] == -3).all()
+    # the float16 entry points: the signs of numpy's own float64 products of the widened values, summed in order
+    w16 = x["w16"].astype(np.float64)
+    for l in range(cpu_twins.HL):
+        for slot, blk in final.items():
+            k = x["keys16"][l][blk].astype(np.float64)                          # [tokens, kv heads, 128]
+            acc = np.zeros(k.shape[:2] + (128,))
+            for d_ in range(cpu_twins.HD):
+                acc += k[..., d_, None] * w16[d_]
+            codes = np.packbits(acc > 0, axis=-1, bitorder="little")
+            assert np.array_equal(got["token_codes_f16"][l, slot], codes)
+            assert np.array_equal(got["colsum_f16"][l, slot], O.hash_colsum(codes[None])[0])
+            assert np.array_equal(got["block_codes_f16"][l, slot], O.hash_majority(codes[None])[0])
+        for r, row in enumerate(x["q_rows"]):
+            qv = x["q16"][l, row].astype(np.float64)
+            acc = np.zeros((qv.shape[0], 128))
+            for d_ in range(cpu_twins.HD):
+                acc += qv[:, d_, None] * w16[d_]
+            qc = np.packbits(acc > 0, axis=-1, bitorder="little")
+            assert np.array_equal(got["q_codes_f16"][l, r], qc)
+            assert np.array_equal(got["qbar_f16"][l, r], qc)                    # one head per kv head: the mean is the row
+            assert np.array_equal(got["q_sum_f16"][l, r], (np.unpackbits(qc, axis=-1, bitorder="little").astype(np.int32) * 2 - 1).sum(0))
 
 
 def test_esa_twins_reproduce_the_oracle(ucm):

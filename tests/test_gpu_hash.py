@@ -484,3 +484,161 @@ def test_hash_query_codes_beyond_the_fp32_range(ucm, dev):
     pm = np.unpackbits(want_q, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
     assert np.array_equal(q_sum[0].cpu().numpy(), pm.sum(1))
     assert np.array_equal(qbar[0].cpu().numpy(), want_q)               # a group of one head: the mean is the row
+
+
+# ------------------------------------------------------------ a float16 model
+
+def exact_codes(x64, w64):
+    """Signs of the products summed in float64, d ascending: [..., 128] x [128, 128] -> uint8 [..., 16]."""
+    acc = np.zeros(x64.shape[:-1] + (128,))
+    with np.errstate(all="ignore"):
+        for d_ in range(128):
+            acc = acc + x64[..., d_, None] * w64[d_]
+    return np.packbits(acc > 0, axis=-1, bitorder="little")
+
+
+def f16_dev(a, dev):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+@pytest.mark.parametrize("hkv,bs", [(8, 128), (2, 16), (1, 32), (4, 520), (8, 272)])
+def test_hash_encode_blocks_of_a_float16_model(ucm, dev, hkv, bs):
+    """Float16 keys and weights (ucm_hash_encode_blocks_f16): the codes are the signs of the exactly accumulated
+    float16 products - the oracle's float64 sums of the widened values and numpy's own agree on that - with rows
+    that cancel exactly, rows of subnormal components (the matrix instruction takes them as they are), rows at the
+    top of float16's range, infinities and NaN."""
+    from ucm_amd import ops
+
+    n_layers, nb, rows = 2, 9, 12
+    rng = np.random.default_rng(1500 + hkv + bs)
+    w16 = (rng.standard_normal((128, 128)) * 2.0).astype(np.float16)
+    caches_h = [(rng.standard_normal((nb, bs, hkv, 128)) * rng.choice([1e-3, 1.0, 30.0], size=(nb, bs, hkv, 1))).astype(np.float16)
+                for _ in range(n_layers)]
+    for c in caches_h:
+        c[0, 0, 0, :] = 0
+        c[0, 1, 0, :] = 0
+        c[0, 1, 0, 5] = 3.0
+        c[1, 2, 0, :3] = [1.0e4, -1.0e4, 1.0e-4]
+        c[2, 3, 0, :] = -c[2, 4, 0, :]
+        c[3, 0, 0, :] = (rng.standard_normal(128) * 2e-6).astype(np.float16)          # all components subnormal
+        c[3, 1, 0, :] = (rng.standard_normal(128) * 2e-6).astype(np.float16)
+        c[3, 1, 0, 7] = 0.5                                                            # ... but one
+        c[4, 0, 0, :] = (rng.standard_normal(128) * 3e4).clip(-65504, 65504).astype(np.float16)
+        c[4, 1, 0, 9] = np.inf
+        c[4, 2, 0, 9], c[4, 2, 0, 77] = np.inf, -np.inf
+        c[4, 3, 0, 100] = np.nan
+    caches = [f16_dev(c, dev) for c in caches_h]
+    lp = ops.LayerPointers(caches)
+    ids = synth.permutation(1510, nb)[:7]
+    slots = synth.permutation(1511, rows)[:7]
+    colsum = torch.full((n_layers, rows, hkv, 128), 77, dtype=torch.int16, device=dev)
+    bcodes = torch.full((n_layers, rows, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    tcodes = torch.full((n_layers, rows, bs, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_blocks(lp, i32(ids, dev), i32(slots, dev), len(ids), f16_dev(w16, dev), bs, hkv, nb, colsum, bcodes,
+                           token_codes=tcodes)
+    torch.cuda.synchronize()
+    got_t, got_s, got_b = tcodes.cpu().numpy(), colsum.cpu().numpy(), bcodes.cpu().numpy()
+    w_f32 = w16.astype(np.float32)
+    for l in range(n_layers):
+        with np.errstate(all="ignore"):
+            want_t = O.hash_encode_f32(caches_h[l][ids].astype(np.float32), w_f32)
+        if l == 0:
+            assert np.array_equal(want_t, exact_codes(caches_h[l][ids].astype(np.float64), w16.astype(np.float64)))
+        assert np.array_equal(got_t[l][slots], want_t), l
+        assert np.array_equal(got_s[l][slots], O.hash_colsum(want_t)), l
+        assert np.array_equal(got_b[l][slots], O.hash_majority(want_t)), l
+        rest = np.setdiff1d(np.arange(rows), slots)
+        assert np.all(got_t[l][rest] == 0xEE) and np.all(got_s[l][rest] == 77) and np.all(got_b[l][rest] == 0xEE)
+    colsum2, bcodes2 = torch.zeros_like(colsum), torch.zeros_like(bcodes)
+    ops.hash_encode_blocks(lp, i32(ids, dev), i32(slots, dev), len(ids), f16_dev(w16, dev), bs, hkv, nb, colsum2, bcodes2)
+    at = torch.from_numpy(slots.astype(np.int64)).to(dev)
+    assert torch.equal(colsum2[:, at], colsum[:, at]) and torch.equal(bcodes2[:, at], bcodes[:, at])
+    # keys of one type with weights of the other are refused
+    with pytest.raises(ValueError):
+        ops.hash_encode_blocks(lp, None, None, nb, f16_dev(w16, dev).to(torch.bfloat16), bs, hkv, nb, colsum, bcodes)
+
+
+@pytest.mark.parametrize("paired", ["neighbours", "scattered"])
+def test_hash_encode_float16_projections_built_to_cancel(ucm, dev, paired):
+    """Float16 key vectors built so that their projection on one weight column cancels down to a sliver of
+    ||x|| ||w|| while the partial sums stay large: every sign, the matrix cores' and the redone ones', is the exact one."""
+    from ucm_amd import ops
+
+    hkv, bs, nb = 8, 128, 6
+    n_vec = nb * bs * hkv
+    rng = np.random.default_rng(1520)
+    w16 = (rng.standard_normal((128, 128)) * 2.0).astype(np.float16)
+    w64 = w16.astype(np.float64)
+    perm = np.arange(128) if paired == "neighbours" else rng.permutation(128)
+    cols = rng.integers(0, 128, n_vec)
+    wc = w64.T[cols]
+    rate = rng.random((n_vec, 1)) * 0.12                       # (float16 has 40 binades: the magnitudes fall off slowly)
+    a = (rng.standard_normal((n_vec, 64)) * 2.0 ** (-rate * np.arange(64))).astype(np.float16)
+    x = np.zeros((n_vec, 128), np.float16)
+    r = np.zeros(n_vec)
+    for i in range(64):
+        p0, p1 = perm[2 * i], perm[2 * i + 1]
+        w1 = np.where(wc[:, p1] == 0, 1.0, wc[:, p1])
+        t0 = a[:, i].astype(np.float64) * wc[:, p0]
+        ideal = np.clip(-(r + t0) / w1, -6e4, 6e4)
+        near = ideal.astype(np.float16)
+        cands = np.stack([near, np.nextafter(near, np.float16(np.inf)), np.nextafter(near, np.float16(-np.inf))])
+        cands = np.where(np.isfinite(cands), cands, near[None])
+        err = np.abs(r + t0 + cands.astype(np.float64) * w1)
+        y = np.take_along_axis(cands, err.argmin(0)[None], 0)[0]
+        x[:, p0], x[:, p1] = a[:, i], y
+        r = r + t0 + y.astype(np.float64) * wc[:, p1]
+    x64 = x.astype(np.float64)
+    ratio = np.abs((x64 * wc).sum(1)) / (np.linalg.norm(x64, axis=1) * np.linalg.norm(wc, axis=1))
+    assert np.median(ratio) < 2.0 ** -14 and (ratio < 2.0 ** -17).sum() > 300      # (eleven bits: the slivers are wider than bfloat16's)
+    keys_h = x.reshape(nb, bs, hkv, 128)
+    lp = ops.LayerPointers([f16_dev(keys_h, dev)])
+    colsum = torch.zeros((1, nb, hkv, 128), dtype=torch.int16, device=dev)
+    bcodes = torch.zeros((1, nb, hkv, 16), dtype=torch.uint8, device=dev)
+    tcodes = torch.zeros((1, nb, bs, hkv, 16), dtype=torch.uint8, device=dev)
+    ops.hash_encode_blocks(lp, None, None, nb, f16_dev(w16, dev), bs, hkv, nb, colsum, bcodes, token_codes=tcodes)
+    torch.cuda.synchronize()
+    want = O.hash_encode_f32(keys_h.astype(np.float32), w16.astype(np.float32))
+    assert np.array_equal(tcodes[0].cpu().numpy(), want)
+    assert np.array_equal(colsum[0].cpu().numpy(), O.hash_colsum(want))
+    assert np.array_equal(bcodes[0].cpu().numpy(), O.hash_majority(want))
+
+
+def test_hash_query_codes_of_a_float16_model(ucm, dev):
+    """Float16 queries and weights, one query head per kv head (what the plugin passes after its own group mean):
+    codes, their +-1 sums and the mean codes (the rows' own codes); rows that cancel exactly or down to one small
+    term, rows of subnormal components and rows of large ones.  Several query heads per kv head are refused."""
+    from ucm_amd import _lib, ops
+
+    hkv, n_layers, n_req = 8, 2, 6
+    rng = np.random.default_rng(1530)
+    w16 = (rng.standard_normal((128, 128)) * 2.0).astype(np.float16)
+    w16[1] = w16[0]
+    w16[5] = -w16[4]
+    q = rng.standard_normal((n_layers, n_req, hkv, 128)).astype(np.float32)
+    q[:, 0] = 0
+    q[:, 0, :, 0], q[:, 0, :, 1] = 3.0, -3.0                   # cancels exactly against the equal weight rows
+    q[:, 0, :, 4], q[:, 0, :, 5] = 0.75, 0.75
+    q[:, 0, 1::2, 2] = 2.0 ** -14                              # every second row keeps one small term
+    q[:, 1] *= 2e-6                                            # subnormal components
+    q[:, 2] *= 2000.0
+    q[:, 3] *= (2.0 ** np.linspace(-20, 12, hkv))[None, :, None]
+    q16 = q.astype(np.float16)
+    q_codes = torch.full((n_layers, n_req, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    q_sum = torch.full((n_layers, n_req, 128), 77, dtype=torch.int16, device=dev)
+    qbar = torch.full((n_layers, n_req, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(f16_dev(q16, dev), f16_dev(w16, dev), hkv, q_codes, q_sum, qbar, n_req)
+    torch.cuda.synchronize()
+    for l in range(n_layers):
+        want = exact_codes(q16[l].astype(np.float64), w16.astype(np.float64))
+        assert np.array_equal(want, O.hash_encode_f32(q16[l].astype(np.float32), w16.astype(np.float32)))
+        assert np.array_equal(q_codes[l].cpu().numpy(), want), l
+        assert np.array_equal(qbar[l].cpu().numpy(), want), l
+        pm = np.unpackbits(want, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
+        assert np.array_equal(q_sum[l].cpu().numpy(), pm.sum(1)), l
+        assert not want[0, 0::2].any() and want[0, 1::2].any() and want[1].any()
+    q32 = torch.zeros((1, 2, 32, 128), dtype=torch.float16, device=dev)
+    with pytest.raises(_lib.UcmHipError, match="one per kv head"):
+        ops.hash_encode_queries(q32, f16_dev(w16, dev), hkv, torch.zeros((1, 2, 32, 16), dtype=torch.uint8, device=dev),
+                                torch.zeros((1, 2, 128), dtype=torch.int16, device=dev),
+                                torch.zeros((1, 2, hkv, 16), dtype=torch.uint8, device=dev), 2)

@@ -51,11 +51,20 @@ def test_hash_encoder_surface(ucm, dev):
     assert pm.dtype == torch.float16 and pm.shape == (9, 128)
     want = np.unpackbits(codes.cpu().numpy(), axis=-1, bitorder="little").astype(np.float32) * 2 - 1
     assert np.array_equal(pm.float().cpu().numpy(), want)
+    # a float16 model's encoder: float16 weights, codes of the float16 products; float32 is refused
+    enc16 = HashEncoder(128, 128, torch.float16, dev)
+    assert enc16.hash_weights.dtype == torch.float16 and 1.5 < float(enc16.hash_weights.float().std()) < 2.5
+    x16 = (torch.from_numpy(synth.normal_f32(961, (5, 7, 128))).to(dev) * 3.0).to(torch.float16)
+    want16 = O.hash_encode_f32(x16.float().cpu().numpy(), enc16.hash_weights.float().cpu().numpy())
+    assert np.array_equal(enc16.compute_hash(x16).cpu().numpy(), want16)
+    with pytest.raises(ValueError):
+        HashEncoder(128, 128, torch.float32, dev)
 
 
-@pytest.mark.parametrize("device_loads,hole,delta", [(True, False, False), (False, False, False), (True, True, False),
-                                                     (True, False, True), (True, True, True)])
-def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
+@pytest.mark.parametrize("device_loads,hole,delta,model", [
+    (True, False, False, "bfloat16"), (False, False, False, "bfloat16"), (True, True, False, "bfloat16"),
+    (True, False, True, "bfloat16"), (True, True, True, "bfloat16"), (True, False, False, "float16"), (False, False, False, "float16")])
+def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta, model):
     """Prefill of 20 full blocks + 5 tokens, then decode on the sparsified block list: windows restored at step 1,
     retrieval at steps 1 and 5 picks what the oracle picks from the same keys, the chosen blocks land in the
     request's middle cache blocks in ascending order, a block filled during decode is dumped and hashed.  Once
@@ -63,7 +72,8 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
     through the per-request path that works with any store.  ``hole``: at the first retrieval the store lacks every
     other block - the load leaves those out, says so (a warning, a counter), and finds them at the next retrieval,
     by which time they are back.  ``delta``: the load moves only the picks that are not in the middle cache blocks
-    already - the same set of blocks there, each in the block the plan names, fewer bytes moved."""
+    already - the same set of blocks there, each in the block the plan names, fewer bytes moved.  ``model``: the type
+    of the cache, the queries and the hash weights (a float16 model's codes are those of its float16 products)."""
     from ucm_amd.sparse.base import INVALID_SLOT, UcmSparseRole
     from ucm_amd.sparse.factory import UcmSparseFactory
     from ucm_amd.sparse.kvcomp.kvcomp import KvComp
@@ -87,11 +97,13 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
     assert plugin.estimate_num_slots_sparsed(req) == INVALID_SLOT
     g = torch.Generator(device=dev)
     g.manual_seed(11)
-    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    model = getattr(torch, model)
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(model) for _ in range(L)]
     original = [c.clone() for c in caches]
     names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
     fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0,
             attn_metadata=ns(query_start_loc=torch.tensor([0, 1])))
+    codes_of = lambda t: O.hash_encode_f32(t.float().cpu().numpy(), w_f32)      # (either type widens exactly)
     ib = ns(req_id_to_index={"A": 0})
 
     def run_step(n_tok):
@@ -99,7 +111,7 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
         plugin.build_sparse_meta(so, {"A": req}, ib)
         qs = []
         for l in range(L):
-            q = torch.randn(n_tok, hq, d, device=dev, generator=g).to(torch.bfloat16)
+            q = torch.randn(n_tok, hq, d, device=dev, generator=g).to(model)
             qs.append(q)
             plugin.attention_begin(q, None, None, names[l], fc)
             plugin.attention_finished(q, None, None, None, names[l], fc)
@@ -114,7 +126,8 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
     key_codes = []                                           # per layer: [20, bs, hkv, 16] of the original blocks
     for l in range(L):
         assert states[l].num_blocks_hashed == 20
-        want = O.hash_encode(bf16_bits(original[l][0][full_ids[:20]]), w_f32)
+        assert plugin.hash_encoder.hash_weights.dtype == model
+        want = codes_of(original[l][0][full_ids[:20]])
         assert np.array_equal(plugin.token_codes[l, base : base + 20].cpu().numpy(), want)
         assert np.array_equal(plugin.colsum[l, base : base + 20].cpu().numpy(), O.hash_colsum(want))
         key_codes.append(want)
@@ -134,7 +147,7 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
 
     def expected(l, q, n_hashed):
         qm = q[0].view(hkv, hq // hkv, d).mean(1)                                        # bf16 group mean, as the plugin takes it
-        q_codes = O.hash_encode(bf16_bits(qm), w_f32)                                    # [hkv, 16]
+        q_codes = codes_of(qm)                                                           # [hkv, 16]
         first, end = 1, n_hashed - 2 + 1
         kc = key_codes[l][first:end].transpose(0, 2, 1, 3)                               # [n, hkv, bs, 16]
         sc = O.hash_scores_sum(q_codes, kc).astype(np.float16)                           # the reference's fp16 scores
@@ -208,12 +221,12 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta):
     req.num_tokens = n_prompt + 18
     req.num_computed_tokens = n_prompt + 10                  # 335 tokens computed: this step completes block 20
     for l in range(L):
-        caches[l][0][kept[-1]] = torch.randn(bs, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+        caches[l][0][kept[-1]] = torch.randn(bs, hkv, d, device=dev, generator=g).to(model)
     run_step(1)
     torch.cuda.synchronize()
     for l in range(L):
         assert states[l].num_blocks_hashed == 21
-        want = O.hash_encode(bf16_bits(caches[l][0][kept[-1]])[None], w_f32)
+        want = codes_of(caches[l][0][kept[-1]][None])
         assert np.array_equal(plugin.token_codes[l, base + 20].cpu().numpy(), want[0])
         assert "req_A_blk_20" in store.slot_of
     assert (plugin._dev is not None) == device_loads

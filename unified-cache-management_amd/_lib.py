@@ -40,7 +40,9 @@ SIGNATURES = {
     "ucm_prefetch_plan": [_p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _p],
     "ucm_delta_plan": [_p, _p, _p, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_encode_blocks": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _i, _p],
+    "ucm_hash_encode_blocks_f16": [_p, _i, _i, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p, _i64, _p, _i64, _p, _i64, _i, _p],
     "ucm_hash_encode_queries": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
+    "ucm_hash_encode_queries_f16": [_p, _i64, _p, _i, _i, _i, _i, _i, _p, _i, _p, _p, _p, _p],
     "ucm_hash_score_blocks": [_i, _p, _p, _p, _i64, _p, _i64, _i64, _p, _p, _i, _i64, _i, _i, _i, _p, _i64, _i, _p],
     "ucm_copy_batch": [_p, _p, _sz, _sz, _p],
     "ucm_park_rows": [_p, _i64, _p, _p, _i64, _p, _i, _sz, _p],

@@ -68,15 +68,50 @@ struct __attribute__((aligned(16))) WaveScratch {
 };
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-// sum of squares of 8 bf16 values added to s (v_dot2c_f32_bf16); only used for error bounds
+// Keys, queries and weights are bfloat16 (kF16 false) or float16 (true): a model's own type.  What the two share:
+// 16-bit elements with the sign in bit 15, products of two of them exact in fp32 (8 x 8 or 11 x 11 significant
+// bits; the smallest float16 product, 2^-48, is a normal fp32 number, and the matrix instruction takes float16
+// subnormals as they are), a matrix instruction of the same shape.
+template <bool kF16>
+__device__ __forceinline__ float dot2_self(unsigned e, float s)
+{
+    if (kF16) { const f16x2 p = __builtin_bit_cast(f16x2, e); return __builtin_amdgcn_fdot2(p, p, s, false); }
+    const bf16x2 p = __builtin_bit_cast(bf16x2, e);
+    return __builtin_amdgcn_fdot2_f32_bf16(p, p, s, false);
+}
+
+// the two 16-bit elements of a word, widened exactly
+template <bool kF16>
+__device__ __forceinline__ float widen_lo(unsigned e)
+{
+    if (kF16) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(e & 0xffffu))); }
+    return __uint_as_float(e << 16);
+}
+template <bool kF16>
+__device__ __forceinline__ float widen_hi(unsigned e)
+{
+    if (kF16) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(e >> 16))); }
+    return __uint_as_float(e & 0xffff0000u);
+}
+
+template <bool kF16>
+__device__ __forceinline__ f32x16 mfma_32x32x16(const u32x4 a, const u32x4 b, const f32x16 c)
+{
+    if (kF16) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0); }
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// sum of squares of 8 elements added to s (v_dot2c_f32_bf16 / v_dot2_f32_f16); only used for error bounds
+template <bool kF16>
 __device__ __forceinline__ float norm2_acc(const u32x4 v, float s)
 {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const unsigned e = v[j];   // (a bit_cast of v[j] itself reads element 0 four times with this compiler)
-        const bf16x2 p = __builtin_bit_cast(bf16x2, e);
-        s = __builtin_amdgcn_fdot2_f32_bf16(p, p, s, false);
+        s = dot2_self<kF16>(e, s);
     }
     return s;
 }
@@ -86,6 +121,7 @@ __device__ __forceinline__ float norm2_acc(const u32x4 v, float s)
 // rounding is symmetric, so the sum is the oracle's with its sign flipped).
 // Both 256-byte rows are fetched with sixteen 16-byte loads issued together, so
 // the redo costs one memory latency, not 128 of them.
+template <bool kF16>
 __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict__ x,
                                                const unsigned short* __restrict__ neg_wt_col)
 {
@@ -101,10 +137,9 @@ __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict_
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const unsigned xa = xv[i][j], wa = wv[i][j];
-            // (a product of two bf16 values is exact in fp64, so the fused form rounds exactly as multiply-then-add does)
-            acc = __builtin_fma(static_cast<double>(__uint_as_float(xa << 16)), static_cast<double>(__uint_as_float(wa << 16)), acc);
-            acc = __builtin_fma(static_cast<double>(__uint_as_float(xa & 0xffff0000u)),
-                                static_cast<double>(__uint_as_float(wa & 0xffff0000u)), acc);
+            // (a product of two such values is exact in fp64, so the fused form rounds exactly as multiply-then-add does)
+            acc = __builtin_fma(static_cast<double>(widen_lo<kF16>(xa)), static_cast<double>(widen_lo<kF16>(wa)), acc);
+            acc = __builtin_fma(static_cast<double>(widen_hi<kF16>(xa)), static_cast<double>(widen_hi<kF16>(wa)), acc);
         }
     }
     return acc < 0.0;
@@ -113,6 +148,7 @@ __device__ __forceinline__ bool exact_positive(const unsigned short* __restrict_
 // Queued results are redone exactly, 64 at a time, one per lane.  Entries are
 // queued after their tile's code words were stored, so the fix goes to memory.
 // Kept out of line: it has several call sites and runs rarely.
+template <bool kF16>
 __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen, int lane,
                                                       const unsigned short* __restrict__ blk,
                                                       const unsigned short* __restrict__ neg_wt,
@@ -128,7 +164,7 @@ __device__ __attribute__((noinline)) void drain_exact(WaveScratch& ws, int qlen,
         if (base + lane < qlen) {
             const unsigned e = ws.queue[base + lane];
             const unsigned v = e >> 8, col = (e >> 1) & 127u, prov = e & 1u;
-            const bool pos = exact_positive(blk + static_cast<size_t>(v) * kDim, &neg_wt[row_of_col(col) * kWtStride]);
+            const bool pos = exact_positive<kF16>(blk + static_cast<size_t>(v) * kDim, &neg_wt[row_of_col(col) * kWtStride]);
             if (static_cast<unsigned>(pos) != prov) {
                 if (tc_out) { atomicXor(&tc_out[v * 4 + (col >> 5)], 1u << (col & 31)); }
                 atomicAdd(&ws.colsum[v % kv_heads][col], pos ? 1 : -1);
@@ -238,7 +274,7 @@ __device__ __forceinline__ void planes_flush_owner(unsigned (&pl)[kPlanes], int*
 // Workgroups are persistent over the list of blocks so that staging the weight
 // matrix is paid once per workgroup, not once per four blocks.
 // grid: x = workgroup (wave w of workgroup g takes items g*kWaves + w, then steps by the grid), y = layer
-template <bool kTokenCodes>
+template <bool kTokenCodes, bool kF16>
 __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
     const void* const* __restrict__ k_layers, const int32_t* __restrict__ block_ids,
     const int32_t* __restrict__ slots, unsigned num_blocks, unsigned n_items, unsigned rows,
@@ -267,7 +303,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         float s = 0.0f;
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            s = norm2_acc(*reinterpret_cast<const u32x4*>(&wt[c * kWtStride + part * 64 + k * 8]), s);
+            s = norm2_acc<kF16>(*reinterpret_cast<const u32x4*>(&wt[c * kWtStride + part * 64 + k * 8]), s);
         }
         s += __shfl_xor(s, 1, 64);
         if (part == 0) { w_norm2[c] = s; }
@@ -378,7 +414,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         };
         auto drain_queue = [&]() {
             store_codes();
-            drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads);
+            drain_exact<kF16>(ws, qlen, lane, blk, wt, tc_out, kv_heads);
             qlen = 0;
             if (kTokenCodes) {
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the patches have been applied
@@ -400,19 +436,19 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
         // the LDS reads is gone.  With token codes the fragments are requested first thing in a tile, ahead of
         // the wait for the keys and of their norms.
         constexpr bool kResidentFirst = !kTokenCodes;
-        bf16x8 wf_first[4];
+        u32x4 wf_first[4];
         if (kResidentFirst) {
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-                wf_first[nb] = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 8]);
+                wf_first[nb] = *reinterpret_cast<const u32x4*>(&wt[(nb * 32 + lr) * kWtStride + half * 8]);
             }
         }
         auto process = [&](u32x4 (&kb)[8], unsigned tile) {
-            bf16x8 wf[2][4];
+            u32x4 wf[2][4];
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
                 if (kResidentFirst) { wf[0][nb] = wf_first[nb]; }
-                else { wf[0][nb] = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 8]); }
+                else { wf[0][nb] = *reinterpret_cast<const u32x4*>(&wt[(nb * 32 + lr) * kWtStride + half * 8]); }
             }
             __builtin_amdgcn_sched_barrier(0);
             store_codes();
@@ -425,8 +461,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const unsigned e = kb[ks][j];
-                    const bf16x2 p = __builtin_bit_cast(bf16x2, e);
-                    xp[j] = __builtin_amdgcn_fdot2_f32_bf16(p, p, xp[j], false);
+                    xp[j] = dot2_self<kF16>(e, xp[j]);
                 }
             }
             float xn2 = (xp[0] + xp[1]) + (xp[2] + xp[3]);
@@ -442,17 +477,17 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
             // the weight fragments of a step are read from LDS while the matrix instructions of the step before run
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                const bf16x8 kf = __builtin_bit_cast(bf16x8, kb[ks]);
+                const u32x4 kf = kb[ks];
                 if (ks < 7) {
 #pragma unroll
                     for (int nb = 0; nb < 4; ++nb) {
-                        wf[(ks + 1) & 1][nb] = *reinterpret_cast<const bf16x8*>(&wt[(nb * 32 + lr) * kWtStride + half * 8 + (ks + 1) * 16]);
+                        wf[(ks + 1) & 1][nb] = *reinterpret_cast<const u32x4*>(&wt[(nb * 32 + lr) * kWtStride + half * 8 + (ks + 1) * 16]);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int nb = 0; nb < 4; ++nb) {
-                    acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[ks & 1][nb], kf, acc[nb], 0, 0, 0);
+                    acc[nb] = mfma_32x32x16<kF16>(wf[ks & 1][nb], kf, acc[nb]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -562,7 +597,7 @@ __global__ __launch_bounds__(kThreads, 2) void hash_encode_blocks_kernel(
             }
         }
         store_codes();
-        if (qlen > 0) { drain_exact(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
+        if (qlen > 0) { drain_exact<kF16>(ws, qlen, lane, blk, wt, tc_out, kv_heads); }
         flush_planes_last();
 
         // ---- block summaries
@@ -619,24 +654,28 @@ __device__ __forceinline__ float wave_max32(float m)
     return m;
 }
 
+template <bool kF16>
 __device__ __forceinline__ void widen8(const u32x4 v, float (&x)[8])
 {
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) { x[2 * j] = __uint_as_float(v[j] << 16); x[2 * j + 1] = __uint_as_float(v[j] & 0xffff0000u); }
+    for (int j = 0; j < 4; ++j) { x[2 * j] = widen_lo<kF16>(w[j]); x[2 * j + 1] = widen_hi<kF16>(w[j]); }
 }
 
 // acc += x[0..7] . W[d0 .. d0+7][col], d ascending (exact products, fp64 sums: the oracle's arithmetic)
+template <bool kF16>
 __device__ __forceinline__ double dot8_exact(const float (&x)[8], const unsigned short* w_s, unsigned d0, unsigned col, double acc)
 {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        const float wf = __uint_as_float(static_cast<unsigned>(w_s[(d0 + j) * kBits + col]) << 16);
+        const float wf = widen_lo<kF16>(static_cast<unsigned>(w_s[(d0 + j) * kBits + col]));
         acc += static_cast<double>(x[j]) * static_cast<double>(wf);
     }
     return acc;
 }
 
 // exact sign of a query row . column: the row is fetched in four groups of four 16-byte pieces
+template <bool kF16>
 __device__ __forceinline__ bool row_exact_positive(const unsigned short* __restrict__ row, const unsigned short* w_s, unsigned col)
 {
     double acc = 0.0;
@@ -648,30 +687,35 @@ __device__ __forceinline__ bool row_exact_positive(const unsigned short* __restr
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             float x[8];
-            widen8(xv[k], x);
-            acc = dot8_exact(x, w_s, 32 * c + 8 * k, col, acc);
+            widen8<kF16>(xv[k], x);
+            acc = dot8_exact<kF16>(x, w_s, 32 * c + 8 * k, col, acc);
         }
     }
     return acc > 0.0;
 }
 
 // exact sign of a staged group mean . column; (hi + mid) + lo is the mean again, exactly
+template <bool kF16>
 __device__ __forceinline__ bool mean_exact_positive(const QueryLds& s, unsigned h, unsigned col)
 {
     double acc = 0.0;
 #pragma unroll 1
     for (int k = 0; k < kDim / 8; ++k) {
         float hi[8], mid[8], lo[8], x[8];
-        widen8(*reinterpret_cast<const u32x4*>(&s.mean[0][h][8 * k]), hi);
-        widen8(*reinterpret_cast<const u32x4*>(&s.mean[1][h][8 * k]), mid);
-        widen8(*reinterpret_cast<const u32x4*>(&s.mean[2][h][8 * k]), lo);
+        widen8<kF16>(*reinterpret_cast<const u32x4*>(&s.mean[0][h][8 * k]), hi);
+        widen8<kF16>(*reinterpret_cast<const u32x4*>(&s.mean[1][h][8 * k]), mid);
+        widen8<kF16>(*reinterpret_cast<const u32x4*>(&s.mean[2][h][8 * k]), lo);
 #pragma unroll
         for (int j = 0; j < 8; ++j) { x[j] = (hi[j] + mid[j]) + lo[j]; }
-        acc = dot8_exact(x, s.w, 8 * k, col, acc);
+        acc = dot8_exact<kF16>(x, s.w, 8 * k, col, acc);
     }
     return acc > 0.0;
 }
 
+// kF16: float16 queries and weights, one query head per kv head only (host checked): the "mean" is the row itself,
+// which is its own first term - an fp32 mean of several float16 rows does not split into float16 terms exactly
+// (its low bits fall below what float16 can hold).
+template <bool kF16>
 __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
     const unsigned short* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows,
     unsigned q_heads, unsigned kv_heads, const unsigned short* __restrict__ w, unsigned n_req,
@@ -701,11 +745,11 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         if (h < kv_heads) {
             const unsigned short* first = qp + (h * g) * kDim + 8 * piece;
             float x[8];
-            widen8(ucm::gload16(first), x);
+            widen8<kF16>(ucm::gload16(first), x);
 #pragma unroll 4
             for (unsigned rr = 1; rr < g; ++rr) {
                 float y[8];
-                widen8(ucm::gload16(first + rr * kDim), y);
+                widen8<kF16>(ucm::gload16(first + rr * kDim), y);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) { x[j] = x[j] + y[j]; }
             }
@@ -713,13 +757,18 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float xm = g != 1 ? x[j] * inv : x[j];
-                const float hi = __uint_as_float(__float_as_uint(xm) & 0xffff0000u);
-                const float r1 = xm - hi;                                     // exact: the trailing bits of xm
-                const float mid = __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
-                const float lo = r1 - mid;                                    // exact, at most 8 significant bits
-                term[0][j] = __float_as_uint(hi) >> 16;
-                term[1][j] = __float_as_uint(mid) >> 16;
-                term[2][j] = __float_as_uint(lo) >> 16;
+                if (kF16) {                                                   // (g == 1: xm is a float16 value)
+                    term[0][j] = __builtin_bit_cast(unsigned short, static_cast<_Float16>(xm));
+                    term[1][j] = term[2][j] = 0u;
+                } else {
+                    const float hi = __uint_as_float(__float_as_uint(xm) & 0xffff0000u);
+                    const float r1 = xm - hi;                                 // exact: the trailing bits of xm
+                    const float mid = __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+                    const float lo = r1 - mid;                                // exact, at most 8 significant bits
+                    term[0][j] = __float_as_uint(hi) >> 16;
+                    term[1][j] = __float_as_uint(mid) >> 16;
+                    term[2][j] = __float_as_uint(lo) >> 16;
+                }
                 nx2 = nx2 + xm * xm;
             }
 #pragma unroll
@@ -752,7 +801,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         for (int j = 0; j < 4; ++j) {
             wb[ks][j] = static_cast<unsigned>(wp[(2 * j) * kBits]) | (static_cast<unsigned>(wp[(2 * j + 1) * kBits]) << 16);
         }
-        nw2 = norm2_acc(wb[ks], nw2);
+        nw2 = norm2_acc<kF16>(wb[ks], nw2);
     }
     nw2 += __shfl_xor(nw2, 32, 64);                      // the column's squared norm
 
@@ -766,7 +815,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         for (int ks = 0; ks < 8; ++ks) {
             if (m_in < q_heads) { xa[ks] = ucm::gload16(qp + m_in * kDim + 16 * ks + 8 * half); }
             else { xa[ks] = u32x4{0u, 0u, 0u, 0u}; }
-            nx2 = norm2_acc(xa[ks], nx2);
+            nx2 = norm2_acc<kF16>(xa[ks], nx2);
         }
         nx2 += __shfl_xor(nx2, 32, 64);
         const float max2 = wave_max32(nx2);
@@ -777,8 +826,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         for (int i = 0; i < 16; ++i) { acc[i] = 0.0f; }
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xa[ks]), __builtin_bit_cast(bf16x8, wb[ks]),
-                                                          acc, 0, 0, 0);
+            acc = mfma_32x32x16<kF16>(xa[ks], wb[ks], acc);
         }
         // result register i is row t0 + 8*(i/4) + 4*half + i%4
         unsigned positive = 0, redo = 0;
@@ -792,7 +840,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
             const unsigned i = static_cast<unsigned>(__builtin_ctz(redo));
             redo &= redo - 1;
             const unsigned m = t0 + 8 * (i >> 2) + 4 * half + (i & 3);
-            const bool pos = row_exact_positive(qp + m * kDim, s.w, col);
+            const bool pos = row_exact_positive<kF16>(qp + m * kDim, s.w, col);
             positive = (positive & ~(1u << i)) | (static_cast<unsigned>(pos) << i);
         }
 #pragma unroll
@@ -821,8 +869,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         for (int ks = 0; ks < 8; ++ks) {
             u32x4 xa = u32x4{0u, 0u, 0u, 0u};
             if (feeds) { xa = *reinterpret_cast<const u32x4*>(&s.mean[term][h_in][16 * ks + 8 * half]); }
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, xa), __builtin_bit_cast(bf16x8, wb[ks]),
-                                                          acc, 0, 0, 0);
+            acc = mfma_32x32x16<kF16>(xa, wb[ks], acc);
         }
         const float max2 = fmaxf(s.mean_max2[0], s.mean_max2[1]);
         const bool all_exact = (max2 > 0.0f && !(max2 >= 0x1p-120f)) || !(max2 < __builtin_inff());   // tiny norms, or none that is finite
@@ -837,7 +884,7 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
         while (redo) {
             const unsigned i = static_cast<unsigned>(__builtin_ctz(redo));
             redo &= redo - 1;
-            const bool pos = mean_exact_positive(s, 4 * half + i, col);
+            const bool pos = mean_exact_positive<kF16>(s, 4 * half + i, col);
             positive = (positive & ~(1u << i)) | (static_cast<unsigned>(pos) << i);
         }
 #pragma unroll
@@ -974,12 +1021,14 @@ __global__ __launch_bounds__(256) void hash_code_score_kernel(
 
 }  // namespace
 
-extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers, int num_blocks,
-                                      const int32_t* block_ids, const int32_t* slots, int n, int block_size,
-                                      int kv_heads, int head_dim, const void* w_bf16, int bits, int rows,
-                                      uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
-                                      int64_t colsum_layer_stride, uint8_t* block_codes,
-                                      int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream)
+namespace {
+
+int hash_encode_blocks(bool f16, const void* const* k_layers, int n_layers, int num_blocks,
+                       const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                       int kv_heads, int head_dim, const void* w_bf16, int bits, int rows,
+                       uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                       int64_t colsum_layer_stride, uint8_t* block_codes,
+                       int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream)
 {
     UCM_REQUIRE(n >= 0, "ucm_hash_encode_blocks: n=%d", n);
     UCM_REQUIRE(workgroups >= 0 && workgroups <= (1 << 20), "ucm_hash_encode_blocks: workgroups=%d", workgroups);
@@ -1005,16 +1054,50 @@ extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers,
         static_cast<unsigned>(block_size), static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16),  \
         reinterpret_cast<unsigned*>(token_codes), token_codes_layer_stride / 4, colsum, colsum_layer_stride,             \
         reinterpret_cast<unsigned*>(block_codes), block_codes_layer_stride / 4
-    if (token_codes) { hipLaunchKernelGGL(hash_encode_blocks_kernel<true>, UCM_HASH_ENCODE_ARGS); }
-    else { hipLaunchKernelGGL(hash_encode_blocks_kernel<false>, UCM_HASH_ENCODE_ARGS); }
+    if (f16) {
+        if (token_codes) { hipLaunchKernelGGL((hash_encode_blocks_kernel<true, true>), UCM_HASH_ENCODE_ARGS); }
+        else { hipLaunchKernelGGL((hash_encode_blocks_kernel<false, true>), UCM_HASH_ENCODE_ARGS); }
+    } else {
+        if (token_codes) { hipLaunchKernelGGL((hash_encode_blocks_kernel<true, false>), UCM_HASH_ENCODE_ARGS); }
+        else { hipLaunchKernelGGL((hash_encode_blocks_kernel<false, false>), UCM_HASH_ENCODE_ARGS); }
+    }
 #undef UCM_HASH_ENCODE_ARGS
     UCM_LAUNCH_CHECK("ucm_hash_encode_blocks");
 }
 
-extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows,
-                                       int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
-                                       const void* w_bf16, int bits, uint8_t* q_codes, int16_t* q_sum,
-                                       uint8_t* qbar_codes, ucm_stream_t stream)
+}  // namespace
+
+extern "C" int ucm_hash_encode_blocks(const void* const* k_layers, int n_layers, int num_blocks,
+                                      const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                                      int kv_heads, int head_dim, const void* w_bf16, int bits, int rows,
+                                      uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                                      int64_t colsum_layer_stride, uint8_t* block_codes,
+                                      int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream)
+{
+    return hash_encode_blocks(false, k_layers, n_layers, num_blocks, block_ids, slots, n, block_size, kv_heads, head_dim, w_bf16,
+                              bits, rows, token_codes, token_codes_layer_stride, colsum, colsum_layer_stride, block_codes,
+                              block_codes_layer_stride, workgroups, stream);
+}
+
+extern "C" int ucm_hash_encode_blocks_f16(const void* const* k_layers, int n_layers, int num_blocks,
+                                          const int32_t* block_ids, const int32_t* slots, int n, int block_size,
+                                          int kv_heads, int head_dim, const void* w_f16, int bits, int rows,
+                                          uint8_t* token_codes, int64_t token_codes_layer_stride, int16_t* colsum,
+                                          int64_t colsum_layer_stride, uint8_t* block_codes,
+                                          int64_t block_codes_layer_stride, int workgroups, ucm_stream_t stream)
+{
+    return hash_encode_blocks(true, k_layers, n_layers, num_blocks, block_ids, slots, n, block_size, kv_heads, head_dim, w_f16,
+                              bits, rows, token_codes, token_codes_layer_stride, colsum, colsum_layer_stride, block_codes,
+                              block_codes_layer_stride, workgroups, stream);
+}
+
+
+namespace {
+
+int hash_encode_queries(bool f16, const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows,
+                        int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
+                        const void* w_bf16, int bits, uint8_t* q_codes, int16_t* q_sum,
+                        uint8_t* qbar_codes, ucm_stream_t stream)
 {
     UCM_REQUIRE(n_req >= 0 && n_layers > 0 && n_layers <= 65535, "ucm_hash_encode_queries: n_req=%d n_layers=%d", n_req, n_layers);
     if (n_req == 0) { return UCM_OK; }
@@ -1027,13 +1110,38 @@ extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_strid
                 static_cast<long long>(q_layer_stride));
     UCM_SUPPORTED(q_heads <= kMaxQHeads && kv_heads <= kMaxHeads, "ucm_hash_encode_queries: q_heads=%d kv_heads=%d (at most %d and %d)",
                   q_heads, kv_heads, kMaxQHeads, kMaxHeads);
-    hipLaunchKernelGGL(hash_query_kernel, dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),
-                       static_cast<const unsigned short*>(q_bf16), q_layer_stride, q_rows,
-                       static_cast<unsigned>(q_heads), static_cast<unsigned>(kv_heads),
-                       static_cast<const unsigned short*>(w_bf16), static_cast<unsigned>(n_req),
-                       reinterpret_cast<unsigned*>(q_codes), q_sum, reinterpret_cast<unsigned*>(qbar_codes));
+    UCM_SUPPORTED(!f16 || q_heads == kv_heads, "ucm_hash_encode_queries_f16: q_heads=%d kv_heads=%d (float16 queries: one per kv head, "
+                  "the caller's own group mean)", q_heads, kv_heads);
+#define UCM_HASH_QUERY_ARGS dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),                    \
+        static_cast<const unsigned short*>(q_bf16), q_layer_stride, q_rows, static_cast<unsigned>(q_heads),          \
+        static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16), static_cast<unsigned>(n_req),   \
+        reinterpret_cast<unsigned*>(q_codes), q_sum, reinterpret_cast<unsigned*>(qbar_codes)
+    if (f16) { hipLaunchKernelGGL(hash_query_kernel<true>, UCM_HASH_QUERY_ARGS); }
+    else { hipLaunchKernelGGL(hash_query_kernel<false>, UCM_HASH_QUERY_ARGS); }
+#undef UCM_HASH_QUERY_ARGS
     UCM_LAUNCH_CHECK("ucm_hash_encode_queries");
 }
+
+}  // namespace
+
+extern "C" int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const int32_t* q_rows,
+                                       int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
+                                       const void* w_bf16, int bits, uint8_t* q_codes, int16_t* q_sum,
+                                       uint8_t* qbar_codes, ucm_stream_t stream)
+{
+    return hash_encode_queries(false, q_bf16, q_layer_stride, q_rows, n_req, n_layers, q_heads, kv_heads, head_dim, w_bf16, bits,
+                               q_codes, q_sum, qbar_codes, stream);
+}
+
+extern "C" int ucm_hash_encode_queries_f16(const void* q_f16, int64_t q_layer_stride, const int32_t* q_rows,
+                                           int n_req, int n_layers, int q_heads, int kv_heads, int head_dim,
+                                           const void* w_f16, int bits, uint8_t* q_codes, int16_t* q_sum,
+                                           uint8_t* qbar_codes, ucm_stream_t stream)
+{
+    return hash_encode_queries(true, q_f16, q_layer_stride, q_rows, n_req, n_layers, q_heads, kv_heads, head_dim, w_f16, bits,
+                               q_codes, q_sum, qbar_codes, stream);
+}
+
 
 extern "C" int ucm_hash_score_blocks(int mode, const int16_t* q_sum, const uint8_t* qbar_codes,
                                      const int16_t* colsum, int64_t colsum_layer_stride,

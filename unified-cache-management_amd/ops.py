@@ -114,11 +114,6 @@ class LayerPointers:
         return self.table.data_ptr() + 8 * first_layer
 
 
-def _bf16_keys_only(layers: LayerPointers, what: str) -> None:
-    if layers.tensors and layers.tensors[0].dtype == torch.float16:
-        raise ValueError(f"{what} reads bfloat16 key caches only (a float16 cache is taken by block_mean, kvstar_block_repre and the scoring calls)")
-
-
 def block_mean(k_layers: LayerPointers, block_ids: torch.Tensor, slots: torch.Tensor, repre: torch.Tensor,
                block_size: int, kv_heads: int, head_dim: int, num_blocks: int, mode: int = MEAN_F32,
                first_layer: int = 0, n_layers: Optional[int] = None) -> None:
@@ -444,12 +439,14 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
                        n: int, w: torch.Tensor, block_size: int, kv_heads: int, num_blocks: int,
                        colsum: torch.Tensor, block_codes: torch.Tensor,
                        token_codes: Optional[torch.Tensor] = None, workgroups: int = 0) -> None:
-    """w bf16 [128, 128]; colsum int16 [L, rows, kv_heads, 128]; block_codes uint8 [L, rows, kv_heads, 16];
-    token_codes uint8 [L, rows, block_size, kv_heads, 16] or None; workgroups: persistent workgroups over all
-    layers, 0 = the library's choice (benchmarks and tests)."""
-    _bf16_keys_only(k_layers, "hash_encode_blocks")
+    """w [128, 128] in the caches' type (bfloat16 or float16); colsum int16 [L, rows, kv_heads, 128]; block_codes uint8
+    [L, rows, kv_heads, 16]; token_codes uint8 [L, rows, block_size, kv_heads, 16] or None; workgroups: persistent
+    workgroups over all layers, 0 = the library's choice (benchmarks and tests)."""
+    key_dtype = k_layers.tensors[0].dtype if k_layers.tensors else w.dtype
+    if key_dtype not in (torch.bfloat16, torch.float16) or w.dtype != key_dtype:
+        raise ValueError("hash_encode_blocks takes bfloat16 or float16 key caches and weights of the same type")
     if w.shape != (128, 128):
-        raise ValueError("w must be [128, 128] bfloat16")
+        raise ValueError("w must be [128, 128]")
     n_layers, rows = colsum.shape[0], colsum.shape[1]
     if colsum.shape != (n_layers, rows, kv_heads, 128) or block_codes.shape != (n_layers, rows, kv_heads, 16):
         raise ValueError("colsum [L,rows,Hkv,128] / block_codes [L,rows,Hkv,16] expected")
@@ -457,8 +454,9 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
         raise ValueError("one output layer per cache layer")
     if token_codes is not None and token_codes.shape != (n_layers, rows, block_size, kv_heads, 16):
         raise ValueError("token_codes must be [L, rows, block_size, kv_heads, 16]")
-    _lib.call("ucm_hash_encode_blocks", k_layers.ptr(), n_layers, num_blocks, _opt(block_ids, torch.int32, "block_ids"),
-              _opt(slots, torch.int32, "slots"), n, block_size, kv_heads, 128, _dev(w, torch.bfloat16, "w"), 128, rows,
+    _lib.call("ucm_hash_encode_blocks_f16" if key_dtype == torch.float16 else "ucm_hash_encode_blocks", k_layers.ptr(), n_layers,
+              num_blocks, _opt(block_ids, torch.int32, "block_ids"),
+              _opt(slots, torch.int32, "slots"), n, block_size, kv_heads, 128, _dev(w, key_dtype, "w"), 128, rows,
               _opt(token_codes, torch.uint8, "token_codes"), 0 if token_codes is None else token_codes.stride(0),
               _dev(colsum, torch.int16, "colsum"), colsum.stride(0), _dev(block_codes, torch.uint8, "block_codes"),
               block_codes.stride(0), int(workgroups), _stream())
@@ -466,16 +464,18 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
 
 def hash_encode_queries(q: torch.Tensor, w: torch.Tensor, kv_heads: int, q_codes: torch.Tensor, q_sum: torch.Tensor,
                         qbar_codes: torch.Tensor, n_req: int, q_rows: Optional[torch.Tensor] = None) -> None:
-    """q bf16 [L, rows, q_heads, 128]; q_codes u8 [L, n_req, q_heads, 16]; q_sum int16 [L, n_req, 128];
-    qbar_codes u8 [L, n_req, kv_heads, 16]."""
+    """q bf16 [L, rows, q_heads, 128] (or float16 with float16 weights and q_heads == kv_heads); q_codes u8
+    [L, n_req, q_heads, 16]; q_sum int16 [L, n_req, 128]; qbar_codes u8 [L, n_req, kv_heads, 16]."""
     n_layers, _, q_heads, d = q.shape
+    if q.dtype not in (torch.bfloat16, torch.float16) or w.dtype != q.dtype:
+        raise ValueError("hash_encode_queries takes bfloat16 or float16 queries and weights of the same type")
     if q_codes.shape != (n_layers, n_req, q_heads, 16) or q_sum.shape != (n_layers, n_req, 128) \
             or qbar_codes.shape != (n_layers, n_req, kv_heads, 16):
         raise ValueError("query code outputs have the wrong shape")
     if q_rows is None and q.shape[1] < n_req:
         raise ValueError("q has fewer rows than requests")
-    _lib.call("ucm_hash_encode_queries", _dev(q, torch.bfloat16, "q"), q.stride(0), _opt(q_rows, torch.int32, "q_rows"),
-              n_req, n_layers, q_heads, kv_heads, d, _dev(w, torch.bfloat16, "w"), 128,
+    _lib.call("ucm_hash_encode_queries_f16" if q.dtype == torch.float16 else "ucm_hash_encode_queries", _dev(q, q.dtype, "q"),
+              q.stride(0), _opt(q_rows, torch.int32, "q_rows"), n_req, n_layers, q_heads, kv_heads, d, _dev(w, q.dtype, "w"), 128,
               _dev(q_codes, torch.uint8, "q_codes"), _dev(q_sum, torch.int16, "q_sum"),
               _dev(qbar_codes, torch.uint8, "qbar_codes"), _stream())
 

@@ -201,7 +201,7 @@ class KvCompDevicePath:
             q = q.view(b, h, -1, d).mean(2)
         elif hq < h:
             q = torch.repeat_interleave(q, h // hq, 1)
-        q = q.to(torch.bfloat16).reshape(1, b, h, d).contiguous()
+        q = q.to(p.hash_encoder.dtype).reshape(1, b, h, d).contiguous()
         q_codes, q_sum, qbar = self.q_codes[:, :b], self.q_sum[:, :b], self.qbar[:, :b]
         ops.hash_encode_queries(q, p.hash_encoder.hash_weights, h, q_codes, q_sum, qbar, b)
         l = slice(layer_id, layer_id + 1)

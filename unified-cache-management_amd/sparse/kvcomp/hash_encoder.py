@@ -12,7 +12,8 @@ that library's accumulation order gives; here the projection runs on the matrix
 cores and every sign is that of the exactly accumulated product (results within
 rounding of zero are redone in fp64), so codes do not depend on a GEMM's
 summation order.  The kernels are built for ``input_dim == hash_bits == 128`` in
-bfloat16; anything else is refused, there is no other path.
+bfloat16 or float16 (the model's type: keys, queries and weights alike); anything
+else is refused, there is no other path.
 """
 from __future__ import annotations
 
@@ -29,8 +30,8 @@ class HashEncoder:
             raise ValueError("hash_bits must be a multiple of 8")
         if input_dim != 128 or hash_bits != 128:
             raise ValueError(f"the hash kernels are built for input_dim = hash_bits = 128, got {input_dim} / {hash_bits}")
-        if dtype != torch.bfloat16:
-            raise ValueError(f"the hash kernels take bfloat16 keys, queries and weights, got {dtype}")
+        if dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError(f"the hash kernels take bfloat16 or float16 keys, queries and weights, got {dtype}")
         self.input_dim, self.hash_bits = input_dim, hash_bits
         self.hash_numbers = hash_bits // 8
         self.dtype, self.device = dtype, torch.device(device)

@@ -332,7 +332,7 @@ class KvComp(UcmSparseBase):
         request and returns the top_k of them, as offsets from ``first``, ascending."""
         dev = self.colsum.device
         t, h, d = query.shape
-        q = query.to(torch.bfloat16).reshape(1, 1, t * h, d).contiguous()
+        q = query.to(self.hash_encoder.dtype).reshape(1, 1, t * h, d).contiguous()
         q_codes = torch.empty((1, 1, t * h, 16), dtype=torch.uint8, device=dev)
         q_sum = torch.empty((1, 1, 128), dtype=torch.int16, device=dev)
         qbar = torch.empty((1, 1, h, 16), dtype=torch.uint8, device=dev)
