@@ -39,8 +39,8 @@ def _config(hq, hkv, d, layers, bs, max_model_len, max_num_seqs, esa_cfg):
               kv_transfer_config=ns(kv_connector_extra_config={"ucm_sparse_config": {"ESA": esa_cfg}}))
 
 
-@pytest.mark.parametrize("pool_where", ["cuda", "pinned"])
-def test_esa_device_path_flow(ucm, dev, pool_where):
+@pytest.mark.parametrize("pool_where,model_dtype", [("cuda", "bfloat16"), ("pinned", "bfloat16"), ("cuda", "float16")])
+def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
     from ucm_amd import ops
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.esa.esa import ESA
@@ -59,7 +59,8 @@ def test_esa_device_path_flow(ucm, dev, pool_where):
     plugin = ESA(cfg, UcmSparseRole.WORKER, store=store)
     g = torch.Generator(device=dev)
     g.manual_seed(5)
-    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+    model_dtype = getattr(torch, model_dtype)       # the cache's and the queries' type: the means are rounded to it
+    caches = [torch.randn(2, nb, bs, hkv, d, device=dev, generator=g).to(model_dtype) for _ in range(L)]
     original = [c.clone() for c in caches]
     all_layers = ops.LayerPointers(caches)
     names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
@@ -94,7 +95,7 @@ def test_esa_device_path_flow(ucm, dev, pool_where):
         ib = ns(req_id_to_index={r.request_id: j for j, r in enumerate(active)})
         md = ns(query_start_loc=torch.tensor(qsl + [pos]))
         so = ns(num_scheduled_tokens=sched)
-        qs = [torch.randn(pos, hq, d, device=dev, generator=g).to(torch.bfloat16) for _ in range(L)]
+        qs = [torch.randn(pos, hq, d, device=dev, generator=g).to(model_dtype) for _ in range(L)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         plugin.build_sparse_meta(so, {r.request_id: r for r in active}, ib, md)
@@ -145,7 +146,8 @@ def test_esa_device_path_flow(ucm, dev, pool_where):
                 for l in range(L):
                     kc = original[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
                     want = np.zeros((plugin.num_slots, hkv * d), np.float32)
-                    O.block_mean_paged(kc, ids[:sparse_range], m["slots"][l], want, round_bf16=True)
+                    O.block_mean_paged(kc, ids[:sparse_range], m["slots"][l], want, round_bf16=True,
+                                       keys_f16=(model_dtype == torch.float16))
                     got = plugin.data[l][m["slots"][l]].cpu().numpy()
                     assert np.array_equal(bits(got), bits(want[m["slots"][l]])), (rid, l)
                     m["rep"].append(want)
