@@ -131,13 +131,21 @@ __device__ __forceinline__ float quad_dot(const f32x4 (&qr)[kSteps], const f32x4
 // request owns at least one tile, which the fused kernel needs: a request's last tile runs its selection.
 __device__ __forceinline__ int clamped_len(int n, int max_seg_len) { return min(max(n, 0), max_seg_len); }
 
-__device__ __forceinline__ bool find_tile(const int32_t* __restrict__ seg_len, int n_req, int tile_blocks, int max_seg_len,
-                                          int min_tiles, int w, int lane, int& r_out, int& tile_out)
+// The owner's other descriptors come back with it: every lane fetches its request's first row and query row together
+// with its length, so the workgroup waits for memory once here, not once for the lengths and again for what they lead to.
+__device__ __forceinline__ bool find_tile(const int32_t* __restrict__ seg_len, const int32_t* __restrict__ seg_off,
+                                          const int32_t* __restrict__ q_rows, int n_req, int tile_blocks, int max_seg_len,
+                                          int min_tiles, int w, int lane, int& r_out, int& tile_out, int& len_out,
+                                          int& off_out, int& q_row_out)
 {
     int base = 0;
     for (int c = 0; c < n_req; c += 64) {
         const int r = c + lane;
-        const int t = r < n_req ? max((clamped_len(seg_len[r], max_seg_len) + tile_blocks - 1) / tile_blocks, min_tiles) : 0;
+        const bool live = r < n_req;
+        const int len = live ? clamped_len(seg_len[r], max_seg_len) : 0;
+        const int off = live ? seg_off[r] : 0;
+        const int qr = live && q_rows ? q_rows[r] : r;
+        const int t = live ? max((len + tile_blocks - 1) / tile_blocks, min_tiles) : 0;
         int incl = t;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -149,6 +157,9 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ seg_len, i
             const int src = __builtin_ctzll(owner);
             r_out = c + src;
             tile_out = w - (base + __shfl(incl - t, src, 64));
+            len_out = __builtin_amdgcn_readlane(len, src);       // (scalar results: what follows stays uniform)
+            off_out = __builtin_amdgcn_readlane(off, src);
+            q_row_out = __builtin_amdgcn_readlane(qr, src);
             return true;
         }
         base += __shfl(incl, 63, 64);
@@ -188,14 +199,16 @@ struct TileInfo {
 template <int kD>
 __device__ __forceinline__ bool locate(const ScoreArgs& a, int lane, TileInfo& t)
 {
-    if (!find_tile(a.seg_len, a.n_req, a.tile_blocks, a.max_seg_len, a.tickets ? 1 : 0, blockIdx.y, lane, t.r, t.tile)) {
+    int len = 0, off = 0, q_row = 0;
+    if (!find_tile(a.seg_len, a.seg_off, a.q_rows, a.n_req, a.tile_blocks, a.max_seg_len, a.tickets ? 1 : 0, blockIdx.y, lane,
+                   t.r, t.tile, len, off, q_row)) {
         return false;
     }
-    t.n = clamped_len(a.seg_len[t.r], a.max_seg_len);
-    t.seg0 = a.seg_off[t.r];
+    t.n = len;
+    t.seg0 = off;
     // indices that came from device memory are followed only inside their tables: the request's query row
     // inside the layer's query block, its rows inside a layer of the representative table
-    t.q_row = a.q_rows ? static_cast<int64_t>(a.q_rows[t.r]) : t.r;
+    t.q_row = q_row;
     t.ok = !(a.q_rows && (t.q_row < 0 || (t.q_row + 1) * a.q_heads * kD > a.q_layer_stride)) &&
            t.seg0 >= 0 && t.seg0 + t.n <= a.repre_rows;
     return true;
