@@ -319,8 +319,8 @@ def test_gsa_plugin_decode_flow(ucm, dev, repre_dtype, model, lag):
 
 
 def test_gsa_retrieval_lag_with_a_request_that_arrives_later(ucm, dev):
-    """retrieval_lag 1 while the batch changes: request A decodes from step 1, request C's prompt arrives at step 4 (A
-    decoding beside it) and C decodes from step 5.  Every selection a layer's attention sees must be the oracle's for
+    """retrieval_lag 1 while the batch changes: request A decodes from step 1 and leaves after step 7, request C's prompt
+    arrives at step 4 (A decoding beside it) and C decodes from step 5, request D arrives at step 8.  Every selection a layer's attention sees must be the oracle's for
     the query the request had in the step before - for C's first decode step that is the last token of its prompt, kept
     during the step that prefilled it - over the representatives and block lists of the step that uses it."""
     from ucm_amd.sparse.base import UcmSparseRole
@@ -338,14 +338,17 @@ def test_gsa_retrieval_lag_with_a_request_that_arrives_later(ucm, dev):
     names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
     fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
     free_blocks = [int(x) for x in synth.permutation(731, nb)]
-    prompts, arrives = {"A": 290, "C": 410}, {"A": 0, "C": 4}
+    prompts, arrives, leaves = {"A": 290, "C": 410, "D": 330}, {"A": 0, "C": 4, "D": 8}, {"A": 7}
     reqs = {r: ns(block_ids=[[]], num_computed_tokens=0, prompt_token_ids=[1] * n, output_token_ids=[]) for r, n in prompts.items()}
     repre_h = {r: [np.zeros((60, hkv * d), np.float32) for _ in range(L)] for r in prompts}
     done_blocks = {r: 0 for r in prompts}
     q_before = {r: [None] * L for r in prompts}
     lagged, checked = [], 0
-    for step in range(10):
-        live = [r for r in prompts if arrives[r] <= step]
+    for step in range(12):
+        for r, last in leaves.items():
+            if step == last + 1:
+                plugin.request_finished_in_worker(r)             # A is done
+        live = [r for r in prompts if arrives[r] <= step <= leaves.get(r, 99)]
         sched = {r: (prompts[r] if step == arrives[r] else 1) for r in live}
         for r in live:
             need = -(-(reqs[r].num_computed_tokens + sched[r]) // bs)
@@ -396,9 +399,10 @@ def test_gsa_retrieval_lag_with_a_request_that_arrives_later(ucm, dev):
             reqs[r].output_token_ids.append(7)
         plugin.execute_finished()
     # step 1 scores layer by layer (nothing was kept during the prefill-only step 0); from step 2 on one launch per step,
-    # the step C's prompt runs beside A's decode and C's first decode step included
-    assert lagged == [False, False] + [True] * 8
-    assert checked == L * (9 + 5)
+    # the step C's prompt runs beside A's decode, C's first decode step, the step after A has left and D's arrival included
+    assert lagged == [False, False] + [True] * 10
+    assert "A" not in plugin.gsa_stats and "A" not in plugin._parked and set(plugin.gsa_stats) == {"C", "D"}
+    assert checked == L * (7 + 7 + 3)
 
 
 @pytest.mark.parametrize("lag", [0, 1])
