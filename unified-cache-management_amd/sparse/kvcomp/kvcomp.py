@@ -288,6 +288,7 @@ class KvComp(UcmSparseBase):
         self._device_loads = bool(self.cfg.get("device_loads", True)) and self.tp_size == 1
         self._dev: Optional[KvCompDevicePath] = None
         self._dev_step_built = True
+        self._quiet = False
         self._kv_caches: Dict[int, torch.Tensor] = {}
 
     # ---- device tables -------------------------------------------------------------------
@@ -390,6 +391,8 @@ class KvComp(UcmSparseBase):
         return self._dev
 
     def attention_begin(self, query, key, value, layer_name: str, forward_context) -> None:
+        if self._quiet:
+            return
         dev = self._device_step(layer_name, forward_context)
         batched = set(dev.active) if dev is not None else ()
         for req_meta in self._sparse_metadata.requests:
@@ -411,6 +414,8 @@ class KvComp(UcmSparseBase):
     def attention_finished(self, query, key, value, attn_output, layer_name: str, forward_context) -> None:
         # with a device-addressable store the full blocks of all requests are dumped and hashed in one go, and the
         # windows of those that finish their prefill copied aside in one go
+        if self._quiet:
+            return
         dev = self._batched(layer_name, forward_context)
         batch = [] if dev is not None else None
         for req_meta in self._sparse_metadata.requests:
@@ -440,6 +445,23 @@ class KvComp(UcmSparseBase):
                                  sparsed.get(req_id, INVALID_SLOT), req.block_ids[0])
         self._sparse_metadata = meta
         self._dev_step_built = False
+        self._quiet = self._quiet_step(meta.requests)
+
+    def _quiet_step(self, metas) -> bool:
+        """True when no hook of this step has anything to do on the batched path: every request decodes, none is at
+        a retrieval step or at its first decode step (windows), none fills a block, and every layer has seen every
+        request before.  The hooks then return at once instead of walking the requests in every layer (three decode
+        steps of four with the default stride)."""
+        if self._dev is None:
+            return False
+        stride, bs = self.cfg["retrieval_stride"], self.block_size
+        for m in metas:
+            states = self.req_states.get(m.request_id)
+            if m.is_prefill or m.step % stride == 1 or states is None or any(st is None or not st.block_size for st in states):
+                return False
+            if (m.num_computed_tokens + m.num_scheduled_tokens) // bs > states[0].num_blocks_hashed or states[0].tasks:
+                return False
+        return True
 
     def request_finished_in_worker(self, request_id: ReqType) -> None:
         self.req_states.pop(request_id, None)
