@@ -50,7 +50,10 @@ class ReprePool:
 
     def allocate(self, num_new_slots: int) -> List[int]:
         assert len(self.free_slots) >= num_new_slots, "Not enough free slots"
-        got = [self.free_slots.pop() for _ in range(num_new_slots)]
+        if num_new_slots <= 0:
+            return []
+        got = self.free_slots[-num_new_slots:][::-1]           # the order repeated pop() hands them out in
+        del self.free_slots[-num_new_slots:]
         self.allocated.update(got)
         return got
 
