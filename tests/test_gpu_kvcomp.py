@@ -235,7 +235,7 @@ def test_kvcomp_plugin_flow(ucm, dev, device_loads, hole, delta, model):
 
 
 def kvcomp_scenario(dev, device_loads, timing=None, shape=(8, 2, 128, 3, 16, 256), prompts=None, start=None, n_steps=12,
-                    keep_caches=True):
+                    keep_caches=True, delta_loads=False):
     """Three sparsified requests at different stages (one prefilled two steps after the others, so that some steps
     mix a prompt with decode tokens and the retrieval steps of the requests do not coincide) plus one short request
     the plugin leaves alone; returns, per engine step, every request's selections per layer and the bytes of all
@@ -250,7 +250,8 @@ def kvcomp_scenario(dev, device_loads, timing=None, shape=(8, 2, 128, 3, 16, 256
     torch.manual_seed(5)                                           # the plugin draws its hash weights from the global generator
     hq, hkv, d, L, bs, nb = shape
     cfg = make_config(hq, hkv, d, L, bs, bs * 64, {})
-    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KvComp": {"device_loads": device_loads}}}
+    cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KvComp": {"device_loads": device_loads,
+                                                                                         "delta_loads": delta_loads}}}
     cfg.scheduler_config.max_num_seqs = max(cfg.scheduler_config.max_num_seqs, len(prompts or ()) + 1)
     plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
     slice_bytes = bs * hkv * d * 2
@@ -328,6 +329,28 @@ def test_kvcomp_batched_path_equals_per_request_path(ucm, dev):
     busy_host = sorted(t for s, t in t_host if s >= 4)
     print(f"\nhost time of a step's hooks, median over steps 4-11: batched {busy_dev[len(busy_dev) // 2] * 1e3:.2f} ms, "
           f"per request {busy_host[len(busy_host) // 2] * 1e3:.2f} ms; slowest {busy_dev[-1] * 1e3:.2f} / {busy_host[-1] * 1e3:.2f} ms")
+
+
+def test_kvcomp_delta_loads_leave_the_same_blocks_in_the_cache(ucm, dev):
+    """Twenty engine steps with and without delta loads (three sparsified requests whose retrieval steps do not
+    coincide, one that arrives later): the same selections at every retrieval, and after every step every layer's
+    cache holds the same blocks - K and V together, the same number of times - only in other middle blocks."""
+    a = kvcomp_scenario(dev, True, n_steps=20, delta_loads=True)
+    b = kvcomp_scenario(dev, True, n_steps=20)
+
+    def contents(cache):                                           # one number per cache block over its K and V bytes
+        v = cache.view(torch.int16).to(torch.int64).reshape(2, cache.shape[1], -1)
+        w = torch.arange(1, v.shape[2] + 1, device=v.device, dtype=torch.int64)
+        h = (v * w).sum(2)
+        return torch.sort(h[0] * 1000003 + h[1]).values
+
+    moved_elsewhere = 0
+    for step, ((sel_a, caches_a), (sel_b, caches_b)) in enumerate(zip(a, b)):
+        assert sel_a == sel_b, step
+        for l, (x, y) in enumerate(zip(caches_a, caches_b)):
+            assert torch.equal(contents(x), contents(y)), (step, l)
+            moved_elsewhere += int(not torch.equal(x, y))
+    assert moved_elsewhere > 10                                    # the placement really differs: the test compares something
 
 
 @pytest.mark.parametrize("seed", range(6))
