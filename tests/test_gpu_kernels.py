@@ -964,3 +964,34 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
     for name in ("votes", "votes_tables", "votes_bad0", "votes_bad1", "votes_bad2"):
         assert np.allclose(got[name], want[name], rtol=2e-4, atol=2e-6), name
         assert np.array_equal(got[name] == -3, want[name] == -3), name        # the same tasks were skipped
+
+
+@pytest.mark.parametrize("dtype,row", [("bfloat16", (32, 128)), ("float32", (8, 64)), ("float16", (3, 8))])
+def test_park_rows_against_torch_indexing(ucm, dev, dtype, row):
+    """ucm_park_rows: rows of a query tensor into rows of a kept-queries table, picked and placed by device index
+    arrays - a thousand pairs, some naming rows outside either array (skipped), with and without destination
+    indices - against torch's own indexing."""
+    from ucm_amd import ops
+
+    dt = getattr(torch, dtype)
+    g = torch.Generator(device=dev)
+    g.manual_seed(77)
+    src = torch.randn((700,) + row, device=dev, generator=g).to(dt)
+    dst = torch.full((1000,) + row, 3.0, dtype=dt, device=dev)
+    rng = np.random.default_rng(78)
+    pick = rng.integers(-5, 710, 1000).astype(np.int32)                  # a few below 0, a few past the end
+    put = rng.permutation(1010)[:1000].astype(np.int32) - 3              # distinct; a few outside [0, 1000)
+    ops.park_rows(src, torch.from_numpy(pick).to(dev), dst, torch.from_numpy(put).to(dev))
+    want = torch.full_like(dst, 3.0)
+    ok = (pick >= 0) & (pick < 700) & (put >= 0) & (put < 1000)
+    want[torch.from_numpy(put[ok].astype(np.int64)).to(dev)] = src[torch.from_numpy(pick[ok].astype(np.int64)).to(dev)]
+    assert 900 < ok.sum() < 1000 and torch.equal(dst.view(torch.uint8), want.view(torch.uint8))
+    dst2 = torch.full((1000,) + row, 3.0, dtype=dt, device=dev)
+    ops.park_rows(src, torch.from_numpy(pick).to(dev), dst2)            # pair i goes to row i
+    want2 = torch.full_like(dst2, 3.0)
+    ok2 = (pick >= 0) & (pick < 700)
+    at = torch.from_numpy(np.nonzero(ok2)[0]).to(dev)
+    want2[at] = src[torch.from_numpy(pick[ok2].astype(np.int64)).to(dev)]
+    assert torch.equal(dst2.view(torch.uint8), want2.view(torch.uint8))
+    with pytest.raises(ValueError):
+        ops.park_rows(src, torch.from_numpy(pick).to(dev), dst.float() if dt != torch.float32 else dst.half())
