@@ -159,6 +159,10 @@ def test_gsa_plugin_metadata_without_a_gpu(ucm):
     plugin.execute_finished()
     plugin.request_finished_in_worker("x")
     assert "x" not in plugin.gsa_stats and plugin.topk_kpre_manger.free_cache[-1] == 0
+    # the options that choose when a selection is made and applied
+    assert plugin.retrieval_lag == 0 and GSA(make_config(cfg={"retrieval_lag": 1}), UcmSparseRole.WORKER).retrieval_lag == 1
+    with pytest.raises(ValueError, match="retrieval_lag"):
+        GSA(make_config(cfg={"retrieval_lag": 2}), UcmSparseRole.WORKER)
 
 
 def test_esa_scheduler_side_and_helpers(ucm):
