@@ -463,8 +463,8 @@ int ucm_hash_encode_queries(const void* q_bf16, int64_t q_layer_stride, const in
 /*
  * The same two calls for a float16 model: keys (or queries) and weights are float16 - HashEncoder draws its weights
  * in the model's type (ucm/sparse/kvcomp/hash_encoder.py:65-71) - and the codes are the signs of the exactly
- * accumulated float16 products.  The query call takes one query head per kv head only (q_heads == kv_heads, what the
- * plugin passes after its own group mean, kvcomp.py:228-233); UCM_ENOTSUP otherwise.
+ * accumulated float16 products.  With several query heads per kv head the group means are fp32 numbers, as in the
+ * bf16 call, and the mean codes are the signs of their exactly accumulated products with the float16 weights.
  */
 int ucm_hash_encode_blocks_f16(const void* const* k_layers, int n_layers, int num_blocks,
                                const int32_t* block_ids, const int32_t* slots, int n, int block_size,

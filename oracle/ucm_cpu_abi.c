@@ -607,7 +607,7 @@ static int hash_encode_queries_host(int f16, const void* q_bf16, int64_t q_layer
         q_heads % kv_heads != 0) {
         return UCM_EINVAL;
     }
-    if (head_dim != 128 || bits != 128 || (f16 && q_heads != kv_heads)) { return UCM_ENOTSUP; }
+    if (head_dim != 128 || bits != 128) { return UCM_ENOTSUP; }
     const uint32_t nbytes = (uint32_t)bits / 8;
     const size_t qrow = (size_t)q_heads * head_dim;
     float* w = widen_weights(w_bf16, f16, head_dim, bits);

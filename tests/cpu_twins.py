@@ -310,7 +310,14 @@ def run_hash(call, side):
     qb16 = side.up(np.full((HL, 3, HHKV, 16), 0xEE, np.uint8))
     call("ucm_hash_encode_queries_f16", side.ptr(q16), 4 * HHKV * HD, side.ptr(q_rows), 3, HL, HHKV, HHKV, HD, side.ptr(w16), 128,
          side.ptr(qc16), side.ptr(qs16), side.ptr(qb16), None)
-    out.update(token_codes_f16=t16, colsum_f16=c16, block_codes_f16=b16, q_codes_f16=qc16, q_sum_f16=qs16, qbar_f16=qb16)
+    # the same queries as HHKV heads around one kv head: the mean codes of a grouped float16 model
+    qcg = side.up(np.full((HL, 3, HHKV, 16), 0xEE, np.uint8))
+    qsg = side.up(np.full((HL, 3, 128), 77, np.int16))
+    qbg = side.up(np.full((HL, 3, 1, 16), 0xEE, np.uint8))
+    call("ucm_hash_encode_queries_f16", side.ptr(q16), 4 * HHKV * HD, side.ptr(q_rows), 3, HL, HHKV, 1, HD, side.ptr(w16), 128,
+         side.ptr(qcg), side.ptr(qsg), side.ptr(qbg), None)
+    out.update(token_codes_f16=t16, colsum_f16=c16, block_codes_f16=b16, q_codes_f16=qc16, q_sum_f16=qs16, qbar_f16=qb16,
+               q_codes_f16_grouped=qcg, q_sum_f16_grouped=qsg, qbar_f16_grouped=qbg)
     side.sync()
     return {k: np.array(side.down(v)) for k, v in out.items()}, x
 

@@ -130,6 +130,18 @@ def test_hash_twins_reproduce_the_oracle(ucm):
             assert np.array_equal(got["q_codes_f16"][l, r], qc)
             assert np.array_equal(got["qbar_f16"][l, r], qc)                    # one head per kv head: the mean is the row
             assert np.array_equal(got["q_sum_f16"][l, r], (np.unpackbits(qc, axis=-1, bitorder="little").astype(np.int32) * 2 - 1).sum(0))
+            # all heads around one kv head: the fp32 mean in head order, then its exact signs
+            q32 = x["q16"][l, row].astype(np.float32)
+            mean = q32[0]
+            for h in range(1, q32.shape[0]):
+                mean = mean + q32[h]
+            mean = mean * (np.float32(1.0) / np.float32(q32.shape[0]))
+            accm = np.zeros(128)
+            for d_ in range(cpu_twins.HD):
+                accm += np.float64(mean[d_]) * w16[d_]
+            assert np.array_equal(got["qbar_f16_grouped"][l, r, 0], np.packbits(accm > 0, bitorder="little"))
+            assert np.array_equal(got["q_codes_f16_grouped"][l, r], qc)
+            assert np.array_equal(got["q_sum_f16_grouped"][l, r], got["q_sum_f16"][l, r])
 
 
 def test_esa_twins_reproduce_the_oracle(ucm):

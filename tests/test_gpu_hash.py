@@ -604,11 +604,54 @@ def test_hash_encode_float16_projections_built_to_cancel(ucm, dev, paired):
     assert np.array_equal(bcodes[0].cpu().numpy(), O.hash_majority(want))
 
 
+@pytest.mark.parametrize("g", [2, 3, 4, 8])
+def test_hash_query_mean_codes_of_a_float16_model_with_grouped_heads(ucm, dev, g):
+    """Several float16 query heads per kv head: the mean codes are the exact signs of (fp32 sequential sum * 1/g) . w,
+    also where the heads of a group cancel down to a few low bits, for subnormal rows and for large ones; the
+    per-head codes and their sums are unchanged by the grouping."""
+    from ucm_amd import ops
+
+    hkv, n_layers, n_req = 8, 2, 5
+    hq = hkv * g
+    rng = np.random.default_rng(1531 + g)
+    w16 = (rng.standard_normal((128, 128)) * 2.0).astype(np.float16)
+    q = rng.standard_normal((n_layers, n_req, hq, 128)).astype(np.float32)
+    q[:, 1] *= 3e-6                                            # subnormal components
+    q[:, 2] *= 1500.0
+    q16 = q.astype(np.float16)
+    # request 3: the heads of a group cancel but for the last bit of one component of one of them
+    q16[:, 3, 1::g] = -q16[:, 3, 0::g]
+    if g > 2:
+        q16[:, 3].reshape(n_layers, hkv, g, 128)[:, :, 2:] = 0
+    q16[:, 3, 0::g, 7] = np.nextafter(q16[:, 3, 0::g, 7], np.float16(np.inf))
+    q_codes = torch.full((n_layers, n_req, hq, 16), 0xEE, dtype=torch.uint8, device=dev)
+    q_sum = torch.full((n_layers, n_req, 128), 77, dtype=torch.int16, device=dev)
+    qbar = torch.full((n_layers, n_req, hkv, 16), 0xEE, dtype=torch.uint8, device=dev)
+    ops.hash_encode_queries(f16_dev(q16, dev), f16_dev(w16, dev), hkv, q_codes, q_sum, qbar, n_req)
+    torch.cuda.synchronize()
+    inv = np.float32(1.0) / np.float32(g)
+    for l in range(n_layers):
+        want = exact_codes(q16[l].astype(np.float64), w16.astype(np.float64))
+        assert np.array_equal(q_codes[l].cpu().numpy(), want), l
+        pm = np.unpackbits(want, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
+        assert np.array_equal(q_sum[l].cpu().numpy(), pm.sum(1)), l
+        grouped = q16[l].astype(np.float32).reshape(n_req, hkv, g, 128)
+        mean = grouped[:, :, 0]
+        for j in range(1, g):
+            mean = mean + grouped[:, :, j]                     # fp32, head order
+        mean = mean * inv
+        want_bar = exact_codes(mean.astype(np.float64), w16.astype(np.float64))
+        for r in range(n_req):
+            assert np.array_equal(O.q_head_mean(q16[l, r].astype(np.float32), hkv), mean[r])
+        assert np.array_equal(qbar[l].cpu().numpy(), want_bar), l
+        assert want_bar[3].any() and not np.array_equal(want_bar[3], want_bar[0])
+
+
 def test_hash_query_codes_of_a_float16_model(ucm, dev):
     """Float16 queries and weights, one query head per kv head (what the plugin passes after its own group mean):
     codes, their +-1 sums and the mean codes (the rows' own codes); rows that cancel exactly or down to one small
-    term, rows of subnormal components and rows of large ones.  Several query heads per kv head are refused."""
-    from ucm_amd import _lib, ops
+    term, rows of subnormal components and rows of large ones."""
+    from ucm_amd import ops
 
     hkv, n_layers, n_req = 8, 2, 6
     rng = np.random.default_rng(1530)
@@ -637,8 +680,3 @@ def test_hash_query_codes_of_a_float16_model(ucm, dev):
         pm = np.unpackbits(want, axis=-1, bitorder="little").astype(np.int32) * 2 - 1
         assert np.array_equal(q_sum[l].cpu().numpy(), pm.sum(1)), l
         assert not want[0, 0::2].any() and want[0, 1::2].any() and want[1].any()
-    q32 = torch.zeros((1, 2, 32, 128), dtype=torch.float16, device=dev)
-    with pytest.raises(_lib.UcmHipError, match="one per kv head"):
-        ops.hash_encode_queries(q32, f16_dev(w16, dev), hkv, torch.zeros((1, 2, 32, 16), dtype=torch.uint8, device=dev),
-                                torch.zeros((1, 2, 128), dtype=torch.int16, device=dev),
-                                torch.zeros((1, 2, hkv, 16), dtype=torch.uint8, device=dev), 2)

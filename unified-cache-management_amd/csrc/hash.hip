@@ -647,6 +647,8 @@ struct __attribute__((aligned(16))) QueryLds {
     float mean_max2[2];                                  // largest squared norm of the means staged by waves 0 and 1
 };
 
+static_assert(sizeof(QueryLds::mean) >= kMaxHeads * kDim * sizeof(float), "the term area also holds the means as fp32 rows");
+
 __device__ __forceinline__ float wave_max32(float m)
 {
 #pragma unroll
@@ -712,9 +714,24 @@ __device__ __forceinline__ bool mean_exact_positive(const QueryLds& s, unsigned 
     return acc > 0.0;
 }
 
-// kF16: float16 queries and weights, one query head per kv head only (host checked): the "mean" is the row itself,
-// which is its own first term - an fp32 mean of several float16 rows does not split into float16 terms exactly
-// (its low bits fall below what float16 can hold).
+// exact sign of an fp32 mean . column (float16 model, several query heads per kv head: the means wait in the
+// term area as plain fp32 rows; an fp32 times a float16 value is exact in fp64 as well)
+__device__ __forceinline__ bool mean_f32_exact_positive(const QueryLds& s, unsigned h, unsigned col)
+{
+    const float* m = reinterpret_cast<const float*>(&s.mean[0][0][0]) + h * kDim;
+    double acc = 0.0;
+#pragma unroll 8
+    for (int d = 0; d < kDim; ++d) {
+        const float wf = widen_lo<true>(static_cast<unsigned>(s.w[d * kBits + col]));
+        acc += static_cast<double>(m[d]) * static_cast<double>(wf);
+    }
+    return acc > 0.0;
+}
+
+// kF16: float16 queries and weights.  With one query head per kv head the "mean" is the row itself, which is its own
+// first term.  An fp32 mean of several float16 rows does not split into float16 terms exactly (its low bits fall
+// below what float16 can hold), so these few means (kv_heads per request) skip the matrix cores: they are kept in
+// fp32 and every one of their signs is taken the exact way.
 template <bool kF16>
 __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
     const unsigned short* __restrict__ q, int64_t q_layer_stride, const int32_t* __restrict__ q_rows,
@@ -754,9 +771,11 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
                 for (int j = 0; j < 8; ++j) { x[j] = x[j] + y[j]; }
             }
             unsigned term[3][8];
+            float xmean[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float xm = g != 1 ? x[j] * inv : x[j];
+                xmean[j] = xm;
                 if (kF16) {                                                   // (g == 1: xm is a float16 value)
                     term[0][j] = __builtin_bit_cast(unsigned short, static_cast<_Float16>(xm));
                     term[1][j] = term[2][j] = 0u;
@@ -771,12 +790,18 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
                 }
                 nx2 = nx2 + xm * xm;
             }
+            if (kF16 && g != 1) {
+                float* m = reinterpret_cast<float*>(&s.mean[0][0][0]) + h * kDim + 8 * piece;
 #pragma unroll
-            for (int p = 0; p < 3; ++p) {
-                u32x4 packed;
+                for (int j = 0; j < 8; ++j) { m[j] = xmean[j]; }
+            } else {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) { packed[j] = term[p][2 * j] | (term[p][2 * j + 1] << 16); }
-                *reinterpret_cast<u32x4*>(&s.mean[p][h][8 * piece]) = packed;
+                for (int p = 0; p < 3; ++p) {
+                    u32x4 packed;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) { packed[j] = term[p][2 * j] | (term[p][2 * j + 1] << 16); }
+                    *reinterpret_cast<u32x4*>(&s.mean[p][h][8 * piece]) = packed;
+                }
             }
         }
         if (wave < 2) {                                  // (waves 0 and 1 hold the at most eight heads)
@@ -858,8 +883,19 @@ __global__ __launch_bounds__(kQueryThreads, 4) void hash_query_kernel(
     sum += __shfl_xor(sum, 32, 64);
     if (half == 0) { q_sum[lrq * kBits + col] = static_cast<short>(sum); }
 
-    // ---- the group means: row 8*term + h of the tile is that term of head h's mean
-    {
+    // ---- the group means
+    if (kF16 && g != 1) {
+#pragma unroll 1
+        for (unsigned i = 0; i < 4; ++i) {
+            const unsigned h = 4 * half + i;
+            const bool valid = h < kv_heads;
+            const bool pos = valid && mean_f32_exact_positive(s, h, col);
+            const unsigned long long mask = __ballot(pos);
+            if (valid && lr32 == 0) {
+                qbar_codes[(lrq * kv_heads + h) * 4 + wave] = static_cast<unsigned>(half ? mask >> 32 : mask);
+            }
+        }
+    } else {                                             // row 8*term + h of the tile is that term of head h's mean
         const unsigned term = lr32 >> 3, h_in = lr32 & 7;
         const bool feeds = term < 3 && h_in < kv_heads;
         f32x16 acc;
@@ -1121,8 +1157,6 @@ int hash_encode_queries(bool f16, const void* q_bf16, int64_t q_layer_stride, co
                 static_cast<long long>(q_layer_stride));
     UCM_SUPPORTED(q_heads <= kMaxQHeads && kv_heads <= kMaxHeads, "ucm_hash_encode_queries: q_heads=%d kv_heads=%d (at most %d and %d)",
                   q_heads, kv_heads, kMaxQHeads, kMaxHeads);
-    UCM_SUPPORTED(!f16 || q_heads == kv_heads, "ucm_hash_encode_queries_f16: q_heads=%d kv_heads=%d (float16 queries: one per kv head, "
-                  "the caller's own group mean)", q_heads, kv_heads);
 #define UCM_HASH_QUERY_ARGS dim3(n_req, n_layers), dim3(kQueryThreads), 0, ucm::as_stream(stream),                    \
         static_cast<const unsigned short*>(q_bf16), q_layer_stride, q_rows, static_cast<unsigned>(q_heads),          \
         static_cast<unsigned>(kv_heads), static_cast<const unsigned short*>(w_bf16), static_cast<unsigned>(n_req),   \

@@ -464,7 +464,7 @@ def hash_encode_blocks(k_layers: LayerPointers, block_ids: Optional[torch.Tensor
 
 def hash_encode_queries(q: torch.Tensor, w: torch.Tensor, kv_heads: int, q_codes: torch.Tensor, q_sum: torch.Tensor,
                         qbar_codes: torch.Tensor, n_req: int, q_rows: Optional[torch.Tensor] = None) -> None:
-    """q bf16 [L, rows, q_heads, 128] (or float16 with float16 weights and q_heads == kv_heads); q_codes u8
+    """q bf16 [L, rows, q_heads, 128] (or float16 with float16 weights); q_codes u8
     [L, n_req, q_heads, 16]; q_sum int16 [L, n_req, 128]; qbar_codes u8 [L, n_req, kv_heads, 16]."""
     n_layers, _, q_heads, d = q.shape
     if q.dtype not in (torch.bfloat16, torch.float16) or w.dtype != q.dtype:
