@@ -406,6 +406,128 @@ def test_gsa_retrieval_lag_with_a_request_that_arrives_later(ucm, dev):
 
 
 @pytest.mark.parametrize("lag", [0, 1])
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_gsa_drawn_scenarios(ucm, dev, seed, lag):
+    """Thirty steps of a drawn batch: up to four requests at a time, prompts of 40 to 520 tokens (those of at most
+    100 are never sparsified; those above 256 are prefilled in two chunks), arrivals and departures at random steps,
+    a request id coming back with another request behind it, batch indices that shift when a request leaves.  After
+    every layer's attention_begin a sparsified request's row of the block table and its length are the oracle's
+    selection - from the query of the step before wherever the step was scored ahead of the model - and a request that
+    is not sparsified keeps its own blocks; after every step the table of representatives holds the oracle's rows."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 64, 2, 16, 200
+    lo, hi, threshold, chunk = 6, 10, 100, 256
+    cfg = make_config(hq, hkv, d, L, bs, 16 * 60, {"seg_prefill_threshold": threshold, "min_topk_len": lo, "max_topk_len": hi,
+                                                   "repre_dtype": "bfloat16", "retrieval_lag": lag})
+    plugin = GSA(cfg, UcmSparseRole.WORKER)
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    rng = np.random.RandomState(seed)
+    caches = [torch.zeros(2, nb, bs, hkv, d, dtype=torch.bfloat16, device=dev) for _ in range(L)]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=None)
+    free_blocks = [int(x) for x in synth.permutation(740 + seed, nb)]
+    ids = ["A", "B", "C", "D", "E"]
+    reqs, prompts, repre_h, done_blocks, q_before = {}, {}, {}, {}, {}
+    live, leaving = [], []
+    checked = kept_whole = lagged_steps = came_back = 0
+    seen = set()
+    for step in range(30):
+        for r in leaving:
+            plugin.request_finished_in_worker(r)
+            free_blocks.extend(reqs[r].block_ids[0])
+            live.remove(r)
+        leaving = []
+        new = []
+        idle = [r for r in ids if r not in live]
+        if idle and len(live) < 4 and (step == 0 or rng.rand() < 0.4):
+            r = idle[rng.randint(len(idle))]
+            came_back += int(r in seen)
+            seen.add(r)
+            prompts[r] = int(rng.choice([rng.randint(40, 101), rng.randint(101, 257), rng.randint(257, 521)], p=[0.2, 0.4, 0.4]))
+            reqs[r] = ns(block_ids=[[]], num_computed_tokens=0, prompt_token_ids=[1] * prompts[r], output_token_ids=[])
+            repre_h[r] = [np.zeros((60, hkv * d), np.float32) for _ in range(L)]
+            done_blocks[r], q_before[r] = 0, [None] * L
+            live.append(r)
+            new.append(r)
+        if not live:
+            continue
+        sched = {r: (min(chunk, prompts[r] - reqs[r].num_computed_tokens) if reqs[r].num_computed_tokens < prompts[r] else 1)
+                 for r in live}
+        for r in live:
+            need = -(-(reqs[r].num_computed_tokens + sched[r]) // bs)
+            while len(reqs[r].block_ids[0]) < need:
+                reqs[r].block_ids[0].append(free_blocks.pop())
+        so = ns(num_scheduled_tokens=sched, scheduled_new_reqs=[ns(req_id=r) for r in new])
+        ib = ns(req_id_to_index={r: i for i, r in enumerate(live)})
+        seq_lens = {r: reqs[r].num_computed_tokens + sched[r] for r in live}
+        sparsified = {r: prompts[r] > threshold and reqs[r].num_computed_tokens >= prompts[r] for r in live}
+        plugin.build_sparse_meta(so, {r: reqs[r] for r in live}, ib, None)
+        plugin.execute_begin(so)
+        lagged = plugin._lagged is not None
+        assert not lagged or lag == 1
+        lagged_steps += int(lagged)
+        for l in range(L):
+            md = ns(block_table=None, seq_lens=None)
+            fc.attn_metadata = {names[l]: md}
+            n_tok = sum(sched.values())
+            query = torch.randn(n_tok, hq, d, device=dev, generator=g).to(torch.bfloat16)
+            key = torch.randn(n_tok, hkv, d, device=dev, generator=g).to(torch.bfloat16)
+            t0, last_row = 0, {}
+            for r in live:
+                for t in range(sched[r]):
+                    pos = reqs[r].num_computed_tokens + t
+                    caches[l][0, reqs[r].block_ids[0][pos // bs], pos % bs] = key[t0 + t]
+                t0 += sched[r]
+                last_row[r] = t0 - 1
+            plugin.attention_begin(query, key, key, names[l], fc)
+            torch.cuda.synchronize()
+            assert (md.block_table is not None) == any(sparsified.values()), (step, l)
+            for i, r in enumerate(live):
+                q_now = query[last_row[r]].float().cpu().numpy()
+                n = len(reqs[r].block_ids[0])
+                if sparsified[r]:
+                    q_use = q_before[r][l] if lagged else q_now
+                    want_idx, _ = O.select_topk(q_use, repre_h[r][l][:n].reshape(n, hkv, 1, d), topk_len(n, lo, hi))
+                    phys, want_len = O.block_table_gather(reqs[r].block_ids[0], want_idx, seq_lens[r], bs)
+                    assert int(md.seq_lens[i]) == want_len, (step, l, r)
+                    assert np.array_equal(md.block_table[i, : len(phys)].cpu().numpy(), phys), (step, l, r)
+                    checked += 1
+                elif md.block_table is not None:
+                    assert int(md.seq_lens[i]) == seq_lens[r], (step, l, r)
+                    assert np.array_equal(md.block_table[i, :n].cpu().numpy(), reqs[r].block_ids[0]), (step, l, r)
+                    kept_whole += 1
+                q_before[r][l] = q_now
+            plugin.attention_finished(query, key, key, None, names[l], fc)
+            for r in live:
+                full = min(seq_lens[r] // bs, len(reqs[r].block_ids[0]))
+                todo = list(range(done_blocks[r], full))
+                if todo:
+                    kc = caches[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+                    O.block_mean_paged(kc, [reqs[r].block_ids[0][i] for i in todo], todo, repre_h[r][l], round_bf16=True)
+        plugin.execute_finished()
+        torch.cuda.synchronize()
+        for r in live:
+            done_blocks[r] = max(done_blocks[r], min(seq_lens[r] // bs, len(reqs[r].block_ids[0])))
+            off = plugin.gsa_stats[r].slot_offset
+            for l in range(L):
+                got = plugin.kpre_caches[l, off : off + done_blocks[r]].float().cpu().numpy()
+                assert np.array_equal(bits(got), bits(repre_h[r][l][: done_blocks[r]])), (step, l, r)
+            reqs[r].num_computed_tokens += sched[r]
+            if reqs[r].num_computed_tokens > prompts[r] - 1:
+                reqs[r].output_token_ids.append(7)
+            if reqs[r].num_computed_tokens >= prompts[r] + 2 and rng.rand() < 0.12:
+                leaving.append(r)
+    assert checked >= 15 * L and kept_whole >= L, (checked, kept_whole, came_back)
+    assert set(plugin.gsa_stats) == set(live)
+    if lag:
+        assert lagged_steps >= 8
+
+
+@pytest.mark.parametrize("lag", [0, 1])
 def test_gsa_retrieval_stride_reuses_scores(ucm, dev, lag):
     """With retrieval_stride 3 the scores of the last retrieval are re-selected with the current lengths
     on the steps in between (the last two blocks are always kept, so the newest block is never missing);
