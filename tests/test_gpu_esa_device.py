@@ -39,8 +39,11 @@ def _config(hq, hkv, d, layers, bs, max_model_len, max_num_seqs, esa_cfg):
               kv_transfer_config=ns(kv_connector_extra_config={"ucm_sparse_config": {"ESA": esa_cfg}}))
 
 
-@pytest.mark.parametrize("pool_where,model_dtype", [("cuda", "bfloat16"), ("pinned", "bfloat16"), ("cuda", "float16")])
-def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
+@pytest.mark.parametrize("pool_where,model_dtype,churn", [("cuda", "bfloat16", False), ("pinned", "bfloat16", False),
+                                                          ("cuda", "float16", False), ("cuda", "bfloat16", True)])
+def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype, churn):
+    """churn: three requests finish before step 7 and three others start at step 8, in the table rows, representative
+    slots and batch positions the first three gave back."""
     from ucm_amd import ops
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.esa.esa import ESA
@@ -69,7 +72,8 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
     # requests: different prompt lengths, each starting its prefill at a different engine step
     perm = synth.permutation(77, nb)
     reqs, used = {}, 0
-    for i in range(n_req):
+    late = 3 if churn else 0
+    for i in range(n_req + late):
         n_blocks = int(synth.ints(300 + i, 1, 12, 100)[0])
         n_prompt = n_blocks * bs + (0 if i % 3 == 0 else int(synth.ints(400 + i, 1, 1, bs - 1)[0]))
         total = n_blocks + 3
@@ -77,7 +81,8 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
         used += total
         prompt = [int(x) for x in synth.ints(500 + i, n_prompt, 0, 30000)]
         reqs[f"r{i}"] = ns(request_id=f"r{i}", block_ids=[ids], num_computed_tokens=0, prompt_token_ids=prompt,
-                           output_token_ids=[], num_prompt_tokens=n_prompt, start=i % 4, index=i)
+                           output_token_ids=[], num_prompt_tokens=n_prompt, start=i % 4 if i < n_req else 8, index=i,
+                           done=False)
     assert used <= nb
 
     # host model of every (request, layer)
@@ -85,7 +90,7 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
     host_ms = {"prefill": [], "first": [], "retrieve": [], "load": [], "idle": []}
 
     def engine_step(t):
-        active = [r for r in reqs.values() if r.start <= t]
+        active = [r for r in reqs.values() if r.start <= t and not r.done]
         sched, qsl, pos = {}, [], 0
         for r in active:
             n_tok = r.num_prompt_tokens if r.num_computed_tokens == 0 else 1
@@ -130,6 +135,11 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
 
     n_steps = 14
     for t in range(n_steps):
+        if churn and t == 7:
+            for rid in ("r0", "r5", "r10"):
+                plugin.request_finished_in_worker(rid)
+                reqs[rid].done = True
+            assert len(plugin._dev.tables.free_rows) == 24 - (n_req - 3)
         active, qsl, qs = engine_step(t)
         for j, r in enumerate(active):
             rid = r.request_id
@@ -183,7 +193,8 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
             r.num_computed_tokens += 1
             r.output_token_ids.append(1)
     # every kind of step was seen; everything outside the requests' sparse slots is untouched
-    assert all(host_ms[k] for k in ("prefill", "first", "retrieve", "load"))
+    # (a step is named for the first kind of work it holds; with late arrivals some kinds are never alone in a step)
+    assert all(host_ms[k] for k in (("prefill", "first") if churn else ("prefill", "first", "retrieve", "load")))
     touched = torch.zeros(nb, dtype=torch.bool, device=dev)
     for rid, m in model.items():
         touched[torch.tensor(reqs[rid].block_ids[0][: m["top_k"]], dtype=torch.long, device=dev)] = True
@@ -191,8 +202,10 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype):
         assert torch.equal(caches[l][:, ~touched], original[l][:, ~touched])
     print("\nESA device path, %d requests x %d layers, host ms per engine step (hooks only): " % (n_req, L) +
           ", ".join(f"{k} {np.median(v):.2f} (n={len(v)})" for k, v in host_ms.items() if v))
-    for rid in list(reqs):
-        plugin.request_finished_in_worker(rid)
+    assert len(plugin._dev.reqs) == n_req
+    for rid, r in reqs.items():
+        if not r.done:
+            plugin.request_finished_in_worker(rid)
     assert not plugin._dev.reqs and len(plugin.layer_pools[0].allocated) == 0
     assert len(plugin._dev.tables.free_rows) == 24
 
