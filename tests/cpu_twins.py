@@ -2,6 +2,7 @@
 delta plan, gathers and the block moves - written once against the C ABI's prototypes and run either through
 libucm_hip.so on device buffers or through the oracle's `_cpu` twins (oracle/ucm_cpu_abi.c) on host buffers.
 The argument lists of the two runs are identical except for where the pointers point."""
+import contextlib
 import ctypes as C
 import os
 
@@ -17,6 +18,21 @@ TWINS = ["ucm_block_mean", "ucm_score_blocks", "ucm_topk_windows", "ucm_score_se
          "ucm_kv_load_planned", "ucm_kvstar_topk", "ucm_kvstar_order", "ucm_prefetch_plan", "ucm_kvstar_block_repre",
          "ucm_kvstar_votes", "ucm_kvstar_votes_tables", "ucm_kvstar_park_queries", "ucm_park_rows", "ucm_kvstar_block_repre_keys",
          "ucm_hash_encode_blocks_f16", "ucm_hash_encode_queries_f16"]
+
+
+@contextlib.contextmanager
+def reseeded(offset: int):
+    """Every input of the scripted passes drawn from other seeds (the shapes, the ids that are out of range on purpose
+    and the order of the calls stay as they are): synth's generators take seed + offset while the block runs."""
+    names = ("normal_f32", "normal_bf16_bits", "normal_bf16_as_f32", "ints", "permutation")
+    kept = {n: getattr(synth, n) for n in names}
+    try:
+        for n, f in kept.items():
+            setattr(synth, n, (lambda f: lambda seed, *a, **k: f(seed + offset, *a, **k))(f))
+        yield
+    finally:
+        for n, f in kept.items():
+            setattr(synth, n, f)
 
 
 def twin_caller(signatures):

@@ -966,6 +966,30 @@ def test_device_and_host_twins_give_the_same_bytes(ucm, dev):
         assert np.array_equal(got[name] == -3, want[name] == -3), name        # the same tasks were skipped
 
 
+def test_device_and_host_twins_on_other_seeds(ucm, dev):
+    """The scripted passes of the test above on inputs drawn from other seeds - 150 sets by default,
+    UCM_TWIN_SEED_SETS of them when that is set (6000 sets take three minutes) - with the same comparison."""
+    import os
+
+    import cpu_twins
+    from ucm_amd import _lib, ops
+
+    exact = ("table_full", "table_pruned", "table_by_block", "park_f32", "park_bf16", "park_f16", "rows_indexed", "rows_in_order")
+    for it in range(1, int(os.environ.get("UCM_TWIN_SEED_SETS", "150")) + 1):
+        with cpu_twins.reseeded(it * 100003):
+            for run in (cpu_twins.run, cpu_twins.run_bounds, cpu_twins.run_hash, cpu_twins.run_esa, cpu_twins.run_more):
+                want, _ = run(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+                got, _ = run(_lib.call, cpu_twins.DeviceSide(ops, dev))
+                for name in want:
+                    assert np.array_equal(got[name].view(np.uint8), want[name].view(np.uint8)), (it, run.__name__, name)
+            want, _ = cpu_twins.run_kvstar(cpu_twins.twin_caller(_lib.SIGNATURES), cpu_twins.HostSide())
+            got, _ = cpu_twins.run_kvstar(_lib.call, cpu_twins.DeviceSide(ops, dev))
+        for name in exact:
+            assert np.array_equal(got[name], want[name]), (it, name)
+        for name in ("votes", "votes_tables", "votes_bad0", "votes_bad1", "votes_bad2"):
+            assert np.allclose(got[name], want[name], rtol=2e-4, atol=2e-6), (it, name)
+
+
 @pytest.mark.parametrize("dtype,row", [("bfloat16", (32, 128)), ("float32", (8, 64)), ("float16", (3, 8))])
 def test_park_rows_against_torch_indexing(ucm, dev, dtype, row):
     """ucm_park_rows: rows of a query tensor into rows of a kept-queries table, picked and placed by device index
