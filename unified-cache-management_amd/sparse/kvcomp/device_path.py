@@ -279,8 +279,14 @@ class KvCompDevicePath:
                 else:
                     blocks = self._window_blocks(meta.vllm_block_ids, *self.win_shape[rid])
                 n, ptr = len(blocks), self.windows[rid].data_ptr()
+                # a request whose new block list is shorter than its two windows together gets a cache block named
+                # twice on the way back: the reference writes the first window, then the last one over it
+                # (kvcomp.py:392-404), so of the copies into one block only the last is made
+                last = {b: j for j, b in enumerate(blocks)}
                 for kv in range(2):
                     for j, b in enumerate(blocks):
+                        if not to_windows and last[b] != j:
+                            continue
                         cache_off.append(kv * kv_stride + b * block_bytes)
                         win_addr.append(ptr + (kv * n + j) * block_bytes)
                         win_lstride.append(2 * n * block_bytes)

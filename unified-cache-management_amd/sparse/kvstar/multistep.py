@@ -600,6 +600,13 @@ class KVStarMultiStep(UcmSparseBase):
         if missing:
             self._report_missing(missing)
         if src:
+            # a request whose block list is shorter than its two windows together names a cache block twice on the
+            # way back: the reference writes the init window, then the local one over it (multistep.py:348-362), so
+            # of the copies into one block only the last is made (the copies of one launch are not ordered)
+            last = {d: i for i, d in enumerate(dst)}
+            if len(last) != len(dst):
+                keep = [i for i, d in enumerate(dst) if last[d] == i]
+                dst, src = [dst[i] for i in keep], [src[i] for i in keep]
             ptrs = ops.upload(torch.tensor([dst, src], dtype=torch.int64), kv.device)
             ops.copy_batch(ptrs[0], ptrs[1], block_bytes)
         held.release()
