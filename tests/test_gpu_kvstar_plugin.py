@@ -348,3 +348,77 @@ def test_kvstar_plugin_at_serving_size(ucm, dev):
     for kind in t_dev:
         print(f"KVStar hooks, 16 requests x 32 layers, {kind}: {np.median(t_dev[kind]):.1f} ms of host time per step "
               f"(lists on the host {np.median(t_host[kind]):.1f} ms, the reference's flow {np.median(t_ref[kind]):.1f} ms)")
+
+
+@pytest.mark.parametrize("n_full", [2, 3, 4])
+def test_kvstar_windows_of_a_short_request(ucm, dev, n_full):
+    """A prompt of two to four full blocks and a few tokens - no more blocks than the init and local windows cover, so
+    nothing lies between them to choose from: prefill, the scheduler's shrink and the first decode step through the
+    batched path (one launch for all window copies) and through the per-request path (torch's indexed assignments, one
+    after the other) leave the same bytes in every cache, and the request's last two blocks hold its local window."""
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.factory import UcmSparseFactory
+    from ucm_amd.store.hip_block_store import UcmHipBlockStore
+
+    ns = types.SimpleNamespace
+    hq, hkv, d, L, bs, nb = 8, 2, 128, 2, 16, 24
+    n_prompt = n_full * bs + 5
+    full_ids = [int(x) + 2 for x in synth.permutation(1410 + n_full, nb - 2)[: n_full + 1]]
+    names = [f"model.layers.{l}.self_attn.attn" for l in range(L)]
+    results = []
+    for device_loads in (True, False):
+        cfg = make_config(hq, hkv, d, L, bs, 16 * 64, {})
+        cfg.kv_transfer_config.kv_connector_extra_config = {"ucm_sparse_config": {"KVStarMultiStep": {
+            "retrieval_stride": 4, "sparse_ratio": 0.25, "blk_repre_dim_prune_ratio": 1.0, "blk_repre_inner_token_merge": 4,
+            "device_loads": device_loads, "device_plans": device_loads}}}
+        slice_bytes = bs * hkv * d * 2
+        plugin = UcmSparseFactory.create_sparse_method(cfg, UcmSparseRole.WORKER)
+        plugin.connector = UcmHipBlockStore({"kv_block_size": L * 2 * slice_bytes, "max_cache_size": 16 * L * 2 * slice_bytes})
+        g = torch.Generator(device=dev)
+        g.manual_seed(33)
+        caches = [(torch.randn(2, nb, bs, hkv, d, device=dev, generator=g) * 0.3).to(torch.bfloat16) for _ in range(L)]
+        original = [c.clone() for c in caches]
+        req = ns(block_ids=[list(full_ids)], num_computed_tokens=0, prompt_token_ids=list(range(7, 7 + n_prompt)), output_token_ids=[],
+                 num_prompt_tokens=n_prompt, num_output_tokens=0, num_tokens=n_prompt, request_id="9")
+        ib = ns(req_id_to_index={"9": 0})
+
+        def run_step(n_tok):
+            so = ns(num_scheduled_tokens={"9": n_tok}, req_sparsed_slots={"9": 0})
+            md = ns(query_start_loc=torch.tensor([0, n_tok]))
+            fc = ns(no_compile_layers={names[l]: ns(kv_cache=[caches[l]]) for l in range(L)}, virtual_engine=0, attn_metadata=md)
+            plugin.build_sparse_meta(so, {"9": req}, ib, md)
+            for l in range(L):
+                q = (torch.randn(n_tok, hq, d, device=dev, generator=g) * 0.3).to(torch.bfloat16)
+                plugin.attention_begin(q, None, None, names[l], fc)
+                plugin.attention_finished(q, None, None, None, names[l], fc)
+            req.num_computed_tokens += n_tok
+
+        run_step(n_prompt)
+        hashes = plugin.req_states["9"][0].block_hashes
+        store = plugin.connector
+        assert store.create(hashes) == [0] * len(hashes)
+        from ucm_amd.sparse.esa.esa import get_offset
+        for l in range(L):
+            for kv in range(2):
+                off = get_offset((bs, hkv, d), 0, 1, 2, l, bool(kv))
+                store.wait(store.dump(hashes, [off] * len(hashes), [original[l][kv][full_ids[i]] for i in range(len(hashes))]))
+        store.commit(hashes)
+        req.output_token_ids.append(1)
+        req.num_output_tokens, req.num_tokens = 1, n_prompt + 1
+        slots = plugin.estimate_num_slots_sparsed(req)
+        kept = full_ids[-math.ceil(slots / bs):] if slots > 0 else list(full_ids)
+        req.block_ids = [list(kept)]
+        run_step(1)
+        torch.cuda.synchronize()
+        for l in range(L):
+            plugin.req_states["9"][l].wait_for_blk_transfer_task_done()
+        torch.cuda.synchronize()
+        results.append((kept, [c.clone() for c in caches], original))
+    (kept_a, caches_a, original), (kept_b, caches_b, _) = results
+    assert kept_a == kept_b
+    for l in range(L):
+        assert torch.equal(caches_a[l], caches_b[l]), l
+        # the request's last two blocks hold the local window, whatever else the list is short for
+        n_local = min(2, len(kept_a))
+        want = original[l][:, full_ids[: n_full + 1][-2:][-n_local:]]
+        assert torch.equal(caches_a[l][:, kept_a[-n_local:]], want), l

@@ -600,9 +600,10 @@ class KVStarMultiStep(UcmSparseBase):
         if missing:
             self._report_missing(missing)
         if src:
-            # a request whose block list is shorter than its two windows together names a cache block twice on the
-            # way back: the reference writes the init window, then the local one over it (multistep.py:348-362), so
-            # of the copies into one block only the last is made (the copies of one launch are not ordered)
+            # a block list shorter than the request's two windows together (this plugin's own slot estimate never
+            # leaves one; another scheduler might) names a cache block twice on the way back: the reference writes
+            # the init window, then the local one over it (multistep.py:348-362), so of the copies into one block
+            # only the last is made (the copies of one launch are not ordered)
             last = {d: i for i, d in enumerate(dst)}
             if len(last) != len(dst):
                 keep = [i for i, d in enumerate(dst) if last[d] == i]
