@@ -78,7 +78,9 @@ class DeviceSide:
         view = a.view(np.int16) if a.dtype == np.uint16 else a      # torch has no uint16 arithmetic type to hold bf16 bits
         t = self.torch.from_numpy(view.copy()).to(self.dev)
         if a.dtype == np.uint16:
-            self._u16 = getattr(self, "_u16", set()) | {t.data_ptr()}
+            # (the tensor itself is kept, not its address: a freed tensor's address comes back with another type behind it)
+            self._u16 = getattr(self, "_u16", {})
+            self._u16[id(t)] = t
         return t
 
     def ptr(self, t):
@@ -90,7 +92,7 @@ class DeviceSide:
 
     def down(self, t):
         a = t.cpu().numpy()
-        return a.view(np.uint16) if t.data_ptr() in getattr(self, "_u16", set()) else a
+        return a.view(np.uint16) if getattr(self, "_u16", {}).get(id(t)) is t else a
 
     def sync(self):
         self.torch.cuda.synchronize()
