@@ -277,7 +277,12 @@ class KvCompDevicePath:
                     self.win_shape[rid] = (n_head, len(blocks) - n_head)
                     self.windows[rid] = torch.empty(L * 2 * len(blocks) * block_bytes, dtype=torch.uint8, device=self.device)
                 else:
-                    blocks = self._window_blocks(meta.vllm_block_ids, *self.win_shape[rid])
+                    n_head, n_tail = self.win_shape[rid]
+                    if len(meta.vllm_block_ids) < max(n_head, n_tail):
+                        # (upstream's indexed assignment fails on the same lists: kvcomp.py:392-404)
+                        raise ValueError(f"KvComp: request {rid} holds {len(meta.vllm_block_ids)} cache blocks, fewer than "
+                                         f"one of its saved windows ({n_head} and {n_tail} blocks)")
+                    blocks = self._window_blocks(meta.vllm_block_ids, n_head, n_tail)
                 n, ptr = len(blocks), self.windows[rid].data_ptr()
                 # a request whose new block list is shorter than its two windows together gets a cache block named
                 # twice on the way back: the reference writes the first window, then the last one over it
