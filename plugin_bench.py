@@ -102,6 +102,7 @@ class Harness:
                 qs = [(self.rho * a.float() + math.sqrt(1.0 - self.rho ** 2) * b.float()).to(torch.bfloat16)
                       for a, b in zip(self._last_q, qs)]
             self._last_q = qs
+        self.last_queries = qs         # what this step's hooks are handed, layer by layer (tests look at them)
         so = ns(num_scheduled_tokens=dict((rid, n_tokens[rid]) for rid in live), req_sparsed_slots={rid: 0 for rid in live},
                 scheduled_new_reqs=[ns(req_id=rid) for rid in live if self.reqs[rid].num_computed_tokens == 0],
                 scheduled_cached_reqs=ns(req_ids=[rid for rid in live if self.reqs[rid].num_computed_tokens > 0]))

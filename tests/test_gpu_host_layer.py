@@ -528,6 +528,61 @@ def test_gsa_drawn_scenarios(ucm, dev, seed, lag):
 
 
 @pytest.mark.parametrize("lag", [0, 1])
+def test_gsa_plugin_at_serving_size(ucm, dev, lag):
+    """Sixteen requests of 280 to 400 blocks of 128 tokens, 32 layers, Llama-3-8B head shape, through the plugin's
+    hooks as the benchmark's plugin leg drives them (two cache tensors stand behind the 32 layers): after each of four
+    decode steps every layer's row of the block table and its length are the oracle's selection for every request,
+    from the representatives the plugin's own table holds and the queries the layer was handed - this step's, or
+    with retrieval_lag 1 and from the second decode step on the step before's."""
+    import plugin_bench as PB
+    from ucm_amd.sparse.base import UcmSparseRole
+    from ucm_amd.sparse.gsa.gsa import GSA
+
+    L, n_req, bs = 32, 16, PB.BS
+    rng = np.random.default_rng(41)
+    lens = rng.integers(280, 401, n_req)
+    nb = int(lens.sum()) + 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(42)
+    two = [torch.empty((2, nb, bs, PB.HKV, PB.D), dtype=torch.bfloat16, device=dev).normal_(0.0, 1.0, generator=g) for _ in range(2)]
+    caches = [two[l % 2] for l in range(L)]
+    perm = rng.permutation(nb)
+    starts = np.concatenate([[0], np.cumsum(lens)])
+    block_lists = [[int(x) for x in perm[starts[r] : starts[r + 1]]] for r in range(n_req)]
+    cfg = PB.make_config(L, 65536, n_req, "GSA", {"seg_prefill_threshold": 0, "repre_dtype": "bfloat16", "retrieval_lag": lag})
+    plugin = GSA(cfg, UcmSparseRole.WORKER)
+    h = PB.Harness(torch, dev, plugin, caches, PB._prompt_shape(lens), block_lists, 43, with_execute_hooks=True)
+    h.step("prefill", {rid: r.num_prompt_tokens for rid, r in h.reqs.items()}, query_rows=16)
+    torch.cuda.synchronize()
+    q_before, dropped = None, 0
+    for step in range(1, 5):
+        h.decode_token()
+        h.step("decode", {rid: 1 for rid in h.reqs})
+        torch.cuda.synchronize()
+        qs = [q.float().cpu().numpy() for q in h.last_queries]
+        lagged = lag == 1 and step >= 2
+        tables = plugin.block_tables_mp.cpu().numpy()
+        seq_out = plugin.gsa_seq_len.cpu().numpy()
+        for l in range(L):
+            table = plugin.kpre_caches[l].float().cpu().numpy()
+            for i, rid in enumerate(h.order):
+                st = plugin.gsa_stats[rid]
+                n = len(block_lists[i])
+                q = (q_before if lagged else qs)[l][i]
+                k = plugin._topk_len(n)
+                want_idx, _ = O.select_topk(q, table[st.slot_offset : st.slot_offset + n].reshape(n, PB.HKV, 1, PB.D), k)
+                seq_len = h.reqs[rid].num_computed_tokens          # (the harness has already counted this step's token)
+                phys, want_len = O.block_table_gather(block_lists[i], want_idx, seq_len, bs)
+                assert seq_out[l, i] == want_len, (step, l, rid)
+                assert np.array_equal(tables[l, i, : len(phys)], phys), (step, l, rid)
+                dropped += int(len(phys) < n)
+        q_before = qs
+    assert dropped == 4 * L * n_req
+    for rid in list(h.reqs):
+        plugin.request_finished_in_worker(rid)
+
+
+@pytest.mark.parametrize("lag", [0, 1])
 def test_gsa_retrieval_stride_reuses_scores(ucm, dev, lag):
     """With retrieval_stride 3 the scores of the last retrieval are re-selected with the current lengths
     on the steps in between (the last two blocks are always kept, so the newest block is never missing);
