@@ -39,17 +39,19 @@ def _config(hq, hkv, d, layers, bs, max_model_len, max_num_seqs, esa_cfg):
               kv_transfer_config=ns(kv_connector_extra_config={"ucm_sparse_config": {"ESA": esa_cfg}}))
 
 
-@pytest.mark.parametrize("pool_where,model_dtype,churn", [("cuda", "bfloat16", False), ("pinned", "bfloat16", False),
-                                                          ("cuda", "float16", False), ("cuda", "bfloat16", True)])
-def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype, churn):
+@pytest.mark.parametrize("pool_where,model_dtype,churn,serving", [
+    ("cuda", "bfloat16", False, False), ("pinned", "bfloat16", False, False), ("cuda", "float16", False, False),
+    ("cuda", "bfloat16", True, False), ("cuda", "bfloat16", True, True)])
+def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype, churn, serving):
     """churn: three requests finish before step 7 and three others start at step 8, in the table rows, representative
-    slots and batch positions the first three gave back."""
+    slots and batch positions the first three gave back.  serving: Llama-3-8B's head shape and blocks of 128 tokens
+    (eight layers), instead of the small shape the other cases run in 32 layers."""
     from ucm_amd import ops
     from ucm_amd.sparse.base import UcmSparseRole
     from ucm_amd.sparse.esa.esa import ESA
     from ucm_amd.store.hip_block_store import UcmHipBlockStore
 
-    hq, hkv, d, L, bs = 8, 2, 64, 32, 16
+    hq, hkv, d, L, bs = (32, 8, 128, 8, 128) if serving else (8, 2, 64, 32, 16)
     n_req = 16 if pool_where == "cuda" else 5
     nb = 2048
     stride_cfg = 5
@@ -86,7 +88,7 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype, churn):
     assert used <= nb
 
     # host model of every (request, layer)
-    model = {}
+    model, keys_h = {}, {}
     host_ms = {"prefill": [], "first": [], "retrieve": [], "load": [], "idle": []}
 
     def engine_step(t):
@@ -154,7 +156,9 @@ def test_esa_device_path_flow(ucm, dev, pool_where, model_dtype, churn):
                          resident=[np.full(top_k, -1, np.int32) for _ in range(L)])
                 ids = r.block_ids[0]
                 for l in range(L):
-                    kc = original[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+                    if l not in keys_h:                    # (a layer's keys as the oracle reads them, fetched once)
+                        keys_h[l] = original[l][0].view(torch.int16).cpu().numpy().view(np.uint16)
+                    kc = keys_h[l]
                     want = np.zeros((plugin.num_slots, hkv * d), np.float32)
                     O.block_mean_paged(kc, ids[:sparse_range], m["slots"][l], want, round_bf16=True,
                                        keys_f16=(model_dtype == torch.float16))
