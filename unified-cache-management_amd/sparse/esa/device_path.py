@@ -28,7 +28,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ... import ops
+from ... import _lib, ops
 from ..utils import HeldBlocks
 
 
@@ -126,6 +126,10 @@ class EsaDevicePath:
         self._kv_one: List[Optional[ops.LayerPointers]] = [None] * esa.total_num_hidden_layers
         self._kv_all: Optional[ops.LayerPointers] = None
         self.device = device
+        # a layer's retrieval and plan go to the library with addresses taken once: the tables are this object's own,
+        # and slicing and re-validating a dozen tensors per layer and step took twice the time of the calls themselves
+        self._retr_const: List[Optional[tuple]] = [None] * esa.total_num_hidden_layers
+        self._plan_const: List[Optional[tuple]] = [None] * esa.total_num_hidden_layers
 
     # ---- caches ----------------------------------------------------------------------------
     def register_kv_cache(self, layer_id: int, kv_cache: torch.Tensor) -> None:
@@ -265,14 +269,42 @@ class EsaDevicePath:
 
     def _retrieve(self, layer_id: int, query: torch.Tensor, rows: torch.Tensor, qpos: torch.Tensor, m: int) -> None:
         t = self.tables
-        ops.esa_retrieve_rows(self.esa.data[layer_id], self._queries(query, qpos), t.slot_table[layer_id], m, rows,
-                              t.topk_rows, t.max_slots, t.scores_ws, t.out_idx[layer_id], t.out_pos[layer_id],
-                              t.out_scores[layer_id], t.out_count[layer_id])
+        q = self._queries(query, qpos)
+        table = self.esa.data                                # [layers, slots, dim]
+        c = self._retr_const[layer_id]
+        if c is None or c[0] is not table:                   # first call of a layer: through the checked wrapper
+            data = table[layer_id]
+            ops.esa_retrieve_rows(data, q, t.slot_table[layer_id], m, rows, t.topk_rows, t.max_slots, t.scores_ws,
+                                  t.out_idx[layer_id], t.out_pos[layer_id], t.out_scores[layer_id], t.out_count[layer_id])
+            self._retr_const[layer_id] = (table, data.data_ptr(), data.shape[0], data.shape[1], t.slot_table[layer_id].data_ptr(),
+                                          t.max_rows, t.max_blocks, t.topk_rows.data_ptr(), t.max_slots, t.scores_ws.data_ptr(),
+                                          t.out_idx[layer_id].data_ptr(), t.out_pos[layer_id].data_ptr(),
+                                          t.out_scores[layer_id].data_ptr(), t.out_count[layer_id].data_ptr())
+            return
+        batch = rows.numel()
+        if m > c[6] or batch > c[5] or q.shape != (batch, c[3]) or q.dtype is not torch.float32 or not q.is_contiguous() \
+                or rows.dtype is not torch.int32 or not rows.is_cuda:
+            raise ValueError("ESA device path: queries or rows do not fit the tables")
+        rc = _lib.lib().ucm_esa_retrieve_rows(c[1], c[2], c[3], q.data_ptr(), c[4], c[5], c[6], m, rows.data_ptr(), batch, c[7],
+                                             c[8], c[9], c[10], c[11], c[12], c[13], c[8], ops.current_stream())
+        if rc != 0:
+            raise _lib.UcmHipError("ucm_esa_retrieve_rows", rc, _lib.lib().ucm_last_error().decode())
 
     def _plan(self, layer_id: int, rows: torch.Tensor) -> None:
         t, l = self.tables, slice(layer_id, layer_id + 1)
-        ops.delta_plan_rows(t.out_pos[l], t.out_pos[l], t.out_count[l], rows, t.resident[l], t.load_sel[l],
-                            t.slot_of_sel[l], t.miss_count[l])
+        c = self._plan_const[layer_id]
+        if c is None:
+            ops.delta_plan_rows(t.out_pos[l], t.out_pos[l], t.out_count[l], rows, t.resident[l], t.load_sel[l],
+                                t.slot_of_sel[l], t.miss_count[l])
+            self._plan_const[layer_id] = (t.out_pos[l].data_ptr(), t.out_count[l].data_ptr(), t.resident[l].data_ptr(),
+                                          t.load_sel[l].data_ptr(), t.slot_of_sel[l].data_ptr(), t.miss_count[l].data_ptr())
+            return
+        if rows.numel() > t.max_rows or rows.dtype is not torch.int32 or not rows.is_cuda:
+            raise ValueError("ESA device path: rows do not fit the tables")
+        rc = _lib.lib().ucm_delta_plan_rows(c[0], c[0], c[1], rows.data_ptr(), rows.numel(), t.max_rows, 1, t.max_slots, c[2],
+                                           t.max_slots, c[3], c[4], c[5], ops.current_stream())
+        if rc != 0:
+            raise _lib.UcmHipError("ucm_delta_plan_rows", rc, _lib.lib().ucm_last_error().decode())
 
     def _load(self, first_layer: int, n_layers: int, rows: torch.Tensor) -> None:
         t = self.tables
